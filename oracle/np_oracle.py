@@ -1,0 +1,305 @@
+"""NumPy restatement of the reference conv_nd / max_pool algorithm.
+
+TEST INFRASTRUCTURE: this module is the checker (and the timed CPU baseline of
+the benchmark); the shipped package never imports it.
+
+Every function follows the reference implementation named in its docstring
+(paths relative to the reference checkout) and hands the bulk arithmetic to the
+same NumPy routines the reference uses, so that on one NumPy/BLAS build it
+produces the reference's numbers: bit-for-bit for pooling, and up to BLAS
+summation order for convolution.
+
+``validate=False`` switches off the exact-integer output-shape check of the
+Operation layer, leaving the flooring placement rule of the window helper; the
+benchmark shapes that the reference's validation rejects are checked that way.
+
+Pinning (what holds each function to the reference without importing it):
+
+  window_view      definition ``out[g] == arr[..., g*S : g*S + W*D : D]`` on
+                   random cases + the reference's docstring / memory vectors
+  conv_forward     reference known answers (1-D, 2-D, triangle response,
+                   padding-only image), brute-force loops
+  conv_backward_x  reference docstring gradient, brute-force loops,
+  conv_backward_w  adjoint identity <conv(x,w),g> = <x,dx> = <w,dw>,
+                   central differences
+  pool_forward     three reference known-answer cases + the docstring case
+  pool_backward    with a tie, brute-force loops on tie-heavy integer inputs
+"""
+
+from numbers import Integral
+
+import numpy as np
+from numpy.lib.stride_tricks import as_strided
+
+__all__ = [
+    "window_view",
+    "normalize_conv_args",
+    "conv_out_shape",
+    "conv_forward",
+    "conv_backward_x",
+    "conv_backward_w",
+    "pool_out_shape",
+    "pool_forward",
+    "pool_backward",
+]
+
+
+# --------------------------------------------------------------------------- #
+# window helper
+# --------------------------------------------------------------------------- #
+def window_view(arr, window_shape, step, dilation=None):
+    """Read-only strided window view, shape ``(G..., lead..., W...)``.
+
+    Follows src/mygrad/nnet/layers/utils.py:123-228 (validation :123-196,
+    stride arithmetic :198-228).  ``view[g, lead, w] = arr[lead, g*S + w*D]``
+    with ``G = (x - ((W-1)*D + 1)) // S + 1`` (floor).
+    """
+    if not hasattr(window_shape, "__iter__"):
+        raise TypeError(f"`window_shape` must be a sequence of positive integers, got: {window_shape}")
+    window_shape = tuple(window_shape)
+    if any(not isinstance(w, Integral) or w <= 0 for w in window_shape):
+        raise TypeError(f"`window_shape` must be a sequence of positive integers, got: {window_shape}")
+    m = len(window_shape)
+    if m > arr.ndim:
+        raise ValueError(
+            f"`window_shape` ({window_shape}) cannot specify more values than `arr.ndim` ({arr.ndim})."
+        )
+
+    if isinstance(step, Integral):
+        step = (int(step),) * m
+    elif hasattr(step, "__iter__"):
+        step = tuple(step)
+    else:
+        raise TypeError(f"`step` must be a positive integer or a sequence of positive integers, got: {step}")
+    if any(not isinstance(s, Integral) or s <= 0 for s in step):
+        raise ValueError(f"`step` must be a positive integer or a sequence of positive integers, got: {step}")
+
+    trailing = arr.shape[arr.ndim - m :] if m else ()
+    if any(w > x for w, x in zip(window_shape[::-1], arr.shape[::-1])):
+        raise ValueError(
+            f"Each size of the window-shape must fit within the trailing dimensions of `arr`."
+            f"{window_shape} does not fit in {trailing}"
+        )
+
+    if dilation is None:
+        dilation = (1,) * m
+    else:
+        if isinstance(dilation, Integral):
+            dilation = (int(dilation),) * m
+        elif not hasattr(dilation, "__iter__"):
+            raise TypeError(
+                f"`dilation` must be None, a positive integer, or a sequence of positive integers, got: {dilation}"
+            )
+        if len(dilation) != m or any(not isinstance(d, Integral) or d <= 0 for d in dilation):
+            raise ValueError(
+                f"`dilation` must be None, a positive integer, or a sequence of positive integers "
+                f"with the same length as `window_shape` ({window_shape}), got: {dilation}"
+            )
+        dilation = tuple(dilation)
+        # the reference rejects w*d > dim (stricter than the true span (w-1)*d+1)
+        if any(w * d > x for w, d, x in zip(window_shape[::-1], dilation[::-1], arr.shape[::-1])):
+            raise ValueError(
+                f"The dilated window ({tuple(w * d for w, d in zip(window_shape, dilation))}) must fit "
+                f"within the trailing dimensions of `arr` ({trailing})"
+            )
+
+    if not arr.flags["C_CONTIGUOUS"]:
+        arr = np.ascontiguousarray(arr)
+
+    item = arr.itemsize
+    elem_strides = _c_elem_strides(arr.shape)
+    lead = arr.ndim - m
+    grid, grid_strides, win_strides = [], [], []
+    for k in range(m):
+        x_k, es = arr.shape[lead + k], elem_strides[lead + k]
+        span = (window_shape[k] - 1) * int(dilation[k]) + 1
+        grid.append((x_k - span) // int(step[k]) + 1)
+        grid_strides.append(int(step[k]) * es)
+        win_strides.append(int(dilation[k]) * es)
+
+    shape = tuple(grid) + arr.shape[:lead] + tuple(int(w) for w in window_shape)
+    strides = tuple(item * s for s in (*grid_strides, *elem_strides[:lead], *win_strides))
+    return as_strided(arr, shape=shape, strides=strides, writeable=False)
+
+
+def _c_elem_strides(shape):
+    """Row-major element strides as plain shape products (utils.py:207)."""
+    out, acc = [], 1
+    for n in reversed(shape):
+        out.append(acc)
+        acc *= int(n)
+    return out[::-1]
+
+
+# --------------------------------------------------------------------------- #
+# convolution
+# --------------------------------------------------------------------------- #
+def _per_axis(value, m, name, lowest):
+    """int-or-sequence -> int array of length m; AssertionError like
+    src/mygrad/nnet/layers/conv.py:35-61."""
+    if isinstance(value, Integral):
+        arr = np.array((value,) * m)
+    else:
+        arr = np.array(value, dtype=int)
+    if len(arr) != m or not all(v >= lowest and isinstance(v, Integral) for v in arr):
+        raise AssertionError(f"bad {name}: {value}")
+    return arr
+
+
+def normalize_conv_args(m, stride, padding, dilation):
+    dilation = _per_axis(dilation, m, "dilation", 1)
+    padding = _per_axis(padding, m, "padding", 0)
+    stride = _per_axis(stride, m, "stride", 1)
+    return stride, padding, dilation
+
+
+def conv_out_shape(x_spatial, w_spatial, stride, padding, dilation, validate=True):
+    """Grid shape ``(G0, ...)``.  Exact-integer rule of conv.py:63-74 when
+    ``validate``; otherwise the window helper's floor rule (utils.py:221-222)."""
+    xs, ws = np.array(x_spatial), np.array(w_spatial)
+    span = (ws - 1) * dilation + 1
+    if validate:
+        exact = (xs + 2 * padding - span) / stride + 1
+        if not all(g.is_integer() and g > 0 for g in exact):
+            raise ValueError(
+                "Stride and kernel dimensions are incompatible: \n"
+                f"Input dimensions: {tuple(xs)}\n"
+                f"Stride dimensions: {tuple(stride)}\n"
+                f"Kernel dimensions: {tuple(ws)}\n"
+                f"Padding dimensions: {tuple(padding)}\n"
+                f"Dilation dimensions: {tuple(dilation)}\n"
+            )
+    return tuple(int(g) for g in (xs + 2 * padding - span) // stride + 1)
+
+
+def _zero_pad(x, padding):
+    if not sum(padding):
+        return x
+    return np.pad(x, ((0, 0), (0, 0), *((int(p), int(p)) for p in padding)), mode="constant")
+
+
+def conv_forward(x, w, *, stride, padding=0, dilation=1, validate=True):
+    """``out[n,f,g] = sum_{c,t} w[f,c,t] * xpad[n,c,g*s+t*d]`` as pad -> window
+    view -> tensordot -> move N to the front.  Follows conv.py:15-103."""
+    assert x.ndim > 2 and x.ndim == w.ndim and x.shape[1] == w.shape[1]
+    m = x.ndim - 2
+    stride, padding, dilation = normalize_conv_args(m, stride, padding, dilation)
+    conv_out_shape(x.shape[2:], w.shape[2:], stride, padding, dilation, validate)
+
+    windows = window_view(_zero_pad(x, padding), w.shape[2:], tuple(stride), tuple(dilation))
+    # w: (F, C, W...) ; windows: (G..., N, C, W...)  ->  (F, G..., N)
+    w_axes = list(range(1, m + 2))
+    win_axes = list(range(m + 1, 2 * m + 2))
+    out = np.moveaxis(np.tensordot(w, windows, axes=[w_axes, win_axes]), -1, 0)
+    return np.ascontiguousarray(out)
+
+
+def conv_backward_x(grad, x_shape, x_dtype, w, *, stride, padding=0, dilation=1):
+    """dx: GEMM ``(N, G..., F) @ (F, C*W...)`` then a col2im loop over grid
+    positions in row-major order, accumulating in ``x_dtype``; padding cropped.
+    Follows conv.py:114-138."""
+    m = grad.ndim - 2
+    stride, padding, dilation = normalize_conv_args(m, stride, padding, dilation)
+    padded = tuple(x_shape[:2]) + tuple(int(n + 2 * p) for n, p in zip(x_shape[2:], padding))
+    dx = np.zeros(padded, dtype=x_dtype)
+
+    spread = np.tensordot(grad, w, axes=[[1], [0]])  # (N, G..., C, W...)
+    taps = w.shape[2:]
+    for g in np.ndindex(*grad.shape[2:]):
+        where = tuple(
+            slice(gk * sk, gk * sk + tk * dk, dk) for gk, tk, sk, dk in zip(g, taps, stride, dilation)
+        )
+        dx[(Ellipsis, *where)] += spread[(slice(None), *g, Ellipsis)]
+
+    if sum(padding):
+        dx = dx[(Ellipsis, *(slice(int(p), -int(p) if p else None) for p in padding))]
+    return dx
+
+
+def conv_backward_w(grad, x, w_shape, *, stride, padding=0, dilation=1):
+    """dw: pad -> window view -> tensordot over ``(G..., N)``.  Follows
+    conv.py:140-155."""
+    m = grad.ndim - 2
+    stride, padding, dilation = normalize_conv_args(m, stride, padding, dilation)
+    windows = window_view(_zero_pad(x, padding), tuple(w_shape[2:]), tuple(stride), tuple(dilation))
+    grad_axes = list(range(2, m + 2)) + [0]
+    win_axes = list(range(m + 1))
+    return np.tensordot(grad, windows, axes=[grad_axes, win_axes])
+
+
+# --------------------------------------------------------------------------- #
+# max-pool
+# --------------------------------------------------------------------------- #
+def _pool_args(x, pool, stride):
+    """AssertionErrors of src/mygrad/nnet/layers/pooling.py:52-68."""
+    if not isinstance(pool, (tuple, list, np.ndarray)) or not all(
+        p >= 0 and isinstance(p, Integral) for p in pool
+    ):
+        raise AssertionError(f"bad pool: {pool}")
+    pool = np.asarray(pool, dtype=int)
+    if not all(p > 0 for p in pool):
+        raise AssertionError(f"bad pool: {pool}")
+    if x.ndim < len(pool):
+        raise AssertionError("The number of pooled dimensions cannot exceed the dimensionality of the data.")
+    if isinstance(stride, Integral):
+        stride = np.array([stride] * len(pool))
+    else:
+        stride = np.asarray(stride, dtype=int)
+    if len(stride) != len(pool) or not all(s >= 1 and isinstance(s, Integral) for s in stride):
+        raise AssertionError(f"bad stride: {stride}")
+    return pool, stride
+
+
+def pool_out_shape(x_pooled_dims, pool, stride, validate=True):
+    """Exact-integer rule of pooling.py:79-86 when ``validate``, else floor."""
+    xs = np.array(x_pooled_dims)
+    if validate:
+        exact = (xs - pool) / stride + 1
+        if not all(g.is_integer() and g > 0 for g in exact):
+            raise ValueError(
+                "Stride and kernel dimensions are incompatible: \n"
+                f"Input dimensions: {tuple(xs)}\n"
+                f"Stride dimensions: {tuple(stride)}\n"
+                f"Pooling dimensions: {tuple(pool)}\n"
+            )
+    return tuple(int(g) for g in (xs - pool) // stride + 1)
+
+
+def pool_forward(x, pool, stride, validate=True):
+    """Windowed max over the trailing ``len(pool)`` axes.  Follows
+    pooling.py:49-98."""
+    pool, stride = _pool_args(x, pool, stride)
+    m = len(pool)
+    lead = x.ndim - m
+    pool_out_shape(x.shape[lead:], pool, stride, validate)
+    peak = window_view(x, tuple(pool), tuple(stride)).max(axis=tuple(range(-m, 0)))  # (G..., lead...)
+    order = tuple(range(m, m + lead)) + tuple(range(m))
+    return np.ascontiguousarray(peak.transpose(order))
+
+
+def pool_backward(x, grad, pool, stride):
+    """Route ``grad`` to the first-occurrence argmax of every window with an
+    unbuffered, C-ordered ``np.add.at`` into a float64 image.  Follows
+    pooling.py:100-149 (argmax :111, index algebra :119-144, add.at :147-148).
+    The result is float64 whatever ``x.dtype`` is, like the reference."""
+    pool, stride = _pool_args(x, pool, stride)
+    m = len(pool)
+    lead_shape, pooled_shape = x.shape[: x.ndim - m], x.shape[x.ndim - m :]
+
+    windows = window_view(x, tuple(pool), tuple(stride))  # (G..., lead..., P...)
+    grid = windows.shape[:m]
+    winner = windows.reshape(*windows.shape[: windows.ndim - m], -1).argmax(-1)  # (G..., lead...)
+    nd = winner.ndim
+    winner = winner.transpose(tuple(range(m, nd)) + tuple(range(m)))  # (lead..., G...)
+
+    unit = _c_elem_strides(pooled_shape)  # flat offset of one step along each pooled axis
+    inside = sum(a * u for a, u in zip(np.unravel_index(winner, tuple(pool)), unit))
+    corner = sum(g * int(s) * u for g, s, u in zip(np.indices(grid), stride, unit))
+
+    flat_shape = (*lead_shape, int(np.prod(grid)))
+    where = np.indices(flat_shape)
+    where[-1] = (inside + corner).reshape(flat_shape)
+
+    dx = np.zeros((*lead_shape, int(np.prod(pooled_shape))))
+    np.add.at(dx, tuple(where), grad.reshape(flat_shape))
+    return dx.reshape(x.shape)

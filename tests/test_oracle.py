@@ -1,0 +1,298 @@
+"""Pins the CPU oracle: reference known answers, definition-level brute force,
+adjoint identity, finite differences, and NumPy library routines on tiny cases.
+A dropped term, a wrong sign/index or a transposed axis list fails one of these."""
+
+import itertools
+
+import numpy as np
+import pytest
+from hypothesis import given, settings
+from hypothesis import strategies as st
+
+from oracle import brute, direct
+from oracle import np_oracle as ora
+
+
+# ----------------------------------------------------------------------------- window helper
+def test_window_docstring_vectors(kats):
+    case = kats["window"][0]
+    x = np.arange(36).reshape(6, 6)
+    y = ora.window_view(x, case["window_shape"], case["step"])
+    assert list(y.shape) == case["shape"]
+    for key, want in case["picks"].items():
+        i, j = map(int, key.split(","))
+        assert np.array_equal(y[i, j], np.array(want))
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int64, np.float16, np.float32, np.float64])
+def test_window_memory_details(kats, dtype):
+    case = kats["window"][1]
+    want = np.array(case["view"])
+    x = np.asfortranarray(np.arange(20).reshape(2, 10).astype(dtype))
+    y = ora.window_view(x, (5,), 5)
+    assert not y.flags["WRITEABLE"]
+    assert np.array_equal(y, want)
+    x = np.ascontiguousarray(np.arange(20).reshape(2, 10))
+    y = ora.window_view(x, (5,), 5)
+    assert not y.flags["WRITEABLE"] and np.shares_memory(x, y)
+    assert np.array_equal(y, want)
+
+
+@settings(deadline=None, max_examples=150)
+@given(data=st.data(), shape=st.lists(st.integers(1, 7), min_size=1, max_size=4))
+def test_window_matches_slicing(data, shape):
+    x = np.arange(int(np.prod(shape))).reshape(shape)
+    m = data.draw(st.integers(1, len(shape)))
+    tail = shape[-m:]
+    win = tuple(data.draw(st.integers(1, s)) for s in tail)
+    step = tuple(data.draw(st.integers(1, s)) for s in tail)
+    dil = tuple(data.draw(st.integers(1, s // w)) for s, w in zip(tail, win))
+    y = ora.window_view(x, win, step, dil)
+    grid = tuple((s - ((w - 1) * d + 1)) // st_ + 1 for s, w, st_, d in zip(tail, win, step, dil))
+    assert y.shape == grid + tuple(shape[:-m]) + win
+    for g in np.ndindex(*grid):
+        sl = tuple(slice(i * s, i * s + w * d, d) for i, w, s, d in zip(g, win, step, dil))
+        assert np.array_equal(y[g], x[(Ellipsis, *sl)])
+
+
+@pytest.mark.parametrize(
+    "kwargs",
+    [
+        dict(step=None),
+        dict(step=-1),
+        dict(window_shape=None),
+        dict(window_shape=1),
+        dict(window_shape=(1, 1, 1)),
+        dict(window_shape=(-1, 1)),
+        dict(window_shape=(1.0, 2.0)),
+        dict(window_shape=(7, 5)),
+        dict(dilation=-1),
+        dict(dilation=(1, 0)),
+        dict(dilation="aa"),
+        dict(dilation=(1, 1, 1)),
+        dict(dilation=1.0),
+        dict(dilation=7),
+        dict(dilation=(1, 7)),
+    ],
+)
+def test_window_validation(kwargs):
+    args = dict(arr=np.arange(36).reshape(6, 6), window_shape=(1, 1), step=1, dilation=None)
+    args.update(kwargs)
+    with pytest.raises((ValueError, TypeError)):
+        ora.window_view(**args)
+
+
+# ----------------------------------------------------------------------------- convolution
+def test_conv_reference_known_answers(kats):
+    for case in kats["conv"]:
+        x, w = np.array(case["x"], dtype=float), np.array(case["w"], dtype=float)
+        conf = dict(stride=tuple(case["stride"]), padding=tuple(case["padding"]), dilation=tuple(case["dilation"]))
+        out = ora.conv_forward(x, w, **conf)
+        assert np.array_equal(out, np.array(case["out"], dtype=float)), case["source"]
+        if "dx_of_ones" in case:
+            g = np.ones_like(out)
+            dx = ora.conv_backward_x(g, x.shape, x.dtype, w, **conf)
+            dw = ora.conv_backward_w(g, x, w.shape, **conf)
+            assert np.array_equal(dx, np.array(case["dx_of_ones"], dtype=float))
+            assert np.array_equal(dw, np.array(case["dw_of_ones"], dtype=float))
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
+def test_conv_padding_only_image_is_zero(m):
+    # reference tests/nnet/layers/test_conv.py:247-273: an empty image padded by p
+    # and a kernel of extent 2p gives the single output 0.0
+    rng = np.random.default_rng(m)
+    pad = tuple(int(p) for p in rng.integers(1, 4, m))
+    x = np.zeros((1, 1) + (0,) * m)
+    w = rng.standard_normal((1, 1) + tuple(2 * p for p in pad))
+    out = ora.conv_forward(x, w, stride=1, padding=pad)
+    assert out.shape == (1,) * (m + 2) and out.item() == 0.0
+    dx = ora.conv_backward_x(np.ones_like(out), x.shape, x.dtype, w, stride=1, padding=pad)
+    assert dx.shape == x.shape
+
+
+def _random_conv_case(rng, m):
+    N, C, F = (int(v) for v in rng.integers(1, 4, 3))
+    taps = tuple(int(v) for v in rng.integers(1, 4, m))
+    dil = tuple(int(v) for v in rng.integers(1, 3, m))
+    stride = tuple(int(v) for v in rng.integers(1, 4, m))
+    pad = tuple(int(v) for v in rng.integers(0, 3, m))
+    grid = tuple(int(v) for v in rng.integers(1, 4, m))
+    X = tuple((g - 1) * s + (t - 1) * d + 1 - 2 * p for g, s, t, d, p in zip(grid, stride, taps, dil, pad))
+    if any(v < 1 for v in X):
+        return None
+    # the reference's window helper rejects taps*dilation > padded extent (utils.py:188-196)
+    if any(t * d > v + 2 * p for t, d, v, p in zip(taps, dil, X, pad)):
+        return None
+    x = rng.standard_normal((N, C, *X))
+    w = rng.standard_normal((F, C, *taps))
+    g = rng.standard_normal((N, F, *grid))
+    return x, w, g, dict(stride=stride, padding=pad, dilation=dil)
+
+
+@pytest.mark.parametrize("m", [1, 2, 3])
+def test_conv_oracle_vs_bruteforce_and_direct(m):
+    rng = np.random.default_rng(100 + m)
+    done = 0
+    while done < 12:
+        case = _random_conv_case(rng, m)
+        if case is None:
+            continue
+        x, w, g, conf = case
+        s, p, d = conf["stride"], conf["padding"], conf["dilation"]
+        out = ora.conv_forward(x, w, **conf)
+        dx = ora.conv_backward_x(g, x.shape, x.dtype, w, **conf)
+        dw = ora.conv_backward_w(g, x, w.shape, **conf)
+        assert out.shape == g.shape
+        np.testing.assert_allclose(out, brute.conv_forward(x, w, s, p, d), rtol=1e-12, atol=1e-12)
+        np.testing.assert_allclose(dx, brute.conv_backward_x(g, x.shape, w, s, p, d), rtol=1e-12, atol=1e-12)
+        np.testing.assert_allclose(dw, brute.conv_backward_w(g, x, w.shape, s, p, d), rtol=1e-12, atol=1e-12)
+        np.testing.assert_allclose(out, direct.conv_forward(x, w, s, p, d), rtol=1e-12, atol=1e-12)
+        np.testing.assert_allclose(dx, direct.conv_backward_x(g, x.shape, w, s, p, d), rtol=1e-12, atol=1e-12)
+        np.testing.assert_allclose(dw, direct.conv_backward_w(g, x, w.shape, s, p, d), rtol=1e-12, atol=1e-12)
+        done += 1
+
+
+def test_conv_floor_placement_ignores_trailing_rows():
+    # shapes the Operation-level validator rejects still run with the floor rule
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((2, 3, 8, 8))
+    w = rng.standard_normal((4, 3, 3, 3))
+    conf = dict(stride=2, padding=1, dilation=1)
+    with pytest.raises(ValueError):
+        ora.conv_forward(x, w, **conf)
+    out = ora.conv_forward(x, w, validate=False, **conf)
+    assert out.shape == (2, 4, 4, 4)
+    np.testing.assert_allclose(out, brute.conv_forward(x, w, (2, 2), (1, 1), (1, 1)), rtol=1e-12, atol=1e-12)
+    g = rng.standard_normal(out.shape)
+    dx = ora.conv_backward_x(g, x.shape, x.dtype, w, **conf)
+    np.testing.assert_allclose(dx, brute.conv_backward_x(g, x.shape, w, (2, 2), (1, 1), (1, 1)), rtol=1e-12, atol=1e-12)
+
+
+def test_conv_adjoint_identity_and_finite_differences():
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((3, 4, 9, 7))
+    w = rng.standard_normal((5, 4, 3, 2))
+    conf = dict(stride=(2, 1), padding=(1, 2), dilation=(1, 2))
+    out = ora.conv_forward(x, w, **conf)
+    g = rng.standard_normal(out.shape)
+    dx = ora.conv_backward_x(g, x.shape, x.dtype, w, **conf)
+    dw = ora.conv_backward_w(g, x, w.shape, **conf)
+    lhs = np.vdot(out, g)
+    assert abs(lhs - np.vdot(x, dx)) < 1e-10 * abs(lhs)
+    assert abs(lhs - np.vdot(w, dw)) < 1e-10 * abs(lhs)
+    # conv is linear in each argument: central differences are exact up to rounding
+    h = 1e-3
+    for _ in range(5):
+        i = tuple(int(rng.integers(0, n)) for n in x.shape)
+        e = np.zeros_like(x)
+        e[i] = h
+        num = (np.vdot(ora.conv_forward(x + e, w, **conf), g) - np.vdot(ora.conv_forward(x - e, w, **conf), g)) / (2 * h)
+        assert abs(num - dx[i]) < 1e-8 * max(1.0, abs(dx[i]))
+        j = tuple(int(rng.integers(0, n)) for n in w.shape)
+        e = np.zeros_like(w)
+        e[j] = h
+        num = (np.vdot(ora.conv_forward(x, w + e, **conf), g) - np.vdot(ora.conv_forward(x, w - e, **conf), g)) / (2 * h)
+        assert abs(num - dw[j]) < 1e-8 * max(1.0, abs(dw[j]))
+
+
+def test_conv_dtype_rules():
+    x = np.ones((1, 1, 5), dtype=np.float32)
+    w = np.ones((1, 1, 2), dtype=np.float32)
+    out = ora.conv_forward(x, w, stride=1)
+    assert out.dtype == np.float32
+    assert ora.conv_forward(x, w.astype(np.float64), stride=1).dtype == np.float64
+    assert ora.conv_backward_x(out, x.shape, x.dtype, w, stride=1).dtype == np.float32
+
+
+def test_conv_error_contract():
+    x = np.zeros((1, 2, 2, 2))
+    w = np.zeros((1, 2, 2, 2))
+    with pytest.raises(ValueError):
+        ora.conv_forward(x, np.zeros((1, 2, 3, 2)), stride=1, padding=0)
+    with pytest.raises(AssertionError):
+        ora.conv_forward(x, w, stride=0)
+    with pytest.raises(AssertionError):
+        ora.conv_forward(x, w, stride=[1, 2, 3])
+    with pytest.raises(AssertionError):
+        ora.conv_forward(x, w, stride=1, padding=-1)
+    with pytest.raises(AssertionError):
+        ora.conv_forward(x, w, stride=1, padding=[1, 2, 3])
+    with pytest.raises(ValueError):
+        ora.conv_forward(x, w, stride=3, padding=1)
+
+
+# ----------------------------------------------------------------------------- max-pool
+def test_pool_reference_known_answers(kats):
+    for case in kats["pool"]:
+        x = np.array(case["x"], dtype=case["dtype"])
+        out = ora.pool_forward(x, tuple(case["pool"]), tuple(case["stride"]))
+        assert out.dtype == x.dtype
+        assert np.array_equal(out, np.array(case["out"], dtype=x.dtype)), case["source"]
+        if case["grad"] is None:
+            continue
+        g = np.ones(out.shape) if case["grad"] == "ones" else np.arange(out.size).reshape(out.shape)
+        dx = ora.pool_backward(x, g, tuple(case["pool"]), tuple(case["stride"]))
+        assert dx.dtype == np.float64
+        assert np.array_equal(dx, np.array(case["dx"], dtype=float)), case["source"]
+        b_out, b_dx = brute.pool_forward_backward(x, g, case["pool"], case["stride"])
+        assert np.array_equal(b_out, out) and np.array_equal(b_dx, dx)
+        d_out, d_dx = direct.pool(x, g, case["pool"], case["stride"])
+        assert np.array_equal(d_out, out) and np.array_equal(d_dx, dx)
+
+
+@pytest.mark.parametrize("m,lead", [(1, (3,)), (2, (2, 2)), (3, (2,)), (2, ())])
+def test_pool_ties_overlap_bit_exact_vs_bruteforce(m, lead):
+    rng = np.random.default_rng(200 + m)
+    for trial in range(10):
+        pool = tuple(int(v) for v in rng.integers(1, 4, m))
+        stride = tuple(int(v) for v in rng.integers(1, 4, m))
+        grid = tuple(int(v) for v in rng.integers(1, 4, m))
+        slack = tuple(int(v) for v in rng.integers(0, 2, m))  # rows the floor rule never covers
+        X = tuple((g - 1) * s + p + e for g, s, p, e in zip(grid, stride, pool, slack))
+        X = tuple(x if (x - p) // s + 1 == g else (g - 1) * s + p for x, p, s, g in zip(X, pool, stride, grid))
+        dtype = np.float32 if trial % 2 else np.float64
+        x = rng.integers(0, 4, (*lead, *X)).astype(dtype)  # few distinct values: ties everywhere
+        g = rng.standard_normal((*lead, *grid)) * 10.0 ** rng.integers(-8, 8, (*lead, *grid))
+        out = ora.pool_forward(x, pool, stride, validate=False)
+        dx = ora.pool_backward(x, g, pool, stride)
+        b_out, b_dx = brute.pool_forward_backward(x, g, pool, stride)
+        assert np.array_equal(out.view(np.uint8), b_out.view(np.uint8))
+        assert np.array_equal(dx.view(np.uint64), b_dx.view(np.uint64))
+        d_out, d_dx = direct.pool(x, g.astype(dtype), pool, stride)
+        dx_t = ora.pool_backward(x, g.astype(dtype), pool, stride)
+        assert np.array_equal(d_out.view(np.uint8), out.view(np.uint8))
+        assert np.array_equal(d_dx.view(np.uint64), dx_t.view(np.uint64))
+
+
+def test_pool_accumulation_order_is_sequential_from_plus_zero():
+    # one input element wins three overlapping windows; a sequential sum keeps
+    # the 1.0 that a pairwise/reordered sum would lose
+    x = np.array([0.0, 0.0, 9.0, 0.0, 0.0])
+    g = np.array([1e16, 1.0, -1e16])
+    dx = ora.pool_backward(x, g, (3,), (1,))
+    assert dx[2] == (1e16 + 1.0) + -1e16 == 0.0
+    g = np.array([1e16, -1e16, 1.0])
+    assert ora.pool_backward(x, g, (3,), (1,))[2] == 1.0
+    # an element whose only contribution is -0.0 ends as +0.0; untouched ones are +0.0
+    dx = ora.pool_backward(np.array([1.0, 0.0]), np.array([-0.0]), (2,), (2,))
+    assert not np.signbit(dx).any()
+
+
+def test_pool_nan_routing():
+    x = np.array([1.0, np.nan, 5.0, np.nan])
+    assert np.isnan(ora.pool_forward(x, (4,), (1,))).all()
+    dx = ora.pool_backward(x, np.array([2.0]), (4,), (1,))
+    assert np.array_equal(dx, [0.0, 2.0, 0.0, 0.0])  # first NaN wins
+
+
+def test_pool_error_contract():
+    x = np.zeros((1, 2, 2, 2), dtype=np.float32)
+    with pytest.raises(ValueError):
+        ora.pool_forward(x, (3,) * 3, (1,) * 3)
+    with pytest.raises(AssertionError):
+        ora.pool_forward(x, (2,) * 3, (0,) * 3)
+    with pytest.raises(AssertionError):
+        ora.pool_forward(x, (2,) * 2, [1, 2, 3])
+    with pytest.raises(ValueError):
+        ora.pool_forward(x, (1,) * 3, (3,) * 3)
