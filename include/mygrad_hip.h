@@ -1,0 +1,134 @@
+/* libmygrad_hip.so -- C ABI of the MI355X (gfx950) conv_nd / max_pool kernels.
+ *
+ * Every function returns an mg_status (0 = OK, negative = error) and never
+ * aborts or throws; mg_last_error() gives the message of the calling thread's
+ * last failure.  All tensor arguments are DEVICE pointers obtained from
+ * mg_malloc() (plain pointers, C-contiguous row-major, NCHW-style).  Work is
+ * enqueued on one library-owned HIP stream; mg_sync() or a device-to-host copy
+ * fences it.  The library is not re-entrant: entry points take one global lock.
+ *
+ * "Reference" below is MyGrad (paths relative to its checkout).
+ */
+#ifndef MYGRAD_HIP_H
+#define MYGRAD_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MG_MAX_ND 3 /* spatial / pooled rank handled by the kernels */
+
+typedef enum {
+  MG_OK = 0,
+  MG_ERR_BAD_ARG = -1,     /* null pointer, non-positive extent, inconsistent shapes */
+  MG_ERR_UNSUPPORTED = -2, /* dtype / rank / size outside what the kernels handle */
+  MG_ERR_NO_DEVICE = -3,   /* no usable gfx950 device */
+  MG_ERR_OOM = -4,         /* device or pinned-host allocation failed */
+  MG_ERR_HIP = -5,         /* any other HIP runtime failure */
+  MG_ERR_NOT_INIT = -6     /* mg_init() has not succeeded */
+} mg_status;
+
+typedef enum { MG_F32 = 0, MG_F64 = 1 } mg_dtype;
+
+/* Shapes of one convolution  x:(N,C,X...) * w:(F,C,W...) -> out:(N,F,G...).
+ * Axes are right-aligned: a rank-nd problem fills the LAST nd entries of each
+ * array and leaves the leading ones at X=W=G=stride=dil=1, pad=0.  G is passed
+ * in, G[k] <= (X[k]+2*pad[k]-((W[k]-1)*dil[k]+1))/stride[k]+1 (floor), so the
+ * caller decides between the reference's exact-integer rule
+ * (src/mygrad/nnet/layers/conv.py:63-74) and the flooring placement of its
+ * window helper (src/mygrad/nnet/layers/utils.py:221-222). */
+typedef struct {
+  int32_t dtype; /* mg_dtype of x, w, out, grad, dx, dw alike */
+  int32_t nd;    /* 1..MG_MAX_ND */
+  int64_t N, C, F;
+  int64_t X[MG_MAX_ND], W[MG_MAX_ND], G[MG_MAX_ND];
+  int64_t stride[MG_MAX_ND], pad[MG_MAX_ND], dil[MG_MAX_ND];
+} mg_conv_desc;
+
+/* Shapes of one max-pool over the trailing nd axes of x:(lead, X...) ->
+ * out:(lead, G...), window P, step S, no padding, no dilation; `lead` is the
+ * product of the un-pooled leading axes (1 if there are none).  Right-aligned
+ * like mg_conv_desc.  G[k] <= (X[k]-P[k])/S[k]+1 (floor). */
+typedef struct {
+  int32_t dtype;    /* mg_dtype of x, out, grad */
+  int32_t dx_dtype; /* mg_dtype of dx: same as dtype, or MG_F64 for f32 input (the
+                       reference builds dx in float64, pooling.py:147) */
+  int32_t nd;       /* 1..MG_MAX_ND */
+  int32_t reserved;
+  int64_t lead;
+  int64_t X[MG_MAX_ND], P[MG_MAX_ND], S[MG_MAX_ND], G[MG_MAX_ND];
+} mg_pool_desc;
+
+typedef struct {
+  char name[64];      /* hipDeviceProp_t::gcnArchName */
+  int32_t compute_units;
+  int32_t clock_khz;
+  int32_t wavefront;
+  int32_t lds_bytes_per_block;
+  int64_t hbm_bytes;
+  int32_t l2_bytes;
+  int32_t memory_clock_khz;
+  int32_t memory_bus_bits;
+  int32_t reserved;
+} mg_device_info_t;
+
+/* ---- runtime (no reference counterpart: the reference is host-only NumPy) ---- */
+int mg_init(int device);           /* idempotent; picks the device, creates the stream */
+int mg_shutdown(void);             /* frees the stream, workspace and cached plans */
+const char *mg_last_error(void);   /* message of this thread's last failing call */
+int mg_device_info(mg_device_info_t *info);
+
+int mg_malloc(void **dptr, size_t nbytes);
+int mg_free(void *dptr);
+int mg_host_alloc(void **hptr, size_t nbytes); /* pinned host memory (hipHostMalloc) */
+int mg_host_free(void *hptr);
+int mg_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes); /* stream-ordered, returns when src may be reused */
+int mg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes); /* returns when dst holds the data */
+int mg_memcpy_d2d(void *dst_dev, const void *src_dev, size_t nbytes);  /* stream-ordered */
+int mg_memset_zero(void *dst_dev, size_t nbytes);                      /* stream-ordered fill kernel */
+int mg_sync(void);
+
+/* HIP events on the library stream, for timing kernels from the host. */
+int mg_event_create(void **event);
+int mg_event_record(void *event);
+int mg_event_elapsed_ms(void *start, void *stop, float *ms); /* synchronizes on `stop` */
+int mg_event_destroy(void *event);
+
+/* ---- convolution ---- */
+
+/* out[n,f,g] = sum_{c,t} w[f,c,t] * x[n,c,g*stride+t*dil-pad] (zero outside x).
+ * Replaces ConvND.__call__, src/mygrad/nnet/layers/conv.py:81-103 (np.pad +
+ * sliding_window_view + np.tensordot + moveaxis copy). */
+int mg_conv_fwd(const mg_conv_desc *desc, const void *x, const void *w, void *out);
+
+/* dx[n,c,i] = sum over (f,t,g) with g*stride+t*dil-pad == i of grad[n,f,g]*w[f,c,t].
+ * Replaces ConvND.backward_var(grad, 0), src/mygrad/nnet/layers/conv.py:114-138
+ * (tensordot + Python col2im loop + crop). */
+int mg_conv_dgrad(const mg_conv_desc *desc, const void *grad, const void *w, void *dx);
+
+/* dw[f,c,t] = sum_{n,g} grad[n,f,g] * x[n,c,g*stride+t*dil-pad].
+ * Replaces ConvND.backward_var(grad, 1), src/mygrad/nnet/layers/conv.py:140-155.
+ * Split over the (n,g) sum with a fixed-order second stage: run-to-run identical. */
+int mg_conv_wgrad(const mg_conv_desc *desc, const void *grad, const void *x, void *dw);
+
+/* ---- max-pool ---- */
+
+/* out[lead,g] = max_a x[lead, g*S+a]; NaN propagates; among equal maxima the
+ * value of the first (row-major in the window) is returned.
+ * Replaces MaxPoolND.__call__, src/mygrad/nnet/layers/pooling.py:93-98. */
+int mg_maxpool_fwd(const mg_pool_desc *desc, const void *x, void *out);
+
+/* dx[lead,i] = sum, in ascending row-major window order starting from +0.0 and
+ * accumulated in double, of grad[lead,g] over the windows g whose first-occurrence
+ * argmax is i (first NaN wins); rounded once to dx_dtype.  Atomic-free.
+ * Replaces MaxPoolND.backward_var, src/mygrad/nnet/layers/pooling.py:100-149
+ * (argmax :111, np.add.at :147-148). */
+int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, void *dx);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MYGRAD_HIP_H */

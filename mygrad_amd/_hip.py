@@ -1,0 +1,247 @@
+"""ctypes binding of ``libmygrad_hip.so`` (declared in ``include/mygrad_hip.h``).
+
+The library is loaded lazily on first use.  There is no CPU fallback: when the
+shared library is missing or no gfx950 device can be initialised, every kernel
+entry point raises :class:`HipUnavailable`.
+"""
+
+import ctypes
+import os
+import threading
+
+MG_MAX_ND = 3
+MG_F32, MG_F64 = 0, 1
+
+MG_OK = 0
+MG_ERR_BAD_ARG = -1
+MG_ERR_UNSUPPORTED = -2
+MG_ERR_NO_DEVICE = -3
+MG_ERR_OOM = -4
+MG_ERR_HIP = -5
+MG_ERR_NOT_INIT = -6
+
+_STATUS_NAMES = {
+    MG_ERR_BAD_ARG: "MG_ERR_BAD_ARG",
+    MG_ERR_UNSUPPORTED: "MG_ERR_UNSUPPORTED",
+    MG_ERR_NO_DEVICE: "MG_ERR_NO_DEVICE",
+    MG_ERR_OOM: "MG_ERR_OOM",
+    MG_ERR_HIP: "MG_ERR_HIP",
+    MG_ERR_NOT_INIT: "MG_ERR_NOT_INIT",
+}
+
+_I64x3 = ctypes.c_int64 * MG_MAX_ND
+
+
+class HipUnavailable(RuntimeError):
+    """The HIP library could not be loaded or no gfx950 device is usable."""
+
+
+class HipError(RuntimeError):
+    """A library call returned a non-zero status."""
+
+    def __init__(self, status, message):
+        super().__init__(f"{_STATUS_NAMES.get(status, status)}: {message}")
+        self.status = status
+
+
+class ConvDesc(ctypes.Structure):
+    _fields_ = [
+        ("dtype", ctypes.c_int32),
+        ("nd", ctypes.c_int32),
+        ("N", ctypes.c_int64),
+        ("C", ctypes.c_int64),
+        ("F", ctypes.c_int64),
+        ("X", _I64x3),
+        ("W", _I64x3),
+        ("G", _I64x3),
+        ("stride", _I64x3),
+        ("pad", _I64x3),
+        ("dil", _I64x3),
+    ]
+
+
+class PoolDesc(ctypes.Structure):
+    _fields_ = [
+        ("dtype", ctypes.c_int32),
+        ("dx_dtype", ctypes.c_int32),
+        ("nd", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+        ("lead", ctypes.c_int64),
+        ("X", _I64x3),
+        ("P", _I64x3),
+        ("S", _I64x3),
+        ("G", _I64x3),
+    ]
+
+
+class DeviceInfo(ctypes.Structure):
+    _fields_ = [
+        ("name", ctypes.c_char * 64),
+        ("compute_units", ctypes.c_int32),
+        ("clock_khz", ctypes.c_int32),
+        ("wavefront", ctypes.c_int32),
+        ("lds_bytes_per_block", ctypes.c_int32),
+        ("hbm_bytes", ctypes.c_int64),
+        ("l2_bytes", ctypes.c_int32),
+        ("memory_clock_khz", ctypes.c_int32),
+        ("memory_bus_bits", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+    ]
+
+
+_vp = ctypes.c_void_p
+_SIGNATURES = {
+    "mg_init": [ctypes.c_int],
+    "mg_shutdown": [],
+    "mg_device_info": [ctypes.POINTER(DeviceInfo)],
+    "mg_malloc": [ctypes.POINTER(_vp), ctypes.c_size_t],
+    "mg_free": [_vp],
+    "mg_host_alloc": [ctypes.POINTER(_vp), ctypes.c_size_t],
+    "mg_host_free": [_vp],
+    "mg_memcpy_h2d": [_vp, _vp, ctypes.c_size_t],
+    "mg_memcpy_d2h": [_vp, _vp, ctypes.c_size_t],
+    "mg_memcpy_d2d": [_vp, _vp, ctypes.c_size_t],
+    "mg_memset_zero": [_vp, ctypes.c_size_t],
+    "mg_sync": [],
+    "mg_event_create": [ctypes.POINTER(_vp)],
+    "mg_event_record": [_vp],
+    "mg_event_elapsed_ms": [_vp, _vp, ctypes.POINTER(ctypes.c_float)],
+    "mg_event_destroy": [_vp],
+    "mg_conv_fwd": [ctypes.POINTER(ConvDesc), _vp, _vp, _vp],
+    "mg_conv_dgrad": [ctypes.POINTER(ConvDesc), _vp, _vp, _vp],
+    "mg_conv_wgrad": [ctypes.POINTER(ConvDesc), _vp, _vp, _vp],
+    "mg_maxpool_fwd": [ctypes.POINTER(PoolDesc), _vp, _vp],
+    "mg_maxpool_bwd": [ctypes.POINTER(PoolDesc), _vp, _vp, _vp],
+}
+EXPORTED_SYMBOLS = tuple(_SIGNATURES) + ("mg_last_error",)
+
+_lock = threading.Lock()
+_lib = None
+_ready = False
+
+
+def library_path():
+    """Path of the shared library: ``$MYGRAD_HIP_LIB`` or the in-tree build."""
+    return os.environ.get("MYGRAD_HIP_LIB") or os.path.join(
+        os.path.dirname(os.path.abspath(__file__)), "libmygrad_hip.so"
+    )
+
+
+def load_library():
+    """dlopen the library and declare the prototypes (no device needed)."""
+    global _lib
+    with _lock:
+        if _lib is None:
+            path = library_path()
+            if not os.path.exists(path):
+                raise HipUnavailable(
+                    f"{path} does not exist; build it with `python -m mygrad_amd.build` "
+                    "(there is no CPU fallback)"
+                )
+            try:
+                lib = ctypes.CDLL(path)
+            except OSError as exc:
+                raise HipUnavailable(f"cannot load {path}: {exc}") from exc
+            for name, argtypes in _SIGNATURES.items():
+                fn = getattr(lib, name)
+                fn.argtypes = argtypes
+                fn.restype = ctypes.c_int
+            lib.mg_last_error.argtypes = []
+            lib.mg_last_error.restype = ctypes.c_char_p
+            _lib = lib
+    return _lib
+
+
+def last_error():
+    return load_library().mg_last_error().decode("utf-8", "replace")
+
+
+def check(status):
+    if status != MG_OK:
+        raise HipError(status, last_error())
+
+
+def lib():
+    """The loaded library with the device initialised; raises HipUnavailable otherwise."""
+    global _ready
+    handle = load_library()
+    if not _ready:
+        device = int(os.environ.get("MYGRAD_HIP_DEVICE", "0"))
+        status = handle.mg_init(device)
+        if status != MG_OK:
+            raise HipUnavailable(
+                f"mg_init({device}) failed: {_STATUS_NAMES.get(status, status)}: {last_error()} "
+                "(there is no CPU fallback)"
+            )
+        _ready = True
+    return handle
+
+
+def is_available():
+    """True when the library loads and a gfx950 device initialises."""
+    try:
+        lib()
+        return True
+    except HipUnavailable:
+        return False
+
+
+def device_info():
+    info = DeviceInfo()
+    check(lib().mg_device_info(ctypes.byref(info)))
+    return {name: (getattr(info, name).decode() if name == "name" else getattr(info, name))
+            for name, _ in DeviceInfo._fields_ if name != "reserved"}
+
+
+def synchronize():
+    check(lib().mg_sync())
+
+
+def _right_aligned(values, fill):
+    values = [int(v) for v in values]
+    if len(values) > MG_MAX_ND:
+        raise ValueError(f"rank {len(values)} exceeds {MG_MAX_ND}")
+    return _I64x3(*([fill] * (MG_MAX_ND - len(values)) + values))
+
+
+def dtype_code(dtype):
+    import numpy as np
+
+    dtype = np.dtype(dtype)
+    if dtype == np.float32:
+        return MG_F32
+    if dtype == np.float64:
+        return MG_F64
+    raise TypeError(f"the HIP kernels handle float32 and float64 only, got {dtype}")
+
+
+def conv_desc(dtype, x_shape, w_shape, grid, stride, padding, dilation):
+    """Descriptor for x:(N,C,X...) * w:(F,C,W...) -> (N,F,grid...)."""
+    m = len(x_shape) - 2
+    return ConvDesc(
+        dtype=dtype_code(dtype),
+        nd=m,
+        N=int(x_shape[0]),
+        C=int(x_shape[1]),
+        F=int(w_shape[0]),
+        X=_right_aligned(x_shape[2:], 1),
+        W=_right_aligned(w_shape[2:], 1),
+        G=_right_aligned(grid, 1),
+        stride=_right_aligned(stride, 1),
+        pad=_right_aligned(padding, 0),
+        dil=_right_aligned(dilation, 1),
+    )
+
+
+def pool_desc(dtype, lead, pooled_shape, pool, stride, grid, dx_dtype=None):
+    return PoolDesc(
+        dtype=dtype_code(dtype),
+        dx_dtype=dtype_code(dtype if dx_dtype is None else dx_dtype),
+        nd=len(pool),
+        reserved=0,
+        lead=int(lead),
+        X=_right_aligned(pooled_shape, 1),
+        P=_right_aligned(pool, 1),
+        S=_right_aligned(stride, 1),
+        G=_right_aligned(grid, 1),
+    )

@@ -1,0 +1,822 @@
+// conv_nd forward / data-gradient / filter-gradient as implicit GEMMs on the
+// gfx950 matrix cores (v_mfma_f32_16x16x4_f32, v_mfma_f64_16x16x4_f64).
+//
+// No im2col matrix is ever written to HBM.  A block gathers its operand tiles
+// straight from the NCHW tensors into LDS -- zero padding is a predicate on the
+// gathered coordinate -- and the 64-wide wavefronts feed the MFMA units from
+// LDS.  Three GEMM views (the closed-form sums are in the header):
+//
+//   forward   M = F, K = (c, tap),        N = (n, g)     gathers x
+//   dgrad     M = C, K = (f, tap),        N = (n, i)     gathers grad; a stride
+//             > 1 splits the input pixels i into prod(stride) phases, each a
+//             dense smaller convolution with its own slice of the (f, tap) table
+//   wgrad     M = F, N = (c, tap),        K = (n, g)     gathers grad and x; the
+//             long K is split over blocks, partial sums are added in a fixed
+//             order by a second kernel (no atomics, run-to-run identical)
+#include "conv_kernels.h"
+#include "internal.h"
+
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+namespace mg {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+
+// D(16x16) += A(16x4) * B(4x16) on one wavefront.  Lane l supplies A[l%16][l/16]
+// and B[l/16][l%16].  Lane l receives four elements of column l%16 of D; their
+// rows are row_of(l, r), r = 0..3, which differs between the two instructions.
+template <typename T>
+struct Mma;
+
+template <>
+struct Mma<float> {
+  using Acc = f32x4;
+  static __device__ __forceinline__ Acc run(float a, float b, Acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ int row_of(int lane, int r) { return 4 * (lane >> 4) + r; }
+};
+
+template <>
+struct Mma<double> {
+  using Acc = f64x4;
+  static __device__ __forceinline__ Acc run(double a, double b, Acc c) {
+    return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ int row_of(int lane, int r) { return 4 * r + (lane >> 4); }
+};
+
+// ------------------------------------------------------------------------------------------
+// filter packing: the GEMMs want the filter operand with M contiguous
+//   mode 0 (forward): Ap[(c*Wvol + t)][f] = w[f][c][t]
+//   mode 1 (dgrad)  : Ap[(f*Wvol + t)][c] = w[f][c][t]
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256) pack_filters_kernel(const T *__restrict__ w, T *__restrict__ ap, int F, int C,
+                                                           int wvol, int mode) {
+  const int total = F * C * wvol;
+  for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+    // idx enumerates the packed layout so that stores are coalesced
+    int m, f, c, t;
+    if (mode == 0) {
+      m = F;
+      f = idx % F;
+      const int row = idx / F;
+      t = row % wvol;
+      c = row / wvol;
+    } else {
+      m = C;
+      c = idx % C;
+      const int row = idx / C;
+      t = row % wvol;
+      f = row / wvol;
+    }
+    (void)m;
+    ap[idx] = w[((long long)f * C + c) * wvol + t];
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// gather-GEMM (forward and data gradient)
+// ------------------------------------------------------------------------------------------
+template <typename T, int BM, int BN, int BK, int WM, int WN>
+__global__ void __launch_bounds__(256) gather_gemm_kernel(const GemmParams p) {
+  static_assert((BM / WM) * (BN / WN) == 4, "four wavefronts per block");
+  static_assert(BK % 4 == 0 && WM % 16 == 0 && WN % 16 == 0, "MFMA 16x16x4 tiling");
+  constexpr int TM = WM / 16, TN = WN / 16;
+  constexpr int WAVES_N = BN / WN;
+  constexpr int AROWS = 256 / BM;  // table rows covered by one pass of the block over the A tile
+  constexpr int ALOADS = (BK + AROWS - 1) / AROWS;
+  constexpr int BROWS = 256 / BN;
+  constexpr int BLOADS = (BK + BROWS - 1) / BROWS;
+  constexpr int LDA = BM + 4, LDB = BN + 4;
+
+  __shared__ T As[2][BK][LDA];
+  __shared__ T Bs[2][BK][LDB];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm0 = (wave / WAVES_N) * WM;
+  const int wn0 = (wave % WAVES_N) * WN;
+
+  // which phase does this block belong to
+  int pi = 0;
+  while (pi + 1 < p.nphases && (int)blockIdx.x >= p.phases[pi + 1].blk_begin) ++pi;
+  const Phase ph = p.phases[pi];
+  const int pos0 = ((int)blockIdx.x - ph.blk_begin) * BN;
+  const int m0 = blockIdx.y * BM;
+  const int j12 = ph.J[1] * ph.J[2];
+  const int jvol = ph.J[0] * j12;
+
+  const T *__restrict__ A = static_cast<const T *>(p.A);
+  const TabEntry *__restrict__ tab = p.tab + ph.k_begin;
+  const int *__restrict__ arow = p.arow + ph.k_begin;
+
+  // ---- loader state: this thread's position in the B tile
+  const int bcol = tid % BN;
+  const int brow0 = tid / BN;
+  int qb0 = 0, qb1 = 0, qb2 = 0, lin = 0;
+  bool pos_ok = false;
+  const T *__restrict__ srcn = static_cast<const T *>(p.src);
+  {
+    const long long pos = (long long)pos0 + bcol;
+    if (pos < ph.npos) {
+      pos_ok = true;
+      const int n = (int)(pos / jvol);
+      int r = (int)(pos - (long long)n * jvol);
+      const int j0 = r / j12;
+      r -= j0 * j12;
+      const int j1 = r / ph.J[2];
+      const int j2 = r - j1 * ph.J[2];
+      qb0 = j0 * p.sj[0];
+      qb1 = j1 * p.sj[1];
+      qb2 = j2 * p.sj[2];
+      lin = qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2];
+      srcn += (long long)n * p.src_nstride;
+    }
+  }
+  const int acol = tid % BM;
+  const int arow0 = tid / BM;
+  const bool m_ok = (m0 + acol) < p.M;
+
+  T ra[ALOADS], rb[BLOADS];
+
+  auto fetch = [&](int kt) {
+    const int kbase = kt * BK;
+#pragma unroll
+    for (int r = 0; r < ALOADS; ++r) {
+      const int kk = arow0 + r * AROWS;
+      const int kidx = kbase + kk;
+      T v = T(0);
+      if (kk < BK && kidx < ph.k_count && m_ok) v = A[(long long)arow[kidx] * p.M + m0 + acol];
+      ra[r] = v;
+    }
+#pragma unroll
+    for (int r = 0; r < BLOADS; ++r) {
+      const int kk = brow0 + r * BROWS;
+      const int kidx = kbase + kk;
+      T v = T(0);
+      if (kk < BK && kidx < ph.k_count && pos_ok) {
+        const TabEntry e = tab[kidx];
+        const bool ok = (unsigned)(qb0 + e.d0) < (unsigned)p.Q[0] && (unsigned)(qb1 + e.d1) < (unsigned)p.Q[1] &&
+                        (unsigned)(qb2 + e.d2) < (unsigned)p.Q[2];
+        if (ok) v = srcn[lin + e.off];
+      }
+      rb[r] = v;
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int r = 0; r < ALOADS; ++r) {
+      const int kk = arow0 + r * AROWS;
+      if (kk < BK) As[buf][kk][acol] = ra[r];
+    }
+#pragma unroll
+    for (int r = 0; r < BLOADS; ++r) {
+      const int kk = brow0 + r * BROWS;
+      if (kk < BK) Bs[buf][kk][bcol] = rb[r];
+    }
+  };
+
+  typename Mma<T>::Acc acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = typename Mma<T>::Acc{0, 0, 0, 0};
+
+  const int ktiles = (ph.k_count + BK - 1) / BK;
+  int buf = 0;
+  if (ktiles > 0) {
+    fetch(0);
+    stash(0);
+  }
+  __syncthreads();
+  for (int kt = 0; kt < ktiles; ++kt) {
+    const bool more = kt + 1 < ktiles;
+    if (more) fetch(kt + 1);
+    const int l16 = lane & 15, lk = lane >> 4;
+#pragma unroll
+    for (int k4 = 0; k4 < BK / 4; ++k4) {
+      T a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) a[i] = As[buf][k4 * 4 + lk][wm0 + i * 16 + l16];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) b[j] = Bs[buf][k4 * 4 + lk][wn0 + j * 16 + l16];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::run(a[i], b[j], acc[i][j]);
+    }
+    if (more) stash(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+  }
+
+  // ---- epilogue: lane owns column (lane % 16) of every 16x16 tile
+  T *__restrict__ dst = static_cast<T *>(p.dst);
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const long long pos = (long long)pos0 + wn0 + j * 16 + (lane & 15);
+    if (pos >= ph.npos) continue;
+    const int n = (int)(pos / jvol);
+    int r = (int)(pos - (long long)n * jvol);
+    const int j0 = r / j12;
+    r -= j0 * j12;
+    const int j1 = r / ph.J[2];
+    const int j2 = r - j1 * ph.J[2];
+    T *out = dst + (long long)n * p.dst_nstride + (long long)(ph.o0[0] + j0 * p.oj[0]) * p.os[0] +
+             (long long)(ph.o0[1] + j1 * p.oj[1]) * p.os[1] + (long long)(ph.o0[2] + j2 * p.oj[2]) * p.os[2];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int m = m0 + wm0 + i * 16 + Mma<T>::row_of(lane, q);
+        if (m < p.M) out[(long long)m * p.dst_mstride] = acc[i][j][q];
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// filter gradient: split-K GEMM over positions, then a fixed-order reduction
+// ------------------------------------------------------------------------------------------
+template <typename T, int BM, int BN, int BK, int WM, int WN>
+__global__ void __launch_bounds__(256) wgrad_kernel(const WgradParams p) {
+  static_assert((BM / WM) * (BN / WN) == 4, "four wavefronts per block");
+  static_assert(256 % BK == 0 && BK % 4 == 0, "K tile");
+  constexpr int TM = WM / 16, TN = WN / 16;
+  constexpr int WAVES_N = BN / WN;
+  constexpr int ROWS = 256 / BK;  // tile rows covered by one pass of the block
+  constexpr int ALOADS = (BM + ROWS - 1) / ROWS;
+  constexpr int BLOADS = (BN + ROWS - 1) / ROWS;
+  constexpr int LDK = BK + 2;
+
+  __shared__ T As[2][BM][LDK];  // grad tile   [f][position]
+  __shared__ T Bs[2][BN][LDK];  // window tile [column][position]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm0 = (wave / WAVES_N) * WM;
+  const int wn0 = (wave % WAVES_N) * WN;
+  const int n0 = blockIdx.x * BN;  // first column (c, tap)
+  const int m0 = blockIdx.y * BM;  // first filter
+  const long long kbeg = (long long)blockIdx.z * p.kchunk;
+  const long long kend = min(kbeg + p.kchunk, p.kpos);
+
+  const T *__restrict__ grad = static_cast<const T *>(p.grad);
+  const T *__restrict__ x = static_cast<const T *>(p.x);
+  const int kcol = tid % BK;  // this thread's position inside the K tile
+  const int row0 = tid / BK;
+  const int g12 = p.G[1] * p.G[2];
+
+  T ra[ALOADS], rb[BLOADS];
+
+  auto fetch = [&](int kt) {
+    const long long pos = kbeg + (long long)kt * BK + kcol;
+    const bool pos_ok = pos < kend;
+    int n = 0, gflat = 0, qb0 = 0, qb1 = 0, qb2 = 0, lin = 0;
+    if (pos_ok) {
+      n = (int)(pos / p.gvol);
+      gflat = (int)(pos - (long long)n * p.gvol);
+      const int g0 = gflat / g12;
+      const int r = gflat - g0 * g12;
+      const int g1 = r / p.G[2];
+      const int g2 = r - g1 * p.G[2];
+      qb0 = g0 * p.sj[0];
+      qb1 = g1 * p.sj[1];
+      qb2 = g2 * p.sj[2];
+      lin = qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2];
+    }
+    const T *gn = grad + (long long)n * p.g_nstride + gflat;
+    const T *xn = x + (long long)n * p.x_nstride;
+#pragma unroll
+    for (int r = 0; r < ALOADS; ++r) {
+      const int row = row0 + r * ROWS;
+      T v = T(0);
+      if (row < BM && pos_ok && m0 + row < p.F) v = gn[(long long)(m0 + row) * p.gvol];
+      ra[r] = v;
+    }
+#pragma unroll
+    for (int r = 0; r < BLOADS; ++r) {
+      const int row = row0 + r * ROWS;
+      T v = T(0);
+      if (row < BN && pos_ok && n0 + row < p.CT) {
+        const TabEntry e = p.tab[n0 + row];
+        const bool ok = (unsigned)(qb0 + e.d0) < (unsigned)p.Q[0] && (unsigned)(qb1 + e.d1) < (unsigned)p.Q[1] &&
+                        (unsigned)(qb2 + e.d2) < (unsigned)p.Q[2];
+        if (ok) v = xn[lin + e.off];
+      }
+      rb[r] = v;
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int r = 0; r < ALOADS; ++r) {
+      const int row = row0 + r * ROWS;
+      if (row < BM) As[buf][row][kcol] = ra[r];
+    }
+#pragma unroll
+    for (int r = 0; r < BLOADS; ++r) {
+      const int row = row0 + r * ROWS;
+      if (row < BN) Bs[buf][row][kcol] = rb[r];
+    }
+  };
+
+  typename Mma<T>::Acc acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = typename Mma<T>::Acc{0, 0, 0, 0};
+
+  const int ktiles = kend > kbeg ? (int)((kend - kbeg + BK - 1) / BK) : 0;
+  int buf = 0;
+  if (ktiles > 0) {
+    fetch(0);
+    stash(0);
+  }
+  __syncthreads();
+  for (int kt = 0; kt < ktiles; ++kt) {
+    const bool more = kt + 1 < ktiles;
+    if (more) fetch(kt + 1);
+    const int l16 = lane & 15, lk = lane >> 4;
+#pragma unroll
+    for (int k4 = 0; k4 < BK / 4; ++k4) {
+      T a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) a[i] = As[buf][wm0 + i * 16 + l16][k4 * 4 + lk];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) b[j] = Bs[buf][wn0 + j * 16 + l16][k4 * 4 + lk];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::run(a[i], b[j], acc[i][j]);
+    }
+    if (more) stash(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+  }
+
+  T *__restrict__ out = static_cast<T *>(p.out) + (long long)blockIdx.z * p.F * p.CT;
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int col = n0 + wn0 + j * 16 + (lane & 15);
+    if (col >= p.CT) continue;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int f = m0 + wm0 + i * 16 + Mma<T>::row_of(lane, q);
+        if (f < p.F) out[(long long)f * p.CT + col] = acc[i][j][q];
+      }
+  }
+}
+
+// dw[i] = ((part[0][i] + part[1][i]) + part[2][i]) + ...   (fixed order)
+template <typename T>
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const T *__restrict__ part, T *__restrict__ dw, int count,
+                                                            int splits) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= count) return;
+  T s = part[i];
+  for (int k = 1; k < splits; ++k) s += part[(long long)k * count + i];
+  dw[i] = s;
+}
+
+// ------------------------------------------------------------------------------------------
+// host side: descriptor checks, cached plans (tables live in device memory), launches
+// ------------------------------------------------------------------------------------------
+namespace {
+
+enum ConvOp { OP_FWD = 0, OP_DGRAD = 1, OP_WGRAD = 2 };
+
+struct Geometry {
+  int nd, dtype;
+  int N, C, F;
+  int X[3], W[3], G[3], S[3], P[3], D[3];
+  long long xvol, wvol, gvol;
+};
+
+struct Plan {
+  void *blob = nullptr;  // one device allocation: [TabEntry table][arow][phases]
+  TabEntry *tab = nullptr;
+  int *arow = nullptr;
+  Phase *phases = nullptr;
+  int nphases = 0;
+  int pos_blocks = 0;  // grid.x for the gather-GEMM
+  int bm = 0, bn = 0;
+  // wgrad
+  int splits = 1;
+  long long kchunk = 0;
+};
+
+std::map<std::string, Plan> &plans() {
+  static std::map<std::string, Plan> m;
+  return m;
+}
+
+int check_desc(const mg_conv_desc *d, Geometry *g) {
+  if (!d) return fail(MG_ERR_BAD_ARG, "conv descriptor is null");
+  if (d->dtype != MG_F32 && d->dtype != MG_F64)
+    return fail(MG_ERR_UNSUPPORTED, "conv dtype %d (only float32=0 / float64=1)", d->dtype);
+  if (d->nd < 1 || d->nd > MG_MAX_ND) return fail(MG_ERR_UNSUPPORTED, "spatial rank %d (1..%d)", d->nd, MG_MAX_ND);
+  if (d->N < 1 || d->C < 1 || d->F < 1)
+    return fail(MG_ERR_BAD_ARG, "N=%lld C=%lld F=%lld must be positive", (long long)d->N, (long long)d->C,
+                (long long)d->F);
+  const long long lim = (1ll << 31) - 1;
+  long long xvol = 1, wvol = 1, gvol = 1;
+  for (int k = 0; k < 3; ++k) {
+    if (d->X[k] < 1 || d->W[k] < 1 || d->G[k] < 1 || d->stride[k] < 1 || d->dil[k] < 1 || d->pad[k] < 0)
+      return fail(MG_ERR_BAD_ARG, "axis %d: X=%lld W=%lld G=%lld stride=%lld dil=%lld pad=%lld", k, (long long)d->X[k],
+                  (long long)d->W[k], (long long)d->G[k], (long long)d->stride[k], (long long)d->dil[k],
+                  (long long)d->pad[k]);
+    if (k < 3 - d->nd &&
+        (d->X[k] != 1 || d->W[k] != 1 || d->G[k] != 1 || d->stride[k] != 1 || d->dil[k] != 1 || d->pad[k] != 0))
+      return fail(MG_ERR_BAD_ARG, "axis %d lies outside rank %d and must be trivial", k, d->nd);
+    if (d->X[k] > lim || d->W[k] > lim || d->stride[k] > lim || d->dil[k] > lim || d->pad[k] > lim)
+      return fail(MG_ERR_UNSUPPORTED, "axis %d: extent beyond 2^31", k);
+    const long long span = (d->W[k] - 1) * d->dil[k] + 1;
+    const long long room = d->X[k] + 2 * d->pad[k] - span;
+    if (room < 0 || d->G[k] > room / d->stride[k] + 1)
+      return fail(MG_ERR_BAD_ARG, "axis %d: G=%lld exceeds (X+2*pad-span)/stride+1", k, (long long)d->G[k]);
+    xvol *= d->X[k];
+    wvol *= d->W[k];
+    gvol *= d->G[k];
+    if (xvol > lim || wvol > lim || gvol > lim) return fail(MG_ERR_UNSUPPORTED, "per-sample volume beyond 2^31");
+    g->X[k] = (int)d->X[k];
+    g->W[k] = (int)d->W[k];
+    g->G[k] = (int)d->G[k];
+    g->S[k] = (int)d->stride[k];
+    g->P[k] = (int)d->pad[k];
+    g->D[k] = (int)d->dil[k];
+  }
+  // Offsets inside one batch item and position counts are 32-bit in the kernels.
+  if (d->N > lim || d->C > lim || d->F > lim || d->C * xvol > lim || d->F * gvol > lim || d->N * gvol > lim ||
+      d->N * xvol > lim || d->F * d->C * wvol > lim)
+    return fail(MG_ERR_UNSUPPORTED, "tensor too large for 32-bit in-sample offsets");
+  g->nd = d->nd;
+  g->dtype = d->dtype;
+  g->N = (int)d->N;
+  g->C = (int)d->C;
+  g->F = (int)d->F;
+  g->xvol = xvol;
+  g->wvol = wvol;
+  g->gvol = gvol;
+  return MG_OK;
+}
+
+// Largest row tile whose round-up waste stays small.
+int pick_bm(int M) {
+  const int cands[4] = {128, 64, 32, 16};
+  for (int c : cands) {
+    const int padded = (int)ceil_div(M, c) * c;
+    if (padded - M <= M / 8) return c;
+  }
+  return 16;
+}
+
+void fwd_table(const Geometry &g, std::vector<TabEntry> &tab) {
+  // row (c, t0, t1, t2) in the filter's own row-major order
+  const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
+  tab.clear();
+  tab.reserve((size_t)g.C * g.wvol);
+  for (int c = 0; c < g.C; ++c)
+    for (int t0 = 0; t0 < g.W[0]; ++t0)
+      for (int t1 = 0; t1 < g.W[1]; ++t1)
+        for (int t2 = 0; t2 < g.W[2]; ++t2) {
+          TabEntry e;
+          e.d0 = t0 * g.D[0] - g.P[0];
+          e.d1 = t1 * g.D[1] - g.P[1];
+          e.d2 = t2 * g.D[2] - g.P[2];
+          e.off = (int)(c * g.xvol) + e.d0 * qs[0] + e.d1 * qs[1] + e.d2 * qs[2];
+          tab.push_back(e);
+        }
+}
+
+int upload_plan(Plan &pl, const std::vector<TabEntry> &tab, const std::vector<int> &arow,
+                const std::vector<Phase> &phases) {
+  const size_t tab_b = (tab.size() * sizeof(TabEntry) + 255) & ~size_t(255);
+  const size_t arow_b = (arow.size() * sizeof(int) + 255) & ~size_t(255);
+  const size_t ph_b = (phases.size() * sizeof(Phase) + 255) & ~size_t(255);
+  std::vector<char> host(tab_b + arow_b + ph_b + 256, 0);
+  if (!tab.empty()) memcpy(host.data(), tab.data(), tab.size() * sizeof(TabEntry));
+  if (!arow.empty()) memcpy(host.data() + tab_b, arow.data(), arow.size() * sizeof(int));
+  if (!phases.empty()) memcpy(host.data() + tab_b + arow_b, phases.data(), phases.size() * sizeof(Phase));
+  MG_HIP(hipMalloc(&pl.blob, host.size()));
+  hipError_t err = hipMemcpy(pl.blob, host.data(), host.size(), hipMemcpyHostToDevice);
+  if (err != hipSuccess) {
+    (void)hipFree(pl.blob);
+    pl.blob = nullptr;
+    return hip_fail(err, "hipMemcpy(plan tables)", __FILE__, __LINE__);
+  }
+  char *base = static_cast<char *>(pl.blob);
+  pl.tab = reinterpret_cast<TabEntry *>(base);
+  pl.arow = reinterpret_cast<int *>(base + tab_b);
+  pl.phases = reinterpret_cast<Phase *>(base + tab_b + arow_b);
+  pl.nphases = (int)phases.size();
+  return MG_OK;
+}
+
+int build_fwd_plan(const Geometry &g, Plan &pl) {
+  std::vector<TabEntry> tab;
+  fwd_table(g, tab);
+  std::vector<int> arow(tab.size());
+  for (size_t i = 0; i < arow.size(); ++i) arow[i] = (int)i;
+  pl.bm = pick_bm(g.F);
+  pl.bn = pl.bm == 128 ? 128 : 256;
+  Phase ph{};
+  for (int k = 0; k < 3; ++k) {
+    ph.J[k] = g.G[k];
+    ph.o0[k] = 0;
+  }
+  ph.k_begin = 0;
+  ph.k_count = (int)tab.size();
+  ph.blk_begin = 0;
+  ph.npos = (long long)g.N * g.gvol;
+  pl.pos_blocks = (int)ceil_div(ph.npos, pl.bn);
+  return upload_plan(pl, tab, arow, std::vector<Phase>{ph});
+}
+
+int build_dgrad_plan(const Geometry &g, Plan &pl) {
+  pl.bm = pick_bm(g.C);
+  pl.bn = pl.bm == 128 ? 128 : 256;
+  std::vector<TabEntry> tab;
+  std::vector<int> arow;
+  std::vector<Phase> phases;
+  const int gs[3] = {g.G[1] * g.G[2], g.G[2], 1};
+  int blk = 0;
+  long long nphase = (long long)g.S[0] * g.S[1] * g.S[2];
+  if (nphase > 4096) return fail(MG_ERR_UNSUPPORTED, "prod(stride) = %lld phases (limit 4096)", nphase);
+  for (int r0 = 0; r0 < g.S[0]; ++r0)
+    for (int r1 = 0; r1 < g.S[1]; ++r1)
+      for (int r2 = 0; r2 < g.S[2]; ++r2) {
+        const int rho[3] = {r0, r1, r2};
+        Phase ph{};
+        bool empty = false;
+        std::vector<int> taps[3], offs[3];
+        for (int k = 0; k < 3; ++k) {
+          // input pixels i with (i + pad) % stride == rho
+          const int i0 = ((rho[k] - g.P[k]) % g.S[k] + g.S[k]) % g.S[k];
+          ph.o0[k] = i0;
+          ph.J[k] = i0 < g.X[k] ? (g.X[k] - i0 + g.S[k] - 1) / g.S[k] : 0;
+          if (ph.J[k] == 0) empty = true;
+          // taps that can reach them: t*dil % stride == rho; the window index is then
+          // g = j + (i0 + pad - t*dil) / stride  (exact division)
+          for (int t = 0; t < g.W[k]; ++t)
+            if ((t * g.D[k]) % g.S[k] == rho[k]) {
+              taps[k].push_back(t);
+              offs[k].push_back((i0 + g.P[k] - t * g.D[k]) / g.S[k]);
+            }
+        }
+        if (empty) continue;
+        ph.k_begin = (int)tab.size();
+        for (int f = 0; f < g.F; ++f)
+          for (size_t a = 0; a < taps[0].size(); ++a)
+            for (size_t b = 0; b < taps[1].size(); ++b)
+              for (size_t c = 0; c < taps[2].size(); ++c) {
+                TabEntry e;
+                e.d0 = offs[0][a];
+                e.d1 = offs[1][b];
+                e.d2 = offs[2][c];
+                e.off = (int)(f * g.gvol) + e.d0 * gs[0] + e.d1 * gs[1] + e.d2 * gs[2];
+                tab.push_back(e);
+                arow.push_back((int)(f * g.wvol) + (taps[0][a] * g.W[1] + taps[1][b]) * g.W[2] + taps[2][c]);
+              }
+        ph.k_count = (int)tab.size() - ph.k_begin;
+        ph.npos = (long long)g.N * ph.J[0] * ph.J[1] * ph.J[2];
+        ph.blk_begin = blk;
+        blk += (int)ceil_div(ph.npos, pl.bn);
+        phases.push_back(ph);
+      }
+  pl.pos_blocks = blk;
+  return upload_plan(pl, tab, arow, phases);
+}
+
+int build_wgrad_plan(const Geometry &g, Plan &pl) {
+  std::vector<TabEntry> tab;
+  fwd_table(g, tab);
+  pl.bm = g.F <= 16 ? 16 : (g.F <= 32 ? 32 : 64);
+  pl.bn = 64;
+  const int bk = g.dtype == MG_F64 ? 32 : 64;
+  const long long ct = (long long)g.C * g.wvol;
+  const long long tiles = ceil_div(g.F, pl.bm) * ceil_div(ct, pl.bn);
+  const long long kpos = (long long)g.N * g.gvol;
+  const long long ktiles = ceil_div(kpos, bk);
+  // aim at about three blocks per compute unit, at least 8 K tiles per block
+  const long long want_blocks = 3ll * runtime().props.multiProcessorCount;
+  long long splits = ceil_div(want_blocks, tiles);
+  const long long max_splits = ktiles >= 8 ? ktiles / 8 : 1;
+  if (splits > max_splits) splits = max_splits;
+  if (splits < 1) splits = 1;
+  if (splits > 1024) splits = 1024;
+  const long long tiles_per_split = ceil_div(ktiles, splits);
+  pl.kchunk = tiles_per_split * bk;
+  pl.splits = (int)ceil_div(kpos, pl.kchunk);
+  return upload_plan(pl, tab, std::vector<int>(), std::vector<Phase>());
+}
+
+int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
+  std::string key(reinterpret_cast<const char *>(d), sizeof *d);
+  key.push_back((char)op);
+  auto it = plans().find(key);
+  if (it == plans().end()) {
+    if (plans().size() >= 256) release_conv_plans();  // crude bound on cached tables
+    Plan pl;
+    int rc = op == OP_FWD ? build_fwd_plan(g, pl) : op == OP_DGRAD ? build_dgrad_plan(g, pl) : build_wgrad_plan(g, pl);
+    if (rc) return rc;
+    it = plans().emplace(key, pl).first;
+  }
+  *out = &it->second;
+  return MG_OK;
+}
+
+template <typename T, int BM, int BN, int BK, int WM, int WN>
+void launch_gemm(const GemmParams &gp, int pos_blocks, hipStream_t s) {
+  const dim3 grid((unsigned)pos_blocks, (unsigned)ceil_div(gp.M, BM));
+  hipLaunchKernelGGL((gather_gemm_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, gp);
+}
+
+template <typename T>
+int run_gemm(const GemmParams &gp, const Plan &pl, hipStream_t s) {
+  constexpr int BK = sizeof(T) == 8 ? 8 : 16;
+  if (pl.pos_blocks <= 0) return MG_OK;
+  switch (pl.bm) {
+    case 128: launch_gemm<T, 128, 128, BK, 64, 64>(gp, pl.pos_blocks, s); break;
+    case 64: launch_gemm<T, 64, 256, BK, 64, 64>(gp, pl.pos_blocks, s); break;
+    case 32: launch_gemm<T, 32, 256, BK, 32, 64>(gp, pl.pos_blocks, s); break;
+    default: launch_gemm<T, 16, 256, BK, 16, 64>(gp, pl.pos_blocks, s); break;
+  }
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
+template <typename T>
+int pack_filters(const Geometry &g, const void *w, int mode, void **packed) {
+  const size_t count = (size_t)g.F * g.C * g.wvol;
+  if (int rc = workspace(count * sizeof(T), packed)) return rc;
+  const unsigned blocks = (unsigned)std::min<long long>(ceil_div((long long)count, 256), 4096);
+  hipLaunchKernelGGL(pack_filters_kernel<T>, dim3(blocks), dim3(256), 0, runtime().stream, static_cast<const T *>(w),
+                     static_cast<T *>(*packed), g.F, g.C, (int)g.wvol, mode);
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
+template <typename T>
+int conv_fwd_impl(const Geometry &g, const Plan &pl, const void *x, const void *w, void *out) {
+  void *packed = nullptr;
+  if (int rc = pack_filters<T>(g, w, 0, &packed)) return rc;
+  GemmParams gp{};
+  gp.A = packed;
+  gp.src = x;
+  gp.dst = out;
+  gp.tab = pl.tab;
+  gp.arow = pl.arow;
+  gp.phases = pl.phases;
+  gp.nphases = pl.nphases;
+  gp.M = g.F;
+  const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
+  const int os[3] = {g.G[1] * g.G[2], g.G[2], 1};
+  for (int k = 0; k < 3; ++k) {
+    gp.Q[k] = g.X[k];
+    gp.sj[k] = g.S[k];
+    gp.qs[k] = qs[k];
+    gp.oj[k] = 1;
+    gp.os[k] = os[k];
+  }
+  gp.dst_mstride = (int)g.gvol;
+  gp.src_nstride = (long long)g.C * g.xvol;
+  gp.dst_nstride = (long long)g.F * g.gvol;
+  return run_gemm<T>(gp, pl, runtime().stream);
+}
+
+template <typename T>
+int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const void *w, void *dx) {
+  void *packed = nullptr;
+  if (int rc = pack_filters<T>(g, w, 1, &packed)) return rc;
+  GemmParams gp{};
+  gp.A = packed;
+  gp.src = grad;
+  gp.dst = dx;
+  gp.tab = pl.tab;
+  gp.arow = pl.arow;
+  gp.phases = pl.phases;
+  gp.nphases = pl.nphases;
+  gp.M = g.C;
+  const int qs[3] = {g.G[1] * g.G[2], g.G[2], 1};
+  const int os[3] = {g.X[1] * g.X[2], g.X[2], 1};
+  for (int k = 0; k < 3; ++k) {
+    gp.Q[k] = g.G[k];
+    gp.sj[k] = 1;
+    gp.qs[k] = qs[k];
+    gp.oj[k] = g.S[k];
+    gp.os[k] = os[k];
+  }
+  gp.dst_mstride = (int)g.xvol;
+  gp.src_nstride = (long long)g.F * g.gvol;
+  gp.dst_nstride = (long long)g.C * g.xvol;
+  return run_gemm<T>(gp, pl, runtime().stream);
+}
+
+template <typename T, int BM, int BN, int BK, int WM, int WN>
+void launch_wgrad(const WgradParams &wp, hipStream_t s) {
+  const dim3 grid((unsigned)ceil_div(wp.CT, BN), (unsigned)ceil_div(wp.F, BM), (unsigned)wp.splits);
+  hipLaunchKernelGGL((wgrad_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, wp);
+}
+
+template <typename T>
+int conv_wgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const void *x, void *dw) {
+  constexpr int BK = sizeof(T) == 8 ? 32 : 64;
+  hipStream_t s = runtime().stream;
+  const int ct = (int)(g.C * g.wvol);
+  void *target = dw;
+  if (pl.splits > 1)
+    if (int rc = workspace((size_t)pl.splits * g.F * ct * sizeof(T), &target)) return rc;
+  WgradParams wp{};
+  wp.grad = grad;
+  wp.x = x;
+  wp.out = target;
+  wp.tab = pl.tab;
+  wp.F = g.F;
+  wp.CT = ct;
+  const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
+  for (int k = 0; k < 3; ++k) {
+    wp.G[k] = g.G[k];
+    wp.Q[k] = g.X[k];
+    wp.sj[k] = g.S[k];
+    wp.qs[k] = qs[k];
+  }
+  wp.gvol = (int)g.gvol;
+  wp.x_nstride = (long long)g.C * g.xvol;
+  wp.g_nstride = (long long)g.F * g.gvol;
+  wp.kpos = (long long)g.N * g.gvol;
+  wp.kchunk = pl.kchunk;
+  wp.splits = pl.splits;
+  switch (pl.bm) {
+    case 64: launch_wgrad<T, 64, 64, BK, 32, 32>(wp, s); break;
+    case 32: launch_wgrad<T, 32, 64, BK, 32, 16>(wp, s); break;
+    default: launch_wgrad<T, 16, 64, BK, 16, 16>(wp, s); break;
+  }
+  MG_HIP(hipGetLastError());
+  if (pl.splits > 1) {
+    const int count = g.F * ct;
+    hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, s,
+                       static_cast<const T *>(target), static_cast<T *>(dw), count, pl.splits);
+    MG_HIP(hipGetLastError());
+  }
+  return MG_OK;
+}
+
+}  // namespace
+
+void release_conv_plans() {
+  for (auto &kv : plans())
+    if (kv.second.blob) (void)hipFree(kv.second.blob);
+  plans().clear();
+}
+
+}  // namespace mg
+
+using namespace mg;
+
+extern "C" {
+
+int mg_conv_fwd(const mg_conv_desc *desc, const void *x, const void *w, void *out) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  Geometry g;
+  if (int rc = check_desc(desc, &g)) return rc;
+  if (!x || !w || !out) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_conv_fwd");
+  Plan *pl = nullptr;
+  if (int rc = get_plan(OP_FWD, desc, g, &pl)) return rc;
+  return g.dtype == MG_F32 ? conv_fwd_impl<float>(g, *pl, x, w, out) : conv_fwd_impl<double>(g, *pl, x, w, out);
+}
+
+int mg_conv_dgrad(const mg_conv_desc *desc, const void *grad, const void *w, void *dx) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  Geometry g;
+  if (int rc = check_desc(desc, &g)) return rc;
+  if (!grad || !w || !dx) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_conv_dgrad");
+  Plan *pl = nullptr;
+  if (int rc = get_plan(OP_DGRAD, desc, g, &pl)) return rc;
+  return g.dtype == MG_F32 ? conv_dgrad_impl<float>(g, *pl, grad, w, dx)
+                           : conv_dgrad_impl<double>(g, *pl, grad, w, dx);
+}
+
+int mg_conv_wgrad(const mg_conv_desc *desc, const void *grad, const void *x, void *dw) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  Geometry g;
+  if (int rc = check_desc(desc, &g)) return rc;
+  if (!grad || !x || !dw) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_conv_wgrad");
+  Plan *pl = nullptr;
+  if (int rc = get_plan(OP_WGRAD, desc, g, &pl)) return rc;
+  return g.dtype == MG_F32 ? conv_wgrad_impl<float>(g, *pl, grad, x, dw)
+                           : conv_wgrad_impl<double>(g, *pl, grad, x, dw);
+}
+
+}  // extern "C"

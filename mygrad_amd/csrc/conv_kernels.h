@@ -1,0 +1,67 @@
+// Device-side parameter blocks shared by the convolution plan builder (host)
+// and the implicit-GEMM kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+namespace mg {
+
+// One row of the contraction table.  For the forward pass a row is one (c, tap);
+// for the data gradient one (f, tap) of a stride phase.  `off` is the element
+// offset that the row adds to a position's base offset inside one batch item of
+// the gathered tensor; d[k] is what it adds to the position's coordinate on axis
+// k, which must land in [0, Q[k]) for the element to exist (otherwise it is a
+// padding zero).
+struct TabEntry {
+  int off;
+  int d0, d1, d2;
+};
+
+// A stride phase of the data gradient (the forward pass has exactly one phase).
+// Positions of a phase are (n, j0, j1, j2), j_k in [0, J[k]); position j maps to
+// the destination coordinate o0[k] + j_k * oj[k].
+struct Phase {
+  int J[3];
+  int o0[3];
+  int k_begin, k_count;  // rows [k_begin, k_begin + k_count) of the table
+  int blk_begin;         // first block (along positions) that works on this phase
+  int pad_;
+  long long npos;        // N * J0 * J1 * J2
+};
+
+// Gather-GEMM:  dst[n, m, pos] = sum_k A[arow[k]][m] * src[n, row k, pos]
+struct GemmParams {
+  const void *A;  // packed filters, [rows][M] with M contiguous
+  const void *src;
+  void *dst;
+  const TabEntry *tab;
+  const int *arow;  // table row -> row of A
+  const Phase *phases;
+  int nphases;
+  int M;
+  int Q[3];   // extents of the gathered tensor's spatial axes
+  int sj[3];  // source coordinate advance per position step
+  int qs[3];  // source element strides of the spatial axes
+  int oj[3];  // destination coordinate advance per position step
+  int os[3];  // destination element strides of the spatial axes
+  int dst_mstride;
+  long long src_nstride, dst_nstride;
+};
+
+// Filter gradient:  out[split][f][col] = sum over the split's positions (n, g) of
+//   grad[n, f, g] * x[n, column col at g]
+struct WgradParams {
+  const void *grad;
+  const void *x;
+  void *out;            // dw itself when splits == 1, else the partial-sum workspace
+  const TabEntry *tab;  // one row per column (c, tap): the forward table
+  int F, CT;            // rows and columns of dw viewed as a matrix
+  int G[3], Q[3], sj[3], qs[3];
+  int gvol;
+  long long x_nstride, g_nstride;
+  long long kpos;    // N * gvol, the length of the sum
+  long long kchunk;  // positions per split (multiple of the K tile)
+  int splits;
+};
+
+}  // namespace mg

@@ -1,0 +1,59 @@
+// Internal declarations shared by the translation units of libmygrad_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <mutex>
+
+#include "mygrad_hip.h"
+
+namespace mg {
+
+// One global lock: the library is single-stream and not re-entrant.
+std::recursive_mutex &api_mutex();
+
+// Records the message that mg_last_error() returns and passes `code` through.
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+// Maps a hipError_t to an mg_status, recording file:line and the HIP message.
+int hip_fail(hipError_t err, const char *what, const char *file, int line);
+
+struct Runtime {
+  bool ready = false;
+  int device = -1;
+  hipStream_t stream = nullptr;
+  hipDeviceProp_t props{};
+  // Grow-only device scratch used by the convolution entry points (packed
+  // filters, split-K partial sums).  Never handed to callers.
+  void *workspace = nullptr;
+  size_t workspace_bytes = 0;
+};
+
+Runtime &runtime();
+
+// Returns a device scratch area of at least `nbytes` (256-byte aligned), growing
+// the allocation when needed.  Stream-ordered users may rely on its contents only
+// until the next call that asks for workspace.
+int workspace(size_t nbytes, void **ptr);
+
+// Drops every cached convolution plan (device tables); called by mg_shutdown.
+void release_conv_plans();
+
+#define MG_HIP(expr)                                                   \
+  do {                                                                 \
+    hipError_t mg_err_ = (expr);                                       \
+    if (mg_err_ != hipSuccess) return ::mg::hip_fail(mg_err_, #expr, __FILE__, __LINE__); \
+  } while (0)
+
+#define MG_REQUIRE_INIT()                                              \
+  do {                                                                 \
+    if (!::mg::runtime().ready)                                        \
+      return ::mg::fail(MG_ERR_NOT_INIT, "mg_init() has not been called (or failed)"); \
+  } while (0)
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+}  // namespace mg

@@ -1,0 +1,269 @@
+// Device selection, the library stream, buffers, copies, events and scratch.
+#include "internal.h"
+
+#include <cstring>
+
+namespace mg {
+
+std::recursive_mutex &api_mutex() {
+  static std::recursive_mutex m;
+  return m;
+}
+
+static thread_local char g_error[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof g_error, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_fail(hipError_t err, const char *what, const char *file, int line) {
+  const char *base = strrchr(file, '/');
+  int code = (err == hipErrorOutOfMemory || err == hipErrorMemoryAllocation) ? MG_ERR_OOM
+             : (err == hipErrorNoDevice || err == hipErrorInvalidDevice)     ? MG_ERR_NO_DEVICE
+                                                                             : MG_ERR_HIP;
+  (void)hipGetLastError();  // clear the sticky error so that later calls start clean
+  return fail(code, "%s:%d: %s -> %s (%s)", base ? base + 1 : file, line, what, hipGetErrorName(err),
+              hipGetErrorString(err));
+}
+
+Runtime &runtime() {
+  static Runtime r;
+  return r;
+}
+
+int workspace(size_t nbytes, void **ptr) {
+  Runtime &rt = runtime();
+  if (nbytes > rt.workspace_bytes) {
+    // Work already enqueued may still be reading the old block.
+    MG_HIP(hipStreamSynchronize(rt.stream));
+    if (rt.workspace) MG_HIP(hipFree(rt.workspace));
+    rt.workspace = nullptr;
+    rt.workspace_bytes = 0;
+    size_t want = (nbytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+    MG_HIP(hipMalloc(&rt.workspace, want));
+    rt.workspace_bytes = want;
+  }
+  *ptr = rt.workspace;
+  return MG_OK;
+}
+
+__global__ void fill_zero_kernel(uint32_t *p, size_t nwords) {
+  size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = size_t(gridDim.x) * blockDim.x;
+  for (; i < nwords; i += step) p[i] = 0u;
+}
+
+__global__ void fill_zero_bytes_kernel(uint8_t *p, size_t n) {
+  size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+}  // namespace mg
+
+using namespace mg;
+
+#define MG_LOCK() std::lock_guard<std::recursive_mutex> mg_guard_(::mg::api_mutex())
+
+extern "C" {
+
+const char *mg_last_error(void) { return g_error; }
+
+int mg_init(int device) {
+  MG_LOCK();
+  Runtime &rt = runtime();
+  if (rt.ready) {
+    if (device >= 0 && device != rt.device)
+      return fail(MG_ERR_BAD_ARG, "already initialised on device %d, asked for %d", rt.device, device);
+    return MG_OK;
+  }
+  int count = 0;
+  hipError_t err = hipGetDeviceCount(&count);
+  if (err != hipSuccess || count <= 0) {
+    (void)hipGetLastError();
+    return fail(MG_ERR_NO_DEVICE, "no HIP device visible (%s)", err == hipSuccess ? "count == 0" : hipGetErrorName(err));
+  }
+  if (device < 0) device = 0;
+  if (device >= count) return fail(MG_ERR_NO_DEVICE, "device %d requested but only %d visible", device, count);
+  MG_HIP(hipSetDevice(device));
+  MG_HIP(hipGetDeviceProperties(&rt.props, device));
+  if (strncmp(rt.props.gcnArchName, "gfx950", 6) != 0)
+    return fail(MG_ERR_NO_DEVICE, "device %d is %s; this library carries gfx950 code only", device,
+                rt.props.gcnArchName);
+  MG_HIP(hipStreamCreateWithFlags(&rt.stream, hipStreamNonBlocking));
+  rt.device = device;
+  rt.ready = true;
+  return MG_OK;
+}
+
+int mg_shutdown(void) {
+  MG_LOCK();
+  Runtime &rt = runtime();
+  if (!rt.ready) return MG_OK;
+  MG_HIP(hipStreamSynchronize(rt.stream));
+  release_conv_plans();
+  if (rt.workspace) MG_HIP(hipFree(rt.workspace));
+  rt.workspace = nullptr;
+  rt.workspace_bytes = 0;
+  MG_HIP(hipStreamDestroy(rt.stream));
+  rt.stream = nullptr;
+  rt.ready = false;
+  rt.device = -1;
+  return MG_OK;
+}
+
+int mg_device_info(mg_device_info_t *info) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  if (!info) return fail(MG_ERR_BAD_ARG, "info is null");
+  const hipDeviceProp_t &p = runtime().props;
+  memset(info, 0, sizeof *info);
+  strncpy(info->name, p.gcnArchName, sizeof info->name - 1);
+  info->compute_units = p.multiProcessorCount;
+  info->clock_khz = p.clockRate;
+  info->wavefront = p.warpSize;
+  info->lds_bytes_per_block = (int32_t)p.sharedMemPerBlock;
+  info->hbm_bytes = (int64_t)p.totalGlobalMem;
+  info->l2_bytes = p.l2CacheSize;
+  info->memory_clock_khz = p.memoryClockRate;
+  info->memory_bus_bits = p.memoryBusWidth;
+  return MG_OK;
+}
+
+int mg_malloc(void **dptr, size_t nbytes) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  if (!dptr) return fail(MG_ERR_BAD_ARG, "dptr is null");
+  *dptr = nullptr;
+  if (nbytes == 0) nbytes = 256;  // keep a distinct, valid pointer for empty tensors
+  MG_HIP(hipMalloc(dptr, nbytes));
+  return MG_OK;
+}
+
+int mg_free(void *dptr) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  if (!dptr) return MG_OK;
+  // hipFree waits for the device, so no kernel can still be using the block.
+  MG_HIP(hipFree(dptr));
+  return MG_OK;
+}
+
+int mg_host_alloc(void **hptr, size_t nbytes) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  if (!hptr) return fail(MG_ERR_BAD_ARG, "hptr is null");
+  *hptr = nullptr;
+  if (nbytes == 0) nbytes = 64;
+  MG_HIP(hipHostMalloc(hptr, nbytes, hipHostMallocDefault));
+  return MG_OK;
+}
+
+int mg_host_free(void *hptr) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  if (!hptr) return MG_OK;
+  MG_HIP(hipHostFree(hptr));
+  return MG_OK;
+}
+
+int mg_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  if (nbytes == 0) return MG_OK;
+  if (!dst_dev || !src_host) return fail(MG_ERR_BAD_ARG, "null pointer in mg_memcpy_h2d");
+  Runtime &rt = runtime();
+  MG_HIP(hipMemcpyAsync(dst_dev, src_host, nbytes, hipMemcpyHostToDevice, rt.stream));
+  // The source may be pageable and may be reused by the caller right away.
+  MG_HIP(hipStreamSynchronize(rt.stream));
+  return MG_OK;
+}
+
+int mg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  if (nbytes == 0) return MG_OK;
+  if (!dst_host || !src_dev) return fail(MG_ERR_BAD_ARG, "null pointer in mg_memcpy_d2h");
+  Runtime &rt = runtime();
+  MG_HIP(hipMemcpyAsync(dst_host, src_dev, nbytes, hipMemcpyDeviceToHost, rt.stream));
+  MG_HIP(hipStreamSynchronize(rt.stream));
+  return MG_OK;
+}
+
+int mg_memcpy_d2d(void *dst_dev, const void *src_dev, size_t nbytes) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  if (nbytes == 0) return MG_OK;
+  if (!dst_dev || !src_dev) return fail(MG_ERR_BAD_ARG, "null pointer in mg_memcpy_d2d");
+  MG_HIP(hipMemcpyAsync(dst_dev, src_dev, nbytes, hipMemcpyDeviceToDevice, runtime().stream));
+  return MG_OK;
+}
+
+int mg_memset_zero(void *dst_dev, size_t nbytes) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  if (nbytes == 0) return MG_OK;
+  if (!dst_dev) return fail(MG_ERR_BAD_ARG, "null pointer in mg_memset_zero");
+  Runtime &rt = runtime();
+  const size_t nwords = nbytes / 4, tail = nbytes % 4;
+  if ((reinterpret_cast<uintptr_t>(dst_dev) & 3u) != 0)
+    return fail(MG_ERR_BAD_ARG, "mg_memset_zero needs a 4-byte aligned pointer");
+  if (nwords) {
+    size_t blocks = (nwords + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, rt.stream,
+                       static_cast<uint32_t *>(dst_dev), nwords);
+  }
+  if (tail)
+    hipLaunchKernelGGL(fill_zero_bytes_kernel, dim3(1), dim3(64), 0, rt.stream,
+                       static_cast<uint8_t *>(dst_dev) + nwords * 4, tail);
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
+int mg_sync(void) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  MG_HIP(hipStreamSynchronize(runtime().stream));
+  return MG_OK;
+}
+
+int mg_event_create(void **event) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  if (!event) return fail(MG_ERR_BAD_ARG, "event is null");
+  hipEvent_t ev;
+  MG_HIP(hipEventCreate(&ev));
+  *event = ev;
+  return MG_OK;
+}
+
+int mg_event_record(void *event) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  if (!event) return fail(MG_ERR_BAD_ARG, "event is null");
+  MG_HIP(hipEventRecord(static_cast<hipEvent_t>(event), runtime().stream));
+  return MG_OK;
+}
+
+int mg_event_elapsed_ms(void *start, void *stop, float *ms) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  if (!start || !stop || !ms) return fail(MG_ERR_BAD_ARG, "null argument in mg_event_elapsed_ms");
+  MG_HIP(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
+  MG_HIP(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+  return MG_OK;
+}
+
+int mg_event_destroy(void *event) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  if (!event) return MG_OK;
+  MG_HIP(hipEventDestroy(static_cast<hipEvent_t>(event)));
+  return MG_OK;
+}
+
+}  // extern "C"

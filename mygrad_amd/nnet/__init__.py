@@ -1,0 +1,3 @@
+from .layers import conv_nd, max_pool
+
+__all__ = ["conv_nd", "max_pool"]

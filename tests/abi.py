@@ -1,0 +1,92 @@
+"""Test helper: call the C-ABI kernels of libmygrad_hip.so on NumPy arrays
+(upload -> kernel -> download), with the output grid chosen by the floor rule so
+that shapes the Operation layer rejects can be exercised too."""
+
+import numpy as np
+
+from mygrad_amd import _device, _hip
+
+
+def _grid(x_spatial, taps, stride, padding, dilation):
+    return tuple(
+        (int(x) + 2 * int(p) - ((int(t) - 1) * int(d) + 1)) // int(s) + 1
+        for x, t, s, p, d in zip(x_spatial, taps, stride, padding, dilation)
+    )
+
+
+def _tup(v, m):
+    return (int(v),) * m if np.isscalar(v) else tuple(int(i) for i in v)
+
+
+def _up(arr):
+    arr = np.ascontiguousarray(arr)
+    buf = _device.DeviceBuffer(arr.nbytes)
+    buf.upload(arr)
+    return buf
+
+
+def _down(buf, shape, dtype):
+    out = np.empty(shape, dtype=dtype)
+    buf.download_into(out)
+    return out
+
+
+def conv_desc(x_shape, w_shape, dtype, stride, padding, dilation):
+    m = len(x_shape) - 2
+    stride, padding, dilation = _tup(stride, m), _tup(padding, m), _tup(dilation, m)
+    grid = _grid(x_shape[2:], w_shape[2:], stride, padding, dilation)
+    return _hip.conv_desc(dtype, x_shape, w_shape, grid, stride, padding, dilation), grid
+
+
+def conv_fwd(x, w, stride, padding=0, dilation=1):
+    desc, grid = conv_desc(x.shape, w.shape, x.dtype, stride, padding, dilation)
+    xb, wb = _up(x), _up(w)
+    shape = (x.shape[0], w.shape[0], *grid)
+    ob = _device.DeviceBuffer(int(np.prod(shape)) * x.dtype.itemsize)
+    _hip.check(_hip.lib().mg_conv_fwd(desc, xb.ptr, wb.ptr, ob.ptr))
+    return _down(ob, shape, x.dtype)
+
+
+def conv_dgrad(grad, x_shape, w, stride, padding=0, dilation=1):
+    desc, grid = conv_desc(x_shape, w.shape, w.dtype, stride, padding, dilation)
+    assert tuple(grad.shape[2:]) == grid, (grad.shape, grid)
+    gb, wb = _up(grad), _up(w)
+    db = _device.DeviceBuffer(int(np.prod(x_shape)) * w.dtype.itemsize)
+    _hip.check(_hip.lib().mg_conv_dgrad(desc, gb.ptr, wb.ptr, db.ptr))
+    return _down(db, tuple(x_shape), w.dtype)
+
+
+def conv_wgrad(grad, x, w_shape, stride, padding=0, dilation=1):
+    desc, grid = conv_desc(x.shape, w_shape, x.dtype, stride, padding, dilation)
+    assert tuple(grad.shape[2:]) == grid, (grad.shape, grid)
+    gb, xb = _up(grad), _up(x)
+    db = _device.DeviceBuffer(int(np.prod(w_shape)) * x.dtype.itemsize)
+    _hip.check(_hip.lib().mg_conv_wgrad(desc, gb.ptr, xb.ptr, db.ptr))
+    return _down(db, tuple(w_shape), x.dtype)
+
+
+def pool_desc(x_shape, dtype, pool, stride, dx_dtype=None):
+    m = len(pool)
+    stride = _tup(stride, m)
+    lead_shape, pooled = x_shape[: len(x_shape) - m], x_shape[len(x_shape) - m :]
+    grid = tuple((int(x) - int(p)) // int(s) + 1 for x, p, s in zip(pooled, pool, stride))
+    lead = int(np.prod(lead_shape, dtype=np.int64))
+    return _hip.pool_desc(dtype, lead, pooled, pool, stride, grid, dx_dtype=dx_dtype), (*lead_shape, *grid)
+
+
+def pool_fwd(x, pool, stride):
+    desc, out_shape = pool_desc(x.shape, x.dtype, pool, stride)
+    xb = _up(x)
+    ob = _device.DeviceBuffer(int(np.prod(out_shape)) * x.dtype.itemsize)
+    _hip.check(_hip.lib().mg_maxpool_fwd(desc, xb.ptr, ob.ptr))
+    return _down(ob, out_shape, x.dtype)
+
+
+def pool_bwd(x, grad, pool, stride, dx_dtype=None):
+    dx_dtype = np.dtype(x.dtype if dx_dtype is None else dx_dtype)
+    desc, out_shape = pool_desc(x.shape, x.dtype, pool, stride, dx_dtype=dx_dtype)
+    assert tuple(grad.shape) == tuple(out_shape)
+    xb, gb = _up(x), _up(np.ascontiguousarray(grad, dtype=x.dtype))
+    db = _device.DeviceBuffer(x.size * dx_dtype.itemsize)
+    _hip.check(_hip.lib().mg_maxpool_bwd(desc, xb.ptr, gb.ptr, db.ptr))
+    return _down(db, x.shape, dx_dtype)

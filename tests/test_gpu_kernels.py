@@ -1,0 +1,276 @@
+"""Parity of the HIP kernels (called through the C ABI) against the CPU oracle.
+
+Bars: pooling bit-exact (raw bit patterns); convolution
+max|gpu - ref| / max|ref| <= 1e-10 in float64 and <= 2e-4 in float32.
+"""
+
+import numpy as np
+import pytest
+
+from oracle import direct
+from oracle import np_oracle as ora
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.dtype(np.float64): 1e-10, np.dtype(np.float32): 2e-4}
+
+
+@pytest.fixture(scope="module")
+def abi():
+    import mygrad_amd
+
+    if not mygrad_amd.is_available():
+        pytest.fail("libmygrad_hip.so / gfx950 device not available: the GPU tests need both")
+    from tests import abi as module
+
+    return module
+
+
+def rel_err(got, want):
+    scale = float(np.max(np.abs(want))) or 1.0
+    return float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) / scale
+
+
+def bits(a):
+    return a.view(np.uint32 if a.dtype == np.float32 else np.uint64)
+
+
+# ----------------------------------------------------------------------------- pooling
+def test_pool_reference_known_answers(abi, kats):
+    for case in kats["pool"]:
+        x = np.array(case["x"], dtype=case["dtype"])
+        pool, stride = tuple(case["pool"]), tuple(case["stride"])
+        out = abi.pool_fwd(x, pool, stride)
+        assert np.array_equal(out, np.array(case["out"], dtype=x.dtype)), case["source"]
+        if case["grad"] is None:
+            continue
+        g = np.ones(out.shape) if case["grad"] == "ones" else np.arange(out.size).reshape(out.shape)
+        for dx_dtype in (x.dtype, np.float64):
+            dx = abi.pool_bwd(x, g, pool, stride, dx_dtype=dx_dtype)
+            assert dx.dtype == dx_dtype
+            assert np.array_equal(dx, np.array(case["dx"], dtype=float)), case["source"]
+
+
+@pytest.mark.parametrize("m,lead", [(1, (3,)), (1, (2, 5)), (2, (2, 3)), (3, (2,)), (2, ()), (3, (1, 2))])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_pool_ties_and_overlap_bit_exact(abi, m, lead, dtype):
+    rng = np.random.default_rng(300 + 10 * m + len(lead))
+    for trial in range(12):
+        pool = tuple(int(v) for v in rng.integers(1, 5, m))
+        stride = tuple(int(v) for v in rng.integers(1, 5, m))
+        grid = tuple(int(v) for v in rng.integers(1, 9, m))
+        slack = tuple(int(v) for v in rng.integers(0, 2, m))
+        X = tuple((g - 1) * s + p + (e if e < s else 0) for g, s, p, e in zip(grid, stride, pool, slack))
+        print("pool case", m, lead, dtype.__name__, pool, stride, X, flush=True)
+        if trial % 3 == 0:
+            x = rng.standard_normal((*lead, *X)).astype(dtype)
+        else:
+            x = rng.integers(0, 4, (*lead, *X)).astype(dtype)  # few distinct values: ties everywhere
+        out_shape = (*lead, *(((xk - pk) // sk + 1) for xk, pk, sk in zip(X, pool, stride)))
+        g = (rng.standard_normal(out_shape) * 10.0 ** rng.integers(-6, 6, out_shape)).astype(dtype)
+        want_out = ora.pool_forward(x, pool, stride, validate=False)
+        want_dx = ora.pool_backward(x, g, pool, stride)  # float64
+        out = abi.pool_fwd(x, pool, stride)
+        assert np.array_equal(bits(out), bits(want_out))
+        dx64 = abi.pool_bwd(x, g, pool, stride, dx_dtype=np.float64)
+        assert np.array_equal(bits(dx64), bits(want_dx))
+        dx = abi.pool_bwd(x, g, pool, stride)
+        assert np.array_equal(bits(dx), bits(want_dx.astype(dtype)))
+        hits = abi.pool_bwd(x, np.ones(out_shape, dtype), pool, stride)
+        assert np.array_equal(hits, ora.pool_backward(x, np.ones(out_shape), pool, stride))
+
+
+def test_pool_order_of_summation_and_signed_zero(abi):
+    x = np.array([[0.0, 0.0, 9.0, 0.0, 0.0]])
+    for g in ([1e16, 1.0, -1e16], [1e16, -1e16, 1.0], [-0.0, -0.0, -0.0]):
+        g = np.array([g])
+        dx = abi.pool_bwd(x, g, (3,), (1,))
+        assert np.array_equal(bits(dx), bits(ora.pool_backward(x, g, (3,), (1,))))
+    dx = abi.pool_bwd(np.array([[1.0, 0.0]]), np.array([[-0.0]]), (2,), (2,))
+    assert not np.signbit(dx).any()
+
+
+def test_pool_nan_first_nan_wins(abi):
+    x = np.array([[1.0, np.nan, 5.0, np.nan, 2.0, 3.0]])
+    out = abi.pool_fwd(x, (4,), (1,))
+    want = ora.pool_forward(x, (4,), (1,))
+    assert np.array_equal(np.isnan(out), np.isnan(want)) and np.isnan(out).all()
+    g = np.array([[2.0, 3.0, 5.0]])
+    assert np.array_equal(abi.pool_bwd(x, g, (4,), (1,)), ora.pool_backward(x, g, (4,), (1,)))
+
+
+@pytest.mark.parametrize("ties", [False, True])
+def test_pool_config2_literal_full_size(abi, ties):
+    # x (64,64,56,56) f64, pool 3x3 stride 2, floor placement -> (64,64,27,27);
+    # the reference's validator rejects it ((56-3)/2+1 = 27.5), its window helper floors
+    rng = np.random.default_rng(1002)
+    shape = (64, 64, 56, 56)
+    x = rng.integers(0, 8, shape).astype(np.float64) if ties else rng.standard_normal(shape)
+    g = rng.standard_normal((64, 64, 27, 27))
+    out = abi.pool_fwd(x, (3, 3), 2)
+    dx = abi.pool_bwd(x, g, (3, 3), 2)
+    want_out, want_dx = direct.pool(x, g, (3, 3), (2, 2))
+    assert np.array_equal(bits(out), bits(want_out))
+    assert np.array_equal(bits(dx), bits(want_dx))
+    assert not dx[..., 55, :].any() and not dx[..., :, 55].any()  # never covered by a window
+    # the NumPy restatement of the reference agrees on a slice it finishes quickly
+    sl = slice(0, 4)
+    assert np.array_equal(bits(out[sl]), bits(ora.pool_forward(x[sl], (3, 3), 2, validate=False)))
+    assert np.array_equal(bits(dx[sl]), bits(ora.pool_backward(x[sl], g[sl], (3, 3), 2)))
+
+
+def test_pool_config5_shape_full_size(abi):
+    rng = np.random.default_rng(1006)
+    x = rng.standard_normal((8, 32, 32, 64, 64)).astype(np.float32)
+    g = rng.standard_normal((8, 32, 16, 32, 32)).astype(np.float32)
+    out = abi.pool_fwd(x, (2, 2, 2), 2)
+    dx = abi.pool_bwd(x, g, (2, 2, 2), 2)
+    want_out, want_dx = direct.pool(x, g, (2, 2, 2), (2, 2, 2))
+    assert np.array_equal(bits(out), bits(want_out))
+    assert np.array_equal(bits(dx), bits(want_dx.astype(np.float32)))
+
+
+# ----------------------------------------------------------------------------- convolution
+def test_conv_reference_known_answers(abi, kats):
+    for dtype in (np.float64, np.float32):
+        for case in kats["conv"]:
+            x, w = np.array(case["x"], dtype=dtype), np.array(case["w"], dtype=dtype)
+            conf = (tuple(case["stride"]), tuple(case["padding"]), tuple(case["dilation"]))
+            out = abi.conv_fwd(x, w, *conf)
+            assert np.array_equal(out, np.array(case["out"], dtype=dtype)), case["source"]
+            if "dx_of_ones" in case:
+                g = np.ones_like(out)
+                assert np.array_equal(abi.conv_dgrad(g, x.shape, w, *conf), np.array(case["dx_of_ones"], dtype=dtype))
+                assert np.array_equal(abi.conv_wgrad(g, x, w.shape, *conf), np.array(case["dw_of_ones"], dtype=dtype))
+
+
+def _random_case(rng, m, big):
+    hi = 40 if big else 6
+    N = int(rng.integers(1, 4))
+    C = int(rng.integers(1, hi))
+    F = int(rng.integers(1, hi))
+    taps = tuple(int(v) for v in rng.integers(1, 4, m))
+    dil = tuple(int(v) for v in rng.integers(1, 3, m))
+    stride = tuple(int(v) for v in rng.integers(1, 4, m))
+    pad = tuple(int(v) for v in rng.integers(0, 3, m))
+    grid = tuple(int(v) for v in rng.integers(1, 12 if m < 3 else 6, m))
+    extra = tuple(int(v) for v in rng.integers(0, 2, m))  # rows the floor rule never uses
+    X = tuple(
+        (g - 1) * s + (t - 1) * d + 1 - 2 * p + (e if e < s else 0)
+        for g, s, t, d, p, e in zip(grid, stride, taps, dil, pad, extra)
+    )
+    if any(v < 1 for v in X):
+        return None
+    return (N, C, *X), (F, C, *taps), stride, pad, dil
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("m", [1, 2, 3])
+@pytest.mark.parametrize("big", [False, True])
+def test_conv_random_cases_vs_oracle(abi, dtype, m, big):
+    rng = np.random.default_rng(400 + 10 * m + big)
+    tol = TOL[np.dtype(dtype)]
+    done = 0
+    while done < 10:
+        case = _random_case(rng, m, big)
+        if case is None:
+            continue
+        x_shape, w_shape, s, p, d = case
+        print("conv case", np.dtype(dtype).name, x_shape, w_shape, s, p, d, flush=True)
+        x = rng.standard_normal(x_shape).astype(dtype)
+        w = rng.standard_normal(w_shape).astype(dtype)
+        want_out = direct.conv_forward(x, w, s, p, d)
+        g = rng.standard_normal(want_out.shape).astype(dtype)
+        out = abi.conv_fwd(x, w, s, p, d)
+        assert out.shape == want_out.shape and out.dtype == dtype
+        assert rel_err(out, want_out) <= tol
+        assert rel_err(abi.conv_dgrad(g, x_shape, w, s, p, d), direct.conv_backward_x(g, x_shape, w, s, p, d)) <= tol
+        assert rel_err(abi.conv_wgrad(g, x, w_shape, s, p, d), direct.conv_backward_w(g, x, w_shape, s, p, d)) <= tol
+        done += 1
+
+
+def _check_conv_config(abi, seed, dtype, x_shape, w_shape, w_scale, s, p, d, np_oracle_batch):
+    """Full-size check: against the definition-level C reference everywhere, and
+    against the NumPy restatement of the reference on the leading batch items."""
+    rng = np.random.default_rng(seed)
+    tol = TOL[np.dtype(dtype)]
+    x = rng.standard_normal(x_shape).astype(dtype)
+    w = (rng.standard_normal(w_shape) * w_scale).astype(dtype)
+    out = abi.conv_fwd(x, w, s, p, d)
+    g = rng.standard_normal(out.shape).astype(dtype)
+    dx = abi.conv_dgrad(g, x_shape, w, s, p, d)
+    dw = abi.conv_wgrad(g, x, w_shape, s, p, d)
+
+    assert rel_err(out, direct.conv_forward(x, w, s, p, d)) <= tol
+    assert rel_err(dx, direct.conv_backward_x(g, x_shape, w, s, p, d)) <= tol
+    assert rel_err(dw, direct.conv_backward_w(g, x, w_shape, s, p, d)) <= tol
+
+    # adjoint identity <conv(x,w), g> = <x, dx> = <w, dw>, in float64
+    lhs = np.vdot(out.astype(np.float64), g.astype(np.float64))
+    eps = 1e-9 if dtype == np.float64 else 1e-3
+    scale = np.linalg.norm(out.astype(np.float64)) * np.linalg.norm(g.astype(np.float64))
+    assert abs(lhs - np.vdot(x.astype(np.float64), dx.astype(np.float64))) <= eps * scale
+    assert abs(lhs - np.vdot(w.astype(np.float64), dw.astype(np.float64))) <= eps * scale
+
+    nb = np_oracle_batch
+    conf = dict(stride=s, padding=p, dilation=d)
+    ref_out = ora.conv_forward(x[:nb], w, validate=False, **conf)
+    assert rel_err(out[:nb], ref_out) <= tol
+    ref_dx = ora.conv_backward_x(g[:nb], x[:nb].shape, x.dtype, w, **conf)
+    assert rel_err(dx[:nb], ref_dx) <= tol
+    if nb == x_shape[0]:
+        assert rel_err(dw, ora.conv_backward_w(g, x, w_shape, **conf)) <= tol
+
+
+def test_conv_config1(abi):
+    _check_conv_config(abi, 1001, np.float64, (32, 3, 32, 32), (16, 3, 3, 3), 1 / np.sqrt(27), (1, 1), (1, 1), (1, 1), 32)
+
+
+def test_conv_config3a(abi):
+    _check_conv_config(abi, 1003, np.float32, (128, 64, 56, 56), (64, 64, 3, 3), np.sqrt(2 / 576), (1, 1), (1, 1), (1, 1), 2)
+
+
+def test_conv_config3b_literal(abi):
+    _check_conv_config(abi, 1004, np.float32, (128, 128, 28, 28), (256, 128, 3, 3), np.sqrt(2 / 1152), (2, 2), (1, 1), (1, 1), 4)
+
+
+def test_conv_config4_shape(abi):
+    _check_conv_config(abi, 1005, np.float64, (16, 32, 128, 128), (32, 32, 5, 5), 1 / np.sqrt(800), (2, 1), (4, 4), (2, 2), 1)
+
+
+def test_conv_config4_literal(abi):
+    _check_conv_config(abi, 1005, np.float64, (16, 32, 128, 128), (32, 32, 5, 5), 1 / np.sqrt(800), (2, 1), (4, 2), (2, 2), 1)
+
+
+def test_conv_config5(abi):
+    _check_conv_config(abi, 1006, np.float32, (8, 16, 32, 64, 64), (32, 16, 3, 3, 3), np.sqrt(2 / 432), (1, 1, 1), (1, 1, 1), (1, 1, 1), 1)
+
+
+def test_conv_wgrad_is_run_to_run_identical(abi):
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((16, 24, 30, 30)).astype(np.float32)
+    g = rng.standard_normal((16, 40, 28, 28)).astype(np.float32)
+    first = abi.conv_wgrad(g, x, (40, 24, 3, 3), 1, 0, 1)
+    for _ in range(3):
+        assert np.array_equal(bits(first), bits(abi.conv_wgrad(g, x, (40, 24, 3, 3), 1, 0, 1)))
+
+
+def test_abi_rejects_bad_arguments(abi):
+    import ctypes
+
+    from mygrad_amd import _hip
+
+    lib = _hip.lib()
+    desc, _ = abi.conv_desc((1, 1, 4, 4), (1, 1, 3, 3), np.float32, 1, 0, 1)
+    assert lib.mg_conv_fwd(desc, None, None, None) == _hip.MG_ERR_BAD_ARG
+    assert "null" in _hip.last_error()
+    desc.dtype = 7
+    assert lib.mg_conv_fwd(desc, 1, 1, 1) == _hip.MG_ERR_UNSUPPORTED
+    desc.dtype = 0
+    desc.G[2] = 99
+    assert lib.mg_conv_fwd(desc, 1, 1, 1) == _hip.MG_ERR_BAD_ARG
+    pdesc, _ = abi.pool_desc((2, 4, 4), np.float32, (2, 2), 2)
+    pdesc.nd = 5
+    assert lib.mg_maxpool_fwd(pdesc, 1, 1) == _hip.MG_ERR_UNSUPPORTED
+    huge = ctypes.c_void_p()
+    assert lib.mg_malloc(ctypes.byref(huge), 1 << 60) == _hip.MG_ERR_OOM
