@@ -1,0 +1,307 @@
+#!/usr/bin/env python3
+"""Benchmark of the conv_nd / max_pool hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all]
+
+A step is one pass of the hot path over one batch of synthetic input that is
+already resident in HBM: forward + data gradient + filter gradient for a
+convolution workload, forward + backward for a pooling workload, each through
+the C ABI of libmygrad_hip.so.  The script prints ONE JSON line:
+
+* ``value``        whole-step throughput from the host clock around the K steps
+                   (algorithmic flops or bytes / wall time, library stream drained
+                   on both sides);
+* ``roofline``     the dominant kernel of the step: algorithmic flops (or bytes)
+                   of one launch / its mean duration between HIP events recorded
+                   on the library stream inside the timed region;
+* ``cpu_baseline`` the NumPy restatement of the reference algorithm timed on the
+                   host cores on a bounded sample of the same workload;
+* ``secondary``    (with --all) the same figures for the other workloads.
+
+Algorithmic work:  convolution 2*N*F*prod(G)*C*prod(W) flops per pass (padding
+taps count, dense definition); pooling |x|+|out| bytes forward and
+|x|+|grad|+|dx| bytes backward.
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"f32": 157.3, "f64": 78.6}  # MI355X dense matrix peaks
+PEAK_HBM_GBS = 8000.0
+
+# name -> definition.  "lit" shapes use the flooring placement of the window
+# helper (the Operation-level validator of the reference rejects them).
+WORKLOADS = {
+    "conv1": dict(kind="conv", dtype="f64", seed=1001, x=(32, 3, 32, 32), w=(16, 3, 3, 3), wscale=27 ** -0.5,
+                  stride=(1, 1), padding=(1, 1), dilation=(1, 1), cpu_batch=32),
+    "conv3a": dict(kind="conv", dtype="f32", seed=1003, x=(128, 64, 56, 56), w=(64, 64, 3, 3), wscale=(2 / 576) ** 0.5,
+                   stride=(1, 1), padding=(1, 1), dilation=(1, 1), cpu_batch=16),
+    "conv3b": dict(kind="conv", dtype="f32", seed=1004, x=(128, 128, 28, 28), w=(256, 128, 3, 3),
+                   wscale=(2 / 1152) ** 0.5, stride=(2, 2), padding=(1, 1), dilation=(1, 1), cpu_batch=32),
+    "conv4": dict(kind="conv", dtype="f64", seed=1005, x=(16, 32, 128, 128), w=(32, 32, 5, 5), wscale=800 ** -0.5,
+                  stride=(2, 1), padding=(4, 4), dilation=(2, 2), cpu_batch=4),
+    "conv5": dict(kind="conv", dtype="f32", seed=1006, x=(8, 16, 32, 64, 64), w=(32, 16, 3, 3, 3),
+                  wscale=(2 / 432) ** 0.5, stride=(1, 1, 1), padding=(1, 1, 1), dilation=(1, 1, 1), cpu_batch=1),
+    "pool2": dict(kind="pool", dtype="f64", seed=1002, x=(64, 64, 56, 56), pool=(3, 3), stride=(2, 2), cpu_lead=16),
+    "pool5": dict(kind="pool", dtype="f32", seed=1006, x=(8, 32, 32, 64, 64), pool=(2, 2, 2), stride=(2, 2, 2),
+                  cpu_lead=2),
+}
+NP_DTYPE = {"f32": np.float32, "f64": np.float64}
+
+
+def conv_grid(wl):
+    return tuple(
+        (x + 2 * p - ((t - 1) * d + 1)) // s + 1
+        for x, t, s, p, d in zip(wl["x"][2:], wl["w"][2:], wl["stride"], wl["padding"], wl["dilation"])
+    )
+
+
+def conv_flops_per_pass(wl, batch=None):
+    n = wl["x"][0] if batch is None else batch
+    return 2.0 * n * wl["w"][0] * np.prod(conv_grid(wl)) * wl["x"][1] * np.prod(wl["w"][2:])
+
+
+def pool_shapes(wl):
+    m = len(wl["pool"])
+    lead, pooled = wl["x"][: len(wl["x"]) - m], wl["x"][len(wl["x"]) - m:]
+    grid = tuple((x - p) // s + 1 for x, p, s in zip(pooled, wl["pool"], wl["stride"]))
+    return lead, pooled, grid
+
+
+def describe(name):
+    wl = WORKLOADS[name]
+    if wl["kind"] == "conv":
+        return (f"{name}: conv_nd {wl['dtype']} x{wl['x']} * w{wl['w']} stride{wl['stride']} pad{wl['padding']} "
+                f"dil{wl['dilation']} -> grid{conv_grid(wl)} fwd+dx+dw")
+    lead, pooled, grid = pool_shapes(wl)
+    return f"{name}: max_pool {wl['dtype']} x{wl['x']} pool{wl['pool']} stride{wl['stride']} -> grid{grid} fwd+bwd"
+
+
+class Step:
+    """Device-resident inputs and outputs of one workload and its step function."""
+
+    def __init__(self, name):
+        from mygrad_amd import _device, _hip
+
+        self.name, self.wl = name, WORKLOADS[name]
+        wl, dt = self.wl, NP_DTYPE[WORKLOADS[name]["dtype"]]
+        rng = np.random.default_rng(wl["seed"])
+        self.lib = _hip.lib()
+        self.check = _hip.check
+        item = np.dtype(dt).itemsize
+
+        def resident(arr):
+            buf = _device.DeviceBuffer(arr.nbytes)
+            buf.upload(arr)
+            return buf
+
+        if wl["kind"] == "conv":
+            grid = conv_grid(wl)
+            out_shape = (wl["x"][0], wl["w"][0], *grid)
+            x = rng.standard_normal(wl["x"]).astype(dt)
+            w = (rng.standard_normal(wl["w"]) * wl["wscale"]).astype(dt)
+            g = rng.standard_normal(out_shape).astype(dt)
+            self.desc = _hip.conv_desc(dt, wl["x"], wl["w"], grid, wl["stride"], wl["padding"], wl["dilation"])
+            self.x, self.w, self.g = resident(x), resident(w), resident(g)
+            self.out = _device.DeviceBuffer(int(np.prod(out_shape)) * item)
+            self.dx = _device.DeviceBuffer(x.nbytes)
+            self.dw = _device.DeviceBuffer(w.nbytes)
+            per_pass = conv_flops_per_pass(wl)
+            self.work = {"conv_fwd": per_pass, "conv_dgrad": per_pass, "conv_wgrad": per_pass}
+            self.total_work = 3 * per_pass
+            self.unit, self.bound, self.peak = "TFLOP/s", "mfma", PEAK_TFLOPS[wl["dtype"]]
+            self.scale = 1e-12
+        else:
+            lead, pooled, grid = pool_shapes(wl)
+            out_shape = (*lead, *grid)
+            x = rng.standard_normal(wl["x"]).astype(dt)
+            g = rng.standard_normal(out_shape).astype(dt)
+            self.desc = _hip.pool_desc(dt, int(np.prod(lead)), pooled, wl["pool"], wl["stride"], grid)
+            self.x, self.g = resident(x), resident(g)
+            self.out = _device.DeviceBuffer(g.nbytes)
+            self.dx = _device.DeviceBuffer(x.nbytes)
+            self.work = {"maxpool_fwd": float(x.nbytes + g.nbytes), "maxpool_bwd": float(2 * x.nbytes + g.nbytes)}
+            self.total_work = sum(self.work.values())
+            self.unit, self.bound, self.peak = "GB/s", "hbm", PEAK_HBM_GBS
+            self.scale = 1e-9
+
+    def __call__(self):
+        lib, d, check = self.lib, self.desc, self.check
+        if self.wl["kind"] == "conv":
+            check(lib.mg_conv_fwd(d, self.x.ptr, self.w.ptr, self.out.ptr))
+            check(lib.mg_conv_dgrad(d, self.g.ptr, self.w.ptr, self.dx.ptr))
+            check(lib.mg_conv_wgrad(d, self.g.ptr, self.x.ptr, self.dw.ptr))
+        else:
+            check(lib.mg_maxpool_fwd(d, self.x.ptr, self.out.ptr))
+            check(lib.mg_maxpool_bwd(d, self.x.ptr, self.g.ptr, self.dx.ptr))
+
+
+def run_gpu(name, steps, warmup):
+    from mygrad_amd import _hip
+
+    step = Step(name)
+    for _ in range(warmup):
+        step()
+    _hip.synchronize()
+    _hip.timing_enable(True)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    _hip.synchronize()
+    elapsed = time.perf_counter() - t0
+    records = _hip.timing_read()
+    _hip.timing_enable(False)
+
+    per_kernel = {}
+    for kname, ms in records:
+        per_kernel.setdefault(kname, []).append(ms)
+    kernels = {
+        k: {"launches": len(v), "avg_ms": float(np.mean(v)), "min_ms": float(np.min(v))} for k, v in per_kernel.items()
+    }
+    for k, info in kernels.items():
+        if k in step.work:
+            info["achieved"] = step.work[k] * step.scale / (info["avg_ms"] * 1e-3)
+            info["unit"] = step.unit
+            info["frac"] = info["achieved"] / step.peak
+    dominant = max((k for k in kernels if k in step.work), key=lambda k: kernels[k]["avg_ms"] * kernels[k]["launches"])
+    dom = kernels[dominant]
+    ms_per_step = elapsed * 1e3 / steps
+    return {
+        "value": step.total_work * step.scale / (elapsed / steps),
+        "unit": step.unit,
+        "ms_per_step": ms_per_step,
+        "kernel_ms_per_step": float(sum(np.sum(v) for v in per_kernel.values()) / steps),
+        "roofline": {
+            "bound": step.bound,
+            "kernel": dominant,
+            "achieved": dom["achieved"],
+            "peak": step.peak,
+            "unit": step.unit,
+            "frac": dom["frac"],
+            "traffic": measured_traffic(name, dominant),
+            "avg_kernel_ms": dom["avg_ms"],
+            "work_per_launch": step.work[dominant],
+        },
+        "kernels": kernels,
+    }
+
+
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch from committed rocprofv3 --pmc runs, if recorded."""
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as fh:
+            return json.load(fh).get(workload, {}).get(kernel)
+    except (OSError, ValueError):
+        return None
+
+
+def blas_threads():
+    try:
+        from threadpoolctl import threadpool_info
+
+        counts = [p.get("num_threads", 1) for p in threadpool_info() if p.get("user_api") == "blas"]
+        return max(counts) if counts else 1
+    except Exception:
+        return int(os.environ.get("OMP_NUM_THREADS", "1"))
+
+
+def run_cpu_baseline(name):
+    """Time the NumPy restatement of the reference on a bounded sample."""
+    from oracle import np_oracle as ora
+
+    wl, dt = WORKLOADS[name], NP_DTYPE[WORKLOADS[name]["dtype"]]
+    rng = np.random.default_rng(wl["seed"])
+    if wl["kind"] == "conv":
+        nb = min(wl["cpu_batch"], wl["x"][0])
+        x = rng.standard_normal((nb, *wl["x"][1:])).astype(dt)
+        w = (rng.standard_normal(wl["w"]) * wl["wscale"]).astype(dt)
+        conf = dict(stride=wl["stride"], padding=wl["padding"], dilation=wl["dilation"])
+        g = rng.standard_normal((nb, wl["w"][0], *conv_grid(wl))).astype(dt)
+        t0 = time.perf_counter()
+        ora.conv_forward(x, w, validate=False, **conf)
+        ora.conv_backward_x(g, x.shape, x.dtype, w, **conf)
+        ora.conv_backward_w(g, x, w.shape, **conf)
+        dt_s = time.perf_counter() - t0
+        value = 3 * conv_flops_per_pass(wl, nb) * 1e-12 / dt_s
+        sample = f"batch {nb} of {wl['x'][0]}, fwd+dx+dw once, {dt_s:.2f} s"
+        unit = "TFLOP/s"
+    else:
+        m = len(wl["pool"])
+        nl = min(wl["cpu_lead"], wl["x"][0])
+        x = rng.standard_normal((nl, *wl["x"][1:])).astype(dt)
+        lead, pooled, grid = pool_shapes(wl)
+        g = rng.standard_normal((nl, *lead[1:], *grid)).astype(dt)
+        t0 = time.perf_counter()
+        ora.pool_forward(x, wl["pool"], wl["stride"], validate=False)
+        ora.pool_backward(x, g, wl["pool"], wl["stride"])
+        dt_s = time.perf_counter() - t0
+        value = (3 * x.nbytes + 2 * g.nbytes) * 1e-9 / dt_s
+        sample = f"leading {nl} of {wl['x'][0]} along axis 0, fwd+bwd once, {dt_s:.2f} s"
+        unit = "GB/s"
+    return {"value": value, "unit": unit, "cores": blas_threads() if wl["kind"] == "conv" else 1, "kind": "port",
+            "sample": sample, "numpy": np.__version__}
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="conv3a", choices=sorted(WORKLOADS))
+    ap.add_argument("--all", action="store_true", help="also run every other workload (reported under 'secondary')")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (--gpus 1); the path shards over the batch axis "
+                 "by design but no multi-GPU code is part of it")
+
+    wl = WORKLOADS[args.workload]
+    res = run_gpu(args.workload, args.steps, args.warmup)
+    line = {
+        "metric": ("conv_nd fwd+bwd TFLOP/s" if wl["kind"] == "conv" else "max_pool fwd+bwd GB/s"),
+        "value": res["value"],
+        "unit": res["unit"],
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": res["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": wl["dtype"],
+        "data": "synthetic (seeded N(0,1) inputs and upstream gradient, He-normal filters), resident in HBM",
+        "config": {"workload": describe(args.workload)},
+        "roofline": res["roofline"],
+        "kernel_ms_per_step": res["kernel_ms_per_step"],
+        "kernels": res["kernels"],
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = run_cpu_baseline(args.workload)
+    if args.all:
+        secondary = {}
+        for name in WORKLOADS:
+            if name == args.workload:
+                continue
+            r = run_gpu(name, args.steps, args.warmup)
+            entry = {"config": describe(name), "value": r["value"], "unit": r["unit"], "dtype": WORKLOADS[name]["dtype"],
+                     "ms_per_step": r["ms_per_step"], "roofline": r["roofline"], "kernels": r["kernels"]}
+            if not args.no_cpu_baseline:
+                entry["cpu_baseline"] = run_cpu_baseline(name)
+            secondary[name] = entry
+        line["secondary"] = secondary
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

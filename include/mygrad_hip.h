@@ -97,6 +97,15 @@ int mg_event_record(void *event);
 int mg_event_elapsed_ms(void *start, void *stop, float *ms); /* synchronizes on `stop` */
 int mg_event_destroy(void *event);
 
+/* Per-launch kernel timing.  After mg_timing_enable(1) every kernel the library
+ * launches is bracketed by a pair of HIP events on the library stream;
+ * mg_timing_read() waits for the stream, returns up to `capacity` (tag, ms)
+ * records in launch order, sets *count to the number recorded and starts over.
+ * Tags: 1 conv forward, 2 conv dgrad, 3 conv wgrad, 4 wgrad split-K reduction,
+ * 5 filter packing, 6 max-pool forward, 7 max-pool backward. */
+int mg_timing_enable(int on);
+int mg_timing_read(int32_t *tags, float *ms, int capacity, int *count);
+
 /* ---- convolution ---- */
 
 /* out[n,f,g] = sum_{c,t} w[f,c,t] * x[n,c,g*stride+t*dil-pad] (zero outside x).

@@ -103,6 +103,9 @@ _SIGNATURES = {
     "mg_memcpy_d2d": [_vp, _vp, ctypes.c_size_t],
     "mg_memset_zero": [_vp, ctypes.c_size_t],
     "mg_sync": [],
+    "mg_timing_enable": [ctypes.c_int],
+    "mg_timing_read": [ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_float), ctypes.c_int,
+                       ctypes.POINTER(ctypes.c_int)],
     "mg_event_create": [ctypes.POINTER(_vp)],
     "mg_event_record": [_vp],
     "mg_event_elapsed_ms": [_vp, _vp, ctypes.POINTER(ctypes.c_float)],
@@ -195,6 +198,32 @@ def device_info():
 
 def synchronize():
     check(lib().mg_sync())
+
+
+KERNEL_TAGS = {
+    1: "conv_fwd",
+    2: "conv_dgrad",
+    3: "conv_wgrad",
+    4: "wgrad_reduce",
+    5: "pack_filters",
+    6: "maxpool_fwd",
+    7: "maxpool_bwd",
+}
+
+
+def timing_enable(on=True):
+    """Start (or stop) bracketing every kernel launch with HIP events."""
+    check(lib().mg_timing_enable(1 if on else 0))
+
+
+def timing_read(capacity=1 << 16):
+    """[(kernel name, milliseconds), ...] for the launches since the last read."""
+    tags = (ctypes.c_int32 * capacity)()
+    ms = (ctypes.c_float * capacity)()
+    count = ctypes.c_int()
+    check(lib().mg_timing_read(tags, ms, capacity, ctypes.byref(count)))
+    n = min(count.value, capacity)
+    return [(KERNEL_TAGS.get(tags[i], str(tags[i])), float(ms[i])) for i in range(n)]
 
 
 def _right_aligned(values, fill):

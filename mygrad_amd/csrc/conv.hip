@@ -641,9 +641,10 @@ void launch_gemm(const GemmParams &gp, int pos_blocks, hipStream_t s) {
 }
 
 template <typename T>
-int run_gemm(const GemmParams &gp, const Plan &pl, hipStream_t s) {
+int run_gemm(const GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
   constexpr int BK = sizeof(T) == 8 ? 8 : 16;
   if (pl.pos_blocks <= 0) return MG_OK;
+  ScopedTiming timed(tag);
   switch (pl.bm) {
     case 128: launch_gemm<T, 128, 128, BK, 64, 64>(gp, pl.pos_blocks, s); break;
     case 64: launch_gemm<T, 64, 256, BK, 64, 64>(gp, pl.pos_blocks, s); break;
@@ -659,6 +660,7 @@ int pack_filters(const Geometry &g, const void *w, int mode, void **packed) {
   const size_t count = (size_t)g.F * g.C * g.wvol;
   if (int rc = workspace(count * sizeof(T), packed)) return rc;
   const unsigned blocks = (unsigned)std::min<long long>(ceil_div((long long)count, 256), 4096);
+  ScopedTiming timed(TAG_PACK_FILTERS);
   hipLaunchKernelGGL(pack_filters_kernel<T>, dim3(blocks), dim3(256), 0, runtime().stream, static_cast<const T *>(w),
                      static_cast<T *>(*packed), g.F, g.C, (int)g.wvol, mode);
   MG_HIP(hipGetLastError());
@@ -690,7 +692,7 @@ int conv_fwd_impl(const Geometry &g, const Plan &pl, const void *x, const void *
   gp.dst_mstride = (int)g.gvol;
   gp.src_nstride = (long long)g.C * g.xvol;
   gp.dst_nstride = (long long)g.F * g.gvol;
-  return run_gemm<T>(gp, pl, runtime().stream);
+  return run_gemm<T>(gp, pl, TAG_CONV_FWD, runtime().stream);
 }
 
 template <typename T>
@@ -718,7 +720,7 @@ int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   gp.dst_mstride = (int)g.xvol;
   gp.src_nstride = (long long)g.F * g.gvol;
   gp.dst_nstride = (long long)g.C * g.xvol;
-  return run_gemm<T>(gp, pl, runtime().stream);
+  return run_gemm<T>(gp, pl, TAG_CONV_DGRAD, runtime().stream);
 }
 
 template <typename T, int BM, int BN, int BK, int WM, int WN>
@@ -755,14 +757,18 @@ int conv_wgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   wp.kpos = (long long)g.N * g.gvol;
   wp.kchunk = pl.kchunk;
   wp.splits = pl.splits;
-  switch (pl.bm) {
-    case 64: launch_wgrad<T, 64, 64, BK, 32, 32>(wp, s); break;
-    case 32: launch_wgrad<T, 32, 64, BK, 32, 16>(wp, s); break;
-    default: launch_wgrad<T, 16, 64, BK, 16, 16>(wp, s); break;
+  {
+    ScopedTiming timed(TAG_CONV_WGRAD);
+    switch (pl.bm) {
+      case 64: launch_wgrad<T, 64, 64, BK, 32, 32>(wp, s); break;
+      case 32: launch_wgrad<T, 32, 64, BK, 32, 16>(wp, s); break;
+      default: launch_wgrad<T, 16, 64, BK, 16, 16>(wp, s); break;
+    }
   }
   MG_HIP(hipGetLastError());
   if (pl.splits > 1) {
     const int count = g.F * ct;
+    ScopedTiming timed(TAG_WGRAD_REDUCE);
     hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, s,
                        static_cast<const T *>(target), static_cast<T *>(dw), count, pl.splits);
     MG_HIP(hipGetLastError());

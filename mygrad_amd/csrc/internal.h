@@ -39,6 +39,25 @@ Runtime &runtime();
 // until the next call that asks for workspace.
 int workspace(size_t nbytes, void **ptr);
 
+// Optional per-launch timing with HIP events on the library stream (off by
+// default).  A launch site brackets its kernel with timing_begin/timing_end.
+enum KernelTag {
+  TAG_CONV_FWD = 1,
+  TAG_CONV_DGRAD = 2,
+  TAG_CONV_WGRAD = 3,
+  TAG_WGRAD_REDUCE = 4,
+  TAG_PACK_FILTERS = 5,
+  TAG_POOL_FWD = 6,
+  TAG_POOL_BWD = 7,
+};
+void timing_begin(int tag);
+void timing_end();
+
+struct ScopedTiming {
+  explicit ScopedTiming(int tag) { timing_begin(tag); }
+  ~ScopedTiming() { timing_end(); }
+};
+
 // Drops every cached convolution plan (device tables); called by mg_shutdown.
 void release_conv_plans();
 

@@ -147,6 +147,7 @@ int mg_maxpool_fwd(const mg_pool_desc *desc, const void *x, void *out) {
   if (!x || !out) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_maxpool_fwd");
   const unsigned grid = grid_for(p.lead * p.gvol);
   hipStream_t s = runtime().stream;
+  ScopedTiming timed(TAG_POOL_FWD);
   if (desc->dtype == MG_F32)
     hipLaunchKernelGGL(maxpool_fwd_kernel<float>, dim3(grid), dim3(256), 0, s, p, (const float *)x, (float *)out);
   else
@@ -163,6 +164,7 @@ int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, vo
   if (!x || !grad || !dx) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_maxpool_bwd");
   const unsigned grid = grid_for(p.lead * p.xvol);
   hipStream_t s = runtime().stream;
+  ScopedTiming timed(TAG_POOL_BWD);
   if (desc->dtype == MG_F64)
     hipLaunchKernelGGL((maxpool_bwd_kernel<double, double>), dim3(grid), dim3(256), 0, s, p, (const double *)x,
                        (const double *)grad, (double *)dx);

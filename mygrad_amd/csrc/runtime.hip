@@ -2,6 +2,7 @@
 #include "internal.h"
 
 #include <cstring>
+#include <vector>
 
 namespace mg {
 
@@ -49,6 +50,51 @@ int workspace(size_t nbytes, void **ptr) {
   }
   *ptr = rt.workspace;
   return MG_OK;
+}
+
+// ---- per-launch timing -------------------------------------------------------------------
+namespace {
+struct TimingRecord {
+  int tag;
+  hipEvent_t start, stop;
+};
+struct Timing {
+  bool on = false;
+  std::vector<TimingRecord> records;  // event pairs are created once and reused
+  size_t used = 0;
+} g_timing;
+}  // namespace
+
+void timing_begin(int tag) {
+  if (!g_timing.on) return;
+  if (g_timing.used == g_timing.records.size()) {
+    TimingRecord r{tag, nullptr, nullptr};
+    if (hipEventCreate(&r.start) != hipSuccess || hipEventCreate(&r.stop) != hipSuccess) {
+      (void)hipGetLastError();
+      g_timing.on = false;
+      return;
+    }
+    g_timing.records.push_back(r);
+  }
+  TimingRecord &r = g_timing.records[g_timing.used];
+  r.tag = tag;
+  (void)hipEventRecord(r.start, runtime().stream);
+}
+
+void timing_end() {
+  if (!g_timing.on) return;
+  (void)hipEventRecord(g_timing.records[g_timing.used].stop, runtime().stream);
+  ++g_timing.used;
+}
+
+static void timing_release() {
+  for (auto &r : g_timing.records) {
+    (void)hipEventDestroy(r.start);
+    (void)hipEventDestroy(r.stop);
+  }
+  g_timing.records.clear();
+  g_timing.used = 0;
+  g_timing.on = false;
 }
 
 __global__ void fill_zero_kernel(uint32_t *p, size_t nwords) {
@@ -105,6 +151,7 @@ int mg_shutdown(void) {
   if (!rt.ready) return MG_OK;
   MG_HIP(hipStreamSynchronize(rt.stream));
   release_conv_plans();
+  timing_release();
   if (rt.workspace) MG_HIP(hipFree(rt.workspace));
   rt.workspace = nullptr;
   rt.workspace_bytes = 0;
@@ -228,6 +275,30 @@ int mg_sync(void) {
   MG_LOCK();
   MG_REQUIRE_INIT();
   MG_HIP(hipStreamSynchronize(runtime().stream));
+  return MG_OK;
+}
+
+int mg_timing_enable(int on) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  MG_HIP(hipStreamSynchronize(runtime().stream));
+  g_timing.used = 0;
+  g_timing.on = on != 0;
+  return MG_OK;
+}
+
+int mg_timing_read(int32_t *tags, float *ms, int capacity, int *count) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  if (!count || (capacity > 0 && (!tags || !ms))) return fail(MG_ERR_BAD_ARG, "null argument in mg_timing_read");
+  MG_HIP(hipStreamSynchronize(runtime().stream));
+  const int n = (int)g_timing.used;
+  *count = n;
+  for (int i = 0; i < n && i < capacity; ++i) {
+    tags[i] = g_timing.records[i].tag;
+    MG_HIP(hipEventElapsedTime(&ms[i], g_timing.records[i].start, g_timing.records[i].stop));
+  }
+  g_timing.used = 0;
   return MG_OK;
 }
 

@@ -1,0 +1,246 @@
+"""The drop-in path on the GPU: conv_nd / max_pool called like the reference's
+functions, gradients through Tensor.backward(), checked against the CPU oracle.
+Bars: pooling bit-exact; convolution 1e-10 (float64) / 2e-4 (float32) in
+max-abs error normalised by the reference's max-abs."""
+
+import numpy as np
+import pytest
+
+import mygrad_amd as mg
+from mygrad_amd import _device, _graph
+from mygrad_amd.nnet import conv_nd, max_pool
+from oracle import direct
+from oracle import np_oracle as ora
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.dtype(np.float64): 1e-10, np.dtype(np.float32): 2e-4}
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu():
+    if not mg.is_available():
+        pytest.fail("libmygrad_hip.so / gfx950 device not available: the GPU tests need both")
+
+
+def rel_err(got, want):
+    scale = float(np.max(np.abs(want))) or 1.0
+    return float(np.max(np.abs(np.asarray(got, np.float64) - np.asarray(want, np.float64)))) / scale
+
+
+def test_reference_docstring_and_known_answers(kats):
+    for case in kats["conv"]:
+        x, w = mg.Tensor(np.array(case["x"], dtype=float)), mg.Tensor(np.array(case["w"], dtype=float))
+        conf = dict(stride=tuple(case["stride"]), padding=tuple(case["padding"]), dilation=tuple(case["dilation"]))
+        out = conv_nd(x, w, **conf)
+        assert isinstance(out, mg.Tensor) and out.constant is False
+        assert np.array_equal(out.data, np.array(case["out"], dtype=float)), case["source"]
+        out.backward()
+        if "dx_of_ones" in case:
+            assert np.array_equal(x.grad, np.array(case["dx_of_ones"], dtype=float))
+            assert np.array_equal(w.grad, np.array(case["dw_of_ones"], dtype=float))
+        assert conv_nd(x, w, constant=True, **conf).constant is True
+        x.clear_graph(), w.clear_graph()
+    for case in kats["pool"]:
+        x = mg.Tensor(np.array(case["x"]), dtype=case["dtype"])
+        out = max_pool(x, tuple(case["pool"]), tuple(case["stride"]))
+        assert np.array_equal(out.data, np.array(case["out"], dtype=x.dtype)), case["source"]
+        if case["grad"] is None:
+            out.clear_graph()
+            continue
+        if case["grad"] == "ones":
+            out.backward()
+        else:
+            out.backward(np.arange(out.size).reshape(out.shape))
+        assert x.grad.dtype == x.dtype
+        assert np.array_equal(x.grad, np.array(case["dx"], dtype=float)), case["source"]
+        assert max_pool(x, tuple(case["pool"]), tuple(case["stride"]), constant=True).constant is True
+    assert _graph.held_count() == 0
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
+def test_padding_only_image_gives_zero(m):
+    rng = np.random.default_rng(m)
+    pad = tuple(int(p) for p in rng.integers(1, 4, m))
+    x = mg.Tensor(np.zeros((1, 1) + (0,) * m))
+    w = rng.standard_normal((1, 1) + tuple(2 * p for p in pad))
+    if m > 3:
+        with pytest.raises(NotImplementedError):
+            conv_nd(x, w, padding=pad, stride=1)
+        return
+    out = conv_nd(x, w, padding=pad, stride=1)
+    assert out.shape == (1,) * (m + 2) and out.item() == 0.0
+    out.backward()
+    assert x.grad.shape == x.shape
+
+
+def _drop_in_conv(seed, dtype, x_shape, w_shape, wscale, conf):
+    rng = np.random.default_rng(seed)
+    x = mg.Tensor(rng.standard_normal(x_shape).astype(dtype))
+    w = mg.Tensor((rng.standard_normal(w_shape) * wscale).astype(dtype))
+    out = conv_nd(x, w, **conf)
+    g = rng.standard_normal(out.shape).astype(dtype)
+    assert not x.data.flags.writeable and not out.data.flags.writeable
+    out_data = out.data
+    out.backward(g)
+    assert x.data.flags.writeable and out_data.flags.writeable and _graph.held_count() == 0
+    assert x.grad.dtype == dtype and w.grad.dtype == dtype and out.grad.dtype == dtype
+    assert x.grad.shape == x.shape and w.grad.shape == w.shape
+    assert not np.shares_memory(x.grad, g) and not np.shares_memory(w.grad, g)
+    return x, w, g, out_data
+
+
+def test_config1_through_backward():
+    conf = dict(stride=1, padding=1, dilation=1)
+    x, w, g, out = _drop_in_conv(1001, np.float64, (32, 3, 32, 32), (16, 3, 3, 3), 27 ** -0.5, conf)
+    assert rel_err(out, ora.conv_forward(x.data, w.data, **conf)) <= 1e-10
+    assert rel_err(x.grad, ora.conv_backward_x(g, x.shape, x.dtype, w.data, **conf)) <= 1e-10
+    assert rel_err(w.grad, ora.conv_backward_w(g, x.data, w.shape, **conf)) <= 1e-10
+
+
+def test_config3b_valid_through_backward():
+    # (128,128,27,27): the neighbouring shape the reference accepts, same output (128,256,14,14)
+    conf = dict(stride=2, padding=1, dilation=1)
+    x, w, g, out = _drop_in_conv(1004, np.float32, (128, 128, 27, 27), (256, 128, 3, 3), (2 / 1152) ** 0.5, conf)
+    assert out.shape == (128, 256, 14, 14)
+    s, p, d = (2, 2), (1, 1), (1, 1)
+    assert rel_err(out, direct.conv_forward(x.data, w.data, s, p, d)) <= 2e-4
+    assert rel_err(x.grad, direct.conv_backward_x(g, x.shape, w.data, s, p, d)) <= 2e-4
+    assert rel_err(w.grad, direct.conv_backward_w(g, x.data, w.shape, s, p, d)) <= 2e-4
+    nb = 4
+    assert rel_err(out[:nb], ora.conv_forward(x.data[:nb], w.data, **conf)) <= 2e-4
+    assert rel_err(x.grad[:nb], ora.conv_backward_x(g[:nb], x.data[:nb].shape, x.dtype, w.data, **conf)) <= 2e-4
+
+
+def test_config4_valid_through_backward():
+    # (16,32,127,128) with padding (4,4): exact placements, output (16,32,64,128)
+    conf = dict(stride=(2, 1), padding=(4, 4), dilation=(2, 2))
+    x, w, g, out = _drop_in_conv(1005, np.float64, (16, 32, 127, 128), (32, 32, 5, 5), 800 ** -0.5, conf)
+    assert out.shape == (16, 32, 64, 128)
+    s, p, d = (2, 1), (4, 4), (2, 2)
+    assert rel_err(out, direct.conv_forward(x.data, w.data, s, p, d)) <= 1e-10
+    assert rel_err(x.grad, direct.conv_backward_x(g, x.shape, w.data, s, p, d)) <= 1e-10
+    assert rel_err(w.grad, direct.conv_backward_w(g, x.data, w.shape, s, p, d)) <= 1e-10
+    assert rel_err(out[:1], ora.conv_forward(x.data[:1], w.data, **conf)) <= 1e-10
+
+
+@pytest.mark.parametrize("ties", [False, True])
+def test_config2_valid_through_backward(ties):
+    rng = np.random.default_rng(1002)
+    shape = (64, 64, 55, 55)
+    xv = rng.integers(0, 8, shape).astype(np.float64) if ties else rng.standard_normal(shape)
+    x = mg.Tensor(xv)
+    out = max_pool(x, (3, 3), 2)
+    assert out.shape == (64, 64, 27, 27)
+    g = rng.standard_normal(out.shape)
+    out_data = out.data
+    out.backward(g)
+    want_out, want_dx = direct.pool(xv, g, (3, 3), (2, 2))
+    assert np.array_equal(out_data.view(np.uint64), want_out.view(np.uint64))
+    assert np.array_equal(x.grad.view(np.uint64), want_dx.view(np.uint64))
+    sl = slice(0, 3)
+    assert np.array_equal(out_data[sl], ora.pool_forward(xv[sl], (3, 3), 2))
+    assert np.array_equal(x.grad[sl].view(np.uint64), ora.pool_backward(xv[sl], g[sl], (3, 3), 2).view(np.uint64))
+
+
+def test_config5_chain_keeps_activations_on_the_device():
+    rng = np.random.default_rng(1006)
+    dtype = np.float32
+    x = mg.Tensor(rng.standard_normal((8, 16, 32, 64, 64)).astype(dtype))
+    w = mg.Tensor((rng.standard_normal((32, 16, 3, 3, 3)) * (2 / 432) ** 0.5).astype(dtype))
+    g = rng.standard_normal((8, 32, 16, 32, 32)).astype(dtype)
+    before = dict(_device.stats)
+    y = conv_nd(x, w, stride=1, padding=1)
+    z = max_pool(y, (2, 2, 2), 2)
+    y_data, z_data = y.data, z.data
+    z.backward(g)
+    uploads = _device.stats["uploads"] - before["uploads"]
+    assert uploads == 3, uploads  # x, w and the seed gradient; nothing is uploaded twice
+    assert _device.stats["mirror_hits"] - before["mirror_hits"] >= 5
+
+    s = p = d = (1, 1, 1)
+    assert rel_err(y_data, direct.conv_forward(x.data, w.data, s, p, d)) <= 2e-4
+    want_z, want_dy = direct.pool(y_data, g, (2, 2, 2), (2, 2, 2))
+    assert np.array_equal(z_data, want_z)
+    assert np.array_equal(y.grad.view(np.uint32), want_dy.astype(dtype).view(np.uint32))
+    assert rel_err(x.grad, direct.conv_backward_x(y.grad, x.shape, w.data, s, p, d)) <= 2e-4
+    assert rel_err(w.grad, direct.conv_backward_w(y.grad, x.data, w.shape, s, p, d)) <= 2e-4
+    assert _graph.held_count() == 0
+
+
+def test_mirror_is_dropped_when_host_data_may_change():
+    rng = np.random.default_rng(9)
+    x = mg.Tensor(rng.standard_normal((2, 3, 8, 8)))
+    w = mg.Tensor(rng.standard_normal((4, 3, 3, 3)))
+    conv_nd(x, w, stride=1).backward()
+    w.data[...] *= 2.0  # an optimiser step on the host between two graphs
+    out = conv_nd(x, w, stride=1)
+    assert rel_err(out.data, ora.conv_forward(x.data, w.data, stride=1)) <= 1e-10
+    out.clear_graph()
+
+
+def test_operand_variety():
+    rng = np.random.default_rng(10)
+    x64 = rng.standard_normal((2, 3, 9, 9))
+    w32 = rng.standard_normal((4, 3, 3, 3)).astype(np.float32)
+    # mixed precision promotes like NumPy; gradients come back in each operand's dtype
+    x, w = mg.Tensor(x64), mg.Tensor(w32)
+    out = conv_nd(x, w, stride=2)
+    assert out.dtype == np.float64
+    out.backward()
+    assert x.grad.dtype == np.float64 and w.grad.dtype == np.float32
+    assert rel_err(out.data, ora.conv_forward(x64, w32, stride=2)) <= 1e-10
+    # non-contiguous operands and integer (constant) data
+    xt = mg.Tensor(np.asfortranarray(x64))
+    xi = mg.Tensor(rng.integers(-3, 4, (2, 3, 9, 9)))
+    wt = mg.Tensor(w32.astype(np.float64))
+    assert rel_err(conv_nd(xt, wt, stride=1).data, ora.conv_forward(x64, wt.data, stride=1)) <= 1e-10
+    out = conv_nd(xi, wt, stride=1, dilation=2)
+    assert out.dtype == np.float64
+    assert rel_err(out.data, ora.conv_forward(xi.data, wt.data, stride=1, dilation=2)) <= 1e-10
+    out.backward()
+    assert xi.grad is None and wt.grad is not None
+    # only one non-constant input: only that gradient is computed
+    xc = mg.Tensor(x64, constant=True)
+    out = conv_nd(xc, wt, stride=1)
+    out.backward()
+    assert xc.grad is None
+    assert rel_err(wt.grad, ora.conv_backward_w(np.ones(out.shape), x64, wt.shape, stride=1)) <= 1e-10
+    # pooling over all axes of a 2-D tensor (no leading axes) and over a non-contiguous one
+    p = mg.Tensor(np.asfortranarray(rng.integers(0, 5, (6, 8)).astype(np.float64)))
+    out = max_pool(p, (2, 2), (2, 2))
+    assert np.array_equal(out.data, ora.pool_forward(p.data, (2, 2), 2))
+    out.backward()
+    assert np.array_equal(p.grad, ora.pool_backward(p.data, np.ones(out.shape), (2, 2), 2))
+    assert _graph.held_count() == 0
+
+
+def test_tensor_feeding_two_pools_accumulates_like_the_reference():
+    # second contribution is added to an existing float32 gradient: the reference adds
+    # the unrounded float64 dx (pooling.py:147, operation_base.py:227-228)
+    rng = np.random.default_rng(12)
+    xv = rng.integers(0, 3, (3, 9, 9)).astype(np.float32)
+    x = mg.Tensor(xv)
+
+    class Twice(mg.Operation):
+        def __call__(self, a, b):
+            self.variables = (a, b)
+            return a.data + b.data
+
+        def backward_var(self, grad, index, **kwargs):
+            return grad * np.float32(1.0 if index == 0 else 3.0)
+
+    a = max_pool(x, (3, 3), 1)
+    b = max_pool(x, (3, 3), 1)
+    out = mg.execute_op(Twice, a, b)
+    g = (rng.standard_normal(out.shape) * 1e3).astype(np.float32)
+    out.backward(g)
+    first = ora.pool_backward(xv, g * np.float32(1.0), (3, 3), 1)
+    second = ora.pool_backward(xv, g * np.float32(3.0), (3, 3), 1)
+    # backward visits `b` (the later consumer in topological order) or `a` first;
+    # either way: float32(first-visited), then += the other in float64
+    want_ab = first.astype(np.float32)
+    want_ab += second
+    want_ba = second.astype(np.float32)
+    want_ba += first
+    assert np.array_equal(x.grad, want_ab) or np.array_equal(x.grad, want_ba)

@@ -1,0 +1,314 @@
+"""Host-side logic that needs no GPU: the C-ABI library loads and exports what
+the header declares, argument validation raises the reference's exception types
+before anything is launched, the window helper, and the graph semantics of the
+Tensor / Operation shim (exercised with a tiny NumPy-only operation defined
+here)."""
+
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import mygrad_amd as mg
+from mygrad_amd import _graph, _hip
+from mygrad_amd.nnet import conv_nd, max_pool
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ----------------------------------------------------------------------------- C ABI
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "mygrad_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mg_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _hip.load_library()
+    declared = _declared_symbols()
+    assert len(declared) >= 20
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in mygrad_hip.h but not exported"
+    assert sorted(_hip.EXPORTED_SYMBOLS) == declared
+
+
+def test_struct_layouts_match_header():
+    # int32 x2 + int64 x3 + 6 * int64[3]
+    assert ctypes.sizeof(_hip.ConvDesc) == 8 + 24 + 6 * 24
+    assert ctypes.sizeof(_hip.PoolDesc) == 16 + 8 + 4 * 24
+    assert ctypes.sizeof(_hip.DeviceInfo) == 64 + 16 + 8 + 16
+
+
+def test_calls_before_init_report_not_initialised():
+    if _hip._ready:
+        pytest.skip("a device is initialised in this process")
+    lib = _hip.load_library()
+    assert lib.mg_sync() == _hip.MG_ERR_NOT_INIT
+    assert "mg_init" in _hip.last_error()
+    ptr = ctypes.c_void_p()
+    assert lib.mg_malloc(ctypes.byref(ptr), 16) == _hip.MG_ERR_NOT_INIT
+
+
+def test_no_device_fails_loudly_without_fallback():
+    if mg.is_available():
+        pytest.skip("a GPU is present")
+    x = np.zeros((1, 1, 4, 4))
+    with pytest.raises(mg.HipUnavailable):
+        conv_nd(x, np.zeros((1, 1, 2, 2)), stride=1)
+    with pytest.raises(mg.HipUnavailable):
+        max_pool(x, (2, 2), 2)
+    assert _graph.held_count() == 0  # a failing op releases its locks
+    assert x.flags.writeable
+
+
+# ----------------------------------------------------------------------------- validation (no launch)
+@pytest.mark.parametrize(
+    "x_shape,w_shape",
+    [((4,), (1, 1, 2)), ((3, 3), (1, 3, 2)), ((1, 2, 5), (1, 2)), ((1, 2, 5, 5), (1, 2, 3)), ((1, 2, 5), (1, 3, 2))],
+)
+def test_conv_shape_mismatch_is_value_error(x_shape, w_shape):
+    with pytest.raises(ValueError):
+        conv_nd(np.zeros(x_shape), np.zeros(w_shape), stride=1)
+
+
+def test_conv_error_contract():
+    x = np.zeros((1, 2, 2, 2))
+    w = np.zeros((1, 2, 2, 2))
+    with pytest.raises(ValueError):
+        conv_nd(x, np.zeros((1, 3, 2, 2)), stride=1, padding=0)  # mismatched channels
+    with pytest.raises(ValueError):
+        conv_nd(x, np.zeros((1, 2, 3, 2)), stride=1, padding=0)  # filter larger than data
+    with pytest.raises(AssertionError):
+        conv_nd(x, w, stride=0, padding=0)
+    with pytest.raises(AssertionError):
+        conv_nd(x, w, stride=[1, 2, 3])
+    with pytest.raises(AssertionError):
+        conv_nd(x, w, stride=1, padding=-1)
+    with pytest.raises(AssertionError):
+        conv_nd(x, w, stride=1, padding=[1, 2, 3])
+    with pytest.raises(AssertionError):
+        conv_nd(x, w, stride=1, dilation=0)
+    with pytest.raises(ValueError) as info:
+        conv_nd(x, w, stride=3, padding=1)  # non-integer output extent
+    assert "Stride and kernel dimensions are incompatible" in str(info.value)
+    # the benchmark shapes the reference rejects are rejected here too
+    with pytest.raises(ValueError):
+        conv_nd(np.zeros((1, 1, 28, 28), np.float32), np.zeros((1, 1, 3, 3), np.float32), stride=2, padding=1)
+    # the window helper's w*d <= extent rule, applied to the padded data
+    with pytest.raises(ValueError):
+        conv_nd(np.zeros((1, 1, 3)), np.zeros((1, 1, 2)), stride=1, dilation=2)
+    assert _graph.held_count() == 0 and x.flags.writeable and w.flags.writeable
+
+
+def test_pool_error_contract():
+    x = mg.Tensor(np.zeros((1, 2, 2, 2)), dtype="float32")
+    with pytest.raises(ValueError):
+        max_pool(x, (3,) * 3, (1,) * 3)
+    with pytest.raises(AssertionError):
+        max_pool(x, (2,) * 3, (0,) * 3)
+    with pytest.raises(AssertionError):
+        max_pool(x, (2,) * 2, [1, 2, 3])
+    with pytest.raises(AssertionError):
+        max_pool(x, 2, 1)  # pool must be a sequence
+    with pytest.raises(AssertionError):
+        max_pool(x, (2, 0), 1)
+    with pytest.raises(ValueError) as info:
+        max_pool(x, (1,) * 3, (3,) * 3)
+    assert "Pooling dimensions" in str(info.value)
+    with pytest.raises(ValueError):
+        max_pool(np.zeros((1, 1, 56, 56)), (3, 3), 2)  # 27.5 placements
+    assert _graph.held_count() == 0
+
+
+def test_unsupported_inputs_are_rejected_not_computed_on_the_cpu():
+    with pytest.raises(NotImplementedError):
+        conv_nd(np.zeros((1, 1, 2, 2, 2, 2)), np.zeros((1, 1, 1, 1, 1, 1)), stride=1)
+    with pytest.raises(TypeError):
+        conv_nd(np.zeros((1, 1, 4), np.float16), np.zeros((1, 1, 2), np.float16), stride=1)
+    with pytest.raises(TypeError):
+        max_pool(np.zeros((1, 4), np.int64), (2,), 2)
+    with pytest.raises(NotImplementedError):
+        max_pool(np.zeros((2, 2, 2, 2)), (1, 1, 1, 1), 1)
+
+
+# ----------------------------------------------------------------------------- window helper
+def test_sliding_window_view_vectors(kats):
+    case = kats["window"][0]
+    y = mg.sliding_window_view(np.arange(36).reshape(6, 6), window_shape=case["window_shape"], step=case["step"])
+    assert list(y.shape) == case["shape"]
+    for key, want in case["picks"].items():
+        i, j = map(int, key.split(","))
+        assert np.array_equal(y[i, j], np.array(want))
+    want = np.array(kats["window"][1]["view"])
+    x = np.asfortranarray(np.arange(20).reshape(2, 10))
+    y = mg.sliding_window_view(x, (5,), 5)
+    assert not y.flags.writeable and np.array_equal(y, want)
+    x = np.arange(20).reshape(2, 10)
+    y = mg.sliding_window_view(x, (5,), 5)
+    assert np.shares_memory(x, y) and np.array_equal(y, want)
+
+
+def test_sliding_window_view_matches_slicing():
+    rng = np.random.default_rng(3)
+    for _ in range(200):
+        nd = int(rng.integers(1, 5))
+        shape = tuple(int(v) for v in rng.integers(1, 8, nd))
+        x = rng.integers(0, 100, shape)
+        m = int(rng.integers(1, nd + 1))
+        tail = shape[-m:]
+        win = tuple(int(rng.integers(1, s + 1)) for s in tail)
+        step = tuple(int(rng.integers(1, s + 1)) for s in tail)
+        dil = tuple(int(rng.integers(1, s // w + 1)) for s, w in zip(tail, win))
+        y = mg.sliding_window_view(x, win, step, dil)
+        for g in np.ndindex(*y.shape[:m]):
+            sl = tuple(slice(i * s, i * s + w * d, d) for i, w, s, d in zip(g, win, step, dil))
+            assert np.array_equal(y[g], x[(Ellipsis, *sl)])
+
+
+@pytest.mark.parametrize(
+    "kwargs",
+    [dict(step=None), dict(step=-1), dict(window_shape=None), dict(window_shape=1), dict(window_shape=(1, 1, 1)),
+     dict(window_shape=(-1, 1)), dict(window_shape=(1.0, 2.0)), dict(window_shape=(7, 5)), dict(dilation=-1),
+     dict(dilation=(1, 0)), dict(dilation="aa"), dict(dilation=(1, 1, 1)), dict(dilation=1.0), dict(dilation=7),
+     dict(dilation=(1, 7)), dict(dilation=(10, 1))],
+)
+def test_sliding_window_view_validation(kwargs):
+    args = dict(arr=np.arange(36).reshape(6, 6), window_shape=(1, 1), step=1, dilation=None)
+    args.update(kwargs)
+    with pytest.raises((ValueError, TypeError)):
+        mg.sliding_window_view(**args)
+
+
+# ----------------------------------------------------------------------------- graph semantics
+class Scale(mg.Operation):
+    """out = a * x + b * y, a NumPy-only stand-in used to drive the shim."""
+
+    def __call__(self, x, y, a=2.0, b=3.0):
+        self.variables = (x, y)
+        self.a, self.b = a, b
+        return a * x.data + b * y.data
+
+    def backward_var(self, grad, index, **kwargs):
+        return (self.a if index == 0 else self.b) * grad
+
+
+class Identity(mg.Operation):
+    def __call__(self, x):
+        self.variables = (x,)
+        return x.data.copy()
+
+    def backward_var(self, grad, index, **kwargs):
+        return grad  # the incoming gradient itself: the caller must copy it
+
+
+def test_op_wraps_output_without_copy_and_locks_arrays():
+    x = mg.Tensor([1.0, 2.0])
+    y = np.array([3.0, 4.0])
+    captured = {}
+
+    class Spy(Scale):
+        def __call__(self, *a, **k):
+            captured["out"] = super().__call__(*a, **k)
+            return captured["out"]
+
+    out = mg.execute_op(Spy, x, y)
+    assert out.data is captured["out"]
+    assert isinstance(out.creator, Spy) and out.creator.variables[0] is x
+    assert out.creator.variables[1].data is y and out.creator.variables[1].constant
+    assert not x.data.flags.writeable and not y.flags.writeable and not out.data.flags.writeable
+    out.backward()
+    assert x.data.flags.writeable and y.flags.writeable and out.data.flags.writeable
+    assert out.creator is None and _graph.held_count() == 0
+    assert np.array_equal(x.grad, [2.0, 2.0])
+
+
+def test_constant_propagation():
+    f, c = mg.Tensor([1.0]), mg.Tensor([1.0], constant=True)
+    assert mg.execute_op(Scale, f, c).constant is False
+    assert mg.execute_op(Scale, c, c).constant is True
+    assert mg.execute_op(Scale, f, f, constant=True).constant is True
+    assert mg.execute_op(Scale, c, [1.0]).constant is True
+    assert mg.Tensor([1, 2]).constant is True
+    with pytest.raises(ValueError):
+        mg.Tensor([1, 2], constant=False)
+    with pytest.raises(TypeError):
+        mg.Tensor([1.0], constant="yes")
+    out = mg.execute_op(Scale, c, c)
+    out.backward()  # constant terminal: clears the graph, computes nothing
+    assert c.grad is None and out.grad is None and _graph.held_count() == 0
+    for t in (f,):
+        t.clear_graph()
+
+
+def test_backward_seed_accumulation_dtype_and_aliasing():
+    x = mg.Tensor(np.array([1.0, 2.0, 3.0], dtype=np.float32))
+    out = mg.execute_op(Scale, x, x)  # x feeds the op twice: 2*g then += 3*g
+    g = np.array([1.0, 10.0, 100.0])
+    out.backward(g)
+    assert x.grad.dtype == np.float32
+    assert np.array_equal(x.grad, 5 * g.astype(np.float32))
+    assert np.array_equal(g, [1.0, 10.0, 100.0]) and out.grad.dtype == np.float32
+    assert out.grad is not g
+
+    x = mg.Tensor([1.0, 2.0])
+    out = mg.execute_op(Identity, x)
+    out.backward()
+    assert x.grad is not out.grad and not np.shares_memory(x.grad, out.grad)
+    out2 = mg.execute_op(Identity, x)  # entering a new graph nulls the old gradient
+    assert x.grad is None
+    out2.backward(2.0)  # broadcast seed
+    assert np.array_equal(x.grad, [2.0, 2.0])
+    with pytest.raises(ValueError):
+        mg.execute_op(Identity, x).backward(np.ones(3))
+    x.clear_graph()
+
+
+def test_invalid_gradient_and_cleared_graph():
+    class Bad(Identity):
+        def backward_var(self, grad, index, **kwargs):
+            return "not an array"
+
+    x = mg.Tensor([1.0])
+    with pytest.raises(mg.InvalidGradient):
+        mg.execute_op(Bad, x).backward()
+    x.clear_graph()
+
+    x = mg.Tensor([1.0])
+    mid = mg.execute_op(Identity, x)
+    out = mg.execute_op(Identity, mid)
+    x._ops.clear()  # what clearing the upstream part of the graph leaves behind
+    with pytest.raises(mg.InvalidBackprop):
+        out.backward()
+    out.clear_graph()
+
+
+def test_chain_and_fan_out_topological_order():
+    x = mg.Tensor([1.0, 2.0])
+    a = mg.execute_op(Scale, x, x, op_kwargs=dict(a=1.0, b=1.0))  # 2x
+    b = mg.execute_op(Scale, a, x, op_kwargs=dict(a=1.0, b=1.0))  # 3x
+    c = mg.execute_op(Scale, a, b, op_kwargs=dict(a=1.0, b=1.0))  # 5x
+    c.backward()
+    assert np.array_equal(x.grad, [5.0, 5.0]) and np.array_equal(a.grad, [2.0, 2.0])
+    assert _graph.held_count() == 0
+
+
+def test_no_autodiff_and_mem_guard_switches():
+    x = mg.Tensor([1.0])
+    with mg.no_autodiff:
+        out = mg.execute_op(Identity, x)
+        assert out.creator is None and x.data.flags.writeable
+        out.backward()  # no-op
+    assert x.grad is None
+
+    @mg.no_autodiff
+    def run(t):
+        return mg.execute_op(Identity, t)
+
+    assert run(x).creator is None and _graph.TRACK_GRAPH is True
+    with mg.mem_guard_off:
+        out = mg.execute_op(Identity, x)
+        assert x.data.flags.writeable and out.creator is not None
+        out.backward()
+    assert np.array_equal(x.grad, [1.0])
