@@ -23,6 +23,24 @@
 
 namespace mg {
 
+// Tables that every lane of a wavefront reads at the same index are addressed
+// through the constant address space, which lets the compiler fetch them with
+// scalar loads (one request per wavefront, no vector-memory wait) instead of 64
+// identical vector loads.
+#define MG_CONSTANT __attribute__((address_space(4)))
+typedef int int4v __attribute__((ext_vector_type(4)));
+static_assert(sizeof(TabEntry) == sizeof(int4v), "a table row is read as one 16-byte vector");
+__device__ __forceinline__ const int4v MG_CONSTANT *as_constant(const TabEntry *p) {
+  return (const int4v MG_CONSTANT *)(p);
+}
+__device__ __forceinline__ const int MG_CONSTANT *as_constant(const int *p) { return (const int MG_CONSTANT *)(p); }
+__device__ __forceinline__ TabEntry table_row(const int4v MG_CONSTANT *tab, int i) {
+  const int4v v = tab[i];
+  return TabEntry{v.x, v.y, v.z, v.w};
+}
+// The wavefront-uniform value of x as a scalar register.
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef double f64x4 __attribute__((ext_vector_type(4)));
 
@@ -114,72 +132,73 @@ __global__ void __launch_bounds__(256) gather_gemm_kernel(const GemmParams p) {
   const int jvol = ph.J[0] * j12;
 
   const T *__restrict__ A = static_cast<const T *>(p.A);
-  const TabEntry *__restrict__ tab = p.tab + ph.k_begin;
-  const int *__restrict__ arow = p.arow + ph.k_begin;
+  const int4v MG_CONSTANT *tab = as_constant(p.tab + ph.k_begin);
+  const int MG_CONSTANT *arow = as_constant(p.arow + ph.k_begin);
 
   // ---- loader state: this thread's position in the B tile
+  static_assert(BN % 64 == 0, "a wavefront loads one table row of the B tile at a time");
   const int bcol = tid % BN;
-  const int brow0 = tid / BN;
+  const int brow0 = uniform(tid / BN);
   int qb0 = 0, qb1 = 0, qb2 = 0, lin = 0;
-  bool pos_ok = false;
+  const bool pos_ok = pos0 + bcol < ph.npos;
   const T *__restrict__ srcn = static_cast<const T *>(p.src);
   {
-    const long long pos = (long long)pos0 + bcol;
-    if (pos < ph.npos) {
-      pos_ok = true;
-      const int n = (int)(pos / jvol);
-      int r = (int)(pos - (long long)n * jvol);
-      const int j0 = r / j12;
-      r -= j0 * j12;
-      const int j1 = r / ph.J[2];
-      const int j2 = r - j1 * ph.J[2];
-      qb0 = j0 * p.sj[0];
-      qb1 = j1 * p.sj[1];
-      qb2 = j2 * p.sj[2];
-      lin = qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2];
-      srcn += (long long)n * p.src_nstride;
-    }
+    const unsigned pos = pos_ok ? (unsigned)(pos0 + bcol) : 0u;
+    const unsigned n = ph.by_jvol.div(pos);
+    unsigned r = pos - n * (unsigned)jvol;
+    const unsigned j0 = ph.by_j12.div(r);
+    r -= j0 * (unsigned)j12;
+    const unsigned j1 = ph.by_j2.div(r);
+    const unsigned j2 = r - j1 * (unsigned)ph.J[2];
+    qb0 = (int)j0 * p.sj[0];
+    qb1 = (int)j1 * p.sj[1];
+    qb2 = (int)j2 * p.sj[2];
+    lin = qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2];
+    srcn += (long long)n * p.src_nstride;
   }
   const int acol = tid % BM;
-  const int arow0 = tid / BM;
+  const int arow0 = BM % 64 == 0 ? uniform(tid / BM) : tid / BM;
   const bool m_ok = (m0 + acol) < p.M;
+  const int acol_safe = m_ok ? m0 + acol : 0;
+  const int klast = ph.k_count - 1;
 
   T ra[ALOADS], rb[BLOADS];
+  bool oka[ALOADS], okb[BLOADS];
 
+  // Every load is issued unconditionally from a clamped (always valid) address and
+  // the padding zeros are selected afterwards, so that the loads of a tile go out
+  // back to back instead of sitting behind one branch each.
   auto fetch = [&](int kt) {
     const int kbase = kt * BK;
 #pragma unroll
     for (int r = 0; r < ALOADS; ++r) {
       const int kk = arow0 + r * AROWS;
       const int kidx = kbase + kk;
-      T v = T(0);
-      if (kk < BK && kidx < ph.k_count && m_ok) v = A[(long long)arow[kidx] * p.M + m0 + acol];
-      ra[r] = v;
+      oka[r] = (kk < BK) & (kidx <= klast) & m_ok;
+      const int row = arow[min(kidx, klast)];
+      ra[r] = A[(long long)row * p.M + acol_safe];
     }
 #pragma unroll
     for (int r = 0; r < BLOADS; ++r) {
       const int kk = brow0 + r * BROWS;
       const int kidx = kbase + kk;
-      T v = T(0);
-      if (kk < BK && kidx < ph.k_count && pos_ok) {
-        const TabEntry e = tab[kidx];
-        const bool ok = (unsigned)(qb0 + e.d0) < (unsigned)p.Q[0] && (unsigned)(qb1 + e.d1) < (unsigned)p.Q[1] &&
-                        (unsigned)(qb2 + e.d2) < (unsigned)p.Q[2];
-        if (ok) v = srcn[lin + e.off];
-      }
-      rb[r] = v;
+      const TabEntry e = table_row(tab, min(kidx, klast));
+      const bool ok = (kk < BK) & (kidx <= klast) & pos_ok & ((unsigned)(qb0 + e.d0) < (unsigned)p.Q[0]) &
+                      ((unsigned)(qb1 + e.d1) < (unsigned)p.Q[1]) & ((unsigned)(qb2 + e.d2) < (unsigned)p.Q[2]);
+      okb[r] = ok;
+      rb[r] = srcn[ok ? lin + e.off : 0];
     }
   };
   auto stash = [&](int buf) {
 #pragma unroll
     for (int r = 0; r < ALOADS; ++r) {
       const int kk = arow0 + r * AROWS;
-      if (kk < BK) As[buf][kk][acol] = ra[r];
+      if (kk < BK) As[buf][kk][acol] = oka[r] ? ra[r] : T(0);
     }
 #pragma unroll
     for (int r = 0; r < BLOADS; ++r) {
       const int kk = brow0 + r * BROWS;
-      if (kk < BK) Bs[buf][kk][bcol] = rb[r];
+      if (kk < BK) Bs[buf][kk][bcol] = okb[r] ? rb[r] : T(0);
     }
   };
 
@@ -221,14 +240,15 @@ __global__ void __launch_bounds__(256) gather_gemm_kernel(const GemmParams p) {
   T *__restrict__ dst = static_cast<T *>(p.dst);
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
-    const long long pos = (long long)pos0 + wn0 + j * 16 + (lane & 15);
-    if (pos >= ph.npos) continue;
-    const int n = (int)(pos / jvol);
-    int r = (int)(pos - (long long)n * jvol);
-    const int j0 = r / j12;
-    r -= j0 * j12;
-    const int j1 = r / ph.J[2];
-    const int j2 = r - j1 * ph.J[2];
+    const int ipos = pos0 + wn0 + j * 16 + (lane & 15);
+    if (ipos >= ph.npos) continue;
+    const unsigned pos = (unsigned)ipos;
+    const unsigned n = ph.by_jvol.div(pos);
+    unsigned r = pos - n * (unsigned)jvol;
+    const int j0 = (int)ph.by_j12.div(r);
+    r -= (unsigned)j0 * (unsigned)j12;
+    const int j1 = (int)ph.by_j2.div(r);
+    const int j2 = (int)r - j1 * ph.J[2];
     T *out = dst + (long long)n * p.dst_nstride + (long long)(ph.o0[0] + j0 * p.oj[0]) * p.os[0] +
              (long long)(ph.o0[1] + j1 * p.oj[1]) * p.os[1] + (long long)(ph.o0[2] + j2 * p.oj[2]) * p.os[2];
 #pragma unroll
@@ -265,65 +285,66 @@ __global__ void __launch_bounds__(256) wgrad_kernel(const WgradParams p) {
   const int wn0 = (wave % WAVES_N) * WN;
   const int n0 = blockIdx.x * BN;  // first column (c, tap)
   const int m0 = blockIdx.y * BM;  // first filter
-  const long long kbeg = (long long)blockIdx.z * p.kchunk;
-  const long long kend = min(kbeg + p.kchunk, p.kpos);
+  const int kbeg = (int)blockIdx.z * p.kchunk;
+  const int kend = min(kbeg + p.kchunk, p.kpos);
 
   const T *__restrict__ grad = static_cast<const T *>(p.grad);
   const T *__restrict__ x = static_cast<const T *>(p.x);
   const int kcol = tid % BK;  // this thread's position inside the K tile
-  const int row0 = tid / BK;
+  const int row0 = BK % 64 == 0 ? uniform(tid / BK) : tid / BK;
   const int g12 = p.G[1] * p.G[2];
+  const int4v MG_CONSTANT *tab = as_constant(p.tab);
 
   T ra[ALOADS], rb[BLOADS];
+  bool oka[ALOADS], okb[BLOADS];
 
+  // Unconditional loads from clamped addresses, zeros selected afterwards (see the
+  // gather-GEMM above).  A thread keeps one position of the K tile and walks the
+  // tile's rows, so the position is decoded once per tile.
   auto fetch = [&](int kt) {
-    const long long pos = kbeg + (long long)kt * BK + kcol;
-    const bool pos_ok = pos < kend;
-    int n = 0, gflat = 0, qb0 = 0, qb1 = 0, qb2 = 0, lin = 0;
-    if (pos_ok) {
-      n = (int)(pos / p.gvol);
-      gflat = (int)(pos - (long long)n * p.gvol);
-      const int g0 = gflat / g12;
-      const int r = gflat - g0 * g12;
-      const int g1 = r / p.G[2];
-      const int g2 = r - g1 * p.G[2];
-      qb0 = g0 * p.sj[0];
-      qb1 = g1 * p.sj[1];
-      qb2 = g2 * p.sj[2];
-      lin = qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2];
-    }
+    const int ipos = kbeg + kt * BK + kcol;
+    const bool pos_ok = ipos < kend;
+    const unsigned pos = pos_ok ? (unsigned)ipos : (unsigned)kbeg;
+    const unsigned n = p.by_gvol.div(pos);
+    const unsigned gflat = pos - n * (unsigned)p.gvol;
+    const unsigned g0 = p.by_g12.div(gflat);
+    const unsigned r12 = gflat - g0 * (unsigned)g12;
+    const unsigned g1 = p.by_g2.div(r12);
+    const unsigned g2 = r12 - g1 * (unsigned)p.G[2];
+    const int qb0 = (int)g0 * p.sj[0];
+    const int qb1 = (int)g1 * p.sj[1];
+    const int qb2 = (int)g2 * p.sj[2];
+    const int lin = qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2];
     const T *gn = grad + (long long)n * p.g_nstride + gflat;
     const T *xn = x + (long long)n * p.x_nstride;
 #pragma unroll
     for (int r = 0; r < ALOADS; ++r) {
       const int row = row0 + r * ROWS;
-      T v = T(0);
-      if (row < BM && pos_ok && m0 + row < p.F) v = gn[(long long)(m0 + row) * p.gvol];
-      ra[r] = v;
+      const int f = m0 + row;
+      oka[r] = (row < BM) & pos_ok & (f < p.F);
+      ra[r] = gn[(long long)min(f, p.F - 1) * p.gvol];
     }
 #pragma unroll
     for (int r = 0; r < BLOADS; ++r) {
       const int row = row0 + r * ROWS;
-      T v = T(0);
-      if (row < BN && pos_ok && n0 + row < p.CT) {
-        const TabEntry e = p.tab[n0 + row];
-        const bool ok = (unsigned)(qb0 + e.d0) < (unsigned)p.Q[0] && (unsigned)(qb1 + e.d1) < (unsigned)p.Q[1] &&
-                        (unsigned)(qb2 + e.d2) < (unsigned)p.Q[2];
-        if (ok) v = xn[lin + e.off];
-      }
-      rb[r] = v;
+      const int col = n0 + row;
+      const TabEntry e = table_row(tab, min(col, p.CT - 1));
+      const bool ok = (row < BN) & pos_ok & (col < p.CT) & ((unsigned)(qb0 + e.d0) < (unsigned)p.Q[0]) &
+                      ((unsigned)(qb1 + e.d1) < (unsigned)p.Q[1]) & ((unsigned)(qb2 + e.d2) < (unsigned)p.Q[2]);
+      okb[r] = ok;
+      rb[r] = xn[ok ? lin + e.off : 0];
     }
   };
   auto stash = [&](int buf) {
 #pragma unroll
     for (int r = 0; r < ALOADS; ++r) {
       const int row = row0 + r * ROWS;
-      if (row < BM) As[buf][row][kcol] = ra[r];
+      if (row < BM) As[buf][row][kcol] = oka[r] ? ra[r] : T(0);
     }
 #pragma unroll
     for (int r = 0; r < BLOADS; ++r) {
       const int row = row0 + r * ROWS;
-      if (row < BN) Bs[buf][row][kcol] = rb[r];
+      if (row < BN) Bs[buf][row][kcol] = okb[r] ? rb[r] : T(0);
     }
   };
 
@@ -333,7 +354,7 @@ __global__ void __launch_bounds__(256) wgrad_kernel(const WgradParams p) {
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = typename Mma<T>::Acc{0, 0, 0, 0};
 
-  const int ktiles = kend > kbeg ? (int)((kend - kbeg + BK - 1) / BK) : 0;
+  const int ktiles = kend > kbeg ? (kend - kbeg + BK - 1) / BK : 0;
   int buf = 0;
   if (ktiles > 0) {
     fetch(0);
@@ -411,7 +432,7 @@ struct Plan {
   int bm = 0, bn = 0;
   // wgrad
   int splits = 1;
-  long long kchunk = 0;
+  int kchunk = 0;
 };
 
 std::map<std::string, Plan> &plans() {
@@ -479,6 +500,12 @@ int pick_bm(int M) {
   return 16;
 }
 
+void set_divisors(Phase &ph) {
+  ph.by_jvol = make_fastdiv((unsigned)(ph.J[0] * ph.J[1] * ph.J[2]));
+  ph.by_j12 = make_fastdiv((unsigned)(ph.J[1] * ph.J[2]));
+  ph.by_j2 = make_fastdiv((unsigned)ph.J[2]);
+}
+
 void fwd_table(const Geometry &g, std::vector<TabEntry> &tab) {
   // row (c, t0, t1, t2) in the filter's own row-major order
   const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
@@ -536,7 +563,8 @@ int build_fwd_plan(const Geometry &g, Plan &pl) {
   ph.k_begin = 0;
   ph.k_count = (int)tab.size();
   ph.blk_begin = 0;
-  ph.npos = (long long)g.N * g.gvol;
+  ph.npos = (int)((long long)g.N * g.gvol);
+  set_divisors(ph);
   pl.pos_blocks = (int)ceil_div(ph.npos, pl.bn);
   return upload_plan(pl, tab, arow, std::vector<Phase>{ph});
 }
@@ -587,7 +615,8 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
                 arow.push_back((int)(f * g.wvol) + (taps[0][a] * g.W[1] + taps[1][b]) * g.W[2] + taps[2][c]);
               }
         ph.k_count = (int)tab.size() - ph.k_begin;
-        ph.npos = (long long)g.N * ph.J[0] * ph.J[1] * ph.J[2];
+        ph.npos = (int)((long long)g.N * ph.J[0] * ph.J[1] * ph.J[2]);
+        set_divisors(ph);
         ph.blk_begin = blk;
         blk += (int)ceil_div(ph.npos, pl.bn);
         phases.push_back(ph);
@@ -614,7 +643,7 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
   if (splits < 1) splits = 1;
   if (splits > 1024) splits = 1024;
   const long long tiles_per_split = ceil_div(ktiles, splits);
-  pl.kchunk = tiles_per_split * bk;
+  pl.kchunk = (int)(tiles_per_split * bk);
   pl.splits = (int)ceil_div(kpos, pl.kchunk);
   return upload_plan(pl, tab, std::vector<int>(), std::vector<Phase>());
 }
@@ -754,9 +783,12 @@ int conv_wgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   wp.gvol = (int)g.gvol;
   wp.x_nstride = (long long)g.C * g.xvol;
   wp.g_nstride = (long long)g.F * g.gvol;
-  wp.kpos = (long long)g.N * g.gvol;
+  wp.kpos = (int)((long long)g.N * g.gvol);
   wp.kchunk = pl.kchunk;
   wp.splits = pl.splits;
+  wp.by_gvol = make_fastdiv((unsigned)g.gvol);
+  wp.by_g12 = make_fastdiv((unsigned)(g.G[1] * g.G[2]));
+  wp.by_g2 = make_fastdiv((unsigned)g.G[2]);
   {
     ScopedTiming timed(TAG_CONV_WGRAD);
     switch (pl.bm) {

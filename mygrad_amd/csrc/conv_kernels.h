@@ -6,6 +6,28 @@
 
 namespace mg {
 
+// Division of a non-negative n < 2^31 by a divisor fixed at plan time:
+// q = umulhi(n, mul) >> shr  (mul = ceil(2^(31+ceil_log2(d)) / d)); d == 1 is
+// special-cased because its multiplier does not fit 32 bits.
+struct FastDiv {
+  unsigned mul, shr, d, pad_;
+#ifdef __HIPCC__
+  __device__ __forceinline__ unsigned div(unsigned n) const { return d == 1u ? n : __umulhi(n, mul) >> shr; }
+#endif
+};
+
+inline FastDiv make_fastdiv(unsigned d) {
+  FastDiv f{0u, 0u, d, 0u};
+  if (d > 1u) {
+    unsigned lg = 0;
+    while ((1ull << lg) < d) ++lg;  // ceil(log2(d))
+    const unsigned p = 31u + lg;
+    f.mul = (unsigned)(((1ull << p) + d - 1ull) / d);
+    f.shr = p - 32u;
+  }
+  return f;
+}
+
 // One row of the contraction table.  For the forward pass a row is one (c, tap);
 // for the data gradient one (f, tap) of a stride phase.  `off` is the element
 // offset that the row adds to a position's base offset inside one batch item of
@@ -25,8 +47,8 @@ struct Phase {
   int o0[3];
   int k_begin, k_count;  // rows [k_begin, k_begin + k_count) of the table
   int blk_begin;         // first block (along positions) that works on this phase
-  int pad_;
-  long long npos;        // N * J0 * J1 * J2
+  int npos;              // N * J0 * J1 * J2
+  FastDiv by_jvol, by_j12, by_j2;  // divisions that turn a position into (n, j0, j1, j2)
 };
 
 // Gather-GEMM:  dst[n, m, pos] = sum_k A[arow[k]][m] * src[n, row k, pos]
@@ -59,9 +81,10 @@ struct WgradParams {
   int G[3], Q[3], sj[3], qs[3];
   int gvol;
   long long x_nstride, g_nstride;
-  long long kpos;    // N * gvol, the length of the sum
-  long long kchunk;  // positions per split (multiple of the K tile)
+  int kpos;    // N * gvol, the length of the sum
+  int kchunk;  // positions per split (multiple of the K tile)
   int splits;
+  FastDiv by_gvol, by_g12, by_g2;  // divisions that turn a position into (n, g0, g1, g2)
 };
 
 }  // namespace mg
