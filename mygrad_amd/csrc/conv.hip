@@ -70,8 +70,10 @@ struct Mma<double> {
 
 // ------------------------------------------------------------------------------------------
 // filter packing: the GEMMs want the filter operand with M contiguous
-//   mode 0 (forward): Ap[(c*Wvol + t)][f] = w[f][c][t]
-//   mode 1 (dgrad)  : Ap[(f*Wvol + t)][c] = w[f][c][t]
+//   mode 0 (forward)            : Ap[(c*Wvol + t)][f] = w[f][c][t]
+//   mode 1 (dgrad)              : Ap[(f*Wvol + t)][c] = w[f][c][t]
+//   mode 2 (forward, tap-major) : Ap[(t*C + c)][f]    = w[f][c][t]
+//   mode 3 (dgrad, tap-major)   : Ap[(t*F + f)][c]    = w[f][c][t]
 // ------------------------------------------------------------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(256) pack_filters_kernel(const T *__restrict__ w, T *__restrict__ ap, int F, int C,
@@ -79,21 +81,28 @@ __global__ void __launch_bounds__(256) pack_filters_kernel(const T *__restrict__
   const int total = F * C * wvol;
   for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
     // idx enumerates the packed layout so that stores are coalesced
-    int m, f, c, t;
-    if (mode == 0) {
-      m = F;
+    int f, c, t;
+    if (mode == 0 || mode == 2) {
       f = idx % F;
       const int row = idx / F;
-      t = row % wvol;
-      c = row / wvol;
+      if (mode == 0) {
+        t = row % wvol;
+        c = row / wvol;
+      } else {
+        c = row % C;
+        t = row / C;
+      }
     } else {
-      m = C;
       c = idx % C;
       const int row = idx / C;
-      t = row % wvol;
-      f = row / wvol;
+      if (mode == 1) {
+        t = row % wvol;
+        f = row / wvol;
+      } else {
+        f = row % F;
+        t = row / F;
+      }
     }
-    (void)m;
     ap[idx] = w[((long long)f * C + c) * wvol + t];
   }
 }
@@ -408,6 +417,12 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const T *__restrict_
   dw[i] = s;
 }
 
+}  // namespace mg
+
+#include "conv_tap_kernels.h"
+
+namespace mg {
+
 // ------------------------------------------------------------------------------------------
 // host side: descriptor checks, cached plans (tables live in device memory), launches
 // ------------------------------------------------------------------------------------------
@@ -422,14 +437,24 @@ struct Geometry {
   long long xvol, wvol, gvol;
 };
 
+// K tile of the gather-GEMMs (positions x filters-or-channels x BK).
+int gemm_bk(int dtype) { return dtype == MG_F64 ? 8 : 16; }
+// K tile of the filter gradient (positions).
+int wgrad_bk(int dtype) { return dtype == MG_F64 ? 32 : 64; }
+
 struct Plan {
-  void *blob = nullptr;  // one device allocation: [TabEntry table][arow][phases]
+  void *blob = nullptr;  // one device allocation holding every table below
   TabEntry *tab = nullptr;
   int *arow = nullptr;
   Phase *phases = nullptr;
+  KTile *ktiles = nullptr;
+  WGroup *groups = nullptr;
+  void *zeros = nullptr;
   int nphases = 0;
-  int pos_blocks = 0;  // grid.x for the gather-GEMM
+  int pos_blocks = 0;  // grid.x of the gather-GEMM
   int bm = 0, bn = 0;
+  bool tap_major = false;  // which kernel family the tables are for
+  bool single_dense_phase = false;  // positions enumerate the destination tensor in order
   // wgrad
   int splits = 1;
   int kchunk = 0;
@@ -448,7 +473,7 @@ int check_desc(const mg_conv_desc *d, Geometry *g) {
   if (d->N < 1 || d->C < 1 || d->F < 1)
     return fail(MG_ERR_BAD_ARG, "N=%lld C=%lld F=%lld must be positive", (long long)d->N, (long long)d->C,
                 (long long)d->F);
-  const long long lim = (1ll << 31) - 1;
+  const long long lim = (1ll << 31) - 4096;
   long long xvol = 1, wvol = 1, gvol = 1;
   for (int k = 0; k < 3; ++k) {
     if (d->X[k] < 1 || d->W[k] < 1 || d->G[k] < 1 || d->stride[k] < 1 || d->dil[k] < 1 || d->pad[k] < 0)
@@ -506,8 +531,56 @@ void set_divisors(Phase &ph) {
   ph.by_j2 = make_fastdiv((unsigned)ph.J[2]);
 }
 
+struct Tables {
+  std::vector<TabEntry> tab;
+  std::vector<int> arow;
+  std::vector<Phase> phases;
+  std::vector<KTile> ktiles;
+  std::vector<WGroup> groups;
+};
+
+template <typename V>
+size_t padded_bytes(const V &v) {
+  return (v.size() * sizeof(typename V::value_type) + 255) & ~size_t(255);
+}
+
+int upload_plan(Plan &pl, const Tables &t) {
+  const size_t zero_b = 256;
+  const size_t off_tab = zero_b;
+  const size_t off_arow = off_tab + padded_bytes(t.tab);
+  const size_t off_ph = off_arow + padded_bytes(t.arow);
+  const size_t off_kt = off_ph + padded_bytes(t.phases);
+  const size_t off_gr = off_kt + padded_bytes(t.ktiles);
+  const size_t total = off_gr + padded_bytes(t.groups) + 256;
+  std::vector<char> host(total, 0);
+  auto put = [&](size_t off, const void *src, size_t n) {
+    if (n) memcpy(host.data() + off, src, n);
+  };
+  put(off_tab, t.tab.data(), t.tab.size() * sizeof(TabEntry));
+  put(off_arow, t.arow.data(), t.arow.size() * sizeof(int));
+  put(off_ph, t.phases.data(), t.phases.size() * sizeof(Phase));
+  put(off_kt, t.ktiles.data(), t.ktiles.size() * sizeof(KTile));
+  put(off_gr, t.groups.data(), t.groups.size() * sizeof(WGroup));
+  MG_HIP(hipMalloc(&pl.blob, host.size()));
+  hipError_t err = hipMemcpy(pl.blob, host.data(), host.size(), hipMemcpyHostToDevice);
+  if (err != hipSuccess) {
+    (void)hipFree(pl.blob);
+    pl.blob = nullptr;
+    return hip_fail(err, "hipMemcpy(plan tables)", __FILE__, __LINE__);
+  }
+  char *base = static_cast<char *>(pl.blob);
+  pl.zeros = base;  // the first 256 bytes stay zero: target of padding loads
+  pl.tab = reinterpret_cast<TabEntry *>(base + off_tab);
+  pl.arow = reinterpret_cast<int *>(base + off_arow);
+  pl.phases = reinterpret_cast<Phase *>(base + off_ph);
+  pl.ktiles = reinterpret_cast<KTile *>(base + off_kt);
+  pl.groups = reinterpret_cast<WGroup *>(base + off_gr);
+  pl.nphases = (int)t.phases.size();
+  return MG_OK;
+}
+
+// rows (c, t0, t1, t2) in the filter's own row-major order
 void fwd_table(const Geometry &g, std::vector<TabEntry> &tab) {
-  // row (c, t0, t1, t2) in the filter's own row-major order
   const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
   tab.clear();
   tab.reserve((size_t)g.C * g.wvol);
@@ -524,57 +597,57 @@ void fwd_table(const Geometry &g, std::vector<TabEntry> &tab) {
         }
 }
 
-int upload_plan(Plan &pl, const std::vector<TabEntry> &tab, const std::vector<int> &arow,
-                const std::vector<Phase> &phases) {
-  const size_t tab_b = (tab.size() * sizeof(TabEntry) + 255) & ~size_t(255);
-  const size_t arow_b = (arow.size() * sizeof(int) + 255) & ~size_t(255);
-  const size_t ph_b = (phases.size() * sizeof(Phase) + 255) & ~size_t(255);
-  std::vector<char> host(tab_b + arow_b + ph_b + 256, 0);
-  if (!tab.empty()) memcpy(host.data(), tab.data(), tab.size() * sizeof(TabEntry));
-  if (!arow.empty()) memcpy(host.data() + tab_b, arow.data(), arow.size() * sizeof(int));
-  if (!phases.empty()) memcpy(host.data() + tab_b + arow_b, phases.data(), phases.size() * sizeof(Phase));
-  MG_HIP(hipMalloc(&pl.blob, host.size()));
-  hipError_t err = hipMemcpy(pl.blob, host.data(), host.size(), hipMemcpyHostToDevice);
-  if (err != hipSuccess) {
-    (void)hipFree(pl.blob);
-    pl.blob = nullptr;
-    return hip_fail(err, "hipMemcpy(plan tables)", __FILE__, __LINE__);
-  }
-  char *base = static_cast<char *>(pl.blob);
-  pl.tab = reinterpret_cast<TabEntry *>(base);
-  pl.arow = reinterpret_cast<int *>(base + tab_b);
-  pl.phases = reinterpret_cast<Phase *>(base + tab_b + arow_b);
-  pl.nphases = (int)phases.size();
-  return MG_OK;
-}
-
 int build_fwd_plan(const Geometry &g, Plan &pl) {
-  std::vector<TabEntry> tab;
-  fwd_table(g, tab);
-  std::vector<int> arow(tab.size());
-  for (size_t i = 0; i < arow.size(); ++i) arow[i] = (int)i;
+  Tables t;
+  const int bk = gemm_bk(g.dtype);
   pl.bm = pick_bm(g.F);
   pl.bn = pl.bm == 128 ? 128 : 256;
+  pl.tap_major = g.C % bk == 0;
+  pl.single_dense_phase = true;
   Phase ph{};
   for (int k = 0; k < 3; ++k) {
     ph.J[k] = g.G[k];
     ph.o0[k] = 0;
   }
   ph.k_begin = 0;
-  ph.k_count = (int)tab.size();
   ph.blk_begin = 0;
   ph.npos = (int)((long long)g.N * g.gvol);
   set_divisors(ph);
+  if (pl.tap_major) {
+    const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
+    for (int t0 = 0; t0 < g.W[0]; ++t0)
+      for (int t1 = 0; t1 < g.W[1]; ++t1)
+        for (int t2 = 0; t2 < g.W[2]; ++t2) {
+          const int tflat = (t0 * g.W[1] + t1) * g.W[2] + t2;
+          for (int c0 = 0; c0 < g.C; c0 += bk) {
+            KTile e{};
+            e.d0 = t0 * g.D[0] - g.P[0];
+            e.d1 = t1 * g.D[1] - g.P[1];
+            e.d2 = t2 * g.D[2] - g.P[2];
+            e.a_row0 = tflat * g.C + c0;
+            e.coff = (int)(c0 * g.xvol) + e.d0 * qs[0] + e.d1 * qs[1] + e.d2 * qs[2];
+            t.ktiles.push_back(e);
+          }
+        }
+    ph.k_count = (int)t.ktiles.size();
+  } else {
+    fwd_table(g, t.tab);
+    t.arow.resize(t.tab.size());
+    for (size_t i = 0; i < t.arow.size(); ++i) t.arow[i] = (int)i;
+    ph.k_count = (int)t.tab.size();
+  }
+  t.phases.push_back(ph);
   pl.pos_blocks = (int)ceil_div(ph.npos, pl.bn);
-  return upload_plan(pl, tab, arow, std::vector<Phase>{ph});
+  return upload_plan(pl, t);
 }
 
 int build_dgrad_plan(const Geometry &g, Plan &pl) {
+  Tables t;
+  const int bk = gemm_bk(g.dtype);
   pl.bm = pick_bm(g.C);
   pl.bn = pl.bm == 128 ? 128 : 256;
-  std::vector<TabEntry> tab;
-  std::vector<int> arow;
-  std::vector<Phase> phases;
+  pl.tap_major = g.F % bk == 0;
+  pl.single_dense_phase = g.S[0] == 1 && g.S[1] == 1 && g.S[2] == 1;
   const int gs[3] = {g.G[1] * g.G[2], g.G[2], 1};
   int blk = 0;
   long long nphase = (long long)g.S[0] * g.S[1] * g.S[2];
@@ -594,45 +667,64 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
           if (ph.J[k] == 0) empty = true;
           // taps that can reach them: t*dil % stride == rho; the window index is then
           // g = j + (i0 + pad - t*dil) / stride  (exact division)
-          for (int t = 0; t < g.W[k]; ++t)
-            if ((t * g.D[k]) % g.S[k] == rho[k]) {
-              taps[k].push_back(t);
-              offs[k].push_back((i0 + g.P[k] - t * g.D[k]) / g.S[k]);
+          for (int tt = 0; tt < g.W[k]; ++tt)
+            if ((tt * g.D[k]) % g.S[k] == rho[k]) {
+              taps[k].push_back(tt);
+              offs[k].push_back((i0 + g.P[k] - tt * g.D[k]) / g.S[k]);
             }
         }
         if (empty) continue;
-        ph.k_begin = (int)tab.size();
-        for (int f = 0; f < g.F; ++f)
+        ph.k_begin = pl.tap_major ? (int)t.ktiles.size() : (int)t.tab.size();
+        if (pl.tap_major) {
           for (size_t a = 0; a < taps[0].size(); ++a)
             for (size_t b = 0; b < taps[1].size(); ++b)
               for (size_t c = 0; c < taps[2].size(); ++c) {
-                TabEntry e;
-                e.d0 = offs[0][a];
-                e.d1 = offs[1][b];
-                e.d2 = offs[2][c];
-                e.off = (int)(f * g.gvol) + e.d0 * gs[0] + e.d1 * gs[1] + e.d2 * gs[2];
-                tab.push_back(e);
-                arow.push_back((int)(f * g.wvol) + (taps[0][a] * g.W[1] + taps[1][b]) * g.W[2] + taps[2][c]);
+                const int tflat = (taps[0][a] * g.W[1] + taps[1][b]) * g.W[2] + taps[2][c];
+                for (int f0 = 0; f0 < g.F; f0 += bk) {
+                  KTile e{};
+                  e.d0 = offs[0][a];
+                  e.d1 = offs[1][b];
+                  e.d2 = offs[2][c];
+                  e.a_row0 = tflat * g.F + f0;
+                  e.coff = (int)(f0 * g.gvol) + e.d0 * gs[0] + e.d1 * gs[1] + e.d2 * gs[2];
+                  t.ktiles.push_back(e);
+                }
               }
-        ph.k_count = (int)tab.size() - ph.k_begin;
+          ph.k_count = (int)t.ktiles.size() - ph.k_begin;
+        } else {
+          for (int f = 0; f < g.F; ++f)
+            for (size_t a = 0; a < taps[0].size(); ++a)
+              for (size_t b = 0; b < taps[1].size(); ++b)
+                for (size_t c = 0; c < taps[2].size(); ++c) {
+                  TabEntry e;
+                  e.d0 = offs[0][a];
+                  e.d1 = offs[1][b];
+                  e.d2 = offs[2][c];
+                  e.off = (int)(f * g.gvol) + e.d0 * gs[0] + e.d1 * gs[1] + e.d2 * gs[2];
+                  t.tab.push_back(e);
+                  t.arow.push_back((int)(f * g.wvol) + (taps[0][a] * g.W[1] + taps[1][b]) * g.W[2] + taps[2][c]);
+                }
+          ph.k_count = (int)t.tab.size() - ph.k_begin;
+        }
         ph.npos = (int)((long long)g.N * ph.J[0] * ph.J[1] * ph.J[2]);
         set_divisors(ph);
         ph.blk_begin = blk;
         blk += (int)ceil_div(ph.npos, pl.bn);
-        phases.push_back(ph);
+        t.phases.push_back(ph);
       }
   pl.pos_blocks = blk;
-  return upload_plan(pl, tab, arow, phases);
+  return upload_plan(pl, t);
 }
 
 int build_wgrad_plan(const Geometry &g, Plan &pl) {
-  std::vector<TabEntry> tab;
-  fwd_table(g, tab);
+  Tables t;
   pl.bm = g.F <= 16 ? 16 : (g.F <= 32 ? 32 : 64);
   pl.bn = 64;
-  const int bk = g.dtype == MG_F64 ? 32 : 64;
+  pl.tap_major = g.C % 16 == 0 && g.F % pl.bm == 0;
+  const int bk = wgrad_bk(g.dtype);
   const long long ct = (long long)g.C * g.wvol;
-  const long long tiles = ceil_div(g.F, pl.bm) * ceil_div(ct, pl.bn);
+  const long long col_tiles = ceil_div(ct, pl.bn);
+  const long long tiles = ceil_div(g.F, pl.bm) * col_tiles;
   const long long kpos = (long long)g.N * g.gvol;
   const long long ktiles = ceil_div(kpos, bk);
   // aim at about three blocks per compute unit, at least 8 K tiles per block
@@ -645,7 +737,27 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
   const long long tiles_per_split = ceil_div(ktiles, splits);
   pl.kchunk = (int)(tiles_per_split * bk);
   pl.splits = (int)ceil_div(kpos, pl.kchunk);
-  return upload_plan(pl, tab, std::vector<int>(), std::vector<Phase>());
+  if (pl.tap_major) {
+    const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
+    const long long ngroups = col_tiles * (pl.bn / 16);
+    for (long long gi = 0; gi < ngroups; ++gi) {
+      WGroup e{};
+      const long long col = gi * 16;  // tap-major column t*C + c
+      if (col < ct) {
+        const int tflat = (int)(col / g.C), c0 = (int)(col % g.C);
+        const int t2 = tflat % g.W[2], t1 = (tflat / g.W[2]) % g.W[1], t0 = tflat / (g.W[2] * g.W[1]);
+        e.d0 = t0 * g.D[0] - g.P[0];
+        e.d1 = t1 * g.D[1] - g.P[1];
+        e.d2 = t2 * g.D[2] - g.P[2];
+        e.coff = (int)(c0 * g.xvol) + e.d0 * qs[0] + e.d1 * qs[1] + e.d2 * qs[2];
+        e.valid = 1;
+      }
+      t.groups.push_back(e);
+    }
+  } else {
+    fwd_table(g, t.tab);
+  }
+  return upload_plan(pl, t);
 }
 
 int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
@@ -653,7 +765,11 @@ int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
   key.push_back((char)op);
   auto it = plans().find(key);
   if (it == plans().end()) {
-    if (plans().size() >= 256) release_conv_plans();  // crude bound on cached tables
+    if (plans().size() >= 256) {
+      // crude bound on cached tables; kernels in flight may still read the old ones
+      MG_HIP(hipStreamSynchronize(runtime().stream));
+      release_conv_plans();
+    }
     Plan pl;
     int rc = op == OP_FWD ? build_fwd_plan(g, pl) : op == OP_DGRAD ? build_dgrad_plan(g, pl) : build_wgrad_plan(g, pl);
     if (rc) return rc;
@@ -664,21 +780,35 @@ int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
 }
 
 template <typename T, int BM, int BN, int BK, int WM, int WN>
-void launch_gemm(const GemmParams &gp, int pos_blocks, hipStream_t s) {
+void launch_gemm(const GemmParams &gp, int pos_blocks, bool tap_major, hipStream_t s) {
   const dim3 grid((unsigned)pos_blocks, (unsigned)ceil_div(gp.M, BM));
-  hipLaunchKernelGGL((gather_gemm_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, gp);
+  if (tap_major)
+    hipLaunchKernelGGL((tap_gemm_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, gp);
+  else
+    hipLaunchKernelGGL((gather_gemm_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, gp);
 }
 
 template <typename T>
-int run_gemm(const GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
+int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
   constexpr int BK = sizeof(T) == 8 ? 8 : 16;
   if (pl.pos_blocks <= 0) return MG_OK;
+  gp.tab = pl.tab;
+  gp.arow = pl.arow;
+  gp.phases = pl.phases;
+  gp.nphases = pl.nphases;
+  gp.ktiles = pl.ktiles;
+  gp.zeros = pl.zeros;
+  // a lane may store its 4 positions as one vector when they are adjacent in dst
+  // (positions run through dst in order, the per-sample volume is a multiple of 4,
+  // and every row starts 16-byte aligned)
+  gp.vec_store = pl.single_dense_phase && gp.dst_mstride % 4 == 0 && gp.dst_nstride % 4 == 0 &&
+                 reinterpret_cast<uintptr_t>(gp.dst) % 16 == 0;
   ScopedTiming timed(tag);
   switch (pl.bm) {
-    case 128: launch_gemm<T, 128, 128, BK, 64, 64>(gp, pl.pos_blocks, s); break;
-    case 64: launch_gemm<T, 64, 256, BK, 64, 64>(gp, pl.pos_blocks, s); break;
-    case 32: launch_gemm<T, 32, 256, BK, 32, 64>(gp, pl.pos_blocks, s); break;
-    default: launch_gemm<T, 16, 256, BK, 16, 64>(gp, pl.pos_blocks, s); break;
+    case 128: launch_gemm<T, 128, 128, BK, 64, 64>(gp, pl.pos_blocks, pl.tap_major, s); break;
+    case 64: launch_gemm<T, 64, 256, BK, 64, 64>(gp, pl.pos_blocks, pl.tap_major, s); break;
+    case 32: launch_gemm<T, 32, 256, BK, 32, 64>(gp, pl.pos_blocks, pl.tap_major, s); break;
+    default: launch_gemm<T, 16, 256, BK, 16, 64>(gp, pl.pos_blocks, pl.tap_major, s); break;
   }
   MG_HIP(hipGetLastError());
   return MG_OK;
@@ -699,15 +829,11 @@ int pack_filters(const Geometry &g, const void *w, int mode, void **packed) {
 template <typename T>
 int conv_fwd_impl(const Geometry &g, const Plan &pl, const void *x, const void *w, void *out) {
   void *packed = nullptr;
-  if (int rc = pack_filters<T>(g, w, 0, &packed)) return rc;
+  if (int rc = pack_filters<T>(g, w, pl.tap_major ? 2 : 0, &packed)) return rc;
   GemmParams gp{};
   gp.A = packed;
   gp.src = x;
   gp.dst = out;
-  gp.tab = pl.tab;
-  gp.arow = pl.arow;
-  gp.phases = pl.phases;
-  gp.nphases = pl.nphases;
   gp.M = g.F;
   const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
   const int os[3] = {g.G[1] * g.G[2], g.G[2], 1};
@@ -719,6 +845,7 @@ int conv_fwd_impl(const Geometry &g, const Plan &pl, const void *x, const void *
     gp.os[k] = os[k];
   }
   gp.dst_mstride = (int)g.gvol;
+  gp.src_cstride = (int)g.xvol;
   gp.src_nstride = (long long)g.C * g.xvol;
   gp.dst_nstride = (long long)g.F * g.gvol;
   return run_gemm<T>(gp, pl, TAG_CONV_FWD, runtime().stream);
@@ -727,15 +854,11 @@ int conv_fwd_impl(const Geometry &g, const Plan &pl, const void *x, const void *
 template <typename T>
 int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const void *w, void *dx) {
   void *packed = nullptr;
-  if (int rc = pack_filters<T>(g, w, 1, &packed)) return rc;
+  if (int rc = pack_filters<T>(g, w, pl.tap_major ? 3 : 1, &packed)) return rc;
   GemmParams gp{};
   gp.A = packed;
   gp.src = grad;
   gp.dst = dx;
-  gp.tab = pl.tab;
-  gp.arow = pl.arow;
-  gp.phases = pl.phases;
-  gp.nphases = pl.nphases;
   gp.M = g.C;
   const int qs[3] = {g.G[1] * g.G[2], g.G[2], 1};
   const int os[3] = {g.X[1] * g.X[2], g.X[2], 1};
@@ -747,15 +870,19 @@ int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
     gp.os[k] = os[k];
   }
   gp.dst_mstride = (int)g.xvol;
+  gp.src_cstride = (int)g.gvol;
   gp.src_nstride = (long long)g.F * g.gvol;
   gp.dst_nstride = (long long)g.C * g.xvol;
   return run_gemm<T>(gp, pl, TAG_CONV_DGRAD, runtime().stream);
 }
 
 template <typename T, int BM, int BN, int BK, int WM, int WN>
-void launch_wgrad(const WgradParams &wp, hipStream_t s) {
+void launch_wgrad(const WgradParams &wp, bool tap_major, hipStream_t s) {
   const dim3 grid((unsigned)ceil_div(wp.CT, BN), (unsigned)ceil_div(wp.F, BM), (unsigned)wp.splits);
-  hipLaunchKernelGGL((wgrad_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, wp);
+  if (tap_major)
+    hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, wp);
+  else
+    hipLaunchKernelGGL((wgrad_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, wp);
 }
 
 template <typename T>
@@ -763,14 +890,19 @@ int conv_wgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   constexpr int BK = sizeof(T) == 8 ? 32 : 64;
   hipStream_t s = runtime().stream;
   const int ct = (int)(g.C * g.wvol);
+  // The tap-major kernel writes its columns in (tap, channel) order, so its result
+  // always goes through the reduction kernel, which also restores (channel, tap).
+  const bool staged = pl.splits > 1 || pl.tap_major;
   void *target = dw;
-  if (pl.splits > 1)
+  if (staged)
     if (int rc = workspace((size_t)pl.splits * g.F * ct * sizeof(T), &target)) return rc;
   WgradParams wp{};
   wp.grad = grad;
   wp.x = x;
   wp.out = target;
   wp.tab = pl.tab;
+  wp.groups = pl.groups;
+  wp.zeros = pl.zeros;
   wp.F = g.F;
   wp.CT = ct;
   const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
@@ -781,6 +913,7 @@ int conv_wgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
     wp.qs[k] = qs[k];
   }
   wp.gvol = (int)g.gvol;
+  wp.x_cstride = (int)g.xvol;
   wp.x_nstride = (long long)g.C * g.xvol;
   wp.g_nstride = (long long)g.F * g.gvol;
   wp.kpos = (int)((long long)g.N * g.gvol);
@@ -792,17 +925,21 @@ int conv_wgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   {
     ScopedTiming timed(TAG_CONV_WGRAD);
     switch (pl.bm) {
-      case 64: launch_wgrad<T, 64, 64, BK, 32, 32>(wp, s); break;
-      case 32: launch_wgrad<T, 32, 64, BK, 32, 16>(wp, s); break;
-      default: launch_wgrad<T, 16, 64, BK, 16, 16>(wp, s); break;
+      case 64: launch_wgrad<T, 64, 64, BK, 32, 32>(wp, pl.tap_major, s); break;
+      case 32: launch_wgrad<T, 32, 64, BK, 32, 16>(wp, pl.tap_major, s); break;
+      default: launch_wgrad<T, 16, 64, BK, 16, 16>(wp, pl.tap_major, s); break;
     }
   }
   MG_HIP(hipGetLastError());
-  if (pl.splits > 1) {
+  if (staged) {
     const int count = g.F * ct;
     ScopedTiming timed(TAG_WGRAD_REDUCE);
-    hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, s,
-                       static_cast<const T *>(target), static_cast<T *>(dw), count, pl.splits);
+    if (pl.tap_major)
+      hipLaunchKernelGGL(tap_reduce_kernel<T>, dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, s,
+                         static_cast<const T *>(target), static_cast<T *>(dw), g.F, g.C, (int)g.wvol, pl.splits);
+    else
+      hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, s,
+                         static_cast<const T *>(target), static_cast<T *>(dw), count, pl.splits);
     MG_HIP(hipGetLastError());
   }
   return MG_OK;

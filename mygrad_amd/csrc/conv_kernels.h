@@ -39,6 +39,26 @@ struct TabEntry {
   int d0, d1, d2;
 };
 
+// One K tile of the tap-major gather-GEMM: BK consecutive channels (forward) or
+// filters (data gradient) under one filter tap.  Rows a_row0.. of the packed
+// filter matrix multiply the gathered elements at `coff` + i * channel stride;
+// all of them share the tap's coordinate offsets d[k], hence one validity test.
+struct KTile {
+  int a_row0;
+  int coff;
+  int d0, d1, d2;
+  int pad0_, pad1_, pad2_;
+};
+
+// Sixteen consecutive columns of the tap-major filter-gradient matrix: one tap,
+// channels c0..c0+15.  `coff` = c0 * channel stride + the tap's element offset.
+struct WGroup {
+  int coff;
+  int d0, d1, d2;
+  int valid;
+  int pad0_, pad1_, pad2_;
+};
+
 // A stride phase of the data gradient (the forward pass has exactly one phase).
 // Positions of a phase are (n, j0, j1, j2), j_k in [0, J[k]); position j maps to
 // the destination coordinate o0[k] + j_k * oj[k].
@@ -68,6 +88,11 @@ struct GemmParams {
   int os[3];  // destination element strides of the spatial axes
   int dst_mstride;
   long long src_nstride, dst_nstride;
+  // tap-major kernels only
+  const KTile *ktiles;  // Phase::k_begin / k_count index this table
+  const void *zeros;    // a few zero elements in device memory: where padding loads point
+  int src_cstride;      // element stride between consecutive channels of the gathered tensor
+  int vec_store;        // positions are contiguous in dst: a lane may store its TN positions as one vector
 };
 
 // Filter gradient:  out[split][f][col] = sum over the split's positions (n, g) of
@@ -85,6 +110,10 @@ struct WgradParams {
   int kchunk;  // positions per split (multiple of the K tile)
   int splits;
   FastDiv by_gvol, by_g12, by_g2;  // divisions that turn a position into (n, g0, g1, g2)
+  // tap-major kernel only
+  const WGroup *groups;
+  const void *zeros;
+  int x_cstride;
 };
 
 }  // namespace mg

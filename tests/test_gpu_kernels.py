@@ -189,6 +189,44 @@ def test_conv_random_cases_vs_oracle(abi, dtype, m, big):
         done += 1
 
 
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("m", [1, 2, 3])
+def test_conv_channel_counts_that_take_the_tap_major_kernels(abi, dtype, m):
+    # channel / filter counts that are multiples of the K tile (8 or 16) select the
+    # tap-major kernels; mix them with counts that do not, strides, dilation, padding
+    rng = np.random.default_rng(500 + m)
+    tol = TOL[np.dtype(dtype)]
+    done = 0
+    while done < 14:
+        C = int(rng.choice([8, 16, 32, 48, 64]))
+        F = int(rng.choice([8, 16, 24, 32, 64, 80, 128, 144]))
+        N = int(rng.integers(1, 4))
+        taps = tuple(int(v) for v in rng.integers(1, 4, m))
+        dil = tuple(int(v) for v in rng.integers(1, 3, m))
+        stride = tuple(int(v) for v in rng.integers(1, 4, m))
+        pad = tuple(int(v) for v in rng.integers(0, 3, m))
+        grid = tuple(int(v) for v in rng.integers(1, [40, 14, 7][m - 1], m))
+        extra = tuple(int(v) for v in rng.integers(0, 2, m))
+        X = tuple(
+            (g - 1) * s + (t - 1) * d + 1 - 2 * p + (e if e < s else 0)
+            for g, s, t, d, p, e in zip(grid, stride, taps, dil, pad, extra)
+        )
+        if any(v < 1 for v in X):
+            continue
+        x_shape, w_shape = (N, C, *X), (F, C, *taps)
+        print("tap-major case", np.dtype(dtype).name, x_shape, w_shape, stride, pad, dil, flush=True)
+        x = rng.standard_normal(x_shape).astype(dtype)
+        w = rng.standard_normal(w_shape).astype(dtype)
+        want_out = direct.conv_forward(x, w, stride, pad, dil)
+        g = rng.standard_normal(want_out.shape).astype(dtype)
+        assert rel_err(abi.conv_fwd(x, w, stride, pad, dil), want_out) <= tol
+        assert rel_err(abi.conv_dgrad(g, x_shape, w, stride, pad, dil),
+                       direct.conv_backward_x(g, x_shape, w, stride, pad, dil)) <= tol
+        assert rel_err(abi.conv_wgrad(g, x, w_shape, stride, pad, dil),
+                       direct.conv_backward_w(g, x, w_shape, stride, pad, dil)) <= tol
+        done += 1
+
+
 def _check_conv_config(abi, seed, dtype, x_shape, w_shape, w_scale, s, p, d, np_oracle_batch):
     """Full-size check: against the definition-level C reference everywhere, and
     against the NumPy restatement of the reference on the leading batch items."""
