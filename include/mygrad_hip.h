@@ -87,7 +87,8 @@ int mg_host_alloc(void **hptr, size_t nbytes); /* pinned host memory (hipHostMal
 int mg_host_free(void *hptr);
 int mg_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes); /* stream-ordered, returns when src may be reused */
 int mg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes); /* returns when dst holds the data */
-int mg_memcpy_d2d(void *dst_dev, const void *src_dev, size_t nbytes);  /* stream-ordered */
+int mg_memcpy_d2d(void *dst_dev, const void *src_dev, size_t nbytes);  /* stream-ordered; a plain 16-byte-per-lane
+                                                                          copy kernel when everything is 16-byte aligned */
 int mg_memset_zero(void *dst_dev, size_t nbytes);                      /* stream-ordered fill kernel */
 int mg_sync(void);
 
@@ -102,7 +103,7 @@ int mg_event_destroy(void *event);
  * mg_timing_read() waits for the stream, returns up to `capacity` (tag, ms)
  * records in launch order, sets *count to the number recorded and starts over.
  * Tags: 1 conv forward, 2 conv dgrad, 3 conv wgrad, 4 wgrad split-K reduction,
- * 5 filter packing, 6 max-pool forward, 7 max-pool backward. */
+ * 5 filter packing, 6 max-pool forward, 7 max-pool backward, 8 device copy. */
 int mg_timing_enable(int on);
 int mg_timing_read(int32_t *tags, float *ms, int capacity, int *count);
 

@@ -208,6 +208,7 @@ KERNEL_TAGS = {
     5: "pack_filters",
     6: "maxpool_fwd",
     7: "maxpool_bwd",
+    8: "copy",
 }
 
 

@@ -49,6 +49,7 @@ enum KernelTag {
   TAG_PACK_FILTERS = 5,
   TAG_POOL_FWD = 6,
   TAG_POOL_BWD = 7,
+  TAG_COPY = 8,
 };
 void timing_begin(int tag);
 void timing_end();

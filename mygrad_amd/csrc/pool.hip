@@ -8,6 +8,8 @@
 //                +0.0 and carried in double.
 #include "internal.h"
 
+#include <algorithm>
+
 namespace mg {
 
 struct PoolParams {
@@ -95,6 +97,186 @@ __global__ void __launch_bounds__(256) maxpool_bwd_kernel(PoolParams p, const T 
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// LDS-tiled kernels
+//
+// A block stages one contiguous chunk of x in LDS with wide coalesced loads --
+// either a band of rows of one pooled volume plus the halo its windows need, or
+// several whole small volumes -- so that every element of x crosses HBM once.
+// Forward: each thread then reduces windows out of LDS.  Backward: the block first
+// records every window's first-occurrence argmax (as an LDS index), then each
+// thread owns input elements and walks the few windows that cover them in
+// ascending row-major order, adding grad where the window's argmax is the
+// element itself: a gather, so no atomics, and the sum order of np.add.at.
+// ------------------------------------------------------------------------------------------
+struct FastDivP {
+  unsigned mul, shr, d, pad_;
+  __device__ __forceinline__ unsigned div(unsigned n) const { return d == 1u ? n : __umulhi(n, mul) >> shr; }
+};
+
+static FastDivP make_fastdiv_p(unsigned d) {
+  FastDivP f{0u, 0u, d, 0u};
+  if (d > 1u) {
+    unsigned lg = 0;
+    while ((1ull << lg) < d) ++lg;
+    const unsigned p = 31u + lg;
+    f.mul = (unsigned)(((1ull << p) + d - 1ull) / d);
+    f.shr = p - 32u;
+  }
+  return f;
+}
+
+struct PoolTileParams {
+  int X[3], P[3], S[3], G[3];
+  int axis;     // first pooled axis with extent > 1: the one that is cut into bands
+  int inner_x;  // elements of x per unit of that axis
+  int inner_g;  // windows per unit of that axis
+  int band;     // forward: windows per band; backward: input rows owned per band
+  int bands;    // bands per volume (1 when a block takes whole volumes)
+  int volumes;  // whole volumes per block (1 when a volume is cut into bands)
+  int xvol, gvol;
+  long long lead;
+  FastDivP by_x12, by_x2, by_g12, by_g2, by_xvol, by_gvol;
+  FastDivP by_s[3];
+};
+
+template <typename T>
+__device__ __forceinline__ void stage_chunk(T *tile, const T *__restrict__ src, long long start, int len, int pad) {
+  // tile[pad + e] = src[start + e]; pad = start % VEC makes both sides 16-byte aligned together
+  constexpr int VEC = 16 / sizeof(T);
+  typedef T Vec __attribute__((ext_vector_type(VEC)));
+  const int head = min(len, (VEC - pad) % VEC);
+  for (int e = threadIdx.x; e < head; e += blockDim.x) tile[pad + e] = src[start + e];
+  const int body = (len - head) / VEC;
+  const Vec *vsrc = reinterpret_cast<const Vec *>(src + start + head);
+  Vec *vdst = reinterpret_cast<Vec *>(tile + pad + head);
+  for (int v = threadIdx.x; v < body; v += blockDim.x) vdst[v] = vsrc[v];
+  for (int e = head + body * VEC + threadIdx.x; e < len; e += blockDim.x) tile[pad + e] = src[start + e];
+}
+
+template <typename T, typename TD, bool BWD>
+__global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, const T *__restrict__ x,
+                                                           const T *__restrict__ grad, void *__restrict__ result,
+                                                           int tile_elems, int win_slots) {
+  // LDS: [x tile | argmax slot per window | grad of those windows]; win_slots is a multiple of 4
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  T *tile = reinterpret_cast<T *>(smem);
+  int *winner = reinterpret_cast<int *>(smem + (size_t)tile_elems * sizeof(T));
+  T *gtile = reinterpret_cast<T *>(smem + (size_t)tile_elems * sizeof(T) + (size_t)win_slots * sizeof(int));
+  constexpr int VEC = 16 / sizeof(T);
+
+  const long long blk = blockIdx.x;
+  const long long l0 = (blk / p.bands) * p.volumes;
+  const int band = (int)(blk % p.bands);
+  const int nvol = (int)min((long long)p.volumes, p.lead - l0);
+  const int a = p.axis;
+  const int XA = p.X[a], GA = p.G[a], PA = p.P[a], SA = p.S[a];
+
+  // rows of the band axis: [own_lo, own_hi) is what this block writes (backward),
+  // windows [g_lo, g_hi] along the axis are what it evaluates, rows [row_lo, row_hi)
+  // are what those windows (and the owned rows) read
+  int own_lo = 0, own_hi = XA, g_lo = 0, g_hi = GA - 1;
+  if (p.bands > 1) {
+    if (BWD) {
+      own_lo = band * p.band;
+      own_hi = min(own_lo + p.band, XA);
+      const int first = own_lo - PA + 1;
+      g_lo = first > 0 ? (first + SA - 1) / SA : 0;
+      g_hi = min(GA - 1, (own_hi - 1) / SA);
+    } else {
+      g_lo = band * p.band;
+      g_hi = min(g_lo + p.band, GA) - 1;
+    }
+  }
+  const bool any_window = g_lo <= g_hi;
+  int row_lo, row_hi;
+  if (BWD) {
+    row_lo = any_window ? min(own_lo, g_lo * SA) : own_lo;
+    row_hi = any_window ? max(own_hi, g_hi * SA + PA) : own_hi;
+  } else {
+    row_lo = g_lo * SA;
+    row_hi = g_hi * SA + PA;
+  }
+  const int first_flat = row_lo * p.inner_x;  // flat index (inside a volume) of tile element 0
+  const int chunk_len = p.bands > 1 ? (row_hi - row_lo) * p.inner_x : nvol * p.xvol;
+  const long long chunk_start = l0 * p.xvol + first_flat;
+  const int pad = (int)(chunk_start % VEC);
+  stage_chunk(tile, x, chunk_start, chunk_len, pad);
+  const int nwin = any_window ? (p.bands > 1 ? (g_hi - g_lo + 1) * p.inner_g : nvol * p.gvol) : 0;
+  const int win_base = p.bands > 1 ? g_lo * p.inner_g : 0;  // flat window index of winner[0]
+  int gpad = 0;
+  if (BWD) {
+    // the windows' gradients are one contiguous run of grad: keep them next to the tile
+    const long long gstart = l0 * p.gvol + win_base;
+    gpad = (int)(gstart % VEC);
+    stage_chunk(gtile, grad, gstart, nwin, gpad);
+  }
+  __syncthreads();
+  const int x12 = p.X[1] * p.X[2], g12 = p.G[1] * p.G[2];
+
+  // ---- one thread per window: the maximum (forward) or where it is (backward)
+  for (int w = threadIdx.x; w < nwin; w += blockDim.x) {
+    const unsigned vol = p.by_gvol.div((unsigned)w);  // 0 when a volume is cut into bands
+    const unsigned wf = (unsigned)w - vol * (unsigned)p.gvol + (unsigned)win_base;
+    const unsigned g0 = p.by_g12.div(wf);
+    const unsigned r = wf - g0 * (unsigned)g12;
+    const unsigned g1 = p.by_g2.div(r);
+    const unsigned g2 = r - g1 * (unsigned)p.G[2];
+    const int origin = (int)((g0 * p.S[0] * p.X[1] + g1 * p.S[1]) * p.X[2] + g2 * p.S[2]) - first_flat +
+                       (int)vol * p.xvol + pad;
+    T best = tile[origin];
+    int where = origin;
+    for (int a0 = 0; a0 < p.P[0]; ++a0)
+      for (int a1 = 0; a1 < p.P[1]; ++a1) {
+        const int rowoff = origin + (a0 * p.X[1] + a1) * p.X[2];
+        for (int a2 = 0; a2 < p.P[2]; ++a2) {
+          const T v = tile[rowoff + a2];
+          if (takes_over(v, best)) {
+            best = v;
+            where = rowoff + a2;
+          }
+        }
+      }
+    if (BWD)
+      winner[w] = where;
+    else
+      static_cast<T *>(result)[l0 * p.gvol + win_base + w] = best;
+  }
+  if (!BWD) return;
+  __syncthreads();
+
+  // ---- one thread per owned input element: gather from the windows that cover it
+  const int own_first = p.bands > 1 ? own_lo * p.inner_x : 0;
+  const int own_len = p.bands > 1 ? (own_hi - own_lo) * p.inner_x : nvol * p.xvol;
+  TD *dx = static_cast<TD *>(result);
+  for (int e = threadIdx.x; e < own_len; e += blockDim.x) {
+    const unsigned vol = p.by_xvol.div((unsigned)e);
+    const unsigned flat = (unsigned)e - vol * (unsigned)p.xvol + (unsigned)own_first;  // inside the volume
+    const unsigned i0 = p.by_x12.div(flat);
+    const unsigned r = flat - i0 * (unsigned)x12;
+    const unsigned i1 = p.by_x2.div(r);
+    const unsigned i2 = r - i1 * (unsigned)p.X[2];
+    const int i[3] = {(int)i0, (int)i1, (int)i2};
+    int lo[3], hi[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      const int first = i[k] - p.P[k] + 1;  // windows starting before this cannot cover i
+      lo[k] = first > 0 ? (int)p.by_s[k].div((unsigned)(first + p.S[k] - 1)) : 0;
+      hi[k] = min(p.G[k] - 1, (int)p.by_s[k].div((unsigned)i[k]));
+    }
+    const int me = (int)flat - first_flat + (int)vol * p.xvol + pad;  // my index in the tile
+    const int wshift = (int)vol * p.gvol - win_base;
+    double acc = 0.0;
+    for (int g0 = lo[0]; g0 <= hi[0]; ++g0)
+      for (int g1 = lo[1]; g1 <= hi[1]; ++g1)
+        for (int g2 = lo[2]; g2 <= hi[2]; ++g2) {
+          const int w = (g0 * p.G[1] + g1) * p.G[2] + g2 + wshift;
+          if (winner[w] == me) acc += (double)gtile[gpad + w];
+        }
+    dx[l0 * p.xvol + own_first + e] = (TD)acc;
+  }
+}
+
 static int check_pool_desc(const mg_pool_desc *d, PoolParams *p) {
   if (!d) return fail(MG_ERR_BAD_ARG, "pool descriptor is null");
   if (d->dtype != MG_F32 && d->dtype != MG_F64)
@@ -127,6 +309,117 @@ static int check_pool_desc(const mg_pool_desc *d, PoolParams *p) {
   return MG_OK;
 }
 
+// LDS the tiled kernels may use per block: small enough for several blocks per
+// compute unit (160 KB each), large enough for whole 2-D planes of common sizes.
+static const int kTileBudgetBytes = 48 * 1024;
+
+// Chooses bands / volumes per block; returns false when not even one row of the
+// band axis plus its halo fits (the thread-per-element kernels handle that).
+static bool plan_tiles(const PoolParams &pp, size_t elem, bool bwd, PoolTileParams *t, int *tile_elems,
+                       int *win_slots, size_t *lds_bytes, long long *blocks) {
+  PoolTileParams q{};
+  int a = 0;
+  while (a < 2 && pp.X[a] == 1) ++a;
+  for (int k = 0; k < 3; ++k) {
+    q.X[k] = pp.X[k];
+    q.P[k] = pp.P[k];
+    q.S[k] = pp.S[k];
+    q.G[k] = pp.G[k];
+  }
+  q.axis = a;
+  q.inner_x = 1;
+  q.inner_g = 1;
+  for (int k = a + 1; k < 3; ++k) {
+    q.inner_x *= pp.X[k];
+    q.inner_g *= pp.G[k];
+  }
+  q.xvol = (int)pp.xvol;
+  q.gvol = (int)pp.gvol;
+  q.lead = pp.lead;
+  const int vec = (int)(16 / elem);
+  // backward keeps, per window, an argmax slot (int) and its gradient (one element)
+  const long long per_win = bwd ? 4 + (long long)elem : 0;
+  const long long per_vol = (long long)pp.xvol * elem + pp.gvol * per_win;
+  long long tile = 0, nwin = 0;
+  if (per_vol + 64 <= kTileBudgetBytes) {
+    // whole volumes: as many as fit, but keep enough blocks to fill the device
+    long long fit = (kTileBudgetBytes - 64) / per_vol;
+    const long long want_blocks = 8ll * runtime().props.multiProcessorCount;
+    const long long spread = std::max<long long>(1, pp.lead / want_blocks);
+    q.volumes = (int)std::max<long long>(1, std::min<long long>(std::min(fit, spread), 64));
+    q.bands = 1;
+    q.band = bwd ? pp.X[a] : pp.G[a];
+    tile = (long long)q.volumes * pp.xvol;
+    nwin = (long long)q.volumes * pp.gvol;
+    *blocks = ceil_div(pp.lead, q.volumes);
+  } else {
+    q.volumes = 1;
+    const int P = pp.P[a], S = pp.S[a], XA = pp.X[a], GA = pp.G[a];
+    // rows of x and windows a band needs, exactly as the kernel derives them
+    auto need = [&](int band, long long *rows, long long *wins) {
+      *rows = 0;
+      *wins = 0;
+      const int count = (int)ceil_div(bwd ? XA : GA, band);
+      for (int b = 0; b < count; ++b) {
+        int g_lo, g_hi, row_lo, row_hi;
+        if (bwd) {
+          const int own_lo = b * band, own_hi = std::min(own_lo + band, XA);
+          const int first = own_lo - P + 1;
+          g_lo = first > 0 ? (first + S - 1) / S : 0;
+          g_hi = std::min(GA - 1, (own_hi - 1) / S);
+          const bool any = g_lo <= g_hi;
+          row_lo = any ? std::min(own_lo, g_lo * S) : own_lo;
+          row_hi = any ? std::max(own_hi, g_hi * S + P) : own_hi;
+          if (any) *wins = std::max<long long>(*wins, (long long)(g_hi - g_lo + 1) * q.inner_g);
+        } else {
+          g_lo = b * band;
+          g_hi = std::min(g_lo + band, GA) - 1;
+          row_lo = g_lo * S;
+          row_hi = g_hi * S + P;
+        }
+        *rows = std::max<long long>(*rows, row_hi - row_lo);
+      }
+    };
+    // largest band that fits; backward bands are whole multiples of the stride
+    // when possible so that neighbouring bands share as few windows as possible
+    const int limit = bwd ? XA : GA;
+    int best = 0;
+    long long best_rows = 0, best_wins = 0;
+    for (int band = limit; band >= 1; --band) {
+      if (bwd && band > S && band % S != 0) continue;
+      long long rows, wins;
+      need(band, &rows, &wins);
+      if (rows * q.inner_x * (long long)elem + wins * per_win + 64 <= kTileBudgetBytes) {
+        best = band;
+        best_rows = rows;
+        best_wins = wins;
+        break;
+      }
+      if (limit > 4096 && band > 64) band = std::max(64, band / 2) + 1;  // keep the search short
+    }
+    if (best == 0) return false;
+    q.band = best;
+    q.bands = (int)ceil_div(limit, best);
+    tile = best_rows * q.inner_x;
+    nwin = best_wins;
+    *blocks = pp.lead * q.bands;
+  }
+  if (*blocks >= (1ll << 31)) return false;
+  q.by_x12 = make_fastdiv_p((unsigned)(pp.X[1] * pp.X[2]));
+  q.by_x2 = make_fastdiv_p((unsigned)pp.X[2]);
+  q.by_g12 = make_fastdiv_p((unsigned)(pp.G[1] * pp.G[2]));
+  q.by_g2 = make_fastdiv_p((unsigned)pp.G[2]);
+  q.by_xvol = make_fastdiv_p((unsigned)pp.xvol);
+  q.by_gvol = make_fastdiv_p((unsigned)pp.gvol);
+  for (int k = 0; k < 3; ++k) q.by_s[k] = make_fastdiv_p((unsigned)pp.S[k]);
+  *tile_elems = (int)(tile + vec);  // room for the alignment shift
+  *tile_elems = (*tile_elems + 3) & ~3;
+  *win_slots = bwd ? (int)((nwin + 3) & ~3ll) : 0;
+  *lds_bytes = (size_t)*tile_elems * elem + (bwd ? (size_t)*win_slots * 4 + ((size_t)nwin + vec) * elem : 0);
+  *t = q;
+  return true;
+}
+
 static unsigned grid_for(long long total) {
   long long blocks = ceil_div(total, 256);
   const long long cap = (long long)runtime().props.multiProcessorCount * 32;
@@ -145,9 +438,23 @@ int mg_maxpool_fwd(const mg_pool_desc *desc, const void *x, void *out) {
   PoolParams p;
   if (int rc = check_pool_desc(desc, &p)) return rc;
   if (!x || !out) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_maxpool_fwd");
-  const unsigned grid = grid_for(p.lead * p.gvol);
   hipStream_t s = runtime().stream;
   ScopedTiming timed(TAG_POOL_FWD);
+  PoolTileParams tp;
+  int tile_elems = 0, win_slots = 0;
+  size_t lds = 0;
+  long long blocks = 0;
+  if (plan_tiles(p, desc->dtype == MG_F32 ? 4 : 8, false, &tp, &tile_elems, &win_slots, &lds, &blocks)) {
+    if (desc->dtype == MG_F32)
+      hipLaunchKernelGGL((maxpool_tile_kernel<float, float, false>), dim3((unsigned)blocks), dim3(256), lds, s, tp,
+                         (const float *)x, (const float *)nullptr, out, tile_elems, win_slots);
+    else
+      hipLaunchKernelGGL((maxpool_tile_kernel<double, double, false>), dim3((unsigned)blocks), dim3(256), lds, s, tp,
+                         (const double *)x, (const double *)nullptr, out, tile_elems, win_slots);
+    MG_HIP(hipGetLastError());
+    return MG_OK;
+  }
+  const unsigned grid = grid_for(p.lead * p.gvol);
   if (desc->dtype == MG_F32)
     hipLaunchKernelGGL(maxpool_fwd_kernel<float>, dim3(grid), dim3(256), 0, s, p, (const float *)x, (float *)out);
   else
@@ -162,9 +469,27 @@ int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, vo
   PoolParams p;
   if (int rc = check_pool_desc(desc, &p)) return rc;
   if (!x || !grad || !dx) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_maxpool_bwd");
-  const unsigned grid = grid_for(p.lead * p.xvol);
   hipStream_t s = runtime().stream;
   ScopedTiming timed(TAG_POOL_BWD);
+  PoolTileParams tp;
+  int tile_elems = 0, win_slots = 0;
+  size_t lds = 0;
+  long long blocks = 0;
+  if (plan_tiles(p, desc->dtype == MG_F32 ? 4 : 8, true, &tp, &tile_elems, &win_slots, &lds, &blocks)) {
+    const dim3 grid((unsigned)blocks), block(256);
+    if (desc->dtype == MG_F64)
+      hipLaunchKernelGGL((maxpool_tile_kernel<double, double, true>), grid, block, lds, s, tp, (const double *)x,
+                         (const double *)grad, dx, tile_elems, win_slots);
+    else if (desc->dx_dtype == MG_F64)
+      hipLaunchKernelGGL((maxpool_tile_kernel<float, double, true>), grid, block, lds, s, tp, (const float *)x,
+                         (const float *)grad, dx, tile_elems, win_slots);
+    else
+      hipLaunchKernelGGL((maxpool_tile_kernel<float, float, true>), grid, block, lds, s, tp, (const float *)x,
+                         (const float *)grad, dx, tile_elems, win_slots);
+    MG_HIP(hipGetLastError());
+    return MG_OK;
+  }
+  const unsigned grid = grid_for(p.lead * p.xvol);
   if (desc->dtype == MG_F64)
     hipLaunchKernelGGL((maxpool_bwd_kernel<double, double>), dim3(grid), dim3(256), 0, s, p, (const double *)x,
                        (const double *)grad, (double *)dx);
