@@ -138,6 +138,8 @@ struct PoolTileParams {
   long long lead;
   FastDivP by_x12, by_x2, by_g12, by_g2, by_xvol, by_gvol;
   FastDivP by_s[3];
+  int cand[3];  // windows that can cover one element, per axis: ceil(P/S)
+  int nranks;   // their product
 };
 
 template <typename T>
@@ -154,15 +156,18 @@ __device__ __forceinline__ void stage_chunk(T *tile, const T *__restrict__ src, 
   for (int e = head + body * VEC + threadIdx.x; e < len; e += blockDim.x) tile[pad + e] = src[start + e];
 }
 
-template <typename T, typename TD, bool BWD>
+template <typename T, typename TD, typename ACC, bool BWD>
 __global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, const T *__restrict__ x,
                                                            const T *__restrict__ grad, void *__restrict__ result,
-                                                           int tile_elems, int win_slots) {
-  // LDS: [x tile | argmax slot per window | grad of those windows]; win_slots is a multiple of 4
+                                                           int tile_elems, int win_slots, int acc_offset) {
+  // LDS: [x tile | one packed int per window | grad of those windows | accumulators];
+  // win_slots is a multiple of 4.  The accumulators alias the x tile (acc_offset == 0)
+  // when they are no wider than T: x is dead once every window knows its argmax.
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   T *tile = reinterpret_cast<T *>(smem);
   int *winner = reinterpret_cast<int *>(smem + (size_t)tile_elems * sizeof(T));
   T *gtile = reinterpret_cast<T *>(smem + (size_t)tile_elems * sizeof(T) + (size_t)win_slots * sizeof(int));
+  ACC *acc = reinterpret_cast<ACC *>(smem + acc_offset);
   constexpr int VEC = 16 / sizeof(T);
 
   const long long blk = blockIdx.x;
@@ -237,44 +242,54 @@ __global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, con
           }
         }
       }
-    if (BWD)
-      winner[w] = where;
-    else
+    if (BWD) {
+      // Rank of this window among the windows that cover its argmax element, in
+      // ascending row-major window order: per axis min(g, (P-1-a)/S) with a the
+      // argmax's offset inside the window.  Two windows with the same argmax
+      // element never share a rank, and adding ranks 0, 1, 2, ... in turn is the
+      // order np.add.at visits them in.
+      const unsigned off = (unsigned)(where - origin);
+      const unsigned a0 = p.by_x12.div(off);
+      const unsigned r12 = off - a0 * (unsigned)x12;
+      const unsigned a1 = p.by_x2.div(r12);
+      const unsigned a2 = r12 - a1 * (unsigned)p.X[2];
+      const unsigned k0 = min(g0, p.by_s[0].div((unsigned)p.P[0] - 1u - a0));
+      const unsigned k1 = min(g1, p.by_s[1].div((unsigned)p.P[1] - 1u - a1));
+      const unsigned k2 = min(g2, p.by_s[2].div((unsigned)p.P[2] - 1u - a2));
+      const unsigned rank = (k0 * (unsigned)p.cand[1] + k1) * (unsigned)p.cand[2] + k2;
+      winner[w] = where | (int)(rank << 20);
+    } else {
       static_cast<T *>(result)[l0 * p.gvol + win_base + w] = best;
+    }
   }
   if (!BWD) return;
   __syncthreads();
 
-  // ---- one thread per owned input element: gather from the windows that cover it
+  // ---- accumulators start at +0.0 (they may sit where the x tile was)
+  const int used = chunk_len + pad;
+  for (int e = threadIdx.x; e < used; e += blockDim.x) acc[e] = ACC(0);
+  __syncthreads();
+
+  // ---- one pass per rank: every window of that rank adds its gradient to its argmax
+  // element.  Within a pass no two windows touch the same element, so plain LDS
+  // read-modify-writes are race-free; across passes the barrier orders them.
+  for (int rank = 0; rank < p.nranks; ++rank) {
+    for (int w = threadIdx.x; w < nwin; w += blockDim.x) {
+      const int packed = winner[w];
+      if ((packed >> 20) == rank) {
+        const int e = packed & 0xFFFFF;
+        acc[e] = acc[e] + (ACC)gtile[gpad + w];
+      }
+    }
+    __syncthreads();
+  }
+
+  // ---- write the rows this block owns
   const int own_first = p.bands > 1 ? own_lo * p.inner_x : 0;
   const int own_len = p.bands > 1 ? (own_hi - own_lo) * p.inner_x : nvol * p.xvol;
-  TD *dx = static_cast<TD *>(result);
-  for (int e = threadIdx.x; e < own_len; e += blockDim.x) {
-    const unsigned vol = p.by_xvol.div((unsigned)e);
-    const unsigned flat = (unsigned)e - vol * (unsigned)p.xvol + (unsigned)own_first;  // inside the volume
-    const unsigned i0 = p.by_x12.div(flat);
-    const unsigned r = flat - i0 * (unsigned)x12;
-    const unsigned i1 = p.by_x2.div(r);
-    const unsigned i2 = r - i1 * (unsigned)p.X[2];
-    const int i[3] = {(int)i0, (int)i1, (int)i2};
-    int lo[3], hi[3];
-#pragma unroll
-    for (int k = 0; k < 3; ++k) {
-      const int first = i[k] - p.P[k] + 1;  // windows starting before this cannot cover i
-      lo[k] = first > 0 ? (int)p.by_s[k].div((unsigned)(first + p.S[k] - 1)) : 0;
-      hi[k] = min(p.G[k] - 1, (int)p.by_s[k].div((unsigned)i[k]));
-    }
-    const int me = (int)flat - first_flat + (int)vol * p.xvol + pad;  // my index in the tile
-    const int wshift = (int)vol * p.gvol - win_base;
-    double acc = 0.0;
-    for (int g0 = lo[0]; g0 <= hi[0]; ++g0)
-      for (int g1 = lo[1]; g1 <= hi[1]; ++g1)
-        for (int g2 = lo[2]; g2 <= hi[2]; ++g2) {
-          const int w = (g0 * p.G[1] + g1) * p.G[2] + g2 + wshift;
-          if (winner[w] == me) acc += (double)gtile[gpad + w];
-        }
-    dx[l0 * p.xvol + own_first + e] = (TD)acc;
-  }
+  const int shift = own_first - first_flat + pad;
+  TD *dx = static_cast<TD *>(result) + (l0 * p.xvol + own_first);
+  for (int e = threadIdx.x; e < own_len; e += blockDim.x) dx[e] = (TD)acc[e + shift];
 }
 
 static int check_pool_desc(const mg_pool_desc *d, PoolParams *p) {
@@ -315,8 +330,10 @@ static const int kTileBudgetBytes = 48 * 1024;
 
 // Chooses bands / volumes per block; returns false when not even one row of the
 // band axis plus its halo fits (the thread-per-element kernels handle that).
-static bool plan_tiles(const PoolParams &pp, size_t elem, bool bwd, PoolTileParams *t, int *tile_elems,
-                       int *win_slots, size_t *lds_bytes, long long *blocks) {
+static bool plan_tiles(const PoolParams &pp, size_t elem, size_t acc_elem, bool bwd, PoolTileParams *t,
+                       int *tile_elems, int *win_slots, int *acc_offset, size_t *lds_bytes, long long *blocks) {
+  // accumulators wider than an element of x cannot reuse the x tile
+  const size_t acc_extra = (bwd && acc_elem > elem) ? acc_elem : 0;
   PoolTileParams q{};
   int a = 0;
   while (a < 2 && pp.X[a] == 1) ++a;
@@ -339,7 +356,8 @@ static bool plan_tiles(const PoolParams &pp, size_t elem, bool bwd, PoolTilePara
   const int vec = (int)(16 / elem);
   // backward keeps, per window, an argmax slot (int) and its gradient (one element)
   const long long per_win = bwd ? 4 + (long long)elem : 0;
-  const long long per_vol = (long long)pp.xvol * elem + pp.gvol * per_win;
+  const long long per_x = (long long)(elem + acc_extra);
+  const long long per_vol = (long long)pp.xvol * per_x + pp.gvol * per_win;
   long long tile = 0, nwin = 0;
   if (per_vol + 64 <= kTileBudgetBytes) {
     // whole volumes: as many as fit, but keep enough blocks to fill the device
@@ -389,7 +407,7 @@ static bool plan_tiles(const PoolParams &pp, size_t elem, bool bwd, PoolTilePara
       if (bwd && band > S && band % S != 0) continue;
       long long rows, wins;
       need(band, &rows, &wins);
-      if (rows * q.inner_x * (long long)elem + wins * per_win + 64 <= kTileBudgetBytes) {
+      if (rows * q.inner_x * per_x + wins * per_win + 64 <= kTileBudgetBytes) {
         best = band;
         best_rows = rows;
         best_wins = wins;
@@ -412,10 +430,24 @@ static bool plan_tiles(const PoolParams &pp, size_t elem, bool bwd, PoolTilePara
   q.by_xvol = make_fastdiv_p((unsigned)pp.xvol);
   q.by_gvol = make_fastdiv_p((unsigned)pp.gvol);
   for (int k = 0; k < 3; ++k) q.by_s[k] = make_fastdiv_p((unsigned)pp.S[k]);
+  q.nranks = 1;
+  for (int k = 0; k < 3; ++k) {
+    q.cand[k] = (pp.P[k] - 1) / pp.S[k] + 1;
+    q.nranks *= q.cand[k];
+  }
+  if (q.nranks > 2047) return false;  // the rank shares a packed int with the argmax index
   *tile_elems = (int)(tile + vec);  // room for the alignment shift
   *tile_elems = (*tile_elems + 3) & ~3;
   *win_slots = bwd ? (int)((nwin + 3) & ~3ll) : 0;
-  *lds_bytes = (size_t)*tile_elems * elem + (bwd ? (size_t)*win_slots * 4 + ((size_t)nwin + vec) * elem : 0);
+  size_t bytes = (size_t)*tile_elems * elem + (bwd ? (size_t)*win_slots * 4 + ((size_t)nwin + vec) * elem : 0);
+  bytes = (bytes + 15) & ~size_t(15);
+  *acc_offset = 0;
+  if (acc_extra) {
+    *acc_offset = (int)bytes;
+    bytes += (size_t)*tile_elems * acc_elem;
+  }
+  if (*tile_elems >= (1 << 20) || bytes > 64 * 1024) return false;
+  *lds_bytes = bytes;
   *t = q;
   return true;
 }
@@ -441,16 +473,17 @@ int mg_maxpool_fwd(const mg_pool_desc *desc, const void *x, void *out) {
   hipStream_t s = runtime().stream;
   ScopedTiming timed(TAG_POOL_FWD);
   PoolTileParams tp;
-  int tile_elems = 0, win_slots = 0;
+  int tile_elems = 0, win_slots = 0, acc_offset = 0;
   size_t lds = 0;
   long long blocks = 0;
-  if (plan_tiles(p, desc->dtype == MG_F32 ? 4 : 8, false, &tp, &tile_elems, &win_slots, &lds, &blocks)) {
+  const size_t elem = desc->dtype == MG_F32 ? 4 : 8;
+  if (plan_tiles(p, elem, elem, false, &tp, &tile_elems, &win_slots, &acc_offset, &lds, &blocks)) {
     if (desc->dtype == MG_F32)
-      hipLaunchKernelGGL((maxpool_tile_kernel<float, float, false>), dim3((unsigned)blocks), dim3(256), lds, s, tp,
-                         (const float *)x, (const float *)nullptr, out, tile_elems, win_slots);
+      hipLaunchKernelGGL((maxpool_tile_kernel<float, float, float, false>), dim3((unsigned)blocks), dim3(256), lds, s,
+                         tp, (const float *)x, (const float *)nullptr, out, tile_elems, win_slots, acc_offset);
     else
-      hipLaunchKernelGGL((maxpool_tile_kernel<double, double, false>), dim3((unsigned)blocks), dim3(256), lds, s, tp,
-                         (const double *)x, (const double *)nullptr, out, tile_elems, win_slots);
+      hipLaunchKernelGGL((maxpool_tile_kernel<double, double, double, false>), dim3((unsigned)blocks), dim3(256), lds,
+                         s, tp, (const double *)x, (const double *)nullptr, out, tile_elems, win_slots, acc_offset);
     MG_HIP(hipGetLastError());
     return MG_OK;
   }
@@ -472,20 +505,33 @@ int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, vo
   hipStream_t s = runtime().stream;
   ScopedTiming timed(TAG_POOL_BWD);
   PoolTileParams tp;
-  int tile_elems = 0, win_slots = 0;
+  int tile_elems = 0, win_slots = 0, acc_offset = 0;
   size_t lds = 0;
   long long blocks = 0;
-  if (plan_tiles(p, desc->dtype == MG_F32 ? 4 : 8, true, &tp, &tile_elems, &win_slots, &lds, &blocks)) {
+  // float32 input whose windows overlap sums several float32 terms per element: that
+  // sum is carried in double (the reference's dx is float64) and rounded once.  When
+  // no two windows overlap an element gets at most one term and float32 is exact.
+  bool overlap = false;
+  for (int k = 0; k < 3; ++k) overlap |= p.P[k] > p.S[k];
+  const bool f32 = desc->dtype == MG_F32;
+  const size_t elem = f32 ? 4 : 8, acc_elem = (f32 && !overlap) ? 4 : 8;
+  if (plan_tiles(p, elem, acc_elem, true, &tp, &tile_elems, &win_slots, &acc_offset, &lds, &blocks)) {
     const dim3 grid((unsigned)blocks), block(256);
-    if (desc->dtype == MG_F64)
-      hipLaunchKernelGGL((maxpool_tile_kernel<double, double, true>), grid, block, lds, s, tp, (const double *)x,
-                         (const double *)grad, dx, tile_elems, win_slots);
-    else if (desc->dx_dtype == MG_F64)
-      hipLaunchKernelGGL((maxpool_tile_kernel<float, double, true>), grid, block, lds, s, tp, (const float *)x,
-                         (const float *)grad, dx, tile_elems, win_slots);
+    const bool wide = desc->dx_dtype == MG_F64;
+#define MG_POOL_BWD(T, TD, ACC)                                                                                  \
+  hipLaunchKernelGGL((maxpool_tile_kernel<T, TD, ACC, true>), grid, block, lds, s, tp, (const T *)x, (const T *)grad, \
+                     dx, tile_elems, win_slots, acc_offset)
+    if (!f32)
+      MG_POOL_BWD(double, double, double);
+    else if (overlap && wide)
+      MG_POOL_BWD(float, double, double);
+    else if (overlap)
+      MG_POOL_BWD(float, float, double);
+    else if (wide)
+      MG_POOL_BWD(float, double, float);
     else
-      hipLaunchKernelGGL((maxpool_tile_kernel<float, float, true>), grid, block, lds, s, tp, (const float *)x,
-                         (const float *)grad, dx, tile_elems, win_slots);
+      MG_POOL_BWD(float, float, float);
+#undef MG_POOL_BWD
     MG_HIP(hipGetLastError());
     return MG_OK;
   }
