@@ -142,44 +142,31 @@ struct PoolTileParams {
   int nranks;   // their product
 };
 
-template <typename T>
-__device__ __forceinline__ void stage_chunk(T *tile, const T *__restrict__ src, long long start, int len, int pad) {
-  // tile[pad + e] = src[start + e]; pad = start % VEC makes both sides 16-byte aligned together
-  constexpr int VEC = 16 / sizeof(T);
-  typedef T Vec __attribute__((ext_vector_type(VEC)));
-  const int head = min(len, (VEC - pad) % VEC);
-  for (int e = threadIdx.x; e < head; e += blockDim.x) tile[pad + e] = src[start + e];
-  const int body = (len - head) / VEC;
-  const Vec *vsrc = reinterpret_cast<const Vec *>(src + start + head);
-  Vec *vdst = reinterpret_cast<Vec *>(tile + pad + head);
-  for (int v = threadIdx.x; v < body; v += blockDim.x) vdst[v] = vsrc[v];
-  for (int e = head + body * VEC + threadIdx.x; e < len; e += blockDim.x) tile[pad + e] = src[start + e];
-}
+// What one block-iteration works on: a contiguous chunk of x and the windows in it.
+struct TileGeom {
+  long long l0;           // first leading index
+  long long chunk_start;  // element offset of the chunk in x
+  long long gstart;       // element offset of the windows' run in grad / out
+  int nvol;               // whole volumes in the chunk (1 when a volume is cut into bands)
+  int own_lo, own_hi;     // rows of the band axis this tile writes (backward)
+  int first_flat;         // flat index inside a volume of chunk element 0
+  int chunk_len;          // elements of x staged
+  int pad;                // chunk_start % VEC: shift that aligns LDS and global together
+  int nwin, win_base;     // windows evaluated; flat window index of the first
+  int gpad;               // gstart % VEC
+};
 
-template <typename T, typename TD, typename ACC, bool BWD>
-__global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, const T *__restrict__ x,
-                                                           const T *__restrict__ grad, void *__restrict__ result,
-                                                           int tile_elems, int win_slots, int acc_offset) {
-  // LDS: [x tile | one packed int per window | grad of those windows | accumulators];
-  // win_slots is a multiple of 4.  The accumulators alias the x tile (acc_offset == 0)
-  // when they are no wider than T: x is dead once every window knows its argmax.
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  T *tile = reinterpret_cast<T *>(smem);
-  int *winner = reinterpret_cast<int *>(smem + (size_t)tile_elems * sizeof(T));
-  T *gtile = reinterpret_cast<T *>(smem + (size_t)tile_elems * sizeof(T) + (size_t)win_slots * sizeof(int));
-  ACC *acc = reinterpret_cast<ACC *>(smem + acc_offset);
+template <typename T, bool BWD>
+__device__ __forceinline__ TileGeom tile_geom(const PoolTileParams &p, long long blk) {
   constexpr int VEC = 16 / sizeof(T);
-
-  const long long blk = blockIdx.x;
-  const long long l0 = (blk / p.bands) * p.volumes;
+  TileGeom t;
+  t.l0 = (blk / p.bands) * p.volumes;
   const int band = (int)(blk % p.bands);
-  const int nvol = (int)min((long long)p.volumes, p.lead - l0);
+  t.nvol = (int)min((long long)p.volumes, p.lead - t.l0);
   const int a = p.axis;
   const int XA = p.X[a], GA = p.G[a], PA = p.P[a], SA = p.S[a];
-
-  // rows of the band axis: [own_lo, own_hi) is what this block writes (backward),
-  // windows [g_lo, g_hi] along the axis are what it evaluates, rows [row_lo, row_hi)
-  // are what those windows (and the owned rows) read
+  // rows [own_lo, own_hi) are written (backward); windows [g_lo, g_hi] along the band
+  // axis are evaluated; rows [row_lo, row_hi) are what those windows and rows read
   int own_lo = 0, own_hi = XA, g_lo = 0, g_hi = GA - 1;
   if (p.bands > 1) {
     if (BWD) {
@@ -202,94 +189,173 @@ __global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, con
     row_lo = g_lo * SA;
     row_hi = g_hi * SA + PA;
   }
-  const int first_flat = row_lo * p.inner_x;  // flat index (inside a volume) of tile element 0
-  const int chunk_len = p.bands > 1 ? (row_hi - row_lo) * p.inner_x : nvol * p.xvol;
-  const long long chunk_start = l0 * p.xvol + first_flat;
-  const int pad = (int)(chunk_start % VEC);
-  stage_chunk(tile, x, chunk_start, chunk_len, pad);
-  const int nwin = any_window ? (p.bands > 1 ? (g_hi - g_lo + 1) * p.inner_g : nvol * p.gvol) : 0;
-  const int win_base = p.bands > 1 ? g_lo * p.inner_g : 0;  // flat window index of winner[0]
-  int gpad = 0;
-  if (BWD) {
-    // the windows' gradients are one contiguous run of grad: keep them next to the tile
-    const long long gstart = l0 * p.gvol + win_base;
-    gpad = (int)(gstart % VEC);
-    stage_chunk(gtile, grad, gstart, nwin, gpad);
+  t.own_lo = own_lo;
+  t.own_hi = own_hi;
+  t.first_flat = row_lo * p.inner_x;
+  t.chunk_len = p.bands > 1 ? (row_hi - row_lo) * p.inner_x : t.nvol * p.xvol;
+  t.chunk_start = t.l0 * p.xvol + t.first_flat;
+  t.pad = (int)(t.chunk_start % VEC);
+  t.nwin = any_window ? (p.bands > 1 ? (g_hi - g_lo + 1) * p.inner_g : t.nvol * p.gvol) : 0;
+  t.win_base = p.bands > 1 ? g_lo * p.inner_g : 0;
+  t.gstart = t.l0 * p.gvol + t.win_base;
+  t.gpad = (int)(t.gstart % VEC);
+  return t;
+}
+
+// A chunk on its way from global memory to LDS.  issue() sends DEPTH 16-byte loads per
+// thread and returns at once; commit() stores what came back, and moves whatever the
+// registers did not cover (the unaligned head and tail, anything beyond DEPTH) directly.
+// tile[pad + e] = src[start + e], with pad = start % VEC so both sides align together.
+template <typename T, int DEPTH>
+struct ChunkInFlight {
+  static constexpr int VEC = 16 / sizeof(T);
+  typedef T Vec __attribute__((ext_vector_type(VEC)));
+  Vec held[DEPTH];
+
+  __device__ __forceinline__ static int head_of(int len, int pad) { return min(len, (VEC - pad) % VEC); }
+
+  __device__ __forceinline__ void issue(const T *__restrict__ src, long long start, int len, int pad) {
+    const int head = head_of(len, pad);
+    const int body = (len - head) / VEC;
+    const Vec *vsrc = reinterpret_cast<const Vec *>(src + start + head);
+    // clamped, never predicated: a load behind a branch would wait for the one before it
+    const int last = max(body - 1, 0);
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) held[u] = vsrc[min(u * 256 + (int)threadIdx.x, last)];
   }
-  __syncthreads();
+
+  __device__ __forceinline__ void commit(T *tile, const T *__restrict__ src, long long start, int len, int pad) {
+    const int head = head_of(len, pad);
+    const int body = (len - head) / VEC;
+    Vec *vdst = reinterpret_cast<Vec *>(tile + pad + head);
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u) {
+      const int v = u * 256 + (int)threadIdx.x;
+      if (v < body) vdst[v] = held[u];
+    }
+    const Vec *vsrc = reinterpret_cast<const Vec *>(src + start + head);
+    for (int v = DEPTH * 256 + (int)threadIdx.x; v < body; v += 256) vdst[v] = vsrc[v];
+    for (int e = threadIdx.x; e < head; e += 256) tile[pad + e] = src[start + e];
+    for (int e = head + body * VEC + (int)threadIdx.x; e < len; e += 256) tile[pad + e] = src[start + e];
+  }
+};
+
+// Persistent blocks: each walks tiles blk, blk + gridDim.x, ...  While a tile is being
+// processed out of LDS, the next tile's x (and grad) are already on their way into
+// registers, so the memory system always has this block's next 16-48 KB in flight.
+template <typename T, typename TD, typename ACC, bool BWD, int DEPTH>
+__global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, const T *__restrict__ x,
+                                                           const T *__restrict__ grad, void *__restrict__ result,
+                                                           long long ntiles, int tile_elems, int win_slots,
+                                                           int acc_offset) {
+  // LDS: [x tile | one packed int per window | grad of those windows | accumulators];
+  // win_slots is a multiple of 4.  The accumulators alias the x tile (acc_offset == 0)
+  // when they are no wider than T: x is dead once every window knows its argmax.
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  T *tile = reinterpret_cast<T *>(smem);
+  int *winner = reinterpret_cast<int *>(smem + (size_t)tile_elems * sizeof(T));
+  T *gtile = reinterpret_cast<T *>(smem + (size_t)tile_elems * sizeof(T) + (size_t)win_slots * sizeof(int));
+  ACC *acc = reinterpret_cast<ACC *>(smem + acc_offset);
+  constexpr int GDEPTH = 2;
   const int x12 = p.X[1] * p.X[2], g12 = p.G[1] * p.G[2];
 
-  // ---- one thread per window: the maximum (forward) or where it is (backward)
-  for (int w = threadIdx.x; w < nwin; w += blockDim.x) {
-    const unsigned vol = p.by_gvol.div((unsigned)w);  // 0 when a volume is cut into bands
-    const unsigned wf = (unsigned)w - vol * (unsigned)p.gvol + (unsigned)win_base;
-    const unsigned g0 = p.by_g12.div(wf);
-    const unsigned r = wf - g0 * (unsigned)g12;
-    const unsigned g1 = p.by_g2.div(r);
-    const unsigned g2 = r - g1 * (unsigned)p.G[2];
-    const int origin = (int)((g0 * p.S[0] * p.X[1] + g1 * p.S[1]) * p.X[2] + g2 * p.S[2]) - first_flat +
-                       (int)vol * p.xvol + pad;
-    T best = tile[origin];
-    int where = origin;
-    for (int a0 = 0; a0 < p.P[0]; ++a0)
-      for (int a1 = 0; a1 < p.P[1]; ++a1) {
-        const int rowoff = origin + (a0 * p.X[1] + a1) * p.X[2];
-        for (int a2 = 0; a2 < p.P[2]; ++a2) {
-          const T v = tile[rowoff + a2];
-          if (takes_over(v, best)) {
-            best = v;
-            where = rowoff + a2;
+  ChunkInFlight<T, DEPTH> xin;
+  ChunkInFlight<T, GDEPTH> gin;
+  long long blk = blockIdx.x;
+  if (blk >= ntiles) return;
+  TileGeom t = tile_geom<T, BWD>(p, blk);
+  xin.issue(x, t.chunk_start, t.chunk_len, t.pad);
+  if (BWD) gin.issue(grad, t.gstart, t.nwin, t.gpad);
+
+  for (; blk < ntiles; blk += gridDim.x) {
+    xin.commit(tile, x, t.chunk_start, t.chunk_len, t.pad);
+    if (BWD) gin.commit(gtile, grad, t.gstart, t.nwin, t.gpad);
+    __syncthreads();
+
+    // next tile: loads go out now and land while this tile is processed
+    const long long nblk = blk + gridDim.x;
+    TileGeom tn = t;
+    if (nblk < ntiles) {
+      tn = tile_geom<T, BWD>(p, nblk);
+      xin.issue(x, tn.chunk_start, tn.chunk_len, tn.pad);
+      if (BWD) gin.issue(grad, tn.gstart, tn.nwin, tn.gpad);
+    }
+
+    // ---- one thread per window: the maximum (forward) or where it is (backward)
+    for (int w = threadIdx.x; w < t.nwin; w += 256) {
+      const unsigned vol = p.by_gvol.div((unsigned)w);  // 0 when a volume is cut into bands
+      const unsigned wf = (unsigned)w - vol * (unsigned)p.gvol + (unsigned)t.win_base;
+      const unsigned g0 = p.by_g12.div(wf);
+      const unsigned r = wf - g0 * (unsigned)g12;
+      const unsigned g1 = p.by_g2.div(r);
+      const unsigned g2 = r - g1 * (unsigned)p.G[2];
+      const int origin = (int)((g0 * p.S[0] * p.X[1] + g1 * p.S[1]) * p.X[2] + g2 * p.S[2]) - t.first_flat +
+                         (int)vol * p.xvol + t.pad;
+      T best = tile[origin];
+      int where = origin;
+      for (int a0 = 0; a0 < p.P[0]; ++a0)
+        for (int a1 = 0; a1 < p.P[1]; ++a1) {
+          const int rowoff = origin + (a0 * p.X[1] + a1) * p.X[2];
+          for (int a2 = 0; a2 < p.P[2]; ++a2) {
+            const T v = tile[rowoff + a2];
+            if (takes_over(v, best)) {
+              best = v;
+              where = rowoff + a2;
+            }
           }
         }
+      if (BWD) {
+        // Rank of this window among the windows that cover its argmax element, in
+        // ascending row-major window order: per axis min(g, (P-1-a)/S) with a the
+        // argmax's offset inside the window.  Two windows with the same argmax
+        // element never share a rank, and adding ranks 0, 1, 2, ... in turn is the
+        // order np.add.at visits them in.
+        const unsigned off = (unsigned)(where - origin);
+        const unsigned a0 = p.by_x12.div(off);
+        const unsigned r12 = off - a0 * (unsigned)x12;
+        const unsigned a1 = p.by_x2.div(r12);
+        const unsigned a2 = r12 - a1 * (unsigned)p.X[2];
+        const unsigned k0 = min(g0, p.by_s[0].div((unsigned)p.P[0] - 1u - a0));
+        const unsigned k1 = min(g1, p.by_s[1].div((unsigned)p.P[1] - 1u - a1));
+        const unsigned k2 = min(g2, p.by_s[2].div((unsigned)p.P[2] - 1u - a2));
+        const unsigned rank = (k0 * (unsigned)p.cand[1] + k1) * (unsigned)p.cand[2] + k2;
+        winner[w] = where | (int)(rank << 20);
+      } else {
+        static_cast<T *>(result)[t.gstart + w] = best;
       }
+    }
+
     if (BWD) {
-      // Rank of this window among the windows that cover its argmax element, in
-      // ascending row-major window order: per axis min(g, (P-1-a)/S) with a the
-      // argmax's offset inside the window.  Two windows with the same argmax
-      // element never share a rank, and adding ranks 0, 1, 2, ... in turn is the
-      // order np.add.at visits them in.
-      const unsigned off = (unsigned)(where - origin);
-      const unsigned a0 = p.by_x12.div(off);
-      const unsigned r12 = off - a0 * (unsigned)x12;
-      const unsigned a1 = p.by_x2.div(r12);
-      const unsigned a2 = r12 - a1 * (unsigned)p.X[2];
-      const unsigned k0 = min(g0, p.by_s[0].div((unsigned)p.P[0] - 1u - a0));
-      const unsigned k1 = min(g1, p.by_s[1].div((unsigned)p.P[1] - 1u - a1));
-      const unsigned k2 = min(g2, p.by_s[2].div((unsigned)p.P[2] - 1u - a2));
-      const unsigned rank = (k0 * (unsigned)p.cand[1] + k1) * (unsigned)p.cand[2] + k2;
-      winner[w] = where | (int)(rank << 20);
-    } else {
-      static_cast<T *>(result)[l0 * p.gvol + win_base + w] = best;
-    }
-  }
-  if (!BWD) return;
-  __syncthreads();
+      __syncthreads();
+      // ---- accumulators start at +0.0 (they may sit where the x tile was)
+      const int used = t.chunk_len + t.pad;
+      for (int e = threadIdx.x; e < used; e += 256) acc[e] = ACC(0);
+      __syncthreads();
 
-  // ---- accumulators start at +0.0 (they may sit where the x tile was)
-  const int used = chunk_len + pad;
-  for (int e = threadIdx.x; e < used; e += blockDim.x) acc[e] = ACC(0);
-  __syncthreads();
-
-  // ---- one pass per rank: every window of that rank adds its gradient to its argmax
-  // element.  Within a pass no two windows touch the same element, so plain LDS
-  // read-modify-writes are race-free; across passes the barrier orders them.
-  for (int rank = 0; rank < p.nranks; ++rank) {
-    for (int w = threadIdx.x; w < nwin; w += blockDim.x) {
-      const int packed = winner[w];
-      if ((packed >> 20) == rank) {
-        const int e = packed & 0xFFFFF;
-        acc[e] = acc[e] + (ACC)gtile[gpad + w];
+      // ---- one pass per rank: every window of that rank adds its gradient to its
+      // argmax element.  Within a pass no two windows touch the same element, so plain
+      // LDS read-modify-writes are race-free; across passes the barrier orders them.
+      for (int rank = 0; rank < p.nranks; ++rank) {
+        for (int w = threadIdx.x; w < t.nwin; w += 256) {
+          const int packed = winner[w];
+          if ((packed >> 20) == rank) {
+            const int e = packed & 0xFFFFF;
+            acc[e] = acc[e] + (ACC)gtile[t.gpad + w];
+          }
+        }
+        __syncthreads();
       }
-    }
-    __syncthreads();
-  }
 
-  // ---- write the rows this block owns
-  const int own_first = p.bands > 1 ? own_lo * p.inner_x : 0;
-  const int own_len = p.bands > 1 ? (own_hi - own_lo) * p.inner_x : nvol * p.xvol;
-  const int shift = own_first - first_flat + pad;
-  TD *dx = static_cast<TD *>(result) + (l0 * p.xvol + own_first);
-  for (int e = threadIdx.x; e < own_len; e += blockDim.x) dx[e] = (TD)acc[e + shift];
+      // ---- write the rows this tile owns
+      const int own_first = p.bands > 1 ? t.own_lo * p.inner_x : 0;
+      const int own_len = p.bands > 1 ? (t.own_hi - t.own_lo) * p.inner_x : t.nvol * p.xvol;
+      const int shift = own_first - t.first_flat + t.pad;
+      TD *dx = static_cast<TD *>(result) + (t.l0 * p.xvol + own_first);
+      for (int e = threadIdx.x; e < own_len; e += 256) dx[e] = (TD)acc[e + shift];
+    }
+    __syncthreads();  // LDS is about to be overwritten by the next tile
+    t = tn;
+  }
 }
 
 static int check_pool_desc(const mg_pool_desc *d, PoolParams *p) {
@@ -452,6 +518,16 @@ static bool plan_tiles(const PoolParams &pp, size_t elem, size_t acc_elem, bool 
   return true;
 }
 
+// Blocks of the persistent tile kernels: as many as fit on the device at once
+// (LDS-limited, at most 8 per compute unit), never more than there are tiles.
+static unsigned persistent_grid(long long tiles, size_t lds_bytes) {
+  const hipDeviceProp_t &pr = runtime().props;
+  const size_t lds_per_cu = 160 * 1024;
+  long long per_cu = (long long)(lds_per_cu / std::max<size_t>(lds_bytes, 1));
+  per_cu = std::max<long long>(1, std::min<long long>(per_cu, 8));
+  return (unsigned)std::min<long long>(tiles, per_cu * pr.multiProcessorCount);
+}
+
 static unsigned grid_for(long long total) {
   long long blocks = ceil_div(total, 256);
   const long long cap = (long long)runtime().props.multiProcessorCount * 32;
@@ -478,12 +554,19 @@ int mg_maxpool_fwd(const mg_pool_desc *desc, const void *x, void *out) {
   long long blocks = 0;
   const size_t elem = desc->dtype == MG_F32 ? 4 : 8;
   if (plan_tiles(p, elem, elem, false, &tp, &tile_elems, &win_slots, &acc_offset, &lds, &blocks)) {
-    if (desc->dtype == MG_F32)
-      hipLaunchKernelGGL((maxpool_tile_kernel<float, float, float, false>), dim3((unsigned)blocks), dim3(256), lds, s,
-                         tp, (const float *)x, (const float *)nullptr, out, tile_elems, win_slots, acc_offset);
-    else
-      hipLaunchKernelGGL((maxpool_tile_kernel<double, double, double, false>), dim3((unsigned)blocks), dim3(256), lds,
-                         s, tp, (const double *)x, (const double *)nullptr, out, tile_elems, win_slots, acc_offset);
+    // one tile per block measured faster than persistent blocks for the forward pass:
+    // its stores trail the next tile's loads in the same in-order memory counter
+    const dim3 grid((unsigned)blocks), block(256);
+    const bool deep = (size_t)tile_elems * elem > 8 * 4096;  // 16-byte loads per thread to cover the tile
+#define MG_POOL_FWD(T, DEPTH)                                                                                   \
+  hipLaunchKernelGGL((maxpool_tile_kernel<T, T, T, false, DEPTH>), grid, block, lds, s, tp, (const T *)x,       \
+                     (const T *)nullptr, out, blocks, tile_elems, win_slots, acc_offset)
+    if (desc->dtype == MG_F32) {
+      if (deep) MG_POOL_FWD(float, 12); else MG_POOL_FWD(float, 8);
+    } else {
+      if (deep) MG_POOL_FWD(double, 12); else MG_POOL_FWD(double, 8);
+    }
+#undef MG_POOL_FWD
     MG_HIP(hipGetLastError());
     return MG_OK;
   }
@@ -516,11 +599,18 @@ int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, vo
   const bool f32 = desc->dtype == MG_F32;
   const size_t elem = f32 ? 4 : 8, acc_elem = (f32 && !overlap) ? 4 : 8;
   if (plan_tiles(p, elem, acc_elem, true, &tp, &tile_elems, &win_slots, &acc_offset, &lds, &blocks)) {
-    const dim3 grid((unsigned)blocks), block(256);
+    const dim3 grid(persistent_grid(blocks, lds)), block(256);
     const bool wide = desc->dx_dtype == MG_F64;
-#define MG_POOL_BWD(T, TD, ACC)                                                                                  \
-  hipLaunchKernelGGL((maxpool_tile_kernel<T, TD, ACC, true>), grid, block, lds, s, tp, (const T *)x, (const T *)grad, \
-                     dx, tile_elems, win_slots, acc_offset)
+    const bool deep = (size_t)tile_elems * elem > 8 * 4096;
+#define MG_POOL_BWD(T, TD, ACC)                                                                                 \
+  do {                                                                                                          \
+    if (deep)                                                                                                   \
+      hipLaunchKernelGGL((maxpool_tile_kernel<T, TD, ACC, true, 12>), grid, block, lds, s, tp, (const T *)x,    \
+                         (const T *)grad, dx, blocks, tile_elems, win_slots, acc_offset);                       \
+    else                                                                                                        \
+      hipLaunchKernelGGL((maxpool_tile_kernel<T, TD, ACC, true, 8>), grid, block, lds, s, tp, (const T *)x,     \
+                         (const T *)grad, dx, blocks, tile_elems, win_slots, acc_offset);                       \
+  } while (0)
     if (!f32)
       MG_POOL_BWD(double, double, double);
     else if (overlap && wide)
