@@ -42,18 +42,17 @@ PEAK_HBM_GBS = 8000.0
 # helper (the Operation-level validator of the reference rejects them).
 WORKLOADS = {
     "conv1": dict(kind="conv", dtype="f64", seed=1001, x=(32, 3, 32, 32), w=(16, 3, 3, 3), wscale=27 ** -0.5,
-                  stride=(1, 1), padding=(1, 1), dilation=(1, 1), cpu_batch=32),
+                  stride=(1, 1), padding=(1, 1), dilation=(1, 1)),
     "conv3a": dict(kind="conv", dtype="f32", seed=1003, x=(128, 64, 56, 56), w=(64, 64, 3, 3), wscale=(2 / 576) ** 0.5,
-                   stride=(1, 1), padding=(1, 1), dilation=(1, 1), cpu_batch=16),
+                   stride=(1, 1), padding=(1, 1), dilation=(1, 1)),
     "conv3b": dict(kind="conv", dtype="f32", seed=1004, x=(128, 128, 28, 28), w=(256, 128, 3, 3),
-                   wscale=(2 / 1152) ** 0.5, stride=(2, 2), padding=(1, 1), dilation=(1, 1), cpu_batch=32),
+                   wscale=(2 / 1152) ** 0.5, stride=(2, 2), padding=(1, 1), dilation=(1, 1)),
     "conv4": dict(kind="conv", dtype="f64", seed=1005, x=(16, 32, 128, 128), w=(32, 32, 5, 5), wscale=800 ** -0.5,
-                  stride=(2, 1), padding=(4, 4), dilation=(2, 2), cpu_batch=4),
+                  stride=(2, 1), padding=(4, 4), dilation=(2, 2)),
     "conv5": dict(kind="conv", dtype="f32", seed=1006, x=(8, 16, 32, 64, 64), w=(32, 16, 3, 3, 3),
-                  wscale=(2 / 432) ** 0.5, stride=(1, 1, 1), padding=(1, 1, 1), dilation=(1, 1, 1), cpu_batch=1),
-    "pool2": dict(kind="pool", dtype="f64", seed=1002, x=(64, 64, 56, 56), pool=(3, 3), stride=(2, 2), cpu_lead=16),
-    "pool5": dict(kind="pool", dtype="f32", seed=1006, x=(8, 32, 32, 64, 64), pool=(2, 2, 2), stride=(2, 2, 2),
-                  cpu_lead=2),
+                  wscale=(2 / 432) ** 0.5, stride=(1, 1, 1), padding=(1, 1, 1), dilation=(1, 1, 1)),
+    "pool2": dict(kind="pool", dtype="f64", seed=1002, x=(64, 64, 56, 56), pool=(3, 3), stride=(2, 2)),
+    "pool5": dict(kind="pool", dtype="f32", seed=1006, x=(8, 32, 32, 64, 64), pool=(2, 2, 2), stride=(2, 2, 2)),
 }
 NP_DTYPE = {"f32": np.float32, "f64": np.float64}
 
@@ -215,41 +214,73 @@ def blas_threads():
         return int(os.environ.get("OMP_NUM_THREADS", "1"))
 
 
-def run_cpu_baseline(name):
-    """Time the NumPy restatement of the reference on a bounded sample."""
+def run_cpu_baseline(name, min_seconds=10.0, max_reps=200):
+    """Time the NumPy restatement of the reference on the host cores: the whole
+    workload, repeated until at least ``min_seconds`` of CPU work have been done."""
     from oracle import np_oracle as ora
 
     wl, dt = WORKLOADS[name], NP_DTYPE[WORKLOADS[name]["dtype"]]
     rng = np.random.default_rng(wl["seed"])
     if wl["kind"] == "conv":
-        nb = min(wl["cpu_batch"], wl["x"][0])
-        x = rng.standard_normal((nb, *wl["x"][1:])).astype(dt)
+        x = rng.standard_normal(wl["x"]).astype(dt)
         w = (rng.standard_normal(wl["w"]) * wl["wscale"]).astype(dt)
         conf = dict(stride=wl["stride"], padding=wl["padding"], dilation=wl["dilation"])
-        g = rng.standard_normal((nb, wl["w"][0], *conv_grid(wl))).astype(dt)
-        t0 = time.perf_counter()
-        ora.conv_forward(x, w, validate=False, **conf)
-        ora.conv_backward_x(g, x.shape, x.dtype, w, **conf)
-        ora.conv_backward_w(g, x, w.shape, **conf)
-        dt_s = time.perf_counter() - t0
-        value = 3 * conv_flops_per_pass(wl, nb) * 1e-12 / dt_s
-        sample = f"batch {nb} of {wl['x'][0]}, fwd+dx+dw once, {dt_s:.2f} s"
-        unit = "TFLOP/s"
+        g = rng.standard_normal((wl["x"][0], wl["w"][0], *conv_grid(wl))).astype(dt)
+
+        def once():
+            ora.conv_forward(x, w, validate=False, **conf)
+            ora.conv_backward_x(g, x.shape, x.dtype, w, **conf)
+            ora.conv_backward_w(g, x, w.shape, **conf)
+
+        work, scale, unit = 3 * conv_flops_per_pass(wl), 1e-12, "TFLOP/s"
+        what = "fwd+dx+dw"
     else:
-        m = len(wl["pool"])
-        nl = min(wl["cpu_lead"], wl["x"][0])
-        x = rng.standard_normal((nl, *wl["x"][1:])).astype(dt)
+        x = rng.standard_normal(wl["x"]).astype(dt)
         lead, pooled, grid = pool_shapes(wl)
-        g = rng.standard_normal((nl, *lead[1:], *grid)).astype(dt)
-        t0 = time.perf_counter()
-        ora.pool_forward(x, wl["pool"], wl["stride"], validate=False)
-        ora.pool_backward(x, g, wl["pool"], wl["stride"])
-        dt_s = time.perf_counter() - t0
-        value = (3 * x.nbytes + 2 * g.nbytes) * 1e-9 / dt_s
-        sample = f"leading {nl} of {wl['x'][0]} along axis 0, fwd+bwd once, {dt_s:.2f} s"
-        unit = "GB/s"
-    return {"value": value, "unit": unit, "cores": blas_threads() if wl["kind"] == "conv" else 1, "kind": "port",
-            "sample": sample, "numpy": np.__version__}
+        g = rng.standard_normal((*lead, *grid)).astype(dt)
+
+        def once():
+            ora.pool_forward(x, wl["pool"], wl["stride"], validate=False)
+            ora.pool_backward(x, g, wl["pool"], wl["stride"])
+
+        work, scale, unit = 3 * x.nbytes + 2 * g.nbytes, 1e-9, "GB/s"
+        what = "fwd+bwd"
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        once()
+        reps += 1
+        elapsed = time.perf_counter() - t0
+        if elapsed >= min_seconds or reps >= max_reps:
+            break
+    return {
+        "value": float(reps * work * scale / elapsed),
+        "unit": unit,
+        "cores": blas_threads() if wl["kind"] == "conv" else 1,
+        "kind": "port",
+        "sample": f"the whole workload ({what}), {reps} repetition(s), {elapsed:.1f} s of host time",
+        "numpy": np.__version__,
+    }
+
+
+def run_copy_calibration(mib=1024, reps=20):
+    """A plain 16-byte-per-lane device copy of known size: what the HBM traffic
+    counters of a profile are scaled against, and the practical bandwidth ceiling."""
+    from mygrad_amd import _device, _hip
+
+    n = mib << 20
+    a, b = _device.DeviceBuffer(n), _device.DeviceBuffer(n)
+    lib = _hip.lib()
+    _hip.check(lib.mg_memset_zero(a.ptr, n))
+    for _ in range(3):
+        _hip.check(lib.mg_memcpy_d2d(b.ptr, a.ptr, n))
+    _hip.timing_enable(True)
+    for _ in range(reps):
+        _hip.check(lib.mg_memcpy_d2d(b.ptr, a.ptr, n))
+    ms = [m for k, m in _hip.timing_read() if k == "copy"]
+    _hip.timing_enable(False)
+    avg = float(np.mean(ms))
+    return {"metric": "device copy", "bytes_read": n, "bytes_written": n, "avg_kernel_ms": avg,
+            "value": 2 * n * 1e-9 / (avg * 1e-3), "unit": "GB/s", "launches": len(ms)}
 
 
 def main():
@@ -260,11 +291,17 @@ def main():
     ap.add_argument("--workload", default="conv3a", choices=sorted(WORKLOADS))
     ap.add_argument("--all", action="store_true", help="also run every other workload (reported under 'secondary')")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only a 1 GiB device copy (the reference point for HBM traffic counters)")
     args = ap.parse_args()
 
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (--gpus 1); the path shards over the batch axis "
                  "by design but no multi-GPU code is part of it")
+
+    if args.calibrate_copy:
+        print(json.dumps(run_copy_calibration()))
+        return
 
     wl = WORKLOADS[args.workload]
     res = run_gpu(args.workload, args.steps, args.warmup)

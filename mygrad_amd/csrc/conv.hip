@@ -614,12 +614,15 @@ int build_fwd_plan(const Geometry &g, Plan &pl) {
   ph.npos = (int)((long long)g.N * g.gvol);
   set_divisors(ph);
   if (pl.tap_major) {
+    // K tiles run channel block by channel block, all taps of a block back to back:
+    // the taps of one channel block re-read the same few rows of x, which then come
+    // from L1/L2 instead of crossing HBM once per tap.
     const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
-    for (int t0 = 0; t0 < g.W[0]; ++t0)
-      for (int t1 = 0; t1 < g.W[1]; ++t1)
-        for (int t2 = 0; t2 < g.W[2]; ++t2) {
-          const int tflat = (t0 * g.W[1] + t1) * g.W[2] + t2;
-          for (int c0 = 0; c0 < g.C; c0 += bk) {
+    for (int c0 = 0; c0 < g.C; c0 += bk)
+      for (int t0 = 0; t0 < g.W[0]; ++t0)
+        for (int t1 = 0; t1 < g.W[1]; ++t1)
+          for (int t2 = 0; t2 < g.W[2]; ++t2) {
+            const int tflat = (t0 * g.W[1] + t1) * g.W[2] + t2;
             KTile e{};
             e.d0 = t0 * g.D[0] - g.P[0];
             e.d1 = t1 * g.D[1] - g.P[1];
@@ -628,7 +631,6 @@ int build_fwd_plan(const Geometry &g, Plan &pl) {
             e.coff = (int)(c0 * g.xvol) + e.d0 * qs[0] + e.d1 * qs[1] + e.d2 * qs[2];
             t.ktiles.push_back(e);
           }
-        }
     ph.k_count = (int)t.ktiles.size();
   } else {
     fwd_table(g, t.tab);
@@ -676,11 +678,11 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
         if (empty) continue;
         ph.k_begin = pl.tap_major ? (int)t.ktiles.size() : (int)t.tab.size();
         if (pl.tap_major) {
-          for (size_t a = 0; a < taps[0].size(); ++a)
-            for (size_t b = 0; b < taps[1].size(); ++b)
-              for (size_t c = 0; c < taps[2].size(); ++c) {
-                const int tflat = (taps[0][a] * g.W[1] + taps[1][b]) * g.W[2] + taps[2][c];
-                for (int f0 = 0; f0 < g.F; f0 += bk) {
+          for (int f0 = 0; f0 < g.F; f0 += bk)  // filter block outermost: its taps share rows of grad
+            for (size_t a = 0; a < taps[0].size(); ++a)
+              for (size_t b = 0; b < taps[1].size(); ++b)
+                for (size_t c = 0; c < taps[2].size(); ++c) {
+                  const int tflat = (taps[0][a] * g.W[1] + taps[1][b]) * g.W[2] + taps[2][c];
                   KTile e{};
                   e.d0 = offs[0][a];
                   e.d1 = offs[1][b];
@@ -689,7 +691,6 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
                   e.coff = (int)(f0 * g.gvol) + e.d0 * gs[0] + e.d1 * gs[1] + e.d2 * gs[2];
                   t.ktiles.push_back(e);
                 }
-              }
           ph.k_count = (int)t.ktiles.size() - ph.k_begin;
         } else {
           for (int f = 0; f < g.F; ++f)
