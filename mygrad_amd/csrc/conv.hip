@@ -16,6 +16,7 @@
 #include "conv_kernels.h"
 #include "internal.h"
 
+#include <algorithm>
 #include <cstring>
 #include <map>
 #include <string>
@@ -406,15 +407,30 @@ __global__ void __launch_bounds__(256) wgrad_kernel(const WgradParams p) {
   }
 }
 
+// ((p[0] + p[stride]) + p[2*stride]) + ... over `terms` terms: always this order, so
+// the result does not change from run to run; eight loads are in flight at a time.
+template <typename T>
+__device__ __forceinline__ T sum_in_order(const T *__restrict__ p, long long stride, int terms) {
+  T s = p[0];
+  int k = 1;
+  for (; k + 8 <= terms; k += 8) {
+    T v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = p[(long long)(k + u) * stride];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) s += v[u];
+  }
+  for (; k < terms; ++k) s += p[(long long)k * stride];
+  return s;
+}
+
 // dw[i] = ((part[0][i] + part[1][i]) + part[2][i]) + ...   (fixed order)
 template <typename T>
 __global__ void __launch_bounds__(256) splitk_reduce_kernel(const T *__restrict__ part, T *__restrict__ dw, int count,
                                                             int splits) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= count) return;
-  T s = part[i];
-  for (int k = 1; k < splits; ++k) s += part[(long long)k * count + i];
-  dw[i] = s;
+  dw[i] = sum_in_order(part + i, count, splits);
 }
 
 }  // namespace mg
@@ -717,6 +733,26 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
   return upload_plan(pl, t);
 }
 
+template <typename K>
+int resident_blocks(K kernel) {
+  int n = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, 0) != hipSuccess || n < 1) {
+    (void)hipGetLastError();
+    n = 1;
+  }
+  return n;
+}
+
+// Blocks of the filter-gradient kernel that fit on one compute unit at a time.
+int wgrad_blocks_per_cu(int dtype, int bm, bool tap_major) {
+#define MG_OCC(T, BM, BK, WM, WN)                                                    \
+  (tap_major ? resident_blocks(tap_wgrad_kernel<T, BM, 64, BK, WM, WN>)              \
+             : resident_blocks(wgrad_kernel<T, BM, 64, BK, WM, WN>))
+  if (dtype == MG_F32) return bm == 64 ? MG_OCC(float, 64, 64, 32, 32) : bm == 32 ? MG_OCC(float, 32, 64, 32, 16) : MG_OCC(float, 16, 64, 16, 16);
+  return bm == 64 ? MG_OCC(double, 64, 32, 32, 32) : bm == 32 ? MG_OCC(double, 32, 32, 32, 16) : MG_OCC(double, 16, 32, 16, 16);
+#undef MG_OCC
+}
+
 int build_wgrad_plan(const Geometry &g, Plan &pl) {
   Tables t;
   pl.bm = g.F <= 16 ? 16 : (g.F <= 32 ? 32 : 64);
@@ -728,14 +764,14 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
   const long long tiles = ceil_div(g.F, pl.bm) * col_tiles;
   const long long kpos = (long long)g.N * g.gvol;
   const long long ktiles = ceil_div(kpos, bk);
-  // aim at about three blocks per compute unit, at least 8 K tiles per block
-  const long long want_blocks = 3ll * runtime().props.multiProcessorCount;
-  long long splits = ceil_div(want_blocks, tiles);
-  const long long max_splits = ktiles >= 8 ? ktiles / 8 : 1;
-  if (splits > max_splits) splits = max_splits;
-  if (splits < 1) splits = 1;
-  if (splits > 1024) splits = 1024;
-  const long long tiles_per_split = ceil_div(ktiles, splits);
+  // Split K so that all blocks are resident at once (one round: no half-empty second
+  // round), with at least 4 K tiles per block.  The tap-major kernel hands whole
+  // splits to the 8 XCDs, so a multiple of 8 is preferred when one fits.
+  const long long slots = (long long)wgrad_blocks_per_cu(g.dtype, pl.bm, pl.tap_major) * runtime().props.multiProcessorCount;
+  const long long max_splits = std::max<long long>(1, std::min<long long>(ktiles / 4, 1024));
+  long long splits = std::max<long long>(1, std::min(slots / tiles, max_splits));
+  if (splits >= 8) splits = splits / 8 * 8;
+  long long tiles_per_split = ceil_div(ktiles, splits);
   pl.kchunk = (int)(tiles_per_split * bk);
   pl.splits = (int)ceil_div(kpos, pl.kchunk);
   if (pl.tap_major) {
@@ -743,9 +779,9 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
     const long long ngroups = col_tiles * (pl.bn / 16);
     for (long long gi = 0; gi < ngroups; ++gi) {
       WGroup e{};
-      const long long col = gi * 16;  // tap-major column t*C + c
+      const long long col = gi * 16;  // group gi = (channel block, tap), taps innermost
       if (col < ct) {
-        const int tflat = (int)(col / g.C), c0 = (int)(col % g.C);
+        const int tflat = (int)(gi % g.wvol), c0 = (int)(gi / g.wvol) * 16;
         const int t2 = tflat % g.W[2], t1 = (tflat / g.W[2]) % g.W[1], t0 = tflat / (g.W[2] * g.W[1]);
         e.d0 = t0 * g.D[0] - g.P[0];
         e.d1 = t1 * g.D[1] - g.P[1];
@@ -878,12 +914,17 @@ int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
 }
 
 template <typename T, int BM, int BN, int BK, int WM, int WN>
-void launch_wgrad(const WgradParams &wp, bool tap_major, hipStream_t s) {
-  const dim3 grid((unsigned)ceil_div(wp.CT, BN), (unsigned)ceil_div(wp.F, BM), (unsigned)wp.splits);
-  if (tap_major)
-    hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, wp);
-  else
+void launch_wgrad(WgradParams &wp, bool tap_major, hipStream_t s) {
+  wp.col_tiles = (int)ceil_div(wp.CT, BN);
+  wp.row_tiles = (int)ceil_div(wp.F, BM);
+  if (tap_major) {
+    // one-dimensional grid, whole K splits per XCD (see the kernel)
+    const long long blocks = (long long)wp.splits * wp.col_tiles * wp.row_tiles;
+    hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN>), dim3((unsigned)blocks), dim3(256), 0, s, wp);
+  } else {
+    const dim3 grid((unsigned)wp.col_tiles, (unsigned)wp.row_tiles, (unsigned)wp.splits);
     hipLaunchKernelGGL((wgrad_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, wp);
+  }
 }
 
 template <typename T>

@@ -50,8 +50,10 @@ struct KTile {
   int pad0_, pad1_, pad2_;
 };
 
-// Sixteen consecutive columns of the tap-major filter-gradient matrix: one tap,
-// channels c0..c0+15.  `coff` = c0 * channel stride + the tap's element offset.
+// Sixteen consecutive columns of the filter-gradient matrix as the tap-major kernel
+// lays it out: one tap, channels c0..c0+15 (c0 a multiple of 16); the groups of one
+// channel block follow each other, one per tap.  `coff` = c0 * channel stride + the
+// tap's element offset.
 struct WGroup {
   int coff;
   int d0, d1, d2;
@@ -114,6 +116,7 @@ struct WgradParams {
   const WGroup *groups;
   const void *zeros;
   int x_cstride;
+  int col_tiles, row_tiles;  // tiles of the output matrix along columns / filters
 };
 
 }  // namespace mg

@@ -8,7 +8,7 @@
 // pointer select per tile and one add per load, instead of a table row, three
 // compares and two selects per element.  Padding loads are pointed at a block
 // of zeros in device memory, so no select follows the load either.  The filter
-// gradient uses the same ordering for its columns.
+// gradient orders its columns by channel block of 16, then tap, then channel.
 //
 // Needs the channel count (filter count for dgrad) to be a multiple of BK; other
 // shapes take the table-driven kernels.
@@ -255,9 +255,24 @@ __global__ void __launch_bounds__(256) tap_wgrad_kernel(const WgradParams p) {
   const int wm0 = (wave / WAVES_N) * WM;
   const int wn0 = (wave % WAVES_N) * WN;
   const int l16 = lane & 15, lk = lane >> 4;
-  const int n0 = blockIdx.x * BN;  // first column (tap-major)
-  const int m0 = blockIdx.y * BM;  // first filter (F % BM == 0)
-  const int kbeg = (int)blockIdx.z * p.kchunk;
+  // Blocks are handed to the 8 XCDs round-robin, and each XCD has its own L2.  All
+  // tiles of one K split read the same positions of grad and x, so they are given to
+  // one XCD, next to each other in its dispatch order: block b is the (b/8)-th block
+  // of XCD b%8, and an XCD takes whole splits.
+  // (Only when the number of splits is a multiple of 8; otherwise plain order.)
+  const int tiles_per_split = p.col_tiles * p.row_tiles;
+  int split, tile;
+  if (p.splits % 8 == 0) {
+    const int xcd = blockIdx.x % 8, nth = blockIdx.x / 8;
+    split = (nth / tiles_per_split) * 8 + xcd;
+    tile = nth % tiles_per_split;
+  } else {
+    split = blockIdx.x / tiles_per_split;
+    tile = blockIdx.x % tiles_per_split;
+  }
+  const int n0 = (tile % p.col_tiles) * BN;  // first column
+  const int m0 = (tile / p.col_tiles) * BM;  // first filter (F % BM == 0)
+  const int kbeg = split * p.kchunk;
   const int kend = min(kbeg + p.kchunk, p.kpos);
 
   const T *__restrict__ grad = static_cast<const T *>(p.grad);
@@ -372,8 +387,8 @@ __global__ void __launch_bounds__(256) tap_wgrad_kernel(const WgradParams p) {
     buf ^= 1;
   }
 
-  // partial sums [split][f][tap-major column]
-  T *__restrict__ out = static_cast<T *>(p.out) + (long long)blockIdx.z * p.F * p.CT;
+  // partial sums [split][f][column]
+  T *__restrict__ out = static_cast<T *>(p.out) + (long long)split * p.F * p.CT;
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int col = n0 + wn0 + j * 16 + l16;
@@ -388,7 +403,9 @@ __global__ void __launch_bounds__(256) tap_wgrad_kernel(const WgradParams p) {
   }
 }
 
-// dw[f][c][t] = ((part[0] + part[1]) + part[2]) + ...  of  part[s][f][t*C + c]
+// dw[f][c][t] = ((part[0] + part[1]) + part[2]) + ...  of  part[s][f][col], where the
+// columns run over channel blocks of 16, then taps, then the channel inside the block:
+// col = ((c/16) * wvol + t) * 16 + c%16
 template <typename T>
 __global__ void __launch_bounds__(256) tap_reduce_kernel(const T *__restrict__ part, T *__restrict__ dw, int F, int C,
                                                          int wvol, int splits) {
@@ -400,10 +417,8 @@ __global__ void __launch_bounds__(256) tap_reduce_kernel(const T *__restrict__ p
   const int r = i - f * ct;
   const int c = r / wvol;
   const int t = r - c * wvol;
-  const int src = f * ct + t * C + c;
-  T s = part[src];
-  for (int k = 1; k < splits; ++k) s += part[(long long)k * count + src];
-  dw[i] = s;
+  const int src = f * ct + ((c / 16) * wvol + t) * 16 + c % 16;
+  dw[i] = sum_in_order(part + src, count, splits);
 }
 
 }  // namespace mg
