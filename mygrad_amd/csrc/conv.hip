@@ -467,8 +467,11 @@ struct Plan {
   WGroup *groups = nullptr;
   void *zeros = nullptr;
   int nphases = 0;
-  int pos_blocks = 0;  // grid.x of the gather-GEMM
+  int pos_blocks = 0;  // position blocks of the gather-GEMM (all phases)
   int bm = 0, bn = 0;
+  int m_tiles = 1;     // row tiles per position block
+  int full_tiles = 0;  // tiles computed whole by one block (tap-major kernel)
+  int tail_split = 1;  // blocks sharing each of the remaining tiles
   bool tap_major = false;  // which kernel family the tables are for
   bool single_dense_phase = false;  // positions enumerate the destination tensor in order
   // wgrad
@@ -539,6 +542,67 @@ int pick_bm(int M) {
     if (padded - M <= M / 8) return c;
   }
   return 16;
+}
+
+// Picks the tile of the gather-GEMM and how its last, partial round of tiles is
+// shared out.  Blocks reach the compute units round-robin, so after floor(T / CUs)
+// whole tiles per unit, T % CUs tiles are left that would keep only some units busy
+// for a full tile time; the tap-major kernel cuts each of those into `split` K slices
+// so that every unit gets about the same share of them.  Smaller tiles give more
+// tiles (finer balance, less padding) at some cost in operand reuse.
+struct TileChoice {
+  int bm, bn, m_tiles, full_tiles, tail_split;
+  long long tiles;
+};
+
+TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_ktiles, bool tap_major, size_t elem) {
+  struct Cfg {
+    int bm, bn;
+    double penalty;  // relative cost of a flop in this tile shape
+    bool tap_only;
+  };
+  static const Cfg cfgs[] = {{128, 128, 1.00, false}, {128, 64, 1.10, true}, {64, 256, 1.00, false}, {64, 128, 1.08, true},
+                             {32, 256, 1.00, false},  {32, 128, 1.10, true}, {16, 256, 1.00, false}};
+  const int bm = pick_bm(M);
+  const int cus = runtime().props.multiProcessorCount;
+  TileChoice best{};
+  double best_cost = 0;
+  for (const Cfg &c : cfgs) {
+    if (c.bm != bm || (c.tap_only && !tap_major)) continue;
+    TileChoice t{};
+    t.bm = c.bm;
+    t.bn = c.bn;
+    t.m_tiles = (int)ceil_div(M, c.bm);
+    long long pos_blocks = 0;
+    for (long long n : phase_npos) pos_blocks += ceil_div(n, c.bn);
+    t.tiles = pos_blocks * t.m_tiles;
+    t.full_tiles = (int)t.tiles;
+    t.tail_split = 1;
+    double tail = 0;
+    const long long rem = t.tiles % cus;
+    if (rem > 0) {
+      tail = 1.0;
+      if (tap_major) {
+        // slices of at least two K tiles, at most 32 MB of partial sums
+        const long long tile_bytes = (long long)c.bm * c.bn * (long long)elem;
+        const int smax = (int)std::max<long long>(1, std::min<long long>({(long long)min_ktiles / 2, 32ll, (32ll << 20) / (rem * tile_bytes)}));
+        for (int sp = 2; sp <= smax; ++sp) {
+          const double share = (double)ceil_div(rem * sp, cus) / sp + 0.01 * sp;  // + a little for the fix-up pass
+          if (share < tail - 1e-9) {
+            tail = share;
+            t.tail_split = sp;
+          }
+        }
+        if (t.tail_split > 1) t.full_tiles = (int)(t.tiles - rem);
+      }
+    }
+    const double cost = ((double)(t.tiles / cus) + tail) * c.bm * c.bn * c.penalty;
+    if (best.bm == 0 || cost < best_cost) {
+      best = t;
+      best_cost = cost;
+    }
+  }
+  return best;
 }
 
 void set_divisors(Phase &ph) {
@@ -616,10 +680,13 @@ void fwd_table(const Geometry &g, std::vector<TabEntry> &tab) {
 int build_fwd_plan(const Geometry &g, Plan &pl) {
   Tables t;
   const int bk = gemm_bk(g.dtype);
-  pl.bm = pick_bm(g.F);
-  pl.bn = pl.bm == 128 ? 128 : 256;
   pl.tap_major = g.C % bk == 0;
   pl.single_dense_phase = true;
+  {
+    const long long ktiles = pl.tap_major ? g.wvol * (g.C / bk) : ceil_div((long long)g.C * g.wvol, bk);
+    const TileChoice tc = choose_tile(g.F, {(long long)g.N * g.gvol}, (int)ktiles, pl.tap_major, g.dtype == MG_F64 ? 8 : 4);
+    pl.bm = tc.bm, pl.bn = tc.bn, pl.m_tiles = tc.m_tiles, pl.full_tiles = tc.full_tiles, pl.tail_split = tc.tail_split;
+  }
   Phase ph{};
   for (int k = 0; k < 3; ++k) {
     ph.J[k] = g.G[k];
@@ -662,73 +729,96 @@ int build_fwd_plan(const Geometry &g, Plan &pl) {
 int build_dgrad_plan(const Geometry &g, Plan &pl) {
   Tables t;
   const int bk = gemm_bk(g.dtype);
-  pl.bm = pick_bm(g.C);
-  pl.bn = pl.bm == 128 ? 128 : 256;
   pl.tap_major = g.F % bk == 0;
   pl.single_dense_phase = g.S[0] == 1 && g.S[1] == 1 && g.S[2] == 1;
   const int gs[3] = {g.G[1] * g.G[2], g.G[2], 1};
-  int blk = 0;
   long long nphase = (long long)g.S[0] * g.S[1] * g.S[2];
   if (nphase > 4096) return fail(MG_ERR_UNSUPPORTED, "prod(stride) = %lld phases (limit 4096)", nphase);
+
+  // ---- the stride phases: which input pixels, which taps reach them
+  struct PhaseTaps {
+    Phase ph;
+    std::vector<int> taps[3], offs[3];
+  };
+  std::vector<PhaseTaps> found;
   for (int r0 = 0; r0 < g.S[0]; ++r0)
     for (int r1 = 0; r1 < g.S[1]; ++r1)
       for (int r2 = 0; r2 < g.S[2]; ++r2) {
         const int rho[3] = {r0, r1, r2};
-        Phase ph{};
+        PhaseTaps pt{};
         bool empty = false;
-        std::vector<int> taps[3], offs[3];
         for (int k = 0; k < 3; ++k) {
           // input pixels i with (i + pad) % stride == rho
           const int i0 = ((rho[k] - g.P[k]) % g.S[k] + g.S[k]) % g.S[k];
-          ph.o0[k] = i0;
-          ph.J[k] = i0 < g.X[k] ? (g.X[k] - i0 + g.S[k] - 1) / g.S[k] : 0;
-          if (ph.J[k] == 0) empty = true;
+          pt.ph.o0[k] = i0;
+          pt.ph.J[k] = i0 < g.X[k] ? (g.X[k] - i0 + g.S[k] - 1) / g.S[k] : 0;
+          if (pt.ph.J[k] == 0) empty = true;
           // taps that can reach them: t*dil % stride == rho; the window index is then
           // g = j + (i0 + pad - t*dil) / stride  (exact division)
           for (int tt = 0; tt < g.W[k]; ++tt)
             if ((tt * g.D[k]) % g.S[k] == rho[k]) {
-              taps[k].push_back(tt);
-              offs[k].push_back((i0 + g.P[k] - tt * g.D[k]) / g.S[k]);
+              pt.taps[k].push_back(tt);
+              pt.offs[k].push_back((i0 + g.P[k] - tt * g.D[k]) / g.S[k]);
             }
         }
         if (empty) continue;
-        ph.k_begin = pl.tap_major ? (int)t.ktiles.size() : (int)t.tab.size();
-        if (pl.tap_major) {
-          for (int f0 = 0; f0 < g.F; f0 += bk)  // filter block outermost: its taps share rows of grad
-            for (size_t a = 0; a < taps[0].size(); ++a)
-              for (size_t b = 0; b < taps[1].size(); ++b)
-                for (size_t c = 0; c < taps[2].size(); ++c) {
-                  const int tflat = (taps[0][a] * g.W[1] + taps[1][b]) * g.W[2] + taps[2][c];
-                  KTile e{};
-                  e.d0 = offs[0][a];
-                  e.d1 = offs[1][b];
-                  e.d2 = offs[2][c];
-                  e.a_row0 = tflat * g.F + f0;
-                  e.coff = (int)(f0 * g.gvol) + e.d0 * gs[0] + e.d1 * gs[1] + e.d2 * gs[2];
-                  t.ktiles.push_back(e);
-                }
-          ph.k_count = (int)t.ktiles.size() - ph.k_begin;
-        } else {
-          for (int f = 0; f < g.F; ++f)
-            for (size_t a = 0; a < taps[0].size(); ++a)
-              for (size_t b = 0; b < taps[1].size(); ++b)
-                for (size_t c = 0; c < taps[2].size(); ++c) {
-                  TabEntry e;
-                  e.d0 = offs[0][a];
-                  e.d1 = offs[1][b];
-                  e.d2 = offs[2][c];
-                  e.off = (int)(f * g.gvol) + e.d0 * gs[0] + e.d1 * gs[1] + e.d2 * gs[2];
-                  t.tab.push_back(e);
-                  t.arow.push_back((int)(f * g.wvol) + (taps[0][a] * g.W[1] + taps[1][b]) * g.W[2] + taps[2][c]);
-                }
-          ph.k_count = (int)t.tab.size() - ph.k_begin;
-        }
-        ph.npos = (int)((long long)g.N * ph.J[0] * ph.J[1] * ph.J[2]);
-        set_divisors(ph);
-        ph.blk_begin = blk;
-        blk += (int)ceil_div(ph.npos, pl.bn);
-        t.phases.push_back(ph);
+        pt.ph.npos = (int)((long long)g.N * pt.ph.J[0] * pt.ph.J[1] * pt.ph.J[2]);
+        set_divisors(pt.ph);
+        found.push_back(pt);
       }
+
+  // ---- tile shape and tail sharing
+  {
+    std::vector<long long> npos;
+    long long min_ktiles = 1 << 30;
+    for (const PhaseTaps &pt : found) {
+      npos.push_back(pt.ph.npos);
+      const long long ntaps = (long long)pt.taps[0].size() * pt.taps[1].size() * pt.taps[2].size();
+      min_ktiles = std::min(min_ktiles, pl.tap_major ? ntaps * (g.F / bk) : ceil_div(ntaps * g.F, bk));
+    }
+    const TileChoice tc = choose_tile(g.C, npos, (int)std::max<long long>(min_ktiles, 0), pl.tap_major, g.dtype == MG_F64 ? 8 : 4);
+    pl.bm = tc.bm, pl.bn = tc.bn, pl.m_tiles = tc.m_tiles, pl.full_tiles = tc.full_tiles, pl.tail_split = tc.tail_split;
+  }
+
+  // ---- tables
+  int blk = 0;
+  for (PhaseTaps &pt : found) {
+    Phase &ph = pt.ph;
+    ph.k_begin = pl.tap_major ? (int)t.ktiles.size() : (int)t.tab.size();
+    if (pl.tap_major) {
+      for (int f0 = 0; f0 < g.F; f0 += bk)  // filter block outermost: its taps share rows of grad
+        for (size_t a = 0; a < pt.taps[0].size(); ++a)
+          for (size_t b = 0; b < pt.taps[1].size(); ++b)
+            for (size_t c = 0; c < pt.taps[2].size(); ++c) {
+              const int tflat = (pt.taps[0][a] * g.W[1] + pt.taps[1][b]) * g.W[2] + pt.taps[2][c];
+              KTile e{};
+              e.d0 = pt.offs[0][a];
+              e.d1 = pt.offs[1][b];
+              e.d2 = pt.offs[2][c];
+              e.a_row0 = tflat * g.F + f0;
+              e.coff = (int)(f0 * g.gvol) + e.d0 * gs[0] + e.d1 * gs[1] + e.d2 * gs[2];
+              t.ktiles.push_back(e);
+            }
+      ph.k_count = (int)t.ktiles.size() - ph.k_begin;
+    } else {
+      for (int f = 0; f < g.F; ++f)
+        for (size_t a = 0; a < pt.taps[0].size(); ++a)
+          for (size_t b = 0; b < pt.taps[1].size(); ++b)
+            for (size_t c = 0; c < pt.taps[2].size(); ++c) {
+              TabEntry e;
+              e.d0 = pt.offs[0][a];
+              e.d1 = pt.offs[1][b];
+              e.d2 = pt.offs[2][c];
+              e.off = (int)(f * g.gvol) + e.d0 * gs[0] + e.d1 * gs[1] + e.d2 * gs[2];
+              t.tab.push_back(e);
+              t.arow.push_back((int)(f * g.wvol) + (pt.taps[0][a] * g.W[1] + pt.taps[1][b]) * g.W[2] + pt.taps[2][c]);
+            }
+      ph.k_count = (int)t.tab.size() - ph.k_begin;
+    }
+    ph.blk_begin = blk;
+    blk += (int)ceil_div(ph.npos, pl.bn);
+    t.phases.push_back(ph);
+  }
   pl.pos_blocks = blk;
   return upload_plan(pl, t);
 }
@@ -817,12 +907,25 @@ int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
 }
 
 template <typename T, int BM, int BN, int BK, int WM, int WN>
-void launch_gemm(const GemmParams &gp, int pos_blocks, bool tap_major, hipStream_t s) {
-  const dim3 grid((unsigned)pos_blocks, (unsigned)ceil_div(gp.M, BM));
-  if (tap_major)
-    hipLaunchKernelGGL((tap_gemm_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, gp);
-  else
+void launch_gemm(const GemmParams &gp, const Plan &pl, hipStream_t s) {
+  if (pl.tap_major) {
+    const long long tiles = (long long)pl.pos_blocks * pl.m_tiles;
+    const long long tail_tiles = tiles - pl.full_tiles;
+    hipLaunchKernelGGL((tap_gemm_kernel<T, BM, BN, BK, WM, WN>), dim3((unsigned)(pl.full_tiles + tail_tiles * pl.tail_split)),
+                       dim3(256), 0, s, gp);
+    if (tail_tiles > 0)
+      hipLaunchKernelGGL((tail_fixup_kernel<T, BM, BN>), dim3((unsigned)ceil_div(BM * BN, 256), (unsigned)tail_tiles),
+                         dim3(256), 0, s, gp);
+  } else {
+    const dim3 grid((unsigned)pl.pos_blocks, (unsigned)pl.m_tiles);
     hipLaunchKernelGGL((gather_gemm_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, gp);
+  }
+}
+
+// Bytes of partial sums the shared tail tiles of this plan need.
+size_t tail_bytes(const Plan &pl, size_t elem) {
+  const long long tail_tiles = (long long)pl.pos_blocks * pl.m_tiles - pl.full_tiles;
+  return pl.tap_major ? (size_t)tail_tiles * pl.tail_split * pl.bm * pl.bn * elem : 0;
 }
 
 template <typename T>
@@ -835,26 +938,38 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
   gp.nphases = pl.nphases;
   gp.ktiles = pl.ktiles;
   gp.zeros = pl.zeros;
+  gp.m_tiles = pl.m_tiles;
+  gp.full_tiles = pl.tap_major ? pl.full_tiles : pl.pos_blocks * pl.m_tiles;
+  gp.tail_split = pl.tail_split;
   // a lane may store its 4 positions as one vector when they are adjacent in dst
   // (positions run through dst in order, the per-sample volume is a multiple of 4,
   // and every row starts 16-byte aligned)
   gp.vec_store = pl.single_dense_phase && gp.dst_mstride % 4 == 0 && gp.dst_nstride % 4 == 0 &&
                  reinterpret_cast<uintptr_t>(gp.dst) % 16 == 0;
   ScopedTiming timed(tag);
-  switch (pl.bm) {
-    case 128: launch_gemm<T, 128, 128, BK, 64, 64>(gp, pl.pos_blocks, pl.tap_major, s); break;
-    case 64: launch_gemm<T, 64, 256, BK, 64, 64>(gp, pl.pos_blocks, pl.tap_major, s); break;
-    case 32: launch_gemm<T, 32, 256, BK, 32, 64>(gp, pl.pos_blocks, pl.tap_major, s); break;
-    default: launch_gemm<T, 16, 256, BK, 16, 64>(gp, pl.pos_blocks, pl.tap_major, s); break;
+  const int shape = pl.bm * 1000 + pl.bn;
+  switch (shape) {
+    case 128128: launch_gemm<T, 128, 128, BK, 64, 64>(gp, pl, s); break;
+    case 128064: launch_gemm<T, 128, 64, BK, 64, 32>(gp, pl, s); break;
+    case 64256: launch_gemm<T, 64, 256, BK, 64, 64>(gp, pl, s); break;
+    case 64128: launch_gemm<T, 64, 128, BK, 32, 64>(gp, pl, s); break;
+    case 32256: launch_gemm<T, 32, 256, BK, 32, 64>(gp, pl, s); break;
+    case 32128: launch_gemm<T, 32, 128, BK, 16, 64>(gp, pl, s); break;
+    case 16256: launch_gemm<T, 16, 256, BK, 16, 64>(gp, pl, s); break;
+    default: return fail(MG_ERR_UNSUPPORTED, "no kernel for tile %d x %d", pl.bm, pl.bn);
   }
   MG_HIP(hipGetLastError());
   return MG_OK;
 }
 
+// Packs the filters into the front of the library workspace; `extra` more bytes
+// behind them (256-byte aligned) are reserved for the caller and returned in *behind.
 template <typename T>
-int pack_filters(const Geometry &g, const void *w, int mode, void **packed) {
+int pack_filters(const Geometry &g, const void *w, int mode, void **packed, size_t extra = 0, void **behind = nullptr) {
   const size_t count = (size_t)g.F * g.C * g.wvol;
-  if (int rc = workspace(count * sizeof(T), packed)) return rc;
+  const size_t packed_bytes = (count * sizeof(T) + 255) & ~size_t(255);
+  if (int rc = workspace(packed_bytes + extra, packed)) return rc;
+  if (behind) *behind = static_cast<char *>(*packed) + packed_bytes;
   const unsigned blocks = (unsigned)std::min<long long>(ceil_div((long long)count, 256), 4096);
   ScopedTiming timed(TAG_PACK_FILTERS);
   hipLaunchKernelGGL(pack_filters_kernel<T>, dim3(blocks), dim3(256), 0, runtime().stream, static_cast<const T *>(w),
@@ -866,8 +981,10 @@ int pack_filters(const Geometry &g, const void *w, int mode, void **packed) {
 template <typename T>
 int conv_fwd_impl(const Geometry &g, const Plan &pl, const void *x, const void *w, void *out) {
   void *packed = nullptr;
-  if (int rc = pack_filters<T>(g, w, pl.tap_major ? 2 : 0, &packed)) return rc;
+  void *partial = nullptr;
+  if (int rc = pack_filters<T>(g, w, pl.tap_major ? 2 : 0, &packed, tail_bytes(pl, sizeof(T)), &partial)) return rc;
   GemmParams gp{};
+  gp.partial = partial;
   gp.A = packed;
   gp.src = x;
   gp.dst = out;
@@ -891,8 +1008,10 @@ int conv_fwd_impl(const Geometry &g, const Plan &pl, const void *x, const void *
 template <typename T>
 int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const void *w, void *dx) {
   void *packed = nullptr;
-  if (int rc = pack_filters<T>(g, w, pl.tap_major ? 3 : 1, &packed)) return rc;
+  void *partial = nullptr;
+  if (int rc = pack_filters<T>(g, w, pl.tap_major ? 3 : 1, &packed, tail_bytes(pl, sizeof(T)), &partial)) return rc;
   GemmParams gp{};
+  gp.partial = partial;
   gp.A = packed;
   gp.src = grad;
   gp.dst = dx;

@@ -95,6 +95,10 @@ struct GemmParams {
   const void *zeros;    // a few zero elements in device memory: where padding loads point
   int src_cstride;      // element stride between consecutive channels of the gathered tensor
   int vec_store;        // positions are contiguous in dst: a lane may store its TN positions as one vector
+  int m_tiles;          // row tiles per position block
+  int full_tiles;       // tiles computed whole by one block each
+  int tail_split;       // blocks that share each remaining tile (K slices), >= 1
+  void *partial;        // [tail tile][slice][BM][BN] partial sums of the shared tiles
 };
 
 // Filter gradient:  out[split][f][col] = sum over the split's positions (n, g) of

@@ -75,11 +75,26 @@ __global__ void __launch_bounds__(256) tap_gemm_kernel(const GemmParams p) {
   const int wn0 = (wave % WAVES_N) * WN;
   const int l16 = lane & 15, lk = lane >> 4;
 
+  // Tiles are numbered with the row tile (m) innermost, so that the row tiles of one
+  // position block, which gather the same elements, run next to each other.  The
+  // first p.full_tiles blocks compute one whole tile each.  The tiles that remain
+  // would fill only part of the device in a last round, so each of them is shared
+  // by p.tail_split blocks, each taking a slice of the K loop and leaving its partial
+  // sums in a workspace for tail_fixup_kernel.
+  const int bid = blockIdx.x;
+  int tile = bid, piece = 0;
+  const bool partial = bid >= p.full_tiles;
+  if (partial) {
+    const int j = bid - p.full_tiles;
+    tile = p.full_tiles + j / p.tail_split;
+    piece = j % p.tail_split;
+  }
+  const int pblk = tile / p.m_tiles;
   int pi = 0;
-  while (pi + 1 < p.nphases && (int)blockIdx.x >= p.phases[pi + 1].blk_begin) ++pi;
+  while (pi + 1 < p.nphases && pblk >= p.phases[pi + 1].blk_begin) ++pi;
   const Phase ph = p.phases[pi];
-  const int pos0 = ((int)blockIdx.x - ph.blk_begin) * BN;
-  const int m0 = blockIdx.y * BM;
+  const int pos0 = (pblk - ph.blk_begin) * BN;
+  const int m0 = (tile % p.m_tiles) * BM;
   const int j12 = ph.J[1] * ph.J[2];
   const int jvol = ph.J[0] * j12;
 
@@ -146,15 +161,20 @@ __global__ void __launch_bounds__(256) tap_gemm_kernel(const GemmParams p) {
   // Lane (l16, lk) feeds row/column l16 of every 16x16 tile.  Tile i of the wave
   // takes the rows m = wm0 + l16*TM + i (and tile j the positions wn0 + l16*TN + j),
   // so the TM (TN) operands of a lane are adjacent in LDS and come in one read.
-  const int ktiles = ph.k_count;
+  int kt_begin = 0, kt_end = ph.k_count;
+  if (partial) {
+    const int per = (ph.k_count + p.tail_split - 1) / p.tail_split;
+    kt_begin = min(piece * per, ph.k_count);
+    kt_end = min(kt_begin + per, ph.k_count);
+  }
   int buf = 0;
-  if (ktiles > 0) {
-    fetch(0);
+  if (kt_begin < kt_end) {
+    fetch(kt_begin);
     stash(0);
   }
   __syncthreads();
-  for (int kt = 0; kt < ktiles; ++kt) {
-    const bool more = kt + 1 < ktiles;
+  for (int kt = kt_begin; kt < kt_end; ++kt) {
+    const bool more = kt + 1 < kt_end;
     if (more) fetch(kt + 1);
 #pragma unroll
     for (int k4 = 0; k4 < BK / 4; ++k4) {
@@ -172,6 +192,33 @@ __global__ void __launch_bounds__(256) tap_gemm_kernel(const GemmParams p) {
   }
 
   // ---- epilogue
+  if (partial) {
+    // raw tile [BM][BN] of this slice, lane's TN positions stored as one vector
+    T *slot = static_cast<T *>(p.partial) +
+              ((long long)(tile - p.full_tiles) * p.tail_split + piece) * (BM * BN) + (wn0 + l16 * TN);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int ml = wm0 + Mma<T>::row_of(lane, q) * TM + i;
+        T v[TN];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) v[j] = acc[i][j][q];
+        if constexpr (sizeof(T) * TN <= 16) {
+          store_vec<T, TN>(slot + ml * BN, v);
+        } else {
+          T lo[TN / 2], hi[TN / 2];
+#pragma unroll
+          for (int j = 0; j < TN / 2; ++j) {
+            lo[j] = v[j];
+            hi[j] = v[TN / 2 + j];
+          }
+          store_vec<T, TN / 2>(slot + ml * BN, lo);
+          store_vec<T, TN / 2>(slot + ml * BN + TN / 2, hi);
+        }
+      }
+    return;
+  }
   T *__restrict__ dst = static_cast<T *>(p.dst);
   auto dst_of = [&](int ipos) -> T * {
     const unsigned pos = (unsigned)ipos;
@@ -227,6 +274,36 @@ __global__ void __launch_bounds__(256) tap_gemm_kernel(const GemmParams p) {
         }
     }
   }
+}
+
+// Adds the K slices of the shared tail tiles in slice order (always the same order,
+// so results repeat exactly) and stores them where the tile's epilogue would have.
+// One thread per tile element; blockIdx.y is the tail tile.
+template <typename T, int BM, int BN>
+__global__ void __launch_bounds__(256) tail_fixup_kernel(const GemmParams p) {
+  const int e = blockIdx.x * 256 + threadIdx.x;  // element of the [BM][BN] tile
+  if (e >= BM * BN) return;
+  const int tile = p.full_tiles + blockIdx.y;
+  const int pblk = tile / p.m_tiles;
+  int pi = 0;
+  while (pi + 1 < p.nphases && pblk >= p.phases[pi + 1].blk_begin) ++pi;
+  const Phase ph = p.phases[pi];
+  const int ipos = (pblk - ph.blk_begin) * BN + e % BN;
+  const int m = (tile % p.m_tiles) * BM + e / BN;
+  if (ipos >= ph.npos || m >= p.M) return;
+  const T *slot = static_cast<const T *>(p.partial) + (long long)blockIdx.y * p.tail_split * (BM * BN) + e;
+  const T sum = sum_in_order(slot, (long long)BM * BN, p.tail_split);
+  const int j12 = ph.J[1] * ph.J[2];
+  const unsigned pos = (unsigned)ipos;
+  const unsigned n = ph.by_jvol.div(pos);
+  unsigned r = pos - n * (unsigned)(ph.J[0] * j12);
+  const int j0 = (int)ph.by_j12.div(r);
+  r -= (unsigned)j0 * (unsigned)j12;
+  const int j1 = (int)ph.by_j2.div(r);
+  const int j2 = (int)r - j1 * ph.J[2];
+  T *out = static_cast<T *>(p.dst) + (long long)n * p.dst_nstride + (long long)(ph.o0[0] + j0 * p.oj[0]) * p.os[0] +
+           (long long)(ph.o0[1] + j1 * p.oj[1]) * p.os[1] + (long long)(ph.o0[2] + j2 * p.oj[2]) * p.os[2];
+  out[(long long)m * p.dst_mstride] = sum;
 }
 
 // ------------------------------------------------------------------------------------------
