@@ -262,6 +262,50 @@ def run_cpu_baseline(name, min_seconds=10.0, max_reps=200):
     }
 
 
+def run_dropin(name, steps=5):
+    """Wall time of the same step through the drop-in API (host arrays in, host arrays
+    out): includes the ctypes calls, uploads over PCIe and the download of every result."""
+    import mygrad_amd as mg
+    from mygrad_amd.nnet import conv_nd, max_pool
+
+    wl, dt = WORKLOADS[name], NP_DTYPE[WORKLOADS[name]["dtype"]]
+    rng = np.random.default_rng(wl["seed"])
+    x = rng.standard_normal(wl["x"]).astype(dt)
+    if wl["kind"] == "conv":
+        w = (rng.standard_normal(wl["w"]) * wl["wscale"]).astype(dt)
+        g = rng.standard_normal((wl["x"][0], wl["w"][0], *conv_grid(wl))).astype(dt)
+        valid = all((xx + 2 * p - ((t - 1) * d + 1)) % s == 0
+                    for xx, t, s, p, d in zip(wl["x"][2:], wl["w"][2:], wl["stride"], wl["padding"], wl["dilation"]))
+        if not valid:
+            return {"skipped": "the reference's validator rejects this shape; the drop-in raises ValueError like it"}
+
+        def once():
+            xt, wt = mg.Tensor(x, copy=False), mg.Tensor(w, copy=False)
+            out = conv_nd(xt, wt, stride=wl["stride"], padding=wl["padding"], dilation=wl["dilation"])
+            out.backward(g)
+
+        work, scale, unit = 3 * conv_flops_per_pass(wl), 1e-12, "TFLOP/s"
+    else:
+        lead, pooled, grid = pool_shapes(wl)
+        g = rng.standard_normal((*lead, *grid)).astype(dt)
+        if any((xx - p) % s for xx, p, s in zip(pooled, wl["pool"], wl["stride"])):
+            return {"skipped": "the reference's validator rejects this shape; the drop-in raises ValueError like it"}
+
+        def once():
+            xt = mg.Tensor(x, copy=False)
+            out = max_pool(xt, wl["pool"], wl["stride"])
+            out.backward(g)
+
+        work, scale, unit = 3 * x.nbytes + 2 * g.nbytes, 1e-9, "GB/s"
+    once()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        once()
+    elapsed = (time.perf_counter() - t0) / steps
+    return {"ms_per_step": elapsed * 1e3, "value": float(work * scale / elapsed), "unit": unit,
+            "note": "through Tensor.backward(), host ndarrays in and out (PCIe included)"}
+
+
 def run_copy_calibration(mib=1024, reps=20):
     """A plain 16-byte-per-lane device copy of known size: what the HBM traffic
     counters of a profile are scaled against, and the practical bandwidth ceiling."""
@@ -291,6 +335,8 @@ def main():
     ap.add_argument("--workload", default="conv3a", choices=sorted(WORKLOADS))
     ap.add_argument("--all", action="store_true", help="also run every other workload (reported under 'secondary')")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--dropin", action="store_true",
+                    help="also time the step through the Python drop-in API (reported under 'dropin', never as value)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a 1 GiB device copy (the reference point for HBM traffic counters)")
     args = ap.parse_args()
@@ -325,6 +371,8 @@ def main():
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = run_cpu_baseline(args.workload)
+    if args.dropin:
+        line["dropin"] = run_dropin(args.workload)
     if args.all:
         secondary = {}
         for name in WORKLOADS:
@@ -335,6 +383,8 @@ def main():
                      "ms_per_step": r["ms_per_step"], "roofline": r["roofline"], "kernels": r["kernels"]}
             if not args.no_cpu_baseline:
                 entry["cpu_baseline"] = run_cpu_baseline(name)
+            if args.dropin:
+                entry["dropin"] = run_dropin(name)
             secondary[name] = entry
         line["secondary"] = secondary
     print(json.dumps(line))
