@@ -569,6 +569,9 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
   double best_cost = 0;
   for (const Cfg &c : cfgs) {
     if (c.bm != bm || (c.tap_only && !tap_major)) continue;
+    // 64x64 fp64 wave tiles hold 128 accumulator registers: only one 8-wave block
+    // fits on a compute unit, so the tap-major kernels use the half-size shapes
+    if (tap_major && elem == 8 && c.bn * c.bm >= 128 * 128) continue;
     TileChoice t{};
     t.bm = c.bm;
     t.bn = c.bn;
@@ -912,7 +915,7 @@ void launch_gemm(const GemmParams &gp, const Plan &pl, hipStream_t s) {
     const long long tiles = (long long)pl.pos_blocks * pl.m_tiles;
     const long long tail_tiles = tiles - pl.full_tiles;
     hipLaunchKernelGGL((tap_gemm_kernel<T, BM, BN, BK, WM, WN>), dim3((unsigned)(pl.full_tiles + tail_tiles * pl.tail_split)),
-                       dim3(256), 0, s, gp);
+                       dim3(512), 0, s, gp);
     if (tail_tiles > 0)
       hipLaunchKernelGGL((tail_fixup_kernel<T, BM, BN>), dim3((unsigned)ceil_div(BM * BN, 256), (unsigned)tail_tiles),
                          dim3(256), 0, s, gp);

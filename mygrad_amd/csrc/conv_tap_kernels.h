@@ -53,7 +53,7 @@ __device__ __forceinline__ void store_vec(T *dst, const T (&src)[N]) {
 // forward and data gradient
 // ------------------------------------------------------------------------------------------
 template <typename T, int BM, int BN, int BK, int WM, int WN>
-__global__ void __launch_bounds__(256) tap_gemm_kernel(const GemmParams p) {
+__global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
   static_assert((BM / WM) * (BN / WN) == 4, "four wavefronts per block");
   static_assert(BK % 4 == 0 && WM % 16 == 0 && WN % 16 == 0 && BN % 64 == 0, "MFMA 16x16x4 tiling");
   constexpr int TM = WM / 16, TN = WN / 16;
@@ -68,11 +68,17 @@ __global__ void __launch_bounds__(256) tap_gemm_kernel(const GemmParams p) {
   __shared__ __attribute__((aligned(16))) T As[2][BK][LDA];
   __shared__ __attribute__((aligned(16))) T Bs[2][BK][LDB];
 
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wm0 = (wave / WAVES_N) * WM;
-  const int wn0 = (wave % WAVES_N) * WN;
+  // Eight wavefronts with two roles.  Waves 0-3 only read LDS and issue MFMAs; waves
+  // 4-7 only gather: global loads -> registers -> LDS, one tile ahead.  One of each
+  // sits on every SIMD, so the gather's address arithmetic, memory instructions and
+  // LDS stores are issued in the shadow of the other wave's MFMAs instead of taking
+  // turns with them in one instruction stream.
+  const int lane = threadIdx.x & 63;
+  const int wave = uniform(threadIdx.x >> 6);
+  const bool loader = wave >= 4;
+  const int tid = threadIdx.x & 255;  // index inside the role
+  const int wm0 = ((wave & 3) / WAVES_N) * WM;
+  const int wn0 = ((wave & 3) % WAVES_N) * WN;
   const int l16 = lane & 15, lk = lane >> 4;
 
   // Tiles are numbered with the row tile (m) innermost, so that the row tiles of one
@@ -152,12 +158,6 @@ __global__ void __launch_bounds__(256) tap_gemm_kernel(const GemmParams p) {
     for (int r = 0; r < BLOADS; ++r) Bs[buf][brow0 + r * BROWS][bcol] = rb[r];
   };
 
-  typename Mma<T>::Acc acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) acc[i][j] = typename Mma<T>::Acc{0, 0, 0, 0};
-
   // Lane (l16, lk) feeds row/column l16 of every 16x16 tile.  Tile i of the wave
   // takes the rows m = wm0 + l16*TM + i (and tile j the positions wn0 + l16*TN + j),
   // so the TM (TN) operands of a lane are adjacent in LDS and come in one read.
@@ -167,28 +167,51 @@ __global__ void __launch_bounds__(256) tap_gemm_kernel(const GemmParams p) {
     kt_begin = min(piece * per, ph.k_count);
     kt_end = min(kt_begin + per, ph.k_count);
   }
-  int buf = 0;
-  if (kt_begin < kt_end) {
-    fetch(kt_begin);
-    stash(0);
-  }
-  __syncthreads();
-  for (int kt = kt_begin; kt < kt_end; ++kt) {
-    const bool more = kt + 1 < kt_end;
-    if (more) fetch(kt + 1);
-#pragma unroll
-    for (int k4 = 0; k4 < BK / 4; ++k4) {
-      T a[TM], b[TN];
-      load_vec<T, TM>(&As[buf][k4 * 4 + lk][wm0 + l16 * TM], a);
-      load_vec<T, TN>(&Bs[buf][k4 * 4 + lk][wn0 + l16 * TN], b);
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::run(a[i], b[j], acc[i][j]);
+  // The two roles run separate loops (their registers never coexist) that meet at
+  // the same barriers: one after the first tile is in LDS, one per K tile.
+  if (loader) {
+    if (kt_begin < kt_end) {
+      fetch(kt_begin);
+      stash(0);
+      if (kt_begin + 1 < kt_end) fetch(kt_begin + 1);
     }
-    if (more) stash(buf ^ 1);
     __syncthreads();
-    buf ^= 1;
+    int buf = 0;
+    for (int kt = kt_begin; kt < kt_end; ++kt) {
+      // tile kt+1 was requested one iteration ago: park it in the idle buffer, then
+      // request tile kt+2
+      if (kt + 1 < kt_end) {
+        stash(buf ^ 1);
+        if (kt + 2 < kt_end) fetch(kt + 2);
+      }
+      __syncthreads();
+      buf ^= 1;
+    }
+    return;
+  }
+
+  typename Mma<T>::Acc acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = typename Mma<T>::Acc{0, 0, 0, 0};
+  __syncthreads();
+  {
+    int buf = 0;
+    for (int kt = kt_begin; kt < kt_end; ++kt) {
+#pragma unroll
+      for (int k4 = 0; k4 < BK / 4; ++k4) {
+        T a[TM], b[TN];
+        load_vec<T, TM>(&As[buf][k4 * 4 + lk][wm0 + l16 * TM], a);
+        load_vec<T, TN>(&Bs[buf][k4 * 4 + lk][wn0 + l16 * TN], b);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::run(a[i], b[j], acc[i][j]);
+      }
+      __syncthreads();
+      buf ^= 1;
+    }
   }
 
   // ---- epilogue
