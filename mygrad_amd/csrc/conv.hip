@@ -17,6 +17,7 @@
 #include "internal.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <string>
@@ -569,6 +570,7 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
   double best_cost = 0;
   for (const Cfg &c : cfgs) {
     if (c.bm != bm || (c.tap_only && !tap_major)) continue;
+    if (const char *force = getenv("MG_EXP_BN")) if (tap_major && atoi(force) != c.bn) continue;
     // 64x64 fp64 wave tiles hold 128 accumulator registers: only one 8-wave block
     // fits on a compute unit, so the tap-major kernels use the half-size shapes
     if (tap_major && elem == 8 && c.bn * c.bm >= 128 * 128) continue;

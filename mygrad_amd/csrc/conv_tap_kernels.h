@@ -134,9 +134,10 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
   const T *__restrict__ an = A + ((long long)arow0 * p.M + m0 + acol);
   const long long astep = a_ok ? (long long)AROWS * p.M : 0;
 
-  T ra[ALOADS], rb[BLOADS];
+  // two register sets: a tile is requested two iterations before it is parked in LDS
+  T ra0[ALOADS], rb0[BLOADS], ra1[ALOADS], rb1[BLOADS];
 
-  auto fetch = [&](int kt) {
+  auto fetch = [&](T(&ra)[ALOADS], T(&rb)[BLOADS], int kt) {
     const int8v e = ktab[kt];  // a_row0, coff, d0, d1, d2
     const T *ap = a_ok ? an + (long long)e[0] * p.M : zeros;
 #pragma unroll
@@ -148,7 +149,7 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
 #pragma unroll
     for (int r = 0; r < BLOADS; ++r) rb[r] = bp[r * bstep];
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](const T(&ra)[ALOADS], const T(&rb)[BLOADS], int buf) {
 #pragma unroll
     for (int r = 0; r < ALOADS; ++r) {
       const int kk = arow0 + r * AROWS;
@@ -170,22 +171,29 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
   // The two roles run separate loops (their registers never coexist) that meet at
   // the same barriers: one after the first tile is in LDS, one per K tile.
   if (loader) {
+    // tile kt_begin + i travels in register set i % 2
     if (kt_begin < kt_end) {
-      fetch(kt_begin);
-      stash(0);
-      if (kt_begin + 1 < kt_end) fetch(kt_begin + 1);
+      fetch(ra0, rb0, kt_begin);
+      stash(ra0, rb0, 0);
+      if (kt_begin + 1 < kt_end) fetch(ra1, rb1, kt_begin + 1);
+      if (kt_begin + 2 < kt_end) fetch(ra0, rb0, kt_begin + 2);
     }
     __syncthreads();
-    int buf = 0;
-    for (int kt = kt_begin; kt < kt_end; ++kt) {
-      // tile kt+1 was requested one iteration ago: park it in the idle buffer, then
-      // request tile kt+2
+    // each half of the loop body parks tile kt+1 (requested two iterations ago) in
+    // the idle buffer and requests tile kt+3 into the registers that just emptied
+    for (int kt = kt_begin; kt < kt_end; kt += 2) {
       if (kt + 1 < kt_end) {
-        stash(buf ^ 1);
-        if (kt + 2 < kt_end) fetch(kt + 2);
+        stash(ra1, rb1, 1);
+        if (kt + 3 < kt_end) fetch(ra1, rb1, kt + 3);
       }
       __syncthreads();
-      buf ^= 1;
+      if (kt + 1 < kt_end) {
+        if (kt + 2 < kt_end) {
+          stash(ra0, rb0, 0);
+          if (kt + 4 < kt_end) fetch(ra0, rb0, kt + 4);
+        }
+        __syncthreads();
+      }
     }
     return;
   }
