@@ -829,9 +829,9 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
 }
 
 template <typename K>
-int resident_blocks(K kernel) {
+int resident_blocks(K kernel, int threads) {
   int n = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, 0) != hipSuccess || n < 1) {
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, threads, 0) != hipSuccess || n < 1) {
     (void)hipGetLastError();
     n = 1;
   }
@@ -841,8 +841,8 @@ int resident_blocks(K kernel) {
 // Blocks of the filter-gradient kernel that fit on one compute unit at a time.
 int wgrad_blocks_per_cu(int dtype, int bm, bool tap_major) {
 #define MG_OCC(T, BM, BK, WM, WN)                                                    \
-  (tap_major ? resident_blocks(tap_wgrad_kernel<T, BM, 64, BK, WM, WN>)              \
-             : resident_blocks(wgrad_kernel<T, BM, 64, BK, WM, WN>))
+  (tap_major ? resident_blocks(tap_wgrad_kernel<T, BM, 64, BK, WM, WN>, 512)         \
+             : resident_blocks(wgrad_kernel<T, BM, 64, BK, WM, WN>, 256))
   if (dtype == MG_F32) return bm == 64 ? MG_OCC(float, 64, 64, 32, 32) : bm == 32 ? MG_OCC(float, 32, 64, 32, 16) : MG_OCC(float, 16, 64, 16, 16);
   return bm == 64 ? MG_OCC(double, 64, 32, 32, 32) : bm == 32 ? MG_OCC(double, 32, 32, 32, 16) : MG_OCC(double, 16, 32, 16, 16);
 #undef MG_OCC
@@ -1044,7 +1044,7 @@ void launch_wgrad(WgradParams &wp, bool tap_major, hipStream_t s) {
   if (tap_major) {
     // one-dimensional grid, whole K splits per XCD (see the kernel)
     const long long blocks = (long long)wp.splits * wp.col_tiles * wp.row_tiles;
-    hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN>), dim3((unsigned)blocks), dim3(256), 0, s, wp);
+    hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN>), dim3((unsigned)blocks), dim3(512), 0, s, wp);
   } else {
     const dim3 grid((unsigned)wp.col_tiles, (unsigned)wp.row_tiles, (unsigned)wp.splits);
     hipLaunchKernelGGL((wgrad_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, wp);

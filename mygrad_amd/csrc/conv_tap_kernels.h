@@ -341,7 +341,7 @@ __global__ void __launch_bounds__(256) tail_fixup_kernel(const GemmParams p) {
 // filter gradient
 // ------------------------------------------------------------------------------------------
 template <typename T, int BM, int BN, int BK, int WM, int WN>
-__global__ void __launch_bounds__(256) tap_wgrad_kernel(const WgradParams p) {
+__global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
   static_assert((BM / WM) * (BN / WN) == 4, "four wavefronts per block");
   static_assert(256 % BK == 0 && BK % 16 == 0 && BN % 16 == 0, "K tile");
   constexpr int TM = WM / 16, TN = WN / 16;
@@ -357,11 +357,14 @@ __global__ void __launch_bounds__(256) tap_wgrad_kernel(const WgradParams p) {
   __shared__ __attribute__((aligned(16))) T As[2][BM][LDK];  // grad tile   [f][position]
   __shared__ __attribute__((aligned(16))) T Bs[2][BN][LDK];  // window tile [column][position]
 
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wm0 = (wave / WAVES_N) * WM;
-  const int wn0 = (wave % WAVES_N) * WN;
+  // eight wavefronts, two roles, as in tap_gemm_kernel: waves 0-3 issue the MFMAs,
+  // waves 4-7 gather grad and x two K tiles ahead
+  const int lane = threadIdx.x & 63;
+  const int wave = uniform(threadIdx.x >> 6);
+  const bool loader = wave >= 4;
+  const int tid = threadIdx.x & 255;  // index inside the role
+  const int wm0 = ((wave & 3) / WAVES_N) * WM;
+  const int wn0 = ((wave & 3) % WAVES_N) * WN;
   const int l16 = lane & 15, lk = lane >> 4;
   // Blocks are handed to the 8 XCDs round-robin, and each XCD has its own L2.  All
   // tiles of one K split read the same positions of grad and x, so they are given to
@@ -396,9 +399,10 @@ __global__ void __launch_bounds__(256) tap_wgrad_kernel(const WgradParams p) {
 #pragma unroll
   for (int j = 0; j < NGROUPS; ++j) grp[j] = gtab[j];
 
-  T ra[ALOADS], rb[NGROUPS * GLOADS];
+  constexpr int NB = NGROUPS * GLOADS;
+  T ra0[ALOADS], rb0[NB], ra1[ALOADS], rb1[NB];
 
-  auto fetch = [&](int kt) {
+  auto fetch = [&](T(&ra)[ALOADS], T(&rb)[NB], int kt) {
     const int ipos = kbeg + kt * BK + kcol;
     const bool pos_ok = ipos < kend;
     const unsigned pos = pos_ok ? (unsigned)ipos : (unsigned)kbeg;
@@ -428,7 +432,7 @@ __global__ void __launch_bounds__(256) tap_wgrad_kernel(const WgradParams p) {
       for (int r = 0; r < GLOADS; ++r) rb[j * GLOADS + r] = bp[r * bstep];
     }
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](const T(&ra)[ALOADS], const T(&rb)[NB], int buf) {
 #pragma unroll
     for (int r = 0; r < ALOADS; ++r) As[buf][row0 + r * ROWS][kcol] = ra[r];
 #pragma unroll
@@ -436,6 +440,33 @@ __global__ void __launch_bounds__(256) tap_wgrad_kernel(const WgradParams p) {
 #pragma unroll
       for (int r = 0; r < GLOADS; ++r) Bs[buf][j * 16 + row0 + r * ROWS][kcol] = rb[j * GLOADS + r];
   };
+
+  const int ktiles = kend > kbeg ? (kend - kbeg + BK - 1) / BK : 0;
+  if (loader) {
+    // tile i travels in register set i % 2 and lands in LDS buffer i % 2
+    if (ktiles > 0) {
+      fetch(ra0, rb0, 0);
+      stash(ra0, rb0, 0);
+      if (1 < ktiles) fetch(ra1, rb1, 1);
+      if (2 < ktiles) fetch(ra0, rb0, 2);
+    }
+    __syncthreads();
+    for (int kt = 0; kt < ktiles; kt += 2) {
+      if (kt + 1 < ktiles) {
+        stash(ra1, rb1, 1);
+        if (kt + 3 < ktiles) fetch(ra1, rb1, kt + 3);
+      }
+      __syncthreads();
+      if (kt + 1 < ktiles) {
+        if (kt + 2 < ktiles) {
+          stash(ra0, rb0, 0);
+          if (kt + 4 < ktiles) fetch(ra0, rb0, kt + 4);
+        }
+        __syncthreads();
+      }
+    }
+    return;
+  }
 
   typename Mma<T>::Acc acc[TM][TN];
 #pragma unroll
@@ -446,16 +477,9 @@ __global__ void __launch_bounds__(256) tap_wgrad_kernel(const WgradParams p) {
   // The order in which the K tile is contracted is free: quarter-wave lk takes the
   // K indices lk*KQ .. lk*KQ+KQ-1, one per MFMA step, so that four steps' operands
   // of a lane are adjacent in LDS and come in one read.
-  const int ktiles = kend > kbeg ? (kend - kbeg + BK - 1) / BK : 0;
-  int buf = 0;
-  if (ktiles > 0) {
-    fetch(0);
-    stash(0);
-  }
   __syncthreads();
+  int buf = 0;
   for (int kt = 0; kt < ktiles; ++kt) {
-    const bool more = kt + 1 < ktiles;
-    if (more) fetch(kt + 1);
 #pragma unroll
     for (int s4 = 0; s4 < KQ / 4; ++s4) {
       T a[TM][4], b[TN][4];
@@ -490,7 +514,6 @@ __global__ void __launch_bounds__(256) tap_wgrad_kernel(const WgradParams p) {
 #pragma unroll
           for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::run(a[i][u], b[j][u], acc[i][j]);
     }
-    if (more) stash(buf ^ 1);
     __syncthreads();
     buf ^= 1;
   }
