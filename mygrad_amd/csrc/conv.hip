@@ -772,6 +772,12 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
         found.push_back(pt);
       }
 
+  // Phases with more taps have longer K loops; their blocks go first so that the
+  // short ones fill in at the end (blocks are dispatched in index order).
+  std::stable_sort(found.begin(), found.end(), [](const PhaseTaps &a, const PhaseTaps &b) {
+    return a.taps[0].size() * a.taps[1].size() * a.taps[2].size() > b.taps[0].size() * b.taps[1].size() * b.taps[2].size();
+  });
+
   // ---- tile shape and tail sharing
   {
     std::vector<long long> npos;
