@@ -243,7 +243,10 @@ struct ChunkInFlight {
 // Persistent blocks: each walks tiles blk, blk + gridDim.x, ...  While a tile is being
 // processed out of LDS, the next tile's x (and grad) are already on their way into
 // registers, so the memory system always has this block's next 16-48 KB in flight.
-template <typename T, typename TD, typename ACC, bool BWD, int DEPTH>
+// PSIG names a pool extent known at compile time, P0*100 + P1*10 + P2 (each 1..3), whose
+// window scan is fully unrolled: all its LDS reads are issued before the first compare
+// instead of one read-compare round trip per element; 0 = any extent, looped.
+template <typename T, typename TD, typename ACC, bool BWD, int DEPTH, int PSIG>
 __global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, const T *__restrict__ x,
                                                            const T *__restrict__ grad, void *__restrict__ result,
                                                            long long ntiles, int tile_elems, int win_slots,
@@ -293,17 +296,40 @@ __global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, con
                          (int)vol * p.xvol + t.pad;
       T best = tile[origin];
       int where = origin;
-      for (int a0 = 0; a0 < p.P[0]; ++a0)
-        for (int a1 = 0; a1 < p.P[1]; ++a1) {
-          const int rowoff = origin + (a0 * p.X[1] + a1) * p.X[2];
-          for (int a2 = 0; a2 < p.P[2]; ++a2) {
-            const T v = tile[rowoff + a2];
-            if (takes_over(v, best)) {
-              best = v;
-              where = rowoff + a2;
+      if constexpr (PSIG != 0) {
+        constexpr int Q0 = PSIG / 100, Q1 = (PSIG / 10) % 10, Q2 = PSIG % 10;
+        T v[Q0 * Q1 * Q2];
+#pragma unroll
+        for (int a0 = 0; a0 < Q0; ++a0)
+#pragma unroll
+          for (int a1 = 0; a1 < Q1; ++a1)
+#pragma unroll
+            for (int a2 = 0; a2 < Q2; ++a2) v[(a0 * Q1 + a1) * Q2 + a2] = tile[origin + (a0 * p.X[1] + a1) * p.X[2] + a2];
+#pragma unroll
+        for (int a0 = 0; a0 < Q0; ++a0)
+#pragma unroll
+          for (int a1 = 0; a1 < Q1; ++a1)
+#pragma unroll
+            for (int a2 = 0; a2 < Q2; ++a2) {
+              const T c = v[(a0 * Q1 + a1) * Q2 + a2];
+              if (takes_over(c, best)) {
+                best = c;
+                where = origin + (a0 * p.X[1] + a1) * p.X[2] + a2;
+              }
+            }
+      } else {
+        for (int a0 = 0; a0 < p.P[0]; ++a0)
+          for (int a1 = 0; a1 < p.P[1]; ++a1) {
+            const int rowoff = origin + (a0 * p.X[1] + a1) * p.X[2];
+            for (int a2 = 0; a2 < p.P[2]; ++a2) {
+              const T v = tile[rowoff + a2];
+              if (takes_over(v, best)) {
+                best = v;
+                where = rowoff + a2;
+              }
             }
           }
-        }
+      }
       if (BWD) {
         // Rank of this window among the windows that cover its argmax element, in
         // ascending row-major window order: per axis min(g, (P-1-a)/S) with a the
@@ -528,6 +554,12 @@ static unsigned persistent_grid(long long tiles, size_t lds_bytes) {
   return (unsigned)std::min<long long>(tiles, per_cu * pr.multiProcessorCount);
 }
 
+// Pool extents with an unrolled kernel instance (see PSIG); 0 selects the looped one.
+static int pool_signature(const PoolParams &p) {
+  const int sig = p.P[0] * 100 + p.P[1] * 10 + p.P[2];
+  return (p.P[0] <= 3 && p.P[1] <= 3 && p.P[2] <= 3 && (sig == 133 || sig == 122 || sig == 222)) ? sig : 0;
+}
+
 static unsigned grid_for(long long total) {
   long long blocks = ceil_div(total, 256);
   const long long cap = (long long)runtime().props.multiProcessorCount * 32;
@@ -558,15 +590,26 @@ int mg_maxpool_fwd(const mg_pool_desc *desc, const void *x, void *out) {
     // its stores trail the next tile's loads in the same in-order memory counter
     const dim3 grid((unsigned)blocks), block(256);
     const bool deep = (size_t)tile_elems * elem > 8 * 4096;  // 16-byte loads per thread to cover the tile
-#define MG_POOL_FWD(T, DEPTH)                                                                                   \
-  hipLaunchKernelGGL((maxpool_tile_kernel<T, T, T, false, DEPTH>), grid, block, lds, s, tp, (const T *)x,       \
+    const int sig = pool_signature(p);
+#define MG_POOL_FWD_SIG(T, DEPTH, SIG)                                                                          \
+  hipLaunchKernelGGL((maxpool_tile_kernel<T, T, T, false, DEPTH, SIG>), grid, block, lds, s, tp, (const T *)x,  \
                      (const T *)nullptr, out, blocks, tile_elems, win_slots, acc_offset)
+#define MG_POOL_FWD(T, DEPTH)                          \
+  do {                                                 \
+    switch (sig) {                                     \
+      case 133: MG_POOL_FWD_SIG(T, DEPTH, 133); break; \
+      case 122: MG_POOL_FWD_SIG(T, DEPTH, 122); break; \
+      case 222: MG_POOL_FWD_SIG(T, DEPTH, 222); break; \
+      default: MG_POOL_FWD_SIG(T, DEPTH, 0); break;    \
+    }                                                  \
+  } while (0)
     if (desc->dtype == MG_F32) {
       if (deep) MG_POOL_FWD(float, 12); else MG_POOL_FWD(float, 8);
     } else {
       if (deep) MG_POOL_FWD(double, 12); else MG_POOL_FWD(double, 8);
     }
 #undef MG_POOL_FWD
+#undef MG_POOL_FWD_SIG
     MG_HIP(hipGetLastError());
     return MG_OK;
   }
@@ -602,14 +645,25 @@ int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, vo
     const dim3 grid(persistent_grid(blocks, lds)), block(256);
     const bool wide = desc->dx_dtype == MG_F64;
     const bool deep = (size_t)tile_elems * elem > 8 * 4096;
-#define MG_POOL_BWD(T, TD, ACC)                                                                                 \
-  do {                                                                                                          \
-    if (deep)                                                                                                   \
-      hipLaunchKernelGGL((maxpool_tile_kernel<T, TD, ACC, true, 12>), grid, block, lds, s, tp, (const T *)x,    \
-                         (const T *)grad, dx, blocks, tile_elems, win_slots, acc_offset);                       \
-    else                                                                                                        \
-      hipLaunchKernelGGL((maxpool_tile_kernel<T, TD, ACC, true, 8>), grid, block, lds, s, tp, (const T *)x,     \
-                         (const T *)grad, dx, blocks, tile_elems, win_slots, acc_offset);                       \
+    const int sig = pool_signature(p);
+#define MG_POOL_BWD_SIG(T, TD, ACC, DEPTH, SIG)                                                                   \
+  hipLaunchKernelGGL((maxpool_tile_kernel<T, TD, ACC, true, DEPTH, SIG>), grid, block, lds, s, tp, (const T *)x,  \
+                     (const T *)grad, dx, blocks, tile_elems, win_slots, acc_offset)
+#define MG_POOL_BWD_D(T, TD, ACC, DEPTH)                          \
+  do {                                                            \
+    switch (sig) {                                                \
+      case 133: MG_POOL_BWD_SIG(T, TD, ACC, DEPTH, 133); break;   \
+      case 122: MG_POOL_BWD_SIG(T, TD, ACC, DEPTH, 122); break;   \
+      case 222: MG_POOL_BWD_SIG(T, TD, ACC, DEPTH, 222); break;   \
+      default: MG_POOL_BWD_SIG(T, TD, ACC, DEPTH, 0); break;      \
+    }                                                             \
+  } while (0)
+#define MG_POOL_BWD(T, TD, ACC)                   \
+  do {                                            \
+    if (deep)                                     \
+      MG_POOL_BWD_D(T, TD, ACC, 12);              \
+    else                                          \
+      MG_POOL_BWD_D(T, TD, ACC, 8);               \
   } while (0)
     if (!f32)
       MG_POOL_BWD(double, double, double);
@@ -622,6 +676,8 @@ int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, vo
     else
       MG_POOL_BWD(float, float, float);
 #undef MG_POOL_BWD
+#undef MG_POOL_BWD_D
+#undef MG_POOL_BWD_SIG
     MG_HIP(hipGetLastError());
     return MG_OK;
   }
