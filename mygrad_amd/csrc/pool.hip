@@ -354,8 +354,18 @@ __global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, con
     if (BWD) {
       __syncthreads();
       // ---- accumulators start at +0.0 (they may sit where the x tile was)
+      // in 16-byte stores; the round-up stays inside the tile's own LDS region
       const int used = t.chunk_len + t.pad;
-      for (int e = threadIdx.x; e < used; e += 256) acc[e] = ACC(0);
+      {
+        constexpr int VA = 16 / sizeof(ACC);
+        typedef ACC AVec __attribute__((ext_vector_type(VA), aligned(16)));
+        AVec zero;
+#pragma unroll
+        for (int i = 0; i < VA; ++i) zero[i] = ACC(0);
+        AVec *vacc = reinterpret_cast<AVec *>(acc);
+        const int nvec = (used + VA - 1) / VA;
+        for (int v = threadIdx.x; v < nvec; v += 256) vacc[v] = zero;
+      }
       __syncthreads();
 
       // ---- one pass per rank: every window of that rank adds its gradient to its
@@ -376,8 +386,27 @@ __global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, con
       const int own_first = p.bands > 1 ? t.own_lo * p.inner_x : 0;
       const int own_len = p.bands > 1 ? (t.own_hi - t.own_lo) * p.inner_x : t.nvol * p.xvol;
       const int shift = own_first - t.first_flat + t.pad;
-      TD *dx = static_cast<TD *>(result) + (t.l0 * p.xvol + own_first);
-      for (int e = threadIdx.x; e < own_len; e += 256) dx[e] = (TD)acc[e + shift];
+      // in 16-byte stores: dx index and LDS index are congruent modulo a 16-byte load
+      // of x (that is what pad is for), hence also modulo a 16-byte store of dx
+      constexpr int VD = 16 / sizeof(TD);
+      typedef TD DVec __attribute__((ext_vector_type(VD)));
+      constexpr int AALIGN = VD * sizeof(ACC) < 16 ? VD * sizeof(ACC) : 16;
+      typedef ACC SVec __attribute__((ext_vector_type(VD), aligned(AALIGN)));
+      const long long d0 = t.l0 * p.xvol + own_first;
+      TD *dx = static_cast<TD *>(result) + d0;
+      const int head = min(own_len, (VD - (int)(d0 % VD)) % VD);
+      const int body = (own_len - head) / VD;
+      DVec *vdx = reinterpret_cast<DVec *>(dx + head);
+      const SVec *from = reinterpret_cast<const SVec *>(acc + shift + head);
+      for (int v = threadIdx.x; v < body; v += 256) {
+        const SVec a = from[v];
+        DVec d;
+#pragma unroll
+        for (int i = 0; i < VD; ++i) d[i] = (TD)a[i];
+        vdx[v] = d;
+      }
+      for (int e = threadIdx.x; e < head; e += 256) dx[e] = (TD)acc[e + shift];
+      for (int e = head + body * VD + (int)threadIdx.x; e < own_len; e += 256) dx[e] = (TD)acc[e + shift];
     }
     __syncthreads();  // LDS is about to be overwritten by the next tile
     t = tn;
