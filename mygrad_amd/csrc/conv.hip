@@ -454,6 +454,15 @@ struct Geometry {
   long long xvol, wvol, gvol;
 };
 
+// The tap-major kernels address their operands with 32-bit byte offsets and mark
+// padding with an offset of 2 GiB, so every tensor they read must be smaller.
+bool fits_buffer_loads(const Geometry &g) {
+  const long long elem = g.dtype == MG_F64 ? 8 : 4;
+  const long long limit = 1ll << 31;
+  return (long long)g.N * g.C * g.xvol * elem < limit && (long long)g.N * g.F * g.gvol * elem < limit &&
+         (long long)g.F * g.C * g.wvol * elem < limit;
+}
+
 // K tile of the gather-GEMMs (positions x filters-or-channels x BK).
 int gemm_bk(int dtype) { return dtype == MG_F64 ? 8 : 16; }
 // K tile of the filter gradient (positions).
@@ -570,7 +579,6 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
   double best_cost = 0;
   for (const Cfg &c : cfgs) {
     if (c.bm != bm || (c.tap_only && !tap_major)) continue;
-    if (const char *force = getenv("MG_EXP_BN")) if (tap_major && atoi(force) != c.bn) continue;
     // 64x64 fp64 wave tiles hold 128 accumulator registers: only one 8-wave block
     // fits on a compute unit, so the tap-major kernels use the half-size shapes
     if (tap_major && elem == 8 && c.bn * c.bm >= 128 * 128) continue;
@@ -685,7 +693,7 @@ void fwd_table(const Geometry &g, std::vector<TabEntry> &tab) {
 int build_fwd_plan(const Geometry &g, Plan &pl) {
   Tables t;
   const int bk = gemm_bk(g.dtype);
-  pl.tap_major = g.C % bk == 0;
+  pl.tap_major = g.C % bk == 0 && fits_buffer_loads(g);
   pl.single_dense_phase = true;
   {
     const long long ktiles = pl.tap_major ? g.wvol * (g.C / bk) : ceil_div((long long)g.C * g.wvol, bk);
@@ -734,7 +742,7 @@ int build_fwd_plan(const Geometry &g, Plan &pl) {
 int build_dgrad_plan(const Geometry &g, Plan &pl) {
   Tables t;
   const int bk = gemm_bk(g.dtype);
-  pl.tap_major = g.F % bk == 0;
+  pl.tap_major = g.F % bk == 0 && fits_buffer_loads(g);
   pl.single_dense_phase = g.S[0] == 1 && g.S[1] == 1 && g.S[2] == 1;
   const int gs[3] = {g.G[1] * g.G[2], g.G[2], 1};
   long long nphase = (long long)g.S[0] * g.S[1] * g.S[2];
@@ -858,7 +866,7 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
   Tables t;
   pl.bm = g.F <= 16 ? 16 : (g.F <= 32 ? 32 : 64);
   pl.bn = 64;
-  pl.tap_major = g.C % 16 == 0 && g.F % pl.bm == 0;
+  pl.tap_major = g.C % 16 == 0 && g.F % pl.bm == 0 && fits_buffer_loads(g);
   const int bk = wgrad_bk(g.dtype);
   const long long ct = (long long)g.C * g.wvol;
   const long long col_tiles = ceil_div(ct, pl.bn);
@@ -1013,6 +1021,8 @@ int conv_fwd_impl(const Geometry &g, const Plan &pl, const void *x, const void *
   gp.src_cstride = (int)g.xvol;
   gp.src_nstride = (long long)g.C * g.xvol;
   gp.dst_nstride = (long long)g.F * g.gvol;
+  gp.a_bytes = (unsigned)((size_t)g.F * g.C * g.wvol * sizeof(T));
+  gp.src_bytes = pl.tap_major ? (unsigned)((size_t)g.N * g.C * g.xvol * sizeof(T)) : 0;
   return run_gemm<T>(gp, pl, TAG_CONV_FWD, runtime().stream);
 }
 
@@ -1040,6 +1050,8 @@ int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   gp.src_cstride = (int)g.gvol;
   gp.src_nstride = (long long)g.F * g.gvol;
   gp.dst_nstride = (long long)g.C * g.xvol;
+  gp.a_bytes = (unsigned)((size_t)g.F * g.C * g.wvol * sizeof(T));
+  gp.src_bytes = pl.tap_major ? (unsigned)((size_t)g.N * g.F * g.gvol * sizeof(T)) : 0;
   return run_gemm<T>(gp, pl, TAG_CONV_DGRAD, runtime().stream);
 }
 
@@ -1086,6 +1098,8 @@ int conv_wgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   }
   wp.gvol = (int)g.gvol;
   wp.x_cstride = (int)g.xvol;
+  wp.grad_bytes = pl.tap_major ? (unsigned)((size_t)g.N * g.F * g.gvol * sizeof(T)) : 0;
+  wp.x_bytes = pl.tap_major ? (unsigned)((size_t)g.N * g.C * g.xvol * sizeof(T)) : 0;
   wp.x_nstride = (long long)g.C * g.xvol;
   wp.g_nstride = (long long)g.F * g.gvol;
   wp.kpos = (int)((long long)g.N * g.gvol);

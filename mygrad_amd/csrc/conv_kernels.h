@@ -92,7 +92,8 @@ struct GemmParams {
   long long src_nstride, dst_nstride;
   // tap-major kernels only
   const KTile *ktiles;  // Phase::k_begin / k_count index this table
-  const void *zeros;    // a few zero elements in device memory: where padding loads point
+  const void *zeros;    // a few zero elements in device memory
+  unsigned a_bytes, src_bytes;  // sizes of A and src (each below 2 GiB)
   int src_cstride;      // element stride between consecutive channels of the gathered tensor
   int vec_store;        // positions are contiguous in dst: a lane may store its TN positions as one vector
   int m_tiles;          // row tiles per position block
@@ -120,6 +121,7 @@ struct WgradParams {
   const WGroup *groups;
   const void *zeros;
   int x_cstride;
+  unsigned grad_bytes, x_bytes;  // sizes of grad and x (each below 2 GiB)
   int col_tiles, row_tiles;  // tiles of the output matrix along columns / filters
 };
 

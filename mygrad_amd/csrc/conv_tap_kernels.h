@@ -49,6 +49,48 @@ __device__ __forceinline__ void store_vec(T *dst, const T (&src)[N]) {
   }
 }
 
+// Gathers go through buffer loads: address = base + per-lane byte offset (VGPR) +
+// wave-uniform byte offset (SGPR).  The channel step of a K tile's rows is uniform,
+// so it rides in the SGPR and costs no vector instruction per load, and a lane
+// whose tap falls in the padding gets a byte offset past the end of the buffer,
+// for which the hardware returns zero without touching memory.  Vector ALU
+// instructions of the loader waves are what the MFMA waves on the same SIMD wait
+// for, so the loaders issue as few of them as possible.
+// Tensors must be smaller than 2 GiB (kOutside must lie past the end).
+constexpr unsigned kOutside = 0x80000000u;
+
+template <typename T>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const void *base, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+
+template <typename T>
+__device__ __forceinline__ T buffer_load(__amdgpu_buffer_rsrc_t rsrc, unsigned lane_bytes, unsigned uniform_bytes) {
+  if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)lane_bytes, (int)uniform_bytes, 0));
+  } else {
+    return __builtin_bit_cast(T, __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)lane_bytes, (int)uniform_bytes, 0));
+  }
+}
+
+// Double precision runs on v_mfma_f64_4x4x4_4b_f64: four independent 4x4x4 products
+// ("blocks") per instruction, 16 cycles each, which reaches the device's fp64 matrix
+// peak; v_mfma_f64_16x16x4_f64 measured 105 cycles on gfx950, 61 % of that peak.
+// Lane l = 16*k + 4*b + r holds A[b][r][k], B[b][k][r] and (with k read as the row)
+// D[b][k][r].  The four blocks are laid out 2x2 over an 8x8 patch of the output:
+// block b covers rows 4*(b/2).. and columns 4*(b%2)..  With l16 = l % 16, lk = l / 16:
+//   lane feeds row  quad_row(l16) = 4*(l16/8) + l16%4  of the patch (two lanes share each),
+//        feeds column             l16 % 8              of the patch,
+//        holds D at row 4*(l16/8) + lk, column l16 % 8.
+struct Quad {
+  static __device__ __forceinline__ int feed_row(int l16) { return ((l16 >> 3) << 2) | (l16 & 3); }
+  static __device__ __forceinline__ int feed_col(int l16) { return l16 & 7; }
+  static __device__ __forceinline__ int held_row(int l16, int lk) { return ((l16 >> 3) << 2) | lk; }
+  static __device__ __forceinline__ double run(double a, double b, double c) {
+    return __builtin_amdgcn_mfma_f64_4x4x4f64(a, b, c, 0, 0, 0);
+  }
+};
+
 // ------------------------------------------------------------------------------------------
 // forward and data gradient
 // ------------------------------------------------------------------------------------------
@@ -104,8 +146,8 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
   const int j12 = ph.J[1] * ph.J[2];
   const int jvol = ph.J[0] * j12;
 
-  const T *__restrict__ A = static_cast<const T *>(p.A);
-  const T *__restrict__ zeros = static_cast<const T *>(p.zeros);
+  const __amdgpu_buffer_rsrc_t a_buf = buffer_of<T>(p.A, p.a_bytes);
+  const __amdgpu_buffer_rsrc_t src_buf = buffer_of<T>(p.src, p.src_bytes);
   const int8v MG_CONSTANT *ktab = (const int8v MG_CONSTANT *)(p.ktiles + ph.k_begin);
 
   // ---- this thread's column of the B tile: one output position
@@ -113,7 +155,7 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
   const int brow0 = uniform(tid / BN);
   int qb0, qb1, qb2;
   const bool pos_ok = pos0 + bcol < ph.npos;
-  const T *__restrict__ srcn = static_cast<const T *>(p.src);
+  unsigned src_at;  // byte offset of the position's tap (0,0,0), channel brow0
   {
     const unsigned pos = pos_ok ? (unsigned)(pos0 + bcol) : 0u;
     const unsigned n = ph.by_jvol.div(pos);
@@ -125,29 +167,30 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
     qb0 = (int)j0 * p.sj[0];
     qb1 = (int)j1 * p.sj[1];
     qb2 = (int)j2 * p.sj[2];
-    srcn += (long long)n * p.src_nstride + (qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2]) + brow0 * p.src_cstride;
+    src_at = (unsigned)((long long)n * p.src_nstride + (qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2]) +
+                        brow0 * p.src_cstride) * (unsigned)sizeof(T);
   }
   // ---- this thread's column of the A tile: one row m of the packed filters
   const int acol = tid % BM;
   const int arow0 = BM % 64 == 0 ? uniform(tid / BM) : tid / BM;
   const bool a_ok = (m0 + acol < p.M) & (arow0 < BK);
-  const T *__restrict__ an = A + ((long long)arow0 * p.M + m0 + acol);
-  const long long astep = a_ok ? (long long)AROWS * p.M : 0;
+  const unsigned a_at = a_ok ? (unsigned)(arow0 * p.M + m0 + acol) * (unsigned)sizeof(T) : kOutside;
+  const unsigned a_row_bytes = (unsigned)p.M * (unsigned)sizeof(T);
+  const unsigned b_step = (unsigned)(BROWS * p.src_cstride) * (unsigned)sizeof(T);
 
   // two register sets: a tile is requested two iterations before it is parked in LDS
   T ra0[ALOADS], rb0[BLOADS], ra1[ALOADS], rb1[BLOADS];
 
   auto fetch = [&](T(&ra)[ALOADS], T(&rb)[BLOADS], int kt) {
     const int8v e = ktab[kt];  // a_row0, coff, d0, d1, d2
-    const T *ap = a_ok ? an + (long long)e[0] * p.M : zeros;
+    const unsigned a_tile = (unsigned)e[0] * a_row_bytes;
 #pragma unroll
-    for (int r = 0; r < ALOADS; ++r) ra[r] = ap[r * astep];
+    for (int r = 0; r < ALOADS; ++r) ra[r] = buffer_load<T>(a_buf, a_at, a_tile + (unsigned)(r * AROWS) * a_row_bytes);
     const bool ok = pos_ok & ((unsigned)(qb0 + e[2]) < (unsigned)p.Q[0]) & ((unsigned)(qb1 + e[3]) < (unsigned)p.Q[1]) &
                     ((unsigned)(qb2 + e[4]) < (unsigned)p.Q[2]);
-    const T *bp = ok ? srcn + e[1] : zeros;
-    const long long bstep = ok ? (long long)(BROWS * p.src_cstride) : 0;
+    const unsigned at = ok ? src_at + (unsigned)(e[1] * (int)sizeof(T)) : kOutside;
 #pragma unroll
-    for (int r = 0; r < BLOADS; ++r) rb[r] = bp[r * bstep];
+    for (int r = 0; r < BLOADS; ++r) rb[r] = buffer_load<T>(src_buf, at, (unsigned)r * b_step);
   };
   auto stash = [&](const T(&ra)[ALOADS], const T(&rb)[BLOADS], int buf) {
 #pragma unroll
@@ -171,28 +214,123 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
   // The two roles run separate loops (their registers never coexist) that meet at
   // the same barriers: one after the first tile is in LDS, one per K tile.
   if (loader) {
-    // tile kt_begin + i travels in register set i % 2
+    // Tile kt_begin + i travels in register set i % 2.  Every path through this loop
+    // issues the same loads in the same order (tile indices past the end are clamped
+    // and their data is never read): only then can the compiler wait for exactly the
+    // older register set and leave the newer one's loads in flight.
+    const int last = kt_end - 1;
     if (kt_begin < kt_end) {
       fetch(ra0, rb0, kt_begin);
       stash(ra0, rb0, 0);
-      if (kt_begin + 1 < kt_end) fetch(ra1, rb1, kt_begin + 1);
-      if (kt_begin + 2 < kt_end) fetch(ra0, rb0, kt_begin + 2);
+      fetch(ra1, rb1, min(kt_begin + 1, last));
+      fetch(ra0, rb0, min(kt_begin + 2, last));
     }
     __syncthreads();
     // each half of the loop body parks tile kt+1 (requested two iterations ago) in
     // the idle buffer and requests tile kt+3 into the registers that just emptied
-    for (int kt = kt_begin; kt < kt_end; kt += 2) {
-      if (kt + 1 < kt_end) {
-        stash(ra1, rb1, 1);
-        if (kt + 3 < kt_end) fetch(ra1, rb1, kt + 3);
+    int kt = kt_begin;
+    for (; kt + 1 < kt_end; kt += 2) {
+      stash(ra1, rb1, 1);
+      fetch(ra1, rb1, min(kt + 3, last));
+      __syncthreads();
+      stash(ra0, rb0, 0);
+      fetch(ra0, rb0, min(kt + 4, last));
+      __syncthreads();
+    }
+    if (kt < kt_end) __syncthreads();
+    return;
+  }
+
+  T *__restrict__ dst = static_cast<T *>(p.dst);
+  auto dst_of = [&](int ipos) -> T * {
+    const unsigned pos = (unsigned)ipos;
+    const unsigned n = ph.by_jvol.div(pos);
+    unsigned r = pos - n * (unsigned)jvol;
+    const int j0 = (int)ph.by_j12.div(r);
+    r -= (unsigned)j0 * (unsigned)j12;
+    const int j1 = (int)ph.by_j2.div(r);
+    const int j2 = (int)r - j1 * ph.J[2];
+    return dst + (long long)n * p.dst_nstride + (long long)(ph.o0[0] + j0 * p.oj[0]) * p.os[0] +
+           (long long)(ph.o0[1] + j1 * p.oj[1]) * p.os[1] + (long long)(ph.o0[2] + j2 * p.oj[2]) * p.os[2];
+  };
+
+  if constexpr (sizeof(T) == 8) {
+    // The wave tile is cut into 8-row and 8-column groups; group pairs are interleaved
+    // (row = pair*16 + 2*patch_row + half) so that a lane's two operands of a pair are
+    // adjacent in LDS and the 8 distinct lanes of a read cover 128 contiguous bytes.
+    constexpr int GM = WM / 8, GN = WN / 8;
+    const int arow = wm0 + Quad::feed_row(l16) * 2;
+    const int bcol8 = wn0 + Quad::feed_col(l16) * 2;
+    const int drow = wm0 + Quad::held_row(l16, lk) * 2;
+    double acc[GM][GN];
+#pragma unroll
+    for (int i = 0; i < GM; ++i)
+#pragma unroll
+      for (int j = 0; j < GN; ++j) acc[i][j] = 0.0;
+    __syncthreads();
+    int buf = 0;
+    for (int kt = kt_begin; kt < kt_end; ++kt) {
+#pragma unroll
+      for (int k4 = 0; k4 < BK / 4; ++k4) {
+        T a[GM], b[GN];
+#pragma unroll
+        for (int g = 0; g < GM / 2; ++g) {
+          T two[2];
+          load_vec<T, 2>(&As[buf][k4 * 4 + lk][arow + g * 16], two);
+          a[2 * g] = two[0], a[2 * g + 1] = two[1];
+        }
+#pragma unroll
+        for (int g = 0; g < GN / 2; ++g) {
+          T two[2];
+          load_vec<T, 2>(&Bs[buf][k4 * 4 + lk][bcol8 + g * 16], two);
+          b[2 * g] = two[0], b[2 * g + 1] = two[1];
+        }
+#pragma unroll
+        for (int i = 0; i < GM; ++i)
+#pragma unroll
+          for (int j = 0; j < GN; ++j) acc[i][j] = Quad::run(a[i], b[j], acc[i][j]);
       }
       __syncthreads();
-      if (kt + 1 < kt_end) {
-        if (kt + 2 < kt_end) {
-          stash(ra0, rb0, 0);
-          if (kt + 4 < kt_end) fetch(ra0, rb0, kt + 4);
+      buf ^= 1;
+    }
+    // ---- epilogue: acc[i][j] is row drow + (i/2)*16 + i%2, column bcol8 + (j/2)*16 + j%2
+    if (partial) {
+      T *slot = static_cast<T *>(p.partial) + ((long long)(tile - p.full_tiles) * p.tail_split + piece) * (BM * BN);
+#pragma unroll
+      for (int i = 0; i < GM; ++i) {
+        const int ml = drow + (i / 2) * 16 + i % 2;
+#pragma unroll
+        for (int g = 0; g < GN / 2; ++g) {
+          const T two[2] = {acc[i][2 * g], acc[i][2 * g + 1]};
+          store_vec<T, 2>(slot + ml * BN + bcol8 + g * 16, two);
         }
-        __syncthreads();
+      }
+      return;
+    }
+#pragma unroll
+    for (int g = 0; g < GN / 2; ++g) {
+      const int first = pos0 + bcol8 + g * 16;
+      if (p.vec_store) {
+        // both positions exist (npos % 4 == 0) and are adjacent in dst
+        if (first >= ph.npos) continue;
+        T *out = dst_of(first);
+#pragma unroll
+        for (int i = 0; i < GM; ++i) {
+          const int m = m0 + drow + (i / 2) * 16 + i % 2;
+          const T two[2] = {acc[i][2 * g], acc[i][2 * g + 1]};
+          if (m < p.M) store_vec<T, 2>(out + (long long)m * p.dst_mstride, two);
+        }
+      } else {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          if (first + h >= ph.npos) continue;
+          T *out = dst_of(first + h);
+#pragma unroll
+          for (int i = 0; i < GM; ++i) {
+            const int m = m0 + drow + (i / 2) * 16 + i % 2;
+            if (m < p.M) out[(long long)m * p.dst_mstride] = acc[i][2 * g + h];
+          }
+        }
       }
     }
     return;
@@ -250,18 +388,6 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
       }
     return;
   }
-  T *__restrict__ dst = static_cast<T *>(p.dst);
-  auto dst_of = [&](int ipos) -> T * {
-    const unsigned pos = (unsigned)ipos;
-    const unsigned n = ph.by_jvol.div(pos);
-    unsigned r = pos - n * (unsigned)jvol;
-    const int j0 = (int)ph.by_j12.div(r);
-    r -= (unsigned)j0 * (unsigned)j12;
-    const int j1 = (int)ph.by_j2.div(r);
-    const int j2 = (int)r - j1 * ph.J[2];
-    return dst + (long long)n * p.dst_nstride + (long long)(ph.o0[0] + j0 * p.oj[0]) * p.os[0] +
-           (long long)(ph.o0[1] + j1 * p.oj[1]) * p.os[1] + (long long)(ph.o0[2] + j2 * p.oj[2]) * p.os[2];
-  };
   const int first = pos0 + wn0 + l16 * TN;
   if (p.vec_store) {
     // the TN positions of this lane are adjacent in dst and all exist (npos % TN == 0)
@@ -386,9 +512,8 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
   const int kbeg = split * p.kchunk;
   const int kend = min(kbeg + p.kchunk, p.kpos);
 
-  const T *__restrict__ grad = static_cast<const T *>(p.grad);
-  const T *__restrict__ x = static_cast<const T *>(p.x);
-  const T *__restrict__ zeros = static_cast<const T *>(p.zeros);
+  const __amdgpu_buffer_rsrc_t grad_buf = buffer_of<T>(p.grad, p.grad_bytes);
+  const __amdgpu_buffer_rsrc_t x_buf = buffer_of<T>(p.x, p.x_bytes);
   const int kcol = tid % BK;
   const int row0 = BK % 64 == 0 ? uniform(tid / BK) : tid / BK;
   const int g12 = p.G[1] * p.G[2];
@@ -401,6 +526,8 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
 
   constexpr int NB = NGROUPS * GLOADS;
   T ra0[ALOADS], rb0[NB], ra1[ALOADS], rb1[NB];
+  const unsigned a_step = (unsigned)(ROWS * p.gvol) * (unsigned)sizeof(T);
+  const unsigned b_step = (unsigned)(ROWS * p.x_cstride) * (unsigned)sizeof(T);
 
   auto fetch = [&](T(&ra)[ALOADS], T(&rb)[NB], int kt) {
     const int ipos = kbeg + kt * BK + kcol;
@@ -415,21 +542,20 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
     const int qb0 = (int)g0 * p.sj[0];
     const int qb1 = (int)g1 * p.sj[1];
     const int qb2 = (int)g2 * p.sj[2];
-    const T *ap = pos_ok ? grad + ((long long)n * p.g_nstride + gflat + (long long)(m0 + row0) * p.gvol) : zeros;
-    const long long astep = pos_ok ? (long long)ROWS * p.gvol : 0;
+    const unsigned g_at =
+        pos_ok ? (unsigned)((long long)n * p.g_nstride + gflat + (long long)(m0 + row0) * p.gvol) * (unsigned)sizeof(T) : kOutside;
 #pragma unroll
-    for (int r = 0; r < ALOADS; ++r) ra[r] = ap[r * astep];
-    const T *xn = x + ((long long)n * p.x_nstride + (qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2]) +
-                       (long long)row0 * p.x_cstride);
+    for (int r = 0; r < ALOADS; ++r) ra[r] = buffer_load<T>(grad_buf, g_at, (unsigned)r * a_step);
+    const unsigned x_at = (unsigned)((long long)n * p.x_nstride + (qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2]) +
+                                     (long long)row0 * p.x_cstride) * (unsigned)sizeof(T);
 #pragma unroll
     for (int j = 0; j < NGROUPS; ++j) {
       const int8v e = grp[j];  // coff, d0, d1, d2, valid
       const bool ok = pos_ok & (e[4] != 0) & ((unsigned)(qb0 + e[1]) < (unsigned)p.Q[0]) &
                       ((unsigned)(qb1 + e[2]) < (unsigned)p.Q[1]) & ((unsigned)(qb2 + e[3]) < (unsigned)p.Q[2]);
-      const T *bp = ok ? xn + e[0] : zeros;
-      const long long bstep = ok ? (long long)ROWS * p.x_cstride : 0;
+      const unsigned at = ok ? x_at + (unsigned)(e[0] * (int)sizeof(T)) : kOutside;
 #pragma unroll
-      for (int r = 0; r < GLOADS; ++r) rb[j * GLOADS + r] = bp[r * bstep];
+      for (int r = 0; r < GLOADS; ++r) rb[j * GLOADS + r] = buffer_load<T>(x_buf, at, (unsigned)r * b_step);
     }
   };
   auto stash = [&](const T(&ra)[ALOADS], const T(&rb)[NB], int buf) {
@@ -443,26 +569,82 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
 
   const int ktiles = kend > kbeg ? (kend - kbeg + BK - 1) / BK : 0;
   if (loader) {
-    // tile i travels in register set i % 2 and lands in LDS buffer i % 2
+    // tile i travels in register set i % 2 and lands in LDS buffer i % 2; the loads
+    // of every path are the same (see tap_gemm_kernel), tiles past the end are clamped
+    const int last = ktiles - 1;
     if (ktiles > 0) {
       fetch(ra0, rb0, 0);
       stash(ra0, rb0, 0);
-      if (1 < ktiles) fetch(ra1, rb1, 1);
-      if (2 < ktiles) fetch(ra0, rb0, 2);
+      fetch(ra1, rb1, min(1, last));
+      fetch(ra0, rb0, min(2, last));
     }
     __syncthreads();
-    for (int kt = 0; kt < ktiles; kt += 2) {
-      if (kt + 1 < ktiles) {
-        stash(ra1, rb1, 1);
-        if (kt + 3 < ktiles) fetch(ra1, rb1, kt + 3);
+    int kt = 0;
+    for (; kt + 1 < ktiles; kt += 2) {
+      stash(ra1, rb1, 1);
+      fetch(ra1, rb1, min(kt + 3, last));
+      __syncthreads();
+      stash(ra0, rb0, 0);
+      fetch(ra0, rb0, min(kt + 4, last));
+      __syncthreads();
+    }
+    if (kt < ktiles) __syncthreads();
+    return;
+  }
+
+  if constexpr (sizeof(T) == 8) {
+    // 4x4x4 four-block MFMAs on 8-row x 8-column patches (see Quad); quarter-wave lk
+    // contracts the K indices lk*KQ .. lk*KQ+KQ-1, four adjacent ones per LDS read
+    constexpr int GM = WM / 8, GN = WN / 8;
+    const int arow = wm0 + Quad::feed_row(l16);
+    const int bcol8 = wn0 + Quad::feed_col(l16);
+    const int drow = wm0 + Quad::held_row(l16, lk);
+    double acc[GM][GN];
+#pragma unroll
+    for (int i = 0; i < GM; ++i)
+#pragma unroll
+      for (int j = 0; j < GN; ++j) acc[i][j] = 0.0;
+    __syncthreads();
+    int buf = 0;
+    for (int kt = 0; kt < ktiles; ++kt) {
+#pragma unroll
+      for (int s4 = 0; s4 < KQ / 4; ++s4) {
+        T a[GM][4], b[GN][4];
+#pragma unroll
+        for (int i = 0; i < GM; ++i) {
+          const T *src = &As[buf][arow + i * 8][lk * KQ + s4 * 4];
+          T lo[2], hi[2];
+          load_vec<T, 2>(src, lo);
+          load_vec<T, 2>(src + 2, hi);
+          a[i][0] = lo[0], a[i][1] = lo[1], a[i][2] = hi[0], a[i][3] = hi[1];
+        }
+#pragma unroll
+        for (int j = 0; j < GN; ++j) {
+          const T *src = &Bs[buf][bcol8 + j * 8][lk * KQ + s4 * 4];
+          T lo[2], hi[2];
+          load_vec<T, 2>(src, lo);
+          load_vec<T, 2>(src + 2, hi);
+          b[j][0] = lo[0], b[j][1] = lo[1], b[j][2] = hi[0], b[j][3] = hi[1];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int i = 0; i < GM; ++i)
+#pragma unroll
+            for (int j = 0; j < GN; ++j) acc[i][j] = Quad::run(a[i][u], b[j][u], acc[i][j]);
       }
       __syncthreads();
-      if (kt + 1 < ktiles) {
-        if (kt + 2 < ktiles) {
-          stash(ra0, rb0, 0);
-          if (kt + 4 < ktiles) fetch(ra0, rb0, kt + 4);
-        }
-        __syncthreads();
+      buf ^= 1;
+    }
+    T *__restrict__ out = static_cast<T *>(p.out) + (long long)split * p.F * p.CT;
+#pragma unroll
+    for (int j = 0; j < GN; ++j) {
+      const int col = n0 + bcol8 + j * 8;
+      if (col >= p.CT) continue;
+#pragma unroll
+      for (int i = 0; i < GM; ++i) {
+        const int f = m0 + drow + i * 8;
+        if (f < p.F) out[(long long)f * p.CT + col] = acc[i][j];
       }
     }
     return;
