@@ -465,8 +465,6 @@ bool fits_buffer_loads(const Geometry &g) {
 
 // K tile of the gather-GEMMs (positions x filters-or-channels x BK).
 int gemm_bk(int dtype) { return dtype == MG_F64 ? 8 : 16; }
-// K tile of the filter gradient (positions).
-int wgrad_bk(int dtype) { return dtype == MG_F64 ? 32 : 64; }
 
 struct Plan {
   void *blob = nullptr;  // one device allocation holding every table below
@@ -479,6 +477,7 @@ struct Plan {
   int nphases = 0;
   int pos_blocks = 0;  // position blocks of the gather-GEMM (all phases)
   int bm = 0, bn = 0;
+  int bk = 0;           // K tile of the filter-gradient kernel chosen for this plan
   int m_tiles = 1;     // row tiles per position block
   int full_tiles = 0;  // tiles computed whole by one block (tap-major kernel)
   int tail_split = 1;  // blocks sharing each of the remaining tiles
@@ -852,36 +851,85 @@ int resident_blocks(K kernel, int threads) {
   return n;
 }
 
+// Tile shapes of the filter-gradient kernels: rows (filters) x columns x K tile, and the
+// wave tile.  The table-driven kernel has the 64-column shapes only.
+#define MG_WGRAD_SHAPES(T, X)                                                          \
+  X(T, 128, 128, (sizeof(T) == 8 ? 16 : 32), 64, 64)                                   \
+  X(T, 64, 128, (sizeof(T) == 8 ? 16 : 32), 32, 64)                                    \
+  X(T, 64, 64, (sizeof(T) == 8 ? 32 : 64), 32, 32)                                     \
+  X(T, 32, 64, (sizeof(T) == 8 ? 32 : 64), 32, 16)                                     \
+  X(T, 16, 64, (sizeof(T) == 8 ? 32 : 64), 16, 16)
+
 // Blocks of the filter-gradient kernel that fit on one compute unit at a time.
-int wgrad_blocks_per_cu(int dtype, int bm, bool tap_major) {
-#define MG_OCC(T, BM, BK, WM, WN)                                                    \
-  (tap_major ? resident_blocks(tap_wgrad_kernel<T, BM, 64, BK, WM, WN>, 512)         \
-             : resident_blocks(wgrad_kernel<T, BM, 64, BK, WM, WN>, 256))
-  if (dtype == MG_F32) return bm == 64 ? MG_OCC(float, 64, 64, 32, 32) : bm == 32 ? MG_OCC(float, 32, 64, 32, 16) : MG_OCC(float, 16, 64, 16, 16);
-  return bm == 64 ? MG_OCC(double, 64, 32, 32, 32) : bm == 32 ? MG_OCC(double, 32, 32, 32, 16) : MG_OCC(double, 16, 32, 16, 16);
+template <typename T>
+int wgrad_blocks_per_cu(int bm, int bn, bool tap_major) {
+#define MG_OCC(TT, BM, BN, BK, WM, WN)                                                     \
+  if (bm == BM && bn == BN) {                                                              \
+    if (tap_major) return resident_blocks(tap_wgrad_kernel<TT, BM, BN, BK, WM, WN>, 512);  \
+    if constexpr (BN == 64) return resident_blocks(wgrad_kernel<TT, BM, BN, BK, WM, WN>, 256); \
+  }
+  MG_WGRAD_SHAPES(T, MG_OCC)
 #undef MG_OCC
+  return 1;
 }
 
 int build_wgrad_plan(const Geometry &g, Plan &pl) {
   Tables t;
-  pl.bm = g.F <= 16 ? 16 : (g.F <= 32 ? 32 : 64);
-  pl.bn = 64;
-  pl.tap_major = g.C % 16 == 0 && g.F % pl.bm == 0 && fits_buffer_loads(g);
-  const int bk = wgrad_bk(g.dtype);
+  const bool f64 = g.dtype == MG_F64;
   const long long ct = (long long)g.C * g.wvol;
-  const long long col_tiles = ceil_div(ct, pl.bn);
-  const long long tiles = ceil_div(g.F, pl.bm) * col_tiles;
   const long long kpos = (long long)g.N * g.gvol;
-  const long long ktiles = ceil_div(kpos, bk);
+  const int cus = runtime().props.multiProcessorCount;
   // Split K so that all blocks are resident at once (one round: no half-empty second
   // round), with at least 4 K tiles per block.  The tap-major kernel hands whole
   // splits to the 8 XCDs, so a multiple of 8 is preferred when one fits.
-  const long long slots = (long long)wgrad_blocks_per_cu(g.dtype, pl.bm, pl.tap_major) * runtime().props.multiProcessorCount;
-  const long long max_splits = std::max<long long>(1, std::min<long long>(ktiles / 4, 1024));
-  long long splits = std::max<long long>(1, std::min(slots / tiles, max_splits));
-  if (splits >= 8) splits = splits / 8 * 8;
-  long long tiles_per_split = ceil_div(ktiles, splits);
-  pl.kchunk = (int)(tiles_per_split * bk);
+  auto splits_for = [&](int bm, int bn, int bk, bool tap) {
+    const long long tiles = ceil_div(ct, bn) * ceil_div(g.F, bm);
+    const long long ktiles = ceil_div(kpos, bk);
+    const int per_cu = f64 ? wgrad_blocks_per_cu<double>(bm, bn, tap) : wgrad_blocks_per_cu<float>(bm, bn, tap);
+    const long long slots = (long long)per_cu * cus;
+    const long long max_splits = std::max<long long>(1, std::min<long long>(ktiles / 4, 1024));
+    long long splits = std::max<long long>(1, std::min(slots / tiles, max_splits));
+    if (splits >= 8) splits = splits / 8 * 8;
+    return splits;
+  };
+  // Tap-major candidates, largest first.  A larger tile re-reads grad and x less often
+  // (the kernel is limited by what it pulls through L1, not by HBM), so the first
+  // shape wins that divides F, wastes little on padding the columns to whole tiles
+  // and still fills most block slots of the device with tiles x K splits.
+  struct Cand {
+    int bm, bn, bk;
+  };
+  const Cand cands[] = {{128, 128, f64 ? 16 : 32}, {64, 128, f64 ? 16 : 32}, {64, 64, f64 ? 32 : 64},
+                        {32, 64, f64 ? 32 : 64},   {16, 64, f64 ? 32 : 64}};
+  long long best_splits = 1;
+  pl.bm = 0;
+  if (g.C % 16 == 0 && fits_buffer_loads(g)) {
+    for (const Cand &c : cands) {
+      if (g.F % c.bm != 0) continue;
+      const long long col_tiles = ceil_div(ct, c.bn), row_tiles = g.F / c.bm;
+      const long long splits = splits_for(c.bm, c.bn, c.bk, true);
+      if (c.bn > 64) {
+        const int per_cu = f64 ? wgrad_blocks_per_cu<double>(c.bm, c.bn, true) : wgrad_blocks_per_cu<float>(c.bm, c.bn, true);
+        const double waste = (double)(col_tiles * c.bn - ct) / (double)ct;
+        const double filled = (double)(col_tiles * row_tiles * splits) / ((double)per_cu * cus);
+        if (waste > 0.06 || filled < 0.75) continue;
+      }
+      best_splits = splits;
+      pl.bm = c.bm, pl.bn = c.bn, pl.bk = c.bk;
+      break;
+    }
+  }
+  pl.tap_major = pl.bm != 0;
+  if (!pl.tap_major) {
+    pl.bm = g.F <= 16 ? 16 : (g.F <= 32 ? 32 : 64);
+    pl.bn = 64;
+    pl.bk = f64 ? 32 : 64;
+    best_splits = splits_for(pl.bm, pl.bn, pl.bk, false);
+  }
+  const long long col_tiles = ceil_div(ct, pl.bn);
+  const long long ktiles = ceil_div(kpos, pl.bk);
+  const long long tiles_per_split = ceil_div(ktiles, best_splits);
+  pl.kchunk = (int)(tiles_per_split * pl.bk);
   pl.splits = (int)ceil_div(kpos, pl.kchunk);
   if (pl.tap_major) {
     const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
@@ -1063,7 +1111,7 @@ void launch_wgrad(WgradParams &wp, bool tap_major, hipStream_t s) {
     // one-dimensional grid, whole K splits per XCD (see the kernel)
     const long long blocks = (long long)wp.splits * wp.col_tiles * wp.row_tiles;
     hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN>), dim3((unsigned)blocks), dim3(512), 0, s, wp);
-  } else {
+  } else if constexpr (BN == 64) {
     const dim3 grid((unsigned)wp.col_tiles, (unsigned)wp.row_tiles, (unsigned)wp.splits);
     hipLaunchKernelGGL((wgrad_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, wp);
   }
@@ -1071,7 +1119,6 @@ void launch_wgrad(WgradParams &wp, bool tap_major, hipStream_t s) {
 
 template <typename T>
 int conv_wgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const void *x, void *dw) {
-  constexpr int BK = sizeof(T) == 8 ? 32 : 64;
   hipStream_t s = runtime().stream;
   const int ct = (int)(g.C * g.wvol);
   // The tap-major kernel writes its columns in (tap, channel) order, so its result
@@ -1110,11 +1157,15 @@ int conv_wgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   wp.by_g2 = make_fastdiv((unsigned)g.G[2]);
   {
     ScopedTiming timed(TAG_CONV_WGRAD);
-    switch (pl.bm) {
-      case 64: launch_wgrad<T, 64, 64, BK, 32, 32>(wp, pl.tap_major, s); break;
-      case 32: launch_wgrad<T, 32, 64, BK, 32, 16>(wp, pl.tap_major, s); break;
-      default: launch_wgrad<T, 16, 64, BK, 16, 16>(wp, pl.tap_major, s); break;
-    }
+    bool launched = false;
+#define MG_LAUNCH(TT, BM, BN, BK, WM, WN)                               \
+  if (!launched && pl.bm == BM && pl.bn == BN) {                        \
+    launch_wgrad<TT, BM, BN, BK, WM, WN>(wp, pl.tap_major, s);          \
+    launched = true;                                                    \
+  }
+    MG_WGRAD_SHAPES(T, MG_LAUNCH)
+#undef MG_LAUNCH
+    if (!launched) return fail(MG_ERR_UNSUPPORTED, "no filter-gradient kernel for tile %d x %d", pl.bm, pl.bn);
   }
   MG_HIP(hipGetLastError());
   if (staged) {

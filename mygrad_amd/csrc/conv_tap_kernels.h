@@ -476,7 +476,15 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
   static_assert(16 % ROWS == 0 && BM % ROWS == 0, "row passes must not straddle a column group");
   constexpr int ALOADS = BM / ROWS;
   constexpr int NGROUPS = BN / 16;
-  constexpr int GLOADS = 16 / ROWS;  // loads per thread per column group
+  // A loader thread owns one position of the K tile and one of ROWS row slots.  The
+  // padding test is per (position, column group), so the slots share out the groups
+  // first (GSPLIT ways) and only then the 16 channels of a group (CSPLIT ways): a
+  // thread tests MYGROUPS groups per K tile and loads CLOADS channels of each.
+  constexpr int GSPLIT = ROWS < NGROUPS ? ROWS : NGROUPS;
+  constexpr int MYGROUPS = NGROUPS / GSPLIT;
+  constexpr int CSPLIT = ROWS / GSPLIT;
+  constexpr int CLOADS = 16 / CSPLIT;
+  static_assert(NGROUPS % GSPLIT == 0 && ROWS % GSPLIT == 0 && 16 % CSPLIT == 0, "loader slots");
   constexpr int LDK = BK + 16 / sizeof(T);
   constexpr int KQ = BK / 4;  // K indices owned by one quarter-wave
 
@@ -518,16 +526,18 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
   const int row0 = BK % 64 == 0 ? uniform(tid / BK) : tid / BK;
   const int g12 = p.G[1] * p.G[2];
 
-  // the block's column groups never change: keep their table rows in registers
-  const int8v MG_CONSTANT *gtab = (const int8v MG_CONSTANT *)(p.groups) + n0 / 16;
-  int8v grp[NGROUPS];
-#pragma unroll
-  for (int j = 0; j < NGROUPS; ++j) grp[j] = gtab[j];
+  const int gsel = row0 % GSPLIT, csel = row0 / GSPLIT;
 
-  constexpr int NB = NGROUPS * GLOADS;
+  // the thread's column groups never change: keep their table rows in registers
+  const int8v MG_CONSTANT *gtab = (const int8v MG_CONSTANT *)(p.groups) + n0 / 16;
+  int8v grp[MYGROUPS];
+#pragma unroll
+  for (int i = 0; i < MYGROUPS; ++i) grp[i] = gtab[gsel + i * GSPLIT];
+
+  constexpr int NB = MYGROUPS * CLOADS;
   T ra0[ALOADS], rb0[NB], ra1[ALOADS], rb1[NB];
   const unsigned a_step = (unsigned)(ROWS * p.gvol) * (unsigned)sizeof(T);
-  const unsigned b_step = (unsigned)(ROWS * p.x_cstride) * (unsigned)sizeof(T);
+  const unsigned b_step = (unsigned)(CSPLIT * p.x_cstride) * (unsigned)sizeof(T);
 
   auto fetch = [&](T(&ra)[ALOADS], T(&rb)[NB], int kt) {
     const int ipos = kbeg + kt * BK + kcol;
@@ -547,24 +557,24 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
 #pragma unroll
     for (int r = 0; r < ALOADS; ++r) ra[r] = buffer_load<T>(grad_buf, g_at, (unsigned)r * a_step);
     const unsigned x_at = (unsigned)((long long)n * p.x_nstride + (qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2]) +
-                                     (long long)row0 * p.x_cstride) * (unsigned)sizeof(T);
+                                     (long long)csel * p.x_cstride) * (unsigned)sizeof(T);
 #pragma unroll
-    for (int j = 0; j < NGROUPS; ++j) {
+    for (int j = 0; j < MYGROUPS; ++j) {
       const int8v e = grp[j];  // coff, d0, d1, d2, valid
       const bool ok = pos_ok & (e[4] != 0) & ((unsigned)(qb0 + e[1]) < (unsigned)p.Q[0]) &
                       ((unsigned)(qb1 + e[2]) < (unsigned)p.Q[1]) & ((unsigned)(qb2 + e[3]) < (unsigned)p.Q[2]);
       const unsigned at = ok ? x_at + (unsigned)(e[0] * (int)sizeof(T)) : kOutside;
 #pragma unroll
-      for (int r = 0; r < GLOADS; ++r) rb[j * GLOADS + r] = buffer_load<T>(x_buf, at, (unsigned)r * b_step);
+      for (int r = 0; r < CLOADS; ++r) rb[j * CLOADS + r] = buffer_load<T>(x_buf, at, (unsigned)r * b_step);
     }
   };
   auto stash = [&](const T(&ra)[ALOADS], const T(&rb)[NB], int buf) {
 #pragma unroll
     for (int r = 0; r < ALOADS; ++r) As[buf][row0 + r * ROWS][kcol] = ra[r];
 #pragma unroll
-    for (int j = 0; j < NGROUPS; ++j)
+    for (int j = 0; j < MYGROUPS; ++j)
 #pragma unroll
-      for (int r = 0; r < GLOADS; ++r) Bs[buf][j * 16 + row0 + r * ROWS][kcol] = rb[j * GLOADS + r];
+      for (int r = 0; r < CLOADS; ++r) Bs[buf][(gsel + j * GSPLIT) * 16 + csel + r * CSPLIT][kcol] = rb[j * CLOADS + r];
   };
 
   const int ktiles = kend > kbeg ? (kend - kbeg + BK - 1) / BK : 0;
