@@ -855,6 +855,7 @@ int resident_blocks(K kernel, int threads) {
 // wave tile.  The table-driven kernel has the 64-column shapes only.
 #define MG_WGRAD_SHAPES(T, X)                                                          \
   X(T, 128, 128, (sizeof(T) == 8 ? 16 : 32), 64, 64)                                   \
+  X(T, 64, 192, (sizeof(T) == 8 ? 16 : 32), 32, 96)                                    \
   X(T, 64, 128, (sizeof(T) == 8 ? 16 : 32), 32, 64)                                    \
   X(T, 64, 64, (sizeof(T) == 8 ? 32 : 64), 32, 32)                                     \
   X(T, 32, 64, (sizeof(T) == 8 ? 32 : 64), 32, 16)                                     \
@@ -899,13 +900,14 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
   struct Cand {
     int bm, bn, bk;
   };
-  const Cand cands[] = {{128, 128, f64 ? 16 : 32}, {64, 128, f64 ? 16 : 32}, {64, 64, f64 ? 32 : 64},
+  const Cand cands[] = {{128, 128, f64 ? 16 : 32}, {64, 192, f64 ? 16 : 32}, {64, 128, f64 ? 16 : 32}, {64, 64, f64 ? 32 : 64},
                         {32, 64, f64 ? 32 : 64},   {16, 64, f64 ? 32 : 64}};
   long long best_splits = 1;
   pl.bm = 0;
   if (g.C % 16 == 0 && fits_buffer_loads(g)) {
     for (const Cand &c : cands) {
       if (g.F % c.bm != 0) continue;
+      if (f64 && c.bn == 192) continue;  // its accumulators leave room for one block per compute unit only
       const long long col_tiles = ceil_div(ct, c.bn), row_tiles = g.F / c.bm;
       const long long splits = splits_for(c.bm, c.bn, c.bk, true);
       if (c.bn > 64) {

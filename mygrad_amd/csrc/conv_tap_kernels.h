@@ -59,6 +59,8 @@ __device__ __forceinline__ void store_vec(T *dst, const T (&src)[N]) {
 // Tensors must be smaller than 2 GiB (kOutside must lie past the end).
 constexpr unsigned kOutside = 0x80000000u;
 
+constexpr int gcd_of(int a, int b) { return b == 0 ? a : gcd_of(b, a % b); }
+
 template <typename T>
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const void *base, unsigned bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
@@ -480,7 +482,7 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
   // padding test is per (position, column group), so the slots share out the groups
   // first (GSPLIT ways) and only then the 16 channels of a group (CSPLIT ways): a
   // thread tests MYGROUPS groups per K tile and loads CLOADS channels of each.
-  constexpr int GSPLIT = ROWS < NGROUPS ? ROWS : NGROUPS;
+  constexpr int GSPLIT = gcd_of(ROWS, NGROUPS);
   constexpr int MYGROUPS = NGROUPS / GSPLIT;
   constexpr int CSPLIT = ROWS / GSPLIT;
   constexpr int CLOADS = 16 / CSPLIT;
