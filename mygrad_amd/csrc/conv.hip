@@ -17,6 +17,7 @@
 #include "internal.h"
 
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -553,12 +554,44 @@ int pick_bm(int M) {
   return 16;
 }
 
+template <typename K>
+int resident_blocks(K kernel, int threads) {
+  int n = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, threads, 0) != hipSuccess || n < 1) {
+    (void)hipGetLastError();
+    n = 1;
+  }
+  return n;
+}
+
+// Tile shapes of the gather-GEMM kernels: rows x positions, and the wave tile.
+#define MG_GEMM_SHAPES(T, X) \
+  X(T, 128, 128, 64, 64)     \
+  X(T, 128, 64, 64, 32)      \
+  X(T, 64, 256, 64, 64)      \
+  X(T, 64, 128, 32, 64)      \
+  X(T, 32, 256, 32, 64)      \
+  X(T, 32, 128, 16, 64)      \
+  X(T, 16, 256, 16, 64)
+
+// Blocks of the persistent tap-major gather-GEMM that a compute unit holds at once.
+template <typename T>
+int gemm_blocks_per_cu(int bm, int bn) {
+  constexpr int BK = sizeof(T) == 8 ? 8 : 16;
+#define MG_OCC(TT, BM, BN, WM, WN) \
+  if (bm == BM && bn == BN) return resident_blocks(tap_gemm_kernel<TT, BM, BN, BK, WM, WN>, 512);
+  MG_GEMM_SHAPES(T, MG_OCC)
+#undef MG_OCC
+  return 1;
+}
+
 // Picks the tile of the gather-GEMM and how its last, partial round of tiles is
-// shared out.  Blocks reach the compute units round-robin, so after floor(T / CUs)
-// whole tiles per unit, T % CUs tiles are left that would keep only some units busy
-// for a full tile time; the tap-major kernel cuts each of those into `split` K slices
-// so that every unit gets about the same share of them.  Smaller tiles give more
-// tiles (finer balance, less padding) at some cost in operand reuse.
+// shared out.  The tap-major kernel runs as many persistent blocks as the device
+// holds at once ("slots"); block b takes tiles b, b + slots, ...  After
+// floor(T / slots) whole tiles per block, T % slots tiles are left that would keep
+// only some blocks busy for a full tile time, so each of those is cut into `split`
+// K slices and every block gets about the same share of them.  Smaller tiles give
+// more tiles (finer balance, less padding) at some cost in operand reuse.
 struct TileChoice {
   int bm, bn, m_tiles, full_tiles, tail_split;
   long long tiles;
@@ -591,7 +624,12 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
     t.full_tiles = (int)t.tiles;
     t.tail_split = 1;
     double tail = 0;
-    const long long rem = t.tiles % cus;
+    // blocks sharing a compute unit share its MFMA pipes: a round of `slots` tiles
+    // takes per_cu tile times
+    const int per_cu = !tap_major ? 1 : elem == 8 ? gemm_blocks_per_cu<double>(c.bm, c.bn) : gemm_blocks_per_cu<float>(c.bm, c.bn);
+    const bool stream = tap_major && tap_gemm_streams(c.bm, (int)elem);
+    const long long slots = stream ? (long long)per_cu * cus : cus;
+    const long long rem = t.tiles % slots;
     if (rem > 0) {
       tail = 1.0;
       if (tap_major) {
@@ -599,7 +637,7 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
         const long long tile_bytes = (long long)c.bm * c.bn * (long long)elem;
         const int smax = (int)std::max<long long>(1, std::min<long long>({(long long)min_ktiles / 2, 32ll, (32ll << 20) / (rem * tile_bytes)}));
         for (int sp = 2; sp <= smax; ++sp) {
-          const double share = (double)ceil_div(rem * sp, cus) / sp + 0.01 * sp;  // + a little for the fix-up pass
+          const double share = (double)ceil_div(rem * sp, slots) / sp + 0.01 * sp;  // + a little for the fix-up pass
           if (share < tail - 1e-9) {
             tail = share;
             t.tail_split = sp;
@@ -608,7 +646,7 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
         if (t.tail_split > 1) t.full_tiles = (int)(t.tiles - rem);
       }
     }
-    const double cost = ((double)(t.tiles / cus) + tail) * c.bm * c.bn * c.penalty;
+    const double cost = ((double)(t.tiles / slots) + tail) * (stream ? per_cu : 1) * c.bm * c.bn * c.penalty;
     if (best.bm == 0 || cost < best_cost) {
       best = t;
       best_cost = cost;
@@ -841,16 +879,6 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
   return upload_plan(pl, t);
 }
 
-template <typename K>
-int resident_blocks(K kernel, int threads) {
-  int n = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, threads, 0) != hipSuccess || n < 1) {
-    (void)hipGetLastError();
-    n = 1;
-  }
-  return n;
-}
-
 // Tile shapes of the filter-gradient kernels: rows (filters) x columns x K tile, and the
 // wave tile.  The table-driven kernel has the 64-column shapes only.
 #define MG_WGRAD_SHAPES(T, X)                                                          \
@@ -969,6 +997,12 @@ int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
     Plan pl;
     int rc = op == OP_FWD ? build_fwd_plan(g, pl) : op == OP_DGRAD ? build_dgrad_plan(g, pl) : build_wgrad_plan(g, pl);
     if (rc) return rc;
+    // MYGRAD_HIP_TRACE=1 reports, once per new descriptor, what was planned
+    static const bool trace = getenv("MYGRAD_HIP_TRACE") != nullptr;
+    if (trace)
+      fprintf(stderr, "[mygrad_hip] %s plan: %s tile %dx%d, %d phase(s), %d position blocks x %d row tiles, %d whole tiles + tail split %d, K splits %d (chunk %d)\n",
+              op == OP_FWD ? "fwd" : op == OP_DGRAD ? "dgrad" : "wgrad", pl.tap_major ? "tap-major" : "table-driven", pl.bm,
+              pl.bn, pl.nphases, pl.pos_blocks, pl.m_tiles, pl.full_tiles, pl.tail_split, pl.splits, pl.kchunk);
     it = plans().emplace(key, pl).first;
   }
   *out = &it->second;
@@ -976,12 +1010,15 @@ int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
 }
 
 template <typename T, int BM, int BN, int BK, int WM, int WN>
-void launch_gemm(const GemmParams &gp, const Plan &pl, hipStream_t s) {
+void launch_gemm(GemmParams &gp, const Plan &pl, hipStream_t s) {
   if (pl.tap_major) {
     const long long tiles = (long long)pl.pos_blocks * pl.m_tiles;
     const long long tail_tiles = tiles - pl.full_tiles;
-    hipLaunchKernelGGL((tap_gemm_kernel<T, BM, BN, BK, WM, WN>), dim3((unsigned)(pl.full_tiles + tail_tiles * pl.tail_split)),
-                       dim3(512), 0, s, gp);
+    static const int per_cu = resident_blocks(tap_gemm_kernel<T, BM, BN, BK, WM, WN>, 512);
+    const long long slots = tap_gemm_streams(BM, (int)sizeof(T)) ? (long long)per_cu * runtime().props.multiProcessorCount : (1ll << 40);
+    gp.items = (int)(pl.full_tiles + tail_tiles * pl.tail_split);
+    hipLaunchKernelGGL((tap_gemm_kernel<T, BM, BN, BK, WM, WN>), dim3((unsigned)std::min<long long>(gp.items, slots)), dim3(512),
+                       0, s, gp);
     if (tail_tiles > 0)
       hipLaunchKernelGGL((tail_fixup_kernel<T, BM, BN>), dim3((unsigned)ceil_div(BM * BN, 256), (unsigned)tail_tiles),
                          dim3(256), 0, s, gp);
@@ -1016,17 +1053,15 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
   gp.vec_store = pl.single_dense_phase && gp.dst_mstride % 4 == 0 && gp.dst_nstride % 4 == 0 &&
                  reinterpret_cast<uintptr_t>(gp.dst) % 16 == 0;
   ScopedTiming timed(tag);
-  const int shape = pl.bm * 1000 + pl.bn;
-  switch (shape) {
-    case 128128: launch_gemm<T, 128, 128, BK, 64, 64>(gp, pl, s); break;
-    case 128064: launch_gemm<T, 128, 64, BK, 64, 32>(gp, pl, s); break;
-    case 64256: launch_gemm<T, 64, 256, BK, 64, 64>(gp, pl, s); break;
-    case 64128: launch_gemm<T, 64, 128, BK, 32, 64>(gp, pl, s); break;
-    case 32256: launch_gemm<T, 32, 256, BK, 32, 64>(gp, pl, s); break;
-    case 32128: launch_gemm<T, 32, 128, BK, 16, 64>(gp, pl, s); break;
-    case 16256: launch_gemm<T, 16, 256, BK, 16, 64>(gp, pl, s); break;
-    default: return fail(MG_ERR_UNSUPPORTED, "no kernel for tile %d x %d", pl.bm, pl.bn);
+  bool launched = false;
+#define MG_LAUNCH(TT, BM, BN, WM, WN)                     \
+  if (!launched && pl.bm == BM && pl.bn == BN) {          \
+    launch_gemm<TT, BM, BN, BK, WM, WN>(gp, pl, s);       \
+    launched = true;                                      \
   }
+  MG_GEMM_SHAPES(T, MG_LAUNCH)
+#undef MG_LAUNCH
+  if (!launched) return fail(MG_ERR_UNSUPPORTED, "no kernel for tile %d x %d", pl.bm, pl.bn);
   MG_HIP(hipGetLastError());
   return MG_OK;
 }

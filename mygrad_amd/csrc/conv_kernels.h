@@ -71,7 +71,9 @@ struct Phase {
   int blk_begin;         // first block (along positions) that works on this phase
   int npos;              // N * J0 * J1 * J2
   FastDiv by_jvol, by_j12, by_j2;  // divisions that turn a position into (n, j0, j1, j2)
+  int pad_[2];                     // 96 bytes: three 32-byte scalar loads
 };
+static_assert(sizeof(Phase) == 96, "Phase is read as three 32-byte rows");
 
 // Gather-GEMM:  dst[n, m, pos] = sum_k A[arow[k]][m] * src[n, row k, pos]
 struct GemmParams {
@@ -97,6 +99,7 @@ struct GemmParams {
   int src_cstride;      // element stride between consecutive channels of the gathered tensor
   int vec_store;        // positions are contiguous in dst: a lane may store its TN positions as one vector
   int m_tiles;          // row tiles per position block
+  int items;            // work items: full_tiles whole tiles, then tail_split K slices of each remaining tile
   int full_tiles;       // tiles computed whole by one block each
   int tail_split;       // blocks that share each remaining tile (K slices), >= 1
   void *partial;        // [tail tile][slice][BM][BN] partial sums of the shared tiles

@@ -49,6 +49,24 @@ __device__ __forceinline__ void store_vec(T *dst, const T (&src)[N]) {
   }
 }
 
+// A row of the phase table through the scalar data path (the index is wave-uniform).
+__device__ __forceinline__ Phase load_phase(const Phase *phases, int i) {
+  const int8v MG_CONSTANT *q = (const int8v MG_CONSTANT *)(phases + uniform(i));
+  const int8v a = q[0], b = q[1], c = q[2];
+  Phase ph;
+  ph.J[0] = a[0], ph.J[1] = a[1], ph.J[2] = a[2];
+  ph.o0[0] = a[3], ph.o0[1] = a[4], ph.o0[2] = a[5];
+  ph.k_begin = a[6], ph.k_count = a[7];
+  ph.blk_begin = b[0], ph.npos = b[1];
+  ph.by_jvol = FastDiv{(unsigned)b[2], (unsigned)b[3], (unsigned)b[4], 0u};
+  ph.by_j12 = FastDiv{(unsigned)b[6], (unsigned)b[7], (unsigned)c[0], 0u};
+  ph.by_j2 = FastDiv{(unsigned)c[2], (unsigned)c[3], (unsigned)c[4], 0u};
+  return ph;
+}
+__device__ __forceinline__ int phase_first_block(const Phase *phases, int i) {
+  return ((const int MG_CONSTANT *)(phases + uniform(i)))[8];
+}
+
 // Gathers go through buffer loads: address = base + per-lane byte offset (VGPR) +
 // wave-uniform byte offset (SGPR).  The channel step of a K tile's rows is uniform,
 // so it rides in the SGPR and costs no vector instruction per load, and a lane
@@ -60,6 +78,10 @@ __device__ __forceinline__ void store_vec(T *dst, const T (&src)[N]) {
 constexpr unsigned kOutside = 0x80000000u;
 
 constexpr int gcd_of(int a, int b) { return b == 0 ? a : gcd_of(b, a % b); }
+
+// Whether tap_gemm_kernel with BM rows per tile runs persistent blocks that stream
+// through several work items (else: one block per item).
+constexpr bool tap_gemm_streams(int bm, int elem) { return bm >= 64 || elem == 8; }
 
 template <typename T>
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_of(const void *base, unsigned bytes) {
@@ -98,6 +120,12 @@ struct Quad {
 // ------------------------------------------------------------------------------------------
 template <typename T, int BM, int BN, int BK, int WM, int WN>
 __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
+  // Tiles of 64 rows and more, and all double-precision tiles, run as persistent
+  // blocks (see below).  The short float tiles of thin filter banks get one block per
+  // item instead: moving the gather on to the next item from inside the K loop keeps
+  // that code's inputs in scalar registers, which costs those shapes a resident block
+  // per compute unit and more than the streaming gains them.
+  constexpr bool STREAM = tap_gemm_streams(BM, (int)sizeof(T));
   static_assert((BM / WM) * (BN / WN) == 4, "four wavefronts per block");
   static_assert(BK % 4 == 0 && WM % 16 == 0 && WN % 16 == 0 && BN % 64 == 0, "MFMA 16x16x4 tiling");
   constexpr int TM = WM / 16, TN = WN / 16;
@@ -113,10 +141,17 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
   __shared__ __attribute__((aligned(16))) T Bs[2][BK][LDB];
 
   // Eight wavefronts with two roles.  Waves 0-3 only read LDS and issue MFMAs; waves
-  // 4-7 only gather: global loads -> registers -> LDS, one tile ahead.  One of each
-  // sits on every SIMD, so the gather's address arithmetic, memory instructions and
-  // LDS stores are issued in the shadow of the other wave's MFMAs instead of taking
-  // turns with them in one instruction stream.
+  // 4-7 only gather: global loads -> registers -> LDS, ahead of the MFMA waves.  One of
+  // each sits on every SIMD, so the gather's memory instructions and LDS stores are
+  // issued in the shadow of the other wave's MFMAs.
+  //
+  // Blocks are persistent: block b works through the items b, b + gridDim.x, ...  An
+  // item is a whole tile or, for the tiles of the last partial round, one K slice of a
+  // tile (its partial sums go to a workspace for tail_fixup_kernel).  The K tiles of a
+  // block's items form one stream: stream element s lives in LDS buffer s % 2, and the
+  // loader waves run ahead of the MFMA waves across item boundaries, so the first
+  // operands of the next tile are already on their way while this tile is finished
+  // and stored.  One barrier at the start, then one per stream element.
   const int lane = threadIdx.x & 63;
   const int wave = uniform(threadIdx.x >> 6);
   const bool loader = wave >= 4;
@@ -125,312 +160,319 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
   const int wn0 = ((wave & 3) % WAVES_N) * WN;
   const int l16 = lane & 15, lk = lane >> 4;
 
-  // Tiles are numbered with the row tile (m) innermost, so that the row tiles of one
-  // position block, which gather the same elements, run next to each other.  The
-  // first p.full_tiles blocks compute one whole tile each.  The tiles that remain
-  // would fill only part of the device in a last round, so each of them is shared
-  // by p.tail_split blocks, each taking a slice of the K loop and leaving its partial
-  // sums in a workspace for tail_fixup_kernel.
-  const int bid = blockIdx.x;
-  int tile = bid, piece = 0;
-  const bool partial = bid >= p.full_tiles;
-  if (partial) {
-    const int j = bid - p.full_tiles;
-    tile = p.full_tiles + j / p.tail_split;
-    piece = j % p.tail_split;
-  }
-  const int pblk = tile / p.m_tiles;
-  int pi = 0;
-  while (pi + 1 < p.nphases && pblk >= p.phases[pi + 1].blk_begin) ++pi;
-  const Phase ph = p.phases[pi];
-  const int pos0 = (pblk - ph.blk_begin) * BN;
-  const int m0 = (tile % p.m_tiles) * BM;
-  const int j12 = ph.J[1] * ph.J[2];
-  const int jvol = ph.J[0] * j12;
-
-  const __amdgpu_buffer_rsrc_t a_buf = buffer_of<T>(p.A, p.a_bytes);
-  const __amdgpu_buffer_rsrc_t src_buf = buffer_of<T>(p.src, p.src_bytes);
-  const int8v MG_CONSTANT *ktab = (const int8v MG_CONSTANT *)(p.ktiles + ph.k_begin);
-
-  // ---- this thread's column of the B tile: one output position
-  const int bcol = tid % BN;
-  const int brow0 = uniform(tid / BN);
-  int qb0, qb1, qb2;
-  const bool pos_ok = pos0 + bcol < ph.npos;
-  unsigned src_at;  // byte offset of the position's tap (0,0,0), channel brow0
-  {
-    const unsigned pos = pos_ok ? (unsigned)(pos0 + bcol) : 0u;
-    const unsigned n = ph.by_jvol.div(pos);
-    unsigned r = pos - n * (unsigned)jvol;
-    const unsigned j0 = ph.by_j12.div(r);
-    r -= j0 * (unsigned)j12;
-    const unsigned j1 = ph.by_j2.div(r);
-    const unsigned j2 = r - j1 * (unsigned)ph.J[2];
-    qb0 = (int)j0 * p.sj[0];
-    qb1 = (int)j1 * p.sj[1];
-    qb2 = (int)j2 * p.sj[2];
-    src_at = (unsigned)((long long)n * p.src_nstride + (qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2]) +
-                        brow0 * p.src_cstride) * (unsigned)sizeof(T);
-  }
-  // ---- this thread's column of the A tile: one row m of the packed filters
-  const int acol = tid % BM;
-  const int arow0 = BM % 64 == 0 ? uniform(tid / BM) : tid / BM;
-  const bool a_ok = (m0 + acol < p.M) & (arow0 < BK);
-  const unsigned a_at = a_ok ? (unsigned)(arow0 * p.M + m0 + acol) * (unsigned)sizeof(T) : kOutside;
-  const unsigned a_row_bytes = (unsigned)p.M * (unsigned)sizeof(T);
-  const unsigned b_step = (unsigned)(BROWS * p.src_cstride) * (unsigned)sizeof(T);
-
-  // two register sets: a tile is requested two iterations before it is parked in LDS
-  T ra0[ALOADS], rb0[BLOADS], ra1[ALOADS], rb1[BLOADS];
-
-  auto fetch = [&](T(&ra)[ALOADS], T(&rb)[BLOADS], int kt) {
-    const int8v e = ktab[kt];  // a_row0, coff, d0, d1, d2
-    const unsigned a_tile = (unsigned)e[0] * a_row_bytes;
-#pragma unroll
-    for (int r = 0; r < ALOADS; ++r) ra[r] = buffer_load<T>(a_buf, a_at, a_tile + (unsigned)(r * AROWS) * a_row_bytes);
-    const bool ok = pos_ok & ((unsigned)(qb0 + e[2]) < (unsigned)p.Q[0]) & ((unsigned)(qb1 + e[3]) < (unsigned)p.Q[1]) &
-                    ((unsigned)(qb2 + e[4]) < (unsigned)p.Q[2]);
-    const unsigned at = ok ? src_at + (unsigned)(e[1] * (int)sizeof(T)) : kOutside;
-#pragma unroll
-    for (int r = 0; r < BLOADS; ++r) rb[r] = buffer_load<T>(src_buf, at, (unsigned)r * b_step);
+  // ---- one work item (all wave-uniform).  Tiles are numbered with the row tile (m)
+  // innermost, so that the row tiles of one position block, which gather the same
+  // elements, run next to each other; items >= p.full_tiles are K slices.
+  struct Item {
+    int tile, piece, pos0, m0, kt_begin, kt_end;
+    bool partial;
+    Phase ph;
   };
-  auto stash = [&](const T(&ra)[ALOADS], const T(&rb)[BLOADS], int buf) {
-#pragma unroll
-    for (int r = 0; r < ALOADS; ++r) {
-      const int kk = arow0 + r * AROWS;
-      if (kk < BK) As[buf][kk][acol] = ra[r];
+  auto locate = [&](int item, int &pi, Item &it) {  // pi: phase of the previous item of this cursor (items ascend)
+    it.tile = item;
+    it.piece = 0;
+    it.partial = item >= p.full_tiles;
+    if (it.partial) {
+      const int j = item - p.full_tiles;
+      it.tile = p.full_tiles + j / p.tail_split;
+      it.piece = j % p.tail_split;
     }
-#pragma unroll
-    for (int r = 0; r < BLOADS; ++r) Bs[buf][brow0 + r * BROWS][bcol] = rb[r];
+    const int pblk = it.tile / p.m_tiles;
+    while (pi + 1 < p.nphases && pblk >= phase_first_block(p.phases, pi + 1)) ++pi;
+    it.ph = load_phase(p.phases, pi);
+    it.pos0 = (pblk - it.ph.blk_begin) * BN;
+    it.m0 = (it.tile % p.m_tiles) * BM;
+    it.kt_begin = 0;
+    it.kt_end = it.ph.k_count;
+    if (it.partial) {
+      const int per = (it.ph.k_count + p.tail_split - 1) / p.tail_split;
+      it.kt_begin = min(it.piece * per, it.ph.k_count);
+      it.kt_end = min(it.kt_begin + per, it.ph.k_count);
+    }
   };
 
-  // Lane (l16, lk) feeds row/column l16 of every 16x16 tile.  Tile i of the wave
-  // takes the rows m = wm0 + l16*TM + i (and tile j the positions wn0 + l16*TN + j),
-  // so the TM (TN) operands of a lane are adjacent in LDS and come in one read.
-  int kt_begin = 0, kt_end = ph.k_count;
-  if (partial) {
-    const int per = (ph.k_count + p.tail_split - 1) / p.tail_split;
-    kt_begin = min(piece * per, ph.k_count);
-    kt_end = min(kt_begin + per, ph.k_count);
-  }
-  // The two roles run separate loops (their registers never coexist) that meet at
-  // the same barriers: one after the first tile is in LDS, one per K tile.
   if (loader) {
-    // Tile kt_begin + i travels in register set i % 2.  Every path through this loop
-    // issues the same loads in the same order (tile indices past the end are clamped
-    // and their data is never read): only then can the compiler wait for exactly the
-    // older register set and leave the newer one's loads in flight.
-    const int last = kt_end - 1;
-    if (kt_begin < kt_end) {
-      fetch(ra0, rb0, kt_begin);
+    const __amdgpu_buffer_rsrc_t a_buf = buffer_of<T>(p.A, p.a_bytes);
+    const __amdgpu_buffer_rsrc_t src_buf = buffer_of<T>(p.src, p.src_bytes);
+    const int bcol = tid % BN;
+    const int brow0 = uniform(tid / BN);
+    const int acol = tid % BM;
+    const int arow0 = BM % 64 == 0 ? uniform(tid / BM) : tid / BM;
+    const unsigned a_row_bytes = (unsigned)p.M * (unsigned)sizeof(T);
+    const unsigned b_step = (unsigned)(BROWS * p.src_cstride) * (unsigned)sizeof(T);
+
+    // ---- fetch cursor: the item being gathered and this thread's place in it
+    Item it;
+    int pi = 0, item = -1, kt = 0;
+    const int8v MG_CONSTANT *ktab = nullptr;
+    int qb0 = 0, qb1 = 0, qb2 = 0;
+    bool pos_ok = false;
+    unsigned src_at = 0;  // byte offset of the position's tap (0,0,0), channel brow0
+    unsigned a_at = kOutside;
+    // moves the cursor to the first item at or after `from` that has K tiles; false if none
+    auto enter = [&](int from) -> bool {
+      for (int i = from; i < p.items; i += (int)gridDim.x) {
+        locate(i, pi, it);
+        if (it.kt_begin >= it.kt_end) continue;
+        item = i;
+        kt = it.kt_begin;
+        ktab = (const int8v MG_CONSTANT *)(p.ktiles + it.ph.k_begin);
+        const int j12 = it.ph.J[1] * it.ph.J[2];
+        pos_ok = it.pos0 + bcol < it.ph.npos;
+        const unsigned pos = pos_ok ? (unsigned)(it.pos0 + bcol) : 0u;
+        const unsigned n = it.ph.by_jvol.div(pos);
+        unsigned r = pos - n * (unsigned)(it.ph.J[0] * j12);
+        const unsigned j0 = it.ph.by_j12.div(r);
+        r -= j0 * (unsigned)j12;
+        const unsigned j1 = it.ph.by_j2.div(r);
+        const unsigned j2 = r - j1 * (unsigned)it.ph.J[2];
+        qb0 = (int)j0 * p.sj[0];
+        qb1 = (int)j1 * p.sj[1];
+        qb2 = (int)j2 * p.sj[2];
+        src_at = (unsigned)((long long)n * p.src_nstride + (qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2]) +
+                            brow0 * p.src_cstride) * (unsigned)sizeof(T);
+        const bool a_ok = (it.m0 + acol < p.M) & (arow0 < BK);
+        a_at = a_ok ? (unsigned)(arow0 * p.M + it.m0 + acol) * (unsigned)sizeof(T) : kOutside;
+        return true;
+      }
+      return false;
+    };
+    // K tile under the cursor -> registers; then the cursor moves on.  Past the end of
+    // the stream it stays on the last K tile (the data is never used): every call
+    // issues the same loads, so the compiler can count them exactly.
+    bool live = false;  // the cursor is on a K tile that has not been requested yet
+    int requested = 0;  // stream elements requested so far
+    auto fetch = [&](T(&ra)[ALOADS], T(&rb)[BLOADS]) {
+      const int8v e = ktab[kt];  // a_row0, coff, d0, d1, d2
+      const unsigned a_tile = (unsigned)e[0] * a_row_bytes;
+#pragma unroll
+      for (int r = 0; r < ALOADS; ++r) ra[r] = buffer_load<T>(a_buf, a_at, a_tile + (unsigned)(r * AROWS) * a_row_bytes);
+      const bool ok = pos_ok & ((unsigned)(qb0 + e[2]) < (unsigned)p.Q[0]) & ((unsigned)(qb1 + e[3]) < (unsigned)p.Q[1]) &
+                      ((unsigned)(qb2 + e[4]) < (unsigned)p.Q[2]);
+      const unsigned at = ok ? src_at + (unsigned)(e[1] * (int)sizeof(T)) : kOutside;
+#pragma unroll
+      for (int r = 0; r < BLOADS; ++r) rb[r] = buffer_load<T>(src_buf, at, (unsigned)r * b_step);
+      if (live) {
+        ++requested;
+        if (kt + 1 < it.kt_end)
+          ++kt;
+        else if constexpr (STREAM)
+          live = enter(item + (int)gridDim.x);  // no further item: the cursor stays where it is
+        else
+          live = false;
+      }
+    };
+    auto stash = [&](const T(&ra)[ALOADS], const T(&rb)[BLOADS], int buf) {
+#pragma unroll
+      for (int r = 0; r < ALOADS; ++r) {
+        const int kk = arow0 + r * AROWS;
+        if (kk < BK) As[buf][kk][acol] = ra[r];
+      }
+#pragma unroll
+      for (int r = 0; r < BLOADS; ++r) Bs[buf][brow0 + r * BROWS][bcol] = rb[r];
+    };
+
+    // two register sets: stream element s travels in set s % 2 and is requested two
+    // elements before it is parked in LDS
+    T ra0[ALOADS], rb0[BLOADS], ra1[ALOADS], rb1[BLOADS];
+    live = enter((int)blockIdx.x);
+    if (live) {
+      fetch(ra0, rb0);
       stash(ra0, rb0, 0);
-      fetch(ra1, rb1, min(kt_begin + 1, last));
-      fetch(ra0, rb0, min(kt_begin + 2, last));
+      fetch(ra1, rb1);
+      fetch(ra0, rb0);
     }
     __syncthreads();
-    // each half of the loop body parks tile kt+1 (requested two iterations ago) in
-    // the idle buffer and requests tile kt+3 into the registers that just emptied
-    int kt = kt_begin;
-    for (; kt + 1 < kt_end; kt += 2) {
+    // While the MFMA waves work on element s, element s+1 (requested two steps ago) is
+    // parked in the idle buffer and element s+3 requested into the registers it left.
+    // Requests run three elements ahead, so `requested` is final before s reaches it.
+    for (int s = 0; s < requested;) {
       stash(ra1, rb1, 1);
-      fetch(ra1, rb1, min(kt + 3, last));
+      fetch(ra1, rb1);
       __syncthreads();
+      if (++s >= requested) break;
       stash(ra0, rb0, 0);
-      fetch(ra0, rb0, min(kt + 4, last));
+      fetch(ra0, rb0);
       __syncthreads();
+      ++s;
     }
-    if (kt < kt_end) __syncthreads();
     return;
   }
 
+  // ---- MFMA waves
+  Item it;
+  int pi = 0;
+  int buf = 0;
   T *__restrict__ dst = static_cast<T *>(p.dst);
-  auto dst_of = [&](int ipos) -> T * {
-    const unsigned pos = (unsigned)ipos;
-    const unsigned n = ph.by_jvol.div(pos);
-    unsigned r = pos - n * (unsigned)jvol;
-    const int j0 = (int)ph.by_j12.div(r);
-    r -= (unsigned)j0 * (unsigned)j12;
-    const int j1 = (int)ph.by_j2.div(r);
-    const int j2 = (int)r - j1 * ph.J[2];
-    return dst + (long long)n * p.dst_nstride + (long long)(ph.o0[0] + j0 * p.oj[0]) * p.os[0] +
-           (long long)(ph.o0[1] + j1 * p.oj[1]) * p.os[1] + (long long)(ph.o0[2] + j2 * p.oj[2]) * p.os[2];
-  };
+  locate((int)blockIdx.x, pi, it);  // the grid never has more blocks than items
+  __syncthreads();
+  for (int item = (int)blockIdx.x; item < p.items; item += (int)gridDim.x) {
+    if (item != (int)blockIdx.x) locate(item, pi, it);
+    const Phase &ph = it.ph;
+    const int pos0 = it.pos0, m0 = it.m0;
+    const int j12 = ph.J[1] * ph.J[2];
+    const int jvol = ph.J[0] * j12;
+    auto dst_of = [&](int ipos) -> T * {
+      const unsigned pos = (unsigned)ipos;
+      const unsigned n = ph.by_jvol.div(pos);
+      unsigned r = pos - n * (unsigned)jvol;
+      const int j0 = (int)ph.by_j12.div(r);
+      r -= (unsigned)j0 * (unsigned)j12;
+      const int j1 = (int)ph.by_j2.div(r);
+      const int j2 = (int)r - j1 * ph.J[2];
+      return dst + (long long)n * p.dst_nstride + (long long)(ph.o0[0] + j0 * p.oj[0]) * p.os[0] +
+             (long long)(ph.o0[1] + j1 * p.oj[1]) * p.os[1] + (long long)(ph.o0[2] + j2 * p.oj[2]) * p.os[2];
+    };
+    T *slot = static_cast<T *>(p.partial) + ((long long)(it.tile - p.full_tiles) * p.tail_split + it.piece) * (BM * BN);
 
-  if constexpr (sizeof(T) == 8) {
-    // The wave tile is cut into 8-row and 8-column groups; group pairs are interleaved
-    // (row = pair*16 + 2*patch_row + half) so that a lane's two operands of a pair are
-    // adjacent in LDS and the 8 distinct lanes of a read cover 128 contiguous bytes.
-    constexpr int GM = WM / 8, GN = WN / 8;
-    const int arow = wm0 + Quad::feed_row(l16) * 2;
-    const int bcol8 = wn0 + Quad::feed_col(l16) * 2;
-    const int drow = wm0 + Quad::held_row(l16, lk) * 2;
-    double acc[GM][GN];
+    if constexpr (sizeof(T) == 8) {
+      // The wave tile is cut into 8-row and 8-column groups; group pairs are interleaved
+      // (row = pair*16 + 2*patch_row + half) so that a lane's two operands of a pair are
+      // adjacent in LDS and the 8 distinct lanes of a read cover 128 contiguous bytes.
+      constexpr int GM = WM / 8, GN = WN / 8;
+      const int arow = wm0 + Quad::feed_row(l16) * 2;
+      const int bcol8 = wn0 + Quad::feed_col(l16) * 2;
+      const int drow = wm0 + Quad::held_row(l16, lk) * 2;
+      double acc[GM][GN];
 #pragma unroll
-    for (int i = 0; i < GM; ++i)
+      for (int i = 0; i < GM; ++i)
 #pragma unroll
-      for (int j = 0; j < GN; ++j) acc[i][j] = 0.0;
-    __syncthreads();
-    int buf = 0;
-    for (int kt = kt_begin; kt < kt_end; ++kt) {
+        for (int j = 0; j < GN; ++j) acc[i][j] = 0.0;
+      for (int kt = it.kt_begin; kt < it.kt_end; ++kt) {
 #pragma unroll
-      for (int k4 = 0; k4 < BK / 4; ++k4) {
-        T a[GM], b[GN];
+        for (int k4 = 0; k4 < BK / 4; ++k4) {
+          T a[GM], b[GN];
 #pragma unroll
-        for (int g = 0; g < GM / 2; ++g) {
-          T two[2];
-          load_vec<T, 2>(&As[buf][k4 * 4 + lk][arow + g * 16], two);
-          a[2 * g] = two[0], a[2 * g + 1] = two[1];
+          for (int g = 0; g < GM / 2; ++g) {
+            T two[2];
+            load_vec<T, 2>(&As[buf][k4 * 4 + lk][arow + g * 16], two);
+            a[2 * g] = two[0], a[2 * g + 1] = two[1];
+          }
+#pragma unroll
+          for (int g = 0; g < GN / 2; ++g) {
+            T two[2];
+            load_vec<T, 2>(&Bs[buf][k4 * 4 + lk][bcol8 + g * 16], two);
+            b[2 * g] = two[0], b[2 * g + 1] = two[1];
+          }
+#pragma unroll
+          for (int i = 0; i < GM; ++i)
+#pragma unroll
+            for (int j = 0; j < GN; ++j) acc[i][j] = Quad::run(a[i], b[j], acc[i][j]);
         }
-#pragma unroll
-        for (int g = 0; g < GN / 2; ++g) {
-          T two[2];
-          load_vec<T, 2>(&Bs[buf][k4 * 4 + lk][bcol8 + g * 16], two);
-          b[2 * g] = two[0], b[2 * g + 1] = two[1];
-        }
-#pragma unroll
-        for (int i = 0; i < GM; ++i)
-#pragma unroll
-          for (int j = 0; j < GN; ++j) acc[i][j] = Quad::run(a[i], b[j], acc[i][j]);
+        __syncthreads();
+        buf ^= 1;
       }
-      __syncthreads();
-      buf ^= 1;
-    }
-    // ---- epilogue: acc[i][j] is row drow + (i/2)*16 + i%2, column bcol8 + (j/2)*16 + j%2
-    if (partial) {
-      T *slot = static_cast<T *>(p.partial) + ((long long)(tile - p.full_tiles) * p.tail_split + piece) * (BM * BN);
-#pragma unroll
-      for (int i = 0; i < GM; ++i) {
-        const int ml = drow + (i / 2) * 16 + i % 2;
-#pragma unroll
-        for (int g = 0; g < GN / 2; ++g) {
-          const T two[2] = {acc[i][2 * g], acc[i][2 * g + 1]};
-          store_vec<T, 2>(slot + ml * BN + bcol8 + g * 16, two);
-        }
-      }
-      return;
-    }
-#pragma unroll
-    for (int g = 0; g < GN / 2; ++g) {
-      const int first = pos0 + bcol8 + g * 16;
-      if (p.vec_store) {
-        // both positions exist (npos % 4 == 0) and are adjacent in dst
-        if (first >= ph.npos) continue;
-        T *out = dst_of(first);
+      // ---- epilogue: acc[i][j] is row drow + (i/2)*16 + i%2, column bcol8 + (j/2)*16 + j%2
+      if (it.partial) {
 #pragma unroll
         for (int i = 0; i < GM; ++i) {
-          const int m = m0 + drow + (i / 2) * 16 + i % 2;
-          const T two[2] = {acc[i][2 * g], acc[i][2 * g + 1]};
-          if (m < p.M) store_vec<T, 2>(out + (long long)m * p.dst_mstride, two);
-        }
-      } else {
+          const int ml = drow + (i / 2) * 16 + i % 2;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          if (first + h >= ph.npos) continue;
-          T *out = dst_of(first + h);
+          for (int g = 0; g < GN / 2; ++g) {
+            const T two[2] = {acc[i][2 * g], acc[i][2 * g + 1]};
+            store_vec<T, 2>(slot + ml * BN + bcol8 + g * 16, two);
+          }
+        }
+        continue;
+      }
+#pragma unroll
+      for (int g = 0; g < GN / 2; ++g) {
+        const int first = pos0 + bcol8 + g * 16;
+        if (p.vec_store) {
+          // both positions exist (npos % 4 == 0) and are adjacent in dst
+          if (first >= ph.npos) continue;
+          T *out = dst_of(first);
 #pragma unroll
           for (int i = 0; i < GM; ++i) {
             const int m = m0 + drow + (i / 2) * 16 + i % 2;
-            if (m < p.M) out[(long long)m * p.dst_mstride] = acc[i][2 * g + h];
+            const T two[2] = {acc[i][2 * g], acc[i][2 * g + 1]};
+            if (m < p.M) store_vec<T, 2>(out + (long long)m * p.dst_mstride, two);
           }
-        }
-      }
-    }
-    return;
-  }
-
-  typename Mma<T>::Acc acc[TM][TN];
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) acc[i][j] = typename Mma<T>::Acc{0, 0, 0, 0};
-  __syncthreads();
-  {
-    int buf = 0;
-    for (int kt = kt_begin; kt < kt_end; ++kt) {
-#pragma unroll
-      for (int k4 = 0; k4 < BK / 4; ++k4) {
-        T a[TM], b[TN];
-        load_vec<T, TM>(&As[buf][k4 * 4 + lk][wm0 + l16 * TM], a);
-        load_vec<T, TN>(&Bs[buf][k4 * 4 + lk][wn0 + l16 * TN], b);
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::run(a[i], b[j], acc[i][j]);
-      }
-      __syncthreads();
-      buf ^= 1;
-    }
-  }
-
-  // ---- epilogue
-  if (partial) {
-    // raw tile [BM][BN] of this slice, lane's TN positions stored as one vector
-    T *slot = static_cast<T *>(p.partial) +
-              ((long long)(tile - p.full_tiles) * p.tail_split + piece) * (BM * BN) + (wn0 + l16 * TN);
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int ml = wm0 + Mma<T>::row_of(lane, q) * TM + i;
-        T v[TN];
-#pragma unroll
-        for (int j = 0; j < TN; ++j) v[j] = acc[i][j][q];
-        if constexpr (sizeof(T) * TN <= 16) {
-          store_vec<T, TN>(slot + ml * BN, v);
         } else {
-          T lo[TN / 2], hi[TN / 2];
 #pragma unroll
-          for (int j = 0; j < TN / 2; ++j) {
-            lo[j] = v[j];
-            hi[j] = v[TN / 2 + j];
-          }
-          store_vec<T, TN / 2>(slot + ml * BN, lo);
-          store_vec<T, TN / 2>(slot + ml * BN + TN / 2, hi);
-        }
-      }
-    return;
-  }
-  const int first = pos0 + wn0 + l16 * TN;
-  if (p.vec_store) {
-    // the TN positions of this lane are adjacent in dst and all exist (npos % TN == 0)
-    if (first < ph.npos) {
-      T *out = dst_of(first);
+          for (int h = 0; h < 2; ++h) {
+            if (first + h >= ph.npos) continue;
+            T *out = dst_of(first + h);
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int m = m0 + wm0 + Mma<T>::row_of(lane, q) * TM + i;
-          if (m < p.M) {
-            T v[TN];
-#pragma unroll
-            for (int j = 0; j < TN; ++j) v[j] = acc[i][j][q];
-            if constexpr (sizeof(T) * TN <= 16) {
-              store_vec<T, TN>(out + (long long)m * p.dst_mstride, v);
-            } else {
-              T lo[TN / 2], hi[TN / 2];
-#pragma unroll
-              for (int j = 0; j < TN / 2; ++j) {
-                lo[j] = v[j];
-                hi[j] = v[TN / 2 + j];
-              }
-              store_vec<T, TN / 2>(out + (long long)m * p.dst_mstride, lo);
-              store_vec<T, TN / 2>(out + (long long)m * p.dst_mstride + TN / 2, hi);
+            for (int i = 0; i < GM; ++i) {
+              const int m = m0 + drow + (i / 2) * 16 + i % 2;
+              if (m < p.M) out[(long long)m * p.dst_mstride] = acc[i][2 * g + h];
             }
           }
         }
-    }
-  } else {
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      if (first + j >= ph.npos) continue;
-      T *out = dst_of(first + j);
+      }
+    } else {
+      // Lane (l16, lk) feeds row/column l16 of every 16x16 tile.  Tile i of the wave
+      // takes the rows m = wm0 + l16*TM + i (and tile j the positions wn0 + l16*TN + j),
+      // so the TM (TN) operands of a lane are adjacent in LDS and come in one read.
+      typename Mma<T>::Acc acc[TM][TN];
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int m = m0 + wm0 + Mma<T>::row_of(lane, q) * TM + i;
-          if (m < p.M) out[(long long)m * p.dst_mstride] = acc[i][j][q];
+        for (int j = 0; j < TN; ++j) acc[i][j] = typename Mma<T>::Acc{0, 0, 0, 0};
+      for (int kt = it.kt_begin; kt < it.kt_end; ++kt) {
+#pragma unroll
+        for (int k4 = 0; k4 < BK / 4; ++k4) {
+          T a[TM], b[TN];
+          load_vec<T, TM>(&As[buf][k4 * 4 + lk][wm0 + l16 * TM], a);
+          load_vec<T, TN>(&Bs[buf][k4 * 4 + lk][wn0 + l16 * TN], b);
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::run(a[i], b[j], acc[i][j]);
         }
+        __syncthreads();
+        buf ^= 1;
+      }
+
+      // ---- epilogue
+      if (it.partial) {
+        // raw tile [BM][BN] of this slice, lane's TN positions stored as one vector
+        T *mine = slot + (wn0 + l16 * TN);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int ml = wm0 + Mma<T>::row_of(lane, q) * TM + i;
+            T v[TN];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) v[j] = acc[i][j][q];
+            store_vec<T, TN>(mine + ml * BN, v);
+          }
+        continue;
+      }
+      const int first = pos0 + wn0 + l16 * TN;
+      if (p.vec_store) {
+        // the TN positions of this lane are adjacent in dst and all exist (npos % TN == 0)
+        if (first < ph.npos) {
+          T *out = dst_of(first);
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int m = m0 + wm0 + Mma<T>::row_of(lane, q) * TM + i;
+              if (m < p.M) {
+                T v[TN];
+#pragma unroll
+                for (int j = 0; j < TN; ++j) v[j] = acc[i][j][q];
+                store_vec<T, TN>(out + (long long)m * p.dst_mstride, v);
+              }
+            }
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          if (first + j >= ph.npos) continue;
+          T *out = dst_of(first + j);
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int m = m0 + wm0 + Mma<T>::row_of(lane, q) * TM + i;
+              if (m < p.M) out[(long long)m * p.dst_mstride] = acc[i][j][q];
+            }
+        }
+      }
     }
   }
 }
