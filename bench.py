@@ -327,6 +327,22 @@ def run_copy_calibration(mib=1024, reps=20):
             "value": 2 * n * 1e-9 / (avg * 1e-3), "unit": "GB/s", "launches": len(ms)}
 
 
+def run_mfma_probe():
+    """What the matrix cores sustain per MFMA shape with operands in registers and no
+    memory traffic, next to the published peaks: the ceiling of the convolution
+    kernels' inner loops on this device."""
+    from mygrad_amd import _hip
+
+    published = {"f32_16x16x4": PEAK_TFLOPS["f32"], "f64_16x16x4": PEAK_TFLOPS["f64"], "f64_4x4x4_4b": PEAK_TFLOPS["f64"]}
+    out = {}
+    for kind in _hip.MFMA_KINDS:
+        rates = {w: _hip.probe_mfma(kind, w) for w in (1, 2, 4)}
+        best = max(rates.values())
+        out[kind] = {"tflops_by_waves_per_simd": rates, "best": best, "published_peak": published[kind],
+                     "frac_of_published": best / published[kind]}
+    return {"metric": "MFMA issue rate, registers only", "unit": "TFLOP/s", "shapes": out}
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -339,6 +355,8 @@ def main():
                     help="also time the step through the Python drop-in API (reported under 'dropin', never as value)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a 1 GiB device copy (the reference point for HBM traffic counters)")
+    ap.add_argument("--probe-mfma", action="store_true",
+                    help="run only the matrix-core rate probe (registers only, per MFMA shape)")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -347,6 +365,9 @@ def main():
 
     if args.calibrate_copy:
         print(json.dumps(run_copy_calibration()))
+        return
+    if args.probe_mfma:
+        print(json.dumps(run_mfma_probe()))
         return
 
     wl = WORKLOADS[args.workload]

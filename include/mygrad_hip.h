@@ -107,6 +107,15 @@ int mg_event_destroy(void *event);
 int mg_timing_enable(int on);
 int mg_timing_read(int32_t *tags, float *ms, int capacity, int *count);
 
+/* Device diagnostic, no counterpart in the reference: the rate at which the
+ * matrix cores retire one MFMA instruction shape when nothing else is in their way
+ * (independent accumulators in registers, no memory traffic), in TFLOP/s over the
+ * whole device.  kind: 0 = v_mfma_f32_16x16x4_f32, 1 = v_mfma_f64_16x16x4_f64,
+ * 2 = v_mfma_f64_4x4x4_4b_f64.  waves_per_simd: 1..8 wavefronts issuing on every
+ * SIMD.  It is the ceiling the convolution kernels' MFMA loops are measured against
+ * besides the published peak (bench.py --probe-mfma). */
+int mg_probe_mfma(int kind, int waves_per_simd, double *tflops);
+
 /* ---- convolution ---- */
 
 /* out[n,f,g] = sum_{c,t} w[f,c,t] * x[n,c,g*stride+t*dil-pad] (zero outside x).

@@ -106,6 +106,7 @@ _SIGNATURES = {
     "mg_timing_enable": [ctypes.c_int],
     "mg_timing_read": [ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_float), ctypes.c_int,
                        ctypes.POINTER(ctypes.c_int)],
+    "mg_probe_mfma": [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)],
     "mg_event_create": [ctypes.POINTER(_vp)],
     "mg_event_record": [_vp],
     "mg_event_elapsed_ms": [_vp, _vp, ctypes.POINTER(ctypes.c_float)],
@@ -225,6 +226,16 @@ def timing_read(capacity=1 << 16):
     check(lib().mg_timing_read(tags, ms, capacity, ctypes.byref(count)))
     n = min(count.value, capacity)
     return [(KERNEL_TAGS.get(tags[i], str(tags[i])), float(ms[i])) for i in range(n)]
+
+
+MFMA_KINDS = {"f32_16x16x4": 0, "f64_16x16x4": 1, "f64_4x4x4_4b": 2}
+
+
+def probe_mfma(kind, waves_per_simd=2):
+    """TFLOP/s the matrix cores sustain on one MFMA shape with nothing else in the way."""
+    out = ctypes.c_double()
+    check(lib().mg_probe_mfma(MFMA_KINDS[kind], int(waves_per_simd), ctypes.byref(out)))
+    return out.value
 
 
 def _right_aligned(values, fill):

@@ -122,6 +122,46 @@ using namespace mg;
 
 #define MG_LOCK() std::lock_guard<std::recursive_mutex> mg_guard_(::mg::api_mutex())
 
+// ---- matrix-core rate probe ---------------------------------------------------------
+namespace {
+typedef float probe_f32x4 __attribute__((ext_vector_type(4)));
+typedef double probe_f64x4 __attribute__((ext_vector_type(4)));
+
+// 16 independent accumulator tiles (8 for the 4-register fp64 tile) per wave, operands
+// fixed in registers: the loop is MFMA instructions and a counter, nothing else.
+template <int KIND>
+__global__ void __launch_bounds__(256) mfma_probe_kernel(double *sink, int iters) {
+  const double seed = 1.0 + 1e-3 * (threadIdx.x & 63);
+  double total = 0;
+  if constexpr (KIND == 0) {
+    probe_f32x4 acc[16];
+    for (int i = 0; i < 16; ++i) acc[i] = probe_f32x4{0, 0, 0, 0};
+    const float a = (float)seed, b = (float)(2.0 - seed);
+    for (int it = 0; it < iters; ++it)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, acc[i], 0, 0, 0);
+    for (int i = 0; i < 16; ++i) total += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+  } else if constexpr (KIND == 1) {
+    probe_f64x4 acc[8];
+    for (int i = 0; i < 8; ++i) acc[i] = probe_f64x4{0, 0, 0, 0};
+    const double a = seed, b = 2.0 - seed;
+    for (int it = 0; it < iters; ++it)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, acc[i], 0, 0, 0);
+    for (int i = 0; i < 8; ++i) total += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+  } else {
+    double acc[16];
+    for (int i = 0; i < 16; ++i) acc[i] = 0;
+    const double a = seed, b = 2.0 - seed;
+    for (int it = 0; it < iters; ++it)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[i] = __builtin_amdgcn_mfma_f64_4x4x4f64(a, b, acc[i], 0, 0, 0);
+    for (int i = 0; i < 16; ++i) total += acc[i];
+  }
+  sink[blockIdx.x * 256 + threadIdx.x] = total;
+}
+}  // namespace
+
 extern "C" {
 
 const char *mg_last_error(void) { return g_error; }
@@ -320,6 +360,43 @@ int mg_timing_read(int32_t *tags, float *ms, int capacity, int *count) {
     MG_HIP(hipEventElapsedTime(&ms[i], g_timing.records[i].start, g_timing.records[i].stop));
   }
   g_timing.used = 0;
+  return MG_OK;
+}
+
+int mg_probe_mfma(int kind, int waves_per_simd, double *tflops) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  if (!tflops) return fail(MG_ERR_BAD_ARG, "tflops is null");
+  if (kind < 0 || kind > 2) return fail(MG_ERR_BAD_ARG, "mfma probe kind %d (0..2)", kind);
+  if (waves_per_simd < 1 || waves_per_simd > 8) return fail(MG_ERR_BAD_ARG, "waves_per_simd %d (1..8)", waves_per_simd);
+  const int cus = runtime().props.multiProcessorCount;
+  const int blocks = cus * waves_per_simd;  // 256 threads = one wave on each of a unit's 4 SIMDs
+  const int iters = 4000;
+  void *sink = nullptr;
+  if (int rc = workspace((size_t)blocks * 256 * sizeof(double), &sink)) return rc;
+  hipStream_t s = runtime().stream;
+  hipEvent_t t0, t1;
+  MG_HIP(hipEventCreate(&t0));
+  MG_HIP(hipEventCreate(&t1));
+  float best = 0;
+  for (int rep = 0; rep < 4; ++rep) {  // the first repetition warms the clocks up
+    MG_HIP(hipEventRecord(t0, s));
+    if (kind == 0)
+      hipLaunchKernelGGL(mfma_probe_kernel<0>, dim3(blocks), dim3(256), 0, s, (double *)sink, iters);
+    else if (kind == 1)
+      hipLaunchKernelGGL(mfma_probe_kernel<1>, dim3(blocks), dim3(256), 0, s, (double *)sink, iters);
+    else
+      hipLaunchKernelGGL(mfma_probe_kernel<2>, dim3(blocks), dim3(256), 0, s, (double *)sink, iters);
+    MG_HIP(hipEventRecord(t1, s));
+    MG_HIP(hipEventSynchronize(t1));
+    float ms = 0;
+    MG_HIP(hipEventElapsedTime(&ms, t0, t1));
+    if (rep > 0 && (best == 0 || ms < best)) best = ms;
+  }
+  (void)hipEventDestroy(t0);
+  (void)hipEventDestroy(t1);
+  const double per_wave = kind == 0 ? 16 * 2048.0 : kind == 1 ? 8 * 2048.0 : 16 * 512.0;  // flops per loop trip
+  *tflops = (double)blocks * 4 * iters * per_wave / (best * 1e-3) * 1e-12;
   return MG_OK;
 }
 

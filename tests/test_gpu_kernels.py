@@ -312,3 +312,18 @@ def test_abi_rejects_bad_arguments(abi):
     assert lib.mg_maxpool_fwd(pdesc, 1, 1) == _hip.MG_ERR_UNSUPPORTED
     huge = ctypes.c_void_p()
     assert lib.mg_malloc(ctypes.byref(huge), 1 << 60) == _hip.MG_ERR_OOM
+
+
+@pytest.mark.gpu
+def test_mfma_probe_reports_plausible_rates():
+    """The diagnostic entry point runs and its figures are ordered the way the fp64
+    kernels rely on: the four-block 4x4x4 MFMA outruns the 16x16x4 one."""
+    from mygrad_amd import _hip
+
+    f32 = _hip.probe_mfma("f32_16x16x4", 2)
+    wide = _hip.probe_mfma("f64_16x16x4", 2)
+    quad = _hip.probe_mfma("f64_4x4x4_4b", 2)
+    assert 20.0 < f32 < 200.0 and 5.0 < wide < 100.0 and 5.0 < quad < 100.0
+    assert quad > wide
+    with pytest.raises(_hip.HipError):
+        _hip.probe_mfma("f32_16x16x4", 9)
