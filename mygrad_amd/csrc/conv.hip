@@ -1208,12 +1208,18 @@ int conv_wgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   if (staged) {
     const int count = g.F * ct;
     ScopedTiming timed(TAG_WGRAD_REDUCE);
-    if (pl.tap_major)
-      hipLaunchKernelGGL(tap_reduce_kernel<T>, dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, s,
-                         static_cast<const T *>(target), static_cast<T *>(dw), g.F, g.C, (int)g.wvol, pl.splits);
-    else
+    if (pl.tap_major) {
+      // four runs of splits per element when one thread per element would leave units idle
+      if (ceil_div(count, 256) < runtime().props.multiProcessorCount && pl.splits >= 16)
+        hipLaunchKernelGGL((tap_reduce_kernel<T, 4>), dim3((unsigned)ceil_div(count, 64)), dim3(256), 0, s,
+                           static_cast<const T *>(target), static_cast<T *>(dw), g.F, g.C, (int)g.wvol, pl.splits);
+      else
+        hipLaunchKernelGGL((tap_reduce_kernel<T, 1>), dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, s,
+                           static_cast<const T *>(target), static_cast<T *>(dw), g.F, g.C, (int)g.wvol, pl.splits);
+    } else {
       hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, s,
                          static_cast<const T *>(target), static_cast<T *>(dw), count, pl.splits);
+    }
     MG_HIP(hipGetLastError());
   }
   return MG_OK;

@@ -770,22 +770,46 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
   }
 }
 
-// dw[f][c][t] = ((part[0] + part[1]) + part[2]) + ...  of  part[s][f][col], where the
-// columns run over channel blocks of 16, then taps, then the channel inside the block:
-// col = ((c/16) * wvol + t) * 16 + c%16
-template <typename T>
+// dw[f][c][t] = the sum over K splits of part[s][f][col], where the columns run over
+// channel blocks of 16, then taps, then the channel inside the block:
+// col = ((c/16) * wvol + t) * 16 + c%16.
+// The splits are cut into RUNS runs (1 or 4); wave q of the block adds run q in split
+// order for 256 / RUNS consecutive elements, and the run sums are added in run order:
+// always the same association for a given plan, so the result repeats exactly.  Four
+// runs put four times the loads in flight, which pays when dw is too small to fill
+// the device with one thread per element.
+template <typename T, int RUNS>
 __global__ void __launch_bounds__(256) tap_reduce_kernel(const T *__restrict__ part, T *__restrict__ dw, int F, int C,
                                                          int wvol, int splits) {
+  constexpr int WIDTH = 256 / RUNS;
+  __shared__ T runs[4][64];
   const int count = F * C * wvol;
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;  // index into dw
-  if (i >= count) return;
-  const int ct = C * wvol;
-  const int f = i / ct;
-  const int r = i - f * ct;
-  const int c = r / wvol;
-  const int t = r - c * wvol;
-  const int src = f * ct + ((c / 16) * wvol + t) * 16 + c % 16;
-  dw[i] = sum_in_order(part + src, count, splits);
+  const int q = threadIdx.x / WIDTH, lane = threadIdx.x % WIDTH;
+  const int i = blockIdx.x * WIDTH + lane;  // index into dw
+  const int per = (splits + RUNS - 1) / RUNS;
+  const int first = min(q * per, splits), last = min(first + per, splits);
+  T sum = T(0);
+  if (i < count && first < last) {
+    const int ct = C * wvol;
+    const int f = i / ct;
+    const int r = i - f * ct;
+    const int c = r / wvol;
+    const int t = r - c * wvol;
+    const int src = f * ct + ((c / 16) * wvol + t) * 16 + c % 16;
+    sum = sum_in_order(part + (long long)first * count + src, count, last - first);
+  }
+  if constexpr (RUNS == 1) {
+    if (i < count) dw[i] = sum;
+    return;
+  }
+  runs[q][lane] = sum;
+  __syncthreads();
+  if (q == 0 && i < count) {
+    // runs past the last split are empty and hold +0.0; adding them changes nothing
+    // except that a total of -0.0 would read +0.0, which a sum of products starting
+    // from +0.0 accumulators cannot be
+    dw[i] = ((runs[0][lane] + runs[1][lane]) + runs[2][lane]) + runs[3][lane];
+  }
 }
 
 }  // namespace mg
