@@ -730,7 +730,8 @@ void fwd_table(const Geometry &g, std::vector<TabEntry> &tab) {
 int build_fwd_plan(const Geometry &g, Plan &pl) {
   Tables t;
   const int bk = gemm_bk(g.dtype);
-  pl.tap_major = g.C % bk == 0 && fits_buffer_loads(g);
+  // (the packed filter rows are read 16 bytes at a time: F must be a multiple of 4)
+  pl.tap_major = g.C % bk == 0 && g.F % 4 == 0 && fits_buffer_loads(g);
   pl.single_dense_phase = true;
   {
     const long long ktiles = pl.tap_major ? g.wvol * (g.C / bk) : ceil_div((long long)g.C * g.wvol, bk);
@@ -779,7 +780,7 @@ int build_fwd_plan(const Geometry &g, Plan &pl) {
 int build_dgrad_plan(const Geometry &g, Plan &pl) {
   Tables t;
   const int bk = gemm_bk(g.dtype);
-  pl.tap_major = g.F % bk == 0 && fits_buffer_loads(g);
+  pl.tap_major = g.F % bk == 0 && g.C % 4 == 0 && fits_buffer_loads(g);
   pl.single_dense_phase = g.S[0] == 1 && g.S[1] == 1 && g.S[2] == 1;
   const int gs[3] = {g.G[1] * g.G[2], g.G[2], 1};
   long long nphase = (long long)g.S[0] * g.S[1] * g.S[2];

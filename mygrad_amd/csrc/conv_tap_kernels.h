@@ -77,6 +77,15 @@ __device__ __forceinline__ int phase_first_block(const Phase *phases, int i) {
 // Tensors must be smaller than 2 GiB (kOutside must lie past the end).
 constexpr unsigned kOutside = 0x80000000u;
 
+// Sixteen bytes (VEC = 16 / sizeof(T) consecutive elements) per lane.
+template <typename T>
+__device__ __forceinline__ typename VecOf<T, 16 / sizeof(T)>::type buffer_load16(__amdgpu_buffer_rsrc_t rsrc, unsigned lane_bytes,
+                                                                               unsigned uniform_bytes) {
+  typedef unsigned u4 __attribute__((ext_vector_type(4)));
+  const u4 raw = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)lane_bytes, (int)uniform_bytes, 0);
+  return __builtin_bit_cast(typename VecOf<T, 16 / sizeof(T)>::type, raw);
+}
+
 constexpr int gcd_of(int a, int b) { return b == 0 ? a : gcd_of(b, a % b); }
 
 // Whether tap_gemm_kernel with BM rows per tile runs persistent blocks that stream
@@ -130,8 +139,12 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
   static_assert(BK % 4 == 0 && WM % 16 == 0 && WN % 16 == 0 && BN % 64 == 0, "MFMA 16x16x4 tiling");
   constexpr int TM = WM / 16, TN = WN / 16;
   constexpr int WAVES_N = BN / WN;
-  constexpr int AROWS = 256 / BM;
+  // the A tile (BK rows of BM packed filter values) is loaded and parked 16 bytes at a time
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int ALANES = BM / VEC;      // lanes that cover one row
+  constexpr int AROWS = 256 / ALANES;   // rows covered by one pass of the loader waves
   constexpr int ALOADS = (BK + AROWS - 1) / AROWS;
+  typedef typename VecOf<T, VEC>::type AVec;
   constexpr int BROWS = 256 / BN;
   constexpr int BLOADS = BK / BROWS;
   constexpr int PAD = 16 / sizeof(T);  // rows stay 16-byte aligned for the vector reads
@@ -196,8 +209,8 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
     const __amdgpu_buffer_rsrc_t src_buf = buffer_of<T>(p.src, p.src_bytes);
     const int bcol = tid % BN;
     const int brow0 = uniform(tid / BN);
-    const int acol = tid % BM;
-    const int arow0 = BM % 64 == 0 ? uniform(tid / BM) : tid / BM;
+    const int acol = (tid % ALANES) * VEC;
+    const int arow0 = tid / ALANES;
     const unsigned a_row_bytes = (unsigned)p.M * (unsigned)sizeof(T);
     const unsigned b_step = (unsigned)(BROWS * p.src_cstride) * (unsigned)sizeof(T);
 
@@ -242,16 +255,30 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
     // issues the same loads, so the compiler can count them exactly.
     bool live = false;  // the cursor is on a K tile that has not been requested yet
     int requested = 0;  // stream elements requested so far
-    auto fetch = [&](T(&ra)[ALOADS], T(&rb)[BLOADS]) {
+    auto fetch = [&](AVec(&ra)[ALOADS], T(&rb)[BLOADS]) {
+#ifdef EXP_NOFETCH
+      for (int r = 0; r < ALOADS; ++r) ra[r] = AVec(T(kt));
+      for (int r = 0; r < BLOADS; ++r) rb[r] = T(kt);
+      if (live) { ++requested; if (kt + 1 < it.kt_end) ++kt; else if constexpr (STREAM) live = enter(item + (int)gridDim.x); else live = false; }
+      return;
+#endif
       const int8v e = ktab[kt];  // a_row0, coff, d0, d1, d2
+#ifdef EXP_NOA
+      for (int r = 0; r < ALOADS; ++r) ra[r] = AVec(T(kt));
+#else
       const unsigned a_tile = (unsigned)e[0] * a_row_bytes;
 #pragma unroll
-      for (int r = 0; r < ALOADS; ++r) ra[r] = buffer_load<T>(a_buf, a_at, a_tile + (unsigned)(r * AROWS) * a_row_bytes);
+      for (int r = 0; r < ALOADS; ++r) ra[r] = buffer_load16<T>(a_buf, a_at, a_tile + (unsigned)(r * AROWS) * a_row_bytes);
+#endif
       const bool ok = pos_ok & ((unsigned)(qb0 + e[2]) < (unsigned)p.Q[0]) & ((unsigned)(qb1 + e[3]) < (unsigned)p.Q[1]) &
                       ((unsigned)(qb2 + e[4]) < (unsigned)p.Q[2]);
       const unsigned at = ok ? src_at + (unsigned)(e[1] * (int)sizeof(T)) : kOutside;
+#ifdef EXP_NOB
+      for (int r = 0; r < BLOADS; ++r) rb[r] = T(at);
+#else
 #pragma unroll
       for (int r = 0; r < BLOADS; ++r) rb[r] = buffer_load<T>(src_buf, at, (unsigned)r * b_step);
+#endif
       if (live) {
         ++requested;
         if (kt + 1 < it.kt_end)
@@ -262,11 +289,11 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
           live = false;
       }
     };
-    auto stash = [&](const T(&ra)[ALOADS], const T(&rb)[BLOADS], int buf) {
+    auto stash = [&](const AVec(&ra)[ALOADS], const T(&rb)[BLOADS], int buf) {
 #pragma unroll
       for (int r = 0; r < ALOADS; ++r) {
         const int kk = arow0 + r * AROWS;
-        if (kk < BK) As[buf][kk][acol] = ra[r];
+        if (kk < BK) *reinterpret_cast<AVec *>(&As[buf][kk][acol]) = ra[r];
       }
 #pragma unroll
       for (int r = 0; r < BLOADS; ++r) Bs[buf][brow0 + r * BROWS][bcol] = rb[r];
@@ -274,7 +301,8 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
 
     // two register sets: stream element s travels in set s % 2 and is requested two
     // elements before it is parked in LDS
-    T ra0[ALOADS], rb0[BLOADS], ra1[ALOADS], rb1[BLOADS];
+    AVec ra0[ALOADS], ra1[ALOADS];
+    T rb0[BLOADS], rb1[BLOADS];
     live = enter((int)blockIdx.x);
     if (live) {
       fetch(ra0, rb0);
