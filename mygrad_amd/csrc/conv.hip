@@ -77,17 +77,25 @@ struct Mma<double> {
 //   mode 1 (dgrad)              : Ap[(f*Wvol + t)][c] = w[f][c][t]
 //   mode 2 (forward, tap-major) : Ap[(t*C + c)][f]    = w[f][c][t]
 //   mode 3 (dgrad, tap-major)   : Ap[(t*F + f)][c]    = w[f][c][t]
+// Modes 2 and 3 pad every row with zeros to a multiple of four values (`ld` values per
+// row), so that the kernels can read a row sixteen bytes at a time whatever M is.
 // ------------------------------------------------------------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(256) pack_filters_kernel(const T *__restrict__ w, T *__restrict__ ap, int F, int C,
-                                                           int wvol, int mode) {
-  const int total = F * C * wvol;
+                                                           int wvol, int mode, int ld) {
+  const int M = (mode == 0 || mode == 2) ? F : C;
+  const int total = (F * C * wvol / M) * ld;
   for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
     // idx enumerates the packed layout so that stores are coalesced
+    const int m = idx % ld;
+    const int row = idx / ld;
+    if (m >= M) {
+      ap[idx] = T(0);
+      continue;
+    }
     int f, c, t;
     if (mode == 0 || mode == 2) {
-      f = idx % F;
-      const int row = idx / F;
+      f = m;
       if (mode == 0) {
         t = row % wvol;
         c = row / wvol;
@@ -96,8 +104,7 @@ __global__ void __launch_bounds__(256) pack_filters_kernel(const T *__restrict__
         t = row / C;
       }
     } else {
-      c = idx % C;
-      const int row = idx / C;
+      c = m;
       if (mode == 1) {
         t = row % wvol;
         f = row / wvol;
@@ -461,7 +468,7 @@ bool fits_buffer_loads(const Geometry &g) {
   const long long elem = g.dtype == MG_F64 ? 8 : 4;
   const long long limit = 1ll << 31;
   return (long long)g.N * g.C * g.xvol * elem < limit && (long long)g.N * g.F * g.gvol * elem < limit &&
-         (long long)g.F * g.C * g.wvol * elem < limit;
+         (long long)(g.F + 3) * (g.C + 3) * g.wvol * elem < limit;  // packed filter rows are padded to 4 values
 }
 
 // K tile of the gather-GEMMs (positions x filters-or-channels x BK).
@@ -482,6 +489,7 @@ struct Plan {
   int m_tiles = 1;     // row tiles per position block
   int full_tiles = 0;  // tiles computed whole by one block (tap-major kernel)
   int tail_split = 1;  // blocks sharing each of the remaining tiles
+  int blocks_per_cu = 1;  // persistent blocks per compute unit (streaming gather-GEMM)
   bool tap_major = false;  // which kernel family the tables are for
   bool single_dense_phase = false;  // positions enumerate the destination tensor in order
   // wgrad
@@ -585,15 +593,19 @@ int gemm_blocks_per_cu(int bm, int bn) {
   return 1;
 }
 
-// Picks the tile of the gather-GEMM and how its last, partial round of tiles is
-// shared out.  The tap-major kernel runs as many persistent blocks as the device
-// holds at once ("slots"); block b takes tiles b, b + slots, ...  After
-// floor(T / slots) whole tiles per block, T % slots tiles are left that would keep
-// only some blocks busy for a full tile time, so each of those is cut into `split`
-// K slices and every block gets about the same share of them.  Smaller tiles give
-// more tiles (finer balance, less padding) at some cost in operand reuse.
+// Picks the tile of the gather-GEMM, how many persistent blocks run per compute unit
+// and how the last, partial round of tiles is shared out.  With r blocks per unit the
+// grid has r x CUs blocks; block b takes tiles b, b + grid, ...  A unit's MFMA pipes are
+// shared by its blocks, so one round of the grid costs r tile times.  After
+// floor(T / grid) whole rounds, T % grid tiles are left that would keep only some
+// units busy; each of those is cut into `split` K slices so that every unit gets
+// about the same share of them (the busiest gets ceil(rem x split / CUs) slices).
+// Smaller tiles give more tiles (finer balance, less padding) at some cost in operand
+// reuse.  Kernels that do not stream run one block per tile (r = 1 in this arithmetic:
+// the hardware refills a unit as soon as a block leaves).
 struct TileChoice {
   int bm, bn, m_tiles, full_tiles, tail_split;
+  int blocks_per_cu;  // persistent blocks per compute unit (streaming kernels)
   long long tiles;
 };
 
@@ -603,7 +615,7 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
     double penalty;  // relative cost of a flop in this tile shape
     bool tap_only;
   };
-  static const Cfg cfgs[] = {{128, 128, 1.00, false}, {128, 64, 1.10, true}, {64, 256, 1.00, false}, {64, 128, 1.08, true},
+  static const Cfg cfgs[] = {{128, 128, 1.00, false}, {128, 64, 1.05, true}, {64, 256, 1.00, false}, {64, 128, 1.08, true},
                              {32, 256, 1.00, false},  {32, 128, 1.10, true}, {16, 256, 1.00, false}};
   const int bm = pick_bm(M);
   const int cus = runtime().props.multiProcessorCount;
@@ -614,42 +626,46 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
     // 64x64 fp64 wave tiles hold 128 accumulator registers: only one 8-wave block
     // fits on a compute unit, so the tap-major kernels use the half-size shapes
     if (tap_major && elem == 8 && c.bn * c.bm >= 128 * 128) continue;
-    TileChoice t{};
-    t.bm = c.bm;
-    t.bn = c.bn;
-    t.m_tiles = (int)ceil_div(M, c.bm);
+    const bool stream = tap_major && tap_gemm_streams(c.bm, (int)elem);
+    const int per_cu = !stream ? 1 : elem == 8 ? gemm_blocks_per_cu<double>(c.bm, c.bn) : gemm_blocks_per_cu<float>(c.bm, c.bn);
     long long pos_blocks = 0;
     for (long long n : phase_npos) pos_blocks += ceil_div(n, c.bn);
-    t.tiles = pos_blocks * t.m_tiles;
-    t.full_tiles = (int)t.tiles;
-    t.tail_split = 1;
-    double tail = 0;
-    // blocks sharing a compute unit share its MFMA pipes: a round of `slots` tiles
-    // takes per_cu tile times
-    const int per_cu = !tap_major ? 1 : elem == 8 ? gemm_blocks_per_cu<double>(c.bm, c.bn) : gemm_blocks_per_cu<float>(c.bm, c.bn);
-    const bool stream = tap_major && tap_gemm_streams(c.bm, (int)elem);
-    const long long slots = stream ? (long long)per_cu * cus : cus;
-    const long long rem = t.tiles % slots;
-    if (rem > 0) {
-      tail = 1.0;
-      if (tap_major) {
-        // slices of at least two K tiles, at most 32 MB of partial sums
-        const long long tile_bytes = (long long)c.bm * c.bn * (long long)elem;
-        const int smax = (int)std::max<long long>(1, std::min<long long>({(long long)min_ktiles / 2, 32ll, (32ll << 20) / (rem * tile_bytes)}));
-        for (int sp = 2; sp <= smax; ++sp) {
-          const double share = (double)ceil_div(rem * sp, slots) / sp + 0.01 * sp;  // + a little for the fix-up pass
-          if (share < tail - 1e-9) {
-            tail = share;
-            t.tail_split = sp;
+    for (int r = 1; r <= per_cu; ++r) {
+      TileChoice t{};
+      t.bm = c.bm;
+      t.bn = c.bn;
+      t.blocks_per_cu = r;
+      t.m_tiles = (int)ceil_div(M, c.bm);
+      t.tiles = pos_blocks * t.m_tiles;
+      t.full_tiles = (int)t.tiles;
+      t.tail_split = 1;
+      const long long grid = (long long)r * cus;
+      const long long rem = t.tiles % grid;
+      double tail = 0;  // tile times the busiest unit spends on the remaining tiles
+      if (rem > 0) {
+        tail = (double)ceil_div(rem, cus);
+        if (tap_major) {
+          // slices of at least two K tiles, at most 32 MB of partial sums
+          const long long tile_bytes = (long long)c.bm * c.bn * (long long)elem;
+          const int smax = (int)std::max<long long>(1, std::min<long long>({(long long)min_ktiles / 2, 32ll, (32ll << 20) / (rem * tile_bytes)}));
+          for (int sp = 2; sp <= smax; ++sp) {
+            const double share = (double)ceil_div(rem * sp, cus) / sp + 0.01 * sp;  // + a little for the fix-up pass
+            if (share < tail - 1e-9) {
+              tail = share;
+              t.tail_split = sp;
+            }
           }
+          if (t.tail_split > 1) t.full_tiles = (int)(t.tiles - rem);
         }
-        if (t.tail_split > 1) t.full_tiles = (int)(t.tiles - rem);
       }
-    }
-    const double cost = ((double)(t.tiles / slots) + tail) * (stream ? per_cu : 1) * c.bm * c.bn * c.penalty;
-    if (best.bm == 0 || cost < best_cost) {
-      best = t;
-      best_cost = cost;
+      // a streaming block alone on its unit leaves the MFMA pipes idle while it waits
+      // at its barriers; two or more cover for one another
+      const double alone = stream && r == 1 ? 1.4 : 1.0;
+      const double cost = ((double)(t.tiles / grid) * r + tail) * alone * c.bm * c.bn * c.penalty;
+      if (best.bm == 0 || cost < best_cost) {
+        best = t;
+        best_cost = cost;
+      }
     }
   }
   return best;
@@ -730,13 +746,12 @@ void fwd_table(const Geometry &g, std::vector<TabEntry> &tab) {
 int build_fwd_plan(const Geometry &g, Plan &pl) {
   Tables t;
   const int bk = gemm_bk(g.dtype);
-  // (the packed filter rows are read 16 bytes at a time: F must be a multiple of 4)
-  pl.tap_major = g.C % bk == 0 && g.F % 4 == 0 && fits_buffer_loads(g);
+  pl.tap_major = g.C % bk == 0 && fits_buffer_loads(g);
   pl.single_dense_phase = true;
   {
     const long long ktiles = pl.tap_major ? g.wvol * (g.C / bk) : ceil_div((long long)g.C * g.wvol, bk);
     const TileChoice tc = choose_tile(g.F, {(long long)g.N * g.gvol}, (int)ktiles, pl.tap_major, g.dtype == MG_F64 ? 8 : 4);
-    pl.bm = tc.bm, pl.bn = tc.bn, pl.m_tiles = tc.m_tiles, pl.full_tiles = tc.full_tiles, pl.tail_split = tc.tail_split;
+    pl.bm = tc.bm, pl.bn = tc.bn, pl.m_tiles = tc.m_tiles, pl.full_tiles = tc.full_tiles, pl.tail_split = tc.tail_split, pl.blocks_per_cu = tc.blocks_per_cu;
   }
   Phase ph{};
   for (int k = 0; k < 3; ++k) {
@@ -780,7 +795,7 @@ int build_fwd_plan(const Geometry &g, Plan &pl) {
 int build_dgrad_plan(const Geometry &g, Plan &pl) {
   Tables t;
   const int bk = gemm_bk(g.dtype);
-  pl.tap_major = g.F % bk == 0 && g.C % 4 == 0 && fits_buffer_loads(g);
+  pl.tap_major = g.F % bk == 0 && fits_buffer_loads(g);
   pl.single_dense_phase = g.S[0] == 1 && g.S[1] == 1 && g.S[2] == 1;
   const int gs[3] = {g.G[1] * g.G[2], g.G[2], 1};
   long long nphase = (long long)g.S[0] * g.S[1] * g.S[2];
@@ -834,7 +849,7 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
       min_ktiles = std::min(min_ktiles, pl.tap_major ? ntaps * (g.F / bk) : ceil_div(ntaps * g.F, bk));
     }
     const TileChoice tc = choose_tile(g.C, npos, (int)std::max<long long>(min_ktiles, 0), pl.tap_major, g.dtype == MG_F64 ? 8 : 4);
-    pl.bm = tc.bm, pl.bn = tc.bn, pl.m_tiles = tc.m_tiles, pl.full_tiles = tc.full_tiles, pl.tail_split = tc.tail_split;
+    pl.bm = tc.bm, pl.bn = tc.bn, pl.m_tiles = tc.m_tiles, pl.full_tiles = tc.full_tiles, pl.tail_split = tc.tail_split, pl.blocks_per_cu = tc.blocks_per_cu;
   }
 
   // ---- tables
@@ -1015,8 +1030,7 @@ void launch_gemm(GemmParams &gp, const Plan &pl, hipStream_t s) {
   if (pl.tap_major) {
     const long long tiles = (long long)pl.pos_blocks * pl.m_tiles;
     const long long tail_tiles = tiles - pl.full_tiles;
-    static const int per_cu = resident_blocks(tap_gemm_kernel<T, BM, BN, BK, WM, WN>, 512);
-    const long long slots = tap_gemm_streams(BM, (int)sizeof(T)) ? (long long)per_cu * runtime().props.multiProcessorCount : (1ll << 40);
+    const long long slots = tap_gemm_streams(BM, (int)sizeof(T)) ? (long long)pl.blocks_per_cu * runtime().props.multiProcessorCount : (1ll << 40);
     gp.items = (int)(pl.full_tiles + tail_tiles * pl.tail_split);
     hipLaunchKernelGGL((tap_gemm_kernel<T, BM, BN, BK, WM, WN>), dim3((unsigned)std::min<long long>(gp.items, slots)), dim3(512),
                        0, s, gp);
@@ -1069,16 +1083,22 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
 
 // Packs the filters into the front of the library workspace; `extra` more bytes
 // behind them (256-byte aligned) are reserved for the caller and returned in *behind.
+// Values per row of the packed filters: M itself for the table-driven kernels, M rounded
+// up to a multiple of four for the tap-major ones.
+inline int packed_ld(int M, bool tap_major) { return tap_major ? (M + 3) / 4 * 4 : M; }
+
 template <typename T>
 int pack_filters(const Geometry &g, const void *w, int mode, void **packed, size_t extra = 0, void **behind = nullptr) {
-  const size_t count = (size_t)g.F * g.C * g.wvol;
+  const int M = (mode == 0 || mode == 2) ? g.F : g.C;
+  const int ld = packed_ld(M, mode >= 2);
+  const size_t count = (size_t)g.F * g.C * g.wvol / M * ld;
   const size_t packed_bytes = (count * sizeof(T) + 255) & ~size_t(255);
   if (int rc = workspace(packed_bytes + extra, packed)) return rc;
   if (behind) *behind = static_cast<char *>(*packed) + packed_bytes;
   const unsigned blocks = (unsigned)std::min<long long>(ceil_div((long long)count, 256), 4096);
   ScopedTiming timed(TAG_PACK_FILTERS);
   hipLaunchKernelGGL(pack_filters_kernel<T>, dim3(blocks), dim3(256), 0, runtime().stream, static_cast<const T *>(w),
-                     static_cast<T *>(*packed), g.F, g.C, (int)g.wvol, mode);
+                     static_cast<T *>(*packed), g.F, g.C, (int)g.wvol, mode, ld);
   MG_HIP(hipGetLastError());
   return MG_OK;
 }
@@ -1107,7 +1127,8 @@ int conv_fwd_impl(const Geometry &g, const Plan &pl, const void *x, const void *
   gp.src_cstride = (int)g.xvol;
   gp.src_nstride = (long long)g.C * g.xvol;
   gp.dst_nstride = (long long)g.F * g.gvol;
-  gp.a_bytes = (unsigned)((size_t)g.F * g.C * g.wvol * sizeof(T));
+  gp.a_ld = packed_ld(g.F, pl.tap_major);
+  gp.a_bytes = (unsigned)((size_t)g.C * g.wvol * gp.a_ld * sizeof(T));
   gp.src_bytes = pl.tap_major ? (unsigned)((size_t)g.N * g.C * g.xvol * sizeof(T)) : 0;
   return run_gemm<T>(gp, pl, TAG_CONV_FWD, runtime().stream);
 }
@@ -1136,7 +1157,8 @@ int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   gp.src_cstride = (int)g.gvol;
   gp.src_nstride = (long long)g.F * g.gvol;
   gp.dst_nstride = (long long)g.C * g.xvol;
-  gp.a_bytes = (unsigned)((size_t)g.F * g.C * g.wvol * sizeof(T));
+  gp.a_ld = packed_ld(g.C, pl.tap_major);
+  gp.a_bytes = (unsigned)((size_t)g.F * g.wvol * gp.a_ld * sizeof(T));
   gp.src_bytes = pl.tap_major ? (unsigned)((size_t)g.N * g.F * g.gvol * sizeof(T)) : 0;
   return run_gemm<T>(gp, pl, TAG_CONV_DGRAD, runtime().stream);
 }

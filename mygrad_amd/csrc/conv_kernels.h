@@ -96,6 +96,7 @@ struct GemmParams {
   const KTile *ktiles;  // Phase::k_begin / k_count index this table
   const void *zeros;    // a few zero elements in device memory
   unsigned a_bytes, src_bytes;  // sizes of A and src (each below 2 GiB)
+  int a_ld;                     // values per row of A (M rounded up to a multiple of 4)
   int src_cstride;      // element stride between consecutive channels of the gathered tensor
   int vec_store;        // positions are contiguous in dst: a lane may store its TN positions as one vector
   int m_tiles;          // row tiles per position block

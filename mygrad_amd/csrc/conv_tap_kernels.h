@@ -211,7 +211,7 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
     const int brow0 = uniform(tid / BN);
     const int acol = (tid % ALANES) * VEC;
     const int arow0 = tid / ALANES;
-    const unsigned a_row_bytes = (unsigned)p.M * (unsigned)sizeof(T);
+    const unsigned a_row_bytes = (unsigned)p.a_ld * (unsigned)sizeof(T);
     const unsigned b_step = (unsigned)(BROWS * p.src_cstride) * (unsigned)sizeof(T);
 
     // ---- fetch cursor: the item being gathered and this thread's place in it
@@ -244,8 +244,8 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
         qb2 = (int)j2 * p.sj[2];
         src_at = (unsigned)((long long)n * p.src_nstride + (qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2]) +
                             brow0 * p.src_cstride) * (unsigned)sizeof(T);
-        const bool a_ok = (it.m0 + acol < p.M) & (arow0 < BK);
-        a_at = a_ok ? (unsigned)(arow0 * p.M + it.m0 + acol) * (unsigned)sizeof(T) : kOutside;
+        const bool a_ok = (it.m0 + acol < p.a_ld) & (arow0 < BK);  // rows are padded to whole 16-byte pieces
+        a_at = a_ok ? (unsigned)(arow0 * p.a_ld + it.m0 + acol) * (unsigned)sizeof(T) : kOutside;
         return true;
       }
       return false;
@@ -295,8 +295,13 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
         const int kk = arow0 + r * AROWS;
         if (kk < BK) *reinterpret_cast<AVec *>(&As[buf][kk][acol]) = ra[r];
       }
+#ifdef EXP_NOBSTASH
+      for (int r = 1; r < BLOADS; ++r) asm volatile("" ::"v"(rb[r]));
+      Bs[buf][brow0][bcol] = rb[0];
+#else
 #pragma unroll
       for (int r = 0; r < BLOADS; ++r) Bs[buf][brow0 + r * BROWS][bcol] = rb[r];
+#endif
     };
 
     // two register sets: stream element s travels in set s % 2 and is requested two
