@@ -910,7 +910,7 @@ template <typename T>
 int wgrad_blocks_per_cu(int bm, int bn, bool tap_major) {
 #define MG_OCC(TT, BM, BN, BK, WM, WN)                                                     \
   if (bm == BM && bn == BN) {                                                              \
-    if (tap_major) return resident_blocks(tap_wgrad_kernel<TT, BM, BN, BK, WM, WN>, 512);  \
+    if (tap_major) return resident_blocks(tap_wgrad_kernel<TT, BM, BN, BK, WM, WN, true>, 512);  \
     if constexpr (BN == 64) return resident_blocks(wgrad_kernel<TT, BM, BN, BK, WM, WN>, 256); \
   }
   MG_WGRAD_SHAPES(T, MG_OCC)
@@ -1170,7 +1170,10 @@ void launch_wgrad(WgradParams &wp, bool tap_major, hipStream_t s) {
   if (tap_major) {
     // one-dimensional grid, whole K splits per XCD (see the kernel)
     const long long blocks = (long long)wp.splits * wp.col_tiles * wp.row_tiles;
-    hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN>), dim3((unsigned)blocks), dim3(512), 0, s, wp);
+    if (wp.gvol % (int)(16 / sizeof(T)) == 0)
+      hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN, true>), dim3((unsigned)blocks), dim3(512), 0, s, wp);
+    else
+      hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN, false>), dim3((unsigned)blocks), dim3(512), 0, s, wp);
   } else if constexpr (BN == 64) {
     const dim3 grid((unsigned)wp.col_tiles, (unsigned)wp.row_tiles, (unsigned)wp.splits);
     hipLaunchKernelGGL((wgrad_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, wp);

@@ -14,6 +14,8 @@
 // shapes take the table-driven kernels.
 #pragma once
 
+#include <type_traits>
+
 namespace mg {
 
 typedef int int8v __attribute__((ext_vector_type(8)));
@@ -543,7 +545,10 @@ __global__ void __launch_bounds__(256) tail_fixup_kernel(const GemmParams p) {
 // ------------------------------------------------------------------------------------------
 // filter gradient
 // ------------------------------------------------------------------------------------------
-template <typename T, int BM, int BN, int BK, int WM, int WN>
+// WIDE: the positions of one sample are a multiple of 16 bytes, so 16 bytes of grad (4 or
+// 2 consecutive positions of one filter) never straddle two samples and the grad tile
+// is loaded and parked 16 bytes per lane; otherwise element by element.
+template <typename T, int BM, int BN, int BK, int WM, int WN, bool WIDE>
 __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
   static_assert((BM / WM) * (BN / WN) == 4, "four wavefronts per block");
   static_assert(256 % BK == 0 && BK % 16 == 0 && BN % 16 == 0, "K tile");
@@ -551,7 +556,13 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
   constexpr int WAVES_N = BN / WN;
   constexpr int ROWS = 256 / BK;  // tile rows covered by one pass of the block
   static_assert(16 % ROWS == 0 && BM % ROWS == 0, "row passes must not straddle a column group");
-  constexpr int ALOADS = BM / ROWS;
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int APIECES = BK / VEC;      // 16-byte pieces per row of the grad tile
+  constexpr int APASS = 256 / APIECES;   // rows covered by one pass when loading pieces
+  static_assert(!WIDE || BM % APASS == 0, "grad tile passes");
+  constexpr int ALOADS = WIDE ? BM / APASS : BM / ROWS;
+  typedef typename VecOf<T, VEC>::type AVec;
+  typedef typename std::conditional<WIDE, AVec, T>::type AReg;
   constexpr int NGROUPS = BN / 16;
   // A loader thread owns one position of the K tile and one of ROWS row slots.  The
   // padding test is per (position, column group), so the slots share out the groups
@@ -612,11 +623,22 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
   for (int i = 0; i < MYGROUPS; ++i) grp[i] = gtab[gsel + i * GSPLIT];
 
   constexpr int NB = MYGROUPS * CLOADS;
-  T ra0[ALOADS], rb0[NB], ra1[ALOADS], rb1[NB];
-  const unsigned a_step = (unsigned)(ROWS * p.gvol) * (unsigned)sizeof(T);
+  AReg ra0[ALOADS], ra1[ALOADS];
+  T rb0[NB], rb1[NB];
+  const unsigned a_step = (unsigned)((WIDE ? APASS : ROWS) * p.gvol) * (unsigned)sizeof(T);
+  const int apiece = tid % APIECES, arow = tid / APIECES;  // WIDE: this thread's piece of the grad tile
   const unsigned b_step = (unsigned)(CSPLIT * p.x_cstride) * (unsigned)sizeof(T);
 
-  auto fetch = [&](T(&ra)[ALOADS], T(&rb)[NB], int kt) {
+  auto fetch = [&](AReg(&ra)[ALOADS], T(&rb)[NB], int kt) {
+    if constexpr (WIDE) {
+      const int apos = kbeg + kt * BK + apiece * VEC;  // the piece lies inside one sample and inside the split or not at all
+      const unsigned an = p.by_gvol.div((unsigned)apos);
+      const unsigned aflat = (unsigned)apos - an * (unsigned)p.gvol;
+      const unsigned g_at = apos < kend ? (unsigned)((long long)an * p.g_nstride + aflat + (long long)(m0 + arow) * p.gvol) * (unsigned)sizeof(T)
+                                        : kOutside;
+#pragma unroll
+      for (int r = 0; r < ALOADS; ++r) ra[r] = buffer_load16<T>(grad_buf, g_at, (unsigned)r * a_step);
+    }
     const int ipos = kbeg + kt * BK + kcol;
     const bool pos_ok = ipos < kend;
     const unsigned pos = pos_ok ? (unsigned)ipos : (unsigned)kbeg;
@@ -629,10 +651,12 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
     const int qb0 = (int)g0 * p.sj[0];
     const int qb1 = (int)g1 * p.sj[1];
     const int qb2 = (int)g2 * p.sj[2];
-    const unsigned g_at =
-        pos_ok ? (unsigned)((long long)n * p.g_nstride + gflat + (long long)(m0 + row0) * p.gvol) * (unsigned)sizeof(T) : kOutside;
+    if constexpr (!WIDE) {
+      const unsigned g_at =
+          pos_ok ? (unsigned)((long long)n * p.g_nstride + gflat + (long long)(m0 + row0) * p.gvol) * (unsigned)sizeof(T) : kOutside;
 #pragma unroll
-    for (int r = 0; r < ALOADS; ++r) ra[r] = buffer_load<T>(grad_buf, g_at, (unsigned)r * a_step);
+      for (int r = 0; r < ALOADS; ++r) ra[r] = buffer_load<T>(grad_buf, g_at, (unsigned)r * a_step);
+    }
     const unsigned x_at = (unsigned)((long long)n * p.x_nstride + (qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2]) +
                                      (long long)csel * p.x_cstride) * (unsigned)sizeof(T);
 #pragma unroll
@@ -645,9 +669,14 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
       for (int r = 0; r < CLOADS; ++r) rb[j * CLOADS + r] = buffer_load<T>(x_buf, at, (unsigned)r * b_step);
     }
   };
-  auto stash = [&](const T(&ra)[ALOADS], const T(&rb)[NB], int buf) {
+  auto stash = [&](const AReg(&ra)[ALOADS], const T(&rb)[NB], int buf) {
 #pragma unroll
-    for (int r = 0; r < ALOADS; ++r) As[buf][row0 + r * ROWS][kcol] = ra[r];
+    for (int r = 0; r < ALOADS; ++r) {
+      if constexpr (WIDE)
+        *reinterpret_cast<AVec *>(&As[buf][arow + r * APASS][apiece * VEC]) = ra[r];
+      else
+        As[buf][row0 + r * ROWS][kcol] = ra[r];
+    }
 #pragma unroll
     for (int j = 0; j < MYGROUPS; ++j)
 #pragma unroll
