@@ -355,6 +355,7 @@ def main():
                     help="also time the step through the Python drop-in API (reported under 'dropin', never as value)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a 1 GiB device copy (the reference point for HBM traffic counters)")
+    ap.add_argument("--copy-mib", type=int, default=1024, help="size of the --calibrate-copy buffer in MiB (read + written)")
     ap.add_argument("--probe-mfma", action="store_true",
                     help="run only the matrix-core rate probe (registers only, per MFMA shape)")
     args = ap.parse_args()
@@ -364,7 +365,7 @@ def main():
                  "by design but no multi-GPU code is part of it")
 
     if args.calibrate_copy:
-        print(json.dumps(run_copy_calibration()))
+        print(json.dumps(run_copy_calibration(args.copy_mib)))
         return
     if args.probe_mfma:
         print(json.dumps(run_mfma_probe()))

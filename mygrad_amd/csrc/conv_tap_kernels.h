@@ -258,29 +258,15 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
     bool live = false;  // the cursor is on a K tile that has not been requested yet
     int requested = 0;  // stream elements requested so far
     auto fetch = [&](AVec(&ra)[ALOADS], T(&rb)[BLOADS]) {
-#ifdef EXP_NOFETCH
-      for (int r = 0; r < ALOADS; ++r) ra[r] = AVec(T(kt));
-      for (int r = 0; r < BLOADS; ++r) rb[r] = T(kt);
-      if (live) { ++requested; if (kt + 1 < it.kt_end) ++kt; else if constexpr (STREAM) live = enter(item + (int)gridDim.x); else live = false; }
-      return;
-#endif
       const int8v e = ktab[kt];  // a_row0, coff, d0, d1, d2
-#ifdef EXP_NOA
-      for (int r = 0; r < ALOADS; ++r) ra[r] = AVec(T(kt));
-#else
       const unsigned a_tile = (unsigned)e[0] * a_row_bytes;
 #pragma unroll
       for (int r = 0; r < ALOADS; ++r) ra[r] = buffer_load16<T>(a_buf, a_at, a_tile + (unsigned)(r * AROWS) * a_row_bytes);
-#endif
       const bool ok = pos_ok & ((unsigned)(qb0 + e[2]) < (unsigned)p.Q[0]) & ((unsigned)(qb1 + e[3]) < (unsigned)p.Q[1]) &
                       ((unsigned)(qb2 + e[4]) < (unsigned)p.Q[2]);
       const unsigned at = ok ? src_at + (unsigned)(e[1] * (int)sizeof(T)) : kOutside;
-#ifdef EXP_NOB
-      for (int r = 0; r < BLOADS; ++r) rb[r] = T(at);
-#else
 #pragma unroll
       for (int r = 0; r < BLOADS; ++r) rb[r] = buffer_load<T>(src_buf, at, (unsigned)r * b_step);
-#endif
       if (live) {
         ++requested;
         if (kt + 1 < it.kt_end)
@@ -297,13 +283,8 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
         const int kk = arow0 + r * AROWS;
         if (kk < BK) *reinterpret_cast<AVec *>(&As[buf][kk][acol]) = ra[r];
       }
-#ifdef EXP_NOBSTASH
-      for (int r = 1; r < BLOADS; ++r) asm volatile("" ::"v"(rb[r]));
-      Bs[buf][brow0][bcol] = rb[0];
-#else
 #pragma unroll
       for (int r = 0; r < BLOADS; ++r) Bs[buf][brow0 + r * BROWS][bcol] = rb[r];
-#endif
     };
 
     // two register sets: stream element s travels in set s % 2 and is requested two
