@@ -227,6 +227,43 @@ def test_conv_channel_counts_that_take_the_tap_major_kernels(abi, dtype, m):
         done += 1
 
 
+# Shapes picked so that, between them, every tile shape and code path of the tap-major
+# kernels runs: all gather-GEMM tiles (rows 16..128), persistent blocks that stream
+# through several tiles and K slices, strided dgrad phases, filter counts that are not a
+# multiple of four (padded packed rows), the 128x128 / 64x192 / 64x128 / 64x64 / 32x64 /
+# 16x64 filter-gradient tiles, and an odd number of positions per sample (grad tile
+# loaded element by element instead of 16 bytes per lane).
+KERNEL_VARIANT_CASES = [
+    # x shape, w shape, stride, padding, dilation
+    ((8, 128, 28, 28), (128, 128, 3, 3), (1, 1), (1, 1), (1, 1)),   # 128-row tiles, wgrad 128x128
+    ((32, 64, 28, 28), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1)),     # 64x256, wgrad 64x192
+    ((64, 64, 28, 28), (64, 64, 2, 2), (1, 1), (0, 0), (1, 1)),     # wgrad 64x128
+    ((16, 128, 29, 29), (256, 128, 3, 3), (2, 2), (1, 1), (1, 1)),  # four dgrad phases, 128x64 tiles, tail slices
+    ((4, 16, 15, 15), (32, 16, 3, 3), (1, 1), (1, 1), (1, 1)),      # 225 positions per sample (odd)
+    ((6, 16, 20, 20), (10, 16, 3, 3), (1, 1), (1, 1), (1, 1)),      # F = 10: packed rows padded to 12
+    ((5, 48, 9, 33), (16, 48, 3, 5), (1, 2), (1, 0), (1, 2)),       # 16-row tiles, dilation, mixed strides
+    ((3, 32, 12, 12, 12), (32, 32, 3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),  # 3-D, 32-row tiles
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("case", range(len(KERNEL_VARIANT_CASES)))
+def test_conv_shapes_that_reach_every_kernel_variant(abi, dtype, case):
+    x_shape, w_shape, s, p, d = KERNEL_VARIANT_CASES[case]
+    rng = np.random.default_rng(700 + case)
+    tol = TOL[np.dtype(dtype)]
+    print("variant case", np.dtype(dtype).name, x_shape, w_shape, s, p, d, flush=True)
+    x = rng.standard_normal(x_shape).astype(dtype)
+    w = (rng.standard_normal(w_shape) * (2.0 / np.prod(w_shape[1:])) ** 0.5).astype(dtype)
+    want_out = direct.conv_forward(x, w, s, p, d)
+    g = rng.standard_normal(want_out.shape).astype(dtype)
+    assert rel_err(abi.conv_fwd(x, w, s, p, d), want_out) <= tol
+    assert rel_err(abi.conv_dgrad(g, x_shape, w, s, p, d), direct.conv_backward_x(g, x_shape, w, s, p, d)) <= tol
+    dw = abi.conv_wgrad(g, x, w_shape, s, p, d)
+    assert rel_err(dw, direct.conv_backward_w(g, x, w_shape, s, p, d)) <= tol
+    assert np.array_equal(bits(dw), bits(abi.conv_wgrad(g, x, w_shape, s, p, d)))  # fixed summation order
+
+
 def _check_conv_config(abi, seed, dtype, x_shape, w_shape, w_scale, s, p, d, np_oracle_batch):
     """Full-size check: against the definition-level C reference everywhere, and
     against the NumPy restatement of the reference on the leading batch items."""
