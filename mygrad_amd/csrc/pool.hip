@@ -413,6 +413,92 @@ __global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, con
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Windows that tile the input exactly (stride == pool extent, X == G * P on every axis):
+// every element belongs to exactly one window, so nothing is staged or accumulated.  A
+// thread takes one 16-byte piece of a row for each of the P0 x P1 rows of a window
+// slab -- 16 / (P2 * sizeof(T)) whole windows -- straight from global memory, reduces
+// them in registers and stores 16-byte pieces of dx (or its share of out).  Consecutive
+// lanes take consecutive pieces: every access of a wave is one contiguous run.
+// ------------------------------------------------------------------------------------------
+struct PoolExactParams {
+  int X1, X2;            // extents of the two inner pooled axes
+  int G0, G1;            // windows along the two outer pooled axes
+  int pieces;            // 16-byte pieces per row of x
+  long long xvol, gvol;  // elements of x / windows per leading index
+  long long total;       // work items: lead * G0 * G1 * pieces
+  FastDivP by_pieces, by_g1, by_g0;
+};
+
+template <typename T, typename TD, int P0, int P1, int P2, bool BWD>
+__global__ void __launch_bounds__(256) maxpool_exact_kernel(PoolExactParams p, const T *__restrict__ x,
+                                                            const T *__restrict__ grad, void *__restrict__ result) {
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int WPT = VEC / P2;  // windows per thread
+  static_assert(VEC % P2 == 0 && WPT >= 1, "a 16-byte piece holds whole windows");
+  typedef T Vec __attribute__((ext_vector_type(VEC)));
+  typedef T WVec __attribute__((ext_vector_type(WPT)));
+  const long long item = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (item >= p.total) return;
+  // item -> (leading index, g0, g1, piece); total < 2^32 is checked by the host
+  const unsigned u = (unsigned)item;
+  const unsigned q1 = p.by_pieces.div(u), piece = u - q1 * (unsigned)p.pieces;
+  const unsigned q2 = p.by_g1.div(q1), g1 = q1 - q2 * (unsigned)p.G1;
+  const unsigned lead = p.by_g0.div(q2), g0 = q2 - lead * (unsigned)p.G0;
+  const long long xrow0 = (long long)lead * p.xvol + ((long long)(g0 * P0) * p.X1 + g1 * P1) * p.X2 + piece * VEC;
+  Vec v[P0][P1];
+#pragma unroll
+  for (int a0 = 0; a0 < P0; ++a0)
+#pragma unroll
+    for (int a1 = 0; a1 < P1; ++a1) v[a0][a1] = *reinterpret_cast<const Vec *>(x + xrow0 + ((long long)a0 * p.X1 + a1) * p.X2);
+  const long long w0 = (long long)lead * p.gvol + ((long long)g0 * p.G1 + g1) * (p.pieces * WPT) + piece * WPT;
+  // first-occurrence maximum (the first NaN if any) of each window, row-major inside it
+  T best[WPT];
+  int where[WPT];
+#pragma unroll
+  for (int j = 0; j < WPT; ++j) {
+    best[j] = v[0][0][j * P2];
+    where[j] = 0;
+#pragma unroll
+    for (int a0 = 0; a0 < P0; ++a0)
+#pragma unroll
+      for (int a1 = 0; a1 < P1; ++a1)
+#pragma unroll
+        for (int a2 = 0; a2 < P2; ++a2) {
+          const T c = v[a0][a1][j * P2 + a2];
+          if (takes_over(c, best[j])) {
+            best[j] = c;
+            where[j] = (a0 * P1 + a1) * P2 + a2;
+          }
+        }
+  }
+  if constexpr (!BWD) {
+    WVec o;
+#pragma unroll
+    for (int j = 0; j < WPT; ++j) o[j] = best[j];
+    *reinterpret_cast<WVec *>(static_cast<T *>(result) + w0) = o;
+  } else {
+    const WVec g = *reinterpret_cast<const WVec *>(grad + w0);
+    typedef TD DVec __attribute__((ext_vector_type(VEC)));
+    TD *dx = static_cast<TD *>(result);
+#pragma unroll
+    for (int a0 = 0; a0 < P0; ++a0)
+#pragma unroll
+      for (int a1 = 0; a1 < P1; ++a1) {
+        DVec d;
+#pragma unroll
+        for (int j = 0; j < WPT; ++j)
+#pragma unroll
+          for (int a2 = 0; a2 < P2; ++a2) {
+            // the one window's gradient added to +0.0 (so -0.0 becomes +0.0), or +0.0
+            const TD term = (TD)(T(0) + g[j]);
+            d[j * P2 + a2] = where[j] == (a0 * P1 + a1) * P2 + a2 ? term : TD(0);
+          }
+        *reinterpret_cast<DVec *>(dx + xrow0 + ((long long)a0 * p.X1 + a1) * p.X2) = d;
+      }
+  }
+}
+
 static int check_pool_desc(const mg_pool_desc *d, PoolParams *p) {
   if (!d) return fail(MG_ERR_BAD_ARG, "pool descriptor is null");
   if (d->dtype != MG_F32 && d->dtype != MG_F64)
@@ -595,6 +681,35 @@ static unsigned grid_for(long long total) {
   return (unsigned)(blocks < cap ? blocks : cap);
 }
 
+// The exact-tiling kernels apply when stride == pool extent and X == G * P on every axis,
+// the pool extent is one of the instantiated ones, rows are whole 16-byte pieces and the
+// tensors are 16-byte aligned.  Returns 0 if not applicable, else P0*100 + P1*10 + P2.
+static int exact_signature(const PoolParams &p, size_t elem, const void *a, const void *b, const void *c, size_t c_elem,
+                           PoolExactParams *e) {
+  for (int k = 0; k < 3; ++k)
+    if (p.S[k] != p.P[k] || p.X[k] != p.G[k] * p.P[k]) return 0;
+  const int sig = p.P[0] * 100 + p.P[1] * 10 + p.P[2];
+  if (sig != 122 && sig != 222) return 0;
+  const int vec = (int)(16 / elem);
+  if (p.X[2] % vec != 0) return 0;
+  const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c);
+  if (bits % 16 != 0) return 0;
+  (void)c_elem;
+  e->X1 = p.X[1];
+  e->X2 = p.X[2];
+  e->G0 = p.G[0];
+  e->G1 = p.G[1];
+  e->pieces = p.X[2] / vec;
+  e->xvol = p.xvol;
+  e->gvol = p.gvol;
+  e->total = p.lead * p.G[0] * p.G[1] * e->pieces;
+  if (e->total >= (1ll << 32)) return 0;
+  e->by_pieces = make_fastdiv_p((unsigned)e->pieces);
+  e->by_g1 = make_fastdiv_p((unsigned)p.G[1]);
+  e->by_g0 = make_fastdiv_p((unsigned)p.G[0]);
+  return sig;
+}
+
 }  // namespace mg
 
 using namespace mg;
@@ -609,6 +724,21 @@ int mg_maxpool_fwd(const mg_pool_desc *desc, const void *x, void *out) {
   if (!x || !out) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_maxpool_fwd");
   hipStream_t s = runtime().stream;
   ScopedTiming timed(TAG_POOL_FWD);
+  PoolExactParams ep;
+  if (const int sig = exact_signature(p, desc->dtype == MG_F32 ? 4 : 8, x, out, out, 0, &ep)) {
+    const dim3 grid((unsigned)ceil_div(ep.total, 256)), block(256);
+#define MG_POOL_EXACT_FWD(T)                                                                                             \
+  do {                                                                                                                   \
+    if (sig == 122)                                                                                                      \
+      hipLaunchKernelGGL((maxpool_exact_kernel<T, T, 1, 2, 2, false>), grid, block, 0, s, ep, (const T *)x, (const T *)nullptr, out); \
+    else                                                                                                                 \
+      hipLaunchKernelGGL((maxpool_exact_kernel<T, T, 2, 2, 2, false>), grid, block, 0, s, ep, (const T *)x, (const T *)nullptr, out); \
+  } while (0)
+    if (desc->dtype == MG_F32) MG_POOL_EXACT_FWD(float); else MG_POOL_EXACT_FWD(double);
+#undef MG_POOL_EXACT_FWD
+    MG_HIP(hipGetLastError());
+    return MG_OK;
+  }
   PoolTileParams tp;
   int tile_elems = 0, win_slots = 0, acc_offset = 0;
   size_t lds = 0;
@@ -659,6 +789,26 @@ int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, vo
   if (!x || !grad || !dx) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_maxpool_bwd");
   hipStream_t s = runtime().stream;
   ScopedTiming timed(TAG_POOL_BWD);
+  PoolExactParams ep;
+  if (const int sig = exact_signature(p, desc->dtype == MG_F32 ? 4 : 8, x, grad, dx, 0, &ep)) {
+    const dim3 grid((unsigned)ceil_div(ep.total, 256)), block(256);
+#define MG_POOL_EXACT_BWD(T, TD)                                                                                        \
+  do {                                                                                                                  \
+    if (sig == 122)                                                                                                     \
+      hipLaunchKernelGGL((maxpool_exact_kernel<T, TD, 1, 2, 2, true>), grid, block, 0, s, ep, (const T *)x, (const T *)grad, dx); \
+    else                                                                                                                \
+      hipLaunchKernelGGL((maxpool_exact_kernel<T, TD, 2, 2, 2, true>), grid, block, 0, s, ep, (const T *)x, (const T *)grad, dx); \
+  } while (0)
+    if (desc->dtype == MG_F64)
+      MG_POOL_EXACT_BWD(double, double);
+    else if (desc->dx_dtype == MG_F64)
+      MG_POOL_EXACT_BWD(float, double);
+    else
+      MG_POOL_EXACT_BWD(float, float);
+#undef MG_POOL_EXACT_BWD
+    MG_HIP(hipGetLastError());
+    return MG_OK;
+  }
   PoolTileParams tp;
   int tile_elems = 0, win_slots = 0, acc_offset = 0;
   size_t lds = 0;

@@ -80,6 +80,34 @@ def test_pool_ties_and_overlap_bit_exact(abi, m, lead, dtype):
         assert np.array_equal(hits, ora.pool_backward(x, np.ones(out_shape), pool, stride))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("lead,X,pool", [
+    ((3, 5), (8, 12), (2, 2)),        # 2-D, rows of whole 16-byte pieces: the exact-tiling kernel
+    ((2,), (6, 4, 8), (2, 2, 2)),     # 3-D
+    ((7,), (2, 2, 4), (2, 2, 2)),     # a single window slab per volume
+    ((4,), (10, 6), (2, 2)),          # rows that are not whole 16-byte pieces in float32: the tiled kernel
+])
+def test_pool_windows_that_tile_the_input_exactly(abi, dtype, lead, X, pool):
+    """Stride == pool extent and X == G * P: the kernels that work straight from global
+    memory.  Ties, NaNs, -0.0 gradients and the float64 dx of a float32 input included."""
+    rng = np.random.default_rng(350 + len(X) + X[-1])
+    for trial in range(4):
+        if trial == 0:
+            x = rng.standard_normal((*lead, *X)).astype(dtype)
+        else:
+            x = rng.integers(0, 3, (*lead, *X)).astype(dtype)  # ties in almost every window
+        if trial == 2:
+            x[rng.random(x.shape) < 0.1] = np.nan
+        out_shape = (*lead, *(xk // pk for xk, pk in zip(X, pool)))
+        g = (rng.standard_normal(out_shape) * 10.0 ** rng.integers(-6, 6, out_shape)).astype(dtype)
+        g[rng.random(out_shape) < 0.2] = -0.0
+        want_out = ora.pool_forward(x, pool, pool, validate=False)
+        want_dx = ora.pool_backward(x, g, pool, pool)  # float64
+        assert np.array_equal(bits(abi.pool_fwd(x, pool, pool)), bits(want_out))
+        assert np.array_equal(bits(abi.pool_bwd(x, g, pool, pool, dx_dtype=np.float64)), bits(want_dx))
+        assert np.array_equal(bits(abi.pool_bwd(x, g, pool, pool)), bits(want_dx.astype(dtype)))
+
+
 def test_pool_order_of_summation_and_signed_zero(abi):
     x = np.array([[0.0, 0.0, 9.0, 0.0, 0.0]])
     for g in ([1e16, 1.0, -1e16], [1e16, -1e16, 1.0], [-0.0, -0.0, -0.0]):
