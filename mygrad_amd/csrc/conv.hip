@@ -417,19 +417,30 @@ __global__ void __launch_bounds__(256) wgrad_kernel(const WgradParams p) {
 }
 
 // ((p[0] + p[stride]) + p[2*stride]) + ... over `terms` terms: always this order, so
-// the result does not change from run to run; eight loads are in flight at a time.
+// the result does not change from run to run; sixteen loads are in flight at a time
+// (the partial sums were written by other XCDs a moment ago: every load is a trip
+// past this XCD's L2).
 template <typename T>
 __device__ __forceinline__ T sum_in_order(const T *__restrict__ p, long long stride, int terms) {
+  constexpr int BATCH = 16;
   T s = p[0];
   int k = 1;
-  for (; k + 8 <= terms; k += 8) {
-    T v[8];
+  for (; k + BATCH <= terms; k += BATCH) {
+    T v[BATCH];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) v[u] = p[(long long)(k + u) * stride];
+    for (int u = 0; u < BATCH; ++u) v[u] = p[(long long)(k + u) * stride];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) s += v[u];
+    for (int u = 0; u < BATCH; ++u) s += v[u];
   }
-  for (; k < terms; ++k) s += p[(long long)k * stride];
+  if (k < terms) {
+    // the rest in one more batch: loads past the end repeat the last term and are not added
+    T v[BATCH];
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u) v[u] = p[(long long)min(k + u, terms - 1) * stride];
+#pragma unroll
+    for (int u = 0; u < BATCH; ++u)
+      if (k + u < terms) s += v[u];
+  }
   return s;
 }
 

@@ -828,18 +828,21 @@ __global__ void __launch_bounds__(256) tap_reduce_kernel(const T *__restrict__ p
   __shared__ T runs[4][64];
   const int count = F * C * wvol;
   const int q = threadIdx.x / WIDTH, lane = threadIdx.x % WIDTH;
-  const int i = blockIdx.x * WIDTH + lane;  // index into dw
+  // Threads run through the partial sums' own layout, so a wave reads consecutive
+  // addresses of every split (the few stores to dw are the scattered side).
+  const int src = blockIdx.x * WIDTH + lane;  // index into one split: f * C*wvol + column
   const int per = (splits + RUNS - 1) / RUNS;
   const int first = min(q * per, splits), last = min(first + per, splits);
   T sum = T(0);
-  if (i < count && first < last) {
+  int i = count;  // index into dw
+  if (src < count) {
     const int ct = C * wvol;
-    const int f = i / ct;
-    const int r = i - f * ct;
-    const int c = r / wvol;
-    const int t = r - c * wvol;
-    const int src = f * ct + ((c / 16) * wvol + t) * 16 + c % 16;
-    sum = sum_in_order(part + (long long)first * count + src, count, last - first);
+    const int f = src / ct;
+    const int col = src - f * ct;
+    const int group = col / 16;  // (channel block, tap)
+    const int cb = group / wvol, t = group - cb * wvol;
+    i = f * ct + (cb * 16 + col % 16) * wvol + t;
+    if (first < last) sum = sum_in_order(part + (long long)first * count + src, count, last - first);
   }
   if constexpr (RUNS == 1) {
     if (i < count) dw[i] = sum;
