@@ -211,6 +211,7 @@ struct ChunkInFlight {
   static constexpr int VEC = 16 / sizeof(T);
   typedef T Vec __attribute__((ext_vector_type(VEC)));
   Vec held[DEPTH];
+  T edge;  // threads 0 .. VEC-2: one element of the unaligned head; the next VEC-1 threads: one of the tail
 
   __device__ __forceinline__ static int head_of(int len, int pad) { return min(len, (VEC - pad) % VEC); }
 
@@ -222,6 +223,11 @@ struct ChunkInFlight {
     const int last = max(body - 1, 0);
 #pragma unroll
     for (int u = 0; u < DEPTH; ++u) held[u] = vsrc[min(u * 256 + (int)threadIdx.x, last)];
+    // the elements before the first and after the last whole vector travel with them,
+    // one per thread, instead of being fetched when the chunk is parked
+    const int t = (int)threadIdx.x;
+    const int e = t < VEC - 1 ? t : head + body * VEC + (t - (VEC - 1));
+    edge = src[start + min(e, max(len - 1, 0))];
   }
 
   __device__ __forceinline__ void commit(T *tile, const T *__restrict__ src, long long start, int len, int pad) {
@@ -235,8 +241,13 @@ struct ChunkInFlight {
     }
     const Vec *vsrc = reinterpret_cast<const Vec *>(src + start + head);
     for (int v = DEPTH * 256 + (int)threadIdx.x; v < body; v += 256) vdst[v] = vsrc[v];
-    for (int e = threadIdx.x; e < head; e += 256) tile[pad + e] = src[start + e];
-    for (int e = head + body * VEC + (int)threadIdx.x; e < len; e += 256) tile[pad + e] = src[start + e];
+    const int t = (int)threadIdx.x;
+    if (t < VEC - 1) {
+      if (t < head) tile[pad + t] = edge;
+    } else if (t < 2 * (VEC - 1)) {
+      const int e = head + body * VEC + (t - (VEC - 1));
+      if (e < len) tile[pad + e] = edge;
+    }
   }
 };
 
