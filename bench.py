@@ -53,6 +53,8 @@ WORKLOADS = {
                   wscale=(2 / 432) ** 0.5, stride=(1, 1, 1), padding=(1, 1, 1), dilation=(1, 1, 1)),
     "pool2": dict(kind="pool", dtype="f64", seed=1002, x=(64, 64, 56, 56), pool=(3, 3), stride=(2, 2)),
     "pool5": dict(kind="pool", dtype="f32", seed=1006, x=(8, 32, 32, 64, 64), pool=(2, 2, 2), stride=(2, 2, 2)),
+    # relu, multiply and sum (forward and gradients) on a tensor of conv5's output size
+    "elem5": dict(kind="elem", dtype="f32", seed=1007, x=(8, 32, 32, 64, 64)),
 }
 NP_DTYPE = {"f32": np.float32, "f64": np.float64}
 
@@ -78,6 +80,8 @@ def pool_shapes(wl):
 
 def describe(name):
     wl = WORKLOADS[name]
+    if wl["kind"] == "elem":
+        return f"{name}: relu + multiply + sum {wl['dtype']} x{wl['x']} fwd+bwd (7 kernels, 16 |x| bytes)"
     if wl["kind"] == "conv":
         return (f"{name}: conv_nd {wl['dtype']} x{wl['x']} * w{wl['w']} stride{wl['stride']} pad{wl['padding']} "
                 f"dil{wl['dilation']} -> grid{conv_grid(wl)} fwd+dx+dw")
@@ -119,6 +123,18 @@ class Step:
             self.total_work = 3 * per_pass
             self.unit, self.bound, self.peak = "TFLOP/s", "mfma", PEAK_TFLOPS[wl["dtype"]]
             self.scale = 1e-12
+        elif wl["kind"] == "elem":
+            x = rng.standard_normal(wl["x"]).astype(dt)
+            g = rng.standard_normal(wl["x"]).astype(dt)
+            self.n, self.code = x.size, _hip.dtype_code(dt)
+            self.x, self.g = resident(x), resident(g)
+            self.out, self.dx = _device.DeviceBuffer(x.nbytes), _device.DeviceBuffer(x.nbytes)
+            self.scalar = _device.DeviceBuffer(16)
+            # relu fwd 2|x|, relu bwd 3|x|, multiply fwd and two gradients 3|x| each, fill |x|: 6 launches
+            self.work = {"elementwise": 15.0 * x.nbytes / 6, "sum_all": float(x.nbytes)}
+            self.total_work = 16.0 * x.nbytes
+            self.unit, self.bound, self.peak = "GB/s", "hbm", PEAK_HBM_GBS
+            self.scale = 1e-9
         else:
             lead, pooled, grid = pool_shapes(wl)
             out_shape = (*lead, *grid)
@@ -134,7 +150,18 @@ class Step:
             self.scale = 1e-9
 
     def __call__(self):
-        lib, d, check = self.lib, self.desc, self.check
+        lib, check = self.lib, self.check
+        if self.wl["kind"] == "elem":
+            c, n = self.code, self.n
+            check(lib.mg_relu_fwd(c, n, self.x.ptr, self.out.ptr))
+            check(lib.mg_multiply(c, n, self.out.ptr, self.g.ptr, self.dx.ptr))  # relu(x) * g
+            check(lib.mg_sum_all(c, n, self.dx.ptr, self.scalar.ptr))
+            check(lib.mg_fill_from(c, n, self.scalar.ptr, self.dx.ptr))  # d sum
+            check(lib.mg_multiply(c, n, self.dx.ptr, self.g.ptr, self.out.ptr))  # d (a*b) / d a
+            check(lib.mg_multiply(c, n, self.dx.ptr, self.x.ptr, self.out.ptr))  # d (a*b) / d b
+            check(lib.mg_relu_bwd(c, n, self.x.ptr, self.dx.ptr, self.out.ptr))
+            return
+        d = self.desc
         if self.wl["kind"] == "conv":
             check(lib.mg_conv_fwd(d, self.x.ptr, self.w.ptr, self.out.ptr))
             check(lib.mg_conv_dgrad(d, self.g.ptr, self.w.ptr, self.dx.ptr))
@@ -234,6 +261,21 @@ def run_cpu_baseline(name, min_seconds=10.0, max_reps=200):
 
         work, scale, unit = 3 * conv_flops_per_pass(wl), 1e-12, "TFLOP/s"
         what = "fwd+dx+dw"
+    elif wl["kind"] == "elem":
+        x = rng.standard_normal(wl["x"]).astype(dt)
+        g = rng.standard_normal(wl["x"]).astype(dt)
+
+        def once():
+            r = ora.relu_forward(x)
+            p = ora.multiply(r, g)
+            total = ora.sum_all(p)
+            dp = ora.sum_all_backward(p, total)
+            ora.multiply_backward(dp, r, g, 0)
+            dr = ora.multiply_backward(dp, r, g, 1)
+            ora.relu_backward(x, dr)
+
+        work, scale, unit = 16 * x.nbytes, 1e-9, "GB/s"
+        what = "relu, multiply, sum and their gradients"
     else:
         x = rng.standard_normal(wl["x"]).astype(dt)
         lead, pooled, grid = pool_shapes(wl)
@@ -285,6 +327,16 @@ def run_dropin(name, steps=5):
             out.backward(g)
 
         work, scale, unit = 3 * conv_flops_per_pass(wl), 1e-12, "TFLOP/s"
+    elif wl["kind"] == "elem":
+        from mygrad_amd.nnet import relu
+
+        g = rng.standard_normal(wl["x"]).astype(dt)
+
+        def once():
+            xt, gt = mg.Tensor(x, copy=False), mg.Tensor(g, copy=False)
+            mg.sum(relu(xt) * gt).backward()
+
+        work, scale, unit = 16 * x.nbytes, 1e-9, "GB/s"
     else:
         lead, pooled, grid = pool_shapes(wl)
         g = rng.standard_normal((*lead, *grid)).astype(dt)
@@ -374,7 +426,8 @@ def main():
     wl = WORKLOADS[args.workload]
     res = run_gpu(args.workload, args.steps, args.warmup)
     line = {
-        "metric": ("conv_nd fwd+bwd TFLOP/s" if wl["kind"] == "conv" else "max_pool fwd+bwd GB/s"),
+        "metric": {"conv": "conv_nd fwd+bwd TFLOP/s", "pool": "max_pool fwd+bwd GB/s",
+                   "elem": "relu+multiply+sum fwd+bwd GB/s"}[wl["kind"]],
         "value": res["value"],
         "unit": res["unit"],
         "n_gpus": 1,

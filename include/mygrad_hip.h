@@ -103,7 +103,8 @@ int mg_event_destroy(void *event);
  * mg_timing_read() waits for the stream, returns up to `capacity` (tag, ms)
  * records in launch order, sets *count to the number recorded and starts over.
  * Tags: 1 conv forward, 2 conv dgrad, 3 conv wgrad, 4 wgrad split-K reduction,
- * 5 filter packing, 6 max-pool forward, 7 max-pool backward, 8 device copy. */
+ * 5 filter packing, 6 max-pool forward, 7 max-pool backward, 8 device copy,
+ * 9 element-wise kernel, 10 whole-array sum. */
 int mg_timing_enable(int on);
 int mg_timing_read(int32_t *tags, float *ms, int capacity, int *count);
 
@@ -146,6 +147,32 @@ int mg_maxpool_fwd(const mg_pool_desc *desc, const void *x, void *out);
  * Replaces MaxPoolND.backward_var, src/mygrad/nnet/layers/pooling.py:100-149
  * (argmax :111, np.add.at :147-148). */
 int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, void *dx);
+
+/* ---- element-wise and whole-array kernels either side of conv / pool ----
+ * dtype: 0 float32, 1 float64; n elements, C-contiguous, same shape; device pointers,
+ * 16-byte aligned (what mg_malloc returns). */
+
+/* out[i] = a[i] * b[i].  Replaces the body of Multiply.__call__ (np.multiply on
+ * same-shape operands, src/mygrad/math/arithmetic/ops.py:45-46) and both branches of
+ * Multiply.backward_var (grad * other, ops.py:48-53). */
+int mg_multiply(int dtype, int64_t n, const void *a, const void *b, void *out);
+
+/* out[i] = x[i] * (x[i] > 0) as one IEEE multiply by 1 or 0: negative x gives -0.0, NaN
+ * stays NaN.  Replaces ReLu.__call__, src/mygrad/nnet/activations/relu.py:11-14. */
+int mg_relu_fwd(int dtype, int64_t n, const void *x, void *out);
+
+/* dx[i] = grad[i] * (x[i] > 0).  Replaces ReLu.backward_var, relu.py:16-17 (the mask the
+ * reference stores in self.back is recomputed from x). */
+int mg_relu_bwd(int dtype, int64_t n, const void *x, const void *grad, void *dx);
+
+/* *out (one element on the device) = sum of x, added in a fixed tree and carried in double,
+ * rounded once.  Replaces Sum.__call__ with axis=None (np.sum,
+ * src/mygrad/math/sequential/ops.py:120-121; src/mygrad/operation_base.py Sequential). */
+int mg_sum_all(int dtype, int64_t n, const void *x, void *out);
+
+/* out[i] = *value (one element on the device).  Replaces Sum.backward_var with axis=None
+ * (np.full(a.shape, grad), sequential/ops.py:123-126). */
+int mg_fill_from(int dtype, int64_t n, const void *value, void *out);
 
 #ifdef __cplusplus
 }

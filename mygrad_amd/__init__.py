@@ -4,6 +4,7 @@
     >>> from mygrad_amd.nnet import conv_nd, max_pool
     >>> out = max_pool(conv_nd(x, w, stride=1, padding=1), (2, 2), 2)
     >>> out.backward(g)        # x.grad, w.grad computed by the HIP kernels
+    >>> loss = mg.sum(mg.nnet.relu(out) * g)   # relu, multiply and sum run on the device too
 
 The arithmetic runs in ``libmygrad_hip.so`` (hand-written gfx950 kernels, called
 through ctypes).  There is no CPU fallback: without the library or without a
@@ -17,6 +18,7 @@ from .errors import InvalidBackprop, InvalidGradient, SkipGradient
 from .nnet.layers.utils import sliding_window_view
 from .operation_base import Operation
 from .tensor_base import Tensor, asarray, tensor
+from .math import multiply, sum  # noqa: A004  (after tensor_base: the ops import Tensor)
 
 execute_op = Tensor._op
 
@@ -30,6 +32,8 @@ __all__ = [
     "mem_guard_off",
     "mem_guard_on",
     "sliding_window_view",
+    "multiply",
+    "sum",
     "nnet",
     "InvalidBackprop",
     "InvalidGradient",

@@ -116,6 +116,11 @@ _SIGNATURES = {
     "mg_conv_wgrad": [ctypes.POINTER(ConvDesc), _vp, _vp, _vp],
     "mg_maxpool_fwd": [ctypes.POINTER(PoolDesc), _vp, _vp],
     "mg_maxpool_bwd": [ctypes.POINTER(PoolDesc), _vp, _vp, _vp],
+    "mg_multiply": [ctypes.c_int, ctypes.c_int64, _vp, _vp, _vp],
+    "mg_relu_fwd": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
+    "mg_relu_bwd": [ctypes.c_int, ctypes.c_int64, _vp, _vp, _vp],
+    "mg_sum_all": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
+    "mg_fill_from": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES) + ("mg_last_error",)
 
@@ -210,6 +215,8 @@ KERNEL_TAGS = {
     6: "maxpool_fwd",
     7: "maxpool_bwd",
     8: "copy",
+    9: "elementwise",
+    10: "sum_all",
 }
 
 

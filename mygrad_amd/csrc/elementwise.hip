@@ -1,0 +1,252 @@
+// Element-wise and whole-array kernels either side of conv_nd / max_pool in a chain
+// such as conv -> relu -> pool -> (. * g) -> sum: bandwidth-bound, 16 bytes per lane.
+//
+//   multiply   out[i] = a[i] * b[i]            (one IEEE multiply: bit-exact with NumPy)
+//   relu       out[i] = x[i] * (x[i] > 0)      (so negative inputs give -0.0, NaN stays NaN)
+//   relu bwd   dx[i]  = grad[i] * (x[i] > 0)
+//   sum        *out   = sum_i x[i]             (fixed summation tree, carried in double)
+//   fill       out[i] = *value
+#include "internal.h"
+
+#include <algorithm>
+
+namespace mg {
+
+namespace {
+
+template <typename T>
+struct Vec16 {
+  static constexpr int N = 16 / sizeof(T);
+  typedef T type __attribute__((ext_vector_type(N)));
+};
+
+enum ElementwiseOp { EW_MUL = 0, EW_RELU = 1, EW_RELU_BWD = 2 };
+
+template <typename T, int OP>
+__device__ __forceinline__ T apply(T a, T b) {
+  if constexpr (OP == EW_MUL) return a * b;
+  if constexpr (OP == EW_RELU) return a * (a > T(0) ? T(1) : T(0));
+  return b * (a > T(0) ? T(1) : T(0));  // a = x, b = grad
+}
+
+// out = op(a, b) over n elements; `a`, `b` and `out` are 16-byte aligned (device
+// allocations are), the last n % VEC elements are handled one by one.
+template <typename T, int OP>
+__global__ void __launch_bounds__(256) elementwise_kernel(const T *__restrict__ a, const T *__restrict__ b,
+                                                          T *__restrict__ out, long long n) {
+  typedef typename Vec16<T>::type V;
+  constexpr int VEC = Vec16<T>::N;
+  const long long nvec = n / VEC;
+  const long long stride = (long long)gridDim.x * 256;
+  const V *va = reinterpret_cast<const V *>(a);
+  const V *vb = reinterpret_cast<const V *>(b);
+  V *vo = reinterpret_cast<V *>(out);
+  long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  for (; i < nvec; i += stride) {
+    const V x = va[i];
+    V y = x;
+    if constexpr (OP != EW_RELU) y = vb[i];
+    V r;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) r[k] = apply<T, OP>(x[k], y[k]);
+    vo[i] = r;
+  }
+  if (blockIdx.x == 0) {
+    const long long i = nvec * VEC + threadIdx.x;
+    if (i < n) out[i] = apply<T, OP>(a[i], OP != EW_RELU ? b[i] : a[i]);
+  }
+}
+
+// Block b adds the elements of chunk b: thread t takes the 16-byte pieces t, t + 256,
+// ... of the chunk in that order (in double), then the 256 thread sums are added in a
+// fixed binary tree.  The chunking depends only on n, so the result repeats exactly.
+template <typename T>
+__global__ void __launch_bounds__(256) sum_chunks_kernel(const T *__restrict__ x, long long n, long long chunk,
+                                                         double *__restrict__ partial) {
+  typedef typename Vec16<T>::type V;
+  constexpr int VEC = Vec16<T>::N;
+  __shared__ double tree[256];
+  const long long begin = (long long)blockIdx.x * chunk;  // chunk is a multiple of VEC
+  const long long end = min(begin + chunk, n);
+  const long long nvec = (end - begin) / VEC;
+  const V *vx = reinterpret_cast<const V *>(x + begin);
+  // four running sums per thread (pieces t, t + 256, t + 512, t + 768 of each round of
+  // 1024), added as (s0 + s1) + (s2 + s3): four loads in flight, still one fixed order
+  double s4[4] = {0.0, 0.0, 0.0, 0.0};
+  long long i = threadIdx.x;
+  for (; i + 768 < nvec; i += 1024) {
+    V v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = vx[i + u * 256];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) s4[u] += (double)v[u][k];
+  }
+  for (int u = 0; i < nvec; i += 256, ++u) {
+    const V v = vx[i];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) s4[u] += (double)v[k];
+  }
+  double s = (s4[0] + s4[1]) + (s4[2] + s4[3]);
+  {
+    const long long i = begin + nvec * VEC + threadIdx.x;  // the array's last n % VEC elements
+    if (i < end) s += (double)x[i];
+  }
+  tree[threadIdx.x] = s;
+  __syncthreads();
+  for (int half = 128; half > 0; half >>= 1) {
+    if ((int)threadIdx.x < half) tree[threadIdx.x] += tree[threadIdx.x + half];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) partial[blockIdx.x] = tree[0];
+}
+
+// One block adds the chunk sums (thread t takes t, t + 256, ... in order, then the same
+// tree) and rounds once to T.
+template <typename T>
+__global__ void __launch_bounds__(256) sum_final_kernel(const double *__restrict__ partial, int count, T *__restrict__ out) {
+  __shared__ double tree[256];
+  double s = 0.0;
+  for (int i = threadIdx.x; i < count; i += 256) s += partial[i];
+  tree[threadIdx.x] = s;
+  __syncthreads();
+  for (int half = 128; half > 0; half >>= 1) {
+    if ((int)threadIdx.x < half) tree[threadIdx.x] += tree[threadIdx.x + half];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) *out = (T)tree[0];
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) fill_from_kernel(const T *__restrict__ value, T *__restrict__ out, long long n) {
+  typedef typename Vec16<T>::type V;
+  constexpr int VEC = Vec16<T>::N;
+  const T v = *value;
+  V vv;
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) vv[k] = v;
+  const long long nvec = n / VEC;
+  V *vo = reinterpret_cast<V *>(out);
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (long long)gridDim.x * 256) vo[i] = vv;
+  if (blockIdx.x == 0) {
+    const long long i = nvec * VEC + threadIdx.x;
+    if (i < n) out[i] = v;
+  }
+}
+
+unsigned streaming_grid(long long n, size_t elem) {
+  const long long pieces = std::max<long long>(1, n / (long long)(16 / elem));
+  const long long cap = (long long)runtime().props.multiProcessorCount * 16;  // 16 blocks of 256 threads per unit
+  return (unsigned)std::min<long long>(ceil_div(pieces, 256), cap);
+}
+
+int check_elementwise(int dtype, int64_t n, const char *who) {
+  if (dtype != MG_F32 && dtype != MG_F64) return fail(MG_ERR_UNSUPPORTED, "%s: dtype %d (only float32=0 / float64=1)", who, dtype);
+  if (n < 0) return fail(MG_ERR_BAD_ARG, "%s: n = %lld", who, (long long)n);
+  return MG_OK;
+}
+
+template <int OP>
+int launch_elementwise(int dtype, int64_t n, const void *a, const void *b, void *out, int tag) {
+  if (n == 0) return MG_OK;
+  hipStream_t s = runtime().stream;
+  ScopedTiming timed(tag);
+  if (dtype == MG_F32)
+    hipLaunchKernelGGL((elementwise_kernel<float, OP>), dim3(streaming_grid(n, 4)), dim3(256), 0, s, (const float *)a,
+                       (const float *)b, (float *)out, (long long)n);
+  else
+    hipLaunchKernelGGL((elementwise_kernel<double, OP>), dim3(streaming_grid(n, 8)), dim3(256), 0, s, (const double *)a,
+                       (const double *)b, (double *)out, (long long)n);
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
+bool misaligned(const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 != 0; }
+
+}  // namespace
+}  // namespace mg
+
+using namespace mg;
+
+extern "C" {
+
+int mg_multiply(int dtype, int64_t n, const void *a, const void *b, void *out) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (int rc = check_elementwise(dtype, n, "mg_multiply")) return rc;
+  if (n > 0 && (!a || !b || !out)) return fail(MG_ERR_BAD_ARG, "null pointer in mg_multiply");
+  if (misaligned(a) || misaligned(b) || misaligned(out)) return fail(MG_ERR_BAD_ARG, "mg_multiply: pointers must be 16-byte aligned");
+  return launch_elementwise<EW_MUL>(dtype, n, a, b, out, TAG_ELEMENTWISE);
+}
+
+int mg_relu_fwd(int dtype, int64_t n, const void *x, void *out) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (int rc = check_elementwise(dtype, n, "mg_relu_fwd")) return rc;
+  if (n > 0 && (!x || !out)) return fail(MG_ERR_BAD_ARG, "null pointer in mg_relu_fwd");
+  if (misaligned(x) || misaligned(out)) return fail(MG_ERR_BAD_ARG, "mg_relu_fwd: pointers must be 16-byte aligned");
+  return launch_elementwise<EW_RELU>(dtype, n, x, x, out, TAG_ELEMENTWISE);
+}
+
+int mg_relu_bwd(int dtype, int64_t n, const void *x, const void *grad, void *dx) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (int rc = check_elementwise(dtype, n, "mg_relu_bwd")) return rc;
+  if (n > 0 && (!x || !grad || !dx)) return fail(MG_ERR_BAD_ARG, "null pointer in mg_relu_bwd");
+  if (misaligned(x) || misaligned(grad) || misaligned(dx)) return fail(MG_ERR_BAD_ARG, "mg_relu_bwd: pointers must be 16-byte aligned");
+  return launch_elementwise<EW_RELU_BWD>(dtype, n, x, grad, dx, TAG_ELEMENTWISE);
+}
+
+int mg_sum_all(int dtype, int64_t n, const void *x, void *out) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (int rc = check_elementwise(dtype, n, "mg_sum_all")) return rc;
+  if (!out || (n > 0 && !x)) return fail(MG_ERR_BAD_ARG, "null pointer in mg_sum_all");
+  if (misaligned(x)) return fail(MG_ERR_BAD_ARG, "mg_sum_all: x must be 16-byte aligned");
+  hipStream_t s = runtime().stream;
+  const size_t elem = dtype == MG_F32 ? 4 : 8;
+  // chunks of 128 KiB, at most 4096 of them (then the chunks grow): a function of n only
+  const long long vec = (long long)(16 / elem);
+  long long chunk = (128 * 1024) / (long long)elem;
+  long long chunks = std::max<long long>(1, ceil_div(n, chunk));
+  if (chunks > 4096) {
+    chunk = ceil_div(ceil_div(n, 4096), vec) * vec;
+    chunks = ceil_div(n, chunk);
+  }
+  void *partial = nullptr;
+  if (int rc = workspace((size_t)chunks * sizeof(double), &partial)) return rc;
+  ScopedTiming timed(TAG_REDUCE_ALL);
+  if (dtype == MG_F32) {
+    hipLaunchKernelGGL(sum_chunks_kernel<float>, dim3((unsigned)chunks), dim3(256), 0, s, (const float *)x, (long long)n, chunk,
+                       (double *)partial);
+    hipLaunchKernelGGL(sum_final_kernel<float>, dim3(1), dim3(256), 0, s, (const double *)partial, (int)chunks, (float *)out);
+  } else {
+    hipLaunchKernelGGL(sum_chunks_kernel<double>, dim3((unsigned)chunks), dim3(256), 0, s, (const double *)x, (long long)n, chunk,
+                       (double *)partial);
+    hipLaunchKernelGGL(sum_final_kernel<double>, dim3(1), dim3(256), 0, s, (const double *)partial, (int)chunks, (double *)out);
+  }
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
+int mg_fill_from(int dtype, int64_t n, const void *value, void *out) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (int rc = check_elementwise(dtype, n, "mg_fill_from")) return rc;
+  if (!value || (n > 0 && !out)) return fail(MG_ERR_BAD_ARG, "null pointer in mg_fill_from");
+  if (misaligned(out)) return fail(MG_ERR_BAD_ARG, "mg_fill_from: out must be 16-byte aligned");
+  if (n == 0) return MG_OK;
+  hipStream_t s = runtime().stream;
+  ScopedTiming timed(TAG_ELEMENTWISE);
+  if (dtype == MG_F32)
+    hipLaunchKernelGGL(fill_from_kernel<float>, dim3(streaming_grid(n, 4)), dim3(256), 0, s, (const float *)value, (float *)out,
+                       (long long)n);
+  else
+    hipLaunchKernelGGL(fill_from_kernel<double>, dim3(streaming_grid(n, 8)), dim3(256), 0, s, (const double *)value, (double *)out,
+                       (long long)n);
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
+}  // extern "C"

@@ -50,6 +50,8 @@ enum KernelTag {
   TAG_POOL_FWD = 6,
   TAG_POOL_BWD = 7,
   TAG_COPY = 8,
+  TAG_ELEMENTWISE = 9,
+  TAG_REDUCE_ALL = 10,
 };
 void timing_begin(int tag);
 void timing_end();

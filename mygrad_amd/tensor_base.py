@@ -121,6 +121,24 @@ class Tensor:
         self._grad = None
         return self
 
+    # ------------------------------------------------------------------ operators
+    # (reference: tensor_base.py:2007-2015, :2378-2384; only what the convolution /
+    # pooling chains use, on the device)
+    def __mul__(self, other):
+        from .math.arithmetic.ops import Multiply
+
+        return self._op(Multiply, self, other)
+
+    def __rmul__(self, other):
+        from .math.arithmetic.ops import Multiply
+
+        return self._op(Multiply, other, self)
+
+    def sum(self, axis=None, keepdims=False, *, constant=None):
+        from .math.sequential.ops import Sum
+
+        return self._op(Sum, self, op_args=(axis, keepdims), constant=constant)
+
     # ------------------------------------------------------------------ graph construction
     @classmethod
     def _op(cls, Op, *input_vars, op_args=None, op_kwargs=None, constant=None):

@@ -24,6 +24,12 @@ Pinning (what holds each function to the reference without importing it):
                    central differences
   pool_forward     three reference known-answer cases + the docstring case
   pool_backward    with a tie, brute-force loops on tie-heavy integer inputs
+  relu_forward     the reference's docstring vectors (``-0.0`` for negative inputs,
+  relu_backward    gradient ``[0, 0, 0, 1, 1]``); one IEEE multiply per element
+  multiply, multiply_backward, sum_all, sum_all_backward
+                   single calls of the NumPy routine the reference calls
+                   (``np.multiply``, ``np.sum``, ``np.full``); ``sum_all`` is
+                   additionally held to ``math.fsum`` and closed forms in the tests
 """
 
 from numbers import Integral
@@ -38,6 +44,12 @@ __all__ = [
     "conv_forward",
     "conv_backward_x",
     "conv_backward_w",
+    "multiply",
+    "multiply_backward",
+    "relu_forward",
+    "relu_backward",
+    "sum_all",
+    "sum_all_backward",
     "pool_out_shape",
     "pool_forward",
     "pool_backward",
@@ -303,3 +315,39 @@ def pool_backward(x, grad, pool, stride):
     dx = np.zeros((*lead_shape, int(np.prod(pooled_shape))))
     np.add.at(dx, tuple(where), grad.reshape(flat_shape))
     return dx.reshape(x.shape)
+
+
+# ------------------------------------------------------------------ element-wise / sum
+def multiply(a, b):
+    """``Multiply.__call__``: ``np.multiply(a, b)`` (mygrad/math/arithmetic/ops.py:45-46)."""
+    return np.multiply(a, b)
+
+
+def multiply_backward(grad, a, b, index):
+    """``Multiply.backward_var``: ``grad * b`` for the first operand, ``grad * a`` for the
+    second (mygrad/math/arithmetic/ops.py:48-53)."""
+    return grad * b if index == 0 else grad * a
+
+
+def relu_forward(x):
+    """``ReLu.__call__``: ``x * asarray(x > 0, dtype=x.dtype)``
+    (mygrad/nnet/activations/relu.py:11-14)."""
+    return x * np.asarray(x > 0, dtype=x.dtype)
+
+
+def relu_backward(x, grad):
+    """``ReLu.backward_var``: ``grad * back`` with ``back`` the forward pass's 0/1 mask
+    (mygrad/nnet/activations/relu.py:16-17)."""
+    return grad * np.asarray(x > 0, dtype=x.dtype)
+
+
+def sum_all(x):
+    """``Sum.__call__`` with ``axis=None``: ``np.sum(x)``
+    (mygrad/math/sequential/ops.py:120-121)."""
+    return np.sum(x)
+
+
+def sum_all_backward(x, grad):
+    """``Sum.backward_var`` with ``axis=None``: ``np.full(a.shape, grad, dtype=a.dtype)``
+    (mygrad/math/sequential/ops.py:123-126)."""
+    return np.full(x.shape, grad, dtype=x.dtype)

@@ -90,3 +90,40 @@ def pool_bwd(x, grad, pool, stride, dx_dtype=None):
     db = _device.DeviceBuffer(x.size * dx_dtype.itemsize)
     _hip.check(_hip.lib().mg_maxpool_bwd(desc, xb.ptr, gb.ptr, db.ptr))
     return _down(db, x.shape, dx_dtype)
+
+
+# ----------------------------------------------------------------- element-wise / sum
+def multiply(a, b):
+    ab, bb = _up(a), _up(b)
+    ob = _device.DeviceBuffer(max(a.nbytes, 16))
+    _hip.check(_hip.lib().mg_multiply(_hip.dtype_code(a.dtype), a.size, ab.ptr, bb.ptr, ob.ptr))
+    return _down(ob, a.shape, a.dtype)
+
+
+def relu_fwd(x):
+    xb = _up(x)
+    ob = _device.DeviceBuffer(max(x.nbytes, 16))
+    _hip.check(_hip.lib().mg_relu_fwd(_hip.dtype_code(x.dtype), x.size, xb.ptr, ob.ptr))
+    return _down(ob, x.shape, x.dtype)
+
+
+def relu_bwd(x, grad):
+    xb, gb = _up(x), _up(grad)
+    ob = _device.DeviceBuffer(max(x.nbytes, 16))
+    _hip.check(_hip.lib().mg_relu_bwd(_hip.dtype_code(x.dtype), x.size, xb.ptr, gb.ptr, ob.ptr))
+    return _down(ob, x.shape, x.dtype)
+
+
+def sum_all(x):
+    xb = _up(x)
+    ob = _device.DeviceBuffer(16)
+    _hip.check(_hip.lib().mg_sum_all(_hip.dtype_code(x.dtype), x.size, xb.ptr, ob.ptr))
+    return _down(ob, (), x.dtype)
+
+
+def fill_from(value, shape, dtype):
+    vb = _up(np.asarray(value, dtype=dtype).reshape(1))
+    n = int(np.prod(shape))
+    ob = _device.DeviceBuffer(max(n * np.dtype(dtype).itemsize, 16))
+    _hip.check(_hip.lib().mg_fill_from(_hip.dtype_code(dtype), n, vb.ptr, ob.ptr))
+    return _down(ob, shape, dtype)

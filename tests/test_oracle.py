@@ -296,3 +296,38 @@ def test_pool_error_contract():
         ora.pool_forward(x, (2,) * 2, [1, 2, 3])
     with pytest.raises(ValueError):
         ora.pool_forward(x, (1,) * 3, (3,) * 3)
+
+
+# ----------------------------------------------------------------- element-wise / sum
+def test_relu_reference_docstring_vectors(kats):
+    for case in kats["relu"]:
+        for dtype in (np.float32, np.float64):
+            x = np.array(case["x"], dtype=dtype)
+            out = ora.relu_forward(x)
+            assert np.array_equal(out, np.array(case["out"], dtype=dtype)), case["source"]
+            assert np.array_equal(np.signbit(out), np.array(case["out_signbit"])), "negative inputs give -0.0"
+            assert np.array_equal(ora.relu_backward(x, np.ones_like(x)), np.array(case["dx_of_ones"], dtype=dtype))
+
+
+def test_relu_special_values_follow_the_multiplication():
+    x = np.array([np.nan, np.inf, -np.inf, -0.0, 1e-45], dtype=np.float32)
+    with np.errstate(invalid="ignore"):
+        out = ora.relu_forward(x)
+    assert np.isnan(out[0]) and out[1] == np.inf and np.isnan(out[2])  # -inf * 0 is NaN
+    assert out[3] == 0.0 and np.signbit(out[3]) and out[4] == x[4]
+
+
+def test_multiply_and_sum_oracle_closed_forms():
+    import math
+
+    rng = np.random.default_rng(7)
+    a, b, g = (rng.standard_normal((3, 4, 5)) for _ in range(3))
+    assert np.array_equal(ora.multiply(a, b), a * b)
+    assert np.array_equal(ora.multiply_backward(g, a, b, 0), g * b)
+    assert np.array_equal(ora.multiply_backward(g, a, b, 1), g * a)
+    n = 100001
+    assert ora.sum_all(np.arange(n, dtype=np.float64)) == n * (n - 1) / 2  # exact in float64
+    x = rng.standard_normal(50000)
+    assert abs(ora.sum_all(x) - math.fsum(x)) <= 1e-13 * np.sum(np.abs(x))
+    assert np.array_equal(ora.sum_all_backward(a.astype(np.float32), np.float64(2.5)), np.full(a.shape, 2.5, np.float32))
+    assert ora.sum_all_backward(a.astype(np.float32), 2.5).dtype == np.float32
