@@ -21,7 +21,7 @@ struct PoolParams {
 // non-NaN best: ties keep the earlier element, a NaN once met is never replaced.
 template <typename T>
 __device__ __forceinline__ bool takes_over(T cand, T best) {
-  return (best == best) && (cand > best || cand != cand);
+  return (best == best) && !(cand <= best);  // "not <=" is true for cand > best and for a NaN cand
 }
 
 template <typename T>
