@@ -55,6 +55,8 @@ WORKLOADS = {
     "pool5": dict(kind="pool", dtype="f32", seed=1006, x=(8, 32, 32, 64, 64), pool=(2, 2, 2), stride=(2, 2, 2)),
     # relu, multiply and sum (forward and gradients) on a tensor of conv5's output size
     "elem5": dict(kind="elem", dtype="f32", seed=1007, x=(8, 32, 32, 64, 64)),
+    # batch normalisation (scaled and shifted) of a tensor of conv3a's output size
+    "bn3a": dict(kind="bn", dtype="f32", seed=1008, x=(128, 64, 56, 56), eps=1e-5),
 }
 NP_DTYPE = {"f32": np.float32, "f64": np.float64}
 
@@ -82,6 +84,8 @@ def describe(name):
     wl = WORKLOADS[name]
     if wl["kind"] == "elem":
         return f"{name}: relu + multiply + sum {wl['dtype']} x{wl['x']} fwd+bwd (7 kernels, 16 |x| bytes)"
+    if wl["kind"] == "bn":
+        return f"{name}: batchnorm {wl['dtype']} x{wl['x']} with gamma and beta, eps={wl['eps']}, fwd + dx, dgamma, dbeta"
     if wl["kind"] == "conv":
         return (f"{name}: conv_nd {wl['dtype']} x{wl['x']} * w{wl['w']} stride{wl['stride']} pad{wl['padding']} "
                 f"dil{wl['dilation']} -> grid{conv_grid(wl)} fwd+dx+dw")
@@ -123,6 +127,23 @@ class Step:
             self.total_work = 3 * per_pass
             self.unit, self.bound, self.peak = "TFLOP/s", "mfma", PEAK_TFLOPS[wl["dtype"]]
             self.scale = 1e-12
+        elif wl["kind"] == "bn":
+            channels = wl["x"][1]
+            x = (rng.standard_normal(wl["x"]) * 2 + 0.5).astype(dt)
+            g = rng.standard_normal(wl["x"]).astype(dt)
+            self.desc = _hip.bn_desc(wl["x"], dt, True, True, wl["eps"])
+            self.x, self.g = resident(x), resident(g)
+            self.gamma = resident(rng.uniform(0.5, 2, channels).astype(dt))
+            self.beta = resident(rng.standard_normal(channels).astype(dt))
+            self.out, self.dx = _device.DeviceBuffer(x.nbytes), _device.DeviceBuffer(x.nbytes)
+            self.mean, self.var, self.dgamma, self.dbeta = (_device.DeviceBuffer(max(channels * item, 16)) for _ in range(4))
+            # per launch: what each kernel must read and write; per step: x in and y out, then
+            # x and grad in and dx out (a step that never re-read anything would move 5 |x|)
+            self.work = {"batchnorm_stats": float(x.nbytes), "batchnorm_apply": 2.0 * x.nbytes,
+                         "batchnorm_bwd_sums": 2.0 * x.nbytes, "batchnorm_bwd_apply": 3.0 * x.nbytes}
+            self.total_work = 5.0 * x.nbytes
+            self.unit, self.bound, self.peak = "GB/s", "hbm", PEAK_HBM_GBS
+            self.scale = 1e-9
         elif wl["kind"] == "elem":
             x = rng.standard_normal(wl["x"]).astype(dt)
             g = rng.standard_normal(wl["x"]).astype(dt)
@@ -162,6 +183,11 @@ class Step:
             check(lib.mg_relu_bwd(c, n, self.x.ptr, self.dx.ptr, self.out.ptr))
             return
         d = self.desc
+        if self.wl["kind"] == "bn":
+            check(lib.mg_batchnorm_fwd(d, self.x.ptr, self.gamma.ptr, self.beta.ptr, self.out.ptr, self.mean.ptr, self.var.ptr))
+            check(lib.mg_batchnorm_bwd(d, self.x.ptr, self.g.ptr, self.gamma.ptr, self.mean.ptr, self.var.ptr,
+                                       self.dx.ptr, self.dgamma.ptr, self.dbeta.ptr))
+            return
         if self.wl["kind"] == "conv":
             check(lib.mg_conv_fwd(d, self.x.ptr, self.w.ptr, self.out.ptr))
             check(lib.mg_conv_dgrad(d, self.g.ptr, self.w.ptr, self.dx.ptr))
@@ -261,6 +287,18 @@ def run_cpu_baseline(name, min_seconds=10.0, max_reps=200):
 
         work, scale, unit = 3 * conv_flops_per_pass(wl), 1e-12, "TFLOP/s"
         what = "fwd+dx+dw"
+    elif wl["kind"] == "bn":
+        x = (rng.standard_normal(wl["x"]) * 2 + 0.5).astype(dt)
+        g = rng.standard_normal(wl["x"]).astype(dt)
+        gamma = rng.uniform(0.5, 2, wl["x"][1]).astype(dt)
+        beta = rng.standard_normal(wl["x"][1]).astype(dt)
+
+        def once():
+            ora.batchnorm_forward(x, gamma, beta, eps=wl["eps"])
+            ora.batchnorm_backward(g, x, gamma, eps=wl["eps"])
+
+        work, scale, unit = 5 * x.nbytes, 1e-9, "GB/s"
+        what = "forward, then dx, dgamma and dbeta (x_norm recomputed in the backward pass)"
     elif wl["kind"] == "elem":
         x = rng.standard_normal(wl["x"]).astype(dt)
         g = rng.standard_normal(wl["x"]).astype(dt)
@@ -327,6 +365,18 @@ def run_dropin(name, steps=5):
             out.backward(g)
 
         work, scale, unit = 3 * conv_flops_per_pass(wl), 1e-12, "TFLOP/s"
+    elif wl["kind"] == "bn":
+        from mygrad_amd.nnet import batchnorm
+
+        g = rng.standard_normal(wl["x"]).astype(dt)
+        gamma = rng.uniform(0.5, 2, wl["x"][1]).astype(dt)
+        beta = rng.standard_normal(wl["x"][1]).astype(dt)
+
+        def once():
+            xt, gt, bt = mg.Tensor(x, copy=False), mg.Tensor(gamma, copy=False), mg.Tensor(beta, copy=False)
+            batchnorm(xt, gamma=gt, beta=bt, eps=wl["eps"]).backward(g)
+
+        work, scale, unit = 5 * x.nbytes, 1e-9, "GB/s"
     elif wl["kind"] == "elem":
         from mygrad_amd.nnet import relu
 
@@ -427,7 +477,7 @@ def main():
     res = run_gpu(args.workload, args.steps, args.warmup)
     line = {
         "metric": {"conv": "conv_nd fwd+bwd TFLOP/s", "pool": "max_pool fwd+bwd GB/s",
-                   "elem": "relu+multiply+sum fwd+bwd GB/s"}[wl["kind"]],
+                   "elem": "relu+multiply+sum fwd+bwd GB/s", "bn": "batchnorm fwd+bwd GB/s"}[wl["kind"]],
         "value": res["value"],
         "unit": res["unit"],
         "n_gpus": 1,

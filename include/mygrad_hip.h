@@ -62,6 +62,18 @@ typedef struct {
   int64_t X[MG_MAX_ND], P[MG_MAX_ND], S[MG_MAX_ND], G[MG_MAX_ND];
 } mg_pool_desc;
 
+/* Shapes of one batch normalisation of x:(N, C, S...) over every axis but axis 1;
+ * S is the product of the axes after the second (1 if there are none).  gamma and beta
+ * are (C,) when announced. */
+typedef struct {
+  int32_t dtype;     /* mg_dtype of every tensor */
+  int32_t has_gamma; /* 0: no scaling (the reference's empty-array gamma, batchnorm.py:48-49) */
+  int32_t has_beta;  /* 0: no shift (batchnorm.py:50-51) */
+  int32_t reserved;
+  int64_t N, C, S;
+  double eps;        /* added to the variance under the root, >= 0 */
+} mg_bn_desc;
+
 typedef struct {
   char name[64];      /* hipDeviceProp_t::gcnArchName */
   int32_t compute_units;
@@ -173,6 +185,26 @@ int mg_sum_all(int dtype, int64_t n, const void *x, void *out);
 /* out[i] = *value (one element on the device).  Replaces Sum.backward_var with axis=None
  * (np.full(a.shape, grad), sequential/ops.py:123-126). */
 int mg_fill_from(int dtype, int64_t n, const void *value, void *out);
+
+/* ---- batch normalisation ---- */
+
+/* mean[c], var[c] = mean and (biased) variance of x[:, c, ...]; y = (x - mean) /
+ * sqrt(var + eps) [* gamma] [+ beta].  The sums run over a fixed partition in double and
+ * are rounded once; the element-wise steps are rounded in dtype in the reference's order.
+ * mean and var, (C,) each, are outputs the caller keeps for mg_batchnorm_bwd.
+ * Replaces BatchNorm.__call__, src/mygrad/nnet/layers/batchnorm.py:26-74. */
+int mg_batchnorm_fwd(const mg_bn_desc *desc, const void *x, const void *gamma, const void *beta, void *y, void *mean,
+                     void *var);
+
+/* With xn = (x - mean) / sqrt(var + eps) recomputed from x (the reference keeps it in
+ * self.x_norm, batchnorm.py:64):
+ *   dx     = ((grad - mean_c(grad)) - xn * sum_c(grad * xn) / (N*S)) / sqrt(var + eps) [* gamma]
+ *            (BatchNorm.backward_var index 0, batchnorm.py:78-99)
+ *   dgamma = sum_c(grad * xn)   (index 1 with gamma, batchnorm.py:101-102)
+ *   dbeta  = sum_c(grad)        (index 2, or 1 without gamma, batchnorm.py:104-106)
+ * Any of dx, dgamma, dbeta may be null (not wanted), not all three. */
+int mg_batchnorm_bwd(const mg_bn_desc *desc, const void *x, const void *grad, const void *gamma, const void *mean,
+                     const void *var, void *dx, void *dgamma, void *dbeta);
 
 #ifdef __cplusplus
 }

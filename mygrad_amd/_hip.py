@@ -74,6 +74,19 @@ class PoolDesc(ctypes.Structure):
     ]
 
 
+class BnDesc(ctypes.Structure):
+    _fields_ = [
+        ("dtype", ctypes.c_int32),
+        ("has_gamma", ctypes.c_int32),
+        ("has_beta", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
+        ("N", ctypes.c_int64),
+        ("C", ctypes.c_int64),
+        ("S", ctypes.c_int64),
+        ("eps", ctypes.c_double),
+    ]
+
+
 class DeviceInfo(ctypes.Structure):
     _fields_ = [
         ("name", ctypes.c_char * 64),
@@ -121,6 +134,8 @@ _SIGNATURES = {
     "mg_relu_bwd": [ctypes.c_int, ctypes.c_int64, _vp, _vp, _vp],
     "mg_sum_all": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
     "mg_fill_from": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
+    "mg_batchnorm_fwd": [ctypes.POINTER(BnDesc), _vp, _vp, _vp, _vp, _vp, _vp],
+    "mg_batchnorm_bwd": [ctypes.POINTER(BnDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES) + ("mg_last_error",)
 
@@ -217,6 +232,10 @@ KERNEL_TAGS = {
     8: "copy",
     9: "elementwise",
     10: "sum_all",
+    11: "batchnorm_stats",
+    12: "batchnorm_apply",
+    13: "batchnorm_bwd_sums",
+    14: "batchnorm_bwd_apply",
 }
 
 
@@ -292,4 +311,21 @@ def pool_desc(dtype, lead, pooled_shape, pool, stride, grid, dx_dtype=None):
         P=_right_aligned(pool, 1),
         S=_right_aligned(stride, 1),
         G=_right_aligned(grid, 1),
+    )
+
+
+def bn_desc(shape, dtype, has_gamma, has_beta, eps):
+    """Descriptor of a batch normalisation of an array of `shape` = (N, C, ...)."""
+    spatial = 1
+    for d in shape[2:]:
+        spatial *= int(d)
+    return BnDesc(
+        dtype=dtype_code(dtype),
+        has_gamma=int(bool(has_gamma)),
+        has_beta=int(bool(has_beta)),
+        reserved=0,
+        N=int(shape[0]),
+        C=int(shape[1]),
+        S=spatial,
+        eps=float(eps),
     )

@@ -52,6 +52,10 @@ enum KernelTag {
   TAG_COPY = 8,
   TAG_ELEMENTWISE = 9,
   TAG_REDUCE_ALL = 10,
+  TAG_BN_STATS = 11,
+  TAG_BN_APPLY = 12,
+  TAG_BN_BWD_SUMS = 13,
+  TAG_BN_BWD_APPLY = 14,
 };
 void timing_begin(int tag);
 void timing_end();

@@ -1,4 +1,4 @@
 from .activations import relu
-from .layers import conv_nd, max_pool
+from .layers import batchnorm, conv_nd, max_pool
 
-__all__ = ["conv_nd", "max_pool", "relu"]
+__all__ = ["batchnorm", "conv_nd", "max_pool", "relu"]

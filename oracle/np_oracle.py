@@ -30,6 +30,15 @@ Pinning (what holds each function to the reference without importing it):
                    single calls of the NumPy routine the reference calls
                    (``np.multiply``, ``np.sum``, ``np.full``); ``sum_all`` is
                    additionally held to ``math.fsum`` and closed forms in the tests
+  batchnorm_forward
+                   the reference's docstring vector; its tests' second formulation
+                   (mean / variance / division composed of primitives); closed forms
+                   (per-channel mean of the output is ``beta``, its variance
+                   ``gamma**2 * var / (var + eps)``)
+  batchnorm_backward
+                   central differences of ``sum(grad * batchnorm(x))`` in x, gamma
+                   and beta; the invariants ``sum_c(dx) == 0`` and, at ``eps == 0``,
+                   ``sum_c(dx * x_norm) == 0``
 """
 
 from numbers import Integral
@@ -50,6 +59,8 @@ __all__ = [
     "relu_backward",
     "sum_all",
     "sum_all_backward",
+    "batchnorm_forward",
+    "batchnorm_backward",
     "pool_out_shape",
     "pool_forward",
     "pool_backward",
@@ -351,3 +362,50 @@ def sum_all_backward(x, grad):
     """``Sum.backward_var`` with ``axis=None``: ``np.full(a.shape, grad, dtype=a.dtype)``
     (mygrad/math/sequential/ops.py:123-126)."""
     return np.full(x.shape, grad, dtype=x.dtype)
+
+
+# ------------------------------------------------------------------ batch normalisation
+def _channel_axes(x):
+    axes = tuple(i for i in range(x.ndim) if i != 1)
+    keep = tuple(1 if n != 1 else d for n, d in enumerate(x.shape))
+    return axes, keep
+
+
+def batchnorm_forward(x, gamma=None, beta=None, *, eps):
+    """BatchNorm.__call__ (src/mygrad/nnet/layers/batchnorm.py:43-74): returns
+    ``(y, mean, var)`` with ``mean`` / ``var`` the (C,) arrays the operation binds."""
+    x = np.asarray(x)
+    axes, keep = _channel_axes(x)
+    mean = x.mean(axis=axes)  # :58
+    var = x.var(axis=axes)  # :59
+    y = x - mean.reshape(keep)  # :61
+    std = np.sqrt(var + eps).reshape(keep)  # :62
+    y /= std  # :63
+    if gamma is not None:
+        y = y * np.asarray(gamma).reshape(keep)  # :69
+    if beta is not None:
+        y = y + np.asarray(beta).reshape(keep)  # :73
+    return y, mean, var
+
+
+def batchnorm_backward(grad, x, gamma=None, *, eps):
+    """BatchNorm.backward_var for indices 0, 1, 2 (batchnorm.py:76-106): returns
+    ``(dx, dgamma, dbeta)``; ``dgamma`` is the x_norm-weighted sum also when the forward
+    pass had no gamma (the reference then never asks for it)."""
+    x = np.asarray(x)
+    grad = np.asarray(grad)
+    axes, keep = _channel_axes(x)
+    std = np.sqrt(x.var(axis=axes) + eps).reshape(keep)
+    x_norm = (x - x.mean(axis=axes).reshape(keep)) / std
+    count = x.size / x.shape[1]  # :81
+    everything = list(range(x.ndim))
+    dot = np.einsum(grad, everything, x_norm, everything, [1])  # :88, :102
+
+    dx = grad - np.mean(grad, axis=axes, keepdims=True)  # :85
+    rterm = x_norm * np.reshape(dot, keep)  # :87-90
+    rterm /= count  # :91
+    dx -= rterm  # :92
+    dx /= std  # :93
+    if gamma is not None:
+        dx *= np.asarray(gamma).reshape(keep)  # :98
+    return dx, dot, grad.sum(axis=axes)  # :99, :102, :106

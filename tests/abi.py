@@ -127,3 +127,52 @@ def fill_from(value, shape, dtype):
     ob = _device.DeviceBuffer(max(n * np.dtype(dtype).itemsize, 16))
     _hip.check(_hip.lib().mg_fill_from(_hip.dtype_code(dtype), n, vb.ptr, ob.ptr))
     return _down(ob, shape, dtype)
+
+
+# ----------------------------------------------------------------- batch normalisation
+def batchnorm_fwd(x, gamma=None, beta=None, *, eps):
+    """-> (y, mean, var) of mg_batchnorm_fwd."""
+    desc = _hip.bn_desc(x.shape, x.dtype, gamma is not None, beta is not None, eps)
+    channels = x.shape[1]
+    xb = _up(x)
+    gb = _up(gamma.astype(x.dtype)) if gamma is not None else None
+    bb = _up(beta.astype(x.dtype)) if beta is not None else None
+    yb = _device.DeviceBuffer(max(x.nbytes, 16))
+    mb = _device.DeviceBuffer(max(channels * x.itemsize, 16))
+    vb = _device.DeviceBuffer(max(channels * x.itemsize, 16))
+    _hip.check(
+        _hip.lib().mg_batchnorm_fwd(
+            desc, xb.ptr, gb.ptr if gb is not None else None, bb.ptr if bb is not None else None, yb.ptr, mb.ptr, vb.ptr
+        )
+    )
+    return _down(yb, x.shape, x.dtype), _down(mb, (channels,), x.dtype), _down(vb, (channels,), x.dtype)
+
+
+def batchnorm_bwd(grad, x, mean, var, gamma=None, *, eps, want=("x", "gamma", "beta")):
+    """-> (dx, dgamma, dbeta) of mg_batchnorm_bwd; entries not in `want` are None."""
+    desc = _hip.bn_desc(x.shape, x.dtype, gamma is not None, False, eps)
+    channels = x.shape[1]
+    xb, gradb, mb, vb = _up(x), _up(grad.astype(x.dtype)), _up(mean), _up(var)
+    gb = _up(gamma.astype(x.dtype)) if gamma is not None else None
+    small = max(channels * x.itemsize, 16)
+    dxb = _device.DeviceBuffer(max(x.nbytes, 16)) if "x" in want else None
+    dgb = _device.DeviceBuffer(small) if "gamma" in want else None
+    dbb = _device.DeviceBuffer(small) if "beta" in want else None
+    _hip.check(
+        _hip.lib().mg_batchnorm_bwd(
+            desc,
+            xb.ptr,
+            gradb.ptr,
+            gb.ptr if gb is not None else None,
+            mb.ptr,
+            vb.ptr,
+            dxb.ptr if dxb is not None else None,
+            dgb.ptr if dgb is not None else None,
+            dbb.ptr if dbb is not None else None,
+        )
+    )
+    return (
+        _down(dxb, x.shape, x.dtype) if dxb is not None else None,
+        _down(dgb, (channels,), x.dtype) if dgb is not None else None,
+        _down(dbb, (channels,), x.dtype) if dbb is not None else None,
+    )

@@ -331,3 +331,90 @@ def test_multiply_and_sum_oracle_closed_forms():
     assert abs(ora.sum_all(x) - math.fsum(x)) <= 1e-13 * np.sum(np.abs(x))
     assert np.array_equal(ora.sum_all_backward(a.astype(np.float32), np.float64(2.5)), np.full(a.shape, 2.5, np.float32))
     assert ora.sum_all_backward(a.astype(np.float32), 2.5).dtype == np.float32
+
+
+# ----------------------------------------------------------------- batch normalisation
+def test_batchnorm_reference_docstring_vector(kats):
+    for case in kats["batchnorm"]:
+        for dtype in (np.float32, np.float64):
+            x = np.array(case["x"], dtype=dtype)
+            y, mean, var = ora.batchnorm_forward(x, eps=case["eps"])
+            assert y.dtype == dtype and mean.shape == var.shape == (x.shape[1],)
+            assert np.allclose(y, np.array(case["out"]), rtol=0, atol=2 * 10.0 ** -case["decimals"] if dtype == np.float64 else 1e-6)
+
+
+def _composed_batchnorm(x, gamma, beta, eps):
+    """The second formulation the reference's tests compare against
+    (tests/nnet/layers/test_batchnorm.py:13-48): variance as the mean of squared
+    deviations, one division by the root."""
+    axes = tuple(i for i in range(x.ndim) if i != 1)
+    keep = tuple(1 if n != 1 else d for n, d in enumerate(x.shape))
+    count = np.prod([x.shape[i] for i in axes])
+    mean = x.sum(axis=axes, keepdims=True) / count
+    var = ((x - mean) ** 2).sum(axis=axes, keepdims=True) / count
+    out = (x - mean) / np.sqrt(var + eps)
+    if gamma is not None:
+        out = out * gamma.reshape(keep)
+    if beta is not None:
+        out = out + beta.reshape(keep)
+    return out
+
+
+BN_SHAPES = [(5, 3), (4, 3, 7), (3, 2, 5, 6), (2, 4, 3, 2, 3)]
+
+
+@pytest.mark.parametrize("shape", BN_SHAPES)
+@pytest.mark.parametrize("affine", [(False, False), (True, False), (False, True), (True, True)])
+def test_batchnorm_forward_second_formulation_and_closed_forms(shape, affine):
+    rng = np.random.default_rng([len(shape), int(np.prod(shape)), int(affine[0]), int(affine[1])])
+    x = rng.uniform(-100, 100, shape)
+    gamma = rng.uniform(-10, 10, shape[1]) if affine[0] else None
+    beta = rng.uniform(-10, 10, shape[1]) if affine[1] else None
+    eps = 1e-3
+    y, mean, var = ora.batchnorm_forward(x, gamma, beta, eps=eps)
+    assert np.allclose(y, _composed_batchnorm(x, gamma, beta, eps), rtol=1e-12, atol=1e-12)
+    axes = tuple(i for i in range(x.ndim) if i != 1)
+    g = np.ones(shape[1]) if gamma is None else gamma
+    b = np.zeros(shape[1]) if beta is None else beta
+    assert np.allclose(y.mean(axis=axes), b, atol=1e-12)
+    assert np.allclose(y.var(axis=axes), g**2 * var / (var + eps), rtol=1e-11)
+    assert np.allclose(mean, np.moveaxis(x, 1, 0).reshape(shape[1], -1).mean(axis=1))
+
+
+@pytest.mark.parametrize("shape", BN_SHAPES)
+@pytest.mark.parametrize("with_gamma", [False, True])
+def test_batchnorm_backward_against_central_differences(shape, with_gamma):
+    rng = np.random.default_rng([len(shape), int(np.prod(shape)), int(with_gamma), 77])
+    x = rng.standard_normal(shape)
+    gamma = rng.uniform(0.5, 2, shape[1]) * rng.choice([-1, 1], shape[1]) if with_gamma else None
+    beta = rng.standard_normal(shape[1])
+    grad = rng.standard_normal(shape)
+    eps = 1e-2
+
+    def loss(x_, gamma_, beta_):
+        return float(np.sum(grad * ora.batchnorm_forward(x_, gamma_, beta_, eps=eps)[0]))
+
+    dx, dgamma, dbeta = ora.batchnorm_backward(grad, x, gamma, eps=eps)
+    h = 1e-6
+    num_dx = np.zeros_like(x)
+    for idx in np.ndindex(*shape):
+        up, dn = x.copy(), x.copy()
+        up[idx] += h
+        dn[idx] -= h
+        num_dx[idx] = (loss(up, gamma, beta) - loss(dn, gamma, beta)) / (2 * h)
+    assert np.allclose(dx, num_dx, rtol=1e-6, atol=1e-7)
+
+    base_gamma = np.ones(shape[1]) if gamma is None else gamma
+    for c in range(shape[1]):
+        e = np.zeros(shape[1])
+        e[c] = h
+        num_dgamma = (loss(x, base_gamma + e, beta) - loss(x, base_gamma - e, beta)) / (2 * h)
+        num_dbeta = (loss(x, gamma, beta + e) - loss(x, gamma, beta - e)) / (2 * h)
+        assert abs(dgamma[c] - num_dgamma) <= 1e-6 * max(1.0, abs(num_dgamma))
+        assert abs(dbeta[c] - num_dbeta) <= 1e-6 * max(1.0, abs(num_dbeta))
+
+    axes = tuple(i for i in range(x.ndim) if i != 1)
+    assert np.allclose(dx.sum(axis=axes), 0, atol=1e-12)
+    dx0, _, _ = ora.batchnorm_backward(grad, x, gamma, eps=0)
+    xn0 = ora.batchnorm_forward(x, eps=0)[0]
+    assert np.allclose((dx0 * xn0).sum(axis=axes), 0, atol=1e-11)
