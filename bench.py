@@ -57,6 +57,11 @@ WORKLOADS = {
     "elem5": dict(kind="elem", dtype="f32", seed=1007, x=(8, 32, 32, 64, 64)),
     # batch normalisation (scaled and shifted) of a tensor of conv3a's output size
     "bn3a": dict(kind="bn", dtype="f32", seed=1008, x=(128, 64, 56, 56), eps=1e-5),
+    # repeat: twofold nearest-neighbour upsampling of the rows of a tensor of pool5's input size
+    # (forward and gradient), and then of its columns
+    "rep5": dict(kind="repeat", dtype="f32", seed=1009, x=(8, 32, 32, 64, 64), repeats=2, axes=(-2, -1)),
+    # the dense copy of the window view the 3x3 convolution of config 3a reads (a quarter of its batch)
+    "win3a": dict(kind="window", dtype="f32", seed=1010, x=(32, 64, 56, 56), window=(3, 3), step=(1, 1), dilation=(1, 1)),
 }
 NP_DTYPE = {"f32": np.float32, "f64": np.float64}
 
@@ -84,6 +89,11 @@ def describe(name):
     wl = WORKLOADS[name]
     if wl["kind"] == "elem":
         return f"{name}: relu + multiply + sum {wl['dtype']} x{wl['x']} fwd+bwd (7 kernels, 16 |x| bytes)"
+    if wl["kind"] == "repeat":
+        return f"{name}: repeat {wl['dtype']} x{wl['x']} repeats={wl['repeats']} along axis {wl['axes'][0]}, then along axis {wl['axes'][1]}, fwd+bwd each"
+    if wl["kind"] == "window":
+        return (f"{name}: contiguous copy of sliding_window_view {wl['dtype']} x{wl['x']} window{wl['window']} "
+                f"step{wl['step']} dilation{wl['dilation']}")
     if wl["kind"] == "bn":
         return f"{name}: batchnorm {wl['dtype']} x{wl['x']} with gamma and beta, eps={wl['eps']}, fwd + dx, dgamma, dbeta"
     if wl["kind"] == "conv":
@@ -127,6 +137,36 @@ class Step:
             self.total_work = 3 * per_pass
             self.unit, self.bound, self.peak = "TFLOP/s", "mfma", PEAK_TFLOPS[wl["dtype"]]
             self.scale = 1e-12
+        elif wl["kind"] == "repeat":
+            x = rng.standard_normal(wl["x"]).astype(dt)
+            r = wl["repeats"]
+            g = rng.standard_normal((*wl["x"][:-1], wl["x"][-1] * r)).astype(dt)  # same size for either axis
+            self.x, self.g = resident(x), resident(g)
+            self.out, self.dx = _device.DeviceBuffer(g.nbytes), _device.DeviceBuffer(x.nbytes)
+            self.geometry = []
+            for axis in wl["axes"]:
+                axis %= len(wl["x"])
+                outer, n, inner = int(np.prod(wl["x"][:axis])), wl["x"][axis], int(np.prod(wl["x"][axis + 1:]))
+                self.geometry.append((outer, n, inner, r, n * r))
+            self.code = _hip.dtype_code(dt)
+            self.work = {"repeat_fwd": float(x.nbytes + g.nbytes), "repeat_bwd": float(x.nbytes + g.nbytes)}
+            self.total_work = 4.0 * (x.nbytes + g.nbytes)
+            self.unit, self.bound, self.peak = "GB/s", "hbm", PEAK_HBM_GBS
+            self.scale = 1e-9
+        elif wl["kind"] == "window":
+            x = rng.standard_normal(wl["x"]).astype(dt)
+            m = len(wl["window"])
+            tail = wl["x"][len(wl["x"]) - m:]
+            grid = tuple((tail[k] - ((wl["window"][k] - 1) * wl["dilation"][k] + 1)) // wl["step"][k] + 1 for k in range(m))
+            lead = int(np.prod(wl["x"][: len(wl["x"]) - m]))
+            count = int(np.prod(grid)) * lead * int(np.prod(wl["window"]))
+            self.desc = _hip.window_desc(item, lead, tail, wl["window"], wl["step"], wl["dilation"], grid)
+            self.x = resident(x)
+            self.out = _device.DeviceBuffer(count * item)
+            self.work = {"window_gather": float(x.nbytes + count * item)}
+            self.total_work = self.work["window_gather"]
+            self.unit, self.bound, self.peak = "GB/s", "hbm", PEAK_HBM_GBS
+            self.scale = 1e-9
         elif wl["kind"] == "bn":
             channels = wl["x"][1]
             x = (rng.standard_normal(wl["x"]) * 2 + 0.5).astype(dt)
@@ -182,7 +222,15 @@ class Step:
             check(lib.mg_multiply(c, n, self.dx.ptr, self.x.ptr, self.out.ptr))  # d (a*b) / d b
             check(lib.mg_relu_bwd(c, n, self.x.ptr, self.dx.ptr, self.out.ptr))
             return
+        if self.wl["kind"] == "repeat":
+            for outer, n, inner, r, total in self.geometry:
+                check(lib.mg_repeat_fwd(4 if self.code == 0 else 8, outer, n, inner, r, total, None, self.x.ptr, self.out.ptr))
+                check(lib.mg_repeat_bwd(self.code, outer, n, inner, r, total, None, self.g.ptr, self.dx.ptr))
+            return
         d = self.desc
+        if self.wl["kind"] == "window":
+            check(lib.mg_window_gather(d, self.x.ptr, self.out.ptr))
+            return
         if self.wl["kind"] == "bn":
             check(lib.mg_batchnorm_fwd(d, self.x.ptr, self.gamma.ptr, self.beta.ptr, self.out.ptr, self.mean.ptr, self.var.ptr))
             check(lib.mg_batchnorm_bwd(d, self.x.ptr, self.g.ptr, self.gamma.ptr, self.mean.ptr, self.var.ptr,
@@ -287,6 +335,26 @@ def run_cpu_baseline(name, min_seconds=10.0, max_reps=200):
 
         work, scale, unit = 3 * conv_flops_per_pass(wl), 1e-12, "TFLOP/s"
         what = "fwd+dx+dw"
+    elif wl["kind"] == "repeat":
+        x = rng.standard_normal(wl["x"]).astype(dt)
+        g = rng.standard_normal((*wl["x"][:-1], wl["x"][-1] * wl["repeats"])).astype(dt)
+
+        def once():
+            for axis in wl["axes"]:
+                out = ora.repeat_forward(x, wl["repeats"], axis)
+                ora.repeat_backward(g.reshape(out.shape), x, wl["repeats"], axis)
+
+        work, scale, unit = 4 * (x.nbytes + g.nbytes), 1e-9, "GB/s"
+        what = "np.repeat and the windowed-sum gradient along each of the two axes"
+    elif wl["kind"] == "window":
+        x = rng.standard_normal(wl["x"]).astype(dt)
+        count = np.prod(ora.window_view(x, wl["window"], wl["step"], wl["dilation"]).shape)
+
+        def once():
+            np.ascontiguousarray(ora.window_view(x, wl["window"], wl["step"], wl["dilation"]))
+
+        work, scale, unit = x.nbytes + int(count) * x.itemsize, 1e-9, "GB/s"
+        what = "np.ascontiguousarray of the view"
     elif wl["kind"] == "bn":
         x = (rng.standard_normal(wl["x"]) * 2 + 0.5).astype(dt)
         g = rng.standard_normal(wl["x"]).astype(dt)
@@ -365,6 +433,23 @@ def run_dropin(name, steps=5):
             out.backward(g)
 
         work, scale, unit = 3 * conv_flops_per_pass(wl), 1e-12, "TFLOP/s"
+    elif wl["kind"] == "repeat":
+        g = rng.standard_normal((*wl["x"][:-1], wl["x"][-1] * wl["repeats"])).astype(dt)
+
+        def once():
+            for axis in wl["axes"]:
+                xt = mg.Tensor(x, copy=False)
+                out = mg.repeat(xt, wl["repeats"], axis)
+                out.backward(g.reshape(out.shape))
+
+        work, scale, unit = 4 * (x.nbytes + g.nbytes), 1e-9, "GB/s"
+    elif wl["kind"] == "window":
+        count = int(np.prod(mg.sliding_window_view(x, wl["window"], wl["step"], wl["dilation"]).shape))
+
+        def once():
+            mg.sliding_window_copy(x, wl["window"], wl["step"], wl["dilation"])
+
+        work, scale, unit = x.nbytes + count * x.itemsize, 1e-9, "GB/s"
     elif wl["kind"] == "bn":
         from mygrad_amd.nnet import batchnorm
 
@@ -477,7 +562,8 @@ def main():
     res = run_gpu(args.workload, args.steps, args.warmup)
     line = {
         "metric": {"conv": "conv_nd fwd+bwd TFLOP/s", "pool": "max_pool fwd+bwd GB/s",
-                   "elem": "relu+multiply+sum fwd+bwd GB/s", "bn": "batchnorm fwd+bwd GB/s"}[wl["kind"]],
+                   "elem": "relu+multiply+sum fwd+bwd GB/s", "bn": "batchnorm fwd+bwd GB/s",
+                   "repeat": "repeat fwd+bwd GB/s", "window": "sliding-window copy GB/s"}[wl["kind"]],
         "value": res["value"],
         "unit": res["unit"],
         "n_gpus": 1,

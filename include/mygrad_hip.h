@@ -74,6 +74,16 @@ typedef struct {
   double eps;        /* added to the variance under the root, >= 0 */
 } mg_bn_desc;
 
+/* A sliding-window view of x:(lead, X...) over its trailing nd axes: window W placed every
+ * S elements, its own elements D apart; G[k] <= (X[k] - ((W[k]-1)*D[k]+1)) / S[k] + 1 placements
+ * per axis (src/mygrad/nnet/layers/utils.py:201-228).  Right-aligned like mg_conv_desc. */
+typedef struct {
+  int32_t elem_bytes; /* 1, 2, 4 or 8: the copy moves bytes, any dtype of that size */
+  int32_t nd;         /* 1..MG_MAX_ND */
+  int64_t lead;
+  int64_t X[MG_MAX_ND], W[MG_MAX_ND], S[MG_MAX_ND], D[MG_MAX_ND], G[MG_MAX_ND];
+} mg_window_desc;
+
 typedef struct {
   char name[64];      /* hipDeviceProp_t::gcnArchName */
   int32_t compute_units;
@@ -205,6 +215,31 @@ int mg_batchnorm_fwd(const mg_bn_desc *desc, const void *x, const void *gamma, c
  * Any of dx, dgamma, dbeta may be null (not wanted), not all three. */
 int mg_batchnorm_bwd(const mg_bn_desc *desc, const void *x, const void *grad, const void *gamma, const void *mean,
                      const void *var, void *dx, void *dgamma, void *dbeta);
+
+/* ---- repeat and the window view ---- */
+
+/* out[o, j, i] = a[o, src(j), i] with a seen as (outer, n, inner) around the repeated axis
+ * (outer = inner = 1 for the flattened axis=None case) and out as (outer, total, inner).
+ * src_of == NULL: every entry `repeats` times, src(j) = j / repeats, total = n * repeats.
+ * Otherwise src_of[total] (int32, on the device) names the source entry of each output entry
+ * (np.repeat(arange(n), repeats)).  Moves bytes: elem_bytes in {1, 2, 4, 8}, any dtype.
+ * Replaces Repeat.__call__ (np.repeat), src/mygrad/tensor_manip/tiling/ops.py:16-22. */
+int mg_repeat_fwd(int elem_bytes, int64_t outer, int64_t n, int64_t inner, int64_t repeats, int64_t total,
+                  const int32_t *src_of, const void *a, void *out);
+
+/* da[o, s, i] = sum of grad[o, j, i] over the run of output entries j that came from s, in
+ * ascending j starting from +0.0, every addition rounded in dtype.  offsets == NULL: runs of
+ * `repeats` (the reference sums a windowed view of grad, tiling/ops.py:36-56); otherwise
+ * offsets[n + 1] (int64, on the device), run s = [offsets[s], offsets[s+1]), offsets[n] = total
+ * (the reference's np.add.at over repeated flat indices, tiling/ops.py:58-72: same order, same
+ * arithmetic).  dtype: 0 float32, 1 float64. */
+int mg_repeat_bwd(int dtype, int64_t outer, int64_t n, int64_t inner, int64_t repeats, int64_t total,
+                  const int64_t *offsets, const void *grad, void *da);
+
+/* out:(G..., lead, W...) contiguous, out[g, l, w] = x[l, g*S + w*D]: the C-contiguous copy of
+ * sliding_window_view(x, W, S, D), src/mygrad/nnet/layers/utils.py:7-228 (the view itself is a
+ * host-side stride trick and moves nothing). */
+int mg_window_gather(const mg_window_desc *desc, const void *x, void *out);
 
 #ifdef __cplusplus
 }

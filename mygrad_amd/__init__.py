@@ -15,10 +15,11 @@ from . import _device, _graph, _hip, nnet
 from ._graph import mem_guard_off, mem_guard_on, no_autodiff
 from ._hip import HipError, HipUnavailable, device_info, is_available, synchronize
 from .errors import InvalidBackprop, InvalidGradient, SkipGradient
-from .nnet.layers.utils import sliding_window_view
+from .nnet.layers.utils import sliding_window_copy, sliding_window_view
 from .operation_base import Operation
 from .tensor_base import Tensor, asarray, tensor
 from .math import multiply, sum  # noqa: A004  (after tensor_base: the ops import Tensor)
+from .tensor_manip import repeat
 
 execute_op = Tensor._op
 
@@ -32,8 +33,10 @@ __all__ = [
     "mem_guard_off",
     "mem_guard_on",
     "sliding_window_view",
+    "sliding_window_copy",
     "multiply",
     "sum",
+    "repeat",
     "nnet",
     "InvalidBackprop",
     "InvalidGradient",

@@ -87,6 +87,19 @@ class BnDesc(ctypes.Structure):
     ]
 
 
+class WindowDesc(ctypes.Structure):
+    _fields_ = [
+        ("elem_bytes", ctypes.c_int32),
+        ("nd", ctypes.c_int32),
+        ("lead", ctypes.c_int64),
+        ("X", _I64x3),
+        ("W", _I64x3),
+        ("S", _I64x3),
+        ("D", _I64x3),
+        ("G", _I64x3),
+    ]
+
+
 class DeviceInfo(ctypes.Structure):
     _fields_ = [
         ("name", ctypes.c_char * 64),
@@ -136,6 +149,9 @@ _SIGNATURES = {
     "mg_fill_from": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
     "mg_batchnorm_fwd": [ctypes.POINTER(BnDesc), _vp, _vp, _vp, _vp, _vp, _vp],
     "mg_batchnorm_bwd": [ctypes.POINTER(BnDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
+    "mg_repeat_fwd": [ctypes.c_int] + [ctypes.c_int64] * 5 + [_vp, _vp, _vp],
+    "mg_repeat_bwd": [ctypes.c_int] + [ctypes.c_int64] * 5 + [_vp, _vp, _vp],
+    "mg_window_gather": [ctypes.POINTER(WindowDesc), _vp, _vp],
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES) + ("mg_last_error",)
 
@@ -236,6 +252,9 @@ KERNEL_TAGS = {
     12: "batchnorm_apply",
     13: "batchnorm_bwd_sums",
     14: "batchnorm_bwd_apply",
+    15: "repeat_fwd",
+    16: "repeat_bwd",
+    17: "window_gather",
 }
 
 
@@ -328,4 +347,18 @@ def bn_desc(shape, dtype, has_gamma, has_beta, eps):
         C=int(shape[1]),
         S=spatial,
         eps=float(eps),
+    )
+
+
+def window_desc(itemsize, lead, windowed_shape, window_shape, step, dilation, grid):
+    """Descriptor of a sliding-window view over the trailing axes of an array."""
+    return WindowDesc(
+        elem_bytes=int(itemsize),
+        nd=len(window_shape),
+        lead=int(lead),
+        X=_right_aligned(windowed_shape, 1),
+        W=_right_aligned(window_shape, 1),
+        S=_right_aligned(step, 1),
+        D=_right_aligned(dilation, 1),
+        G=_right_aligned(grid, 1),
     )

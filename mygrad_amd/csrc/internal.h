@@ -56,6 +56,9 @@ enum KernelTag {
   TAG_BN_APPLY = 12,
   TAG_BN_BWD_SUMS = 13,
   TAG_BN_BWD_APPLY = 14,
+  TAG_REPEAT_FWD = 15,
+  TAG_REPEAT_BWD = 16,
+  TAG_WINDOW_GATHER = 17,
 };
 void timing_begin(int tag);
 void timing_end();

@@ -8,7 +8,9 @@ read-only view -- and stays on the host.  Its index map
 
 is the address function the convolution and pooling kernels evaluate on the
 device; ``check_window_args`` is the part of it that the operations reuse to
-raise the reference's errors before anything is launched.
+raise the reference's errors before anything is launched.  ``sliding_window_copy``
+evaluates the same map on the device and returns the C-contiguous copy of the view
+(what ``np.ascontiguousarray(sliding_window_view(...))`` gives).
 """
 
 from numbers import Integral
@@ -16,7 +18,7 @@ from numbers import Integral
 import numpy as np
 from numpy.lib.stride_tricks import as_strided
 
-__all__ = ["sliding_window_view", "check_window_args"]
+__all__ = ["sliding_window_view", "sliding_window_copy", "check_window_args"]
 
 
 def check_window_args(shape, window_shape, step, dilation=None):
@@ -126,3 +128,34 @@ def sliding_window_view(arr, window_shape, step, dilation=None):
         strides=tuple(arr.itemsize * s for s in elem_strides),
         writeable=False,
     )
+
+
+def sliding_window_copy(arr, window_shape, step, dilation=None):
+    """C-contiguous copy of ``sliding_window_view(arr, window_shape, step, dilation)``,
+    gathered on the device (same arguments, same errors, same shape; writable).
+
+    The view costs nothing and is the right tool on the host; the copy is for consumers
+    that need the windows laid out densely, and it is produced at memory speed instead of
+    by NumPy's strided copy loop.  At most three windowed axes; elements of 1, 2, 4 or 8
+    bytes."""
+    from ... import _device, _hip
+
+    arr = np.asarray(arr)
+    window, step, dilation = check_window_args(arr.shape, window_shape, step, dilation)
+    m = len(window)
+    if not 1 <= m <= _hip.MG_MAX_ND:
+        raise NotImplementedError(f"sliding_window_copy handles 1 to {_hip.MG_MAX_ND} windowed axes, got {m} (no CPU fallback)")
+    if arr.dtype.itemsize not in (1, 2, 4, 8) or arr.dtype.hasobject:
+        raise TypeError(f"sliding_window_copy moves elements of 1, 2, 4 or 8 bytes, got {arr.dtype} (no CPU fallback)")
+    lead_shape, tail = arr.shape[: arr.ndim - m], arr.shape[arr.ndim - m :]
+    grid = tuple((tail[k] - ((window[k] - 1) * dilation[k] + 1)) // step[k] + 1 for k in range(m))
+    out_shape = grid + lead_shape + window
+    count = int(np.prod(out_shape, dtype=np.int64))
+    if count == 0:
+        return np.empty(out_shape, dtype=arr.dtype)
+    lead = int(np.prod(lead_shape, dtype=np.int64))
+    desc = _hip.window_desc(arr.dtype.itemsize, lead, tail, window, step, dilation, grid)
+    xb = _device.to_device(arr)
+    ob = _device.DeviceBuffer(max(count * arr.dtype.itemsize, 16))
+    _hip.check(_hip.lib().mg_window_gather(desc, xb.ptr, ob.ptr))
+    return _device.download(ob, out_shape, arr.dtype)

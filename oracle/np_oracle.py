@@ -39,6 +39,10 @@ Pinning (what holds each function to the reference without importing it):
                    central differences of ``sum(grad * batchnorm(x))`` in x, gamma
                    and beta; the invariants ``sum_c(dx) == 0`` and, at ``eps == 0``,
                    ``sum_c(dx * x_norm) == 0``
+  repeat_forward   a single call of ``np.repeat`` (what the reference calls); the
+                   reference's four docstring vectors
+  repeat_backward  element-by-element loops; the adjoint identity
+                   ``<repeat(a), g> == <a, repeat_backward(g)>`` (repeat is linear)
 """
 
 from numbers import Integral
@@ -61,6 +65,8 @@ __all__ = [
     "sum_all_backward",
     "batchnorm_forward",
     "batchnorm_backward",
+    "repeat_forward",
+    "repeat_backward",
     "pool_out_shape",
     "pool_forward",
     "pool_backward",
@@ -409,3 +415,39 @@ def batchnorm_backward(grad, x, gamma=None, *, eps):
     if gamma is not None:
         dx *= np.asarray(gamma).reshape(keep)  # :98
     return dx, dot, grad.sum(axis=axes)  # :99, :102, :106
+
+
+# ------------------------------------------------------------------ repeat
+def repeat_forward(a, repeats, axis=None):
+    """Repeat.__call__ (src/mygrad/tensor_manip/tiling/ops.py:16-22)."""
+    return np.repeat(np.asarray(a), repeats=repeats, axis=axis)
+
+
+def repeat_backward(grad, a, repeats, axis=None):
+    """Repeat.backward_var (tiling/ops.py:24-72): equal repeats sum a windowed view of the
+    gradient whose windows span the runs of copies (:36-56); unequal repeats add the
+    gradient into place through repeated flat indices (:58-72)."""
+    a = np.asarray(a)
+    grad = np.asarray(grad)
+    if isinstance(repeats, Integral) or len(repeats) == 1:
+        if not isinstance(repeats, Integral):
+            (repeats,) = repeats
+        if not repeats:
+            return np.zeros(a.shape, dtype=grad.dtype)  # :32-34
+        if axis is None:
+            grad = grad.ravel()  # :38
+            window_shape = (repeats,)
+        else:
+            window_shape = [1] * max(1, a.ndim)  # :43
+            window_shape[axis] = repeats
+            window_shape = tuple(window_shape)
+        view = window_view(grad, window_shape, window_shape)  # :51-53
+        out = view.sum(axis=tuple(range(-len(window_shape), 0)))  # :54
+        if axis is None:
+            out.shape = a.shape
+        return out
+    out = np.zeros((a.size,), dtype=grad.dtype)  # :67
+    indices = np.arange(a.size).reshape(a.shape)
+    indices = np.repeat(indices, repeats=repeats, axis=axis)
+    np.add.at(out, indices.ravel(), grad.ravel())  # :70
+    return out.reshape(a.shape)

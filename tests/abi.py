@@ -176,3 +176,62 @@ def batchnorm_bwd(grad, x, mean, var, gamma=None, *, eps, want=("x", "gamma", "b
         _down(dgb, (channels,), x.dtype) if dgb is not None else None,
         _down(dbb, (channels,), x.dtype) if dbb is not None else None,
     )
+
+
+# ----------------------------------------------------------------- repeat, window copy
+def _around_axis(shape, axis):
+    if axis is None:
+        return 1, int(np.prod(shape, dtype=np.int64)), 1
+    axis = axis % len(shape)
+    return (
+        int(np.prod(shape[:axis], dtype=np.int64)),
+        int(shape[axis]),
+        int(np.prod(shape[axis + 1 :], dtype=np.int64)),
+    )
+
+
+def repeat_fwd(a, repeats, axis=None):
+    """np.repeat through mg_repeat_fwd (a: at least 1-D)."""
+    outer, n, inner = _around_axis(a.shape, axis)
+    src_of = np.repeat(np.arange(n, dtype=np.int32), repeats)
+    total = src_of.size
+    uniform = np.ndim(repeats) == 0
+    out_shape = (total,) if axis is None else (*a.shape[: axis % a.ndim], total, *a.shape[axis % a.ndim + 1 :])
+    ab = _up(a)
+    sb = None if uniform else _up(src_of)
+    ob = _device.DeviceBuffer(max(int(np.prod(out_shape, dtype=np.int64)) * a.itemsize, 16))
+    _hip.check(
+        _hip.lib().mg_repeat_fwd(
+            a.itemsize, outer, n, inner, int(repeats) if uniform else 0, total, sb.ptr if sb is not None else None, ab.ptr, ob.ptr
+        )
+    )
+    return _down(ob, out_shape, a.dtype)
+
+
+def repeat_bwd(grad, a_shape, repeats, axis=None):
+    outer, n, inner = _around_axis(a_shape, axis)
+    uniform = np.ndim(repeats) == 0
+    offsets = None if uniform else np.concatenate([[0], np.cumsum(repeats)]).astype(np.int64)
+    total = n * int(repeats) if uniform else int(offsets[-1])
+    gb = _up(grad)
+    fb = None if uniform else _up(offsets)
+    ob = _device.DeviceBuffer(max(int(np.prod(a_shape, dtype=np.int64)) * grad.itemsize, 16))
+    _hip.check(
+        _hip.lib().mg_repeat_bwd(
+            _hip.dtype_code(grad.dtype), outer, n, inner, int(repeats) if uniform else 0, total,
+            fb.ptr if fb is not None else None, gb.ptr, ob.ptr,
+        )
+    )
+    return _down(ob, tuple(a_shape), grad.dtype)
+
+
+def window_gather(x, window, step, dilation):
+    m = len(window)
+    lead_shape, tail = x.shape[: x.ndim - m], x.shape[x.ndim - m :]
+    grid = tuple((tail[k] - ((window[k] - 1) * dilation[k] + 1)) // step[k] + 1 for k in range(m))
+    out_shape = grid + lead_shape + tuple(window)
+    desc = _hip.window_desc(x.itemsize, int(np.prod(lead_shape, dtype=np.int64)), tail, window, step, dilation, grid)
+    xb = _up(x)
+    ob = _device.DeviceBuffer(max(int(np.prod(out_shape, dtype=np.int64)) * x.itemsize, 16))
+    _hip.check(_hip.lib().mg_window_gather(desc, xb.ptr, ob.ptr))
+    return _down(ob, out_shape, x.dtype)

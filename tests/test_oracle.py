@@ -418,3 +418,50 @@ def test_batchnorm_backward_against_central_differences(shape, with_gamma):
     dx0, _, _ = ora.batchnorm_backward(grad, x, gamma, eps=0)
     xn0 = ora.batchnorm_forward(x, eps=0)[0]
     assert np.allclose((dx0 * xn0).sum(axis=axes), 0, atol=1e-11)
+
+
+# ----------------------------------------------------------------- repeat
+def test_repeat_reference_docstring_vectors(kats):
+    for case in kats["repeat"]:
+        out = ora.repeat_forward(np.array(case["a"]), case["repeats"], case["axis"])
+        assert np.array_equal(out, np.array(case["out"])), case["source"]
+
+
+def _repeat_backward_by_loops(grad, a_shape, repeats, axis):
+    """dx[i] = sum of grad over the copies of entry i, located by repeating the flat indices."""
+    size = int(np.prod(a_shape, dtype=np.int64))
+    where = np.repeat(np.arange(size).reshape(a_shape), repeats, axis=axis).ravel()
+    out = np.zeros(size, dtype=np.float64)
+    for j, i in enumerate(where):
+        out[i] += grad.ravel()[j]
+    return out.reshape(a_shape)
+
+
+REPEAT_CASES = [
+    ((), 3, None),
+    ((), 2, 0),
+    ((5,), 0, None),
+    ((5,), 4, 0),
+    ((2, 3), 2, None),
+    ((2, 3), 3, 1),
+    ((2, 3, 4), 2, -2),
+    ((2, 3, 4), [3], 0),
+    ((2, 3), [1, 2], 0),
+    ((2, 3), [0, 2, 5], 1),
+    ((2, 2), [2, 0, 1, 3], None),
+    ((3, 1, 2), [0, 0, 0], 0),
+]
+
+
+@pytest.mark.parametrize("shape, repeats, axis", REPEAT_CASES)
+def test_repeat_backward_by_loops_and_adjoint(shape, repeats, axis):
+    rng = np.random.default_rng([len(shape), int(np.prod(shape, dtype=np.int64)), 5])
+    a = rng.standard_normal(shape)
+    out = ora.repeat_forward(a, repeats, axis)
+    grad = rng.standard_normal(out.shape)
+    da = ora.repeat_backward(grad, a, repeats, axis)
+    # a scalar repeated along axis 0 comes back as one entry; Operation.backward reshapes it
+    assert da.shape == (a.shape or ((1,) if axis == 0 else ()))
+    da = da.reshape(a.shape)
+    assert np.allclose(da, _repeat_backward_by_loops(grad, a.shape, repeats, axis), rtol=0, atol=1e-13)
+    assert abs(float(np.sum(out * grad)) - float(np.sum(a * da))) <= 1e-12 * max(1.0, float(np.sum(np.abs(out * grad))))
