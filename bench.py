@@ -57,6 +57,8 @@ WORKLOADS = {
     "elem5": dict(kind="elem", dtype="f32", seed=1007, x=(8, 32, 32, 64, 64)),
     # batch normalisation (scaled and shifted) of a tensor of conv3a's output size
     "bn3a": dict(kind="bn", dtype="f32", seed=1008, x=(128, 64, 56, 56), eps=1e-5),
+    # matrix product on the convolution kernels: one dense layer's three products
+    "mm4k": dict(kind="matmul", dtype="f32", seed=1011, M=4096, K=4096, N=4096),
     # repeat: twofold nearest-neighbour upsampling of the rows of a tensor of pool5's input size
     # (forward and gradient), and then of its columns
     "rep5": dict(kind="repeat", dtype="f32", seed=1009, x=(8, 32, 32, 64, 64), repeats=2, axes=(-2, -1)),
@@ -89,6 +91,8 @@ def describe(name):
     wl = WORKLOADS[name]
     if wl["kind"] == "elem":
         return f"{name}: relu + multiply + sum {wl['dtype']} x{wl['x']} fwd+bwd (7 kernels, 16 |x| bytes)"
+    if wl["kind"] == "matmul":
+        return f"{name}: matmul {wl['dtype']} ({wl['M']},{wl['K']}) @ ({wl['K']},{wl['N']}): product + both gradients"
     if wl["kind"] == "repeat":
         return f"{name}: repeat {wl['dtype']} x{wl['x']} repeats={wl['repeats']} along axis {wl['axes'][0]}, then along axis {wl['axes'][1]}, fwd+bwd each"
     if wl["kind"] == "window":
@@ -133,6 +137,19 @@ class Step:
             self.dx = _device.DeviceBuffer(x.nbytes)
             self.dw = _device.DeviceBuffer(w.nbytes)
             per_pass = conv_flops_per_pass(wl)
+            self.work = {"conv_fwd": per_pass, "conv_dgrad": per_pass, "conv_wgrad": per_pass}
+            self.total_work = 3 * per_pass
+            self.unit, self.bound, self.peak = "TFLOP/s", "mfma", PEAK_TFLOPS[wl["dtype"]]
+            self.scale = 1e-12
+        elif wl["kind"] == "matmul":
+            M, K, N = wl["M"], wl["K"], wl["N"]
+            a = (rng.standard_normal((M, K)) * K ** -0.5).astype(dt)
+            x = rng.standard_normal((K, N)).astype(dt)
+            g = rng.standard_normal((M, N)).astype(dt)
+            self.w, self.x, self.g = resident(a), resident(x), resident(g)
+            self.out, self.dx, self.dw = (_device.DeviceBuffer(n * item) for n in (M * N, K * N, M * K))
+            self.code, self.dims = _hip.dtype_code(dt), (1, M, K, N)
+            per_pass = 2.0 * M * K * N
             self.work = {"conv_fwd": per_pass, "conv_dgrad": per_pass, "conv_wgrad": per_pass}
             self.total_work = 3 * per_pass
             self.unit, self.bound, self.peak = "TFLOP/s", "mfma", PEAK_TFLOPS[wl["dtype"]]
@@ -221,6 +238,11 @@ class Step:
             check(lib.mg_multiply(c, n, self.dx.ptr, self.g.ptr, self.out.ptr))  # d (a*b) / d a
             check(lib.mg_multiply(c, n, self.dx.ptr, self.x.ptr, self.out.ptr))  # d (a*b) / d b
             check(lib.mg_relu_bwd(c, n, self.x.ptr, self.dx.ptr, self.out.ptr))
+            return
+        if self.wl["kind"] == "matmul":
+            check(lib.mg_matmul(self.code, *self.dims, self.w.ptr, self.x.ptr, self.out.ptr))
+            check(lib.mg_matmul_dx(self.code, *self.dims, self.g.ptr, self.w.ptr, self.dx.ptr))
+            check(lib.mg_matmul_da(self.code, *self.dims, self.g.ptr, self.x.ptr, self.dw.ptr))
             return
         if self.wl["kind"] == "repeat":
             for outer, n, inner, r, total in self.geometry:
@@ -335,6 +357,19 @@ def run_cpu_baseline(name, min_seconds=10.0, max_reps=200):
 
         work, scale, unit = 3 * conv_flops_per_pass(wl), 1e-12, "TFLOP/s"
         what = "fwd+dx+dw"
+    elif wl["kind"] == "matmul":
+        M, K, N = wl["M"], wl["K"], wl["N"]
+        a = (rng.standard_normal((M, K)) * K ** -0.5).astype(dt)
+        x = rng.standard_normal((K, N)).astype(dt)
+        g = rng.standard_normal((M, N)).astype(dt)
+
+        def once():
+            ora.matmul_forward(a, x)
+            ora.matmul_backward(g, a, x, 0)
+            ora.matmul_backward(g, a, x, 1)
+
+        work, scale, unit = 6.0 * M * K * N, 1e-12, "TFLOP/s"
+        what = "product and both gradients (three BLAS sgemm calls)"
     elif wl["kind"] == "repeat":
         x = rng.standard_normal(wl["x"]).astype(dt)
         g = rng.standard_normal((*wl["x"][:-1], wl["x"][-1] * wl["repeats"])).astype(dt)
@@ -403,7 +438,7 @@ def run_cpu_baseline(name, min_seconds=10.0, max_reps=200):
     return {
         "value": float(reps * work * scale / elapsed),
         "unit": unit,
-        "cores": blas_threads() if wl["kind"] == "conv" else 1,
+        "cores": blas_threads() if wl["kind"] in ("conv", "matmul") else 1,
         "kind": "port",
         "sample": f"the whole workload ({what}), {reps} repetition(s), {elapsed:.1f} s of host time",
         "numpy": np.__version__,
@@ -418,7 +453,7 @@ def run_dropin(name, steps=5):
 
     wl, dt = WORKLOADS[name], NP_DTYPE[WORKLOADS[name]["dtype"]]
     rng = np.random.default_rng(wl["seed"])
-    x = rng.standard_normal(wl["x"]).astype(dt)
+    x = rng.standard_normal(wl["x"]).astype(dt) if "x" in wl else None
     if wl["kind"] == "conv":
         w = (rng.standard_normal(wl["w"]) * wl["wscale"]).astype(dt)
         g = rng.standard_normal((wl["x"][0], wl["w"][0], *conv_grid(wl))).astype(dt)
@@ -433,6 +468,17 @@ def run_dropin(name, steps=5):
             out.backward(g)
 
         work, scale, unit = 3 * conv_flops_per_pass(wl), 1e-12, "TFLOP/s"
+    elif wl["kind"] == "matmul":
+        M, K, N = wl["M"], wl["K"], wl["N"]
+        a = (rng.standard_normal((M, K)) * K ** -0.5).astype(dt)
+        x = rng.standard_normal((K, N)).astype(dt)
+        g = rng.standard_normal((M, N)).astype(dt)
+
+        def once():
+            at, xt = mg.Tensor(a, copy=False), mg.Tensor(x, copy=False)
+            (at @ xt).backward(g)
+
+        work, scale, unit = 6.0 * M * K * N, 1e-12, "TFLOP/s"
     elif wl["kind"] == "repeat":
         g = rng.standard_normal((*wl["x"][:-1], wl["x"][-1] * wl["repeats"])).astype(dt)
 
@@ -563,7 +609,7 @@ def main():
     line = {
         "metric": {"conv": "conv_nd fwd+bwd TFLOP/s", "pool": "max_pool fwd+bwd GB/s",
                    "elem": "relu+multiply+sum fwd+bwd GB/s", "bn": "batchnorm fwd+bwd GB/s",
-                   "repeat": "repeat fwd+bwd GB/s", "window": "sliding-window copy GB/s"}[wl["kind"]],
+                   "repeat": "repeat fwd+bwd GB/s", "matmul": "matmul fwd+bwd TFLOP/s", "window": "sliding-window copy GB/s"}[wl["kind"]],
         "value": res["value"],
         "unit": res["unit"],
         "n_gpus": 1,

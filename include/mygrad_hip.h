@@ -216,6 +216,23 @@ int mg_batchnorm_fwd(const mg_bn_desc *desc, const void *x, const void *gamma, c
 int mg_batchnorm_bwd(const mg_bn_desc *desc, const void *x, const void *grad, const void *gamma, const void *mean,
                      const void *var, void *dx, void *dgamma, void *dbeta);
 
+/* ---- matrix product ---- */
+
+/* out[b] = a @ x[b], a:(M, K) shared by the batch, x:(batch, K, N), out:(batch, M, N), all
+ * C-contiguous.  Runs as the convolution of x with M one-tap filters (the same implicit-GEMM
+ * kernels; the reduction has length K).  A stack of left operands times one right operand,
+ * (batch, M, K) @ (K, N), is the same call with batch = 1 and M := batch * M.
+ * Replaces np.matmul in MatMul.__call__, src/mygrad/math/misc/ops.py:91-93. */
+int mg_matmul(int dtype, int64_t batch, int64_t M, int64_t K, int64_t N, const void *a, const void *x, void *out);
+
+/* da = sum_b grad[b] @ x[b]^T (M, K): MatMul.backward_var index 0 (np.matmul(grad,
+ * b.swapaxes(-1, -2)) summed over the broadcast batch, ops.py:107-114); fixed summation order. */
+int mg_matmul_da(int dtype, int64_t batch, int64_t M, int64_t K, int64_t N, const void *grad, const void *x, void *da);
+
+/* dx[b] = a^T @ grad[b] (batch, K, N): MatMul.backward_var index 1 (np.matmul(a.swapaxes(-1, -2),
+ * grad), ops.py:116-124). */
+int mg_matmul_dx(int dtype, int64_t batch, int64_t M, int64_t K, int64_t N, const void *grad, const void *a, void *dx);
+
 /* ---- repeat and the window view ---- */
 
 /* out[o, j, i] = a[o, src(j), i] with a seen as (outer, n, inner) around the repeated axis

@@ -18,8 +18,9 @@ from .errors import InvalidBackprop, InvalidGradient, SkipGradient
 from .nnet.layers.utils import sliding_window_copy, sliding_window_view
 from .operation_base import Operation
 from .tensor_base import Tensor, asarray, tensor
-from .math import multiply, sum  # noqa: A004  (after tensor_base: the ops import Tensor)
+from .math import matmul, multiply, sum  # noqa: A004  (after tensor_base: the ops import Tensor)
 from .tensor_manip import repeat
+from ._io import load, save
 
 execute_op = Tensor._op
 
@@ -35,8 +36,11 @@ __all__ = [
     "sliding_window_view",
     "sliding_window_copy",
     "multiply",
+    "matmul",
     "sum",
     "repeat",
+    "save",
+    "load",
     "nnet",
     "InvalidBackprop",
     "InvalidGradient",

@@ -30,6 +30,7 @@ __all__ = [
     "to_device",
     "attach",
     "attach_transient",
+    "hold_gradient",
     "evict",
     "drop_transients",
     "lookup",
@@ -161,6 +162,20 @@ def attach(arr, buf):
 def attach_transient(arr, buf):
     """Record ``buf`` as the device copy of a gradient array until backward() ends."""
     _transient[_key(arr)] = buf
+
+
+def hold_gradient(arr):
+    """Upload ``arr`` now and keep the copy until backward() ends: an operation with several
+    non-constant inputs is asked for one gradient per input with the same incoming ``arr``,
+    which would otherwise cross PCIe once per request."""
+    if not isinstance(arr, np.ndarray) or not arr.flags["C_CONTIGUOUS"] or arr.size == 0:
+        return
+    if arr.dtype not in (np.float32, np.float64) or lookup(arr) is not None:
+        return
+    buf = DeviceBuffer(arr.nbytes)
+    buf.upload(arr)
+    stats["uploads"] += 1
+    attach_transient(arr, buf)
 
 
 def evict(arr):

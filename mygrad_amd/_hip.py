@@ -149,6 +149,9 @@ _SIGNATURES = {
     "mg_fill_from": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
     "mg_batchnorm_fwd": [ctypes.POINTER(BnDesc), _vp, _vp, _vp, _vp, _vp, _vp],
     "mg_batchnorm_bwd": [ctypes.POINTER(BnDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
+    "mg_matmul": [ctypes.c_int] + [ctypes.c_int64] * 4 + [_vp, _vp, _vp],
+    "mg_matmul_da": [ctypes.c_int] + [ctypes.c_int64] * 4 + [_vp, _vp, _vp],
+    "mg_matmul_dx": [ctypes.c_int] + [ctypes.c_int64] * 4 + [_vp, _vp, _vp],
     "mg_repeat_fwd": [ctypes.c_int] + [ctypes.c_int64] * 5 + [_vp, _vp, _vp],
     "mg_repeat_bwd": [ctypes.c_int] + [ctypes.c_int64] * 5 + [_vp, _vp, _vp],
     "mg_window_gather": [ctypes.POINTER(WindowDesc), _vp, _vp],

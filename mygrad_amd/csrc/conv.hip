@@ -1316,4 +1316,44 @@ int mg_conv_wgrad(const mg_conv_desc *desc, const void *grad, const void *x, voi
                            : conv_wgrad_impl<double>(g, *pl, grad, x, dw);
 }
 
+// ---- matrix product: a convolution with a window of one element -------------------------
+//
+// out[b] = a @ x[b] with a:(M, K) shared by the batch and x:(batch, K, N) is the convolution of
+// x (batch entries, K channels, N positions) with M filters of one tap: the same implicit-GEMM
+// kernels with a reduction of length K.  Its two gradients are the convolution's.
+namespace {
+int matmul_desc(const char *who, int dtype, int64_t batch, int64_t M, int64_t K, int64_t N, mg_conv_desc *d) {
+  if (batch < 1 || M < 1 || K < 1 || N < 1)
+    return fail(MG_ERR_BAD_ARG, "%s: batch=%lld M=%lld K=%lld N=%lld must be positive", who, (long long)batch, (long long)M,
+                (long long)K, (long long)N);
+  *d = mg_conv_desc{};
+  d->dtype = dtype;
+  d->nd = 1;
+  d->N = batch;
+  d->C = K;
+  d->F = M;
+  for (int k = 0; k < MG_MAX_ND; ++k) d->X[k] = d->W[k] = d->G[k] = d->stride[k] = d->dil[k] = 1;
+  d->X[MG_MAX_ND - 1] = d->G[MG_MAX_ND - 1] = N;
+  return MG_OK;
+}
+}  // namespace
+
+int mg_matmul(int dtype, int64_t batch, int64_t M, int64_t K, int64_t N, const void *a, const void *x, void *out) {
+  mg_conv_desc d;
+  if (int rc = matmul_desc("mg_matmul", dtype, batch, M, K, N, &d)) return rc;
+  return mg_conv_fwd(&d, x, a, out);
+}
+
+int mg_matmul_da(int dtype, int64_t batch, int64_t M, int64_t K, int64_t N, const void *grad, const void *x, void *da) {
+  mg_conv_desc d;
+  if (int rc = matmul_desc("mg_matmul_da", dtype, batch, M, K, N, &d)) return rc;
+  return mg_conv_wgrad(&d, grad, x, da);
+}
+
+int mg_matmul_dx(int dtype, int64_t batch, int64_t M, int64_t K, int64_t N, const void *grad, const void *a, void *dx) {
+  mg_conv_desc d;
+  if (int rc = matmul_desc("mg_matmul_dx", dtype, batch, M, K, N, &d)) return rc;
+  return mg_conv_dgrad(&d, grad, a, dx);
+}
+
 }  // extern "C"

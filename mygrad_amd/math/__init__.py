@@ -1,7 +1,8 @@
-"""Element-wise and sequential operations that sit either side of ``conv_nd`` /
-``max_pool`` in a chain and run on the device: ``multiply`` and ``sum``."""
+"""Element-wise, sequential and matrix operations that sit either side of ``conv_nd`` /
+``max_pool`` in a chain and run on the device: ``multiply``, ``sum`` and ``matmul``."""
 
 from .arithmetic.funcs import multiply
+from .misc.funcs import matmul
 from .sequential.funcs import sum  # noqa: A004 (same name as the reference's mygrad.sum)
 
-__all__ = ["multiply", "sum"]
+__all__ = ["multiply", "matmul", "sum"]

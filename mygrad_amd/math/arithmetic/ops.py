@@ -36,6 +36,8 @@ def device_multiply(a, b, dtype):
 class Multiply(Operation):
     """``f(a, b) -> a * b`` element-wise."""
 
+    gradient_on_device = True
+
     def __call__(self, a, b):
         self.variables = (a, b)
         dtype = _same_shape_floats("multiply", a.data, b.data)

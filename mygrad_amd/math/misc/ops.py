@@ -1,0 +1,110 @@
+"""``MatMul`` on the MI355X (reference: ``mygrad/math/misc/ops.py:91-126``).
+
+A matrix product is a convolution whose window has one element: ``a @ b`` with ``a:(M, K)``
+and ``b:(K, N)`` is the convolution of ``b`` -- K channels, N positions -- with M filters, and
+its two gradients are the convolution's.  The operation therefore runs on the convolution's
+implicit-GEMM kernels (``mg_matmul*`` in ``libmygrad_hip.so``) with no kernel of its own.
+
+Operand patterns that run: both operands at most 2-D (vectors are promoted like
+``np.matmul`` does); one operand a stack and the other at most 2-D (one launch: the stack is
+the convolution's batch, or folds into the rows of the left operand); two stacks of the same
+batch shape (one launch per matrix pair).  Stacks that broadcast against each other raise
+``NotImplementedError`` (there is no CPU fallback)."""
+
+import numpy as np
+
+from ... import _device, _hip
+from ...operation_base import Operation
+
+__all__ = ["MatMul"]
+
+
+def _prod(shape):
+    return int(np.prod(shape, dtype=np.int64))
+
+
+class MatMul(Operation):
+    gradient_on_device = True
+
+    def __call__(self, a, b):
+        self.variables = (a, b)
+        x, y = a.data, b.data
+        # NumPy's own checks (scalars, core dimensions, batch broadcasting) on operands
+        # without rows and columns: the same errors, the batch shape of the result, no arithmetic
+        probe = np.matmul(
+            np.empty(x.shape if x.ndim < 2 else (*x.shape[:-2], 0, x.shape[-1]), dtype=np.int8),
+            np.empty(y.shape if y.ndim < 2 else (*y.shape[:-2], y.shape[-2], 0), dtype=np.int8),
+        )
+        dtype = np.dtype(np.result_type(x, y))
+        if dtype not in (np.float32, np.float64):
+            raise TypeError(f"matmul runs on the GPU in float32 or float64, got {x.dtype} and {y.dtype} (there is no CPU fallback)")
+
+        x2 = x if x.ndim > 1 else x[None, :]
+        y2 = y if y.ndim > 1 else y[:, None]
+        M, K, N = x2.shape[-2], x2.shape[-1], y2.shape[-1]
+        stack_a, stack_b = x2.shape[:-2], y2.shape[:-2]
+        if stack_a and stack_b and stack_a != stack_b:
+            raise NotImplementedError(
+                f"matmul on the GPU does not broadcast two stacks against each other, got {x.shape} and {y.shape} "
+                "(no CPU fallback)"
+            )
+        batch_shape = stack_a or stack_b
+        out_shape = batch_shape + (() if x.ndim == 1 else (M,)) + (() if y.ndim == 1 else (N,))
+        assert len(out_shape) == probe.ndim
+        self._dtype, self._dims = dtype, (M, K, N)
+        self._stacks = (stack_a, stack_b)
+        self._promoted = (x2.shape, y2.shape)
+        if 0 in out_shape or K == 0:
+            return np.zeros(out_shape, dtype=dtype)
+
+        ab, bb = _device.to_device(x, dtype), _device.to_device(y, dtype)
+        ob = _device.DeviceBuffer(max(_prod(out_shape) * dtype.itemsize, 16))
+        self._launch("mg_matmul", ab, bb, ob, a_like=0, x_like=1, out_like=2)
+        out = _device.download(ob, out_shape, dtype)
+        _device.attach(out, ob)
+        return out
+
+    def _launch(self, entry, first, second, result, a_like, x_like, out_like):
+        """Call ``entry(dtype, batch, M, K, N, first, second, result)`` once, or once per
+        matrix pair for two stacks.  ``*_like`` say which of (a, b, out) each buffer has the
+        layout of (0: a, 1: b, 2: out) so that the per-pair offsets can be formed."""
+        M, K, N = self._dims
+        stack_a, stack_b = self._stacks
+        code, item = _hip.dtype_code(self._dtype), self._dtype.itemsize
+        fn = getattr(_hip.lib(), entry)
+        if not stack_a:
+            _hip.check(fn(code, _prod(stack_b), M, K, N, first.ptr, second.ptr, result.ptr))
+        elif not stack_b:
+            _hip.check(fn(code, 1, _prod(stack_a) * M, K, N, first.ptr, second.ptr, result.ptr))
+        else:
+            per = (M * K * item, K * N * item, M * N * item)
+            for i in range(_prod(stack_a)):
+                _hip.check(
+                    fn(code, 1, M, K, N, first.ptr + i * per[a_like], second.ptr + i * per[x_like], result.ptr + i * per[out_like])
+                )
+
+    def backward_var(self, grad, index, **kwargs):
+        a, b = self.variables
+        dtype = self._dtype
+        var = (a, b)[index].data
+        if var.size == 0 or grad.size == 0:
+            return np.zeros(var.shape, dtype=dtype)
+        M, K, N = self._dims
+        stack_a, stack_b = self._stacks
+        batch = _prod(stack_a or stack_b)
+        if grad.size != batch * M * N:
+            raise ValueError(f"matmul backward: gradient of shape {grad.shape} does not match the product")
+        gb = _device.to_device(grad, dtype)
+        if index == 0:
+            # d a = grad @ b^T, summed over a batch that `a` was shared by (ops.py:107-114)
+            other = _device.to_device(b.data, dtype)
+            ob = _device.DeviceBuffer(max(var.size * dtype.itemsize, 16))
+            self._launch("mg_matmul_da", gb, other, ob, a_like=2, x_like=1, out_like=0)
+        else:
+            # d b = a^T @ grad, summed over a stack of left operands that `b` was shared by (ops.py:116-124)
+            other = _device.to_device(a.data, dtype)
+            ob = _device.DeviceBuffer(max(var.size * dtype.itemsize, 16))
+            self._launch("mg_matmul_dx", gb, other, ob, a_like=2, x_like=0, out_like=1)
+        out = _device.download(ob, var.shape, dtype)
+        _device.attach_transient(out, ob)
+        return out

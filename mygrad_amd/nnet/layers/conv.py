@@ -49,6 +49,8 @@ class ConvND(Operation):
     ``(N, C, X0, ...) * (F, C, W0, ...) -> (N, F, G0, ...)``
     """
 
+    gradient_on_device = True
+
     def __call__(self, x, w, *, stride, padding=0, dilation=1):
         self.variables = (x, w)
         xd, wd = x.data, w.data

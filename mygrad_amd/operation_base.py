@@ -26,6 +26,10 @@ class Operation(ABC):
 
     variables = ()
 
+    # True for operations whose backward_var hands the incoming gradient to a device kernel
+    # for more than one input: backward() then uploads it once for all of them
+    gradient_on_device = False
+
     @abstractmethod
     def __call__(self, *input_vars, **kwargs):
         """Forward pass; must bind the tuple of input tensors to ``self.variables``
@@ -41,6 +45,8 @@ class Operation(ABC):
     def backward(self, grad, **kwargs):
         """Back-propagate ``grad`` to every non-constant input
         (reference: operation_base.py:162-228)."""
+        if self.gradient_on_device and sum(not var.constant for var in self.variables) > 1:
+            _device.hold_gradient(grad)
         for index, var in enumerate(self.variables):
             if var.constant:
                 continue

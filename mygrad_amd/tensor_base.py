@@ -134,6 +134,16 @@ class Tensor:
 
         return self._op(Multiply, other, self)
 
+    def __matmul__(self, other):
+        from .math.misc.ops import MatMul
+
+        return self._op(MatMul, self, other)
+
+    def __rmatmul__(self, other):
+        from .math.misc.ops import MatMul
+
+        return self._op(MatMul, other, self)
+
     def sum(self, axis=None, keepdims=False, *, constant=None):
         from .math.sequential.ops import Sum
 

@@ -39,6 +39,10 @@ Pinning (what holds each function to the reference without importing it):
                    central differences of ``sum(grad * batchnorm(x))`` in x, gamma
                    and beta; the invariants ``sum_c(dx) == 0`` and, at ``eps == 0``,
                    ``sum_c(dx * x_norm) == 0``
+  matmul_forward   a single call of ``np.matmul`` (what the reference's ufunc calls); the
+                   reference's docstring vectors; triple loops on small operands
+  matmul_backward  triple loops; the adjoint identities
+                   ``<a @ b, g> == <a, da> == <b, db>`` (the product is linear in each)
   repeat_forward   a single call of ``np.repeat`` (what the reference calls); the
                    reference's four docstring vectors
   repeat_backward  element-by-element loops; the adjoint identity
@@ -67,6 +71,8 @@ __all__ = [
     "batchnorm_backward",
     "repeat_forward",
     "repeat_backward",
+    "matmul_forward",
+    "matmul_backward",
     "pool_out_shape",
     "pool_forward",
     "pool_backward",
@@ -451,3 +457,48 @@ def repeat_backward(grad, a, repeats, axis=None):
     indices = np.repeat(indices, repeats=repeats, axis=axis)
     np.add.at(out, indices.ravel(), grad.ravel())  # :70
     return out.reshape(a.shape)
+
+
+# ------------------------------------------------------------------ matmul
+def matmul_forward(a, b):
+    """MatMul.__call__: ``np.matmul`` (src/mygrad/math/misc/ops.py:91-93)."""
+    return np.matmul(np.asarray(a), np.asarray(b))
+
+
+def _sum_to(arr, shape):
+    """Undo broadcasting: what the reference's BinaryUfunc.backward does to a gradient whose
+    shape exceeds its variable's (src/mygrad/operation_base.py:262-330, reduce_broadcast)."""
+    arr = np.asarray(arr)
+    extra = arr.ndim - len(shape)
+    if extra:
+        arr = arr.sum(axis=tuple(range(extra)))
+    keep = tuple(i for i, n in enumerate(shape) if n == 1 and arr.shape[i] != 1)
+    if keep:
+        arr = arr.sum(axis=keep, keepdims=True)
+    return arr
+
+
+def matmul_backward(grad, a, b, index):
+    """MatMul.backward_var (ops.py:95-126), reduced to the operand's shape."""
+    a, b, grad = np.asarray(a), np.asarray(b), np.asarray(grad)
+    if a.ndim == 1 and b.ndim == 1:  # :101-105
+        return grad * b if index == 0 else grad * a
+    if index == 0:
+        if b.ndim > 1:  # :108-111
+            if a.ndim == 1:
+                grad = np.expand_dims(grad, -2)
+            out = np.matmul(grad, b.swapaxes(-1, -2))
+        else:  # :112-113
+            out = np.expand_dims(grad, -1) * b
+        if a.ndim == 1 and out.ndim > 1:
+            out = out.reshape(*out.shape[:-2], out.shape[-1])
+        return _sum_to(out, a.shape)
+    if a.ndim > 1:  # :117-122
+        if b.ndim == 1:
+            grad = np.expand_dims(grad, -1)
+        out = np.matmul(a.swapaxes(-1, -2), grad)
+        if b.ndim == 1:
+            out = out.squeeze(-1)
+    else:  # :123-124
+        out = a[:, np.newaxis] * np.expand_dims(grad, -2)
+    return _sum_to(out, b.shape)

@@ -235,3 +235,31 @@ def window_gather(x, window, step, dilation):
     ob = _device.DeviceBuffer(max(int(np.prod(out_shape, dtype=np.int64)) * x.itemsize, 16))
     _hip.check(_hip.lib().mg_window_gather(desc, xb.ptr, ob.ptr))
     return _down(ob, out_shape, x.dtype)
+
+
+# ----------------------------------------------------------------- matrix product
+def matmul(a, x):
+    """a:(M, K) @ x:(batch, K, N) -> (batch, M, N) through mg_matmul."""
+    batch, K, N = x.shape
+    M = a.shape[0]
+    ab, xb = _up(a), _up(x)
+    ob = _device.DeviceBuffer(max(batch * M * N * a.itemsize, 16))
+    _hip.check(_hip.lib().mg_matmul(_hip.dtype_code(a.dtype), batch, M, K, N, ab.ptr, xb.ptr, ob.ptr))
+    return _down(ob, (batch, M, N), a.dtype)
+
+
+def matmul_da(grad, x, M):
+    batch, K, N = x.shape
+    gb, xb = _up(grad), _up(x)
+    ob = _device.DeviceBuffer(max(M * K * x.itemsize, 16))
+    _hip.check(_hip.lib().mg_matmul_da(_hip.dtype_code(x.dtype), batch, M, K, N, gb.ptr, xb.ptr, ob.ptr))
+    return _down(ob, (M, K), x.dtype)
+
+
+def matmul_dx(grad, a):
+    batch, M, N = grad.shape
+    K = a.shape[1]
+    gb, ab = _up(grad), _up(a)
+    ob = _device.DeviceBuffer(max(batch * K * N * a.itemsize, 16))
+    _hip.check(_hip.lib().mg_matmul_dx(_hip.dtype_code(a.dtype), batch, M, K, N, gb.ptr, ab.ptr, ob.ptr))
+    return _down(ob, (batch, K, N), a.dtype)

@@ -312,3 +312,32 @@ def test_no_autodiff_and_mem_guard_switches():
         assert x.data.flags.writeable and out.creator is not None
         out.backward()
     assert np.array_equal(x.grad, [1.0])
+
+
+def test_save_and_load_round_trip(tmp_path):
+    import io
+
+    import mygrad_amd as mg
+
+    x = mg.Tensor(np.arange(10.0))
+    buf = io.BytesIO()
+    mg.save(buf, x)
+    buf.seek(0)
+    back = mg.load(buf)
+    assert isinstance(back, mg.Tensor) and np.array_equal(back.data, x.data) and back.grad is None
+
+    x.backward(np.arange(10.0) * 2)  # a leaf: the seed becomes its gradient
+    path = tmp_path / "with_grad"
+    mg.save(path, x)
+    back = mg.load(str(path) + ".npz")
+    assert np.array_equal(back.data, x.data) and np.array_equal(back.grad, np.arange(10.0) * 2)
+    with np.load(str(path) + ".npz") as archive:  # the reference's layout
+        assert sorted(archive.files) == ["data", "grad"]
+
+    ints = mg.Tensor(np.arange(4))
+    buf = io.BytesIO()
+    mg.save(buf, ints)
+    buf.seek(0)
+    assert mg.load(buf).dtype == ints.dtype
+    with pytest.raises(TypeError):
+        mg.save(io.BytesIO(), np.arange(3.0))

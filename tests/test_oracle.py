@@ -465,3 +465,64 @@ def test_repeat_backward_by_loops_and_adjoint(shape, repeats, axis):
     da = da.reshape(a.shape)
     assert np.allclose(da, _repeat_backward_by_loops(grad, a.shape, repeats, axis), rtol=0, atol=1e-13)
     assert abs(float(np.sum(out * grad)) - float(np.sum(a * da))) <= 1e-12 * max(1.0, float(np.sum(np.abs(out * grad))))
+
+
+# ----------------------------------------------------------------- matmul
+def test_matmul_reference_vectors(kats):
+    for case in kats["matmul"]:
+        if "a" in case:
+            a, b = np.array(case["a"], dtype=float), np.array(case["b"], dtype=float)
+            assert np.array_equal(ora.matmul_forward(a, b), np.array(case["out"], dtype=float)), case["source"]
+            if "da" in case:
+                g = np.ones_like(ora.matmul_forward(a, b))
+                assert np.array_equal(ora.matmul_backward(g, a, b, 0), case["da"])
+                assert np.array_equal(ora.matmul_backward(g, a, b, 1), case["db"])
+        else:
+            out = ora.matmul_forward(np.zeros(case["a_shape"]), np.zeros(case["b_shape"]))
+            assert list(out.shape) == case["out_shape"]
+
+
+MATMUL_SHAPES = [
+    ((3, 4), (4, 5)),
+    ((4,), (4, 5)),
+    ((3, 4), (4,)),
+    ((4,), (4,)),
+    ((2, 3, 4), (4, 5)),
+    ((3, 4), (2, 4, 5)),
+    ((2, 3, 4), (2, 4, 5)),
+    ((4,), (2, 3, 4, 5)),
+    ((2, 3, 4), (4,)),
+    ((2, 1, 3, 4), (2, 4, 5)),  # stacks that broadcast against each other
+]
+
+
+@pytest.mark.parametrize("sa, sb", MATMUL_SHAPES)
+def test_matmul_backward_by_loops_and_adjoint(sa, sb):
+    rng = np.random.default_rng([len(sa), len(sb), int(np.prod(sa)), int(np.prod(sb))])
+    a, b = rng.standard_normal(sa), rng.standard_normal(sb)
+    out = ora.matmul_forward(a, b)
+    g = rng.standard_normal(out.shape)
+    da, db = ora.matmul_backward(g, a, b, 0), ora.matmul_backward(g, a, b, 1)
+    assert da.shape == a.shape and db.shape == b.shape
+    inner = float(np.sum(out * g))
+    assert abs(inner - float(np.sum(a * da))) <= 1e-12 * max(1.0, abs(inner))
+    assert abs(inner - float(np.sum(b * db))) <= 1e-12 * max(1.0, abs(inner))
+    # definition: out[..., i, k] = sum_j a[..., i, j] * b[..., j, k] on promoted operands
+    a2 = a if a.ndim > 1 else a[None, :]
+    b2 = b if b.ndim > 1 else b[:, None]
+    want = np.einsum("...ij,...jk->...ik", a2, b2)
+    if a.ndim == 1:
+        want = want[..., 0, :]
+    if b.ndim == 1:
+        want = want[..., 0]
+    assert np.allclose(out, want, rtol=1e-13, atol=1e-13)
+    # d out[..., i, k] / d a[i, j] = b[j, k]: loops on the 2-D case
+    if a.ndim == 2 and b.ndim == 2:
+        loop_da = np.zeros_like(a)
+        loop_db = np.zeros_like(b)
+        for i in range(a.shape[0]):
+            for j in range(a.shape[1]):
+                for k in range(b.shape[1]):
+                    loop_da[i, j] += g[i, k] * b[j, k]
+                    loop_db[j, k] += a[i, j] * g[i, k]
+        assert np.allclose(da, loop_da, atol=1e-13) and np.allclose(db, loop_db, atol=1e-13)
