@@ -1,4 +1,5 @@
-from typing import Optional, Sequence, Union
+"""``repeat``: the user-facing function over the ``Repeat`` operation (reference:
+``mygrad/tensor_manip/tiling/funcs.py``, itself modelled on ``numpy.repeat``)."""
 
 from ...tensor_base import Tensor
 from .ops import Repeat
@@ -6,47 +7,25 @@ from .ops import Repeat
 __all__ = ["repeat"]
 
 
-def repeat(a, repeats: Union[int, Sequence[int]], axis: Optional[int] = None, *, constant: Optional[bool] = None) -> Tensor:
-    """
-    Repeat elements of a tensor (the counterpart of ``mygrad.repeat`` / ``numpy.repeat``).
+def repeat(a, repeats, axis=None, *, constant=None):
+    """Copy every entry of ``a`` along ``axis`` a given number of times, on the GPU.
 
-    Parameters
-    ----------
-    a : ArrayLike
-        Input tensor.
+    ``repeats`` is one count for all entries or one count per entry of the axis (zeros
+    allowed); with ``axis=None`` the input is read as flattened and the result is 1-D, as
+    with ``numpy.repeat``.  Any dtype of 1, 2, 4 or 8 bytes is accepted (integer tensors come
+    back constant); the gradient -- each input entry collects the gradient of its copies --
+    is defined for float32 / float64.
 
-    repeats : Union[int, Sequence[int]]
-        The number of repetitions for each element. ``repeats``
-        is broadcasted to fit the shape of the given axis.
-
-    axis : Optional[int]
-        The axis along which to repeat values. By default, use the
-        flattened input array, and return a flat output tensor.
-
-    constant : Optional[bool]
-        If ``True``, the result is a constant and does not take part in
-        back-propagation. Integer-type tensors must be constant.
-
-    Returns
-    -------
-    repeated_tensor : Tensor
-        Output tensor which has the same shape as `a`, except along
-        the given axis.
-
-    Examples
-    --------
     >>> import mygrad_amd as mg
-    >>> mg.repeat(3, 4)
-    Tensor([3, 3, 3, 3])
-    >>> x = mg.Tensor([[1, 2], [3, 4]])
-    >>> mg.repeat(x, 2)
-    Tensor([1, 1, 2, 2, 3, 3, 4, 4])
-    >>> mg.repeat(x, 3, axis=1)
-    Tensor([[1, 1, 1, 2, 2, 2],
-            [3, 3, 3, 4, 4, 4]])
-    >>> mg.repeat(x, [1, 2], axis=0)
-    Tensor([[1, 2],
-            [3, 4],
-            [3, 4]])
+    >>> x = mg.Tensor([[1., 2.], [3., 4.]])
+    >>> y = mg.repeat(x, [1, 2], axis=0)
+    >>> y.data
+    array([[1., 2.],
+           [3., 4.],
+           [3., 4.]])
+    >>> y.backward()
+    >>> x.grad
+    array([[1., 1.],
+           [2., 2.]])
     """
     return Tensor._op(Repeat, a, op_args=(repeats, axis), constant=constant)
