@@ -111,8 +111,6 @@ def test_matmul_through_the_tensor_api(sa, sb, dtype):
 
 def test_reference_vectors_operator_and_errors(kats):
     import mygrad_amd as mg
-    from mygrad_amd import _graph
-
     for case in kats["matmul"]:
         if "a" not in case:
             out = mg.matmul(np.zeros(case["a_shape"]), np.zeros(case["b_shape"]))
@@ -126,7 +124,6 @@ def test_reference_vectors_operator_and_errors(kats):
             assert np.array_equal(a.grad, case["da"]) and np.array_equal(b.grad, case["db"])
     x = mg.Tensor(np.eye(3))
     assert np.array_equal((np.arange(9.0).reshape(3, 3) @ x).data, np.arange(9.0).reshape(3, 3))  # __rmatmul__
-    assert _graph.held_count() == 0 or True
 
     with pytest.raises(ValueError):
         mg.matmul(mg.Tensor(np.ones((2, 3))), 3.0)  # scalars are not allowed
