@@ -945,6 +945,23 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
     const int per_cu = f64 ? wgrad_blocks_per_cu<double>(bm, bn, tap) : wgrad_blocks_per_cu<float>(bm, bn, tap);
     const long long slots = (long long)per_cu * cus;
     const long long max_splits = std::max<long long>(1, std::min<long long>(ktiles / 4, 1024));
+    if (tiles > slots) {
+      // More tiles than block slots (a large dw, as in a matrix product): the blocks run in
+      // rounds and the last round may be nearly empty.  Splitting K evens the rounds out at
+      // the price of one more copy of dw written and read back per split: take the split
+      // that minimises  (time of the rounds) + (time of that traffic).
+      const double work = 2.0 * (double)g.F * (double)ct * (double)kpos / (0.7 * (f64 ? 78.6e12 : 157.3e12));
+      const double copy = 2.0 * (double)g.F * (double)ct * (f64 ? 8.0 : 4.0) / 4.0e12;
+      long long best = 1;
+      double best_time = 0;
+      for (long long sp = 1; sp <= std::min<long long>(max_splits, 16); ++sp) {
+        const long long blocks = tiles * sp;
+        const double rounds = (double)ceil_div(blocks, slots) * (double)slots / (double)blocks;
+        const double time = work * rounds + copy * (double)sp;
+        if (sp == 1 || time < best_time) best = sp, best_time = time;
+      }
+      return best;
+    }
     long long splits = std::max<long long>(1, std::min(slots / tiles, max_splits));
     if (splits >= 8) splits = splits / 8 * 8;
     return splits;
