@@ -1217,9 +1217,10 @@ template <typename T>
 int conv_wgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const void *x, void *dw) {
   hipStream_t s = runtime().stream;
   const int ct = (int)(g.C * g.wvol);
-  // The tap-major kernel writes its columns in (tap, channel) order, so its result
-  // always goes through the reduction kernel, which also restores (channel, tap).
-  const bool staged = pl.splits > 1 || pl.tap_major;
+  // The tap-major kernel writes its columns in (tap, channel) order, so its result goes
+  // through the reduction kernel, which also restores (channel, tap) -- unless there is a
+  // single tap (a matrix product), where the two orders are the same, and a single split.
+  const bool staged = pl.splits > 1 || (pl.tap_major && g.wvol > 1);
   void *target = dw;
   if (staged)
     if (int rc = workspace((size_t)pl.splits * g.F * ct * sizeof(T), &target)) return rc;
