@@ -39,6 +39,8 @@ def test_struct_layouts_match_header():
     assert ctypes.sizeof(_hip.ConvDesc) == 8 + 24 + 6 * 24
     assert ctypes.sizeof(_hip.PoolDesc) == 16 + 8 + 4 * 24
     assert ctypes.sizeof(_hip.DeviceInfo) == 64 + 16 + 8 + 16
+    assert ctypes.sizeof(_hip.BnDesc) == 16 + 24 + 8
+    assert ctypes.sizeof(_hip.WindowDesc) == 8 + 8 + 5 * 24
 
 
 def test_calls_before_init_report_not_initialised():
@@ -61,6 +63,23 @@ def test_no_device_fails_loudly_without_fallback():
         max_pool(x, (2, 2), 2)
     assert _graph.held_count() == 0  # a failing op releases its locks
     assert x.flags.writeable
+    # and so do the operations either side of them
+    from mygrad_amd.nnet import batchnorm, relu
+
+    v = np.ones((2, 3))
+    for call in (
+        lambda: relu(v),
+        lambda: mg.multiply(v, v),
+        lambda: mg.sum(v),
+        lambda: batchnorm(v, eps=1e-5),
+        lambda: mg.repeat(v, 2),
+        lambda: mg.matmul(v, v.T),
+        lambda: mg.Tensor(v) @ v.T,
+        lambda: mg.sliding_window_copy(v, (2, 2), 1),
+    ):
+        with pytest.raises(mg.HipUnavailable):
+            call()
+    assert _graph.held_count() == 0
 
 
 # ----------------------------------------------------------------------------- validation (no launch)
@@ -341,3 +360,57 @@ def test_save_and_load_round_trip(tmp_path):
     assert mg.load(buf).dtype == ints.dtype
     with pytest.raises(TypeError):
         mg.save(io.BytesIO(), np.arange(3.0))
+
+
+def test_argument_checks_of_the_neighbouring_operations_need_no_device():
+    """Everything that is refused is refused before a kernel could be launched, with NumPy's /
+    the reference's exception types; empty results are answered on the host."""
+    from mygrad_amd.nnet import batchnorm
+
+    x = np.ones((4, 3, 5))
+    with pytest.raises(ValueError):
+        batchnorm(np.ones(4), eps=1e-5)  # fewer than two axes
+    with pytest.raises(ValueError):
+        batchnorm(x, gamma=np.ones(2), eps=1e-5)
+    with pytest.raises(TypeError):
+        batchnorm(x.astype(np.float32), gamma=np.ones(3), eps=1e-5)  # gamma in another dtype
+    with pytest.raises(TypeError):
+        batchnorm(np.ones((4, 3), dtype=np.int32), eps=1e-5)
+    with pytest.raises(ValueError):
+        batchnorm(x, eps=-1.0)
+    assert batchnorm(np.ones((0, 3, 5)), eps=1e-5).shape == (0, 3, 5)
+
+    with pytest.raises(ValueError):
+        mg.matmul(x, 3.0)  # scalars are not allowed
+    with pytest.raises(ValueError):
+        mg.matmul(np.ones((2, 3)), np.ones((4, 2)))
+    with pytest.raises(NotImplementedError):
+        mg.matmul(np.ones((2, 1, 3, 4)), np.ones((2, 4, 5)))  # stacks that broadcast against each other
+    with pytest.raises(TypeError):
+        mg.matmul(np.ones((2, 3), dtype=np.int64), np.ones((3, 2), dtype=np.int64))
+    assert mg.matmul(np.ones((0, 3)), np.ones((3, 2))).shape == (0, 2)
+    assert np.array_equal(mg.matmul(np.ones((2, 0)), np.ones((0, 3))).data, np.zeros((2, 3)))
+
+    with pytest.raises(ValueError):
+        mg.repeat(np.ones((2, 3)), [1, 2], axis=1)
+    with pytest.raises(ValueError):
+        mg.repeat(np.ones((2, 3)), -1)
+    with pytest.raises(np.exceptions.AxisError):
+        mg.repeat(np.ones((2, 3)), 2, axis=2)
+    with pytest.raises(TypeError):
+        mg.repeat(np.ones(3, dtype=np.complex128), 2)  # 16-byte elements
+    assert mg.repeat(np.ones((2, 3)), 0, axis=1).shape == (2, 0)
+    assert mg.repeat(np.ones((0, 3)), 2, axis=0).shape == (0, 3)
+
+    with pytest.raises(ValueError):
+        mg.sliding_window_copy(np.ones((3, 3)), (4, 4), 1)
+    with pytest.raises(TypeError):
+        mg.sliding_window_copy(np.ones((3, 3)), 2, 1)
+    with pytest.raises(NotImplementedError):
+        mg.sliding_window_copy(np.ones((2, 2, 2, 2)), (1, 1, 1, 1), 1)
+
+    with pytest.raises(NotImplementedError):
+        mg.multiply(np.ones((2, 3)), np.ones(3))
+    with pytest.raises(NotImplementedError):
+        mg.sum(np.ones((2, 3)), axis=0)
+    assert _graph.held_count() == 0
