@@ -173,7 +173,8 @@ __device__ __forceinline__ double pilot_of(const BnParams &p, const T *__restric
     const int count = min(p.N, 8);
     double sum = 0.0;
     for (int i = 0; i < count; ++i) sum += (double)x[(((long long)i * p.N) >> 3) * p.J + (long long)c * p.S];
-    return sum / count;
+    const double pilot = sum / count;
+    return isfinite(pilot) ? pilot : 0.0;
   } else {
     const int lane = threadIdx.x & 63;
     double sample = 0.0;
@@ -182,7 +183,8 @@ __device__ __forceinline__ double pilot_of(const BnParams &p, const T *__restric
       const unsigned n = p.by_s.div(e);
       sample = (double)x[((long long)n * p.C + c) * p.S + (e - n * (unsigned)p.S)];
     }
-    return wave_sum(sample) / (double)min(p.M, 64);
+    const double pilot = wave_sum(sample) / (double)min(p.M, 64);
+    return isfinite(pilot) ? pilot : 0.0;  // an infinite sample must still give an infinite mean, not inf - inf
   }
 }
 
@@ -191,7 +193,8 @@ template <typename T>
 __device__ __forceinline__ void write_stats(const BnParams &p, int c, double sd, double sdd, double pilot, T *mean, T *var) {
   const double m = sd / p.M;
   mean[c] = (T)(pilot + m);
-  var[c] = (T)fmax(sdd / p.M - m * m, 0.0);
+  const double v = sdd / p.M - m * m;
+  var[c] = (T)(v < 0.0 ? 0.0 : v);  // rounding may leave a tiny negative value; a NaN stays a NaN
 }
 
 // sums[c] = (sum g, sum g * xn) in double from the totals of g and g * (x - mean); dbeta and

@@ -138,6 +138,23 @@ def test_constant_channel_and_single_element_channels(abi):
     assert np.isnan(y).all()
 
 
+@pytest.mark.parametrize("bad", [np.nan, np.inf])
+@pytest.mark.parametrize("shape, where", [((6, 3, 20, 20), (4, 1, 7, 3)), ((500, 3), (321, 1))])
+def test_a_non_finite_element_poisons_its_own_channel_only(abi, bad, shape, where):
+    """As in the reference: the channel's mean, variance and normalised values become NaN
+    (an infinite mean for an infinite element), the other channels are untouched."""
+    x, _, _, _ = _case(shape, np.dtype(np.float64), 9)
+    clean = abi.batchnorm_fwd(x, eps=1e-5)
+    x[where] = bad
+    with np.errstate(invalid="ignore"):
+        y, mean, var = abi.batchnorm_fwd(x, eps=1e-5)
+        want_y, want_mean, want_var = ora.batchnorm_forward(x, eps=1e-5)
+    assert np.isnan(want_var[1]) and np.isnan(var[1]) and np.isnan(y[:, 1]).all()
+    assert np.isnan(mean[1]) if np.isnan(want_mean[1]) else mean[1] == want_mean[1]
+    for c in (0, 2):
+        assert np.array_equal(y[:, c], clean[0][:, c]) and mean[c] == clean[1][c] and var[c] == clean[2][c]
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_results_are_identical_from_run_to_run_and_outputs_are_optional(abi, dtype):
     x, gamma, beta, grad = _case((8, 6, 30, 30), np.dtype(dtype), 3)
