@@ -53,6 +53,12 @@ WORKLOADS = {
                   wscale=(2 / 432) ** 0.5, stride=(1, 1, 1), padding=(1, 1, 1), dilation=(1, 1, 1)),
     "pool2": dict(kind="pool", dtype="f64", seed=1002, x=(64, 64, 56, 56), pool=(3, 3), stride=(2, 2)),
     "pool5": dict(kind="pool", dtype="f32", seed=1006, x=(8, 32, 32, 64, 64), pool=(2, 2, 2), stride=(2, 2, 2)),
+    # the same two with each window's argmax recomputed from x in the backward pass (the stateless
+    # pair of entry points) instead of remembered from the forward pass
+    "pool2-recompute": dict(kind="pool", dtype="f64", seed=1002, x=(64, 64, 56, 56), pool=(3, 3), stride=(2, 2),
+                            recompute=True),
+    "pool5-recompute": dict(kind="pool", dtype="f32", seed=1006, x=(8, 32, 32, 64, 64), pool=(2, 2, 2),
+                            stride=(2, 2, 2), recompute=True),
     # relu, multiply and sum (forward and gradients) on a tensor of conv5's output size
     "elem5": dict(kind="elem", dtype="f32", seed=1007, x=(8, 32, 32, 64, 64)),
     # batch normalisation (scaled and shifted) of a tensor of conv3a's output size
@@ -104,7 +110,8 @@ def describe(name):
         return (f"{name}: conv_nd {wl['dtype']} x{wl['x']} * w{wl['w']} stride{wl['stride']} pad{wl['padding']} "
                 f"dil{wl['dilation']} -> grid{conv_grid(wl)} fwd+dx+dw")
     lead, pooled, grid = pool_shapes(wl)
-    return f"{name}: max_pool {wl['dtype']} x{wl['x']} pool{wl['pool']} stride{wl['stride']} -> grid{grid} fwd+bwd"
+    how = "argmax recomputed from x in bwd" if wl.get("recompute") else "argmax kept from fwd, one byte per window"
+    return f"{name}: max_pool {wl['dtype']} x{wl['x']} pool{wl['pool']} stride{wl['stride']} -> grid{grid} fwd+bwd ({how})"
 
 
 class Step:
@@ -222,6 +229,9 @@ class Step:
             self.x, self.g = resident(x), resident(g)
             self.out = _device.DeviceBuffer(g.nbytes)
             self.dx = _device.DeviceBuffer(x.nbytes)
+            self.argmax = None if wl.get("recompute") else _device.DeviceBuffer(g.size)
+            # algorithmic bytes of the stateless definition, |x| + |out| and |x| + |grad| + |dx|, whichever
+            # pair runs: remembering the argmax moves fewer bytes than that in the backward pass
             self.work = {"maxpool_fwd": float(x.nbytes + g.nbytes), "maxpool_bwd": float(2 * x.nbytes + g.nbytes)}
             self.total_work = sum(self.work.values())
             self.unit, self.bound, self.peak = "GB/s", "hbm", PEAK_HBM_GBS
@@ -262,9 +272,12 @@ class Step:
             check(lib.mg_conv_fwd(d, self.x.ptr, self.w.ptr, self.out.ptr))
             check(lib.mg_conv_dgrad(d, self.g.ptr, self.w.ptr, self.dx.ptr))
             check(lib.mg_conv_wgrad(d, self.g.ptr, self.x.ptr, self.dw.ptr))
-        else:
+        elif self.argmax is None:
             check(lib.mg_maxpool_fwd(d, self.x.ptr, self.out.ptr))
             check(lib.mg_maxpool_bwd(d, self.x.ptr, self.g.ptr, self.dx.ptr))
+        else:
+            check(lib.mg_maxpool_fwd_argmax(d, self.x.ptr, self.out.ptr, self.argmax.ptr))
+            check(lib.mg_maxpool_bwd_argmax(d, self.argmax.ptr, self.g.ptr, self.dx.ptr))
 
 
 def run_gpu(name, steps, warmup):

@@ -170,6 +170,19 @@ int mg_maxpool_fwd(const mg_pool_desc *desc, const void *x, void *out);
  * (argmax :111, np.add.at :147-148). */
 int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, void *dx);
 
+/* The same pair with the argmax remembered between the passes instead of recomputed:
+ * the forward pass also writes argmax[lead,g] (one byte per window, lead * prod(G) bytes:
+ * the row-major offset (a0*P1 + a1)*P2 + a2 inside the window of the first-occurrence
+ * maximum, the first NaN if any), and the backward pass routes grad from those bytes
+ * without reading x.  Same results, bit for bit, as mg_maxpool_fwd / mg_maxpool_bwd while
+ * x is unchanged between the two calls.  A window of more than 256 elements is refused
+ * (unsupported): use the pair above.
+ * mg_maxpool_fwd_argmax replaces MaxPoolND.__call__, src/mygrad/nnet/layers/pooling.py:93-98,
+ * and performs the argmax of :109-111 early; mg_maxpool_bwd_argmax replaces the rest of
+ * MaxPoolND.backward_var, pooling.py:113-149 (index arithmetic and np.add.at). */
+int mg_maxpool_fwd_argmax(const mg_pool_desc *desc, const void *x, void *out, void *argmax);
+int mg_maxpool_bwd_argmax(const mg_pool_desc *desc, const void *argmax, const void *grad, void *dx);
+
 /* ---- element-wise and whole-array kernels either side of conv / pool ----
  * dtype: 0 float32, 1 float64; n elements, C-contiguous, same shape; device pointers,
  * 16-byte aligned (what mg_malloc returns). */

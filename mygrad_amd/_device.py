@@ -143,6 +143,12 @@ def note_released(arr):
     _mirrors.pop(key, None)
 
 
+def is_locked(arr):
+    """True while the graph holds ``arr`` read-only (so nothing derived from its values on
+    the device can have gone stale)."""
+    return _key(arr) in _locked
+
+
 def _evict_key(key):
     _mirrors.pop(key, None)
     _transient.pop(key, None)

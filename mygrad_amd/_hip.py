@@ -142,6 +142,8 @@ _SIGNATURES = {
     "mg_conv_wgrad": [ctypes.POINTER(ConvDesc), _vp, _vp, _vp],
     "mg_maxpool_fwd": [ctypes.POINTER(PoolDesc), _vp, _vp],
     "mg_maxpool_bwd": [ctypes.POINTER(PoolDesc), _vp, _vp, _vp],
+    "mg_maxpool_fwd_argmax": [ctypes.POINTER(PoolDesc), _vp, _vp, _vp],
+    "mg_maxpool_bwd_argmax": [ctypes.POINTER(PoolDesc), _vp, _vp, _vp],
     "mg_multiply": [ctypes.c_int, ctypes.c_int64, _vp, _vp, _vp],
     "mg_relu_fwd": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
     "mg_relu_bwd": [ctypes.c_int, ctypes.c_int64, _vp, _vp, _vp],

@@ -24,9 +24,12 @@ __device__ __forceinline__ bool takes_over(T cand, T best) {
   return (best == best) && !(cand <= best);  // "not <=" is true for cand > best and for a NaN cand
 }
 
-template <typename T>
+// MARK (here and below): also record, one byte per window, where its maximum sits:
+// the row-major offset (a0 * P1 + a1) * P2 + a2 of the first-occurrence argmax inside
+// the window.  The backward pass can then route gradients without reading x again.
+template <typename T, bool MARK>
 __global__ void __launch_bounds__(256) maxpool_fwd_kernel(PoolParams p, const T *__restrict__ x,
-                                                          T *__restrict__ out) {
+                                                          T *__restrict__ out, unsigned char *__restrict__ mark) {
   const long long total = p.lead * p.gvol;
   for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
        idx += (long long)gridDim.x * blockDim.x) {
@@ -38,15 +41,20 @@ __global__ void __launch_bounds__(256) maxpool_fwd_kernel(PoolParams p, const T 
     const int g0 = r / p.G[1];
     const T *w = x + l * p.xvol + ((long long)(g0 * p.S[0]) * p.X[1] + g1 * p.S[1]) * p.X[2] + g2 * p.S[2];
     T best = w[0];
+    int code = 0;
     for (int a0 = 0; a0 < p.P[0]; ++a0)
       for (int a1 = 0; a1 < p.P[1]; ++a1) {
         const T *row = w + ((long long)a0 * p.X[1] + a1) * p.X[2];
         for (int a2 = 0; a2 < p.P[2]; ++a2) {
           const T v = row[a2];
-          if (takes_over(v, best)) best = v;
+          if (takes_over(v, best)) {
+            best = v;
+            code = (a0 * p.P[1] + a1) * p.P[2] + a2;
+          }
         }
       }
     out[idx] = best;
+    if constexpr (MARK) mark[idx] = (unsigned char)code;
   }
 }
 
@@ -138,6 +146,7 @@ struct PoolTileParams {
   long long lead;
   FastDivP by_x12, by_x2, by_g12, by_g2, by_xvol, by_gvol;
   FastDivP by_s[3];
+  FastDivP by_p12, by_p2;  // a recorded argmax offset back to (a0, a1, a2)
   int cand[3];  // windows that can cover one element, per axis: ceil(P/S)
   int nranks;   // their product
 };
@@ -257,11 +266,16 @@ struct ChunkInFlight {
 // PSIG names a pool extent known at compile time, P0*100 + P1*10 + P2 (each 1..3), whose
 // window scan is fully unrolled: all its LDS reads are issued before the first compare
 // instead of one read-compare round trip per element; 0 = any extent, looped.
-template <typename T, typename TD, typename ACC, bool BWD, int DEPTH, int PSIG>
+// FROM_MARK (backward only): x is neither loaded nor scanned; each window's argmax comes from
+// the byte a MARK forward pass recorded, staged through LDS at mark_offset like the gradients.
+template <typename T, typename TD, typename ACC, bool BWD, int DEPTH, int PSIG, bool MARK = false,
+          bool FROM_MARK = false>
 __global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, const T *__restrict__ x,
                                                            const T *__restrict__ grad, void *__restrict__ result,
                                                            long long ntiles, int tile_elems, int win_slots,
-                                                           int acc_offset) {
+                                                           int acc_offset, unsigned char *__restrict__ mark = nullptr,
+                                                           int mark_offset = 0) {
+  static_assert(!FROM_MARK || BWD, "only the backward pass reads recorded positions");
   // LDS: [x tile | one packed int per window | grad of those windows | accumulators];
   // win_slots is a multiple of 4.  The accumulators alias the x tile (acc_offset == 0)
   // when they are no wider than T: x is dead once every window knows its argmax.
@@ -270,19 +284,28 @@ __global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, con
   int *winner = reinterpret_cast<int *>(smem + (size_t)tile_elems * sizeof(T));
   T *gtile = reinterpret_cast<T *>(smem + (size_t)tile_elems * sizeof(T) + (size_t)win_slots * sizeof(int));
   ACC *acc = reinterpret_cast<ACC *>(smem + acc_offset);
+  unsigned char *mtile = smem + mark_offset;
   constexpr int GDEPTH = 2;
   const int x12 = p.X[1] * p.X[2], g12 = p.G[1] * p.G[2];
 
   ChunkInFlight<T, DEPTH> xin;
   ChunkInFlight<T, GDEPTH> gin;
+  ChunkInFlight<unsigned char, 1> marks_in;
   long long blk = blockIdx.x;
   if (blk >= ntiles) return;
   TileGeom t = tile_geom<T, BWD>(p, blk);
-  xin.issue(x, t.chunk_start, t.chunk_len, t.pad);
+  if constexpr (FROM_MARK)
+    marks_in.issue(mark, t.gstart, t.nwin, (int)(t.gstart % 16));
+  else
+    xin.issue(x, t.chunk_start, t.chunk_len, t.pad);
   if (BWD) gin.issue(grad, t.gstart, t.nwin, t.gpad);
 
   for (; blk < ntiles; blk += gridDim.x) {
-    xin.commit(tile, x, t.chunk_start, t.chunk_len, t.pad);
+    const int mpad = (int)(t.gstart % 16);
+    if constexpr (FROM_MARK)
+      marks_in.commit(mtile, mark, t.gstart, t.nwin, mpad);
+    else
+      xin.commit(tile, x, t.chunk_start, t.chunk_len, t.pad);
     if (BWD) gin.commit(gtile, grad, t.gstart, t.nwin, t.gpad);
     __syncthreads();
 
@@ -291,7 +314,10 @@ __global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, con
     TileGeom tn = t;
     if (nblk < ntiles) {
       tn = tile_geom<T, BWD>(p, nblk);
-      xin.issue(x, tn.chunk_start, tn.chunk_len, tn.pad);
+      if constexpr (FROM_MARK)
+        marks_in.issue(mark, tn.gstart, tn.nwin, (int)(tn.gstart % 16));
+      else
+        xin.issue(x, tn.chunk_start, tn.chunk_len, tn.pad);
       if (BWD) gin.issue(grad, tn.gstart, tn.nwin, tn.gpad);
     }
 
@@ -305,9 +331,25 @@ __global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, con
       const unsigned g2 = r - g1 * (unsigned)p.G[2];
       const int origin = (int)((g0 * p.S[0] * p.X[1] + g1 * p.S[1]) * p.X[2] + g2 * p.S[2]) - t.first_flat +
                          (int)vol * p.xvol + t.pad;
-      T best = tile[origin];
+      T best = FROM_MARK ? T(0) : tile[origin];
       int where = origin;
-      if constexpr (PSIG != 0) {
+      int code = 0;  // the argmax as an offset inside the window (what MARK records)
+      if constexpr (FROM_MARK) {
+        const unsigned recorded = mtile[mpad + w];
+        unsigned a0, a1, a2;
+        if constexpr (PSIG != 0) {
+          constexpr unsigned Q1 = (PSIG / 10) % 10, Q2 = PSIG % 10;
+          a0 = recorded / (Q1 * Q2);
+          a1 = (recorded - a0 * Q1 * Q2) / Q2;
+          a2 = recorded - (a0 * Q1 + a1) * Q2;
+        } else {
+          a0 = p.by_p12.div(recorded);
+          const unsigned r12 = recorded - a0 * (unsigned)(p.P[1] * p.P[2]);
+          a1 = p.by_p2.div(r12);
+          a2 = r12 - a1 * (unsigned)p.P[2];
+        }
+        where = origin + (int)((a0 * p.X[1] + a1) * p.X[2] + a2);
+      } else if constexpr (PSIG != 0) {
         constexpr int Q0 = PSIG / 100, Q1 = (PSIG / 10) % 10, Q2 = PSIG % 10;
         T v[Q0 * Q1 * Q2];
 #pragma unroll
@@ -326,6 +368,7 @@ __global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, con
               if (takes_over(c, best)) {
                 best = c;
                 where = origin + (a0 * p.X[1] + a1) * p.X[2] + a2;
+                code = (a0 * Q1 + a1) * Q2 + a2;
               }
             }
       } else {
@@ -337,6 +380,7 @@ __global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, con
               if (takes_over(v, best)) {
                 best = v;
                 where = rowoff + a2;
+                code = (a0 * p.P[1] + a1) * p.P[2] + a2;
               }
             }
           }
@@ -359,6 +403,7 @@ __global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, con
         winner[w] = where | (int)(rank << 20);
       } else {
         static_cast<T *>(result)[t.gstart + w] = best;
+        if constexpr (MARK) mark[t.gstart + w] = (unsigned char)code;
       }
     }
 
@@ -441,18 +486,22 @@ struct PoolExactParams {
   FastDivP by_pieces, by_g1, by_g0;
 };
 
-template <typename T, typename TD, int P0, int P1, int P2, bool BWD>
+template <typename T, typename TD, int P0, int P1, int P2, bool BWD, bool MARK = false>
 __global__ void __launch_bounds__(256) maxpool_exact_kernel(PoolExactParams p, const T *__restrict__ x,
-                                                            const T *__restrict__ grad, void *__restrict__ result) {
+                                                            const T *__restrict__ grad, void *__restrict__ result,
+                                                            unsigned char *__restrict__ mark = nullptr) {
   constexpr int VEC = 16 / sizeof(T);
   constexpr int WPT = VEC / P2;  // windows per thread
   static_assert(VEC % P2 == 0 && WPT >= 1, "a 16-byte piece holds whole windows");
   typedef T Vec __attribute__((ext_vector_type(VEC)));
   typedef T WVec __attribute__((ext_vector_type(WPT)));
   const long long item = (long long)blockIdx.x * 256 + threadIdx.x;
-  if (item >= p.total) return;
+  // with MARK every thread stays for the block-wide store of the recorded bytes: a thread
+  // past the end works on the last item again and stores nothing
+  const bool live = item < p.total;
+  if (!MARK && !live) return;
   // item -> (leading index, g0, g1, piece); total < 2^32 is checked by the host
-  const unsigned u = (unsigned)item;
+  const unsigned u = (unsigned)(live ? item : p.total - 1);
   const unsigned q1 = p.by_pieces.div(u), piece = u - q1 * (unsigned)p.pieces;
   const unsigned q2 = p.by_g1.div(q1), g1 = q1 - q2 * (unsigned)p.G1;
   const unsigned lead = p.by_g0.div(q2), g0 = q2 - lead * (unsigned)p.G0;
@@ -487,7 +536,24 @@ __global__ void __launch_bounds__(256) maxpool_exact_kernel(PoolExactParams p, c
     WVec o;
 #pragma unroll
     for (int j = 0; j < WPT; ++j) o[j] = best[j];
-    *reinterpret_cast<WVec *>(static_cast<T *>(result) + w0) = o;
+    if (live) *reinterpret_cast<WVec *>(static_cast<T *>(result) + w0) = o;
+    if constexpr (MARK) {
+      // The windows of item i are windows i * WPT ... of the whole tensor, so a block's
+      // bytes are one contiguous run: gathered in LDS and stored 16 at a time.
+      __shared__ __attribute__((aligned(16))) unsigned char stage[256 * WPT];
+#pragma unroll
+      for (int j = 0; j < WPT; ++j) stage[threadIdx.x * WPT + j] = (unsigned char)where[j];
+      __syncthreads();
+      const long long run0 = (long long)blockIdx.x * 256 * WPT, run_end = p.total * WPT;
+      const int at = (int)threadIdx.x * 16;
+      if (at < 256 * WPT) {
+        if (run0 + at + 16 <= run_end) {
+          *reinterpret_cast<uint4 *>(mark + run0 + at) = *reinterpret_cast<const uint4 *>(stage + at);
+        } else {
+          for (int b = 0; b < 16 && run0 + at + b < run_end; ++b) mark[run0 + at + b] = stage[at + b];
+        }
+      }
+    }
   } else {
     const WVec g = *reinterpret_cast<const WVec *>(grad + w0);
     typedef TD DVec __attribute__((ext_vector_type(VEC)));
@@ -508,6 +574,128 @@ __global__ void __launch_bounds__(256) maxpool_exact_kernel(PoolExactParams p, c
         *reinterpret_cast<DVec *>(dx + xrow0 + ((long long)a0 * p.X1 + a1) * p.X2) = d;
       }
   }
+}
+
+// ------------------------------------------------------------------------------------------
+// Backward from the argmax positions a MARK forward pass recorded: x is not read again.
+// A thread owns VD consecutive elements of dx (one 16-byte store).  Each element walks the
+// windows that cover it in ascending row-major order and adds grad where the window's
+// recorded offset is the element's own offset inside that window: the order and the
+// +0.0 start of np.add.at, carried in double and rounded once.
+// ------------------------------------------------------------------------------------------
+struct PoolMarkParams {
+  int X[3], P[3], S[3], G[3];
+  int xvol, gvol, x12;
+  int leads;        // leading indices per blockIdx.y: leads * xvol < 2^31
+  long long lead;   // leading indices in all
+  FastDivP by_xvol, by_x12, by_x2, by_s[3];
+};
+
+template <typename T, typename TD, int VD>
+__global__ void __launch_bounds__(256) maxpool_from_mark_kernel(PoolMarkParams p, const unsigned char *__restrict__ mark,
+                                                                const T *__restrict__ grad, TD *__restrict__ dx) {
+  const long long lead0 = (long long)blockIdx.y * p.leads;
+  const unsigned here = (unsigned)min((long long)p.leads, p.lead - lead0) * (unsigned)p.xvol;  // elements in this slice
+  const unsigned first = (blockIdx.x * 256u + threadIdx.x) * (unsigned)VD;
+  if (first >= here) return;
+  const unsigned l = p.by_xvol.div(first);
+  unsigned r = first - l * (unsigned)p.xvol;
+  int i0 = (int)p.by_x12.div(r);
+  r -= (unsigned)i0 * (unsigned)p.x12;
+  int i1 = (int)p.by_x2.div(r);
+  int i2 = (int)r - i1 * p.X[2];
+  const unsigned char *m = mark + (lead0 + l) * p.gvol;
+  const T *g = grad + (lead0 + l) * p.gvol;
+
+  // windows g_k in [lo, hi] cover coordinate i along axis k
+  auto lo_of = [&](int k, int i) { return i >= p.P[k] ? (int)p.by_s[k].div((unsigned)(i - p.P[k] + p.S[k])) : 0; };
+  auto hi_of = [&](int k, int i) { return min(p.G[k] - 1, (int)p.by_s[k].div((unsigned)i)); };
+  int lo0 = lo_of(0, i0), hi0 = hi_of(0, i0), lo1 = lo_of(1, i1), hi1 = hi_of(1, i1);
+
+  TD vals[VD];
+#pragma unroll
+  for (int v = 0; v < VD; ++v) {
+    double acc = 0.0;
+    if (first + v < here) {
+      const int lo2 = lo_of(2, i2), hi2 = hi_of(2, i2);
+      for (int g0 = lo0; g0 <= hi0; ++g0)
+        for (int g1 = lo1; g1 <= hi1; ++g1) {
+          const int row = (g0 * p.G[1] + g1) * p.G[2];
+          const int mine01 = ((i0 - g0 * p.S[0]) * p.P[1] + (i1 - g1 * p.S[1])) * p.P[2];
+          for (int g2 = lo2; g2 <= hi2; ++g2)
+            if ((int)m[row + g2] == mine01 + (i2 - g2 * p.S[2])) acc += (double)g[row + g2];
+        }
+      // the next element: along the row, wrapping into the next row / plane / leading index
+      if (++i2 == p.X[2]) {
+        i2 = 0;
+        if (++i1 == p.X[1]) {
+          i1 = 0;
+          if (++i0 == p.X[0]) {
+            i0 = 0;
+            m += p.gvol;
+            g += p.gvol;
+          }
+          lo0 = lo_of(0, i0);
+          hi0 = hi_of(0, i0);
+        }
+        lo1 = lo_of(1, i1);
+        hi1 = hi_of(1, i1);
+      }
+    }
+    vals[v] = (TD)acc;
+  }
+  TD *to = dx + lead0 * p.xvol + first;
+  if (VD > 1 && first + VD <= here) {
+    typedef TD DVec __attribute__((ext_vector_type(VD)));
+    DVec d;
+#pragma unroll
+    for (int v = 0; v < VD; ++v) d[v] = vals[v];
+    *reinterpret_cast<DVec *>(to) = d;
+  } else {
+#pragma unroll
+    for (int v = 0; v < VD; ++v)
+      if (first + v < here) to[v] = vals[v];
+  }
+}
+
+// The same for windows that tile the input exactly: an element belongs to one window, so a
+// thread reads the recorded offsets and gradients of its 16 / (P2 * sizeof(T)) windows and
+// writes their P0 x P1 rows of dx.
+template <typename T, typename TD, int P0, int P1, int P2>
+__global__ void __launch_bounds__(256) maxpool_exact_from_mark_kernel(PoolExactParams p,
+                                                                      const unsigned char *__restrict__ mark,
+                                                                      const T *__restrict__ grad, TD *__restrict__ dx) {
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int WPT = VEC / P2;
+  static_assert(VEC % P2 == 0 && WPT >= 1, "a 16-byte piece holds whole windows");
+  typedef T WVec __attribute__((ext_vector_type(WPT)));
+  typedef TD DVec __attribute__((ext_vector_type(VEC)));
+  const long long item = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (item >= p.total) return;
+  const unsigned u = (unsigned)item;
+  const unsigned q1 = p.by_pieces.div(u), piece = u - q1 * (unsigned)p.pieces;
+  const unsigned q2 = p.by_g1.div(q1), g1 = q1 - q2 * (unsigned)p.G1;
+  const unsigned lead = p.by_g0.div(q2), g0 = q2 - lead * (unsigned)p.G0;
+  const long long xrow0 = (long long)lead * p.xvol + ((long long)(g0 * P0) * p.X1 + g1 * P1) * p.X2 + piece * VEC;
+  const long long w0 = (long long)lead * p.gvol + ((long long)g0 * p.G1 + g1) * (p.pieces * WPT) + piece * WPT;
+  const WVec g = *reinterpret_cast<const WVec *>(grad + w0);
+  int where[WPT];
+#pragma unroll
+  for (int j = 0; j < WPT; ++j) where[j] = (int)mark[w0 + j];
+#pragma unroll
+  for (int a0 = 0; a0 < P0; ++a0)
+#pragma unroll
+    for (int a1 = 0; a1 < P1; ++a1) {
+      DVec d;
+#pragma unroll
+      for (int j = 0; j < WPT; ++j)
+#pragma unroll
+        for (int a2 = 0; a2 < P2; ++a2) {
+          const TD term = (TD)(T(0) + g[j]);  // added to +0.0, so -0.0 becomes +0.0
+          d[j * P2 + a2] = where[j] == (a0 * P1 + a1) * P2 + a2 ? term : TD(0);
+        }
+      *reinterpret_cast<DVec *>(dx + xrow0 + ((long long)a0 * p.X1 + a1) * p.X2) = d;
+    }
 }
 
 static int check_pool_desc(const mg_pool_desc *d, PoolParams *p) {
@@ -648,6 +836,8 @@ static bool plan_tiles(const PoolParams &pp, size_t elem, size_t acc_elem, bool 
   q.by_xvol = make_fastdiv_p((unsigned)pp.xvol);
   q.by_gvol = make_fastdiv_p((unsigned)pp.gvol);
   for (int k = 0; k < 3; ++k) q.by_s[k] = make_fastdiv_p((unsigned)pp.S[k]);
+  q.by_p12 = make_fastdiv_p((unsigned)(pp.P[1] * pp.P[2]));
+  q.by_p2 = make_fastdiv_p((unsigned)pp.P[2]);
   q.nranks = 1;
   for (int k = 0; k < 3; ++k) {
     q.cand[k] = (pp.P[k] - 1) / pp.S[k] + 1;
@@ -721,31 +911,33 @@ static int exact_signature(const PoolParams &p, size_t elem, const void *a, cons
   return sig;
 }
 
-}  // namespace mg
-
-using namespace mg;
-
-extern "C" {
-
-int mg_maxpool_fwd(const mg_pool_desc *desc, const void *x, void *out) {
-  std::lock_guard<std::recursive_mutex> guard(api_mutex());
-  MG_REQUIRE_INIT();
+// Forward pass; `mark`, when not null, receives one byte per window (see MARK).
+static int maxpool_fwd_impl(const mg_pool_desc *desc, const void *x, void *out, unsigned char *mark) {
   PoolParams p;
   if (int rc = check_pool_desc(desc, &p)) return rc;
-  if (!x || !out) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_maxpool_fwd");
+  if (!x || !out) return fail(MG_ERR_BAD_ARG, "null tensor pointer in the max-pool forward pass");
+  if (mark && (long long)p.P[0] * p.P[1] * p.P[2] > 256)
+    return fail(MG_ERR_UNSUPPORTED, "a window of %lld elements does not fit the one-byte argmax record (at most 256)",
+                (long long)p.P[0] * p.P[1] * p.P[2]);
   hipStream_t s = runtime().stream;
   ScopedTiming timed(TAG_POOL_FWD);
   PoolExactParams ep;
-  if (const int sig = exact_signature(p, desc->dtype == MG_F32 ? 4 : 8, x, out, out, 0, &ep)) {
+  if (const int sig = exact_signature(p, desc->dtype == MG_F32 ? 4 : 8, x, out, mark ? (const void *)mark : out, 0, &ep)) {
     const dim3 grid((unsigned)ceil_div(ep.total, 256)), block(256);
-#define MG_POOL_EXACT_FWD(T)                                                                                             \
-  do {                                                                                                                   \
-    if (sig == 122)                                                                                                      \
-      hipLaunchKernelGGL((maxpool_exact_kernel<T, T, 1, 2, 2, false>), grid, block, 0, s, ep, (const T *)x, (const T *)nullptr, out); \
-    else                                                                                                                 \
-      hipLaunchKernelGGL((maxpool_exact_kernel<T, T, 2, 2, 2, false>), grid, block, 0, s, ep, (const T *)x, (const T *)nullptr, out); \
+#define MG_POOL_EXACT_FWD(T, MK)                                                                              \
+  do {                                                                                                        \
+    if (sig == 122)                                                                                           \
+      hipLaunchKernelGGL((maxpool_exact_kernel<T, T, 1, 2, 2, false, MK>), grid, block, 0, s, ep, (const T *)x, \
+                         (const T *)nullptr, out, mark);                                                      \
+    else                                                                                                      \
+      hipLaunchKernelGGL((maxpool_exact_kernel<T, T, 2, 2, 2, false, MK>), grid, block, 0, s, ep, (const T *)x, \
+                         (const T *)nullptr, out, mark);                                                      \
   } while (0)
-    if (desc->dtype == MG_F32) MG_POOL_EXACT_FWD(float); else MG_POOL_EXACT_FWD(double);
+    if (desc->dtype == MG_F32) {
+      if (mark) MG_POOL_EXACT_FWD(float, true); else MG_POOL_EXACT_FWD(float, false);
+    } else {
+      if (mark) MG_POOL_EXACT_FWD(double, true); else MG_POOL_EXACT_FWD(double, false);
+    }
 #undef MG_POOL_EXACT_FWD
     MG_HIP(hipGetLastError());
     return MG_OK;
@@ -761,17 +953,21 @@ int mg_maxpool_fwd(const mg_pool_desc *desc, const void *x, void *out) {
     const dim3 grid((unsigned)blocks), block(256);
     const bool deep = (size_t)tile_elems * elem > 8 * 4096;  // 16-byte loads per thread to cover the tile
     const int sig = pool_signature(p);
-#define MG_POOL_FWD_SIG(T, DEPTH, SIG)                                                                          \
-  hipLaunchKernelGGL((maxpool_tile_kernel<T, T, T, false, DEPTH, SIG>), grid, block, lds, s, tp, (const T *)x,  \
-                     (const T *)nullptr, out, blocks, tile_elems, win_slots, acc_offset)
-#define MG_POOL_FWD(T, DEPTH)                          \
-  do {                                                 \
-    switch (sig) {                                     \
-      case 133: MG_POOL_FWD_SIG(T, DEPTH, 133); break; \
-      case 122: MG_POOL_FWD_SIG(T, DEPTH, 122); break; \
-      case 222: MG_POOL_FWD_SIG(T, DEPTH, 222); break; \
-      default: MG_POOL_FWD_SIG(T, DEPTH, 0); break;    \
-    }                                                  \
+#define MG_POOL_FWD_SIG(T, DEPTH, SIG, MK)                                                                         \
+  hipLaunchKernelGGL((maxpool_tile_kernel<T, T, T, false, DEPTH, SIG, MK>), grid, block, lds, s, tp, (const T *)x, \
+                     (const T *)nullptr, out, blocks, tile_elems, win_slots, acc_offset, mark)
+#define MG_POOL_FWD_MK(T, DEPTH, MK)                       \
+  do {                                                     \
+    switch (sig) {                                         \
+      case 133: MG_POOL_FWD_SIG(T, DEPTH, 133, MK); break; \
+      case 122: MG_POOL_FWD_SIG(T, DEPTH, 122, MK); break; \
+      case 222: MG_POOL_FWD_SIG(T, DEPTH, 222, MK); break; \
+      default: MG_POOL_FWD_SIG(T, DEPTH, 0, MK); break;    \
+    }                                                      \
+  } while (0)
+#define MG_POOL_FWD(T, DEPTH)                                                         \
+  do {                                                                                \
+    if (mark) MG_POOL_FWD_MK(T, DEPTH, true); else MG_POOL_FWD_MK(T, DEPTH, false);   \
   } while (0)
     if (desc->dtype == MG_F32) {
       if (deep) MG_POOL_FWD(float, 12); else MG_POOL_FWD(float, 8);
@@ -779,17 +975,172 @@ int mg_maxpool_fwd(const mg_pool_desc *desc, const void *x, void *out) {
       if (deep) MG_POOL_FWD(double, 12); else MG_POOL_FWD(double, 8);
     }
 #undef MG_POOL_FWD
+#undef MG_POOL_FWD_MK
 #undef MG_POOL_FWD_SIG
     MG_HIP(hipGetLastError());
     return MG_OK;
   }
   const unsigned grid = grid_for(p.lead * p.gvol);
-  if (desc->dtype == MG_F32)
-    hipLaunchKernelGGL(maxpool_fwd_kernel<float>, dim3(grid), dim3(256), 0, s, p, (const float *)x, (float *)out);
-  else
-    hipLaunchKernelGGL(maxpool_fwd_kernel<double>, dim3(grid), dim3(256), 0, s, p, (const double *)x, (double *)out);
+#define MG_POOL_FWD_PLAIN(T, MK) \
+  hipLaunchKernelGGL((maxpool_fwd_kernel<T, MK>), dim3(grid), dim3(256), 0, s, p, (const T *)x, (T *)out, mark)
+  if (desc->dtype == MG_F32) {
+    if (mark) MG_POOL_FWD_PLAIN(float, true); else MG_POOL_FWD_PLAIN(float, false);
+  } else {
+    if (mark) MG_POOL_FWD_PLAIN(double, true); else MG_POOL_FWD_PLAIN(double, false);
+  }
+#undef MG_POOL_FWD_PLAIN
   MG_HIP(hipGetLastError());
   return MG_OK;
+}
+
+// Backward pass from recorded argmax offsets.
+static int maxpool_bwd_from_mark(const mg_pool_desc *desc, const unsigned char *mark, const void *grad, void *dx) {
+  PoolParams p;
+  if (int rc = check_pool_desc(desc, &p)) return rc;
+  if (!mark || !grad || !dx) return fail(MG_ERR_BAD_ARG, "null tensor pointer in the max-pool backward pass");
+  if ((long long)p.P[0] * p.P[1] * p.P[2] > 256)
+    return fail(MG_ERR_UNSUPPORTED, "a window of %lld elements does not fit the one-byte argmax record (at most 256)",
+                (long long)p.P[0] * p.P[1] * p.P[2]);
+  hipStream_t s = runtime().stream;
+  ScopedTiming timed(TAG_POOL_BWD);
+  const bool f32 = desc->dtype == MG_F32, wide = desc->dx_dtype == MG_F64;
+  PoolExactParams ep;
+  // the exact-tiling test looks at the alignment of x; grad stands in for it here
+  if (const int sig = exact_signature(p, f32 ? 4 : 8, grad, grad, dx, 0, &ep)) {
+    const dim3 grid((unsigned)ceil_div(ep.total, 256)), block(256);
+#define MG_POOL_EXACT_MARK(T, TD)                                                                                  \
+  do {                                                                                                             \
+    if (sig == 122)                                                                                                \
+      hipLaunchKernelGGL((maxpool_exact_from_mark_kernel<T, TD, 1, 2, 2>), grid, block, 0, s, ep, mark, (const T *)grad, \
+                         (TD *)dx);                                                                                \
+    else                                                                                                           \
+      hipLaunchKernelGGL((maxpool_exact_from_mark_kernel<T, TD, 2, 2, 2>), grid, block, 0, s, ep, mark, (const T *)grad, \
+                         (TD *)dx);                                                                                \
+  } while (0)
+    if (!f32)
+      MG_POOL_EXACT_MARK(double, double);
+    else if (wide)
+      MG_POOL_EXACT_MARK(float, double);
+    else
+      MG_POOL_EXACT_MARK(float, float);
+#undef MG_POOL_EXACT_MARK
+    MG_HIP(hipGetLastError());
+    return MG_OK;
+  }
+  {
+    PoolTileParams tp;
+    int tile_elems = 0, win_slots = 0, acc_offset = 0;
+    size_t lds = 0;
+    long long blocks = 0;
+    bool overlap = false;
+    for (int k = 0; k < 3; ++k) overlap |= p.P[k] > p.S[k];
+    const size_t elem = f32 ? 4 : 8, acc_elem = (f32 && !overlap) ? 4 : 8;
+    if (plan_tiles(p, elem, acc_elem, true, &tp, &tile_elems, &win_slots, &acc_offset, &lds, &blocks) &&
+        lds + (size_t)win_slots + 32 <= 64 * 1024) {
+      // the staged bytes go behind everything else; 16 spare bytes for the alignment shift
+      const int mark_offset = (int)lds;
+      lds += ((size_t)win_slots + 16 + 15) & ~size_t(15);
+      const dim3 grid(persistent_grid(blocks, lds)), block(256);
+      const int sig = pool_signature(p);
+      unsigned char *marks = const_cast<unsigned char *>(mark);  // only read in this mode
+#define MG_POOL_MARK_SIG(T, TD, ACC, SIG)                                                                          \
+  hipLaunchKernelGGL((maxpool_tile_kernel<T, TD, ACC, true, 1, SIG, false, true>), grid, block, lds, s, tp,         \
+                     (const T *)nullptr, (const T *)grad, dx, blocks, tile_elems, win_slots, acc_offset, marks,     \
+                     mark_offset)
+#define MG_POOL_MARK_TILED(T, TD, ACC)                      \
+  do {                                                      \
+    switch (sig) {                                          \
+      case 133: MG_POOL_MARK_SIG(T, TD, ACC, 133); break;   \
+      case 122: MG_POOL_MARK_SIG(T, TD, ACC, 122); break;   \
+      case 222: MG_POOL_MARK_SIG(T, TD, ACC, 222); break;   \
+      default: MG_POOL_MARK_SIG(T, TD, ACC, 0); break;      \
+    }                                                       \
+  } while (0)
+      if (!f32)
+        MG_POOL_MARK_TILED(double, double, double);
+      else if (overlap && wide)
+        MG_POOL_MARK_TILED(float, double, double);
+      else if (overlap)
+        MG_POOL_MARK_TILED(float, float, double);
+      else if (wide)
+        MG_POOL_MARK_TILED(float, double, float);
+      else
+        MG_POOL_MARK_TILED(float, float, float);
+#undef MG_POOL_MARK_TILED
+#undef MG_POOL_MARK_SIG
+      MG_HIP(hipGetLastError());
+      return MG_OK;
+    }
+  }
+  PoolMarkParams q{};
+  for (int k = 0; k < 3; ++k) {
+    q.X[k] = p.X[k];
+    q.P[k] = p.P[k];
+    q.S[k] = p.S[k];
+    q.G[k] = p.G[k];
+    q.by_s[k] = make_fastdiv_p((unsigned)p.S[k]);
+  }
+  q.xvol = (int)p.xvol;
+  q.gvol = (int)p.gvol;
+  q.x12 = p.X[1] * p.X[2];
+  q.lead = p.lead;
+  q.by_xvol = make_fastdiv_p((unsigned)p.xvol);
+  q.by_x12 = make_fastdiv_p((unsigned)q.x12);
+  q.by_x2 = make_fastdiv_p((unsigned)p.X[2]);
+  // slices of whole leading indices whose element count stays below 2^31 (32-bit index
+  // arithmetic inside a slice); a multiple of 4 of them so every slice starts 16-byte aligned
+  const long long cap = ((1ll << 31) - 1024) / p.xvol;
+  long long leads = std::min<long long>(p.lead, cap);
+  if (leads < p.lead) leads -= leads % 4;
+  const size_t dx_elem = (f32 && !wide) ? 4 : 8;
+  const bool vector_ok = leads >= 1 && reinterpret_cast<uintptr_t>(dx) % 16 == 0;
+  if (leads < 1) leads = 1;
+  q.leads = (int)leads;
+  const int vd = vector_ok ? (int)(16 / dx_elem) : 1;
+  const long long slice = leads * p.xvol;
+  const dim3 grid((unsigned)ceil_div(ceil_div(slice, vd), 256), (unsigned)ceil_div(p.lead, leads)), block(256);
+#define MG_POOL_MARK(T, TD)                                                                                        \
+  do {                                                                                                             \
+    if (vd > 1)                                                                                                    \
+      hipLaunchKernelGGL((maxpool_from_mark_kernel<T, TD, 16 / sizeof(TD)>), grid, block, 0, s, q, mark,           \
+                         (const T *)grad, (TD *)dx);                                                               \
+    else                                                                                                           \
+      hipLaunchKernelGGL((maxpool_from_mark_kernel<T, TD, 1>), grid, block, 0, s, q, mark, (const T *)grad, (TD *)dx); \
+  } while (0)
+  if (!f32)
+    MG_POOL_MARK(double, double);
+  else if (wide)
+    MG_POOL_MARK(float, double);
+  else
+    MG_POOL_MARK(float, float);
+#undef MG_POOL_MARK
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
+}  // namespace mg
+
+using namespace mg;
+
+extern "C" {
+
+int mg_maxpool_fwd(const mg_pool_desc *desc, const void *x, void *out) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  return maxpool_fwd_impl(desc, x, out, nullptr);
+}
+
+int mg_maxpool_fwd_argmax(const mg_pool_desc *desc, const void *x, void *out, void *argmax) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (!argmax) return fail(MG_ERR_BAD_ARG, "null argmax pointer in mg_maxpool_fwd_argmax");
+  return maxpool_fwd_impl(desc, x, out, static_cast<unsigned char *>(argmax));
+}
+
+int mg_maxpool_bwd_argmax(const mg_pool_desc *desc, const void *argmax, const void *grad, void *dx) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  return maxpool_bwd_from_mark(desc, static_cast<const unsigned char *>(argmax), grad, dx);
 }
 
 int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, void *dx) {

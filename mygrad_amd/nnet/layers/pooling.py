@@ -21,6 +21,8 @@ class MaxPoolND(Operation):
     every ``(S0, ...)``; only placements that fit entirely inside the data.
     """
 
+    _argmax = None  # device buffer, one byte per window, written by the forward pass
+
     def __call__(self, x, pool, stride):
         self.variables = (x,)
         xd = x.data
@@ -69,8 +71,17 @@ class MaxPoolND(Operation):
 
         desc = _hip.pool_desc(xd.dtype, self._lead, pooled, pool, stride, grid)
         xb = _device.to_device(xd)
-        ob = _device.DeviceBuffer(int(np.prod(out_full)) * xd.dtype.itemsize)
-        _hip.check(_hip.lib().mg_maxpool_fwd(desc, xb.ptr, ob.ptr))
+        windows = int(np.prod(out_full))
+        ob = _device.DeviceBuffer(windows * xd.dtype.itemsize)
+        if int(np.prod(pool)) <= 256:
+            # Each window's argmax (pooling.py:109-111) is found here, while x is being read
+            # anyway, and kept on the device as one byte per window: the backward pass then
+            # needs grad and these bytes only.  x is read-only for as long as the graph holds
+            # it, so the positions cannot go stale; backward_var checks that this still holds.
+            self._argmax = _device.DeviceBuffer(windows)
+            _hip.check(_hip.lib().mg_maxpool_fwd_argmax(desc, xb.ptr, ob.ptr, self._argmax.ptr))
+        else:
+            _hip.check(_hip.lib().mg_maxpool_fwd(desc, xb.ptr, ob.ptr))
         out = _device.download(ob, out_full, xd.dtype)
         _device.attach(out, ob)
         return out
@@ -89,10 +100,13 @@ class MaxPoolND(Operation):
         dx_dtype = np.dtype(np.float64) if var._grad is not None else x.dtype
         desc = _hip.pool_desc(x.dtype, self._lead, x.shape[x.ndim - m :], self.pool, self.stride, self._grid,
                               dx_dtype=dx_dtype)
-        xb = _device.to_device(x)
         gb = _device.to_device(grad, x.dtype)
         db = _device.DeviceBuffer(x.size * dx_dtype.itemsize)
-        _hip.check(_hip.lib().mg_maxpool_bwd(desc, xb.ptr, gb.ptr, db.ptr))
+        if self._argmax is not None and _device.is_locked(x):
+            _hip.check(_hip.lib().mg_maxpool_bwd_argmax(desc, self._argmax.ptr, gb.ptr, db.ptr))
+        else:  # x may have been written to since the forward pass: find the maxima again
+            xb = _device.to_device(x)
+            _hip.check(_hip.lib().mg_maxpool_bwd(desc, xb.ptr, gb.ptr, db.ptr))
         out = _device.download(db, x.shape, dx_dtype)
         _device.attach_transient(out, db)
         return out

@@ -312,6 +312,18 @@ def pool_forward(x, pool, stride, validate=True):
     return np.ascontiguousarray(peak.transpose(order))
 
 
+def pool_argmax(x, pool, stride):
+    """Per window, the position of its maximum inside the flattened (row-major) window:
+    the first of equal maxima, the first NaN if there is one (``argmax(-1)`` of
+    pooling.py:109-111), laid out ``(lead..., G...)`` like the pooled output."""
+    pool, stride = _pool_args(x, pool, stride)
+    m = len(pool)
+    windows = window_view(x, tuple(pool), tuple(stride))  # (G..., lead..., P...)
+    winner = windows.reshape(*windows.shape[: windows.ndim - m], -1).argmax(-1)  # (G..., lead...)
+    nd = winner.ndim
+    return winner.transpose(tuple(range(m, nd)) + tuple(range(m)))  # (lead..., G...)
+
+
 def pool_backward(x, grad, pool, stride):
     """Route ``grad`` to the first-occurrence argmax of every window with an
     unbuffered, C-ordered ``np.add.at`` into a float64 image.  Follows
@@ -321,11 +333,8 @@ def pool_backward(x, grad, pool, stride):
     m = len(pool)
     lead_shape, pooled_shape = x.shape[: x.ndim - m], x.shape[x.ndim - m :]
 
-    windows = window_view(x, tuple(pool), tuple(stride))  # (G..., lead..., P...)
-    grid = windows.shape[:m]
-    winner = windows.reshape(*windows.shape[: windows.ndim - m], -1).argmax(-1)  # (G..., lead...)
-    nd = winner.ndim
-    winner = winner.transpose(tuple(range(m, nd)) + tuple(range(m)))  # (lead..., G...)
+    winner = pool_argmax(x, pool, stride)  # (lead..., G...)
+    grid = winner.shape[winner.ndim - m :]
 
     unit = _c_elem_strides(pooled_shape)  # flat offset of one step along each pooled axis
     inside = sum(a * u for a, u in zip(np.unravel_index(winner, tuple(pool)), unit))

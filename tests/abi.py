@@ -92,6 +92,28 @@ def pool_bwd(x, grad, pool, stride, dx_dtype=None):
     return _down(db, x.shape, dx_dtype)
 
 
+def pool_fwd_argmax(x, pool, stride):
+    """(out, argmax): argmax holds one byte per window, its maximum's offset inside the window."""
+    desc, out_shape = pool_desc(x.shape, x.dtype, pool, stride)
+    xb = _up(x)
+    windows = int(np.prod(out_shape))
+    ob = _device.DeviceBuffer(max(windows * x.dtype.itemsize, 16))
+    ab = _device.DeviceBuffer(max(windows, 16))
+    _hip.check(_hip.lib().mg_maxpool_fwd_argmax(desc, xb.ptr, ob.ptr, ab.ptr))
+    return _down(ob, out_shape, x.dtype), _down(ab, out_shape, np.uint8)
+
+
+def pool_bwd_argmax(argmax, x_shape, x_dtype, grad, pool, stride, dx_dtype=None):
+    x_dtype = np.dtype(x_dtype)
+    dx_dtype = np.dtype(x_dtype if dx_dtype is None else dx_dtype)
+    desc, out_shape = pool_desc(x_shape, x_dtype, pool, stride, dx_dtype=dx_dtype)
+    assert tuple(grad.shape) == tuple(out_shape) == tuple(argmax.shape)
+    ab, gb = _up(np.ascontiguousarray(argmax, dtype=np.uint8)), _up(np.ascontiguousarray(grad, dtype=x_dtype))
+    db = _device.DeviceBuffer(int(np.prod(x_shape)) * dx_dtype.itemsize)
+    _hip.check(_hip.lib().mg_maxpool_bwd_argmax(desc, ab.ptr, gb.ptr, db.ptr))
+    return _down(db, tuple(x_shape), dx_dtype)
+
+
 # ----------------------------------------------------------------- element-wise / sum
 def multiply(a, b):
     ab, bb = _up(a), _up(b)

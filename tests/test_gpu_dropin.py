@@ -168,6 +168,37 @@ def test_config5_chain_keeps_activations_on_the_device():
     assert _graph.held_count() == 0
 
 
+def test_max_pool_keeps_each_windows_argmax_only_while_x_is_guarded():
+    """The forward pass records where every window's maximum sits and the backward pass
+    routes by that record; with the memory guard off x may change in between, and then
+    the maxima are found again from the x of that moment, as the reference does."""
+    rng = np.random.default_rng(77)
+    xv = rng.integers(0, 4, (3, 2, 9, 11)).astype(np.float32)  # ties everywhere
+    g = rng.standard_normal((3, 2, 4, 5)).astype(np.float32)
+    x = mg.Tensor(xv.copy())
+    out = max_pool(x, (3, 3), 2)
+    assert out.creator._argmax is not None and _device.is_locked(x.data)
+    out.backward(g)
+    want = ora.pool_backward(xv, g, (3, 3), 2).astype(np.float32)
+    assert np.array_equal(x.grad.view(np.uint32), want.view(np.uint32))
+
+    big = mg.Tensor(rng.integers(0, 30, (2, 20, 20)).astype(np.float64))  # 272 positions per window
+    out = max_pool(big, (17, 16), 1)
+    assert out.creator._argmax is None
+    out.backward()
+    assert np.array_equal(big.grad, ora.pool_backward(big.data, np.ones((2, 4, 5)), (17, 16), 1))
+
+    with mg.mem_guard_off:
+        x = mg.Tensor(xv.copy())
+        out = max_pool(x, (3, 3), 2)
+        assert not _device.is_locked(x.data)
+        x.data[...] = x.data[..., ::-1].copy()  # allowed without the guard
+        out.backward(g)
+        want = ora.pool_backward(xv[..., ::-1], g, (3, 3), 2).astype(np.float32)
+        assert np.array_equal(x.grad.view(np.uint32), want.view(np.uint32))
+    assert _graph.held_count() == 0
+
+
 def test_mirror_is_dropped_when_host_data_may_change():
     rng = np.random.default_rng(9)
     x = mg.Tensor(rng.standard_normal((2, 3, 8, 8)))

@@ -36,24 +36,48 @@ def bits(a):
 
 
 # ----------------------------------------------------------------------------- pooling
-def test_pool_reference_known_answers(abi, kats):
+class _Remembered:
+    """The pair of entry points that keeps each window's argmax from the forward pass,
+    behind the calling convention of the pair that recomputes it from x."""
+
+    def __init__(self, abi):
+        self.abi = abi
+
+    def pool_fwd(self, x, pool, stride):
+        out, argmax = self.abi.pool_fwd_argmax(x, pool, stride)
+        # what was recorded is np.argmax over each flattened window (pooling.py:109-111)
+        if x.size <= 1 << 22:
+            assert argmax.dtype == np.uint8 and np.array_equal(argmax, ora.pool_argmax(x, pool, stride))
+        return out
+
+    def pool_bwd(self, x, grad, pool, stride, dx_dtype=None):
+        _, argmax = self.abi.pool_fwd_argmax(x, pool, stride)
+        return self.abi.pool_bwd_argmax(argmax, x.shape, x.dtype, grad, pool, stride, dx_dtype=dx_dtype)
+
+
+@pytest.fixture(params=["recompute", "remember"])
+def pools(request, abi):
+    return abi if request.param == "recompute" else _Remembered(abi)
+
+
+def test_pool_reference_known_answers(pools, kats):
     for case in kats["pool"]:
         x = np.array(case["x"], dtype=case["dtype"])
         pool, stride = tuple(case["pool"]), tuple(case["stride"])
-        out = abi.pool_fwd(x, pool, stride)
+        out = pools.pool_fwd(x, pool, stride)
         assert np.array_equal(out, np.array(case["out"], dtype=x.dtype)), case["source"]
         if case["grad"] is None:
             continue
         g = np.ones(out.shape) if case["grad"] == "ones" else np.arange(out.size).reshape(out.shape)
         for dx_dtype in (x.dtype, np.float64):
-            dx = abi.pool_bwd(x, g, pool, stride, dx_dtype=dx_dtype)
+            dx = pools.pool_bwd(x, g, pool, stride, dx_dtype=dx_dtype)
             assert dx.dtype == dx_dtype
             assert np.array_equal(dx, np.array(case["dx"], dtype=float)), case["source"]
 
 
 @pytest.mark.parametrize("m,lead", [(1, (3,)), (1, (2, 5)), (2, (2, 3)), (3, (2,)), (2, ()), (3, (1, 2))])
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
-def test_pool_ties_and_overlap_bit_exact(abi, m, lead, dtype):
+def test_pool_ties_and_overlap_bit_exact(pools, m, lead, dtype):
     rng = np.random.default_rng(300 + 10 * m + len(lead))
     for trial in range(12):
         pool = tuple(int(v) for v in rng.integers(1, 5, m))
@@ -70,13 +94,13 @@ def test_pool_ties_and_overlap_bit_exact(abi, m, lead, dtype):
         g = (rng.standard_normal(out_shape) * 10.0 ** rng.integers(-6, 6, out_shape)).astype(dtype)
         want_out = ora.pool_forward(x, pool, stride, validate=False)
         want_dx = ora.pool_backward(x, g, pool, stride)  # float64
-        out = abi.pool_fwd(x, pool, stride)
+        out = pools.pool_fwd(x, pool, stride)
         assert np.array_equal(bits(out), bits(want_out))
-        dx64 = abi.pool_bwd(x, g, pool, stride, dx_dtype=np.float64)
+        dx64 = pools.pool_bwd(x, g, pool, stride, dx_dtype=np.float64)
         assert np.array_equal(bits(dx64), bits(want_dx))
-        dx = abi.pool_bwd(x, g, pool, stride)
+        dx = pools.pool_bwd(x, g, pool, stride)
         assert np.array_equal(bits(dx), bits(want_dx.astype(dtype)))
-        hits = abi.pool_bwd(x, np.ones(out_shape, dtype), pool, stride)
+        hits = pools.pool_bwd(x, np.ones(out_shape, dtype), pool, stride)
         assert np.array_equal(hits, ora.pool_backward(x, np.ones(out_shape), pool, stride))
 
 
@@ -87,7 +111,7 @@ def test_pool_ties_and_overlap_bit_exact(abi, m, lead, dtype):
     ((7,), (2, 2, 4), (2, 2, 2)),     # a single window slab per volume
     ((4,), (10, 6), (2, 2)),          # rows that are not whole 16-byte pieces in float32: the tiled kernel
 ])
-def test_pool_windows_that_tile_the_input_exactly(abi, dtype, lead, X, pool):
+def test_pool_windows_that_tile_the_input_exactly(pools, dtype, lead, X, pool):
     """Stride == pool extent and X == G * P: the kernels that work straight from global
     memory.  Ties, NaNs, -0.0 gradients and the float64 dx of a float32 input included."""
     rng = np.random.default_rng(350 + len(X) + X[-1])
@@ -103,40 +127,63 @@ def test_pool_windows_that_tile_the_input_exactly(abi, dtype, lead, X, pool):
         g[rng.random(out_shape) < 0.2] = -0.0
         want_out = ora.pool_forward(x, pool, pool, validate=False)
         want_dx = ora.pool_backward(x, g, pool, pool)  # float64
-        assert np.array_equal(bits(abi.pool_fwd(x, pool, pool)), bits(want_out))
-        assert np.array_equal(bits(abi.pool_bwd(x, g, pool, pool, dx_dtype=np.float64)), bits(want_dx))
-        assert np.array_equal(bits(abi.pool_bwd(x, g, pool, pool)), bits(want_dx.astype(dtype)))
+        assert np.array_equal(bits(pools.pool_fwd(x, pool, pool)), bits(want_out))
+        assert np.array_equal(bits(pools.pool_bwd(x, g, pool, pool, dx_dtype=np.float64)), bits(want_dx))
+        assert np.array_equal(bits(pools.pool_bwd(x, g, pool, pool)), bits(want_dx.astype(dtype)))
 
 
-def test_pool_order_of_summation_and_signed_zero(abi):
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("X,pool,stride", [((7, 9001), (3, 3), (2, 2)), ((2, 5, 7000), (2, 3, 2), (1, 2, 3))])
+def test_pool_rows_too_long_for_the_staged_kernels(pools, dtype, X, pool, stride):
+    """One row of windows with its halo exceeds the LDS budget: the kernels that work
+    element by element from global memory take over."""
+    rng = np.random.default_rng(360 + len(X))
+    x = rng.integers(0, 5, (3, *X)).astype(dtype)
+    out_shape = (3, *(((xk - pk) // sk + 1) for xk, pk, sk in zip(X, pool, stride)))
+    g = (rng.standard_normal(out_shape) * 10.0 ** rng.integers(-6, 6, out_shape)).astype(dtype)
+    want_dx = ora.pool_backward(x, g, pool, stride)
+    assert np.array_equal(bits(pools.pool_fwd(x, pool, stride)), bits(ora.pool_forward(x, pool, stride, validate=False)))
+    assert np.array_equal(bits(pools.pool_bwd(x, g, pool, stride, dx_dtype=np.float64)), bits(want_dx))
+    assert np.array_equal(bits(pools.pool_bwd(x, g, pool, stride)), bits(want_dx.astype(dtype)))
+
+
+def test_pool_window_of_256_positions_fills_the_argmax_byte(pools):
+    rng = np.random.default_rng(361)
+    x = rng.integers(0, 50, (2, 20, 19)).astype(np.float64)
+    g = rng.standard_normal((2, 5, 4))
+    assert np.array_equal(pools.pool_fwd(x, (16, 16), 1), ora.pool_forward(x, (16, 16), 1))
+    assert np.array_equal(bits(pools.pool_bwd(x, g, (16, 16), 1)), bits(ora.pool_backward(x, g, (16, 16), 1)))
+
+
+def test_pool_order_of_summation_and_signed_zero(pools):
     x = np.array([[0.0, 0.0, 9.0, 0.0, 0.0]])
     for g in ([1e16, 1.0, -1e16], [1e16, -1e16, 1.0], [-0.0, -0.0, -0.0]):
         g = np.array([g])
-        dx = abi.pool_bwd(x, g, (3,), (1,))
+        dx = pools.pool_bwd(x, g, (3,), (1,))
         assert np.array_equal(bits(dx), bits(ora.pool_backward(x, g, (3,), (1,))))
-    dx = abi.pool_bwd(np.array([[1.0, 0.0]]), np.array([[-0.0]]), (2,), (2,))
+    dx = pools.pool_bwd(np.array([[1.0, 0.0]]), np.array([[-0.0]]), (2,), (2,))
     assert not np.signbit(dx).any()
 
 
-def test_pool_nan_first_nan_wins(abi):
+def test_pool_nan_first_nan_wins(pools):
     x = np.array([[1.0, np.nan, 5.0, np.nan, 2.0, 3.0]])
-    out = abi.pool_fwd(x, (4,), (1,))
+    out = pools.pool_fwd(x, (4,), (1,))
     want = ora.pool_forward(x, (4,), (1,))
     assert np.array_equal(np.isnan(out), np.isnan(want)) and np.isnan(out).all()
     g = np.array([[2.0, 3.0, 5.0]])
-    assert np.array_equal(abi.pool_bwd(x, g, (4,), (1,)), ora.pool_backward(x, g, (4,), (1,)))
+    assert np.array_equal(pools.pool_bwd(x, g, (4,), (1,)), ora.pool_backward(x, g, (4,), (1,)))
 
 
 @pytest.mark.parametrize("ties", [False, True])
-def test_pool_config2_literal_full_size(abi, ties):
+def test_pool_config2_literal_full_size(pools, ties):
     # x (64,64,56,56) f64, pool 3x3 stride 2, floor placement -> (64,64,27,27);
     # the reference's validator rejects it ((56-3)/2+1 = 27.5), its window helper floors
     rng = np.random.default_rng(1002)
     shape = (64, 64, 56, 56)
     x = rng.integers(0, 8, shape).astype(np.float64) if ties else rng.standard_normal(shape)
     g = rng.standard_normal((64, 64, 27, 27))
-    out = abi.pool_fwd(x, (3, 3), 2)
-    dx = abi.pool_bwd(x, g, (3, 3), 2)
+    out = pools.pool_fwd(x, (3, 3), 2)
+    dx = pools.pool_bwd(x, g, (3, 3), 2)
     want_out, want_dx = direct.pool(x, g, (3, 3), (2, 2))
     assert np.array_equal(bits(out), bits(want_out))
     assert np.array_equal(bits(dx), bits(want_dx))
@@ -147,12 +194,12 @@ def test_pool_config2_literal_full_size(abi, ties):
     assert np.array_equal(bits(dx[sl]), bits(ora.pool_backward(x[sl], g[sl], (3, 3), 2)))
 
 
-def test_pool_config5_shape_full_size(abi):
+def test_pool_config5_shape_full_size(pools):
     rng = np.random.default_rng(1006)
     x = rng.standard_normal((8, 32, 32, 64, 64)).astype(np.float32)
     g = rng.standard_normal((8, 32, 16, 32, 32)).astype(np.float32)
-    out = abi.pool_fwd(x, (2, 2, 2), 2)
-    dx = abi.pool_bwd(x, g, (2, 2, 2), 2)
+    out = pools.pool_fwd(x, (2, 2, 2), 2)
+    dx = pools.pool_bwd(x, g, (2, 2, 2), 2)
     want_out, want_dx = direct.pool(x, g, (2, 2, 2), (2, 2, 2))
     assert np.array_equal(bits(out), bits(want_out))
     assert np.array_equal(bits(dx), bits(want_dx.astype(np.float32)))
@@ -375,6 +422,13 @@ def test_abi_rejects_bad_arguments(abi):
     pdesc, _ = abi.pool_desc((2, 4, 4), np.float32, (2, 2), 2)
     pdesc.nd = 5
     assert lib.mg_maxpool_fwd(pdesc, 1, 1) == _hip.MG_ERR_UNSUPPORTED
+    pdesc, _ = abi.pool_desc((2, 4, 4), np.float32, (2, 2), 2)
+    assert lib.mg_maxpool_fwd_argmax(pdesc, 1, 1, None) == _hip.MG_ERR_BAD_ARG
+    assert lib.mg_maxpool_bwd_argmax(pdesc, None, 1, 1) == _hip.MG_ERR_BAD_ARG
+    wide, _ = abi.pool_desc((2, 20, 20), np.float32, (17, 16), 1)  # 272 positions: more than a byte tells apart
+    assert lib.mg_maxpool_fwd_argmax(wide, 1, 1, 1) == _hip.MG_ERR_UNSUPPORTED
+    assert lib.mg_maxpool_bwd_argmax(wide, 1, 1, 1) == _hip.MG_ERR_UNSUPPORTED
+    assert "256" in _hip.last_error()
     huge = ctypes.c_void_p()
     assert lib.mg_malloc(ctypes.byref(huge), 1 << 60) == _hip.MG_ERR_OOM
 
