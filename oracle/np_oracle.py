@@ -24,6 +24,7 @@ Pinning (what holds each function to the reference without importing it):
                    central differences
   pool_forward     three reference known-answer cases + the docstring case
   pool_backward    with a tie, brute-force loops on tie-heavy integer inputs
+  pool_argmax      the docstring tie case read as offsets, first-NaN case, loops
   relu_forward     the reference's docstring vectors (``-0.0`` for negative inputs,
   relu_backward    gradient ``[0, 0, 0, 1, 1]``); one IEEE multiply per element
   multiply, multiply_backward, sum_all, sum_all_backward
@@ -75,6 +76,7 @@ __all__ = [
     "matmul_backward",
     "pool_out_shape",
     "pool_forward",
+    "pool_argmax",
     "pool_backward",
 ]
 

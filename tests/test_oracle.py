@@ -265,6 +265,34 @@ def test_pool_ties_overlap_bit_exact_vs_bruteforce(m, lead):
         assert np.array_equal(d_dx.view(np.uint64), dx_t.view(np.uint64))
 
 
+def test_pool_argmax_is_the_first_of_equal_maxima_in_row_major_window_order():
+    # the reference's docstring case (pooling.py:203-214): window [[2, 7], [5, 7]] holds 7 twice and
+    # its gradient goes to row 1 of x, i.e. to offset 1 of the flattened window, not offset 3
+    x = np.array([[0.0, 10.0, 8.0], [2.0, 7.0, 3.0], [5.0, 7.0, 20.0]])
+    assert np.array_equal(ora.pool_argmax(x, (2, 2), 1), [[1, 0], [1, 3]])
+    # the first NaN wins over everything, also over a later, larger value
+    assert np.array_equal(ora.pool_argmax(np.array([1.0, np.nan, 5.0, np.nan, 2.0, 3.0]), (4,), 1), [1, 0, 1])
+    # against loops: per window, walk it in row-major order and keep the first strict improvement
+    rng = np.random.default_rng(207)
+    for trial in range(8):
+        m = 1 + trial % 3
+        pool = tuple(int(v) for v in rng.integers(1, 4, m))
+        stride = tuple(int(v) for v in rng.integers(1, 4, m))
+        grid = tuple(int(v) for v in rng.integers(1, 4, m))
+        X = tuple((g - 1) * s + p for g, s, p in zip(grid, stride, pool))
+        x = rng.integers(0, 3, (2, *X)).astype(np.float64)
+        got = ora.pool_argmax(x, pool, stride)
+        assert got.shape == (2, *grid)
+        for lead in range(2):
+            for g in np.ndindex(*grid):
+                best, where = None, -1
+                for k, a in enumerate(np.ndindex(*pool)):
+                    v = x[(lead, *(gi * si + ai for gi, si, ai in zip(g, stride, a)))]
+                    if best is None or v > best:
+                        best, where = v, k
+                assert got[(lead, *g)] == where
+
+
 def test_pool_accumulation_order_is_sequential_from_plus_zero():
     # one input element wins three overlapping windows; a sequential sum keeps
     # the 1.0 that a pairwise/reordered sum would lose
