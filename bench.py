@@ -310,6 +310,13 @@ def run_gpu(name, steps, warmup):
     dominant = max((k for k in kernels if k in step.work), key=lambda k: kernels[k]["avg_ms"] * kernels[k]["launches"])
     dom = kernels[dominant]
     ms_per_step = elapsed * 1e3 / steps
+    traffic = measured_traffic(name, dominant)
+    extra = {}
+    if step.bound == "hbm" and traffic:
+        # the rate at which bytes really crossed HBM: below `achieved` where a kernel avoids part
+        # of the algorithmic bytes (the pool backward pass that routes from the recorded argmax)
+        extra["moved"] = traffic * step.scale / (dom["avg_ms"] * 1e-3)
+        extra["moved_frac"] = extra["moved"] / step.peak
     return {
         "value": step.total_work * step.scale / (elapsed / steps),
         "unit": step.unit,
@@ -322,9 +329,10 @@ def run_gpu(name, steps, warmup):
             "peak": step.peak,
             "unit": step.unit,
             "frac": dom["frac"],
-            "traffic": measured_traffic(name, dominant),
+            "traffic": traffic,
             "avg_kernel_ms": dom["avg_ms"],
             "work_per_launch": step.work[dominant],
+            **extra,
         },
         "kernels": kernels,
     }

@@ -229,6 +229,18 @@ int mg_batchnorm_fwd(const mg_bn_desc *desc, const void *x, const void *gamma, c
 int mg_batchnorm_bwd(const mg_bn_desc *desc, const void *x, const void *grad, const void *gamma, const void *mean,
                      const void *var, void *dx, void *dgamma, void *dbeta);
 
+/* ---- sums over some of the axes ----
+ * x is seen as (outer, n, inner), C-contiguous (the caller merges neighbouring axes that are
+ * all summed or all kept).  over_middle = 1: out[o, i] = sum_m x[o, m, i], out:(outer, inner).
+ * over_middle = 0: out[m] = sum_{o, i} x[o, m, i], out:(n).  Carried in double over a fixed
+ * partition, rounded once; run-to-run identical.  More than one kept and one summed group on
+ * each side takes several calls.
+ * Replaces np.sum(a, axis=...) in Sum.__call__ (Sequential.__call__,
+ * src/mygrad/operation_base.py:400-452, src/mygrad/math/sequential/ops.py:120-121) and the
+ * sums of reduce_broadcast (src/mygrad/_utils/__init__.py:131-168) behind a broadcasting
+ * Multiply. */
+int mg_sum_over(int dtype, int64_t outer, int64_t n, int64_t inner, int over_middle, const void *x, void *out);
+
 /* ---- matrix product ---- */
 
 /* out[b] = a @ x[b], a:(M, K) shared by the batch, x:(batch, K, N), out:(batch, M, N), all

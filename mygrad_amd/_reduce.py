@@ -1,0 +1,84 @@
+"""Sums over axes and broadcasts on device buffers, in terms of the two kernels that do
+them: ``mg_sum_over`` (a C-contiguous array seen as ``(outer, n, inner)``, summed over the
+middle axis or over the outer and inner ones) and ``mg_repeat_fwd`` (an axis of length one
+repeated).  Neighbouring axes that are treated alike are merged first, so the usual
+cases -- a bias gradient, a per-channel scale, a reduction over the last axes -- take one
+launch; anything else takes one launch per remaining group of axes.
+"""
+
+import numpy as np
+
+from . import _device, _hip
+
+__all__ = ["sum_axes", "broadcast"]
+
+
+def _merge(pairs):
+    """``[(size, kind), ...]`` without the axes of length one and with neighbours of one kind
+    multiplied together."""
+    merged = []
+    for size, kind in pairs:
+        if size == 1:
+            continue
+        if merged and merged[-1][1] == kind:
+            merged[-1][0] *= size
+        else:
+            merged.append([int(size), kind])
+    return merged
+
+
+def _product(groups):
+    total = 1
+    for size, _ in groups:
+        total *= size
+    return total
+
+
+def sum_axes(buf, shape, axes, dtype):
+    """Device buffer with ``x.sum(axis=axes)`` of the C-contiguous ``x`` of ``shape`` in
+    ``buf`` (``axes``: normalised, unique).  The array must not be empty."""
+    lib, code = _hip.lib(), _hip.dtype_code(dtype)
+    summed = set(axes)
+    groups = _merge([(size, axis in summed) for axis, size in enumerate(shape)])
+    while any(kind for _, kind in groups):
+        kinds = [kind for _, kind in groups]
+        if kinds in ([True], [True, False], [False, True], [True, False, True]):
+            # one kept group at most, summed groups around it: a single pass
+            if kinds == [True]:
+                outer, n, inner = groups[0][0], 1, 1
+            elif kinds == [True, False]:
+                outer, n, inner = groups[0][0], groups[1][0], 1
+            elif kinds == [False, True]:
+                outer, n, inner = 1, groups[0][0], groups[1][0]
+            else:
+                outer, n, inner = (g[0] for g in groups)
+            out = _device.DeviceBuffer(max(n * dtype.itemsize, 16))
+            _hip.check(lib.mg_sum_over(code, outer, n, inner, 0, buf.ptr, out.ptr))
+            return out
+        # several kept groups: take out the largest summed group, the rest next time round
+        j = max((i for i, (_, kind) in enumerate(groups) if kind), key=lambda i: groups[i][0])
+        outer, n, inner = _product(groups[:j]), groups[j][0], _product(groups[j + 1 :])
+        out = _device.DeviceBuffer(max(outer * inner * dtype.itemsize, 16))
+        _hip.check(lib.mg_sum_over(code, outer, n, inner, 1, buf.ptr, out.ptr))
+        buf = out
+        groups = _merge([tuple(g) for g in groups[:j] + groups[j + 1 :]])
+    return buf
+
+
+def broadcast(buf, shape, to_shape, dtype):
+    """Device buffer with ``np.broadcast_to(x, to_shape)`` made contiguous, for the
+    C-contiguous ``x`` of ``shape`` in ``buf``.  ``to_shape`` must not be empty of elements."""
+    shape = (1,) * (len(to_shape) - len(shape)) + tuple(shape)
+    groups = _merge([(to, "copy" if have == to else "grow") for have, to in zip(shape, to_shape)])
+    lib = _hip.lib()
+    current = [size if kind == "copy" else 1 for size, kind in groups]
+    for j, (size, kind) in enumerate(groups):
+        if kind != "grow":
+            continue
+        outer = int(np.prod(current[:j], dtype=np.int64))
+        inner = int(np.prod(current[j + 1 :], dtype=np.int64))
+        out = _device.DeviceBuffer(max(outer * size * inner * dtype.itemsize, 16))
+        _hip.check(lib.mg_repeat_fwd(dtype.itemsize, outer, 1, inner, size, size, None, buf.ptr, out.ptr))
+        buf = out
+        current[j] = size
+    return buf

@@ -53,6 +53,7 @@ struct BnParams {
   int chunk;      // ROWS*: elements of a channel per block; COLS: rows per block
   int terms;      // partial sums per channel: chunks (ROWS*) or chunks * S (COLS)
   FastDivB by_s;  // division by S
+  int c0;         // row walks: channel of blockIdx.y == 0 (launches of at most 65535 channels each)
   double eps;
   int has_gamma, has_beta;
 };
@@ -96,7 +97,7 @@ __device__ __forceinline__ int my_channel(const BnParams &p, bool *active) {
     return (int)p.by_s.div((unsigned)min(j, p.J - 1));
   } else {
     *active = true;
-    return blockIdx.y;
+    return p.c0 + blockIdx.y;
   }
 }
 
@@ -111,7 +112,7 @@ __device__ __forceinline__ void visit(const BnParams &p, F f) {
     for (int n = first; n < last; ++n) f((long long)n * p.J + j);
   } else {
     constexpr int VEC = WALK == ROWS_WIDE ? Wide<T>::N : 1;
-    const int c = blockIdx.y;
+    const int c = p.c0 + blockIdx.y;
     const int begin = blockIdx.x * p.chunk, end = min(begin + p.chunk, p.M);
 #pragma unroll 4
     for (int e = begin + (int)threadIdx.x * VEC; e < end; e += 256 * VEC) {
@@ -367,11 +368,102 @@ __global__ void __launch_bounds__(256) bn_bwd_apply_kernel(BnParams p, const T *
   });
 }
 
-int make_params(const mg_bn_desc *d, BnParams *p, const char *who) {
+// ------------------------------------------------------------------------------------------
+// Plain sums over the same walks: out[c] = sum over n and s of x[n, c, s], carried in double
+// over the same fixed partition and trees as the statistics above.
+// ------------------------------------------------------------------------------------------
+template <typename T, int WALK>
+__global__ void __launch_bounds__(256) axis_sum_kernel(BnParams p, const T *__restrict__ x, double *__restrict__ partial) {
+  typedef typename Wide<T>::type V;
+  __shared__ double slots[8];
+  bool active;
+  const int c = my_channel<WALK>(p, &active);
+  double even = 0.0, odd = 0.0;  // two running sums, added at the end
+  if (active)
+    visit<T, WALK>(p, [&](long long at) {
+      if constexpr (WALK == ROWS_WIDE) {
+        const V v = *reinterpret_cast<const V *>(x + at);
+#pragma unroll
+        for (int k = 0; k < Wide<T>::N; k += 2) {
+          even += (double)v[k];
+          odd += (double)v[k + 1];
+        }
+      } else {
+        even += (double)x[at];
+      }
+    });
+  put_partial<WALK>(p, c, active, even, odd, partial, slots);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) axis_sum_finish_kernel(BnParams p, const double *__restrict__ partial, T *__restrict__ out) {
+  const int c = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (c >= p.C) return;
+  double even, odd;
+  channel_totals(p, c, partial, &even, &odd);
+  if ((threadIdx.x & 63) == 0) out[c] = (T)(even + odd);
+}
+
+// out[o, i] = sum over m of x[o, m, i] for x:(outer, n, inner).  A thread owns VEC consecutive
+// i of one o and walks `chunk` of the n entries of the middle axis, inner elements apart;
+// lanes are consecutive in i, so each step of the walk is one coalesced access.  With more
+// than one chunk the sums go to `partial` as doubles and a second kernel adds them in order.
+struct MiddleParams {
+  long long outer, outs;  // outs = outer * inner, results
+  int n, inner;
+  int chunk, chunks;
+};
+
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256) sum_middle_kernel(MiddleParams p, const T *__restrict__ x, T *__restrict__ out,
+                                                         double *__restrict__ partial) {
+  typedef T V __attribute__((ext_vector_type(VEC)));
+  const long long piece = (long long)blockIdx.x * 256 + threadIdx.x;
+  const int per_row = p.inner / VEC;
+  if (piece >= p.outer * per_row) return;
+  const long long o = piece / per_row;
+  const int i = (int)(piece - o * per_row) * VEC;
+  const int first = blockIdx.y * p.chunk, last = min(first + p.chunk, p.n);
+  const T *src = x + (o * p.n + first) * p.inner + i;
+  double acc[VEC];
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) acc[k] = 0.0;
+#pragma unroll 4
+  for (int m = first; m < last; ++m) {
+    if constexpr (VEC == 1) {
+      acc[0] += (double)*src;
+    } else {
+      const V v = *reinterpret_cast<const V *>(src);
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) acc[k] += (double)v[k];
+    }
+    src += p.inner;
+  }
+  const long long at = o * p.inner + i;
+  if (p.chunks == 1) {
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) out[at + k] = (T)acc[k];
+  } else {
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) partial[(long long)blockIdx.y * p.outs + at + k] = acc[k];
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) sum_middle_finish_kernel(MiddleParams p, const double *__restrict__ partial, T *__restrict__ out) {
+  const long long e = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= p.outs) return;
+  double total = 0.0;
+  for (int c = 0; c < p.chunks; ++c) total += partial[(long long)c * p.outs + e];
+  out[e] = (T)total;
+}
+
+// many_channels: the caller cuts its launches to the grid's y extent of 65535 itself
+int make_params(const mg_bn_desc *d, BnParams *p, const char *who, bool many_channels = false) {
   if (!d) return fail(MG_ERR_BAD_ARG, "%s: descriptor is null", who);
   if (d->dtype != MG_F32 && d->dtype != MG_F64) return fail(MG_ERR_UNSUPPORTED, "%s: dtype %d (only float32=0 / float64=1)", who, d->dtype);
   if (d->N < 1 || d->C < 1 || d->S < 1) return fail(MG_ERR_BAD_ARG, "%s: N=%lld C=%lld S=%lld must be positive", who, (long long)d->N, (long long)d->C, (long long)d->S);
-  if (d->N * d->S >= (1ll << 31) || d->C * d->S >= (1ll << 31) || d->C > 65535)
+  if (d->N * d->S >= (1ll << 31) || d->C * d->S >= (1ll << 31) || (d->C > 65535 && !many_channels))
     return fail(MG_ERR_UNSUPPORTED, "%s: 2^31 or more elements per channel or per batch entry, or more than 65535 channels", who);
   if (!(d->eps >= 0.0)) return fail(MG_ERR_BAD_ARG, "%s: eps = %g must be non-negative", who, d->eps);
   p->N = (int)d->N;
@@ -383,6 +475,7 @@ int make_params(const mg_bn_desc *d, BnParams *p, const char *who) {
   p->has_gamma = d->has_gamma != 0;
   p->has_beta = d->has_beta != 0;
   p->by_s = make_fastdiv_b((unsigned)d->S);
+  p->c0 = 0;
   const long long slots = 16ll * runtime().props.multiProcessorCount;  // blocks wanted: 16 per compute unit
   if (d->S < 64) {
     // short rows: walk columns.  32 to 256 rows per block: enough blocks to fill the device
@@ -476,6 +569,67 @@ int bwd_impl(const BnParams &p, const void *x, const void *grad, const void *gam
   return MG_OK;
 }
 
+// out[c] = sum over n, s of x[n, c, s]
+template <typename T>
+int axis_sum_impl(BnParams p, const void *x, void *out) {
+  hipStream_t s = runtime().stream;
+  void *partial = nullptr;
+  if (int rc = workspace((size_t)p.C * p.terms * 2 * sizeof(double), &partial)) return rc;
+  const dim3 block(256);
+  const int walk = walk_for(p, sizeof(T), {x});
+  ScopedTiming timed(TAG_SUM_OVER);
+  if (p.walk == COLS) {
+    const dim3 grid = grid_for(p);
+    MG_BN_LAUNCH(axis_sum_kernel, walk, p, (const T *)x, (double *)partial);
+  } else {
+    const int channels = p.C;
+    for (int c0 = 0; c0 < channels; c0 += 65535) {  // the grid's y extent
+      p.c0 = c0;
+      const dim3 grid((unsigned)p.chunks, (unsigned)std::min(65535, channels - c0));
+      MG_BN_LAUNCH(axis_sum_kernel, walk, p, (const T *)x, (double *)partial);
+    }
+    p.c0 = 0;
+  }
+  hipLaunchKernelGGL(axis_sum_finish_kernel<T>, dim3((unsigned)ceil_div(p.C, 4)), block, 0, s, p, (const double *)partial, (T *)out);
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
+// out[o, i] = sum over m of x[o, m, i]
+template <typename T>
+int middle_sum_impl(long long outer, long long n, long long inner, const void *x, void *out) {
+  hipStream_t s = runtime().stream;
+  constexpr int WIDE = 16 / sizeof(T);
+  const bool wide = inner % WIDE == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  const int vec = wide ? WIDE : 1;
+  MiddleParams p;
+  p.outer = outer;
+  p.outs = outer * inner;
+  p.n = (int)n;
+  p.inner = (int)inner;
+  const long long blocks = ceil_div(outer * (inner / vec), 256);
+  // few results and a long middle axis: cut the axis so that about four blocks per compute
+  // unit are in flight, no piece shorter than 16 entries
+  const long long want = 4ll * runtime().props.multiProcessorCount;
+  long long chunks = std::max<long long>(1, std::min<long long>(ceil_div(want, blocks), n / 16));
+  chunks = std::min<long long>(chunks, 65535);
+  p.chunk = (int)ceil_div(n, chunks);
+  p.chunks = (int)ceil_div(n, p.chunk);
+  void *partial = nullptr;
+  if (p.chunks > 1)
+    if (int rc = workspace((size_t)p.chunks * p.outs * sizeof(double), &partial)) return rc;
+  const dim3 grid((unsigned)blocks, (unsigned)p.chunks), block(256);
+  ScopedTiming timed(TAG_SUM_OVER);
+  if (wide)
+    hipLaunchKernelGGL((sum_middle_kernel<T, WIDE>), grid, block, 0, s, p, (const T *)x, (T *)out, (double *)partial);
+  else
+    hipLaunchKernelGGL((sum_middle_kernel<T, 1>), grid, block, 0, s, p, (const T *)x, (T *)out, (double *)partial);
+  if (p.chunks > 1)
+    hipLaunchKernelGGL(sum_middle_finish_kernel<T>, dim3((unsigned)ceil_div(p.outs, 256)), block, 0, s, p, (const double *)partial, (T *)out);
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
 #undef MG_BN_LAUNCH
 
 }  // namespace
@@ -506,6 +660,29 @@ int mg_batchnorm_bwd(const mg_bn_desc *desc, const void *x, const void *grad, co
   if (!dx && !dgamma && !dbeta) return fail(MG_ERR_BAD_ARG, "mg_batchnorm_bwd: nothing to compute (dx, dgamma and dbeta are all null)");
   return desc->dtype == MG_F32 ? bwd_impl<float>(p, x, grad, gamma, mean, var, dx, dgamma, dbeta)
                                : bwd_impl<double>(p, x, grad, gamma, mean, var, dx, dgamma, dbeta);
+}
+
+int mg_sum_over(int dtype, int64_t outer, int64_t n, int64_t inner, int over_middle, const void *x, void *out) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (dtype != MG_F32 && dtype != MG_F64) return fail(MG_ERR_UNSUPPORTED, "mg_sum_over: dtype %d (only float32=0 / float64=1)", dtype);
+  if (outer < 1 || n < 1 || inner < 1)
+    return fail(MG_ERR_BAD_ARG, "mg_sum_over: outer=%lld n=%lld inner=%lld must be positive", (long long)outer, (long long)n, (long long)inner);
+  if (!x || !out) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_sum_over");
+  if (over_middle) {
+    if (n >= (1ll << 31) || inner >= (1ll << 31) || ceil_div(outer * inner, 256) >= (1ll << 31))
+      return fail(MG_ERR_UNSUPPORTED, "mg_sum_over: an axis of 2^31 or more entries, or 2^39 or more results");
+    return dtype == MG_F32 ? middle_sum_impl<float>(outer, n, inner, x, out) : middle_sum_impl<double>(outer, n, inner, x, out);
+  }
+  mg_bn_desc desc{};
+  desc.dtype = dtype;
+  desc.N = outer;
+  desc.C = n;
+  desc.S = inner;
+  desc.eps = 0.0;
+  BnParams p;
+  if (int rc = make_params(&desc, &p, "mg_sum_over", true)) return rc;
+  return dtype == MG_F32 ? axis_sum_impl<float>(p, x, out) : axis_sum_impl<double>(p, x, out);
 }
 
 }  // extern "C"

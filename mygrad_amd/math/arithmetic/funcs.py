@@ -10,7 +10,7 @@ def multiply(x1, x2, *, constant=None):
     Parameters
     ----------
     x1, x2 : ArrayLike
-        Operands of the same shape, float32 or float64.
+        float32 or float64 operands that broadcast against each other.
     constant : Optional[bool]
         If True, the resulting Tensor is a constant.
 
@@ -26,5 +26,9 @@ def multiply(x1, x2, *, constant=None):
     >>> y.backward()
     >>> x.grad
     array([2., 2., 2.])
+    >>> scale = mg.Tensor([10.0, 100.0])
+    >>> mg.multiply(mg.Tensor([[1.0, 2.0], [3.0, 4.0]]), scale).backward()
+    >>> scale.grad   # summed over the axis it was broadcast along
+    array([4., 6.])
     """
     return Tensor._op(Multiply, x1, x2, constant=constant)

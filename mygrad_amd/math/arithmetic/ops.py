@@ -1,57 +1,78 @@
 """``Multiply`` on the MI355X (reference: ``mygrad/math/arithmetic/ops.py:45-53``).
 
 The reference's ``Multiply`` is ``np.multiply`` with broadcasting and gradients
-``grad * other``.  This build runs the case that occurs between the convolution /
-pooling kernels -- two operands of the same shape and floating-point dtype -- as one
-bandwidth-bound kernel; other argument patterns raise (there is no CPU fallback)."""
+``grad * other``, summed back to the operand's shape over the axes it was broadcast along
+(``mygrad/_utils/__init__.py:131-168``).  Operands of one shape -- the case between the
+convolution / pooling kernels -- take one bandwidth-bound kernel; an operand that is
+broadcast is first spread to the common shape on the device, and its gradient is summed
+back there (carried in double, rounded once: equal to NumPy's pairwise sum to rounding).
+Floating-point operands only; other argument patterns raise (there is no CPU fallback)."""
 
 import numpy as np
 
-from ... import _device, _hip
+from ... import _device, _hip, _reduce
 from ...operation_base import Operation
 
 __all__ = ["Multiply"]
 
 
-def _same_shape_floats(op, a, b):
-    if a.shape != b.shape:
-        raise NotImplementedError(
-            f"{op} on the GPU takes operands of one shape, got {a.shape} and {b.shape} "
-            "(broadcasting is not part of this build; there is no CPU fallback)"
-        )
+def _float_dtype(op, a, b):
     dtype = np.result_type(a, b)
     if dtype not in (np.float32, np.float64):
         raise TypeError(f"{op} runs on the GPU in float32 or float64, got {a.dtype} and {b.dtype} (there is no CPU fallback)")
     return np.dtype(dtype)
 
 
-def device_multiply(a, b, dtype):
-    """``a * b`` for two same-shape host arrays -> (host result, its device buffer)."""
-    ab, bb = _device.to_device(a, dtype), _device.to_device(b, dtype)
-    ob = _device.DeviceBuffer(max(a.size * dtype.itemsize, 16))
-    _hip.check(_hip.lib().mg_multiply(_hip.dtype_code(dtype), a.size, ab.ptr, bb.ptr, ob.ptr))
-    return _device.download(ob, a.shape, dtype), ob
+def _spread(arr, shape, dtype):
+    """Device buffer with ``arr`` cast to ``dtype`` and broadcast to ``shape``."""
+    buf = _device.to_device(arr, dtype)
+    return buf if arr.shape == tuple(shape) else _reduce.broadcast(buf, arr.shape, shape, dtype)
+
+
+def device_multiply(a, b, dtype, shape=None):
+    """``a * b`` for two host arrays that broadcast to ``shape`` -> (host result, its device buffer)."""
+    shape = a.shape if shape is None else tuple(shape)
+    size = int(np.prod(shape, dtype=np.int64))
+    if size == 0:
+        return np.empty(shape, dtype=dtype), None
+    ab, bb = _spread(a, shape, dtype), _spread(b, shape, dtype)
+    ob = _device.DeviceBuffer(max(size * dtype.itemsize, 16))
+    _hip.check(_hip.lib().mg_multiply(_hip.dtype_code(dtype), size, ab.ptr, bb.ptr, ob.ptr))
+    return _device.download(ob, shape, dtype), ob
 
 
 class Multiply(Operation):
-    """``f(a, b) -> a * b`` element-wise."""
+    """``f(a, b) -> a * b`` element-wise, with NumPy's broadcasting."""
 
     gradient_on_device = True
 
     def __call__(self, a, b):
         self.variables = (a, b)
-        dtype = _same_shape_floats("multiply", a.data, b.data)
+        dtype = _float_dtype("multiply", a.data, b.data)
         self._dtype = dtype
-        out, ob = device_multiply(a.data, b.data, dtype)
-        _device.attach(out, ob)
+        self._shape = np.broadcast_shapes(a.shape, b.shape)  # ValueError for shapes that do not go together
+        out, ob = device_multiply(a.data, b.data, dtype, self._shape)
+        if ob is not None:
+            _device.attach(out, ob)
         return out
 
     def backward_var(self, grad, index, **kwargs):
         a, b = self.variables
-        other = b.data if index == 0 else a.data
-        dtype = np.dtype(np.result_type(grad, other))
-        if grad.shape != other.shape or dtype not in (np.float32, np.float64):
+        var, other = (a, b) if index == 0 else (b, a)
+        dtype = np.dtype(np.result_type(grad, other.data))
+        if grad.shape != self._shape or dtype not in (np.float32, np.float64):
             raise NotImplementedError(f"multiply backward for gradient {grad.shape} {grad.dtype} (no CPU fallback)")
-        out, ob = device_multiply(grad, other, dtype)
-        _device.attach_transient(out, ob)
-        return out
+        out, ob = device_multiply(grad, other.data, dtype, self._shape)
+        if ob is None:
+            return np.zeros(var.shape, dtype=dtype)
+        if var.shape == self._shape:
+            _device.attach_transient(out, ob)
+            return out
+        # the operand was broadcast: add its gradient up over the axes it was spread along
+        # (reduce_broadcast: the leading axes it lacks and those where it has length one)
+        lead = len(self._shape) - var.ndim
+        axes = tuple(range(lead)) + tuple(lead + i for i, n in enumerate(var.shape) if n == 1 and self._shape[lead + i] != 1)
+        rb = _reduce.sum_axes(ob, self._shape, axes, dtype)
+        back = _device.download(rb, var.shape, dtype)
+        _device.attach_transient(back, rb)
+        return back

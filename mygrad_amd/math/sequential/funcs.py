@@ -5,17 +5,17 @@ __all__ = ["sum"]
 
 
 def sum(x, axis=None, keepdims=False, *, constant=None):  # noqa: A001
-    """Sum of all tensor elements (reference: ``mygrad.sum``).
+    """Sum of tensor elements over the given axes (reference: ``mygrad.sum``).
 
     Parameters
     ----------
     x : ArrayLike
         float32 or float64.
-    axis : None
-        Only the full reduction runs on the GPU; anything else raises
-        ``NotImplementedError``.
+    axis : Optional[int, Tuple[int, ...]]
+        The axis or axes to sum over, counted from the end when negative; ``None`` sums
+        over all of them.
     keepdims : bool
-        Keep the reduced axes with length one.
+        Keep the summed axes with length one, so that the result broadcasts against ``x``.
     constant : Optional[bool]
         If True, the resulting Tensor is a constant.
 
@@ -30,5 +30,7 @@ def sum(x, axis=None, keepdims=False, *, constant=None):  # noqa: A001
     >>> mg.sum(x).backward()
     >>> x.grad
     array([1., 1., 1.])
+    >>> mg.sum(mg.Tensor([[1.0, 2.0], [3.0, 4.0]]), axis=0)
+    Tensor([4., 6.])
     """
     return Tensor._op(Sum, x, op_args=(axis, keepdims), constant=constant)

@@ -31,6 +31,11 @@ Pinning (what holds each function to the reference without importing it):
                    single calls of the NumPy routine the reference calls
                    (``np.multiply``, ``np.sum``, ``np.full``); ``sum_all`` is
                    additionally held to ``math.fsum`` and closed forms in the tests
+  sum_axes, sum_axes_backward, reduce_broadcast, multiply_broadcast_backward
+                   ``np.sum`` itself, held to ``math.fsum`` per kept entry and to loops;
+                   the two gradients to loops over every index and to the adjoint
+                   identities <sum(x), g> = <x, backward(g)> and
+                   <a * b, g> = <a, grad_a> = <b, grad_b>
   batchnorm_forward
                    the reference's docstring vector; its tests' second formulation
                    (mean / variance / division composed of primitives); closed forms
@@ -75,6 +80,10 @@ __all__ = [
     "matmul_forward",
     "matmul_backward",
     "pool_out_shape",
+    "sum_axes",
+    "sum_axes_backward",
+    "reduce_broadcast",
+    "multiply_broadcast_backward",
     "pool_forward",
     "pool_argmax",
     "pool_backward",
@@ -373,6 +382,53 @@ def relu_backward(x, grad):
     """``ReLu.backward_var``: ``grad * back`` with ``back`` the forward pass's 0/1 mask
     (mygrad/nnet/activations/relu.py:16-17)."""
     return grad * np.asarray(x > 0, dtype=x.dtype)
+
+
+def sum_axes(x, axis=None, keepdims=False):
+    """``Sum.__call__``: ``np.sum(x, axis=axis, keepdims=keepdims)``
+    (mygrad/operation_base.py:400-452 with ``numpy_func = np.sum``,
+    mygrad/math/sequential/ops.py:120-121)."""
+    return np.sum(x, axis=axis, keepdims=keepdims)
+
+
+def sum_axes_backward(x, grad, axis=None, keepdims=False):
+    """``Sum.backward_var`` (mygrad/math/sequential/ops.py:123-133): ``np.full`` for a sum
+    over everything; otherwise the summed axes are put back into ``grad`` as axes of length
+    one (unless they were kept) and the result is broadcast to ``x.shape``."""
+    if axis is None:
+        return np.full(x.shape, grad, dtype=x.dtype)
+    axes = axis if hasattr(axis, "__iter__") else (axis,)
+    grad = np.asarray(grad)
+    if not keepdims:
+        index = [slice(None)] * x.ndim
+        for i in axes:
+            index[i] = np.newaxis
+        grad = grad[tuple(index)]
+    return np.broadcast_to(grad, x.shape).astype(x.dtype, copy=False)
+
+
+def reduce_broadcast(grad, var_shape):
+    """Sum ``grad`` back to the shape of an operand that was broadcast
+    (mygrad/_utils/__init__.py:131-168): first over the leading axes the operand lacks, then,
+    keeping them, over the axes where the shapes differ."""
+    if grad.shape == tuple(var_shape):
+        return grad
+    if grad.ndim != len(var_shape):
+        if grad.ndim < len(var_shape):
+            raise ValueError("the gradient has fewer axes than the operand it belongs to")
+        grad = grad.sum(axis=tuple(range(grad.ndim - len(var_shape))))
+    keep = tuple(n for n, i in enumerate(grad.shape) if i != var_shape[n])
+    if keep:
+        grad = grad.sum(axis=keep, keepdims=True)
+    return grad
+
+
+def multiply_broadcast_backward(grad, a, b, index):
+    """What reaches operand ``index`` of a broadcasting ``Multiply``: ``grad * other``
+    (mygrad/math/arithmetic/ops.py:48-53) summed back to the operand's shape by
+    ``Operation.backward`` (mygrad/operation_base.py:89-97, :213)."""
+    var, other = (a, b) if index == 0 else (b, a)
+    return reduce_broadcast(grad * other, var.shape)
 
 
 def sum_all(x):

@@ -136,6 +136,16 @@ def relu_bwd(x, grad):
     return _down(ob, x.shape, x.dtype)
 
 
+def sum_over(x3, over_middle):
+    """x3:(outer, n, inner) -> sums over the middle axis (outer, inner) or over the other two (n,)."""
+    outer, n, inner = x3.shape
+    xb = _up(x3)
+    out_shape = (outer, inner) if over_middle else (n,)
+    ob = _device.DeviceBuffer(max(int(np.prod(out_shape)) * x3.dtype.itemsize, 16))
+    _hip.check(_hip.lib().mg_sum_over(_hip.dtype_code(x3.dtype), outer, n, inner, int(over_middle), xb.ptr, ob.ptr))
+    return _down(ob, out_shape, x3.dtype)
+
+
 def sum_all(x):
     xb = _up(x)
     ob = _device.DeviceBuffer(16)

@@ -84,6 +84,124 @@ def test_sum_closed_forms_and_fill(abi):
             assert np.array_equal(abi.fill_from(2.5, shape, dtype), want)
 
 
+SUM_OVER_SHAPES = [
+    (1, 1, 1), (3, 1, 5), (1, 7, 1), (5, 3, 1), (1, 4, 9), (6, 5, 4), (2, 3, 64), (128, 64, 3136 // 16),
+    (70000, 3, 1), (1, 70000, 3), (4, 70000, 64), (3, 2, 100003), (40000, 5, 2), (2, 100000, 4), (1, 1000, 1000),
+    (500, 33, 130), (9, 4000, 7),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("shape", SUM_OVER_SHAPES)
+def test_sum_over_both_forms_against_exact_sums(abi, dtype, shape):
+    """mg_sum_over: x:(outer, n, inner) summed over the middle axis, and over the two outer
+    ones.  Bar: |got - exact| <= 1e-6 (float32) / 1e-14 (float64) of the sum of magnitudes
+    of what was added, the exact sum being NumPy's in extended precision; and the same
+    against np.sum in the array's own precision, with twice the allowance."""
+    dtype = np.dtype(dtype)
+    rng = np.random.default_rng(list(shape))
+    x = (rng.standard_normal(shape) * 10.0 ** rng.integers(-2, 3, shape)).astype(dtype)
+    wide = x.astype(np.longdouble)
+    for over_middle, axes in ((True, (1,)), (False, (0, 2))):
+        got = abi.sum_over(x, over_middle)
+        exact = wide.sum(axis=axes)
+        scale = np.abs(wide).sum(axis=axes) + 1e-300
+        assert got.dtype == dtype and got.shape == exact.shape
+        assert np.all(np.abs(got - exact) <= SUM_TOL[dtype] * scale)
+        assert np.all(np.abs(got - ora.sum_axes(x, axes)) <= 2 * SUM_TOL[dtype] * scale)
+        assert np.array_equal(bits(abi.sum_over(x, over_middle)), bits(got))  # the same partition and trees every run
+
+
+def test_sum_over_closed_forms_and_bad_arguments(abi):
+    from mygrad_amd import _device, _hip
+
+    x = np.arange(2 * 3 * 4, dtype=np.float64).reshape(2, 3, 4)
+    assert np.array_equal(abi.sum_over(x, True), x.sum(axis=1))
+    assert np.array_equal(abi.sum_over(x, False), x.sum(axis=(0, 2)))
+    ones = np.ones((300, 70, 50), dtype=np.float32)
+    assert np.array_equal(abi.sum_over(ones, True), np.full((300, 50), 70.0, np.float32))
+    assert np.array_equal(abi.sum_over(ones, False), np.full(70, 15000.0, np.float32))
+    nan = np.ones((4, 3, 5))
+    nan[2, 1, 3] = np.nan
+    assert np.isnan(abi.sum_over(nan, False)[1]) and np.isnan(abi.sum_over(nan, True)[2, 3])
+    assert np.isnan(abi.sum_over(nan, True)).sum() == 1 and np.isnan(abi.sum_over(nan, False)).sum() == 1
+    buf = _device.DeviceBuffer(64)
+    lib = _hip.lib()
+    assert lib.mg_sum_over(0, 1, 2, 3, 0, None, buf.ptr) == _hip.MG_ERR_BAD_ARG
+    assert lib.mg_sum_over(0, 0, 2, 3, 1, buf.ptr, buf.ptr) == _hip.MG_ERR_BAD_ARG
+    assert lib.mg_sum_over(3, 1, 2, 3, 1, buf.ptr, buf.ptr) == _hip.MG_ERR_UNSUPPORTED
+
+
+TENSOR_SUM_CASES = [
+    ((4, 5), 0, False), ((4, 5), -1, True), ((2, 3, 4), (0, 2), False), ((2, 3, 4), (1,), True), ((2, 1, 3, 2), (1, 3), False),
+    ((3,), None, True), ((2, 3, 2, 2, 3), (1, 3), True), ((2, 3), (), False), ((2, 3, 4, 5, 2), (0, 2, 4), False),
+    ((8, 16, 12, 12), (0, 2, 3), False), ((8, 16, 12, 12), 1, True), ((64, 1000), 0, False), ((64, 1000), 1, False),
+    ((1, 5, 1), (0, 2), False), ((0, 3), 0, False), ((0, 3), 1, True), ((), None, False),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("shape,axis,keepdims", TENSOR_SUM_CASES)
+def test_sum_over_axes_through_the_tensor_api(dtype, shape, axis, keepdims):
+    import mygrad_amd as mg
+
+    dtype = np.dtype(dtype)
+    rng = np.random.default_rng([len(shape), int(np.prod(shape)), 5])
+    xv = rng.standard_normal(shape).astype(dtype)
+    x = mg.Tensor(xv)
+    out = mg.sum(x, axis=axis, keepdims=keepdims)
+    want = ora.sum_axes(xv, axis, keepdims)
+    assert out.shape == want.shape and out.dtype == want.dtype
+    scale = np.abs(xv.astype(np.float64)).sum(axis=axis, keepdims=keepdims)
+    assert np.all(np.abs(out.data.astype(np.float64) - want) <= 2 * SUM_TOL[dtype] * (scale + 1e-300))
+    g = rng.standard_normal(want.shape).astype(dtype)
+    out.backward(g)
+    back = ora.sum_axes_backward(xv, g, axis, keepdims)
+    assert x.grad.dtype == back.dtype and np.array_equal(x.grad, back)  # a copy of values: exact
+
+
+def test_sum_axis_errors_through_the_tensor_api():
+    import mygrad_amd as mg
+
+    x = mg.Tensor(np.ones((2, 3)))
+    with pytest.raises(np.exceptions.AxisError):
+        mg.sum(x, axis=2)
+    with pytest.raises(ValueError):
+        mg.sum(x, axis=(0, 0))
+    assert float(mg.sum(mg.Tensor(3.0), axis=0).data) == 3.0
+
+
+BROADCAST_CASES = [
+    ((4, 5), (5,)), ((4, 5), (4, 1)), ((2, 3, 4), (3, 1)), ((3, 1, 2), (1, 4, 1)), ((2, 3), ()), ((1,), (2, 3)),
+    ((2, 3, 4, 5), (1, 3, 1, 1)), ((5,), (5,)), ((8, 16, 12, 12), (16, 1, 1)), ((64, 1000), (1000,)), ((64, 1000), (64, 1)),
+    ((2, 1, 3, 1, 2), (3, 1, 4, 1)), ((0, 3), (3,)), ((2, 3), (1,)),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("sa,sb", BROADCAST_CASES)
+def test_broadcasting_multiply_through_the_tensor_api(dtype, sa, sb):
+    """The product is one IEEE multiply per element, so it equals NumPy's bit for bit; the
+    gradient of a broadcast operand is a sum, held to the bar of the sums above."""
+    import mygrad_amd as mg
+
+    dtype = np.dtype(dtype)
+    rng = np.random.default_rng([len(sa), len(sb), int(np.prod(sa)) + int(np.prod(sb))])
+    av, bv = rng.standard_normal(sa).astype(dtype), rng.standard_normal(sb).astype(dtype)
+    a, b = mg.Tensor(av), mg.Tensor(bv)
+    out = a * b
+    want = ora.multiply(av, bv)
+    assert out.shape == want.shape and out.dtype == want.dtype and np.array_equal(bits(out.data), bits(want))
+    g = rng.standard_normal(want.shape).astype(dtype)
+    out.backward(g)
+    for index, var in enumerate((a, b)):
+        back = ora.multiply_broadcast_backward(g.astype(np.float64), av.astype(np.float64), bv.astype(np.float64), index)
+        other = bv if index == 0 else av
+        scale = ora.reduce_broadcast(np.abs(g.astype(np.float64) * other), var.shape)
+        assert var.grad.shape == var.shape and var.grad.dtype == dtype
+        assert np.all(np.abs(var.grad - back) <= 4 * SUM_TOL[dtype] * (scale + 1e-300))
+
+
 def test_abi_rejects_bad_arguments(abi):
     from mygrad_amd import _device, _hip
 
@@ -114,10 +232,14 @@ def test_docstring_examples_through_the_tensor_api():
     s.backward()
     assert np.array_equal(a.grad, [4.0, 5.0, 6.0]) and np.array_equal(b.grad, [1.0, 2.0, 3.0])
 
-    with pytest.raises(NotImplementedError):
-        mg.multiply(mg.Tensor(np.ones((2, 3))), np.ones(3))
-    with pytest.raises(NotImplementedError):
-        mg.sum(mg.Tensor(np.ones((2, 3))), axis=0)
+    scale = mg.Tensor([10.0, 100.0])
+    prod = mg.multiply(mg.Tensor([[1.0, 2.0], [3.0, 4.0]]), scale)
+    assert np.array_equal(prod.data, [[10.0, 200.0], [30.0, 400.0]])
+    prod.backward()
+    assert np.array_equal(scale.grad, [4.0, 6.0])
+    assert np.array_equal(mg.sum(mg.Tensor([[1.0, 2.0], [3.0, 4.0]]), axis=0).data, [4.0, 6.0])
+    with pytest.raises(ValueError):
+        mg.multiply(mg.Tensor(np.ones((2, 3))), np.ones(4))
     with pytest.raises(TypeError):
         relu(mg.Tensor(np.arange(4)))
 

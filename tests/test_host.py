@@ -409,8 +409,17 @@ def test_argument_checks_of_the_neighbouring_operations_need_no_device():
     with pytest.raises(NotImplementedError):
         mg.sliding_window_copy(np.ones((2, 2, 2, 2)), (1, 1, 1, 1), 1)
 
-    with pytest.raises(NotImplementedError):
-        mg.multiply(np.ones((2, 3)), np.ones(3))
-    with pytest.raises(NotImplementedError):
-        mg.sum(np.ones((2, 3)), axis=0)
+    with pytest.raises(ValueError):
+        mg.multiply(np.ones((2, 3)), np.ones(4))  # shapes that do not broadcast
+    with pytest.raises(TypeError):
+        mg.multiply(np.ones((2, 3), dtype=np.int64), np.ones(3, dtype=np.int64))
+    assert mg.multiply(np.ones((0, 3)), np.ones(3)).shape == (0, 3)
+    with pytest.raises(np.exceptions.AxisError):
+        mg.sum(np.ones((2, 3)), axis=2)
+    with pytest.raises(ValueError):
+        mg.sum(np.ones((2, 3)), axis=(1, 1))
+    with pytest.raises(TypeError):
+        mg.sum(np.ones((2, 3), dtype=np.int32), axis=0)
+    assert np.array_equal(mg.sum(np.ones((0, 3)), axis=0).data, np.zeros(3))
+    assert mg.sum(np.ones((0, 3)), axis=1, keepdims=True).shape == (0, 1)
     assert _graph.held_count() == 0

@@ -3,6 +3,7 @@ adjoint identity, finite differences, and NumPy library routines on tiny cases.
 A dropped term, a wrong sign/index or a transposed axis list fails one of these."""
 
 import itertools
+import math
 
 import numpy as np
 import pytest
@@ -554,3 +555,79 @@ def test_matmul_backward_by_loops_and_adjoint(sa, sb):
                     loop_da[i, j] += g[i, k] * b[j, k]
                     loop_db[j, k] += a[i, j] * g[i, k]
         assert np.allclose(da, loop_da, atol=1e-13) and np.allclose(db, loop_db, atol=1e-13)
+
+
+# ----------------------------------------------------------------- sums over axes, broadcasting
+SUM_CASES = [((4, 5), 0, False), ((4, 5), -1, True), ((2, 3, 4), (0, 2), False), ((2, 3, 4), (1,), True),
+             ((2, 1, 3, 2), (1, 3), False), ((3,), None, False), ((2, 3, 2, 2, 3), (1, 3), True), ((2, 3), (), False)]
+
+
+@pytest.mark.parametrize("shape,axis,keepdims", SUM_CASES)
+def test_sum_over_axes_against_exact_sums_and_loops(shape, axis, keepdims):
+    rng = np.random.default_rng(len(shape) * 31 + (0 if axis is None else len(np.atleast_1d(axis))))
+    x = rng.standard_normal(shape) * 10.0 ** rng.integers(-3, 4, shape)
+    got = ora.sum_axes(x, axis, keepdims)
+    axes = tuple(range(x.ndim)) if axis is None else tuple(a % x.ndim for a in np.atleast_1d(axis).astype(int))
+    kept = [i for i in range(x.ndim) if i not in axes]
+    want = np.zeros([shape[i] for i in kept])
+    for k in np.ndindex(*want.shape):
+        terms = []
+        for r in np.ndindex(*[shape[i] for i in axes]):
+            full = [0] * x.ndim
+            for i, v in zip(kept, k):
+                full[i] = v
+            for i, v in zip(axes, r):
+                full[i] = v
+            terms.append(x[tuple(full)])
+        want[k] = math.fsum(terms)
+    assert got.shape == (tuple(1 if i in axes else n for i, n in enumerate(shape)) if keepdims else want.shape)
+    assert np.allclose(got.reshape(want.shape), want, rtol=1e-13, atol=1e-13 * np.abs(x).sum())
+
+    # gradient: every element of x receives the gradient of the entry it was added into
+    g = rng.standard_normal(got.shape)
+    back = ora.sum_axes_backward(x, g, axis, keepdims)
+    assert back.shape == x.shape and back.dtype == x.dtype
+    g_kept = g.reshape(want.shape)
+    for full in np.ndindex(*shape):
+        assert back[full] == g_kept[tuple(full[i] for i in kept)]
+    # adjoint identity <sum(x), g> = <x, backward(g)>
+    assert math.isclose(float(np.sum(got * g)), float(np.sum(x * back)), rel_tol=1e-10, abs_tol=1e-10)
+
+
+def test_sum_axis_errors_are_numpys():
+    x = np.zeros((2, 3))
+    with pytest.raises(np.exceptions.AxisError):
+        ora.sum_axes(x, 2)
+    with pytest.raises(ValueError):
+        ora.sum_axes(x, (0, 0))
+    assert ora.sum_axes(np.array(3.0), 0) == 3.0  # NumPy lets a scalar be summed over axis 0
+
+
+BROADCAST_CASES = [((4, 5), (5,)), ((4, 5), (4, 1)), ((2, 3, 4), (3, 1)), ((3, 1, 2), (1, 4, 1)), ((2, 3), ()),
+                   ((1,), (2, 3)), ((2, 3, 4, 5), (1, 3, 1, 1)), ((5,), (5,))]
+
+
+@pytest.mark.parametrize("sa,sb", BROADCAST_CASES)
+def test_broadcast_multiply_gradients_against_loops_and_adjoints(sa, sb):
+    rng = np.random.default_rng(len(sa) * 7 + len(sb))
+    a, b = rng.standard_normal(sa), rng.standard_normal(sb)
+    out = ora.multiply(a, b)
+    shape = np.broadcast_shapes(sa, sb)
+    assert out.shape == shape
+    g = rng.standard_normal(shape)
+    for index, (var, other) in enumerate(((a, b), (b, a))):
+        got = ora.multiply_broadcast_backward(g, a, b, index)
+        assert got.shape == var.shape
+        # loops: walk every element of the result and add its term to the operand entry it read
+        want = np.zeros(var.shape)
+        pad_v = (1,) * (len(shape) - var.ndim) + var.shape
+        pad_o = (1,) * (len(shape) - other.ndim) + other.shape
+        v3, o3 = want.reshape(pad_v), other.reshape(pad_o)
+        for full in np.ndindex(*shape):
+            iv = tuple(0 if n == 1 else i for i, n in zip(full, pad_v))
+            io = tuple(0 if n == 1 else i for i, n in zip(full, pad_o))
+            v3[iv] += g[full] * o3[io]
+        assert np.allclose(got, want, rtol=1e-12, atol=1e-12)
+        assert math.isclose(float(np.sum(out * g)), float(np.sum(var * got)), rel_tol=1e-9, abs_tol=1e-9)
+    with pytest.raises(ValueError):
+        ora.reduce_broadcast(np.zeros(3), (2, 3))
