@@ -65,6 +65,9 @@ WORKLOADS = {
     "bn3a": dict(kind="bn", dtype="f32", seed=1008, x=(128, 64, 56, 56), eps=1e-5),
     # matrix product on the convolution kernels: one dense layer's three products
     "mm4k": dict(kind="matmul", dtype="f32", seed=1011, M=4096, K=4096, N=4096),
+    # sums over axes of a tensor of conv5's output size: per channel (the gradient of a bias or of a
+    # per-channel scale: every axis but axis 1), then over the channel axis alone
+    "sum5": dict(kind="sumover", dtype="f32", seed=1012, x=(8, 32, 32, 64, 64), axes=((0, 2, 3, 4), (1,))),
     # repeat: twofold nearest-neighbour upsampling of the rows of a tensor of pool5's input size
     # (forward and gradient), and then of its columns
     "rep5": dict(kind="repeat", dtype="f32", seed=1009, x=(8, 32, 32, 64, 64), repeats=2, axes=(-2, -1)),
@@ -99,6 +102,8 @@ def describe(name):
         return f"{name}: relu + multiply + sum {wl['dtype']} x{wl['x']} fwd+bwd (7 kernels, 16 |x| bytes)"
     if wl["kind"] == "matmul":
         return f"{name}: matmul {wl['dtype']} ({wl['M']},{wl['K']}) @ ({wl['K']},{wl['N']}): product + both gradients"
+    if wl["kind"] == "sumover":
+        return f"{name}: sum {wl['dtype']} x{wl['x']} over axes {wl['axes'][0]}, then over axes {wl['axes'][1]}"
     if wl["kind"] == "repeat":
         return f"{name}: repeat {wl['dtype']} x{wl['x']} repeats={wl['repeats']} along axis {wl['axes'][0]}, then along axis {wl['axes'][1]}, fwd+bwd each"
     if wl["kind"] == "window":
@@ -161,6 +166,17 @@ class Step:
             self.total_work = 3 * per_pass
             self.unit, self.bound, self.peak = "TFLOP/s", "mfma", PEAK_TFLOPS[wl["dtype"]]
             self.scale = 1e-12
+        elif wl["kind"] == "sumover":
+            x = rng.standard_normal(wl["x"]).astype(dt)
+            outer, n, inner = wl["x"][0], wl["x"][1], int(np.prod(wl["x"][2:]))
+            self.dims, self.code = (outer, n, inner), _hip.dtype_code(dt)
+            self.x = resident(x)
+            self.out = _device.DeviceBuffer(outer * inner * item)
+            # each launch reads x once; what it writes is 1/32 of that at most
+            self.work = {"sum_over": float(x.nbytes)}
+            self.total_work = 2.0 * x.nbytes
+            self.unit, self.bound, self.peak = "GB/s", "hbm", PEAK_HBM_GBS
+            self.scale = 1e-9
         elif wl["kind"] == "repeat":
             x = rng.standard_normal(wl["x"]).astype(dt)
             r = wl["repeats"]
@@ -253,6 +269,10 @@ class Step:
             check(lib.mg_matmul(self.code, *self.dims, self.w.ptr, self.x.ptr, self.out.ptr))
             check(lib.mg_matmul_dx(self.code, *self.dims, self.g.ptr, self.w.ptr, self.dx.ptr))
             check(lib.mg_matmul_da(self.code, *self.dims, self.g.ptr, self.x.ptr, self.dw.ptr))
+            return
+        if self.wl["kind"] == "sumover":
+            check(lib.mg_sum_over(self.code, *self.dims, 0, self.x.ptr, self.out.ptr))
+            check(lib.mg_sum_over(self.code, *self.dims, 1, self.x.ptr, self.out.ptr))
             return
         if self.wl["kind"] == "repeat":
             for outer, n, inner, r, total in self.geometry:
@@ -391,6 +411,15 @@ def run_cpu_baseline(name, min_seconds=10.0, max_reps=200):
 
         work, scale, unit = 6.0 * M * K * N, 1e-12, "TFLOP/s"
         what = "product and both gradients (three BLAS sgemm calls)"
+    elif wl["kind"] == "sumover":
+        x = rng.standard_normal(wl["x"]).astype(dt)
+
+        def once():
+            for axes in wl["axes"]:
+                ora.sum_axes(x, axes)
+
+        work, scale, unit = 2 * x.nbytes, 1e-9, "GB/s"
+        what = "np.sum over each of the two sets of axes"
     elif wl["kind"] == "repeat":
         x = rng.standard_normal(wl["x"]).astype(dt)
         g = rng.standard_normal((*wl["x"][:-1], wl["x"][-1] * wl["repeats"])).astype(dt)
@@ -500,6 +529,13 @@ def run_dropin(name, steps=5):
             (at @ xt).backward(g)
 
         work, scale, unit = 6.0 * M * K * N, 1e-12, "TFLOP/s"
+    elif wl["kind"] == "sumover":
+
+        def once():
+            for axes in wl["axes"]:
+                mg.sum(mg.Tensor(x, copy=False), axis=axes).clear_graph()
+
+        work, scale, unit = 2 * x.nbytes, 1e-9, "GB/s"
     elif wl["kind"] == "repeat":
         g = rng.standard_normal((*wl["x"][:-1], wl["x"][-1] * wl["repeats"])).astype(dt)
 
@@ -630,7 +666,8 @@ def main():
     line = {
         "metric": {"conv": "conv_nd fwd+bwd TFLOP/s", "pool": "max_pool fwd+bwd GB/s",
                    "elem": "relu+multiply+sum fwd+bwd GB/s", "bn": "batchnorm fwd+bwd GB/s",
-                   "repeat": "repeat fwd+bwd GB/s", "matmul": "matmul fwd+bwd TFLOP/s", "window": "sliding-window copy GB/s"}[wl["kind"]],
+                   "repeat": "repeat fwd+bwd GB/s", "matmul": "matmul fwd+bwd TFLOP/s", "window": "sliding-window copy GB/s",
+                   "sumover": "sum over axes GB/s"}[wl["kind"]],
         "value": res["value"],
         "unit": res["unit"],
         "n_gpus": 1,
