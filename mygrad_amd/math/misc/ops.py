@@ -8,12 +8,13 @@ implicit-GEMM kernels (``mg_matmul*`` in ``libmygrad_hip.so``) with no kernel of
 Operand patterns that run: both operands at most 2-D (vectors are promoted like
 ``np.matmul`` does); one operand a stack and the other at most 2-D (one launch: the stack is
 the convolution's batch, or folds into the rows of the left operand); two stacks of the same
-batch shape (one launch per matrix pair).  Stacks that broadcast against each other raise
-``NotImplementedError`` (there is no CPU fallback)."""
+batch shape (one launch per matrix pair); two stacks that broadcast against each other
+(each is first spread to the common batch shape on the device, and the gradient of a stack
+that was spread is summed back over the axes it was spread along)."""
 
 import numpy as np
 
-from ... import _device, _hip
+from ... import _device, _hip, _reduce
 from ...operation_base import Operation
 
 __all__ = ["MatMul"]
@@ -43,11 +44,11 @@ class MatMul(Operation):
         y2 = y if y.ndim > 1 else y[:, None]
         M, K, N = x2.shape[-2], x2.shape[-1], y2.shape[-1]
         stack_a, stack_b = x2.shape[:-2], y2.shape[:-2]
-        if stack_a and stack_b and stack_a != stack_b:
-            raise NotImplementedError(
-                f"matmul on the GPU does not broadcast two stacks against each other, got {x.shape} and {y.shape} "
-                "(no CPU fallback)"
-            )
+        # two different stacks: both are spread to the batch shape they broadcast to
+        self._spread = bool(stack_a and stack_b and stack_a != stack_b)
+        self._own_stacks = (stack_a, stack_b)
+        if self._spread:
+            stack_a = stack_b = tuple(probe.shape[: probe.ndim - 2])
         batch_shape = stack_a or stack_b
         out_shape = batch_shape + (() if x.ndim == 1 else (M,)) + (() if y.ndim == 1 else (N,))
         assert len(out_shape) == probe.ndim
@@ -57,12 +58,22 @@ class MatMul(Operation):
         if 0 in out_shape or K == 0:
             return np.zeros(out_shape, dtype=dtype)
 
-        ab, bb = _device.to_device(x, dtype), _device.to_device(y, dtype)
+        ab, bb = self._operand(x, 0), self._operand(y, 1)
         ob = _device.DeviceBuffer(max(_prod(out_shape) * dtype.itemsize, 16))
         self._launch("mg_matmul", ab, bb, ob, a_like=0, x_like=1, out_like=2)
         out = _device.download(ob, out_shape, dtype)
         _device.attach(out, ob)
         return out
+
+    def _operand(self, arr, index):
+        """Device buffer of operand ``index``, spread over the common batch shape if its own
+        stack is a different one."""
+        buf = _device.to_device(arr, self._dtype)
+        own, batch = self._own_stacks[index], self._stacks[index]
+        if not self._spread or own == batch:
+            return buf
+        core = self._promoted[index][-2:]
+        return _reduce.broadcast(buf, own + core, batch + core, self._dtype)
 
     def _launch(self, entry, first, second, result, a_like, x_like, out_like):
         """Call ``entry(dtype, batch, M, K, N, first, second, result)`` once, or once per
@@ -95,16 +106,22 @@ class MatMul(Operation):
         if grad.size != batch * M * N:
             raise ValueError(f"matmul backward: gradient of shape {grad.shape} does not match the product")
         gb = _device.to_device(grad, dtype)
+        own, full = self._own_stacks[index], self._stacks[index]
+        widened = self._spread and own != full
+        core = self._promoted[index][-2:]
+        count = _prod(full + core) if widened else var.size
+        ob = _device.DeviceBuffer(max(count * dtype.itemsize, 16))
         if index == 0:
             # d a = grad @ b^T, summed over a batch that `a` was shared by (ops.py:107-114)
-            other = _device.to_device(b.data, dtype)
-            ob = _device.DeviceBuffer(max(var.size * dtype.itemsize, 16))
-            self._launch("mg_matmul_da", gb, other, ob, a_like=2, x_like=1, out_like=0)
+            self._launch("mg_matmul_da", gb, self._operand(b.data, 1), ob, a_like=2, x_like=1, out_like=0)
         else:
             # d b = a^T @ grad, summed over a stack of left operands that `b` was shared by (ops.py:116-124)
-            other = _device.to_device(a.data, dtype)
-            ob = _device.DeviceBuffer(max(var.size * dtype.itemsize, 16))
-            self._launch("mg_matmul_dx", gb, other, ob, a_like=2, x_like=0, out_like=1)
+            self._launch("mg_matmul_dx", gb, self._operand(a.data, 0), ob, a_like=2, x_like=0, out_like=1)
+        if widened:
+            # one gradient per matrix pair: add up those of the pairs that shared this operand's matrix
+            lead = len(full) - len(own)
+            axes = tuple(range(lead)) + tuple(lead + i for i, n in enumerate(own) if n == 1 and full[lead + i] != 1)
+            ob = _reduce.sum_axes(ob, full + core, axes, dtype)
         out = _device.download(ob, var.shape, dtype)
         _device.attach_transient(out, ob)
         return out

@@ -87,6 +87,11 @@ SHAPES = [
     ((2, 3, 4), (4,)),
     ((2, 2, 30, 40), (2, 2, 40, 50)),
     ((60, 70), (70, 80)),
+    # stacks that broadcast against each other
+    ((2, 1, 3, 4), (2, 4, 5)),
+    ((1, 3, 4), (2, 4, 5)),
+    ((3, 1, 2, 6, 4), (2, 1, 4, 5)),
+    ((2, 3, 4), (5, 1, 4, 3)),
 ]
 
 
@@ -129,8 +134,8 @@ def test_reference_vectors_operator_and_errors(kats):
         mg.matmul(mg.Tensor(np.ones((2, 3))), 3.0)  # scalars are not allowed
     with pytest.raises(ValueError):
         mg.matmul(mg.Tensor(np.ones((2, 3))), np.ones((4, 2)))  # core dimensions differ
-    with pytest.raises(NotImplementedError):
-        mg.matmul(mg.Tensor(np.ones((2, 1, 3, 4))), np.ones((2, 4, 5)))
+    with pytest.raises(ValueError):
+        mg.matmul(mg.Tensor(np.ones((2, 1, 3, 4))), np.ones((3, 2, 4, 5)))  # stacks that do not broadcast
     with pytest.raises(TypeError):
         mg.matmul(mg.Tensor(np.ones((2, 3), dtype=np.int64)), np.ones((3, 2), dtype=np.int64))
     assert mg.matmul(np.ones((0, 3)), np.ones((3, 2))).shape == (0, 2)

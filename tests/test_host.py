@@ -384,8 +384,8 @@ def test_argument_checks_of_the_neighbouring_operations_need_no_device():
         mg.matmul(x, 3.0)  # scalars are not allowed
     with pytest.raises(ValueError):
         mg.matmul(np.ones((2, 3)), np.ones((4, 2)))
-    with pytest.raises(NotImplementedError):
-        mg.matmul(np.ones((2, 1, 3, 4)), np.ones((2, 4, 5)))  # stacks that broadcast against each other
+    with pytest.raises(ValueError):
+        mg.matmul(np.ones((2, 1, 3, 4)), np.ones((3, 2, 4, 5)))  # stacks that do not broadcast against each other
     with pytest.raises(TypeError):
         mg.matmul(np.ones((2, 3), dtype=np.int64), np.ones((3, 2), dtype=np.int64))
     assert mg.matmul(np.ones((0, 3)), np.ones((3, 2))).shape == (0, 2)
