@@ -241,6 +241,16 @@ int mg_batchnorm_bwd(const mg_bn_desc *desc, const void *x, const void *grad, co
  * Multiply. */
 int mg_sum_over(int dtype, int64_t outer, int64_t n, int64_t inner, int over_middle, const void *x, void *out);
 
+/* ---- transposition ----
+ * out = x.transpose(perm) made C-contiguous: x has `nd` axes of extents shape[], output axis i
+ * is input axis perm[i]; elements of 4 or 8 bytes, fewer than 2^31 of them; at most 6 axes
+ * after those of length one are dropped and runs that stay together are merged.
+ * Brings the operands of an Einstein summation into the order (batch, rows, contracted) /
+ * (batch, contracted, columns) that the matrix-product entry points take, and the result back
+ * into the order the subscripts ask for: part of what np.einsum does in EinSum.__call__ and
+ * EinSum.backward_var, src/mygrad/linalg/ops.py:79-110 and :112-262. */
+int mg_permute(int elem_bytes, int nd, const int64_t *shape, const int32_t *perm, const void *x, void *out);
+
 /* ---- matrix product ---- */
 
 /* out[b] = a @ x[b], a:(M, K) shared by the batch, x:(batch, K, N), out:(batch, M, N), all

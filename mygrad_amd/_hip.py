@@ -158,6 +158,7 @@ _SIGNATURES = {
     "mg_repeat_fwd": [ctypes.c_int] + [ctypes.c_int64] * 5 + [_vp, _vp, _vp],
     "mg_repeat_bwd": [ctypes.c_int] + [ctypes.c_int64] * 5 + [_vp, _vp, _vp],
     "mg_window_gather": [ctypes.POINTER(WindowDesc), _vp, _vp],
+    "mg_permute": [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int32), _vp, _vp],
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES) + ("mg_last_error",)
 
@@ -262,6 +263,7 @@ KERNEL_TAGS = {
     16: "repeat_bwd",
     17: "window_gather",
     18: "sum_over",
+    19: "permute",
 }
 
 

@@ -10,7 +10,7 @@ import numpy as np
 
 from . import _device, _hip
 
-__all__ = ["sum_axes", "broadcast"]
+__all__ = ["sum_axes", "broadcast", "permute"]
 
 
 def _merge(pairs):
@@ -82,3 +82,18 @@ def broadcast(buf, shape, to_shape, dtype):
         buf = out
         current[j] = size
     return buf
+
+
+def permute(buf, shape, perm, dtype):
+    """Device buffer with ``x.transpose(perm)`` made contiguous, for the C-contiguous ``x`` of
+    ``shape`` in ``buf`` (not empty).  The same buffer comes back when nothing moves."""
+    import ctypes
+
+    perm = tuple(int(p) for p in perm)
+    moving = [p for p in perm if shape[p] != 1]
+    if moving == sorted(moving):
+        return buf
+    nd = len(shape)
+    out = _device.DeviceBuffer(max(int(np.prod(shape, dtype=np.int64)) * dtype.itemsize, 16))
+    _hip.check(_hip.lib().mg_permute(dtype.itemsize, nd, (ctypes.c_int64 * nd)(*shape), (ctypes.c_int32 * nd)(*perm), buf.ptr, out.ptr))
+    return out

@@ -60,6 +60,7 @@ enum KernelTag {
   TAG_REPEAT_BWD = 16,
   TAG_WINDOW_GATHER = 17,
   TAG_SUM_OVER = 18,
+  TAG_PERMUTE = 19,
 };
 void timing_begin(int tag);
 void timing_end();

@@ -335,6 +335,89 @@ void launch_repeat_bwd(const RepeatParams &p, bool wide, const long long *offset
     hipLaunchKernelGGL((repeat_bwd_kernel<T, 1>), grid, block, 0, runtime().stream, p, offsets, (const T *)grad, (T *)da, count);
 }
 
+// ------------------------------------------------------------------------------------------
+// Transposition: out = x.transpose(perm), C-contiguous.  The host drops axes of length one
+// and merges output axes that are neighbours in the input as well; what is left has at most
+// kMaxPermuteAxes axes, described per OUTPUT axis by its extent and its stride in the input.
+//   rows  the last output axis is also the input's fastest one: whole runs are copied, 16
+//         bytes per lane where the runs allow it;
+//   tile  otherwise some other output axis p is the input's fastest one: 32 x 32 tiles over
+//         (axis p, last axis) go through LDS, read along p and written along the last axis,
+//         so that both sides are coalesced.
+// ------------------------------------------------------------------------------------------
+constexpr int kMaxPermuteAxes = 6;
+
+struct PermuteParams {
+  int nd;
+  unsigned size[kMaxPermuteAxes];
+  long long in_stride[kMaxPermuteAxes];  // rows: in pieces; tile: in elements
+  FastDivT by_size[kMaxPermuteAxes];
+  unsigned pieces;  // rows: pieces per run
+  FastDivT by_pieces;
+  unsigned count;   // rows: pieces in all
+  int p_axis;       // tile: the output axis that is the input's fastest
+  long long p_out_stride;
+  unsigned tiles_c, tiles_r, nrest;
+  FastDivT by_tiles_c;
+};
+
+template <int PIECE>
+__global__ void __launch_bounds__(256) permute_rows_kernel(PermuteParams p, const typename Word<PIECE>::type *__restrict__ x,
+                                                           typename Word<PIECE>::type *__restrict__ out) {
+  const unsigned t = blockIdx.x * 256u + threadIdx.x;
+  if (t >= p.count) return;
+  unsigned row = p.by_pieces.div(t);
+  long long at = t - row * p.pieces;
+  for (int k = p.nd - 2; k >= 0; --k) {
+    const unsigned q = p.by_size[k].div(row);
+    at += (long long)(row - q * p.size[k]) * p.in_stride[k];
+    row = q;
+  }
+  out[t] = x[at];
+}
+
+template <int BYTES>
+__global__ void __launch_bounds__(256) permute_tile_kernel(PermuteParams p, const typename Word<BYTES>::type *__restrict__ x,
+                                                           typename Word<BYTES>::type *__restrict__ out) {
+  typedef typename Word<BYTES>::type W;
+  __shared__ W tile[32][33];
+  const int last = p.nd - 1;
+  const unsigned tr = p.by_tiles_c.div(blockIdx.x), tc = blockIdx.x - tr * p.tiles_c;
+  const unsigned r0 = tr * 32u, c0 = tc * 32u;
+  const unsigned tx = threadIdx.x & 31u, ty = threadIdx.x >> 5;
+  const unsigned rn = p.size[p.p_axis], cn = p.size[last];
+  const long long sc = p.in_stride[last];
+  for (unsigned rest = blockIdx.y; rest < p.nrest; rest += gridDim.y) {
+    // the other axes: offsets of this tile's plane in the input and in the output
+    long long in0 = 0, out0 = 0, out_stride = cn;
+    unsigned rem = rest;
+    for (int k = last - 1; k >= 0; --k) {
+      if (k == p.p_axis) {
+        out_stride *= p.size[k];
+        continue;
+      }
+      const unsigned q = p.by_size[k].div(rem);
+      const unsigned i = rem - q * p.size[k];
+      rem = q;
+      in0 += (long long)i * p.in_stride[k];
+      out0 += (long long)i * out_stride;
+      out_stride *= p.size[k];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const unsigned r = r0 + tx, c = c0 + ty + 8u * j;
+      if (r < rn && c < cn) tile[ty + 8 * j][tx] = x[in0 + r + (long long)c * sc];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const unsigned c = c0 + tx, r = r0 + ty + 8u * j;
+      if (r < rn && c < cn) out[out0 + (long long)r * p.p_out_stride + c] = tile[tx][ty + 8 * j];
+    }
+    __syncthreads();
+  }
+}
+
 }  // namespace
 }  // namespace mg
 
@@ -503,6 +586,98 @@ int mg_window_gather(const mg_window_desc *d, const void *x, void *out) {
     case 4: hipLaunchKernelGGL(window_gather_kernel<4>, grid, block, 0, s, p, (const unsigned *)x, (unsigned *)out); break;
     case 2: hipLaunchKernelGGL(window_gather_kernel<2>, grid, block, 0, s, p, (const unsigned short *)x, (unsigned short *)out); break;
     default: hipLaunchKernelGGL(window_gather_kernel<1>, grid, block, 0, s, p, (const unsigned char *)x, (unsigned char *)out); break;
+  }
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
+int mg_permute(int elem_bytes, int nd, const int64_t *shape, const int32_t *perm, const void *x, void *out) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (elem_bytes != 4 && elem_bytes != 8) return fail(MG_ERR_UNSUPPORTED, "mg_permute: element size %d (4 or 8 bytes)", elem_bytes);
+  if (nd < 0 || nd > 16 || (nd > 0 && (!shape || !perm))) return fail(MG_ERR_BAD_ARG, "mg_permute: nd = %d or null shape / perm", nd);
+  long long total = 1;
+  long long stride[16];
+  bool seen[16] = {false};
+  for (int k = nd - 1; k >= 0; --k) {
+    if (shape[k] < 0) return fail(MG_ERR_BAD_ARG, "mg_permute: negative extent");
+    if (perm[k] < 0 || perm[k] >= nd || seen[perm[k]]) return fail(MG_ERR_BAD_ARG, "mg_permute: perm is not a permutation of 0..%d", nd - 1);
+    seen[perm[k]] = true;
+    stride[k] = total;
+    total *= shape[k];
+    if (total >= (1ll << 31)) return fail(MG_ERR_UNSUPPORTED, "mg_permute: 2^31 or more elements");
+  }
+  if (total == 0) return MG_OK;
+  if (!x || !out) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_permute");
+  // output axes as (extent, stride in the input); length-one axes dropped, neighbours that are
+  // neighbours in the input too merged
+  long long size[16], from[16];
+  int m = 0;
+  for (int i = 0; i < nd; ++i) {
+    const long long n = shape[perm[i]], st = stride[perm[i]];
+    if (n == 1) continue;
+    if (m > 0 && from[m - 1] == st * n) {
+      size[m - 1] *= n;
+      from[m - 1] = st;
+    } else {
+      size[m] = n;
+      from[m] = st;
+      ++m;
+    }
+  }
+  hipStream_t s = runtime().stream;
+  ScopedTiming timed(TAG_PERMUTE);
+  if (m <= 1) {  // the same order in memory
+    MG_HIP(hipMemcpyAsync(out, x, (size_t)total * elem_bytes, hipMemcpyDeviceToDevice, s));
+    return MG_OK;
+  }
+  if (m > kMaxPermuteAxes) return fail(MG_ERR_UNSUPPORTED, "mg_permute: %d axes left after merging (at most %d)", m, kMaxPermuteAxes);
+  PermuteParams p{};
+  p.nd = m;
+  for (int k = 0; k < m; ++k) {
+    p.size[k] = (unsigned)size[k];
+    p.in_stride[k] = from[k];
+    p.by_size[k] = make_fastdiv_t((unsigned)size[k]);
+  }
+  const dim3 block(256);
+  if (from[m - 1] == 1) {
+    // runs of size[m-1] elements; every other stride is a multiple of that run
+    const long long run_bytes = size[m - 1] * elem_bytes;
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out);
+    const int piece = (run_bytes % 16 == 0 && bits % 16 == 0) ? 16 : elem_bytes;
+    const long long epp = piece / elem_bytes;
+    p.pieces = (unsigned)(run_bytes / piece);
+    p.by_pieces = make_fastdiv_t(p.pieces);
+    p.count = (unsigned)(total / epp);
+    for (int k = 0; k < m - 1; ++k) p.in_stride[k] = from[k] / epp;
+    const dim3 grid((unsigned)ceil_div((long long)p.count, 256));
+    switch (piece) {
+      case 16: hipLaunchKernelGGL(permute_rows_kernel<16>, grid, block, 0, s, p, (const Word16 *)x, (Word16 *)out); break;
+      case 8: hipLaunchKernelGGL(permute_rows_kernel<8>, grid, block, 0, s, p, (const unsigned long long *)x, (unsigned long long *)out); break;
+      default: hipLaunchKernelGGL(permute_rows_kernel<4>, grid, block, 0, s, p, (const unsigned *)x, (unsigned *)out); break;
+    }
+  } else {
+    p.p_axis = -1;
+    long long out_stride = 1, rest = 1;
+    for (int k = m - 1; k >= 0; --k) {
+      if (from[k] == 1) {
+        p.p_axis = k;
+        p.p_out_stride = out_stride;
+      } else if (k != m - 1) {
+        rest *= size[k];
+      }
+      out_stride *= size[k];
+    }
+    if (p.p_axis < 0) return fail(MG_ERR_HIP, "mg_permute: no output axis is the input's fastest one");
+    p.tiles_c = (unsigned)ceil_div(size[m - 1], 32);
+    p.tiles_r = (unsigned)ceil_div(size[p.p_axis], 32);
+    p.by_tiles_c = make_fastdiv_t(p.tiles_c);
+    p.nrest = (unsigned)rest;
+    const dim3 grid(p.tiles_c * p.tiles_r, (unsigned)std::min<long long>(rest, 65535));
+    if (elem_bytes == 8)
+      hipLaunchKernelGGL(permute_tile_kernel<8>, grid, block, 0, s, p, (const unsigned long long *)x, (unsigned long long *)out);
+    else
+      hipLaunchKernelGGL(permute_tile_kernel<4>, grid, block, 0, s, p, (const unsigned *)x, (unsigned *)out);
   }
   MG_HIP(hipGetLastError());
   return MG_OK;

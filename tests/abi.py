@@ -136,6 +136,17 @@ def relu_bwd(x, grad):
     return _down(ob, x.shape, x.dtype)
 
 
+def permute(x, perm):
+    import ctypes
+
+    nd = x.ndim
+    xb = _up(x)
+    ob = _device.DeviceBuffer(max(x.nbytes, 16))
+    shape, order = (ctypes.c_int64 * max(nd, 1))(*x.shape), (ctypes.c_int32 * max(nd, 1))(*perm)
+    _hip.check(_hip.lib().mg_permute(x.dtype.itemsize, nd, shape, order, xb.ptr, ob.ptr))
+    return _down(ob, tuple(x.shape[p] for p in perm), x.dtype)
+
+
 def sum_over(x3, over_middle):
     """x3:(outer, n, inner) -> sums over the middle axis (outer, inner) or over the other two (n,)."""
     outer, n, inner = x3.shape

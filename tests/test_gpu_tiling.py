@@ -196,3 +196,40 @@ def test_abi_rejects_bad_arguments(abi):
     assert lib.mg_window_gather(_hip.window_desc(4, 1, (10,), (3,), (1,), (1,), (9,)), p, p) == -1  # a placement too many
     assert lib.mg_window_gather(_hip.window_desc(3, 1, (10,), (3,), (1,), (1,), (8,)), p, p) == -2
     assert lib.mg_window_gather(None, p, p) == -1
+
+
+# ----------------------------------------------------------------------------- transposition
+PERMUTE_CASES = [
+    ((5,), (0,)), ((3, 4), (1, 0)), ((3, 4), (0, 1)), ((33, 65), (1, 0)), ((2, 3, 4), (2, 0, 1)), ((2, 3, 4), (0, 2, 1)),
+    ((2, 3, 4), (1, 0, 2)), ((7, 1, 5), (2, 1, 0)), ((4, 5, 6, 7), (3, 1, 0, 2)), ((4, 5, 6, 8), (1, 0, 2, 3)),
+    ((2, 3, 4, 5, 6), (4, 3, 2, 1, 0)), ((2, 3, 2, 3, 2, 3), (5, 3, 1, 4, 2, 0)), ((64, 100, 36), (0, 2, 1)),
+    ((100, 257), (1, 0)), ((8, 16, 12, 12), (0, 2, 3, 1)), ((8, 12, 12, 16), (0, 3, 1, 2)), ((1, 1, 1), (2, 0, 1)),
+    ((300, 2, 70), (1, 2, 0)), ((1000, 1000), (1, 0)), ((3, 70000), (1, 0)), ((70000, 3), (1, 0)),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("shape, perm", PERMUTE_CASES)
+def test_permute_is_numpys_transpose(abi, dtype, shape, perm):
+    rng = np.random.default_rng([len(shape), int(np.prod(shape))])
+    x = rng.standard_normal(shape).astype(dtype)
+    got = abi.permute(x, perm)
+    want = np.ascontiguousarray(np.transpose(x, perm))
+    assert got.shape == want.shape and np.array_equal(got.view(np.uint8), want.view(np.uint8))
+
+
+def test_permute_rejects_bad_arguments(abi):
+    import ctypes
+
+    from mygrad_amd import _device, _hip
+
+    buf = _device.DeviceBuffer(256)
+    lib = _hip.lib()
+    shape, perm = (ctypes.c_int64 * 2)(3, 4), (ctypes.c_int32 * 2)(1, 1)
+    assert lib.mg_permute(4, 2, shape, perm, buf.ptr, buf.ptr) == _hip.MG_ERR_BAD_ARG  # not a permutation
+    perm = (ctypes.c_int32 * 2)(1, 0)
+    assert lib.mg_permute(2, 2, shape, perm, buf.ptr, buf.ptr) == _hip.MG_ERR_UNSUPPORTED  # 2-byte elements
+    assert lib.mg_permute(4, 2, shape, perm, None, buf.ptr) == _hip.MG_ERR_BAD_ARG
+    seven = (ctypes.c_int64 * 7)(*([2] * 7))
+    reverse = (ctypes.c_int32 * 7)(*range(6, -1, -1))
+    assert lib.mg_permute(4, 7, seven, reverse, buf.ptr, buf.ptr) == _hip.MG_ERR_UNSUPPORTED  # seven axes that all move
