@@ -20,6 +20,8 @@ from .operation_base import Operation
 from .tensor_base import Tensor, asarray, tensor
 from .math import matmul, multiply, sum  # noqa: A004  (after tensor_base: the ops import Tensor)
 from .tensor_manip import repeat
+from .linalg import einsum
+from . import linalg
 from ._io import load, save
 
 execute_op = Tensor._op
@@ -36,6 +38,8 @@ __all__ = [
     "sliding_window_view",
     "sliding_window_copy",
     "multiply",
+    "einsum",
+    "linalg",
     "matmul",
     "sum",
     "repeat",

@@ -44,8 +44,10 @@ def sum_axes(buf, shape, axes, dtype):
         kinds = [kind for _, kind in groups]
         if kinds in ([True], [True, False], [False, True], [True, False, True]):
             # one kept group at most, summed groups around it: a single pass
-            if kinds == [True]:
-                outer, n, inner = groups[0][0], 1, 1
+            if kinds == [True]:  # everything that is left is summed: the whole-array kernel
+                out = _device.DeviceBuffer(16)
+                _hip.check(lib.mg_sum_all(code, groups[0][0], buf.ptr, out.ptr))
+                return out
             elif kinds == [True, False]:
                 outer, n, inner = groups[0][0], groups[1][0], 1
             elif kinds == [False, True]:

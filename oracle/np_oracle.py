@@ -31,6 +31,9 @@ Pinning (what holds each function to the reference without importing it):
                    single calls of the NumPy routine the reference calls
                    (``np.multiply``, ``np.sum``, ``np.full``); ``sum_all`` is
                    additionally held to ``math.fsum`` and closed forms in the tests
+  einsum_forward   ``np.einsum`` itself, held to the reference's docstring vectors
+  einsum_backward  central differences, the adjoint identity <einsum(a, b), g> =
+                   <a, grad_a> = <b, grad_b>, loops over every index
   sum_axes, sum_axes_backward, reduce_broadcast, multiply_broadcast_backward
                    ``np.sum`` itself, held to ``math.fsum`` per kept entry and to loops;
                    the two gradients to loops over every index and to the adjoint
@@ -84,6 +87,8 @@ __all__ = [
     "sum_axes_backward",
     "reduce_broadcast",
     "multiply_broadcast_backward",
+    "einsum_forward",
+    "einsum_backward",
     "pool_forward",
     "pool_argmax",
     "pool_backward",
@@ -569,3 +574,43 @@ def matmul_backward(grad, a, b, index):
     else:  # :123-124
         out = a[:, np.newaxis] * np.expand_dims(grad, -2)
     return _sum_to(out, b.shape)
+
+
+# ------------------------------------------------------------------ einsum
+def einsum_forward(in_lbls, out_lbls, *arrays):
+    """``EinSum.__call__``: ``np.einsum("<in_lbls>-><out_lbls>", *arrays)``
+    (mygrad/linalg/ops.py:82-110); ``in_lbls`` is the comma-separated string."""
+    return np.einsum(f"{in_lbls}->{out_lbls}", *arrays)
+
+
+def einsum_backward(grad, index, in_lbls, out_lbls, arrays, factor=1):
+    """``EinSum.backward_var`` for operands without a repeated label
+    (mygrad/linalg/ops.py:124-218): the operand's gradient is the summation of ``grad`` (in
+    the operand's place, labelled like the result) with the other operands onto the
+    operand's labels.  Labels of the operand that occur nowhere else were summed away on
+    their own, so ``grad`` is first given an axis for each of them, broadcast to its length.
+    ``factor`` is the number of times the same (tensor, labels) pair occurs among the
+    operands (the reference computes one gradient for all of them and scales it)."""
+    lbls = in_lbls.split(",")
+    var_lbl = lbls.pop(index)
+    if len(set(var_lbl)) != len(var_lbl):
+        raise NotImplementedError("repeated labels within an operand (traces) are not restated")
+    var_shape = arrays[index].shape
+    rest = tuple(a for n, a in enumerate(arrays) if n != index)
+    known = set("".join(lbls)) | set(out_lbls)
+    grad = np.asarray(grad)
+    grad_lbl = out_lbls
+    if set(var_lbl) - known:
+        slots = [slice(None)] * grad.ndim
+        shape = list(grad.shape)
+        for n, lbl in enumerate(var_lbl):
+            if lbl not in known:
+                grad_lbl = grad_lbl[:n] + lbl + grad_lbl[n:]
+                slots.insert(n, np.newaxis)
+                shape.insert(n, var_shape[n])
+        grad = np.broadcast_to(grad[tuple(slots)] if grad.ndim else grad, shape)
+    back = np.einsum(",".join([grad_lbl] + lbls) + "->" + var_lbl, grad, *rest)
+    back = reduce_broadcast(back, var_shape)
+    if back.shape != var_shape:
+        back = np.broadcast_to(back, var_shape)
+    return back * factor if factor > 1 else back

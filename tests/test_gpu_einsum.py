@@ -1,0 +1,120 @@
+"""Einstein summation on the device against the NumPy restatement of the reference
+(``np.einsum`` forward; the reference's gradient rule), through ``Tensor.backward()``.
+
+Bar (maximum absolute error relative to the largest magnitude of the expected array):
+1e-10 in float64, 2e-4 in float32 -- the bar of the matrix product it runs on.  Pure
+rearrangements (a transpose, an outer product with a scalar) are exact."""
+
+import numpy as np
+import pytest
+
+from oracle import np_oracle as ora
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.dtype(np.float32): 2e-4, np.dtype(np.float64): 1e-10}
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_gpu():
+    import mygrad_amd as mg
+
+    if not mg.is_available():
+        pytest.fail("libmygrad_hip.so / gfx950 device not available: the GPU tests need both")
+
+
+def err(got, want):
+    want = np.asarray(want, dtype=np.float64)
+    scale = float(np.max(np.abs(want))) if want.size else 1.0
+    return float(np.max(np.abs(np.asarray(got, dtype=np.float64) - want), initial=0.0)) / (scale or 1.0)
+
+
+CASES = [
+    ("ij,jk->ik", [(3, 4), (4, 5)]), ("ij,kj->ik", [(3, 4), (5, 4)]), ("ji,jk->ik", [(4, 3), (4, 5)]),
+    ("bij,bjk->bik", [(2, 3, 4), (2, 4, 5)]), ("ijk,jil->kl", [(3, 4, 5), (4, 3, 2)]), ("i,i->", [(6,), (6,)]),
+    ("i,j->ji", [(3,), (4,)]), ("ij->ji", [(3, 4)]), ("ijk->j", [(2, 3, 4)]), ("ij,jk->i", [(3, 4), (4, 5)]),
+    ("ij,k->", [(2, 3), (4,)]), ("abc,cd->dab", [(2, 3, 4), (4, 5)]), (",ij->ij", [(), (2, 3)]),
+    ("aib,ajb->abij", [(2, 3, 4), (2, 5, 4)]), ("ij->", [(3, 4)]), ("ij->ij", [(2, 3)]), ("ijkl->lkji", [(2, 3, 4, 5)]),
+    ("bhqd,bhkd->bhqk", [(2, 3, 16, 8), (2, 3, 12, 8)]), ("nchw,fc->nfhw", [(2, 16, 5, 5), (8, 16)]),
+    ("ij,jk->ik", [(128, 256), (256, 64)]), ("ab,ab->", [(7, 9), (7, 9)]), ("ab,ab->ab", [(7, 9), (7, 9)]),
+    ("i,i->i", [(5,), (5,)]), ("ij,j->i", [(0, 3), (3,)]), ("ij,jk->ik", [(2, 0), (0, 3)]),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("subscripts, shapes", CASES)
+def test_einsum_and_its_gradients_match_the_oracle(subscripts, shapes, dtype):
+    import mygrad_amd as mg
+
+    dtype = np.dtype(dtype)
+    rng = np.random.default_rng([len(subscripts), sum(int(np.prod(s)) for s in shapes)])
+    arrays = [rng.standard_normal(s).astype(dtype) for s in shapes]
+    tensors = [mg.Tensor(a) for a in arrays]
+    out = mg.einsum(subscripts, *tensors)
+    in_lbls, out_lbls = subscripts.split("->")
+    wide = [a.astype(np.float64) for a in arrays]
+    want = ora.einsum_forward(in_lbls, out_lbls, *wide)
+    assert out.shape == want.shape and out.dtype == dtype
+    assert err(out.data, want) <= TOL[dtype]
+    g = rng.standard_normal(want.shape).astype(dtype)
+    out.backward(g)
+    for index, t in enumerate(tensors):
+        back = ora.einsum_backward(g.astype(np.float64), index, in_lbls, out_lbls, wide)
+        assert t.grad.shape == t.shape and t.grad.dtype == dtype
+        assert err(t.grad, back) <= TOL[dtype]
+
+
+def test_reference_docstring_vectors_in_both_calling_conventions(kats):
+    import mygrad_amd as mg
+
+    def operand(text):
+        return np.asarray(eval(text, {"arange": lambda n: np.arange(float(n))}), dtype=np.float64)  # noqa: S307
+
+    for case in kats["einsum"]:
+        got = mg.einsum(case["subscripts"], *[operand(t) for t in case["operands"]])
+        assert np.array_equal(got.data, np.array(case["out"], dtype=float)), case["source"]
+    a, b = np.arange(60.0).reshape(3, 4, 5), np.arange(24.0).reshape(4, 3, 2)
+    got = mg.einsum(mg.Tensor(a), [0, 1, 2], mg.Tensor(b), [1, 0, 3], [2, 3])
+    assert np.array_equal(got.data, [[4400, 4730], [4532, 4874], [4664, 5018], [4796, 5162], [4928, 5306]])
+    # rearrangements are copies of values: exact, and never a view of the operand
+    c = mg.Tensor(np.arange(6.0).reshape(2, 3))
+    t = mg.einsum("ij->ji", c)
+    assert np.array_equal(t.data, c.data.T) and not np.shares_memory(t.data, c.data)
+    t.clear_graph()
+
+
+def test_a_tensor_that_occurs_twice_gets_one_gradient_scaled_by_two():
+    import mygrad_amd as mg
+
+    x = mg.Tensor(np.arange(1.0, 5.0))
+    mg.einsum("i,i->", x, x).backward()
+    assert np.array_equal(x.grad, 2 * x.data)  # d (x.x) / dx
+    y = mg.Tensor(np.arange(6.0).reshape(2, 3))
+    mg.einsum("ij,ij->j", y, y).backward(np.array([1.0, 10.0, 100.0]))
+    assert np.array_equal(y.grad, 2 * y.data * np.array([1.0, 10.0, 100.0]))
+    # the same tensor under different labels is two different pairs
+    z = mg.Tensor(np.arange(4.0).reshape(2, 2))
+    mg.einsum("ij,jk->ik", z, z).backward()
+    want = ora.einsum_backward(np.ones((2, 2)), 0, "ij,jk", "ik", [z.data, z.data]) + ora.einsum_backward(
+        np.ones((2, 2)), 1, "ij,jk", "ik", [z.data, z.data])
+    assert np.array_equal(z.grad, want)
+
+
+def test_errors_and_what_is_refused():
+    import mygrad_amd as mg
+
+    a, b = mg.Tensor(np.ones((2, 3))), mg.Tensor(np.ones((3, 4)))
+    with pytest.raises(ValueError):
+        mg.einsum("ij,jk->ik", a, mg.Tensor(np.ones((4, 4))))  # lengths of j differ
+    with pytest.raises(ValueError):
+        mg.einsum("ijk,jk->i", a, b)  # three labels for two axes
+    with pytest.raises(ValueError):
+        mg.einsum("ij,jk->ii", a, b)
+    with pytest.raises(NotImplementedError):
+        mg.einsum("ii->i", mg.Tensor(np.ones((3, 3))))  # a diagonal
+    with pytest.raises(NotImplementedError):
+        mg.einsum("ij,jk,kl->il", a, b, mg.Tensor(np.ones((4, 2))))
+    with pytest.raises(NotImplementedError):
+        mg.einsum("ij,ij->ij", a, mg.Tensor(np.ones((1, 3))))  # a label of length one broadcast
+    with pytest.raises(TypeError):
+        mg.einsum("ij,jk->ik", mg.Tensor(np.ones((2, 3), dtype=np.int64)), mg.Tensor(np.ones((3, 4), dtype=np.int64)))

@@ -76,6 +76,10 @@ def test_no_device_fails_loudly_without_fallback():
         lambda: mg.matmul(v, v.T),
         lambda: mg.Tensor(v) @ v.T,
         lambda: mg.sliding_window_copy(v, (2, 2), 1),
+        lambda: mg.sum(v, axis=0),
+        lambda: mg.multiply(v, np.ones(3)),
+        lambda: mg.einsum("ij,kj->ik", v, v),
+        lambda: mg.einsum("ij->ji", v),
     ):
         with pytest.raises(mg.HipUnavailable):
             call()
@@ -408,6 +412,18 @@ def test_argument_checks_of_the_neighbouring_operations_need_no_device():
         mg.sliding_window_copy(np.ones((3, 3)), 2, 1)
     with pytest.raises(NotImplementedError):
         mg.sliding_window_copy(np.ones((2, 2, 2, 2)), (1, 1, 1, 1), 1)
+
+    with pytest.raises(ValueError):
+        mg.einsum("ij,jk->ik", np.ones((2, 3)), np.ones((4, 4)))
+    with pytest.raises(ValueError):
+        mg.einsum("ij,jk->ii", np.ones((2, 3)), np.ones((3, 4)))
+    with pytest.raises(NotImplementedError):
+        mg.einsum("ii", np.ones((3, 3)))
+    with pytest.raises(NotImplementedError):
+        mg.einsum("i,i,i", np.ones(3), np.ones(3), np.ones(3))
+    with pytest.raises(TypeError):
+        mg.einsum("i,i", np.arange(3), np.arange(3))
+    assert mg.einsum("ij,jk->ik", np.ones((2, 0)), np.ones((0, 3))).shape == (2, 3)
 
     with pytest.raises(ValueError):
         mg.multiply(np.ones((2, 3)), np.ones(4))  # shapes that do not broadcast

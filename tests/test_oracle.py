@@ -631,3 +631,66 @@ def test_broadcast_multiply_gradients_against_loops_and_adjoints(sa, sb):
         assert math.isclose(float(np.sum(out * g)), float(np.sum(var * got)), rel_tol=1e-9, abs_tol=1e-9)
     with pytest.raises(ValueError):
         ora.reduce_broadcast(np.zeros(3), (2, 3))
+
+
+# ----------------------------------------------------------------- einsum
+def _kat_operand(text):
+    return np.asarray(eval(text, {"arange": lambda n: np.arange(float(n))}), dtype=np.float64)  # noqa: S307 (fixture text)
+
+
+EINSUM_CASES = [
+    ("ij,jk->ik", [(3, 4), (4, 5)]), ("ij,kj->ik", [(3, 4), (5, 4)]), ("bij,bjk->bik", [(2, 3, 4), (2, 4, 5)]),
+    ("ijk,jil->kl", [(3, 4, 5), (4, 3, 2)]), ("i,i->", [(6,), (6,)]), ("i,j->ji", [(3,), (4,)]), ("ij->ji", [(3, 4)]),
+    ("ijk->j", [(2, 3, 4)]), ("ij,jk->i", [(3, 4), (4, 5)]), ("ij,k->", [(2, 3), (4,)]), ("abc,cd->dab", [(2, 3, 4), (4, 5)]),
+    (",ij->ij", [(), (2, 3)]), ("aib,ajb->abij", [(2, 3, 4), (2, 5, 4)]), ("ij->", [(3, 4)]), ("ij->ij", [(2, 3)]),
+]
+
+
+def test_einsum_reference_docstring_vectors(kats):
+    from numpy._core.einsumfunc import _parse_einsum_input
+
+    for case in kats["einsum"]:
+        arrays = [_kat_operand(t) for t in case["operands"]]
+        in_lbls, out_lbls, _ = _parse_einsum_input([case["subscripts"], *arrays])
+        got = ora.einsum_forward(in_lbls, out_lbls, *arrays)
+        assert np.array_equal(got, np.array(case["out"], dtype=float)), case["source"]
+
+
+@pytest.mark.parametrize("subscripts, shapes", EINSUM_CASES)
+def test_einsum_backward_against_differences_adjoints_and_loops(subscripts, shapes):
+    rng = np.random.default_rng(len(subscripts) * 13 + len(shapes))
+    in_lbls, out_lbls = subscripts.split("->")
+    arrays = [rng.standard_normal(s) for s in shapes]
+    out = ora.einsum_forward(in_lbls, out_lbls, *arrays)
+    g = rng.standard_normal(out.shape)
+    lbls = in_lbls.split(",")
+    sizes = {l: n for ls, a in zip(lbls, arrays) for l, n in zip(ls, a.shape)}
+    every = sorted(sizes)
+    for index, var in enumerate(arrays):
+        back = ora.einsum_backward(g, index, in_lbls, out_lbls, arrays)
+        assert back.shape == var.shape
+        # adjoint identity (the summation is linear in each operand)
+        assert math.isclose(float(np.sum(out * g)), float(np.sum(var * back)), rel_tol=1e-9, abs_tol=1e-9)
+        # loops over the whole index space: each term of the result, times its gradient, goes to
+        # the element of this operand that it read
+        want = np.zeros(var.shape)
+        for values in np.ndindex(*[sizes[l] for l in every]):
+            at = dict(zip(every, values))
+            term = g[tuple(at[l] for l in out_lbls)]
+            for n, (ls, a) in enumerate(zip(lbls, arrays)):
+                if n != index:
+                    term = term * a[tuple(at[l] for l in ls)]
+            want[tuple(at[l] for l in lbls[index])] += term
+        assert np.allclose(back, want, rtol=1e-10, atol=1e-10)
+        # central difference along one random direction
+        direction = rng.standard_normal(var.shape)
+        eps = 1e-6
+        plus = [a + eps * direction if n == index else a for n, a in enumerate(arrays)]
+        minus = [a - eps * direction if n == index else a for n, a in enumerate(arrays)]
+        slope = float(np.sum((ora.einsum_forward(in_lbls, out_lbls, *plus) - ora.einsum_forward(in_lbls, out_lbls, *minus)) * g)) / (2 * eps)
+        assert math.isclose(slope, float(np.sum(back * direction)), rel_tol=1e-6, abs_tol=1e-6)
+
+
+def test_einsum_backward_scales_a_repeated_pair():
+    x = np.arange(4.0)
+    assert np.array_equal(ora.einsum_backward(np.array(1.0), 0, "i,i", "", [x, x], factor=2), 2 * x)  # d(x.x)/dx
