@@ -103,6 +103,12 @@ int mg_shutdown(void);             /* frees the stream, workspace and cached pla
 const char *mg_last_error(void);   /* message of this thread's last failing call */
 int mg_device_info(mg_device_info_t *info);
 
+/* Device memory.  A block given back with mg_free is kept by the library and handed out again
+ * by a later mg_malloc of a like size (no driver call, no wait for the device): work that the
+ * library enqueued on the block before mg_free runs before anything its next owner enqueues,
+ * because there is one stream.  A caller that touches a block from a stream of its own must
+ * wait for that work before mg_free.  MYGRAD_HIP_POOL=0 (read by mg_init) switches the reuse
+ * off; at most a quarter of the device's memory is kept idle. */
 int mg_malloc(void **dptr, size_t nbytes);
 int mg_free(void *dptr);
 int mg_host_alloc(void **hptr, size_t nbytes); /* pinned host memory (hipHostMalloc) */

@@ -1,7 +1,10 @@
 // Device selection, the library stream, buffers, copies, events and scratch.
 #include "internal.h"
 
+#include <cstdlib>
 #include <cstring>
+#include <map>
+#include <unordered_map>
 #include <vector>
 
 namespace mg {
@@ -162,6 +165,40 @@ __global__ void __launch_bounds__(256) mfma_probe_kernel(double *sink, int iters
 }
 }  // namespace
 
+// Blocks given back with mg_free are kept and handed out again: hipMalloc costs tens of
+// microseconds and hipFree waits for the whole device, once per result of every operation.
+// Everything the library does to a block is ordered on its one stream, so a block may be
+// reused as soon as it is given back: whatever was enqueued on it before runs first.
+namespace {
+struct BlockPool {
+  std::multimap<size_t, void *> idle;           // size -> block, not in use
+  std::unordered_map<void *, size_t> size_of;   // every block of the pool, in use or idle
+  size_t idle_bytes = 0;
+  bool off = false;                             // MYGRAD_HIP_POOL=0: plain hipMalloc / hipFree
+};
+BlockPool &pool() {
+  static BlockPool p;
+  return p;
+}
+size_t pool_round(size_t n) {
+  const size_t unit = n <= (size_t(1) << 20) ? 512 : (size_t(1) << 21);
+  return (n + unit - 1) / unit * unit;
+}
+// Gives idle blocks back to the driver until at most `keep` bytes of them are left.
+void pool_trim(size_t keep) {
+  BlockPool &bp = pool();
+  if (bp.idle_bytes <= keep) return;
+  (void)hipStreamSynchronize(runtime().stream);  // work enqueued before the blocks were given back
+  while (bp.idle_bytes > keep && !bp.idle.empty()) {
+    auto largest = std::prev(bp.idle.end());
+    (void)hipFree(largest->second);
+    bp.idle_bytes -= largest->first;
+    bp.size_of.erase(largest->second);
+    bp.idle.erase(largest);
+  }
+}
+}  // namespace
+
 extern "C" {
 
 const char *mg_last_error(void) { return g_error; }
@@ -188,6 +225,10 @@ int mg_init(int device) {
     return fail(MG_ERR_NO_DEVICE, "device %d is %s; this library carries gfx950 code only", device,
                 rt.props.gcnArchName);
   MG_HIP(hipStreamCreateWithFlags(&rt.stream, hipStreamNonBlocking));
+  {
+    const char *flag = getenv("MYGRAD_HIP_POOL");
+    pool().off = flag && flag[0] == '0';
+  }
   rt.device = device;
   rt.ready = true;
   return MG_OK;
@@ -203,6 +244,7 @@ int mg_shutdown(void) {
   if (rt.workspace) MG_HIP(hipFree(rt.workspace));
   rt.workspace = nullptr;
   rt.workspace_bytes = 0;
+  pool_trim(0);  // idle blocks go back to the driver; blocks still held by callers stay theirs
   MG_HIP(hipStreamDestroy(rt.stream));
   rt.stream = nullptr;
   rt.ready = false;
@@ -234,7 +276,30 @@ int mg_malloc(void **dptr, size_t nbytes) {
   if (!dptr) return fail(MG_ERR_BAD_ARG, "dptr is null");
   *dptr = nullptr;
   if (nbytes == 0) nbytes = 256;  // keep a distinct, valid pointer for empty tensors
-  MG_HIP(hipMalloc(dptr, nbytes));
+  BlockPool &bp = pool();
+  if (bp.off) {
+    MG_HIP(hipMalloc(dptr, nbytes));
+    return MG_OK;
+  }
+  const size_t want = pool_round(nbytes);
+  auto fit = bp.idle.lower_bound(want);
+  if (fit != bp.idle.end() && fit->first <= want + want / 4) {  // at most a quarter of it unused
+    *dptr = fit->second;
+    bp.idle_bytes -= fit->first;
+    bp.idle.erase(fit);
+    return MG_OK;
+  }
+  hipError_t err = hipMalloc(dptr, want);
+  if ((err == hipErrorOutOfMemory || err == hipErrorMemoryAllocation) && bp.idle_bytes > 0) {
+    (void)hipGetLastError();
+    pool_trim(0);
+    err = hipMalloc(dptr, want);
+  }
+  if (err != hipSuccess) {
+    *dptr = nullptr;
+    return hip_fail(err, "hipMalloc", __FILE__, __LINE__);
+  }
+  bp.size_of[*dptr] = want;
   return MG_OK;
 }
 
@@ -242,8 +307,18 @@ int mg_free(void *dptr) {
   MG_LOCK();
   MG_REQUIRE_INIT();
   if (!dptr) return MG_OK;
-  // hipFree waits for the device, so no kernel can still be using the block.
-  MG_HIP(hipFree(dptr));
+  BlockPool &bp = pool();
+  auto known = bp.size_of.find(dptr);
+  if (known == bp.size_of.end()) {
+    // not from the pool: hipFree waits for the device, so no kernel can still be using it
+    MG_HIP(hipFree(dptr));
+    return MG_OK;
+  }
+  bp.idle.emplace(known->second, dptr);
+  bp.idle_bytes += known->second;
+  // keep at most a quarter of the device's memory idle
+  const size_t limit = runtime().props.totalGlobalMem / 4;
+  if (bp.idle_bytes > limit) pool_trim(limit / 2);
   return MG_OK;
 }
 

@@ -433,6 +433,34 @@ def test_abi_rejects_bad_arguments(abi):
     assert lib.mg_malloc(ctypes.byref(huge), 1 << 60) == _hip.MG_ERR_OOM
 
 
+def test_blocks_given_back_are_handed_out_again_in_stream_order(abi):
+    """mg_free keeps the block, mg_malloc of a like size returns it without touching the
+    driver; work enqueued on the block before it was given back runs before its next use."""
+    from mygrad_amd import _device, _hip
+
+    size = 3 << 20
+    first = _device.DeviceBuffer(size)
+    ptr = first.ptr
+    first.free()
+    again = _device.DeviceBuffer(size - 4096)  # rounds to the same block size
+    assert again.ptr == ptr
+    # a kernel still writing the block when it is given back: the next owner's upload lands after it
+    x = np.arange(size // 8, dtype=np.float64)
+    src = _device.DeviceBuffer(size)
+    src.upload(x)
+    _hip.check(_hip.lib().mg_memcpy_d2d(again.ptr, src.ptr, size))  # enqueued, not waited for
+    again.free()
+    reused = _device.DeviceBuffer(size)
+    assert reused.ptr == ptr
+    reused.upload(-x)
+    got = np.empty_like(x)
+    reused.download_into(got)
+    assert np.array_equal(got, -x)
+    # a block of another size class does not take this one
+    small = _device.DeviceBuffer(1024)
+    assert small.ptr != ptr
+
+
 @pytest.mark.gpu
 def test_mfma_probe_reports_plausible_rates():
     """The diagnostic entry point runs and its figures are ordered the way the fp64
