@@ -68,6 +68,12 @@ WORKLOADS = {
     # sums over axes of a tensor of conv5's output size: per channel (the gradient of a bias or of a
     # per-channel scale: every axis but axis 1), then over the channel axis alone
     "sum5": dict(kind="sumover", dtype="f32", seed=1012, x=(8, 32, 32, 64, 64), axes=((0, 2, 3, 4), (1,))),
+    # transposition of a tensor of conv5's output size: channels last (N,C,D,H,W -> N,D,H,W,C) and back
+    "perm5": dict(kind="permute", dtype="f32", seed=1013, x=(8, 32, 32, 64, 64), perms=((0, 2, 3, 4, 1), (0, 4, 1, 2, 3))),
+    # Einstein summation: a 1x1 convolution written as 'nchw,fc->nfhw' and its two gradients
+    # (operands transposed on the device, product on the convolution kernels, result transposed back)
+    "ein1x1": dict(kind="einsum", dtype="f32", seed=1014, x=(32, 256, 56, 56), w=(256, 256),
+                   subscripts=("nchw", "fc", "nfhw")),
     # repeat: twofold nearest-neighbour upsampling of the rows of a tensor of pool5's input size
     # (forward and gradient), and then of its columns
     "rep5": dict(kind="repeat", dtype="f32", seed=1009, x=(8, 32, 32, 64, 64), repeats=2, axes=(-2, -1)),
@@ -102,6 +108,11 @@ def describe(name):
         return f"{name}: relu + multiply + sum {wl['dtype']} x{wl['x']} fwd+bwd (7 kernels, 16 |x| bytes)"
     if wl["kind"] == "matmul":
         return f"{name}: matmul {wl['dtype']} ({wl['M']},{wl['K']}) @ ({wl['K']},{wl['N']}): product + both gradients"
+    if wl["kind"] == "permute":
+        return f"{name}: transpose {wl['dtype']} x{wl['x']} by {wl['perms'][0]}, then the result by {wl['perms'][1]}"
+    if wl["kind"] == "einsum":
+        a, b, o = wl["subscripts"]
+        return f"{name}: einsum '{a},{b}->{o}' {wl['dtype']} x{wl['x']} w{wl['w']} and both gradients"
     if wl["kind"] == "sumover":
         return f"{name}: sum {wl['dtype']} x{wl['x']} over axes {wl['axes'][0]}, then over axes {wl['axes'][1]}"
     if wl["kind"] == "repeat":
@@ -163,6 +174,33 @@ class Step:
             self.code, self.dims = _hip.dtype_code(dt), (1, M, K, N)
             per_pass = 2.0 * M * K * N
             self.work = {"conv_fwd": per_pass, "conv_dgrad": per_pass, "conv_wgrad": per_pass}
+            self.total_work = 3 * per_pass
+            self.unit, self.bound, self.peak = "TFLOP/s", "mfma", PEAK_TFLOPS[wl["dtype"]]
+            self.scale = 1e-12
+        elif wl["kind"] == "permute":
+            import ctypes
+
+            x = rng.standard_normal(wl["x"]).astype(dt)
+            self.x, self.out, self.back = resident(x), _device.DeviceBuffer(x.nbytes), _device.DeviceBuffer(x.nbytes)
+            nd = x.ndim
+            mid = tuple(wl["x"][p] for p in wl["perms"][0])
+            self.calls = [((ctypes.c_int64 * nd)(*wl["x"]), (ctypes.c_int32 * nd)(*wl["perms"][0])),
+                          ((ctypes.c_int64 * nd)(*mid), (ctypes.c_int32 * nd)(*wl["perms"][1]))]
+            self.nd = nd
+            self.work = {"permute": 2.0 * x.nbytes}
+            self.total_work = 4.0 * x.nbytes
+            self.unit, self.bound, self.peak = "GB/s", "hbm", PEAK_HBM_GBS
+            self.scale = 1e-9
+        elif wl["kind"] == "einsum":
+            x = rng.standard_normal(wl["x"]).astype(dt)
+            w = (rng.standard_normal(wl["w"]) * wl["w"][1] ** -0.5).astype(dt)
+            la, lb, lo = wl["subscripts"]
+            self.sizes = {**dict(zip(la, wl["x"])), **dict(zip(lb, wl["w"]))}
+            g = rng.standard_normal(tuple(self.sizes[l] for l in lo)).astype(dt)
+            self.x, self.w, self.g = resident(x), resident(w), resident(g)
+            self.np_dtype = np.dtype(dt)
+            per_pass = 2.0 * np.prod([float(v) for v in self.sizes.values()])
+            self.work = {"conv_fwd": per_pass, "conv_wgrad": per_pass}
             self.total_work = 3 * per_pass
             self.unit, self.bound, self.peak = "TFLOP/s", "mfma", PEAK_TFLOPS[wl["dtype"]]
             self.scale = 1e-12
@@ -269,6 +307,19 @@ class Step:
             check(lib.mg_matmul(self.code, *self.dims, self.w.ptr, self.x.ptr, self.out.ptr))
             check(lib.mg_matmul_dx(self.code, *self.dims, self.g.ptr, self.w.ptr, self.dx.ptr))
             check(lib.mg_matmul_da(self.code, *self.dims, self.g.ptr, self.x.ptr, self.dw.ptr))
+            return
+        if self.wl["kind"] == "permute":
+            item = 4 if self.wl["dtype"] == "f32" else 8
+            check(lib.mg_permute(item, self.nd, *self.calls[0], self.x.ptr, self.out.ptr))
+            check(lib.mg_permute(item, self.nd, *self.calls[1], self.out.ptr, self.back.ptr))
+            return
+        if self.wl["kind"] == "einsum":
+            from mygrad_amd.linalg.ops import contract
+
+            la, lb, lo = self.wl["subscripts"]
+            contract([(self.x, la), (self.w, lb)], lo, self.sizes, self.np_dtype)
+            contract([(self.g, lo), (self.w, lb)], la, self.sizes, self.np_dtype)
+            contract([(self.g, lo), (self.x, la)], lb, self.sizes, self.np_dtype)
             return
         if self.wl["kind"] == "sumover":
             check(lib.mg_sum_over(self.code, *self.dims, 0, self.x.ptr, self.out.ptr))
@@ -411,6 +462,35 @@ def run_cpu_baseline(name, min_seconds=10.0, max_reps=200):
 
         work, scale, unit = 6.0 * M * K * N, 1e-12, "TFLOP/s"
         what = "product and both gradients (three BLAS sgemm calls)"
+    elif wl["kind"] == "permute":
+        x = rng.standard_normal(wl["x"]).astype(dt)
+
+        def once():
+            mid = np.ascontiguousarray(np.transpose(x, wl["perms"][0]))
+            np.ascontiguousarray(np.transpose(mid, wl["perms"][1]))
+
+        work, scale, unit = 4 * x.nbytes, 1e-9, "GB/s"
+        what = "np.ascontiguousarray(np.transpose(...)) twice"
+    elif wl["kind"] == "einsum":
+        x = rng.standard_normal(wl["x"]).astype(dt)
+        w = rng.standard_normal(wl["w"]).astype(dt)
+        la, lb, lo = wl["subscripts"]
+        sizes = {**dict(zip(la, wl["x"])), **dict(zip(lb, wl["w"]))}
+        g = rng.standard_normal(tuple(sizes[l] for l in lo)).astype(dt)
+        # np.einsum without optimize=True (the reference's default) does not call BLAS: an eighth
+        # of the batch keeps one repetition to a few seconds
+        part = max(1, wl["x"][0] // 8)
+        x, g = np.ascontiguousarray(x[:part]), np.ascontiguousarray(g[:part])
+        sizes[la[0]] = part
+
+        def once():
+            ora.einsum_forward(f"{la},{lb}", lo, x, w)
+            ora.einsum_backward(g, 0, f"{la},{lb}", lo, [x, w])
+            ora.einsum_backward(g, 1, f"{la},{lb}", lo, [x, w])
+
+        work, scale, unit = 6.0 * np.prod([float(v) for v in sizes.values()]), 1e-12, "TFLOP/s"
+        what = f"np.einsum for the product and both gradients on {part} of the {wl['x'][0]} batch entries"
+        whole = False
     elif wl["kind"] == "sumover":
         x = rng.standard_normal(wl["x"]).astype(dt)
 
@@ -478,6 +558,7 @@ def run_cpu_baseline(name, min_seconds=10.0, max_reps=200):
 
         work, scale, unit = 3 * x.nbytes + 2 * g.nbytes, 1e-9, "GB/s"
         what = "fwd+bwd"
+    whole = locals().get("whole", True)
     reps, t0 = 0, time.perf_counter()
     while True:
         once()
@@ -490,7 +571,7 @@ def run_cpu_baseline(name, min_seconds=10.0, max_reps=200):
         "unit": unit,
         "cores": blas_threads() if wl["kind"] in ("conv", "matmul") else 1,
         "kind": "port",
-        "sample": f"the whole workload ({what}), {reps} repetition(s), {elapsed:.1f} s of host time",
+        "sample": f"{'the whole workload' if whole else 'a part of the workload'} ({what}), {reps} repetition(s), {elapsed:.1f} s of host time",
         "numpy": np.__version__,
     }
 
@@ -529,6 +610,18 @@ def run_dropin(name, steps=5):
             (at @ xt).backward(g)
 
         work, scale, unit = 6.0 * M * K * N, 1e-12, "TFLOP/s"
+    elif wl["kind"] == "permute":
+        return {"skipped": "transposition is a building block of einsum here, not an operation of its own"}
+    elif wl["kind"] == "einsum":
+        w = rng.standard_normal(wl["w"]).astype(dt)
+        la, lb, lo = wl["subscripts"]
+        sizes = {**dict(zip(la, wl["x"])), **dict(zip(lb, wl["w"]))}
+        g = rng.standard_normal(tuple(sizes[l] for l in lo)).astype(dt)
+
+        def once():
+            mg.einsum(f"{la},{lb}->{lo}", mg.Tensor(x, copy=False), mg.Tensor(w, copy=False)).backward(g)
+
+        work, scale, unit = 6.0 * np.prod([float(v) for v in sizes.values()]), 1e-12, "TFLOP/s"
     elif wl["kind"] == "sumover":
 
         def once():
@@ -667,7 +760,7 @@ def main():
         "metric": {"conv": "conv_nd fwd+bwd TFLOP/s", "pool": "max_pool fwd+bwd GB/s",
                    "elem": "relu+multiply+sum fwd+bwd GB/s", "bn": "batchnorm fwd+bwd GB/s",
                    "repeat": "repeat fwd+bwd GB/s", "matmul": "matmul fwd+bwd TFLOP/s", "window": "sliding-window copy GB/s",
-                   "sumover": "sum over axes GB/s"}[wl["kind"]],
+                   "sumover": "sum over axes GB/s", "permute": "transposition GB/s", "einsum": "einsum fwd+bwd TFLOP/s"}[wl["kind"]],
         "value": res["value"],
         "unit": res["unit"],
         "n_gpus": 1,

@@ -7,8 +7,12 @@ contracted labels (both operands, not the result), row labels (first operand and
 and column labels (second operand and result); the operands are transposed on the device
 to ``(batch, rows, contracted)`` and ``(batch, contracted, columns)`` (``mg_permute``),
 multiplied (``mg_matmul``, one launch per batch entry), and the product is transposed into
-the order the subscripts ask for.  The gradient of an operand is, as in the reference, the
-same kind of summation with the incoming gradient in the operand's place.
+the order the subscripts ask for.  Two arrangements need no transposition of the large
+tensors and are recognised first: a convolution with a one-element window written as a
+summation (``"nchw,fc->nfhw"`` and its input gradient: ``mg_matmul`` with the leading labels
+as the batch) and its filter gradient (``"nfhw,nchw->fc"``: ``mg_matmul_da``); a plain
+matrix product is the first of them.  The gradient of an operand is, as in the reference,
+the same kind of summation with the incoming gradient in the operand's place.
 
 What runs: one or two float32 / float64 operands, no label repeated within one operand (no
 traces or diagonals), every label of the same length wherever it occurs.  Anything else
@@ -49,6 +53,65 @@ def _ordered(buf, lbls, order, sizes, dtype):
     return _reduce.permute(buf, tuple(sizes[lbl] for lbl in lbls), perm, dtype)
 
 
+def _block(lbls, members):
+    """Where the labels ``members`` sit in ``lbls`` if they form one run there: (start, stop),
+    (n, n) for no members at all; None if they are scattered."""
+    at = [n for n, lbl in enumerate(lbls) if lbl in members]
+    if not at:
+        return len(lbls), len(lbls)
+    return (at[0], at[-1] + 1) if at == list(range(at[0], at[-1] + 1)) else None
+
+
+def _shared_filter_form(operands, out_lbls, sizes, dtype):
+    """``out[o, m, i] = sum_k a[m, k] x[o, k, i]`` without moving ``x`` or the result: one operand
+    (``x``) already has its contracted labels in one run with free labels before (``o``) and
+    after (``i``) it, and the result is those with the other operand's free labels (``m``) in
+    between -- a convolution with a one-element window read straight from its tensors
+    (``mg_matmul`` with ``o`` as the batch).  Only the other operand is re-ordered."""
+    lib, code, item = _hip.lib(), _hip.dtype_code(dtype), dtype.itemsize
+    for which in sorted((0, 1), key=lambda n: -_prod(sizes[lbl] for lbl in operands[n][1])):  # the larger one as x
+        (xbuf, xl), (abuf, al) = operands[which], operands[1 - which]
+        summed = [lbl for lbl in xl if lbl in al]
+        if not summed or any(lbl in out_lbls for lbl in summed):
+            continue
+        run = _block(xl, summed)
+        if run is None:
+            continue
+        outer, inner = xl[: run[0]], xl[run[1] :]
+        rows = "".join(lbl for lbl in out_lbls if lbl in al)
+        if out_lbls != outer + rows + inner:
+            continue
+        abuf = _ordered(abuf, al, rows + xl[run[0] : run[1]], sizes, dtype)
+        B, M, K, N = (_prod(sizes[lbl] for lbl in group) for group in (outer, rows, summed, inner))
+        out = _device.DeviceBuffer(max(B * M * N * item, 16))
+        _hip.check(lib.mg_matmul(code, B, M, K, N, abuf.ptr, xbuf.ptr, out.ptr))
+        return out
+    return None
+
+
+def _joint_sum_form(operands, out_lbls, sizes, dtype):
+    """``out[r, c] = sum_{o, i} g[o, r, i] x[o, c, i]``: both operands carry the contracted labels
+    as the same run before and the same run after their own free labels -- the filter gradient
+    of that convolution (``mg_matmul_da`` with ``o`` as the batch).  Neither operand moves; the
+    (small) result is put into the order asked for."""
+    lib, code, item = _hip.lib(), _hip.dtype_code(dtype), dtype.itemsize
+    (gbuf, gl), (xbuf, xl) = operands
+    summed = set(gl) & set(xl)
+    if not summed or summed & set(out_lbls):
+        return None
+    grun, xrun = _block(gl, set(gl) - summed), _block(xl, set(xl) - summed)
+    if grun is None or xrun is None:
+        return None
+    if gl[: grun[0]] != xl[: xrun[0]] or gl[grun[1] :] != xl[xrun[1] :]:
+        return None
+    outer, inner = gl[: grun[0]], gl[grun[1] :]
+    rows, cols = gl[grun[0] : grun[1]], xl[xrun[0] : xrun[1]]
+    B, M, K, N = (_prod(sizes[lbl] for lbl in group) for group in (outer, rows, cols, inner))
+    out = _device.DeviceBuffer(max(M * K * item, 16))
+    _hip.check(lib.mg_matmul_da(code, B, M, K, N, gbuf.ptr, xbuf.ptr, out.ptr))
+    return _ordered(out, rows + cols, out_lbls, sizes, dtype)
+
+
 def contract(operands, out_lbls, sizes, dtype):
     """Device buffer with ``einsum(operands -> out_lbls)``: ``operands`` is one or two pairs
     (device buffer, labels), ``sizes`` maps each label to its length (none of them zero)."""
@@ -60,14 +123,35 @@ def contract(operands, out_lbls, sizes, dtype):
     (abuf, albl), (bbuf, blbl) = operands
     abuf, albl = _sum_away(abuf, albl, set(albl) - set(blbl) - set(out_lbls), sizes, dtype)
     bbuf, blbl = _sum_away(bbuf, blbl, set(blbl) - set(albl) - set(out_lbls), sizes, dtype)
+    operands = [(abuf, albl), (bbuf, blbl)]
+
+    # the two forms that leave the large tensors where they are
+    long_sum = _prod(sizes[lbl] for lbl in set(albl) & set(blbl)) >= _prod(sizes[lbl] for lbl in out_lbls)
+    forms = (_joint_sum_form, _shared_filter_form) if long_sum else (_shared_filter_form, _joint_sum_form)
+    for form in forms:
+        out = form(operands, out_lbls, sizes, dtype)
+        if out is not None:
+            return out
+
+    # the general way: both operands transposed to (batch, free, summed) order
     batch = "".join(lbl for lbl in out_lbls if lbl in albl and lbl in blbl)
     summed = "".join(lbl for lbl in albl if lbl in blbl and lbl not in out_lbls)
     rows = "".join(lbl for lbl in out_lbls if lbl in albl and lbl not in blbl)
     cols = "".join(lbl for lbl in out_lbls if lbl in blbl and lbl not in albl)
-    abuf = _ordered(abuf, albl, batch + rows + summed, sizes, dtype)
-    bbuf = _ordered(bbuf, blbl, batch + summed + cols, sizes, dtype)
     B, M, K, N = (_prod(sizes[lbl] for lbl in group) for group in (batch, rows, summed, cols))
     out = _device.DeviceBuffer(max(B * M * N * item, 16))
+    if K >= 4 * max(M, N):
+        # a long sum and a small result: the filter-gradient kernels, out = a @ b^T over the long axis
+        abuf = _ordered(abuf, albl, batch + rows + summed, sizes, dtype)
+        bbuf = _ordered(bbuf, blbl, batch + cols + summed, sizes, dtype)
+        for b in range(B):
+            _hip.check(lib.mg_matmul_da(code, 1, M, N, K, abuf.ptr + b * M * K * item, bbuf.ptr + b * N * K * item,
+                                        out.ptr + b * M * N * item))
+        return _ordered(out, batch + rows + cols, out_lbls, sizes, dtype)
+    if N < M:  # the longer free axis plays the positions of the convolution, the other its filters
+        (abuf, albl, rows, M), (bbuf, blbl, cols, N) = (bbuf, blbl, cols, N), (abuf, albl, rows, M)
+    abuf = _ordered(abuf, albl, batch + rows + summed, sizes, dtype)
+    bbuf = _ordered(bbuf, blbl, batch + summed + cols, sizes, dtype)
     for b in range(B):
         _hip.check(lib.mg_matmul(code, 1, M, K, N, abuf.ptr + b * M * K * item, bbuf.ptr + b * K * N * item, out.ptr + b * M * N * item))
     return _ordered(out, batch + rows + cols, out_lbls, sizes, dtype)

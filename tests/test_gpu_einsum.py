@@ -38,6 +38,13 @@ CASES = [
     ("bhqd,bhkd->bhqk", [(2, 3, 16, 8), (2, 3, 12, 8)]), ("nchw,fc->nfhw", [(2, 16, 5, 5), (8, 16)]),
     ("ij,jk->ik", [(128, 256), (256, 64)]), ("ab,ab->", [(7, 9), (7, 9)]), ("ab,ab->ab", [(7, 9), (7, 9)]),
     ("i,i->i", [(5,), (5,)]), ("ij,j->i", [(0, 3), (3,)]), ("ij,jk->ik", [(2, 0), (0, 3)]),
+    # the arrangements that leave the large operand in place: a one-element-window convolution,
+    # its input gradient and its filter gradient
+    ("nchw,fc->nfhw", [(3, 16, 6, 5), (8, 16)]), ("nfhw,fc->nchw", [(3, 8, 6, 5), (8, 16)]), ("nfhw,nchw->fc", [(3, 8, 6, 5), (3, 16, 6, 5)]),
+    ("nfhw,nchw->cf", [(3, 8, 6, 5), (3, 16, 6, 5)]), ("fc,nchw->nfhw", [(8, 16), (3, 16, 6, 5)]),
+    # and ones that fit neither: a long scattered sum (filter-gradient kernels), a tall result (roles swapped)
+    ("iaj,jbi->ab", [(40, 2, 30), (30, 3, 40)]), ("ai,ib->ba", [(50, 4), (4, 3)]), ("ij,j->i", [(300, 7), (7,)]),
+    ("j,jk->k", [(9,), (9, 4)]),
 ]
 
 
