@@ -376,15 +376,19 @@ __global__ void __launch_bounds__(256) permute_rows_kernel(PermuteParams p, cons
   out[t] = x[at];
 }
 
-template <int BYTES>
+// VEC elements (16 bytes, or one element when the extents or the pointers do not allow it) per
+// lane on both sides: along axis p when reading, along the last axis when writing.
+template <int BYTES, int VEC>
 __global__ void __launch_bounds__(256) permute_tile_kernel(PermuteParams p, const typename Word<BYTES>::type *__restrict__ x,
                                                            typename Word<BYTES>::type *__restrict__ out) {
   typedef typename Word<BYTES>::type W;
+  typedef W WV __attribute__((ext_vector_type(VEC)));
+  constexpr int LX = 32 / VEC, LY = 256 / LX, ITERS = 32 / LY;
   __shared__ W tile[32][33];
   const int last = p.nd - 1;
   const unsigned tr = p.by_tiles_c.div(blockIdx.x), tc = blockIdx.x - tr * p.tiles_c;
   const unsigned r0 = tr * 32u, c0 = tc * 32u;
-  const unsigned tx = threadIdx.x & 31u, ty = threadIdx.x >> 5;
+  const unsigned tx = threadIdx.x % LX, ty = threadIdx.x / LX;
   const unsigned rn = p.size[p.p_axis], cn = p.size[last];
   const long long sc = p.in_stride[last];
   for (unsigned rest = blockIdx.y; rest < p.nrest; rest += gridDim.y) {
@@ -404,15 +408,34 @@ __global__ void __launch_bounds__(256) permute_tile_kernel(PermuteParams p, cons
       out_stride *= p.size[k];
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const unsigned r = r0 + tx, c = c0 + ty + 8u * j;
-      if (r < rn && c < cn) tile[ty + 8 * j][tx] = x[in0 + r + (long long)c * sc];
+    for (int j = 0; j < ITERS; ++j) {
+      const unsigned r = r0 + tx * VEC, row = ty + LY * j, c = c0 + row;
+      if (r < rn && c < cn) {  // VEC > 1: rn is a multiple of VEC, so the whole piece is inside
+        const W *src = x + in0 + r + (long long)c * sc;
+        if constexpr (VEC == 1) {
+          tile[row][tx] = *src;
+        } else {
+          const WV v = *reinterpret_cast<const WV *>(src);
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) tile[row][tx * VEC + k] = v[k];
+        }
+      }
     }
     __syncthreads();
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const unsigned c = c0 + tx, r = r0 + ty + 8u * j;
-      if (r < rn && c < cn) out[out0 + (long long)r * p.p_out_stride + c] = tile[tx][ty + 8 * j];
+    for (int j = 0; j < ITERS; ++j) {
+      const unsigned c = c0 + tx * VEC, row = ty + LY * j, r = r0 + row;
+      if (r < rn && c < cn) {
+        W *dst = out + out0 + (long long)r * p.p_out_stride + c;
+        if constexpr (VEC == 1) {
+          *dst = tile[tx][row];
+        } else {
+          WV v;
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) v[k] = tile[tx * VEC + k][row];
+          *reinterpret_cast<WV *>(dst) = v;
+        }
+      }
     }
     __syncthreads();
   }
@@ -674,10 +697,22 @@ int mg_permute(int elem_bytes, int nd, const int64_t *shape, const int32_t *perm
     p.by_tiles_c = make_fastdiv_t(p.tiles_c);
     p.nrest = (unsigned)rest;
     const dim3 grid(p.tiles_c * p.tiles_r, (unsigned)std::min<long long>(rest, 65535));
-    if (elem_bytes == 8)
-      hipLaunchKernelGGL(permute_tile_kernel<8>, grid, block, 0, s, p, (const unsigned long long *)x, (unsigned long long *)out);
-    else
-      hipLaunchKernelGGL(permute_tile_kernel<4>, grid, block, 0, s, p, (const unsigned *)x, (unsigned *)out);
+    // 16 bytes per lane when both tiled extents are whole pieces (every other stride on either
+    // side is a multiple of one of them) and the tensors are aligned
+    const long long per16 = 16 / elem_bytes;
+    const uintptr_t bits = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out);
+    const bool wide = size[p.p_axis] % per16 == 0 && size[m - 1] % per16 == 0 && bits % 16 == 0;
+    if (elem_bytes == 8) {
+      if (wide)
+        hipLaunchKernelGGL((permute_tile_kernel<8, 2>), grid, block, 0, s, p, (const unsigned long long *)x, (unsigned long long *)out);
+      else
+        hipLaunchKernelGGL((permute_tile_kernel<8, 1>), grid, block, 0, s, p, (const unsigned long long *)x, (unsigned long long *)out);
+    } else {
+      if (wide)
+        hipLaunchKernelGGL((permute_tile_kernel<4, 4>), grid, block, 0, s, p, (const unsigned *)x, (unsigned *)out);
+      else
+        hipLaunchKernelGGL((permute_tile_kernel<4, 1>), grid, block, 0, s, p, (const unsigned *)x, (unsigned *)out);
+    }
   }
   MG_HIP(hipGetLastError());
   return MG_OK;
