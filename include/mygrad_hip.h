@@ -111,7 +111,7 @@ int mg_device_info(mg_device_info_t *info);
  * off; at most a quarter of the device's memory is kept idle. */
 int mg_malloc(void **dptr, size_t nbytes);
 int mg_free(void *dptr);
-int mg_host_alloc(void **hptr, size_t nbytes); /* pinned host memory (hipHostMalloc) */
+int mg_host_alloc(void **hptr, size_t nbytes); /* pinned host memory (hipHostMalloc); blocks given back are reused like device blocks, at most 8 GiB kept idle */
 int mg_host_free(void *hptr);
 int mg_memcpy_h2d(void *dst_dev, const void *src_host, size_t nbytes); /* stream-ordered, returns when src may be reused */
 int mg_memcpy_d2h(void *dst_host, const void *src_dev, size_t nbytes); /* returns when dst holds the data */

@@ -175,9 +175,17 @@ struct BlockPool {
   std::unordered_map<void *, size_t> size_of;   // every block of the pool, in use or idle
   size_t idle_bytes = 0;
   bool off = false;                             // MYGRAD_HIP_POOL=0: plain hipMalloc / hipFree
+  bool pinned = false;                          // blocks of pinned host memory (hipHostMalloc)
 };
 BlockPool &pool() {
   static BlockPool p;
+  return p;
+}
+// Pinned host blocks (results are downloaded into them): allocating and releasing 100 MB
+// of pinned memory costs about as much as copying it over the link.
+BlockPool &host_pool() {
+  static BlockPool p;
+  p.pinned = true;
   return p;
 }
 size_t pool_round(size_t n) {
@@ -185,13 +193,15 @@ size_t pool_round(size_t n) {
   return (n + unit - 1) / unit * unit;
 }
 // Gives idle blocks back to the driver until at most `keep` bytes of them are left.
-void pool_trim(size_t keep) {
-  BlockPool &bp = pool();
+void pool_trim(size_t keep, BlockPool &bp = pool()) {
   if (bp.idle_bytes <= keep) return;
   (void)hipStreamSynchronize(runtime().stream);  // work enqueued before the blocks were given back
   while (bp.idle_bytes > keep && !bp.idle.empty()) {
     auto largest = std::prev(bp.idle.end());
-    (void)hipFree(largest->second);
+    if (bp.pinned)
+      (void)hipHostFree(largest->second);
+    else
+      (void)hipFree(largest->second);
     bp.idle_bytes -= largest->first;
     bp.size_of.erase(largest->second);
     bp.idle.erase(largest);
@@ -245,6 +255,7 @@ int mg_shutdown(void) {
   rt.workspace = nullptr;
   rt.workspace_bytes = 0;
   pool_trim(0);  // idle blocks go back to the driver; blocks still held by callers stay theirs
+  pool_trim(0, host_pool());
   MG_HIP(hipStreamDestroy(rt.stream));
   rt.stream = nullptr;
   rt.ready = false;
@@ -328,7 +339,30 @@ int mg_host_alloc(void **hptr, size_t nbytes) {
   if (!hptr) return fail(MG_ERR_BAD_ARG, "hptr is null");
   *hptr = nullptr;
   if (nbytes == 0) nbytes = 64;
-  MG_HIP(hipHostMalloc(hptr, nbytes, hipHostMallocDefault));
+  BlockPool &bp = host_pool();
+  if (pool().off) {
+    MG_HIP(hipHostMalloc(hptr, nbytes, hipHostMallocDefault));
+    return MG_OK;
+  }
+  const size_t want = pool_round(nbytes);
+  auto fit = bp.idle.lower_bound(want);
+  if (fit != bp.idle.end() && fit->first <= want + want / 4) {
+    *hptr = fit->second;
+    bp.idle_bytes -= fit->first;
+    bp.idle.erase(fit);
+    return MG_OK;
+  }
+  hipError_t err = hipHostMalloc(hptr, want, hipHostMallocDefault);
+  if (err != hipSuccess && bp.idle_bytes > 0) {
+    (void)hipGetLastError();
+    pool_trim(0, bp);
+    err = hipHostMalloc(hptr, want, hipHostMallocDefault);
+  }
+  if (err != hipSuccess) {
+    *hptr = nullptr;
+    return hip_fail(err, "hipHostMalloc", __FILE__, __LINE__);
+  }
+  bp.size_of[*hptr] = want;
   return MG_OK;
 }
 
@@ -336,7 +370,17 @@ int mg_host_free(void *hptr) {
   MG_LOCK();
   MG_REQUIRE_INIT();
   if (!hptr) return MG_OK;
-  MG_HIP(hipHostFree(hptr));
+  BlockPool &bp = host_pool();
+  auto known = bp.size_of.find(hptr);
+  if (known == bp.size_of.end()) {
+    MG_HIP(hipHostFree(hptr));
+    return MG_OK;
+  }
+  // copies into and out of pinned blocks return only when they are done, so nothing is in flight
+  bp.idle.emplace(known->second, hptr);
+  bp.idle_bytes += known->second;
+  const size_t limit = size_t(8) << 30;  // at most 8 GiB of pinned memory kept idle
+  if (bp.idle_bytes > limit) pool_trim(limit / 2, bp);
   return MG_OK;
 }
 
