@@ -1,6 +1,6 @@
 """``EinSum`` on the MI355X (reference: ``mygrad/linalg/ops.py:79-262``).
 
-An Einstein summation of one or two operands is brought into the form the matrix-product
+An Einstein summation (of one or two operands at a time) is brought into the form the matrix-product
 kernels take: labels that occur in one operand only and not in the result are summed away
 first (``mg_sum_over``); the others fall into batch labels (both operands and the result),
 contracted labels (both operands, not the result), row labels (first operand and result)
@@ -14,8 +14,9 @@ as the batch) and its filter gradient (``"nfhw,nchw->fc"``: ``mg_matmul_da``); a
 matrix product is the first of them.  The gradient of an operand is, as in the reference,
 the same kind of summation with the incoming gradient in the operand's place.
 
-What runs: one or two float32 / float64 operands, no label repeated within one operand (no
-traces or diagonals), every label of the same length wherever it occurs.  Anything else
+What runs: float32 / float64 operands (more than two are contracted pairwise from the
+left), no label repeated within one operand (no traces or diagonals), every label of the
+same length wherever it occurs.  Anything else
 raises ``NotImplementedError``; there is no CPU fallback.  The result is always a new
 array, never a view of an operand."""
 
@@ -157,6 +158,18 @@ def contract(operands, out_lbls, sizes, dtype):
     return _ordered(out, batch + rows + cols, out_lbls, sizes, dtype)
 
 
+def contract_all(operands, out_lbls, sizes, dtype):
+    """``contract`` for any number of operands: the first two are contracted onto the labels
+    that are still needed (by the operands that follow, or by the result) until two are left."""
+    operands = list(operands)
+    while len(operands) > 2:
+        (abuf, albl), (bbuf, blbl) = operands[:2]
+        needed = set(out_lbls) | set(chain.from_iterable(lbls for _, lbls in operands[2:]))
+        keep = "".join(dict.fromkeys(lbl for lbl in albl + blbl if lbl in needed))
+        operands[:2] = [(contract([(abuf, albl), (bbuf, blbl)], keep, sizes, dtype), keep)]
+    return contract(operands, out_lbls, sizes, dtype)
+
+
 class EinSum(Operation):
     gradient_on_device = True
 
@@ -189,8 +202,6 @@ class EinSum(Operation):
         if not set(out_lbls) <= set(sizes):
             raise ValueError(f"einstein sum subscripts string included output subscript which never appeared in an input: '{out_lbls}'")
 
-        if len(arrays) not in (1, 2):
-            raise NotImplementedError(f"einsum on the GPU takes one or two operands, got {len(arrays)} (no CPU fallback)")
         if any(len(set(lbls)) != len(lbls) for lbls in self.in_lbls):
             raise NotImplementedError("einsum on the GPU does not take a label twice within one operand (traces, diagonals)")
         dtype = np.dtype(np.result_type(*arrays))
@@ -202,7 +213,7 @@ class EinSum(Operation):
         if 0 in sizes.values():  # an empty sum is zero, an empty result has nothing in it
             return np.zeros(out_shape, dtype=dtype)
         operands = [(_device.to_device(arr, dtype), lbls) for arr, lbls in zip(arrays, self.in_lbls)]
-        ob = contract(operands, out_lbls, sizes, dtype)
+        ob = contract_all(operands, out_lbls, sizes, dtype)
         if any(ob is buf for buf, _ in operands):  # nothing was summed or moved: the result is a copy
             copy = _device.DeviceBuffer(max(_prod(out_shape) * dtype.itemsize, 16))
             _hip.check(_hip.lib().mg_memcpy_d2d(copy.ptr, ob.ptr, _prod(out_shape) * dtype.itemsize))
@@ -242,7 +253,7 @@ class EinSum(Operation):
         operands = [(_device.to_device(np.ascontiguousarray(grad), dtype), self.out_lbls)]
         operands += [(_device.to_device(v.data, dtype), lbls)
                      for n, (v, lbls) in enumerate(zip(self.variables, self.in_lbls)) if n != index]
-        ob = contract(operands, found, sizes, dtype)
+        ob = contract_all(operands, found, sizes, dtype)
         if found != var_lbl:
             ob = _reduce.broadcast(ob, tuple(sizes[lbl] if lbl in elsewhere else 1 for lbl in var_lbl), var.shape, dtype)
         nbytes = var.data.size * dtype.itemsize

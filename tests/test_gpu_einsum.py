@@ -45,6 +45,9 @@ CASES = [
     # and ones that fit neither: a long scattered sum (filter-gradient kernels), a tall result (roles swapped)
     ("iaj,jbi->ab", [(40, 2, 30), (30, 3, 40)]), ("ai,ib->ba", [(50, 4), (4, 3)]), ("ij,j->i", [(300, 7), (7,)]),
     ("j,jk->k", [(9,), (9, 4)]),
+    # more than two operands: contracted pairwise from the left
+    ("ij,jk,kl->il", [(3, 4), (4, 5), (5, 2)]), ("bi,bj,bk->ijk", [(4, 2), (4, 3), (4, 5)]), ("i,ij,j->", [(3,), (3, 4), (4,)]),
+    ("ab,bc,cd,da->", [(2, 3), (3, 4), (4, 5), (5, 2)]),
 ]
 
 
@@ -99,6 +102,9 @@ def test_a_tensor_that_occurs_twice_gets_one_gradient_scaled_by_two():
     y = mg.Tensor(np.arange(6.0).reshape(2, 3))
     mg.einsum("ij,ij->j", y, y).backward(np.array([1.0, 10.0, 100.0]))
     assert np.array_equal(y.grad, 2 * y.data * np.array([1.0, 10.0, 100.0]))
+    w = mg.Tensor(np.arange(1.0, 4.0))
+    mg.einsum("i,i,i->", w, w, w).backward()
+    assert np.array_equal(w.grad, 3 * w.data**2)
     # the same tensor under different labels is two different pairs
     z = mg.Tensor(np.arange(4.0).reshape(2, 2))
     mg.einsum("ij,jk->ik", z, z).backward()
@@ -119,8 +125,6 @@ def test_errors_and_what_is_refused():
         mg.einsum("ij,jk->ii", a, b)
     with pytest.raises(NotImplementedError):
         mg.einsum("ii->i", mg.Tensor(np.ones((3, 3))))  # a diagonal
-    with pytest.raises(NotImplementedError):
-        mg.einsum("ij,jk,kl->il", a, b, mg.Tensor(np.ones((4, 2))))
     with pytest.raises(NotImplementedError):
         mg.einsum("ij,ij->ij", a, mg.Tensor(np.ones((1, 3))))  # a label of length one broadcast
     with pytest.raises(TypeError):

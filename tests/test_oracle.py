@@ -643,6 +643,7 @@ EINSUM_CASES = [
     ("ijk,jil->kl", [(3, 4, 5), (4, 3, 2)]), ("i,i->", [(6,), (6,)]), ("i,j->ji", [(3,), (4,)]), ("ij->ji", [(3, 4)]),
     ("ijk->j", [(2, 3, 4)]), ("ij,jk->i", [(3, 4), (4, 5)]), ("ij,k->", [(2, 3), (4,)]), ("abc,cd->dab", [(2, 3, 4), (4, 5)]),
     (",ij->ij", [(), (2, 3)]), ("aib,ajb->abij", [(2, 3, 4), (2, 5, 4)]), ("ij->", [(3, 4)]), ("ij->ij", [(2, 3)]),
+    ("ij,jk,kl->il", [(3, 4), (4, 5), (5, 2)]), ("bi,bj,bk->ijk", [(4, 2), (4, 3), (4, 5)]),
 ]
 
 
