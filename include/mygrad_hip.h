@@ -257,6 +257,18 @@ int mg_sum_over(int dtype, int64_t outer, int64_t n, int64_t inner, int over_mid
  * EinSum.backward_var, src/mygrad/linalg/ops.py:79-110 and :112-262. */
 int mg_permute(int elem_bytes, int nd, const int64_t *shape, const int32_t *perm, const void *x, void *out);
 
+/* Copy between a dense array of `shape` (C-contiguous) and an array of `extent` elements
+ * addressed through `strides` (in elements, not negative): element (i_0, ...) of the dense side
+ * pairs with offset sum_k i_k * strides[k] of the other.  scatter = 0: out (dense) takes its
+ * values from x at those offsets; scatter = 1: x (dense) is written to out at those offsets,
+ * which must differ between elements, the rest of out is left as it is.  At most 6 axes.
+ * With the sum of several of a tensor's strides as one stride this takes out, and writes back,
+ * the diagonals behind a label that occurs twice in one operand of an Einstein summation:
+ * np.einsum("ii->i") in EinSum.__call__ and the as_strided view that EinSum.backward_var
+ * writes through, src/mygrad/linalg/ops.py:220-262. */
+int mg_strided_copy(int elem_bytes, int nd, const int64_t *shape, const int64_t *strides, int64_t extent, int scatter, const void *x,
+                    void *out);
+
 /* ---- matrix product ---- */
 
 /* out[b] = a @ x[b], a:(M, K) shared by the batch, x:(batch, K, N), out:(batch, M, N), all

@@ -158,6 +158,8 @@ _SIGNATURES = {
     "mg_repeat_fwd": [ctypes.c_int] + [ctypes.c_int64] * 5 + [_vp, _vp, _vp],
     "mg_repeat_bwd": [ctypes.c_int] + [ctypes.c_int64] * 5 + [_vp, _vp, _vp],
     "mg_window_gather": [ctypes.POINTER(WindowDesc), _vp, _vp],
+    "mg_strided_copy": [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64), ctypes.c_int64,
+                        ctypes.c_int, _vp, _vp],
     "mg_permute": [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int32), _vp, _vp],
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES) + ("mg_last_error",)

@@ -441,6 +441,39 @@ __global__ void __launch_bounds__(256) permute_tile_kernel(PermuteParams p, cons
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Copy between a dense array and an array addressed through arbitrary strides: element
+// (i_0, ..., i_{nd-1}) of the dense side pairs with offset sum_k i_k * stride_k of the other.
+// With a stride that is the sum of two of a tensor's strides this walks a diagonal:
+// gather takes it out (dense[t] = strided[off]), scatter writes it back (strided[off] =
+// dense[t]; the offsets of distinct elements must differ).
+// ------------------------------------------------------------------------------------------
+struct StridedParams {
+  int nd;
+  unsigned size[kMaxPermuteAxes];
+  long long stride[kMaxPermuteAxes];
+  FastDivT by_size[kMaxPermuteAxes];
+  unsigned total;
+};
+
+template <int BYTES, bool SCATTER>
+__global__ void __launch_bounds__(256) strided_copy_kernel(StridedParams p, const typename Word<BYTES>::type *__restrict__ src,
+                                                           typename Word<BYTES>::type *__restrict__ dst) {
+  const unsigned t = blockIdx.x * 256u + threadIdx.x;
+  if (t >= p.total) return;
+  unsigned rem = t;
+  long long off = 0;
+  for (int k = p.nd - 1; k >= 0; --k) {
+    const unsigned q = p.by_size[k].div(rem);
+    off += (long long)(rem - q * p.size[k]) * p.stride[k];
+    rem = q;
+  }
+  if (SCATTER)
+    dst[off] = src[t];
+  else
+    dst[t] = src[off];
+}
+
 }  // namespace
 }  // namespace mg
 
@@ -714,6 +747,48 @@ int mg_permute(int elem_bytes, int nd, const int64_t *shape, const int32_t *perm
         hipLaunchKernelGGL((permute_tile_kernel<4, 1>), grid, block, 0, s, p, (const unsigned *)x, (unsigned *)out);
     }
   }
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
+int mg_strided_copy(int elem_bytes, int nd, const int64_t *shape, const int64_t *strides, int64_t extent, int scatter, const void *x,
+                    void *out) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (elem_bytes != 4 && elem_bytes != 8) return fail(MG_ERR_UNSUPPORTED, "mg_strided_copy: element size %d (4 or 8 bytes)", elem_bytes);
+  if (nd < 1 || nd > kMaxPermuteAxes || !shape || !strides)
+    return fail(MG_ERR_BAD_ARG, "mg_strided_copy: nd = %d (1..%d) or null shape / strides", nd, kMaxPermuteAxes);
+  StridedParams p{};
+  p.nd = nd;
+  long long total = 1, reach = 0;
+  for (int k = 0; k < nd; ++k) {
+    if (shape[k] < 0 || strides[k] < 0) return fail(MG_ERR_BAD_ARG, "mg_strided_copy: negative extent or stride");
+    total *= shape[k];
+    if (total >= (1ll << 31)) return fail(MG_ERR_UNSUPPORTED, "mg_strided_copy: 2^31 or more elements");
+    if (shape[k] > 0) reach += (shape[k] - 1) * strides[k];
+    p.size[k] = (unsigned)shape[k];
+    p.stride[k] = strides[k];
+    p.by_size[k] = make_fastdiv_t((unsigned)std::max<int64_t>(shape[k], 1));
+  }
+  if (total == 0) return MG_OK;
+  if (reach >= extent) return fail(MG_ERR_BAD_ARG, "mg_strided_copy: the strides reach element %lld of %lld", reach, (long long)extent);
+  if (!x || !out) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_strided_copy");
+  p.total = (unsigned)total;
+  hipStream_t s = runtime().stream;
+  const dim3 grid((unsigned)ceil_div(total, 256)), block(256);
+  ScopedTiming timed(TAG_PERMUTE);
+#define MG_STRIDED(BYTES, W)                                                                                        \
+  do {                                                                                                              \
+    if (scatter)                                                                                                    \
+      hipLaunchKernelGGL((strided_copy_kernel<BYTES, true>), grid, block, 0, s, p, (const W *)x, (W *)out);         \
+    else                                                                                                            \
+      hipLaunchKernelGGL((strided_copy_kernel<BYTES, false>), grid, block, 0, s, p, (const W *)x, (W *)out);        \
+  } while (0)
+  if (elem_bytes == 8)
+    MG_STRIDED(8, unsigned long long);
+  else
+    MG_STRIDED(4, unsigned);
+#undef MG_STRIDED
   MG_HIP(hipGetLastError());
   return MG_OK;
 }

@@ -27,8 +27,8 @@ def einsum(*operands, optimize=False, out=None, constant=None):
         The labels of each operand's axes, separated by commas, and optionally those of
         the result after ``->``.
     operands : ArrayLike
-        float32 / float64 operands.  No label may occur twice within one operand,
-        and a label has the same length wherever it occurs (see the notes).
+        float32 / float64 operands; a label has the same length wherever it occurs
+        (see the notes).
     optimize : bool
         Accepted for compatibility; the order of evaluation is fixed.
     constant : Optional[bool]
@@ -41,8 +41,9 @@ def einsum(*operands, optimize=False, out=None, constant=None):
     Notes
     -----
     The summation runs on the matrix-product kernels after the operands have been transposed
-    on the device.  More than two operands are contracted pairwise from the left.  Traces and
-    diagonals (``"ii"``), broadcasting of a label of length one, and ``out=`` raise
+    on the device.  More than two operands are contracted pairwise from the left; a label
+    that occurs twice in one operand (``"ii"``: a trace or a diagonal) is taken along its
+    diagonal first.  Broadcasting of a label of length one and ``out=`` raise
     ``NotImplementedError``.  A tensor that occurs
     twice with the same labels receives one gradient, scaled by two, as in the reference.
     The result is a new array, where ``numpy.einsum`` may return a view.

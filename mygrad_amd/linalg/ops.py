@@ -15,8 +15,9 @@ matrix product is the first of them.  The gradient of an operand is, as in the r
 the same kind of summation with the incoming gradient in the operand's place.
 
 What runs: float32 / float64 operands (more than two are contracted pairwise from the
-left), no label repeated within one operand (no traces or diagonals), every label of the
-same length wherever it occurs.  Anything else
+left); a label repeated within one operand is taken along its diagonal first
+(``mg_strided_copy``), and its gradient is written back along that diagonal into zeros; every
+label has the same length wherever it occurs.  Anything else
 raises ``NotImplementedError``; there is no CPU fallback.  The result is always a new
 array, never a view of an operand."""
 
@@ -113,6 +114,40 @@ def _joint_sum_form(operands, out_lbls, sizes, dtype):
     return _ordered(out, rows + cols, out_lbls, sizes, dtype)
 
 
+def _last_of_each(lbls):
+    """``lbls`` with every label kept once, at its last position: "ijikik" -> "jik"
+    (the order the reference reduces a repeated label to, linalg/ops.py:21-42)."""
+    return "".join(lbl for n, lbl in enumerate(lbls) if lbl not in lbls[n + 1 :])
+
+
+def _diagonal_strides(lbls, once, sizes):
+    """Element strides that walk the C-contiguous operand labelled ``lbls`` along ``once``:
+    a label that occurs several times moves along all of its axes together."""
+    strides, step = {}, 1
+    for lbl in reversed(lbls):
+        strides[lbl] = strides.get(lbl, 0) + step
+        step *= sizes[lbl]
+    return [strides[lbl] for lbl in once]
+
+
+def _strided(buf, lbls, once, sizes, dtype, scatter):
+    """gather: the operand ``buf`` (labels ``lbls``, some repeated) -> its diagonal array labelled
+    ``once``.  scatter: the array ``buf`` labelled ``once`` -> zeros of the operand's shape with
+    ``buf`` written along those diagonals."""
+    import ctypes
+
+    lib, item = _hip.lib(), dtype.itemsize
+    full = _prod(sizes[lbl] for lbl in lbls)
+    dense = _prod(sizes[lbl] for lbl in once)
+    shape = (ctypes.c_int64 * len(once))(*(sizes[lbl] for lbl in once))
+    strides = (ctypes.c_int64 * len(once))(*_diagonal_strides(lbls, once, sizes))
+    out = _device.DeviceBuffer(max((full if scatter else dense) * item, 16))
+    if scatter:
+        _hip.check(lib.mg_memset_zero(out.ptr, full * item))
+    _hip.check(lib.mg_strided_copy(item, len(once), shape, strides, full, int(scatter), buf.ptr, out.ptr))
+    return out
+
+
 def contract(operands, out_lbls, sizes, dtype):
     """Device buffer with ``einsum(operands -> out_lbls)``: ``operands`` is one or two pairs
     (device buffer, labels), ``sizes`` maps each label to its length (none of them zero)."""
@@ -202,8 +237,8 @@ class EinSum(Operation):
         if not set(out_lbls) <= set(sizes):
             raise ValueError(f"einstein sum subscripts string included output subscript which never appeared in an input: '{out_lbls}'")
 
-        if any(len(set(lbls)) != len(lbls) for lbls in self.in_lbls):
-            raise NotImplementedError("einsum on the GPU does not take a label twice within one operand (traces, diagonals)")
+        if any(len(lbls) - len(set(lbls)) > 0 and len(set(lbls)) > 6 for lbls in self.in_lbls):
+            raise NotImplementedError("einsum on the GPU walks diagonals of operands with at most six distinct labels")
         dtype = np.dtype(np.result_type(*arrays))
         if dtype not in (np.float32, np.float64):
             raise TypeError(f"einsum runs on the GPU in float32 or float64, got {[str(a.dtype) for a in arrays]} (there is no CPU fallback)")
@@ -212,7 +247,7 @@ class EinSum(Operation):
         out_shape = tuple(sizes[lbl] for lbl in out_lbls)
         if 0 in sizes.values():  # an empty sum is zero, an empty result has nothing in it
             return np.zeros(out_shape, dtype=dtype)
-        operands = [(_device.to_device(arr, dtype), lbls) for arr, lbls in zip(arrays, self.in_lbls)]
+        operands = [self._operand(arr, lbls) for arr, lbls in zip(arrays, self.in_lbls)]
         ob = contract_all(operands, out_lbls, sizes, dtype)
         if any(ob is buf for buf, _ in operands):  # nothing was summed or moved: the result is a copy
             copy = _device.DeviceBuffer(max(_prod(out_shape) * dtype.itemsize, 16))
@@ -221,6 +256,15 @@ class EinSum(Operation):
         result = _device.download(ob, out_shape, dtype)
         _device.attach(result, ob)
         return result
+
+    def _operand(self, arr, lbls):
+        """(device buffer, labels) of one operand; a label that occurs twice is taken along its
+        diagonal first, which leaves every label once."""
+        buf = _device.to_device(arr, self._dtype)
+        once = _last_of_each(lbls)
+        if once == lbls:
+            return buf, lbls
+        return _strided(buf, lbls, once, self._sizes, self._dtype, scatter=False), once
 
     @property
     def cache(self):
@@ -249,13 +293,18 @@ class EinSum(Operation):
         # labels of this operand that were summed away on their own occur nowhere else: the
         # gradient is the same along them (linalg/ops.py:170-190)
         elsewhere = set(chain.from_iterable(others)) | set(self.out_lbls)
-        found = "".join(lbl for lbl in var_lbl if lbl in elsewhere)
+        once = _last_of_each(var_lbl)  # the operand's labels with its diagonals taken (linalg/ops.py:147-163)
+        found = "".join(lbl for lbl in once if lbl in elsewhere)
         operands = [(_device.to_device(np.ascontiguousarray(grad), dtype), self.out_lbls)]
-        operands += [(_device.to_device(v.data, dtype), lbls)
-                     for n, (v, lbls) in enumerate(zip(self.variables, self.in_lbls)) if n != index]
+        operands += [self._operand(v.data, lbls) for n, (v, lbls) in enumerate(zip(self.variables, self.in_lbls)) if n != index]
         ob = contract_all(operands, found, sizes, dtype)
-        if found != var_lbl:
-            ob = _reduce.broadcast(ob, tuple(sizes[lbl] if lbl in elsewhere else 1 for lbl in var_lbl), var.shape, dtype)
+        if found != once:
+            ob = _reduce.broadcast(ob, tuple(sizes[lbl] if lbl in elsewhere else 1 for lbl in once),
+                                   tuple(sizes[lbl] for lbl in once), dtype)
+        if once != var_lbl:
+            # the gradient lives on the diagonals the forward pass read; everything off them is
+            # zero (the reference writes through a strided view of zeros, linalg/ops.py:220-262)
+            ob = _strided(ob, var_lbl, once, sizes, dtype, scatter=True)
         nbytes = var.data.size * dtype.itemsize
         if factor > 1 or any(ob is buf for buf, _ in operands):
             # a buffer of its own, scaled by the number of times the pair occurs

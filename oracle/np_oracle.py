@@ -584,18 +584,21 @@ def einsum_forward(in_lbls, out_lbls, *arrays):
 
 
 def einsum_backward(grad, index, in_lbls, out_lbls, arrays, factor=1):
-    """``EinSum.backward_var`` for operands without a repeated label
-    (mygrad/linalg/ops.py:124-218): the operand's gradient is the summation of ``grad`` (in
-    the operand's place, labelled like the result) with the other operands onto the
-    operand's labels.  Labels of the operand that occur nowhere else were summed away on
-    their own, so ``grad`` is first given an axis for each of them, broadcast to its length.
-    ``factor`` is the number of times the same (tensor, labels) pair occurs among the
-    operands (the reference computes one gradient for all of them and scales it)."""
+    """``EinSum.backward_var`` (mygrad/linalg/ops.py:124-262): the operand's gradient is the
+    summation of ``grad`` (in the operand's place, labelled like the result) with the other
+    operands onto the operand's labels.  Labels of the operand that occur nowhere else were
+    summed away on their own, so ``grad`` is first given an axis for each of them, broadcast
+    to its length.  An operand with a repeated label (a trace or a diagonal) only ever read
+    its diagonal: the summation is made onto the labels taken once (each at its last
+    position, :21-42) and written along that diagonal into zeros (the reference writes
+    through a strided view, :220-262).  ``factor`` is the number of times the same (tensor,
+    labels) pair occurs among the operands (one gradient for all of them, scaled)."""
     lbls = in_lbls.split(",")
-    var_lbl = lbls.pop(index)
-    if len(set(var_lbl)) != len(var_lbl):
-        raise NotImplementedError("repeated labels within an operand (traces) are not restated")
-    var_shape = arrays[index].shape
+    full_lbl = lbls.pop(index)
+    var_lbl = "".join(lbl for n, lbl in enumerate(full_lbl) if lbl not in full_lbl[n + 1 :])
+    full_shape = arrays[index].shape
+    size = dict(zip(full_lbl, full_shape))
+    var_shape = tuple(size[lbl] for lbl in var_lbl)
     rest = tuple(a for n, a in enumerate(arrays) if n != index)
     known = set("".join(lbls)) | set(out_lbls)
     grad = np.asarray(grad)
@@ -613,4 +616,9 @@ def einsum_backward(grad, index, in_lbls, out_lbls, arrays, factor=1):
     back = reduce_broadcast(back, var_shape)
     if back.shape != var_shape:
         back = np.broadcast_to(back, var_shape)
+    if var_lbl != full_lbl:
+        along = np.indices(var_shape)
+        placed = np.zeros(full_shape, dtype=back.dtype)
+        placed[tuple(along[var_lbl.index(lbl)] for lbl in full_lbl)] = back
+        back = placed
     return back * factor if factor > 1 else back

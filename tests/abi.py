@@ -147,6 +147,24 @@ def permute(x, perm):
     return _down(ob, tuple(x.shape[p] for p in perm), x.dtype)
 
 
+def strided_copy(x, shape, strides, out_elems=None):
+    """gather (out_elems None): dense array of `shape` read from x at the strided offsets;
+    scatter: x (dense, of `shape`) written at those offsets into zeros of out_elems elements."""
+    import ctypes
+
+    nd = len(shape)
+    cs, ct = (ctypes.c_int64 * nd)(*shape), (ctypes.c_int64 * nd)(*strides)
+    xb = _up(x)
+    if out_elems is None:
+        ob = _device.DeviceBuffer(max(int(np.prod(shape)) * x.dtype.itemsize, 16))
+        _hip.check(_hip.lib().mg_strided_copy(x.dtype.itemsize, nd, cs, ct, x.size, 0, xb.ptr, ob.ptr))
+        return _down(ob, tuple(shape), x.dtype)
+    ob = _device.DeviceBuffer(max(out_elems * x.dtype.itemsize, 16))
+    _hip.check(_hip.lib().mg_memset_zero(ob.ptr, out_elems * x.dtype.itemsize))
+    _hip.check(_hip.lib().mg_strided_copy(x.dtype.itemsize, nd, cs, ct, out_elems, 1, xb.ptr, ob.ptr))
+    return _down(ob, (out_elems,), x.dtype)
+
+
 def sum_over(x3, over_middle):
     """x3:(outer, n, inner) -> sums over the middle axis (outer, inner) or over the other two (n,)."""
     outer, n, inner = x3.shape

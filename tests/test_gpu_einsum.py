@@ -48,6 +48,9 @@ CASES = [
     # more than two operands: contracted pairwise from the left
     ("ij,jk,kl->il", [(3, 4), (4, 5), (5, 2)]), ("bi,bj,bk->ijk", [(4, 2), (4, 3), (4, 5)]), ("i,ij,j->", [(3,), (3, 4), (4,)]),
     ("ab,bc,cd,da->", [(2, 3), (3, 4), (4, 5), (5, 2)]),
+    # a label twice within an operand: traces and diagonals
+    ("ii->", [(4, 4)]), ("ii->i", [(4, 4)]), ("iji->j", [(3, 2, 3)]), ("ijikik->jk", [(2, 3, 2, 4, 2, 4)]), ("ii,ij->j", [(3, 3), (3, 4)]),
+    ("ijj,jk->ik", [(2, 3, 3), (3, 4)]), ("iij->", [(3, 3, 2)]), ("bii->b", [(70, 65, 65)]), ("ii,jj->ij", [(3, 3), (4, 4)]),
 ]
 
 
@@ -86,6 +89,12 @@ def test_reference_docstring_vectors_in_both_calling_conventions(kats):
     a, b = np.arange(60.0).reshape(3, 4, 5), np.arange(24.0).reshape(4, 3, 2)
     got = mg.einsum(mg.Tensor(a), [0, 1, 2], mg.Tensor(b), [1, 0, 3], [2, 3])
     assert np.array_equal(got.data, [[4400, 4730], [4532, 4874], [4664, 5018], [4796, 5162], [4928, 5306]])
+    sq = mg.Tensor(np.arange(25.0).reshape(5, 5))
+    assert float(mg.einsum("ii", sq).data) == 60.0  # the docstring's trace
+    diag = mg.einsum("ii->i", sq)
+    assert np.array_equal(diag.data, [0, 6, 12, 18, 24])
+    diag.backward(np.arange(5.0))
+    assert np.array_equal(sq.grad, np.diag(np.arange(5.0)))
     # rearrangements are copies of values: exact, and never a view of the operand
     c = mg.Tensor(np.arange(6.0).reshape(2, 3))
     t = mg.einsum("ij->ji", c)
@@ -123,8 +132,8 @@ def test_errors_and_what_is_refused():
         mg.einsum("ijk,jk->i", a, b)  # three labels for two axes
     with pytest.raises(ValueError):
         mg.einsum("ij,jk->ii", a, b)
-    with pytest.raises(NotImplementedError):
-        mg.einsum("ii->i", mg.Tensor(np.ones((3, 3))))  # a diagonal
+    with pytest.raises(ValueError):
+        mg.einsum("ii->i", mg.Tensor(np.ones((3, 4))))  # the two axes of a diagonal differ in length
     with pytest.raises(NotImplementedError):
         mg.einsum("ij,ij->ij", a, mg.Tensor(np.ones((1, 3))))  # a label of length one broadcast
     with pytest.raises(TypeError):

@@ -233,3 +233,36 @@ def test_permute_rejects_bad_arguments(abi):
     seven = (ctypes.c_int64 * 7)(*([2] * 7))
     reverse = (ctypes.c_int32 * 7)(*range(6, -1, -1))
     assert lib.mg_permute(4, 7, seven, reverse, buf.ptr, buf.ptr) == _hip.MG_ERR_UNSUPPORTED  # seven axes that all move
+
+
+# ----------------------------------------------------------------------------- strided copy
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_strided_copy_walks_diagonals_both_ways(abi, dtype):
+    rng = np.random.default_rng(91)
+    x = rng.standard_normal((5, 7, 5)).astype(dtype)
+    # the diagonal over axes 0 and 2, laid out (i, j): strides (35 + 1, 5)
+    got = abi.strided_copy(x, (5, 7), (36, 5))
+    assert np.array_equal(got, np.einsum("iji->ij", x))
+    back = abi.strided_copy(got, (5, 7), (36, 5), out_elems=x.size).reshape(x.shape)
+    want = np.zeros_like(x)
+    i = np.arange(5)
+    want[i, :, i] = got
+    assert np.array_equal(back, want)
+    # a plain transposition is the same call
+    y = rng.standard_normal((30, 41)).astype(dtype)
+    assert np.array_equal(abi.strided_copy(y, (41, 30), (1, 41)), y.T)
+
+
+def test_strided_copy_rejects_what_would_leave_the_buffer(abi):
+    import ctypes
+
+    from mygrad_amd import _device, _hip
+
+    buf = _device.DeviceBuffer(4096)
+    lib = _hip.lib()
+    shape, strides = (ctypes.c_int64 * 2)(4, 4), (ctypes.c_int64 * 2)(5, 1)
+    assert lib.mg_strided_copy(4, 2, shape, strides, 19, 0, buf.ptr, buf.ptr) == _hip.MG_OK  # reaches element 3*5 + 3 = 18
+    assert lib.mg_strided_copy(4, 2, shape, strides, 18, 0, buf.ptr, buf.ptr) == _hip.MG_ERR_BAD_ARG
+    negative = (ctypes.c_int64 * 2)(5, -1)
+    assert lib.mg_strided_copy(4, 2, shape, negative, 64, 0, buf.ptr, buf.ptr) == _hip.MG_ERR_BAD_ARG
+    assert lib.mg_strided_copy(2, 2, shape, strides, 64, 0, buf.ptr, buf.ptr) == _hip.MG_ERR_UNSUPPORTED

@@ -417,8 +417,8 @@ def test_argument_checks_of_the_neighbouring_operations_need_no_device():
         mg.einsum("ij,jk->ik", np.ones((2, 3)), np.ones((4, 4)))
     with pytest.raises(ValueError):
         mg.einsum("ij,jk->ii", np.ones((2, 3)), np.ones((3, 4)))
-    with pytest.raises(NotImplementedError):
-        mg.einsum("ii", np.ones((3, 3)))
+    with pytest.raises(ValueError):
+        mg.einsum("ii", np.ones((3, 4)))
     with pytest.raises(TypeError):
         mg.einsum("i,i", np.arange(3), np.arange(3))
     assert mg.einsum("ij,jk->ik", np.ones((2, 0)), np.ones((0, 3))).shape == (2, 3)

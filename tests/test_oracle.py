@@ -644,6 +644,9 @@ EINSUM_CASES = [
     ("ijk->j", [(2, 3, 4)]), ("ij,jk->i", [(3, 4), (4, 5)]), ("ij,k->", [(2, 3), (4,)]), ("abc,cd->dab", [(2, 3, 4), (4, 5)]),
     (",ij->ij", [(), (2, 3)]), ("aib,ajb->abij", [(2, 3, 4), (2, 5, 4)]), ("ij->", [(3, 4)]), ("ij->ij", [(2, 3)]),
     ("ij,jk,kl->il", [(3, 4), (4, 5), (5, 2)]), ("bi,bj,bk->ijk", [(4, 2), (4, 3), (4, 5)]),
+    # a label twice within an operand: traces and diagonals
+    ("ii->", [(4, 4)]), ("ii->i", [(4, 4)]), ("iji->j", [(3, 2, 3)]), ("ijikik->jk", [(2, 3, 2, 4, 2, 4)]), ("ii,ij->j", [(3, 3), (3, 4)]),
+    ("ijj,jk->ik", [(2, 3, 3), (3, 4)]), ("iij->", [(3, 3, 2)]),
 ]
 
 
@@ -690,6 +693,15 @@ def test_einsum_backward_against_differences_adjoints_and_loops(subscripts, shap
         minus = [a - eps * direction if n == index else a for n, a in enumerate(arrays)]
         slope = float(np.sum((ora.einsum_forward(in_lbls, out_lbls, *plus) - ora.einsum_forward(in_lbls, out_lbls, *minus)) * g)) / (2 * eps)
         assert math.isclose(slope, float(np.sum(back * direction)), rel_tol=1e-6, abs_tol=1e-6)
+
+
+def test_einsum_reference_docstring_trace_and_diagonal():
+    a = np.arange(25.0).reshape(5, 5)
+    assert ora.einsum_forward("ii", "", a) == 60.0  # linalg/funcs.py docstring: the trace
+    assert np.array_equal(ora.einsum_forward("ii", "i", a), [0, 6, 12, 18, 24])  # and the diagonal
+    # their gradients: ones on the diagonal, nothing off it
+    assert np.array_equal(ora.einsum_backward(np.array(1.0), 0, "ii", "", [a]), np.eye(5))
+    assert np.array_equal(ora.einsum_backward(np.arange(5.0), 0, "ii", "i", [a]), np.diag(np.arange(5.0)))
 
 
 def test_einsum_backward_scales_a_repeated_pair():
