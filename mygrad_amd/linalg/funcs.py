@@ -27,8 +27,7 @@ def einsum(*operands, optimize=False, out=None, constant=None):
         The labels of each operand's axes, separated by commas, and optionally those of
         the result after ``->``.
     operands : ArrayLike
-        float32 / float64 operands; a label has the same length wherever it occurs
-        (see the notes).
+        float32 / float64 operands.
     optimize : bool
         Accepted for compatibility; the order of evaluation is fixed.
     constant : Optional[bool]
@@ -43,8 +42,8 @@ def einsum(*operands, optimize=False, out=None, constant=None):
     The summation runs on the matrix-product kernels after the operands have been transposed
     on the device.  More than two operands are contracted pairwise from the left; a label
     that occurs twice in one operand (``"ii"``: a trace or a diagonal) is taken along its
-    diagonal first.  Broadcasting of a label of length one and ``out=`` raise
-    ``NotImplementedError``.  A tensor that occurs
+    diagonal first; an axis of length one is broadcast against a longer one under the
+    same label.  ``out=`` raises ``NotImplementedError``.  A tensor that occurs
     twice with the same labels receives one gradient, scaled by two, as in the reference.
     The result is a new array, where ``numpy.einsum`` may return a view.
 

@@ -16,8 +16,8 @@ the same kind of summation with the incoming gradient in the operand's place.
 
 What runs: float32 / float64 operands (more than two are contracted pairwise from the
 left); a label repeated within one operand is taken along its diagonal first
-(``mg_strided_copy``), and its gradient is written back along that diagonal into zeros; every
-label has the same length wherever it occurs.  Anything else
+(``mg_strided_copy``), and its gradient is written back along that diagonal into zeros; an
+axis of length one under a label that is longer elsewhere is broadcast.  Anything else
 raises ``NotImplementedError``; there is no CPU fallback.  The result is always a new
 array, never a view of an operand."""
 
@@ -228,16 +228,26 @@ class EinSum(Operation):
             if len(lbls) != arr.ndim:
                 raise ValueError(f"einstein sum subscripts string '{lbls}' does not match the {arr.ndim} axes of its operand")
             for lbl, n in zip(lbls, arr.shape):
-                if sizes.setdefault(lbl, n) != n:
-                    if 1 in (sizes[lbl], n):
-                        raise NotImplementedError(f"einsum on the GPU does not broadcast label '{lbl}' (lengths {sizes[lbl]} and {n})")
-                    raise ValueError(f"operands could not be broadcast together: label '{lbl}' has lengths {sizes[lbl]} and {n}")
+                have = sizes.get(lbl)
+                if have is None or have == 1:
+                    sizes[lbl] = n
+                elif n not in (1, have):
+                    raise ValueError(f"operands could not be broadcast together: label '{lbl}' has lengths {have} and {n}")
+        # An axis of length one under a label that is longer elsewhere is broadcast: the operand
+        # does not depend on that label, so the label is struck from it (same memory), and
+        # its gradient is summed over the label like over any label it does not carry.
+        self._lbls = []
+        for lbls, arr in zip(self.in_lbls, arrays):
+            kept = "".join(lbl for lbl, n in zip(lbls, arr.shape) if n == sizes[lbl])
+            if kept != lbls and len(set(lbls)) != len(lbls):
+                raise NotImplementedError(f"einsum on the GPU does not broadcast an operand with a repeated label ('{lbls}')")
+            self._lbls.append(kept)
         if len(set(out_lbls)) != len(out_lbls):
             raise ValueError(f"einstein sum subscripts string includes output subscript more than once: '{out_lbls}'")
         if not set(out_lbls) <= set(sizes):
             raise ValueError(f"einstein sum subscripts string included output subscript which never appeared in an input: '{out_lbls}'")
 
-        if any(len(lbls) - len(set(lbls)) > 0 and len(set(lbls)) > 6 for lbls in self.in_lbls):
+        if any(len(lbls) - len(set(lbls)) > 0 and len(set(lbls)) > 6 for lbls in self._lbls):
             raise NotImplementedError("einsum on the GPU walks diagonals of operands with at most six distinct labels")
         dtype = np.dtype(np.result_type(*arrays))
         if dtype not in (np.float32, np.float64):
@@ -247,7 +257,7 @@ class EinSum(Operation):
         out_shape = tuple(sizes[lbl] for lbl in out_lbls)
         if 0 in sizes.values():  # an empty sum is zero, an empty result has nothing in it
             return np.zeros(out_shape, dtype=dtype)
-        operands = [self._operand(arr, lbls) for arr, lbls in zip(arrays, self.in_lbls)]
+        operands = [self._operand(arr, lbls) for arr, lbls in zip(arrays, self._lbls)]
         ob = contract_all(operands, out_lbls, sizes, dtype)
         if any(ob is buf for buf, _ in operands):  # nothing was summed or moved: the result is a copy
             copy = _device.DeviceBuffer(max(_prod(out_shape) * dtype.itemsize, 16))
@@ -277,13 +287,14 @@ class EinSum(Operation):
     def backward_var(self, grad, index, **kwargs):
         """forward ``"ijk,k->ji", x, y``: the gradient of x is ``"ji,k->ijk", grad, y`` and that of
         y is ``"ji,ijk->k", grad, x`` (linalg/ops.py:124-218)."""
-        others = list(self.in_lbls)
-        var_lbl = others.pop(index)
         var = self.variables[index]
-        factor = self.cache[(id(var), var_lbl)]
+        pair = (id(var), self.in_lbls[index])
+        factor = self.cache[pair]
         if factor == 0:  # this (tensor, labels) pair has had its gradient, scaled by its count
             raise SkipGradient()
-        self.cache[(id(var), var_lbl)] = 0
+        self.cache[pair] = 0
+        others = list(self._lbls)  # labels with broadcast axes struck
+        var_lbl = others.pop(index)
         dtype, sizes = self._dtype, self._sizes
         if var.data.size == 0:
             return np.zeros(var.shape, dtype=dtype)
@@ -296,7 +307,7 @@ class EinSum(Operation):
         once = _last_of_each(var_lbl)  # the operand's labels with its diagonals taken (linalg/ops.py:147-163)
         found = "".join(lbl for lbl in once if lbl in elsewhere)
         operands = [(_device.to_device(np.ascontiguousarray(grad), dtype), self.out_lbls)]
-        operands += [self._operand(v.data, lbls) for n, (v, lbls) in enumerate(zip(self.variables, self.in_lbls)) if n != index]
+        operands += [self._operand(v.data, lbls) for n, (v, lbls) in enumerate(zip(self.variables, self._lbls)) if n != index]
         ob = contract_all(operands, found, sizes, dtype)
         if found != once:
             ob = _reduce.broadcast(ob, tuple(sizes[lbl] if lbl in elsewhere else 1 for lbl in once),

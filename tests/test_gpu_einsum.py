@@ -51,6 +51,9 @@ CASES = [
     # a label twice within an operand: traces and diagonals
     ("ii->", [(4, 4)]), ("ii->i", [(4, 4)]), ("iji->j", [(3, 2, 3)]), ("ijikik->jk", [(2, 3, 2, 4, 2, 4)]), ("ii,ij->j", [(3, 3), (3, 4)]),
     ("ijj,jk->ik", [(2, 3, 3), (3, 4)]), ("iij->", [(3, 3, 2)]), ("bii->b", [(70, 65, 65)]), ("ii,jj->ij", [(3, 3), (4, 4)]),
+    # an axis of length one broadcast against a longer one under the same label
+    ("ij,ij->ij", [(2, 3), (1, 3)]), ("bij,bjk->bik", [(1, 3, 4), (5, 4, 2)]), ("bij,bjk->bik", [(5, 3, 4), (1, 4, 2)]),
+    ("ai,ai->a", [(4, 1), (4, 6)]), ("ij,jk->ik", [(3, 1), (4, 5)]),
 ]
 
 
@@ -135,6 +138,6 @@ def test_errors_and_what_is_refused():
     with pytest.raises(ValueError):
         mg.einsum("ii->i", mg.Tensor(np.ones((3, 4))))  # the two axes of a diagonal differ in length
     with pytest.raises(NotImplementedError):
-        mg.einsum("ij,ij->ij", a, mg.Tensor(np.ones((1, 3))))  # a label of length one broadcast
+        mg.einsum("ii,ij->j", mg.Tensor(np.ones((1, 1))), mg.Tensor(np.ones((3, 2))))  # a diagonal that is broadcast as well
     with pytest.raises(TypeError):
         mg.einsum("ij,jk->ik", mg.Tensor(np.ones((2, 3), dtype=np.int64)), mg.Tensor(np.ones((3, 4), dtype=np.int64)))
