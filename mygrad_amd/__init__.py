@@ -18,7 +18,7 @@ from .errors import InvalidBackprop, InvalidGradient, SkipGradient
 from .nnet.layers.utils import sliding_window_copy, sliding_window_view
 from .operation_base import Operation
 from .tensor_base import Tensor, asarray, tensor
-from .math import matmul, multiply, sum  # noqa: A004  (after tensor_base: the ops import Tensor)
+from .math import matmul, multi_matmul, multiply, sum  # noqa: A004  (after tensor_base: the ops import Tensor)
 from .tensor_manip import repeat
 from .linalg import einsum
 from . import linalg
@@ -41,6 +41,7 @@ __all__ = [
     "einsum",
     "linalg",
     "matmul",
+    "multi_matmul",
     "sum",
     "repeat",
     "save",

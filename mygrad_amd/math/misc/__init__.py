@@ -1,3 +1,3 @@
-from .funcs import matmul
+from .funcs import matmul, multi_matmul
 
-__all__ = ["matmul"]
+__all__ = ["matmul", "multi_matmul"]

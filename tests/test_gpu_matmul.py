@@ -164,3 +164,42 @@ def test_dense_layer_chain_stays_on_the_device():
     assert err(w2.grad, ora.matmul_backward(g, want_h, w2.data, 1)) <= 1e-10
     assert err(w1.grad, ora.matmul_backward(dh, x.data, w1.data, 1)) <= 1e-10
     assert err(x.grad, ora.matmul_backward(dh, x.data, w1.data, 0)) <= 1e-10
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("shapes", [
+    [(10, 100), (100, 5), (5, 50)], [(3, 4), (4, 5), (5, 6), (6, 2)], [(4,), (4, 5), (5, 3)], [(3, 4), (4, 5), (5,)],
+    [(4,), (4, 6), (6, 5), (5,)], [(7, 2), (2, 9), (9, 1), (1, 8), (8, 3)], [(3, 4), (4, 5)],
+])
+def test_multi_matmul_and_its_gradients(shapes, dtype):
+    """Same bar as the single product; the expected values are NumPy's chained product and the
+    chain rule through the restated matmul gradients, in float64."""
+    import mygrad_amd as mg
+
+    dtype = np.dtype(dtype)
+    rng = np.random.default_rng([len(shapes), sum(int(np.prod(s)) for s in shapes)])
+    arrays = [rng.standard_normal(s).astype(dtype) for s in shapes]
+    tensors = [mg.Tensor(a) for a in arrays]
+    out = mg.multi_matmul(tensors)
+    wide = [a.astype(np.float64) for a in arrays]
+    want = wide[0]
+    for w in wide[1:]:
+        want = ora.matmul_forward(want, w)
+    assert out.shape == want.shape and out.dtype == dtype and err(out.data, want) <= TOL[dtype]
+    g = rng.standard_normal(want.shape).astype(dtype)
+    out.backward(g)
+    # d out / d A_i = (A_0 ... A_{i-1})^T g (A_{i+1} ... A_n)^T, by the chain rule from the left
+    for i, t in enumerate(tensors):
+        left = None
+        for w in wide[:i]:
+            left = w if left is None else ora.matmul_forward(left, w)
+        right = None
+        for w in wide[i + 1:]:
+            right = w if right is None else ora.matmul_forward(right, w)
+        grad = g.astype(np.float64)
+        chain = wide[i] if right is None else ora.matmul_forward(wide[i], right)
+        if left is not None:
+            grad = ora.matmul_backward(grad, left, chain, 1)  # through left @ (A_i right)
+        if right is not None:
+            grad = ora.matmul_backward(grad, wide[i], right, 0)  # through A_i @ right
+        assert t.grad.shape == t.shape and err(t.grad, grad) <= TOL[dtype]

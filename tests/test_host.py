@@ -437,3 +437,32 @@ def test_argument_checks_of_the_neighbouring_operations_need_no_device():
     assert np.array_equal(mg.sum(np.ones((0, 3)), axis=0).data, np.zeros(3))
     assert mg.sum(np.ones((0, 3)), axis=1, keepdims=True).shape == (0, 1)
     assert _graph.held_count() == 0
+
+
+def test_multi_matmul_picks_the_cheapest_order_and_checks_its_arguments():
+    from mygrad_amd.math.misc.funcs import _chain_split
+
+    def cheapest(dims, i, j):
+        if i == j:
+            return 0
+        return min(cheapest(dims, i, k) + cheapest(dims, k + 1, j) + dims[i] * dims[k + 1] * dims[j + 1] for k in range(i, j))
+
+    def cost_of(cut, dims, i, j):
+        if i == j:
+            return 0
+        k = cut[i][j]
+        return cost_of(cut, dims, i, k) + cost_of(cut, dims, k + 1, j) + dims[i] * dims[k + 1] * dims[j + 1]
+
+    # the textbook case: A 10x100, B 100x5, C 5x50 -> (A B) C at 7500 multiplications, not 75000
+    assert cost_of(_chain_split([10, 100, 5, 50]), [10, 100, 5, 50], 0, 2) == 7500
+    rng = np.random.default_rng(3)
+    for n in range(2, 8):
+        for _ in range(10):
+            dims = [int(v) for v in rng.integers(1, 30, n + 1)]
+            assert cost_of(_chain_split(dims), dims, 0, n - 1) == cheapest(dims, 0, n - 1)
+    with pytest.raises(ValueError):
+        mg.multi_matmul([np.ones((2, 2))])
+    with pytest.raises(ValueError):
+        mg.multi_matmul([np.ones((2, 2)), np.ones((2, 2, 2)), np.ones((2, 2))])
+    with pytest.raises(ValueError):
+        mg.multi_matmul([np.ones((2, 3)), np.ones(3), np.ones((3, 2))])  # a vector in the middle
