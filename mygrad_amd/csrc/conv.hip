@@ -80,6 +80,27 @@ struct Mma<double> {
 // Modes 2 and 3 pad every row with zeros to a multiple of four values (`ld` values per
 // row), so that the kernels can read a row sixteen bytes at a time whatever M is.
 // ------------------------------------------------------------------------------------------
+// One tap, forward, tap-major (mode 2 with wvol == 1 and ld == F): Ap[c][f] = w[f][c], a plain
+// transposition of an F x C matrix -- what a matrix product's left operand needs.  32 x 32
+// tiles through LDS: read along c, written along f, both coalesced.
+template <typename T>
+__global__ void __launch_bounds__(256) pack_transpose_kernel(const T *__restrict__ w, T *__restrict__ ap, int F, int C) {
+  __shared__ T tile[32][33];
+  const int c0 = blockIdx.x * 32, f0 = blockIdx.y * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int f = f0 + ty + 8 * j, c = c0 + tx;
+    if (f < F && c < C) tile[ty + 8 * j][tx] = w[(long long)f * C + c];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c = c0 + ty + 8 * j, f = f0 + tx;
+    if (f < F && c < C) ap[(long long)c * F + f] = tile[tx][ty + 8 * j];
+  }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256) pack_filters_kernel(const T *__restrict__ w, T *__restrict__ ap, int F, int C,
                                                            int wvol, int mode, int ld) {
@@ -1126,8 +1147,24 @@ int pack_filters(const Geometry &g, const void *w, int mode, void **packed, size
   const int ld = packed_ld(M, mode >= 2);
   const size_t count = (size_t)g.F * g.C * g.wvol / M * ld;
   const size_t packed_bytes = (count * sizeof(T) + 255) & ~size_t(255);
+  if (mode == 3 && g.wvol == 1 && ld == g.C && reinterpret_cast<uintptr_t>(w) % 16 == 0) {
+    // one tap, input gradient: the packed layout [f][c] is w's own, nothing to do
+    void *scratch = nullptr;
+    if (int rc = workspace(extra, &scratch)) return rc;
+    *packed = const_cast<void *>(w);
+    if (behind) *behind = scratch;
+    return MG_OK;
+  }
   if (int rc = workspace(packed_bytes + extra, packed)) return rc;
   if (behind) *behind = static_cast<char *>(*packed) + packed_bytes;
+  if (mode == 2 && g.wvol == 1 && ld == g.F) {
+    // one tap, forward: a transposition of the F x C matrix
+    ScopedTiming timed(TAG_PACK_FILTERS);
+    hipLaunchKernelGGL(pack_transpose_kernel<T>, dim3((unsigned)ceil_div(g.C, 32), (unsigned)ceil_div(g.F, 32)), dim3(256), 0,
+                       runtime().stream, static_cast<const T *>(w), static_cast<T *>(*packed), (int)g.F, (int)g.C);
+    MG_HIP(hipGetLastError());
+    return MG_OK;
+  }
   const unsigned blocks = (unsigned)std::min<long long>(ceil_div((long long)count, 256), 4096);
   ScopedTiming timed(TAG_PACK_FILTERS);
   hipLaunchKernelGGL(pack_filters_kernel<T>, dim3(blocks), dim3(256), 0, runtime().stream, static_cast<const T *>(w),
