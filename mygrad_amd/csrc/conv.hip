@@ -1334,6 +1334,67 @@ void release_conv_plans() {
 
 using namespace mg;
 
+// The fast (tap-major) kernels need the reduction -- K for the product and for da, M for dx --
+// and da's row count M to be multiples of 16.  A large product whose extents are not is run on
+// zero-padded copies of its operands (two bandwidth-bound passes over the operands against a
+// matrix product that runs more than twice as fast); small ones take the table-driven kernels.
+namespace {
+constexpr int64_t kMatmulUnit = 16;
+inline int64_t padded(int64_t n) { return (n + kMatmulUnit - 1) / kMatmulUnit * kMatmulUnit; }
+inline bool worth_padding(int64_t batch, int64_t M, int64_t K, int64_t N) {
+  return 2.0 * (double)batch * (double)M * (double)K * (double)N >= 2.0e8;
+}
+
+// dst:(batch, drows, dcols) takes src:(batch, srows, scols) where both have an element, zero elsewhere
+template <typename T>
+__global__ void __launch_bounds__(256) pad2d_kernel(const T *__restrict__ src, T *__restrict__ dst, long long total, int srows,
+                                                    int scols, int drows, int dcols) {
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const long long plane = (long long)drows * dcols;
+  const long long b = idx / plane;
+  const int rem = (int)(idx - b * plane);
+  const int r = rem / dcols, c = rem - r * dcols;
+  dst[idx] = (r < srows && c < scols) ? src[(b * srows + r) * scols + c] : T(0);
+}
+
+// src:(batch, srows, scols) re-laid as (batch, drows, dcols) into dst
+int relay_into(int dtype, const void *src, int64_t batch, int64_t srows, int64_t scols, int64_t drows, int64_t dcols, void *dst) {
+  void *where = dst;
+  void **block = &where;
+  const long long total = batch * drows * dcols;
+  if (srows >= (1ll << 31) || scols >= (1ll << 31) || drows * dcols >= (1ll << 31) || ceil_div(total, 256) >= (1ll << 31))
+    return fail(MG_ERR_UNSUPPORTED, "matrix product: an extent of 2^31 or more");
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  const dim3 grid((unsigned)ceil_div(total, 256)), blk(256);
+  ScopedTiming timed(TAG_COPY);
+  if (dtype == MG_F32)
+    hipLaunchKernelGGL(pad2d_kernel<float>, grid, blk, 0, runtime().stream, (const float *)src, (float *)*block, total, (int)srows,
+                       (int)scols, (int)drows, (int)dcols);
+  else
+    hipLaunchKernelGGL(pad2d_kernel<double>, grid, blk, 0, runtime().stream, (const double *)src, (double *)*block, total, (int)srows,
+                       (int)scols, (int)drows, (int)dcols);
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
+// a pooled block holding src:(batch, srows, scols) re-laid as (batch, drows, dcols)
+int relaid(int dtype, const void *src, int64_t batch, int64_t srows, int64_t scols, int64_t drows, int64_t dcols, void **block) {
+  if (int rc = mg_malloc(block, (size_t)(batch * drows * dcols) * (dtype == MG_F32 ? 4 : 8))) return rc;
+  return relay_into(dtype, src, batch, srows, scols, drows, dcols, *block);
+}
+
+// frees pooled blocks when the call that used them returns (the pool keeps them in stream order)
+struct Blocks {
+  void *held[4] = {nullptr, nullptr, nullptr, nullptr};
+  ~Blocks() {
+    for (void *p : held)
+      if (p) (void)mg_free(p);
+  }
+};
+}  // namespace
+
+
 extern "C" {
 
 int mg_conv_fwd(const mg_conv_desc *desc, const void *x, const void *w, void *out) {
@@ -1396,18 +1457,57 @@ int matmul_desc(const char *who, int dtype, int64_t batch, int64_t M, int64_t K,
 int mg_matmul(int dtype, int64_t batch, int64_t M, int64_t K, int64_t N, const void *a, const void *x, void *out) {
   mg_conv_desc d;
   if (int rc = matmul_desc("mg_matmul", dtype, batch, M, K, N, &d)) return rc;
+  if (K % kMatmulUnit != 0 && (dtype == MG_F32 || dtype == MG_F64) && a && x && out && worth_padding(batch, M, K, N)) {
+    const int64_t Kp = padded(K);
+    Blocks tmp;
+    if (int rc = relaid(dtype, a, 1, M, K, M, Kp, &tmp.held[0])) return rc;          // zero columns
+    if (int rc = relaid(dtype, x, batch, K, N, Kp, N, &tmp.held[1])) return rc;      // zero rows
+    if (int rc = matmul_desc("mg_matmul", dtype, batch, M, Kp, N, &d)) return rc;
+    return mg_conv_fwd(&d, tmp.held[1], tmp.held[0], out);
+  }
   return mg_conv_fwd(&d, x, a, out);
 }
 
 int mg_matmul_da(int dtype, int64_t batch, int64_t M, int64_t K, int64_t N, const void *grad, const void *x, void *da) {
   mg_conv_desc d;
   if (int rc = matmul_desc("mg_matmul_da", dtype, batch, M, K, N, &d)) return rc;
+  // da's rows are the filter-gradient kernel's tile rows, which must divide M: a large M is padded
+  // to whole 128-row (64-row) tiles rather than left to the 16- or 32-row ones
+  const int64_t row_unit = M >= 1024 ? 128 : (M >= 256 ? 64 : kMatmulUnit);
+  const int64_t Mp = (M + row_unit - 1) / row_unit * row_unit;
+  if ((K % kMatmulUnit != 0 || Mp != M) && (dtype == MG_F32 || dtype == MG_F64) && grad && x && da &&
+      worth_padding(batch, M, K, N)) {
+    const int64_t Kp = padded(K);
+    Blocks tmp;
+    const void *g2 = grad, *x2 = x;
+    if (Mp != M) {
+      if (int rc = relaid(dtype, grad, batch, M, N, Mp, N, &tmp.held[0])) return rc;
+      g2 = tmp.held[0];
+    }
+    if (Kp != K) {
+      if (int rc = relaid(dtype, x, batch, K, N, Kp, N, &tmp.held[1])) return rc;
+      x2 = tmp.held[1];
+    }
+    if (int rc = mg_malloc(&tmp.held[2], (size_t)Mp * Kp * (dtype == MG_F32 ? 4 : 8))) return rc;
+    if (int rc = matmul_desc("mg_matmul_da", dtype, batch, Mp, Kp, N, &d)) return rc;
+    if (int rc = mg_conv_wgrad(&d, g2, x2, tmp.held[2])) return rc;
+    // the rows and columns that belong to da
+    return relay_into(dtype, tmp.held[2], 1, Mp, Kp, M, K, da);
+  }
   return mg_conv_wgrad(&d, grad, x, da);
 }
 
 int mg_matmul_dx(int dtype, int64_t batch, int64_t M, int64_t K, int64_t N, const void *grad, const void *a, void *dx) {
   mg_conv_desc d;
   if (int rc = matmul_desc("mg_matmul_dx", dtype, batch, M, K, N, &d)) return rc;
+  if (M % kMatmulUnit != 0 && (dtype == MG_F32 || dtype == MG_F64) && grad && a && dx && worth_padding(batch, M, K, N)) {
+    const int64_t Mp = padded(M);
+    Blocks tmp;
+    if (int rc = relaid(dtype, a, 1, M, K, Mp, K, &tmp.held[0])) return rc;          // zero rows
+    if (int rc = relaid(dtype, grad, batch, M, N, Mp, N, &tmp.held[1])) return rc;   // zero rows
+    if (int rc = matmul_desc("mg_matmul_dx", dtype, batch, Mp, K, N, &d)) return rc;
+    return mg_conv_dgrad(&d, tmp.held[1], tmp.held[0], dx);
+  }
   return mg_conv_dgrad(&d, grad, a, dx);
 }
 

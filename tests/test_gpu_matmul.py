@@ -49,6 +49,11 @@ SIZES = [
     (1, 1024, 64, 16),
     (5, 16, 64, 1024),
     (1, 513, 257, 255),
+    # large enough, with a reduction or a row count that is no multiple of 16: zero-padded operands
+    (1, 520, 1000, 700),
+    (2, 300, 330, 1100),
+    (1, 512, 1000, 512),
+    (1, 1001, 512, 512),
 ]
 
 
