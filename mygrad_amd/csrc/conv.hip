@@ -1341,8 +1341,17 @@ using namespace mg;
 namespace {
 constexpr int64_t kMatmulUnit = 16;
 inline int64_t padded(int64_t n) { return (n + kMatmulUnit - 1) / kMatmulUnit * kMatmulUnit; }
+// MYGRAD_HIP_PAD=0 leaves every operand as it is (the table-driven kernels then take the
+// awkward extents): for comparisons
+inline bool padding_allowed() {
+  static const bool on = [] {
+    const char *flag = getenv("MYGRAD_HIP_PAD");
+    return !(flag && flag[0] == '0');
+  }();
+  return on;
+}
 inline bool worth_padding(int64_t batch, int64_t M, int64_t K, int64_t N) {
-  return 2.0 * (double)batch * (double)M * (double)K * (double)N >= 2.0e8;
+  return padding_allowed() && 2.0 * (double)batch * (double)M * (double)K * (double)N >= 2.0e8;
 }
 
 // dst:(batch, drows, dcols) takes src:(batch, srows, scols) where both have an element, zero elsewhere
@@ -1384,6 +1393,18 @@ int relaid(int dtype, const void *src, int64_t batch, int64_t srows, int64_t sco
   return relay_into(dtype, src, batch, srows, scols, drows, dcols, *block);
 }
 
+// Channel (or filter) count to zero-pad `channels` to so that the tap-major kernels apply, or 0
+// to leave it: already a multiple of 16, too small a problem to repay two extra passes over
+// the operands, or more than a third of padding.
+inline double conv_flops(const Geometry &g) {
+  return 2.0 * (double)g.N * (double)g.F * (double)g.gvol * (double)g.C * (double)g.wvol;
+}
+inline int64_t channels_to_pad_to(int64_t channels, double flops) {
+  if (channels % kMatmulUnit == 0 || flops < 2.0e8 || !padding_allowed()) return 0;
+  const int64_t up = padded(channels);
+  return 3 * up <= 4 * channels ? up : 0;
+}
+
 // frees pooled blocks when the call that used them returns (the pool keeps them in stream order)
 struct Blocks {
   void *held[4] = {nullptr, nullptr, nullptr, nullptr};
@@ -1403,6 +1424,15 @@ int mg_conv_fwd(const mg_conv_desc *desc, const void *x, const void *w, void *ou
   Geometry g;
   if (int rc = check_desc(desc, &g)) return rc;
   if (!x || !w || !out) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_conv_fwd");
+  if (const int64_t Cp = channels_to_pad_to(g.C, conv_flops(g))) {
+    // zero channels added to x and to the filters: the same sums, on the tap-major kernels
+    Blocks tmp;
+    if (int rc = relaid(g.dtype, x, g.N, g.C, g.xvol, Cp, g.xvol, &tmp.held[0])) return rc;
+    if (int rc = relaid(g.dtype, w, g.F, g.C, g.wvol, Cp, g.wvol, &tmp.held[1])) return rc;
+    mg_conv_desc wider = *desc;
+    wider.C = Cp;
+    return mg_conv_fwd(&wider, tmp.held[0], tmp.held[1], out);
+  }
   Plan *pl = nullptr;
   if (int rc = get_plan(OP_FWD, desc, g, &pl)) return rc;
   return g.dtype == MG_F32 ? conv_fwd_impl<float>(g, *pl, x, w, out) : conv_fwd_impl<double>(g, *pl, x, w, out);
@@ -1414,6 +1444,15 @@ int mg_conv_dgrad(const mg_conv_desc *desc, const void *grad, const void *w, voi
   Geometry g;
   if (int rc = check_desc(desc, &g)) return rc;
   if (!grad || !w || !dx) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_conv_dgrad");
+  if (const int64_t Fp = channels_to_pad_to(g.F, conv_flops(g))) {
+    // zero filters added to grad and to the filter bank
+    Blocks tmp;
+    if (int rc = relaid(g.dtype, grad, g.N, g.F, g.gvol, Fp, g.gvol, &tmp.held[0])) return rc;
+    if (int rc = relaid(g.dtype, w, 1, g.F, (int64_t)g.C * g.wvol, Fp, (int64_t)g.C * g.wvol, &tmp.held[1])) return rc;
+    mg_conv_desc wider = *desc;
+    wider.F = Fp;
+    return mg_conv_dgrad(&wider, tmp.held[0], tmp.held[1], dx);
+  }
   Plan *pl = nullptr;
   if (int rc = get_plan(OP_DGRAD, desc, g, &pl)) return rc;
   return g.dtype == MG_F32 ? conv_dgrad_impl<float>(g, *pl, grad, w, dx)
@@ -1426,6 +1465,29 @@ int mg_conv_wgrad(const mg_conv_desc *desc, const void *grad, const void *x, voi
   Geometry g;
   if (int rc = check_desc(desc, &g)) return rc;
   if (!grad || !x || !dw) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_conv_wgrad");
+  {
+    const int64_t Cp = channels_to_pad_to(g.C, conv_flops(g)), Fp = channels_to_pad_to(g.F, conv_flops(g));
+    if (Cp || Fp) {
+      // zero channels / filters added to x / grad; the rows and columns of dw that exist are kept
+      const int64_t C2 = Cp ? Cp : g.C, F2 = Fp ? Fp : g.F;
+      Blocks tmp;
+      const void *x2 = x, *g2 = grad;
+      if (Cp) {
+        if (int rc = relaid(g.dtype, x, g.N, g.C, g.xvol, Cp, g.xvol, &tmp.held[0])) return rc;
+        x2 = tmp.held[0];
+      }
+      if (Fp) {
+        if (int rc = relaid(g.dtype, grad, g.N, g.F, g.gvol, Fp, g.gvol, &tmp.held[1])) return rc;
+        g2 = tmp.held[1];
+      }
+      if (int rc = mg_malloc(&tmp.held[2], (size_t)(F2 * C2 * g.wvol) * (g.dtype == MG_F32 ? 4 : 8))) return rc;
+      mg_conv_desc wider = *desc;
+      wider.C = C2;
+      wider.F = F2;
+      if (int rc = mg_conv_wgrad(&wider, g2, x2, tmp.held[2])) return rc;
+      return relay_into(g.dtype, tmp.held[2], g.F, C2, g.wvol, g.C, g.wvol, dw);
+    }
+  }
   Plan *pl = nullptr;
   if (int rc = get_plan(OP_WGRAD, desc, g, &pl)) return rc;
   return g.dtype == MG_F32 ? conv_wgrad_impl<float>(g, *pl, grad, x, dw)

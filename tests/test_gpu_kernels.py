@@ -308,6 +308,32 @@ def test_conv_channel_counts_that_take_the_tap_major_kernels(abi, dtype, m):
 # multiple of four (padded packed rows), the 128x128 / 64x192 / 64x128 / 64x64 / 32x64 /
 # 16x64 filter-gradient tiles, and an odd number of positions per sample (grad tile
 # loaded element by element instead of 16 bytes per lane).
+PADDED_CHANNEL_CASES = [
+    # (x shape, w shape, stride, pad, dilation): large enough, channel / filter counts that are no
+    # multiple of 16 but within a third of one: run on zero-padded copies by the tap-major kernels
+    ((8, 24, 48, 48), (40, 24, 3, 3), (1, 1), (1, 1), (1, 1)),
+    ((6, 40, 40, 40), (32, 40, 3, 3), (2, 2), (1, 1), (1, 1)),
+    ((4, 32, 64, 64), (56, 32, 3, 3), (1, 1), (0, 0), (2, 2)),
+    ((16, 100, 400), (72, 100, 5), (1,), (2,), (1,)),
+    ((2, 24, 12, 20, 20), (24, 24, 3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("case", range(len(PADDED_CHANNEL_CASES)))
+def test_conv_awkward_channel_counts_on_padded_copies(abi, dtype, case):
+    x_shape, w_shape, s, p, d = PADDED_CHANNEL_CASES[case]
+    rng = np.random.default_rng(700 + case)
+    tol = TOL[np.dtype(dtype)]
+    x = rng.standard_normal(x_shape).astype(dtype)
+    w = (rng.standard_normal(w_shape) / np.sqrt(np.prod(w_shape[1:]))).astype(dtype)
+    want_out = direct.conv_forward(x, w, s, p, d)
+    g = rng.standard_normal(want_out.shape).astype(dtype)
+    assert rel_err(abi.conv_fwd(x, w, s, p, d), want_out) <= tol
+    assert rel_err(abi.conv_dgrad(g, x_shape, w, s, p, d), direct.conv_backward_x(g, x_shape, w, s, p, d)) <= tol
+    assert rel_err(abi.conv_wgrad(g, x, w_shape, s, p, d), direct.conv_backward_w(g, x, w_shape, s, p, d)) <= tol
+
+
 KERNEL_VARIANT_CASES = [
     # x shape, w shape, stride, padding, dilation
     ((8, 128, 28, 28), (128, 128, 3, 3), (1, 1), (1, 1), (1, 1)),   # 128-row tiles, wgrad 128x128
