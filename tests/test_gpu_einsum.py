@@ -141,3 +141,23 @@ def test_errors_and_what_is_refused():
         mg.einsum("ii,ij->j", mg.Tensor(np.ones((1, 1))), mg.Tensor(np.ones((3, 2))))  # a diagonal that is broadcast as well
     with pytest.raises(TypeError):
         mg.einsum("ij,jk->ik", mg.Tensor(np.ones((2, 3), dtype=np.int64)), mg.Tensor(np.ones((3, 4), dtype=np.int64)))
+
+
+def test_one_element_window_convolution_full_size():
+    """The benchmark's summation, 'nchw,fc->nfhw' on (32,256,56,56) x (256,256) with both
+    gradients, against BLAS products of the same operands in float64 (2e-4 bar)."""
+    import mygrad_amd as mg
+
+    rng = np.random.default_rng(95)
+    xv = rng.standard_normal((32, 256, 56, 56), dtype=np.float32)
+    wv = (rng.standard_normal((256, 256)) / 16).astype(np.float32)
+    x, w = mg.Tensor(xv), mg.Tensor(wv)
+    out = mg.einsum("nchw,fc->nfhw", x, w)
+    x64, w64 = xv.astype(np.float64), wv.astype(np.float64)
+    want = np.tensordot(w64, x64, axes=([1], [1])).transpose(1, 0, 2, 3)
+    assert err(out.data, want) <= 2e-4
+    g = rng.standard_normal(out.shape, dtype=np.float32)
+    out.backward(g)
+    g64 = g.astype(np.float64)
+    assert err(x.grad, np.tensordot(w64, g64, axes=([0], [1])).transpose(1, 0, 2, 3)) <= 2e-4
+    assert err(w.grad, np.tensordot(g64, x64, axes=([0, 2, 3], [0, 2, 3]))) <= 2e-4

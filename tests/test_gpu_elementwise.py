@@ -112,6 +112,19 @@ def test_sum_over_both_forms_against_exact_sums(abi, dtype, shape):
         assert np.array_equal(bits(abi.sum_over(x, over_middle)), bits(got))  # the same partition and trees every run
 
 
+def test_sum_over_full_size(abi):
+    """The benchmark's tensor (134 MB) summed per channel and over the channel axis, against
+    NumPy's sums of the same values in float64."""
+    rng = np.random.default_rng(94)
+    x = rng.standard_normal((8, 32, 32 * 64 * 64), dtype=np.float32)
+    wide = x.astype(np.float64)
+    for over_middle, axes in ((False, (0, 2)), (True, (1,))):
+        got = abi.sum_over(x, over_middle)
+        want = wide.sum(axis=axes)
+        scale = np.abs(wide).sum(axis=axes)
+        assert np.all(np.abs(got - want) <= SUM_TOL[np.dtype(np.float32)] * scale)
+
+
 def test_sum_over_closed_forms_and_bad_arguments(abi):
     from mygrad_amd import _device, _hip
 

@@ -266,3 +266,12 @@ def test_strided_copy_rejects_what_would_leave_the_buffer(abi):
     negative = (ctypes.c_int64 * 2)(5, -1)
     assert lib.mg_strided_copy(4, 2, shape, negative, 64, 0, buf.ptr, buf.ptr) == _hip.MG_ERR_BAD_ARG
     assert lib.mg_strided_copy(2, 2, shape, strides, 64, 0, buf.ptr, buf.ptr) == _hip.MG_ERR_UNSUPPORTED
+
+
+def test_permute_full_size_round_trip(abi):
+    """The benchmark's tensor (134 MB): channels last and back gives the input, bit for bit."""
+    rng = np.random.default_rng(93)
+    x = rng.standard_normal((8, 32, 32, 64, 64), dtype=np.float32)
+    there = abi.permute(x, (0, 2, 3, 4, 1))
+    assert np.array_equal(there[3, 5, 7, 11], x[3, :, 5, 7, 11])
+    assert np.array_equal(abi.permute(there, (0, 4, 1, 2, 3)), x)
