@@ -90,6 +90,12 @@ def conv_grid(wl):
     )
 
 
+def elem_bytes(x):
+    """Algorithmic bytes of sum(relu(x) * g) and its gradients: 15 passes over an array of x's
+    size and relu's mask, one bit per element, written once and read once."""
+    return 15.0 * x.nbytes + 2.0 * ((x.size + 7) // 8)
+
+
 def conv_flops_per_pass(wl, batch=None):
     n = wl["x"][0] if batch is None else batch
     return 2.0 * n * wl["w"][0] * np.prod(conv_grid(wl)) * wl["x"][1] * np.prod(wl["w"][2:])
@@ -269,9 +275,11 @@ class Step:
             self.x, self.g = resident(x), resident(g)
             self.out, self.dx = _device.DeviceBuffer(x.nbytes), _device.DeviceBuffer(x.nbytes)
             self.scalar = _device.DeviceBuffer(16)
-            # relu fwd 2|x|, relu bwd 3|x|, multiply fwd and two gradients 3|x| each, fill |x|: 6 launches
-            self.work = {"elementwise": 15.0 * x.nbytes / 6, "sum_all": float(x.nbytes)}
-            self.total_work = 16.0 * x.nbytes
+            self.mask = _device.DeviceBuffer((x.size + 7) // 8)
+            # relu fwd and bwd 2|x| + the mask (one bit per element) each, multiply fwd and two
+            # gradients 3|x| each, fill |x|: 6 launches
+            self.work = {"elementwise": (elem_bytes(x) - x.nbytes) / 6, "sum_all": float(x.nbytes)}
+            self.total_work = elem_bytes(x)
             self.unit, self.bound, self.peak = "GB/s", "hbm", PEAK_HBM_GBS
             self.scale = 1e-9
         else:
@@ -295,13 +303,13 @@ class Step:
         lib, check = self.lib, self.check
         if self.wl["kind"] == "elem":
             c, n = self.code, self.n
-            check(lib.mg_relu_fwd(c, n, self.x.ptr, self.out.ptr))
+            check(lib.mg_relu_fwd_mask(c, n, self.x.ptr, self.out.ptr, self.mask.ptr))
             check(lib.mg_multiply(c, n, self.out.ptr, self.g.ptr, self.dx.ptr))  # relu(x) * g
             check(lib.mg_sum_all(c, n, self.dx.ptr, self.scalar.ptr))
             check(lib.mg_fill_from(c, n, self.scalar.ptr, self.dx.ptr))  # d sum
             check(lib.mg_multiply(c, n, self.dx.ptr, self.g.ptr, self.out.ptr))  # d (a*b) / d a
             check(lib.mg_multiply(c, n, self.dx.ptr, self.x.ptr, self.out.ptr))  # d (a*b) / d b
-            check(lib.mg_relu_bwd(c, n, self.x.ptr, self.dx.ptr, self.out.ptr))
+            check(lib.mg_relu_bwd_mask(c, n, self.mask.ptr, self.dx.ptr, self.out.ptr))
             return
         if self.wl["kind"] == "matmul":
             check(lib.mg_matmul(self.code, *self.dims, self.w.ptr, self.x.ptr, self.out.ptr))
@@ -545,7 +553,7 @@ def run_cpu_baseline(name, min_seconds=10.0, max_reps=200):
             dr = ora.multiply_backward(dp, r, g, 1)
             ora.relu_backward(x, dr)
 
-        work, scale, unit = 16 * x.nbytes, 1e-9, "GB/s"
+        work, scale, unit = elem_bytes(x), 1e-9, "GB/s"
         what = "relu, multiply, sum and their gradients"
     else:
         x = rng.standard_normal(wl["x"]).astype(dt)
@@ -667,7 +675,7 @@ def run_dropin(name, steps=5):
             xt, gt = mg.Tensor(x, copy=False), mg.Tensor(g, copy=False)
             mg.sum(relu(xt) * gt).backward()
 
-        work, scale, unit = 16 * x.nbytes, 1e-9, "GB/s"
+        work, scale, unit = elem_bytes(x), 1e-9, "GB/s"
     else:
         lead, pooled, grid = pool_shapes(wl)
         g = rng.standard_normal((*lead, *grid)).astype(dt)

@@ -206,6 +206,14 @@ int mg_relu_fwd(int dtype, int64_t n, const void *x, void *out);
  * reference stores in self.back is recomputed from x). */
 int mg_relu_bwd(int dtype, int64_t n, const void *x, const void *grad, void *dx);
 
+/* The same pair with the mask kept between the passes, as the reference keeps it
+ * (self.back, src/mygrad/nnet/activations/relu.py:11-17): the forward pass also writes one bit
+ * per element, bit i % 8 of mask[i / 8] = (x[i] > 0), (n + 7) / 8 bytes; the backward pass
+ * multiplies grad by those bits and does not read x (so it uses the x of the forward pass
+ * even if x has changed since, like the reference). */
+int mg_relu_fwd_mask(int dtype, int64_t n, const void *x, void *out, void *mask);
+int mg_relu_bwd_mask(int dtype, int64_t n, const void *mask, const void *grad, void *dx);
+
 /* *out (one element on the device) = sum of x, added in a fixed tree and carried in double,
  * rounded once.  Replaces Sum.__call__ with axis=None (np.sum,
  * src/mygrad/math/sequential/ops.py:120-121; src/mygrad/operation_base.py Sequential). */

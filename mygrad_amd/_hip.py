@@ -147,6 +147,8 @@ _SIGNATURES = {
     "mg_multiply": [ctypes.c_int, ctypes.c_int64, _vp, _vp, _vp],
     "mg_relu_fwd": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
     "mg_relu_bwd": [ctypes.c_int, ctypes.c_int64, _vp, _vp, _vp],
+    "mg_relu_fwd_mask": [ctypes.c_int, ctypes.c_int64, _vp, _vp, _vp],
+    "mg_relu_bwd_mask": [ctypes.c_int, ctypes.c_int64, _vp, _vp, _vp],
     "mg_sum_all": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
     "mg_fill_from": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
     "mg_sum_over": [ctypes.c_int] + [ctypes.c_int64] * 3 + [ctypes.c_int, _vp, _vp],

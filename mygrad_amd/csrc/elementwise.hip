@@ -164,6 +164,74 @@ int launch_elementwise(int dtype, int64_t n, const void *a, const void *b, void 
 
 bool misaligned(const void *p) { return reinterpret_cast<uintptr_t>(p) % 16 != 0; }
 
+// relu with its mask kept as one bit per element: bit i % 8 of mask[i / 8] is x[i] > 0.  A
+// thread takes eight consecutive elements (two or four 16-byte pieces) and one byte of the mask.
+//   forward:  out[i] = x[i] * (x[i] > 0), and the mask
+//   backward: dx[i]  = grad[i] * (bit i)          -- x is not read
+template <typename T, bool BACKWARD>
+__global__ void __launch_bounds__(256) relu_mask_kernel(const T *__restrict__ in, T *__restrict__ out, unsigned char *__restrict__ mask,
+                                                        long long n) {
+  typedef typename Vec16<T>::type V;
+  constexpr int VEC = Vec16<T>::N, PIECES = 8 / VEC;
+  const long long groups = (n + 7) / 8;
+  for (long long grp = (long long)blockIdx.x * 256 + threadIdx.x; grp < groups; grp += (long long)gridDim.x * 256) {
+    const long long first = grp * 8;
+    unsigned bits = BACKWARD ? (unsigned)mask[grp] : 0u;
+    if (first + 8 <= n) {
+      const V *vi = reinterpret_cast<const V *>(in + first);
+      V *vo = reinterpret_cast<V *>(out + first);
+      V v[PIECES];
+#pragma unroll
+      for (int q = 0; q < PIECES; ++q) v[q] = vi[q];
+#pragma unroll
+      for (int q = 0; q < PIECES; ++q) {
+        V r;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+          const int bit = q * VEC + k;
+          if constexpr (BACKWARD) {
+            r[k] = v[q][k] * (((bits >> bit) & 1u) ? T(1) : T(0));
+          } else {
+            const bool positive = v[q][k] > T(0);
+            bits |= (positive ? 1u : 0u) << bit;
+            r[k] = v[q][k] * (positive ? T(1) : T(0));
+          }
+        }
+        vo[q] = r;
+      }
+    } else {  // the array's last, partial group
+      for (int bit = 0; first + bit < n; ++bit) {
+        const T value = in[first + bit];
+        if constexpr (BACKWARD) {
+          out[first + bit] = value * (((bits >> bit) & 1u) ? T(1) : T(0));
+        } else {
+          const bool positive = value > T(0);
+          bits |= (positive ? 1u : 0u) << bit;
+          out[first + bit] = value * (positive ? T(1) : T(0));
+        }
+      }
+    }
+    if constexpr (!BACKWARD) mask[grp] = (unsigned char)bits;
+  }
+}
+
+template <bool BACKWARD>
+int launch_relu_mask(int dtype, int64_t n, const void *in, void *out, void *mask) {
+  if (n == 0) return MG_OK;
+  hipStream_t s = runtime().stream;
+  const long long groups = ((long long)n + 7) / 8;
+  const unsigned grid = (unsigned)std::min<long long>(ceil_div(groups, 256), (long long)runtime().props.multiProcessorCount * 16);
+  ScopedTiming timed(TAG_ELEMENTWISE);
+  if (dtype == MG_F32)
+    hipLaunchKernelGGL((relu_mask_kernel<float, BACKWARD>), dim3(grid), dim3(256), 0, s, (const float *)in, (float *)out,
+                       (unsigned char *)mask, (long long)n);
+  else
+    hipLaunchKernelGGL((relu_mask_kernel<double, BACKWARD>), dim3(grid), dim3(256), 0, s, (const double *)in, (double *)out,
+                       (unsigned char *)mask, (long long)n);
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
 }  // namespace
 }  // namespace mg
 
@@ -196,6 +264,24 @@ int mg_relu_bwd(int dtype, int64_t n, const void *x, const void *grad, void *dx)
   if (n > 0 && (!x || !grad || !dx)) return fail(MG_ERR_BAD_ARG, "null pointer in mg_relu_bwd");
   if (misaligned(x) || misaligned(grad) || misaligned(dx)) return fail(MG_ERR_BAD_ARG, "mg_relu_bwd: pointers must be 16-byte aligned");
   return launch_elementwise<EW_RELU_BWD>(dtype, n, x, grad, dx, TAG_ELEMENTWISE);
+}
+
+int mg_relu_fwd_mask(int dtype, int64_t n, const void *x, void *out, void *mask) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (int rc = check_elementwise(dtype, n, "mg_relu_fwd_mask")) return rc;
+  if (n > 0 && (!x || !out || !mask)) return fail(MG_ERR_BAD_ARG, "null pointer in mg_relu_fwd_mask");
+  if (misaligned(x) || misaligned(out)) return fail(MG_ERR_BAD_ARG, "mg_relu_fwd_mask: x and out must be 16-byte aligned");
+  return launch_relu_mask<false>(dtype, n, x, out, mask);
+}
+
+int mg_relu_bwd_mask(int dtype, int64_t n, const void *mask, const void *grad, void *dx) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (int rc = check_elementwise(dtype, n, "mg_relu_bwd_mask")) return rc;
+  if (n > 0 && (!mask || !grad || !dx)) return fail(MG_ERR_BAD_ARG, "null pointer in mg_relu_bwd_mask");
+  if (misaligned(grad) || misaligned(dx)) return fail(MG_ERR_BAD_ARG, "mg_relu_bwd_mask: grad and dx must be 16-byte aligned");
+  return launch_relu_mask<true>(dtype, n, grad, dx, const_cast<void *>(mask));
 }
 
 int mg_sum_all(int dtype, int64_t n, const void *x, void *out) {

@@ -2,7 +2,8 @@
 
 ``f(x) = x * (x > 0)`` computed, like the reference, as a multiplication by a 0/1 mask:
 negative inputs give ``-0.0`` and NaN stays NaN.  The mask the reference keeps in
-``self.back`` is recomputed from ``x`` in the backward kernel."""
+``self.back`` is kept here as well, on the device, as one bit per element: the backward
+kernel reads the gradient and the bits, not ``x``."""
 
 import numpy as np
 
@@ -23,7 +24,8 @@ class ReLu(Operation):
             return np.empty(x.shape, dtype=x.dtype)
         xb = _device.to_device(x)
         ob = _device.DeviceBuffer(max(x.nbytes, 16))
-        _hip.check(_hip.lib().mg_relu_fwd(_hip.dtype_code(x.dtype), x.size, xb.ptr, ob.ptr))
+        self._mask = _device.DeviceBuffer(max((x.size + 7) // 8, 16))  # the reference's self.back, packed
+        _hip.check(_hip.lib().mg_relu_fwd_mask(_hip.dtype_code(x.dtype), x.size, xb.ptr, ob.ptr, self._mask.ptr))
         out = _device.download(ob, x.shape, x.dtype)
         _device.attach(out, ob)
         return out
@@ -34,10 +36,9 @@ class ReLu(Operation):
             return np.empty(x.shape, dtype=x.dtype)
         if grad.shape != x.shape:
             raise NotImplementedError(f"relu backward for gradient of shape {grad.shape} (no CPU fallback)")
-        xb = _device.to_device(x)
         gb = _device.to_device(grad, x.dtype)
         ob = _device.DeviceBuffer(max(x.nbytes, 16))
-        _hip.check(_hip.lib().mg_relu_bwd(_hip.dtype_code(x.dtype), x.size, xb.ptr, gb.ptr, ob.ptr))
+        _hip.check(_hip.lib().mg_relu_bwd_mask(_hip.dtype_code(x.dtype), x.size, self._mask.ptr, gb.ptr, ob.ptr))
         out = _device.download(ob, x.shape, x.dtype)
         _device.attach_transient(out, ob)
         return out

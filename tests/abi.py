@@ -136,6 +136,23 @@ def relu_bwd(x, grad):
     return _down(ob, x.shape, x.dtype)
 
 
+def relu_fwd_mask(x):
+    """(out, mask): mask holds one bit per element of x, bit i % 8 of byte i // 8."""
+    xb = _up(x)
+    ob = _device.DeviceBuffer(max(x.nbytes, 16))
+    nbytes = (x.size + 7) // 8
+    mb = _device.DeviceBuffer(max(nbytes, 16))
+    _hip.check(_hip.lib().mg_relu_fwd_mask(_hip.dtype_code(x.dtype), x.size, xb.ptr, ob.ptr, mb.ptr))
+    return _down(ob, x.shape, x.dtype), _down(mb, (nbytes,), np.uint8)
+
+
+def relu_bwd_mask(mask, grad):
+    mb, gb = _up(mask), _up(grad)
+    ob = _device.DeviceBuffer(max(grad.nbytes, 16))
+    _hip.check(_hip.lib().mg_relu_bwd_mask(_hip.dtype_code(grad.dtype), grad.size, mb.ptr, gb.ptr, ob.ptr))
+    return _down(ob, grad.shape, grad.dtype)
+
+
 def permute(x, perm):
     import ctypes
 
