@@ -24,6 +24,7 @@ taps count, dense definition); pooling |x|+|out| bytes forward and
 """
 
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -67,6 +68,7 @@ WORKLOADS = {
     "mm4k": dict(kind="matmul", dtype="f32", seed=1011, M=4096, K=4096, N=4096),
     # sums over axes of a tensor of conv5's output size: per channel (the gradient of a bias or of a
     # per-channel scale: every axis but axis 1), then over the channel axis alone
+    "scale5": dict(kind="scale", dtype="f32", seed=1015, x=(8, 32, 32, 64, 64), others=((32, 1, 1, 1), (64,))),
     "sum5": dict(kind="sumover", dtype="f32", seed=1012, x=(8, 32, 32, 64, 64), axes=((0, 2, 3, 4), (1,))),
     # transposition of a tensor of conv5's output size: channels last (N,C,D,H,W -> N,D,H,W,C) and back
     "perm5": dict(kind="permute", dtype="f32", seed=1013, x=(8, 32, 32, 64, 64), perms=((0, 2, 3, 4, 1), (0, 4, 1, 2, 3))),
@@ -119,6 +121,8 @@ def describe(name):
     if wl["kind"] == "einsum":
         a, b, o = wl["subscripts"]
         return f"{name}: einsum '{a},{b}->{o}' {wl['dtype']} x{wl['x']} w{wl['w']} and both gradients"
+    if wl["kind"] == "scale":
+        return f"{name}: multiply {wl['dtype']} x{wl['x']} by an operand of shape {wl['others'][0]}, then by one of shape {wl['others'][1]}"
     if wl["kind"] == "sumover":
         return f"{name}: sum {wl['dtype']} x{wl['x']} over axes {wl['axes'][0]}, then over axes {wl['axes'][1]}"
     if wl["kind"] == "repeat":
@@ -184,8 +188,6 @@ class Step:
             self.unit, self.bound, self.peak = "TFLOP/s", "mfma", PEAK_TFLOPS[wl["dtype"]]
             self.scale = 1e-12
         elif wl["kind"] == "permute":
-            import ctypes
-
             x = rng.standard_normal(wl["x"]).astype(dt)
             self.x, self.out, self.back = resident(x), _device.DeviceBuffer(x.nbytes), _device.DeviceBuffer(x.nbytes)
             nd = x.ndim
@@ -219,6 +221,22 @@ class Step:
             # each launch reads x once; what it writes is 1/32 of that at most
             self.work = {"sum_over": float(x.nbytes)}
             self.total_work = 2.0 * x.nbytes
+            self.unit, self.bound, self.peak = "GB/s", "hbm", PEAK_HBM_GBS
+            self.scale = 1e-9
+        elif wl["kind"] == "scale":
+            from mygrad_amd import _reduce
+
+            x = rng.standard_normal(wl["x"]).astype(dt)
+            self.x, self.out, self.code = resident(x), _device.DeviceBuffer(x.nbytes), _hip.dtype_code(dt)
+            self.others = []
+            for shape in wl["others"]:
+                extents, sa, sb = _reduce.multiply_plan(wl["x"], shape, wl["x"])
+                as_array = ctypes.c_int64 * len(extents)
+                self.others.append((len(extents), as_array(*extents), as_array(*sa), as_array(*sb),
+                                    resident(rng.standard_normal(shape).astype(dt))))
+            # each launch reads x and writes the product; the other operand is 1/1000 of that at most
+            self.work = {"elementwise": 2.0 * x.nbytes}
+            self.total_work = 4.0 * x.nbytes
             self.unit, self.bound, self.peak = "GB/s", "hbm", PEAK_HBM_GBS
             self.scale = 1e-9
         elif wl["kind"] == "repeat":
@@ -332,6 +350,10 @@ class Step:
         if self.wl["kind"] == "sumover":
             check(lib.mg_sum_over(self.code, *self.dims, 0, self.x.ptr, self.out.ptr))
             check(lib.mg_sum_over(self.code, *self.dims, 1, self.x.ptr, self.out.ptr))
+            return
+        if self.wl["kind"] == "scale":
+            for nd, extents, sa, sb, other in self.others:
+                check(lib.mg_multiply_broadcast(self.code, nd, extents, sa, sb, self.x.ptr, other.ptr, self.out.ptr))
             return
         if self.wl["kind"] == "repeat":
             for outer, n, inner, r, total in self.geometry:
@@ -508,6 +530,16 @@ def run_cpu_baseline(name, min_seconds=10.0, max_reps=200):
 
         work, scale, unit = 2 * x.nbytes, 1e-9, "GB/s"
         what = "np.sum over each of the two sets of axes"
+    elif wl["kind"] == "scale":
+        x = rng.standard_normal(wl["x"]).astype(dt)
+        others = [rng.standard_normal(shape).astype(dt) for shape in wl["others"]]
+
+        def once():
+            for other in others:
+                ora.multiply(x, other)
+
+        work, scale, unit = 4 * x.nbytes, 1e-9, "GB/s"
+        what = "np.multiply by a per-channel scale and by a row"
     elif wl["kind"] == "repeat":
         x = rng.standard_normal(wl["x"]).astype(dt)
         g = rng.standard_normal((*wl["x"][:-1], wl["x"][-1] * wl["repeats"])).astype(dt)
@@ -637,6 +669,14 @@ def run_dropin(name, steps=5):
                 mg.sum(mg.Tensor(x, copy=False), axis=axes).clear_graph()
 
         work, scale, unit = 2 * x.nbytes, 1e-9, "GB/s"
+    elif wl["kind"] == "scale":
+        others = [rng.standard_normal(shape).astype(dt) for shape in wl["others"]]
+
+        def once():
+            for other in others:
+                (mg.Tensor(x, copy=False) * mg.Tensor(other, copy=False)).clear_graph()
+
+        work, scale, unit = 4 * x.nbytes, 1e-9, "GB/s"
     elif wl["kind"] == "repeat":
         g = rng.standard_normal((*wl["x"][:-1], wl["x"][-1] * wl["repeats"])).astype(dt)
 
@@ -768,7 +808,7 @@ def main():
         "metric": {"conv": "conv_nd fwd+bwd TFLOP/s", "pool": "max_pool fwd+bwd GB/s",
                    "elem": "relu+multiply+sum fwd+bwd GB/s", "bn": "batchnorm fwd+bwd GB/s",
                    "repeat": "repeat fwd+bwd GB/s", "matmul": "matmul fwd+bwd TFLOP/s", "window": "sliding-window copy GB/s",
-                   "sumover": "sum over axes GB/s", "permute": "transposition GB/s", "einsum": "einsum fwd+bwd TFLOP/s"}[wl["kind"]],
+                   "sumover": "sum over axes GB/s", "scale": "broadcasting multiply GB/s", "permute": "transposition GB/s", "einsum": "einsum fwd+bwd TFLOP/s"}[wl["kind"]],
         "value": res["value"],
         "unit": res["unit"],
         "n_gpus": 1,

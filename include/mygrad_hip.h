@@ -198,6 +198,15 @@ int mg_maxpool_bwd_argmax(const mg_pool_desc *desc, const void *argmax, const vo
  * Multiply.backward_var (grad * other, ops.py:48-53). */
 int mg_multiply(int dtype, int64_t n, const void *a, const void *b, void *out);
 
+/* out = a * b with NumPy's broadcasting (np.multiply in Multiply.__call__, ops.py:45-46, and
+ * grad * other in backward_var, ops.py:48-53, before reduce_broadcast sums it back).  `out` is
+ * C-contiguous of `shape` (nd axes, 1 to 6: merge neighbouring axes that both operands treat
+ * alike first; fewer than 2^31 elements); a_strides / b_strides are the operands' strides in
+ * elements along those axes, 0 along an axis the operand is broadcast on, and 1 or 0 along the
+ * last axis.  One pass: an operand is read where it lies, never spread out in memory. */
+int mg_multiply_broadcast(int dtype, int nd, const int64_t *shape, const int64_t *a_strides, const int64_t *b_strides, const void *a,
+                          const void *b, void *out);
+
 /* out[i] = x[i] * (x[i] > 0) as one IEEE multiply by 1 or 0: negative x gives -0.0, NaN
  * stays NaN.  Replaces ReLu.__call__, src/mygrad/nnet/activations/relu.py:11-14. */
 int mg_relu_fwd(int dtype, int64_t n, const void *x, void *out);

@@ -145,6 +145,8 @@ _SIGNATURES = {
     "mg_maxpool_fwd_argmax": [ctypes.POINTER(PoolDesc), _vp, _vp, _vp],
     "mg_maxpool_bwd_argmax": [ctypes.POINTER(PoolDesc), _vp, _vp, _vp],
     "mg_multiply": [ctypes.c_int, ctypes.c_int64, _vp, _vp, _vp],
+    "mg_multiply_broadcast": [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64),
+                              ctypes.POINTER(ctypes.c_int64), _vp, _vp, _vp],
     "mg_relu_fwd": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
     "mg_relu_bwd": [ctypes.c_int, ctypes.c_int64, _vp, _vp, _vp],
     "mg_relu_fwd_mask": [ctypes.c_int, ctypes.c_int64, _vp, _vp, _vp],

@@ -4,13 +4,19 @@ middle axis or over the outer and inner ones) and ``mg_repeat_fwd`` (an axis of 
 repeated).  Neighbouring axes that are treated alike are merged first, so the usual
 cases -- a bias gradient, a per-channel scale, a reduction over the last axes -- take one
 launch; anything else takes one launch per remaining group of axes.
+
+A product of two operands that broadcast against each other needs neither: ``multiply_plan``
+gives the merged axes and the strides with which ``mg_multiply_broadcast`` reads each operand
+where it lies.
 """
+
+import ctypes
 
 import numpy as np
 
 from . import _device, _hip
 
-__all__ = ["sum_axes", "broadcast", "permute"]
+__all__ = ["sum_axes", "broadcast", "permute", "multiply_plan", "multiply_broadcast"]
 
 
 def _merge(pairs):
@@ -89,8 +95,6 @@ def broadcast(buf, shape, to_shape, dtype):
 def permute(buf, shape, perm, dtype):
     """Device buffer with ``x.transpose(perm)`` made contiguous, for the C-contiguous ``x`` of
     ``shape`` in ``buf`` (not empty).  The same buffer comes back when nothing moves."""
-    import ctypes
-
     perm = tuple(int(p) for p in perm)
     moving = [p for p in perm if shape[p] != 1]
     if moving == sorted(moving):
@@ -98,4 +102,48 @@ def permute(buf, shape, perm, dtype):
     nd = len(shape)
     out = _device.DeviceBuffer(max(int(np.prod(shape, dtype=np.int64)) * dtype.itemsize, 16))
     _hip.check(_hip.lib().mg_permute(dtype.itemsize, nd, (ctypes.c_int64 * nd)(*shape), (ctypes.c_int32 * nd)(*perm), buf.ptr, out.ptr))
+    return out
+
+
+def multiply_plan(a_shape, b_shape, shape):
+    """``(extents, a_strides, b_strides)`` of ``a * b`` broadcast to ``shape``: neighbouring
+    axes that both operands treat alike -- each is either there or broadcast -- are merged, axes
+    of length one are dropped, strides are in elements of the C-contiguous operands and 0 where
+    an operand is broadcast.  At least one axis comes back (``shape`` has no empty axis)."""
+    nd = len(shape)
+    a_shape = (1,) * (nd - len(a_shape)) + tuple(a_shape)
+    b_shape = (1,) * (nd - len(b_shape)) + tuple(b_shape)
+    groups = _merge([(size, (a_shape[i] == size, b_shape[i] == size)) for i, size in enumerate(shape)])
+    if not groups:
+        return [1], [0], [0]
+    extents = [size for size, _ in groups]
+    strides = ([], [])
+    for which in (0, 1):
+        step = 1
+        for size, there in reversed(groups):
+            strides[which].insert(0, step if there[which] else 0)
+            if there[which]:
+                step *= size
+    return extents, strides[0], strides[1]
+
+
+MAX_MULTIPLY_AXES = 6  # of mg_multiply_broadcast, after merging
+
+
+def multiply_broadcast(a_buf, a_shape, b_buf, b_shape, shape, dtype):
+    """Device buffer with ``a * b`` of ``shape``, for C-contiguous operands that broadcast to
+    it, in one pass; ``None`` when the pattern has more axes than the kernel takes or the
+    result 2^31 elements or more (the caller then spreads the operands first)."""
+    extents, a_strides, b_strides = multiply_plan(a_shape, b_shape, shape)
+    size = int(np.prod(shape, dtype=np.int64))
+    if len(extents) > MAX_MULTIPLY_AXES or size >= 2**31:
+        return None
+    nd = len(extents)
+    out = _device.DeviceBuffer(max(size * dtype.itemsize, 16))
+    as_array = ctypes.c_int64 * nd
+    _hip.check(
+        _hip.lib().mg_multiply_broadcast(
+            _hip.dtype_code(dtype), nd, as_array(*extents), as_array(*a_strides), as_array(*b_strides), a_buf.ptr, b_buf.ptr, out.ptr
+        )
+    )
     return out

@@ -2,6 +2,7 @@
 // such as conv -> relu -> pool -> (. * g) -> sum: bandwidth-bound, 16 bytes per lane.
 //
 //   multiply   out[i] = a[i] * b[i]            (one IEEE multiply: bit-exact with NumPy)
+//              also with operands that are broadcast along some of the axes
 //   relu       out[i] = x[i] * (x[i] > 0)      (so negative inputs give -0.0, NaN stays NaN)
 //   relu bwd   dx[i]  = grad[i] * (x[i] > 0)
 //   sum        *out   = sum_i x[i]             (fixed summation tree, carried in double)
@@ -54,6 +55,65 @@ __global__ void __launch_bounds__(256) elementwise_kernel(const T *__restrict__ 
   if (blockIdx.x == 0) {
     const long long i = nvec * VEC + threadIdx.x;
     if (i < n) out[i] = apply<T, OP>(a[i], OP != EW_RELU ? b[i] : a[i]);
+  }
+}
+
+// out = a * b where each operand lacks some of the axes of `out` (NumPy's broadcasting).  The
+// host merges neighbouring axes that both operands treat alike, so `out` is (d[0], ..., d[nd-1])
+// with the last axis `inner` long; an operand's stride along an axis is 0 where it is
+// broadcast, and along the last axis 1 or 0.  A thread makes VEC consecutive results of one
+// row: an operand present along the last axis is read 16 bytes at a time, a broadcast one once.
+struct BroadcastParams {
+  int outer_dims;         // axes before the last one (at most 5)
+  unsigned extent[5];     // their lengths, first axis first
+  unsigned a_step[5], b_step[5];  // element strides of a and b along them
+  unsigned a_inner, b_inner;      // 1 or 0: strides along the last axis
+  unsigned inner, pieces;         // length of the last axis, ceil(inner / VEC)
+  unsigned threads;               // rows x pieces
+};
+
+template <typename T, bool ALIGNED>
+__global__ void __launch_bounds__(256) multiply_broadcast_kernel(const T *__restrict__ a, const T *__restrict__ b, T *__restrict__ out,
+                                                                 BroadcastParams p) {
+  typedef typename Vec16<T>::type V;
+  constexpr int VEC = Vec16<T>::N;
+  for (unsigned t = blockIdx.x * 256u + threadIdx.x; t < p.threads; t += gridDim.x * 256u) {
+    const unsigned piece = t % p.pieces;
+    unsigned row = t / p.pieces;
+    const size_t at = (size_t)row * p.inner + (size_t)piece * VEC;  // in `out`
+    unsigned ia = 0, ib = 0;
+    for (int d = p.outer_dims - 1; d >= 0; --d) {
+      const unsigned c = row % p.extent[d];
+      row /= p.extent[d];
+      ia += c * p.a_step[d];
+      ib += c * p.b_step[d];
+    }
+    if constexpr (ALIGNED) {  // inner is a multiple of VEC: every piece is whole and 16-byte aligned in all three
+      V x, y, r;
+      if (p.a_inner) {
+        x = *reinterpret_cast<const V *>(a + ia + piece * VEC);
+      } else {
+        const T v = a[ia];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) x[k] = v;
+      }
+      if (p.b_inner) {
+        y = *reinterpret_cast<const V *>(b + ib + piece * VEC);
+      } else {
+        const T v = b[ib];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) y[k] = v;
+      }
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) r[k] = x[k] * y[k];
+      *reinterpret_cast<V *>(out + at) = r;
+    } else {
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) {
+        const unsigned col = piece * VEC + k;
+        if (col < p.inner) out[at + k] = a[ia + col * p.a_inner] * b[ib + col * p.b_inner];
+      }
+    }
   }
 }
 
@@ -282,6 +342,60 @@ int mg_relu_bwd_mask(int dtype, int64_t n, const void *mask, const void *grad, v
   if (n > 0 && (!mask || !grad || !dx)) return fail(MG_ERR_BAD_ARG, "null pointer in mg_relu_bwd_mask");
   if (misaligned(grad) || misaligned(dx)) return fail(MG_ERR_BAD_ARG, "mg_relu_bwd_mask: grad and dx must be 16-byte aligned");
   return launch_relu_mask<true>(dtype, n, grad, dx, const_cast<void *>(mask));
+}
+
+int mg_multiply_broadcast(int dtype, int nd, const int64_t *shape, const int64_t *a_strides, const int64_t *b_strides, const void *a,
+                          const void *b, void *out) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (dtype != MG_F32 && dtype != MG_F64) return fail(MG_ERR_UNSUPPORTED, "mg_multiply_broadcast: dtype %d (only float32=0 / float64=1)", dtype);
+  if (nd < 1 || nd > 6) return fail(MG_ERR_UNSUPPORTED, "mg_multiply_broadcast: %d axes (1 to 6 after merging)", nd);
+  if (!shape || !a_strides || !b_strides) return fail(MG_ERR_BAD_ARG, "null pointer in mg_multiply_broadcast");
+  const int vec = dtype == MG_F32 ? 4 : 2;  // elements in 16 bytes
+  long long n = 1, a_span = 1, b_span = 1;  // elements of out; one past the farthest element read of a and b
+  for (int d = 0; d < nd; ++d) {
+    if (shape[d] < 0 || a_strides[d] < 0 || b_strides[d] < 0) return fail(MG_ERR_BAD_ARG, "mg_multiply_broadcast: negative extent or stride");
+    if (shape[d] == 0) return MG_OK;
+    n *= shape[d];
+    if (n >= (1ll << 31)) return fail(MG_ERR_UNSUPPORTED, "mg_multiply_broadcast: 2^31 elements or more");
+    a_span += (shape[d] - 1) * a_strides[d];
+    b_span += (shape[d] - 1) * b_strides[d];
+  }
+  if (a_span > n || b_span > n) return fail(MG_ERR_BAD_ARG, "mg_multiply_broadcast: an operand reaches beyond the extent of the result");
+  if (a_strides[nd - 1] > 1 || b_strides[nd - 1] > 1)
+    return fail(MG_ERR_BAD_ARG, "mg_multiply_broadcast: the stride along the last axis must be 1 or 0");
+  if (!a || !b || !out) return fail(MG_ERR_BAD_ARG, "null pointer in mg_multiply_broadcast");
+  if (misaligned(a) || misaligned(b) || misaligned(out)) return fail(MG_ERR_BAD_ARG, "mg_multiply_broadcast: buffers must be 16-byte aligned");
+  BroadcastParams p{};
+  p.outer_dims = nd - 1;
+  bool aligned = shape[nd - 1] % vec == 0;
+  for (int d = 0; d < nd - 1; ++d) {
+    p.extent[d] = (unsigned)shape[d];
+    p.a_step[d] = (unsigned)a_strides[d];
+    p.b_step[d] = (unsigned)b_strides[d];
+    // 16-byte pieces of an operand must start on 16 bytes: every stride a multiple of the piece
+    aligned = aligned && (a_strides[nd - 1] == 0 || a_strides[d] % vec == 0) && (b_strides[nd - 1] == 0 || b_strides[d] % vec == 0);
+  }
+  p.a_inner = (unsigned)a_strides[nd - 1];
+  p.b_inner = (unsigned)b_strides[nd - 1];
+  p.inner = (unsigned)shape[nd - 1];
+  p.pieces = (unsigned)ceil_div(shape[nd - 1], (long long)vec);
+  const long long threads = (n / shape[nd - 1]) * p.pieces;
+  if (threads >= (1ll << 32) - 256 * 4096) return fail(MG_ERR_UNSUPPORTED, "mg_multiply_broadcast: too many rows of a short last axis");
+  p.threads = (unsigned)threads;
+  const unsigned grid = (unsigned)std::min<long long>(ceil_div(threads, 256), (long long)runtime().props.multiProcessorCount * 16);
+  hipStream_t s = runtime().stream;
+  ScopedTiming timed(TAG_ELEMENTWISE);
+#define MG_LAUNCH(T, ALIGNED) \
+  hipLaunchKernelGGL((multiply_broadcast_kernel<T, ALIGNED>), dim3(grid), dim3(256), 0, s, (const T *)a, (const T *)b, (T *)out, p)
+  if (dtype == MG_F32) {
+    if (aligned) MG_LAUNCH(float, true); else MG_LAUNCH(float, false);
+  } else {
+    if (aligned) MG_LAUNCH(double, true); else MG_LAUNCH(double, false);
+  }
+#undef MG_LAUNCH
+  MG_HIP(hipGetLastError());
+  return MG_OK;
 }
 
 int mg_sum_all(int dtype, int64_t n, const void *x, void *out) {

@@ -3,9 +3,11 @@
 The reference's ``Multiply`` is ``np.multiply`` with broadcasting and gradients
 ``grad * other``, summed back to the operand's shape over the axes it was broadcast along
 (``mygrad/_utils/__init__.py:131-168``).  Operands of one shape -- the case between the
-convolution / pooling kernels -- take one bandwidth-bound kernel; an operand that is
-broadcast is first spread to the common shape on the device, and its gradient is summed
-back there (carried in double, rounded once: equal to NumPy's pairwise sum to rounding).
+convolution / pooling kernels -- take one bandwidth-bound kernel; so do operands that are
+broadcast (``mg_multiply_broadcast`` reads each where it lies; only a pattern with more than
+six groups of axes is first spread to the common shape on the device), and the gradient of a
+broadcast operand is summed back on the device (carried in double, rounded once: equal to
+NumPy's pairwise sum to rounding).
 Floating-point operands only; other argument patterns raise (there is no CPU fallback)."""
 
 import numpy as np
@@ -35,9 +37,14 @@ def device_multiply(a, b, dtype, shape=None):
     size = int(np.prod(shape, dtype=np.int64))
     if size == 0:
         return np.empty(shape, dtype=dtype), None
-    ab, bb = _spread(a, shape, dtype), _spread(b, shape, dtype)
-    ob = _device.DeviceBuffer(max(size * dtype.itemsize, 16))
-    _hip.check(_hip.lib().mg_multiply(_hip.dtype_code(dtype), size, ab.ptr, bb.ptr, ob.ptr))
+    ob = None
+    if a.shape != shape or b.shape != shape:
+        # one pass that reads each operand where it lies
+        ob = _reduce.multiply_broadcast(_device.to_device(a, dtype), a.shape, _device.to_device(b, dtype), b.shape, shape, dtype)
+    if ob is None:
+        ab, bb = _spread(a, shape, dtype), _spread(b, shape, dtype)
+        ob = _device.DeviceBuffer(max(size * dtype.itemsize, 16))
+        _hip.check(_hip.lib().mg_multiply(_hip.dtype_code(dtype), size, ab.ptr, bb.ptr, ob.ptr))
     return _device.download(ob, shape, dtype), ob
 
 

@@ -122,6 +122,17 @@ def multiply(a, b):
     return _down(ob, a.shape, a.dtype)
 
 
+def multiply_broadcast(a, b):
+    """a * b with NumPy's broadcasting through mg_multiply_broadcast (the merged axes and the
+    strides come from the host's plan)."""
+    from mygrad_amd import _reduce
+
+    shape = np.broadcast_shapes(a.shape, b.shape)
+    dtype = np.dtype(np.result_type(a, b))
+    ob = _reduce.multiply_broadcast(_up(a.astype(dtype)), a.shape, _up(b.astype(dtype)), b.shape, shape, dtype)
+    return None if ob is None else _down(ob, shape, dtype)
+
+
 def relu_fwd(x):
     xb = _up(x)
     ob = _device.DeviceBuffer(max(x.nbytes, 16))

@@ -193,7 +193,49 @@ BROADCAST_CASES = [
     ((4, 5), (5,)), ((4, 5), (4, 1)), ((2, 3, 4), (3, 1)), ((3, 1, 2), (1, 4, 1)), ((2, 3), ()), ((1,), (2, 3)),
     ((2, 3, 4, 5), (1, 3, 1, 1)), ((5,), (5,)), ((8, 16, 12, 12), (16, 1, 1)), ((64, 1000), (1000,)), ((64, 1000), (64, 1)),
     ((2, 1, 3, 1, 2), (3, 1, 4, 1)), ((0, 3), (3,)), ((2, 3), (1,)),
+    # rows of whole 16-byte pieces with either operand, or neither, along them; rows that are not
+    ((6, 1, 64), (1, 5, 64)), ((6, 5, 1), (1, 1, 64)), ((3, 7, 1), (7, 62)), ((16, 1), (1, 16)), ((1, 1), (1,)),
+    ((4, 1, 6, 1, 8), (3, 1, 5, 1)), ((2, 1, 2, 1, 2, 1), (1, 3, 1, 3, 1, 8)),
+    # seven groups of axes after merging: more than the one-pass kernel takes, the operands are spread first
+    ((2, 1, 2, 1, 2, 1, 2), (1, 3, 1, 3, 1, 3, 1)),
 ]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("sa,sb", [c for c in BROADCAST_CASES if 0 not in c[0] + c[1]])
+def test_multiply_broadcast_bit_exact(abi, dtype, sa, sb):
+    rng = np.random.default_rng([7, len(sa), len(sb), int(np.prod(sa)) + int(np.prod(sb))])
+    a, b = rng.standard_normal(sa).astype(dtype), rng.standard_normal(sb).astype(dtype)
+    flat = a.reshape(-1)  # a view: special values at both ends and in the middle
+    flat[0], flat[-1], flat[a.size // 2] = np.nan, -0.0, np.inf
+    got = abi.multiply_broadcast(a, b)
+    from mygrad_amd import _reduce
+
+    if len(_reduce.multiply_plan(sa, sb, np.broadcast_shapes(sa, sb))[0]) > _reduce.MAX_MULTIPLY_AXES:
+        assert got is None
+        return
+    with np.errstate(invalid="ignore"):
+        want = ora.multiply(a, b)
+    assert got.shape == want.shape and np.array_equal(bits(got), bits(want))
+
+
+def test_multiply_broadcast_rejects_bad_arguments(abi):
+    import ctypes
+
+    from mygrad_amd import _device, _hip
+
+    lib, buf = _hip.lib(), _device.DeviceBuffer(4096)
+    arr = lambda *v: (ctypes.c_int64 * len(v))(*v)
+    call = lambda nd, shape, sa, sb, dtype=0: lib.mg_multiply_broadcast(dtype, nd, shape, sa, sb, buf.ptr, buf.ptr, buf.ptr)
+    assert call(2, arr(4, 8), arr(8, 1), arr(0, 1)) == _hip.MG_OK
+    assert call(2, arr(4, 8), arr(8, 2), arr(0, 1)) == _hip.MG_ERR_BAD_ARG  # stride along the last axis
+    assert call(2, arr(4, 8), arr(16, 1), arr(0, 1)) == _hip.MG_ERR_BAD_ARG  # an operand larger than the result
+    assert call(2, arr(4, 8), arr(-8, 1), arr(0, 1)) == _hip.MG_ERR_BAD_ARG
+    assert call(7, arr(*[2] * 7), arr(*[0] * 7), arr(*[0] * 7)) == _hip.MG_ERR_UNSUPPORTED
+    assert call(0, arr(1), arr(0), arr(0)) == _hip.MG_ERR_UNSUPPORTED
+    assert call(2, arr(1 << 16, 1 << 15), arr(0, 0), arr(0, 0)) == _hip.MG_ERR_UNSUPPORTED  # 2^31 elements
+    assert call(2, arr(4, 8), arr(8, 1), arr(0, 1), dtype=2) == _hip.MG_ERR_UNSUPPORTED
+    assert call(2, arr(0, 8), arr(8, 1), arr(0, 1)) == _hip.MG_OK  # nothing to do
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])

@@ -466,3 +466,26 @@ def test_multi_matmul_picks_the_cheapest_order_and_checks_its_arguments():
         mg.multi_matmul([np.ones((2, 2)), np.ones((2, 2, 2)), np.ones((2, 2))])
     with pytest.raises(ValueError):
         mg.multi_matmul([np.ones((2, 3)), np.ones(3), np.ones((3, 2))])  # a vector in the middle
+
+
+@pytest.mark.parametrize(
+    "sa,sb",
+    [((4, 5), (5,)), ((4, 5), (4, 1)), ((3, 1, 2), (1, 4, 1)), ((2, 3), ()), ((1,), (2, 3)), ((8, 16, 12, 12), (16, 1, 1)),
+     ((2, 1, 3, 1, 2), (3, 1, 4, 1)), ((1, 1), (1,)), ((2, 1, 2, 1, 2, 1, 2), (1, 3, 1, 3, 1, 3, 1)), ((2, 3, 4), (2, 3, 4))],
+)
+def test_multiply_plan_reads_each_operand_where_it_lies(sa, sb):
+    """The merged axes and strides of the one-pass broadcasting product, walked with NumPy's
+    own strided views, give NumPy's product."""
+    from numpy.lib.stride_tricks import as_strided
+
+    from mygrad_amd import _reduce
+
+    rng = np.random.default_rng(len(sa) * 10 + len(sb))
+    a, b = rng.standard_normal(sa), rng.standard_normal(sb)
+    shape = np.broadcast_shapes(sa, sb)
+    extents, a_strides, b_strides = _reduce.multiply_plan(sa, sb, shape)
+    assert int(np.prod(extents)) == int(np.prod(shape)) and a_strides[-1] in (0, 1) and b_strides[-1] in (0, 1)
+    assert all(x > 1 for x in extents) or extents == [1]
+    va = as_strided(a.reshape(-1) if a.size else a, shape=extents, strides=[8 * s for s in a_strides], writeable=False)
+    vb = as_strided(b.reshape(-1) if b.size else b, shape=extents, strides=[8 * s for s in b_strides], writeable=False)
+    assert np.array_equal((va * vb).reshape(shape), a * b)
