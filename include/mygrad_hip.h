@@ -264,6 +264,13 @@ int mg_batchnorm_bwd(const mg_bn_desc *desc, const void *x, const void *grad, co
  * Multiply. */
 int mg_sum_over(int dtype, int64_t outer, int64_t n, int64_t inner, int over_middle, const void *x, void *out);
 
+/* The same sums of x * y for two arrays of one shape, in one pass over both: the product is
+ * rounded to dtype before it is added, so the result is that of mg_multiply followed by
+ * mg_sum_over.  Replaces grad * other followed by reduce_broadcast's sums in
+ * Multiply.backward_var for an operand that was broadcast
+ * (src/mygrad/math/arithmetic/ops.py:48-53, src/mygrad/_utils/__init__.py:131-168). */
+int mg_sum_product_over(int dtype, int64_t outer, int64_t n, int64_t inner, int over_middle, const void *x, const void *y, void *out);
+
 /* ---- transposition ----
  * out = x.transpose(perm) made C-contiguous: x has `nd` axes of extents shape[], output axis i
  * is input axis perm[i]; elements of 4 or 8 bytes, fewer than 2^31 of them; at most 6 axes

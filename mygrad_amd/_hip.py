@@ -154,6 +154,7 @@ _SIGNATURES = {
     "mg_sum_all": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
     "mg_fill_from": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
     "mg_sum_over": [ctypes.c_int] + [ctypes.c_int64] * 3 + [ctypes.c_int, _vp, _vp],
+    "mg_sum_product_over": [ctypes.c_int] + [ctypes.c_int64] * 3 + [ctypes.c_int, _vp, _vp, _vp],
     "mg_batchnorm_fwd": [ctypes.POINTER(BnDesc), _vp, _vp, _vp, _vp, _vp, _vp],
     "mg_batchnorm_bwd": [ctypes.POINTER(BnDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
     "mg_matmul": [ctypes.c_int] + [ctypes.c_int64] * 4 + [_vp, _vp, _vp],

@@ -40,20 +40,35 @@ def _product(groups):
     return total
 
 
-def sum_axes(buf, shape, axes, dtype):
+def sum_axes(buf, shape, axes, dtype, times=None):
     """Device buffer with ``x.sum(axis=axes)`` of the C-contiguous ``x`` of ``shape`` in
-    ``buf`` (``axes``: normalised, unique).  The array must not be empty."""
+    ``buf`` (``axes``: normalised, unique).  The array must not be empty.  With ``times``, the
+    buffer of a ``y`` of the same shape, the sums are those of ``x * y`` (the product rounded
+    before it is added, as if it had been formed first), in the same number of passes."""
     lib, code = _hip.lib(), _hip.dtype_code(dtype)
+
+    def sum_over(outer, n, inner, over_middle, out):
+        nonlocal times
+        if times is None:
+            _hip.check(lib.mg_sum_over(code, outer, n, inner, over_middle, buf.ptr, out.ptr))
+        else:  # the first pass takes the product; what is left to sum afterwards is plain
+            _hip.check(lib.mg_sum_product_over(code, outer, n, inner, over_middle, buf.ptr, times.ptr, out.ptr))
+            times = None
+
     summed = set(axes)
     groups = _merge([(size, axis in summed) for axis, size in enumerate(shape)])
+    if times is not None and not any(kind for _, kind in groups):
+        raise ValueError("sum_axes with a second operand needs an axis to sum over")
     while any(kind for _, kind in groups):
         kinds = [kind for _, kind in groups]
         if kinds in ([True], [True, False], [False, True], [True, False, True]):
             # one kept group at most, summed groups around it: a single pass
-            if kinds == [True]:  # everything that is left is summed: the whole-array kernel
+            if kinds == [True] and times is None:  # everything that is left is summed: the whole-array kernel
                 out = _device.DeviceBuffer(16)
                 _hip.check(lib.mg_sum_all(code, groups[0][0], buf.ptr, out.ptr))
                 return out
+            elif kinds == [True]:  # of a product: one kept entry between nothing and the whole array
+                outer, n, inner = 1, 1, groups[0][0]
             elif kinds == [True, False]:
                 outer, n, inner = groups[0][0], groups[1][0], 1
             elif kinds == [False, True]:
@@ -61,13 +76,13 @@ def sum_axes(buf, shape, axes, dtype):
             else:
                 outer, n, inner = (g[0] for g in groups)
             out = _device.DeviceBuffer(max(n * dtype.itemsize, 16))
-            _hip.check(lib.mg_sum_over(code, outer, n, inner, 0, buf.ptr, out.ptr))
+            sum_over(outer, n, inner, 0, out)
             return out
         # several kept groups: take out the largest summed group, the rest next time round
         j = max((i for i, (_, kind) in enumerate(groups) if kind), key=lambda i: groups[i][0])
         outer, n, inner = _product(groups[:j]), groups[j][0], _product(groups[j + 1 :])
         out = _device.DeviceBuffer(max(outer * inner * dtype.itemsize, 16))
-        _hip.check(lib.mg_sum_over(code, outer, n, inner, 1, buf.ptr, out.ptr))
+        sum_over(outer, n, inner, 1, out)
         buf = out
         groups = _merge([tuple(g) for g in groups[:j] + groups[j + 1 :]])
     return buf

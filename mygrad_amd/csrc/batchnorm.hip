@@ -372,8 +372,8 @@ __global__ void __launch_bounds__(256) bn_bwd_apply_kernel(BnParams p, const T *
 // Plain sums over the same walks: out[c] = sum over n and s of x[n, c, s], carried in double
 // over the same fixed partition and trees as the statistics above.
 // ------------------------------------------------------------------------------------------
-template <typename T, int WALK>
-__global__ void __launch_bounds__(256) axis_sum_kernel(BnParams p, const T *__restrict__ x, double *__restrict__ partial) {
+template <typename T, int WALK, bool PRODUCT>
+__device__ __forceinline__ void axis_sum_body(const BnParams &p, const T *__restrict__ x, const T *__restrict__ y, double *__restrict__ partial) {
   typedef typename Wide<T>::type V;
   __shared__ double slots[8];
   bool active;
@@ -381,18 +381,35 @@ __global__ void __launch_bounds__(256) axis_sum_kernel(BnParams p, const T *__re
   double even = 0.0, odd = 0.0;  // two running sums, added at the end
   if (active)
     visit<T, WALK>(p, [&](long long at) {
+#pragma clang fp contract(off)  // the product is rounded to T, like a product formed first: no fused multiply-add
       if constexpr (WALK == ROWS_WIDE) {
-        const V v = *reinterpret_cast<const V *>(x + at);
+        V v = *reinterpret_cast<const V *>(x + at);
+        if constexpr (PRODUCT) v = v * *reinterpret_cast<const V *>(y + at);
 #pragma unroll
         for (int k = 0; k < Wide<T>::N; k += 2) {
           even += (double)v[k];
           odd += (double)v[k + 1];
         }
       } else {
-        even += (double)x[at];
+        T v = x[at];
+        if constexpr (PRODUCT) v = v * y[at];
+        even += (double)v;
       }
     });
   put_partial<WALK>(p, c, active, even, odd, partial, slots);
+}
+
+template <typename T, int WALK>
+__global__ void __launch_bounds__(256) axis_sum_kernel(BnParams p, const T *__restrict__ x, double *__restrict__ partial) {
+  axis_sum_body<T, WALK, false>(p, x, nullptr, partial);
+}
+
+// The same sum of x * y: the product is rounded to T before it is added, so the result is
+// that of multiplying first and summing afterwards, in one pass over both operands.
+template <typename T, int WALK>
+__global__ void __launch_bounds__(256) axis_sum_product_kernel(BnParams p, const T *__restrict__ x, const T *__restrict__ y,
+                                                               double *__restrict__ partial) {
+  axis_sum_body<T, WALK, true>(p, x, y, partial);
 }
 
 template <typename T>
@@ -414,9 +431,9 @@ struct MiddleParams {
   int chunk, chunks;
 };
 
-template <typename T, int VEC>
-__global__ void __launch_bounds__(256) sum_middle_kernel(MiddleParams p, const T *__restrict__ x, T *__restrict__ out,
-                                                         double *__restrict__ partial) {
+template <typename T, int VEC, bool PRODUCT>
+__global__ void __launch_bounds__(256) sum_middle_kernel(MiddleParams p, const T *__restrict__ x, const T *__restrict__ y,
+                                                         T *__restrict__ out, double *__restrict__ partial) {
   typedef T V __attribute__((ext_vector_type(VEC)));
   const long long piece = (long long)blockIdx.x * 256 + threadIdx.x;
   const int per_row = p.inner / VEC;
@@ -424,20 +441,27 @@ __global__ void __launch_bounds__(256) sum_middle_kernel(MiddleParams p, const T
   const long long o = piece / per_row;
   const int i = (int)(piece - o * per_row) * VEC;
   const int first = blockIdx.y * p.chunk, last = min(first + p.chunk, p.n);
-  const T *src = x + (o * p.n + first) * p.inner + i;
+  const long long start = (o * p.n + first) * p.inner + i;
+  const T *src = x + start;
+  const T *other = PRODUCT ? y + start : nullptr;  // x * y is rounded to T before it is added
   double acc[VEC];
 #pragma unroll
   for (int k = 0; k < VEC; ++k) acc[k] = 0.0;
 #pragma unroll 4
   for (int m = first; m < last; ++m) {
+#pragma clang fp contract(off)  // no fused multiply-add: the product is rounded first
     if constexpr (VEC == 1) {
-      acc[0] += (double)*src;
+      T v = *src;
+      if constexpr (PRODUCT) v = v * *other;
+      acc[0] += (double)v;
     } else {
-      const V v = *reinterpret_cast<const V *>(src);
+      V v = *reinterpret_cast<const V *>(src);
+      if constexpr (PRODUCT) v = v * *reinterpret_cast<const V *>(other);
 #pragma unroll
       for (int k = 0; k < VEC; ++k) acc[k] += (double)v[k];
     }
     src += p.inner;
+    if constexpr (PRODUCT) other += p.inner;
   }
   const long long at = o * p.inner + i;
   if (p.chunks == 1) {
@@ -569,24 +593,28 @@ int bwd_impl(const BnParams &p, const void *x, const void *grad, const void *gam
   return MG_OK;
 }
 
-// out[c] = sum over n, s of x[n, c, s]
+// out[c] = sum over n, s of x[n, c, s] (times y[n, c, s] if y is given)
 template <typename T>
-int axis_sum_impl(BnParams p, const void *x, void *out) {
+int axis_sum_impl(BnParams p, const void *x, const void *y, void *out) {
   hipStream_t s = runtime().stream;
   void *partial = nullptr;
   if (int rc = workspace((size_t)p.C * p.terms * 2 * sizeof(double), &partial)) return rc;
   const dim3 block(256);
-  const int walk = walk_for(p, sizeof(T), {x});
+  const int walk = y ? walk_for(p, sizeof(T), {x, y}) : walk_for(p, sizeof(T), {x});
   ScopedTiming timed(TAG_SUM_OVER);
+  auto launch = [&](const dim3 grid) {
+    if (y)
+      MG_BN_LAUNCH(axis_sum_product_kernel, walk, p, (const T *)x, (const T *)y, (double *)partial);
+    else
+      MG_BN_LAUNCH(axis_sum_kernel, walk, p, (const T *)x, (double *)partial);
+  };
   if (p.walk == COLS) {
-    const dim3 grid = grid_for(p);
-    MG_BN_LAUNCH(axis_sum_kernel, walk, p, (const T *)x, (double *)partial);
+    launch(grid_for(p));
   } else {
     const int channels = p.C;
     for (int c0 = 0; c0 < channels; c0 += 65535) {  // the grid's y extent
       p.c0 = c0;
-      const dim3 grid((unsigned)p.chunks, (unsigned)std::min(65535, channels - c0));
-      MG_BN_LAUNCH(axis_sum_kernel, walk, p, (const T *)x, (double *)partial);
+      launch(dim3((unsigned)p.chunks, (unsigned)std::min(65535, channels - c0)));
     }
     p.c0 = 0;
   }
@@ -595,12 +623,13 @@ int axis_sum_impl(BnParams p, const void *x, void *out) {
   return MG_OK;
 }
 
-// out[o, i] = sum over m of x[o, m, i]
+// out[o, i] = sum over m of x[o, m, i] (times y[o, m, i] if y is given)
 template <typename T>
-int middle_sum_impl(long long outer, long long n, long long inner, const void *x, void *out) {
+int middle_sum_impl(long long outer, long long n, long long inner, const void *x, const void *y, void *out) {
   hipStream_t s = runtime().stream;
   constexpr int WIDE = 16 / sizeof(T);
-  const bool wide = inner % WIDE == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  const bool wide = inner % WIDE == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0 &&
+                    reinterpret_cast<uintptr_t>(out) % 16 == 0;
   const int vec = wide ? WIDE : 1;
   MiddleParams p;
   p.outer = outer;
@@ -620,10 +649,14 @@ int middle_sum_impl(long long outer, long long n, long long inner, const void *x
     if (int rc = workspace((size_t)p.chunks * p.outs * sizeof(double), &partial)) return rc;
   const dim3 grid((unsigned)blocks, (unsigned)p.chunks), block(256);
   ScopedTiming timed(TAG_SUM_OVER);
-  if (wide)
-    hipLaunchKernelGGL((sum_middle_kernel<T, WIDE>), grid, block, 0, s, p, (const T *)x, (T *)out, (double *)partial);
-  else
-    hipLaunchKernelGGL((sum_middle_kernel<T, 1>), grid, block, 0, s, p, (const T *)x, (T *)out, (double *)partial);
+#define MG_MIDDLE(VEC, PRODUCT) \
+  hipLaunchKernelGGL((sum_middle_kernel<T, VEC, PRODUCT>), grid, block, 0, s, p, (const T *)x, (const T *)y, (T *)out, (double *)partial)
+  if (wide) {
+    if (y) MG_MIDDLE(WIDE, true); else MG_MIDDLE(WIDE, false);
+  } else {
+    if (y) MG_MIDDLE(1, true); else MG_MIDDLE(1, false);
+  }
+#undef MG_MIDDLE
   if (p.chunks > 1)
     hipLaunchKernelGGL(sum_middle_finish_kernel<T>, dim3((unsigned)ceil_div(p.outs, 256)), block, 0, s, p, (const double *)partial, (T *)out);
   MG_HIP(hipGetLastError());
@@ -662,17 +695,36 @@ int mg_batchnorm_bwd(const mg_bn_desc *desc, const void *x, const void *grad, co
                                : bwd_impl<double>(p, x, grad, gamma, mean, var, dx, dgamma, dbeta);
 }
 
+namespace {
+int sum_over(const char *who, int dtype, int64_t outer, int64_t n, int64_t inner, int over_middle, const void *x, const void *y, void *out);
+}
+
 int mg_sum_over(int dtype, int64_t outer, int64_t n, int64_t inner, int over_middle, const void *x, void *out) {
   std::lock_guard<std::recursive_mutex> guard(api_mutex());
   MG_REQUIRE_INIT();
-  if (dtype != MG_F32 && dtype != MG_F64) return fail(MG_ERR_UNSUPPORTED, "mg_sum_over: dtype %d (only float32=0 / float64=1)", dtype);
+  return sum_over("mg_sum_over", dtype, outer, n, inner, over_middle, x, nullptr, out);
+}
+
+int mg_sum_product_over(int dtype, int64_t outer, int64_t n, int64_t inner, int over_middle, const void *x, const void *y, void *out) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (!y) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_sum_product_over");
+  return sum_over("mg_sum_product_over", dtype, outer, n, inner, over_middle, x, y, out);
+}
+
+}  // extern "C"
+
+namespace {
+
+int sum_over(const char *who, int dtype, int64_t outer, int64_t n, int64_t inner, int over_middle, const void *x, const void *y, void *out) {
+  if (dtype != MG_F32 && dtype != MG_F64) return fail(MG_ERR_UNSUPPORTED, "%s: dtype %d (only float32=0 / float64=1)", who, dtype);
   if (outer < 1 || n < 1 || inner < 1)
-    return fail(MG_ERR_BAD_ARG, "mg_sum_over: outer=%lld n=%lld inner=%lld must be positive", (long long)outer, (long long)n, (long long)inner);
-  if (!x || !out) return fail(MG_ERR_BAD_ARG, "null tensor pointer in mg_sum_over");
+    return fail(MG_ERR_BAD_ARG, "%s: outer=%lld n=%lld inner=%lld must be positive", who, (long long)outer, (long long)n, (long long)inner);
+  if (!x || !out) return fail(MG_ERR_BAD_ARG, "null tensor pointer in %s", who);
   if (over_middle) {
     if (n >= (1ll << 31) || inner >= (1ll << 31) || ceil_div(outer * inner, 256) >= (1ll << 31))
-      return fail(MG_ERR_UNSUPPORTED, "mg_sum_over: an axis of 2^31 or more entries, or 2^39 or more results");
-    return dtype == MG_F32 ? middle_sum_impl<float>(outer, n, inner, x, out) : middle_sum_impl<double>(outer, n, inner, x, out);
+      return fail(MG_ERR_UNSUPPORTED, "%s: an axis of 2^31 or more entries, or 2^39 or more results", who);
+    return dtype == MG_F32 ? middle_sum_impl<float>(outer, n, inner, x, y, out) : middle_sum_impl<double>(outer, n, inner, x, y, out);
   }
   mg_bn_desc desc{};
   desc.dtype = dtype;
@@ -681,8 +733,8 @@ int mg_sum_over(int dtype, int64_t outer, int64_t n, int64_t inner, int over_mid
   desc.S = inner;
   desc.eps = 0.0;
   BnParams p;
-  if (int rc = make_params(&desc, &p, "mg_sum_over", true)) return rc;
-  return dtype == MG_F32 ? axis_sum_impl<float>(p, x, out) : axis_sum_impl<double>(p, x, out);
+  if (int rc = make_params(&desc, &p, who, true)) return rc;
+  return dtype == MG_F32 ? axis_sum_impl<float>(p, x, y, out) : axis_sum_impl<double>(p, x, y, out);
 }
 
-}  // extern "C"
+}  // namespace

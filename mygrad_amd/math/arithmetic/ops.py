@@ -69,17 +69,25 @@ class Multiply(Operation):
         dtype = np.dtype(np.result_type(grad, other.data))
         if grad.shape != self._shape or dtype not in (np.float32, np.float64):
             raise NotImplementedError(f"multiply backward for gradient {grad.shape} {grad.dtype} (no CPU fallback)")
-        out, ob = device_multiply(grad, other.data, dtype, self._shape)
-        if ob is None:
-            return np.zeros(var.shape, dtype=dtype)
-        if var.shape == self._shape:
+        if var.size == int(np.prod(self._shape, dtype=np.int64)):  # nothing to add up (axes of length one at most)
+            out, ob = device_multiply(grad, other.data, dtype, self._shape)
+            if ob is None:
+                return np.zeros(var.shape, dtype=dtype)
+            out = out.reshape(var.shape)
             _device.attach_transient(out, ob)
             return out
+        if 0 in self._shape:
+            return np.zeros(var.shape, dtype=dtype)
         # the operand was broadcast: add its gradient up over the axes it was spread along
         # (reduce_broadcast: the leading axes it lacks and those where it has length one)
         lead = len(self._shape) - var.ndim
         axes = tuple(range(lead)) + tuple(lead + i for i, n in enumerate(var.shape) if n == 1 and self._shape[lead + i] != 1)
-        rb = _reduce.sum_axes(ob, self._shape, axes, dtype)
+        if other.shape == self._shape:
+            # product and sums in one pass over the gradient and the other operand
+            rb = _reduce.sum_axes(_device.to_device(grad, dtype), self._shape, axes, dtype, times=_device.to_device(other.data, dtype))
+        else:
+            _, ob = device_multiply(grad, other.data, dtype, self._shape)
+            rb = _reduce.sum_axes(ob, self._shape, axes, dtype)
         back = _device.download(rb, var.shape, dtype)
         _device.attach_transient(back, rb)
         return back

@@ -203,6 +203,16 @@ def sum_over(x3, over_middle):
     return _down(ob, out_shape, x3.dtype)
 
 
+def sum_product_over(x3, y3, over_middle):
+    """The same sums of x3 * y3, in one pass."""
+    outer, n, inner = x3.shape
+    xb, yb = _up(x3), _up(y3)
+    out_shape = (outer, inner) if over_middle else (n,)
+    ob = _device.DeviceBuffer(max(int(np.prod(out_shape)) * x3.dtype.itemsize, 16))
+    _hip.check(_hip.lib().mg_sum_product_over(_hip.dtype_code(x3.dtype), outer, n, inner, int(over_middle), xb.ptr, yb.ptr, ob.ptr))
+    return _down(ob, out_shape, x3.dtype)
+
+
 def sum_all(x):
     xb = _up(x)
     ob = _device.DeviceBuffer(16)

@@ -117,6 +117,34 @@ def test_sum_over_both_forms_against_exact_sums(abi, dtype, shape):
         assert np.array_equal(bits(abi.sum_over(x, over_middle)), bits(got))  # the same partition and trees every run
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("shape", SUM_OVER_SHAPES)
+def test_sum_product_over_equals_product_then_sum(abi, dtype, shape):
+    """mg_sum_product_over rounds each product to the array's precision before adding it and
+    adds in mg_sum_over's order, so it gives bit for bit what mg_multiply followed by
+    mg_sum_over gives (both of which are checked against NumPy on their own)."""
+    dtype = np.dtype(dtype)
+    rng = np.random.default_rng([3, *shape])
+    x = (rng.standard_normal(shape) * 10.0 ** rng.integers(-2, 3, shape)).astype(dtype)
+    y = rng.standard_normal(shape).astype(dtype)
+    product = abi.multiply(x, y)
+    assert np.array_equal(bits(product), bits(x * y))
+    for over_middle in (True, False):
+        got = abi.sum_product_over(x, y, over_middle)
+        assert np.array_equal(bits(got), bits(abi.sum_over(product, over_middle)))
+
+
+def test_sum_product_over_bad_arguments(abi):
+    from mygrad_amd import _device, _hip
+
+    buf, lib = _device.DeviceBuffer(64), _hip.lib()
+    assert lib.mg_sum_product_over(0, 1, 2, 3, 0, buf.ptr, None, buf.ptr) == _hip.MG_ERR_BAD_ARG
+    assert lib.mg_sum_product_over(0, 1, 2, 3, 0, None, buf.ptr, buf.ptr) == _hip.MG_ERR_BAD_ARG
+    assert lib.mg_sum_product_over(0, 1, 0, 3, 1, buf.ptr, buf.ptr, buf.ptr) == _hip.MG_ERR_BAD_ARG
+    assert lib.mg_sum_product_over(2, 1, 2, 3, 1, buf.ptr, buf.ptr, buf.ptr) == _hip.MG_ERR_UNSUPPORTED
+    assert "mg_sum_product_over" in _hip.last_error()
+
+
 def test_sum_over_full_size(abi):
     """The benchmark's tensor (134 MB) summed per channel and over the channel axis, against
     NumPy's sums of the same values in float64."""
