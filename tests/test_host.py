@@ -489,3 +489,38 @@ def test_multiply_plan_reads_each_operand_where_it_lies(sa, sb):
     va = as_strided(a.reshape(-1) if a.size else a, shape=extents, strides=[8 * s for s in a_strides], writeable=False)
     vb = as_strided(b.reshape(-1) if b.size else b, shape=extents, strides=[8 * s for s in b_strides], writeable=False)
     assert np.array_equal((va * vb).reshape(shape), a * b)
+
+
+def test_multiply_plan_on_drawn_shapes():
+    """The same property on shapes drawn by hypothesis: any two shapes that broadcast."""
+    from hypothesis import given, settings
+    from hypothesis import strategies as st
+    from numpy.lib.stride_tricks import as_strided
+
+    from mygrad_amd import _reduce
+
+    @st.composite
+    def pairs(draw):
+        full = draw(st.lists(st.integers(1, 4), min_size=0, max_size=7))
+        def operand():
+            keep = draw(st.integers(0, len(full)))
+            tail = full[len(full) - keep:]
+            return tuple(n if draw(st.booleans()) else 1 for n in tail)
+        return operand(), operand()
+
+    @settings(max_examples=300, deadline=None)
+    @given(pairs())
+    def check(pair):
+        sa, sb = pair
+        shape = np.broadcast_shapes(sa, sb)
+        a = np.arange(1, 1 + int(np.prod(sa)), dtype=np.float64).reshape(sa)
+        b = np.arange(2, 2 + int(np.prod(sb)), dtype=np.float64).reshape(sb) * 0.5
+        extents, a_strides, b_strides = _reduce.multiply_plan(sa, sb, shape)
+        assert int(np.prod(extents)) == int(np.prod(shape))
+        assert 1 + sum((n - 1) * s for n, s in zip(extents, a_strides)) == a.size  # reaches a's last element, no further
+        assert 1 + sum((n - 1) * s for n, s in zip(extents, b_strides)) == b.size
+        va = as_strided(a.reshape(-1), shape=extents, strides=[8 * s for s in a_strides], writeable=False)
+        vb = as_strided(b.reshape(-1), shape=extents, strides=[8 * s for s in b_strides], writeable=False)
+        assert np.array_equal((va * vb).reshape(shape), a * b)
+
+    check()
