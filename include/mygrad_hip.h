@@ -310,6 +310,16 @@ int mg_matmul_da(int dtype, int64_t batch, int64_t M, int64_t K, int64_t N, cons
  * grad), ops.py:116-124). */
 int mg_matmul_dx(int dtype, int64_t batch, int64_t M, int64_t K, int64_t N, const void *grad, const void *a, void *dx);
 
+/* out[p] = op(a[p]) @ op(b[p]) for p < batch: op(a[p]):(M, K), op(b[p]):(K, N), out[p]:(M, N);
+ * with trans_a the matrix a[p] is stored as (K, M), with trans_b the matrix b[p] as (N, K); the
+ * stacks are C-contiguous.  One launch for the whole stack (a wavefront per 16 x 16 tile of one
+ * product), meant for stacks of matrices too small to fill the device one pair at a time; the
+ * two gradients are the same call with the transpositions set.  Replaces np.matmul on two
+ * stacks in MatMul.__call__ and the products of MatMul.backward_var,
+ * src/mygrad/math/misc/ops.py:91-126. */
+int mg_matmul_batched(int dtype, int64_t batch, int64_t M, int64_t K, int64_t N, int trans_a, int trans_b, const void *a, const void *b,
+                      void *out);
+
 /* ---- repeat and the window view ---- */
 
 /* out[o, j, i] = a[o, src(j), i] with a seen as (outer, n, inner) around the repeated axis

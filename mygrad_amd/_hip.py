@@ -158,6 +158,7 @@ _SIGNATURES = {
     "mg_batchnorm_fwd": [ctypes.POINTER(BnDesc), _vp, _vp, _vp, _vp, _vp, _vp],
     "mg_batchnorm_bwd": [ctypes.POINTER(BnDesc), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
     "mg_matmul": [ctypes.c_int] + [ctypes.c_int64] * 4 + [_vp, _vp, _vp],
+    "mg_matmul_batched": [ctypes.c_int] + [ctypes.c_int64] * 4 + [ctypes.c_int, ctypes.c_int, _vp, _vp, _vp],
     "mg_matmul_da": [ctypes.c_int] + [ctypes.c_int64] * 4 + [_vp, _vp, _vp],
     "mg_matmul_dx": [ctypes.c_int] + [ctypes.c_int64] * 4 + [_vp, _vp, _vp],
     "mg_repeat_fwd": [ctypes.c_int] + [ctypes.c_int64] * 5 + [_vp, _vp, _vp],
@@ -271,6 +272,7 @@ KERNEL_TAGS = {
     17: "window_gather",
     18: "sum_over",
     19: "permute",
+    20: "batched_product",
 }
 
 

@@ -1,0 +1,125 @@
+// Products of many small matrix pairs in one launch: out[p] = op(a[p]) @ op(b[p]), p < batch,
+// where op transposes or not.  A pair of stacks whose matrices are too small to fill the device
+// one pair at a time (np.matmul on two stacks, an einsum with a label that both operands and
+// the result carry) is bound by launches, not arithmetic, when each pair gets a launch of the
+// convolution kernels; here a wavefront makes one 16x16 tile of one product on the matrix cores,
+// reading its operands where they lie (a transposed operand is a pair of swapped strides), so the
+// whole stack is one grid.  Large pairs stay with the tiled kernels, which re-use operands
+// through LDS.
+#include "internal.h"
+
+#include <algorithm>
+
+namespace mg {
+
+namespace {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+
+// D(16x16) += A(16x4) * B(4x16) on one wavefront: lane l supplies A[l%16][l/16] and
+// B[l/16][l%16] and receives four elements of column l%16 of D, in rows row_of(l, r).
+template <typename T>
+struct Tile;
+
+template <>
+struct Tile<float> {
+  using Acc = f32x4;
+  static __device__ __forceinline__ Acc run(float a, float b, Acc c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ int row_of(int lane, int r) { return 4 * (lane >> 4) + r; }
+};
+
+template <>
+struct Tile<double> {
+  using Acc = f64x4;
+  static __device__ __forceinline__ Acc run(double a, double b, Acc c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+  static __device__ __forceinline__ int row_of(int lane, int r) { return 4 * r + (lane >> 4); }
+};
+
+struct BatchedParams {
+  int M, K, N;
+  int row_tiles, col_tiles;
+  long long tiles;                   // batch * row_tiles * col_tiles
+  long long a_pair, a_row, a_col;    // element strides of op(a): between pairs, along M, along K
+  long long b_pair, b_row, b_col;    // of op(b): between pairs, along K, along N
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) batched_product_kernel(BatchedParams p, const T *__restrict__ a, const T *__restrict__ b,
+                                                              T *__restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  const long long tile = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);  // the same for a whole wavefront
+  if (tile >= p.tiles) return;
+  const int per_pair = p.row_tiles * p.col_tiles;
+  const long long pair = tile / per_pair;
+  const int within = (int)(tile - pair * per_pair);
+  const int row0 = (within / p.col_tiles) * 16, col0 = (within % p.col_tiles) * 16;
+  const int i = row0 + (lane & 15), j = col0 + (lane & 15), kk = lane >> 4;
+  // rows and columns beyond the matrix supply zeros and are not stored
+  const bool row_in = i < p.M, col_in = j < p.N;
+  const T *pa = a + pair * p.a_pair + (row_in ? (long long)i * p.a_row : 0);
+  const T *pb = b + pair * p.b_pair + (col_in ? (long long)j * p.b_col : 0);
+  typename Tile<T>::Acc acc = {0, 0, 0, 0};
+  const int whole = p.K & ~3;
+#pragma unroll 4
+  for (int k0 = 0; k0 < whole; k0 += 4) {
+    const int k = k0 + kk;
+    const T av = row_in ? pa[(long long)k * p.a_col] : T(0);
+    const T bv = col_in ? pb[(long long)k * p.b_row] : T(0);
+    acc = Tile<T>::run(av, bv, acc);
+  }
+  if (whole < p.K) {  // the last one to three columns of op(a) / rows of op(b)
+    const int k = whole + kk;
+    const bool k_in = k < p.K;
+    const T av = row_in && k_in ? pa[(long long)k * p.a_col] : T(0);
+    const T bv = col_in && k_in ? pb[(long long)k * p.b_row] : T(0);
+    acc = Tile<T>::run(av, bv, acc);
+  }
+  if (!col_in) return;
+  T *po = out + pair * ((long long)p.M * p.N) + j;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int row = row0 + Tile<T>::row_of(lane, r);
+    if (row < p.M) po[(long long)row * p.N] = acc[r];
+  }
+}
+
+}  // namespace
+}  // namespace mg
+
+using namespace mg;
+
+extern "C" {
+
+int mg_matmul_batched(int dtype, int64_t batch, int64_t M, int64_t K, int64_t N, int trans_a, int trans_b, const void *a, const void *b,
+                      void *out) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (dtype != MG_F32 && dtype != MG_F64) return fail(MG_ERR_UNSUPPORTED, "mg_matmul_batched: dtype %d (only float32=0 / float64=1)", dtype);
+  if (batch < 0 || M < 0 || K < 0 || N < 0)
+    return fail(MG_ERR_BAD_ARG, "mg_matmul_batched: batch=%lld M=%lld K=%lld N=%lld", (long long)batch, (long long)M, (long long)K, (long long)N);
+  if (batch == 0 || M == 0 || N == 0) return MG_OK;
+  if (M >= (1 << 24) || K >= (1 << 24) || N >= (1 << 24) || batch >= (1ll << 31))
+    return fail(MG_ERR_UNSUPPORTED, "mg_matmul_batched: an extent of 2^24 or more, or 2^31 pairs or more");
+  if (!out || (K > 0 && (!a || !b))) return fail(MG_ERR_BAD_ARG, "null pointer in mg_matmul_batched");
+  BatchedParams p{};
+  p.M = (int)M, p.K = (int)K, p.N = (int)N;
+  p.row_tiles = (int)ceil_div(M, 16);
+  p.col_tiles = (int)ceil_div(N, 16);
+  p.tiles = batch * p.row_tiles * p.col_tiles;
+  if (ceil_div(p.tiles, 4) >= (1ll << 31)) return fail(MG_ERR_UNSUPPORTED, "mg_matmul_batched: 2^33 tiles of 16 x 16 results or more");
+  p.a_pair = M * K, p.b_pair = K * N;
+  p.a_row = trans_a ? 1 : K, p.a_col = trans_a ? M : 1;  // a[p] is stored (K, M) when transposed
+  p.b_row = trans_b ? 1 : N, p.b_col = trans_b ? K : 1;  // b[p] is stored (N, K) when transposed
+  hipStream_t s = runtime().stream;
+  ScopedTiming timed(TAG_BATCHED_PRODUCT);
+  const dim3 grid((unsigned)ceil_div(p.tiles, 4)), block(256);
+  if (dtype == MG_F32)
+    hipLaunchKernelGGL(batched_product_kernel<float>, grid, block, 0, s, p, (const float *)a, (const float *)b, (float *)out);
+  else
+    hipLaunchKernelGGL(batched_product_kernel<double>, grid, block, 0, s, p, (const double *)a, (const double *)b, (double *)out);
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
+}  // extern "C"

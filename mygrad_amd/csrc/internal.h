@@ -61,6 +61,7 @@ enum KernelTag {
   TAG_WINDOW_GATHER = 17,
   TAG_SUM_OVER = 18,
   TAG_PERMUTE = 19,
+  TAG_BATCHED_PRODUCT = 20,
 };
 void timing_begin(int tag);
 void timing_end();

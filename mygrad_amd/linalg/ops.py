@@ -6,7 +6,8 @@ first (``mg_sum_over``); the others fall into batch labels (both operands and th
 contracted labels (both operands, not the result), row labels (first operand and result)
 and column labels (second operand and result); the operands are transposed on the device
 to ``(batch, rows, contracted)`` and ``(batch, contracted, columns)`` (``mg_permute``),
-multiplied (``mg_matmul``, one launch per batch entry), and the product is transposed into
+multiplied (``mg_matmul_batched`` for a stack of small products, else ``mg_matmul`` with one
+launch per batch entry), and the product is transposed into
 the order the subscripts ask for.  Two arrangements need no transposition of the large
 tensors and are recognised first: a convolution with a one-element window written as a
 summation (``"nchw,fc->nfhw"`` and its input gradient: ``mg_matmul`` with the leading labels
@@ -28,6 +29,7 @@ import numpy as np
 
 from .. import _device, _hip, _reduce
 from ..errors import SkipGradient
+from ..math.misc.ops import SMALL_PAIR_FLOPS
 from ..operation_base import Operation
 
 __all__ = ["EinSum"]
@@ -176,6 +178,17 @@ def contract(operands, out_lbls, sizes, dtype):
     cols = "".join(lbl for lbl in out_lbls if lbl in blbl and lbl not in albl)
     B, M, K, N = (_prod(sizes[lbl] for lbl in group) for group in (batch, rows, summed, cols))
     out = _device.DeviceBuffer(max(B * M * N * item, 16))
+    if B > 1 and 2 * M * K * N <= SMALL_PAIR_FLOPS:
+        # many small products: one launch for all of them; an operand that already lies
+        # transposed is read that way instead of being moved
+        trans_a = albl == batch + summed + rows and M > 1 and K > 1
+        trans_b = blbl == batch + cols + summed and N > 1 and K > 1
+        if not trans_a:
+            abuf = _ordered(abuf, albl, batch + rows + summed, sizes, dtype)
+        if not trans_b:
+            bbuf = _ordered(bbuf, blbl, batch + summed + cols, sizes, dtype)
+        _hip.check(lib.mg_matmul_batched(code, B, M, K, N, int(trans_a), int(trans_b), abuf.ptr, bbuf.ptr, out.ptr))
+        return _ordered(out, batch + rows + cols, out_lbls, sizes, dtype)
     if K >= 4 * max(M, N):
         # a long sum and a small result: the filter-gradient kernels, out = a @ b^T over the long axis
         abuf = _ordered(abuf, albl, batch + rows + summed, sizes, dtype)

@@ -8,7 +8,8 @@ implicit-GEMM kernels (``mg_matmul*`` in ``libmygrad_hip.so``) with no kernel of
 Operand patterns that run: both operands at most 2-D (vectors are promoted like
 ``np.matmul`` does); one operand a stack and the other at most 2-D (one launch: the stack is
 the convolution's batch, or folds into the rows of the left operand); two stacks of the same
-batch shape (one launch per matrix pair); two stacks that broadcast against each other
+batch shape (one launch for all pairs when the matrices are small, ``mg_matmul_batched``,
+else one launch of the tiled kernels per matrix pair); two stacks that broadcast against each other
 (each is first spread to the common batch shape on the device, and the gradient of a stack
 that was spread is summed back over the axes it was spread along)."""
 
@@ -18,6 +19,14 @@ from ... import _device, _hip, _reduce
 from ...operation_base import Operation
 
 __all__ = ["MatMul"]
+
+
+# Two stacks are multiplied pair by pair on the tiled kernels when a pair has more than this
+# many floating-point operations (it then fills the device by itself), else in one launch of the
+# kernel that gives every 16 x 16 tile of every product a wavefront.  Measured on float32 squares:
+# that kernel sustains 16-18 TFLOP/s from 128^3 up, a launch of the tiled kernels costs 8-12 us,
+# so the two meet near 450^3 per pair.
+SMALL_PAIR_FLOPS = 2 * 384**3
 
 
 def _prod(shape):
@@ -87,6 +96,18 @@ class MatMul(Operation):
             _hip.check(fn(code, _prod(stack_b), M, K, N, first.ptr, second.ptr, result.ptr))
         elif not stack_b:
             _hip.check(fn(code, 1, _prod(stack_a) * M, K, N, first.ptr, second.ptr, result.ptr))
+        elif 2 * M * K * N <= SMALL_PAIR_FLOPS:
+            # a stack of small pairs: one launch, the gradients by transposed reads
+            # (entry: first, second -> result)   mg_matmul: a, b -> a @ b;
+            # mg_matmul_da: grad, b -> grad @ b^T;   mg_matmul_dx: grad, a -> a^T @ grad
+            pairs = _prod(stack_a)
+            batched = _hip.lib().mg_matmul_batched
+            if entry == "mg_matmul":
+                _hip.check(batched(code, pairs, M, K, N, 0, 0, first.ptr, second.ptr, result.ptr))
+            elif entry == "mg_matmul_da":
+                _hip.check(batched(code, pairs, M, N, K, 0, 1, first.ptr, second.ptr, result.ptr))
+            else:
+                _hip.check(batched(code, pairs, K, M, N, 1, 0, second.ptr, first.ptr, result.ptr))
         else:
             per = (M * K * item, K * N * item, M * N * item)
             for i in range(_prod(stack_a)):

@@ -347,6 +347,18 @@ def matmul(a, x):
     return _down(ob, (batch, M, N), a.dtype)
 
 
+def matmul_batched(a, b, trans_a=False, trans_b=False):
+    """op(a[p]) @ op(b[p]) for stacks a:(batch, M, K) -- (batch, K, M) with trans_a -- and
+    b:(batch, K, N) -- (batch, N, K) with trans_b -- through mg_matmul_batched."""
+    batch = a.shape[0]
+    K, M = a.shape[1:] if trans_a else a.shape[:0:-1]
+    N = b.shape[1] if trans_b else b.shape[2]
+    ab, bb = _up(a), _up(b)
+    ob = _device.DeviceBuffer(max(batch * M * N * a.itemsize, 16))
+    _hip.check(_hip.lib().mg_matmul_batched(_hip.dtype_code(a.dtype), batch, M, K, N, int(trans_a), int(trans_b), ab.ptr, bb.ptr, ob.ptr))
+    return _down(ob, (batch, M, N), a.dtype)
+
+
 def matmul_da(grad, x, M):
     batch, K, N = x.shape
     gb, xb = _up(grad), _up(x)

@@ -80,6 +80,42 @@ def test_results_repeat_exactly(abi):
         assert np.array_equal(fn(*args), fn(*args))
 
 
+BATCHED = [(1, 1, 1, 1), (3, 16, 16, 16), (5, 17, 3, 33), (2, 1, 70, 1), (300, 8, 8, 8), (7, 64, 40, 48), (4, 33, 6, 2), (2, 5, 0, 4),
+           (3, 100, 129, 50)]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("batch, M, K, N", BATCHED)
+def test_batched_product_with_and_without_transposed_operands(abi, batch, M, K, N, dtype):
+    """mg_matmul_batched against float64 products of the same values, to the bar of the other
+    matrix products (max abs error over the largest |entry|: 2e-4 float32, 1e-10 float64)."""
+    dtype = np.dtype(dtype)
+    rng = np.random.default_rng([batch, M, K, N])
+    a, b = rng.standard_normal((batch, M, K)).astype(dtype), rng.standard_normal((batch, K, N)).astype(dtype)
+    want = np.matmul(a.astype(np.float64), b.astype(np.float64))
+    at, bt = np.ascontiguousarray(a.transpose(0, 2, 1)), np.ascontiguousarray(b.transpose(0, 2, 1))
+    for ta, tb in ((False, False), (True, False), (False, True), (True, True)):
+        got = abi.matmul_batched(at if ta else a, bt if tb else b, ta, tb)
+        assert got.shape == want.shape and got.dtype == dtype
+        assert err(got, want) <= TOL[dtype], (ta, tb)
+    if K:  # a column and a row of the result must not see their neighbours: exact small integers
+        ai, bi = np.round(a * 2), np.round(b * 2)
+        assert np.array_equal(abi.matmul_batched(ai, bi), np.matmul(ai, bi))
+
+
+def test_batched_product_bad_arguments(abi):
+    from mygrad_amd import _device, _hip
+
+    buf, lib = _device.DeviceBuffer(4096), _hip.lib()
+    assert lib.mg_matmul_batched(0, 2, 4, 4, 4, 0, 0, buf.ptr, buf.ptr, buf.ptr) == _hip.MG_OK
+    assert lib.mg_matmul_batched(2, 2, 4, 4, 4, 0, 0, buf.ptr, buf.ptr, buf.ptr) == _hip.MG_ERR_UNSUPPORTED
+    assert lib.mg_matmul_batched(0, 2, -1, 4, 4, 0, 0, buf.ptr, buf.ptr, buf.ptr) == _hip.MG_ERR_BAD_ARG
+    assert lib.mg_matmul_batched(0, 2, 4, 4, 4, 0, 0, None, buf.ptr, buf.ptr) == _hip.MG_ERR_BAD_ARG
+    assert lib.mg_matmul_batched(0, 2, 4, 4, 4, 0, 0, buf.ptr, buf.ptr, None) == _hip.MG_ERR_BAD_ARG
+    assert lib.mg_matmul_batched(0, 2, 1 << 24, 4, 4, 0, 0, buf.ptr, buf.ptr, buf.ptr) == _hip.MG_ERR_UNSUPPORTED
+    assert lib.mg_matmul_batched(0, 0, 4, 4, 4, 0, 0, None, None, None) == _hip.MG_OK  # nothing to do
+
+
 SHAPES = [
     ((3, 4), (4, 5)),
     ((4,), (4, 5)),
@@ -91,6 +127,7 @@ SHAPES = [
     ((4,), (2, 3, 4, 5)),
     ((2, 3, 4), (4,)),
     ((2, 2, 30, 40), (2, 2, 40, 50)),
+    ((2, 400, 410), (2, 410, 390)),  # pairs large enough for a launch of the tiled kernels each
     ((60, 70), (70, 80)),
     # stacks that broadcast against each other
     ((2, 1, 3, 4), (2, 4, 5)),
