@@ -65,6 +65,7 @@ WORKLOADS = {
     # batch normalisation (scaled and shifted) of a tensor of conv3a's output size
     "bn3a": dict(kind="bn", dtype="f32", seed=1008, x=(128, 64, 56, 56), eps=1e-5),
     # matrix product on the convolution kernels: one dense layer's three products
+    "bmm64": dict(kind="bmm", dtype="f32", seed=1016, batch=512, M=64, K=64, N=64),
     "mm4k": dict(kind="matmul", dtype="f32", seed=1011, M=4096, K=4096, N=4096),
     # sums over axes of a tensor of conv5's output size: per channel (the gradient of a bias or of a
     # per-channel scale: every axis but axis 1), then over the channel axis alone
@@ -113,7 +114,10 @@ def pool_shapes(wl):
 def describe(name):
     wl = WORKLOADS[name]
     if wl["kind"] == "elem":
-        return f"{name}: relu + multiply + sum {wl['dtype']} x{wl['x']} fwd+bwd (7 kernels, 16 |x| bytes)"
+        return f"{name}: relu + multiply + sum {wl['dtype']} x{wl['x']} fwd+bwd (7 kernels, 15 |x| bytes + relu's mask)"
+    if wl["kind"] == "bmm":
+        return (f"{name}: matmul {wl['dtype']} of two stacks ({wl['batch']},{wl['M']},{wl['K']}) @ ({wl['batch']},{wl['K']},{wl['N']}): "
+                "product + both gradients")
     if wl["kind"] == "matmul":
         return f"{name}: matmul {wl['dtype']} ({wl['M']},{wl['K']}) @ ({wl['K']},{wl['N']}): product + both gradients"
     if wl["kind"] == "permute":
@@ -172,6 +176,16 @@ class Step:
             per_pass = conv_flops_per_pass(wl)
             self.work = {"conv_fwd": per_pass, "conv_dgrad": per_pass, "conv_wgrad": per_pass}
             self.total_work = 3 * per_pass
+            self.unit, self.bound, self.peak = "TFLOP/s", "mfma", PEAK_TFLOPS[wl["dtype"]]
+            self.scale = 1e-12
+        elif wl["kind"] == "bmm":
+            B, M, K, N = wl["batch"], wl["M"], wl["K"], wl["N"]
+            self.w = resident((rng.standard_normal((B, M, K)) * K ** -0.5).astype(dt))
+            self.x, self.g = resident(rng.standard_normal((B, K, N)).astype(dt)), resident(rng.standard_normal((B, M, N)).astype(dt))
+            self.out, self.dx, self.dw = (_device.DeviceBuffer(B * n * item) for n in (M * N, K * N, M * K))
+            self.code, self.dims = _hip.dtype_code(dt), (B, M, K, N)
+            self.work = {"batched_product": 2.0 * B * M * K * N}
+            self.total_work = 6.0 * B * M * K * N
             self.unit, self.bound, self.peak = "TFLOP/s", "mfma", PEAK_TFLOPS[wl["dtype"]]
             self.scale = 1e-12
         elif wl["kind"] == "matmul":
@@ -329,6 +343,12 @@ class Step:
             check(lib.mg_multiply(c, n, self.dx.ptr, self.x.ptr, self.out.ptr))  # d (a*b) / d b
             check(lib.mg_relu_bwd_mask(c, n, self.mask.ptr, self.dx.ptr, self.out.ptr))
             return
+        if self.wl["kind"] == "bmm":
+            B, M, K, N = self.dims
+            check(lib.mg_matmul_batched(self.code, B, M, K, N, 0, 0, self.w.ptr, self.x.ptr, self.out.ptr))
+            check(lib.mg_matmul_batched(self.code, B, M, N, K, 0, 1, self.g.ptr, self.x.ptr, self.dw.ptr))  # grad @ x^T
+            check(lib.mg_matmul_batched(self.code, B, K, M, N, 1, 0, self.w.ptr, self.g.ptr, self.dx.ptr))  # a^T @ grad
+            return
         if self.wl["kind"] == "matmul":
             check(lib.mg_matmul(self.code, *self.dims, self.w.ptr, self.x.ptr, self.out.ptr))
             check(lib.mg_matmul_dx(self.code, *self.dims, self.g.ptr, self.w.ptr, self.dx.ptr))
@@ -479,6 +499,18 @@ def run_cpu_baseline(name, min_seconds=10.0, max_reps=200):
 
         work, scale, unit = 3 * conv_flops_per_pass(wl), 1e-12, "TFLOP/s"
         what = "fwd+dx+dw"
+    elif wl["kind"] == "bmm":
+        B, M, K, N = wl["batch"], wl["M"], wl["K"], wl["N"]
+        a = (rng.standard_normal((B, M, K)) * K ** -0.5).astype(dt)
+        x, g = rng.standard_normal((B, K, N)).astype(dt), rng.standard_normal((B, M, N)).astype(dt)
+
+        def once():
+            ora.matmul_forward(a, x)
+            ora.matmul_backward(g, a, x, 0)
+            ora.matmul_backward(g, a, x, 1)
+
+        work, scale, unit = 6.0 * B * M * K * N, 1e-12, "TFLOP/s"
+        what = "np.matmul on the two stacks and both gradients"
     elif wl["kind"] == "matmul":
         M, K, N = wl["M"], wl["K"], wl["N"]
         a = (rng.standard_normal((M, K)) * K ** -0.5).astype(dt)
@@ -650,6 +682,16 @@ def run_dropin(name, steps=5):
             (at @ xt).backward(g)
 
         work, scale, unit = 6.0 * M * K * N, 1e-12, "TFLOP/s"
+    elif wl["kind"] == "bmm":
+        B, M, K, N = wl["batch"], wl["M"], wl["K"], wl["N"]
+        a = (rng.standard_normal((B, M, K)) * K ** -0.5).astype(dt)
+        x, g = rng.standard_normal((B, K, N)).astype(dt), rng.standard_normal((B, M, N)).astype(dt)
+
+        def once():
+            at, xt = mg.Tensor(a, copy=False), mg.Tensor(x, copy=False)
+            (at @ xt).backward(g)
+
+        work, scale, unit = 6.0 * B * M * K * N, 1e-12, "TFLOP/s"
     elif wl["kind"] == "permute":
         return {"skipped": "transposition is a building block of einsum here, not an operation of its own"}
     elif wl["kind"] == "einsum":
@@ -807,7 +849,7 @@ def main():
     line = {
         "metric": {"conv": "conv_nd fwd+bwd TFLOP/s", "pool": "max_pool fwd+bwd GB/s",
                    "elem": "relu+multiply+sum fwd+bwd GB/s", "bn": "batchnorm fwd+bwd GB/s",
-                   "repeat": "repeat fwd+bwd GB/s", "matmul": "matmul fwd+bwd TFLOP/s", "window": "sliding-window copy GB/s",
+                   "repeat": "repeat fwd+bwd GB/s", "matmul": "matmul fwd+bwd TFLOP/s", "bmm": "matmul of two stacks fwd+bwd TFLOP/s", "window": "sliding-window copy GB/s",
                    "sumover": "sum over axes GB/s", "scale": "broadcasting multiply GB/s", "permute": "transposition GB/s", "einsum": "einsum fwd+bwd TFLOP/s"}[wl["kind"]],
         "value": res["value"],
         "unit": res["unit"],

@@ -44,9 +44,15 @@ struct BatchedParams {
   long long b_pair, b_row, b_col;    // of op(b): between pairs, along K, along N
 };
 
-template <typename T>
+// AV / BV: op(a) / op(b) is contiguous along K and K is a multiple of the 16-byte piece, so a
+// lane reads a piece of VEC consecutive k at once.  The sum over k may run in any order as long
+// as both operands use the same one: in a block of 4 * VEC values of k, the four lane groups
+// (lane / 16 = q) take k = k0 + VEC * q + s at step s, which makes a lane's VEC steps one piece.
+template <typename T, bool AV, bool BV>
 __global__ void __launch_bounds__(256) batched_product_kernel(BatchedParams p, const T *__restrict__ a, const T *__restrict__ b,
                                                               T *__restrict__ out) {
+  constexpr int VEC = 16 / sizeof(T);
+  typedef T V __attribute__((ext_vector_type(VEC)));
   const int lane = threadIdx.x & 63;
   const long long tile = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);  // the same for a whole wavefront
   if (tile >= p.tiles) return;
@@ -61,12 +67,45 @@ __global__ void __launch_bounds__(256) batched_product_kernel(BatchedParams p, c
   const T *pb = b + pair * p.b_pair + (col_in ? (long long)j * p.b_col : 0);
   typename Tile<T>::Acc acc = {0, 0, 0, 0};
   const int whole = p.K & ~3;
-#pragma unroll 4
-  for (int k0 = 0; k0 < whole; k0 += 4) {
+  int done = 0;
+  if constexpr (AV || BV) {
+    const int blocked = p.K - p.K % (4 * VEC);
+    for (; done < blocked; done += 4 * VEC) {
+      const int k = done + VEC * kk;
+      T av[VEC], bv[VEC];
+      if constexpr (AV) {
+        V v = {};
+        if (row_in) v = *reinterpret_cast<const V *>(pa + k);
+#pragma unroll
+        for (int s = 0; s < VEC; ++s) av[s] = v[s];
+      } else {
+#pragma unroll
+        for (int s = 0; s < VEC; ++s) av[s] = row_in ? pa[(long long)(k + s) * p.a_col] : T(0);
+      }
+      if constexpr (BV) {
+        V v = {};
+        if (col_in) v = *reinterpret_cast<const V *>(pb + k);
+#pragma unroll
+        for (int s = 0; s < VEC; ++s) bv[s] = v[s];
+      } else {
+#pragma unroll
+        for (int s = 0; s < VEC; ++s) bv[s] = col_in ? pb[(long long)(k + s) * p.b_row] : T(0);
+      }
+#pragma unroll
+      for (int s = 0; s < VEC; ++s) acc = Tile<T>::run(av[s], bv[s], acc);
+    }
+  }
+  auto step = [&](int k0) {
     const int k = k0 + kk;
     const T av = row_in ? pa[(long long)k * p.a_col] : T(0);
     const T bv = col_in ? pb[(long long)k * p.b_row] : T(0);
     acc = Tile<T>::run(av, bv, acc);
+  };
+  if constexpr (AV || BV) {
+    for (int k0 = done; k0 < whole; k0 += 4) step(k0);  // at most 4 * VEC - 1 values of k are left
+  } else {
+#pragma unroll 4
+    for (int k0 = 0; k0 < whole; k0 += 4) step(k0);
   }
   if (whole < p.K) {  // the last one to three columns of op(a) / rows of op(b)
     const int k = whole + kk;
@@ -114,10 +153,23 @@ int mg_matmul_batched(int dtype, int64_t batch, int64_t M, int64_t K, int64_t N,
   hipStream_t s = runtime().stream;
   ScopedTiming timed(TAG_BATCHED_PRODUCT);
   const dim3 grid((unsigned)ceil_div(p.tiles, 4)), block(256);
-  if (dtype == MG_F32)
-    hipLaunchKernelGGL(batched_product_kernel<float>, grid, block, 0, s, p, (const float *)a, (const float *)b, (float *)out);
-  else
-    hipLaunchKernelGGL(batched_product_kernel<double>, grid, block, 0, s, p, (const double *)a, (const double *)b, (double *)out);
+  // 16-byte pieces along K: the operand is contiguous there, K is a whole number of pieces (so
+  // every row starts on one) and the stack itself is aligned
+  const int vec = dtype == MG_F32 ? 4 : 2;
+  const bool av = p.a_col == 1 && K % vec == 0 && reinterpret_cast<uintptr_t>(a) % 16 == 0;
+  const bool bv = p.b_row == 1 && K % vec == 0 && reinterpret_cast<uintptr_t>(b) % 16 == 0;
+#define MG_BATCHED(T, AV, BV) \
+  hipLaunchKernelGGL((batched_product_kernel<T, AV, BV>), grid, block, 0, s, p, (const T *)a, (const T *)b, (T *)out)
+#define MG_BATCHED_T(T)                 \
+  do {                                  \
+    if (av && bv) MG_BATCHED(T, true, true);        \
+    else if (av) MG_BATCHED(T, true, false);        \
+    else if (bv) MG_BATCHED(T, false, true);        \
+    else MG_BATCHED(T, false, false);               \
+  } while (0)
+  if (dtype == MG_F32) MG_BATCHED_T(float); else MG_BATCHED_T(double);
+#undef MG_BATCHED_T
+#undef MG_BATCHED
   MG_HIP(hipGetLastError());
   return MG_OK;
 }

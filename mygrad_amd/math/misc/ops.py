@@ -24,9 +24,9 @@ __all__ = ["MatMul"]
 # Two stacks are multiplied pair by pair on the tiled kernels when a pair has more than this
 # many floating-point operations (it then fills the device by itself), else in one launch of the
 # kernel that gives every 16 x 16 tile of every product a wavefront.  Measured on float32 squares:
-# that kernel sustains 16-18 TFLOP/s from 128^3 up, a launch of the tiled kernels costs 8-12 us,
-# so the two meet near 450^3 per pair.
-SMALL_PAIR_FLOPS = 2 * 384**3
+# that kernel sustains 36-49 TFLOP/s from 128^3 up, a launch of the tiled kernels costs 8-12 us
+# and reaches 55 TFLOP/s at 1024^3, where the two meet.
+SMALL_PAIR_FLOPS = 2 * 768**3
 
 
 def _prod(shape):

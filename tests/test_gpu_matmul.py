@@ -127,7 +127,7 @@ SHAPES = [
     ((4,), (2, 3, 4, 5)),
     ((2, 3, 4), (4,)),
     ((2, 2, 30, 40), (2, 2, 40, 50)),
-    ((2, 400, 410), (2, 410, 390)),  # pairs large enough for a launch of the tiled kernels each
+    ((2, 800, 810), (2, 810, 790)),  # pairs large enough for a launch of the tiled kernels each
     ((60, 70), (70, 80)),
     # stacks that broadcast against each other
     ((2, 1, 3, 4), (2, 4, 5)),
