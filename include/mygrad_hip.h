@@ -228,6 +228,19 @@ int mg_relu_bwd_mask(int dtype, int64_t n, const void *mask, const void *grad, v
  * src/mygrad/math/sequential/ops.py:120-121; src/mygrad/operation_base.py Sequential). */
 int mg_sum_all(int dtype, int64_t n, const void *x, void *out);
 
+/* mg_sum_all for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc); it has no counterpart in the reference.  Same
+ * kernels, same chunking, the same result bit for bit, but the chunk sums go to a fixed 32 KiB
+ * array in the library's device image (resolved per device by mg_init) instead of the library's
+ * growing workspace, and no timing events are recorded: the call allocates nothing on the host
+ * side of HIP or on the device.  n above MG_SUM_STATIC_MAX_N is refused (MG_ERR_UNSUPPORTED).
+ * Every call on a device shares that device's array: calls that overlap on one device (two
+ * host threads are serialised by the library's lock, but two processes' or streams' kernels
+ * are not) race.  Nothing needs clearing between calls: each call writes every chunk sum it
+ * reads. */
+#define MG_SUM_STATIC_MAX_N ((int64_t)1 << 31)
+int mg_sum_all_static(int dtype, int64_t n, const void *x, void *out);
+
 /* out[i] = *value (one element on the device).  Replaces Sum.backward_var with axis=None
  * (np.full(a.shape, grad), sequential/ops.py:123-126). */
 int mg_fill_from(int dtype, int64_t n, const void *value, void *out);

@@ -152,6 +152,7 @@ _SIGNATURES = {
     "mg_relu_fwd_mask": [ctypes.c_int, ctypes.c_int64, _vp, _vp, _vp],
     "mg_relu_bwd_mask": [ctypes.c_int, ctypes.c_int64, _vp, _vp, _vp],
     "mg_sum_all": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
+    "mg_sum_all_static": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
     "mg_fill_from": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
     "mg_sum_over": [ctypes.c_int] + [ctypes.c_int64] * 3 + [ctypes.c_int, _vp, _vp],
     "mg_sum_product_over": [ctypes.c_int] + [ctypes.c_int64] * 3 + [ctypes.c_int, _vp, _vp, _vp],

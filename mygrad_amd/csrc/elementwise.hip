@@ -292,7 +292,70 @@ int launch_relu_mask(int dtype, int64_t n, const void *in, void *out, void *mask
   return MG_OK;
 }
 
+// How mg_sum_all cuts x: chunks of 128 KiB, at most 4096 of them (then the chunks grow); a
+// function of n and the element size only, so that the order of the additions is too.
+struct SumChunking {
+  long long chunk, chunks;
+};
+SumChunking sum_chunking(int dtype, int64_t n) {
+  const long long elem = dtype == MG_F32 ? 4 : 8;
+  const long long vec = 16 / elem;
+  long long chunk = (128 * 1024) / elem;
+  long long chunks = std::max<long long>(1, ceil_div(n, chunk));
+  if (chunks > 4096) {
+    chunk = ceil_div(ceil_div(n, 4096), vec) * vec;
+    chunks = ceil_div(n, chunk);
+  }
+  return {chunk, chunks};
+}
+
+int check_sum_all(int dtype, int64_t n, const void *x, const void *out, const char *who) {
+  if (int rc = check_elementwise(dtype, n, who)) return rc;
+  if (!out || (n > 0 && !x)) return fail(MG_ERR_BAD_ARG, "null pointer in %s", who);
+  if (misaligned(x)) return fail(MG_ERR_BAD_ARG, "%s: x must be 16-byte aligned", who);
+  return MG_OK;
+}
+
+// The two kernels of the whole-array sum; `partial` holds one double per chunk.
+int launch_sum_all(int dtype, int64_t n, const void *x, void *out, double *partial) {
+  hipStream_t s = runtime().stream;
+  const SumChunking c = sum_chunking(dtype, n);
+  if (dtype == MG_F32) {
+    hipLaunchKernelGGL(sum_chunks_kernel<float>, dim3((unsigned)c.chunks), dim3(256), 0, s, (const float *)x, (long long)n, c.chunk,
+                       partial);
+    hipLaunchKernelGGL(sum_final_kernel<float>, dim3(1), dim3(256), 0, s, (const double *)partial, (int)c.chunks, (float *)out);
+  } else {
+    hipLaunchKernelGGL(sum_chunks_kernel<double>, dim3((unsigned)c.chunks), dim3(256), 0, s, (const double *)x, (long long)n, c.chunk,
+                       partial);
+    hipLaunchKernelGGL(sum_final_kernel<double>, dim3(1), dim3(256), 0, s, (const double *)partial, (int)c.chunks, (double *)out);
+  }
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
 }  // namespace
+
+// Chunk sums of mg_sum_all_static: device memory that belongs to the code object, so that entry
+// point needs no allocation.  Every device the library runs on holds its own copy at its own
+// address; the array's name is only a host-side handle for hipGetSymbolAddress, the kernels get
+// the resolved pointer.  Every chunk sum a call reads is written by that call first, so nothing
+// has to be cleared between calls; two calls that overlap on one device would race on it.
+constexpr int kStaticChunks = 4096;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) double scratch[kStaticChunks];
+static double *scratch_ptr[kMaxDevices];
+
+// Called by mg_init with `device` current: looks up where this device keeps `scratch`.
+int resolve_static_scratch(int device) {
+  if (device < 0 || device >= kMaxDevices) return fail(MG_ERR_UNSUPPORTED, "device index %d beyond the %d this library keeps scratch pointers for", device, kMaxDevices);
+  if (scratch_ptr[device]) return MG_OK;
+  double *ptr = nullptr;
+  MG_HIP(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+  if (!ptr) return fail(MG_ERR_HIP, "hipGetSymbolAddress returned a null address for the static scratch array");
+  scratch_ptr[device] = ptr;
+  return MG_OK;
+}
+
 }  // namespace mg
 
 using namespace mg;
@@ -401,33 +464,26 @@ int mg_multiply_broadcast(int dtype, int nd, const int64_t *shape, const int64_t
 int mg_sum_all(int dtype, int64_t n, const void *x, void *out) {
   std::lock_guard<std::recursive_mutex> guard(api_mutex());
   MG_REQUIRE_INIT();
-  if (int rc = check_elementwise(dtype, n, "mg_sum_all")) return rc;
-  if (!out || (n > 0 && !x)) return fail(MG_ERR_BAD_ARG, "null pointer in mg_sum_all");
-  if (misaligned(x)) return fail(MG_ERR_BAD_ARG, "mg_sum_all: x must be 16-byte aligned");
-  hipStream_t s = runtime().stream;
-  const size_t elem = dtype == MG_F32 ? 4 : 8;
-  // chunks of 128 KiB, at most 4096 of them (then the chunks grow): a function of n only
-  const long long vec = (long long)(16 / elem);
-  long long chunk = (128 * 1024) / (long long)elem;
-  long long chunks = std::max<long long>(1, ceil_div(n, chunk));
-  if (chunks > 4096) {
-    chunk = ceil_div(ceil_div(n, 4096), vec) * vec;
-    chunks = ceil_div(n, chunk);
-  }
+  if (int rc = check_sum_all(dtype, n, x, out, "mg_sum_all")) return rc;
   void *partial = nullptr;
-  if (int rc = workspace((size_t)chunks * sizeof(double), &partial)) return rc;
+  if (int rc = workspace((size_t)sum_chunking(dtype, n).chunks * sizeof(double), &partial)) return rc;
   ScopedTiming timed(TAG_REDUCE_ALL);
-  if (dtype == MG_F32) {
-    hipLaunchKernelGGL(sum_chunks_kernel<float>, dim3((unsigned)chunks), dim3(256), 0, s, (const float *)x, (long long)n, chunk,
-                       (double *)partial);
-    hipLaunchKernelGGL(sum_final_kernel<float>, dim3(1), dim3(256), 0, s, (const double *)partial, (int)chunks, (float *)out);
-  } else {
-    hipLaunchKernelGGL(sum_chunks_kernel<double>, dim3((unsigned)chunks), dim3(256), 0, s, (const double *)x, (long long)n, chunk,
-                       (double *)partial);
-    hipLaunchKernelGGL(sum_final_kernel<double>, dim3(1), dim3(256), 0, s, (const double *)partial, (int)chunks, (double *)out);
-  }
-  MG_HIP(hipGetLastError());
-  return MG_OK;
+  return launch_sum_all(dtype, n, x, out, (double *)partial);
+}
+
+int mg_sum_all_static(int dtype, int64_t n, const void *x, void *out) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (int rc = check_sum_all(dtype, n, x, out, "mg_sum_all_static")) return rc;
+  if (n > MG_SUM_STATIC_MAX_N)
+    return fail(MG_ERR_UNSUPPORTED, "mg_sum_all_static: n = %lld exceeds the %lld elements its fixed scratch array is sized for",
+                (long long)n, (long long)MG_SUM_STATIC_MAX_N);
+  const int device = runtime().device;
+  double *partial = device >= 0 && device < kMaxDevices ? scratch_ptr[device] : nullptr;
+  if (!partial) return fail(MG_ERR_NOT_INIT, "mg_sum_all_static: the scratch array was not resolved on device %d", device);
+  if (sum_chunking(dtype, n).chunks > kStaticChunks) return fail(MG_ERR_UNSUPPORTED, "mg_sum_all_static: more chunks than the scratch array holds");
+  // no timing events here: creating them allocates
+  return launch_sum_all(dtype, n, x, out, partial);
 }
 
 int mg_fill_from(int dtype, int64_t n, const void *value, void *out) {

@@ -74,6 +74,10 @@ struct ScopedTiming {
 // Drops every cached convolution plan (device tables); called by mg_shutdown.
 void release_conv_plans();
 
+// Looks up the address of the file-scope device array behind mg_sum_all_static on `device`,
+// which must be the current device; called once per device by mg_init.
+int resolve_static_scratch(int device);
+
 #define MG_HIP(expr)                                                   \
   do {                                                                 \
     hipError_t mg_err_ = (expr);                                       \

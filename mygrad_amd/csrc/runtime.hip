@@ -234,6 +234,7 @@ int mg_init(int device) {
   if (strncmp(rt.props.gcnArchName, "gfx950", 6) != 0)
     return fail(MG_ERR_NO_DEVICE, "device %d is %s; this library carries gfx950 code only", device,
                 rt.props.gcnArchName);
+  if (int rc = resolve_static_scratch(device)) return rc;
   MG_HIP(hipStreamCreateWithFlags(&rt.stream, hipStreamNonBlocking));
   {
     const char *flag = getenv("MYGRAD_HIP_POOL");
