@@ -16,7 +16,9 @@ the C ABI of libmygrad_hip.so.  The script prints ONE JSON line:
                    on the library stream inside the timed region;
 * ``cpu_baseline`` the NumPy restatement of the reference algorithm timed on the
                    host cores on a bounded sample of the same workload;
-* ``secondary``    (with --all) the same figures for the other workloads.
+* ``secondary``    the same figures for the hot path's other configurations (the max_pool
+                   half of the metric and the other convolution shapes; every workload
+                   with --all, none with --no-secondary).
 
 Algorithmic work:  convolution 2*N*F*prod(G)*C*prod(W) flops per pass (padding
 taps count, dense definition); pooling |x|+|out| bytes forward and
@@ -84,6 +86,8 @@ WORKLOADS = {
     "win3a": dict(kind="window", dtype="f32", seed=1010, x=(32, 64, 56, 56), window=(3, 3), step=(1, 1), dilation=(1, 1)),
 }
 NP_DTYPE = {"f32": np.float32, "f64": np.float64}
+# the configurations of the hot path itself: reported by every default run
+HOT_PATH = ["conv3a", "conv3b", "conv4", "conv5", "conv1", "pool2", "pool5", "pool2-recompute", "pool5-recompute"]
 
 
 def conv_grid(wl):
@@ -822,7 +826,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="conv3a", choices=sorted(WORKLOADS))
-    ap.add_argument("--all", action="store_true", help="also run every other workload (reported under 'secondary')")
+    ap.add_argument("--all", action="store_true",
+                    help="report every other workload under 'secondary', not only the hot path's other configurations")
+    ap.add_argument("--no-secondary", action="store_true", help="run the one workload only")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--dropin", action="store_true",
                     help="also time the step through the Python drop-in API (reported under 'dropin', never as value)")
@@ -871,16 +877,20 @@ def main():
         line["cpu_baseline"] = run_cpu_baseline(args.workload)
     if args.dropin:
         line["dropin"] = run_dropin(args.workload)
-    if args.all:
+    if not args.no_secondary:
+        # the other half of the metric (max_pool GB/s) and the other convolution configurations,
+        # each with its own roofline and a short CPU baseline
+        names = list(WORKLOADS) if args.all else HOT_PATH
         secondary = {}
-        for name in WORKLOADS:
+        for name in names:
             if name == args.workload:
                 continue
             r = run_gpu(name, args.steps, args.warmup)
             entry = {"config": describe(name), "value": r["value"], "unit": r["unit"], "dtype": WORKLOADS[name]["dtype"],
-                     "ms_per_step": r["ms_per_step"], "roofline": r["roofline"], "kernels": r["kernels"]}
+                     "ms_per_step": r["ms_per_step"], "kernel_ms_per_step": r["kernel_ms_per_step"], "roofline": r["roofline"],
+                     "kernels": r["kernels"]}
             if not args.no_cpu_baseline:
-                entry["cpu_baseline"] = run_cpu_baseline(name)
+                entry["cpu_baseline"] = run_cpu_baseline(name, min_seconds=2.0)
             if args.dropin:
                 entry["dropin"] = run_dropin(name)
             secondary[name] = entry
