@@ -653,14 +653,25 @@ def run_cpu_baseline(name, min_seconds=10.0, max_reps=200):
 
 
 def run_dropin(name, steps=5):
-    """Wall time of the same step through the drop-in API (host arrays in, host arrays
-    out): includes the ctypes calls, uploads over PCIe and the download of every result."""
+    """Wall time of the same step through the drop-in API (conv_nd / max_pool / ... called on
+    tensors, gradients through Tensor.backward()), two ways:
+
+    ``resident``  inputs are device tensors (uploaded once), nothing is read during the loop;
+                  the gradients are read once after the last step (``read_back_ms``).  Next to
+                  it the kernel time of the same loop from the library's HIP events.
+    ``host``      host ndarrays in and every gradient read on the host after every step: the
+                  PCIe-inclusive figure.
+    Neither is ever ``value``."""
     import mygrad_amd as mg
+    from mygrad_amd import _hip
     from mygrad_amd.nnet import conv_nd, max_pool
 
     wl, dt = WORKLOADS[name], NP_DTYPE[WORKLOADS[name]["dtype"]]
     rng = np.random.default_rng(wl["seed"])
     x = rng.standard_normal(wl["x"]).astype(dt) if "x" in wl else None
+    chain = None
+    # every branch defines once(T, C): T wraps an input that takes a gradient, C a constant one
+    # (both return tensors); it runs one step and returns the tensors whose gradients it left
     if wl["kind"] == "conv":
         w = (rng.standard_normal(wl["w"]) * wl["wscale"]).astype(dt)
         g = rng.standard_normal((wl["x"][0], wl["w"][0], *conv_grid(wl))).astype(dt)
@@ -668,22 +679,32 @@ def run_dropin(name, steps=5):
                     for xx, t, s, p, d in zip(wl["x"][2:], wl["w"][2:], wl["stride"], wl["padding"], wl["dilation"]))
         if not valid:
             return {"skipped": "the reference's validator rejects this shape; the drop-in raises ValueError like it"}
+        conf = dict(stride=wl["stride"], padding=wl["padding"], dilation=wl["dilation"])
 
-        def once():
-            xt, wt = mg.Tensor(x, copy=False), mg.Tensor(w, copy=False)
-            out = conv_nd(xt, wt, stride=wl["stride"], padding=wl["padding"], dilation=wl["dilation"])
-            out.backward(g)
+        def once(T, C):
+            xt, wt = T(x), T(w)
+            conv_nd(xt, wt, **conf).backward(C(g))
+            return xt, wt
 
         work, scale, unit = 3 * conv_flops_per_pass(wl), 1e-12, "TFLOP/s"
+        if name == "conv5":
+            # the whole of configuration 5: conv -> max_pool (2,2,2) -> loss = sum(pool_out * g)
+            g5 = rng.standard_normal((wl["x"][0], wl["w"][0], *(n // 2 for n in conv_grid(wl)))).astype(dt)
+
+            def chain(T, C):
+                xt, wt = T(x), T(w)
+                mg.sum(max_pool(conv_nd(xt, wt, **conf), (2, 2, 2), 2) * C(g5)).backward()
+                return xt, wt
     elif wl["kind"] == "matmul":
         M, K, N = wl["M"], wl["K"], wl["N"]
         a = (rng.standard_normal((M, K)) * K ** -0.5).astype(dt)
         x = rng.standard_normal((K, N)).astype(dt)
         g = rng.standard_normal((M, N)).astype(dt)
 
-        def once():
-            at, xt = mg.Tensor(a, copy=False), mg.Tensor(x, copy=False)
-            (at @ xt).backward(g)
+        def once(T, C):
+            at, xt = T(a), T(x)
+            (at @ xt).backward(C(g))
+            return at, xt
 
         work, scale, unit = 6.0 * M * K * N, 1e-12, "TFLOP/s"
     elif wl["kind"] == "bmm":
@@ -691,9 +712,10 @@ def run_dropin(name, steps=5):
         a = (rng.standard_normal((B, M, K)) * K ** -0.5).astype(dt)
         x, g = rng.standard_normal((B, K, N)).astype(dt), rng.standard_normal((B, M, N)).astype(dt)
 
-        def once():
-            at, xt = mg.Tensor(a, copy=False), mg.Tensor(x, copy=False)
-            (at @ xt).backward(g)
+        def once(T, C):
+            at, xt = T(a), T(x)
+            (at @ xt).backward(C(g))
+            return at, xt
 
         work, scale, unit = 6.0 * B * M * K * N, 1e-12, "TFLOP/s"
     elif wl["kind"] == "permute":
@@ -704,40 +726,51 @@ def run_dropin(name, steps=5):
         sizes = {**dict(zip(la, wl["x"])), **dict(zip(lb, wl["w"]))}
         g = rng.standard_normal(tuple(sizes[l] for l in lo)).astype(dt)
 
-        def once():
-            mg.einsum(f"{la},{lb}->{lo}", mg.Tensor(x, copy=False), mg.Tensor(w, copy=False)).backward(g)
+        def once(T, C):
+            xt, wt = T(x), T(w)
+            mg.einsum(f"{la},{lb}->{lo}", xt, wt).backward(C(g))
+            return xt, wt
 
         work, scale, unit = 6.0 * np.prod([float(v) for v in sizes.values()]), 1e-12, "TFLOP/s"
     elif wl["kind"] == "sumover":
 
-        def once():
-            for axes in wl["axes"]:
-                mg.sum(mg.Tensor(x, copy=False), axis=axes).clear_graph()
+        def once(T, C):
+            outs = [mg.sum(C(x), axis=axes) for axes in wl["axes"]]
+            for out in outs:
+                out.clear_graph()
+            return ()
 
         work, scale, unit = 2 * x.nbytes, 1e-9, "GB/s"
     elif wl["kind"] == "scale":
         others = [rng.standard_normal(shape).astype(dt) for shape in wl["others"]]
 
-        def once():
+        def once(T, C):
             for other in others:
-                (mg.Tensor(x, copy=False) * mg.Tensor(other, copy=False)).clear_graph()
+                (C(x) * C(other)).clear_graph()
+            return ()
 
         work, scale, unit = 4 * x.nbytes, 1e-9, "GB/s"
     elif wl["kind"] == "repeat":
         g = rng.standard_normal((*wl["x"][:-1], wl["x"][-1] * wl["repeats"])).astype(dt)
+        seeds = {}
 
-        def once():
+        def once(T, C):
+            leaves = []
             for axis in wl["axes"]:
-                xt = mg.Tensor(x, copy=False)
+                xt = T(x)
                 out = mg.repeat(xt, wl["repeats"], axis)
-                out.backward(g.reshape(out.shape))
+                seeds.setdefault(axis, np.ascontiguousarray(g.reshape(out.shape)))
+                out.backward(C(seeds[axis]))
+                leaves.append(xt)
+            return leaves[-1:]
 
         work, scale, unit = 4 * (x.nbytes + g.nbytes), 1e-9, "GB/s"
     elif wl["kind"] == "window":
         count = int(np.prod(mg.sliding_window_view(x, wl["window"], wl["step"], wl["dilation"]).shape))
 
-        def once():
+        def once(T, C):
             mg.sliding_window_copy(x, wl["window"], wl["step"], wl["dilation"])
+            return ()
 
         work, scale, unit = x.nbytes + count * x.itemsize, 1e-9, "GB/s"
     elif wl["kind"] == "bn":
@@ -747,9 +780,10 @@ def run_dropin(name, steps=5):
         gamma = rng.uniform(0.5, 2, wl["x"][1]).astype(dt)
         beta = rng.standard_normal(wl["x"][1]).astype(dt)
 
-        def once():
-            xt, gt, bt = mg.Tensor(x, copy=False), mg.Tensor(gamma, copy=False), mg.Tensor(beta, copy=False)
-            batchnorm(xt, gamma=gt, beta=bt, eps=wl["eps"]).backward(g)
+        def once(T, C):
+            xt, gt, bt = T(x), T(gamma), T(beta)
+            batchnorm(xt, gamma=gt, beta=bt, eps=wl["eps"]).backward(C(g))
+            return xt, gt, bt
 
         work, scale, unit = 5 * x.nbytes, 1e-9, "GB/s"
     elif wl["kind"] == "elem":
@@ -757,9 +791,10 @@ def run_dropin(name, steps=5):
 
         g = rng.standard_normal(wl["x"]).astype(dt)
 
-        def once():
-            xt, gt = mg.Tensor(x, copy=False), mg.Tensor(g, copy=False)
+        def once(T, C):
+            xt, gt = T(x), T(g)
             mg.sum(relu(xt) * gt).backward()
+            return xt, gt
 
         work, scale, unit = elem_bytes(x), 1e-9, "GB/s"
     else:
@@ -768,19 +803,70 @@ def run_dropin(name, steps=5):
         if any((xx - p) % s for xx, p, s in zip(pooled, wl["pool"], wl["stride"])):
             return {"skipped": "the reference's validator rejects this shape; the drop-in raises ValueError like it"}
 
-        def once():
-            xt = mg.Tensor(x, copy=False)
-            out = max_pool(xt, wl["pool"], wl["stride"])
-            out.backward(g)
+        def once(T, C):
+            xt = T(x)
+            max_pool(xt, wl["pool"], wl["stride"]).backward(C(g))
+            return (xt,)
 
         work, scale, unit = 3 * x.nbytes + 2 * g.nbytes, 1e-9, "GB/s"
-    once()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        once()
-    elapsed = (time.perf_counter() - t0) / steps
-    return {"ms_per_step": elapsed * 1e3, "value": float(work * scale / elapsed), "unit": unit,
-            "note": "through Tensor.backward(), host ndarrays in and out (PCIe included)"}
+
+    def measure(step):
+        def read(leaves):
+            for t in leaves:
+                t.grad
+
+        # host arrays in, gradients read every step
+        host_T = lambda a: mg.Tensor(a, copy=False)
+        host_C = lambda a: mg.Tensor(a, copy=False, constant=True)
+        read(step(host_T, host_C))
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            read(step(host_T, host_C))
+        host_ms = (time.perf_counter() - t0) / steps * 1e3
+        if wl["kind"] == "window":
+            return {"host": {"ms_per_step": host_ms, "note": "host ndarray in, host ndarray out"}}
+
+        # device tensors in, nothing read until the loop is over
+        held = {}
+
+        def dev_T(a, constant=None):
+            if id(a) not in held:
+                held[id(a)] = (a, mg.device_tensor(a, constant=constant))
+            return held[id(a)][1]
+
+        dev_C = lambda a: dev_T(a, constant=True)
+        many = max(steps, 20)
+        step(dev_T, dev_C)
+        _hip.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(many):
+            leaves = step(dev_T, dev_C)
+        _hip.synchronize()
+        wall_ms = (time.perf_counter() - t0) / many * 1e3
+        t0 = time.perf_counter()
+        read(leaves)
+        read_ms = (time.perf_counter() - t0) * 1e3
+        _hip.timing_enable(True)
+        for _ in range(many):
+            step(dev_T, dev_C)
+        _hip.synchronize()
+        kernel_ms = sum(ms for _, ms in _hip.timing_read()) / many
+        _hip.timing_enable(False)
+        return {
+            "resident": {"ms_per_step": wall_ms, "kernel_ms_per_step": kernel_ms, "over_kernels": wall_ms / kernel_ms if kernel_ms else None,
+                         "read_back_ms": read_ms, "steps": many,
+                         "note": "device tensors in, Tensor.backward() every step, gradients read once after the last step"},
+            "host": {"ms_per_step": host_ms, "note": "host ndarrays in, every gradient read on the host after every step (PCIe included)"},
+        }
+
+    result = measure(once)
+    for entry in result.values():
+        entry["value"] = float(work * scale / (entry["ms_per_step"] * 1e-3))
+        entry["unit"] = unit
+    if chain is not None:
+        result["chain"] = measure(chain)
+        result["chain"]["what"] = "conv_nd -> max_pool((2,2,2), 2) -> sum(pool_out * g) and backward()"
+    return result
 
 
 def run_copy_calibration(mib=1024, reps=20):

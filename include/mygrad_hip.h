@@ -245,6 +245,24 @@ int mg_sum_all_static(int dtype, int64_t n, const void *x, void *out);
  * (np.full(a.shape, grad), sequential/ops.py:123-126). */
 int mg_fill_from(int dtype, int64_t n, const void *value, void *out);
 
+/* ---- gradient bookkeeping between operations, on the device ----
+ * What Operation.backward does to a gradient that backward_var returned before it becomes, or
+ * joins, var.grad (src/mygrad/operation_base.py:216-228), and how Tensor.backward seeds the
+ * terminal tensor (src/mygrad/tensor_base.py:1308-1334), for gradients that never leave the
+ * device.  Buffers from mg_malloc (32-byte aligned for the first two). */
+
+/* out[i] = (to_dtype) x[i]: `backed.astype(var.dtype)`, operation_base.py:223-224 (the float64
+ * gradient of a float32 max_pool input, pooling.py:147). */
+int mg_cast(int from_dtype, int to_dtype, int64_t n, const void *x, void *out);
+
+/* acc[i] = (acc_dtype)(acc[i] + inc[i]), the sum formed in the wider of the two types:
+ * `var._grad += backed`, operation_base.py:227-228, with NumPy's rule for a narrower `acc`. */
+int mg_accumulate(int acc_dtype, int inc_dtype, int64_t n, void *acc, const void *inc);
+
+/* out[i] = value: `np.full_like(self.data, fill_value=1.0)`, the seed of Tensor.backward()
+ * without an argument, tensor_base.py:1330-1334. */
+int mg_fill_value(int dtype, int64_t n, double value, void *out);
+
 /* ---- batch normalisation ---- */
 
 /* mean[c], var[c] = mean and (biased) variance of x[:, c, ...]; y = (x - mean) /

@@ -17,7 +17,7 @@ from ._hip import HipError, HipUnavailable, device_info, is_available, synchroni
 from .errors import InvalidBackprop, InvalidGradient, SkipGradient
 from .nnet.layers.utils import sliding_window_copy, sliding_window_view
 from .operation_base import Operation
-from .tensor_base import Tensor, asarray, tensor
+from .tensor_base import Tensor, asarray, device_tensor, tensor
 from .math import matmul, multi_matmul, multiply, sum  # noqa: A004  (after tensor_base: the ops import Tensor)
 from .tensor_manip import repeat
 from .linalg import einsum
@@ -29,6 +29,7 @@ execute_op = Tensor._op
 __all__ = [
     "Tensor",
     "tensor",
+    "device_tensor",
     "asarray",
     "Operation",
     "execute_op",

@@ -15,6 +15,14 @@ than once, every array that enters or leaves an op keeps its device copy (its
 A mirror is dropped when the graph releases its lock on the host array (the host
 copy may change from then on), when the host array is garbage collected, or
 explicitly via :func:`evict`.
+
+Under the package's own ``Tensor`` no result crosses PCIe until somebody reads it:
+while :func:`deferring` is active, :func:`download` hands back a :class:`DeviceArray`
+-- shape, dtype and the device buffer -- instead of copying, ``Tensor.data`` /
+``Tensor.grad`` turn it into a host array on first read, and operations take such
+values from :func:`to_device` without any copy.  Called directly (or from another
+caller of the Operation contract) the operations return host arrays as the contract
+says.
 """
 
 import ctypes
@@ -25,7 +33,11 @@ import numpy as np
 from . import _hip
 
 __all__ = [
+    "DeviceArray",
     "DeviceBuffer",
+    "deferring",
+    "full",
+    "value_of",
     "pinned_empty",
     "to_device",
     "attach",
@@ -108,10 +120,158 @@ def pinned_empty(shape, dtype):
     return np.ndarray(shape, dtype=dtype, buffer=raw)  # .base is `raw` itself, not a view chain
 
 
+# --------------------------------------------------------------------------- results kept on the device
+_defer = 0
+
+
+class deferring:
+    """While active, :func:`download` returns :class:`DeviceArray` objects instead of copying
+    results to the host (the package's ``Tensor`` wraps its calls of an operation in it)."""
+
+    def __enter__(self):
+        global _defer
+        _defer += 1
+        return self
+
+    def __exit__(self, *exc):
+        global _defer
+        _defer -= 1
+        return False
+
+
+class _Flags(dict):
+    c_contiguous = True
+    writeable = False
+
+
+_DEVICE_FLAGS = _Flags(C_CONTIGUOUS=True, WRITEABLE=False)
+
+
+def _resolve_shape(size, shape):
+    """``shape`` with a single -1 filled in, checked against ``size`` like ndarray.reshape."""
+    shape = [int(n) for n in shape]
+    known = 1
+    for n in shape:
+        if n != -1:
+            known *= n
+    if shape.count(-1) == 1 and known and size % known == 0:
+        shape[shape.index(-1)] = size // known
+        known = size
+    if -1 in shape or known != size:
+        raise ValueError(f"cannot reshape array of size {size} into shape {tuple(shape)}")
+    return tuple(shape)
+
+
+class DeviceArray:
+    """A C-contiguous array that so far exists on the device only: shape, dtype and the
+    buffer a kernel wrote.  It answers the questions operations ask of an input before
+    launching (``shape``, ``dtype``, ``ndim``, ``size``, ``nbytes``, ``reshape``) without
+    touching the data; :meth:`host` copies it into pinned host memory, once.
+
+    ``base`` is the array whose buffer this one shares (a reshape), None for the owner of
+    a buffer -- the rule ``Operation.backward`` uses to decide whether a gradient must be
+    copied before it may be updated in place.
+    """
+
+    __slots__ = ("buf", "shape", "dtype", "base", "_host", "__weakref__")
+    flags = _DEVICE_FLAGS
+
+    def __init__(self, buf, shape, dtype, base=None):
+        self.buf = buf
+        self.shape = tuple(int(n) for n in shape)
+        self.dtype = np.dtype(dtype)
+        self.base = base
+        self._host = None
+
+    @property
+    def ndim(self):
+        return len(self.shape)
+
+    @property
+    def size(self):
+        return int(np.prod(self.shape, dtype=np.int64))
+
+    @property
+    def itemsize(self):
+        return self.dtype.itemsize
+
+    @property
+    def nbytes(self):
+        return self.size * self.dtype.itemsize
+
+    def reshape(self, *shape):
+        if len(shape) == 1 and not isinstance(shape[0], (int, np.integer)):
+            shape = tuple(shape[0])
+        shape = _resolve_shape(self.size, shape)
+        return DeviceArray(self.buf, shape, self.dtype, base=self if self.base is None else self.base)
+
+    def host(self):
+        """The values as a (pinned) host array; copied on the first call."""
+        if self._host is None:
+            out = pinned_empty(self.shape, self.dtype)
+            if self.size:
+                self.buf.download_into(out)
+            self._host = out
+        return self._host
+
+    def __array__(self, dtype=None, copy=None):
+        out = self.host()
+        if dtype is not None and np.dtype(dtype) != out.dtype:
+            return out.astype(dtype)
+        return out.copy() if copy else out
+
+    def copy(self):
+        """A new array with a buffer of its own (device-to-device copy)."""
+        buf = DeviceBuffer(max(self.nbytes, 16))
+        if self.nbytes:
+            _hip.check(_hip.lib().mg_memcpy_d2d(buf.ptr, self.buf.ptr, self.nbytes))
+        return DeviceArray(buf, self.shape, self.dtype)
+
+    def astype(self, dtype):
+        """The values cast to float32 / float64 on the device (a new buffer)."""
+        dtype = np.dtype(dtype)
+        if dtype == self.dtype:
+            return self
+        buf = DeviceBuffer(max(self.size * dtype.itemsize, 16))
+        _hip.check(_hip.lib().mg_cast(_hip.dtype_code(self.dtype), _hip.dtype_code(dtype), self.size, self.buf.ptr, buf.ptr))
+        return DeviceArray(buf, self.shape, dtype)
+
+    def add_into(self, other):
+        """``self += other`` on the device, with NumPy's rule for a narrower ``self`` (the sum is
+        formed in the wider type and rounded once).  ``self`` must own its buffer and must not
+        have been copied to the host yet."""
+        assert self.base is None and self._host is None and other.shape == self.shape
+        _hip.check(_hip.lib().mg_accumulate(_hip.dtype_code(self.dtype), _hip.dtype_code(other.dtype), self.size,
+                                            self.buf.ptr, other.buf.ptr))
+
+    def __repr__(self):
+        return f"DeviceArray(shape={self.shape}, dtype={self.dtype})"
+
+
+def value_of(tensor):
+    """What an operation works on: the tensor's DeviceArray while its values exist on the
+    device only, else its host array (``tensor.data``; a tensor class other than this
+    package's has nothing else)."""
+    try:
+        return tensor._value
+    except AttributeError:
+        return tensor.data
+
+
+def full(shape, dtype, value):
+    """``np.full(shape, value, dtype)`` made on the device."""
+    dtype = np.dtype(dtype)
+    count = int(np.prod(shape, dtype=np.int64))
+    buf = DeviceBuffer(max(count * dtype.itemsize, 16))
+    _hip.check(_hip.lib().mg_fill_value(_hip.dtype_code(dtype), count, float(value), buf.ptr))
+    return DeviceArray(buf, shape, dtype)
+
+
 # --------------------------------------------------------------------------- mirrors
 _mirrors = {}  # key -> DeviceBuffer, for arrays the graph holds read-only
 _transient = {}  # key -> DeviceBuffer, for gradients in flight during one backward()
 _locked = {}  # key -> number of graph locks on that memory
+_pending = {}  # key -> DeviceBuffer offered by the last attach(), a mirror once the array is locked
 
 
 def _key(arr):
@@ -130,6 +290,13 @@ def note_locked(arr):
     """The graph now holds ``arr`` read-only: its mirror may be cached."""
     key = _key(arr)
     _locked[key] = _locked.get(key, 0) + 1
+    offered = _pending.pop(key, None)
+    if offered is not None:
+        _mirrors[key] = offered
+        try:
+            weakref.finalize(_root(arr), _evict_key, key)
+        except TypeError:  # owner not weak-referenceable: do not cache
+            _mirrors.pop(key, None)
 
 
 def note_released(arr):
@@ -145,8 +312,9 @@ def note_released(arr):
 
 def is_locked(arr):
     """True while the graph holds ``arr`` read-only (so nothing derived from its values on
-    the device can have gone stale)."""
-    return _key(arr) in _locked
+    the device can have gone stale).  A value that exists on the device only cannot be
+    written to from the host at all."""
+    return isinstance(arr, DeviceArray) or _key(arr) in _locked
 
 
 def _evict_key(key):
@@ -156,25 +324,44 @@ def _evict_key(key):
 
 
 def attach(arr, buf):
-    """Record ``buf`` as the device copy of ``arr`` (which the graph is about to lock)."""
-    key = _key(arr)
-    _mirrors[key] = buf
-    try:
-        weakref.finalize(_root(arr), _evict_key, key)
-    except TypeError:  # owner not weak-referenceable: do not cache
-        _mirrors.pop(key, None)
+    """Offer ``buf`` as the device copy of the result ``arr``.  The offer stands only if the
+    graph locks ``arr`` next (``Tensor._op`` does, right after the operation returns): an array
+    that is handed out writeable -- under ``no_autodiff`` or with the memory guard off -- may
+    be edited on the host, and a copy cached for it would go stale unnoticed."""
+    if isinstance(arr, DeviceArray):
+        return
+    _pending.clear()
+    _pending[_key(arr)] = buf
+
+
+def drop_pending():
+    """Forget the offer of the last :func:`attach` (its array was not locked)."""
+    _pending.clear()
 
 
 def attach_transient(arr, buf):
-    """Record ``buf`` as the device copy of a gradient array until backward() ends."""
-    _transient[_key(arr)] = buf
+    """Record ``buf`` as the device copy of a gradient array until backward() ends or the
+    array dies, whichever comes first (its memory may be handed out again after that)."""
+    if isinstance(arr, DeviceArray):
+        return
+    key = _key(arr)
+    _transient[key] = buf
+    try:
+        weakref.finalize(_root(arr), _drop_transient, key, buf)
+    except TypeError:  # owner not weak-referenceable: do not cache
+        _transient.pop(key, None)
+
+
+def _drop_transient(key, buf):
+    if _transient.get(key) is buf:
+        del _transient[key]
 
 
 def hold_gradient(arr):
     """Upload ``arr`` now and keep the copy until backward() ends: an operation with several
     non-constant inputs is asked for one gradient per input with the same incoming ``arr``,
     which would otherwise cross PCIe once per request."""
-    if not isinstance(arr, np.ndarray) or not arr.flags["C_CONTIGUOUS"] or arr.size == 0:
+    if isinstance(arr, DeviceArray) or not isinstance(arr, np.ndarray) or not arr.flags["C_CONTIGUOUS"] or arr.size == 0:
         return
     if arr.dtype not in (np.float32, np.float64) or lookup(arr) is not None:
         return
@@ -185,6 +372,8 @@ def hold_gradient(arr):
 
 
 def evict(arr):
+    if isinstance(arr, DeviceArray):
+        return
     key = _key(arr)
     _mirrors.pop(key, None)
     _transient.pop(key, None)
@@ -195,6 +384,8 @@ def drop_transients():
 
 
 def lookup(arr):
+    if isinstance(arr, DeviceArray):
+        return arr.buf
     if not arr.flags["C_CONTIGUOUS"]:
         return None
     key = _key(arr)
@@ -207,6 +398,9 @@ def lookup(arr):
 def to_device(arr, dtype=None):
     """Device buffer holding ``arr`` (cast to ``dtype`` if given): the cached mirror
     when there is one, else a fresh upload (cached if the graph holds ``arr``)."""
+    if isinstance(arr, DeviceArray):
+        stats["mirror_hits"] += 1
+        return (arr if dtype is None else arr.astype(dtype)).buf
     if dtype is not None and arr.dtype != dtype:
         arr = arr.astype(dtype)
     elif not arr.flags["C_CONTIGUOUS"]:
@@ -219,13 +413,21 @@ def to_device(arr, dtype=None):
     buf = DeviceBuffer(arr.nbytes)
     buf.upload(arr)
     stats["uploads"] += 1
-    if _key(arr) in _locked:
-        attach(arr, buf)
+    key = _key(arr)
+    if key in _locked:
+        _mirrors[key] = buf
+        try:
+            weakref.finalize(_root(arr), _evict_key, key)
+        except TypeError:  # owner not weak-referenceable: do not cache
+            _mirrors.pop(key, None)
     return buf
 
 
-def download(buf, shape, dtype):
-    """Copy a device buffer into a new pinned host array."""
+def download(buf, shape, dtype, now=False):
+    """The result a kernel left in ``buf``: copied into a new pinned host array, or -- while
+    :func:`deferring` is active and unless ``now`` -- left where it is as a DeviceArray."""
+    if _defer and not now:
+        return DeviceArray(buf, shape, dtype)
     out = pinned_empty(shape, dtype)
     buf.download_into(out)
     return out

@@ -100,10 +100,13 @@ def release(refs):
 
 
 def arrays_and_bases(tensors):
-    """Each tensor's array, preceded by its ndarray base if it has one (unique)."""
+    """Each tensor's host array, preceded by its ndarray base if it has one (unique).  A
+    tensor whose value is on the device only has no host array that could be written to."""
     seen = set()
     for t in tensors:
-        arr = t.data
+        arr = t._value
+        if not isinstance(arr, np.ndarray):
+            continue
         base = arr.base
         for a in (base, arr):
             if isinstance(a, np.ndarray) and id(a) not in seen:

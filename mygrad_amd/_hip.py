@@ -154,6 +154,9 @@ _SIGNATURES = {
     "mg_sum_all": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
     "mg_sum_all_static": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
     "mg_fill_from": [ctypes.c_int, ctypes.c_int64, _vp, _vp],
+    "mg_cast": [ctypes.c_int, ctypes.c_int, ctypes.c_int64, _vp, _vp],
+    "mg_accumulate": [ctypes.c_int, ctypes.c_int, ctypes.c_int64, _vp, _vp],
+    "mg_fill_value": [ctypes.c_int, ctypes.c_int64, ctypes.c_double, _vp],
     "mg_sum_over": [ctypes.c_int] + [ctypes.c_int64] * 3 + [ctypes.c_int, _vp, _vp],
     "mg_sum_product_over": [ctypes.c_int] + [ctypes.c_int64] * 3 + [ctypes.c_int, _vp, _vp, _vp],
     "mg_batchnorm_fwd": [ctypes.POINTER(BnDesc), _vp, _vp, _vp, _vp, _vp, _vp],

@@ -10,6 +10,7 @@
 #include "internal.h"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace mg {
 
@@ -292,6 +293,65 @@ int launch_relu_mask(int dtype, int64_t n, const void *in, void *out, void *mask
   return MG_OK;
 }
 
+// Kernels of the gradient bookkeeping between operations: out = (B) x, acc = (A)(acc + inc)
+// in the wider of the two types (what NumPy's `acc += inc` computes), out = value.  A thread
+// takes four consecutive elements of each array (16 or 32 bytes).
+template <typename A, typename B, bool ADD>
+__global__ void __launch_bounds__(256) convert_kernel(A *__restrict__ acc, const B *__restrict__ inc, long long n) {
+  typedef A VA __attribute__((ext_vector_type(4)));
+  typedef B VB __attribute__((ext_vector_type(4)));
+  typedef typename std::conditional<(sizeof(A) > sizeof(B)), A, B>::type P;
+  const long long nvec = n / 4;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (long long)gridDim.x * 256) {
+    const VB b = reinterpret_cast<const VB *>(inc)[i];
+    VA r;
+    if constexpr (ADD) {
+      const VA a = reinterpret_cast<const VA *>(acc)[i];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) r[k] = (A)((P)a[k] + (P)b[k]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) r[k] = (A)b[k];
+    }
+    reinterpret_cast<VA *>(acc)[i] = r;
+  }
+  if (blockIdx.x == 0) {
+    const long long i = nvec * 4 + threadIdx.x;
+    if (i < n) acc[i] = ADD ? (A)((P)acc[i] + (P)inc[i]) : (A)inc[i];
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) fill_value_kernel(T *__restrict__ out, T value, long long n) {
+  typedef typename Vec16<T>::type V;
+  constexpr int VEC = Vec16<T>::N;
+  V vv;
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) vv[k] = value;
+  const long long nvec = n / VEC;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (long long)gridDim.x * 256) reinterpret_cast<V *>(out)[i] = vv;
+  if (blockIdx.x == 0) {
+    const long long i = nvec * VEC + threadIdx.x;
+    if (i < n) out[i] = value;
+  }
+}
+
+template <bool ADD>
+int launch_convert(int a_dtype, int b_dtype, int64_t n, void *acc, const void *inc) {
+  if (n == 0) return MG_OK;
+  hipStream_t s = runtime().stream;
+  const unsigned grid = (unsigned)std::min<long long>(ceil_div(ceil_div(n, 4), 256), (long long)runtime().props.multiProcessorCount * 16);
+  ScopedTiming timed(TAG_ELEMENTWISE);
+#define MG_CONVERT(A, B) hipLaunchKernelGGL((convert_kernel<A, B, ADD>), dim3(grid), dim3(256), 0, s, (A *)acc, (const B *)inc, (long long)n)
+  if (a_dtype == MG_F32 && b_dtype == MG_F32) MG_CONVERT(float, float);
+  else if (a_dtype == MG_F32) MG_CONVERT(float, double);
+  else if (b_dtype == MG_F32) MG_CONVERT(double, float);
+  else MG_CONVERT(double, double);
+#undef MG_CONVERT
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
 // How mg_sum_all cuts x: chunks of 128 KiB, at most 4096 of them (then the chunks grow); a
 // function of n and the element size only, so that the order of the additions is too.
 struct SumChunking {
@@ -484,6 +544,45 @@ int mg_sum_all_static(int dtype, int64_t n, const void *x, void *out) {
   if (sum_chunking(dtype, n).chunks > kStaticChunks) return fail(MG_ERR_UNSUPPORTED, "mg_sum_all_static: more chunks than the scratch array holds");
   // no timing events here: creating them allocates
   return launch_sum_all(dtype, n, x, out, partial);
+}
+
+int mg_cast(int from_dtype, int to_dtype, int64_t n, const void *x, void *out) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (int rc = check_elementwise(from_dtype, n, "mg_cast")) return rc;
+  if (int rc = check_elementwise(to_dtype, n, "mg_cast")) return rc;
+  if (n > 0 && (!x || !out)) return fail(MG_ERR_BAD_ARG, "null pointer in mg_cast");
+  if (reinterpret_cast<uintptr_t>(x) % 32 != 0 || reinterpret_cast<uintptr_t>(out) % 32 != 0)
+    return fail(MG_ERR_BAD_ARG, "mg_cast: buffers must be 32-byte aligned");
+  return launch_convert<false>(to_dtype, from_dtype, n, out, x);
+}
+
+int mg_accumulate(int acc_dtype, int inc_dtype, int64_t n, void *acc, const void *inc) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (int rc = check_elementwise(acc_dtype, n, "mg_accumulate")) return rc;
+  if (int rc = check_elementwise(inc_dtype, n, "mg_accumulate")) return rc;
+  if (n > 0 && (!acc || !inc)) return fail(MG_ERR_BAD_ARG, "null pointer in mg_accumulate");
+  if (reinterpret_cast<uintptr_t>(acc) % 32 != 0 || reinterpret_cast<uintptr_t>(inc) % 32 != 0)
+    return fail(MG_ERR_BAD_ARG, "mg_accumulate: buffers must be 32-byte aligned");
+  return launch_convert<true>(acc_dtype, inc_dtype, n, acc, inc);
+}
+
+int mg_fill_value(int dtype, int64_t n, double value, void *out) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  if (int rc = check_elementwise(dtype, n, "mg_fill_value")) return rc;
+  if (n > 0 && !out) return fail(MG_ERR_BAD_ARG, "null pointer in mg_fill_value");
+  if (misaligned(out)) return fail(MG_ERR_BAD_ARG, "mg_fill_value: out must be 16-byte aligned");
+  if (n == 0) return MG_OK;
+  hipStream_t s = runtime().stream;
+  ScopedTiming timed(TAG_ELEMENTWISE);
+  if (dtype == MG_F32)
+    hipLaunchKernelGGL(fill_value_kernel<float>, dim3(streaming_grid(n, 4)), dim3(256), 0, s, (float *)out, (float)value, (long long)n);
+  else
+    hipLaunchKernelGGL(fill_value_kernel<double>, dim3(streaming_grid(n, 8)), dim3(256), 0, s, (double *)out, value, (long long)n);
+  MG_HIP(hipGetLastError());
+  return MG_OK;
 }
 
 int mg_fill_from(int dtype, int64_t n, const void *value, void *out) {

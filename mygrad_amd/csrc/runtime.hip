@@ -317,10 +317,16 @@ int mg_malloc(void **dptr, size_t nbytes) {
 
 int mg_free(void *dptr) {
   MG_LOCK();
-  MG_REQUIRE_INIT();
   if (!dptr) return MG_OK;
   BlockPool &bp = pool();
   auto known = bp.size_of.find(dptr);
+  if (!runtime().ready) {
+    // a block that outlived mg_shutdown: there is no stream left to order its reuse on,
+    // so it goes straight back to the driver (hipFree waits for the device)
+    if (known != bp.size_of.end()) bp.size_of.erase(known);
+    MG_HIP(hipFree(dptr));
+    return MG_OK;
+  }
   if (known == bp.size_of.end()) {
     // not from the pool: hipFree waits for the device, so no kernel can still be using it
     MG_HIP(hipFree(dptr));
@@ -369,10 +375,14 @@ int mg_host_alloc(void **hptr, size_t nbytes) {
 
 int mg_host_free(void *hptr) {
   MG_LOCK();
-  MG_REQUIRE_INIT();
   if (!hptr) return MG_OK;
   BlockPool &bp = host_pool();
   auto known = bp.size_of.find(hptr);
+  if (!runtime().ready) {  // a pinned block that outlived mg_shutdown
+    if (known != bp.size_of.end()) bp.size_of.erase(known);
+    MG_HIP(hipHostFree(hptr));
+    return MG_OK;
+  }
   if (known == bp.size_of.end()) {
     MG_HIP(hipHostFree(hptr));
     return MG_OK;
@@ -495,26 +505,31 @@ int mg_probe_mfma(int kind, int waves_per_simd, double *tflops) {
   void *sink = nullptr;
   if (int rc = workspace((size_t)blocks * 256 * sizeof(double), &sink)) return rc;
   hipStream_t s = runtime().stream;
-  hipEvent_t t0, t1;
-  MG_HIP(hipEventCreate(&t0));
-  MG_HIP(hipEventCreate(&t1));
+  struct EventPair {  // destroyed on every way out
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    ~EventPair() {
+      if (t0) (void)hipEventDestroy(t0);
+      if (t1) (void)hipEventDestroy(t1);
+    }
+  } ev;
+  MG_HIP(hipEventCreate(&ev.t0));
+  MG_HIP(hipEventCreate(&ev.t1));
   float best = 0;
   for (int rep = 0; rep < 4; ++rep) {  // the first repetition warms the clocks up
-    MG_HIP(hipEventRecord(t0, s));
+    MG_HIP(hipEventRecord(ev.t0, s));
     if (kind == 0)
       hipLaunchKernelGGL(mfma_probe_kernel<0>, dim3(blocks), dim3(256), 0, s, (double *)sink, iters);
     else if (kind == 1)
       hipLaunchKernelGGL(mfma_probe_kernel<1>, dim3(blocks), dim3(256), 0, s, (double *)sink, iters);
     else
       hipLaunchKernelGGL(mfma_probe_kernel<2>, dim3(blocks), dim3(256), 0, s, (double *)sink, iters);
-    MG_HIP(hipEventRecord(t1, s));
-    MG_HIP(hipEventSynchronize(t1));
+    MG_HIP(hipEventRecord(ev.t1, s));
+    MG_HIP(hipEventSynchronize(ev.t1));
     float ms = 0;
-    MG_HIP(hipEventElapsedTime(&ms, t0, t1));
-    if (rep > 0 && (best == 0 || ms < best)) best = ms;
+    MG_HIP(hipEventElapsedTime(&ms, ev.t0, ev.t1));
+    if (rep > 0 && ms > 0 && (best == 0 || ms < best)) best = ms;
   }
-  (void)hipEventDestroy(t0);
-  (void)hipEventDestroy(t1);
+  if (!(best > 0)) return fail(MG_ERR_HIP, "mfma probe: every timed repetition reported 0 ms");
   const double per_wave = kind == 0 ? 16 * 2048.0 : kind == 1 ? 8 * 2048.0 : 16 * 512.0;  // flops per loop trip
   *tflops = (double)blocks * 4 * iters * per_wave / (best * 1e-3) * 1e-12;
   return MG_OK;

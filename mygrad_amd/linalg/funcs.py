@@ -11,6 +11,13 @@ except ImportError:  # pragma: no cover
 __all__ = ["einsum"]
 
 
+def _shape_only(tensor):
+    """A stand-in with the tensor's shape and dtype that owns one element: NumPy's parser of the
+    subscripts looks at the operands' shapes only, and a value that is on the device need not
+    be copied to the host for that."""
+    return np.broadcast_to(np.empty((), dtype=tensor.dtype), tensor.shape)
+
+
 def einsum(*operands, optimize=False, out=None, constant=None):
     """einsum(subscripts, *operands)
 
@@ -59,11 +66,11 @@ def einsum(*operands, optimize=False, out=None, constant=None):
     operands = list(operands)
     if isinstance(operands[0], str):
         variables = operands[1:]
-        operands[1:] = (var.data if isinstance(var, Tensor) else var for var in operands[1:])
+        operands[1:] = (_shape_only(var) if isinstance(var, Tensor) else var for var in operands[1:])
     else:
         end = -1 if len(operands) % 2 else None  # the last entry is the result's sublist
         variables = operands[:end:2]
-        operands[:end:2] = (var.data if isinstance(var, Tensor) else np.asarray(var) for var in operands[:end:2])
+        operands[:end:2] = (_shape_only(var) if isinstance(var, Tensor) else np.asarray(var) for var in operands[:end:2])
     in_lbls, out_lbls, _ = _parse_einsum_input(operands)
     return Tensor._op(
         EinSum,

@@ -219,6 +219,8 @@ def contract_all(operands, out_lbls, sizes, dtype):
 
 
 class EinSum(Operation):
+    takes_device_arrays = True
+
     gradient_on_device = True
 
     def __call__(self, *variables, in_lbls, out_lbls, out=None, optimize=False):
@@ -229,7 +231,7 @@ class EinSum(Operation):
         self._cache = None  # how often each (tensor, labels) pair occurs; see backward_var
         if out is not None:
             raise NotImplementedError("einsum on the GPU does not write into an existing array (out=...)")
-        arrays = [v.data for v in variables]
+        arrays = [_device.value_of(v) for v in variables]
 
         # the checks np.einsum makes, with its exception type
         if len(self.in_lbls) != len(arrays):
@@ -262,7 +264,7 @@ class EinSum(Operation):
 
         if any(len(lbls) - len(set(lbls)) > 0 and len(set(lbls)) > 6 for lbls in self._lbls):
             raise NotImplementedError("einsum on the GPU walks diagonals of operands with at most six distinct labels")
-        dtype = np.dtype(np.result_type(*arrays))
+        dtype = np.dtype(np.result_type(*(a.dtype for a in arrays)))
         if dtype not in (np.float32, np.float64):
             raise TypeError(f"einsum runs on the GPU in float32 or float64, got {[str(a.dtype) for a in arrays]} (there is no CPU fallback)")
         self._dtype, self._sizes = dtype, sizes
@@ -309,7 +311,7 @@ class EinSum(Operation):
         others = list(self._lbls)  # labels with broadcast axes struck
         var_lbl = others.pop(index)
         dtype, sizes = self._dtype, self._sizes
-        if var.data.size == 0:
+        if _device.value_of(var).size == 0:
             return np.zeros(var.shape, dtype=dtype)
         if 0 in sizes.values():
             return np.zeros(var.shape, dtype=dtype)
@@ -319,8 +321,8 @@ class EinSum(Operation):
         elsewhere = set(chain.from_iterable(others)) | set(self.out_lbls)
         once = _last_of_each(var_lbl)  # the operand's labels with its diagonals taken (linalg/ops.py:147-163)
         found = "".join(lbl for lbl in once if lbl in elsewhere)
-        operands = [(_device.to_device(np.ascontiguousarray(grad), dtype), self.out_lbls)]
-        operands += [self._operand(v.data, lbls) for n, (v, lbls) in enumerate(zip(self.variables, self._lbls)) if n != index]
+        operands = [(_device.to_device(grad if isinstance(grad, _device.DeviceArray) else np.ascontiguousarray(grad), dtype), self.out_lbls)]
+        operands += [self._operand(_device.value_of(v), lbls) for n, (v, lbls) in enumerate(zip(self.variables, self._lbls)) if n != index]
         ob = contract_all(operands, found, sizes, dtype)
         if found != once:
             ob = _reduce.broadcast(ob, tuple(sizes[lbl] if lbl in elsewhere else 1 for lbl in once),
@@ -329,14 +331,13 @@ class EinSum(Operation):
             # the gradient lives on the diagonals the forward pass read; everything off them is
             # zero (the reference writes through a strided view of zeros, linalg/ops.py:220-262)
             ob = _strided(ob, var_lbl, once, sizes, dtype, scatter=True)
-        nbytes = var.data.size * dtype.itemsize
+        nbytes = _device.value_of(var).size * dtype.itemsize
         if factor > 1 or any(ob is buf for buf, _ in operands):
             # a buffer of its own, scaled by the number of times the pair occurs
-            scale = _device.to_device(np.array(float(factor), dtype=dtype))
             ones = _device.DeviceBuffer(max(nbytes, 16))
-            _hip.check(_hip.lib().mg_fill_from(_hip.dtype_code(dtype), var.data.size, scale.ptr, ones.ptr))
+            _hip.check(_hip.lib().mg_fill_value(_hip.dtype_code(dtype), _device.value_of(var).size, float(factor), ones.ptr))
             scaled = _device.DeviceBuffer(max(nbytes, 16))
-            _hip.check(_hip.lib().mg_multiply(_hip.dtype_code(dtype), var.data.size, ob.ptr, ones.ptr, scaled.ptr))
+            _hip.check(_hip.lib().mg_multiply(_hip.dtype_code(dtype), _device.value_of(var).size, ob.ptr, ones.ptr, scaled.ptr))
             ob = scaled
         out = _device.download(ob, var.shape, dtype)
         _device.attach_transient(out, ob)

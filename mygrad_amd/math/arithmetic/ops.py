@@ -19,7 +19,7 @@ __all__ = ["Multiply"]
 
 
 def _float_dtype(op, a, b):
-    dtype = np.result_type(a, b)
+    dtype = np.result_type(a.dtype, b.dtype)
     if dtype not in (np.float32, np.float64):
         raise TypeError(f"{op} runs on the GPU in float32 or float64, got {a.dtype} and {b.dtype} (there is no CPU fallback)")
     return np.dtype(dtype)
@@ -51,14 +51,16 @@ def device_multiply(a, b, dtype, shape=None):
 class Multiply(Operation):
     """``f(a, b) -> a * b`` element-wise, with NumPy's broadcasting."""
 
+    takes_device_arrays = True
+
     gradient_on_device = True
 
     def __call__(self, a, b):
         self.variables = (a, b)
-        dtype = _float_dtype("multiply", a.data, b.data)
+        dtype = _float_dtype("multiply", _device.value_of(a), _device.value_of(b))
         self._dtype = dtype
         self._shape = np.broadcast_shapes(a.shape, b.shape)  # ValueError for shapes that do not go together
-        out, ob = device_multiply(a.data, b.data, dtype, self._shape)
+        out, ob = device_multiply(_device.value_of(a), _device.value_of(b), dtype, self._shape)
         if ob is not None:
             _device.attach(out, ob)
         return out
@@ -66,14 +68,15 @@ class Multiply(Operation):
     def backward_var(self, grad, index, **kwargs):
         a, b = self.variables
         var, other = (a, b) if index == 0 else (b, a)
-        dtype = np.dtype(np.result_type(grad, other.data))
+        dtype = np.dtype(np.result_type(grad.dtype, other.dtype))
         if grad.shape != self._shape or dtype not in (np.float32, np.float64):
             raise NotImplementedError(f"multiply backward for gradient {grad.shape} {grad.dtype} (no CPU fallback)")
         if var.size == int(np.prod(self._shape, dtype=np.int64)):  # nothing to add up (axes of length one at most)
-            out, ob = device_multiply(grad, other.data, dtype, self._shape)
+            out, ob = device_multiply(grad, _device.value_of(other), dtype, self._shape)
             if ob is None:
                 return np.zeros(var.shape, dtype=dtype)
-            out = out.reshape(var.shape)
+            if out.shape != var.shape:
+                out = out.reshape(var.shape)  # shares its buffer: the caller copies it before keeping it
             _device.attach_transient(out, ob)
             return out
         if 0 in self._shape:
@@ -84,9 +87,9 @@ class Multiply(Operation):
         axes = tuple(range(lead)) + tuple(lead + i for i, n in enumerate(var.shape) if n == 1 and self._shape[lead + i] != 1)
         if other.shape == self._shape:
             # product and sums in one pass over the gradient and the other operand
-            rb = _reduce.sum_axes(_device.to_device(grad, dtype), self._shape, axes, dtype, times=_device.to_device(other.data, dtype))
+            rb = _reduce.sum_axes(_device.to_device(grad, dtype), self._shape, axes, dtype, times=_device.to_device(_device.value_of(other), dtype))
         else:
-            _, ob = device_multiply(grad, other.data, dtype, self._shape)
+            _, ob = device_multiply(grad, _device.value_of(other), dtype, self._shape)
             rb = _reduce.sum_axes(ob, self._shape, axes, dtype)
         back = _device.download(rb, var.shape, dtype)
         _device.attach_transient(back, rb)

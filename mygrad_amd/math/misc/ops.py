@@ -34,25 +34,27 @@ def _prod(shape):
 
 
 class MatMul(Operation):
+    takes_device_arrays = True
+
     gradient_on_device = True
 
     def __call__(self, a, b):
         self.variables = (a, b)
-        x, y = a.data, b.data
+        x, y = _device.value_of(a), _device.value_of(b)
         # NumPy's own checks (scalars, core dimensions, batch broadcasting) on operands
         # without rows and columns: the same errors, the batch shape of the result, no arithmetic
         probe = np.matmul(
             np.empty(x.shape if x.ndim < 2 else (*x.shape[:-2], 0, x.shape[-1]), dtype=np.int8),
             np.empty(y.shape if y.ndim < 2 else (*y.shape[:-2], y.shape[-2], 0), dtype=np.int8),
         )
-        dtype = np.dtype(np.result_type(x, y))
+        dtype = np.dtype(np.result_type(x.dtype, y.dtype))
         if dtype not in (np.float32, np.float64):
             raise TypeError(f"matmul runs on the GPU in float32 or float64, got {x.dtype} and {y.dtype} (there is no CPU fallback)")
 
-        x2 = x if x.ndim > 1 else x[None, :]
-        y2 = y if y.ndim > 1 else y[:, None]
-        M, K, N = x2.shape[-2], x2.shape[-1], y2.shape[-1]
-        stack_a, stack_b = x2.shape[:-2], y2.shape[:-2]
+        x2_shape = tuple(x.shape) if x.ndim > 1 else (1, *x.shape)  # a vector is promoted like np.matmul promotes it
+        y2_shape = tuple(y.shape) if y.ndim > 1 else (*y.shape, 1)
+        M, K, N = x2_shape[-2], x2_shape[-1], y2_shape[-1]
+        stack_a, stack_b = x2_shape[:-2], y2_shape[:-2]
         # two different stacks: both are spread to the batch shape they broadcast to
         self._spread = bool(stack_a and stack_b and stack_a != stack_b)
         self._own_stacks = (stack_a, stack_b)
@@ -63,7 +65,7 @@ class MatMul(Operation):
         assert len(out_shape) == probe.ndim
         self._dtype, self._dims = dtype, (M, K, N)
         self._stacks = (stack_a, stack_b)
-        self._promoted = (x2.shape, y2.shape)
+        self._promoted = (x2_shape, y2_shape)
         if 0 in out_shape or K == 0:
             return np.zeros(out_shape, dtype=dtype)
 
@@ -118,7 +120,7 @@ class MatMul(Operation):
     def backward_var(self, grad, index, **kwargs):
         a, b = self.variables
         dtype = self._dtype
-        var = (a, b)[index].data
+        var = _device.value_of((a, b)[index])
         if var.size == 0 or grad.size == 0:
             return np.zeros(var.shape, dtype=dtype)
         M, K, N = self._dims
@@ -134,10 +136,10 @@ class MatMul(Operation):
         ob = _device.DeviceBuffer(max(count * dtype.itemsize, 16))
         if index == 0:
             # d a = grad @ b^T, summed over a batch that `a` was shared by (ops.py:107-114)
-            self._launch("mg_matmul_da", gb, self._operand(b.data, 1), ob, a_like=2, x_like=1, out_like=0)
+            self._launch("mg_matmul_da", gb, self._operand(_device.value_of(b), 1), ob, a_like=2, x_like=1, out_like=0)
         else:
             # d b = a^T @ grad, summed over a stack of left operands that `b` was shared by (ops.py:116-124)
-            self._launch("mg_matmul_dx", gb, self._operand(a.data, 0), ob, a_like=2, x_like=0, out_like=1)
+            self._launch("mg_matmul_dx", gb, self._operand(_device.value_of(a), 0), ob, a_like=2, x_like=0, out_like=1)
         if widened:
             # one gradient per matrix pair: add up those of the pairs that shared this operand's matrix
             lead = len(full) - len(own)

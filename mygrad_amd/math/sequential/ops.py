@@ -17,9 +17,11 @@ __all__ = ["Sum"]
 
 
 class Sum(Operation):
+    takes_device_arrays = True
+
     def __call__(self, a, axis=None, keepdims=False):
         self.variables = (a,)
-        x = a.data
+        x = _device.value_of(a)
         # the reference keeps a single axis as a one-tuple (operation_base.py:424-431)
         self.axis = axis if axis is None or hasattr(axis, "__iter__") else (axis,)
         self.keepdims = bool(keepdims)
@@ -54,21 +56,22 @@ class Sum(Operation):
 
     def backward_var(self, grad, index, **kwargs):
         (a,) = self.variables
-        x = a.data
-        grad = np.asarray(grad)
+        x = _device.value_of(a)
+        if not isinstance(grad, _device.DeviceArray):
+            grad = np.ascontiguousarray(grad)
         if x.size == 0:
             return np.zeros(x.shape, dtype=x.dtype)
         lib, code = _hip.lib(), _hip.dtype_code(x.dtype)
         if len(self._axes) == x.ndim:
             if grad.size != 1:
                 raise ValueError(f"the gradient of a sum over every axis holds one value, got shape {grad.shape}")
-            gb = _device.to_device(np.ascontiguousarray(grad).reshape(()), x.dtype)
+            gb = _device.to_device(grad.reshape(()), x.dtype)
             ob = _device.DeviceBuffer(max(x.nbytes, 16))
             _hip.check(lib.mg_fill_from(code, x.size, gb.ptr, ob.ptr))
         else:
             if grad.size * int(np.prod([x.shape[i] for i in self._axes], dtype=np.int64)) != x.size:
                 raise ValueError(f"gradient of shape {grad.shape} does not fit a sum of {x.shape} over axes {self._axes}")
-            gb = _device.to_device(np.ascontiguousarray(grad), x.dtype)
+            gb = _device.to_device(grad, x.dtype)
             ob = _reduce.broadcast(gb, self._kept_shape, x.shape, x.dtype)
             if ob is gb:  # nothing to spread: a copy the caller may keep
                 ob = _device.DeviceBuffer(max(x.nbytes, 16))

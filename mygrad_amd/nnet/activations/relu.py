@@ -15,9 +15,11 @@ __all__ = ["relu", "ReLu"]
 
 
 class ReLu(Operation):
+    takes_device_arrays = True
+
     def __call__(self, a):
         self.variables = (a,)
-        x = a.data
+        x = _device.value_of(a)
         if x.dtype not in (np.float32, np.float64):
             raise TypeError(f"relu runs on the GPU in float32 or float64, got {x.dtype} (there is no CPU fallback)")
         if x.size == 0:
@@ -31,7 +33,7 @@ class ReLu(Operation):
         return out
 
     def backward_var(self, grad, index, **kwargs):
-        x = self.variables[index].data
+        x = _device.value_of(self.variables[index])
         if x.size == 0:
             return np.empty(x.shape, dtype=x.dtype)
         if grad.shape != x.shape:

@@ -21,6 +21,8 @@ class BatchNorm(Operation):
     """Per-channel normalisation with optional scale and shift.  Calling the instance binds
     the channel statistics it computed as ``self.mean`` and ``self.var`` (each ``(C,)``)."""
 
+    takes_device_arrays = True
+
     def __call__(self, x, gamma, beta, *, eps):
         """``x:(N, C, ...)``; ``gamma`` / ``beta``: ``(C,)`` tensors, or empty ones for "no
         scale" / "no shift" (how the wrapper passes ``None``); returns the normalised array."""
@@ -35,7 +37,7 @@ class BatchNorm(Operation):
         self.beta = beta
         self.eps = float(eps)
 
-        xd = x.data
+        xd = _device.value_of(x)
         if xd.ndim < 2:
             raise ValueError(f"batchnorm normalises every axis but axis 1: `x` must have at least 2 axes, got shape {xd.shape}")
         if xd.dtype not in (np.float32, np.float64):
@@ -44,25 +46,25 @@ class BatchNorm(Operation):
         for name, t in (("gamma", gamma), ("beta", beta)):
             if t is None:
                 continue
-            if t.data.shape != (channels,):
-                raise ValueError(f"`{name}` must have shape ({channels},), got {t.data.shape}")
-            if t.data.dtype != xd.dtype:
+            if _device.value_of(t).shape != (channels,):
+                raise ValueError(f"`{name}` must have shape ({channels},), got {_device.value_of(t).shape}")
+            if _device.value_of(t).dtype != xd.dtype:
                 raise TypeError(
-                    f"batchnorm on the GPU takes `{name}` in the dtype of `x` ({xd.dtype}), got {t.data.dtype}"
+                    f"batchnorm on the GPU takes `{name}` in the dtype of `x` ({xd.dtype}), got {_device.value_of(t).dtype}"
                 )
         if not self.eps >= 0:
             raise ValueError(f"`eps` must be a non-negative number, got {eps}")
 
         self._bwd = None
         if xd.size == 0:
-            self.mean = np.full((channels,), np.nan, dtype=xd.dtype)
-            self.var = np.full((channels,), np.nan, dtype=xd.dtype)
+            self._mean = np.full((channels,), np.nan, dtype=xd.dtype)
+            self._var = np.full((channels,), np.nan, dtype=xd.dtype)
             return np.empty(xd.shape, dtype=xd.dtype)
 
         desc = self._desc = _hip.bn_desc(xd.shape, xd.dtype, gamma is not None, beta is not None, self.eps)
         xb = _device.to_device(xd)
-        gb = _device.to_device(gamma.data) if gamma is not None else None
-        bb = _device.to_device(beta.data) if beta is not None else None
+        gb = _device.to_device(_device.value_of(gamma)) if gamma is not None else None
+        bb = _device.to_device(_device.value_of(beta)) if beta is not None else None
         yb = _device.DeviceBuffer(max(xd.nbytes, 16))
         self._mean_dev = _device.DeviceBuffer(max(channels * xd.itemsize, 16))
         self._var_dev = _device.DeviceBuffer(max(channels * xd.itemsize, 16))
@@ -77,22 +79,37 @@ class BatchNorm(Operation):
                 self._var_dev.ptr,
             )
         )
-        self.mean = _device.download(self._mean_dev, (channels,), xd.dtype)
-        self.var = _device.download(self._var_dev, (channels,), xd.dtype)
+        # copied to the host when somebody asks for them (the backward pass reads the device copies)
+        self._mean = _device.DeviceArray(self._mean_dev, (channels,), xd.dtype)
+        self._var = _device.DeviceArray(self._var_dev, (channels,), xd.dtype)
         y = _device.download(yb, xd.shape, xd.dtype)
         _device.attach(y, yb)
         return y
 
+    @property
+    def mean(self):
+        """Per-channel mean of the batch (the reference's ``self.mean``, batchnorm.py:57)."""
+        if isinstance(self._mean, _device.DeviceArray):
+            self._mean = self._mean.host()
+        return self._mean
+
+    @property
+    def var(self):
+        """Per-channel (biased) variance of the batch (the reference's ``self.var``, batchnorm.py:58)."""
+        if isinstance(self._var, _device.DeviceArray):
+            self._var = self._var.host()
+        return self._var
+
     def _run_backward(self, grad, want):
         """One pass over (x, grad) for every gradient in ``want`` (a set of "x", "gamma",
         "beta"); returns them as a dict of arrays."""
-        x = self.variables[0].data
+        x = _device.value_of(self.variables[0])
         channels = x.shape[1]
         if grad.shape != x.shape:
             raise NotImplementedError(f"batchnorm backward for gradient of shape {grad.shape} (no CPU fallback)")
         xb = _device.to_device(x)
         gradb = _device.to_device(grad, x.dtype)
-        gb = _device.to_device(self.gamma.data) if self.gamma is not None else None
+        gb = _device.to_device(_device.value_of(self.gamma)) if self.gamma is not None else None
         small = max(channels * x.itemsize, 16)
         dxb = _device.DeviceBuffer(max(x.nbytes, 16)) if "x" in want else None
         dgb = _device.DeviceBuffer(small) if "gamma" in want else None
@@ -131,7 +148,7 @@ class BatchNorm(Operation):
 
     def backward_var(self, grad, index, **kwargs):
         which = self._which(index)
-        x = self.variables[0].data
+        x = _device.value_of(self.variables[0])
         if x.size == 0:
             return np.zeros(x.shape if which == "x" else (x.shape[1],), dtype=x.dtype)
         # backward() asks for each variable in turn with the same `grad`: the first request

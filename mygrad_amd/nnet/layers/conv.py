@@ -26,7 +26,7 @@ def _per_axis(value, m, lowest):
 def _kernel_dtype(*arrays):
     """The dtype the kernels compute in: NumPy's promotion of the operands, which
     must come out as float32 or float64."""
-    dtype = np.result_type(*arrays)
+    dtype = np.result_type(*(a.dtype for a in arrays))
     if dtype not in (np.float32, np.float64):
         raise TypeError(
             f"conv_nd runs on the GPU in float32 or float64; the operands promote to {dtype} "
@@ -49,11 +49,13 @@ class ConvND(Operation):
     ``(N, C, X0, ...) * (F, C, W0, ...) -> (N, F, G0, ...)``
     """
 
+    takes_device_arrays = True
+
     gradient_on_device = True
 
     def __call__(self, x, w, *, stride, padding=0, dilation=1):
         self.variables = (x, w)
-        xd, wd = x.data, w.data
+        xd, wd = _device.value_of(x), _device.value_of(w)
 
         assert xd.ndim > 2
         assert xd.ndim == wd.ndim
@@ -107,7 +109,7 @@ class ConvND(Operation):
         return out
 
     def backward_var(self, grad, index, **kwargs):
-        x, w = (v.data for v in self.variables)
+        x, w = (_device.value_of(v) for v in self.variables)
         dtype = self._dtype
         if self._desc is None:
             return _device_zeros((x if index == 0 else w).shape, dtype)

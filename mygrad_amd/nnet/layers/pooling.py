@@ -21,11 +21,13 @@ class MaxPoolND(Operation):
     every ``(S0, ...)``; only placements that fit entirely inside the data.
     """
 
+    takes_device_arrays = True
+
     _argmax = None  # device buffer, one byte per window, written by the forward pass
 
     def __call__(self, x, pool, stride):
         self.variables = (x,)
-        xd = x.data
+        xd = _device.value_of(x)
 
         assert isinstance(pool, (tuple, list, np.ndarray)) and all(
             i >= 0 and isinstance(i, Integral) for i in pool
@@ -88,9 +90,12 @@ class MaxPoolND(Operation):
 
     def backward_var(self, grad, index, **kwargs):
         var = self.variables[index]
-        x = var.data
+        x = _device.value_of(var)
         if self._lead == 0:
             return np.zeros(x.shape, dtype=np.float64)
+        if grad.shape != (*x.shape[: x.ndim - len(self.pool)], *self._grid):
+            raise ValueError(f"max_pool backward: gradient of shape {grad.shape} for an output of shape "
+                             f"{(*x.shape[: x.ndim - len(self.pool)], *self._grid)}")
         m = len(self.pool)
         # The reference builds dx in float64 whatever x is (pooling.py:147) and the
         # caller rounds it to x.dtype when it becomes var.grad.  The kernel sums in

@@ -26,6 +26,15 @@ class Operation(ABC):
 
     variables = ()
 
+    # True for operations whose backward_var takes a gradient that is still on the device (a
+    # DeviceArray) as it is; any other operation is handed a host array
+    takes_device_arrays = False
+
+    # the list of array locks the graph holds on this operation's behalf (None without the
+    # memory guard); Tensor._op sets it, and a tensor whose value is copied to the host while
+    # the operation is alive appends the lock on that array
+    _guarded = None
+
     # True for operations whose backward_var hands the incoming gradient to a device kernel
     # for more than one input: backward() then uploads it once for all of them
     gradient_on_device = False
@@ -63,6 +72,11 @@ class Operation(ABC):
             except SkipGradient:
                 continue
 
+            if isinstance(backed, _device.DeviceArray):
+                if backed.shape == var.shape:
+                    self._accumulate_on_device(var, backed, grad)
+                    continue
+                backed = backed.host()  # a gradient that still has to be summed to var's shape
             if not isinstance(backed, (np.ndarray, np.number, Real)):
                 raise InvalidGradient(
                     f"An invalid gradient-value was passed to:\n\t`{type(self).__name__}.backward_var("
@@ -86,8 +100,34 @@ class Operation(ABC):
                     backed = backed.astype(var.dtype, copy=False)
                 var._grad = backed
             else:
+                if isinstance(var._grad, _device.DeviceArray):
+                    var._grad = var._grad.host()
                 _device.evict(var._grad)  # the host copy is about to change
                 var._grad += backed
+
+    @staticmethod
+    def _accumulate_on_device(var, backed, grad):
+        """The same bookkeeping for a gradient that is on the device (and has var's shape):
+        copied if it shares its buffer with something else, cast to var's dtype, stored; or
+        added into the gradient var already holds (reference: operation_base.py:216-228)."""
+        if var._grad is None:
+            if backed.base is not None or backed is grad:
+                backed = backed.copy()
+            if backed.dtype != var.dtype:
+                if var.dtype in (np.float32, np.float64):
+                    backed = backed.astype(var.dtype)
+                else:
+                    backed = backed.host().astype(var.dtype)
+            var._grad = backed
+            return
+        held = var._grad
+        if isinstance(held, _device.DeviceArray) and held._host is None and held.base is None and held.dtype in (np.float32, np.float64):
+            held.add_into(backed)
+            return
+        if isinstance(held, _device.DeviceArray):
+            held = var._grad = held.host()
+        _device.evict(held)  # the host copy is about to change
+        held += backed.host()
 
 
 def _is_foreign_buffer(arr):

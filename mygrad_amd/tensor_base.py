@@ -18,7 +18,7 @@ import numpy as np
 
 from . import _device, _graph
 
-__all__ = ["Tensor", "tensor", "asarray"]
+__all__ = ["Tensor", "tensor", "asarray", "device_tensor"]
 
 _CONSTANT_ONLY = (np.integer, np.bool_)
 
@@ -35,6 +35,30 @@ def tensor(x, *, dtype=None, constant=None, copy=True, ndmin=0):
     return Tensor(x, dtype=dtype, constant=constant, copy=copy, ndmin=ndmin)
 
 
+def device_tensor(x, *, dtype=None, constant=None):
+    """A tensor whose values are uploaded once, now, and live on the device from then on (not a
+    function of the reference, whose arrays are all host arrays).
+
+    A tensor made from a host array is uploaded by the first operation that reads it and the
+    copy is kept only while a graph holds the array read-only, so a training loop that feeds the
+    same host array to a new graph every step uploads it every step.  A device tensor has no host
+    array that could change behind the copy: it is never uploaded again, an operation reads it in
+    place, and ``.data`` copies it back only if somebody asks.  float32 / float64 only.
+    """
+    if isinstance(x, Tensor):
+        if x.on_device and (dtype is None or np.dtype(dtype) == x.dtype):
+            return Tensor(x, constant=constant, copy=False)
+        x = x.data
+    arr = np.ascontiguousarray(x, dtype=dtype)
+    if arr.dtype not in (np.float32, np.float64):
+        raise TypeError(f"device_tensor holds float32 or float64 values, got {arr.dtype}")
+    buf = _device.DeviceBuffer(max(arr.nbytes, 16))
+    if arr.nbytes:
+        buf.upload(arr)
+        _device.stats["uploads"] += 1
+    return Tensor(_device.DeviceArray(buf, arr.shape, arr.dtype), constant=constant, copy=False)
+
+
 class Tensor:
     """An N-dimensional array that remembers the operation that produced it."""
 
@@ -46,15 +70,18 @@ class Tensor:
         if not isinstance(ndmin, Integral):
             raise TypeError(f"'{type(ndmin)}' object cannot be interpreted as an integer")
         if isinstance(x, Tensor):
-            x = x.data
+            x = x._value if copy is False else x.data
         self._creator = _creator
-        if copy is False:
+        self._guards = []  # weak references to the operations that hold this tensor's value read-only
+        if isinstance(x, _device.DeviceArray) and copy is False and not ndmin and (dtype is None or np.dtype(dtype) == x.dtype):
+            data = x  # a result that stays on the device until it is read
+        elif copy is False:
             data = np.asarray(x, dtype=dtype)
             if ndmin and data.ndim < ndmin:
                 data = data[(None,) * (ndmin - data.ndim)]
         else:
             data = np.array(x, dtype=dtype, copy=copy, ndmin=ndmin)
-        self.data = data
+        self._value = data
 
         kind = data.dtype.type
         is_float = issubclass(kind, np.floating)
@@ -72,20 +99,55 @@ class Tensor:
 
     # ------------------------------------------------------------------ array-like surface
     @property
+    def data(self):
+        """The tensor's values as a NumPy array.  The result of an operation stays on the
+        device until this is read for the first time (one copy into pinned host memory);
+        while the graph that produced or consumes it is alive the array is read-only, like
+        every array of a live graph."""
+        value = self._value
+        if isinstance(value, _device.DeviceArray):
+            value = self._to_host()
+        return value
+
+    @data.setter
+    def data(self, value):
+        self._value = value
+
+    def _to_host(self):
+        dev = self._value
+        arr = dev.host()
+        self._value = arr
+        holders = [op for op in (ref() for ref in self._guards) if op is not None and op._guarded is not None]
+        self._guards = []
+        if holders:
+            # the graph is alive: the host copy is held read-only like any other array of the
+            # graph, which is also what keeps the device buffer a valid copy of it
+            _device.attach(arr, dev.buf)
+            for op in holders:
+                op._guarded.append(_graph.lock(arr))
+            _device.drop_pending()
+        return arr
+
+    @property
+    def on_device(self):
+        """True while the values exist on the device only (nothing has read ``data`` yet)."""
+        return isinstance(self._value, _device.DeviceArray)
+
+    @property
     def shape(self):
-        return self.data.shape
+        return self._value.shape
 
     @property
     def ndim(self):
-        return self.data.ndim
+        return self._value.ndim
 
     @property
     def size(self):
-        return self.data.size
+        return self._value.size
 
     @property
     def dtype(self):
-        return self.data.dtype
+        return self._value.dtype
 
     @property
     def constant(self):
@@ -101,6 +163,10 @@ class Tensor:
 
     @property
     def grad(self):
+        """The gradient left by the last ``backward()``, as a NumPy array (copied from the
+        device on first read) or None."""
+        if isinstance(self._grad, _device.DeviceArray):
+            self._grad = self._grad.host()
         return self._grad
 
     def item(self):
@@ -162,20 +228,24 @@ class Tensor:
         tensor_vars = tuple(
             var if isinstance(var, Tensor) else cls(var, constant=True, copy=False) for var in input_vars
         )
+        _device.drop_pending()  # an offer left by an operation that was called directly has lapsed
         guarded = []
         guard = _graph.TRACK_GRAPH and _graph.MEM_GUARD
         if guard:
             guarded = [_graph.lock(a) for a in _graph.arrays_and_bases(tensor_vars)]
 
         f = Op()
+        f._guarded = guarded if guard else None
         try:
-            op_out = f(*tensor_vars, *(op_args or ()), **(op_kwargs or {}))
+            with _device.deferring():  # the result stays on the device until somebody reads it
+                op_out = f(*tensor_vars, *(op_args or ()), **(op_kwargs or {}))
         except Exception:
             if guard:
                 _graph.release(guarded)
             raise
 
         if not _graph.TRACK_GRAPH:
+            _device.drop_pending()  # the result is handed out writeable: no device copy is kept for it
             return cls(op_out, constant=constant, copy=False)
 
         for v in input_vars:
@@ -192,8 +262,15 @@ class Tensor:
         out = cls(op_out, constant=constant, copy=False, _creator=f)
 
         if _graph.MEM_GUARD:
-            guarded.append(_graph.lock(out.data))
+            if not out.on_device:
+                guarded.append(_graph.lock(out._value))
+            # values that are still on the device have no host array to lock yet: the tensor
+            # remembers who holds it, and locks the array on their behalf when it is read
+            for t in (*tensor_vars, out):
+                if t.on_device:
+                    t._guards.append(ref_f)
             finalize(f, _graph.release, guarded)
+        _device.drop_pending()
         return out
 
     # ------------------------------------------------------------------ back-propagation
@@ -210,11 +287,15 @@ class Tensor:
         order = deque()
         _collect_and_null(self, set(), order, set())
 
-        if grad is not None:
+        if isinstance(grad, Tensor) and grad.on_device:
+            grad = grad._value
+        if isinstance(grad, _device.DeviceArray) and grad.shape == self.shape and self.dtype in (np.float32, np.float64):
+            seed = grad.astype(self.dtype)  # a gradient that is on the device already stays there
+        elif grad is not None:
             seed = asarray(grad, dtype=self.dtype)
             if seed.shape != self.shape:
                 try:
-                    seed = np.multiply(np.full_like(self.data, fill_value=1.0), seed, dtype=self.dtype)
+                    seed = np.multiply(np.ones(self.shape, dtype=self.dtype), seed, dtype=self.dtype)
                     if seed.shape != self.shape:
                         raise ValueError()
                 except ValueError:
@@ -223,8 +304,10 @@ class Tensor:
                         f"`grad` must be broadcast-compatible with `tensor.shape={self.shape}`\n"
                         f"Got `grad.shape={seed.shape}`"
                     )
+        elif self._creator is not None and self.on_device and self.size:
+            seed = _device.full(self.shape, self.dtype, 1.0)
         else:
-            seed = np.full_like(self.data, fill_value=1.0)
+            seed = np.ones(self.shape, dtype=self.dtype)
         self._grad = seed
 
         try:
@@ -242,7 +325,9 @@ class Tensor:
             f"\ntensor-shape: {self.shape}\ngrad-shape: {self._grad.shape}"
         )
         if self._creator is not None:
-            self._creator.backward(self._grad)
+            grad = self._grad if self._creator.takes_device_arrays else self.grad
+            with _device.deferring():
+                self._creator.backward(grad)
 
     def clear_graph(self):
         """Detach this tensor and everything upstream of it from the graph; the

@@ -15,6 +15,8 @@ __all__ = ["Repeat"]
 
 
 class Repeat(Operation):
+    takes_device_arrays = True
+
     # Repeat can broadcast in the case:
     #    repeat(1, 2) -> [1 1]
 
@@ -22,7 +24,7 @@ class Repeat(Operation):
         self.variables = (a,)
         self._axis = axis
         self._repeats = repeats
-        x = a.data
+        x = _device.value_of(a)
         if x.dtype.itemsize not in (1, 2, 4, 8) or x.dtype.hasobject:
             raise TypeError(f"repeat runs on the GPU for elements of 1, 2, 4 or 8 bytes, got {x.dtype} (no CPU fallback)")
 
@@ -72,7 +74,7 @@ class Repeat(Operation):
         return out
 
     def backward_var(self, grad, index, **kwargs):
-        a = self.variables[index].data
+        a = _device.value_of(self.variables[index])
         outer, n, inner, total = self._geometry
         if grad.dtype not in (np.float32, np.float64):
             raise TypeError(f"repeat's gradient runs on the GPU in float32 or float64, got {grad.dtype} (no CPU fallback)")

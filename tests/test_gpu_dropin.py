@@ -275,3 +275,153 @@ def test_tensor_feeding_two_pools_accumulates_like_the_reference():
     want_ba = second.astype(np.float32)
     want_ba += first
     assert np.array_equal(x.grad, want_ab) or np.array_equal(x.grad, want_ba)
+
+
+def test_config3a_through_backward():
+    conf = dict(stride=1, padding=1, dilation=1)
+    x, w, g, out = _drop_in_conv(1003, np.float32, (128, 64, 56, 56), (64, 64, 3, 3), (2 / 576) ** 0.5, conf)
+    assert out.shape == (128, 64, 56, 56)
+    s = p = d = (1, 1)
+    assert rel_err(out, direct.conv_forward(x.data, w.data, s, p, d)) <= 2e-4
+    assert rel_err(x.grad, direct.conv_backward_x(g, x.shape, w.data, s, p, d)) <= 2e-4
+    assert rel_err(w.grad, direct.conv_backward_w(g, x.data, w.shape, s, p, d)) <= 2e-4
+    nb = 2
+    assert rel_err(out[:nb], ora.conv_forward(x.data[:nb], w.data, **conf)) <= 2e-4
+    assert rel_err(x.grad[:nb], ora.conv_backward_x(g[:nb], x.data[:nb].shape, x.dtype, w.data, **conf)) <= 2e-4
+
+
+def test_config5_chain_copies_back_only_what_is_read():
+    """Nothing a kernel wrote crosses PCIe until somebody reads it: for the conv -> relu -> pool
+    -> sum(. * g) chain the bytes copied device-to-host are those of the loss, x.grad and w.grad."""
+    from mygrad_amd.nnet import relu
+
+    rng = np.random.default_rng(1006)
+    dtype = np.float32
+    xv = rng.standard_normal((8, 16, 32, 64, 64)).astype(dtype)
+    wv = (rng.standard_normal((32, 16, 3, 3, 3)) * (2 / 432) ** 0.5).astype(dtype)
+    gv = rng.standard_normal((8, 32, 16, 32, 32)).astype(dtype)
+    x, w, g = mg.Tensor(xv), mg.Tensor(wv), mg.Tensor(gv, constant=True)
+    before = dict(_device.stats)
+    y = conv_nd(x, w, stride=1, padding=1)
+    z = max_pool(relu(y), (2, 2, 2), 2)
+    loss = mg.sum(z * g)
+    assert y.on_device and z.on_device and loss.on_device
+    loss.backward()
+    assert _device.stats["d2h_bytes"] == before["d2h_bytes"]  # nothing has been read yet
+    assert _device.stats["uploads"] - before["uploads"] == 3  # x, w, g
+    loss_value = loss.item()
+    dx, dw = x.grad, w.grad
+    assert _device.stats["d2h_bytes"] - before["d2h_bytes"] == dx.nbytes + dw.nbytes + 4
+    assert y.on_device and z.on_device and y.grad is not None
+    assert dx.flags.writeable and dw.flags.writeable and dx.dtype == dtype and dw.dtype == dtype
+
+    # the same numbers as the oracle's, step by step (reading y, z now copies them back)
+    s = p = d = (1, 1, 1)
+    y_data = y.data
+    assert rel_err(y_data, direct.conv_forward(xv, wv, s, p, d)) <= 2e-4
+    r = ora.relu_forward(y_data)
+    want_z, dr = direct.pool(r, gv, (2, 2, 2), (2, 2, 2))
+    assert np.array_equal(z.data, want_z)
+    assert abs(loss_value - float(np.sum(want_z.astype(np.float64) * gv))) <= 1e-6 * float(np.sum(np.abs(want_z * gv)))
+    dy = ora.relu_backward(y_data, dr.astype(dtype))
+    assert np.array_equal(y.grad.view(np.uint32), dy.view(np.uint32))
+    assert rel_err(dx, direct.conv_backward_x(dy, xv.shape, wv, s, p, d)) <= 2e-4
+    assert rel_err(dw, direct.conv_backward_w(dy, xv, wv.shape, s, p, d)) <= 2e-4
+    assert _graph.held_count() == 0
+
+
+def test_result_read_while_the_graph_is_alive_is_held_read_only():
+    rng = np.random.default_rng(21)
+    x = mg.Tensor(rng.standard_normal((2, 3, 8, 8)))
+    w = mg.Tensor(rng.standard_normal((4, 3, 3, 3)))
+    y = conv_nd(x, w, stride=1)
+    z = max_pool(y, (2, 2), 2)
+    assert y.on_device and z.on_device
+    y_data = y.data  # read after two operations took hold of it: both must release it
+    assert not y.on_device and not y_data.flags.writeable and y.data is y_data
+    with pytest.raises(ValueError):
+        y_data[...] = 0.0
+    uploads = _device.stats["uploads"]
+    z.backward()
+    assert _device.stats["uploads"] == uploads  # the host copy of y did not have to go back up
+    assert y_data.flags.writeable and _graph.held_count() == 0
+    want_dy = ora.pool_backward(y_data, np.ones(z.shape), (2, 2), 2)
+    assert np.array_equal(y.grad, want_dy)
+    assert rel_err(x.grad, ora.conv_backward_x(want_dy, x.shape, x.dtype, w.data, stride=1)) <= 1e-10
+    # a result read after its graph is gone is an ordinary writeable array
+    y2 = conv_nd(x, w, stride=1)
+    y2.clear_graph()
+    assert y2.data.flags.writeable
+
+
+def test_unguarded_result_edited_on_the_host_is_uploaded_again():
+    """Under no_autodiff (or without the memory guard) a result is handed out writeable; a later
+    operation must see the host's edits, not a device copy kept from before them."""
+    rng = np.random.default_rng(22)
+    x = rng.standard_normal((2, 3, 8, 8))
+    w = rng.standard_normal((4, 3, 3, 3))
+    for switch in (mg.no_autodiff, mg.mem_guard_off):
+        with switch:
+            y = conv_nd(x, w, stride=1)
+        assert y.data.flags.writeable
+        y.data[...] = rng.standard_normal(y.shape)
+        z = max_pool(y, (2, 2), 2)
+        assert np.array_equal(z.data, ora.pool_forward(y.data, (2, 2), 2))
+        z.clear_graph()
+    # the eager contract (an operation called directly returns a host array): same rule
+    from mygrad_amd.nnet.layers.conv import ConvND
+
+    out = ConvND()(mg.Tensor(x), mg.Tensor(w), stride=1)
+    assert isinstance(out, np.ndarray) and out.flags.writeable
+    out[...] = 1.0
+    z = max_pool(out, (2, 2), 2)
+    assert np.array_equal(z.data, np.ones(z.shape))
+    z.clear_graph()
+    assert _graph.held_count() == 0
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_gradients_of_a_tensor_used_twice_are_added_on_the_device(dtype):
+    from mygrad_amd.nnet import relu
+
+    rng = np.random.default_rng(23)
+    xv = rng.standard_normal((3, 4, 9, 9)).astype(dtype)
+    wv = rng.standard_normal((5, 4, 3, 3)).astype(dtype)
+    gv = rng.standard_normal((3, 5, 7, 7)).astype(dtype)
+    x, w = mg.Tensor(xv), mg.Tensor(wv)
+    a = conv_nd(x, w, stride=1)
+    b = conv_nd(x, w, stride=1)  # x and w feed two operations: their gradients are sums of two terms
+    out = relu(a) * b
+    before = _device.stats["d2h_bytes"]
+    out.backward(gv)
+    assert _device.stats["d2h_bytes"] == before
+    ya = ora.conv_forward(xv, wv, stride=1)
+    da = ora.relu_backward(ya, (gv * ya).astype(dtype))
+    db = (gv * ora.relu_forward(ya)).astype(dtype)
+    want_dx = ora.conv_backward_x(da, xv.shape, xv.dtype, wv, stride=1) + ora.conv_backward_x(db, xv.shape, xv.dtype, wv, stride=1)
+    want_dw = ora.conv_backward_w(da, xv, wv.shape, stride=1) + ora.conv_backward_w(db, xv, wv.shape, stride=1)
+    tol = TOL[np.dtype(dtype)]
+    assert x.grad.dtype == dtype and rel_err(x.grad, want_dx) <= tol
+    assert rel_err(w.grad, want_dw) <= tol
+    assert _graph.held_count() == 0
+
+
+def test_device_tensor_is_uploaded_once_and_seeds_backward():
+    rng = np.random.default_rng(24)
+    xv = rng.standard_normal((2, 3, 10, 10)).astype(np.float32)
+    wv = rng.standard_normal((4, 3, 3, 3)).astype(np.float32)
+    gv = rng.standard_normal((2, 4, 8, 8)).astype(np.float32)
+    before = dict(_device.stats)
+    x, w, g = mg.device_tensor(xv), mg.device_tensor(wv), mg.device_tensor(gv, constant=True)
+    assert x.on_device and x.shape == xv.shape and x.dtype == np.float32 and not x.constant
+    for _ in range(3):  # three graphs over the same tensors: nothing goes up or comes down again
+        out = conv_nd(x, w, stride=1)
+        out.backward(g)
+    assert _device.stats["uploads"] - before["uploads"] == 3
+    assert _device.stats["d2h_bytes"] == before["d2h_bytes"]
+    assert rel_err(x.grad, ora.conv_backward_x(gv, xv.shape, xv.dtype, wv, stride=1)) <= 2e-4
+    assert rel_err(w.grad, ora.conv_backward_w(gv, xv, wv.shape, stride=1)) <= 2e-4
+    assert np.array_equal(x.data, xv) and x.data.flags.writeable
+    with pytest.raises(TypeError):
+        mg.device_tensor(np.arange(4))
+    assert _graph.held_count() == 0
