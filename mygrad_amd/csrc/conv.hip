@@ -524,6 +524,11 @@ struct Plan {
   int blocks_per_cu = 1;  // persistent blocks per compute unit (streaming gather-GEMM)
   bool tap_major = false;  // which kernel family the tables are for
   bool single_dense_phase = false;  // positions enumerate the destination tensor in order
+  // fused stride phases of the data gradient (see GemmParams::nph)
+  int nph = 1;
+  int kcut[4] = {0, 0, 0, 0};
+  int po0[4][3] = {};
+  int pJ[4][3] = {};
   // wgrad
   int splits = 1;
   int kchunk = 0;
@@ -614,14 +619,43 @@ int resident_blocks(K kernel, int threads) {
   X(T, 32, 128, 16, 64)      \
   X(T, 16, 256, 16, 64)
 
+// Tile shapes of the data gradient with 2 / 4 fused stride phases (float only): a wave keeps one
+// set of accumulators per phase, so these are the shapes with at most 32 / 16 accumulator
+// registers per set, which leaves room for two blocks on a compute unit.
+#define MG_FUSED2_SHAPES(T, X) \
+  X(T, 128, 64, 64, 32)        \
+  X(T, 64, 128, 32, 64)        \
+  X(T, 32, 256, 32, 64)        \
+  X(T, 16, 256, 16, 64)
+#define MG_FUSED4_SHAPES(T, X) \
+  X(T, 64, 64, 32, 32)         \
+  X(T, 32, 128, 16, 64)        \
+  X(T, 16, 256, 16, 64)
+
 // Blocks of the persistent tap-major gather-GEMM that a compute unit holds at once.
 template <typename T>
-int gemm_blocks_per_cu(int bm, int bn) {
+int gemm_blocks_per_cu(int bm, int bn, int nph = 1) {
   constexpr int BK = sizeof(T) == 8 ? 8 : 16;
 #define MG_OCC(TT, BM, BN, WM, WN) \
   if (bm == BM && bn == BN) return resident_blocks(tap_gemm_kernel<TT, BM, BN, BK, WM, WN>, 512);
+#define MG_OCC2(TT, BM, BN, WM, WN) \
+  if (bm == BM && bn == BN) return resident_blocks(tap_gemm_kernel<TT, BM, BN, BK, WM, WN, 2>, 512);
+#define MG_OCC4(TT, BM, BN, WM, WN) \
+  if (bm == BM && bn == BN) return resident_blocks(tap_gemm_kernel<TT, BM, BN, BK, WM, WN, 4>, 512);
+  if constexpr (sizeof(T) == 4) {
+    if (nph == 2) {
+      MG_FUSED2_SHAPES(T, MG_OCC2)
+      return 1;
+    }
+    if (nph == 4) {
+      MG_FUSED4_SHAPES(T, MG_OCC4)
+      return 1;
+    }
+  }
   MG_GEMM_SHAPES(T, MG_OCC)
 #undef MG_OCC
+#undef MG_OCC2
+#undef MG_OCC4
   return 1;
 }
 
@@ -641,25 +675,30 @@ struct TileChoice {
   long long tiles;
 };
 
-TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_ktiles, bool tap_major, size_t elem) {
+TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_ktiles, bool tap_major, size_t elem, int nph = 1) {
   struct Cfg {
     int bm, bn;
     double penalty;  // relative cost of a flop in this tile shape
     bool tap_only;
   };
-  static const Cfg cfgs[] = {{128, 128, 1.00, false}, {128, 64, 1.05, true}, {64, 256, 1.00, false}, {64, 128, 1.08, true},
-                             {32, 256, 1.00, false},  {32, 128, 1.10, true}, {16, 256, 1.00, false}};
-  const int bm = pick_bm(M);
+  static const Cfg plain[] = {{128, 128, 1.00, false}, {128, 64, 1.05, true}, {64, 256, 1.00, false}, {64, 128, 1.08, true},
+                              {32, 256, 1.00, false},  {32, 128, 1.10, true}, {16, 256, 1.00, false}};
+  static const Cfg fused2[] = {{128, 64, 1.05, true}, {64, 128, 1.08, true}, {32, 256, 1.00, true}, {16, 256, 1.00, true}};
+  static const Cfg fused4[] = {{64, 64, 1.10, true}, {32, 128, 1.10, true}, {16, 256, 1.00, true}};
+  const Cfg *cfgs = nph == 4 ? fused4 : nph == 2 ? fused2 : plain;
+  const int ncfgs = nph == 4 ? 3 : nph == 2 ? 4 : 7;
+  const int bm = nph == 4 ? std::min(pick_bm(M), 64) : pick_bm(M);
   const int cus = runtime().props.multiProcessorCount;
   TileChoice best{};
   double best_cost = 0;
-  for (const Cfg &c : cfgs) {
+  for (int ci = 0; ci < ncfgs; ++ci) {
+    const Cfg &c = cfgs[ci];
     if (c.bm != bm || (c.tap_only && !tap_major)) continue;
     // 64x64 fp64 wave tiles hold 128 accumulator registers: only one 8-wave block
     // fits on a compute unit, so the tap-major kernels use the half-size shapes
     if (tap_major && elem == 8 && c.bn * c.bm >= 128 * 128) continue;
     const bool stream = tap_major && tap_gemm_streams(c.bm, (int)elem);
-    const int per_cu = !stream ? 1 : elem == 8 ? gemm_blocks_per_cu<double>(c.bm, c.bn) : gemm_blocks_per_cu<float>(c.bm, c.bn);
+    const int per_cu = !stream ? 1 : elem == 8 ? gemm_blocks_per_cu<double>(c.bm, c.bn) : gemm_blocks_per_cu<float>(c.bm, c.bn, nph);
     long long pos_blocks = 0;
     for (long long n : phase_npos) pos_blocks += ceil_div(n, c.bn);
     for (int r = 1; r <= per_cu; ++r) {
@@ -678,7 +717,7 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
         tail = (double)ceil_div(rem, cus);
         if (tap_major) {
           // slices of at least two K tiles, at most 32 MB of partial sums
-          const long long tile_bytes = (long long)c.bm * c.bn * (long long)elem;
+          const long long tile_bytes = (long long)c.bm * c.bn * (long long)elem * nph;
           const int smax = (int)std::max<long long>(1, std::min<long long>({(long long)min_ktiles / 2, 32ll, (32ll << 20) / (rem * tile_bytes)}));
           for (int sp = 2; sp <= smax; ++sp) {
             const double share = (double)ceil_div(rem * sp, cus) / sp + 0.01 * sp;  // + a little for the fix-up pass
@@ -697,6 +736,35 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
       if (best.bm == 0 || cost < best_cost) {
         best = t;
         best_cost = cost;
+      }
+      // The same grid with the tail counted per unit instead of per round of the grid: blocks
+      // b, b + CUs, ... share a unit, so a unit gets the tiles t = b (mod CUs): q = T / CUs whole
+      // tiles each, and only the T mod CUs tiles beyond that are cut into slices (at most one
+      // slice per unit: little partial-sum traffic).  Within a unit the r blocks take q / r tiles
+      // each; if r does not divide q the last q mod r tiles run with fewer blocks than r.
+      if (stream && r > 1 && rem > 0) {
+        TileChoice u = t;
+        const long long q = u.tiles / cus, left = u.tiles % cus;
+        const int over = (int)(q % r);
+        double time = (double)(q / r) * r + (over == 1 ? 1.4 : (double)over);
+        u.full_tiles = (int)u.tiles;
+        u.tail_split = 1;
+        if (left > 0) {
+          double share = 1.0;
+          const long long tile_bytes = (long long)c.bm * c.bn * (long long)elem * nph;
+          const int smax = (int)std::max<long long>(1, std::min<long long>({(long long)min_ktiles / 2, 32ll, (32ll << 20) / (left * tile_bytes)}));
+          for (int sp = 2; sp <= smax; ++sp) {
+            const double sh = (double)ceil_div(left * sp, cus) / sp + 0.01 * sp;
+            if (sh < share - 1e-9) share = sh, u.tail_split = sp;
+          }
+          if (u.tail_split > 1) u.full_tiles = (int)(q * cus);
+          time += share;
+        }
+        const double ucost = time * c.bm * c.bn * c.penalty;
+        if (q > 0 && ucost < best_cost) {
+          best = u;
+          best_cost = ucost;
+        }
       }
     }
   }
@@ -864,6 +932,73 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
         set_divisors(pt.ph);
         found.push_back(pt);
       }
+
+  // ---- stride 2 along the last axis: the phases' elements alternate in dx, and phases that
+  // write them at different times make every line of dx cross HBM several times, partly
+  // filled.  With 2 or 4 phases in all, every tile computes all of them for its patch of the
+  // coarse grid J = ceil(X / stride) and writes them together (float only: one set of
+  // accumulators per phase has to fit next to the other registers).
+  static const bool fuse_on = [] {
+    const char *flag = getenv("MYGRAD_HIP_FUSE");
+    return !(flag && flag[0] == '0');
+  }();
+  const bool fused = fuse_on && pl.tap_major && g.dtype == MG_F32 && g.S[2] == 2 && g.S[0] <= 2 && g.S[1] <= 2 &&
+                     (nphase == 2 || nphase == 4) && (long long)found.size() == nphase;
+  if (fused) {
+    std::stable_sort(found.begin(), found.end(), [](const PhaseTaps &a, const PhaseTaps &b) {
+      if (a.ph.o0[0] != b.ph.o0[0]) return a.ph.o0[0] < b.ph.o0[0];
+      if (a.ph.o0[1] != b.ph.o0[1]) return a.ph.o0[1] < b.ph.o0[1];
+      return a.ph.o0[2] < b.ph.o0[2];
+    });
+    pl.nph = (int)nphase;
+    Phase coarse{};
+    long long total_ktiles = 0;
+    for (int k = 0; k < 3; ++k) coarse.J[k] = (g.X[k] + g.S[k] - 1) / g.S[k];
+    int taps_so_far = 0;
+    for (int f = 0; f < pl.nph; ++f) {
+      const PhaseTaps &pt = found[f];
+      for (int k = 0; k < 3; ++k) {
+        pl.po0[f][k] = pt.ph.o0[k];
+        pl.pJ[f][k] = pt.ph.J[k];
+      }
+      taps_so_far += (int)(pt.taps[0].size() * pt.taps[1].size() * pt.taps[2].size());
+      pl.kcut[f] = taps_so_far;  // every filter tap belongs to exactly one phase: W taps in all
+    }
+    // filter block outermost, then the phases, then a phase's taps: all taps of one filter block
+    // read the same neighbourhood of grad, whichever phase they belong to
+    for (int f0 = 0; f0 < g.F; f0 += bk)
+      for (int f = 0; f < pl.nph; ++f) {
+        const PhaseTaps &pt = found[f];
+        for (size_t a = 0; a < pt.taps[0].size(); ++a)
+          for (size_t b = 0; b < pt.taps[1].size(); ++b)
+            for (size_t c = 0; c < pt.taps[2].size(); ++c) {
+              const int tflat = (pt.taps[0][a] * g.W[1] + pt.taps[1][b]) * g.W[2] + pt.taps[2][c];
+              KTile e{};
+              e.d0 = pt.offs[0][a];
+              e.d1 = pt.offs[1][b];
+              e.d2 = pt.offs[2][c];
+              e.a_row0 = tflat * g.F + f0;
+              e.coff = (int)(f0 * g.gvol) + e.d0 * gs[0] + e.d1 * gs[1] + e.d2 * gs[2];
+              t.ktiles.push_back(e);
+            }
+      }
+    total_ktiles = (long long)t.ktiles.size();
+    coarse.k_begin = 0;
+    coarse.k_count = (int)total_ktiles;
+    coarse.blk_begin = 0;
+    coarse.npos = (int)((long long)g.N * coarse.J[0] * coarse.J[1] * coarse.J[2]);
+    set_divisors(coarse);
+    const TileChoice tc = choose_tile(g.C, {(long long)coarse.npos}, (int)total_ktiles, true, 4, pl.nph);
+    if (tc.bm != 0 && total_ktiles > 0) {
+      pl.bm = tc.bm, pl.bn = tc.bn, pl.m_tiles = tc.m_tiles, pl.full_tiles = tc.full_tiles, pl.tail_split = tc.tail_split, pl.blocks_per_cu = tc.blocks_per_cu;
+      t.phases.push_back(coarse);
+      pl.pos_blocks = (int)ceil_div(coarse.npos, pl.bn);
+      return upload_plan(pl, t);
+    }
+    // no tile shape for this row count: the phases run one after the other
+    pl.nph = 1;
+    t.ktiles.clear();
+  }
 
   // Phases with more taps have longer K loops; their blocks go first so that the
   // short ones fill in at the end (blocks are dispatched in index order).
@@ -1070,28 +1205,28 @@ int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
     // MYGRAD_HIP_TRACE=1 reports, once per new descriptor, what was planned
     static const bool trace = getenv("MYGRAD_HIP_TRACE") != nullptr;
     if (trace)
-      fprintf(stderr, "[mygrad_hip] %s plan: %s tile %dx%d, %d phase(s), %d position blocks x %d row tiles, %d whole tiles + tail split %d, K splits %d (chunk %d)\n",
+      fprintf(stderr, "[mygrad_hip] %s plan: %s tile %dx%d, %d phase(s) (%d fused per tile), %d position blocks x %d row tiles, %d whole tiles + tail split %d, %d block(s) per unit, K splits %d (chunk %d)\n",
               op == OP_FWD ? "fwd" : op == OP_DGRAD ? "dgrad" : "wgrad", pl.tap_major ? "tap-major" : "table-driven", pl.bm,
-              pl.bn, pl.nphases, pl.pos_blocks, pl.m_tiles, pl.full_tiles, pl.tail_split, pl.splits, pl.kchunk);
+              pl.bn, pl.nphases, pl.nph, pl.pos_blocks, pl.m_tiles, pl.full_tiles, pl.tail_split, pl.blocks_per_cu, pl.splits, pl.kchunk);
     it = plans().emplace(key, pl).first;
   }
   *out = &it->second;
   return MG_OK;
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int NPH = 1>
 void launch_gemm(GemmParams &gp, const Plan &pl, hipStream_t s) {
   if (pl.tap_major) {
     const long long tiles = (long long)pl.pos_blocks * pl.m_tiles;
     const long long tail_tiles = tiles - pl.full_tiles;
     const long long slots = tap_gemm_streams(BM, (int)sizeof(T)) ? (long long)pl.blocks_per_cu * runtime().props.multiProcessorCount : (1ll << 40);
     gp.items = (int)(pl.full_tiles + tail_tiles * pl.tail_split);
-    hipLaunchKernelGGL((tap_gemm_kernel<T, BM, BN, BK, WM, WN>), dim3((unsigned)std::min<long long>(gp.items, slots)), dim3(512),
+    hipLaunchKernelGGL((tap_gemm_kernel<T, BM, BN, BK, WM, WN, NPH>), dim3((unsigned)std::min<long long>(gp.items, slots)), dim3(512),
                        0, s, gp);
     if (tail_tiles > 0)
-      hipLaunchKernelGGL((tail_fixup_kernel<T, BM, BN>), dim3((unsigned)ceil_div(BM * BN, 256), (unsigned)tail_tiles),
+      hipLaunchKernelGGL((tail_fixup_kernel<T, BM, BN, NPH>), dim3((unsigned)ceil_div(BM * BN, 256), (unsigned)tail_tiles),
                          dim3(256), 0, s, gp);
-  } else {
+  } else if constexpr (NPH == 1) {
     const dim3 grid((unsigned)pl.pos_blocks, (unsigned)pl.m_tiles);
     hipLaunchKernelGGL((gather_gemm_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, gp);
   }
@@ -1100,7 +1235,7 @@ void launch_gemm(GemmParams &gp, const Plan &pl, hipStream_t s) {
 // Bytes of partial sums the shared tail tiles of this plan need.
 size_t tail_bytes(const Plan &pl, size_t elem) {
   const long long tail_tiles = (long long)pl.pos_blocks * pl.m_tiles - pl.full_tiles;
-  return pl.tap_major ? (size_t)tail_tiles * pl.tail_split * pl.bm * pl.bn * elem : 0;
+  return pl.tap_major ? (size_t)tail_tiles * pl.tail_split * pl.nph * pl.bm * pl.bn * elem : 0;
 }
 
 template <typename T>
@@ -1121,6 +1256,17 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
   // and every row starts 16-byte aligned)
   gp.vec_store = pl.single_dense_phase && gp.dst_mstride % 4 == 0 && gp.dst_nstride % 4 == 0 &&
                  reinterpret_cast<uintptr_t>(gp.dst) % 16 == 0;
+  gp.nph = pl.nph;
+  if (pl.nph > 1) {
+    for (int f = 0; f < 4; ++f) {
+      gp.kcut[f] = pl.kcut[f];
+      for (int k = 0; k < 3; ++k) gp.po0[f][k] = pl.po0[f][k], gp.pJ[f][k] = pl.pJ[f][k];
+    }
+    // the two phases of a pair have the same positions (an even extent along the last axis),
+    // and 2 * TN adjacent elements of a row of dst start 16-byte aligned
+    gp.vec_store = pl.pJ[0][2] == pl.pJ[1][2] && gp.os[1] % 4 == 0 && gp.os[0] % 4 == 0 && gp.dst_mstride % 4 == 0 &&
+                   gp.dst_nstride % 4 == 0 && reinterpret_cast<uintptr_t>(gp.dst) % 16 == 0;
+  }
   ScopedTiming timed(tag);
   bool launched = false;
 #define MG_LAUNCH(TT, BM, BN, WM, WN)                     \
@@ -1128,8 +1274,29 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
     launch_gemm<TT, BM, BN, BK, WM, WN>(gp, pl, s);       \
     launched = true;                                      \
   }
-  MG_GEMM_SHAPES(T, MG_LAUNCH)
+#define MG_LAUNCH2(TT, BM, BN, WM, WN)                    \
+  if (!launched && pl.bm == BM && pl.bn == BN) {          \
+    launch_gemm<TT, BM, BN, BK, WM, WN, 2>(gp, pl, s);    \
+    launched = true;                                      \
+  }
+#define MG_LAUNCH4(TT, BM, BN, WM, WN)                    \
+  if (!launched && pl.bm == BM && pl.bn == BN) {          \
+    launch_gemm<TT, BM, BN, BK, WM, WN, 4>(gp, pl, s);    \
+    launched = true;                                      \
+  }
+  if constexpr (sizeof(T) == 4) {
+    if (pl.nph == 2) {
+      MG_FUSED2_SHAPES(T, MG_LAUNCH2)
+    } else if (pl.nph == 4) {
+      MG_FUSED4_SHAPES(T, MG_LAUNCH4)
+    }
+  }
+  if (pl.nph == 1) {
+    MG_GEMM_SHAPES(T, MG_LAUNCH)
+  }
 #undef MG_LAUNCH
+#undef MG_LAUNCH2
+#undef MG_LAUNCH4
   if (!launched) return fail(MG_ERR_UNSUPPORTED, "no kernel for tile %d x %d", pl.bm, pl.bn);
   MG_HIP(hipGetLastError());
   return MG_OK;

@@ -103,7 +103,16 @@ struct GemmParams {
   int items;            // work items: full_tiles whole tiles, then tail_split K slices of each remaining tile
   int full_tiles;       // tiles computed whole by one block each
   int tail_split;       // blocks that share each remaining tile (K slices), >= 1
-  void *partial;        // [tail tile][slice][BM][BN] partial sums of the shared tiles
+  void *partial;        // [tail tile][slice][phase][BM][BN] partial sums of the shared tiles
+  // Fused stride phases (data gradient with a stride, tap-major kernel with NPH > 1): the phase
+  // table holds ONE phase, the coarse grid J[k] = ceil(X[k] / stride[k]); every tile computes all
+  // nph stride phases of its coarse positions, one accumulator set each, and writes them together,
+  // so that the interleaved elements of dx leave the block as whole runs.
+  int nph;              // 1 (not fused), 2 or 4; phases 2q and 2q+1 alternate along the last axis (po0[.][2] = 0, 1)
+  int kcut[4];          // a tile's K tiles run filter block by filter block, kcut[nph-1] tiles each (the taps of all
+                        // phases); tiles [kcut[f-1], kcut[f]) of a block belong to phase f (kcut[-1] = 0)
+  int po0[4][3];        // destination coordinate of coarse position (0,0,0) in phase f
+  int pJ[4][3];         // coarse positions j_k < pJ[f][k] exist in phase f
 };
 
 // Filter gradient:  out[split][f][col] = sum over the split's positions (n, g) of

@@ -129,8 +129,12 @@ struct Quad {
 // ------------------------------------------------------------------------------------------
 // forward and data gradient
 // ------------------------------------------------------------------------------------------
-template <typename T, int BM, int BN, int BK, int WM, int WN>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int NPH = 1>
 __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
+  // NPH > 1: every tile computes NPH stride phases of the data gradient (see GemmParams::nph):
+  // the K tiles of the phases follow each other in the tile's stream, each phase has its own
+  // accumulators, and the epilogue writes the phases together.
+  static_assert(NPH == 1 || NPH == 2 || NPH == 4, "1, 2 or 4 fused stride phases");
   // Tiles of 64 rows and more, and all double-precision tiles, run as persistent
   // blocks (see below).  The short float tiles of thin filter banks get one block per
   // item instead: moving the gather on to the next item from inside the K loop keeps
@@ -328,18 +332,32 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
     const int pos0 = it.pos0, m0 = it.m0;
     const int j12 = ph.J[1] * ph.J[2];
     const int jvol = ph.J[0] * j12;
-    auto dst_of = [&](int ipos) -> T * {
+    // position -> sample and grid coordinates of its phase (the coarse grid when phases are fused)
+    auto split_pos = [&](int ipos, int &n, int &j0, int &j1, int &j2) {
       const unsigned pos = (unsigned)ipos;
-      const unsigned n = ph.by_jvol.div(pos);
-      unsigned r = pos - n * (unsigned)jvol;
-      const int j0 = (int)ph.by_j12.div(r);
+      const unsigned nn = ph.by_jvol.div(pos);
+      unsigned r = pos - nn * (unsigned)jvol;
+      j0 = (int)ph.by_j12.div(r);
       r -= (unsigned)j0 * (unsigned)j12;
-      const int j1 = (int)ph.by_j2.div(r);
-      const int j2 = (int)r - j1 * ph.J[2];
+      j1 = (int)ph.by_j2.div(r);
+      j2 = (int)r - j1 * ph.J[2];
+      n = (int)nn;
+    };
+    auto dst_of = [&](int ipos) -> T * {
+      int n, j0, j1, j2;
+      split_pos(ipos, n, j0, j1, j2);
       return dst + (long long)n * p.dst_nstride + (long long)(ph.o0[0] + j0 * p.oj[0]) * p.os[0] +
              (long long)(ph.o0[1] + j1 * p.oj[1]) * p.os[1] + (long long)(ph.o0[2] + j2 * p.oj[2]) * p.os[2];
     };
-    T *slot = static_cast<T *>(p.partial) + ((long long)(it.tile - p.full_tiles) * p.tail_split + it.piece) * (BM * BN);
+    // fused phases: where coarse position (n, j) of phase f lies in dst, and whether it exists
+    auto fused_dst = [&](int f, int n, int j0, int j1, int j2) -> T * {
+      return dst + (long long)n * p.dst_nstride + (long long)(p.po0[f][0] + j0 * p.oj[0]) * p.os[0] +
+             (long long)(p.po0[f][1] + j1 * p.oj[1]) * p.os[1] + (long long)(p.po0[f][2] + j2 * p.oj[2]) * p.os[2];
+    };
+    auto fused_ok = [&](int f, int j0, int j1, int j2) -> bool {
+      return (j0 < p.pJ[f][0]) & (j1 < p.pJ[f][1]) & (j2 < p.pJ[f][2]);
+    };
+    T *slot = static_cast<T *>(p.partial) + ((long long)(it.tile - p.full_tiles) * p.tail_split + it.piece) * (NPH * BM * BN);
 
     if constexpr (sizeof(T) == 8) {
       // The wave tile is cut into 8-row and 8-column groups; group pairs are interleaved
@@ -349,12 +367,15 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
       const int arow = wm0 + Quad::feed_row(l16) * 2;
       const int bcol8 = wn0 + Quad::feed_col(l16) * 2;
       const int drow = wm0 + Quad::held_row(l16, lk) * 2;
-      double acc[GM][GN];
+      double acc[NPH][GM][GN];
 #pragma unroll
-      for (int i = 0; i < GM; ++i)
+      for (int f = 0; f < NPH; ++f)
 #pragma unroll
-        for (int j = 0; j < GN; ++j) acc[i][j] = 0.0;
-      for (int kt = it.kt_begin; kt < it.kt_end; ++kt) {
+        for (int i = 0; i < GM; ++i)
+#pragma unroll
+          for (int j = 0; j < GN; ++j) acc[f][i][j] = 0.0;
+      auto step = [&](auto fc) {  // one K tile into accumulator set f
+        constexpr int f = decltype(fc)::value;
 #pragma unroll
         for (int k4 = 0; k4 < BK / 4; ++k4) {
           T a[GM], b[GN];
@@ -373,35 +394,95 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
 #pragma unroll
           for (int i = 0; i < GM; ++i)
 #pragma unroll
-            for (int j = 0; j < GN; ++j) acc[i][j] = Quad::run(a[i], b[j], acc[i][j]);
+            for (int j = 0; j < GN; ++j) acc[f][i][j] = Quad::run(a[i], b[j], acc[f][i][j]);
         }
         __syncthreads();
         buf ^= 1;
+      };
+      if constexpr (NPH == 1) {
+        for (int kt = it.kt_begin; kt < it.kt_end; ++kt) step(std::integral_constant<int, 0>{});
+      } else {
+        // K tiles of a fused tile run filter block by filter block; inside a block the taps
+        // of phase 0 come first, then those of phase 1, ...: tile `off` of a block belongs to
+        // the phase f with kcut[f - 1] <= off < kcut[f].
+        int kt = it.kt_begin;
+        int off = kt % p.kcut[NPH - 1];
+        while (kt < it.kt_end) {
+          for (; off < p.kcut[0] && kt < it.kt_end; ++off, ++kt) step(std::integral_constant<int, 0>{});
+          for (; off < p.kcut[1] && kt < it.kt_end; ++off, ++kt) step(std::integral_constant<int, 1>{});
+          if constexpr (NPH == 4) {
+            for (; off < p.kcut[2] && kt < it.kt_end; ++off, ++kt) step(std::integral_constant<int, 2>{});
+            for (; off < p.kcut[3] && kt < it.kt_end; ++off, ++kt) step(std::integral_constant<int, 3>{});
+          }
+          off = 0;
+        }
       }
-      // ---- epilogue: acc[i][j] is row drow + (i/2)*16 + i%2, column bcol8 + (j/2)*16 + j%2
+      // ---- epilogue: acc[.][i][j] is row drow + (i/2)*16 + i%2, column bcol8 + (j/2)*16 + j%2
       if (it.partial) {
 #pragma unroll
-        for (int i = 0; i < GM; ++i) {
-          const int ml = drow + (i / 2) * 16 + i % 2;
+        for (int f = 0; f < NPH; ++f)
 #pragma unroll
-          for (int g = 0; g < GN / 2; ++g) {
-            const T two[2] = {acc[i][2 * g], acc[i][2 * g + 1]};
-            store_vec<T, 2>(slot + ml * BN + bcol8 + g * 16, two);
+          for (int i = 0; i < GM; ++i) {
+            const int ml = drow + (i / 2) * 16 + i % 2;
+#pragma unroll
+            for (int g = 0; g < GN / 2; ++g) {
+              const T two[2] = {acc[f][i][2 * g], acc[f][i][2 * g + 1]};
+              store_vec<T, 2>(slot + f * (BM * BN) + ml * BN + bcol8 + g * 16, two);
+            }
           }
-        }
         continue;
       }
 #pragma unroll
       for (int g = 0; g < GN / 2; ++g) {
         const int first = pos0 + bcol8 + g * 16;
-        if (p.vec_store) {
+        if constexpr (NPH > 1) {
+          if (p.vec_store && ph.J[2] % 2 == 0) {
+            // both coarse positions exist, lie in one row, and their phases are adjacent in dst
+            if (first >= ph.npos) continue;
+            int n, j0, j1, j2;
+            split_pos(first, n, j0, j1, j2);
+            // phases f and f+1 alternate along the last axis: four adjacent elements of dst
+#pragma unroll
+            for (int f = 0; f < NPH; f += 2) {
+              if (!fused_ok(f, j0, j1, j2)) continue;
+              T *out = fused_dst(f, n, j0, j1, j2);
+#pragma unroll
+              for (int i = 0; i < GM; ++i) {
+                const int m = m0 + drow + (i / 2) * 16 + i % 2;
+                const T lo[2] = {acc[f][i][2 * g], acc[f + 1][i][2 * g]};
+                const T hi[2] = {acc[f][i][2 * g + 1], acc[f + 1][i][2 * g + 1]};
+                if (m < p.M) {
+                  store_vec<T, 2>(out + (long long)m * p.dst_mstride, lo);
+                  store_vec<T, 2>(out + (long long)m * p.dst_mstride + 2, hi);
+                }
+              }
+            }
+          } else {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              if (first + h >= ph.npos) continue;
+              int n, j0, j1, j2;
+              split_pos(first + h, n, j0, j1, j2);
+#pragma unroll
+              for (int f = 0; f < NPH; ++f) {
+                if (!fused_ok(f, j0, j1, j2)) continue;
+                T *out = fused_dst(f, n, j0, j1, j2);
+#pragma unroll
+                for (int i = 0; i < GM; ++i) {
+                  const int m = m0 + drow + (i / 2) * 16 + i % 2;
+                  if (m < p.M) out[(long long)m * p.dst_mstride] = acc[f][i][2 * g + h];
+                }
+              }
+            }
+          }
+        } else if (p.vec_store) {
           // both positions exist (npos % 4 == 0) and are adjacent in dst
           if (first >= ph.npos) continue;
           T *out = dst_of(first);
 #pragma unroll
           for (int i = 0; i < GM; ++i) {
             const int m = m0 + drow + (i / 2) * 16 + i % 2;
-            const T two[2] = {acc[i][2 * g], acc[i][2 * g + 1]};
+            const T two[2] = {acc[0][i][2 * g], acc[0][i][2 * g + 1]};
             if (m < p.M) store_vec<T, 2>(out + (long long)m * p.dst_mstride, two);
           }
         } else {
@@ -412,7 +493,7 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
 #pragma unroll
             for (int i = 0; i < GM; ++i) {
               const int m = m0 + drow + (i / 2) * 16 + i % 2;
-              if (m < p.M) out[(long long)m * p.dst_mstride] = acc[i][2 * g + h];
+              if (m < p.M) out[(long long)m * p.dst_mstride] = acc[0][i][2 * g + h];
             }
           }
         }
@@ -421,12 +502,15 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
       // Lane (l16, lk) feeds row/column l16 of every 16x16 tile.  Tile i of the wave
       // takes the rows m = wm0 + l16*TM + i (and tile j the positions wn0 + l16*TN + j),
       // so the TM (TN) operands of a lane are adjacent in LDS and come in one read.
-      typename Mma<T>::Acc acc[TM][TN];
+      typename Mma<T>::Acc acc[NPH][TM][TN];
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+      for (int f = 0; f < NPH; ++f)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = typename Mma<T>::Acc{0, 0, 0, 0};
-      for (int kt = it.kt_begin; kt < it.kt_end; ++kt) {
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) acc[f][i][j] = typename Mma<T>::Acc{0, 0, 0, 0};
+      auto step = [&](auto fc) {  // one K tile into accumulator set f
+        constexpr int f = decltype(fc)::value;
 #pragma unroll
         for (int k4 = 0; k4 < BK / 4; ++k4) {
           T a[TM], b[TN];
@@ -435,30 +519,102 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
 #pragma unroll
           for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::run(a[i], b[j], acc[i][j]);
+            for (int j = 0; j < TN; ++j) acc[f][i][j] = Mma<T>::run(a[i], b[j], acc[f][i][j]);
         }
         __syncthreads();
         buf ^= 1;
+      };
+      if constexpr (NPH == 1) {
+        for (int kt = it.kt_begin; kt < it.kt_end; ++kt) step(std::integral_constant<int, 0>{});
+      } else {
+        // K tiles of a fused tile run filter block by filter block; inside a block the taps
+        // of phase 0 come first, then those of phase 1, ...: tile `off` of a block belongs to
+        // the phase f with kcut[f - 1] <= off < kcut[f].
+        int kt = it.kt_begin;
+        int off = kt % p.kcut[NPH - 1];
+        while (kt < it.kt_end) {
+          for (; off < p.kcut[0] && kt < it.kt_end; ++off, ++kt) step(std::integral_constant<int, 0>{});
+          for (; off < p.kcut[1] && kt < it.kt_end; ++off, ++kt) step(std::integral_constant<int, 1>{});
+          if constexpr (NPH == 4) {
+            for (; off < p.kcut[2] && kt < it.kt_end; ++off, ++kt) step(std::integral_constant<int, 2>{});
+            for (; off < p.kcut[3] && kt < it.kt_end; ++off, ++kt) step(std::integral_constant<int, 3>{});
+          }
+          off = 0;
+        }
       }
 
       // ---- epilogue
       if (it.partial) {
-        // raw tile [BM][BN] of this slice, lane's TN positions stored as one vector
+        // raw tile [BM][BN] of this slice (one per phase), lane's TN positions stored as one vector
         T *mine = slot + (wn0 + l16 * TN);
 #pragma unroll
-        for (int i = 0; i < TM; ++i)
+        for (int f = 0; f < NPH; ++f)
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int ml = wm0 + Mma<T>::row_of(lane, q) * TM + i;
-            T v[TN];
+          for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) v[j] = acc[i][j][q];
-            store_vec<T, TN>(mine + ml * BN, v);
-          }
+            for (int q = 0; q < 4; ++q) {
+              const int ml = wm0 + Mma<T>::row_of(lane, q) * TM + i;
+              T v[TN];
+#pragma unroll
+              for (int j = 0; j < TN; ++j) v[j] = acc[f][i][j][q];
+              store_vec<T, TN>(mine + f * (BM * BN) + ml * BN, v);
+            }
         continue;
       }
       const int first = pos0 + wn0 + l16 * TN;
-      if (p.vec_store) {
+      if constexpr (NPH > 1) {
+        if (p.vec_store && ph.J[2] % TN == 0) {
+          // the lane's TN coarse positions exist and lie in one row of the coarse grid
+          if (first < ph.npos) {
+            int n, j0, j1, j2;
+            split_pos(first, n, j0, j1, j2);
+            // phases f and f+1 alternate along the last axis: 2*TN adjacent elements of dst
+#pragma unroll
+            for (int f = 0; f < NPH; f += 2) {
+              if (!fused_ok(f, j0, j1, j2)) continue;
+              T *out = fused_dst(f, n, j0, j1, j2);
+#pragma unroll
+              for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                  const int m = m0 + wm0 + Mma<T>::row_of(lane, q) * TM + i;
+                  if (m < p.M) {
+                    constexpr int PER = TN < 2 ? TN : 2;  // coarse positions per 16-byte store
+#pragma unroll
+                    for (int h = 0; h < TN / PER; ++h) {
+                      T v[2 * PER];
+#pragma unroll
+                      for (int t = 0; t < PER; ++t) {
+                        v[2 * t] = acc[f][i][h * PER + t][q];
+                        v[2 * t + 1] = acc[f + 1][i][h * PER + t][q];
+                      }
+                      store_vec<T, 2 * PER>(out + (long long)m * p.dst_mstride + 2 * h * PER, v);
+                    }
+                  }
+                }
+            }
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            if (first + j >= ph.npos) continue;
+            int n, j0, j1, j2;
+            split_pos(first + j, n, j0, j1, j2);
+#pragma unroll
+            for (int f = 0; f < NPH; ++f) {
+              if (!fused_ok(f, j0, j1, j2)) continue;
+              T *out = fused_dst(f, n, j0, j1, j2);
+#pragma unroll
+              for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                  const int m = m0 + wm0 + Mma<T>::row_of(lane, q) * TM + i;
+                  if (m < p.M) out[(long long)m * p.dst_mstride] = acc[f][i][j][q];
+                }
+            }
+          }
+        }
+      } else if (p.vec_store) {
         // the TN positions of this lane are adjacent in dst and all exist (npos % TN == 0)
         if (first < ph.npos) {
           T *out = dst_of(first);
@@ -470,7 +626,7 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
               if (m < p.M) {
                 T v[TN];
 #pragma unroll
-                for (int j = 0; j < TN; ++j) v[j] = acc[i][j][q];
+                for (int j = 0; j < TN; ++j) v[j] = acc[0][i][j][q];
                 store_vec<T, TN>(out + (long long)m * p.dst_mstride, v);
               }
             }
@@ -485,7 +641,7 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               const int m = m0 + wm0 + Mma<T>::row_of(lane, q) * TM + i;
-              if (m < p.M) out[(long long)m * p.dst_mstride] = acc[i][j][q];
+              if (m < p.M) out[(long long)m * p.dst_mstride] = acc[0][i][j][q];
             }
         }
       }
@@ -496,7 +652,7 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
 // Adds the K slices of the shared tail tiles in slice order (always the same order,
 // so results repeat exactly) and stores them where the tile's epilogue would have.
 // One thread per tile element; blockIdx.y is the tail tile.
-template <typename T, int BM, int BN>
+template <typename T, int BM, int BN, int NPH = 1>
 __global__ void __launch_bounds__(256) tail_fixup_kernel(const GemmParams p) {
   const int e = blockIdx.x * 256 + threadIdx.x;  // element of the [BM][BN] tile
   if (e >= BM * BN) return;
@@ -508,8 +664,6 @@ __global__ void __launch_bounds__(256) tail_fixup_kernel(const GemmParams p) {
   const int ipos = (pblk - ph.blk_begin) * BN + e % BN;
   const int m = (tile % p.m_tiles) * BM + e / BN;
   if (ipos >= ph.npos || m >= p.M) return;
-  const T *slot = static_cast<const T *>(p.partial) + (long long)blockIdx.y * p.tail_split * (BM * BN) + e;
-  const T sum = sum_in_order(slot, (long long)BM * BN, p.tail_split);
   const int j12 = ph.J[1] * ph.J[2];
   const unsigned pos = (unsigned)ipos;
   const unsigned n = ph.by_jvol.div(pos);
@@ -518,9 +672,17 @@ __global__ void __launch_bounds__(256) tail_fixup_kernel(const GemmParams p) {
   r -= (unsigned)j0 * (unsigned)j12;
   const int j1 = (int)ph.by_j2.div(r);
   const int j2 = (int)r - j1 * ph.J[2];
-  T *out = static_cast<T *>(p.dst) + (long long)n * p.dst_nstride + (long long)(ph.o0[0] + j0 * p.oj[0]) * p.os[0] +
-           (long long)(ph.o0[1] + j1 * p.oj[1]) * p.os[1] + (long long)(ph.o0[2] + j2 * p.oj[2]) * p.os[2];
-  out[(long long)m * p.dst_mstride] = sum;
+  const long long slice = (long long)NPH * BM * BN;  // elements of one K slice of a tile: one [BM][BN] per phase
+  const T *slot = static_cast<const T *>(p.partial) + (long long)blockIdx.y * p.tail_split * slice + e;
+#pragma unroll
+  for (int f = 0; f < NPH; ++f) {
+    const int o0 = NPH == 1 ? ph.o0[0] : p.po0[f][0], o1 = NPH == 1 ? ph.o0[1] : p.po0[f][1], o2 = NPH == 1 ? ph.o0[2] : p.po0[f][2];
+    if (NPH > 1 && !((j0 < p.pJ[f][0]) & (j1 < p.pJ[f][1]) & (j2 < p.pJ[f][2]))) continue;
+    const T sum = sum_in_order(slot + (long long)f * (BM * BN), slice, p.tail_split);
+    T *out = static_cast<T *>(p.dst) + (long long)n * p.dst_nstride + (long long)(o0 + j0 * p.oj[0]) * p.os[0] +
+             (long long)(o1 + j1 * p.oj[1]) * p.os[1] + (long long)(o2 + j2 * p.oj[2]) * p.os[2];
+    out[(long long)m * p.dst_mstride] = sum;
+  }
 }
 
 // ------------------------------------------------------------------------------------------

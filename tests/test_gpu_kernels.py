@@ -302,6 +302,43 @@ def test_conv_channel_counts_that_take_the_tap_major_kernels(abi, dtype, m):
         done += 1
 
 
+# Stride 2 along the last axis (float32, filter count a multiple of 16): every tile of the data
+# gradient computes all 2 / 4 stride phases of its patch and writes them interleaved.  Even and
+# odd extents (vector and element-wise stores, phases with fewer positions than the coarse grid),
+# 1, 2 and 3 convolved axes, channel counts for every fused tile shape (16 .. 128 rows), filters
+# with taps that some phases never see (1x1: three of four phases are all zero), dilation, and
+# enough positions for persistent blocks, tail tiles and K slices.
+FUSED_PHASE_CASES = [
+    ((4, 64, 28, 28), (32, 64, 3, 3), (2, 2), (1, 1), (1, 1)),
+    ((3, 128, 27, 27), (48, 128, 3, 3), (2, 2), (1, 1), (1, 1)),
+    ((2, 32, 30, 36), (16, 32, 1, 1), (2, 2), (0, 0), (1, 1)),
+    ((5, 16, 19, 24), (64, 16, 5, 3), (2, 2), (2, 1), (1, 2)),
+    ((2, 48, 40, 44), (32, 48, 2, 2), (1, 2), (0, 1), (1, 1)),
+    ((3, 64, 130), (16, 64, 7), (2,), (3,), (1,)),
+    ((2, 24, 9, 16, 20), (32, 24, 3, 3, 3), (1, 2, 2), (1, 1, 1), (1, 1, 1)),
+    ((40, 128, 28, 28), (256, 128, 3, 3), (2, 2), (1, 1), (1, 1)),
+    ((2, 8, 12, 10), (16, 8, 3, 3), (2, 2), (0, 0), (1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", range(len(FUSED_PHASE_CASES)))
+def test_conv_dgrad_with_fused_stride_phases(abi, case):
+    x_shape, w_shape, s, p, d = FUSED_PHASE_CASES[case]
+    rng = np.random.default_rng(900 + case)
+    w = (rng.standard_normal(w_shape) / np.sqrt(np.prod(w_shape[1:]))).astype(np.float32)
+    grid = tuple((x + 2 * pp - ((t - 1) * dd + 1)) // ss + 1 for x, t, ss, pp, dd in zip(x_shape[2:], w_shape[2:], s, p, d))
+    g = rng.standard_normal((x_shape[0], w_shape[0], *grid)).astype(np.float32)
+    dx = abi.conv_dgrad(g, x_shape, w, s, p, d)
+    assert rel_err(dx, direct.conv_backward_x(g, x_shape, w, s, p, d)) <= 2e-4
+    assert np.array_equal(dx, abi.conv_dgrad(g, x_shape, w, s, p, d))  # no atomics: run-to-run identical
+    # dx of an all-ones gradient counts, per input element, the windows that reach it: exact
+    # in float32 with a filter of ones, which isolates the routing from the rounding
+    ones_w = np.ones(w_shape, dtype=np.float32)
+    ones_g = np.ones_like(g)
+    assert np.array_equal(abi.conv_dgrad(ones_g, x_shape, ones_w, s, p, d),
+                          direct.conv_backward_x(ones_g, x_shape, ones_w, s, p, d).astype(np.float32))
+
+
 # Shapes picked so that, between them, every tile shape and code path of the tap-major
 # kernels runs: all gather-GEMM tiles (rows 16..128), persistent blocks that stream
 # through several tiles and K slices, strided dgrad phases, filter counts that are not a
