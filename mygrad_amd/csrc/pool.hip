@@ -8,6 +8,8 @@
 //                +0.0 and carried in double.
 #include "internal.h"
 
+#include <cstdlib>
+
 #include <algorithm>
 
 namespace mg {
@@ -658,6 +660,86 @@ __global__ void __launch_bounds__(256) maxpool_from_mark_kernel(PoolMarkParams p
   }
 }
 
+// The same gather for windows over the last two axes whose extent and step are known at compile
+// time (P0 = S0 = 1; P1 x P2 placed every S1, S2).  A thread owns a 16-byte piece of S1
+// consecutive rows of dx: the rows k*S1 .. k*S1 + S1 - 1 are covered by the same ceil(P1/S1)
+// window rows, and the piece's columns by the same ceil(P2/S2) - 1 + VD/S2 windows along the row,
+// whichever thread -- so their recorded offsets and gradients are loaded up front (clamped, never
+// predicated), and every element adds, in ascending window order, the gradient of the windows
+// whose recorded offset names it and +0.0 for the others: no loop bounds to compute, no
+// divisions by runtime values, no LDS.  Needs X2 % VD == 0 and VD % S2 == 0 (a piece starts on a
+// window boundary).
+struct PoolGatherParams {
+  int X1, X2, G1, G2;
+  int pieces;        // 16-byte pieces per row of dx
+  int groups;        // groups of S1 rows per plane: ceil(X1 / S1)
+  long long planes;  // lead * X0
+  FastDivP by_pieces, by_groups;
+};
+
+template <typename T, typename TD, int P1, int P2, int S1, int S2>
+__global__ void __launch_bounds__(256) maxpool_mark_gather_kernel(PoolGatherParams p, const unsigned char *__restrict__ mark,
+                                                                 const T *__restrict__ grad, TD *__restrict__ dx) {
+  constexpr int VD = 16 / sizeof(TD);
+  constexpr int C1 = (P1 + S1 - 1) / S1, C2 = (P2 + S2 - 1) / S2;
+  constexpr int NW2 = (VD - 1) / S2 + C2;  // windows along the row that can reach the piece
+  static_assert(VD % S2 == 0, "a piece starts on a window boundary");
+  typedef TD DVec __attribute__((ext_vector_type(VD)));
+  const long long item = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (item >= p.planes * p.groups * p.pieces) return;
+  const unsigned u = (unsigned)item;
+  const unsigned q = p.by_pieces.div(u), piece = u - q * (unsigned)p.pieces;
+  const unsigned plane = p.by_groups.div(q);
+  const int k = (int)(q - plane * (unsigned)p.groups);
+  const int i2 = (int)piece * VD;
+  const unsigned char *m = mark + (long long)plane * (p.G1 * p.G2);
+  const T *g = grad + (long long)plane * (p.G1 * p.G2);
+  const int g1_first = k - (C1 - 1), g2_first = i2 / S2 - (C2 - 1);
+
+  int code[C1][NW2];
+  double term[C1][NW2];
+#pragma unroll
+  for (int d = 0; d < C1; ++d) {
+    const int g1 = g1_first + d;
+    const bool ok1 = (g1 >= 0) & (g1 < p.G1);
+    const int r = min(max(g1, 0), p.G1 - 1) * p.G2;
+#pragma unroll
+    for (int e = 0; e < NW2; ++e) {
+      const int g2 = g2_first + e;
+      const bool ok = ok1 & (g2 >= 0) & (g2 < p.G2);
+      const int at = r + min(max(g2, 0), p.G2 - 1);
+      const int c = (int)m[at];
+      const double t = (double)g[at];
+      code[d][e] = ok ? c : -1;  // a window that does not exist names no element
+      term[d][e] = t;
+    }
+  }
+  TD *to = dx + ((long long)plane * p.X1 + (long long)k * S1) * p.X2 + i2;
+#pragma unroll
+  for (int rr = 0; rr < S1; ++rr) {
+    if (k * S1 + rr >= p.X1) break;
+    DVec out;
+#pragma unroll
+    for (int v = 0; v < VD; ++v) {
+      double acc = 0.0;
+#pragma unroll
+      for (int d = 0; d < C1; ++d) {
+        const int a1 = rr + (C1 - 1 - d) * S1;  // the row's offset inside window row d: known at compile time
+        if (a1 >= P1) continue;                 // that window row does not reach this row
+#pragma unroll
+        for (int e = 0; e < C2; ++e) {
+          const int w = v / S2 + e;                     // which of the loaded windows
+          const int a2 = (v % S2) + (C2 - 1 - e) * S2;   // the element's offset inside it
+          if (a2 >= P2) continue;
+          acc += code[d][w] == a1 * P2 + a2 ? term[d][w] : 0.0;  // + (+0.0) leaves a sum that started at +0.0 as it is
+        }
+      }
+      out[v] = (TD)acc;
+    }
+    *reinterpret_cast<DVec *>(to + (long long)rr * p.X2) = out;
+  }
+}
+
 // The same for windows that tile the input exactly: an element belongs to one window, so a
 // thread reads the recorded offsets and gradients of its 16 / (P2 * sizeof(T)) windows and
 // writes their P0 x P1 rows of dx.
@@ -1026,6 +1108,47 @@ static int maxpool_bwd_from_mark(const mg_pool_desc *desc, const unsigned char *
 #undef MG_POOL_EXACT_MARK
     MG_HIP(hipGetLastError());
     return MG_OK;
+  }
+  {
+    // windows over the last two axes with an extent and step that have a kernel instance: the
+    // gather with everything but the tensor's extents known at compile time
+    const int vd = (f32 && !wide) ? 4 : 2;
+    const long long rows = p.lead * p.X[0] * p.X[1];
+    static const bool gather_on = [] {
+      const char *flag = getenv("MYGRAD_HIP_POOL_GATHER");
+      return !(flag && flag[0] == '0');
+    }();
+    const int sig4 = ((p.P[1] * 10 + p.P[2]) * 10 + p.S[1]) * 10 + p.S[2];
+    if (gather_on && p.P[0] == 1 && p.S[0] == 1 && (sig4 == 3322 || sig4 == 3311 || sig4 == 2211) && p.X[2] % vd == 0 &&
+        vd % p.S[2] == 0 && reinterpret_cast<uintptr_t>(dx) % 16 == 0 && rows * (p.X[2] / vd) < (1ll << 31) &&
+        (long long)p.G[1] * p.G[2] < (1ll << 30)) {
+      PoolGatherParams q{};
+      q.X1 = p.X[1], q.X2 = p.X[2], q.G1 = p.G[1], q.G2 = p.G[2];
+      q.pieces = p.X[2] / vd;
+      q.groups = (int)ceil_div(p.X[1], p.S[1]);
+      q.planes = p.lead * p.X[0];
+      q.by_pieces = make_fastdiv_p((unsigned)q.pieces);
+      q.by_groups = make_fastdiv_p((unsigned)q.groups);
+      const dim3 grid((unsigned)ceil_div(q.planes * q.groups * q.pieces, 256)), block(256);
+#define MG_POOL_GATHER_SIG(T, TD, A, B, C, D) \
+  hipLaunchKernelGGL((maxpool_mark_gather_kernel<T, TD, A, B, C, D>), grid, block, 0, s, q, mark, (const T *)grad, (TD *)dx)
+#define MG_POOL_GATHER(T, TD)                                     \
+  do {                                                            \
+    if (sig4 == 3322) MG_POOL_GATHER_SIG(T, TD, 3, 3, 2, 2);      \
+    else if (sig4 == 3311) MG_POOL_GATHER_SIG(T, TD, 3, 3, 1, 1); \
+    else MG_POOL_GATHER_SIG(T, TD, 2, 2, 1, 1);                   \
+  } while (0)
+      if (!f32)
+        MG_POOL_GATHER(double, double);
+      else if (wide)
+        MG_POOL_GATHER(float, double);
+      else
+        MG_POOL_GATHER(float, float);
+#undef MG_POOL_GATHER
+#undef MG_POOL_GATHER_SIG
+      MG_HIP(hipGetLastError());
+      return MG_OK;
+    }
   }
   {
     PoolTileParams tp;

@@ -105,6 +105,39 @@ def test_pool_ties_and_overlap_bit_exact(pools, m, lead, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("lead,X,pool,stride", [
+    ((3, 2), (11, 16), (3, 3), (2, 2)),   # an odd number of rows: the last row group is half empty
+    ((5,), (56, 56), (3, 3), (2, 2)),     # the benchmark's plane (rows 55 and columns 55 are never covered)
+    ((2,), (9, 12), (3, 3), (1, 1)),      # every element under up to nine windows
+    ((4,), (7, 8), (2, 2), (1, 1)),
+    ((2,), (3, 6, 8), (1, 3, 3), (1, 2, 2)),  # a leading pooled axis of extent one folds into the planes
+    ((1,), (3, 4), (3, 3), (2, 2)),       # a single window per plane
+])
+def test_pool_backward_gather_for_windows_known_at_compile_time(pools, dtype, lead, X, pool, stride):
+    """2-D windows of 3x3 / stride 2, 3x3 / stride 1 and 2x2 / stride 1 over rows of whole 16-byte
+    pieces: the backward pass from the recorded argmax gathers per element in registers.  Ties,
+    NaNs, gradients of -0.0 and huge / tiny magnitudes (the order of the additions shows), the
+    float64 dx of a float32 input."""
+    rng = np.random.default_rng(370 + X[-1] + X[-2])
+    for trial in range(5):
+        if trial == 0:
+            x = rng.standard_normal((*lead, *X)).astype(dtype)
+        else:
+            x = rng.integers(0, 3, (*lead, *X)).astype(dtype)
+        if trial == 2:
+            x[rng.random(x.shape) < 0.1] = np.nan
+        out_shape = (*lead, *(((xk - pk) // sk + 1) for xk, pk, sk in zip(X, pool, stride)))
+        g = (rng.standard_normal(out_shape) * 10.0 ** rng.integers(-6, 6, out_shape)).astype(dtype)
+        if trial == 3:
+            g = rng.choice(np.array([1e16, 1.0, -1e16], dtype=dtype), out_shape)  # sums that depend on their order
+        g[rng.random(out_shape) < 0.2] = -0.0
+        want_dx = ora.pool_backward(x, g, pool, stride)  # float64
+        assert np.array_equal(bits(pools.pool_fwd(x, pool, stride)), bits(ora.pool_forward(x, pool, stride, validate=False)))
+        assert np.array_equal(bits(pools.pool_bwd(x, g, pool, stride, dx_dtype=np.float64)), bits(want_dx))
+        assert np.array_equal(bits(pools.pool_bwd(x, g, pool, stride)), bits(want_dx.astype(dtype)))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("lead,X,pool", [
     ((3, 5), (8, 12), (2, 2)),        # 2-D, rows of whole 16-byte pieces: the exact-tiling kernel
     ((2,), (6, 4, 8), (2, 2, 2)),     # 3-D
