@@ -660,6 +660,90 @@ __global__ void __launch_bounds__(256) maxpool_from_mark_kernel(PoolMarkParams p
   }
 }
 
+// Forward pass for windows over the last two axes whose extent and step are known at compile time
+// (P0 = S0 = 1; P1 x P2 placed every S1, S2), straight from global memory.  Lane l of a wavefront
+// takes the l-th 16-byte piece of a window row's P1 rows of x -- consecutive lanes, consecutive
+// pieces: every load of the wavefront is one contiguous run -- and reduces the VEC / S2 windows
+// that start inside its piece.  The P2 - S2 columns those reach beyond the piece come from the
+// next lane by a cross-lane move, not from memory; the last lane of a wavefront only supplies them
+// (the next wavefront starts on its piece again).  A window that would need columns of the next
+// row does not exist.  Every element of x crosses HBM once (rows shared by two window rows come
+// the second time out of L1 / L2); nothing is staged.
+// Needs X2 % VEC == 0, VEC % S2 == 0, P2 - S2 <= VEC and rows of x that start 16-byte aligned.
+#define POOL_ROWS_PER_THREAD 3
+struct PoolRowsParams {
+  int X1, X2, G1, G2;
+  int pieces;        // 16-byte pieces per row of x
+  int groups;        // groups of POOL_ROWS_PER_THREAD window rows per plane
+  long long planes;  // lead * X0
+  long long items;   // planes * groups * pieces: one per (group of window rows, piece)
+  FastDivP by_pieces, by_groups;
+};
+
+template <typename T>
+__device__ __forceinline__ T from_next_lane(T value) {
+  return __shfl_down(value, 1, 64);
+}
+
+template <typename T, int P1, int P2, int S1, int S2, bool MARK, bool STORE_OUT = true>
+__global__ void __launch_bounds__(256) maxpool_rows_fwd_kernel(PoolRowsParams p, const T *__restrict__ x, T *__restrict__ out,
+                                                              unsigned char *__restrict__ mark) {
+  constexpr int VEC = 16 / sizeof(T);
+  constexpr int WO = VEC / S2;   // windows that start inside a piece
+  constexpr int HALO = P2 - S2;  // columns the last of them reaches into the next piece
+  constexpr int RW = POOL_ROWS_PER_THREAD;   // window rows per thread: the rows two of them share are loaded once
+  constexpr int NR = (RW - 1) * S1 + P1;     // rows of x under them
+  static_assert(VEC % S2 == 0 && HALO >= 0 && HALO <= VEC, "piece / window geometry");
+  typedef T Vec __attribute__((ext_vector_type(VEC)));
+  const int lane = threadIdx.x & 63;
+  const long long wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const long long item = wave * 63 + lane;  // wavefronts overlap by one lane
+  const unsigned u = (unsigned)(item < p.items ? item : p.items - 1);  // clamped: every lane loads, some do not store
+  const unsigned q = p.by_pieces.div(u), piece = u - q * (unsigned)p.pieces;
+  const unsigned plane = p.by_groups.div(q);
+  const int g1_first = (int)(q - plane * (unsigned)p.groups) * RW;
+  const T *rows = x + (long long)plane * p.X1 * p.X2 + (int)piece * VEC;
+  const int row_first = g1_first * S1;
+  T v[NR][VEC + HALO];
+#pragma unroll
+  for (int r = 0; r < NR; ++r) {
+    // rows beyond the last one belong to window rows that do not exist: read the last row instead
+    const Vec mine = *reinterpret_cast<const Vec *>(rows + (long long)min(row_first + r, p.X1 - 1) * p.X2);
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[r][i] = mine[i];
+  }
+#pragma unroll
+  for (int r = 0; r < NR; ++r)
+#pragma unroll
+    for (int i = 0; i < HALO; ++i) v[r][VEC + i] = from_next_lane(v[r][i]);
+  if (lane == 63 || item >= p.items) return;
+#pragma unroll
+  for (int w = 0; w < RW; ++w) {
+    const int g1 = g1_first + w;
+    if (g1 >= p.G1) break;
+    const long long w0 = ((long long)plane * p.G1 + g1) * p.G2 + (long long)piece * WO;
+#pragma unroll
+    for (int t = 0; t < WO; ++t) {
+      T best = v[w * S1][t * S2];
+      int code = 0;
+#pragma unroll
+      for (int a1 = 0; a1 < P1; ++a1)
+#pragma unroll
+        for (int a2 = 0; a2 < P2; ++a2) {
+          const T c = v[w * S1 + a1][t * S2 + a2];
+          if (takes_over(c, best)) {
+            best = c;
+            code = a1 * P2 + a2;
+          }
+        }
+      if ((int)piece * WO + t < p.G2) {
+        if constexpr (STORE_OUT) out[w0 + t] = best;
+        if constexpr (MARK) mark[w0 + t] = (unsigned char)code;
+      }
+    }
+  }
+}
+
 // The same gather for windows over the last two axes whose extent and step are known at compile
 // time (P0 = S0 = 1; P1 x P2 placed every S1, S2).  A thread owns a 16-byte piece of S1
 // consecutive rows of dx: the rows k*S1 .. k*S1 + S1 - 1 are covered by the same ceil(P1/S1)
@@ -993,6 +1077,103 @@ static int exact_signature(const PoolParams &p, size_t elem, const void *a, cons
   return sig;
 }
 
+// ---- the kernels for 2-D windows known at compile time: when they apply, and their launches
+static int window_signature4(const PoolParams &p) { return ((p.P[1] * 10 + p.P[2]) * 10 + p.S[1]) * 10 + p.S[2]; }
+static bool has_rows_instance(const PoolParams &p) {
+  const int sig4 = window_signature4(p);
+  return p.P[0] == 1 && p.S[0] == 1 && (sig4 == 3322 || sig4 == 3311 || sig4 == 2211);
+}
+
+static bool rows_forward_applies(const PoolParams &p, bool f32, const void *x) {
+  static const bool on = [] {
+    const char *flag = getenv("MYGRAD_HIP_POOL_ROWS");
+    return !(flag && flag[0] == '0');
+  }();
+  const int vec = f32 ? 4 : 2;
+  const long long items = p.lead * p.X[0] * ceil_div(p.G[1], POOL_ROWS_PER_THREAD) * (p.X[2] / vec);
+  return on && has_rows_instance(p) && p.X[2] % vec == 0 && vec % p.S[2] == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+         items < (1ll << 31);
+}
+
+// out may be null (with mark set): only the argmax offsets are wanted
+static int launch_rows_forward(const PoolParams &p, bool f32, const void *x, void *out, unsigned char *mark, hipStream_t s) {
+  const int vec = f32 ? 4 : 2;
+  const int sig4 = window_signature4(p);
+  PoolRowsParams q{};
+  q.X1 = p.X[1], q.X2 = p.X[2], q.G1 = p.G[1], q.G2 = p.G[2];
+  q.pieces = p.X[2] / vec;
+  q.groups = (int)ceil_div(p.G[1], POOL_ROWS_PER_THREAD);
+  q.planes = p.lead * p.X[0];
+  q.items = q.planes * q.groups * q.pieces;
+  q.by_pieces = make_fastdiv_p((unsigned)q.pieces);
+  q.by_groups = make_fastdiv_p((unsigned)q.groups);
+  // a wavefront covers 63 items (its last lane only supplies its neighbour), a block 4 wavefronts
+  const dim3 grid((unsigned)ceil_div(ceil_div(q.items, 63), 4)), block(256);
+#define MG_POOL_ROWS_SIG(T, A, B, C, D, MK, OUT) \
+  hipLaunchKernelGGL((maxpool_rows_fwd_kernel<T, A, B, C, D, MK, OUT>), grid, block, 0, s, q, (const T *)x, (T *)out, mark)
+#define MG_POOL_ROWS_MK(T, MK, OUT)                                  \
+  do {                                                               \
+    if (sig4 == 3322) MG_POOL_ROWS_SIG(T, 3, 3, 2, 2, MK, OUT);      \
+    else if (sig4 == 3311) MG_POOL_ROWS_SIG(T, 3, 3, 1, 1, MK, OUT); \
+    else MG_POOL_ROWS_SIG(T, 2, 2, 1, 1, MK, OUT);                   \
+  } while (0)
+#define MG_POOL_ROWS(T)                                 \
+  do {                                                  \
+    if (!out) MG_POOL_ROWS_MK(T, true, false);          \
+    else if (mark) MG_POOL_ROWS_MK(T, true, true);      \
+    else MG_POOL_ROWS_MK(T, false, true);               \
+  } while (0)
+  if (f32) MG_POOL_ROWS(float); else MG_POOL_ROWS(double);
+#undef MG_POOL_ROWS
+#undef MG_POOL_ROWS_MK
+#undef MG_POOL_ROWS_SIG
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
+static bool mark_gather_applies(const PoolParams &p, bool f32, bool wide, const void *dx) {
+  static const bool on = [] {
+    const char *flag = getenv("MYGRAD_HIP_POOL_GATHER");
+    return !(flag && flag[0] == '0');
+  }();
+  const int vd = (f32 && !wide) ? 4 : 2;
+  const long long items = p.lead * p.X[0] * ceil_div(p.X[1], p.S[1]) * (p.X[2] / vd);
+  return on && has_rows_instance(p) && p.X[2] % vd == 0 && vd % p.S[2] == 0 && reinterpret_cast<uintptr_t>(dx) % 16 == 0 &&
+         items < (1ll << 31) && (long long)p.G[1] * p.G[2] < (1ll << 30);
+}
+
+static int launch_mark_gather(const PoolParams &p, bool f32, bool wide, const unsigned char *mark, const void *grad, void *dx,
+                              hipStream_t s) {
+  const int vd = (f32 && !wide) ? 4 : 2;
+  const int sig4 = window_signature4(p);
+  PoolGatherParams q{};
+  q.X1 = p.X[1], q.X2 = p.X[2], q.G1 = p.G[1], q.G2 = p.G[2];
+  q.pieces = p.X[2] / vd;
+  q.groups = (int)ceil_div(p.X[1], p.S[1]);
+  q.planes = p.lead * p.X[0];
+  q.by_pieces = make_fastdiv_p((unsigned)q.pieces);
+  q.by_groups = make_fastdiv_p((unsigned)q.groups);
+  const dim3 grid((unsigned)ceil_div(q.planes * q.groups * q.pieces, 256)), block(256);
+#define MG_POOL_GATHER_SIG(T, TD, A, B, C, D) \
+  hipLaunchKernelGGL((maxpool_mark_gather_kernel<T, TD, A, B, C, D>), grid, block, 0, s, q, mark, (const T *)grad, (TD *)dx)
+#define MG_POOL_GATHER(T, TD)                                     \
+  do {                                                            \
+    if (sig4 == 3322) MG_POOL_GATHER_SIG(T, TD, 3, 3, 2, 2);      \
+    else if (sig4 == 3311) MG_POOL_GATHER_SIG(T, TD, 3, 3, 1, 1); \
+    else MG_POOL_GATHER_SIG(T, TD, 2, 2, 1, 1);                   \
+  } while (0)
+  if (!f32)
+    MG_POOL_GATHER(double, double);
+  else if (wide)
+    MG_POOL_GATHER(float, double);
+  else
+    MG_POOL_GATHER(float, float);
+#undef MG_POOL_GATHER
+#undef MG_POOL_GATHER_SIG
+  MG_HIP(hipGetLastError());
+  return MG_OK;
+}
+
 // Forward pass; `mark`, when not null, receives one byte per window (see MARK).
 static int maxpool_fwd_impl(const mg_pool_desc *desc, const void *x, void *out, unsigned char *mark) {
   PoolParams p;
@@ -1024,6 +1205,7 @@ static int maxpool_fwd_impl(const mg_pool_desc *desc, const void *x, void *out, 
     MG_HIP(hipGetLastError());
     return MG_OK;
   }
+  if (rows_forward_applies(p, desc->dtype == MG_F32, x)) return launch_rows_forward(p, desc->dtype == MG_F32, x, out, mark, s);
   PoolTileParams tp;
   int tile_elems = 0, win_slots = 0, acc_offset = 0;
   size_t lds = 0;
@@ -1109,47 +1291,7 @@ static int maxpool_bwd_from_mark(const mg_pool_desc *desc, const unsigned char *
     MG_HIP(hipGetLastError());
     return MG_OK;
   }
-  {
-    // windows over the last two axes with an extent and step that have a kernel instance: the
-    // gather with everything but the tensor's extents known at compile time
-    const int vd = (f32 && !wide) ? 4 : 2;
-    const long long rows = p.lead * p.X[0] * p.X[1];
-    static const bool gather_on = [] {
-      const char *flag = getenv("MYGRAD_HIP_POOL_GATHER");
-      return !(flag && flag[0] == '0');
-    }();
-    const int sig4 = ((p.P[1] * 10 + p.P[2]) * 10 + p.S[1]) * 10 + p.S[2];
-    if (gather_on && p.P[0] == 1 && p.S[0] == 1 && (sig4 == 3322 || sig4 == 3311 || sig4 == 2211) && p.X[2] % vd == 0 &&
-        vd % p.S[2] == 0 && reinterpret_cast<uintptr_t>(dx) % 16 == 0 && rows * (p.X[2] / vd) < (1ll << 31) &&
-        (long long)p.G[1] * p.G[2] < (1ll << 30)) {
-      PoolGatherParams q{};
-      q.X1 = p.X[1], q.X2 = p.X[2], q.G1 = p.G[1], q.G2 = p.G[2];
-      q.pieces = p.X[2] / vd;
-      q.groups = (int)ceil_div(p.X[1], p.S[1]);
-      q.planes = p.lead * p.X[0];
-      q.by_pieces = make_fastdiv_p((unsigned)q.pieces);
-      q.by_groups = make_fastdiv_p((unsigned)q.groups);
-      const dim3 grid((unsigned)ceil_div(q.planes * q.groups * q.pieces, 256)), block(256);
-#define MG_POOL_GATHER_SIG(T, TD, A, B, C, D) \
-  hipLaunchKernelGGL((maxpool_mark_gather_kernel<T, TD, A, B, C, D>), grid, block, 0, s, q, mark, (const T *)grad, (TD *)dx)
-#define MG_POOL_GATHER(T, TD)                                     \
-  do {                                                            \
-    if (sig4 == 3322) MG_POOL_GATHER_SIG(T, TD, 3, 3, 2, 2);      \
-    else if (sig4 == 3311) MG_POOL_GATHER_SIG(T, TD, 3, 3, 1, 1); \
-    else MG_POOL_GATHER_SIG(T, TD, 2, 2, 1, 1);                   \
-  } while (0)
-      if (!f32)
-        MG_POOL_GATHER(double, double);
-      else if (wide)
-        MG_POOL_GATHER(float, double);
-      else
-        MG_POOL_GATHER(float, float);
-#undef MG_POOL_GATHER
-#undef MG_POOL_GATHER_SIG
-      MG_HIP(hipGetLastError());
-      return MG_OK;
-    }
-  }
+  if (mark_gather_applies(p, f32, wide, dx)) return launch_mark_gather(p, f32, wide, mark, grad, dx, s);
   {
     PoolTileParams tp;
     int tile_elems = 0, win_slots = 0, acc_offset = 0;
@@ -1293,6 +1435,16 @@ int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, vo
 #undef MG_POOL_EXACT_BWD
     MG_HIP(hipGetLastError());
     return MG_OK;
+  }
+  if (rows_forward_applies(p, desc->dtype == MG_F32, x) &&
+      mark_gather_applies(p, desc->dtype == MG_F32, desc->dx_dtype == MG_F64, dx)) {
+    // two passes straight from global memory: every window's first-occurrence argmax as one
+    // byte in the library workspace (x is read, nothing else is written), then the gather
+    // from those bytes -- less traffic through LDS than finding and routing in one kernel
+    void *marks = nullptr;
+    if (int rc = workspace((size_t)(p.lead * p.gvol), &marks)) return rc;
+    if (int rc = launch_rows_forward(p, desc->dtype == MG_F32, x, nullptr, (unsigned char *)marks, s)) return rc;
+    return launch_mark_gather(p, desc->dtype == MG_F32, desc->dx_dtype == MG_F64, (const unsigned char *)marks, grad, dx, s);
   }
   PoolTileParams tp;
   int tile_elems = 0, win_slots = 0, acc_offset = 0;
