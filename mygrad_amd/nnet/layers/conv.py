@@ -8,6 +8,7 @@ from numbers import Integral
 import numpy as np
 
 from ... import _device, _hip
+from . import _highrank
 from ...operation_base import Operation
 from ...tensor_base import Tensor
 from .utils import check_window_args
@@ -86,24 +87,27 @@ class ConvND(Operation):
         check_window_args(padded, tuple(int(i) for i in w_shape), tuple(int(s) for s in stride),
                           tuple(int(d) for d in dilation))
 
-        if m > _hip.MG_MAX_ND:
-            raise NotImplementedError(
-                f"conv_nd on the GPU handles 1 to {_hip.MG_MAX_ND} convolved axes, got {m} (no CPU fallback)"
-            )
         dtype = _kernel_dtype(xd, wd)
         grid = tuple(int(g) for g in out_shape)
         out_full = (xd.shape[0], wd.shape[0], *grid)
         self._dtype = dtype
+        self._grid = grid
         if xd.size == 0 or wd.size == 0:
             # nothing to gather: every product involves a padding zero
             self._desc = None
             return _device_zeros(out_full, dtype)
 
-        self._desc = _hip.conv_desc(dtype, xd.shape, wd.shape, grid, stride, padding, dilation)
         xb = _device.to_device(xd, dtype)
         wb = _device.to_device(wd, dtype)
-        ob = _device.DeviceBuffer(int(np.prod(out_full)) * dtype.itemsize)
-        _hip.check(_hip.lib().mg_conv_fwd(self._desc, xb.ptr, wb.ptr, ob.ptr))
+        if m > _hip.MG_MAX_ND:
+            # more convolved axes than the kernels take: the leading ones are taken apart on the
+            # host, tap by tap, into convolutions over the last three (same results, more launches)
+            self._desc = "folded"
+            ob = _highrank.conv_forward(xb, wb, dtype, tuple(xd.shape), tuple(wd.shape), grid, stride, padding, dilation)
+        else:
+            self._desc = _hip.conv_desc(dtype, xd.shape, wd.shape, grid, stride, padding, dilation)
+            ob = _device.DeviceBuffer(int(np.prod(out_full)) * dtype.itemsize)
+            _hip.check(_hip.lib().mg_conv_fwd(self._desc, xb.ptr, wb.ptr, ob.ptr))
         out = _device.download(ob, out_full, dtype)
         _device.attach(out, ob)
         return out
@@ -114,16 +118,26 @@ class ConvND(Operation):
         if self._desc is None:
             return _device_zeros((x if index == 0 else w).shape, dtype)
         lib = _hip.lib()
+        if tuple(grad.shape) != (x.shape[0], w.shape[0], *self._grid):
+            raise ValueError(f"conv_nd backward: gradient of shape {tuple(grad.shape)} for an output of shape "
+                             f"{(x.shape[0], w.shape[0], *self._grid)}")
         gb = _device.to_device(grad, dtype)
+        folded = (dtype, tuple(x.shape), tuple(w.shape), self._grid, self.stride, self.padding, self.dilation)
         if index == 0:  # dx
             wb = _device.to_device(w, dtype)
-            db = _device.DeviceBuffer(x.size * dtype.itemsize)
-            _hip.check(lib.mg_conv_dgrad(self._desc, gb.ptr, wb.ptr, db.ptr))
+            if self._desc == "folded":
+                db = _highrank.conv_dgrad(gb, wb, *folded)
+            else:
+                db = _device.DeviceBuffer(x.size * dtype.itemsize)
+                _hip.check(lib.mg_conv_dgrad(self._desc, gb.ptr, wb.ptr, db.ptr))
             out = _device.download(db, x.shape, dtype)
         else:  # dw
             xb = _device.to_device(x, dtype)
-            db = _device.DeviceBuffer(w.size * dtype.itemsize)
-            _hip.check(lib.mg_conv_wgrad(self._desc, gb.ptr, xb.ptr, db.ptr))
+            if self._desc == "folded":
+                db = _highrank.conv_wgrad(gb, xb, *folded)
+            else:
+                db = _device.DeviceBuffer(w.size * dtype.itemsize)
+                _hip.check(lib.mg_conv_wgrad(self._desc, gb.ptr, xb.ptr, db.ptr))
             out = _device.download(db, w.shape, dtype)
         _device.attach_transient(out, db)
         return out

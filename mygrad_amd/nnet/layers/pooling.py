@@ -24,6 +24,7 @@ class MaxPoolND(Operation):
     takes_device_arrays = True
 
     _argmax = None  # device buffer, one byte per window, written by the forward pass
+    _skip = 0  # leading pooled axes with a one-element window, counted as leading axes
 
     def __call__(self, x, pool, stride):
         self.variables = (x,)
@@ -56,10 +57,17 @@ class MaxPoolND(Operation):
                 f"Pooling dimensions: {tuple(pool)}\n"
             )
 
-        if not 1 <= m <= _hip.MG_MAX_ND:
+        # Leading pooled axes with a window of one element placed at every position pool nothing:
+        # they count as un-pooled leading axes.  What is left must fit the kernels' three axes.
+        skip = 0
+        while m - skip > _hip.MG_MAX_ND and pool[skip] == 1 and stride[skip] == 1:
+            skip += 1
+        if not 1 <= m - skip <= _hip.MG_MAX_ND:
             raise NotImplementedError(
-                f"max_pool on the GPU handles 1 to {_hip.MG_MAX_ND} pooled axes, got {m} (no CPU fallback)"
+                f"max_pool on the GPU handles 1 to {_hip.MG_MAX_ND} pooled axes (leading axes with a window of one "
+                f"element aside), got pool={tuple(pool)} stride={tuple(stride)} (no CPU fallback)"
             )
+        self._skip = skip
         if xd.dtype not in (np.float32, np.float64):
             raise TypeError(
                 f"max_pool runs on the GPU in float32 or float64, got {xd.dtype} (there is no CPU fallback)"
@@ -71,7 +79,8 @@ class MaxPoolND(Operation):
         if self._lead == 0:
             return np.empty(out_full, dtype=xd.dtype)
 
-        desc = _hip.pool_desc(xd.dtype, self._lead, pooled, pool, stride, grid)
+        self._lead *= int(np.prod(pooled[:skip], dtype=np.int64))
+        desc = _hip.pool_desc(xd.dtype, self._lead, pooled[skip:], pool[skip:], stride[skip:], grid[skip:])
         xb = _device.to_device(xd)
         windows = int(np.prod(out_full))
         ob = _device.DeviceBuffer(windows * xd.dtype.itemsize)
@@ -103,7 +112,8 @@ class MaxPoolND(Operation):
         # var already holds a gradient that this one is added to, where the
         # unrounded float64 values are needed for the same result.
         dx_dtype = np.dtype(np.float64) if var._grad is not None else x.dtype
-        desc = _hip.pool_desc(x.dtype, self._lead, x.shape[x.ndim - m :], self.pool, self.stride, self._grid,
+        k = self._skip
+        desc = _hip.pool_desc(x.dtype, self._lead, x.shape[x.ndim - m + k :], self.pool[k:], self.stride[k:], self._grid[k:],
                               dx_dtype=dx_dtype)
         gb = _device.to_device(grad, x.dtype)
         db = _device.DeviceBuffer(x.size * dx_dtype.itemsize)

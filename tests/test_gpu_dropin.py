@@ -64,10 +64,6 @@ def test_padding_only_image_gives_zero(m):
     pad = tuple(int(p) for p in rng.integers(1, 4, m))
     x = mg.Tensor(np.zeros((1, 1) + (0,) * m))
     w = rng.standard_normal((1, 1) + tuple(2 * p for p in pad))
-    if m > 3:
-        with pytest.raises(NotImplementedError):
-            conv_nd(x, w, padding=pad, stride=1)
-        return
     out = conv_nd(x, w, padding=pad, stride=1)
     assert out.shape == (1,) * (m + 2) and out.item() == 0.0
     out.backward()
@@ -424,4 +420,51 @@ def test_device_tensor_is_uploaded_once_and_seeds_backward():
     assert np.array_equal(x.data, xv) and x.data.flags.writeable
     with pytest.raises(TypeError):
         mg.device_tensor(np.arange(4))
+    assert _graph.held_count() == 0
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_four_and_five_convolved_axes(dtype):
+    """More convolved axes than the kernels take: the leading ones are taken apart on the host
+    into convolutions over the last three (the reference takes any number, conv.py:23-29)."""
+    from oracle import brute
+
+    rng = np.random.default_rng(31)
+    tol = TOL[np.dtype(dtype)]
+    cases = [
+        # x shape, w shape, stride, padding, dilation
+        ((2, 3, 5, 7, 5, 7), (4, 3, 2, 3, 2, 3), (1, 2, 1, 2), (1, 0, 1, 1), (2, 1, 1, 1)),
+        ((1, 16, 4, 6, 6, 8), (16, 16, 3, 1, 3, 3), (1, 1, 1, 1), (1, 0, 1, 1), (1, 1, 1, 1)),
+        ((2, 2, 3, 4, 3, 4, 5), (3, 2, 2, 2, 1, 2, 2), (1, 1, 1, 1, 1), (0, 1, 0, 0, 1), (1, 1, 1, 1, 1)),
+    ]
+    for x_shape, w_shape, s, p, d in cases:
+        xv = rng.standard_normal(x_shape).astype(dtype)
+        wv = (rng.standard_normal(w_shape) / np.sqrt(np.prod(w_shape[1:]))).astype(dtype)
+        x, w = mg.Tensor(xv), mg.Tensor(wv)
+        out = conv_nd(x, w, stride=s, padding=p, dilation=d)
+        want = ora.conv_forward(xv, wv, stride=s, padding=p, dilation=d)
+        assert out.shape == want.shape and out.dtype == dtype
+        g = rng.standard_normal(out.shape).astype(dtype)
+        out_data = out.data
+        out.backward(g)
+        assert rel_err(out_data, want) <= tol
+        assert rel_err(x.grad, ora.conv_backward_x(g, xv.shape, xv.dtype, wv, stride=s, padding=p, dilation=d)) <= tol
+        assert rel_err(w.grad, ora.conv_backward_w(g, xv, wv.shape, stride=s, padding=p, dilation=d)) <= tol
+        if xv.size * wv.size // wv.shape[1] < 3_000_000:  # the definition itself, in loops
+            assert rel_err(out_data, brute.conv_forward(xv, wv, s, p, d)) <= tol
+    assert _graph.held_count() == 0
+
+
+def test_pooling_over_four_axes_with_a_leading_window_of_one():
+    rng = np.random.default_rng(32)
+    xv = rng.integers(0, 4, (2, 3, 5, 6, 8)).astype(np.float64)
+    x = mg.Tensor(xv)
+    out = max_pool(x, (1, 1, 2, 3, 2), (1, 1, 1, 3, 2))  # five pooled axes, two of them with a window of one element
+    want = ora.pool_forward(xv, (1, 1, 2, 3, 2), (1, 1, 1, 3, 2), validate=False)
+    assert np.array_equal(out.data, want)
+    g = rng.standard_normal(out.shape)
+    out.backward(g)
+    assert np.array_equal(x.grad.view(np.uint64), ora.pool_backward(xv, g, (1, 1, 2, 3, 2), (1, 1, 1, 3, 2)).view(np.uint64))
+    with pytest.raises(NotImplementedError):
+        max_pool(mg.Tensor(np.zeros((4, 4, 4, 4))), (2, 2, 2, 2), 2)
     assert _graph.held_count() == 0
