@@ -54,6 +54,10 @@ WORKLOADS = {
                   stride=(2, 1), padding=(4, 4), dilation=(2, 2)),
     "conv5": dict(kind="conv", dtype="f32", seed=1006, x=(8, 16, 32, 64, 64), w=(32, 16, 3, 3, 3),
                   wscale=(2 / 432) ** 0.5, stride=(1, 1, 1), padding=(1, 1, 1), dilation=(1, 1, 1)),
+    # a ResNet stem: three input channels, a 7x7 filter bank, stride 2 (flooring placement: the last
+    # padded row and column are never read)
+    "stem": dict(kind="conv", dtype="f32", seed=1017, x=(128, 3, 224, 224), w=(64, 3, 7, 7), wscale=(2 / 147) ** 0.5,
+                 stride=(2, 2), padding=(3, 3), dilation=(1, 1)),
     "pool2": dict(kind="pool", dtype="f64", seed=1002, x=(64, 64, 56, 56), pool=(3, 3), stride=(2, 2)),
     "pool5": dict(kind="pool", dtype="f32", seed=1006, x=(8, 32, 32, 64, 64), pool=(2, 2, 2), stride=(2, 2, 2)),
     # the same two with each window's argmax recomputed from x in the backward pass (the stateless

@@ -492,6 +492,11 @@ def test_conv_config5(abi):
     _check_conv_config(abi, 1006, np.float32, (8, 16, 32, 64, 64), (32, 16, 3, 3, 3), np.sqrt(2 / 432), (1, 1, 1), (1, 1, 1), (1, 1, 1), 1)
 
 
+def test_conv_stem_three_channels_seven_by_seven_stride_two(abi):
+    # a quarter of the batch of bench.py's `stem` workload, its literal (flooring) shape
+    _check_conv_config(abi, 1017, np.float32, (32, 3, 224, 224), (64, 3, 7, 7), np.sqrt(2 / 147), (2, 2), (3, 3), (1, 1), 1)
+
+
 def test_conv_wgrad_is_run_to_run_identical(abi):
     rng = np.random.default_rng(5)
     x = rng.standard_normal((16, 24, 30, 30)).astype(np.float32)
