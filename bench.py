@@ -10,7 +10,9 @@ the C ABI of libmygrad_hip.so.  The script prints ONE JSON line:
 
 * ``value``        whole-step throughput from the host clock around the K steps
                    (algorithmic flops or bytes / wall time, library stream drained
-                   on both sides);
+                   on both sides).  Before the W warm-up steps the step runs untimed
+                   for ``--prewarm`` seconds (0.4 by default, reported under
+                   ``prewarm``) so that the device clock has settled;
 * ``roofline``     the dominant kernel of the step: algorithmic flops (or bytes)
                    of one launch / its mean duration between HIP events recorded
                    on the library stream inside the timed region;
@@ -409,10 +411,25 @@ class Step:
             check(lib.mg_maxpool_bwd_argmax(d, self.argmax.ptr, self.g.ptr, self.dx.ptr))
 
 
-def run_gpu(name, steps, warmup):
+PREWARM_SECONDS = 0.4
+
+
+def run_gpu(name, steps, warmup, prewarm=None):
     from mygrad_amd import _hip
 
     step = Step(name)
+    # The device clock climbs for a few hundred milliseconds after an idle period (measured:
+    # 2.15 - 2.3 GHz during the first tens of milliseconds of work, 2.38 - 2.40 GHz from then on,
+    # see profiles/conv3a_sustained.txt): run the step untimed until it has settled, so that the
+    # timed steps show the rate a job sustains rather than the ramp.
+    prewarm = PREWARM_SECONDS if prewarm is None else prewarm
+    t_end = time.perf_counter() + prewarm
+    prewarmed = 0
+    while time.perf_counter() < t_end:
+        for _ in range(10):
+            step()
+        _hip.synchronize()
+        prewarmed += 10
     for _ in range(warmup):
         step()
     _hip.synchronize()
@@ -451,6 +468,7 @@ def run_gpu(name, steps, warmup):
         "unit": step.unit,
         "ms_per_step": ms_per_step,
         "kernel_ms_per_step": float(sum(np.sum(v) for v in per_kernel.values()) / steps),
+        "prewarm": {"seconds": prewarm, "steps": prewarmed},
         "roofline": {
             "bound": step.bound,
             "kernel": dominant,
@@ -920,6 +938,8 @@ def main():
                     help="report every other workload under 'secondary', not only the hot path's other configurations")
     ap.add_argument("--no-secondary", action="store_true", help="run the one workload only")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--prewarm", type=float, default=PREWARM_SECONDS,
+                    help="seconds of untimed steps before the warm-up steps, for the device clock to settle (0: none)")
     ap.add_argument("--dropin", action="store_true",
                     help="also time the step through the Python drop-in API (reported under 'dropin', never as value)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -941,7 +961,7 @@ def main():
         return
 
     wl = WORKLOADS[args.workload]
-    res = run_gpu(args.workload, args.steps, args.warmup)
+    res = run_gpu(args.workload, args.steps, args.warmup, args.prewarm)
     line = {
         "metric": {"conv": "conv_nd fwd+bwd TFLOP/s", "pool": "max_pool fwd+bwd GB/s",
                    "elem": "relu+multiply+sum fwd+bwd GB/s", "bn": "batchnorm fwd+bwd GB/s",
@@ -961,6 +981,7 @@ def main():
         "config": {"workload": describe(args.workload)},
         "roofline": res["roofline"],
         "kernel_ms_per_step": res["kernel_ms_per_step"],
+        "prewarm": res["prewarm"],
         "kernels": res["kernels"],
     }
     if not args.no_cpu_baseline:
@@ -975,7 +996,7 @@ def main():
         for name in names:
             if name == args.workload:
                 continue
-            r = run_gpu(name, args.steps, args.warmup)
+            r = run_gpu(name, args.steps, args.warmup, args.prewarm)
             entry = {"config": describe(name), "value": r["value"], "unit": r["unit"], "dtype": WORKLOADS[name]["dtype"],
                      "ms_per_step": r["ms_per_step"], "kernel_ms_per_step": r["kernel_ms_per_step"], "roofline": r["roofline"],
                      "kernels": r["kernels"]}
