@@ -245,6 +245,103 @@ def test_op_wraps_output_without_copy_and_locks_arrays():
     assert np.array_equal(x.grad, [2.0, 2.0])
 
 
+class _HostBackedBuffer:
+    """Stands in for a device buffer in the tests of the host logic: 'downloads' from a NumPy array."""
+
+    def __init__(self, values):
+        self.values = np.ascontiguousarray(values)
+        self.ptr, self.nbytes, self.downloads = 0, self.values.nbytes, 0
+
+    def download_into(self, arr):
+        self.downloads += 1
+        arr[...] = self.values.reshape(arr.shape)
+
+
+def _pinned_stand_in(monkeypatch):
+    from mygrad_amd import _device
+
+    monkeypatch.setattr(_device, "pinned_empty", lambda shape, dtype: np.empty(shape, dtype))
+    return _device
+
+
+class DeviceScale(mg.Operation):
+    """Doubles its input and returns the result as a value that is 'on the device' only."""
+
+    takes_device_arrays = True
+
+    def __call__(self, x):
+        from mygrad_amd import _device
+
+        self.variables = (x,)
+        self.seen = _device.value_of(x)
+        values = np.asarray(self.seen.buf.values if isinstance(self.seen, _device.DeviceArray) else self.seen) * 2.0
+        return _device.DeviceArray(_HostBackedBuffer(values), values.shape, values.dtype)
+
+    def backward_var(self, grad, index, **kwargs):
+        from mygrad_amd import _device
+
+        self.grad_seen = grad
+        values = np.asarray(grad.buf.values if isinstance(grad, _device.DeviceArray) else grad) * 2.0
+        return _device.DeviceArray(_HostBackedBuffer(values), values.shape, values.dtype)
+
+
+def test_a_result_on_the_device_is_copied_once_when_read_and_guarded_like_any_array(monkeypatch):
+    _device = _pinned_stand_in(monkeypatch)
+    x = mg.Tensor([1.0, 2.0, 3.0])
+    y = mg.execute_op(DeviceScale, x)
+    z = mg.execute_op(DeviceScale, y)
+    assert y.on_device and z.on_device and y.shape == (3,) and y.dtype == np.float64 and y.size == 3 and y.ndim == 1
+    assert isinstance(z.creator.seen, _device.DeviceArray)  # the second operation got the value as it was, no copy
+    buf = y._value.buf
+    data = y.data
+    assert buf.downloads == 1 and y.data is data and not y.on_device
+    assert np.array_equal(data, [2.0, 4.0, 6.0])
+    assert not data.flags.writeable  # two live operations hold it (its creator and its consumer)
+    z.backward(np.array([1.0, 1.0, 1.0]))
+    assert data.flags.writeable and _graph.held_count() == 0
+    assert isinstance(x._grad, _device.DeviceArray)  # a gradient stays where it was made ...
+    grad = x.grad
+    assert isinstance(grad, np.ndarray) and np.array_equal(grad, [4.0, 4.0, 4.0]) and x.grad is grad  # ... until it is read
+    assert grad.flags.writeable
+    # read after its graph is gone: an ordinary writeable array, nothing left to guard
+    w = mg.execute_op(DeviceScale, x)
+    w.clear_graph()
+    assert w.data.flags.writeable
+    # without the graph (or the guard) nothing is locked and nothing is remembered
+    with mg.no_autodiff:
+        v = mg.execute_op(DeviceScale, x)
+    assert v.on_device and v.creator is None and v.data.flags.writeable
+    assert _graph.held_count() == 0
+
+
+def test_an_operation_that_does_not_take_device_arrays_gets_host_arrays(monkeypatch):
+    _device = _pinned_stand_in(monkeypatch)
+    x = mg.Tensor([1.0, 2.0])
+    y = mg.execute_op(DeviceScale, x)
+    out = mg.execute_op(Scale, y, np.array([1.0, 1.0]))  # reads y.data: a host array from here on
+    assert not y.on_device and np.array_equal(out.data, [7.0, 11.0])
+    out.backward()
+    assert np.array_equal(x.grad, [4.0, 4.0])
+    u = mg.Tensor([1.0, 2.0])
+    z = mg.execute_op(DeviceScale, mg.execute_op(Identity, u))
+    z.backward(np.array([1.0, 1.0]))  # DeviceScale hands a DeviceArray back; Identity's backward_var gets an ndarray
+    assert isinstance(z.creator, type(None)) and np.array_equal(u.grad, [2.0, 2.0])
+    assert _graph.held_count() == 0
+
+
+def test_device_array_answers_shape_questions_without_a_copy():
+    from mygrad_amd import _device
+
+    buf = _HostBackedBuffer(np.arange(24.0))
+    a = _device.DeviceArray(buf, (2, 3, 4), np.float64)
+    assert (a.ndim, a.size, a.nbytes, a.itemsize) == (3, 24, 192, 8) and a.flags["C_CONTIGUOUS"] and a.base is None
+    b = a.reshape(6, -1)
+    assert b.shape == (6, 4) and b.buf is buf and b.base is a and b.reshape((24,)).base is a
+    with pytest.raises(ValueError):
+        a.reshape(5, -1)
+    assert buf.downloads == 0 and _device.is_locked(a) and _device.lookup(a) is buf
+
+
 def test_constant_propagation():
     f, c = mg.Tensor([1.0]), mg.Tensor([1.0], constant=True)
     assert mg.execute_op(Scale, f, c).constant is False
