@@ -1093,8 +1093,7 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
   const long long kpos = (long long)g.N * g.gvol;
   const int cus = runtime().props.multiProcessorCount;
   // Split K so that all blocks are resident at once (one round: no half-empty second
-  // round), with at least 4 K tiles per block.  The tap-major kernel hands whole
-  // splits to the 8 XCDs, so a multiple of 8 is preferred when one fits.
+  // round), with at least 4 K tiles per block.
   auto splits_for = [&](int bm, int bn, int bk, bool tap) {
     const long long tiles = ceil_div(ct, bn) * ceil_div(g.F, bm);
     const long long ktiles = ceil_div(kpos, bk);
@@ -1118,9 +1117,7 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
       }
       return best;
     }
-    long long splits = std::max<long long>(1, std::min(slots / tiles, max_splits));
-    if (splits >= 8) splits = splits / 8 * 8;
-    return splits;
+    return std::max<long long>(1, std::min(slots / tiles, max_splits));
   };
   // Tap-major candidates, largest first.  A larger tile re-reads grad and x less often
   // (the kernel is limited by what it pulls through L1, not by HBM), so the first

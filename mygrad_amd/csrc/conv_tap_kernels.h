@@ -732,20 +732,18 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
   const int wn0 = ((wave & 3) % WAVES_N) * WN;
   const int l16 = lane & 15, lk = lane >> 4;
   // Blocks are handed to the 8 XCDs round-robin, and each XCD has its own L2.  All
-  // tiles of one K split read the same positions of grad and x, so they are given to
-  // one XCD, next to each other in its dispatch order: block b is the (b/8)-th block
-  // of XCD b%8, and an XCD takes whole splits.
-  // (Only when the number of splits is a multiple of 8; otherwise plain order.)
+  // tiles of one K split read the same positions of grad and x, so they should meet in
+  // one L2.  The (split, tile) pairs, splits outermost, are cut into 8 runs of equal
+  // length (to within one), one per XCD: block b is the (b/8)-th block of XCD b%8 and
+  // takes the (b/8)-th pair of that XCD's run.  An XCD then works on whole splits, one
+  // after the other, and shares at most the split at either end of its run with a
+  // neighbour; any number of splits can be used.
   const int tiles_per_split = p.col_tiles * p.row_tiles;
-  int split, tile;
-  if (p.splits % 8 == 0) {
-    const int xcd = blockIdx.x % 8, nth = blockIdx.x / 8;
-    split = (nth / tiles_per_split) * 8 + xcd;
-    tile = nth % tiles_per_split;
-  } else {
-    split = blockIdx.x / tiles_per_split;
-    tile = blockIdx.x % tiles_per_split;
-  }
+  const int xcd = blockIdx.x % 8, nth = blockIdx.x / 8;
+  const int per_xcd = gridDim.x / 8, extra = gridDim.x % 8;
+  const int pair = xcd * per_xcd + min(xcd, extra) + nth;
+  const int split = pair / tiles_per_split;
+  const int tile = pair % tiles_per_split;
   const int n0 = (tile % p.col_tiles) * BN;  // first column
   const int m0 = (tile / p.col_tiles) * BM;  // first filter (F % BM == 0)
   const int kbeg = split * p.kchunk;
