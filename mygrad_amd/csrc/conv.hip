@@ -72,13 +72,12 @@ struct Mma<double> {
 };
 
 // ------------------------------------------------------------------------------------------
-// filter packing: the GEMMs want the filter operand with M contiguous
-//   mode 0 (forward)            : Ap[(c*Wvol + t)][f] = w[f][c][t]
-//   mode 1 (dgrad)              : Ap[(f*Wvol + t)][c] = w[f][c][t]
-//   mode 2 (forward, tap-major) : Ap[(t*C + c)][f]    = w[f][c][t]
-//   mode 3 (dgrad, tap-major)   : Ap[(t*F + f)][c]    = w[f][c][t]
-// Modes 2 and 3 pad every row with zeros to a multiple of four values (`ld` values per
-// row), so that the kernels can read a row sixteen bytes at a time whatever M is.
+// filter packing: the tap-major GEMMs want the filter operand with M contiguous
+//   mode 2 (forward) : Ap[(t*C + c)][f] = w[f][c][t]
+//   mode 3 (dgrad)   : Ap[(t*F + f)][c] = w[f][c][t]
+// Every row is padded with zeros to a multiple of four values (`ld` values per row), so
+// that the kernels can read a row sixteen bytes at a time whatever M is.  (The
+// table-driven kernel reads the filter bank in place.)
 // ------------------------------------------------------------------------------------------
 // One tap, forward, tap-major (mode 2 with wvol == 1 and ld == F): Ap[c][f] = w[f][c], a plain
 // transposition of an F x C matrix -- what a matrix product's left operand needs.  32 x 32
@@ -104,7 +103,7 @@ __global__ void __launch_bounds__(256) pack_transpose_kernel(const T *__restrict
 template <typename T>
 __global__ void __launch_bounds__(256) pack_filters_kernel(const T *__restrict__ w, T *__restrict__ ap, int F, int C,
                                                            int wvol, int mode, int ld) {
-  const int M = (mode == 0 || mode == 2) ? F : C;
+  const int M = mode == 2 ? F : C;
   const int total = (F * C * wvol / M) * ld;
   for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
     // idx enumerates the packed layout so that stores are coalesced
@@ -115,24 +114,14 @@ __global__ void __launch_bounds__(256) pack_filters_kernel(const T *__restrict__
       continue;
     }
     int f, c, t;
-    if (mode == 0 || mode == 2) {
+    if (mode == 2) {
       f = m;
-      if (mode == 0) {
-        t = row % wvol;
-        c = row / wvol;
-      } else {
-        c = row % C;
-        t = row / C;
-      }
+      c = row % C;
+      t = row / C;
     } else {
       c = m;
-      if (mode == 1) {
-        t = row % wvol;
-        f = row / wvol;
-      } else {
-        f = row % F;
-        t = row / F;
-      }
+      f = row % F;
+      t = row / F;
     }
     ap[idx] = w[((long long)f * C + c) * wvol + t];
   }
@@ -216,7 +205,7 @@ __global__ void __launch_bounds__(256) gather_gemm_kernel(const GemmParams p) {
       const int kidx = kbase + kk;
       oka[r] = (kk < BK) & (kidx <= klast) & m_ok;
       const int row = arow[min(kidx, klast)];
-      ra[r] = A[(long long)row * p.M + acol_safe];
+      ra[r] = A[(long long)row + (long long)acol_safe * p.a_mstride];
     }
 #pragma unroll
     for (int r = 0; r < BLOADS; ++r) {
@@ -466,12 +455,32 @@ __device__ __forceinline__ T sum_in_order(const T *__restrict__ p, long long str
 }
 
 // dw[i] = ((part[0][i] + part[1][i]) + part[2][i]) + ...   (fixed order)
-template <typename T>
+// RUNS > 1: the splits are cut into RUNS consecutive runs, each summed in order by its own
+// thread, and the runs' totals are added in order (for a small dw, where one thread per
+// element would leave most of the device idle behind a long chain of dependent loads).
+template <typename T, int RUNS>
 __global__ void __launch_bounds__(256) splitk_reduce_kernel(const T *__restrict__ part, T *__restrict__ dw, int count,
                                                             int splits) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= count) return;
-  dw[i] = sum_in_order(part + i, count, splits);
+  constexpr int WIDTH = 256 / RUNS;
+  const int q = threadIdx.x / WIDTH, lane = threadIdx.x % WIDTH;
+  const int i = blockIdx.x * WIDTH + lane;
+  if constexpr (RUNS == 1) {
+    if (i < count) dw[i] = sum_in_order(part + i, count, splits);
+    return;
+  }
+  __shared__ T runs[RUNS][WIDTH];
+  const int per = (splits + RUNS - 1) / RUNS;
+  const int first = min(q * per, splits), last = min(first + per, splits);
+  // an empty run holds +0.0, which changes no total (a total of -0.0 cannot come out of
+  // accumulators that start from +0.0)
+  runs[q][lane] = (i < count && first < last) ? sum_in_order(part + (long long)first * count + i, count, last - first) : T(0);
+  __syncthreads();
+  if (q == 0 && i < count) {
+    T sum = runs[0][lane];
+#pragma unroll
+    for (int r = 1; r < RUNS; ++r) sum += runs[r][lane];
+    dw[i] = sum;
+  }
 }
 
 }  // namespace mg
@@ -524,6 +533,7 @@ struct Plan {
   int blocks_per_cu = 1;  // persistent blocks per compute unit (streaming gather-GEMM)
   bool tap_major = false;  // which kernel family the tables are for
   bool single_dense_phase = false;  // positions enumerate the destination tensor in order
+  bool deep_k = false;              // table-driven, a few microseconds of work: 16 x 64 tiles with a K tile four times as deep
   // fused stride phases of the data gradient (see GemmParams::nph)
   int nph = 1;
   int kcut[4] = {0, 0, 0, 0};
@@ -843,6 +853,27 @@ void fwd_table(const Geometry &g, std::vector<TabEntry> &tab) {
         }
 }
 
+// A problem of a few microseconds is bound by its launches and by the chain of K tiles a
+// block runs through, each a round trip to memory, not by the matrix pipes.
+// MYGRAD_HIP_TINY=0 plans such a problem like a large one (read whenever a plan is built, and
+// part of the plan's key: the parity tests run their small cases both ways).
+bool tiny_plans_enabled() {
+  const char *flag = getenv("MYGRAD_HIP_TINY");
+  return !(flag && flag[0] == '0');
+}
+
+bool is_tiny(const Geometry &g) {
+  return tiny_plans_enabled() &&
+         2.0 * (double)g.N * (double)g.gvol * (double)g.F * (double)g.C * (double)g.wvol < 1e8;
+}
+
+// The table-driven kernel for such a problem: more, smaller tiles and a quarter of the K steps.
+void deepen_if_tiny(const Geometry &g, Plan &pl) {
+  if (pl.tap_major || !is_tiny(g) || pl.bm != 16) return;
+  pl.bn = 64;
+  pl.deep_k = true;
+}
+
 int build_fwd_plan(const Geometry &g, Plan &pl) {
   Tables t;
   const int bk = gemm_bk(g.dtype);
@@ -852,6 +883,7 @@ int build_fwd_plan(const Geometry &g, Plan &pl) {
     const long long ktiles = pl.tap_major ? g.wvol * (g.C / bk) : ceil_div((long long)g.C * g.wvol, bk);
     const TileChoice tc = choose_tile(g.F, {(long long)g.N * g.gvol}, (int)ktiles, pl.tap_major, g.dtype == MG_F64 ? 8 : 4);
     pl.bm = tc.bm, pl.bn = tc.bn, pl.m_tiles = tc.m_tiles, pl.full_tiles = tc.full_tiles, pl.tail_split = tc.tail_split, pl.blocks_per_cu = tc.blocks_per_cu;
+    deepen_if_tiny(g, pl);
   }
   Phase ph{};
   for (int k = 0; k < 3; ++k) {
@@ -895,7 +927,9 @@ int build_fwd_plan(const Geometry &g, Plan &pl) {
 int build_dgrad_plan(const Geometry &g, Plan &pl) {
   Tables t;
   const int bk = gemm_bk(g.dtype);
-  pl.tap_major = g.F % bk == 0 && fits_buffer_loads(g);
+  // a tiny problem is bound by its launches: the table-driven kernel needs neither packed
+  // filters nor a pass over partial sums
+  pl.tap_major = g.F % bk == 0 && fits_buffer_loads(g) && !is_tiny(g);
   pl.single_dense_phase = g.S[0] == 1 && g.S[1] == 1 && g.S[2] == 1;
   const int gs[3] = {g.G[1] * g.G[2], g.G[2], 1};
   long long nphase = (long long)g.S[0] * g.S[1] * g.S[2];
@@ -1017,6 +1051,7 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
     }
     const TileChoice tc = choose_tile(g.C, npos, (int)std::max<long long>(min_ktiles, 0), pl.tap_major, g.dtype == MG_F64 ? 8 : 4);
     pl.bm = tc.bm, pl.bn = tc.bn, pl.m_tiles = tc.m_tiles, pl.full_tiles = tc.full_tiles, pl.tail_split = tc.tail_split, pl.blocks_per_cu = tc.blocks_per_cu;
+    deepen_if_tiny(g, pl);
   }
 
   // ---- tables
@@ -1050,7 +1085,7 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
               e.d2 = pt.offs[2][c];
               e.off = (int)(f * g.gvol) + e.d0 * gs[0] + e.d1 * gs[1] + e.d2 * gs[2];
               t.tab.push_back(e);
-              t.arow.push_back((int)(f * g.wvol) + (pt.taps[0][a] * g.W[1] + pt.taps[1][b]) * g.W[2] + pt.taps[2][c]);
+              t.arow.push_back((int)(f * g.C * g.wvol) + (pt.taps[0][a] * g.W[1] + pt.taps[1][b]) * g.W[2] + pt.taps[2][c]);
             }
       ph.k_count = (int)t.tab.size() - ph.k_begin;
     }
@@ -1189,6 +1224,7 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
 int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
   std::string key(reinterpret_cast<const char *>(d), sizeof *d);
   key.push_back((char)op);
+  key.push_back(tiny_plans_enabled() ? 't' : 'T');
   auto it = plans().find(key);
   if (it == plans().end()) {
     if (plans().size() >= 256) {
@@ -1266,6 +1302,10 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
   }
   ScopedTiming timed(tag);
   bool launched = false;
+  if (pl.deep_k) {
+    launch_gemm<T, 16, 64, 4 * BK, 16, 16>(gp, pl, s);
+    launched = true;
+  }
 #define MG_LAUNCH(TT, BM, BN, WM, WN)                     \
   if (!launched && pl.bm == BM && pl.bn == BN) {          \
     launch_gemm<TT, BM, BN, BK, WM, WN>(gp, pl, s);       \
@@ -1301,14 +1341,13 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
 
 // Packs the filters into the front of the library workspace; `extra` more bytes
 // behind them (256-byte aligned) are reserved for the caller and returned in *behind.
-// Values per row of the packed filters: M itself for the table-driven kernels, M rounded
-// up to a multiple of four for the tap-major ones.
+// Values per row of the packed filters: M rounded up to a multiple of four.
 inline int packed_ld(int M, bool tap_major) { return tap_major ? (M + 3) / 4 * 4 : M; }
 
 template <typename T>
 int pack_filters(const Geometry &g, const void *w, int mode, void **packed, size_t extra = 0, void **behind = nullptr) {
-  const int M = (mode == 0 || mode == 2) ? g.F : g.C;
-  const int ld = packed_ld(M, mode >= 2);
+  const int M = mode == 2 ? g.F : g.C;
+  const int ld = packed_ld(M, true);
   const size_t count = (size_t)g.F * g.C * g.wvol / M * ld;
   const size_t packed_bytes = (count * sizeof(T) + 255) & ~size_t(255);
   if (mode == 3 && g.wvol == 1 && ld == g.C && reinterpret_cast<uintptr_t>(w) % 16 == 0) {
@@ -1341,10 +1380,15 @@ template <typename T>
 int conv_fwd_impl(const Geometry &g, const Plan &pl, const void *x, const void *w, void *out) {
   void *packed = nullptr;
   void *partial = nullptr;
-  if (int rc = pack_filters<T>(g, w, pl.tap_major ? 2 : 0, &packed, tail_bytes(pl, sizeof(T)), &partial)) return rc;
+  if (!pl.tap_major) {
+    packed = const_cast<void *>(w);  // read in place: row k = (c, taps) of filter m lies at w[m * C*taps + k]
+  } else if (int rc = pack_filters<T>(g, w, 2, &packed, tail_bytes(pl, sizeof(T)), &partial)) {
+    return rc;
+  }
   GemmParams gp{};
   gp.partial = partial;
   gp.A = packed;
+  gp.a_mstride = (int)(g.C * g.wvol);
   gp.src = x;
   gp.dst = out;
   gp.M = g.F;
@@ -1371,10 +1415,15 @@ template <typename T>
 int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const void *w, void *dx) {
   void *packed = nullptr;
   void *partial = nullptr;
-  if (int rc = pack_filters<T>(g, w, pl.tap_major ? 3 : 1, &packed, tail_bytes(pl, sizeof(T)), &partial)) return rc;
+  if (!pl.tap_major) {
+    packed = const_cast<void *>(w);  // read in place: row k = (f, tap) of channel m lies at w[(f * C + m) * taps + tap]
+  } else if (int rc = pack_filters<T>(g, w, 3, &packed, tail_bytes(pl, sizeof(T)), &partial)) {
+    return rc;
+  }
   GemmParams gp{};
   gp.partial = partial;
   gp.A = packed;
+  gp.a_mstride = (int)g.wvol;
   gp.src = grad;
   gp.dst = dx;
   gp.M = g.C;
@@ -1478,8 +1527,12 @@ int conv_wgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
         hipLaunchKernelGGL((tap_reduce_kernel<T, 1>), dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, s,
                            static_cast<const T *>(target), static_cast<T *>(dw), g.F, g.C, (int)g.wvol, pl.splits);
     } else {
-      hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, s,
-                         static_cast<const T *>(target), static_cast<T *>(dw), count, pl.splits);
+      if (ceil_div(count, 256) < runtime().props.multiProcessorCount / 8 && pl.splits >= 64)
+        hipLaunchKernelGGL((splitk_reduce_kernel<T, 16>), dim3((unsigned)ceil_div(count, 16)), dim3(256), 0, s,
+                           static_cast<const T *>(target), static_cast<T *>(dw), count, pl.splits);
+      else
+        hipLaunchKernelGGL((splitk_reduce_kernel<T, 1>), dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, s,
+                           static_cast<const T *>(target), static_cast<T *>(dw), count, pl.splits);
     }
     MG_HIP(hipGetLastError());
   }

@@ -75,13 +75,17 @@ struct Phase {
 };
 static_assert(sizeof(Phase) == 96, "Phase is read as three 32-byte rows");
 
-// Gather-GEMM:  dst[n, m, pos] = sum_k A[arow[k]][m] * src[n, row k, pos]
+// Gather-GEMM:  dst[n, m, pos] = sum_k A(k, m) * src[n, row k, pos]
+// The tap-major kernels read A from packed filters, [rows][a_ld] with the M values of a row
+// contiguous; the table-driven kernel reads the filter bank where it lies:
+// A(k, m) = A[arow[k] + m * a_mstride].
 struct GemmParams {
-  const void *A;  // packed filters, [rows][M] with M contiguous
+  const void *A;
   const void *src;
   void *dst;
   const TabEntry *tab;
-  const int *arow;  // table row -> row of A
+  const int *arow;  // table row -> offset of its m = 0 element in the filter bank
+  int a_mstride;    // elements between consecutive m in the filter bank
   const Phase *phases;
   int nphases;
   int M;

@@ -297,9 +297,19 @@ def test_conv_random_cases_vs_oracle(abi, dtype, m, big):
         done += 1
 
 
+@pytest.fixture(params=["small problems planned as such", "planned like large ones"])
+def plan_mode(request, monkeypatch):
+    """A convolution of a few microseconds is planned for few launches (table-driven kernels
+    that read the filter bank in place); MYGRAD_HIP_TINY=0 plans it like a large one, which
+    is how shapes this small reach the tap-major kernels' edge cases."""
+    if request.param == "planned like large ones":
+        monkeypatch.setenv("MYGRAD_HIP_TINY", "0")
+    return request.param
+
+
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("m", [1, 2, 3])
-def test_conv_channel_counts_that_take_the_tap_major_kernels(abi, dtype, m):
+def test_conv_channel_counts_that_take_the_tap_major_kernels(abi, dtype, m, plan_mode):
     # channel / filter counts that are multiples of the K tile (8 or 16) select the
     # tap-major kernels; mix them with counts that do not, strides, dilation, padding
     rng = np.random.default_rng(500 + m)
@@ -355,7 +365,7 @@ FUSED_PHASE_CASES = [
 
 
 @pytest.mark.parametrize("case", range(len(FUSED_PHASE_CASES)))
-def test_conv_dgrad_with_fused_stride_phases(abi, case):
+def test_conv_dgrad_with_fused_stride_phases(abi, case, plan_mode):
     x_shape, w_shape, s, p, d = FUSED_PHASE_CASES[case]
     rng = np.random.default_rng(900 + case)
     w = (rng.standard_normal(w_shape) / np.sqrt(np.prod(w_shape[1:]))).astype(np.float32)
