@@ -81,7 +81,10 @@ def test_results_repeat_exactly(abi):
 
 
 BATCHED = [(1, 1, 1, 1), (3, 16, 16, 16), (5, 17, 3, 33), (2, 1, 70, 1), (300, 8, 8, 8), (7, 64, 40, 48), (4, 33, 6, 2), (2, 5, 0, 4),
-           (3, 100, 129, 50)]
+           (3, 100, 129, 50),
+           # 32 x 32 results or more per pair: 64 x 64 tiles staged in LDS -- whole tiles, ragged edges in M, N
+           # and K, several K chunks, row lengths that are and are not whole 16-byte pieces
+           (9, 64, 64, 64), (3, 130, 70, 96), (2, 32, 200, 32), (5, 47, 33, 61), (2, 128, 64, 192)]
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
