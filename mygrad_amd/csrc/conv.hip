@@ -75,6 +75,11 @@ struct Mma<double> {
 // filter packing: the tap-major GEMMs want the filter operand with M contiguous
 //   mode 2 (forward) : Ap[(t*C + c)][f] = w[f][c][t]
 //   mode 3 (dgrad)   : Ap[(t*F + f)][c] = w[f][c][t]
+//   modes 4 / 5 (dgrad / forward with the three taps t2 of the last axis folded into the rows;
+//           u is the tap of the other axes):
+//           Ap[(u*F + f)][3*c + t2] = w[f][c][u][t2]      Ap[(u*C + c)][3*f + 2 - t2] = w[f][c][u][t2]
+//           (the row of a tap is added to dst one position to the right of the row after it:
+//           the forward pass reads x to the right of a later tap, the gradient to the left)
 // Every row is padded with zeros to a multiple of four values (`ld` values per row), so
 // that the kernels can read a row sixteen bytes at a time whatever M is.  (The
 // table-driven kernel reads the filter bank in place.)
@@ -103,7 +108,7 @@ __global__ void __launch_bounds__(256) pack_transpose_kernel(const T *__restrict
 template <typename T>
 __global__ void __launch_bounds__(256) pack_filters_kernel(const T *__restrict__ w, T *__restrict__ ap, int F, int C,
                                                            int wvol, int mode, int ld) {
-  const int M = mode == 2 ? F : C;
+  const int M = mode == 2 ? F : mode == 3 ? C : mode == 4 ? 3 * C : 3 * F;
   const int total = (F * C * wvol / M) * ld;
   for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
     // idx enumerates the packed layout so that stores are coalesced
@@ -118,10 +123,18 @@ __global__ void __launch_bounds__(256) pack_filters_kernel(const T *__restrict__
       f = m;
       c = row % C;
       t = row / C;
-    } else {
+    } else if (mode == 3) {
       c = m;
       f = row % F;
       t = row / F;
+    } else if (mode == 4) {
+      c = m / 3;
+      f = row % F;
+      t = (row / F) * 3 + m % 3;
+    } else {
+      f = m / 3;
+      c = row % C;
+      t = (row / C) * 3 + 2 - m % 3;
     }
     ap[idx] = w[((long long)f * C + c) * wvol + t];
   }
@@ -533,6 +546,7 @@ struct Plan {
   int blocks_per_cu = 1;  // persistent blocks per compute unit (streaming gather-GEMM)
   bool tap_major = false;  // which kernel family the tables are for
   bool single_dense_phase = false;  // positions enumerate the destination tensor in order
+  int fold_row = 0;                 // data gradient with the last axis' three taps folded into the rows: length of a row of positions
   bool deep_k = false;              // table-driven, a few microseconds of work: 16 x 64 tiles with a K tile four times as deep
   // fused stride phases of the data gradient (see GemmParams::nph)
   int nph = 1;
@@ -853,6 +867,34 @@ void fwd_table(const Geometry &g, std::vector<TabEntry> &tab) {
         }
 }
 
+// Whether the three taps of the last axis can be rows of the GEMM (see GemmParams::fold_row)
+// for a problem with `rows` rows (filters in the forward pass, channels in the data gradient):
+// float, few rows (with 16 or 32 the plain tiles are bound by the gather, not by the matrix
+// pipes: a gathered element feeds three times the MFMAs this way), a 3-tap "same" last axis
+// with unit stride and dilation, and rows of positions that a wave's 64 positions hold whole
+// (a power of two up to 64).  MYGRAD_HIP_FOLD=0 switches it off.
+bool fold_applies(const Geometry &g, int rows) {
+  static const bool fold_on = [] {
+    const char *flag = getenv("MYGRAD_HIP_FOLD");
+    return !(flag && flag[0] == '0');
+  }();
+  const bool row_fits = g.X[2] >= 4 && g.X[2] <= 64 && (g.X[2] & (g.X[2] - 1)) == 0;
+  return fold_on && g.dtype == MG_F32 && rows <= 32 && g.W[2] == 3 && g.P[2] == 1 && g.D[2] == 1 && g.S[2] == 1 &&
+         g.G[2] == g.X[2] && row_fits;
+}
+
+// Tile of a plan with folded taps: 48 rows x 256 positions for up to 16 channels (one block per
+// tile), 96 x 128 for up to 32 (persistent blocks, as many as fit on the device, every tile whole).
+void set_fold_tile(Plan &pl, int rows) {
+  pl.m_tiles = 1, pl.tail_split = 1, pl.blocks_per_cu = 1;
+  if (rows <= 16) {
+    pl.bm = 48, pl.bn = 256;
+  } else {
+    pl.bm = 96, pl.bn = 128;
+    pl.blocks_per_cu = resident_blocks(tap_gemm_kernel<float, 96, 128, 16, 48, 64, 1, true>, 512);
+  }
+}
+
 // A problem of a few microseconds is bound by its launches and by the chain of K tiles a
 // block runs through, each a round trip to memory, not by the matrix pipes.
 // MYGRAD_HIP_TINY=0 plans such a problem like a large one (read whenever a plan is built, and
@@ -894,6 +936,28 @@ int build_fwd_plan(const Geometry &g, Plan &pl) {
   ph.blk_begin = 0;
   ph.npos = (int)((long long)g.N * g.gvol);
   set_divisors(ph);
+  if (pl.tap_major && fold_applies(g, g.F)) {
+    // rows (filter, tap of the last axis); K tiles over the taps of the other axes
+    const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
+    for (int c0 = 0; c0 < g.C; c0 += bk)
+      for (int t0 = 0; t0 < g.W[0]; ++t0)
+        for (int t1 = 0; t1 < g.W[1]; ++t1) {
+          KTile e{};
+          e.d0 = t0 * g.D[0] - g.P[0];
+          e.d1 = t1 * g.D[1] - g.P[1];
+          e.d2 = 0;
+          e.a_row0 = (t0 * g.W[1] + t1) * g.C + c0;
+          e.coff = (int)(c0 * g.xvol) + e.d0 * qs[0] + e.d1 * qs[1];
+          t.ktiles.push_back(e);
+        }
+    ph.k_count = (int)t.ktiles.size();
+    pl.fold_row = g.X[2];
+    set_fold_tile(pl, g.F);
+    pl.pos_blocks = (int)ceil_div(ph.npos, pl.bn);
+    pl.full_tiles = pl.pos_blocks;
+    t.phases.push_back(ph);
+    return upload_plan(pl, t);
+  }
   if (pl.tap_major) {
     // K tiles run channel block by channel block, all taps of a block back to back:
     // the taps of one channel block re-read the same few rows of x, which then come
@@ -966,6 +1030,37 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
         set_divisors(pt.ph);
         found.push_back(pt);
       }
+
+  // ---- few channels, unit strides, a 3-tap "same" last axis (float): the rows of the GEMM are
+  // (channel, tap of the last axis), three times as many as there are channels, and the K tiles
+  // run over the taps of the other axes only.  A gathered element of grad then feeds three
+  // times the MFMAs -- with 16 channels the plain tiles are bound by the gather, not by the
+  // matrix pipes -- and the epilogue adds the three rows of a channel, shifted along the last
+  // axis, into dx.  A wave's 64 positions must be whole rows: X2 a power of two up to 64.
+  if (fold_applies(g, g.C) && pl.tap_major && nphase == 1 && found.size() == 1) {
+    const PhaseTaps &pt = found[0];
+    Phase ph = pt.ph;
+    for (int f0 = 0; f0 < g.F; f0 += bk)
+      for (size_t a = 0; a < pt.taps[0].size(); ++a)
+        for (size_t b = 0; b < pt.taps[1].size(); ++b) {
+          KTile e{};
+          e.d0 = pt.offs[0][a];
+          e.d1 = pt.offs[1][b];
+          e.d2 = 0;
+          e.a_row0 = (pt.taps[0][a] * g.W[1] + pt.taps[1][b]) * g.F + f0;
+          e.coff = (int)(f0 * g.gvol) + e.d0 * gs[0] + e.d1 * gs[1];
+          t.ktiles.push_back(e);
+        }
+    ph.k_begin = 0;
+    ph.k_count = (int)t.ktiles.size();
+    ph.blk_begin = 0;
+    pl.fold_row = g.X[2];
+    set_fold_tile(pl, g.C);
+    pl.pos_blocks = (int)ceil_div(ph.npos, pl.bn);
+    pl.full_tiles = pl.pos_blocks;
+    t.phases.push_back(ph);
+    return upload_plan(pl, t);
+  }
 
   // ---- stride 2 along the last axis: the phases' elements alternate in dx, and phases that
   // write them at different times make every line of dx cross HBM several times, partly
@@ -1247,19 +1342,19 @@ int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
   return MG_OK;
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int NPH = 1>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int NPH = 1, bool FOLD = false>
 void launch_gemm(GemmParams &gp, const Plan &pl, hipStream_t s) {
   if (pl.tap_major) {
     const long long tiles = (long long)pl.pos_blocks * pl.m_tiles;
     const long long tail_tiles = tiles - pl.full_tiles;
     const long long slots = tap_gemm_streams(BM, (int)sizeof(T)) ? (long long)pl.blocks_per_cu * runtime().props.multiProcessorCount : (1ll << 40);
     gp.items = (int)(pl.full_tiles + tail_tiles * pl.tail_split);
-    hipLaunchKernelGGL((tap_gemm_kernel<T, BM, BN, BK, WM, WN, NPH>), dim3((unsigned)std::min<long long>(gp.items, slots)), dim3(512),
-                       0, s, gp);
+    hipLaunchKernelGGL((tap_gemm_kernel<T, BM, BN, BK, WM, WN, NPH, FOLD>), dim3((unsigned)std::min<long long>(gp.items, slots)),
+                       dim3(512), 0, s, gp);
     if (tail_tiles > 0)
       hipLaunchKernelGGL((tail_fixup_kernel<T, BM, BN, NPH>), dim3((unsigned)ceil_div(BM * BN, 256), (unsigned)tail_tiles),
                          dim3(256), 0, s, gp);
-  } else if constexpr (NPH == 1) {
+  } else if constexpr (NPH == 1 && !FOLD) {
     const dim3 grid((unsigned)pl.pos_blocks, (unsigned)pl.m_tiles);
     hipLaunchKernelGGL((gather_gemm_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, gp);
   }
@@ -1306,6 +1401,16 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
     launch_gemm<T, 16, 64, 4 * BK, 16, 16>(gp, pl, s);
     launched = true;
   }
+  gp.fold_row = pl.fold_row;
+  if constexpr (sizeof(T) == 4) {
+    if (pl.fold_row) {
+      if (pl.bm == 48)
+        launch_gemm<T, 48, 256, BK, 48, 64, 1, true>(gp, pl, s);
+      else
+        launch_gemm<T, 96, 128, BK, 48, 64, 1, true>(gp, pl, s);
+      launched = true;
+    }
+  }
 #define MG_LAUNCH(TT, BM, BN, WM, WN)                     \
   if (!launched && pl.bm == BM && pl.bn == BN) {          \
     launch_gemm<TT, BM, BN, BK, WM, WN>(gp, pl, s);       \
@@ -1346,7 +1451,7 @@ inline int packed_ld(int M, bool tap_major) { return tap_major ? (M + 3) / 4 * 4
 
 template <typename T>
 int pack_filters(const Geometry &g, const void *w, int mode, void **packed, size_t extra = 0, void **behind = nullptr) {
-  const int M = mode == 2 ? g.F : g.C;
+  const int M = mode == 2 ? g.F : mode == 3 ? g.C : mode == 4 ? 3 * g.C : 3 * g.F;
   const int ld = packed_ld(M, true);
   const size_t count = (size_t)g.F * g.C * g.wvol / M * ld;
   const size_t packed_bytes = (count * sizeof(T) + 255) & ~size_t(255);
@@ -1382,7 +1487,7 @@ int conv_fwd_impl(const Geometry &g, const Plan &pl, const void *x, const void *
   void *partial = nullptr;
   if (!pl.tap_major) {
     packed = const_cast<void *>(w);  // read in place: row k = (c, taps) of filter m lies at w[m * C*taps + k]
-  } else if (int rc = pack_filters<T>(g, w, 2, &packed, tail_bytes(pl, sizeof(T)), &partial)) {
+  } else if (int rc = pack_filters<T>(g, w, pl.fold_row ? 5 : 2, &packed, tail_bytes(pl, sizeof(T)), &partial)) {
     return rc;
   }
   GemmParams gp{};
@@ -1405,8 +1510,8 @@ int conv_fwd_impl(const Geometry &g, const Plan &pl, const void *x, const void *
   gp.src_cstride = (int)g.xvol;
   gp.src_nstride = (long long)g.C * g.xvol;
   gp.dst_nstride = (long long)g.F * g.gvol;
-  gp.a_ld = packed_ld(g.F, pl.tap_major);
-  gp.a_bytes = (unsigned)((size_t)g.C * g.wvol * gp.a_ld * sizeof(T));
+  gp.a_ld = packed_ld(pl.fold_row ? 3 * g.F : g.F, pl.tap_major);
+  gp.a_bytes = (unsigned)((size_t)g.C * (pl.fold_row ? g.wvol / 3 : g.wvol) * gp.a_ld * sizeof(T));
   gp.src_bytes = pl.tap_major ? (unsigned)((size_t)g.N * g.C * g.xvol * sizeof(T)) : 0;
   return run_gemm<T>(gp, pl, TAG_CONV_FWD, runtime().stream);
 }
@@ -1417,7 +1522,7 @@ int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   void *partial = nullptr;
   if (!pl.tap_major) {
     packed = const_cast<void *>(w);  // read in place: row k = (f, tap) of channel m lies at w[(f * C + m) * taps + tap]
-  } else if (int rc = pack_filters<T>(g, w, 3, &packed, tail_bytes(pl, sizeof(T)), &partial)) {
+  } else if (int rc = pack_filters<T>(g, w, pl.fold_row ? 4 : 3, &packed, tail_bytes(pl, sizeof(T)), &partial)) {
     return rc;
   }
   GemmParams gp{};
@@ -1440,8 +1545,8 @@ int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   gp.src_cstride = (int)g.gvol;
   gp.src_nstride = (long long)g.F * g.gvol;
   gp.dst_nstride = (long long)g.C * g.xvol;
-  gp.a_ld = packed_ld(g.C, pl.tap_major);
-  gp.a_bytes = (unsigned)((size_t)g.F * g.wvol * gp.a_ld * sizeof(T));
+  gp.a_ld = packed_ld(pl.fold_row ? 3 * g.C : g.C, pl.tap_major);
+  gp.a_bytes = (unsigned)((size_t)g.F * (pl.fold_row ? g.wvol / 3 : g.wvol) * gp.a_ld * sizeof(T));
   gp.src_bytes = pl.tap_major ? (unsigned)((size_t)g.N * g.F * g.gvol * sizeof(T)) : 0;
   return run_gemm<T>(gp, pl, TAG_CONV_DGRAD, runtime().stream);
 }

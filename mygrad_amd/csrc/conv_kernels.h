@@ -117,6 +117,11 @@ struct GemmParams {
                         // phases); tiles [kcut[f-1], kcut[f]) of a block belong to phase f (kcut[-1] = 0)
   int po0[4][3];        // destination coordinate of coarse position (0,0,0) in phase f
   int pJ[4][3];         // coarse positions j_k < pJ[f][k] exist in phase f
+  // Taps of the last axis folded into the rows (tap-major kernel with FOLD): row 3*m + t of a tile
+  // holds the sum over the taps of the other axes only, for tap t of the last axis, at the
+  // position's own place along that axis; the epilogue adds the three rows of an m, each shifted
+  // by its tap's offset along the last axis (+1, 0, -1 positions), into the one row of dst.
+  int fold_row;         // 0: not folded; else the length of a row of positions (a power of two, 4 .. 64)
 };
 
 // Filter gradient:  out[split][f][col] = sum over the split's positions (n, g) of

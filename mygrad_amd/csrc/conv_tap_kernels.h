@@ -129,8 +129,12 @@ struct Quad {
 // ------------------------------------------------------------------------------------------
 // forward and data gradient
 // ------------------------------------------------------------------------------------------
-template <typename T, int BM, int BN, int BK, int WM, int WN, int NPH = 1>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int NPH = 1, bool FOLD = false>
 __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
+  // FOLD: the three taps of the last axis are rows of the tile (see GemmParams::fold_row): three
+  // times the rows per gathered element, a third of the K tiles.  A wave makes 48 rows (16
+  // channels x 3 taps) x 64 positions, which are whole rows of the last axis.
+  static_assert(!FOLD || (NPH == 1 && WM == 48 && WN == 64 && sizeof(T) == 4), "folded taps: 48 x 64 float wave tiles");
   // NPH > 1: every tile computes NPH stride phases of the data gradient (see GemmParams::nph):
   // the K tiles of the phases follow each other in the tile's stream, each phase has its own
   // accumulators, and the epilogue writes the phases together.
@@ -514,7 +518,12 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
 #pragma unroll
         for (int k4 = 0; k4 < BK / 4; ++k4) {
           T a[TM], b[TN];
-          load_vec<T, TM>(&As[buf][k4 * 4 + lk][wm0 + l16 * TM], a);
+          if constexpr (TM == 3) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) a[i] = As[buf][k4 * 4 + lk][wm0 + l16 * TM + i];
+          } else {
+            load_vec<T, TM>(&As[buf][k4 * 4 + lk][wm0 + l16 * TM], a);
+          }
           load_vec<T, TN>(&Bs[buf][k4 * 4 + lk][wn0 + l16 * TN], b);
 #pragma unroll
           for (int i = 0; i < TM; ++i)
@@ -611,6 +620,37 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
                   const int m = m0 + wm0 + Mma<T>::row_of(lane, q) * TM + i;
                   if (m < p.M) out[(long long)m * p.dst_mstride] = acc[f][i][j][q];
                 }
+            }
+          }
+        }
+      } else if constexpr (FOLD) {
+        // Tile i of the wave holds tap i of the last axis for the lane's channels 4*lk + q and its
+        // TN = 4 adjacent positions first .. first + 3 of one row:
+        //   dst[pos] = tap1[pos] + tap0[pos + 1] + tap2[pos - 1]
+        // with zeros beyond the ends of the row.  pos + 1 and pos - 1 are in the lane itself or
+        // in its neighbours of the same quarter-wave (a wave's positions are whole rows, so the
+        // first and last lane of a quarter never need a neighbour).
+        static_assert(TM == 3 && TN == 4, "three taps, four positions per lane");
+        const unsigned in_row = (unsigned)first & (unsigned)(p.fold_row - 1);
+        const bool has_prev = in_row != 0, has_next = in_row + TN != (unsigned)p.fold_row;
+        const bool exists = first < ph.npos;
+        T *out = dst_of(exists ? first : 0);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const T from_prev = __shfl_up(acc[0][2][TN - 1][q], 1, 16);
+          const T from_next = __shfl_down(acc[0][0][0][q], 1, 16);
+          T v[TN];
+          v[0] = (acc[0][1][0][q] + acc[0][0][1][q]) + (has_prev ? from_prev : T(0));
+          v[1] = (acc[0][1][1][q] + acc[0][0][2][q]) + acc[0][2][0][q];
+          v[2] = (acc[0][1][2][q] + acc[0][0][3][q]) + acc[0][2][1][q];
+          v[3] = (acc[0][1][3][q] + (has_next ? from_next : T(0))) + acc[0][2][2][q];
+          const int m = (m0 + wm0) / 3 + Mma<T>::row_of(lane, q);
+          if (exists && m < p.M) {
+            if (p.vec_store) {
+              store_vec<T, TN>(out + (long long)m * p.dst_mstride, v);
+            } else {
+#pragma unroll
+              for (int j = 0; j < TN; ++j) out[(long long)m * p.dst_mstride + j] = v[j];
             }
           }
         }

@@ -382,6 +382,57 @@ def test_conv_dgrad_with_fused_stride_phases(abi, case, plan_mode):
                           direct.conv_backward_x(ones_g, x_shape, ones_w, s, p, d).astype(np.float32))
 
 
+# Few channels (filters, in the forward pass), a 3-tap "same" last axis whose rows are a power of
+# two up to 64 long (float32, the other count a multiple of 16): the data gradient and the forward
+# pass compute the three taps of the last axis as separate rows and add them, shifted, in the epilogue.  1, 2 and 3 convolved axes,
+# row lengths 4 .. 64, channel counts that do and do not fill the tile, other axes with padding,
+# dilation and even tap counts, position counts that are no multiple of the tile.
+FOLDED_TAP_CASES = [
+    ((2, 16, 8, 64, 64), (32, 16, 3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
+    ((3, 16, 40, 32), (16, 16, 3, 3), (1, 1), (1, 1), (1, 1)),
+    ((5, 8, 21, 16), (48, 8, 2, 3), (1, 1), (0, 1), (1, 1)),
+    ((7, 5, 9, 8), (16, 5, 5, 3), (1, 1), (4, 1), (2, 1)),
+    ((9, 12, 64), (32, 12, 3), (1,), (1,), (1,)),
+    ((2, 3, 6, 10, 4), (16, 3, 1, 3, 3), (1, 1, 1), (0, 0, 1), (1, 1, 1)),
+    ((1, 16, 33, 64), (64, 16, 1, 3), (1, 1), (0, 1), (1, 1)),
+    ((2, 32, 16, 32), (16, 32, 3, 3), (1, 1), (1, 1), (1, 1)),       # 32 channels: 96-row tiles
+    ((3, 24, 10, 16), (32, 24, 3, 3), (1, 1), (1, 1), (1, 1)),       # 24 channels in a 96-row tile
+    ((2, 48, 12, 9, 32), (24, 48, 2, 3, 3), (2, 1, 1), (0, 2, 1), (1, 2, 1)),  # forward only folds (24 filters; stride on axis 0)
+]
+
+
+@pytest.mark.parametrize("case", range(len(FOLDED_TAP_CASES)))
+def test_conv_with_the_last_axis_taps_folded_into_rows(abi, case, monkeypatch):
+    monkeypatch.setenv("MYGRAD_HIP_TINY", "0")  # small shapes: planned like large ones, or they take the table-driven kernel
+    x_shape, w_shape, s, p, d = FOLDED_TAP_CASES[case]
+    rng = np.random.default_rng(1300 + case)
+    w = (rng.standard_normal(w_shape) / np.sqrt(np.prod(w_shape[1:]))).astype(np.float32)
+    grid = tuple((x + 2 * pp - ((t - 1) * dd + 1)) // ss + 1 for x, t, ss, pp, dd in zip(x_shape[2:], w_shape[2:], s, p, d))
+    g = rng.standard_normal((x_shape[0], w_shape[0], *grid)).astype(np.float32)
+    dx = abi.conv_dgrad(g, x_shape, w, s, p, d)
+    assert rel_err(dx, direct.conv_backward_x(g, x_shape, w, s, p, d)) <= 2e-4
+    assert np.array_equal(dx, abi.conv_dgrad(g, x_shape, w, s, p, d))
+    # exact with ones: per input element, the number of (filter, tap) pairs that reach it -- a
+    # shift in the wrong direction or a neighbour taken across a row end changes the counts
+    ones_w = np.ones(w_shape, dtype=np.float32)
+    ones_g = np.ones_like(g)
+    assert np.array_equal(abi.conv_dgrad(ones_g, x_shape, ones_w, s, p, d),
+                          direct.conv_backward_x(ones_g, x_shape, ones_w, s, p, d).astype(np.float32))
+    # and with a filter that is not symmetric along the last axis (tap t2 weighs t2 + 1), so that
+    # tap 0 and tap 2 cannot be swapped unnoticed
+    ramp_w = np.ones(w_shape, dtype=np.float32) * np.arange(1, w_shape[-1] + 1, dtype=np.float32)
+    assert np.array_equal(abi.conv_dgrad(ones_g, x_shape, ramp_w, s, p, d),
+                          direct.conv_backward_x(ones_g, x_shape, ramp_w, s, p, d).astype(np.float32))
+    # the forward pass folds the same way when there are few filters (and channels in whole K tiles)
+    x = rng.standard_normal(x_shape).astype(np.float32)
+    out = abi.conv_fwd(x, w, s, p, d)
+    assert rel_err(out, direct.conv_forward(x, w, s, p, d)) <= 2e-4
+    assert np.array_equal(out, abi.conv_fwd(x, w, s, p, d))
+    # exact: x counts along the last axis (small integers), ramp filter
+    steps = np.broadcast_to(np.arange(x_shape[-1], dtype=np.float32) % 5, x_shape).copy()
+    assert np.array_equal(abi.conv_fwd(steps, ramp_w, s, p, d), direct.conv_forward(steps, ramp_w, s, p, d).astype(np.float32))
+
+
 # Shapes picked so that, between them, every tile shape and code path of the tap-major
 # kernels runs: all gather-GEMM tiles (rows 16..128), persistent blocks that stream
 # through several tiles and K slices, strided dgrad phases, filter counts that are not a
