@@ -527,6 +527,10 @@ bool fits_buffer_loads(const Geometry &g) {
 
 // K tile of the gather-GEMMs (positions x filters-or-channels x BK).
 int gemm_bk(int dtype) { return dtype == MG_F64 ? 8 : 16; }
+// K tile of a tap-major plan that contracts `channels` channels per tap.  Double precision: 16
+// where the channels allow it -- a K tile of 8 is 64 MFMAs per wave between two barriers, and
+// the barriers then cost a tenth of the time (config 4: forward 122 -> 115 us, dx 130 -> 119 us).
+int tap_bk(int dtype, int channels) { return dtype == MG_F64 && channels % 16 != 0 ? 8 : 16; }
 
 struct Plan {
   void *blob = nullptr;  // one device allocation holding every table below
@@ -539,7 +543,7 @@ struct Plan {
   int nphases = 0;
   int pos_blocks = 0;  // position blocks of the gather-GEMM (all phases)
   int bm = 0, bn = 0;
-  int bk = 0;           // K tile of the filter-gradient kernel chosen for this plan
+  int bk = 0;           // depth of a K tile of the kernel chosen for this plan
   int m_tiles = 1;     // row tiles per position block
   int full_tiles = 0;  // tiles computed whole by one block (tap-major kernel)
   int tail_split = 1;  // blocks sharing each of the remaining tiles
@@ -658,10 +662,12 @@ int resident_blocks(K kernel, int threads) {
 
 // Blocks of the persistent tap-major gather-GEMM that a compute unit holds at once.
 template <typename T>
-int gemm_blocks_per_cu(int bm, int bn, int nph = 1) {
+int gemm_blocks_per_cu(int bm, int bn, int nph = 1, int bk = 0) {
   constexpr int BK = sizeof(T) == 8 ? 8 : 16;
-#define MG_OCC(TT, BM, BN, WM, WN) \
-  if (bm == BM && bn == BN) return resident_blocks(tap_gemm_kernel<TT, BM, BN, BK, WM, WN>, 512);
+#define MG_OCC(TT, BM, BN, WM, WN)                                                                                       \
+  if (bm == BM && bn == BN)                                                                                              \
+    return bk == 2 * BK ? resident_blocks(tap_gemm_kernel<TT, BM, BN, (sizeof(TT) == 8 ? 2 * BK : BK), WM, WN>, 512)     \
+                        : resident_blocks(tap_gemm_kernel<TT, BM, BN, BK, WM, WN>, 512);
 #define MG_OCC2(TT, BM, BN, WM, WN) \
   if (bm == BM && bn == BN) return resident_blocks(tap_gemm_kernel<TT, BM, BN, BK, WM, WN, 2>, 512);
 #define MG_OCC4(TT, BM, BN, WM, WN) \
@@ -699,7 +705,7 @@ struct TileChoice {
   long long tiles;
 };
 
-TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_ktiles, bool tap_major, size_t elem, int nph = 1) {
+TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_ktiles, bool tap_major, size_t elem, int nph = 1, int bk = 0) {
   struct Cfg {
     int bm, bn;
     double penalty;  // relative cost of a flop in this tile shape
@@ -722,7 +728,7 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
     // fits on a compute unit, so the tap-major kernels use the half-size shapes
     if (tap_major && elem == 8 && c.bn * c.bm >= 128 * 128) continue;
     const bool stream = tap_major && tap_gemm_streams(c.bm, (int)elem);
-    const int per_cu = !stream ? 1 : elem == 8 ? gemm_blocks_per_cu<double>(c.bm, c.bn) : gemm_blocks_per_cu<float>(c.bm, c.bn, nph);
+    const int per_cu = !stream ? 1 : elem == 8 ? gemm_blocks_per_cu<double>(c.bm, c.bn, 1, bk) : gemm_blocks_per_cu<float>(c.bm, c.bn, nph);
     long long pos_blocks = 0;
     for (long long n : phase_npos) pos_blocks += ceil_div(n, c.bn);
     for (int r = 1; r <= per_cu; ++r) {
@@ -918,12 +924,13 @@ void deepen_if_tiny(const Geometry &g, Plan &pl) {
 
 int build_fwd_plan(const Geometry &g, Plan &pl) {
   Tables t;
-  const int bk = gemm_bk(g.dtype);
-  pl.tap_major = g.C % bk == 0 && fits_buffer_loads(g);
+  pl.tap_major = g.C % gemm_bk(g.dtype) == 0 && fits_buffer_loads(g);
+  const int bk = pl.tap_major ? tap_bk(g.dtype, g.C) : gemm_bk(g.dtype);
+  pl.bk = bk;
   pl.single_dense_phase = true;
   {
     const long long ktiles = pl.tap_major ? g.wvol * (g.C / bk) : ceil_div((long long)g.C * g.wvol, bk);
-    const TileChoice tc = choose_tile(g.F, {(long long)g.N * g.gvol}, (int)ktiles, pl.tap_major, g.dtype == MG_F64 ? 8 : 4);
+    const TileChoice tc = choose_tile(g.F, {(long long)g.N * g.gvol}, (int)ktiles, pl.tap_major, g.dtype == MG_F64 ? 8 : 4, 1, bk);
     pl.bm = tc.bm, pl.bn = tc.bn, pl.m_tiles = tc.m_tiles, pl.full_tiles = tc.full_tiles, pl.tail_split = tc.tail_split, pl.blocks_per_cu = tc.blocks_per_cu;
     deepen_if_tiny(g, pl);
   }
@@ -990,10 +997,11 @@ int build_fwd_plan(const Geometry &g, Plan &pl) {
 
 int build_dgrad_plan(const Geometry &g, Plan &pl) {
   Tables t;
-  const int bk = gemm_bk(g.dtype);
   // a tiny problem is bound by its launches: the table-driven kernel needs neither packed
   // filters nor a pass over partial sums
-  pl.tap_major = g.F % bk == 0 && fits_buffer_loads(g) && !is_tiny(g);
+  pl.tap_major = g.F % gemm_bk(g.dtype) == 0 && fits_buffer_loads(g) && !is_tiny(g);
+  const int bk = pl.tap_major ? tap_bk(g.dtype, g.F) : gemm_bk(g.dtype);
+  pl.bk = bk;
   pl.single_dense_phase = g.S[0] == 1 && g.S[1] == 1 && g.S[2] == 1;
   const int gs[3] = {g.G[1] * g.G[2], g.G[2], 1};
   long long nphase = (long long)g.S[0] * g.S[1] * g.S[2];
@@ -1144,7 +1152,7 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
       const long long ntaps = (long long)pt.taps[0].size() * pt.taps[1].size() * pt.taps[2].size();
       min_ktiles = std::min(min_ktiles, pl.tap_major ? ntaps * (g.F / bk) : ceil_div(ntaps * g.F, bk));
     }
-    const TileChoice tc = choose_tile(g.C, npos, (int)std::max<long long>(min_ktiles, 0), pl.tap_major, g.dtype == MG_F64 ? 8 : 4);
+    const TileChoice tc = choose_tile(g.C, npos, (int)std::max<long long>(min_ktiles, 0), pl.tap_major, g.dtype == MG_F64 ? 8 : 4, 1, bk);
     pl.bm = tc.bm, pl.bn = tc.bn, pl.m_tiles = tc.m_tiles, pl.full_tiles = tc.full_tiles, pl.tail_split = tc.tail_split, pl.blocks_per_cu = tc.blocks_per_cu;
     deepen_if_tiny(g, pl);
   }
@@ -1400,6 +1408,17 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
   if (pl.deep_k) {
     launch_gemm<T, 16, 64, 4 * BK, 16, 16>(gp, pl, s);
     launched = true;
+  }
+  if constexpr (sizeof(T) == 8) {
+    if (pl.tap_major && pl.bk == 2 * BK) {
+#define MG_LAUNCH_DEEP(TT, BM, BN, WM, WN)                \
+  if (!launched && pl.bm == BM && pl.bn == BN) {          \
+    launch_gemm<TT, BM, BN, 2 * BK, WM, WN>(gp, pl, s);   \
+    launched = true;                                      \
+  }
+      MG_GEMM_SHAPES(T, MG_LAUNCH_DEEP)
+#undef MG_LAUNCH_DEEP
+    }
   }
   gp.fold_row = pl.fold_row;
   if constexpr (sizeof(T) == 4) {
