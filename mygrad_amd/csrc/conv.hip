@@ -670,8 +670,10 @@ int gemm_blocks_per_cu(int bm, int bn, int nph = 1, int bk = 0) {
                         : resident_blocks(tap_gemm_kernel<TT, BM, BN, BK, WM, WN>, 512);
 #define MG_OCC2(TT, BM, BN, WM, WN) \
   if (bm == BM && bn == BN) return resident_blocks(tap_gemm_kernel<TT, BM, BN, BK, WM, WN, 2>, 512);
-#define MG_OCC4(TT, BM, BN, WM, WN) \
-  if (bm == BM && bn == BN) return resident_blocks(tap_gemm_kernel<TT, BM, BN, BK, WM, WN, 4>, 512);
+#define MG_OCC4(TT, BM, BN, WM, WN)                                                                                       \
+  if (bm == BM && bn == BN)                                                                                                \
+    return bk == 2 * BK ? resident_blocks(tap_gemm_kernel<TT, BM, BN, (sizeof(TT) == 4 ? 2 * BK : BK), WM, WN, 4>, 512)     \
+                        : resident_blocks(tap_gemm_kernel<TT, BM, BN, BK, WM, WN, 4>, 512);
   if constexpr (sizeof(T) == 4) {
     if (nph == 2) {
       MG_FUSED2_SHAPES(T, MG_OCC2)
@@ -728,7 +730,7 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
     // fits on a compute unit, so the tap-major kernels use the half-size shapes
     if (tap_major && elem == 8 && c.bn * c.bm >= 128 * 128) continue;
     const bool stream = tap_major && tap_gemm_streams(c.bm, (int)elem);
-    const int per_cu = !stream ? 1 : elem == 8 ? gemm_blocks_per_cu<double>(c.bm, c.bn, 1, bk) : gemm_blocks_per_cu<float>(c.bm, c.bn, nph);
+    const int per_cu = !stream ? 1 : elem == 8 ? gemm_blocks_per_cu<double>(c.bm, c.bn, 1, bk) : gemm_blocks_per_cu<float>(c.bm, c.bn, nph, bk);
     long long pos_blocks = 0;
     for (long long n : phase_npos) pos_blocks += ceil_div(n, c.bn);
     for (int r = 1; r <= per_cu; ++r) {
@@ -995,6 +997,14 @@ int build_fwd_plan(const Geometry &g, Plan &pl) {
   return upload_plan(pl, t);
 }
 
+bool deep_fused_on() {
+  static const bool on = [] {
+    const char *flag = getenv("MYGRAD_HIP_FUSE_BK32");
+    return !(flag && flag[0] == '0');
+  }();
+  return on;
+}
+
 int build_dgrad_plan(const Geometry &g, Plan &pl) {
   Tables t;
   // a tiny problem is bound by its launches: the table-driven kernel needs neither packed
@@ -1088,6 +1098,10 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
       return a.ph.o0[2] < b.ph.o0[2];
     });
     pl.nph = (int)nphase;
+    // Four phases share a tile's time: a K tile of 16 would be 16 MFMAs per wave between two
+    // barriers.  With 32 filters per K tile the barriers cost half as much.
+    const int fbk = nphase == 4 && g.F % 32 == 0 && deep_fused_on() ? 32 : bk;
+    pl.bk = fbk;
     Phase coarse{};
     long long total_ktiles = 0;
     for (int k = 0; k < 3; ++k) coarse.J[k] = (g.X[k] + g.S[k] - 1) / g.S[k];
@@ -1103,7 +1117,7 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
     }
     // filter block outermost, then the phases, then a phase's taps: all taps of one filter block
     // read the same neighbourhood of grad, whichever phase they belong to
-    for (int f0 = 0; f0 < g.F; f0 += bk)
+    for (int f0 = 0; f0 < g.F; f0 += fbk)
       for (int f = 0; f < pl.nph; ++f) {
         const PhaseTaps &pt = found[f];
         for (size_t a = 0; a < pt.taps[0].size(); ++a)
@@ -1125,7 +1139,7 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
     coarse.blk_begin = 0;
     coarse.npos = (int)((long long)g.N * coarse.J[0] * coarse.J[1] * coarse.J[2]);
     set_divisors(coarse);
-    const TileChoice tc = choose_tile(g.C, {(long long)coarse.npos}, (int)total_ktiles, true, 4, pl.nph);
+    const TileChoice tc = choose_tile(g.C, {(long long)coarse.npos}, (int)total_ktiles, true, 4, pl.nph, fbk);
     if (tc.bm != 0 && total_ktiles > 0) {
       pl.bm = tc.bm, pl.bn = tc.bn, pl.m_tiles = tc.m_tiles, pl.full_tiles = tc.full_tiles, pl.tail_split = tc.tail_split, pl.blocks_per_cu = tc.blocks_per_cu;
       t.phases.push_back(coarse);
@@ -1134,6 +1148,7 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
     }
     // no tile shape for this row count: the phases run one after the other
     pl.nph = 1;
+    pl.bk = bk;
     t.ktiles.clear();
   }
 
@@ -1448,6 +1463,14 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
   if constexpr (sizeof(T) == 4) {
     if (pl.nph == 2) {
       MG_FUSED2_SHAPES(T, MG_LAUNCH2)
+    } else if (pl.nph == 4 && pl.bk == 2 * BK) {
+#define MG_LAUNCH4_DEEP(TT, BM, BN, WM, WN)                      \
+  if (!launched && pl.bm == BM && pl.bn == BN) {                 \
+    launch_gemm<TT, BM, BN, 2 * BK, WM, WN, 4>(gp, pl, s);       \
+    launched = true;                                             \
+  }
+      MG_FUSED4_SHAPES(T, MG_LAUNCH4_DEEP)
+#undef MG_LAUNCH4_DEEP
     } else if (pl.nph == 4) {
       MG_FUSED4_SHAPES(T, MG_LAUNCH4)
     }
