@@ -75,6 +75,7 @@ struct Mma<double> {
 // filter packing: the tap-major GEMMs want the filter operand with M contiguous
 //   mode 2 (forward) : Ap[(t*C + c)][f] = w[f][c][t]
 //   mode 3 (dgrad)   : Ap[(t*F + f)][c] = w[f][c][t]
+//   mode 6 (forward, K tiles of table rows) : Ap[(c*taps + t)][f] = w[f][c][t]
 //   modes 4 / 5 (dgrad / forward with the three taps t2 of the last axis folded into the rows;
 //           u is the tap of the other axes):
 //           Ap[(u*F + f)][3*c + t2] = w[f][c][u][t2]      Ap[(u*C + c)][3*f + 2 - t2] = w[f][c][u][t2]
@@ -108,7 +109,7 @@ __global__ void __launch_bounds__(256) pack_transpose_kernel(const T *__restrict
 template <typename T>
 __global__ void __launch_bounds__(256) pack_filters_kernel(const T *__restrict__ w, T *__restrict__ ap, int F, int C,
                                                            int wvol, int mode, int ld) {
-  const int M = mode == 2 ? F : mode == 3 ? C : mode == 4 ? 3 * C : 3 * F;
+  const int M = (mode == 2 || mode == 6) ? F : mode == 3 ? C : mode == 4 ? 3 * C : 3 * F;
   const int total = (F * C * wvol / M) * ld;
   for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
     // idx enumerates the packed layout so that stores are coalesced
@@ -123,6 +124,10 @@ __global__ void __launch_bounds__(256) pack_filters_kernel(const T *__restrict__
       f = m;
       c = row % C;
       t = row / C;
+    } else if (mode == 6) {
+      f = m;
+      t = row % wvol;
+      c = row / wvol;
     } else if (mode == 3) {
       c = m;
       f = row % F;
@@ -550,6 +555,7 @@ struct Plan {
   int blocks_per_cu = 1;  // persistent blocks per compute unit (streaming gather-GEMM)
   bool tap_major = false;  // which kernel family the tables are for
   bool single_dense_phase = false;  // positions enumerate the destination tensor in order
+  bool table_rows = false;          // tap-major kernel whose K tiles are rows of the gather table (channel count no multiple of the K tile)
   int fold_row = 0;                 // data gradient with the last axis' three taps folded into the rows: length of a row of positions
   bool deep_k = false;              // table-driven, a few microseconds of work: 16 x 64 tiles with a K tile four times as deep
   // fused stride phases of the data gradient (see GemmParams::nph)
@@ -927,11 +933,21 @@ void deepen_if_tiny(const Geometry &g, Plan &pl) {
 int build_fwd_plan(const Geometry &g, Plan &pl) {
   Tables t;
   pl.tap_major = g.C % gemm_bk(g.dtype) == 0 && fits_buffer_loads(g);
-  const int bk = pl.tap_major ? tap_bk(g.dtype, g.C) : gemm_bk(g.dtype);
+  // Channels that do not fill K tiles (a first layer's one or three): the same kernel, its K
+  // tiles 16 rows of the gather table each -- unless the problem is tiny (few launches matter
+  // more) or MYGRAD_HIP_TABLE_ROWS=0 asks for the plain table-driven kernel.
+  static const bool rows_on = [] {
+    const char *flag = getenv("MYGRAD_HIP_TABLE_ROWS");
+    return !(flag && flag[0] == '0');
+  }();
+  pl.table_rows = rows_on && !pl.tap_major && fits_buffer_loads(g) && !is_tiny(g);
+  if (pl.table_rows) pl.tap_major = true;
+  const int bk = pl.table_rows ? 16 : pl.tap_major ? tap_bk(g.dtype, g.C) : gemm_bk(g.dtype);
   pl.bk = bk;
   pl.single_dense_phase = true;
   {
-    const long long ktiles = pl.tap_major ? g.wvol * (g.C / bk) : ceil_div((long long)g.C * g.wvol, bk);
+    const long long ktiles = pl.table_rows ? ceil_div((long long)g.C * g.wvol, bk)
+                             : pl.tap_major ? g.wvol * (g.C / bk) : ceil_div((long long)g.C * g.wvol, bk);
     const TileChoice tc = choose_tile(g.F, {(long long)g.N * g.gvol}, (int)ktiles, pl.tap_major, g.dtype == MG_F64 ? 8 : 4, 1, bk);
     pl.bm = tc.bm, pl.bn = tc.bn, pl.m_tiles = tc.m_tiles, pl.full_tiles = tc.full_tiles, pl.tail_split = tc.tail_split, pl.blocks_per_cu = tc.blocks_per_cu;
     deepen_if_tiny(g, pl);
@@ -945,6 +961,25 @@ int build_fwd_plan(const Geometry &g, Plan &pl) {
   ph.blk_begin = 0;
   ph.npos = (int)((long long)g.N * g.gvol);
   set_divisors(ph);
+  if (pl.table_rows) {
+    // the table in the filter's own row order (c, taps), padded to whole K tiles with rows that
+    // lie outside every input (and meet rows of A beyond its end: zeros)
+    fwd_table(g, t.tab);
+    const int rows = (int)t.tab.size();
+    for (int k0 = 0; k0 < rows; k0 += bk) {
+      KTile e{};
+      e.a_row0 = k0;
+      e.coff = k0;  // first table row of the tile
+      t.ktiles.push_back(e);
+    }
+    TabEntry outside{};
+    outside.d0 = outside.d1 = outside.d2 = 1 << 29;
+    while (t.tab.size() % bk != 0) t.tab.push_back(outside);
+    ph.k_count = (int)t.ktiles.size();
+    t.phases.push_back(ph);
+    pl.pos_blocks = (int)ceil_div(ph.npos, pl.bn);
+    return upload_plan(pl, t);
+  }
   if (pl.tap_major && fold_applies(g, g.F)) {
     // rows (filter, tap of the last axis); K tiles over the taps of the other axes
     const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
@@ -1306,17 +1341,38 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
   }
   pl.tap_major = pl.bm != 0;
   if (!pl.tap_major) {
-    pl.bm = g.F <= 16 ? 16 : (g.F <= 32 ? 32 : 64);
-    pl.bn = 64;
-    pl.bk = f64 ? 32 : 64;
-    best_splits = splits_for(pl.bm, pl.bn, pl.bk, false);
+    // Channels that fill no group of 16 columns: the tap-major kernel with one table row per
+    // column (64-column tiles, filters in whole row tiles), unless the problem is tiny or
+    // MYGRAD_HIP_TABLE_ROWS=0 asks for the plain table-driven kernel.
+    static const bool rows_on = [] {
+      const char *flag = getenv("MYGRAD_HIP_TABLE_ROWS");
+      return !(flag && flag[0] == '0');
+    }();
+    const int row_tile = g.F % 64 == 0 ? 64 : g.F % 32 == 0 ? 32 : g.F % 16 == 0 ? 16 : 0;
+    if (rows_on && row_tile && fits_buffer_loads(g) && !is_tiny(g)) {
+      pl.tap_major = pl.table_rows = true;
+      pl.bm = row_tile;
+      pl.bn = 64;
+      pl.bk = f64 ? 32 : 64;
+      best_splits = splits_for(pl.bm, pl.bn, pl.bk, true);
+    } else {
+      pl.bm = g.F <= 16 ? 16 : (g.F <= 32 ? 32 : 64);
+      pl.bn = 64;
+      pl.bk = f64 ? 32 : 64;
+      best_splits = splits_for(pl.bm, pl.bn, pl.bk, false);
+    }
   }
   const long long col_tiles = ceil_div(ct, pl.bn);
   const long long ktiles = ceil_div(kpos, pl.bk);
   const long long tiles_per_split = ceil_div(ktiles, best_splits);
   pl.kchunk = (int)(tiles_per_split * pl.bk);
   pl.splits = (int)ceil_div(kpos, pl.kchunk);
-  if (pl.tap_major) {
+  if (pl.table_rows) {
+    fwd_table(g, t.tab);
+    TabEntry outside{};
+    outside.d0 = outside.d1 = outside.d2 = 1 << 29;
+    while ((long long)t.tab.size() < col_tiles * pl.bn) t.tab.push_back(outside);
+  } else if (pl.tap_major) {
     const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
     const long long ngroups = col_tiles * (pl.bn / 16);
     for (long long gi = 0; gi < ngroups; ++gi) {
@@ -1365,19 +1421,19 @@ int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
   return MG_OK;
 }
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int NPH = 1, bool FOLD = false>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int NPH = 1, bool FOLD = false, bool ROWS = false>
 void launch_gemm(GemmParams &gp, const Plan &pl, hipStream_t s) {
   if (pl.tap_major) {
     const long long tiles = (long long)pl.pos_blocks * pl.m_tiles;
     const long long tail_tiles = tiles - pl.full_tiles;
     const long long slots = tap_gemm_streams(BM, (int)sizeof(T)) ? (long long)pl.blocks_per_cu * runtime().props.multiProcessorCount : (1ll << 40);
     gp.items = (int)(pl.full_tiles + tail_tiles * pl.tail_split);
-    hipLaunchKernelGGL((tap_gemm_kernel<T, BM, BN, BK, WM, WN, NPH, FOLD>), dim3((unsigned)std::min<long long>(gp.items, slots)),
+    hipLaunchKernelGGL((tap_gemm_kernel<T, BM, BN, BK, WM, WN, NPH, FOLD, ROWS>), dim3((unsigned)std::min<long long>(gp.items, slots)),
                        dim3(512), 0, s, gp);
     if (tail_tiles > 0)
       hipLaunchKernelGGL((tail_fixup_kernel<T, BM, BN, NPH>), dim3((unsigned)ceil_div(BM * BN, 256), (unsigned)tail_tiles),
                          dim3(256), 0, s, gp);
-  } else if constexpr (NPH == 1 && !FOLD) {
+  } else if constexpr (NPH == 1 && !FOLD && !ROWS) {
     const dim3 grid((unsigned)pl.pos_blocks, (unsigned)pl.m_tiles);
     hipLaunchKernelGGL((gather_gemm_kernel<T, BM, BN, BK, WM, WN>), grid, dim3(256), 0, s, gp);
   }
@@ -1425,7 +1481,7 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
     launched = true;
   }
   if constexpr (sizeof(T) == 8) {
-    if (pl.tap_major && pl.bk == 2 * BK) {
+    if (pl.tap_major && pl.bk == 2 * BK && !pl.table_rows) {
 #define MG_LAUNCH_DEEP(TT, BM, BN, WM, WN)                \
   if (!launched && pl.bm == BM && pl.bn == BN) {          \
     launch_gemm<TT, BM, BN, 2 * BK, WM, WN>(gp, pl, s);   \
@@ -1434,6 +1490,15 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
       MG_GEMM_SHAPES(T, MG_LAUNCH_DEEP)
 #undef MG_LAUNCH_DEEP
     }
+  }
+  if (pl.table_rows) {
+#define MG_LAUNCH_ROWS(TT, BM, BN, WM, WN)                              \
+  if (!launched && pl.bm == BM && pl.bn == BN) {                        \
+    launch_gemm<TT, BM, BN, 16, WM, WN, 1, false, true>(gp, pl, s);     \
+    launched = true;                                                    \
+  }
+    MG_GEMM_SHAPES(T, MG_LAUNCH_ROWS)
+#undef MG_LAUNCH_ROWS
   }
   gp.fold_row = pl.fold_row;
   if constexpr (sizeof(T) == 4) {
@@ -1493,7 +1558,7 @@ inline int packed_ld(int M, bool tap_major) { return tap_major ? (M + 3) / 4 * 4
 
 template <typename T>
 int pack_filters(const Geometry &g, const void *w, int mode, void **packed, size_t extra = 0, void **behind = nullptr) {
-  const int M = mode == 2 ? g.F : mode == 3 ? g.C : mode == 4 ? 3 * g.C : 3 * g.F;
+  const int M = (mode == 2 || mode == 6) ? g.F : mode == 3 ? g.C : mode == 4 ? 3 * g.C : 3 * g.F;
   const int ld = packed_ld(M, true);
   const size_t count = (size_t)g.F * g.C * g.wvol / M * ld;
   const size_t packed_bytes = (count * sizeof(T) + 255) & ~size_t(255);
@@ -1529,7 +1594,7 @@ int conv_fwd_impl(const Geometry &g, const Plan &pl, const void *x, const void *
   void *partial = nullptr;
   if (!pl.tap_major) {
     packed = const_cast<void *>(w);  // read in place: row k = (c, taps) of filter m lies at w[m * C*taps + k]
-  } else if (int rc = pack_filters<T>(g, w, pl.fold_row ? 5 : 2, &packed, tail_bytes(pl, sizeof(T)), &partial)) {
+  } else if (int rc = pack_filters<T>(g, w, pl.table_rows ? 6 : pl.fold_row ? 5 : 2, &packed, tail_bytes(pl, sizeof(T)), &partial)) {
     return rc;
   }
   GemmParams gp{};
@@ -1594,10 +1659,18 @@ int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
 }
 
 template <typename T, int BM, int BN, int BK, int WM, int WN>
-void launch_wgrad(WgradParams &wp, bool tap_major, hipStream_t s) {
+void launch_wgrad(WgradParams &wp, bool tap_major, bool table_rows, hipStream_t s) {
   wp.col_tiles = (int)ceil_div(wp.CT, BN);
   wp.row_tiles = (int)ceil_div(wp.F, BM);
-  if (tap_major) {
+  if (table_rows) {
+    if constexpr (BN == 64) {
+      const long long blocks = (long long)wp.splits * wp.col_tiles * wp.row_tiles;
+      if (wp.gvol % (int)(16 / sizeof(T)) == 0)
+        hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN, true, true>), dim3((unsigned)blocks), dim3(512), 0, s, wp);
+      else
+        hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN, false, true>), dim3((unsigned)blocks), dim3(512), 0, s, wp);
+    }
+  } else if (tap_major) {
     // one-dimensional grid, whole K splits per XCD (see the kernel)
     const long long blocks = (long long)wp.splits * wp.col_tiles * wp.row_tiles;
     if (wp.gvol % (int)(16 / sizeof(T)) == 0)
@@ -1617,7 +1690,7 @@ int conv_wgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   // The tap-major kernel writes its columns in (tap, channel) order, so its result goes
   // through the reduction kernel, which also restores (channel, tap) -- unless there is a
   // single tap (a matrix product), where the two orders are the same, and a single split.
-  const bool staged = pl.splits > 1 || (pl.tap_major && g.wvol > 1);
+  const bool staged = pl.splits > 1 || (pl.tap_major && !pl.table_rows && g.wvol > 1);
   void *target = dw;
   if (staged)
     if (int rc = workspace((size_t)pl.splits * g.F * ct * sizeof(T), &target)) return rc;
@@ -1654,7 +1727,7 @@ int conv_wgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
     bool launched = false;
 #define MG_LAUNCH(TT, BM, BN, BK, WM, WN)                               \
   if (!launched && pl.bm == BM && pl.bn == BN) {                        \
-    launch_wgrad<TT, BM, BN, BK, WM, WN>(wp, pl.tap_major, s);          \
+    launch_wgrad<TT, BM, BN, BK, WM, WN>(wp, pl.tap_major, pl.table_rows, s);        \
     launched = true;                                                    \
   }
     MG_WGRAD_SHAPES(T, MG_LAUNCH)
@@ -1665,7 +1738,7 @@ int conv_wgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   if (staged) {
     const int count = g.F * ct;
     ScopedTiming timed(TAG_WGRAD_REDUCE);
-    if (pl.tap_major) {
+    if (pl.tap_major && !pl.table_rows) {
       // four runs of splits per element when one thread per element would leave units idle
       if (ceil_div(count, 256) < runtime().props.multiProcessorCount && pl.splits >= 16)
         hipLaunchKernelGGL((tap_reduce_kernel<T, 4>), dim3((unsigned)ceil_div(count, 64)), dim3(256), 0, s,

@@ -129,8 +129,14 @@ struct Quad {
 // ------------------------------------------------------------------------------------------
 // forward and data gradient
 // ------------------------------------------------------------------------------------------
-template <typename T, int BM, int BN, int BK, int WM, int WN, int NPH = 1, bool FOLD = false>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int NPH = 1, bool FOLD = false, bool ROWS = false>
 __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
+  // ROWS: the BK rows of a K tile are any rows of the gather table (GemmParams::tab: element
+  // offset and coordinate offsets of one (channel, tap) each), not BK channels under one tap;
+  // KTile::coff is then the index of the tile's first table row.  For channel counts that are
+  // no multiple of the K tile (a first layer's three): every row costs the gathering waves its
+  // own bounds test, but the structure of the kernel -- and its MFMA waves -- stay the same.
+  static_assert(!ROWS || (NPH == 1 && !FOLD), "table rows: plain tiles only");
   // FOLD: the three taps of the last axis are rows of the tile (see GemmParams::fold_row): three
   // times the rows per gathered element, a third of the K tiles.  A wave makes 48 rows (16
   // channels x 3 taps) x 64 positions, which are whole rows of the last axis.
@@ -253,7 +259,7 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
         qb1 = (int)j1 * p.sj[1];
         qb2 = (int)j2 * p.sj[2];
         src_at = (unsigned)((long long)n * p.src_nstride + (qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2]) +
-                            brow0 * p.src_cstride) * (unsigned)sizeof(T);
+                            (ROWS ? 0 : brow0 * p.src_cstride)) * (unsigned)sizeof(T);
         const bool a_ok = (it.m0 + acol < p.a_ld) & (arow0 < BK);  // rows are padded to whole 16-byte pieces
         a_at = a_ok ? (unsigned)(arow0 * p.a_ld + it.m0 + acol) * (unsigned)sizeof(T) : kOutside;
         return true;
@@ -270,11 +276,22 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
       const unsigned a_tile = (unsigned)e[0] * a_row_bytes;
 #pragma unroll
       for (int r = 0; r < ALOADS; ++r) ra[r] = buffer_load16<T>(a_buf, a_at, a_tile + (unsigned)(r * AROWS) * a_row_bytes);
-      const bool ok = pos_ok & ((unsigned)(qb0 + e[2]) < (unsigned)p.Q[0]) & ((unsigned)(qb1 + e[3]) < (unsigned)p.Q[1]) &
-                      ((unsigned)(qb2 + e[4]) < (unsigned)p.Q[2]);
-      const unsigned at = ok ? src_at + (unsigned)(e[1] * (int)sizeof(T)) : kOutside;
+      if constexpr (ROWS) {
+        const int4v MG_CONSTANT *rows = (const int4v MG_CONSTANT *)(p.tab) + e[1];
 #pragma unroll
-      for (int r = 0; r < BLOADS; ++r) rb[r] = buffer_load<T>(src_buf, at, (unsigned)r * b_step);
+        for (int r = 0; r < BLOADS; ++r) {
+          const int4v t = rows[brow0 + r * BROWS];  // off, d0, d1, d2 (the row is the same for the whole wave)
+          const bool ok = pos_ok & ((unsigned)(qb0 + t[1]) < (unsigned)p.Q[0]) & ((unsigned)(qb1 + t[2]) < (unsigned)p.Q[1]) &
+                          ((unsigned)(qb2 + t[3]) < (unsigned)p.Q[2]);
+          rb[r] = buffer_load<T>(src_buf, ok ? src_at + (unsigned)(t[0] * (int)sizeof(T)) : kOutside, 0u);
+        }
+      } else {
+        const bool ok = pos_ok & ((unsigned)(qb0 + e[2]) < (unsigned)p.Q[0]) & ((unsigned)(qb1 + e[3]) < (unsigned)p.Q[1]) &
+                        ((unsigned)(qb2 + e[4]) < (unsigned)p.Q[2]);
+        const unsigned at = ok ? src_at + (unsigned)(e[1] * (int)sizeof(T)) : kOutside;
+#pragma unroll
+        for (int r = 0; r < BLOADS; ++r) rb[r] = buffer_load<T>(src_buf, at, (unsigned)r * b_step);
+      }
       if (live) {
         ++requested;
         if (kt + 1 < it.kt_end)
@@ -731,7 +748,11 @@ __global__ void __launch_bounds__(256) tail_fixup_kernel(const GemmParams p) {
 // WIDE: the positions of one sample are a multiple of 16 bytes, so 16 bytes of grad (4 or
 // 2 consecutive positions of one filter) never straddle two samples and the grad tile
 // is loaded and parked 16 bytes per lane; otherwise element by element.
-template <typename T, int BM, int BN, int BK, int WM, int WN, bool WIDE>
+// TABLE: the columns are any rows of the gather table (WgradParams::tab, one (channel, tap) each,
+// in dw's own order, padded to whole tiles with rows that lie outside every input), not groups
+// of 16 channels under one tap -- for channel counts that fill no group.  Every column then
+// costs the gathering waves its own bounds test.
+template <typename T, int BM, int BN, int BK, int WM, int WN, bool WIDE, bool TABLE = false>
 __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
   static_assert((BM / WM) * (BN / WN) == 4, "four wavefronts per block");
   static_assert(256 % BK == 0 && BK % 16 == 0 && BN % 16 == 0, "K tile");
@@ -800,8 +821,19 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
   // the thread's column groups never change: keep their table rows in registers
   const int8v MG_CONSTANT *gtab = (const int8v MG_CONSTANT *)(p.groups) + n0 / 16;
   int8v grp[MYGROUPS];
+  if constexpr (!TABLE) {
 #pragma unroll
-  for (int i = 0; i < MYGROUPS; ++i) grp[i] = gtab[gsel + i * GSPLIT];
+    for (int i = 0; i < MYGROUPS; ++i) grp[i] = gtab[gsel + i * GSPLIT];
+  }
+  // TABLE: this thread's columns (gsel + j*GSPLIT)*16 + csel + r*CSPLIT of the tile, one table row each
+  int4v ent[TABLE ? MYGROUPS * CLOADS : 1];
+  if constexpr (TABLE) {
+    const int4v MG_CONSTANT *rows = (const int4v MG_CONSTANT *)(p.tab) + n0;
+#pragma unroll
+    for (int j = 0; j < MYGROUPS; ++j)
+#pragma unroll
+      for (int r = 0; r < CLOADS; ++r) ent[j * CLOADS + r] = rows[(gsel + j * GSPLIT) * 16 + csel + r * CSPLIT];
+  }
 
   constexpr int NB = MYGROUPS * CLOADS;
   AReg ra0[ALOADS], ra1[ALOADS];
@@ -839,15 +871,25 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
       for (int r = 0; r < ALOADS; ++r) ra[r] = buffer_load<T>(grad_buf, g_at, (unsigned)r * a_step);
     }
     const unsigned x_at = (unsigned)((long long)n * p.x_nstride + (qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2]) +
-                                     (long long)csel * p.x_cstride) * (unsigned)sizeof(T);
+                                     (TABLE ? 0ll : (long long)csel * p.x_cstride)) * (unsigned)sizeof(T);
+    if constexpr (TABLE) {
 #pragma unroll
-    for (int j = 0; j < MYGROUPS; ++j) {
-      const int8v e = grp[j];  // coff, d0, d1, d2, valid
-      const bool ok = pos_ok & (e[4] != 0) & ((unsigned)(qb0 + e[1]) < (unsigned)p.Q[0]) &
-                      ((unsigned)(qb1 + e[2]) < (unsigned)p.Q[1]) & ((unsigned)(qb2 + e[3]) < (unsigned)p.Q[2]);
-      const unsigned at = ok ? x_at + (unsigned)(e[0] * (int)sizeof(T)) : kOutside;
+      for (int i = 0; i < NB; ++i) {
+        const int4v e = ent[i];  // off, d0, d1, d2
+        const bool ok = pos_ok & ((unsigned)(qb0 + e[1]) < (unsigned)p.Q[0]) & ((unsigned)(qb1 + e[2]) < (unsigned)p.Q[1]) &
+                        ((unsigned)(qb2 + e[3]) < (unsigned)p.Q[2]);
+        rb[i] = buffer_load<T>(x_buf, ok ? x_at + (unsigned)(e[0] * (int)sizeof(T)) : kOutside, 0u);
+      }
+    } else {
 #pragma unroll
-      for (int r = 0; r < CLOADS; ++r) rb[j * CLOADS + r] = buffer_load<T>(x_buf, at, (unsigned)r * b_step);
+      for (int j = 0; j < MYGROUPS; ++j) {
+        const int8v e = grp[j];  // coff, d0, d1, d2, valid
+        const bool ok = pos_ok & (e[4] != 0) & ((unsigned)(qb0 + e[1]) < (unsigned)p.Q[0]) &
+                        ((unsigned)(qb1 + e[2]) < (unsigned)p.Q[1]) & ((unsigned)(qb2 + e[3]) < (unsigned)p.Q[2]);
+        const unsigned at = ok ? x_at + (unsigned)(e[0] * (int)sizeof(T)) : kOutside;
+#pragma unroll
+        for (int r = 0; r < CLOADS; ++r) rb[j * CLOADS + r] = buffer_load<T>(x_buf, at, (unsigned)r * b_step);
+      }
     }
   };
   auto stash = [&](const AReg(&ra)[ALOADS], const T(&rb)[NB], int buf) {

@@ -433,6 +433,39 @@ def test_conv_with_the_last_axis_taps_folded_into_rows(abi, case, monkeypatch):
     assert np.array_equal(abi.conv_fwd(steps, ramp_w, s, p, d), direct.conv_forward(steps, ramp_w, s, p, d).astype(np.float32))
 
 
+# Channel counts that fill no K tile (the one or three channels of a first layer), on problems
+# large enough not to be planned as tiny: the forward pass runs the tap-major kernel with K tiles
+# made of rows of the gather table (the last tile padded with rows that lie outside every input).
+FIRST_LAYER_CASES = [
+    ((16, 3, 64, 64), (32, 3, 5, 5), (1, 1), (2, 2), (1, 1)),
+    ((8, 3, 115, 115), (64, 3, 7, 7), (2, 2), (3, 3), (1, 1)),      # the stem's geometry, flooring placement
+    ((32, 1, 28, 28), (20, 1, 5, 5), (1, 1), (0, 0), (1, 1)),       # one channel, 20 filters (padded packed rows)
+    ((4, 5, 20, 24, 24), (16, 5, 3, 3, 3), (1, 2, 1), (1, 0, 1), (1, 1, 2)),
+    ((64, 7, 500), (48, 7, 9), (3,), (4,), (2,)),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("case", range(len(FIRST_LAYER_CASES)))
+def test_conv_forward_with_channels_that_fill_no_k_tile(abi, dtype, case):
+    x_shape, w_shape, s, p, d = FIRST_LAYER_CASES[case]
+    rng = np.random.default_rng(1500 + case)
+    tol = TOL[np.dtype(dtype)]
+    x = rng.standard_normal(x_shape).astype(dtype)
+    w = (rng.standard_normal(w_shape) / np.sqrt(np.prod(w_shape[1:]))).astype(dtype)
+    want = direct.conv_forward(x, w, s, p, d)
+    out = abi.conv_fwd(x, w, s, p, d)
+    assert rel_err(out, want) <= tol
+    assert np.array_equal(out, abi.conv_fwd(x, w, s, p, d))
+    # exact: small integers, every (channel, tap) weighted differently
+    xi = rng.integers(-2, 3, x_shape).astype(dtype)
+    wi = (np.arange(np.prod(w_shape[1:])).reshape(w_shape[1:]) % 7 - 3).astype(dtype) * np.ones(w_shape, dtype=dtype)
+    assert np.array_equal(abi.conv_fwd(xi, wi, s, p, d), direct.conv_forward(xi, wi, s, p, d).astype(dtype))
+    g = rng.standard_normal(want.shape).astype(dtype)
+    assert rel_err(abi.conv_dgrad(g, x_shape, w, s, p, d), direct.conv_backward_x(g, x_shape, w, s, p, d)) <= tol
+    assert rel_err(abi.conv_wgrad(g, x, w_shape, s, p, d), direct.conv_backward_w(g, x, w_shape, s, p, d)) <= tol
+
+
 # Shapes picked so that, between them, every tile shape and code path of the tap-major
 # kernels runs: all gather-GEMM tiles (rows 16..128), persistent blocks that stream
 # through several tiles and K slices, strided dgrad phases, filter counts that are not a
