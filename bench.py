@@ -57,9 +57,13 @@ WORKLOADS = {
     "conv5": dict(kind="conv", dtype="f32", seed=1006, x=(8, 16, 32, 64, 64), w=(32, 16, 3, 3, 3),
                   wscale=(2 / 432) ** 0.5, stride=(1, 1, 1), padding=(1, 1, 1), dilation=(1, 1, 1)),
     # a ResNet stem: three input channels, a 7x7 filter bank, stride 2 (flooring placement: the last
-    # padded row and column are never read)
+    # padded row and column are never read).  Its input is the data batch, a constant: like the
+    # reference (Operation.backward skips constant variables, operation_base.py:216-228) a step
+    # computes no dx.  `stem-dx` is the same layer with dx, for an input that does take a gradient.
     "stem": dict(kind="conv", dtype="f32", seed=1017, x=(128, 3, 224, 224), w=(64, 3, 7, 7), wscale=(2 / 147) ** 0.5,
-                 stride=(2, 2), padding=(3, 3), dilation=(1, 1)),
+                 stride=(2, 2), padding=(3, 3), dilation=(1, 1), constant_input=True),
+    "stem-dx": dict(kind="conv", dtype="f32", seed=1017, x=(128, 3, 224, 224), w=(64, 3, 7, 7), wscale=(2 / 147) ** 0.5,
+                    stride=(2, 2), padding=(3, 3), dilation=(1, 1)),
     "pool2": dict(kind="pool", dtype="f64", seed=1002, x=(64, 64, 56, 56), pool=(3, 3), stride=(2, 2)),
     "pool5": dict(kind="pool", dtype="f32", seed=1006, x=(8, 32, 32, 64, 64), pool=(2, 2, 2), stride=(2, 2, 2)),
     # the same two with each window's argmax recomputed from x in the backward pass (the stateless
@@ -109,6 +113,10 @@ def elem_bytes(x):
     return 15.0 * x.nbytes + 2.0 * ((x.size + 7) // 8)
 
 
+def conv_passes(wl):
+    return "fwd+dw (constant input: no dx)" if wl.get("constant_input") else "fwd+dx+dw"
+
+
 def conv_flops_per_pass(wl, batch=None):
     n = wl["x"][0] if batch is None else batch
     return 2.0 * n * wl["w"][0] * np.prod(conv_grid(wl)) * wl["x"][1] * np.prod(wl["w"][2:])
@@ -148,7 +156,7 @@ def describe(name):
         return f"{name}: batchnorm {wl['dtype']} x{wl['x']} with gamma and beta, eps={wl['eps']}, fwd + dx, dgamma, dbeta"
     if wl["kind"] == "conv":
         return (f"{name}: conv_nd {wl['dtype']} x{wl['x']} * w{wl['w']} stride{wl['stride']} pad{wl['padding']} "
-                f"dil{wl['dilation']} -> grid{conv_grid(wl)} fwd+dx+dw")
+                f"dil{wl['dilation']} -> grid{conv_grid(wl)} {conv_passes(wl)}")
     lead, pooled, grid = pool_shapes(wl)
     how = "argmax recomputed from x in bwd" if wl.get("recompute") else "argmax kept from fwd, one byte per window"
     return f"{name}: max_pool {wl['dtype']} x{wl['x']} pool{wl['pool']} stride{wl['stride']} -> grid{grid} fwd+bwd ({how})"
@@ -185,7 +193,7 @@ class Step:
             self.dw = _device.DeviceBuffer(w.nbytes)
             per_pass = conv_flops_per_pass(wl)
             self.work = {"conv_fwd": per_pass, "conv_dgrad": per_pass, "conv_wgrad": per_pass}
-            self.total_work = 3 * per_pass
+            self.total_work = (2 if wl.get("constant_input") else 3) * per_pass
             self.unit, self.bound, self.peak = "TFLOP/s", "mfma", PEAK_TFLOPS[wl["dtype"]]
             self.scale = 1e-12
         elif wl["kind"] == "bmm":
@@ -214,7 +222,7 @@ class Step:
             self.code, self.dims = _hip.dtype_code(dt), (1, M, K, N)
             per_pass = 2.0 * M * K * N
             self.work = {"conv_fwd": per_pass, "conv_dgrad": per_pass, "conv_wgrad": per_pass}
-            self.total_work = 3 * per_pass
+            self.total_work = (2 if wl.get("constant_input") else 3) * per_pass
             self.unit, self.bound, self.peak = "TFLOP/s", "mfma", PEAK_TFLOPS[wl["dtype"]]
             self.scale = 1e-12
         elif wl["kind"] == "permute":
@@ -407,7 +415,8 @@ class Step:
             return
         if self.wl["kind"] == "conv":
             check(lib.mg_conv_fwd(d, self.x.ptr, self.w.ptr, self.out.ptr))
-            check(lib.mg_conv_dgrad(d, self.g.ptr, self.w.ptr, self.dx.ptr))
+            if not self.wl.get("constant_input"):
+                check(lib.mg_conv_dgrad(d, self.g.ptr, self.w.ptr, self.dx.ptr))
             check(lib.mg_conv_wgrad(d, self.g.ptr, self.x.ptr, self.dw.ptr))
         elif self.argmax is None:
             check(lib.mg_maxpool_fwd(d, self.x.ptr, self.out.ptr))
@@ -529,11 +538,12 @@ def run_cpu_baseline(name, min_seconds=10.0, max_reps=200):
 
         def once():
             ora.conv_forward(x, w, validate=False, **conf)
-            ora.conv_backward_x(g, x.shape, x.dtype, w, **conf)
+            if not wl.get("constant_input"):
+                ora.conv_backward_x(g, x.shape, x.dtype, w, **conf)
             ora.conv_backward_w(g, x, w.shape, **conf)
 
-        work, scale, unit = 3 * conv_flops_per_pass(wl), 1e-12, "TFLOP/s"
-        what = "fwd+dx+dw"
+        work, scale, unit = (2 if wl.get("constant_input") else 3) * conv_flops_per_pass(wl), 1e-12, "TFLOP/s"
+        what = conv_passes(wl)
     elif wl["kind"] == "bmm":
         B, M, K, N = wl["batch"], wl["M"], wl["K"], wl["N"]
         a = (rng.standard_normal((B, M, K)) * K ** -0.5).astype(dt)
@@ -713,11 +723,11 @@ def run_dropin(name, steps=5):
         conf = dict(stride=wl["stride"], padding=wl["padding"], dilation=wl["dilation"])
 
         def once(T, C):
-            xt, wt = T(x), T(w)
+            xt, wt = (C(x) if wl.get("constant_input") else T(x)), T(w)
             conv_nd(xt, wt, **conf).backward(C(g))
             return xt, wt
 
-        work, scale, unit = 3 * conv_flops_per_pass(wl), 1e-12, "TFLOP/s"
+        work, scale, unit = (2 if wl.get("constant_input") else 3) * conv_flops_per_pass(wl), 1e-12, "TFLOP/s"
         if name == "conv5":
             # the whole of configuration 5: conv -> max_pool (2,2,2) -> loss = sum(pool_out * g)
             g5 = rng.standard_normal((wl["x"][0], wl["w"][0], *(n // 2 for n in conv_grid(wl)))).astype(dt)
