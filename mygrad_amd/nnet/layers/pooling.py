@@ -14,17 +14,73 @@ from ...tensor_base import Tensor
 __all__ = ["max_pool", "MaxPoolND"]
 
 
+class _Stage:
+    """One launch's worth of pooling: ``lead`` stacked arrays of shape ``shape`` (one to three
+    axes), window ``pool`` placed every ``stride``.  Keeps the argmax bytes of its forward pass
+    (windows of up to 256 elements) and, when it is not the first stage, the buffer it read."""
+
+    def __init__(self, lead, shape, pool, stride):
+        self.lead = int(lead)
+        self.shape = tuple(int(n) for n in shape)
+        self.pool = tuple(int(n) for n in pool)
+        self.stride = tuple(int(n) for n in stride)
+        self.grid = tuple((n - w) // s + 1 for n, w, s in zip(self.shape, self.pool, self.stride))
+        self.windows = self.lead * int(np.prod(self.grid, dtype=np.int64))
+        self.count = self.lead * int(np.prod(self.shape, dtype=np.int64))
+        self.argmax = None
+        self.source = None  # the device buffer read by the forward pass (stages after the first)
+
+    def desc(self, dtype, dx_dtype=None):
+        return _hip.pool_desc(dtype, self.lead, self.shape, self.pool, self.stride, self.grid, dx_dtype=dx_dtype)
+
+    def forward(self, dtype, xb):
+        ob = _device.DeviceBuffer(self.windows * dtype.itemsize)
+        if int(np.prod(self.pool)) <= 256:
+            # Each window's argmax (pooling.py:109-111) is found here, while x is being read
+            # anyway, and kept on the device as one byte per window: the backward pass then
+            # needs grad and these bytes only.
+            self.argmax = _device.DeviceBuffer(self.windows)
+            _hip.check(_hip.lib().mg_maxpool_fwd_argmax(self.desc(dtype), xb.ptr, ob.ptr, self.argmax.ptr))
+        else:
+            self.argmax = None
+            _hip.check(_hip.lib().mg_maxpool_fwd(self.desc(dtype), xb.ptr, ob.ptr))
+        return ob
+
+    def backward(self, x_dtype, g_dtype, gb, dx_dtype, xb, argmax_valid):
+        """Routes ``gb`` (values of ``g_dtype``) to a new buffer of ``dx_dtype`` values."""
+        db = _device.DeviceBuffer(self.count * dx_dtype.itemsize)
+        if self.argmax is not None and argmax_valid:
+            _hip.check(_hip.lib().mg_maxpool_bwd_argmax(self.desc(g_dtype, dx_dtype), self.argmax.ptr, gb.ptr, db.ptr))
+        else:  # find the maxima again in what the forward pass read
+            _hip.check(_hip.lib().mg_maxpool_bwd(self.desc(x_dtype, dx_dtype), xb.ptr, gb.ptr, db.ptr))
+        return db
+
+
 class MaxPoolND(Operation):
     """Max-pooling over the trailing ``len(pool)`` axes of ``x``.
 
     ``(N0, ..., C0, ...) -> (N0, ..., G0, ...)`` with window ``(P0, ...)`` placed
     every ``(S0, ...)``; only placements that fit entirely inside the data.
+
+    The kernels pool over one to three axes.  More pooled axes are taken three at a time, from
+    the last: the maximum over a window is the maximum, over its leading axes, of the maxima
+    over its last three, and the first maximum in row-major order is found the same way (the
+    first leading position that holds the maximum, then the first place inside it).  So the
+    last three axes are pooled with all others counted as leading axes, the three resulting
+    grid axes are merged into one with a window of one element, and the rest is pooled again --
+    the gradient takes the same stages in reverse, in float64 between them as the reference
+    accumulates it (pooling.py:147).
     """
 
     takes_device_arrays = True
 
-    _argmax = None  # device buffer, one byte per window, written by the forward pass
+    _stages = ()
     _skip = 0  # leading pooled axes with a one-element window, counted as leading axes
+
+    @property
+    def _argmax(self):
+        """Argmax bytes of the forward pass (of its one stage, for up to three pooled axes)."""
+        return self._stages[0].argmax if self._stages else None
 
     def __call__(self, x, pool, stride):
         self.variables = (x,)
@@ -56,17 +112,14 @@ class MaxPoolND(Operation):
                 f"Stride dimensions: {tuple(stride)}\n"
                 f"Pooling dimensions: {tuple(pool)}\n"
             )
+        if m == 0:
+            raise NotImplementedError("max_pool on the GPU needs at least one pooled axis (no CPU fallback)")
 
         # Leading pooled axes with a window of one element placed at every position pool nothing:
-        # they count as un-pooled leading axes.  What is left must fit the kernels' three axes.
+        # they count as un-pooled leading axes.
         skip = 0
-        while m - skip > _hip.MG_MAX_ND and pool[skip] == 1 and stride[skip] == 1:
+        while m - skip > 1 and pool[skip] == 1 and stride[skip] == 1:
             skip += 1
-        if not 1 <= m - skip <= _hip.MG_MAX_ND:
-            raise NotImplementedError(
-                f"max_pool on the GPU handles 1 to {_hip.MG_MAX_ND} pooled axes (leading axes with a window of one "
-                f"element aside), got pool={tuple(pool)} stride={tuple(stride)} (no CPU fallback)"
-            )
         self._skip = skip
         if xd.dtype not in (np.float32, np.float64):
             raise TypeError(
@@ -80,21 +133,25 @@ class MaxPoolND(Operation):
             return np.empty(out_full, dtype=xd.dtype)
 
         self._lead *= int(np.prod(pooled[:skip], dtype=np.int64))
-        desc = _hip.pool_desc(xd.dtype, self._lead, pooled[skip:], pool[skip:], stride[skip:], grid[skip:])
-        xb = _device.to_device(xd)
-        windows = int(np.prod(out_full))
-        ob = _device.DeviceBuffer(windows * xd.dtype.itemsize)
-        if int(np.prod(pool)) <= 256:
-            # Each window's argmax (pooling.py:109-111) is found here, while x is being read
-            # anyway, and kept on the device as one byte per window: the backward pass then
-            # needs grad and these bytes only.  x is read-only for as long as the graph holds
-            # it, so the positions cannot go stale; backward_var checks that this still holds.
-            self._argmax = _device.DeviceBuffer(windows)
-            _hip.check(_hip.lib().mg_maxpool_fwd_argmax(desc, xb.ptr, ob.ptr, self._argmax.ptr))
-        else:
-            _hip.check(_hip.lib().mg_maxpool_fwd(desc, xb.ptr, ob.ptr))
-        out = _device.download(ob, out_full, xd.dtype)
-        _device.attach(out, ob)
+        # the stages, in the order the forward pass runs them
+        stages = []
+        shape, window, step = list(pooled[skip:]), list(pool[skip:]), list(stride[skip:])
+        while len(shape) > _hip.MG_MAX_ND:
+            k = _hip.MG_MAX_ND
+            stage = _Stage(self._lead * int(np.prod(shape[:-k], dtype=np.int64)), shape[-k:], window[-k:], step[-k:])
+            stages.append(stage)
+            shape = shape[:-k] + [int(np.prod(stage.grid, dtype=np.int64))]
+            window, step = window[:-k] + [1], step[:-k] + [1]
+        stages.append(_Stage(self._lead, shape, window, step))
+        self._stages = stages
+
+        buf = _device.to_device(xd)
+        for i, stage in enumerate(stages):
+            if i:
+                stage.source = buf
+            buf = stage.forward(xd.dtype, buf)
+        out = _device.download(buf, out_full, xd.dtype)
+        _device.attach(out, buf)
         return out
 
     def backward_var(self, grad, index, **kwargs):
@@ -105,25 +162,48 @@ class MaxPoolND(Operation):
         if grad.shape != (*x.shape[: x.ndim - len(self.pool)], *self._grid):
             raise ValueError(f"max_pool backward: gradient of shape {grad.shape} for an output of shape "
                              f"{(*x.shape[: x.ndim - len(self.pool)], *self._grid)}")
-        m = len(self.pool)
         # The reference builds dx in float64 whatever x is (pooling.py:147) and the
         # caller rounds it to x.dtype when it becomes var.grad.  The kernel sums in
         # double and rounds once, so it can write x.dtype directly -- except when
         # var already holds a gradient that this one is added to, where the
         # unrounded float64 values are needed for the same result.
         dx_dtype = np.dtype(np.float64) if var._grad is not None else x.dtype
-        k = self._skip
-        desc = _hip.pool_desc(x.dtype, self._lead, x.shape[x.ndim - m + k :], self.pool[k:], self.stride[k:], self._grid[k:],
-                              dx_dtype=dx_dtype)
-        gb = _device.to_device(grad, x.dtype)
-        db = _device.DeviceBuffer(x.size * dx_dtype.itemsize)
-        if self._argmax is not None and _device.is_locked(x):
-            _hip.check(_hip.lib().mg_maxpool_bwd_argmax(desc, self._argmax.ptr, gb.ptr, db.ptr))
-        else:  # x may have been written to since the forward pass: find the maxima again
+        wide = np.dtype(np.float64)
+        stages = self._stages
+        # x is read-only for as long as the graph holds it, so the recorded positions cannot go
+        # stale; if it was released and may have been written to, the maxima are found again
+        # (for several stages: all of them, from the values x holds now)
+        fresh = _device.is_locked(x)
+        xb = None
+        if not fresh or stages[0].argmax is None:
             xb = _device.to_device(x)
-            _hip.check(_hip.lib().mg_maxpool_bwd(desc, xb.ptr, gb.ptr, db.ptr))
-        out = _device.download(db, x.shape, dx_dtype)
-        _device.attach_transient(out, db)
+        if not fresh and len(stages) > 1:
+            buf = xb
+            for i, stage in enumerate(stages):
+                if i:
+                    stage.source = buf
+                buf = stage.forward(x.dtype, buf)
+            fresh = True
+        gb = _device.to_device(grad, x.dtype)
+        g_dtype = x.dtype
+        for i in range(len(stages) - 1, -1, -1):
+            stage = stages[i]
+            last = i == 0
+            # between the stages the gradient stays in float64 when the stage can route it from its
+            # argmax bytes (the kernels read x and grad in one precision)
+            out_dtype = dx_dtype if last else (wide if stages[i - 1].argmax is not None else x.dtype)
+            target = out_dtype
+            if g_dtype != x.dtype and out_dtype != wide:
+                target = wide  # a float64 gradient is routed to float64 and rounded afterwards
+            source = xb if last else stage.source
+            db = stage.backward(x.dtype, g_dtype, gb, target, source, fresh)
+            if target != out_dtype:
+                narrow = _device.DeviceBuffer(stage.count * out_dtype.itemsize)
+                _hip.check(_hip.lib().mg_cast(_hip.dtype_code(target), _hip.dtype_code(out_dtype), stage.count, db.ptr, narrow.ptr))
+                db = narrow
+            gb, g_dtype = db, out_dtype
+        out = _device.download(gb, x.shape, dx_dtype)
+        _device.attach_transient(out, gb)
         return out
 
 
