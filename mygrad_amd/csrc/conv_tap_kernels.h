@@ -839,10 +839,12 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
   // takes the (b/8)-th pair of that XCD's run.  An XCD then works on whole splits, one
   // after the other, and shares at most the split at either end of its run with a
   // neighbour; any number of splits can be used.
+  // (A single split -- a matrix product's many tiles -- keeps the plain order: neighbouring
+  // tiles on neighbouring XCDs re-read less of the operands than eight long runs do.)
   const int tiles_per_split = p.col_tiles * p.row_tiles;
   const int xcd = blockIdx.x % 8, nth = blockIdx.x / 8;
   const int per_xcd = gridDim.x / 8, extra = gridDim.x % 8;
-  const int pair = xcd * per_xcd + min(xcd, extra) + nth;
+  const int pair = p.splits == 1 ? (int)blockIdx.x : xcd * per_xcd + min(xcd, extra) + nth;
   const int split = pair / tiles_per_split;
   const int tile = pair % tiles_per_split;
   const int n0 = (tile % p.col_tiles) * BN;  // first column
