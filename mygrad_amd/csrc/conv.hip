@@ -1042,9 +1042,11 @@ bool deep_fused_on() {
 
 int build_dgrad_plan(const Geometry &g, Plan &pl) {
   Tables t;
-  // a tiny problem is bound by its launches: the table-driven kernel needs neither packed
-  // filters nor a pass over partial sums
-  pl.tap_major = g.F % gemm_bk(g.dtype) == 0 && fits_buffer_loads(g) && !is_tiny(g);
+  // a tiny problem with a handful of channels is bound by its launches: the table-driven kernel
+  // with its deep K tiles needs neither packed filters nor a pass over partial sums.  (Measured,
+  // whole steps: 3 channels 38.5 -> 28 us; with 16 channels the tap-major kernels are 4 us
+  // ahead, and with 32 or 64 the table-driven kernel's few, long-running blocks cost 2 - 5 x.)
+  pl.tap_major = g.F % gemm_bk(g.dtype) == 0 && fits_buffer_loads(g) && !(is_tiny(g) && g.C <= 8);
   const int bk = pl.tap_major ? tap_bk(g.dtype, g.F) : gemm_bk(g.dtype);
   pl.bk = bk;
   pl.single_dense_phase = g.S[0] == 1 && g.S[1] == 1 && g.S[2] == 1;
