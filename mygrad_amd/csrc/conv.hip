@@ -887,14 +887,18 @@ void fwd_table(const Geometry &g, std::vector<TabEntry> &tab) {
 // pipes: a gathered element feeds three times the MFMAs this way), a 3-tap "same" last axis
 // with unit stride and dilation, and rows of positions that a wave's 64 positions hold whole
 // (a power of two up to 64).  MYGRAD_HIP_FOLD=0 switches it off.
-bool fold_applies(const Geometry &g, int rows) {
+// `depth`: the channels contracted per tap (channels in the forward pass, filters in the data
+// gradient).  With 17 to 32 rows the plain 32-row tiles are less starved, and measured against
+// them the 96-row folded tile wins with 16 and 32 channels per tap (3 - 8 %) and loses with 256
+// (10 %): taken up to 64.
+bool fold_applies(const Geometry &g, int rows, int depth) {
   static const bool fold_on = [] {
     const char *flag = getenv("MYGRAD_HIP_FOLD");
     return !(flag && flag[0] == '0');
   }();
   const bool row_fits = g.X[2] >= 4 && g.X[2] <= 64 && (g.X[2] & (g.X[2] - 1)) == 0;
-  return fold_on && g.dtype == MG_F32 && rows <= 32 && g.W[2] == 3 && g.P[2] == 1 && g.D[2] == 1 && g.S[2] == 1 &&
-         g.G[2] == g.X[2] && row_fits;
+  return fold_on && g.dtype == MG_F32 && (rows <= 16 || (rows <= 32 && depth <= 64)) && g.W[2] == 3 && g.P[2] == 1 &&
+         g.D[2] == 1 && g.S[2] == 1 && g.G[2] == g.X[2] && row_fits;
 }
 
 // Tile of a plan with folded taps: 48 rows x 256 positions for up to 16 channels (one block per
@@ -980,7 +984,7 @@ int build_fwd_plan(const Geometry &g, Plan &pl) {
     pl.pos_blocks = (int)ceil_div(ph.npos, pl.bn);
     return upload_plan(pl, t);
   }
-  if (pl.tap_major && fold_applies(g, g.F)) {
+  if (pl.tap_major && fold_applies(g, g.F, g.C)) {
     // rows (filter, tap of the last axis); K tiles over the taps of the other axes
     const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
     for (int c0 = 0; c0 < g.C; c0 += bk)
@@ -1092,7 +1096,7 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
   // times the MFMAs -- with 16 channels the plain tiles are bound by the gather, not by the
   // matrix pipes -- and the epilogue adds the three rows of a channel, shifted along the last
   // axis, into dx.  A wave's 64 positions must be whole rows: X2 a power of two up to 64.
-  if (fold_applies(g, g.C) && pl.tap_major && nphase == 1 && found.size() == 1) {
+  if (fold_applies(g, g.C, g.F) && pl.tap_major && nphase == 1 && found.size() == 1) {
     const PhaseTaps &pt = found[0];
     Phase ph = pt.ph;
     for (int f0 = 0; f0 < g.F; f0 += bk)
