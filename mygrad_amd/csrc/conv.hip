@@ -886,19 +886,37 @@ void fwd_table(const Geometry &g, std::vector<TabEntry> &tab) {
 // float, few rows (with 16 or 32 the plain tiles are bound by the gather, not by the matrix
 // pipes: a gathered element feeds three times the MFMAs this way), a 3-tap "same" last axis
 // with unit stride and dilation, and rows of positions that a wave's 64 positions hold whole
-// (a power of two up to 64).  MYGRAD_HIP_FOLD=0 switches it off.
+// (up to 64 long, padded to a power of two).  MYGRAD_HIP_FOLD=0 switches it off.
 // `depth`: the channels contracted per tap (channels in the forward pass, filters in the data
 // gradient).  With 17 to 32 rows the plain 32-row tiles are less starved, and measured against
 // them the 96-row folded tile wins with 16 and 32 channels per tap (3 - 8 %) and loses with 256
 // (10 %): taken up to 64.
+int fold_padded_row(int row) {
+  int padded = 4;
+  while (padded < row) padded *= 2;
+  return padded;
+}
+
 bool fold_applies(const Geometry &g, int rows, int depth) {
   static const bool fold_on = [] {
     const char *flag = getenv("MYGRAD_HIP_FOLD");
     return !(flag && flag[0] == '0');
   }();
-  const bool row_fits = g.X[2] >= 4 && g.X[2] <= 64 && (g.X[2] & (g.X[2] - 1)) == 0;
+  // a row of positions is padded to a power of two (a wave's 64 positions are whole padded rows);
+  // the padding positions cost MFMA time and store nothing: at most an eighth of a row
+  const int padded = fold_padded_row(g.X[2]);
+  const bool row_fits = g.X[2] >= 4 && g.X[2] <= 64 && (padded - g.X[2]) * 8 <= padded &&
+                        (long long)g.N * g.X[0] * g.X[1] * padded < (1ll << 31);
   return fold_on && g.dtype == MG_F32 && (rows <= 16 || (rows <= 32 && depth <= 64)) && g.W[2] == 3 && g.P[2] == 1 &&
          g.D[2] == 1 && g.S[2] == 1 && g.G[2] == g.X[2] && row_fits;
+}
+
+// The positions of a folded plan: rows of the last axis padded to `fold_row` positions each.
+void pad_fold_rows(const Geometry &g, Plan &pl, Phase &ph) {
+  pl.fold_row = fold_padded_row(g.X[2]);
+  ph.J[2] = pl.fold_row;
+  ph.npos = (int)((long long)g.N * ph.J[0] * ph.J[1] * ph.J[2]);
+  set_divisors(ph);
 }
 
 // Tile of a plan with folded taps: 48 rows x 256 positions for up to 16 channels (one block per
@@ -999,7 +1017,7 @@ int build_fwd_plan(const Geometry &g, Plan &pl) {
           t.ktiles.push_back(e);
         }
     ph.k_count = (int)t.ktiles.size();
-    pl.fold_row = g.X[2];
+    pad_fold_rows(g, pl, ph);
     set_fold_tile(pl, g.F);
     pl.pos_blocks = (int)ceil_div(ph.npos, pl.bn);
     pl.full_tiles = pl.pos_blocks;
@@ -1095,7 +1113,8 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
   // run over the taps of the other axes only.  A gathered element of grad then feeds three
   // times the MFMAs -- with 16 channels the plain tiles are bound by the gather, not by the
   // matrix pipes -- and the epilogue adds the three rows of a channel, shifted along the last
-  // axis, into dx.  A wave's 64 positions must be whole rows: X2 a power of two up to 64.
+  // axis, into dx.  A wave's 64 positions must be whole rows: rows of up to 64 positions, padded
+  // to a power of two.
   if (fold_applies(g, g.C, g.F) && pl.tap_major && nphase == 1 && found.size() == 1) {
     const PhaseTaps &pt = found[0];
     Phase ph = pt.ph;
@@ -1113,7 +1132,7 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
     ph.k_begin = 0;
     ph.k_count = (int)t.ktiles.size();
     ph.blk_begin = 0;
-    pl.fold_row = g.X[2];
+    pad_fold_rows(g, pl, ph);
     set_fold_tile(pl, g.C);
     pl.pos_blocks = (int)ceil_div(ph.npos, pl.bn);
     pl.full_tiles = pl.pos_blocks;
@@ -1507,6 +1526,12 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
 #undef MG_LAUNCH_ROWS
   }
   gp.fold_row = pl.fold_row;
+  if (pl.fold_row) {
+    // a lane's four positions are adjacent in dst and all exist or all do not when the rows are
+    // whole 16-byte pieces (positions do not run through dst in order: rows are padded)
+    gp.vec_store = gp.Q[2] % 4 == 0 && gp.dst_mstride % 4 == 0 && gp.dst_nstride % 4 == 0 && gp.os[0] % 4 == 0 &&
+                   gp.os[1] % 4 == 0 && reinterpret_cast<uintptr_t>(gp.dst) % 16 == 0;
+  }
   if constexpr (sizeof(T) == 4) {
     if (pl.fold_row) {
       if (pl.bm == 48)

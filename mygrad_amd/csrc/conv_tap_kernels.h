@@ -688,9 +688,13 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
         // in its neighbours of the same quarter-wave (a wave's positions are whole rows, so the
         // first and last lane of a quarter never need a neighbour).
         static_assert(TM == 3 && TN == 4, "three taps, four positions per lane");
+        // (A row of positions is padded to fold_row, a power of two; the padding positions
+        // gather nothing, so their sums are zero -- which is what the last real position of a
+        // row must see to its right -- and they are not stored.)
         const unsigned in_row = (unsigned)first & (unsigned)(p.fold_row - 1);
         const bool has_prev = in_row != 0, has_next = in_row + TN != (unsigned)p.fold_row;
-        const bool exists = first < ph.npos;
+        const int real = p.Q[2] - (int)in_row;  // positions of this lane that exist: min(real, TN), none if <= 0
+        const bool exists = first < ph.npos && real > 0;
         T *out = dst_of(exists ? first : 0);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
@@ -707,7 +711,8 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
               store_vec<T, TN>(out + (long long)m * p.dst_mstride, v);
             } else {
 #pragma unroll
-              for (int j = 0; j < TN; ++j) out[(long long)m * p.dst_mstride + j] = v[j];
+              for (int j = 0; j < TN; ++j)
+                if (j < real) out[(long long)m * p.dst_mstride + j] = v[j];
             }
           }
         }

@@ -398,6 +398,14 @@ FOLDED_TAP_CASES = [
     ((2, 32, 16, 32), (16, 32, 3, 3), (1, 1), (1, 1), (1, 1)),       # 32 channels: 96-row tiles
     ((3, 24, 10, 16), (32, 24, 3, 3), (1, 1), (1, 1), (1, 1)),       # 24 channels in a 96-row tile
     ((2, 48, 12, 9, 32), (24, 48, 2, 3, 3), (2, 1, 1), (0, 2, 1), (1, 2, 1)),  # forward only folds (24 filters; stride on axis 0)
+    # rows that are no power of two: padded to one (at most an eighth of padding), the padding never stored
+    ((3, 16, 28, 28), (16, 16, 3, 3), (1, 1), (1, 1), (1, 1)),
+    ((2, 8, 5, 14, 14), (32, 8, 3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
+    ((5, 16, 9, 7), (16, 16, 3, 3), (1, 1), (1, 1), (1, 1)),
+    ((2, 16, 20, 56), (32, 16, 3, 3), (1, 1), (1, 1), (1, 1)),
+    ((3, 10, 11, 30), (16, 10, 2, 3), (1, 1), (1, 1), (1, 1)),       # rows of 30: no whole 16-byte pieces, element-wise stores
+    ((4, 16, 6, 15), (16, 16, 3, 3), (1, 1), (1, 1), (1, 1)),
+    ((7, 32, 61), (32, 32, 3), (1,), (1,), (1,)),
 ]
 
 
