@@ -1287,8 +1287,17 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
   X(T, 16, 64, (sizeof(T) == 8 ? 32 : 64), 16, 16)
 
 // Blocks of the filter-gradient kernel that fit on one compute unit at a time.
+// Tile shapes that only the table-row mode of the tap-major filter-gradient kernel has.
+#define MG_WGRAD_TABLE_SHAPES(T, X)                \
+  X(T, 64, 80, (sizeof(T) == 8 ? 32 : 64), 16, 80) \
+  X(T, 64, 32, (sizeof(T) == 8 ? 32 : 64), 32, 16)
+
 template <typename T>
 int wgrad_blocks_per_cu(int bm, int bn, bool tap_major) {
+#define MG_OCC_TABLE(TT, BM, BN, BK, WM, WN) \
+  if (bm == BM && bn == BN && tap_major) return resident_blocks(tap_wgrad_kernel<TT, BM, BN, BK, WM, WN, true, true>, 512);
+  MG_WGRAD_TABLE_SHAPES(T, MG_OCC_TABLE)
+#undef MG_OCC_TABLE
 #define MG_OCC(TT, BM, BN, BK, WM, WN)                                                     \
   if (bm == BM && bn == BN) {                                                              \
     if (tap_major) return resident_blocks(tap_wgrad_kernel<TT, BM, BN, BK, WM, WN, true>, 512);  \
@@ -1379,6 +1388,12 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
       pl.bm = row_tile;
       pl.bn = 64;
       pl.bk = f64 ? 32 : 64;
+      if (row_tile == 64) {
+        // 64-row tiles also come 32 and 80 columns wide: the width that pads the columns least
+        // (a 7x7 filter on three channels: 147 columns are 160 in tiles of 80, 192 in tiles of 64)
+        for (int bn : {80, 32})
+          if (ceil_div(ct, bn) * bn < ceil_div(ct, pl.bn) * pl.bn) pl.bn = bn;
+      }
       best_splits = splits_for(pl.bm, pl.bn, pl.bk, true);
     } else {
       pl.bm = g.F <= 16 ? 16 : (g.F <= 32 ? 32 : 64);
@@ -1690,17 +1705,22 @@ int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
 }
 
 template <typename T, int BM, int BN, int BK, int WM, int WN>
+void launch_table_wgrad(WgradParams &wp, hipStream_t s) {
+  wp.col_tiles = (int)ceil_div(wp.CT, BN);
+  wp.row_tiles = (int)ceil_div(wp.F, BM);
+  const long long blocks = (long long)wp.splits * wp.col_tiles * wp.row_tiles;
+  if (wp.gvol % (int)(16 / sizeof(T)) == 0)
+    hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN, true, true>), dim3((unsigned)blocks), dim3(512), 0, s, wp);
+  else
+    hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN, false, true>), dim3((unsigned)blocks), dim3(512), 0, s, wp);
+}
+
+template <typename T, int BM, int BN, int BK, int WM, int WN>
 void launch_wgrad(WgradParams &wp, bool tap_major, bool table_rows, hipStream_t s) {
   wp.col_tiles = (int)ceil_div(wp.CT, BN);
   wp.row_tiles = (int)ceil_div(wp.F, BM);
   if (table_rows) {
-    if constexpr (BN == 64) {
-      const long long blocks = (long long)wp.splits * wp.col_tiles * wp.row_tiles;
-      if (wp.gvol % (int)(16 / sizeof(T)) == 0)
-        hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN, true, true>), dim3((unsigned)blocks), dim3(512), 0, s, wp);
-      else
-        hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN, false, true>), dim3((unsigned)blocks), dim3(512), 0, s, wp);
-    }
+    if constexpr (BN == 64) launch_table_wgrad<T, BM, BN, BK, WM, WN>(wp, s);
   } else if (tap_major) {
     // one-dimensional grid, whole K splits per XCD (see the kernel)
     const long long blocks = (long long)wp.splits * wp.col_tiles * wp.row_tiles;
@@ -1756,6 +1776,15 @@ int conv_wgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   {
     ScopedTiming timed(TAG_CONV_WGRAD);
     bool launched = false;
+    if (pl.table_rows) {
+#define MG_LAUNCH_TABLE(TT, BM, BN, BK, WM, WN)             \
+  if (!launched && pl.bm == BM && pl.bn == BN) {            \
+    launch_table_wgrad<TT, BM, BN, BK, WM, WN>(wp, s);      \
+    launched = true;                                        \
+  }
+      MG_WGRAD_TABLE_SHAPES(T, MG_LAUNCH_TABLE)
+#undef MG_LAUNCH_TABLE
+    }
 #define MG_LAUNCH(TT, BM, BN, BK, WM, WN)                               \
   if (!launched && pl.bm == BM && pl.bn == BN) {                        \
     launch_wgrad<TT, BM, BN, BK, WM, WN>(wp, pl.tap_major, pl.table_rows, s);        \

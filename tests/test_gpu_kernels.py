@@ -450,6 +450,8 @@ FIRST_LAYER_CASES = [
     ((32, 1, 28, 28), (20, 1, 5, 5), (1, 1), (0, 0), (1, 1)),       # one channel, 20 filters (padded packed rows)
     ((4, 5, 20, 24, 24), (16, 5, 3, 3, 3), (1, 2, 1), (1, 0, 1), (1, 1, 2)),
     ((64, 7, 500), (48, 7, 9), (3,), (4,), (2,)),
+    ((64, 1, 28, 28), (64, 1, 5, 5), (1, 1), (0, 0), (1, 1)),       # 25 columns of dw: one 32-column tile
+    ((16, 3, 48, 48), (128, 3, 7, 7), (1, 1), (3, 3), (1, 1)),      # 147 columns: two 80-column tiles, two row tiles
 ]
 
 
