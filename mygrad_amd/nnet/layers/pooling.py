@@ -56,6 +56,22 @@ class _Stage:
         return db
 
 
+def plan_stages(lead, pooled, pool, stride, most=_hip.MG_MAX_ND):
+    """The stages of a pooling over any number of axes, in the order the forward pass runs them:
+    the last ``most`` axes first, with everything in front of them counted as leading axes; their
+    grid then merges into one axis with a window of one element, and so on until at most ``most``
+    axes are left."""
+    stages = []
+    shape, window, step = [int(n) for n in pooled], [int(n) for n in pool], [int(n) for n in stride]
+    while len(shape) > most:
+        stage = _Stage(int(lead) * int(np.prod(shape[:-most], dtype=np.int64)), shape[-most:], window[-most:], step[-most:])
+        stages.append(stage)
+        shape = shape[:-most] + [int(np.prod(stage.grid, dtype=np.int64))]
+        window, step = window[:-most] + [1], step[:-most] + [1]
+    stages.append(_Stage(lead, shape, window, step))
+    return stages
+
+
 class MaxPoolND(Operation):
     """Max-pooling over the trailing ``len(pool)`` axes of ``x``.
 
@@ -133,16 +149,7 @@ class MaxPoolND(Operation):
             return np.empty(out_full, dtype=xd.dtype)
 
         self._lead *= int(np.prod(pooled[:skip], dtype=np.int64))
-        # the stages, in the order the forward pass runs them
-        stages = []
-        shape, window, step = list(pooled[skip:]), list(pool[skip:]), list(stride[skip:])
-        while len(shape) > _hip.MG_MAX_ND:
-            k = _hip.MG_MAX_ND
-            stage = _Stage(self._lead * int(np.prod(shape[:-k], dtype=np.int64)), shape[-k:], window[-k:], step[-k:])
-            stages.append(stage)
-            shape = shape[:-k] + [int(np.prod(stage.grid, dtype=np.int64))]
-            window, step = window[:-k] + [1], step[:-k] + [1]
-        stages.append(_Stage(self._lead, shape, window, step))
+        stages = plan_stages(self._lead, pooled[skip:], pool[skip:], stride[skip:])
         self._stages = stages
 
         buf = _device.to_device(xd)

@@ -619,3 +619,27 @@ def test_multiply_plan_on_drawn_shapes():
         assert np.array_equal((va * vb).reshape(shape), a * b)
 
     check()
+
+
+def test_pooling_stages_cover_any_number_of_axes():
+    """Stage planning of max_pool over more axes than the kernels take (host logic only): every
+    stage has at most three axes, each stage reads what the one before it wrote, and the last
+    one's windows are the windows of the whole pooling."""
+    from mygrad_amd.nnet.layers.pooling import plan_stages
+
+    rng = np.random.default_rng(5)
+    for m in range(1, 9):
+        pool = rng.integers(1, 4, m)
+        stride = rng.integers(1, 4, m)
+        grid = rng.integers(1, 4, m)
+        pooled = (grid - 1) * stride + pool
+        lead = int(rng.integers(1, 5))
+        stages = plan_stages(lead, pooled, pool, stride)
+        assert all(1 <= len(st.shape) <= 3 for st in stages)
+        assert len(stages) == (1 if m <= 3 else 1 + -(-(m - 3) // 2))
+        assert stages[0].count == lead * int(np.prod(pooled))
+        for before, after in zip(stages, stages[1:]):
+            assert after.count == before.windows  # a stage reads exactly what the one before it wrote
+        assert stages[-1].windows == lead * int(np.prod(grid))
+        # window volumes multiply up to the whole window
+        assert int(np.prod([np.prod(st.pool) for st in stages])) == int(np.prod(pool))
