@@ -1722,7 +1722,7 @@ void launch_wgrad(WgradParams &wp, bool tap_major, bool table_rows, hipStream_t 
   if (table_rows) {
     if constexpr (BN == 64) launch_table_wgrad<T, BM, BN, BK, WM, WN>(wp, s);
   } else if (tap_major) {
-    // one-dimensional grid, whole K splits per XCD (see the kernel)
+    // one-dimensional grid, runs of (split, tile) pairs per XCD (see the kernel)
     const long long blocks = (long long)wp.splits * wp.col_tiles * wp.row_tiles;
     if (wp.gvol % (int)(16 / sizeof(T)) == 0)
       hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN, true>), dim3((unsigned)blocks), dim3(512), 0, s, wp);
