@@ -115,6 +115,20 @@ __global__ void __launch_bounds__(256) pack_filters_kernel(const T *__restrict__
     // idx enumerates the packed layout so that stores are coalesced
     const int m = idx % ld;
     const int row = idx / ld;
+    if (sizeof(T) == 8 && mode >= 4 && mode <= 5) {
+      // double precision orders the folded rows (block of 16, tap, one of the 16): the wave tile of
+      // its MFMA holds a lane's two rows of each tap 16 rows apart
+      const int n = mode == 4 ? C : F;
+      const int one = (m / 48) * 16 + m % 16, tap = (m % 48) / 16;
+      T v = T(0);
+      if (one < n) {
+        const int f = mode == 4 ? row % F : one, c = mode == 4 ? one : row % C;
+        const int t = (row / (mode == 4 ? F : C)) * 3 + (mode == 4 ? tap : 2 - tap);
+        v = w[((long long)f * C + c) * wvol + t];
+      }
+      ap[idx] = v;
+      continue;
+    }
     if (m >= M) {
       ap[idx] = T(0);
       continue;
@@ -907,7 +921,7 @@ bool fold_applies(const Geometry &g, int rows, int depth) {
   const int padded = fold_padded_row(g.X[2]);
   const bool row_fits = g.X[2] >= 4 && g.X[2] <= 64 && (padded - g.X[2]) * 8 <= padded &&
                         (long long)g.N * g.X[0] * g.X[1] * padded < (1ll << 31);
-  return fold_on && g.dtype == MG_F32 && (rows <= 16 || (rows <= 32 && depth <= 64)) && g.W[2] == 3 && g.P[2] == 1 &&
+  return fold_on && (rows <= 16 || (rows <= 32 && depth <= 64)) && g.W[2] == 3 && g.P[2] == 1 &&
          g.D[2] == 1 && g.S[2] == 1 && g.G[2] == g.X[2] && row_fits;
 }
 
@@ -921,12 +935,23 @@ void pad_fold_rows(const Geometry &g, Plan &pl, Phase &ph) {
 
 // Tile of a plan with folded taps: 48 rows x 256 positions for up to 16 channels (one block per
 // tile), 96 x 128 for up to 32 (persistent blocks, as many as fit on the device, every tile whole).
-void set_fold_tile(Plan &pl, int rows) {
+void set_fold_tile(const Geometry &g, Plan &pl, int rows, int bk) {
   pl.m_tiles = 1, pl.tail_split = 1, pl.blocks_per_cu = 1;
   if (rows <= 16) {
     pl.bm = 48, pl.bn = 256;
   } else {
     pl.bm = 96, pl.bn = 128;
+  }
+  // persistent blocks (all double-precision tiles, and float tiles of 64 rows or more): as many
+  // as the device holds
+  if (g.dtype == MG_F64) {
+    if (rows <= 16)
+      pl.blocks_per_cu = bk == 16 ? resident_blocks(tap_gemm_kernel<double, 48, 256, 16, 48, 64, 1, true>, 512)
+                                  : resident_blocks(tap_gemm_kernel<double, 48, 256, 8, 48, 64, 1, true>, 512);
+    else
+      pl.blocks_per_cu = bk == 16 ? resident_blocks(tap_gemm_kernel<double, 96, 128, 16, 48, 64, 1, true>, 512)
+                                  : resident_blocks(tap_gemm_kernel<double, 96, 128, 8, 48, 64, 1, true>, 512);
+  } else if (rows > 16) {
     pl.blocks_per_cu = resident_blocks(tap_gemm_kernel<float, 96, 128, 16, 48, 64, 1, true>, 512);
   }
 }
@@ -1018,7 +1043,7 @@ int build_fwd_plan(const Geometry &g, Plan &pl) {
         }
     ph.k_count = (int)t.ktiles.size();
     pad_fold_rows(g, pl, ph);
-    set_fold_tile(pl, g.F);
+    set_fold_tile(g, pl, g.F, bk);
     pl.pos_blocks = (int)ceil_div(ph.npos, pl.bn);
     pl.full_tiles = pl.pos_blocks;
     t.phases.push_back(ph);
@@ -1133,7 +1158,7 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
     ph.k_count = (int)t.ktiles.size();
     ph.blk_begin = 0;
     pad_fold_rows(g, pl, ph);
-    set_fold_tile(pl, g.C);
+    set_fold_tile(g, pl, g.C, bk);
     pl.pos_blocks = (int)ceil_div(ph.npos, pl.bn);
     pl.full_tiles = pl.pos_blocks;
     t.phases.push_back(ph);
@@ -1521,7 +1546,7 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
     launched = true;
   }
   if constexpr (sizeof(T) == 8) {
-    if (pl.tap_major && pl.bk == 2 * BK && !pl.table_rows) {
+    if (pl.tap_major && pl.bk == 2 * BK && !pl.table_rows && !pl.fold_row) {
 #define MG_LAUNCH_DEEP(TT, BM, BN, WM, WN)                \
   if (!launched && pl.bm == BM && pl.bn == BN) {          \
     launch_gemm<TT, BM, BN, 2 * BK, WM, WN>(gp, pl, s);   \
@@ -1544,17 +1569,22 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
   if (pl.fold_row) {
     // a lane's four positions are adjacent in dst and all exist or all do not when the rows are
     // whole 16-byte pieces (positions do not run through dst in order: rows are padded)
-    gp.vec_store = gp.Q[2] % 4 == 0 && gp.dst_mstride % 4 == 0 && gp.dst_nstride % 4 == 0 && gp.os[0] % 4 == 0 &&
-                   gp.os[1] % 4 == 0 && reinterpret_cast<uintptr_t>(gp.dst) % 16 == 0;
+    const int piece = (int)(16 / sizeof(T));
+    gp.vec_store = gp.Q[2] % piece == 0 && gp.dst_mstride % piece == 0 && gp.dst_nstride % piece == 0 &&
+                   gp.os[0] % piece == 0 && gp.os[1] % piece == 0 && reinterpret_cast<uintptr_t>(gp.dst) % 16 == 0;
   }
-  if constexpr (sizeof(T) == 4) {
-    if (pl.fold_row) {
+  if (pl.fold_row && !launched) {
+    if (pl.bk == 2 * BK && sizeof(T) == 8) {
       if (pl.bm == 48)
-        launch_gemm<T, 48, 256, BK, 48, 64, 1, true>(gp, pl, s);
+        launch_gemm<T, 48, 256, (sizeof(T) == 8 ? 2 * BK : BK), 48, 64, 1, true>(gp, pl, s);
       else
-        launch_gemm<T, 96, 128, BK, 48, 64, 1, true>(gp, pl, s);
-      launched = true;
+        launch_gemm<T, 96, 128, (sizeof(T) == 8 ? 2 * BK : BK), 48, 64, 1, true>(gp, pl, s);
+    } else if (pl.bm == 48) {
+      launch_gemm<T, 48, 256, BK, 48, 64, 1, true>(gp, pl, s);
+    } else {
+      launch_gemm<T, 96, 128, BK, 48, 64, 1, true>(gp, pl, s);
     }
+    launched = true;
   }
 #define MG_LAUNCH(TT, BM, BN, WM, WN)                     \
   if (!launched && pl.bm == BM && pl.bn == BN) {          \
@@ -1602,10 +1632,17 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
 // Values per row of the packed filters: M rounded up to a multiple of four.
 inline int packed_ld(int M, bool tap_major) { return tap_major ? (M + 3) / 4 * 4 : M; }
 
+// Values per packed row when the three taps of the last axis are rows (n channels or filters):
+// 3n rounded up to four in single precision, whole 48-row wave tiles in double.
+template <typename T>
+int folded_ld(int n) {
+  return sizeof(T) == 8 ? 48 * (int)ceil_div(n, 16) : (3 * n + 3) / 4 * 4;
+}
+
 template <typename T>
 int pack_filters(const Geometry &g, const void *w, int mode, void **packed, size_t extra = 0, void **behind = nullptr) {
   const int M = (mode == 2 || mode == 6) ? g.F : mode == 3 ? g.C : mode == 4 ? 3 * g.C : 3 * g.F;
-  const int ld = packed_ld(M, true);
+  const int ld = mode == 4 || mode == 5 ? folded_ld<T>(M / 3) : packed_ld(M, true);
   const size_t count = (size_t)g.F * g.C * g.wvol / M * ld;
   const size_t packed_bytes = (count * sizeof(T) + 255) & ~size_t(255);
   if (mode == 3 && g.wvol == 1 && ld == g.C && reinterpret_cast<uintptr_t>(w) % 16 == 0) {
@@ -1663,7 +1700,7 @@ int conv_fwd_impl(const Geometry &g, const Plan &pl, const void *x, const void *
   gp.src_cstride = (int)g.xvol;
   gp.src_nstride = (long long)g.C * g.xvol;
   gp.dst_nstride = (long long)g.F * g.gvol;
-  gp.a_ld = packed_ld(pl.fold_row ? 3 * g.F : g.F, pl.tap_major);
+  gp.a_ld = pl.fold_row ? folded_ld<T>(g.F) : packed_ld(g.F, pl.tap_major);
   gp.a_bytes = (unsigned)((size_t)g.C * (pl.fold_row ? g.wvol / 3 : g.wvol) * gp.a_ld * sizeof(T));
   gp.src_bytes = pl.tap_major ? (unsigned)((size_t)g.N * g.C * g.xvol * sizeof(T)) : 0;
   return run_gemm<T>(gp, pl, TAG_CONV_FWD, runtime().stream);
@@ -1698,7 +1735,7 @@ int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   gp.src_cstride = (int)g.gvol;
   gp.src_nstride = (long long)g.F * g.gvol;
   gp.dst_nstride = (long long)g.C * g.xvol;
-  gp.a_ld = packed_ld(pl.fold_row ? 3 * g.C : g.C, pl.tap_major);
+  gp.a_ld = pl.fold_row ? folded_ld<T>(g.C) : packed_ld(g.C, pl.tap_major);
   gp.a_bytes = (unsigned)((size_t)g.F * (pl.fold_row ? g.wvol / 3 : g.wvol) * gp.a_ld * sizeof(T));
   gp.src_bytes = pl.tap_major ? (unsigned)((size_t)g.N * g.F * g.gvol * sizeof(T)) : 0;
   return run_gemm<T>(gp, pl, TAG_CONV_DGRAD, runtime().stream);

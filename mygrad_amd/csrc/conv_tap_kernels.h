@@ -140,7 +140,7 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
   // FOLD: the three taps of the last axis are rows of the tile (see GemmParams::fold_row): three
   // times the rows per gathered element, a third of the K tiles.  A wave makes 48 rows (16
   // channels x 3 taps) x 64 positions, which are whole rows of the last axis.
-  static_assert(!FOLD || (NPH == 1 && WM == 48 && WN == 64 && sizeof(T) == 4), "folded taps: 48 x 64 float wave tiles");
+  static_assert(!FOLD || (NPH == 1 && WM == 48 && WN == 64), "folded taps: 48 x 64 wave tiles");
   // NPH > 1: every tile computes NPH stride phases of the data gradient (see GemmParams::nph):
   // the K tiles of the phases follow each other in the tile's stream, each phase has its own
   // accumulators, and the epilogue writes the phases together.
@@ -462,6 +462,55 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
               store_vec<T, 2>(slot + f * (BM * BN) + ml * BN + bcol8 + g * 16, two);
             }
           }
+        continue;
+      }
+      if constexpr (FOLD) {
+        // Double precision with folded taps.  Rows are ordered (tap of the last axis, channel), so
+        // that the lane's row pairs i = 0,1 / 2,3 / 4,5 are taps 0 / 1 / 2 of its two channels
+        // drow, drow + 1.  A lane holds the position pairs first, first + 1 (first = 2q + 16g, q its
+        // place among the eight lanes that share its rows):
+        //   dst[pos] = tap1[pos] + tap0[pos + 1] + tap2[pos - 1]
+        // pos + 1 of an odd position and pos - 1 of an even one are with the lane next door (the
+        // first pair of q = 0 and the last of q = 7: with the lane at the other end, one pair over),
+        // and beyond the ends of a (padded) row there is nothing to add.
+        static_assert(GM == 6 && GN == 8, "three taps x two channels, four position pairs per lane");
+        const int q8 = l16 & 7;
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+          const int m = (m0 + wm0) / 3 + (drow - wm0) + r;  // channel
+          T out_e[GN / 2], out_o[GN / 2];
+#pragma unroll
+          for (int g = 0; g < GN / 2; ++g) {
+            const T t0e = acc[0][r][2 * g], t0o = acc[0][r][2 * g + 1];
+            const T t1e = acc[0][2 + r][2 * g], t1o = acc[0][2 + r][2 * g + 1];
+            const T t2e = acc[0][4 + r][2 * g], t2o = acc[0][4 + r][2 * g + 1];
+            // the odd position to the left of this pair, the even one to its right
+            const T left_near = __shfl_up(t2o, 1, 8);
+            const T left_far = __shfl(g > 0 ? acc[0][4 + r][2 * g - 1] : T(0), 7, 8);
+            const T right_near = __shfl_down(t0e, 1, 8);
+            const T right_far = __shfl(g + 1 < GN / 2 ? acc[0][r][2 * g + 2] : T(0), 0, 8);
+            const int first = pos0 + bcol8 + g * 16;
+            const unsigned in_row = (unsigned)first & (unsigned)(p.fold_row - 1);
+            const T left = in_row == 0 ? T(0) : (q8 > 0 ? left_near : left_far);
+            const T right = in_row + 2 == (unsigned)p.fold_row ? T(0) : (q8 < 7 ? right_near : right_far);
+            out_e[g] = (t1e + t0o) + left;
+            out_o[g] = (t1o + right) + t2e;
+          }
+#pragma unroll
+          for (int g = 0; g < GN / 2; ++g) {
+            const int first = pos0 + bcol8 + g * 16;
+            const int real = p.Q[2] - (int)((unsigned)first & (unsigned)(p.fold_row - 1));
+            if (first >= ph.npos || real <= 0 || m >= p.M) continue;
+            T *out = dst_of(first) + (long long)m * p.dst_mstride;
+            if (p.vec_store) {
+              const T two[2] = {out_e[g], out_o[g]};
+              store_vec<T, 2>(out, two);
+            } else {
+              out[0] = out_e[g];
+              if (real > 1) out[1] = out_o[g];
+            }
+          }
+        }
         continue;
       }
 #pragma unroll

@@ -409,36 +409,38 @@ FOLDED_TAP_CASES = [
 ]
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("case", range(len(FOLDED_TAP_CASES)))
-def test_conv_with_the_last_axis_taps_folded_into_rows(abi, case, monkeypatch):
+def test_conv_with_the_last_axis_taps_folded_into_rows(abi, case, dtype, monkeypatch):
     monkeypatch.setenv("MYGRAD_HIP_TINY", "0")  # small shapes: planned like large ones, or they take the table-driven kernel
     x_shape, w_shape, s, p, d = FOLDED_TAP_CASES[case]
     rng = np.random.default_rng(1300 + case)
-    w = (rng.standard_normal(w_shape) / np.sqrt(np.prod(w_shape[1:]))).astype(np.float32)
+    tol = TOL[np.dtype(dtype)]
+    w = (rng.standard_normal(w_shape) / np.sqrt(np.prod(w_shape[1:]))).astype(dtype)
     grid = tuple((x + 2 * pp - ((t - 1) * dd + 1)) // ss + 1 for x, t, ss, pp, dd in zip(x_shape[2:], w_shape[2:], s, p, d))
-    g = rng.standard_normal((x_shape[0], w_shape[0], *grid)).astype(np.float32)
+    g = rng.standard_normal((x_shape[0], w_shape[0], *grid)).astype(dtype)
     dx = abi.conv_dgrad(g, x_shape, w, s, p, d)
-    assert rel_err(dx, direct.conv_backward_x(g, x_shape, w, s, p, d)) <= 2e-4
+    assert rel_err(dx, direct.conv_backward_x(g, x_shape, w, s, p, d)) <= tol
     assert np.array_equal(dx, abi.conv_dgrad(g, x_shape, w, s, p, d))
     # exact with ones: per input element, the number of (filter, tap) pairs that reach it -- a
     # shift in the wrong direction or a neighbour taken across a row end changes the counts
-    ones_w = np.ones(w_shape, dtype=np.float32)
+    ones_w = np.ones(w_shape, dtype=dtype)
     ones_g = np.ones_like(g)
     assert np.array_equal(abi.conv_dgrad(ones_g, x_shape, ones_w, s, p, d),
-                          direct.conv_backward_x(ones_g, x_shape, ones_w, s, p, d).astype(np.float32))
+                          direct.conv_backward_x(ones_g, x_shape, ones_w, s, p, d).astype(dtype))
     # and with a filter that is not symmetric along the last axis (tap t2 weighs t2 + 1), so that
     # tap 0 and tap 2 cannot be swapped unnoticed
-    ramp_w = np.ones(w_shape, dtype=np.float32) * np.arange(1, w_shape[-1] + 1, dtype=np.float32)
+    ramp_w = np.ones(w_shape, dtype=dtype) * np.arange(1, w_shape[-1] + 1, dtype=dtype)
     assert np.array_equal(abi.conv_dgrad(ones_g, x_shape, ramp_w, s, p, d),
-                          direct.conv_backward_x(ones_g, x_shape, ramp_w, s, p, d).astype(np.float32))
+                          direct.conv_backward_x(ones_g, x_shape, ramp_w, s, p, d).astype(dtype))
     # the forward pass folds the same way when there are few filters (and channels in whole K tiles)
-    x = rng.standard_normal(x_shape).astype(np.float32)
+    x = rng.standard_normal(x_shape).astype(dtype)
     out = abi.conv_fwd(x, w, s, p, d)
-    assert rel_err(out, direct.conv_forward(x, w, s, p, d)) <= 2e-4
+    assert rel_err(out, direct.conv_forward(x, w, s, p, d)) <= tol
     assert np.array_equal(out, abi.conv_fwd(x, w, s, p, d))
     # exact: x counts along the last axis (small integers), ramp filter
-    steps = np.broadcast_to(np.arange(x_shape[-1], dtype=np.float32) % 5, x_shape).copy()
-    assert np.array_equal(abi.conv_fwd(steps, ramp_w, s, p, d), direct.conv_forward(steps, ramp_w, s, p, d).astype(np.float32))
+    steps = np.broadcast_to(np.arange(x_shape[-1], dtype=dtype) % 5, x_shape).copy()
+    assert np.array_equal(abi.conv_fwd(steps, ramp_w, s, p, d), direct.conv_forward(steps, ramp_w, s, p, d).astype(dtype))
 
 
 # Channel counts that fill no K tile (the one or three channels of a first layer), on problems
