@@ -159,6 +159,19 @@ __global__ void __launch_bounds__(256) pack_filters_kernel(const T *__restrict__
   }
 }
 
+// Packed filters of a data gradient on table rows: Ap[k][c] = w[arow[k] + c * taps], where arow[k]
+// is the offset of row k's (filter, tap) for channel 0, or negative for a padding row (zeros).
+template <typename T>
+__global__ void __launch_bounds__(256) pack_rows_kernel(const T *__restrict__ w, T *__restrict__ ap, const int *__restrict__ arow,
+                                                        int rows, int C, int wvol, int ld) {
+  const int total = rows * ld;
+  for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+    const int c = idx % ld, k = idx / ld;
+    const int at = arow[k];
+    ap[idx] = (c < C && at >= 0) ? w[(long long)at + (long long)c * wvol] : T(0);
+  }
+}
+
 // ------------------------------------------------------------------------------------------
 // gather-GEMM (forward and data gradient)
 // ------------------------------------------------------------------------------------------
@@ -570,6 +583,7 @@ struct Plan {
   bool tap_major = false;  // which kernel family the tables are for
   bool single_dense_phase = false;  // positions enumerate the destination tensor in order
   bool table_rows = false;          // tap-major kernel whose K tiles are rows of the gather table (channel count no multiple of the K tile)
+  int table_count = 0;              // data gradient on table rows: rows of the (padded) table = rows of the packed filters
   int fold_row = 0;                 // data gradient with the last axis' three taps folded into the rows: length of a row of positions
   bool deep_k = false;              // table-driven, a few microseconds of work: 16 x 64 tiles with a K tile four times as deep
   // fused stride phases of the data gradient (see GemmParams::nph)
@@ -977,6 +991,14 @@ void deepen_if_tiny(const Geometry &g, Plan &pl) {
   pl.deep_k = true;
 }
 
+bool table_rows_on() {
+  static const bool on = [] {
+    const char *flag = getenv("MYGRAD_HIP_TABLE_ROWS");
+    return !(flag && flag[0] == '0');
+  }();
+  return on;
+}
+
 int build_fwd_plan(const Geometry &g, Plan &pl) {
   Tables t;
   pl.tap_major = g.C % gemm_bk(g.dtype) == 0 && fits_buffer_loads(g);
@@ -1094,7 +1116,11 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
   // whole steps: 3 channels 38.5 -> 28 us; with 16 channels the tap-major kernels are 4 us
   // ahead, and with 32 or 64 the table-driven kernel's few, long-running blocks cost 2 - 5 x.)
   pl.tap_major = g.F % gemm_bk(g.dtype) == 0 && fits_buffer_loads(g) && !(is_tiny(g) && g.C <= 8);
-  const int bk = pl.tap_major ? tap_bk(g.dtype, g.F) : gemm_bk(g.dtype);
+  // filter counts that fill no K tile (10, 20, ...): the tap-major kernel on rows of the gather
+  // table, as in the forward pass (MYGRAD_HIP_TABLE_ROWS=0: the plain table-driven kernel)
+  pl.table_rows = table_rows_on() && g.F % gemm_bk(g.dtype) != 0 && fits_buffer_loads(g) && !is_tiny(g);
+  if (pl.table_rows) pl.tap_major = true;
+  const int bk = pl.table_rows ? 16 : pl.tap_major ? tap_bk(g.dtype, g.F) : gemm_bk(g.dtype);
   pl.bk = bk;
   pl.single_dense_phase = g.S[0] == 1 && g.S[1] == 1 && g.S[2] == 1;
   const int gs[3] = {g.G[1] * g.G[2], g.G[2], 1};
@@ -1140,7 +1166,7 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
   // matrix pipes -- and the epilogue adds the three rows of a channel, shifted along the last
   // axis, into dx.  A wave's 64 positions must be whole rows: rows of up to 64 positions, padded
   // to a power of two.
-  if (fold_applies(g, g.C, g.F) && pl.tap_major && nphase == 1 && found.size() == 1) {
+  if (fold_applies(g, g.C, g.F) && pl.tap_major && !pl.table_rows && nphase == 1 && found.size() == 1) {
     const PhaseTaps &pt = found[0];
     Phase ph = pt.ph;
     for (int f0 = 0; f0 < g.F; f0 += bk)
@@ -1174,7 +1200,7 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
     const char *flag = getenv("MYGRAD_HIP_FUSE");
     return !(flag && flag[0] == '0');
   }();
-  const bool fused = fuse_on && pl.tap_major && g.dtype == MG_F32 && g.S[2] == 2 && g.S[0] <= 2 && g.S[1] <= 2 &&
+  const bool fused = fuse_on && pl.tap_major && !pl.table_rows && g.dtype == MG_F32 && g.S[2] == 2 && g.S[0] <= 2 && g.S[1] <= 2 &&
                      (nphase == 2 || nphase == 4) && (long long)found.size() == nphase;
   if (fused) {
     std::stable_sort(found.begin(), found.end(), [](const PhaseTaps &a, const PhaseTaps &b) {
@@ -1250,7 +1276,7 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
     for (const PhaseTaps &pt : found) {
       npos.push_back(pt.ph.npos);
       const long long ntaps = (long long)pt.taps[0].size() * pt.taps[1].size() * pt.taps[2].size();
-      min_ktiles = std::min(min_ktiles, pl.tap_major ? ntaps * (g.F / bk) : ceil_div(ntaps * g.F, bk));
+      min_ktiles = std::min(min_ktiles, pl.tap_major && !pl.table_rows ? ntaps * (g.F / bk) : ceil_div(ntaps * g.F, bk));
     }
     const TileChoice tc = choose_tile(g.C, npos, (int)std::max<long long>(min_ktiles, 0), pl.tap_major, g.dtype == MG_F64 ? 8 : 4, 1, bk);
     pl.bm = tc.bm, pl.bn = tc.bn, pl.m_tiles = tc.m_tiles, pl.full_tiles = tc.full_tiles, pl.tail_split = tc.tail_split, pl.blocks_per_cu = tc.blocks_per_cu;
@@ -1262,7 +1288,36 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
   for (PhaseTaps &pt : found) {
     Phase &ph = pt.ph;
     ph.k_begin = pl.tap_major ? (int)t.ktiles.size() : (int)t.tab.size();
-    if (pl.tap_major) {
+    if (pl.table_rows) {
+      // the phase's rows (filter, tap), padded to whole K tiles with rows that lie outside every
+      // input and name no element of the filter bank (a zero row of the packed filters)
+      const int first_row = (int)t.tab.size();
+      for (int f = 0; f < g.F; ++f)
+        for (size_t a = 0; a < pt.taps[0].size(); ++a)
+          for (size_t b = 0; b < pt.taps[1].size(); ++b)
+            for (size_t c = 0; c < pt.taps[2].size(); ++c) {
+              TabEntry e;
+              e.d0 = pt.offs[0][a];
+              e.d1 = pt.offs[1][b];
+              e.d2 = pt.offs[2][c];
+              e.off = (int)(f * g.gvol) + e.d0 * gs[0] + e.d1 * gs[1] + e.d2 * gs[2];
+              t.tab.push_back(e);
+              t.arow.push_back((int)(f * g.C * g.wvol) + (pt.taps[0][a] * g.W[1] + pt.taps[1][b]) * g.W[2] + pt.taps[2][c]);
+            }
+      TabEntry outside{};
+      outside.d0 = outside.d1 = outside.d2 = 1 << 29;
+      while ((t.tab.size() - first_row) % bk != 0) {
+        t.tab.push_back(outside);
+        t.arow.push_back(-1);
+      }
+      for (int k0 = first_row; k0 < (int)t.tab.size(); k0 += bk) {
+        KTile e{};
+        e.a_row0 = k0;
+        e.coff = k0;  // first table row of the tile
+        t.ktiles.push_back(e);
+      }
+      ph.k_count = (int)t.ktiles.size() - ph.k_begin;
+    } else if (pl.tap_major) {
       for (int f0 = 0; f0 < g.F; f0 += bk)  // filter block outermost: its taps share rows of grad
         for (size_t a = 0; a < pt.taps[0].size(); ++a)
           for (size_t b = 0; b < pt.taps[1].size(); ++b)
@@ -1297,6 +1352,7 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
     t.phases.push_back(ph);
   }
   pl.pos_blocks = blk;
+  pl.table_count = (int)t.tab.size();
   return upload_plan(pl, t);
 }
 
@@ -1407,8 +1463,10 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
       const char *flag = getenv("MYGRAD_HIP_TABLE_ROWS");
       return !(flag && flag[0] == '0');
     }();
-    const int row_tile = g.F % 64 == 0 ? 64 : g.F % 32 == 0 ? 32 : g.F % 16 == 0 ? 16 : 0;
-    if (rows_on && row_tile && fits_buffer_loads(g) && !is_tiny(g)) {
+    // filters in row tiles of 16, 32 or 64, the last one possibly short: its rows beyond F read
+    // whatever follows in grad (or zeros past its end) and are not stored
+    const int row_tile = g.F <= 16 ? 16 : g.F <= 32 ? 32 : g.F <= 48 ? 16 : 64;
+    if (rows_on && fits_buffer_loads(g) && !is_tiny(g)) {
       pl.tap_major = pl.table_rows = true;
       pl.bm = row_tile;
       pl.bn = 64;
@@ -1712,6 +1770,16 @@ int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   void *partial = nullptr;
   if (!pl.tap_major) {
     packed = const_cast<void *>(w);  // read in place: row k = (f, tap) of channel m lies at w[(f * C + m) * taps + tap]
+  } else if (pl.table_rows) {
+    const int ld = packed_ld(g.C, true);
+    const size_t packed_bytes = ((size_t)pl.table_count * ld * sizeof(T) + 255) & ~size_t(255);
+    if (int rc = workspace(packed_bytes + tail_bytes(pl, sizeof(T)), &packed)) return rc;
+    partial = static_cast<char *>(packed) + packed_bytes;
+    ScopedTiming timed(TAG_PACK_FILTERS);
+    const unsigned blocks = (unsigned)std::min<long long>(ceil_div((long long)pl.table_count * ld, 256), 4096);
+    hipLaunchKernelGGL(pack_rows_kernel<T>, dim3(blocks), dim3(256), 0, runtime().stream, static_cast<const T *>(w),
+                       static_cast<T *>(packed), pl.arow, pl.table_count, (int)g.C, (int)g.wvol, ld);
+    MG_HIP(hipGetLastError());
   } else if (int rc = pack_filters<T>(g, w, pl.fold_row ? 4 : 3, &packed, tail_bytes(pl, sizeof(T)), &partial)) {
     return rc;
   }
@@ -1736,7 +1804,8 @@ int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   gp.src_nstride = (long long)g.F * g.gvol;
   gp.dst_nstride = (long long)g.C * g.xvol;
   gp.a_ld = pl.fold_row ? folded_ld<T>(g.C) : packed_ld(g.C, pl.tap_major);
-  gp.a_bytes = (unsigned)((size_t)g.F * (pl.fold_row ? g.wvol / 3 : g.wvol) * gp.a_ld * sizeof(T));
+  gp.a_bytes = pl.table_rows ? (unsigned)((size_t)pl.table_count * gp.a_ld * sizeof(T))
+                             : (unsigned)((size_t)g.F * (pl.fold_row ? g.wvol / 3 : g.wvol) * gp.a_ld * sizeof(T));
   gp.src_bytes = pl.tap_major ? (unsigned)((size_t)g.N * g.F * g.gvol * sizeof(T)) : 0;
   return run_gemm<T>(gp, pl, TAG_CONV_DGRAD, runtime().stream);
 }

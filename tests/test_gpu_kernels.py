@@ -454,12 +454,19 @@ FIRST_LAYER_CASES = [
     ((64, 7, 500), (48, 7, 9), (3,), (4,), (2,)),
     ((64, 1, 28, 28), (64, 1, 5, 5), (1, 1), (0, 0), (1, 1)),       # 25 columns of dw: one 32-column tile
     ((16, 3, 48, 48), (128, 3, 7, 7), (1, 1), (3, 3), (1, 1)),      # 147 columns: two 80-column tiles, two row tiles
+    # filter counts that fill no K tile either: the data gradient on table rows, the filter gradient
+    # with a short last row tile
+    ((256, 1, 28, 28), (20, 1, 5, 5), (1, 1), (0, 0), (1, 1)),
+    ((256, 20, 12, 12), (10, 20, 5, 5), (1, 1), (0, 0), (1, 1)),
+    ((32, 24, 41, 40), (20, 24, 3, 4), (2, 2), (1, 1), (1, 1)),     # four stride phases with different tap counts
+    ((6, 16, 10, 18, 18), (35, 16, 3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
+    ((64, 40, 301), (19, 40, 7), (2,), (3,), (3,)),
 ]
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("case", range(len(FIRST_LAYER_CASES)))
-def test_conv_forward_with_channels_that_fill_no_k_tile(abi, dtype, case):
+def test_conv_with_channel_or_filter_counts_that_fill_no_k_tile(abi, dtype, case):
     x_shape, w_shape, s, p, d = FIRST_LAYER_CASES[case]
     rng = np.random.default_rng(1500 + case)
     tol = TOL[np.dtype(dtype)]
@@ -476,6 +483,10 @@ def test_conv_forward_with_channels_that_fill_no_k_tile(abi, dtype, case):
     g = rng.standard_normal(want.shape).astype(dtype)
     assert rel_err(abi.conv_dgrad(g, x_shape, w, s, p, d), direct.conv_backward_x(g, x_shape, w, s, p, d)) <= tol
     assert rel_err(abi.conv_wgrad(g, x, w_shape, s, p, d), direct.conv_backward_w(g, x, w_shape, s, p, d)) <= tol
+    # exact: gradients of small integers
+    gi = rng.integers(-2, 3, want.shape).astype(dtype)
+    assert np.array_equal(abi.conv_dgrad(gi, x_shape, wi, s, p, d), direct.conv_backward_x(gi, x_shape, wi, s, p, d).astype(dtype))
+    assert np.array_equal(abi.conv_wgrad(gi, xi, w_shape, s, p, d), direct.conv_backward_w(gi, xi, w_shape, s, p, d).astype(dtype))
 
 
 # Shapes picked so that, between them, every tile shape and code path of the tap-major
