@@ -984,6 +984,17 @@ bool is_tiny(const Geometry &g) {
          2.0 * (double)g.N * (double)g.gvol * (double)g.F * (double)g.C * (double)g.wvol < 1e8;
 }
 
+// Whether a tiny problem with `rows` rows and a contraction of `depth` (channels x taps, or
+// filters x taps) is better off on the table-driven kernel -- one launch, no packing: when a
+// block's chain of K tiles there is at most five long (its K tile is 64 / 32 deep for up to 16
+// rows, 16 / 8 beyond; float / double).  Measured on MNIST-sized layers: a contraction of 25 or
+// 144 is faster there, one of 250 or 500 is 1.3 - 2.4 x slower than the tap-major kernel on
+// table rows.
+bool tiny_table(const Geometry &g, int rows, long long depth) {
+  const int k_tile = (rows <= 16 ? 4 : 1) * gemm_bk(g.dtype);
+  return is_tiny(g) && depth <= 5 * k_tile;
+}
+
 // The table-driven kernel for such a problem: more, smaller tiles and a quarter of the K steps.
 void deepen_if_tiny(const Geometry &g, Plan &pl) {
   if (pl.tap_major || !is_tiny(g) || pl.bm != 16) return;
@@ -1009,7 +1020,7 @@ int build_fwd_plan(const Geometry &g, Plan &pl) {
     const char *flag = getenv("MYGRAD_HIP_TABLE_ROWS");
     return !(flag && flag[0] == '0');
   }();
-  pl.table_rows = rows_on && !pl.tap_major && fits_buffer_loads(g) && !is_tiny(g);
+  pl.table_rows = rows_on && !pl.tap_major && fits_buffer_loads(g) && !tiny_table(g, g.F, (long long)g.C * g.wvol);
   if (pl.table_rows) pl.tap_major = true;
   const int bk = pl.table_rows ? 16 : pl.tap_major ? tap_bk(g.dtype, g.C) : gemm_bk(g.dtype);
   pl.bk = bk;
@@ -1115,10 +1126,10 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
   // with its deep K tiles needs neither packed filters nor a pass over partial sums.  (Measured,
   // whole steps: 3 channels 38.5 -> 28 us; with 16 channels the tap-major kernels are 4 us
   // ahead, and with 32 or 64 the table-driven kernel's few, long-running blocks cost 2 - 5 x.)
-  pl.tap_major = g.F % gemm_bk(g.dtype) == 0 && fits_buffer_loads(g) && !(is_tiny(g) && g.C <= 8);
+  pl.tap_major = g.F % gemm_bk(g.dtype) == 0 && fits_buffer_loads(g) && !(tiny_table(g, g.C, (long long)g.F * g.wvol) && g.C <= 8);
   // filter counts that fill no K tile (10, 20, ...): the tap-major kernel on rows of the gather
   // table, as in the forward pass (MYGRAD_HIP_TABLE_ROWS=0: the plain table-driven kernel)
-  pl.table_rows = table_rows_on() && g.F % gemm_bk(g.dtype) != 0 && fits_buffer_loads(g) && !is_tiny(g);
+  pl.table_rows = table_rows_on() && g.F % gemm_bk(g.dtype) != 0 && fits_buffer_loads(g) && !tiny_table(g, g.C, (long long)g.F * g.wvol);
   if (pl.table_rows) pl.tap_major = true;
   const int bk = pl.table_rows ? 16 : pl.tap_major ? tap_bk(g.dtype, g.F) : gemm_bk(g.dtype);
   pl.bk = bk;
@@ -1466,7 +1477,7 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
     // filters in row tiles of 16, 32 or 64, the last one possibly short: its rows beyond F read
     // whatever follows in grad (or zeros past its end) and are not stored
     const int row_tile = g.F <= 16 ? 16 : g.F <= 32 ? 32 : g.F <= 48 ? 16 : 64;
-    if (rows_on && fits_buffer_loads(g) && !is_tiny(g)) {
+    if (rows_on && fits_buffer_loads(g)) {
       pl.tap_major = pl.table_rows = true;
       pl.bm = row_tile;
       pl.bn = 64;
