@@ -1,6 +1,7 @@
 // Device selection, the library stream, buffers, copies, events and scratch.
 #include "internal.h"
 
+#include <atomic>
 #include <cstdlib>
 #include <cstring>
 #include <map>
@@ -9,8 +10,13 @@
 
 namespace mg {
 
+// entry points called so far (every one of them takes the lock first): lets the per-launch timing
+// tell whether anything can have been enqueued between two timed launches
+static std::atomic<unsigned long long> g_api_calls{0};
+
 std::recursive_mutex &api_mutex() {
   static std::recursive_mutex m;
+  ++g_api_calls;
   return m;
 }
 
@@ -56,47 +62,84 @@ int workspace(size_t nbytes, void **ptr) {
 }
 
 // ---- per-launch timing -------------------------------------------------------------------
+// One event after every timed launch; the event after the launch before it serves as its start
+// when nothing else can have been enqueued in between (the earlier scope ended in this entry
+// point or in the one called just before it) -- an event record costs a few microseconds of
+// stream time, which for launches of 5 - 20 us is a large part of what is being measured.
 namespace {
 struct TimingRecord {
   int tag;
-  hipEvent_t start, stop;
+  size_t start, stop;  // indices into Timing::events
 };
 struct Timing {
   bool on = false;
-  std::vector<TimingRecord> records;  // event pairs are created once and reused
-  size_t used = 0;
+  std::vector<hipEvent_t> events;  // created once and reused
+  std::vector<TimingRecord> records;
+  size_t used_events = 0, used = 0;
+  bool open = false;               // between timing_begin and timing_end
+  size_t open_start = 0;
+  int open_tag = 0;
+  bool chain = false;              // the last thing enqueued by a timed scope was events[last_stop]
+  size_t last_stop = 0;
+  unsigned long long chain_call = 0;
 } g_timing;
+// the next unused event, recorded on the library stream; false if none could be created
+bool record_next_event(size_t *index) {
+  if (g_timing.used_events == g_timing.events.size()) {
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) {
+      (void)hipGetLastError();
+      g_timing.on = false;
+      return false;
+    }
+    g_timing.events.push_back(e);
+  }
+  *index = g_timing.used_events++;
+  (void)hipEventRecord(g_timing.events[*index], runtime().stream);
+  return true;
+}
 }  // namespace
 
 void timing_begin(int tag) {
   if (!g_timing.on) return;
-  if (g_timing.used == g_timing.records.size()) {
-    TimingRecord r{tag, nullptr, nullptr};
-    if (hipEventCreate(&r.start) != hipSuccess || hipEventCreate(&r.stop) != hipSuccess) {
-      (void)hipGetLastError();
-      g_timing.on = false;
-      return;
-    }
-    g_timing.records.push_back(r);
+  const unsigned long long call = g_api_calls.load();
+  g_timing.open_tag = tag;
+  if (g_timing.chain && call - g_timing.chain_call <= 1) {
+    g_timing.open_start = g_timing.last_stop;
+    g_timing.open = true;
+    return;
   }
-  TimingRecord &r = g_timing.records[g_timing.used];
-  r.tag = tag;
-  (void)hipEventRecord(r.start, runtime().stream);
+  g_timing.open = record_next_event(&g_timing.open_start);
 }
 
 void timing_end() {
-  if (!g_timing.on) return;
-  (void)hipEventRecord(g_timing.records[g_timing.used].stop, runtime().stream);
+  if (!g_timing.on || !g_timing.open) return;
+  g_timing.open = false;
+  size_t stop = 0;
+  if (!record_next_event(&stop)) return;
+  TimingRecord r{g_timing.open_tag, g_timing.open_start, stop};
+  if (g_timing.used == g_timing.records.size())
+    g_timing.records.push_back(r);
+  else
+    g_timing.records[g_timing.used] = r;
   ++g_timing.used;
+  g_timing.chain = true;
+  g_timing.last_stop = stop;
+  g_timing.chain_call = g_api_calls.load();
+}
+
+static void timing_reset() {
+  g_timing.used = 0;
+  g_timing.used_events = 0;
+  g_timing.open = false;
+  g_timing.chain = false;
 }
 
 static void timing_release() {
-  for (auto &r : g_timing.records) {
-    (void)hipEventDestroy(r.start);
-    (void)hipEventDestroy(r.stop);
-  }
+  for (hipEvent_t e : g_timing.events) (void)hipEventDestroy(e);
+  g_timing.events.clear();
   g_timing.records.clear();
-  g_timing.used = 0;
+  timing_reset();
   g_timing.on = false;
 }
 
@@ -473,7 +516,7 @@ int mg_timing_enable(int on) {
   MG_LOCK();
   MG_REQUIRE_INIT();
   MG_HIP(hipStreamSynchronize(runtime().stream));
-  g_timing.used = 0;
+  timing_reset();
   g_timing.on = on != 0;
   return MG_OK;
 }
@@ -487,9 +530,9 @@ int mg_timing_read(int32_t *tags, float *ms, int capacity, int *count) {
   *count = n;
   for (int i = 0; i < n && i < capacity; ++i) {
     tags[i] = g_timing.records[i].tag;
-    MG_HIP(hipEventElapsedTime(&ms[i], g_timing.records[i].start, g_timing.records[i].stop));
+    MG_HIP(hipEventElapsedTime(&ms[i], g_timing.events[g_timing.records[i].start], g_timing.events[g_timing.records[i].stop]));
   }
-  g_timing.used = 0;
+  timing_reset();
   return MG_OK;
 }
 
