@@ -50,7 +50,9 @@ def einsum(*operands, optimize=False, out=None, constant=None):
     on the device.  More than two operands are contracted pairwise from the left; a label
     that occurs twice in one operand (``"ii"``: a trace or a diagonal) is taken along its
     diagonal first; an axis of length one is broadcast against a longer one under the
-    same label.  ``out=`` raises ``NotImplementedError``.  A tensor that occurs
+    same label.  ``out=`` takes a NumPy array, which receives the result and becomes the returned
+    tensor's data (a tensor as the target asks for the reference's in-place graph semantics, which
+    this package does not have: ``NotImplementedError``).  A tensor that occurs
     twice with the same labels receives one gradient, scaled by two, as in the reference.
     The result is a new array, where ``numpy.einsum`` may return a view.
 
@@ -63,6 +65,8 @@ def einsum(*operands, optimize=False, out=None, constant=None):
     Tensor([[10., 28., 46., 64.],
             [13., 40., 67., 94.]])
     """
+    if isinstance(out, Tensor):
+        raise NotImplementedError("einsum(..., out=<Tensor>) needs in-place operations on tensors, which are outside this package; pass an ndarray")
     operands = list(operands)
     if isinstance(operands[0], str):
         variables = operands[1:]

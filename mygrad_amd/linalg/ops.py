@@ -18,9 +18,10 @@ the same kind of summation with the incoming gradient in the operand's place.
 What runs: float32 / float64 operands (more than two are contracted pairwise from the
 left); a label repeated within one operand is taken along its diagonal first
 (``mg_strided_copy``), and its gradient is written back along that diagonal into zeros; an
-axis of length one under a label that is longer elsewhere is broadcast.  Anything else
-raises ``NotImplementedError``; there is no CPU fallback.  The result is always a new
-array, never a view of an operand."""
+axis of length one under a label that is longer elsewhere is broadcast (a diagonal of
+length one included); ``out=`` names a NumPy array that receives the result.  Anything else
+raises ``NotImplementedError``; there is no CPU fallback.  Without ``out`` the result is a
+new array, never a view of an operand."""
 
 from collections import Counter
 from itertools import chain
@@ -229,8 +230,8 @@ class EinSum(Operation):
         self.variables = variables
         self.optimize = optimize
         self._cache = None  # how often each (tensor, labels) pair occurs; see backward_var
-        if out is not None:
-            raise NotImplementedError("einsum on the GPU does not write into an existing array (out=...)")
+        if out is not None and not isinstance(out, np.ndarray):
+            raise TypeError("keyword parameter out must be an array for einsum")
         arrays = [_device.value_of(v) for v in variables]
 
         # the checks np.einsum makes, with its exception type
@@ -239,10 +240,14 @@ class EinSum(Operation):
                              if len(arrays) > len(self.in_lbls) else
                              "fewer operands provided to einstein sum function than specified in the subscripts string")
         sizes = {}
-        for lbls, arr in zip(self.in_lbls, arrays):
+        for nth, (lbls, arr) in enumerate(zip(self.in_lbls, arrays)):
             if len(lbls) != arr.ndim:
                 raise ValueError(f"einstein sum subscripts string '{lbls}' does not match the {arr.ndim} axes of its operand")
+            own = {}  # a label repeated within the operand walks a diagonal: its axes must agree
             for lbl, n in zip(lbls, arr.shape):
+                if own.setdefault(lbl, n) != n:
+                    raise ValueError(f"dimensions in operand {nth} for collapsing index '{lbl}' "
+                                     f"don't match ({own[lbl]} != {n})")
                 have = sizes.get(lbl)
                 if have is None or have == 1:
                     sizes[lbl] = n
@@ -250,13 +255,10 @@ class EinSum(Operation):
                     raise ValueError(f"operands could not be broadcast together: label '{lbl}' has lengths {have} and {n}")
         # An axis of length one under a label that is longer elsewhere is broadcast: the operand
         # does not depend on that label, so the label is struck from it (same memory), and
-        # its gradient is summed over the label like over any label it does not carry.
-        self._lbls = []
-        for lbls, arr in zip(self.in_lbls, arrays):
-            kept = "".join(lbl for lbl, n in zip(lbls, arr.shape) if n == sizes[lbl])
-            if kept != lbls and len(set(lbls)) != len(lbls):
-                raise NotImplementedError(f"einsum on the GPU does not broadcast an operand with a repeated label ('{lbls}')")
-            self._lbls.append(kept)
+        # its gradient is summed over the label like over any label it does not carry.  A label
+        # repeated within the operand goes or stays with all of its axes (they agree in length).
+        self._lbls = ["".join(lbl for lbl, n in zip(lbls, arr.shape) if n == sizes[lbl])
+                      for lbls, arr in zip(self.in_lbls, arrays)]
         if len(set(out_lbls)) != len(out_lbls):
             raise ValueError(f"einstein sum subscripts string includes output subscript more than once: '{out_lbls}'")
         if not set(out_lbls) <= set(sizes):
@@ -270,7 +272,21 @@ class EinSum(Operation):
         self._dtype, self._sizes = dtype, sizes
 
         out_shape = tuple(sizes[lbl] for lbl in out_lbls)
+        if out is not None:
+            # the checks np.einsum makes of its target, before anything is computed
+            if out.ndim != len(out_shape):
+                raise ValueError(f"out parameter does not have the correct number of dimensions, has {out.ndim} but should have {len(out_shape)}")
+            if out.shape != out_shape:
+                raise ValueError(f"operands could not be broadcast together: out has shape {out.shape}, the result {out_shape}")
+            if not out.flags.writeable:
+                raise ValueError("operand array with iterator write flag set is read-only")
+            if not np.can_cast(dtype, out.dtype, "safe"):
+                raise TypeError(f"Iterator requested dtype could not be cast from {dtype!r} to {out.dtype!r}, the operand {len(arrays)} dtype, "
+                                "according to the rule 'safe'")
         if 0 in sizes.values():  # an empty sum is zero, an empty result has nothing in it
+            if out is not None:
+                out[...] = 0
+                return out
             return np.zeros(out_shape, dtype=dtype)
         operands = [self._operand(arr, lbls) for arr, lbls in zip(arrays, self._lbls)]
         ob = contract_all(operands, out_lbls, sizes, dtype)
@@ -278,6 +294,15 @@ class EinSum(Operation):
             copy = _device.DeviceBuffer(max(_prod(out_shape) * dtype.itemsize, 16))
             _hip.check(_hip.lib().mg_memcpy_d2d(copy.ptr, ob.ptr, _prod(out_shape) * dtype.itemsize))
             ob = copy
+        if out is not None:
+            # the values cross to the host now, into the caller's array (which may be strided or
+            # of a wider type); the buffer stays its device copy when the two hold the same bytes
+            if out.dtype == dtype and out.flags["C_CONTIGUOUS"]:
+                ob.download_into(out)
+                _device.attach(out, ob)
+            else:
+                np.copyto(out, _device.download(ob, out_shape, dtype, now=True), casting="safe")
+            return out
         result = _device.download(ob, out_shape, dtype)
         _device.attach(result, ob)
         return result

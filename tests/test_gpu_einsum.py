@@ -55,6 +55,8 @@ CASES = [
     # an axis of length one broadcast against a longer one under the same label
     ("ij,ij->ij", [(2, 3), (1, 3)]), ("bij,bjk->bik", [(1, 3, 4), (5, 4, 2)]), ("bij,bjk->bik", [(5, 3, 4), (1, 4, 2)]),
     ("ai,ai->a", [(4, 1), (4, 6)]), ("ij,jk->ik", [(3, 1), (4, 5)]),
+    # both at once: a diagonal of length one under a label that is longer elsewhere
+    ("ii,ij->j", [(1, 1), (3, 4)]), ("iji,ik->jk", [(1, 3, 1), (4, 2)]), ("ii,jj->ij", [(1, 1), (4, 4)]), ("iij,ik->jk", [(1, 1, 5), (6, 2)]),
 ]
 
 
@@ -138,8 +140,8 @@ def test_errors_and_what_is_refused():
         mg.einsum("ij,jk->ii", a, b)
     with pytest.raises(ValueError):
         mg.einsum("ii->i", mg.Tensor(np.ones((3, 4))))  # the two axes of a diagonal differ in length
-    with pytest.raises(NotImplementedError):
-        mg.einsum("ii,ij->j", mg.Tensor(np.ones((1, 1))), mg.Tensor(np.ones((3, 2))))  # a diagonal that is broadcast as well
+    with pytest.raises(ValueError):
+        mg.einsum("ii,ij->j", mg.Tensor(np.ones((3, 1))), mg.Tensor(np.ones((3, 2))))  # one axis of the diagonal broadcast, one not
     with pytest.raises(TypeError):
         mg.einsum("ij,jk->ik", mg.Tensor(np.ones((2, 3), dtype=np.int64)), mg.Tensor(np.ones((3, 4), dtype=np.int64)))
 
@@ -162,3 +164,37 @@ def test_one_element_window_convolution_full_size():
     g64 = g.astype(np.float64)
     assert err(x.grad, np.tensordot(w64, g64, axes=([0], [1])).transpose(1, 0, 2, 3)) <= 2e-4
     assert err(w.grad, np.tensordot(g64, x64, axes=([0, 2, 3], [0, 2, 3]))) <= 2e-4
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_out_receives_the_result_and_becomes_the_data(dtype):
+    """``einsum(..., out=array)`` (reference: mygrad/linalg/funcs.py:445-451 hands the array to
+    ``np.einsum`` through ``Tensor._op``, mygrad/tensor_base.py:1110-1113): the array is written,
+    it is the returned tensor's data, and back-propagation runs as without it."""
+    import mygrad_amd as mg
+
+    rng = np.random.default_rng(31)
+    a, b = rng.standard_normal((6, 7)).astype(dtype), rng.standard_normal((7, 5)).astype(dtype)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    ta, tb = mg.Tensor(a), mg.Tensor(b)
+    target = np.full((6, 5), np.nan, dtype=dtype)
+    res = mg.einsum("ij,jk->ik", ta, tb, out=target)
+    assert res.data is target and err(target, want) <= TOL[np.dtype(dtype)]
+    plain = mg.einsum("ij,jk->ik", a, b)
+    assert np.array_equal(target, plain.data)
+    g = rng.standard_normal((6, 5)).astype(dtype)
+    res.backward(g)
+    assert err(ta.grad, g.astype(np.float64) @ b.T.astype(np.float64)) <= TOL[np.dtype(dtype)]
+    assert err(tb.grad, a.T.astype(np.float64) @ g.astype(np.float64)) <= TOL[np.dtype(dtype)]
+    # a consumer of the result reads the same values (from the device copy or from the array)
+    twice = mg.einsum("ik->ki", res)
+    assert np.array_equal(twice.data, target.T)
+
+    # a strided target and a wider one are filled through the host
+    wide = np.zeros((5, 6), dtype=np.float64).T
+    assert mg.einsum("ij,jk->ik", a, b, out=wide).data is wide
+    assert np.array_equal(wide, plain.data.astype(np.float64))
+    # an empty sum writes zeros
+    empty = np.full((2, 3), 7.0, dtype=dtype)
+    mg.einsum("ij,jk->ik", np.ones((2, 0), dtype=dtype), np.ones((0, 3), dtype=dtype), out=empty)
+    assert np.array_equal(empty, np.zeros((2, 3)))

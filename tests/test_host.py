@@ -517,6 +517,24 @@ def test_argument_checks_of_the_neighbouring_operations_need_no_device():
     with pytest.raises(TypeError):
         mg.einsum("i,i", np.arange(3), np.arange(3))
     assert mg.einsum("ij,jk->ik", np.ones((2, 0)), np.ones((0, 3))).shape == (2, 3)
+    # the target of out=, checked like np.einsum checks it, before anything is computed
+    ab = (np.ones((2, 3)), np.ones((3, 4)))
+    with pytest.raises(TypeError):
+        mg.einsum("ij,jk->ik", *ab, out=[[0.0] * 4] * 2)
+    with pytest.raises(TypeError):
+        mg.einsum("ij,jk->ik", *ab, out=np.zeros((2, 4), dtype=np.float32))  # float64 into float32 is no safe cast
+    with pytest.raises(ValueError):
+        mg.einsum("ij,jk->ik", *ab, out=np.zeros((2, 5)))
+    with pytest.raises(ValueError):
+        mg.einsum("ij,jk->ik", *ab, out=np.zeros((1, 2, 4)))
+    locked = np.zeros((2, 4))
+    locked.flags.writeable = False
+    with pytest.raises(ValueError):
+        mg.einsum("ij,jk->ik", *ab, out=locked)
+    with pytest.raises(NotImplementedError):
+        mg.einsum("ij,jk->ik", *ab, out=mg.Tensor(np.zeros((2, 4))))  # in-place semantics on tensors
+    with pytest.raises(ValueError):
+        mg.einsum("ii,ij->j", np.ones((3, 1)), np.ones((3, 2)))  # a diagonal whose axes differ in length
 
     with pytest.raises(ValueError):
         mg.multiply(np.ones((2, 3)), np.ones(4))  # shapes that do not broadcast

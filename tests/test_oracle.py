@@ -695,6 +695,32 @@ def test_einsum_backward_against_differences_adjoints_and_loops(subscripts, shap
         assert math.isclose(slope, float(np.sum(back * direction)), rel_tol=1e-6, abs_tol=1e-6)
 
 
+@pytest.mark.parametrize("subscripts, shapes", [
+    ("ij,ij->ij", [(2, 3), (1, 3)]), ("bij,bjk->bik", [(1, 3, 4), (5, 4, 2)]), ("ii,ij->j", [(1, 1), (3, 4)]),
+    ("iji,ik->jk", [(1, 3, 1), (4, 2)]), ("ii,jj->ij", [(1, 1), (4, 4)]), ("iij,ik->jk", [(1, 1, 5), (6, 2)]),
+])
+def test_einsum_backward_of_broadcast_operands(subscripts, shapes):
+    """An axis of length one under a label that is longer elsewhere: the gradient is summed over
+    that label.  Pinned by the adjoint identity and central differences (np.einsum itself
+    defines the forward values)."""
+    rng = np.random.default_rng(len(subscripts) * 7 + len(shapes))
+    in_lbls, out_lbls = subscripts.split("->")
+    arrays = [rng.standard_normal(s) for s in shapes]
+    out = ora.einsum_forward(in_lbls, out_lbls, *arrays)
+    g = rng.standard_normal(out.shape)
+    for index, var in enumerate(arrays):
+        back = ora.einsum_backward(g, index, in_lbls, out_lbls, arrays)
+        assert back.shape == var.shape
+        assert math.isclose(float(np.sum(out * g)), float(np.sum(var * back)), rel_tol=1e-9, abs_tol=1e-9)
+        for _ in range(3):
+            direction = rng.standard_normal(var.shape)
+            eps = 1e-6
+            plus = [a + eps * direction if n == index else a for n, a in enumerate(arrays)]
+            minus = [a - eps * direction if n == index else a for n, a in enumerate(arrays)]
+            slope = float(np.sum((ora.einsum_forward(in_lbls, out_lbls, *plus) - ora.einsum_forward(in_lbls, out_lbls, *minus)) * g)) / (2 * eps)
+            assert math.isclose(slope, float(np.sum(back * direction)), rel_tol=1e-6, abs_tol=1e-6)
+
+
 def test_einsum_reference_docstring_trace_and_diagonal():
     a = np.arange(25.0).reshape(5, 5)
     assert ora.einsum_forward("ii", "", a) == 60.0  # linalg/funcs.py docstring: the trace
