@@ -18,7 +18,7 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(ROOT, "include")
 OBJDIR = os.path.join(HERE, "build")
 LIBRARY = os.path.join(HERE, "libmygrad_hip.so")
-SOURCES = ("runtime.hip", "pool.hip", "conv.hip", "elementwise.hip", "batchnorm.hip", "tiling.hip", "batched.hip")
+SOURCES = ("runtime.hip", "pool.hip", "conv.hip", "conv_thin.hip", "elementwise.hip", "batchnorm.hip", "tiling.hip", "batched.hip")
 
 # -packed-fp32-ops is switched off: the compiler must not form packed fp32 VALU
 # instructions from ordinary float code.  (The host pass prints a harmless

@@ -17,6 +17,7 @@
 #include "internal.h"
 
 #include <algorithm>
+#include <array>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -591,6 +592,12 @@ struct Plan {
   int kcut[4] = {0, 0, 0, 0};
   int po0[4][3] = {};
   int pJ[4][3] = {};
+  // at most four rows, single precision: one position per lane on the 4x4x1 MFMA (see ThinParams)
+  bool thin = false;
+  int thin_chunks = 0, thin_kgroups = 0;
+  long long thin_src_group = 0, thin_w_group = 0;  // elements of src / of the filter bank between consecutive groups
+  int thin_w_mstride = 0;
+  Phase thin_grid{};  // J, npos and divisors of the positions (host copy)
   // wgrad
   int splits = 1;
   int kchunk = 0;
@@ -1010,8 +1017,96 @@ bool table_rows_on() {
   return on;
 }
 
+
+// ---- at most four rows (channels of a data gradient, filters of a forward pass), single
+// precision, enough positions to fill the device: the 4x4x1 MFMA kernel, one position per lane.
+// MYGRAD_HIP_THIN=0 switches it off (read whenever a plan is built, and part of the plan's key).
+bool thin_on() {
+  const char *flag = getenv("MYGRAD_HIP_THIN");
+  return !(flag && flag[0] == '0');
+}
+
+// Positions: one wave per SIMD (65536) with several stride phases, where the 16-row tiles take two
+// to three times as long; four waves per SIMD with one phase, where a gathered element feeds a
+// single MFMA and the kernel is bound by its loads (at one wave per SIMD it loses a quarter,
+// at sixteen it is ahead by one).
+bool thin_applies(const Geometry &g, int rows, long long positions, long long depth, long long nph) {
+  return thin_on() && g.dtype == MG_F32 && rows <= 4 && fits_buffer_loads(g) && positions >= (nph == 1 ? 4 : 1) * 65536 &&
+         !tiny_table(g, rows, depth);
+}
+
+// One gathered element of a thin plan: its coordinate offsets and, per phase, the filter tap it
+// meets there (-1: none).
+struct ThinUse {
+  int d[3];
+  int tap[4];
+};
+
+// Lays the entries out in chunks of 16 / nph.  `groups` consecutive source channels may be taken
+// together (their count must divide the channel count) so that fewer slots of a register of
+// packed filters stay empty.  The kernel's time goes with its loads (one per entry and step,
+// plus the register of filters), and a chunk's set-up before its loop over the channel groups
+// costs about two thirds of a load per entry (measured: 25 taps, 32 filters take the same time
+// as 25 chunks x 2 steps and as 2 padded chunks x 32 steps); the cheapest grouping is taken.
+void thin_tables(Plan &pl, Tables &t, const std::vector<ThinUse> &uses, int nph, int channels, long long src_cstride, const int qs[3],
+                 long long w_kstride) {
+  const int epv = 16 / nph;
+  const int ne = (int)uses.size();
+  int groups = 1;
+  long long best = -1;
+  for (int cand : {1, 2, 4, 8, 16}) {
+    if (channels % cand != 0) continue;
+    const long long chunks = ceil_div((long long)cand * ne, epv);
+    const long long cost = chunks * (13 * epv + 20ll * (channels / cand) * (epv + 1));
+    if (best < 0 || cost < best) best = cost, groups = cand;
+  }
+  for (int ksub = 0; ksub < groups; ++ksub)
+    for (const ThinUse &u : uses) {
+      TabEntry e;
+      e.d0 = u.d[0], e.d1 = u.d[1], e.d2 = u.d[2];
+      e.off = (int)(ksub * src_cstride) + u.d[0] * qs[0] + u.d[1] * qs[1] + u.d[2] * qs[2];
+      t.tab.push_back(e);
+      for (int f = 0; f < nph; ++f) t.arow.push_back(u.tap[f] < 0 ? -1 : (int)(ksub * w_kstride) + u.tap[f]);
+    }
+  TabEntry outside{};
+  outside.d0 = outside.d1 = outside.d2 = 1 << 29;
+  while (t.tab.size() % epv != 0) {
+    t.tab.push_back(outside);
+    for (int f = 0; f < nph; ++f) t.arow.push_back(-1);
+  }
+  pl.thin = true;
+  pl.nph = nph;
+  pl.thin_chunks = (int)t.tab.size() / epv;
+  pl.thin_kgroups = channels / groups;
+  pl.thin_src_group = groups * src_cstride;
+  pl.thin_w_group = groups * w_kstride;
+}
+
 int build_fwd_plan(const Geometry &g, Plan &pl) {
   Tables t;
+  if (thin_applies(g, g.F, (long long)g.N * g.gvol, (long long)g.C * g.wvol, 1)) {
+    // up to four filters (single precision): one output position per lane
+    const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
+    std::vector<ThinUse> uses;
+    for (int t0 = 0; t0 < g.W[0]; ++t0)
+      for (int t1 = 0; t1 < g.W[1]; ++t1)
+        for (int t2 = 0; t2 < g.W[2]; ++t2)
+          uses.push_back(ThinUse{{t0 * g.D[0] - g.P[0], t1 * g.D[1] - g.P[1], t2 * g.D[2] - g.P[2]}, {(t0 * g.W[1] + t1) * g.W[2] + t2, -1, -1, -1}});
+    thin_tables(pl, t, uses, 1, g.C, g.xvol, qs, g.wvol);
+    pl.thin_w_mstride = (int)(g.C * g.wvol);
+    Phase grid{};
+    for (int k = 0; k < 3; ++k) {
+      grid.J[k] = g.G[k];
+      pl.po0[0][k] = 0;
+      pl.pJ[0][k] = g.G[k];
+    }
+    grid.npos = (int)((long long)g.N * g.gvol);
+    set_divisors(grid);
+    pl.thin_grid = grid;
+    pl.pos_blocks = (int)ceil_div(grid.npos, 256);
+    pl.bm = 4, pl.bn = 256;
+    return upload_plan(pl, t);
+  }
   pl.tap_major = g.C % gemm_bk(g.dtype) == 0 && fits_buffer_loads(g);
   // Channels that do not fill K tiles (a first layer's one or three): the same kernel, its K
   // tiles 16 rows of the gather table each -- unless the problem is tiny (few launches matter
@@ -1169,6 +1264,49 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
         set_divisors(pt.ph);
         found.push_back(pt);
       }
+
+  // ---- up to four channels (single precision): one position of the coarse grid ceil(X / stride)
+  // per lane, all of its stride phases at once
+  {
+    long long coarse_pos = g.N;
+    for (int k = 0; k < 3; ++k) coarse_pos *= (g.X[k] + g.S[k] - 1) / g.S[k];
+    if (thin_applies(g, g.C, coarse_pos, (long long)g.F * g.wvol, nphase) && (nphase == 1 || nphase == 2 || nphase == 4) &&
+        (long long)found.size() == nphase) {
+      std::stable_sort(found.begin(), found.end(), [](const PhaseTaps &a, const PhaseTaps &b) {
+        if (a.ph.o0[0] != b.ph.o0[0]) return a.ph.o0[0] < b.ph.o0[0];
+        if (a.ph.o0[1] != b.ph.o0[1]) return a.ph.o0[1] < b.ph.o0[1];
+        return a.ph.o0[2] < b.ph.o0[2];
+      });
+      std::map<std::array<int, 3>, ThinUse> seen;  // ordered by offset: neighbours along the last axis share a chunk
+      for (int f = 0; f < (int)nphase; ++f) {
+        const PhaseTaps &pt = found[f];
+        for (int k = 0; k < 3; ++k) {
+          pl.po0[f][k] = pt.ph.o0[k];
+          pl.pJ[f][k] = pt.ph.J[k];
+        }
+        for (size_t a = 0; a < pt.taps[0].size(); ++a)
+          for (size_t b = 0; b < pt.taps[1].size(); ++b)
+            for (size_t c = 0; c < pt.taps[2].size(); ++c) {
+              const std::array<int, 3> d{pt.offs[0][a], pt.offs[1][b], pt.offs[2][c]};
+              auto it = seen.find(d);
+              if (it == seen.end()) it = seen.emplace(d, ThinUse{{d[0], d[1], d[2]}, {-1, -1, -1, -1}}).first;
+              it->second.tap[f] = (pt.taps[0][a] * g.W[1] + pt.taps[1][b]) * g.W[2] + pt.taps[2][c];
+            }
+      }
+      std::vector<ThinUse> uses;
+      for (const auto &kv : seen) uses.push_back(kv.second);
+      thin_tables(pl, t, uses, (int)nphase, g.F, g.gvol, gs, (long long)g.C * g.wvol);
+      pl.thin_w_mstride = (int)g.wvol;
+      Phase coarse{};
+      for (int k = 0; k < 3; ++k) coarse.J[k] = (g.X[k] + g.S[k] - 1) / g.S[k];
+      coarse.npos = (int)coarse_pos;
+      set_divisors(coarse);
+      pl.thin_grid = coarse;
+      pl.pos_blocks = (int)ceil_div(coarse.npos, 256);
+      pl.bm = 4, pl.bn = 256;
+      return upload_plan(pl, t);
+    }
+  }
 
   // ---- few channels, unit strides, a 3-tap "same" last axis (float): the rows of the GEMM are
   // (channel, tap of the last axis), three times as many as there are channels, and the K tiles
@@ -1533,6 +1671,7 @@ int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
   std::string key(reinterpret_cast<const char *>(d), sizeof *d);
   key.push_back((char)op);
   key.push_back(tiny_plans_enabled() ? 't' : 'T');
+  key.push_back(thin_on() ? 'n' : 'N');
   auto it = plans().find(key);
   if (it == plans().end()) {
     if (plans().size() >= 256) {
@@ -1547,7 +1686,7 @@ int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
     static const bool trace = getenv("MYGRAD_HIP_TRACE") != nullptr;
     if (trace)
       fprintf(stderr, "[mygrad_hip] %s plan: %s tile %dx%d, %d phase(s) (%d fused per tile), %d position blocks x %d row tiles, %d whole tiles + tail split %d, %d block(s) per unit, K splits %d (chunk %d)\n",
-              op == OP_FWD ? "fwd" : op == OP_DGRAD ? "dgrad" : "wgrad", pl.tap_major ? "tap-major" : "table-driven", pl.bm,
+              op == OP_FWD ? "fwd" : op == OP_DGRAD ? "dgrad" : "wgrad", pl.thin ? "one position per lane" : pl.tap_major ? "tap-major" : "table-driven", pl.bm,
               pl.bn, pl.nphases, pl.nph, pl.pos_blocks, pl.m_tiles, pl.full_tiles, pl.tail_split, pl.blocks_per_cu, pl.splits, pl.kchunk);
     it = plans().emplace(key, pl).first;
   }
@@ -1740,8 +1879,66 @@ int pack_filters(const Geometry &g, const void *w, int mode, void **packed, size
   return MG_OK;
 }
 
+// The 4x4x1 MFMA kernel for a plan with at most four rows: packs the filters into its
+// register-sized groups, then one position per lane.
+int run_thin(const Plan &pl, ThinParams &tp, const void *w, int tag) {
+  void *packed = nullptr;
+  const size_t a_bytes = (size_t)pl.thin_chunks * pl.thin_kgroups * 256;
+  if (int rc = workspace(a_bytes, &packed)) return rc;
+  {
+    ScopedTiming timed(TAG_PACK_FILTERS);
+    if (int rc = launch_thin_pack(static_cast<const float *>(w), static_cast<float *>(packed), pl.arow, pl.thin_chunks, pl.thin_kgroups,
+                                  pl.thin_w_group, pl.thin_w_mstride, tp.M, runtime().stream))
+      return rc;
+  }
+  tp.A = static_cast<const float *>(packed);
+  tp.a_bytes = (unsigned)a_bytes;
+  tp.tab = pl.tab;
+  tp.chunks = pl.thin_chunks;
+  tp.kgroups = pl.thin_kgroups;
+  tp.group_bytes = (unsigned)(pl.thin_src_group * 4);
+  tp.npos = pl.thin_grid.npos;
+  tp.by_jvol = pl.thin_grid.by_jvol, tp.by_j12 = pl.thin_grid.by_j12, tp.by_j2 = pl.thin_grid.by_j2;
+  tp.nph = pl.nph;
+  for (int k = 0; k < 3; ++k) tp.J[k] = pl.thin_grid.J[k];
+  for (int f = 0; f < pl.nph; ++f)
+    for (int k = 0; k < 3; ++k) {
+      tp.po0[f][k] = pl.po0[f][k];
+      tp.pJ[f][k] = pl.pJ[f][k];
+    }
+  // phases 2q and 2q + 1 side by side along the last axis, every pair 8-byte aligned in dst
+  bool pairs = pl.nph > 1 && tp.oj[2] == 2 && tp.os[2] == 1 && tp.os[1] % 2 == 0 && tp.os[0] % 2 == 0 && tp.dst_mstride % 2 == 0 &&
+               tp.dst_nstride % 2 == 0 && reinterpret_cast<uintptr_t>(tp.dst) % 8 == 0;
+  for (int f = 0; pairs && f + 1 < pl.nph; f += 2)
+    pairs = pl.po0[f][2] == 0 && pl.po0[f + 1][2] == 1 && pl.po0[f][0] == pl.po0[f + 1][0] && pl.po0[f][1] == pl.po0[f + 1][1] &&
+            pl.pJ[f][0] == pl.pJ[f + 1][0] && pl.pJ[f][1] == pl.pJ[f + 1][1] && pl.pJ[f][2] == pl.pJ[f + 1][2];
+  tp.pair_store = pairs ? 1 : 0;
+  ScopedTiming timed(tag);
+  return launch_thin_gemm(tp, runtime().stream);
+}
+
 template <typename T>
 int conv_fwd_impl(const Geometry &g, const Plan &pl, const void *x, const void *w, void *out) {
+  if (pl.thin) {
+    ThinParams tp{};
+    tp.src = static_cast<const float *>(x);
+    tp.dst = static_cast<float *>(out);
+    tp.M = g.F;
+    const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
+    const int os[3] = {g.G[1] * g.G[2], g.G[2], 1};
+    for (int k = 0; k < 3; ++k) {
+      tp.Q[k] = g.X[k];
+      tp.sj[k] = g.S[k];
+      tp.qs[k] = qs[k];
+      tp.oj[k] = 1;
+      tp.os[k] = os[k];
+    }
+    tp.dst_mstride = (int)g.gvol;
+    tp.src_nstride = (long long)g.C * g.xvol;
+    tp.dst_nstride = (long long)g.F * g.gvol;
+    tp.src_bytes = (unsigned)((size_t)g.N * g.C * g.xvol * 4);
+    return run_thin(pl, tp, w, TAG_CONV_FWD);
+  }
   void *packed = nullptr;
   void *partial = nullptr;
   if (!pl.tap_major) {
@@ -1777,6 +1974,26 @@ int conv_fwd_impl(const Geometry &g, const Plan &pl, const void *x, const void *
 
 template <typename T>
 int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const void *w, void *dx) {
+  if (pl.thin) {
+    ThinParams tp{};
+    tp.src = static_cast<const float *>(grad);
+    tp.dst = static_cast<float *>(dx);
+    tp.M = g.C;
+    const int qs[3] = {g.G[1] * g.G[2], g.G[2], 1};
+    const int os[3] = {g.X[1] * g.X[2], g.X[2], 1};
+    for (int k = 0; k < 3; ++k) {
+      tp.Q[k] = g.G[k];
+      tp.sj[k] = 1;
+      tp.qs[k] = qs[k];
+      tp.oj[k] = g.S[k];
+      tp.os[k] = os[k];
+    }
+    tp.dst_mstride = (int)g.xvol;
+    tp.src_nstride = (long long)g.F * g.gvol;
+    tp.dst_nstride = (long long)g.C * g.xvol;
+    tp.src_bytes = (unsigned)((size_t)g.N * g.F * g.gvol * 4);
+    return run_thin(pl, tp, w, TAG_CONV_DGRAD);
+  }
   void *packed = nullptr;
   void *partial = nullptr;
   if (!pl.tap_major) {

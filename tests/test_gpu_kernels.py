@@ -4,6 +4,8 @@ Bars: pooling bit-exact (raw bit patterns); convolution
 max|gpu - ref| / max|ref| <= 1e-10 in float64 and <= 2e-4 in float32.
 """
 
+import os
+
 import numpy as np
 import pytest
 
@@ -487,6 +489,87 @@ def test_conv_with_channel_or_filter_counts_that_fill_no_k_tile(abi, dtype, case
     gi = rng.integers(-2, 3, want.shape).astype(dtype)
     assert np.array_equal(abi.conv_dgrad(gi, x_shape, wi, s, p, d), direct.conv_backward_x(gi, x_shape, wi, s, p, d).astype(dtype))
     assert np.array_equal(abi.conv_wgrad(gi, xi, w_shape, s, p, d), direct.conv_backward_w(gi, xi, w_shape, s, p, d).astype(dtype))
+
+
+# Up to four channels in single precision, on enough positions to fill the device: the data
+# gradient runs one position of the coarse grid ceil(X / stride) per lane on the 4x4x1 MFMA, all
+# stride phases of the position at once (1, 2 or 4 of them).  Between them the cases cover every
+# phase count, entries that fill their chunks of 16 / phases and ones that need padding or
+# several channels per chunk, odd extents (phases with different numbers of positions, no paired
+# stores), dilation, and one to three convolved axes.  float64 runs the other kernels.
+THIN_ROW_CASES = [
+    ((16, 3, 130, 130), (16, 3, 7, 7), (2, 2), (3, 3), (1, 1)),     # the stem's geometry (even extent, flooring placement): 4 phases, 16 entries
+    ((16, 3, 131, 131), (8, 3, 7, 7), (2, 2), (3, 3), (1, 1)),      # odd extents: the phases differ in size
+    ((64, 3, 64, 64), (32, 3, 5, 5), (1, 1), (2, 2), (1, 1)),       # one phase, 25 entries, two filters per chunk step
+    ((64, 1, 128, 128), (10, 1, 3, 3), (1, 1), (1, 1), (1, 1)),     # one channel; 9 entries x 2 filters, padded
+    ((16, 4, 96, 97), (16, 4, 3, 4), (1, 2), (1, 1), (1, 1)),       # two phases along the last axis
+    ((16, 2, 140, 70), (24, 2, 5, 3), (2, 1), (2, 1), (1, 1)),      # two phases along the first axis: no paired stores
+    ((64, 3, 64, 64), (32, 3, 3, 3), (1, 1), (2, 2), (2, 2)),       # dilation 2; 9 entries x 16 filters fill their chunks
+    ((4, 3, 18, 64, 64), (12, 3, 3, 3, 3), (1, 2, 2), (1, 1, 1), (1, 1, 1)),  # three axes, four phases
+    ((64, 2, 2100), (48, 2, 9), (2,), (4,), (1,)),                  # one axis, two phases
+    ((64, 3, 128, 128), (16, 3, 2, 2), (2, 2), (0, 0), (1, 1)),     # window = stride: every phase has one tap
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("case", range(len(THIN_ROW_CASES)))
+def test_data_gradient_with_up_to_four_channels(abi, dtype, case):
+    x_shape, w_shape, s, p, d = THIN_ROW_CASES[case]
+    rng = np.random.default_rng(2300 + case)
+    tol = TOL[np.dtype(dtype)]
+    w = (rng.standard_normal(w_shape) / np.sqrt(np.prod(w_shape[1:]))).astype(dtype)
+    grid = direct.conv_forward(np.zeros(x_shape, dtype=dtype), w, s, p, d).shape
+    g = rng.standard_normal(grid).astype(dtype)
+    got = abi.conv_dgrad(g, x_shape, w, s, p, d)
+    assert rel_err(got, direct.conv_backward_x(g, x_shape, w, s, p, d)) <= tol
+    assert np.array_equal(got, abi.conv_dgrad(g, x_shape, w, s, p, d))
+    # exact: small integers, every (filter, channel, tap) weighted differently
+    gi = rng.integers(-2, 3, grid).astype(dtype)
+    wi = (np.arange(np.prod(w_shape)).reshape(w_shape) % 11 - 5).astype(dtype)
+    assert np.array_equal(abi.conv_dgrad(gi, x_shape, wi, s, p, d), direct.conv_backward_x(gi, x_shape, wi, s, p, d).astype(dtype))
+    if dtype == np.float32:
+        # MYGRAD_HIP_THIN=0 plans the same problem on the 16-row tiles: same bar
+        os.environ["MYGRAD_HIP_THIN"] = "0"
+        try:
+            other = abi.conv_dgrad(g, x_shape, w, s, p, d)
+        finally:
+            del os.environ["MYGRAD_HIP_THIN"]
+        assert rel_err(other, direct.conv_backward_x(g, x_shape, w, s, p, d)) <= tol
+
+
+# Up to four filters in single precision (a layer that ends in one map or in the three colours
+# of an image): the forward pass on the same kernel, one output position per lane.
+THIN_FILTER_CASES = [
+    ((64, 16, 64, 64), (3, 16, 3, 3), (1, 1), (1, 1), (1, 1)),
+    ((256, 64, 64, 64), (1, 64, 1, 1), (1, 1), (0, 0), (1, 1)),     # one tap: sixteen channels per chunk
+    ((112, 8, 97, 97), (4, 8, 7, 7), (2, 2), (3, 3), (1, 1)),       # strided reads
+    ((4, 6, 20, 64, 64), (2, 6, 3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
+    ((128, 48, 2048), (3, 48, 5), (1,), (4,), (2,)),
+    ((64, 9, 64, 64), (4, 9, 5, 5), (1, 1), (2, 2), (1, 1)),        # 25 taps, 9 channels: one channel per group, chunks padded
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("case", range(len(THIN_FILTER_CASES)))
+def test_forward_pass_with_up_to_four_filters(abi, dtype, case):
+    x_shape, w_shape, s, p, d = THIN_FILTER_CASES[case]
+    rng = np.random.default_rng(2400 + case)
+    tol = TOL[np.dtype(dtype)]
+    x = rng.standard_normal(x_shape).astype(dtype)
+    w = (rng.standard_normal(w_shape) / np.sqrt(np.prod(w_shape[1:]))).astype(dtype)
+    got = abi.conv_fwd(x, w, s, p, d)
+    assert rel_err(got, direct.conv_forward(x, w, s, p, d)) <= tol
+    assert np.array_equal(got, abi.conv_fwd(x, w, s, p, d))
+    xi = rng.integers(-2, 3, x_shape).astype(dtype)
+    wi = (np.arange(np.prod(w_shape)).reshape(w_shape) % 11 - 5).astype(dtype)
+    assert np.array_equal(abi.conv_fwd(xi, wi, s, p, d), direct.conv_forward(xi, wi, s, p, d).astype(dtype))
+    if dtype == np.float32:
+        os.environ["MYGRAD_HIP_THIN"] = "0"  # the same problem on the 16-row tiles: same bar
+        try:
+            other = abi.conv_fwd(x, w, s, p, d)
+        finally:
+            del os.environ["MYGRAD_HIP_THIN"]
+        assert rel_err(other, direct.conv_forward(x, w, s, p, d)) <= tol
 
 
 # Shapes picked so that, between them, every tile shape and code path of the tap-major
