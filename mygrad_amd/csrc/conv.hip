@@ -592,8 +592,9 @@ struct Plan {
   int kcut[4] = {0, 0, 0, 0};
   int po0[4][3] = {};
   int pJ[4][3] = {};
-  // at most four rows, single precision: one position per lane on the 4x4x1 MFMA (see ThinParams)
+  // few rows, single precision: one position per lane on the 4x4x1 MFMA (see ThinParams)
   bool thin = false;
+  int thin_rg = 1;  // groups of four rows
   int thin_chunks = 0, thin_kgroups = 0;
   long long thin_src_group = 0, thin_w_group = 0;  // elements of src / of the filter bank between consecutive groups
   int thin_w_mstride = 0;
@@ -1018,20 +1019,28 @@ bool table_rows_on() {
 }
 
 
-// ---- at most four rows (channels of a data gradient, filters of a forward pass), single
-// precision, enough positions to fill the device: the 4x4x1 MFMA kernel, one position per lane.
+// ---- few rows (channels of a data gradient, filters of a forward pass), single precision,
+// enough positions to fill the device: the 4x4x1 MFMA kernel, one position per lane.
 // MYGRAD_HIP_THIN=0 switches it off (read whenever a plan is built, and part of the plan's key).
 bool thin_on() {
   const char *flag = getenv("MYGRAD_HIP_THIN");
   return !(flag && flag[0] == '0');
 }
 
-// Positions: one wave per SIMD (65536) with several stride phases, where the 16-row tiles take two
-// to three times as long; four waves per SIMD with one phase, where a gathered element feeds a
-// single MFMA and the kernel is bound by its loads (at one wave per SIMD it loses a quarter,
-// at sixteen it is ahead by one).
+// Groups of four rows the kernel would run `rows` as (a power of two), 0 if it has no such shape.
+int thin_row_groups(int rows, int nph) {
+  int rg = 1;
+  while (rg * 4 < rows) rg *= 2;
+  return (nph == 1 || nph == 2 || nph == 4) && thin_gemm_has(nph, rg) ? rg : 0;
+}
+
+// Positions: one wave per SIMD (65536) where a gathered element feeds several MFMAs (stride
+// phases, row groups) -- the 16-row tiles take two to three times as long there; four waves per
+// SIMD where it feeds a single one and the kernel is bound by its loads (at one wave per SIMD
+// it loses a quarter, at sixteen it is ahead by one).
 bool thin_applies(const Geometry &g, int rows, long long positions, long long depth, long long nph) {
-  return thin_on() && g.dtype == MG_F32 && rows <= 4 && fits_buffer_loads(g) && positions >= (nph == 1 ? 4 : 1) * 65536 &&
+  const int rg = thin_row_groups(rows, (int)nph);
+  return thin_on() && g.dtype == MG_F32 && rg != 0 && fits_buffer_loads(g) && positions >= (nph * rg == 1 ? 4 : 1) * 65536 &&
          !tiny_table(g, rows, depth);
 }
 
@@ -1048,9 +1057,10 @@ struct ThinUse {
 // plus the register of filters), and a chunk's set-up before its loop over the channel groups
 // costs about two thirds of a load per entry (measured: 25 taps, 32 filters take the same time
 // as 25 chunks x 2 steps and as 2 padded chunks x 32 steps); the cheapest grouping is taken.
-void thin_tables(Plan &pl, Tables &t, const std::vector<ThinUse> &uses, int nph, int channels, long long src_cstride, const int qs[3],
-                 long long w_kstride) {
-  const int epv = 16 / nph;
+void thin_tables(Plan &pl, Tables &t, const std::vector<ThinUse> &uses, int nph, int rows, int channels, long long src_cstride,
+                 const int qs[3], long long w_kstride, long long w_mstride) {
+  const int rg = thin_row_groups(rows, nph);
+  const int epv = 16 / (nph * rg);
   const int ne = (int)uses.size();
   int groups = 1;
   long long best = -1;
@@ -1060,40 +1070,50 @@ void thin_tables(Plan &pl, Tables &t, const std::vector<ThinUse> &uses, int nph,
     const long long cost = chunks * (13 * epv + 20ll * (channels / cand) * (epv + 1));
     if (best < 0 || cost < best) best = cost, groups = cand;
   }
+  // a slot of the packed filters is (entry within its chunk, phase, row group): the offset of the
+  // group's first row in the filter bank, -1 where the phase has no tap for the entry or the group
+  // lies beyond the rows
+  auto push_slots = [&](const ThinUse *u, int ksub) {
+    for (int f = 0; f < nph; ++f)
+      for (int r = 0; r < rg; ++r)
+        t.arow.push_back(u == nullptr || u->tap[f] < 0 || 4 * r >= rows ? -1 : (int)(ksub * w_kstride + u->tap[f] + 4 * r * w_mstride));
+  };
   for (int ksub = 0; ksub < groups; ++ksub)
     for (const ThinUse &u : uses) {
       TabEntry e;
       e.d0 = u.d[0], e.d1 = u.d[1], e.d2 = u.d[2];
       e.off = (int)(ksub * src_cstride) + u.d[0] * qs[0] + u.d[1] * qs[1] + u.d[2] * qs[2];
       t.tab.push_back(e);
-      for (int f = 0; f < nph; ++f) t.arow.push_back(u.tap[f] < 0 ? -1 : (int)(ksub * w_kstride) + u.tap[f]);
+      push_slots(&u, ksub);
     }
   TabEntry outside{};
   outside.d0 = outside.d1 = outside.d2 = 1 << 29;
   while (t.tab.size() % epv != 0) {
     t.tab.push_back(outside);
-    for (int f = 0; f < nph; ++f) t.arow.push_back(-1);
+    push_slots(nullptr, 0);
   }
   pl.thin = true;
   pl.nph = nph;
+  pl.thin_rg = rg;
   pl.thin_chunks = (int)t.tab.size() / epv;
   pl.thin_kgroups = channels / groups;
   pl.thin_src_group = groups * src_cstride;
   pl.thin_w_group = groups * w_kstride;
+  pl.thin_w_mstride = (int)w_mstride;
 }
 
 int build_fwd_plan(const Geometry &g, Plan &pl) {
   Tables t;
-  if (thin_applies(g, g.F, (long long)g.N * g.gvol, (long long)g.C * g.wvol, 1)) {
-    // up to four filters (single precision): one output position per lane
+  if ((g.F <= 4 || (g.F <= 64 && g.C % gemm_bk(g.dtype) != 0)) && thin_applies(g, g.F, (long long)g.N * g.gvol, (long long)g.C * g.wvol, 1)) {
+    // up to four filters, or a first layer (channels that fill no K tile, up to 64 filters), in
+    // single precision: one output position per lane
     const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
     std::vector<ThinUse> uses;
     for (int t0 = 0; t0 < g.W[0]; ++t0)
       for (int t1 = 0; t1 < g.W[1]; ++t1)
         for (int t2 = 0; t2 < g.W[2]; ++t2)
           uses.push_back(ThinUse{{t0 * g.D[0] - g.P[0], t1 * g.D[1] - g.P[1], t2 * g.D[2] - g.P[2]}, {(t0 * g.W[1] + t1) * g.W[2] + t2, -1, -1, -1}});
-    thin_tables(pl, t, uses, 1, g.C, g.xvol, qs, g.wvol);
-    pl.thin_w_mstride = (int)(g.C * g.wvol);
+    thin_tables(pl, t, uses, 1, g.F, g.C, g.xvol, qs, g.wvol, (long long)g.C * g.wvol);
     Phase grid{};
     for (int k = 0; k < 3; ++k) {
       grid.J[k] = g.G[k];
@@ -1270,8 +1290,7 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
   {
     long long coarse_pos = g.N;
     for (int k = 0; k < 3; ++k) coarse_pos *= (g.X[k] + g.S[k] - 1) / g.S[k];
-    if (thin_applies(g, g.C, coarse_pos, (long long)g.F * g.wvol, nphase) && (nphase == 1 || nphase == 2 || nphase == 4) &&
-        (long long)found.size() == nphase) {
+    if (g.C <= 4 && thin_applies(g, g.C, coarse_pos, (long long)g.F * g.wvol, nphase) && (long long)found.size() == nphase) {
       std::stable_sort(found.begin(), found.end(), [](const PhaseTaps &a, const PhaseTaps &b) {
         if (a.ph.o0[0] != b.ph.o0[0]) return a.ph.o0[0] < b.ph.o0[0];
         if (a.ph.o0[1] != b.ph.o0[1]) return a.ph.o0[1] < b.ph.o0[1];
@@ -1295,8 +1314,7 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
       }
       std::vector<ThinUse> uses;
       for (const auto &kv : seen) uses.push_back(kv.second);
-      thin_tables(pl, t, uses, (int)nphase, g.F, g.gvol, gs, (long long)g.C * g.wvol);
-      pl.thin_w_mstride = (int)g.wvol;
+      thin_tables(pl, t, uses, (int)nphase, g.C, g.F, g.gvol, gs, (long long)g.C * g.wvol, g.wvol);
       Phase coarse{};
       for (int k = 0; k < 3; ++k) coarse.J[k] = (g.X[k] + g.S[k] - 1) / g.S[k];
       coarse.npos = (int)coarse_pos;
@@ -1879,7 +1897,7 @@ int pack_filters(const Geometry &g, const void *w, int mode, void **packed, size
   return MG_OK;
 }
 
-// The 4x4x1 MFMA kernel for a plan with at most four rows: packs the filters into its
+// The 4x4x1 MFMA kernel for a plan with few rows: packs the filters into its
 // register-sized groups, then one position per lane.
 int run_thin(const Plan &pl, ThinParams &tp, const void *w, int tag) {
   void *packed = nullptr;
@@ -1888,7 +1906,7 @@ int run_thin(const Plan &pl, ThinParams &tp, const void *w, int tag) {
   {
     ScopedTiming timed(TAG_PACK_FILTERS);
     if (int rc = launch_thin_pack(static_cast<const float *>(w), static_cast<float *>(packed), pl.arow, pl.thin_chunks, pl.thin_kgroups,
-                                  pl.thin_w_group, pl.thin_w_mstride, tp.M, runtime().stream))
+                                  pl.thin_w_group, pl.thin_w_mstride, tp.M, pl.thin_rg, runtime().stream))
       return rc;
   }
   tp.A = static_cast<const float *>(packed);
@@ -1900,6 +1918,7 @@ int run_thin(const Plan &pl, ThinParams &tp, const void *w, int tag) {
   tp.npos = pl.thin_grid.npos;
   tp.by_jvol = pl.thin_grid.by_jvol, tp.by_j12 = pl.thin_grid.by_j12, tp.by_j2 = pl.thin_grid.by_j2;
   tp.nph = pl.nph;
+  tp.rg = pl.thin_rg;
   for (int k = 0; k < 3; ++k) tp.J[k] = pl.thin_grid.J[k];
   for (int f = 0; f < pl.nph; ++f)
     for (int k = 0; k < 3; ++k) {

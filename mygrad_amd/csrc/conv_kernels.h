@@ -124,20 +124,20 @@ struct GemmParams {
   int fold_row;         // 0: not folded; else the length of a row of positions (a power of two, 4 .. 64)
 };
 
-// Gather-GEMM with at most four rows (the data gradient of a layer with up to four channels,
-// the forward pass of one with up to four filters), one position per lane:
+// Gather-GEMM with one position per lane, for few rows (the data gradient of a layer with a
+// handful of channels, the forward pass of one with a handful of filters or of a first layer):
 //   dst[n, m, pos of phase f] = sum over groups kg, entries e of  A(kg, e, f, m) * src[n, base(pos) + kg * group_stride + off_e]
 // `tab` holds the entries in chunks of 16 / nph: entry e adds `off` elements to the
 // position's base offset and d[k] to its source coordinate on axis k, which must land in
 // [0, Q[k]) (else the element is a padding zero).  The packed operand holds, for chunk q and
-// group kg, 64 values [entry within chunk][phase][m]: zero where the entry feeds no tap of that
-// phase, or m is beyond M.
+// group kg, 64 values [entry within chunk][phase][row group][row within group]: zero where the
+// entry feeds no tap of that phase, or the row is beyond M.
 struct ThinParams {
   const float *A;
   const float *src;
   float *dst;
   const TabEntry *tab;
-  int chunks;           // chunks of 16 / nph entries
+  int chunks;           // chunks of 16 / (nph * rg) entries
   int kgroups;          // steps of the inner loop
   unsigned group_bytes; // bytes of src between consecutive groups
   unsigned a_bytes, src_bytes;
@@ -153,6 +153,7 @@ struct ThinParams {
   int dst_mstride;
   long long src_nstride, dst_nstride;
   int nph;          // 1, 2 or 4 stride phases per position
+  int rg;           // groups of four rows (M <= 4 * rg), nph * rg <= 16
   int po0[4][3];    // destination coordinate of position (0,0,0) in phase f
   int pJ[4][3];     // positions j_k < pJ[f][k] exist in phase f
   int pair_store;   // phases 2q and 2q+1 are neighbours along the last axis of dst, stored as one 8-byte piece
@@ -160,8 +161,9 @@ struct ThinParams {
 
 // conv_thin.hip
 int launch_thin_pack(const float *w, float *packed, const int *arow, int chunks, int kgroups, long long group_stride, int m_stride, int M,
-                     hipStream_t s);
+                     int rg, hipStream_t s);
 int launch_thin_gemm(const ThinParams &p, hipStream_t s);
+bool thin_gemm_has(int nph, int rg);
 
 // Filter gradient:  out[split][f][col] = sum over the split's positions (n, g) of
 //   grad[n, f, g] * x[n, column col at g]

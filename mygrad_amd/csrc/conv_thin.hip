@@ -1,8 +1,10 @@
-// Gather-GEMM for convolutions with at most four rows: the data gradient of a layer with up
-// to four channels (the first layer of an image network), the forward pass of a layer with
-// up to four filters.  Single precision.
+// Gather-GEMM with one position per lane, for convolutions whose rows come in few groups of
+// four: the data gradient of a layer with a handful of channels (the first layer of an image
+// network), the forward pass of a layer with a handful of filters, and the forward pass of a
+// first layer itself (up to 64 filters over one or three channels).  Single precision.
 //
-// A 16-row MFMA tile would carry 3 or 4 live rows.  v_mfma_f32_4x4x1_16b_f32 multiplies
+// A 16-row MFMA tile would carry 3 or 4 live rows of such a data gradient, and K tiles of 16
+// suit 3 channels badly.  v_mfma_f32_4x4x1_16b_f32 multiplies
 // sixteen independent 4x1 by 1x4 blocks: lane l supplies B[l] and receives D[i][l], i = 0..3,
 // in its four accumulator registers; with the A operand broadcast from one block (cbsz = 4,
 // abid = the block), D[i][l] += A[4 * abid + i] * B[l].  So a lane IS a position: it gathers its
@@ -11,7 +13,10 @@
 // sixteen MFMAs.  With a stride, a lane owns one position of the coarse grid ceil(X / stride)
 // and all of its stride phases, one accumulator each: the phases read the same neighbourhood
 // of grad, so each gathered element feeds up to nph MFMAs (with weights that are zero where
-// the phase has no tap for it).
+// the phase has no tap for it).  More than four rows are RG groups of four, one accumulator
+// each as well: the sixteen blocks of a register of filters are (entry, phase, row group), and a
+// gathered element feeds NPH * RG MFMAs.  With 64 filters a register holds one (channel, tap)
+// of all of them, and the forward pass of a first layer does sixteen MFMAs per two loads.
 #include "conv_kernels.h"
 #include "internal.h"
 
@@ -33,28 +38,35 @@ __device__ __forceinline__ float buffer_load(__amdgpu_buffer_rsrc_t rsrc, unsign
   return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)lane_bytes, (int)uniform_bytes, 0));
 }
 
-// acc[ph] += A[block I * NPH + ph] * v for every phase; the block index is an immediate of the instruction
-template <int NPH, int I>
-__device__ __forceinline__ void feed(f32x4 (&acc)[NPH], float a, float v) {
-  acc[0] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, v, acc[0], 4, I * NPH, 0);
-  if constexpr (NPH >= 2) acc[1] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, v, acc[1], 4, I * NPH + 1, 0);
-  if constexpr (NPH >= 4) {
-    acc[2] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, v, acc[2], 4, I * NPH + 2, 0);
-    acc[3] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, v, acc[3], 4, I * NPH + 3, 0);
+// acc[j] += A[block I * NACC + j] * v for every accumulator; the block index is an immediate of the instruction
+template <int NACC, int I, int J = 0>
+__device__ __forceinline__ void feed(f32x4 (&acc)[NACC], float a, float v) {
+  if constexpr (J < NACC) {
+    if constexpr (NACC >= 8) {
+      // Many accumulators: written as the instruction itself, accumulating in place.  (Through the
+      // builtin the compiler gives the unrolled steps' results new registers and moves all of
+      // them back at the end of every round of the loop, 128 moves for 16 MFMAs.)  An accumulator
+      // is used again eight or more MFMAs later, long after its result has been written.
+      asm volatile("v_mfma_f32_4x4x1_16b_f32 %0, %1, %2, %0 cbsz:4 abid:%3" : "+a"(acc[J]) : "v"(a), "v"(v), "n"(I * NACC + J));
+    } else {
+      acc[J] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, v, acc[J], 4, I * NACC + J, 0);
+    }
+    feed<NACC, I, J + 1>(acc, a, v);
   }
 }
 
-template <int NPH, int EPV, int I = 0>
-__device__ __forceinline__ void feed_all(f32x4 (&acc)[NPH], float a, const float (&v)[EPV]) {
+template <int NACC, int EPV, int I = 0>
+__device__ __forceinline__ void feed_all(f32x4 (&acc)[NACC], float a, const float (&v)[EPV]) {
   if constexpr (I < EPV) {
-    feed<NPH, I>(acc, a, v[I]);
-    feed_all<NPH, EPV, I + 1>(acc, a, v);
+    feed<NACC, I>(acc, a, v[I]);
+    feed_all<NACC, EPV, I + 1>(acc, a, v);
   }
 }
 
-template <int NPH>
+template <int NPH, int RG>
 __global__ void __launch_bounds__(256) thin_gemm_kernel(ThinParams p) {
-  constexpr int EPV = 16 / NPH;  // entries per register of packed filters
+  constexpr int NACC = NPH * RG;   // accumulators: (stride phase, group of four rows)
+  constexpr int EPV = 16 / NACC;   // entries per register of packed filters
   const int lane = threadIdx.x & 63;
   const int pos = blockIdx.x * 256 + threadIdx.x;
   const bool active = pos < p.npos;
@@ -73,41 +85,84 @@ __global__ void __launch_bounds__(256) thin_gemm_kernel(ThinParams p) {
   const __amdgpu_buffer_rsrc_t src_buf = buffer_of(p.src, p.src_bytes);
   const int4v MG_CONSTANT *tab = (const int4v MG_CONSTANT *)p.tab;
 
-  f32x4 acc[NPH];
+  f32x4 acc[NACC];
 #pragma unroll
-  for (int ph = 0; ph < NPH; ++ph) acc[ph] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < NACC; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // One step = one chunk of entries under one group of channels: a register of filters, EPV
+  // gathered elements, 16 MFMAs.  The steps of all chunks form one pipeline: two sets of
+  // registers take turns, the loads of one step are in flight while the other feeds the MFMAs,
+  // also across the change from one chunk to the next (where the entries' offsets are renewed).
   const unsigned a_lane = (unsigned)lane * 4u;
-  for (int q = 0; q < p.chunks; ++q) {
-    unsigned at[EPV];
+  unsigned at[EPV];
+  // The rows of the table come through the scalar data path; with few entries per chunk the
+  // chunks change often, and the rows of the next chunk are asked for a chunk ahead so that
+  // nobody waits for them.
+  constexpr bool AHEAD = EPV <= 4;
+  int4v rows[EPV];
+  auto ask_rows = [&](int q) {
+#pragma unroll
+    for (int i = 0; i < EPV; ++i) rows[i] = tab[q * EPV + i];  // off, d0, d1, d2: the same for every lane
+  };
+  auto enter_chunk = [&](int q) {
+    if constexpr (!AHEAD) ask_rows(q);
 #pragma unroll
     for (int i = 0; i < EPV; ++i) {
-      const int4v e = tab[q * EPV + i];  // off, d0, d1, d2: the same for every lane
-      const bool ok = active && (unsigned)(c0 + e.y) < (unsigned)p.Q[0] && (unsigned)(c1 + e.z) < (unsigned)p.Q[1] &&
-                      (unsigned)(c2 + e.w) < (unsigned)p.Q[2];
+      const int4v e = rows[i];
+      const bool ok = active & ((unsigned)(c0 + e.y) < (unsigned)p.Q[0]) & ((unsigned)(c1 + e.z) < (unsigned)p.Q[1]) &
+                      ((unsigned)(c2 + e.w) < (unsigned)p.Q[2]);  // no branches: the rows are the same for every lane
       at[i] = ok ? src_at + (unsigned)(e.x * 4) : kOutside;
     }
-    // two sets of registers take turns: the loads of one group are in flight while the other feeds the MFMAs
-    const unsigned a_base = (unsigned)q * (unsigned)p.kgroups * 256u;
-    float a0, a1, v0[EPV], v1[EPV];
-    auto fetch = [&](int kg, float &a, float (&v)[EPV]) {
-      a = buffer_load(a_buf, a_lane, a_base + (unsigned)kg * 256u);
-      const unsigned s_uni = (unsigned)kg * p.group_bytes;
+    if constexpr (AHEAD) ask_rows(min(q + 1, p.chunks - 1));
+  };
+  if constexpr (AHEAD) ask_rows(0);
+  int q = 0, kg = 0;
+  unsigned a_uni = 0u, s_uni = 0u;
+  auto fetch = [&](float &a, float (&v)[EPV]) {
+    a = buffer_load(a_buf, a_lane, a_uni);
 #pragma unroll
-      for (int i = 0; i < EPV; ++i) v[i] = buffer_load(src_buf, at[i], s_uni);
-      __builtin_amdgcn_sched_barrier(0);  // all of a group's loads are issued before the MFMAs that follow in the source
-    };
-    fetch(0, a0, v0);
-    const int last = p.kgroups - 1;
-    for (int kg = 0; kg < last; kg += 2) {
-      fetch(kg + 1, a1, v1);
-      feed_all<NPH, EPV>(acc, a0, v0);
-      fetch(min(kg + 2, last), a0, v0);  // past the end: the last group once more, not fed
-      feed_all<NPH, EPV>(acc, a1, v1);
+    for (int i = 0; i < EPV; ++i) v[i] = buffer_load(src_buf, at[i], s_uni);
+    __builtin_amdgcn_sched_barrier(0);  // all of a step's loads are issued before the MFMAs that follow in the source
+  };
+  // moves on to the next step; past the last one every load lies outside its buffer and reads as
+  // zero (the packed filters end there, the entries' offsets are set outside)
+  auto advance = [&]() {
+    a_uni += 256u;
+    s_uni += p.group_bytes;
+    if (++kg == p.kgroups) {
+      kg = 0;
+      s_uni = 0u;
+      if (++q < p.chunks) {
+        enter_chunk(q);
+      } else {
+#pragma unroll
+        for (int i = 0; i < EPV; ++i) at[i] = kOutside;
+      }
     }
-    if (p.kgroups & 1) feed_all<NPH, EPV>(acc, a0, v0);
+  };
+  // DEPTH sets of registers take turns; the loads of DEPTH - 1 steps are in flight while one step
+  // feeds the MFMAs.  A step with few entries is short (16 MFMAs whatever their number), and its
+  // loads would not be back in time with one step of lead.
+  constexpr int DEPTH = EPV <= 2 ? 4 : 2;
+  float a[DEPTH], v[DEPTH][EPV];
+  enter_chunk(0);
+  fetch(a[0], v[0]);
+#pragma unroll
+  for (int d = 1; d < DEPTH - 1; ++d) {
+    advance();
+    fetch(a[d], v[d]);
+  }
+  const int steps = p.chunks * p.kgroups;
+  for (int step = 0; step < steps; step += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      advance();
+      fetch(a[(d + DEPTH - 1) % DEPTH], v[(d + DEPTH - 1) % DEPTH]);
+      feed_all<NACC, EPV>(acc, a[d], v[d]);
+    }
   }
 
+  if constexpr (NACC >= 8) asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");  // the last MFMAs' results are written before they are read
   if (!active) return;
   float *const dst_n = p.dst + (long long)n * p.dst_nstride;
 #pragma unroll
@@ -119,52 +174,70 @@ __global__ void __launch_bounds__(256) thin_gemm_kernel(ThinParams p) {
       // phases 2q and 2q + 1 lie side by side in dst: one 8-byte store for both
       if ((ph & 1) == 0 && here) {
 #pragma unroll
-        for (int m = 0; m < 4; ++m)
-          if (m < p.M) *reinterpret_cast<f32x2 *>(dst_n + (long long)m * p.dst_mstride + o) = f32x2{acc[ph][m], acc[ph | 1][m]};
+        for (int r = 0; r < RG; ++r)
+#pragma unroll
+          for (int m = 0; m < 4; ++m)
+            if (r * 4 + m < p.M)
+              *reinterpret_cast<f32x2 *>(dst_n + (long long)(r * 4 + m) * p.dst_mstride + o) = f32x2{acc[ph * RG + r][m], acc[(ph | 1) * RG + r][m]};
       }
     } else if (here) {
 #pragma unroll
-      for (int m = 0; m < 4; ++m)
-        if (m < p.M) dst_n[(long long)m * p.dst_mstride + o] = acc[ph][m];
+      for (int r = 0; r < RG; ++r)
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+          if (r * 4 + m < p.M) dst_n[(long long)(r * 4 + m) * p.dst_mstride + o] = acc[ph * RG + r][m];
     }
   }
 }
 
 // packed[(q * kgroups + kg) * 64 + slot * 4 + m] = w[arow[q * 16 + slot] + kg * group_stride + m * m_stride]
-// (zero where arow is negative or m >= M)
+// (zero where arow is negative or the slot's row group, slot % rg, ends before row m)
 __global__ void __launch_bounds__(256) thin_pack_kernel(const float *__restrict__ w, float *__restrict__ packed, const int *__restrict__ arow,
-                                                        int chunks, int kgroups, long long group_stride, int m_stride, int M) {
+                                                        int chunks, int kgroups, long long group_stride, int m_stride, int M, int rg) {
   const long long total = (long long)chunks * kgroups * 64;
   for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long long)gridDim.x * 256) {
     const int m = (int)(i & 3), slot = (int)((i >> 2) & 15);
     const long long qk = i >> 6;
     const int q = (int)(qk / kgroups), kg = (int)(qk - (long long)q * kgroups);
     const int row = arow[q * 16 + slot];
-    packed[i] = (row >= 0 && m < M) ? w[row + kg * group_stride + (long long)m * m_stride] : 0.f;
+    packed[i] = (row >= 0 && (slot % rg) * 4 + m < M) ? w[row + kg * group_stride + (long long)m * m_stride] : 0.f;
   }
 }
 
 }  // namespace
 
 int launch_thin_pack(const float *w, float *packed, const int *arow, int chunks, int kgroups, long long group_stride, int m_stride, int M,
-                     hipStream_t s) {
+                     int rg, hipStream_t s) {
   const long long total = (long long)chunks * kgroups * 64;
   const unsigned blocks = (unsigned)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
-  hipLaunchKernelGGL(thin_pack_kernel, dim3(blocks ? blocks : 1), dim3(256), 0, s, w, packed, arow, chunks, kgroups, group_stride, m_stride, M);
+  hipLaunchKernelGGL(thin_pack_kernel, dim3(blocks ? blocks : 1), dim3(256), 0, s, w, packed, arow, chunks, kgroups, group_stride, m_stride, M,
+                     rg);
   hipError_t err = hipGetLastError();
   return err == hipSuccess ? MG_OK : hip_fail(err, "thin_pack_kernel", __FILE__, __LINE__);
 }
 
+// (stride phases, row groups) the kernel is built for: their product is at most 16
+#define MG_THIN_SHAPES(X) X(1, 1) X(1, 2) X(1, 4) X(1, 8) X(1, 16) X(2, 1) X(2, 2) X(2, 4) X(2, 8) X(4, 1) X(4, 2) X(4, 4)
+
+bool thin_gemm_has(int nph, int rg) {
+#define MG_THIN_HAS(NPH, RG) \
+  if (nph == NPH && rg == RG) return true;
+  MG_THIN_SHAPES(MG_THIN_HAS)
+#undef MG_THIN_HAS
+  return false;
+}
+
 int launch_thin_gemm(const ThinParams &p, hipStream_t s) {
   const unsigned blocks = (unsigned)((p.npos + 255) / 256);
-  if (p.nph == 1)
-    hipLaunchKernelGGL(thin_gemm_kernel<1>, dim3(blocks), dim3(256), 0, s, p);
-  else if (p.nph == 2)
-    hipLaunchKernelGGL(thin_gemm_kernel<2>, dim3(blocks), dim3(256), 0, s, p);
-  else if (p.nph == 4)
-    hipLaunchKernelGGL(thin_gemm_kernel<4>, dim3(blocks), dim3(256), 0, s, p);
-  else
-    return fail(MG_ERR_UNSUPPORTED, "thin gather-GEMM with %d phases", p.nph);
+  bool launched = false;
+#define MG_THIN_LAUNCH(NPH, RG)                                                               \
+  if (p.nph == NPH && p.rg == RG) {                                                            \
+    hipLaunchKernelGGL((thin_gemm_kernel<NPH, RG>), dim3(blocks), dim3(256), 0, s, p);         \
+    launched = true;                                                                           \
+  }
+  MG_THIN_SHAPES(MG_THIN_LAUNCH)
+#undef MG_THIN_LAUNCH
+  if (!launched) return fail(MG_ERR_UNSUPPORTED, "one-position-per-lane gather-GEMM with %d phases x %d row groups", p.nph, p.rg);
   hipError_t err = hipGetLastError();
   return err == hipSuccess ? MG_OK : hip_fail(err, "thin_gemm_kernel", __FILE__, __LINE__);
 }
