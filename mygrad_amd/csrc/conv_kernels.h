@@ -138,7 +138,8 @@ struct ThinParams {
   float *dst;
   const TabEntry *tab;
   int chunks;           // chunks of 16 / (nph * rg) entries
-  int kgroups;          // steps of the inner loop
+  int kgroups;          // groups of source channels: chunks * kgroups steps in all
+  int kblock;           // groups per block: all chunks run under one block of groups before the next block
   unsigned group_bytes; // bytes of src between consecutive groups
   unsigned a_bytes, src_bytes;
   int M;

@@ -113,10 +113,15 @@ __global__ void __launch_bounds__(256) thin_gemm_kernel(ThinParams p) {
                       ((unsigned)(c2 + e.w) < (unsigned)p.Q[2]);  // no branches: the rows are the same for every lane
       at[i] = ok ? src_at + (unsigned)(e.x * 4) : kOutside;
     }
-    if constexpr (AHEAD) ask_rows(min(q + 1, p.chunks - 1));
+    if constexpr (AHEAD) ask_rows(q + 1 < p.chunks ? q + 1 : 0);
   };
   if constexpr (AHEAD) ask_rows(0);
-  int q = 0, kg = 0;
+  // The channel groups are taken in blocks of p.kblock: all chunks under one block, then the
+  // next block.  The chunks read overlapping neighbourhoods of the same channels (the taps of a
+  // window; the rows of grad the stride phases share), and with every channel between two
+  // chunks the second one found nothing of the first in the caches: the stem's data gradient
+  // read grad 4.7 times from HBM.
+  int q = 0, kg = 0, kbegin = 0, kend = min(p.kblock, p.kgroups);
   unsigned a_uni = 0u, s_uni = 0u;
   auto fetch = [&](float &a, float (&v)[EPV]) {
     a = buffer_load(a_buf, a_lane, a_uni);
@@ -129,14 +134,21 @@ __global__ void __launch_bounds__(256) thin_gemm_kernel(ThinParams p) {
   auto advance = [&]() {
     a_uni += 256u;
     s_uni += p.group_bytes;
-    if (++kg == p.kgroups) {
-      kg = 0;
-      s_uni = 0u;
-      if (++q < p.chunks) {
+    if (++kg == kend) {
+      if (++q == p.chunks) {
+        q = 0;
+        kbegin = kend;
+        kend = min(kbegin + p.kblock, p.kgroups);
+      }
+      kg = kbegin;
+      if (kbegin < p.kgroups) {
+        a_uni = (unsigned)(q * p.kgroups + kg) * 256u;
+        s_uni = (unsigned)kg * p.group_bytes;
         enter_chunk(q);
       } else {
 #pragma unroll
         for (int i = 0; i < EPV; ++i) at[i] = kOutside;
+        a_uni = kOutside;
       }
     }
   };
