@@ -78,6 +78,9 @@ WORKLOADS = {
     "bn3a": dict(kind="bn", dtype="f32", seed=1008, x=(128, 64, 56, 56), eps=1e-5),
     # matrix product on the convolution kernels: one dense layer's three products
     "bmm64": dict(kind="bmm", dtype="f32", seed=1016, batch=512, M=64, K=64, N=64),
+    # the same products in a stack sixteen times as tall: 134 MB per launch instead of 8, so that the
+    # kernel's rate shows and not the few microseconds any launch takes
+    "bmm64-tall": dict(kind="bmm", dtype="f32", seed=1016, batch=8192, M=64, K=64, N=64),
     "mm4k": dict(kind="matmul", dtype="f32", seed=1011, M=4096, K=4096, N=4096),
     # sums over axes of a tensor of conv5's output size: per channel (the gradient of a bias or of a
     # per-channel scale: every axis but axis 1), then over the channel axis alone
