@@ -31,7 +31,9 @@ typedef enum {
   MG_ERR_NOT_INIT = -6     /* mg_init() has not succeeded */
 } mg_status;
 
-typedef enum { MG_F32 = 0, MG_F64 = 1 } mg_dtype;
+/* MG_F16 (IEEE binary16) is a storage type only: mg_cast and mg_accumulate take it, every other
+ * entry point computes in float32 or float64 and refuses it (MG_ERR_UNSUPPORTED). */
+typedef enum { MG_F32 = 0, MG_F64 = 1, MG_F16 = 2 } mg_dtype;
 
 /* Shapes of one convolution  x:(N,C,X...) * w:(F,C,W...) -> out:(N,F,G...).
  * Axes are right-aligned: a rank-nd problem fills the LAST nd entries of each
@@ -252,11 +254,14 @@ int mg_fill_from(int dtype, int64_t n, const void *value, void *out);
  * device.  Buffers from mg_malloc (32-byte aligned for the first two). */
 
 /* out[i] = (to_dtype) x[i]: `backed.astype(var.dtype)`, operation_base.py:223-224 (the float64
- * gradient of a float32 max_pool input, pooling.py:147). */
+ * gradient of a float32 max_pool input, pooling.py:147).  Either type may be MG_F16: float16
+ * operands of conv_nd / max_pool are widened to float32 for the kernels and the result is
+ * rounded to float16 once, to nearest even (from float64 in one step, not through float32). */
 int mg_cast(int from_dtype, int to_dtype, int64_t n, const void *x, void *out);
 
 /* acc[i] = (acc_dtype)(acc[i] + inc[i]), the sum formed in the wider of the two types:
- * `var._grad += backed`, operation_base.py:227-228, with NumPy's rule for a narrower `acc`. */
+ * `var._grad += backed`, operation_base.py:227-228, with NumPy's rule for a narrower `acc`.
+ * Either type may be MG_F16. */
 int mg_accumulate(int acc_dtype, int inc_dtype, int64_t n, void *acc, const void *inc);
 
 /* out[i] = value: `np.full_like(self.data, fill_value=1.0)`, the seed of Tensor.backward()

@@ -228,12 +228,12 @@ class DeviceArray:
         return DeviceArray(buf, self.shape, self.dtype)
 
     def astype(self, dtype):
-        """The values cast to float32 / float64 on the device (a new buffer)."""
+        """The values cast to float32 / float64 / float16 on the device (a new buffer)."""
         dtype = np.dtype(dtype)
         if dtype == self.dtype:
             return self
         buf = DeviceBuffer(max(self.size * dtype.itemsize, 16))
-        _hip.check(_hip.lib().mg_cast(_hip.dtype_code(self.dtype), _hip.dtype_code(dtype), self.size, self.buf.ptr, buf.ptr))
+        _hip.check(_hip.lib().mg_cast(_hip.storage_code(self.dtype), _hip.storage_code(dtype), self.size, self.buf.ptr, buf.ptr))
         return DeviceArray(buf, self.shape, dtype)
 
     def add_into(self, other):
@@ -241,7 +241,7 @@ class DeviceArray:
         formed in the wider type and rounded once).  ``self`` must own its buffer and must not
         have been copied to the host yet."""
         assert self.base is None and self._host is None and other.shape == self.shape
-        _hip.check(_hip.lib().mg_accumulate(_hip.dtype_code(self.dtype), _hip.dtype_code(other.dtype), self.size,
+        _hip.check(_hip.lib().mg_accumulate(_hip.storage_code(self.dtype), _hip.storage_code(other.dtype), self.size,
                                             self.buf.ptr, other.buf.ptr))
 
     def __repr__(self):

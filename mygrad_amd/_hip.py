@@ -10,7 +10,7 @@ import os
 import threading
 
 MG_MAX_ND = 3
-MG_F32, MG_F64 = 0, 1
+MG_F32, MG_F64, MG_F16 = 0, 1, 2
 
 MG_OK = 0
 MG_ERR_BAD_ARG = -1
@@ -321,6 +321,14 @@ def dtype_code(dtype):
     if dtype == np.float64:
         return MG_F64
     raise TypeError(f"the HIP kernels handle float32 and float64 only, got {dtype}")
+
+
+def storage_code(dtype):
+    """``dtype_code`` for the two conversions (``mg_cast``, ``mg_accumulate``), which also take
+    float16: a type arrays are stored in, not one any kernel computes in."""
+    import numpy as np
+
+    return MG_F16 if np.dtype(dtype) == np.float16 else dtype_code(dtype)
 
 
 def conv_desc(dtype, x_shape, w_shape, grid, stride, padding, dilation):

@@ -343,10 +343,16 @@ int launch_convert(int a_dtype, int b_dtype, int64_t n, void *acc, const void *i
   const unsigned grid = (unsigned)std::min<long long>(ceil_div(ceil_div(n, 4), 256), (long long)runtime().props.multiProcessorCount * 16);
   ScopedTiming timed(TAG_ELEMENTWISE);
 #define MG_CONVERT(A, B) hipLaunchKernelGGL((convert_kernel<A, B, ADD>), dim3(grid), dim3(256), 0, s, (A *)acc, (const B *)inc, (long long)n)
-  if (a_dtype == MG_F32 && b_dtype == MG_F32) MG_CONVERT(float, float);
-  else if (a_dtype == MG_F32) MG_CONVERT(float, double);
-  else if (b_dtype == MG_F32) MG_CONVERT(double, float);
-  else MG_CONVERT(double, double);
+#define MG_CONVERT_FROM(A)                               \
+  do {                                                   \
+    if (b_dtype == MG_F32) MG_CONVERT(A, float);         \
+    else if (b_dtype == MG_F64) MG_CONVERT(A, double);   \
+    else MG_CONVERT(A, _Float16);                        \
+  } while (0)
+  if (a_dtype == MG_F32) MG_CONVERT_FROM(float);
+  else if (a_dtype == MG_F64) MG_CONVERT_FROM(double);
+  else MG_CONVERT_FROM(_Float16);
+#undef MG_CONVERT_FROM
 #undef MG_CONVERT
   MG_HIP(hipGetLastError());
   return MG_OK;
@@ -546,11 +552,19 @@ int mg_sum_all_static(int dtype, int64_t n, const void *x, void *out) {
   return launch_sum_all(dtype, n, x, out, partial);
 }
 
+// float16 is a storage type: the two conversions take it, nothing else does
+static int check_storage(int dtype, int64_t n, const char *who) {
+  if (dtype != MG_F32 && dtype != MG_F64 && dtype != MG_F16)
+    return fail(MG_ERR_UNSUPPORTED, "%s: dtype %d (float32=0 / float64=1 / float16=2)", who, dtype);
+  if (n < 0) return fail(MG_ERR_BAD_ARG, "%s: n = %lld", who, (long long)n);
+  return MG_OK;
+}
+
 int mg_cast(int from_dtype, int to_dtype, int64_t n, const void *x, void *out) {
   std::lock_guard<std::recursive_mutex> guard(api_mutex());
   MG_REQUIRE_INIT();
-  if (int rc = check_elementwise(from_dtype, n, "mg_cast")) return rc;
-  if (int rc = check_elementwise(to_dtype, n, "mg_cast")) return rc;
+  if (int rc = check_storage(from_dtype, n, "mg_cast")) return rc;
+  if (int rc = check_storage(to_dtype, n, "mg_cast")) return rc;
   if (n > 0 && (!x || !out)) return fail(MG_ERR_BAD_ARG, "null pointer in mg_cast");
   if (reinterpret_cast<uintptr_t>(x) % 32 != 0 || reinterpret_cast<uintptr_t>(out) % 32 != 0)
     return fail(MG_ERR_BAD_ARG, "mg_cast: buffers must be 32-byte aligned");
@@ -560,8 +574,8 @@ int mg_cast(int from_dtype, int to_dtype, int64_t n, const void *x, void *out) {
 int mg_accumulate(int acc_dtype, int inc_dtype, int64_t n, void *acc, const void *inc) {
   std::lock_guard<std::recursive_mutex> guard(api_mutex());
   MG_REQUIRE_INIT();
-  if (int rc = check_elementwise(acc_dtype, n, "mg_accumulate")) return rc;
-  if (int rc = check_elementwise(inc_dtype, n, "mg_accumulate")) return rc;
+  if (int rc = check_storage(acc_dtype, n, "mg_accumulate")) return rc;
+  if (int rc = check_storage(inc_dtype, n, "mg_accumulate")) return rc;
   if (n > 0 && (!acc || !inc)) return fail(MG_ERR_BAD_ARG, "null pointer in mg_accumulate");
   if (reinterpret_cast<uintptr_t>(acc) % 32 != 0 || reinterpret_cast<uintptr_t>(inc) % 32 != 0)
     return fail(MG_ERR_BAD_ARG, "mg_accumulate: buffers must be 32-byte aligned");

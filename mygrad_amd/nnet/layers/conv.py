@@ -25,15 +25,28 @@ def _per_axis(value, m, lowest):
 
 
 def _kernel_dtype(*arrays):
-    """The dtype the kernels compute in: NumPy's promotion of the operands, which
-    must come out as float32 or float64."""
-    dtype = np.result_type(*(a.dtype for a in arrays))
+    """(the dtype the kernels compute in, the dtype of the result): NumPy's promotion of the
+    operands, which must come out as float32, float64 or float16.  float16 is a storage type:
+    NumPy multiplies float16 arrays with float32 sums rounded once at the end
+    (``np.tensordot`` in the reference's conv.py:96-99), so its operands are widened to float32
+    (exactly), the float32 kernels run, and the result is rounded to float16 on the device."""
+    dtype = np.dtype(np.result_type(*(a.dtype for a in arrays)))
+    if dtype == np.float16:
+        return np.dtype(np.float32), dtype
     if dtype not in (np.float32, np.float64):
         raise TypeError(
-            f"conv_nd runs on the GPU in float32 or float64; the operands promote to {dtype} "
-            "(there is no CPU fallback)"
+            f"conv_nd runs on the GPU in float32 or float64 (float16 operands are widened to float32); "
+            f"the operands promote to {dtype} (there is no CPU fallback)"
         )
-    return np.dtype(dtype)
+    return dtype, dtype
+
+
+def _narrowed(buf, shape, dtype, result_dtype):
+    """The kernel's result ``buf`` as the array handed back: rounded to float16 on the device
+    when the operands were float16."""
+    if result_dtype != dtype:
+        buf = _device.DeviceArray(buf, shape, dtype).astype(result_dtype).buf
+    return _device.download(buf, shape, result_dtype), buf
 
 
 def _device_zeros(shape, dtype):
@@ -87,15 +100,18 @@ class ConvND(Operation):
         check_window_args(padded, tuple(int(i) for i in w_shape), tuple(int(s) for s in stride),
                           tuple(int(d) for d in dilation))
 
-        dtype = _kernel_dtype(xd, wd)
+        if np.iscomplexobj(xd) or np.iscomplexobj(wd):
+            return self._complex_forward(xd, wd)
+        dtype, result_dtype = _kernel_dtype(xd, wd)
         grid = tuple(int(g) for g in out_shape)
         out_full = (xd.shape[0], wd.shape[0], *grid)
         self._dtype = dtype
+        self._result_dtype = result_dtype
         self._grid = grid
         if xd.size == 0 or wd.size == 0:
             # nothing to gather: every product involves a padding zero
             self._desc = None
-            return _device_zeros(out_full, dtype)
+            return np.zeros(out_full, dtype=result_dtype) if result_dtype != dtype else _device_zeros(out_full, dtype)
 
         xb = _device.to_device(xd, dtype)
         wb = _device.to_device(wd, dtype)
@@ -108,15 +124,41 @@ class ConvND(Operation):
             self._desc = _hip.conv_desc(dtype, xd.shape, wd.shape, grid, stride, padding, dilation)
             ob = _device.DeviceBuffer(int(np.prod(out_full)) * dtype.itemsize)
             _hip.check(_hip.lib().mg_conv_fwd(self._desc, xb.ptr, wb.ptr, ob.ptr))
-        out = _device.download(ob, out_full, dtype)
+        out, ob = _narrowed(ob, out_full, dtype, result_dtype)
         _device.attach(out, ob)
+        return out
+
+    def _complex_forward(self, xd, wd):
+        """Complex operands (reference: ``np.tensordot`` multiplies whatever it is given,
+        conv.py:96-99; complex arrays reach the operation only under ``no_autodiff``, where the
+        reference's own tests take complex-step derivatives through it).  One real convolution
+        of twice the channels and filters: with x = a + ib laid out as channels [a, b] and the
+        filters as [[p, -q], [q, p]] for w = p + iq, the first F maps of the result are
+        a*p - b*q and the last F are a*q + b*p.  Every product stays among parts of its own
+        magnitude, which is what a complex step of 1e-20 needs."""
+        real = np.float32 if np.result_type(xd.dtype, wd.dtype) == np.complex64 else np.float64
+        xd, wd = np.asarray(xd), np.asarray(wd)
+        a, b = np.real(xd).astype(real, copy=False), np.imag(xd).astype(real, copy=False)
+        p, q = np.real(wd).astype(real, copy=False), np.imag(wd).astype(real, copy=False)
+        planes = np.concatenate([a, b], axis=1)
+        bank = np.concatenate([np.concatenate([p, -q], axis=1), np.concatenate([q, p], axis=1)], axis=0)
+        inner = ConvND()
+        both = np.asarray(inner(Tensor(planes, constant=True, copy=False), Tensor(bank, constant=True, copy=False),
+                                stride=self.stride, padding=self.padding, dilation=self.dilation))
+        filters = wd.shape[0]
+        out = np.empty((both.shape[0], filters, *both.shape[2:]), dtype=np.result_type(xd.dtype, wd.dtype))
+        out.real = both[:, :filters]
+        out.imag = both[:, filters:]
+        self._desc = None
+        self._dtype = self._result_dtype = out.dtype
         return out
 
     def backward_var(self, grad, index, **kwargs):
         x, w = (_device.value_of(v) for v in self.variables)
         dtype = self._dtype
         if self._desc is None:
-            return _device_zeros((x if index == 0 else w).shape, dtype)
+            return np.zeros((x if index == 0 else w).shape, dtype=self._result_dtype) if self._result_dtype != dtype else _device_zeros(
+                (x if index == 0 else w).shape, dtype)
         lib = _hip.lib()
         if tuple(grad.shape) != (x.shape[0], w.shape[0], *self._grid):
             raise ValueError(f"conv_nd backward: gradient of shape {tuple(grad.shape)} for an output of shape "
@@ -130,7 +172,7 @@ class ConvND(Operation):
             else:
                 db = _device.DeviceBuffer(x.size * dtype.itemsize)
                 _hip.check(lib.mg_conv_dgrad(self._desc, gb.ptr, wb.ptr, db.ptr))
-            out = _device.download(db, x.shape, dtype)
+            out, db = _narrowed(db, x.shape, dtype, self._result_dtype)
         else:  # dw
             xb = _device.to_device(x, dtype)
             if self._desc == "folded":
@@ -138,7 +180,7 @@ class ConvND(Operation):
             else:
                 db = _device.DeviceBuffer(w.size * dtype.itemsize)
                 _hip.check(lib.mg_conv_wgrad(self._desc, gb.ptr, xb.ptr, db.ptr))
-            out = _device.download(db, w.shape, dtype)
+            out, db = _narrowed(db, w.shape, dtype, self._result_dtype)
         _device.attach_transient(out, db)
         return out
 

@@ -137,16 +137,22 @@ class MaxPoolND(Operation):
         while m - skip > 1 and pool[skip] == 1 and stride[skip] == 1:
             skip += 1
         self._skip = skip
-        if xd.dtype not in (np.float32, np.float64):
+        if xd.dtype not in (np.float32, np.float64, np.float16):
             raise TypeError(
-                f"max_pool runs on the GPU in float32 or float64, got {xd.dtype} (there is no CPU fallback)"
+                f"max_pool runs on the GPU in float32 or float64 (float16 values are widened to float32), got {xd.dtype} "
+                "(there is no CPU fallback)"
             )
+        # float16 is a storage type here: the values are widened to float32 (exactly), the kernels
+        # pick the same maxima, and the result is narrowed again (exactly: it consists of inputs)
+        result_dtype = xd.dtype
+        if xd.dtype == np.float16:
+            xd = xd.astype(np.float32)  # on the device for a value that lives there, else on the host
         grid = tuple(int(g) for g in out_shape)
         self._grid = grid
         self._lead = int(np.prod(lead_shape, dtype=np.int64))
         out_full = (*lead_shape, *grid)
         if self._lead == 0:
-            return np.empty(out_full, dtype=xd.dtype)
+            return np.empty(out_full, dtype=result_dtype)
 
         self._lead *= int(np.prod(pooled[:skip], dtype=np.int64))
         stages = plan_stages(self._lead, pooled[skip:], pool[skip:], stride[skip:])
@@ -157,7 +163,9 @@ class MaxPoolND(Operation):
             if i:
                 stage.source = buf
             buf = stage.forward(xd.dtype, buf)
-        out = _device.download(buf, out_full, xd.dtype)
+        if result_dtype != xd.dtype:
+            buf = _device.DeviceArray(buf, out_full, xd.dtype).astype(result_dtype).buf
+        out = _device.download(buf, out_full, result_dtype)
         _device.attach(out, buf)
         return out
 
@@ -166,6 +174,10 @@ class MaxPoolND(Operation):
         x = _device.value_of(var)
         if self._lead == 0:
             return np.zeros(x.shape, dtype=np.float64)
+        held = x  # what the graph holds (and locks)
+        half = x.dtype == np.float16
+        if half:
+            x = x.astype(np.float32)
         if grad.shape != (*x.shape[: x.ndim - len(self.pool)], *self._grid):
             raise ValueError(f"max_pool backward: gradient of shape {grad.shape} for an output of shape "
                              f"{(*x.shape[: x.ndim - len(self.pool)], *self._grid)}")
@@ -174,13 +186,14 @@ class MaxPoolND(Operation):
         # double and rounds once, so it can write x.dtype directly -- except when
         # var already holds a gradient that this one is added to, where the
         # unrounded float64 values are needed for the same result.
-        dx_dtype = np.dtype(np.float64) if var._grad is not None else x.dtype
+        # A float16 x gets the float64 sums, which the caller rounds to float16 in one step.
+        dx_dtype = np.dtype(np.float64) if var._grad is not None or half else x.dtype
         wide = np.dtype(np.float64)
         stages = self._stages
         # x is read-only for as long as the graph holds it, so the recorded positions cannot go
         # stale; if it was released and may have been written to, the maxima are found again
         # (for several stages: all of them, from the values x holds now)
-        fresh = _device.is_locked(x)
+        fresh = _device.is_locked(held)
         xb = None
         if not fresh or stages[0].argmax is None:
             xb = _device.to_device(x)

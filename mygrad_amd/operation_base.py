@@ -114,14 +114,14 @@ class Operation(ABC):
             if backed.base is not None or backed is grad:
                 backed = backed.copy()
             if backed.dtype != var.dtype:
-                if var.dtype in (np.float32, np.float64):
+                if var.dtype in (np.float32, np.float64, np.float16):
                     backed = backed.astype(var.dtype)
                 else:
                     backed = backed.host().astype(var.dtype)
             var._grad = backed
             return
         held = var._grad
-        if isinstance(held, _device.DeviceArray) and held._host is None and held.base is None and held.dtype in (np.float32, np.float64):
+        if isinstance(held, _device.DeviceArray) and held._host is None and held.base is None and held.dtype in (np.float32, np.float64, np.float16):
             held.add_into(backed)
             return
         if isinstance(held, _device.DeviceArray):

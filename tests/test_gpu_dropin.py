@@ -514,3 +514,142 @@ def test_pooling_over_four_axes_with_a_leading_window_of_one():
     out.backward(g)
     assert np.array_equal(x.grad.view(np.uint64), ora.pool_backward(xv, g, (1, 1, 2, 3, 2), (1, 1, 1, 3, 2)).view(np.uint64))
     assert _graph.held_count() == 0
+
+
+def _ulp16(a):
+    return np.spacing(np.abs(np.asarray(a, dtype=np.float16))).astype(np.float64)
+
+
+def test_casts_to_and_from_float16_round_like_numpy():
+    """float16 is a storage type of the library: ``mg_cast`` rounds to nearest even in one step
+    (a float64 just above a float16 tie must not be rounded to float32 first), keeps signed zeros,
+    infinities, NaNs and subnormals, and ``mg_accumulate`` forms ``a += b`` in the wider type."""
+    rng = np.random.default_rng(77)
+    tie = 1.0 + 2.0**-11  # halfway between two float16 values
+    special = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 65504.0, 65519.9, 65520.0, -65520.0, 1e-8, 5.96e-8, 2.98e-8,
+                        2.9803e-8, 6.1e-5, tie, tie + 2.0**-40, tie - 2.0**-40, -(tie + 2.0**-40), 3 * 2.0**-11 + 1, 2049.0, 2051.0], dtype=np.float64)
+    values = np.concatenate([special, rng.standard_normal(5000) * 10.0 ** rng.integers(-9, 5, 5000)])
+    for wide in (np.float64, np.float32):
+        src = values.astype(wide)
+        buf = _device.DeviceBuffer(max(src.nbytes, 16))
+        buf.upload(src)
+        with np.errstate(over="ignore"):
+            want = src.astype(np.float16)
+        got = _device.DeviceArray(buf, src.shape, wide).astype(np.float16)
+        assert got.dtype == np.float16
+        assert np.array_equal(got.host().view(np.uint16), want.view(np.uint16))
+        back = got.astype(wide).host()
+        assert np.array_equal(back.view(np.uint64 if wide == np.float64 else np.uint32), want.astype(wide).view(np.uint64 if wide == np.float64 else np.uint32))
+    # a += b with a in float16: the sum is formed in the wider type and rounded once
+    a16 = (rng.standard_normal(1000) * 8).astype(np.float16)
+    for inc_dtype in (np.float16, np.float32, np.float64):
+        inc = (rng.standard_normal(1000) * 8).astype(inc_dtype)
+        abuf, ibuf = _device.DeviceBuffer(a16.nbytes), _device.DeviceBuffer(inc.nbytes)
+        abuf.upload(a16)
+        ibuf.upload(inc)
+        acc = _device.DeviceArray(abuf, a16.shape, np.float16)
+        acc.add_into(_device.DeviceArray(ibuf, inc.shape, inc_dtype))
+        want = a16.copy()
+        want += inc.astype(want.dtype, copy=False) if inc_dtype == np.float16 else inc  # NumPy: same-kind cast of the sum
+        assert np.array_equal(acc.host().view(np.uint16), want.view(np.uint16)), inc_dtype
+
+
+def test_float16_operands_are_widened_and_rounded_once():
+    """float16 tensors (reference: any float dtype, conv.py:20-21; NumPy multiplies float16 arrays
+    with float32 sums rounded to float16 at the end).  Here the operands are widened to float32,
+    the float32 kernels run and the result is rounded once: within one float16 unit in the last
+    place of the reference's value everywhere (the sums run in another order), and within half a
+    unit (+ the float32 sum's own error) of the exact result, which the reference's dx -- rounded
+    after every window it adds -- is not."""
+    rng = np.random.default_rng(78)
+    x16 = rng.standard_normal((4, 6, 12, 12)).astype(np.float16)
+    w16 = (rng.standard_normal((8, 6, 3, 3)) / 7).astype(np.float16)
+    x, w = mg.Tensor(x16), mg.Tensor(w16)
+    out = conv_nd(x, w, stride=1, padding=1)
+    assert out.dtype == np.float16 and out.shape == (4, 8, 12, 12)
+    want = ora.conv_forward(x16, w16, stride=1, padding=1)
+    assert want.dtype == np.float16
+    got = out.data
+    assert np.mean(got == want) > 0.98
+    # the exact result, and what a float32 sum of these terms may be off by (1e-6 of the sum of
+    # their magnitudes: 54 to 576 terms of relative error 6e-8 each)
+    x64, w64 = x16.astype(np.float64), w16.astype(np.float64)
+    exact = ora.conv_forward(x64, w64, stride=1, padding=1)
+    slack = 1e-6 * ora.conv_forward(np.abs(x64), np.abs(w64), stride=1, padding=1)
+    assert np.all(np.abs(got.astype(np.float64) - exact) <= 0.5 * _ulp16(exact) + slack)
+    assert np.all(np.abs(got.astype(np.float64) - want.astype(np.float64)) <= _ulp16(want) + 2 * slack)
+
+    g16 = rng.standard_normal(out.shape).astype(np.float16)
+    out.backward(g16)
+    assert x.grad.dtype == np.float16 and w.grad.dtype == np.float16
+    g64 = g16.astype(np.float64)
+    dx_exact = ora.conv_backward_x(g64, x16.shape, np.float64, w64, stride=1, padding=1)
+    dw_exact = ora.conv_backward_w(g64, x64, w16.shape, stride=1, padding=1)
+    dx_slack = 1e-6 * ora.conv_backward_x(np.abs(g64), x16.shape, np.float64, np.abs(w64), stride=1, padding=1)
+    dw_slack = 1e-6 * ora.conv_backward_w(np.abs(g64), np.abs(x64), w16.shape, stride=1, padding=1)
+    assert np.all(np.abs(x.grad.astype(np.float64) - dx_exact) <= 0.5 * _ulp16(dx_exact) + dx_slack)
+    assert np.all(np.abs(w.grad.astype(np.float64) - dw_exact) <= 0.5 * _ulp16(dw_exact) + dw_slack)
+    # against the reference's own arithmetic: dw has one rounding there too, dx nine more
+    dw_ref = ora.conv_backward_w(g16, x16, w16.shape, stride=1, padding=1)
+    assert np.all(np.abs(w.grad.astype(np.float64) - dw_ref.astype(np.float64)) <= _ulp16(dw_ref) + 2 * dw_slack)
+    dx_ref = ora.conv_backward_x(g16, x16.shape, np.float16, w16, stride=1, padding=1)
+    assert rel_err(x.grad, dx_ref) <= 4e-3
+
+    # float16 against float32 promotes to float32, as in NumPy
+    out = conv_nd(mg.Tensor(x16), mg.Tensor(w16.astype(np.float32)), stride=1)
+    assert out.dtype == np.float32
+    assert rel_err(out.data, ora.conv_forward(x16.astype(np.float64), w16.astype(np.float64), stride=1)) <= 2e-4
+
+
+def test_max_pool_of_float16_is_exact():
+    """Pooling picks inputs and adds gradients in float64 (pooling.py:147), rounded to the tensor's
+    type once: with float16 tensors both passes agree with the reference bit for bit, ties and
+    overlapping windows included."""
+    rng = np.random.default_rng(79)
+    x16 = rng.integers(-4, 5, (3, 5, 13, 13)).astype(np.float16) / np.float16(4)  # many ties
+    x16[0, 0, :4, :4] = rng.standard_normal((4, 4)).astype(np.float16) * 100
+    g16 = (rng.standard_normal((3, 5, 6, 6)) * 3).astype(np.float16)
+    x = mg.Tensor(x16)
+    out = max_pool(x, (3, 3), 2)
+    assert out.dtype == np.float16
+    assert np.array_equal(out.data.view(np.uint16), ora.pool_forward(x16, (3, 3), 2).view(np.uint16))
+    out.backward(g16)
+    want = ora.pool_backward(x16, g16, (3, 3), 2).astype(np.float16)
+    assert x.grad.dtype == np.float16
+    assert np.array_equal(x.grad.view(np.uint16), want.view(np.uint16))
+
+
+def test_complex_operands_under_no_autodiff_carry_a_complex_step():
+    """The reference's tests differentiate conv_nd numerically with a complex step through the
+    operation itself (tests/nnet/layers/test_conv.py:291-300, tests/utils/numerical_gradient.py):
+    complex128 operands under ``no_autodiff``.  Here they run as one real convolution of twice the
+    channels and filters; the imaginary part of a step of 1e-20 comes back with full relative
+    precision and gives the derivative the data gradient gives."""
+    rng = np.random.default_rng(80)
+    x = rng.standard_normal((2, 3, 9, 8))
+    w = rng.standard_normal((4, 3, 3, 2))
+    kwargs = dict(stride=(2, 1), padding=(1, 0), dilation=(1, 2))
+    with mg.no_autodiff:
+        z = conv_nd(x + 1j * rng.standard_normal(x.shape), w + 1j * rng.standard_normal(w.shape), **kwargs)
+    assert z.dtype == np.complex128
+    xc, wc = rng.standard_normal(x.shape) * 1j + x, rng.standard_normal(w.shape) * 1j + w
+    with mg.no_autodiff:
+        z = np.asarray(conv_nd(xc, wc, **kwargs).data)
+    want = ora.conv_forward(xc, wc, **kwargs)
+    assert rel_err(z.real, want.real) <= 1e-10 and rel_err(z.imag, want.imag) <= 1e-10
+
+    # complex step in one element of x: d out / d x[e] for every output at once
+    h = 1e-20
+    e = (1, 2, 4, 3)
+    step = x.astype(np.complex128)
+    step[e] += 1j * h
+    with mg.no_autodiff:
+        slope = np.asarray(conv_nd(step, w.astype(np.complex128), **kwargs).data).imag / h
+    g = rng.standard_normal(slope.shape)
+    tx, tw = mg.Tensor(x), mg.Tensor(w)
+    conv_nd(tx, tw, **kwargs).backward(g)
+    assert abs(float(np.sum(slope * g)) - float(tx.grad[e])) <= 1e-10 * max(1.0, abs(float(tx.grad[e])))
+    # a real operand against a complex one
+    with mg.no_autodiff:
+        z = np.asarray(conv_nd(x, wc, **kwargs).data)
+    assert rel_err(z.imag, ora.conv_forward(x.astype(np.complex128), wc, **kwargs).imag) <= 1e-10
