@@ -1040,8 +1040,10 @@ int thin_row_groups(int rows, int nph) {
 // it loses a quarter, at sixteen it is ahead by one).
 bool thin_applies(const Geometry &g, int rows, long long positions, long long depth, long long nph) {
   const int rg = thin_row_groups(rows, (int)nph);
+  // (the packed filters take up to 128 bytes per element of the contraction and are addressed
+  // with 32-bit offsets like everything else)
   return thin_on() && g.dtype == MG_F32 && rg != 0 && fits_buffer_loads(g) && positions >= (nph * rg == 1 ? 4 : 1) * 65536 &&
-         !tiny_table(g, rows, depth);
+         depth < (1 << 23) && !tiny_table(g, rows, depth);
 }
 
 // One gathered element of a thin plan: its coordinate offsets and, per phase, the filter tap it
