@@ -572,6 +572,57 @@ def test_forward_pass_with_up_to_four_filters(abi, dtype, case):
         assert rel_err(other, direct.conv_forward(x, w, s, p, d)) <= tol
 
 
+def _random_thin_case(rng, m, rows_are_channels):
+    """A random problem with few rows (channels for the data gradient, filters for the forward
+    pass) and enough positions for the one-position-per-lane kernel: strides of 1 or 2 (1, 2 or 4
+    stride phases, or more: then the other kernels run), windows of 1 to 5, dilation, padding."""
+    few = int(rng.integers(1, 5))
+    many = int(rng.choice([8, 16, 20, 33]))
+    C, F = (few, many) if rows_are_channels else (many, few)
+    taps = tuple(int(v) for v in rng.integers(1, 6 if m < 3 else 4, m))
+    dil = tuple(int(v) for v in rng.integers(1, 3, m))
+    stride = tuple(int(v) for v in rng.integers(1, 3, m))
+    pad = tuple(int(v) for v in rng.integers(0, 3, m))
+    grid = tuple(int(v) for v in rng.integers(20, {1: 600, 2: 70, 3: 24}[m], m))
+    X = tuple((g - 1) * s + (t - 1) * d + 1 - 2 * p + int(rng.integers(0, s)) for g, s, t, d, p in zip(grid, stride, taps, dil, pad))
+    if any(v < 1 for v in X):
+        return None
+    coarse = int(np.prod([-(-v // s) for v, s in zip(X, stride)])) if rows_are_channels else int(np.prod(grid))
+    # enough positions, and enough work not to be planned as a problem of a few microseconds
+    N = max(-(-300000 // coarse), -(-120_000_000 // (2 * coarse * C * F * int(np.prod(taps)))))
+    if N * max(C, F) * int(np.prod(X)) > 60_000_000:
+        return None
+    return (N, C, *X), (F, C, *taps), stride, pad, dil
+
+
+@pytest.mark.parametrize("m", [1, 2, 3])
+@pytest.mark.parametrize("which", ["data gradient, few channels", "forward, few filters"])
+def test_random_problems_with_few_rows(abi, m, which):
+    rows_are_channels = which.startswith("data")
+    rng = np.random.default_rng(2500 + 10 * m + rows_are_channels)
+    done = 0
+    while done < 8:
+        case = _random_thin_case(rng, m, rows_are_channels)
+        if case is None:
+            continue
+        x_shape, w_shape, s, p, d = case
+        print("thin case", which, x_shape, w_shape, s, p, d, flush=True)
+        w = (rng.standard_normal(w_shape) / np.sqrt(np.prod(w_shape[1:]))).astype(np.float32)
+        wi = (np.arange(np.prod(w_shape)).reshape(w_shape) % 11 - 5).astype(np.float32)
+        if rows_are_channels:
+            grid = direct.conv_forward(np.zeros(x_shape, dtype=np.float32), w, s, p, d).shape
+            g = rng.standard_normal(grid).astype(np.float32)
+            assert rel_err(abi.conv_dgrad(g, x_shape, w, s, p, d), direct.conv_backward_x(g, x_shape, w, s, p, d)) <= 2e-4
+            gi = rng.integers(-2, 3, grid).astype(np.float32)
+            assert np.array_equal(abi.conv_dgrad(gi, x_shape, wi, s, p, d), direct.conv_backward_x(gi, x_shape, wi, s, p, d).astype(np.float32))
+        else:
+            x = rng.standard_normal(x_shape).astype(np.float32)
+            assert rel_err(abi.conv_fwd(x, w, s, p, d), direct.conv_forward(x, w, s, p, d)) <= 2e-4
+            xi = rng.integers(-2, 3, x_shape).astype(np.float32)
+            assert np.array_equal(abi.conv_fwd(xi, wi, s, p, d), direct.conv_forward(xi, wi, s, p, d).astype(np.float32))
+        done += 1
+
+
 # Shapes picked so that, between them, every tile shape and code path of the tap-major
 # kernels runs: all gather-GEMM tiles (rows 16..128), persistent blocks that stream
 # through several tiles and K slices, strided dgrad phases, filter counts that are not a
