@@ -137,6 +137,10 @@ int mg_event_destroy(void *event);
  * 9 element-wise kernel, 10 whole-array sum. */
 int mg_timing_enable(int on);
 int mg_timing_read(int32_t *tags, float *ms, int capacity, int *count);
+/* Suspends (1) or resumes (0) the recording without waiting for the stream and without
+ * dropping what was recorded: an event costs a few microseconds of stream time, so a caller
+ * that times a long run may record a sample of its steps and let the others run untouched. */
+int mg_timing_pause(int paused);
 
 /* Device diagnostic, no counterpart in the reference: the rate at which the
  * matrix cores retire one MFMA instruction shape when nothing else is in their way

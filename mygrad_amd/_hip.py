@@ -130,6 +130,7 @@ _SIGNATURES = {
     "mg_memset_zero": [_vp, ctypes.c_size_t],
     "mg_sync": [],
     "mg_timing_enable": [ctypes.c_int],
+    "mg_timing_pause": [ctypes.c_int],
     "mg_timing_read": [ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_float), ctypes.c_int,
                        ctypes.POINTER(ctypes.c_int)],
     "mg_probe_mfma": [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)],
@@ -283,6 +284,11 @@ KERNEL_TAGS = {
 def timing_enable(on=True):
     """Start (or stop) bracketing every kernel launch with HIP events."""
     check(lib().mg_timing_enable(1 if on else 0))
+
+
+def timing_pause(paused=True):
+    """Suspend / resume the recording of launches without waiting for the stream."""
+    check(lib().mg_timing_pause(1 if paused else 0))
 
 
 def timing_read(capacity=1 << 16):

@@ -73,6 +73,7 @@ struct TimingRecord {
 };
 struct Timing {
   bool on = false;
+  bool paused = false;             // on, but the launches of the moment are not recorded
   std::vector<hipEvent_t> events;  // created once and reused
   std::vector<TimingRecord> records;
   size_t used_events = 0, used = 0;
@@ -101,7 +102,7 @@ bool record_next_event(size_t *index) {
 }  // namespace
 
 void timing_begin(int tag) {
-  if (!g_timing.on) return;
+  if (!g_timing.on || g_timing.paused) return;
   const unsigned long long call = g_api_calls.load();
   g_timing.open_tag = tag;
   if (g_timing.chain && call - g_timing.chain_call <= 1) {
@@ -518,6 +519,15 @@ int mg_timing_enable(int on) {
   MG_HIP(hipStreamSynchronize(runtime().stream));
   timing_reset();
   g_timing.on = on != 0;
+  g_timing.paused = false;
+  return MG_OK;
+}
+
+int mg_timing_pause(int paused) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  g_timing.paused = paused != 0;
+  g_timing.chain = false;  // whatever is enqueued while paused lies between the last event and the next
   return MG_OK;
 }
 

@@ -830,3 +830,36 @@ def test_mfma_probe_reports_plausible_rates():
     assert quad > wide
     with pytest.raises(_hip.HipError):
         _hip.probe_mfma("f32_16x16x4", 9)
+
+
+def test_per_launch_timing_records_chains_and_pauses():
+    """``mg_timing_enable`` / ``mg_timing_read`` give one (kernel, milliseconds) record per timed
+    launch, in order; ``mg_timing_pause`` suspends the recording without dropping what was
+    recorded (what bench.py uses to time a sample of its steps)."""
+    import mygrad_amd as mg
+    from mygrad_amd import _hip
+
+    a = mg.device_tensor(np.ones((256, 1024), dtype=np.float32))
+    b = mg.device_tensor(np.full((256, 1024), 2.0, dtype=np.float32))
+    with mg.no_autodiff:
+        _hip.timing_enable(True)
+        try:
+            mg.multiply(a, b)
+            _hip.timing_pause(True)
+            for _ in range(3):
+                mg.multiply(a, b)
+            _hip.timing_pause(False)
+            mg.multiply(a, b)
+            mg.multiply(a, b)
+            records = _hip.timing_read()
+        finally:
+            _hip.timing_enable(False)
+    assert [k for k, _ in records] == ["elementwise"] * 3
+    assert all(0.0 < ms < 5.0 for _, ms in records)
+    with mg.no_autodiff:
+        mg.multiply(a, b)  # timing off: nothing is recorded, nothing is left over
+    _hip.timing_enable(True)
+    try:
+        assert _hip.timing_read() == []
+    finally:
+        _hip.timing_enable(False)
