@@ -2031,11 +2031,13 @@ int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
     const size_t packed_bytes = ((size_t)pl.table_count * ld * sizeof(T) + 255) & ~size_t(255);
     if (int rc = workspace(packed_bytes + tail_bytes(pl, sizeof(T)), &packed)) return rc;
     partial = static_cast<char *>(packed) + packed_bytes;
-    ScopedTiming timed(TAG_PACK_FILTERS);
-    const unsigned blocks = (unsigned)std::min<long long>(ceil_div((long long)pl.table_count * ld, 256), 4096);
-    hipLaunchKernelGGL(pack_rows_kernel<T>, dim3(blocks), dim3(256), 0, runtime().stream, static_cast<const T *>(w),
-                       static_cast<T *>(packed), pl.arow, pl.table_count, (int)g.C, (int)g.wvol, ld);
-    MG_HIP(hipGetLastError());
+    if (pl.table_count > 0) {  // no phase may have a tap at all (an axis of one element that every window steps over): dx is zero
+      ScopedTiming timed(TAG_PACK_FILTERS);
+      const unsigned blocks = (unsigned)std::min<long long>(ceil_div((long long)pl.table_count * ld, 256), 4096);
+      hipLaunchKernelGGL(pack_rows_kernel<T>, dim3(blocks), dim3(256), 0, runtime().stream, static_cast<const T *>(w),
+                         static_cast<T *>(packed), pl.arow, pl.table_count, (int)g.C, (int)g.wvol, ld);
+      MG_HIP(hipGetLastError());
+    }
   } else if (int rc = pack_filters<T>(g, w, pl.fold_row ? 4 : 3, &packed, tail_bytes(pl, sizeof(T)), &partial)) {
     return rc;
   }

@@ -572,6 +572,27 @@ def test_forward_pass_with_up_to_four_filters(abi, dtype, case):
         assert rel_err(other, direct.conv_forward(x, w, s, p, d)) <= tol
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("filters", [10, 16])
+def test_conv_whose_windows_step_over_the_only_row(abi, dtype, filters):
+    """An axis of one element, padded by one, under a one-element window with stride 2: the
+    windows sit on the two padding rows and never on x.  The output is zero, dw is zero, and dx
+    is zero because no stride phase has a tap (the data gradient's tables are empty) -- on a
+    problem large enough to be planned like any other."""
+    x_shape, w_shape, s, p, d = (64, 20, 1, 2048), (filters, 20, 1, 3), (2, 1), (1, 1), (1, 1)
+    rng = np.random.default_rng(2600 + filters)
+    x = rng.standard_normal(x_shape).astype(dtype)
+    w = rng.standard_normal(w_shape).astype(dtype)
+    out = abi.conv_fwd(x, w, s, p, d)
+    assert out.shape == (64, filters, 2, 2048) and not out.any()
+    g = rng.standard_normal(out.shape).astype(dtype)
+    dx = abi.conv_dgrad(g, x_shape, w, s, p, d)
+    assert dx.shape == x_shape and not dx.any()
+    assert not direct.conv_backward_x(g, x_shape, w, s, p, d).any()
+    dw = abi.conv_wgrad(g, x, w_shape, s, p, d)
+    assert dw.shape == w_shape and not dw.any()
+
+
 def _random_thin_case(rng, m, rows_are_channels):
     """A random problem with few rows (channels for the data gradient, filters for the forward
     pass) and enough positions for the one-position-per-lane kernel: strides of 1 or 2 (1, 2 or 4
