@@ -274,10 +274,20 @@ def _random_case(rng, m, big):
     return (N, C, *X), (F, C, *taps), stride, pad, dil
 
 
+@pytest.fixture(params=["small problems planned as such", "planned like large ones"])
+def plan_mode(request, monkeypatch):
+    """A convolution of a few microseconds is planned for few launches (table-driven kernels
+    that read the filter bank in place); MYGRAD_HIP_TINY=0 plans it like a large one, which
+    is how shapes this small reach the tap-major kernels' edge cases."""
+    if request.param == "planned like large ones":
+        monkeypatch.setenv("MYGRAD_HIP_TINY", "0")
+    return request.param
+
+
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
 @pytest.mark.parametrize("m", [1, 2, 3])
 @pytest.mark.parametrize("big", [False, True])
-def test_conv_random_cases_vs_oracle(abi, dtype, m, big):
+def test_conv_random_cases_vs_oracle(abi, dtype, m, big, plan_mode):
     rng = np.random.default_rng(400 + 10 * m + big)
     tol = TOL[np.dtype(dtype)]
     done = 0
@@ -297,16 +307,6 @@ def test_conv_random_cases_vs_oracle(abi, dtype, m, big):
         assert rel_err(abi.conv_dgrad(g, x_shape, w, s, p, d), direct.conv_backward_x(g, x_shape, w, s, p, d)) <= tol
         assert rel_err(abi.conv_wgrad(g, x, w_shape, s, p, d), direct.conv_backward_w(g, x, w_shape, s, p, d)) <= tol
         done += 1
-
-
-@pytest.fixture(params=["small problems planned as such", "planned like large ones"])
-def plan_mode(request, monkeypatch):
-    """A convolution of a few microseconds is planned for few launches (table-driven kernels
-    that read the filter bank in place); MYGRAD_HIP_TINY=0 plans it like a large one, which
-    is how shapes this small reach the tap-major kernels' edge cases."""
-    if request.param == "planned like large ones":
-        monkeypatch.setenv("MYGRAD_HIP_TINY", "0")
-    return request.param
 
 
 @pytest.mark.parametrize("dtype", [np.float64, np.float32])
@@ -570,6 +570,48 @@ def test_forward_pass_with_up_to_four_filters(abi, dtype, case):
         finally:
             del os.environ["MYGRAD_HIP_THIN"]
         assert rel_err(other, direct.conv_forward(x, w, s, p, d)) <= tol
+
+
+def _random_medium_case(rng, m):
+    """A random problem of 0.12 - 3 GFLOP: large enough to be planned like the benchmark's
+    layers (whichever family its channel and filter counts select), small enough for the oracle."""
+    C = int(rng.choice([1, 3, 8, 16, 20, 32, 48, 64]))
+    F = int(rng.choice([2, 4, 10, 16, 24, 32, 64, 96]))
+    taps = tuple(int(v) for v in rng.integers(1, 6 if m < 3 else 4, m))
+    dil = tuple(int(v) for v in rng.integers(1, 3, m))
+    stride = tuple(int(v) for v in rng.integers(1, 4, m))
+    pad = tuple(int(v) for v in rng.integers(0, 3, m))
+    grid = tuple(int(v) for v in rng.integers(6, {1: 900, 2: 60, 3: 20}[m], m))
+    X = tuple((g - 1) * s + (t - 1) * d + 1 - 2 * p + int(rng.integers(0, s)) for g, s, t, d, p in zip(grid, stride, taps, dil, pad))
+    if any(v < 1 for v in X):
+        return None
+    per_sample = 2 * int(np.prod(grid)) * C * F * int(np.prod(taps))
+    N = max(1, -(-150_000_000 // per_sample))
+    if N > 512 or N * per_sample > 3_000_000_000 or N * max(C * int(np.prod(X)), F * int(np.prod(grid))) > 50_000_000:
+        return None
+    return (N, C, *X), (F, C, *taps), stride, pad, dil
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("m", [1, 2, 3])
+def test_conv_random_problems_of_benchmark_size(abi, dtype, m):
+    rng = np.random.default_rng(2700 + m)
+    tol = TOL[np.dtype(dtype)]
+    done = 0
+    while done < 10:
+        case = _random_medium_case(rng, m)
+        if case is None:
+            continue
+        x_shape, w_shape, s, p, d = case
+        print("medium case", np.dtype(dtype).name, x_shape, w_shape, s, p, d, flush=True)
+        x = rng.standard_normal(x_shape).astype(dtype)
+        w = (rng.standard_normal(w_shape) / np.sqrt(np.prod(w_shape[1:]))).astype(dtype)
+        want = direct.conv_forward(x, w, s, p, d)
+        g = rng.standard_normal(want.shape).astype(dtype)
+        assert rel_err(abi.conv_fwd(x, w, s, p, d), want) <= tol
+        assert rel_err(abi.conv_dgrad(g, x_shape, w, s, p, d), direct.conv_backward_x(g, x_shape, w, s, p, d)) <= tol
+        assert rel_err(abi.conv_wgrad(g, x, w_shape, s, p, d), direct.conv_backward_w(g, x, w_shape, s, p, d)) <= tol
+        done += 1
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
