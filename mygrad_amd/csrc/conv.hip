@@ -1027,10 +1027,12 @@ bool thin_on() {
   return !(flag && flag[0] == '0');
 }
 
-// Groups of four rows the kernel would run `rows` as (a power of two), 0 if it has no such shape.
+// Groups of four rows the kernel would run `rows` as (a power of two; more than 64 rows without
+// stride phases: sixteen per pass), 0 if it has no such shape.
 int thin_row_groups(int rows, int nph) {
   int rg = 1;
-  while (rg * 4 < rows) rg *= 2;
+  while (rg * 4 < rows && rg < 16) rg *= 2;
+  if (rg * 4 < rows && nph != 1) return 0;
   return (nph == 1 || nph == 2 || nph == 4) && thin_gemm_has(nph, rg) ? rg : 0;
 }
 
@@ -1106,8 +1108,8 @@ void thin_tables(Plan &pl, Tables &t, const std::vector<ThinUse> &uses, int nph,
 
 int build_fwd_plan(const Geometry &g, Plan &pl) {
   Tables t;
-  if ((g.F <= 4 || (g.F <= 64 && g.C % gemm_bk(g.dtype) != 0)) && thin_applies(g, g.F, (long long)g.N * g.gvol, (long long)g.C * g.wvol, 1)) {
-    // up to four filters, or a first layer (channels that fill no K tile, up to 64 filters), in
+  if ((g.F <= 4 || (g.F <= 1024 && g.C % gemm_bk(g.dtype) != 0)) && thin_applies(g, g.F, (long long)g.N * g.gvol, (long long)g.C * g.wvol, 1)) {
+    // up to four filters, or a first layer (channels that fill no K tile; passes of 64 filters), in
     // single precision: one output position per lane
     const int qs[3] = {g.X[1] * g.X[2], g.X[2], 1};
     std::vector<ThinUse> uses;
@@ -1903,12 +1905,13 @@ int pack_filters(const Geometry &g, const void *w, int mode, void **packed, size
 // register-sized groups, then one position per lane.
 int run_thin(const Plan &pl, ThinParams &tp, const void *w, int tag) {
   void *packed = nullptr;
-  const size_t a_bytes = (size_t)pl.thin_chunks * pl.thin_kgroups * 256;
-  if (int rc = workspace(a_bytes, &packed)) return rc;
+  const size_t a_bytes = (size_t)pl.thin_chunks * pl.thin_kgroups * 256;  // per pass
+  const int passes = (int)ceil_div(tp.M, 4 * pl.thin_rg);
+  if (int rc = workspace(a_bytes * passes, &packed)) return rc;
   {
     ScopedTiming timed(TAG_PACK_FILTERS);
     if (int rc = launch_thin_pack(static_cast<const float *>(w), static_cast<float *>(packed), pl.arow, pl.thin_chunks, pl.thin_kgroups,
-                                  pl.thin_w_group, pl.thin_w_mstride, tp.M, pl.thin_rg, runtime().stream))
+                                  pl.thin_w_group, pl.thin_w_mstride, tp.M, pl.thin_rg, passes, runtime().stream))
       return rc;
   }
   tp.A = static_cast<const float *>(packed);
@@ -1928,6 +1931,8 @@ int run_thin(const Plan &pl, ThinParams &tp, const void *w, int tag) {
   tp.by_jvol = pl.thin_grid.by_jvol, tp.by_j12 = pl.thin_grid.by_j12, tp.by_j2 = pl.thin_grid.by_j2;
   tp.nph = pl.nph;
   tp.rg = pl.thin_rg;
+  tp.passes = passes;
+  tp.pass_floats = (long long)(a_bytes / 4);
   for (int k = 0; k < 3; ++k) tp.J[k] = pl.thin_grid.J[k];
   for (int f = 0; f < pl.nph; ++f)
     for (int k = 0; k < 3; ++k) {

@@ -154,7 +154,10 @@ struct ThinParams {
   int dst_mstride;
   long long src_nstride, dst_nstride;
   int nph;          // 1, 2 or 4 stride phases per position
-  int rg;           // groups of four rows (M <= 4 * rg), nph * rg <= 16
+  int rg;           // groups of four rows per pass, nph * rg <= 16
+  int passes;       // blocks of 4 * rg rows (grid.y); M <= 4 * rg * passes.  Pass y reads the packed filters
+                    // from A + y * pass_floats and writes rows 4 * rg * y ...
+  long long pass_floats;
   int po0[4][3];    // destination coordinate of position (0,0,0) in phase f
   int pJ[4][3];     // positions j_k < pJ[f][k] exist in phase f
   int pair_store;   // phases 2q and 2q+1 are neighbours along the last axis of dst, stored as one 8-byte piece
@@ -162,7 +165,7 @@ struct ThinParams {
 
 // conv_thin.hip
 int launch_thin_pack(const float *w, float *packed, const int *arow, int chunks, int kgroups, long long group_stride, int m_stride, int M,
-                     int rg, hipStream_t s);
+                     int rg, int passes, hipStream_t s);
 int launch_thin_gemm(const ThinParams &p, hipStream_t s);
 bool thin_gemm_has(int nph, int rg);
 

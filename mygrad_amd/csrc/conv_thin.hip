@@ -81,7 +81,10 @@ __global__ void __launch_bounds__(256) thin_gemm_kernel(ThinParams p) {
   const unsigned src_at =
       (unsigned)(((long long)n * p.src_nstride + (long long)c0 * p.qs[0] + (long long)c1 * p.qs[1] + (long long)c2 * p.qs[2]) * 4);
 
-  const __amdgpu_buffer_rsrc_t a_buf = buffer_of(p.A, p.a_bytes);
+  // a pass is a block of 4 * RG rows: its own packed filters, its own rows of dst
+  const int pass = blockIdx.y;
+  const int rows_left = p.M - pass * 4 * RG;
+  const __amdgpu_buffer_rsrc_t a_buf = buffer_of(p.A + (long long)pass * p.pass_floats, p.a_bytes);
   const __amdgpu_buffer_rsrc_t src_buf = buffer_of(p.src, p.src_bytes);
   const int4v MG_CONSTANT *tab = (const int4v MG_CONSTANT *)p.tab;
 
@@ -176,7 +179,7 @@ __global__ void __launch_bounds__(256) thin_gemm_kernel(ThinParams p) {
 
   if constexpr (NACC >= 8) asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");  // the last MFMAs' results are written before they are read
   if (!active) return;
-  float *const dst_n = p.dst + (long long)n * p.dst_nstride;
+  float *const dst_n = p.dst + (long long)n * p.dst_nstride + (long long)pass * 4 * RG * p.dst_mstride;
 #pragma unroll
   for (int ph = 0; ph < NPH; ++ph) {
     const bool here = (int)j0 < p.pJ[ph][0] && (int)j1 < p.pJ[ph][1] && (int)j2 < p.pJ[ph][2];
@@ -189,7 +192,7 @@ __global__ void __launch_bounds__(256) thin_gemm_kernel(ThinParams p) {
         for (int r = 0; r < RG; ++r)
 #pragma unroll
           for (int m = 0; m < 4; ++m)
-            if (r * 4 + m < p.M)
+            if (r * 4 + m < rows_left)
               *reinterpret_cast<f32x2 *>(dst_n + (long long)(r * 4 + m) * p.dst_mstride + o) = f32x2{acc[ph * RG + r][m], acc[(ph | 1) * RG + r][m]};
       }
     } else if (here) {
@@ -197,33 +200,39 @@ __global__ void __launch_bounds__(256) thin_gemm_kernel(ThinParams p) {
       for (int r = 0; r < RG; ++r)
 #pragma unroll
         for (int m = 0; m < 4; ++m)
-          if (r * 4 + m < p.M) dst_n[(long long)(r * 4 + m) * p.dst_mstride + o] = acc[ph * RG + r][m];
+          if (r * 4 + m < rows_left) dst_n[(long long)(r * 4 + m) * p.dst_mstride + o] = acc[ph * RG + r][m];
     }
   }
 }
 
-// packed[(q * kgroups + kg) * 64 + slot * 4 + m] = w[arow[q * 16 + slot] + kg * group_stride + m * m_stride]
-// (zero where arow is negative or the slot's row group, slot % rg, ends before row m)
+// packed[((pass * chunks + q) * kgroups + kg) * 64 + slot * 4 + m] =
+//     w[arow[q * 16 + slot] + kg * group_stride + (pass * 4 * rg + m) * m_stride]
+// (zero where arow is negative or the slot's row group, slot % rg, ends before that row)
 __global__ void __launch_bounds__(256) thin_pack_kernel(const float *__restrict__ w, float *__restrict__ packed, const int *__restrict__ arow,
-                                                        int chunks, int kgroups, long long group_stride, int m_stride, int M, int rg) {
-  const long long total = (long long)chunks * kgroups * 64;
+                                                        int chunks, int kgroups, long long group_stride, int m_stride, int M, int rg,
+                                                        int passes) {
+  const long long per_pass = (long long)chunks * kgroups * 64;
+  const long long total = per_pass * passes;
   for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long long)gridDim.x * 256) {
-    const int m = (int)(i & 3), slot = (int)((i >> 2) & 15);
-    const long long qk = i >> 6;
+    const int pass = (int)(i / per_pass);
+    const long long j = i - (long long)pass * per_pass;
+    const int m = (int)(j & 3), slot = (int)((j >> 2) & 15);
+    const long long qk = j >> 6;
     const int q = (int)(qk / kgroups), kg = (int)(qk - (long long)q * kgroups);
     const int row = arow[q * 16 + slot];
-    packed[i] = (row >= 0 && (slot % rg) * 4 + m < M) ? w[row + kg * group_stride + (long long)m * m_stride] : 0.f;
+    const int first = pass * 4 * rg;  // first row of the pass; the slot's group starts (slot % rg) * 4 rows further on
+    packed[i] = (row >= 0 && first + (slot % rg) * 4 + m < M) ? w[row + kg * group_stride + (long long)(first + m) * m_stride] : 0.f;
   }
 }
 
 }  // namespace
 
 int launch_thin_pack(const float *w, float *packed, const int *arow, int chunks, int kgroups, long long group_stride, int m_stride, int M,
-                     int rg, hipStream_t s) {
-  const long long total = (long long)chunks * kgroups * 64;
+                     int rg, int passes, hipStream_t s) {
+  const long long total = (long long)chunks * kgroups * 64 * passes;
   const unsigned blocks = (unsigned)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
   hipLaunchKernelGGL(thin_pack_kernel, dim3(blocks ? blocks : 1), dim3(256), 0, s, w, packed, arow, chunks, kgroups, group_stride, m_stride, M,
-                     rg);
+                     rg, passes);
   hipError_t err = hipGetLastError();
   return err == hipSuccess ? MG_OK : hip_fail(err, "thin_pack_kernel", __FILE__, __LINE__);
 }
@@ -244,7 +253,7 @@ int launch_thin_gemm(const ThinParams &p, hipStream_t s) {
   bool launched = false;
 #define MG_THIN_LAUNCH(NPH, RG)                                                               \
   if (p.nph == NPH && p.rg == RG) {                                                            \
-    hipLaunchKernelGGL((thin_gemm_kernel<NPH, RG>), dim3(blocks), dim3(256), 0, s, p);         \
+    hipLaunchKernelGGL((thin_gemm_kernel<NPH, RG>), dim3(blocks, (unsigned)p.passes), dim3(256), 0, s, p); \
     launched = true;                                                                           \
   }
   MG_THIN_SHAPES(MG_THIN_LAUNCH)

@@ -538,7 +538,8 @@ def test_data_gradient_with_up_to_four_channels(abi, dtype, case):
 
 
 # Up to four filters in single precision (a layer that ends in one map or in the three colours
-# of an image): the forward pass on the same kernel, one output position per lane.
+# of an image), or a first layer (channels that fill no K tile): the forward pass on the same
+# kernel, one output position per lane.
 THIN_FILTER_CASES = [
     ((64, 16, 64, 64), (3, 16, 3, 3), (1, 1), (1, 1), (1, 1)),
     ((256, 64, 64, 64), (1, 64, 1, 1), (1, 1), (0, 0), (1, 1)),     # one tap: sixteen channels per chunk
@@ -546,6 +547,9 @@ THIN_FILTER_CASES = [
     ((4, 6, 20, 64, 64), (2, 6, 3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),
     ((128, 48, 2048), (3, 48, 5), (1,), (4,), (2,)),
     ((64, 9, 64, 64), (4, 9, 5, 5), (1, 1), (2, 2), (1, 1)),        # 25 taps, 9 channels: one channel per group, chunks padded
+    # a first layer with more than 64 filters: passes of 64 rows over the same positions
+    ((128, 3, 64, 64), (96, 3, 4, 4), (2, 2), (1, 1), (1, 1)),      # a pass of 64 and one of 32
+    ((64, 1, 64, 64), (130, 1, 3, 3), (1, 1), (1, 1), (1, 1)),      # three passes, two rows in the last
 ]
 
 
