@@ -1,7 +1,8 @@
 // Gather-GEMM with one position per lane, for convolutions whose rows come in few groups of
 // four: the data gradient of a layer with a handful of channels (the first layer of an image
 // network), the forward pass of a layer with a handful of filters, and the forward pass of a
-// first layer itself (up to 64 filters over one or three channels).  Single precision.
+// first layer itself (one or three channels; more than 64 filters in passes of 64).  Single
+// precision.
 //
 // A 16-row MFMA tile would carry 3 or 4 live rows of such a data gradient, and K tiles of 16
 // suit 3 channels badly.  v_mfma_f32_4x4x1_16b_f32 multiplies
