@@ -178,7 +178,10 @@ __global__ void __launch_bounds__(256) thin_gemm_kernel(ThinParams p) {
     }
   }
 
-  if constexpr (NACC >= 8) asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");  // the last MFMAs' results are written before they are read
+  // The compiler does not know that the statements above are MFMAs, whose results may be read
+  // only a few cycles after issue: sixteen idle cycles before the epilogue (whose reads of the
+  // accumulators lie behind the branches on `active` and on the phase's extent).
+  if constexpr (NACC >= 8) asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
   if (!active) return;
   float *const dst_n = p.dst + (long long)n * p.dst_nstride + (long long)pass * 4 * RG * p.dst_mstride;
 #pragma unroll
