@@ -72,6 +72,15 @@ WORKLOADS = {
                             recompute=True),
     "pool5-recompute": dict(kind="pool", dtype="f32", seed=1006, x=(8, 32, 32, 64, 64), pool=(2, 2, 2),
                             stride=(2, 2, 2), recompute=True),
+    # The neighbours of configurations 2, 3b and 4 that the reference's validator accepts (an exact
+    # window grid: pooling.py:79-86, conv.py:63-74): what max_pool() / conv_nd() can be called with.
+    "pool2-valid": dict(kind="pool", dtype="f64", seed=1002, x=(64, 64, 55, 55), pool=(3, 3), stride=(2, 2)),
+    "pool2-valid-recompute": dict(kind="pool", dtype="f64", seed=1002, x=(64, 64, 55, 55), pool=(3, 3), stride=(2, 2),
+                                  recompute=True),
+    "conv3b-valid": dict(kind="conv", dtype="f32", seed=1004, x=(128, 128, 27, 27), w=(256, 128, 3, 3),
+                         wscale=(2 / 1152) ** 0.5, stride=(2, 2), padding=(1, 1), dilation=(1, 1)),
+    "conv4-valid": dict(kind="conv", dtype="f64", seed=1005, x=(16, 32, 127, 128), w=(32, 32, 5, 5), wscale=800 ** -0.5,
+                        stride=(2, 1), padding=(4, 4), dilation=(2, 2)),
     # relu, multiply and sum (forward and gradients) on a tensor of conv5's output size
     "elem5": dict(kind="elem", dtype="f32", seed=1007, x=(8, 32, 32, 64, 64)),
     # batch normalisation (scaled and shifted) of a tensor of conv3a's output size
@@ -100,7 +109,62 @@ WORKLOADS = {
 }
 NP_DTYPE = {"f32": np.float32, "f64": np.float64}
 # the configurations of the hot path itself: reported by every default run
-HOT_PATH = ["conv3a", "conv3b", "conv4", "conv5", "conv1", "pool2", "pool5", "pool2-recompute", "pool5-recompute"]
+HOT_PATH = ["conv3a", "conv3b", "conv4", "conv5", "conv1", "pool2", "pool5", "pool2-recompute", "pool5-recompute",
+            "pool2-valid", "pool2-valid-recompute", "conv3b-valid", "conv4-valid"]
+
+
+def _sweep_shapes():
+    """Reference-valid shapes around the benchmark's: what `--sweep` runs, pass by pass."""
+    he = lambda w: (2.0 / (w[1] * int(np.prod(w[2:])))) ** 0.5
+    shapes = {}
+
+    def conv(name, dtype, x, w, stride, padding, dilation):
+        m = len(x) - 2
+        as_tuple = lambda v: (v,) * m if isinstance(v, int) else tuple(v)
+        shapes[name] = dict(kind="conv", dtype=dtype, seed=2000 + len(shapes), x=x, w=w, wscale=he(w), stride=as_tuple(stride),
+                            padding=as_tuple(padding), dilation=as_tuple(dilation))
+
+    def pool(name, dtype, x, window, stride):
+        for suffix, extra in (("", {}), ("-recompute", {"recompute": True})):
+            shapes[name + suffix] = dict(kind="pool", dtype=dtype, seed=2100 + len(shapes), x=x, pool=window,
+                                         stride=(stride,) * len(window), **extra)
+
+    # 3x3, stride 1, padding 1: the stages of a residual network
+    conv("c3x3-64@56", "f32", (128, 64, 56, 56), (64, 64, 3, 3), 1, 1, 1)
+    conv("c3x3-128@28", "f32", (128, 128, 28, 28), (128, 128, 3, 3), 1, 1, 1)
+    conv("c3x3-256@14", "f32", (128, 256, 14, 14), (256, 256, 3, 3), 1, 1, 1)
+    conv("c3x3-512@7", "f32", (128, 512, 7, 7), (512, 512, 3, 3), 1, 1, 1)
+    conv("c3x3-64@56-f64", "f64", (64, 64, 56, 56), (64, 64, 3, 3), 1, 1, 1)
+    # 3x3, stride 2, padding 1 on the odd extents an exact grid needs
+    conv("c3x3s2-64@55", "f32", (128, 64, 55, 55), (128, 64, 3, 3), 2, 1, 1)
+    conv("c3x3s2-128@27", "f32", (128, 128, 27, 27), (256, 128, 3, 3), 2, 1, 1)
+    conv("c3x3s2-256@13", "f32", (128, 256, 13, 13), (512, 256, 3, 3), 2, 1, 1)
+    # 1x1: the bottleneck's two ends, and a strided shortcut
+    conv("c1x1-256to64@56", "f32", (128, 256, 56, 56), (64, 256, 1, 1), 1, 0, 1)
+    conv("c1x1-64to256@56", "f32", (128, 64, 56, 56), (256, 64, 1, 1), 1, 0, 1)
+    conv("c1x1s2-256to512@55", "f32", (128, 256, 55, 55), (512, 256, 1, 1), 2, 0, 1)
+    # 5x5, dilation 2
+    conv("c5x5d2-64@56", "f32", (32, 64, 56, 56), (64, 64, 5, 5), 1, 4, 2)
+    conv("c5x5d2s21-32@127-f64", "f64", (16, 32, 127, 128), (32, 32, 5, 5), (2, 1), 4, 2)
+    # three convolved axes
+    conv("c3x3x3-16to32@32x64x64", "f32", (8, 16, 32, 64, 64), (32, 16, 3, 3, 3), 1, 1, 1)
+    conv("c3x3x3-32to64@16x32x32", "f32", (8, 32, 16, 32, 32), (64, 32, 3, 3, 3), 1, 1, 1)
+    # pooling: 3x3 every other position (odd extents), 2x2 tiling, overlapping 3-D windows
+    pool("p3x3s2@55-f64", "f64", (64, 64, 55, 55), (3, 3), 2)
+    pool("p3x3s2@55-f32", "f32", (128, 64, 55, 55), (3, 3), 2)
+    pool("p3x3s2@113-f32", "f32", (32, 64, 113, 113), (3, 3), 2)
+    pool("p3x3s2@113-f64", "f64", (16, 64, 113, 113), (3, 3), 2)
+    pool("p2x2s2@14-f32", "f32", (128, 512, 14, 14), (2, 2), 2)
+    pool("p2x2s2@28-f32", "f32", (128, 256, 28, 28), (2, 2), 2)
+    pool("p2x2s2@112-f32", "f32", (32, 64, 112, 112), (2, 2), 2)
+    pool("p2x2s2@14-f64", "f64", (128, 256, 14, 14), (2, 2), 2)
+    pool("p3x3x3s2@33x65x65-f32", "f32", (4, 32, 33, 65, 65), (3, 3, 3), 2)
+    pool("p2x2x2s2@32x64x64-f32", "f32", (8, 32, 32, 64, 64), (2, 2, 2), 2)
+    return shapes
+
+
+SWEEP = _sweep_shapes()
+WORKLOADS.update(SWEEP)
 
 
 def conv_grid(wl):
@@ -355,8 +419,28 @@ class Step:
             # pair runs: remembering the argmax moves fewer bytes than that in the backward pass
             self.work = {"maxpool_fwd": float(x.nbytes + g.nbytes), "maxpool_bwd": float(2 * x.nbytes + g.nbytes)}
             self.total_work = sum(self.work.values())
+            # what the pair that keeps the argmax has to move: forward x, out and one byte per window,
+            # backward those bytes, grad and dx -- x is not read again
+            if self.argmax is not None:
+                self.moved = {"maxpool_fwd": float(x.nbytes + g.nbytes + g.size), "maxpool_bwd": float(g.size + g.nbytes + x.nbytes)}
             self.unit, self.bound, self.peak = "GB/s", "hbm", PEAK_HBM_GBS
             self.scale = 1e-9
+
+    def passes(self):
+        """(label, callable, key of the pass in self.work) for each pass of a convolution or pooling step."""
+        lib, check, d = self.lib, self.check, self.desc
+        if self.wl["kind"] == "conv":
+            out = [("fwd", lambda: check(lib.mg_conv_fwd(d, self.x.ptr, self.w.ptr, self.out.ptr)), "conv_fwd")]
+            if not self.wl.get("constant_input"):
+                out.append(("dx", lambda: check(lib.mg_conv_dgrad(d, self.g.ptr, self.w.ptr, self.dx.ptr)), "conv_dgrad"))
+            out.append(("dw", lambda: check(lib.mg_conv_wgrad(d, self.g.ptr, self.x.ptr, self.dw.ptr)), "conv_wgrad"))
+            return out
+        assert self.wl["kind"] == "pool", self.wl["kind"]
+        if self.argmax is None:
+            return [("fwd", lambda: check(lib.mg_maxpool_fwd(d, self.x.ptr, self.out.ptr)), "maxpool_fwd"),
+                    ("bwd", lambda: check(lib.mg_maxpool_bwd(d, self.x.ptr, self.g.ptr, self.dx.ptr)), "maxpool_bwd")]
+        return [("fwd", lambda: check(lib.mg_maxpool_fwd_argmax(d, self.x.ptr, self.out.ptr, self.argmax.ptr)), "maxpool_fwd"),
+                ("bwd", lambda: check(lib.mg_maxpool_bwd_argmax(d, self.argmax.ptr, self.g.ptr, self.dx.ptr)), "maxpool_bwd")]
 
     def __call__(self):
         lib, check = self.lib, self.check
@@ -482,11 +566,18 @@ def run_gpu(name, steps, warmup, prewarm=None, time_every=None):
     # the ceiling the kernels are priced against (a workload may quote its throughput in flops
     # and still be bound by HBM)
     roof = getattr(step, "roof", None) or dict(bound=step.bound, work=step.work, scale=step.scale, unit=step.unit, peak=step.peak)
+    # A pooling pair that keeps the argmax does not read x again in its backward pass: it is priced on
+    # the bytes it has to move, not on the stateless definition's |x| + |grad| + |dx| (kept beside it).
+    moved = getattr(step, "moved", None)
+    if moved:
+        roof = dict(roof, work=moved)
     for k, info in kernels.items():
         if k in roof["work"]:
             info["achieved"] = roof["work"][k] * roof["scale"] / (info["avg_ms"] * 1e-3)
             info["unit"] = roof["unit"]
             info["frac"] = info["achieved"] / roof["peak"]
+            if moved:
+                info["on_definition_bytes"] = step.work[k] * roof["scale"] / (info["avg_ms"] * 1e-3)
     dominant = max((k for k in kernels if k in roof["work"]), key=lambda k: kernels[k]["avg_ms"] * kernels[k]["launches"])
     dom = kernels[dominant]
     ms_per_step = elapsed * 1e3 / steps
@@ -497,8 +588,13 @@ def run_gpu(name, steps, warmup, prewarm=None, time_every=None):
         # of the algorithmic bytes (the pool backward pass that routes from the recorded argmax)
         extra["moved"] = traffic * roof["scale"] / (dom["avg_ms"] * 1e-3)
         extra["moved_frac"] = extra["moved"] / roof["peak"]
+    total = sum(moved.values()) if moved else step.total_work
+    if moved:
+        extra["priced_on"] = "bytes the argmax-keeping pair has to move (x, out, one byte per window; bytes, grad, dx)"
+        extra["on_definition_bytes"] = dom["on_definition_bytes"]
     return {
-        "value": step.total_work * step.scale / (elapsed / steps),
+        "value": total * step.scale / (elapsed / steps),
+        **({"value_on_definition_bytes": step.total_work * step.scale / (elapsed / steps)} if moved else {}),
         "unit": step.unit,
         "ms_per_step": ms_per_step,
         "kernel_ms_per_step": float(sum(np.sum(v) for v in per_kernel.values()) / timed_steps),
@@ -518,6 +614,109 @@ def run_gpu(name, steps, warmup, prewarm=None, time_every=None):
         },
         "kernels": kernels,
     }
+
+
+def short_plan(note):
+    """The kernel family, tile and K split out of a plan note of the library."""
+    import re
+
+    m = re.match(r"(\w+): (.*?) tile (\d+x\d+x\d+), (\d+) phase\(s\) \((\d+) fused per tile\).*K splits (\d+)", note)
+    if not m:
+        return note.split(": ", 1)[-1]
+    family, tile, phases, fused, splits = m.group(2), m.group(3), int(m.group(4)), int(m.group(5)), int(m.group(6))
+    extra = (f", {phases} phases" + (f" ({fused} fused)" if fused > 1 else "")) if phases > 1 else ""
+    return f"{family} {tile}{extra}" + (f", {splits} K splits" if m.group(1) == "wgrad" else "")
+
+
+def run_sweep(names, steps=20, prewarm=0.25):
+    """Every pass of every shape on its own: the plan the library chose, the time of `steps`
+    back-to-back calls by the host clock (stream drained on both sides) and the kernels' own
+    time by HIP events, as a share of the roofline that bounds the pass."""
+    from mygrad_amd import _hip
+
+    rows = []
+    for name in names:
+        step = Step(name)
+        wl = step.wl
+        t_end = time.perf_counter() + prewarm
+        while time.perf_counter() < t_end:
+            for _ in range(5):
+                step()
+            _hip.synchronize()
+        work_of = getattr(step, "moved", None) or step.work
+        for label, fn, key in step.passes():
+            fn()
+            plan = _hip.last_plan()
+            _hip.synchronize()
+            _hip.timing_enable(True)
+            for _ in range(steps):
+                fn()
+            records = _hip.timing_read()
+            _hip.timing_enable(False)
+            kernel_ms = sum(ms for _, ms in records) / steps
+            reps = steps
+            while True:
+                _hip.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(reps):
+                    fn()
+                _hip.synchronize()
+                elapsed = time.perf_counter() - t0
+                if elapsed >= 0.02 or reps >= 2000:
+                    break
+                reps *= 4
+            host_ms = elapsed / reps * 1e3
+            work = work_of[key]
+            rows.append({
+                "shape": name, "dtype": wl["dtype"], "kind": wl["kind"], "pass": label, "plan": plan, "launches": len(records) / steps,
+                "host_us": host_ms * 1e3, "kernel_us": kernel_ms * 1e3, "work": work, "unit": step.unit,
+                "achieved": work * step.scale / (host_ms * 1e-3), "frac": work * step.scale / (host_ms * 1e-3) / step.peak,
+                "kernel_frac": work * step.scale / (kernel_ms * 1e-3) / step.peak,
+                "small": wl["kind"] == "conv" and min(wl["x"][1], wl["w"][0]) < 32,
+            })
+        del step
+    return rows
+
+
+def sweep_table(rows):
+    """The sweep as text: one line per pass, then one per pooling pair, then the outliers."""
+    lines = ["shape                          dtype pass  host us  kernels us  launches  achieved        % of roofline (host clock / kernels)  plan",
+             "-" * 170]
+    for r in rows:
+        lines.append(f"{r['shape']:<30} {r['dtype']:<5} {r['pass']:<4} {r['host_us']:>8.1f} {r['kernel_us']:>11.1f} {r['launches']:>9.1f}  "
+                     f"{r['achieved']:>8.1f} {r['unit']:<8} {100 * r['frac']:>6.1f} / {100 * r['kernel_frac']:<6.1f}"
+                     f"                          {short_plan(r['plan'])}")
+    lines += ["", "pooling pairs (forward + backward, bytes each pair has to move / time by the host clock):"]
+    pairs = {}
+    for r in rows:
+        if r["kind"] == "pool":
+            pairs.setdefault(r["shape"], []).append(r)
+    outliers = []
+    for shape, both in pairs.items():
+        work, us = sum(r["work"] for r in both), sum(r["host_us"] for r in both)
+        frac = work * 1e-9 / (us * 1e-6) / PEAK_HBM_GBS
+        lines.append(f"  {shape:<34} {work / 1e6:>8.1f} MB in {us:>7.1f} us = {work * 1e-9 / (us * 1e-6):>7.0f} GB/s = {100 * frac:5.1f} % of {PEAK_HBM_GBS:.0f} GB/s")
+        if frac < 0.65:
+            outliers.append(f"  {shape}: pair at {100 * frac:.1f} % (bar 65 %)")
+    for r in rows:
+        if r["kind"] == "conv" and not r["small"] and r["frac"] < 0.60:
+            outliers.append(f"  {r['shape']} {r['pass']}: {100 * r['frac']:.1f} % (bar 60 %)")
+    lines += ["", "below the bar (convolution passes with C, F >= 32 under 60 % of the MFMA peak, pooling pairs under 65 % of HBM):"]
+    lines += outliers or ["  none"]
+    return "\n".join(lines)
+
+
+def compact_summary(line):
+    """value and the dominant kernel's share of its roofline for the headline workload and every
+    secondary one, short enough to survive a truncated record of the JSON line."""
+    out = {}
+    for name, entry in [(line["config"]["workload"].split(":")[0], line)] + list(line.get("secondary", {}).items()):
+        roof = entry["roofline"]
+        item = [round(entry["value"], 1 if entry["unit"] == "TFLOP/s" else 0), round(roof["frac"], 3)]
+        if "value_on_definition_bytes" in entry:
+            item.append("moved")
+        out[name] = item
+    return out
 
 
 def measured_traffic(workload, kernel):
@@ -983,6 +1182,10 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a 1 GiB device copy (the reference point for HBM traffic counters)")
     ap.add_argument("--copy-mib", type=int, default=1024, help="size of the --calibrate-copy buffer in MiB (read + written)")
+    ap.add_argument("--sweep", action="store_true",
+                    help="run only the sweep over reference-valid shapes around the benchmark's, pass by pass: a text "
+                         "table on stdout (what profiles/sweep_hotpath.txt holds), the rows as one JSON line on stderr")
+    ap.add_argument("--sweep-only", default="", help="with --sweep: only the shapes whose name contains this text")
     ap.add_argument("--probe-mfma", action="store_true",
                     help="run only the matrix-core rate probe (registers only, per MFMA shape)")
     args = ap.parse_args()
@@ -996,6 +1199,11 @@ def main():
         return
     if args.probe_mfma:
         print(json.dumps(run_mfma_probe()))
+        return
+    if args.sweep:
+        rows = run_sweep([n for n in SWEEP if args.sweep_only in n], steps=args.steps)
+        print(sweep_table(rows))
+        print(json.dumps({"sweep": rows}), file=sys.stderr)
         return
 
     wl = WORKLOADS[args.workload]
@@ -1030,7 +1238,7 @@ def main():
     if not args.no_secondary:
         # the other half of the metric (max_pool GB/s) and the other convolution configurations,
         # each with its own roofline and a short CPU baseline
-        names = list(WORKLOADS) if args.all else HOT_PATH
+        names = [n for n in WORKLOADS if n not in SWEEP] if args.all else HOT_PATH
         secondary = {}
         for name in names:
             if name == args.workload:
@@ -1045,6 +1253,7 @@ def main():
                 entry["dropin"] = run_dropin(name)
             secondary[name] = entry
         line["secondary"] = secondary
+    line["summary"] = compact_summary(line)  # last: the end of the line is what a truncated record keeps
     print(json.dumps(line))
 
 

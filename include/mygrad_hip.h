@@ -103,6 +103,8 @@ typedef struct {
 int mg_init(int device);           /* idempotent; picks the device, creates the stream */
 int mg_shutdown(void);             /* frees the stream, workspace and cached plans */
 const char *mg_last_error(void);   /* message of this thread's last failing call */
+const char *mg_last_plan(void);    /* diagnostics: the kernel family, tile and split that the most recent mg_conv_* or
+                                      mg_maxpool_* call ran on; valid until the next call into the library */
 int mg_device_info(mg_device_info_t *info);
 
 /* Device memory.  A block given back with mg_free is kept by the library and handed out again

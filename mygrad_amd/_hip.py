@@ -173,7 +173,7 @@ _SIGNATURES = {
                         ctypes.c_int, _vp, _vp],
     "mg_permute": [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int32), _vp, _vp],
 }
-EXPORTED_SYMBOLS = tuple(_SIGNATURES) + ("mg_last_error",)
+EXPORTED_SYMBOLS = tuple(_SIGNATURES) + ("mg_last_error", "mg_last_plan")
 
 _lock = threading.Lock()
 _lib = None
@@ -208,12 +208,19 @@ def load_library():
                 fn.restype = ctypes.c_int
             lib.mg_last_error.argtypes = []
             lib.mg_last_error.restype = ctypes.c_char_p
+            lib.mg_last_plan.argtypes = []
+            lib.mg_last_plan.restype = ctypes.c_char_p
             _lib = lib
     return _lib
 
 
 def last_error():
     return load_library().mg_last_error().decode("utf-8", "replace")
+
+
+def last_plan():
+    """Which kernel family, tile and split the most recent conv / pool call ran on (diagnostics)."""
+    return lib().mg_last_plan().decode("utf-8", "replace")
 
 
 def check(status):

@@ -602,6 +602,7 @@ struct Plan {
   // wgrad
   int splits = 1;
   int kchunk = 0;
+  char note[200] = "";  // what mg_last_plan() reports after a call that ran this plan
 };
 
 std::map<std::string, Plan> &plans() {
@@ -1704,15 +1705,20 @@ int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
     Plan pl;
     int rc = op == OP_FWD ? build_fwd_plan(g, pl) : op == OP_DGRAD ? build_dgrad_plan(g, pl) : build_wgrad_plan(g, pl);
     if (rc) return rc;
+    snprintf(pl.note, sizeof pl.note,
+             "%s: %s%s%s tile %dx%dx%d, %d phase(s) (%d fused per tile), %d position blocks x %d row tiles, %d whole tiles + tail split %d, "
+             "%d block(s) per unit, K splits %d",
+             op == OP_FWD ? "fwd" : op == OP_DGRAD ? "dgrad" : "wgrad",
+             pl.thin ? "one position per lane" : pl.tap_major ? "tap-major" : "table-driven", pl.table_rows ? ", table rows" : "",
+             pl.fold_row ? ", folded taps" : "", pl.bm, pl.bn, pl.bk, pl.nphases, pl.nph, pl.pos_blocks, pl.m_tiles, pl.full_tiles,
+             pl.tail_split, pl.blocks_per_cu, pl.splits);
     // MYGRAD_HIP_TRACE=1 reports, once per new descriptor, what was planned
     static const bool trace = getenv("MYGRAD_HIP_TRACE") != nullptr;
-    if (trace)
-      fprintf(stderr, "[mygrad_hip] %s plan: %s tile %dx%d, %d phase(s) (%d fused per tile), %d position blocks x %d row tiles, %d whole tiles + tail split %d, %d block(s) per unit, K splits %d (chunk %d)\n",
-              op == OP_FWD ? "fwd" : op == OP_DGRAD ? "dgrad" : "wgrad", pl.thin ? "one position per lane" : pl.tap_major ? "tap-major" : "table-driven", pl.bm,
-              pl.bn, pl.nphases, pl.nph, pl.pos_blocks, pl.m_tiles, pl.full_tiles, pl.tail_split, pl.blocks_per_cu, pl.splits, pl.kchunk);
+    if (trace) fprintf(stderr, "[mygrad_hip] plan %s (K chunk %d)\n", pl.note, pl.kchunk);
     it = plans().emplace(key, pl).first;
   }
   *out = &it->second;
+  note_plan(it->second.note);
   return MG_OK;
 }
 
@@ -2186,6 +2192,7 @@ int conv_wgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
 }  // namespace
 
 void release_conv_plans() {
+  note_plan("");  // it may point into a plan
   for (auto &kv : plans())
     if (kv.second.blob) (void)hipFree(kv.second.blob);
   plans().clear();

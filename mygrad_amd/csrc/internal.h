@@ -71,6 +71,10 @@ struct ScopedTiming {
   ~ScopedTiming() { timing_end(); }
 };
 
+// Remembers which kernel family (and tile) the entry point that is running chose: what
+// mg_last_plan() returns.  `text` must outlive the next call (a literal, or a cached plan's note).
+void note_plan(const char *text);
+
 // Drops every cached convolution plan (device tables); called by mg_shutdown.
 void release_conv_plans();
 

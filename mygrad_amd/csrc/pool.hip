@@ -478,23 +478,25 @@ __global__ void __launch_bounds__(256) maxpool_tile_kernel(PoolTileParams p, con
 // slab -- 16 / (P2 * sizeof(T)) whole windows -- straight from global memory, reduces
 // them in registers and stores 16-byte pieces of dx (or its share of out).  Consecutive
 // lanes take consecutive pieces: every access of a wave is one contiguous run.
+// float32 rows that are whole 8-byte but not whole 16-byte pieces (14, 30, ... columns under
+// two-column windows) take pieces of 8 bytes, one window wide (VEC = 2).
 // ------------------------------------------------------------------------------------------
 struct PoolExactParams {
   int X1, X2;            // extents of the two inner pooled axes
   int G0, G1;            // windows along the two outer pooled axes
-  int pieces;            // 16-byte pieces per row of x
+  int vec;               // elements per piece: 16 bytes, or 8 bytes for float32 rows of 4k + 2 columns
+  int pieces;            // pieces per row of x
   long long xvol, gvol;  // elements of x / windows per leading index
   long long total;       // work items: lead * G0 * G1 * pieces
   FastDivP by_pieces, by_g1, by_g0;
 };
 
-template <typename T, typename TD, int P0, int P1, int P2, bool BWD, bool MARK = false>
+template <typename T, typename TD, int P0, int P1, int P2, bool BWD, bool MARK = false, int VEC = 16 / sizeof(T)>
 __global__ void __launch_bounds__(256) maxpool_exact_kernel(PoolExactParams p, const T *__restrict__ x,
                                                             const T *__restrict__ grad, void *__restrict__ result,
                                                             unsigned char *__restrict__ mark = nullptr) {
-  constexpr int VEC = 16 / sizeof(T);
   constexpr int WPT = VEC / P2;  // windows per thread
-  static_assert(VEC % P2 == 0 && WPT >= 1, "a 16-byte piece holds whole windows");
+  static_assert(VEC % P2 == 0 && WPT >= 1, "a piece holds whole windows");
   typedef T Vec __attribute__((ext_vector_type(VEC)));
   typedef T WVec __attribute__((ext_vector_type(WPT)));
   const long long item = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -669,11 +671,18 @@ __global__ void __launch_bounds__(256) maxpool_from_mark_kernel(PoolMarkParams p
 // (the next wavefront starts on its piece again).  A window that would need columns of the next
 // row does not exist.  Every element of x crosses HBM once (rows shared by two window rows come
 // the second time out of L1 / L2); nothing is staged.
-// Needs X2 % VEC == 0, VEC % S2 == 0, P2 - S2 <= VEC and rows of x that start 16-byte aligned.
+// Pieces are counted in columns, not in addresses: a row need not start on a 16-byte boundary
+// (the loads only assume the alignment of an element), and a row that is no whole number of
+// pieces ends in a short one of `tail` columns.  The lane of a short piece loads the last VEC
+// columns of the row instead and moves its own to the front, so no load leaves the row; what is
+// then behind them belongs to no window.  An exact window grid over 3 x 3 windows placed every
+// other column always has an odd last extent, i.e. such rows.
+// Needs VEC % S2 == 0, P2 - S2 <= VEC and X2 >= VEC.
 #define POOL_ROWS_PER_THREAD 3
 struct PoolRowsParams {
   int X1, X2, G1, G2;
-  int pieces;        // 16-byte pieces per row of x
+  int pieces;        // 16-byte pieces per row of x, the short one included
+  int tail;          // columns of the short piece (X2 % VEC); 0: none
   int groups;        // groups of POOL_ROWS_PER_THREAD window rows per plane
   long long planes;  // lead * X0
   long long items;   // planes * groups * pieces: one per (group of window rows, piece)
@@ -694,7 +703,7 @@ __global__ void __launch_bounds__(256) maxpool_rows_fwd_kernel(PoolRowsParams p,
   constexpr int RW = POOL_ROWS_PER_THREAD;   // window rows per thread: the rows two of them share are loaded once
   constexpr int NR = (RW - 1) * S1 + P1;     // rows of x under them
   static_assert(VEC % S2 == 0 && HALO >= 0 && HALO <= VEC, "piece / window geometry");
-  typedef T Vec __attribute__((ext_vector_type(VEC)));
+  typedef T Vec __attribute__((ext_vector_type(VEC), aligned(sizeof(T))));
   const int lane = threadIdx.x & 63;
   const long long wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
   const long long item = wave * 63 + lane;  // wavefronts overlap by one lane
@@ -702,7 +711,8 @@ __global__ void __launch_bounds__(256) maxpool_rows_fwd_kernel(PoolRowsParams p,
   const unsigned q = p.by_pieces.div(u), piece = u - q * (unsigned)p.pieces;
   const unsigned plane = p.by_groups.div(q);
   const int g1_first = (int)(q - plane * (unsigned)p.groups) * RW;
-  const T *rows = x + (long long)plane * p.X1 * p.X2 + (int)piece * VEC;
+  const bool short_piece = p.tail != 0 && (int)piece == p.pieces - 1;
+  const T *rows = x + (long long)plane * p.X1 * p.X2 + (short_piece ? p.X2 - VEC : (int)piece * VEC);
   const int row_first = g1_first * S1;
   T v[NR][VEC + HALO];
 #pragma unroll
@@ -711,6 +721,19 @@ __global__ void __launch_bounds__(256) maxpool_rows_fwd_kernel(PoolRowsParams p,
     const Vec mine = *reinterpret_cast<const Vec *>(rows + (long long)min(row_first + r, p.X1 - 1) * p.X2);
 #pragma unroll
     for (int i = 0; i < VEC; ++i) v[r][i] = mine[i];
+  }
+  if (p.tail != 0) {
+    // a short piece's own columns are the last `tail` of what it loaded
+#pragma unroll
+    for (int r = 0; r < NR; ++r)
+#pragma unroll
+      for (int i = 0; i < VEC - 1; ++i) {
+        T moved = v[r][i];
+#pragma unroll
+        for (int k = i + 1; k < VEC; ++k)
+          if (p.tail == k) moved = v[r][i + VEC - k];
+        v[r][i] = short_piece ? moved : v[r][i];
+      }
   }
 #pragma unroll
   for (int r = 0; r < NR; ++r)
@@ -751,11 +774,14 @@ __global__ void __launch_bounds__(256) maxpool_rows_fwd_kernel(PoolRowsParams p,
 // whichever thread -- so their recorded offsets and gradients are loaded up front (clamped, never
 // predicated), and every element adds, in ascending window order, the gradient of the windows
 // whose recorded offset names it and +0.0 for the others: no loop bounds to compute, no
-// divisions by runtime values, no LDS.  Needs X2 % VD == 0 and VD % S2 == 0 (a piece starts on a
-// window boundary).
+// divisions by runtime values, no LDS.  Needs VD % S2 == 0 (a piece starts on a window boundary).
+// Pieces are counted in columns: rows of dx need not start on 16-byte boundaries (the stores only
+// assume the alignment of an element), and the short piece at the end of a row that is no whole
+// number of pieces is stored element by element.
 struct PoolGatherParams {
   int X1, X2, G1, G2;
-  int pieces;        // 16-byte pieces per row of dx
+  int pieces;        // 16-byte pieces per row of dx, the short one included
+  int tail;          // columns of the short piece (X2 % VD); 0: none
   int groups;        // groups of S1 rows per plane: ceil(X1 / S1)
   long long planes;  // lead * X0
   FastDivP by_pieces, by_groups;
@@ -768,7 +794,7 @@ __global__ void __launch_bounds__(256) maxpool_mark_gather_kernel(PoolGatherPara
   constexpr int C1 = (P1 + S1 - 1) / S1, C2 = (P2 + S2 - 1) / S2;
   constexpr int NW2 = (VD - 1) / S2 + C2;  // windows along the row that can reach the piece
   static_assert(VD % S2 == 0, "a piece starts on a window boundary");
-  typedef TD DVec __attribute__((ext_vector_type(VD)));
+  typedef TD DVec __attribute__((ext_vector_type(VD), aligned(sizeof(TD))));
   const long long item = (long long)blockIdx.x * 256 + threadIdx.x;
   if (item >= p.planes * p.groups * p.pieces) return;
   const unsigned u = (unsigned)item;
@@ -776,6 +802,7 @@ __global__ void __launch_bounds__(256) maxpool_mark_gather_kernel(PoolGatherPara
   const unsigned plane = p.by_groups.div(q);
   const int k = (int)(q - plane * (unsigned)p.groups);
   const int i2 = (int)piece * VD;
+  const int live = (p.tail != 0 && (int)piece == p.pieces - 1) ? p.tail : VD;  // columns of this piece
   const unsigned char *m = mark + (long long)plane * (p.G1 * p.G2);
   const T *g = grad + (long long)plane * (p.G1 * p.G2);
   const int g1_first = k - (C1 - 1), g2_first = i2 / S2 - (C2 - 1);
@@ -820,20 +847,25 @@ __global__ void __launch_bounds__(256) maxpool_mark_gather_kernel(PoolGatherPara
       }
       out[v] = (TD)acc;
     }
-    *reinterpret_cast<DVec *>(to + (long long)rr * p.X2) = out;
+    if (live == VD) {
+      *reinterpret_cast<DVec *>(to + (long long)rr * p.X2) = out;
+    } else {
+#pragma unroll
+      for (int v = 0; v < VD - 1; ++v)
+        if (v < live) to[(long long)rr * p.X2 + v] = out[v];
+    }
   }
 }
 
 // The same for windows that tile the input exactly: an element belongs to one window, so a
 // thread reads the recorded offsets and gradients of its 16 / (P2 * sizeof(T)) windows and
 // writes their P0 x P1 rows of dx.
-template <typename T, typename TD, int P0, int P1, int P2>
+template <typename T, typename TD, int P0, int P1, int P2, int VEC = 16 / sizeof(T)>
 __global__ void __launch_bounds__(256) maxpool_exact_from_mark_kernel(PoolExactParams p,
                                                                       const unsigned char *__restrict__ mark,
                                                                       const T *__restrict__ grad, TD *__restrict__ dx) {
-  constexpr int VEC = 16 / sizeof(T);
   constexpr int WPT = VEC / P2;
-  static_assert(VEC % P2 == 0 && WPT >= 1, "a 16-byte piece holds whole windows");
+  static_assert(VEC % P2 == 0 && WPT >= 1, "a piece holds whole windows");
   typedef T WVec __attribute__((ext_vector_type(WPT)));
   typedef TD DVec __attribute__((ext_vector_type(VEC)));
   const long long item = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -1057,11 +1089,15 @@ static int exact_signature(const PoolParams &p, size_t elem, const void *a, cons
     if (p.S[k] != p.P[k] || p.X[k] != p.G[k] * p.P[k]) return 0;
   const int sig = p.P[0] * 100 + p.P[1] * 10 + p.P[2];
   if (sig != 122 && sig != 222) return 0;
-  const int vec = (int)(16 / elem);
-  if (p.X[2] % vec != 0) return 0;
+  int vec = (int)(16 / elem);
+  if (p.X[2] % vec != 0) {
+    if (elem != 4 || p.X[2] % 2 != 0) return 0;
+    vec = 2;
+  }
   const uintptr_t bits = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | reinterpret_cast<uintptr_t>(c);
   if (bits % 16 != 0) return 0;
   (void)c_elem;
+  e->vec = vec;
   e->X1 = p.X[1];
   e->X2 = p.X[2];
   e->G0 = p.G[0];
@@ -1090,9 +1126,9 @@ static bool rows_forward_applies(const PoolParams &p, bool f32, const void *x) {
     return !(flag && flag[0] == '0');
   }();
   const int vec = f32 ? 4 : 2;
-  const long long items = p.lead * p.X[0] * ceil_div(p.G[1], POOL_ROWS_PER_THREAD) * (p.X[2] / vec);
-  return on && has_rows_instance(p) && p.X[2] % vec == 0 && vec % p.S[2] == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
-         items < (1ll << 31);
+  const long long items = p.lead * p.X[0] * ceil_div(p.G[1], POOL_ROWS_PER_THREAD) * ceil_div(p.X[2], vec);
+  return on && has_rows_instance(p) && p.X[2] >= vec && vec % p.S[2] == 0 &&
+         reinterpret_cast<uintptr_t>(x) % (f32 ? 4 : 8) == 0 && items < (1ll << 31);
 }
 
 // out may be null (with mark set): only the argmax offsets are wanted
@@ -1101,7 +1137,8 @@ static int launch_rows_forward(const PoolParams &p, bool f32, const void *x, voi
   const int sig4 = window_signature4(p);
   PoolRowsParams q{};
   q.X1 = p.X[1], q.X2 = p.X[2], q.G1 = p.G[1], q.G2 = p.G[2];
-  q.pieces = p.X[2] / vec;
+  q.pieces = (int)ceil_div(p.X[2], vec);
+  q.tail = p.X[2] % vec;
   q.groups = (int)ceil_div(p.G[1], POOL_ROWS_PER_THREAD);
   q.planes = p.lead * p.X[0];
   q.items = q.planes * q.groups * q.pieces;
@@ -1137,8 +1174,8 @@ static bool mark_gather_applies(const PoolParams &p, bool f32, bool wide, const 
     return !(flag && flag[0] == '0');
   }();
   const int vd = (f32 && !wide) ? 4 : 2;
-  const long long items = p.lead * p.X[0] * ceil_div(p.X[1], p.S[1]) * (p.X[2] / vd);
-  return on && has_rows_instance(p) && p.X[2] % vd == 0 && vd % p.S[2] == 0 && reinterpret_cast<uintptr_t>(dx) % 16 == 0 &&
+  const long long items = p.lead * p.X[0] * ceil_div(p.X[1], p.S[1]) * ceil_div(p.X[2], vd);
+  return on && has_rows_instance(p) && vd % p.S[2] == 0 && reinterpret_cast<uintptr_t>(dx) % (16 / vd) == 0 &&
          items < (1ll << 31) && (long long)p.G[1] * p.G[2] < (1ll << 30);
 }
 
@@ -1148,7 +1185,8 @@ static int launch_mark_gather(const PoolParams &p, bool f32, bool wide, const un
   const int sig4 = window_signature4(p);
   PoolGatherParams q{};
   q.X1 = p.X[1], q.X2 = p.X[2], q.G1 = p.G[1], q.G2 = p.G[2];
-  q.pieces = p.X[2] / vd;
+  q.pieces = (int)ceil_div(p.X[2], vd);
+  q.tail = p.X[2] % vd;
   q.groups = (int)ceil_div(p.X[1], p.S[1]);
   q.planes = p.lead * p.X[0];
   q.by_pieces = make_fastdiv_p((unsigned)q.pieces);
@@ -1186,26 +1224,38 @@ static int maxpool_fwd_impl(const mg_pool_desc *desc, const void *x, void *out, 
   ScopedTiming timed(TAG_POOL_FWD);
   PoolExactParams ep;
   if (const int sig = exact_signature(p, desc->dtype == MG_F32 ? 4 : 8, x, out, mark ? (const void *)mark : out, 0, &ep)) {
+    note_plan(ep.vec * (desc->dtype == MG_F32 ? 4 : 8) == 16 ? "pool fwd: exact tiling, registers, 16-byte pieces"
+                                                            : "pool fwd: exact tiling, registers, 8-byte pieces");
     const dim3 grid((unsigned)ceil_div(ep.total, 256)), block(256);
-#define MG_POOL_EXACT_FWD(T, MK)                                                                              \
-  do {                                                                                                        \
-    if (sig == 122)                                                                                           \
-      hipLaunchKernelGGL((maxpool_exact_kernel<T, T, 1, 2, 2, false, MK>), grid, block, 0, s, ep, (const T *)x, \
-                         (const T *)nullptr, out, mark);                                                      \
-    else                                                                                                      \
-      hipLaunchKernelGGL((maxpool_exact_kernel<T, T, 2, 2, 2, false, MK>), grid, block, 0, s, ep, (const T *)x, \
-                         (const T *)nullptr, out, mark);                                                      \
+#define MG_POOL_EXACT_FWD_V(T, MK, V)                                                                            \
+  do {                                                                                                          \
+    if (sig == 122)                                                                                             \
+      hipLaunchKernelGGL((maxpool_exact_kernel<T, T, 1, 2, 2, false, MK, V>), grid, block, 0, s, ep, (const T *)x, \
+                         (const T *)nullptr, out, mark);                                                        \
+    else                                                                                                        \
+      hipLaunchKernelGGL((maxpool_exact_kernel<T, T, 2, 2, 2, false, MK, V>), grid, block, 0, s, ep, (const T *)x, \
+                         (const T *)nullptr, out, mark);                                                        \
+  } while (0)
+#define MG_POOL_EXACT_FWD(T, MK)                                           \
+  do {                                                                     \
+    if (ep.vec == (int)(16 / sizeof(T))) MG_POOL_EXACT_FWD_V(T, MK, 16 / sizeof(T)); \
+    else MG_POOL_EXACT_FWD_V(T, MK, 2);                                    \
   } while (0)
     if (desc->dtype == MG_F32) {
       if (mark) MG_POOL_EXACT_FWD(float, true); else MG_POOL_EXACT_FWD(float, false);
     } else {
       if (mark) MG_POOL_EXACT_FWD(double, true); else MG_POOL_EXACT_FWD(double, false);
     }
+#undef MG_POOL_EXACT_FWD_V
 #undef MG_POOL_EXACT_FWD
     MG_HIP(hipGetLastError());
     return MG_OK;
   }
-  if (rows_forward_applies(p, desc->dtype == MG_F32, x)) return launch_rows_forward(p, desc->dtype == MG_F32, x, out, mark, s);
+  if (rows_forward_applies(p, desc->dtype == MG_F32, x)) {
+    note_plan(p.X[2] % (desc->dtype == MG_F32 ? 4 : 2) ? "pool fwd: compile-time window, registers, rows with a short piece"
+                                                       : "pool fwd: compile-time window, registers, whole pieces");
+    return launch_rows_forward(p, desc->dtype == MG_F32, x, out, mark, s);
+  }
   PoolTileParams tp;
   int tile_elems = 0, win_slots = 0, acc_offset = 0;
   size_t lds = 0;
@@ -1214,6 +1264,7 @@ static int maxpool_fwd_impl(const mg_pool_desc *desc, const void *x, void *out, 
   if (plan_tiles(p, elem, elem, false, &tp, &tile_elems, &win_slots, &acc_offset, &lds, &blocks)) {
     // one tile per block measured faster than persistent blocks for the forward pass:
     // its stores trail the next tile's loads in the same in-order memory counter
+    note_plan(tp.bands > 1 ? "pool fwd: LDS tiles, bands of rows" : "pool fwd: LDS tiles, whole volumes");
     const dim3 grid((unsigned)blocks), block(256);
     const bool deep = (size_t)tile_elems * elem > 8 * 4096;  // 16-byte loads per thread to cover the tile
     const int sig = pool_signature(p);
@@ -1244,6 +1295,7 @@ static int maxpool_fwd_impl(const mg_pool_desc *desc, const void *x, void *out, 
     MG_HIP(hipGetLastError());
     return MG_OK;
   }
+  note_plan("pool fwd: thread per window, no staging");
   const unsigned grid = grid_for(p.lead * p.gvol);
 #define MG_POOL_FWD_PLAIN(T, MK) \
   hipLaunchKernelGGL((maxpool_fwd_kernel<T, MK>), dim3(grid), dim3(256), 0, s, p, (const T *)x, (T *)out, mark)
@@ -1271,15 +1323,22 @@ static int maxpool_bwd_from_mark(const mg_pool_desc *desc, const unsigned char *
   PoolExactParams ep;
   // the exact-tiling test looks at the alignment of x; grad stands in for it here
   if (const int sig = exact_signature(p, f32 ? 4 : 8, grad, grad, dx, 0, &ep)) {
+    note_plan(ep.vec * (f32 ? 4 : 8) == 16 ? "pool bwd from argmax: exact tiling, registers, 16-byte pieces"
+                                          : "pool bwd from argmax: exact tiling, registers, 8-byte pieces");
     const dim3 grid((unsigned)ceil_div(ep.total, 256)), block(256);
-#define MG_POOL_EXACT_MARK(T, TD)                                                                                  \
-  do {                                                                                                             \
-    if (sig == 122)                                                                                                \
-      hipLaunchKernelGGL((maxpool_exact_from_mark_kernel<T, TD, 1, 2, 2>), grid, block, 0, s, ep, mark, (const T *)grad, \
-                         (TD *)dx);                                                                                \
-    else                                                                                                           \
-      hipLaunchKernelGGL((maxpool_exact_from_mark_kernel<T, TD, 2, 2, 2>), grid, block, 0, s, ep, mark, (const T *)grad, \
-                         (TD *)dx);                                                                                \
+#define MG_POOL_EXACT_MARK_V(T, TD, V)                                                                                \
+  do {                                                                                                               \
+    if (sig == 122)                                                                                                  \
+      hipLaunchKernelGGL((maxpool_exact_from_mark_kernel<T, TD, 1, 2, 2, V>), grid, block, 0, s, ep, mark, (const T *)grad, \
+                         (TD *)dx);                                                                                  \
+    else                                                                                                             \
+      hipLaunchKernelGGL((maxpool_exact_from_mark_kernel<T, TD, 2, 2, 2, V>), grid, block, 0, s, ep, mark, (const T *)grad, \
+                         (TD *)dx);                                                                                  \
+  } while (0)
+#define MG_POOL_EXACT_MARK(T, TD)                                              \
+  do {                                                                         \
+    if (ep.vec == (int)(16 / sizeof(T))) MG_POOL_EXACT_MARK_V(T, TD, 16 / sizeof(T)); \
+    else MG_POOL_EXACT_MARK_V(T, TD, 2);                                       \
   } while (0)
     if (!f32)
       MG_POOL_EXACT_MARK(double, double);
@@ -1287,11 +1346,16 @@ static int maxpool_bwd_from_mark(const mg_pool_desc *desc, const unsigned char *
       MG_POOL_EXACT_MARK(float, double);
     else
       MG_POOL_EXACT_MARK(float, float);
+#undef MG_POOL_EXACT_MARK_V
 #undef MG_POOL_EXACT_MARK
     MG_HIP(hipGetLastError());
     return MG_OK;
   }
-  if (mark_gather_applies(p, f32, wide, dx)) return launch_mark_gather(p, f32, wide, mark, grad, dx, s);
+  if (mark_gather_applies(p, f32, wide, dx)) {
+    note_plan(p.X[2] % ((f32 && !wide) ? 4 : 2) ? "pool bwd from argmax: compile-time window, register gather, rows with a short piece"
+                                                : "pool bwd from argmax: compile-time window, register gather, whole pieces");
+    return launch_mark_gather(p, f32, wide, mark, grad, dx, s);
+  }
   {
     PoolTileParams tp;
     int tile_elems = 0, win_slots = 0, acc_offset = 0;
@@ -1303,6 +1367,7 @@ static int maxpool_bwd_from_mark(const mg_pool_desc *desc, const unsigned char *
     if (plan_tiles(p, elem, acc_elem, true, &tp, &tile_elems, &win_slots, &acc_offset, &lds, &blocks) &&
         lds + (size_t)win_slots + 32 <= 64 * 1024) {
       // the staged bytes go behind everything else; 16 spare bytes for the alignment shift
+      note_plan(tp.bands > 1 ? "pool bwd from argmax: LDS tiles, bands of rows" : "pool bwd from argmax: LDS tiles, whole volumes");
       const int mark_offset = (int)lds;
       lds += ((size_t)win_slots + 16 + 15) & ~size_t(15);
       const dim3 grid(persistent_grid(blocks, lds)), block(256);
@@ -1337,6 +1402,7 @@ static int maxpool_bwd_from_mark(const mg_pool_desc *desc, const unsigned char *
       return MG_OK;
     }
   }
+  note_plan("pool bwd from argmax: thread per 16 bytes of dx, no staging");
   PoolMarkParams q{};
   for (int k = 0; k < 3; ++k) {
     q.X[k] = p.X[k];
@@ -1418,13 +1484,20 @@ int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, vo
   ScopedTiming timed(TAG_POOL_BWD);
   PoolExactParams ep;
   if (const int sig = exact_signature(p, desc->dtype == MG_F32 ? 4 : 8, x, grad, dx, 0, &ep)) {
+    note_plan(ep.vec * (desc->dtype == MG_F32 ? 4 : 8) == 16 ? "pool bwd: exact tiling, registers, 16-byte pieces"
+                                                            : "pool bwd: exact tiling, registers, 8-byte pieces");
     const dim3 grid((unsigned)ceil_div(ep.total, 256)), block(256);
-#define MG_POOL_EXACT_BWD(T, TD)                                                                                        \
-  do {                                                                                                                  \
-    if (sig == 122)                                                                                                     \
-      hipLaunchKernelGGL((maxpool_exact_kernel<T, TD, 1, 2, 2, true>), grid, block, 0, s, ep, (const T *)x, (const T *)grad, dx); \
-    else                                                                                                                \
-      hipLaunchKernelGGL((maxpool_exact_kernel<T, TD, 2, 2, 2, true>), grid, block, 0, s, ep, (const T *)x, (const T *)grad, dx); \
+#define MG_POOL_EXACT_BWD_V(T, TD, V)                                                                                      \
+  do {                                                                                                                    \
+    if (sig == 122)                                                                                                       \
+      hipLaunchKernelGGL((maxpool_exact_kernel<T, TD, 1, 2, 2, true, false, V>), grid, block, 0, s, ep, (const T *)x, (const T *)grad, dx); \
+    else                                                                                                                  \
+      hipLaunchKernelGGL((maxpool_exact_kernel<T, TD, 2, 2, 2, true, false, V>), grid, block, 0, s, ep, (const T *)x, (const T *)grad, dx); \
+  } while (0)
+#define MG_POOL_EXACT_BWD(T, TD)                                              \
+  do {                                                                        \
+    if (ep.vec == (int)(16 / sizeof(T))) MG_POOL_EXACT_BWD_V(T, TD, 16 / sizeof(T)); \
+    else MG_POOL_EXACT_BWD_V(T, TD, 2);                                       \
   } while (0)
     if (desc->dtype == MG_F64)
       MG_POOL_EXACT_BWD(double, double);
@@ -1432,6 +1505,7 @@ int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, vo
       MG_POOL_EXACT_BWD(float, double);
     else
       MG_POOL_EXACT_BWD(float, float);
+#undef MG_POOL_EXACT_BWD_V
 #undef MG_POOL_EXACT_BWD
     MG_HIP(hipGetLastError());
     return MG_OK;
@@ -1441,6 +1515,7 @@ int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, vo
     // two passes straight from global memory: every window's first-occurrence argmax as one
     // byte in the library workspace (x is read, nothing else is written), then the gather
     // from those bytes -- less traffic through LDS than finding and routing in one kernel
+    note_plan("pool bwd: compile-time window, argmax pass + register gather");
     void *marks = nullptr;
     if (int rc = workspace((size_t)(p.lead * p.gvol), &marks)) return rc;
     if (int rc = launch_rows_forward(p, desc->dtype == MG_F32, x, nullptr, (unsigned char *)marks, s)) return rc;
@@ -1458,6 +1533,7 @@ int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, vo
   const bool f32 = desc->dtype == MG_F32;
   const size_t elem = f32 ? 4 : 8, acc_elem = (f32 && !overlap) ? 4 : 8;
   if (plan_tiles(p, elem, acc_elem, true, &tp, &tile_elems, &win_slots, &acc_offset, &lds, &blocks)) {
+    note_plan(tp.bands > 1 ? "pool bwd: LDS tiles, bands of rows" : "pool bwd: LDS tiles, whole volumes");
     const dim3 grid(persistent_grid(blocks, lds)), block(256);
     const bool wide = desc->dx_dtype == MG_F64;
     const bool deep = (size_t)tile_elems * elem > 8 * 4096;
@@ -1497,6 +1573,7 @@ int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, vo
     MG_HIP(hipGetLastError());
     return MG_OK;
   }
+  note_plan("pool bwd: thread per element, no staging");
   const unsigned grid = grid_for(p.lead * p.xvol);
   if (desc->dtype == MG_F64)
     hipLaunchKernelGGL((maxpool_bwd_kernel<double, double>), dim3(grid), dim3(256), 0, s, p, (const double *)x,

@@ -22,6 +22,10 @@ std::recursive_mutex &api_mutex() {
 
 static thread_local char g_error[512] = "";
 
+static const char *g_plan = "";
+
+void note_plan(const char *text) { g_plan = text ? text : ""; }
+
 int fail(int code, const char *fmt, ...) {
   va_list ap;
   va_start(ap, fmt);
@@ -256,6 +260,11 @@ void pool_trim(size_t keep, BlockPool &bp = pool()) {
 extern "C" {
 
 const char *mg_last_error(void) { return g_error; }
+
+const char *mg_last_plan(void) {
+  MG_LOCK();
+  return g_plan;
+}
 
 int mg_init(int device) {
   MG_LOCK();

@@ -114,6 +114,16 @@ def test_pool_ties_and_overlap_bit_exact(pools, m, lead, dtype):
     ((4,), (7, 8), (2, 2), (1, 1)),
     ((2,), (3, 6, 8), (1, 3, 3), (1, 2, 2)),  # a leading pooled axis of extent one folds into the planes
     ((1,), (3, 4), (3, 3), (2, 2)),       # a single window per plane
+    # exact window grids over an odd last extent (what the reference's validator admits for 3 x 3 windows
+    # placed every other column): rows start on no 16-byte boundary and end in a short piece
+    ((3, 2), (11, 15), (3, 3), (2, 2)),
+    ((5,), (55, 55), (3, 3), (2, 2)),     # the valid neighbour of the benchmark's plane
+    ((2,), (5, 7), (3, 3), (2, 2)),       # short pieces of three (float32) and one (float64) columns
+    ((2,), (5, 5), (3, 3), (2, 2)),       # of one column in either precision
+    ((3,), (9, 13), (3, 3), (1, 1)),
+    ((3,), (7, 9), (2, 2), (1, 1)),
+    ((2,), (5, 6), (3, 3), (1, 1)),       # a short piece of two float32 columns
+    ((2,), (3, 3), (3, 3), (2, 2)),       # a float32 row shorter than one piece
 ])
 def test_pool_backward_gather_for_windows_known_at_compile_time(pools, dtype, lead, X, pool, stride):
     """2-D windows of 3x3 / stride 2, 3x3 / stride 1 and 2x2 / stride 1 over rows of whole 16-byte
@@ -144,7 +154,10 @@ def test_pool_backward_gather_for_windows_known_at_compile_time(pools, dtype, le
     ((3, 5), (8, 12), (2, 2)),        # 2-D, rows of whole 16-byte pieces: the exact-tiling kernel
     ((2,), (6, 4, 8), (2, 2, 2)),     # 3-D
     ((7,), (2, 2, 4), (2, 2, 2)),     # a single window slab per volume
-    ((4,), (10, 6), (2, 2)),          # rows that are not whole 16-byte pieces in float32: the tiled kernel
+    ((4,), (10, 6), (2, 2)),          # float32 rows of 4k + 2 columns: pieces of 8 bytes
+    ((3, 2), (14, 14), (2, 2)),
+    ((2,), (4, 6, 10), (2, 2, 2)),
+    ((1,), (2, 2), (2, 2)),           # one window in all
 ])
 def test_pool_windows_that_tile_the_input_exactly(pools, dtype, lead, X, pool):
     """Stride == pool extent and X == G * P: the kernels that work straight from global
@@ -227,6 +240,27 @@ def test_pool_config2_literal_full_size(pools, ties):
     sl = slice(0, 4)
     assert np.array_equal(bits(out[sl]), bits(ora.pool_forward(x[sl], (3, 3), 2, validate=False)))
     assert np.array_equal(bits(dx[sl]), bits(ora.pool_backward(x[sl], g[sl], (3, 3), 2)))
+
+
+@pytest.mark.parametrize("ties", [False, True])
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+def test_pool_config2_valid_full_size(pools, ties, dtype):
+    # the neighbour of config 2 that the reference accepts: x (64,64,55,55), pool 3x3 stride 2 ->
+    # (64,64,27,27) exactly; rows of 55 elements start on no 16-byte boundary
+    rng = np.random.default_rng(1002)
+    shape = (64, 64, 55, 55)
+    x = (rng.integers(0, 8, shape) if ties else rng.standard_normal(shape)).astype(dtype)
+    g = rng.standard_normal((64, 64, 27, 27)).astype(dtype)
+    out = pools.pool_fwd(x, (3, 3), 2)
+    dx = pools.pool_bwd(x, g, (3, 3), 2)
+    dx64 = pools.pool_bwd(x, g, (3, 3), 2, dx_dtype=np.float64)
+    want_out, want_dx = direct.pool(x, g, (3, 3), (2, 2))
+    assert np.array_equal(bits(out), bits(want_out))
+    assert np.array_equal(bits(dx64), bits(want_dx))
+    assert np.array_equal(bits(dx), bits(want_dx.astype(dtype)))
+    sl = slice(0, 4)
+    assert np.array_equal(bits(out[sl]), bits(ora.pool_forward(x[sl], (3, 3), 2)))
+    assert np.array_equal(bits(dx64[sl]), bits(ora.pool_backward(x[sl], g[sl], (3, 3), 2)))
 
 
 def test_pool_config5_shape_full_size(pools):
