@@ -232,6 +232,10 @@ class DeviceArray:
         dtype = np.dtype(dtype)
         if dtype == self.dtype:
             return self
+        if not (_is_storage_type(dtype) and _is_storage_type(self.dtype)):
+            # mg_cast converts between the floating-point storage types only; anything else (the
+            # integer or boolean result of a `repeat`) is converted by NumPy and uploaded again
+            return from_host(np.ascontiguousarray(self.host().astype(dtype)))
         buf = DeviceBuffer(max(self.size * dtype.itemsize, 16))
         _hip.check(_hip.lib().mg_cast(_hip.storage_code(self.dtype), _hip.storage_code(dtype), self.size, self.buf.ptr, buf.ptr))
         return DeviceArray(buf, self.shape, dtype)
@@ -258,9 +262,25 @@ def value_of(tensor):
         return tensor.data
 
 
+def _is_storage_type(dtype):
+    return np.dtype(dtype) in (np.dtype(np.float16), np.dtype(np.float32), np.dtype(np.float64))
+
+
+def from_host(arr):
+    """A C-contiguous host array of any dtype as a DeviceArray (one upload)."""
+    buf = DeviceBuffer(max(arr.nbytes, 16))
+    if arr.nbytes:
+        buf.upload(arr)
+        stats["uploads"] += 1
+    return DeviceArray(buf, arr.shape, arr.dtype)
+
+
 def full(shape, dtype, value):
-    """``np.full(shape, value, dtype)`` made on the device."""
+    """``np.full(shape, value, dtype)`` made on the device (float32, float64; float16 is filled as
+    float32 and narrowed, which is exact for the values that fit)."""
     dtype = np.dtype(dtype)
+    if dtype == np.float16:
+        return full(shape, np.float32, value).astype(np.float16)
     count = int(np.prod(shape, dtype=np.int64))
     buf = DeviceBuffer(max(count * dtype.itemsize, 16))
     _hip.check(_hip.lib().mg_fill_value(_hip.dtype_code(dtype), count, float(value), buf.ptr))

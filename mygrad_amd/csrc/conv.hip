@@ -581,6 +581,11 @@ struct Plan {
   int full_tiles = 0;  // tiles computed whole by one block (tap-major kernel)
   int tail_split = 1;  // blocks sharing each of the remaining tiles
   int blocks_per_cu = 1;  // persistent blocks per compute unit (streaming gather-GEMM)
+  // even shares of the last round (GemmParams::share_first): set by upload_plan when tail_split == 0
+  int *share_first = nullptr;
+  ShareSlice *share_slices = nullptr;
+  ShareFix *share_fix = nullptr;
+  int share_grid = 0, share_slots = 0, share_fixes = 0;
   bool tap_major = false;  // which kernel family the tables are for
   bool single_dense_phase = false;  // positions enumerate the destination tensor in order
   bool table_rows = false;          // tap-major kernel whose K tiles are rows of the gather table (channel count no multiple of the K tile)
@@ -744,13 +749,18 @@ int gemm_blocks_per_cu(int bm, int bn, int nph = 1, int bk = 0) {
 // Smaller tiles give more tiles (finer balance, less padding) at some cost in operand
 // reuse.  Kernels that do not stream run one block per tile (r = 1 in this arithmetic:
 // the hardware refills a unit as soon as a block leaves).
+// Fewest K tiles in a block's share of the leftover tiles (see build_shares).
+constexpr long long kMinRun = 8;
+
 struct TileChoice {
   int bm, bn, m_tiles, full_tiles, tail_split;
   int blocks_per_cu;  // persistent blocks per compute unit (streaming kernels)
   long long tiles;
 };
 
-TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_ktiles, bool tap_major, size_t elem, int nph = 1, int bk = 0) {
+TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_ktiles, bool tap_major, size_t elem, int nph = 1, int bk = 0,
+                       int avg_ktiles = -1) {
+  if (avg_ktiles < 0) avg_ktiles = min_ktiles;  // K tiles of an average tile (phases of a data gradient differ)
   struct Cfg {
     int bm, bn;
     double penalty;  // relative cost of a flop in this tile shape
@@ -762,13 +772,29 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
   static const Cfg fused4[] = {{64, 64, 1.10, true}, {32, 128, 1.10, true}, {16, 256, 1.00, true}};
   const Cfg *cfgs = nph == 4 ? fused4 : nph == 2 ? fused2 : plain;
   const int ncfgs = nph == 4 ? 3 : nph == 2 ? 4 : 7;
-  const int bm = nph == 4 ? std::min(pick_bm(M), 64) : pick_bm(M);
+  // MYGRAD_HIP_TILE="rows,positions[,blocks per unit]" (diagnostics; read once): only that tile shape
+  struct Forced {
+    int bm = 0, bn = 0, r = 0;
+  };
+  static const Forced forced = [] {
+    Forced f;
+    if (const char *v = getenv("MYGRAD_HIP_TILE")) sscanf(v, "%d,%d,%d", &f.bm, &f.bn, &f.r);
+    return f;
+  }();
+  // MYGRAD_HIP_SHARES=0: the last round's tiles are cut into equal K slices instead (the older scheme)
+  static const bool shares_on = [] {
+    const char *flag = getenv("MYGRAD_HIP_SHARES");
+    return !(flag && flag[0] == '0');
+  }();
+  bool forced_fits = false;
+  for (int ci = 0; ci < ncfgs; ++ci) forced_fits |= cfgs[ci].bm == forced.bm && cfgs[ci].bn == forced.bn && (!cfgs[ci].tap_only || tap_major);
+  const int bm = forced_fits ? forced.bm : nph == 4 ? std::min(pick_bm(M), 64) : pick_bm(M);
   const int cus = runtime().props.multiProcessorCount;
   TileChoice best{};
   double best_cost = 0;
   for (int ci = 0; ci < ncfgs; ++ci) {
     const Cfg &c = cfgs[ci];
-    if (c.bm != bm || (c.tap_only && !tap_major)) continue;
+    if (c.bm != bm || (c.tap_only && !tap_major) || (forced_fits && c.bn != forced.bn)) continue;
     // 64x64 fp64 wave tiles hold 128 accumulator registers: only one 8-wave block
     // fits on a compute unit, so the tap-major kernels use the half-size shapes
     if (tap_major && elem == 8 && c.bn * c.bm >= 128 * 128) continue;
@@ -777,6 +803,7 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
     long long pos_blocks = 0;
     for (long long n : phase_npos) pos_blocks += ceil_div(n, c.bn);
     for (int r = 1; r <= per_cu; ++r) {
+      if (forced_fits && forced.r > 0 && r != std::min(forced.r, per_cu)) continue;
       TileChoice t{};
       t.bm = c.bm;
       t.bn = c.bn;
@@ -787,6 +814,45 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
       t.tail_split = 1;
       const long long grid = (long long)r * cus;
       const long long rem = t.tiles % grid;
+      // a streaming block alone on its unit leaves the MFMA pipes idle while it waits
+      // at its barriers; two or more cover for one another
+      const double alone = stream && r == 1 ? 1.4 : 1.0;
+      if (stream && shares_on && t.tiles < 2 * (long long)cus) {
+        // Fewer than two tiles per unit (few positions under many channels: the late stages of a
+        // network).  Equal K slices of the leftover tiles then leave a large part of the device idle
+        // in the last round however they are cut (196 tiles of 288 K tiles on 256 units: 0.85 tile
+        // times at best where 0.77 are due, and measured 1.0), and with more tiles per unit the
+        // slices below lose 1 - 3 % less to their partial sums than the shares do.
+        // Persistent blocks take even shares of what the whole tiles leave over (build_shares).
+        // Blocks b, b + CUs, ... share a unit, so a unit gets the tiles t = b (mod CUs): q = T / CUs
+        // whole tiles, worked off by its r blocks, and the T mod CUs tiles beyond that are shared
+        // out as K tiles: every unit gets (T mod CUs) / CUs tile times of them, whatever the
+        // remainder.  What it costs is the partial sums of the tiles that are cut: about one slice
+        // per run and one more per tile that is cut, written and read once (priced in tile times:
+        // a tile's flops at three quarters of the unit's peak against its bytes at 4 TB/s for the
+        // whole device, plus the fix-up launch).
+        const long long q = t.tiles / cus, left = t.tiles % cus;
+        // (within a unit the r blocks take q / r whole tiles each; if r does not divide q the last
+        // q mod r tiles run with fewer blocks than r, a single one without cover for its barriers)
+        const int over = (int)(q % r);
+        double units = (double)(q / r) * r + (over == 1 && r > 1 ? 1.4 : (double)over) + (double)left / cus;
+        if (left > 0) {
+          t.full_tiles = (int)(q * cus);
+          t.tail_split = 0;  // marks the plan for build_shares
+          const double depth = (double)std::max(avg_ktiles, 1) * (bk > 0 ? bk : (elem == 8 ? 8 : 16));
+          const double tile_seconds = 2.0 * c.bm * c.bn * depth / (0.75 * (elem == 8 ? 78.6e12 : 157.3e12) / cus);
+          const long long runs = std::max<long long>(1, std::min<long long>(grid, left * (long long)std::max(avg_ktiles, 1) / kMinRun));
+          const double slices = (double)(runs - 1) + (double)std::min<long long>(left, runs - 1);
+          const double fix_seconds = slices * c.bm * c.bn * (double)elem * nph * 2.0 / 4.0e12 + 4e-6;
+          units += fix_seconds / tile_seconds;
+        }
+        const double cost = units * alone * c.bm * c.bn * c.penalty;
+        if (best.bm == 0 || cost < best_cost) {
+          best = t;
+          best_cost = cost;
+        }
+        continue;
+      }
       double tail = 0;  // tile times the busiest unit spends on the remaining tiles
       if (rem > 0) {
         tail = (double)ceil_div(rem, cus);
@@ -804,9 +870,6 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
           if (t.tail_split > 1) t.full_tiles = (int)(t.tiles - rem);
         }
       }
-      // a streaming block alone on its unit leaves the MFMA pipes idle while it waits
-      // at its barriers; two or more cover for one another
-      const double alone = stream && r == 1 ? 1.4 : 1.0;
       const double cost = ((double)(t.tiles / grid) * r + tail) * alone * c.bm * c.bn * c.penalty;
       if (best.bm == 0 || cost < best_cost) {
         best = t;
@@ -858,21 +921,107 @@ struct Tables {
   std::vector<Phase> phases;
   std::vector<KTile> ktiles;
   std::vector<WGroup> groups;
+  std::vector<int> share_first;
+  std::vector<ShareSlice> share_slices;
+  std::vector<ShareFix> share_fix;
 };
+
+// Even shares of what the whole tiles leave over: the K tiles of the tiles from pl.full_tiles on,
+// laid end to end, are cut into runs of equal length (to within one K tile; at least kMinRun K
+// tiles each, so at most one run per block), one run per block from the last block down (with
+// full_tiles no multiple of the grid those have one whole tile fewer); a run is cut where it
+// crosses from one tile into the next.  A tile that lies in one run is computed whole and stored
+// directly; the slices of any other leave partial sums in consecutive slots, in K order, which
+// the fix-up pass adds in that order.  Tiles without K tiles (a stride phase that no tap reaches)
+// are all zeros: dealt out one by one, stored directly.
+void build_shares(Plan &pl, Tables &t, int grid) {
+  const long long tiles = (long long)pl.pos_blocks * pl.m_tiles;
+  std::vector<int> kcount;  // K tiles of each tail tile
+  long long total = 0;
+  size_t pi = 0;
+  for (long long tile = pl.full_tiles; tile < tiles; ++tile) {
+    const int pblk = (int)(tile / pl.m_tiles);
+    while (pi + 1 < t.phases.size() && pblk >= t.phases[pi + 1].blk_begin) ++pi;
+    kcount.push_back(t.phases[pi].k_count);
+    total += t.phases[pi].k_count;
+  }
+  const long long runs = std::max<long long>(1, std::min<long long>(grid, total / kMinRun));
+  std::vector<std::vector<ShareSlice>> mine((size_t)grid);
+  std::vector<int> slices_of(kcount.size(), 0);
+  size_t cur = 0;      // tail tile the next run starts in
+  long long done = 0;  // K tiles of that tile that earlier runs took
+  for (long long j = 0; j < runs; ++j) {
+    std::vector<ShareSlice> &list = mine[(size_t)(grid - 1 - j)];
+    long long want = total * (j + 1) / runs - total * j / runs;
+    while (want > 0 && cur < kcount.size()) {
+      if (kcount[cur] == 0) {
+        ++cur;
+        continue;
+      }
+      const long long take = std::min<long long>(want, kcount[cur] - done);
+      list.push_back(ShareSlice{(int)(pl.full_tiles + cur), (int)done, (int)(done + take), 0});
+      ++slices_of[cur];
+      done += take;
+      want -= take;
+      if (done == kcount[cur]) ++cur, done = 0;
+    }
+  }
+  int dealt = 0;
+  for (size_t i = 0; i < kcount.size(); ++i)
+    if (kcount[i] == 0) {
+      mine[(size_t)(grid - 1 - dealt % grid)].push_back(ShareSlice{(int)(pl.full_tiles + i), 0, 0, 0});
+      slices_of[i] = 1;
+      ++dealt;
+    }
+  // slots: a tile's slices lie in consecutive runs, i.e. in descending blocks; numbered in K order
+  std::vector<int> first_slot(kcount.size(), -1);
+  int slots = 0;
+  for (size_t i = 0; i < kcount.size(); ++i)
+    if (slices_of[i] > 1) {
+      first_slot[i] = slots;
+      t.share_fix.push_back(ShareFix{(int)(pl.full_tiles + i), slots, slices_of[i], 0});
+      slots += slices_of[i];
+    }
+  std::vector<int> used(kcount.size(), 0);
+  for (long long b = grid - 1; b >= 0; --b)
+    for (ShareSlice &sl : mine[(size_t)b]) {
+      const size_t i = (size_t)(sl.tile - pl.full_tiles);
+      sl.slot = first_slot[i] < 0 ? -1 : first_slot[i] + used[i]++;
+    }
+  t.share_first.assign(grid + 1, 0);
+  for (int b = 0; b < grid; ++b) {
+    t.share_first[b] = (int)t.share_slices.size();
+    // a block's cursor over the phase table only moves forward: its tiles in ascending order
+    std::stable_sort(mine[(size_t)b].begin(), mine[(size_t)b].end(), [](const ShareSlice &x, const ShareSlice &y) { return x.tile < y.tile; });
+    for (const ShareSlice &sl : mine[(size_t)b]) t.share_slices.push_back(sl);
+  }
+  t.share_first[grid] = (int)t.share_slices.size();
+  pl.share_grid = grid;
+  pl.share_slots = slots;
+  pl.share_fixes = (int)t.share_fix.size();
+}
 
 template <typename V>
 size_t padded_bytes(const V &v) {
   return (v.size() * sizeof(typename V::value_type) + 255) & ~size_t(255);
 }
 
-int upload_plan(Plan &pl, const Tables &t) {
+int upload_plan(Plan &pl, Tables &t) {
+  if (pl.tap_major && pl.tail_split == 0) {
+    const long long tiles = (long long)pl.pos_blocks * pl.m_tiles;
+    if (tiles > pl.full_tiles) build_shares(pl, t, pl.blocks_per_cu * runtime().props.multiProcessorCount);
+  }
+  if (pl.tail_split == 0 && pl.share_grid == 0) pl.tail_split = 1;
   const size_t zero_b = 256;
   const size_t off_tab = zero_b;
   const size_t off_arow = off_tab + padded_bytes(t.tab);
   const size_t off_ph = off_arow + padded_bytes(t.arow);
   const size_t off_kt = off_ph + padded_bytes(t.phases);
   const size_t off_gr = off_kt + padded_bytes(t.ktiles);
-  const size_t total = off_gr + padded_bytes(t.groups) + 256;
+  const size_t off_sf = off_gr + padded_bytes(t.groups);
+  const size_t off_ss = off_sf + padded_bytes(t.share_first);
+  const size_t off_sx = off_ss + padded_bytes(t.share_slices);
+  const size_t total = off_sx + padded_bytes(t.share_fix) + 256;
   std::vector<char> host(total, 0);
   auto put = [&](size_t off, const void *src, size_t n) {
     if (n) memcpy(host.data() + off, src, n);
@@ -882,6 +1031,9 @@ int upload_plan(Plan &pl, const Tables &t) {
   put(off_ph, t.phases.data(), t.phases.size() * sizeof(Phase));
   put(off_kt, t.ktiles.data(), t.ktiles.size() * sizeof(KTile));
   put(off_gr, t.groups.data(), t.groups.size() * sizeof(WGroup));
+  put(off_sf, t.share_first.data(), t.share_first.size() * sizeof(int));
+  put(off_ss, t.share_slices.data(), t.share_slices.size() * sizeof(ShareSlice));
+  put(off_sx, t.share_fix.data(), t.share_fix.size() * sizeof(ShareFix));
   MG_HIP(hipMalloc(&pl.blob, host.size()));
   hipError_t err = hipMemcpy(pl.blob, host.data(), host.size(), hipMemcpyHostToDevice);
   if (err != hipSuccess) {
@@ -896,6 +1048,11 @@ int upload_plan(Plan &pl, const Tables &t) {
   pl.phases = reinterpret_cast<Phase *>(base + off_ph);
   pl.ktiles = reinterpret_cast<KTile *>(base + off_kt);
   pl.groups = reinterpret_cast<WGroup *>(base + off_gr);
+  if (pl.share_grid > 0) {
+    pl.share_first = reinterpret_cast<int *>(base + off_sf);
+    pl.share_slices = reinterpret_cast<ShareSlice *>(base + off_ss);
+    pl.share_fix = reinterpret_cast<ShareFix *>(base + off_sx);
+  }
   pl.nphases = (int)t.phases.size();
   return MG_OK;
 }
@@ -1450,7 +1607,14 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
       const long long ntaps = (long long)pt.taps[0].size() * pt.taps[1].size() * pt.taps[2].size();
       min_ktiles = std::min(min_ktiles, pl.tap_major && !pl.table_rows ? ntaps * (g.F / bk) : ceil_div(ntaps * g.F, bk));
     }
-    const TileChoice tc = choose_tile(g.C, npos, (int)std::max<long long>(min_ktiles, 0), pl.tap_major, g.dtype == MG_F64 ? 8 : 4, 1, bk);
+    long long all_ktiles = 0, all_pos = 0;
+    for (const PhaseTaps &pt : found) {
+      const long long ntaps = (long long)pt.taps[0].size() * pt.taps[1].size() * pt.taps[2].size();
+      all_ktiles += ceil_div(ntaps * g.F, bk) * pt.ph.npos;
+      all_pos += pt.ph.npos;
+    }
+    const TileChoice tc = choose_tile(g.C, npos, (int)std::max<long long>(min_ktiles, 0), pl.tap_major, g.dtype == MG_F64 ? 8 : 4, 1, bk,
+                                      (int)(all_ktiles / std::max<long long>(all_pos, 1)));
     pl.bm = tc.bm, pl.bn = tc.bn, pl.m_tiles = tc.m_tiles, pl.full_tiles = tc.full_tiles, pl.tail_split = tc.tail_split, pl.blocks_per_cu = tc.blocks_per_cu;
     deepen_if_tiny(g, pl);
   }
@@ -1705,13 +1869,18 @@ int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
     Plan pl;
     int rc = op == OP_FWD ? build_fwd_plan(g, pl) : op == OP_DGRAD ? build_dgrad_plan(g, pl) : build_wgrad_plan(g, pl);
     if (rc) return rc;
+    char tail[64];
+    if (pl.share_grid > 0)
+      snprintf(tail, sizeof tail, "even shares of the rest (%d partial slices)", pl.share_slots);
+    else
+      snprintf(tail, sizeof tail, "tail split %d", pl.tail_split);
     snprintf(pl.note, sizeof pl.note,
-             "%s: %s%s%s tile %dx%dx%d, %d phase(s) (%d fused per tile), %d position blocks x %d row tiles, %d whole tiles + tail split %d, "
+             "%s: %s%s%s tile %dx%dx%d, %d phase(s) (%d fused per tile), %d position blocks x %d row tiles, %d whole tiles + %s, "
              "%d block(s) per unit, K splits %d",
              op == OP_FWD ? "fwd" : op == OP_DGRAD ? "dgrad" : "wgrad",
              pl.thin ? "one position per lane" : pl.tap_major ? "tap-major" : "table-driven", pl.table_rows ? ", table rows" : "",
-             pl.fold_row ? ", folded taps" : "", pl.bm, pl.bn, pl.bk, pl.nphases, pl.nph, pl.pos_blocks, pl.m_tiles, pl.full_tiles,
-             pl.tail_split, pl.blocks_per_cu, pl.splits);
+             pl.fold_row ? ", folded taps" : "", pl.bm, pl.bn, pl.bk, pl.nphases, pl.nph, pl.pos_blocks, pl.m_tiles, pl.full_tiles, tail,
+             pl.blocks_per_cu, pl.splits);
     // MYGRAD_HIP_TRACE=1 reports, once per new descriptor, what was planned
     static const bool trace = getenv("MYGRAD_HIP_TRACE") != nullptr;
     if (trace) fprintf(stderr, "[mygrad_hip] plan %s (K chunk %d)\n", pl.note, pl.kchunk);
@@ -1728,6 +1897,16 @@ void launch_gemm(GemmParams &gp, const Plan &pl, hipStream_t s) {
     const long long tiles = (long long)pl.pos_blocks * pl.m_tiles;
     const long long tail_tiles = tiles - pl.full_tiles;
     const long long slots = tap_gemm_streams(BM, (int)sizeof(T)) ? (long long)pl.blocks_per_cu * runtime().props.multiProcessorCount : (1ll << 40);
+    gp.share_first = pl.share_first, gp.share_slices = pl.share_slices, gp.share_fix = pl.share_fix;
+    if (pl.share_grid > 0) {
+      // whole tiles b, b + grid, ... and then one even share of the remaining tiles' K tiles per block
+      gp.items = pl.full_tiles;
+      hipLaunchKernelGGL((tap_gemm_kernel<T, BM, BN, BK, WM, WN, NPH, FOLD, ROWS>), dim3((unsigned)pl.share_grid), dim3(512), 0, s, gp);
+      if (pl.share_fixes > 0)
+        hipLaunchKernelGGL((tail_fixup_kernel<T, BM, BN, NPH>), dim3((unsigned)ceil_div(BM * BN, 256), (unsigned)pl.share_fixes),
+                           dim3(256), 0, s, gp);
+      return;
+    }
     gp.items = (int)(pl.full_tiles + tail_tiles * pl.tail_split);
     hipLaunchKernelGGL((tap_gemm_kernel<T, BM, BN, BK, WM, WN, NPH, FOLD, ROWS>), dim3((unsigned)std::min<long long>(gp.items, slots)),
                        dim3(512), 0, s, gp);
@@ -1743,6 +1922,7 @@ void launch_gemm(GemmParams &gp, const Plan &pl, hipStream_t s) {
 // Bytes of partial sums the shared tail tiles of this plan need.
 size_t tail_bytes(const Plan &pl, size_t elem) {
   const long long tail_tiles = (long long)pl.pos_blocks * pl.m_tiles - pl.full_tiles;
+  if (pl.share_grid > 0) return (size_t)pl.share_slots * pl.nph * pl.bm * pl.bn * elem;
   return pl.tap_major ? (size_t)tail_tiles * pl.tail_split * pl.nph * pl.bm * pl.bn * elem : 0;
 }
 
@@ -1764,6 +1944,7 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
   // and every row starts 16-byte aligned)
   gp.vec_store = pl.single_dense_phase && gp.dst_mstride % 4 == 0 && gp.dst_nstride % 4 == 0 &&
                  reinterpret_cast<uintptr_t>(gp.dst) % 16 == 0;
+  gp.run_store = pl.single_dense_phase && !gp.vec_store;
   gp.nph = pl.nph;
   if (pl.nph > 1) {
     for (int f = 0; f < 4; ++f) {

@@ -75,6 +75,16 @@ struct Phase {
 };
 static_assert(sizeof(Phase) == 96, "Phase is read as three 32-byte rows");
 
+// A slice of a tile's K tiles that one block computes (see GemmParams::share_first), and a tile
+// whose slices the fix-up pass adds: its partial sums lie in consecutive slots, in K order.
+struct ShareSlice {
+  int tile, kt_begin, kt_end;
+  int slot;  // of the partial sums; -1: all of the tile's K tiles, stored directly
+};
+struct ShareFix {
+  int tile, first_slot, slots, pad_;
+};
+
 // Gather-GEMM:  dst[n, m, pos] = sum_k A(k, m) * src[n, row k, pos]
 // The tap-major kernels read A from packed filters, [rows][a_ld] with the M values of a row
 // contiguous; the table-driven kernel reads the filter bank where it lies:
@@ -103,11 +113,21 @@ struct GemmParams {
   int a_ld;                     // values per row of A (M rounded up to a multiple of 4)
   int src_cstride;      // element stride between consecutive channels of the gathered tensor
   int vec_store;        // positions are contiguous in dst: a lane may store its TN positions as one vector
+  int run_store;        // positions run through each sample of dst in order, rows not 16-byte aligned: a lane whose
+                        // TN positions lie in one sample stores them as one vector of element alignment
   int m_tiles;          // row tiles per position block
   int items;            // work items: full_tiles whole tiles, then tail_split K slices of each remaining tile
   int full_tiles;       // tiles computed whole by one block each
   int tail_split;       // blocks that share each remaining tile (K slices), >= 1
   void *partial;        // [tail tile][slice][phase][BM][BN] partial sums of the shared tiles
+  // Even shares of the last, partial round (persistent blocks): the K tiles of the tiles beyond
+  // full_tiles, laid end to end, are cut into one run per block; a run is a few slices (a tile's
+  // end, whole tiles, a tile's beginning).  share_first != nullptr switches this on; tail_split is
+  // then not used.  After its whole tiles b, b + grid, ... block b takes the slices
+  // share_first[b] .. share_first[b + 1] - 1.
+  const int *share_first;     // [grid + 1]
+  const ShareSlice *share_slices;
+  const ShareFix *share_fix;  // the tiles that were cut, one thread block row of tail_fixup_kernel each
   // Fused stride phases (data gradient with a stride, tap-major kernel with NPH > 1): the phase
   // table holds ONE phase, the coarse grid J[k] = ceil(X[k] / stride[k]); every tile computes all
   // nph stride phases of its coarse positions, one accumulator set each, and writes them together,

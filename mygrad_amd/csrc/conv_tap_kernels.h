@@ -193,18 +193,39 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
   // innermost, so that the row tiles of one position block, which gather the same
   // elements, run next to each other; items >= p.full_tiles are K slices.
   struct Item {
-    int tile, piece, pos0, m0, kt_begin, kt_end;
+    int tile, piece, pos0, m0, kt_begin, kt_end, slot;
     bool partial;
     Phase ph;
   };
-  auto locate = [&](int item, int &pi, Item &it) {  // pi: phase of the previous item of this cursor (items ascend)
+  // Even shares of the last round (see GemmParams::share_first): the block's own run of slices
+  const bool shares = p.share_first != nullptr;
+  const int share_begin = shares ? ((const int MG_CONSTANT *)p.share_first)[uniform((int)blockIdx.x)] : 0;
+  const int share_end = shares ? ((const int MG_CONSTANT *)p.share_first)[uniform((int)blockIdx.x) + 1] : 0;
+  const int item_end = shares ? p.full_tiles + share_end : p.items;
+  const int item_first = (!shares || (int)blockIdx.x < p.full_tiles) ? (int)blockIdx.x : p.full_tiles + share_begin;
+  auto next_item = [&](int item) -> int {
+    if (!shares) return item + (int)gridDim.x;
+    if (item >= p.full_tiles) return item + 1;
+    return item + (int)gridDim.x < p.full_tiles ? item + (int)gridDim.x : p.full_tiles + share_begin;
+  };
+  auto locate = [&](int item, int &pi, Item &it) {  // pi: phase of the previous item of this cursor (tiles ascend)
     it.tile = item;
     it.piece = 0;
+    it.slot = 0;
     it.partial = item >= p.full_tiles;
+    int4v row = {0, 0, 0, 0};
     if (it.partial) {
-      const int j = item - p.full_tiles;
-      it.tile = p.full_tiles + j / p.tail_split;
-      it.piece = j % p.tail_split;
+      if (shares) {
+        row = ((const int4v MG_CONSTANT *)p.share_slices)[uniform(item - p.full_tiles)];
+        it.tile = row[0];
+        it.slot = row[3];
+        it.partial = row[3] >= 0;
+      } else {
+        const int j = item - p.full_tiles;
+        it.tile = p.full_tiles + j / p.tail_split;
+        it.piece = j % p.tail_split;
+        it.slot = j;
+      }
     }
     const int pblk = it.tile / p.m_tiles;
     while (pi + 1 < p.nphases && pblk >= phase_first_block(p.phases, pi + 1)) ++pi;
@@ -213,7 +234,10 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
     it.m0 = (it.tile % p.m_tiles) * BM;
     it.kt_begin = 0;
     it.kt_end = it.ph.k_count;
-    if (it.partial) {
+    if (shares && item >= p.full_tiles) {
+      it.kt_begin = row[1];
+      it.kt_end = row[2];
+    } else if (it.partial) {
       const int per = (it.ph.k_count + p.tail_split - 1) / p.tail_split;
       it.kt_begin = min(it.piece * per, it.ph.k_count);
       it.kt_end = min(it.kt_begin + per, it.ph.k_count);
@@ -240,7 +264,7 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
     unsigned a_at = kOutside;
     // moves the cursor to the first item at or after `from` that has K tiles; false if none
     auto enter = [&](int from) -> bool {
-      for (int i = from; i < p.items; i += (int)gridDim.x) {
+      for (int i = from; i < item_end; i = next_item(i)) {
         locate(i, pi, it);
         if (it.kt_begin >= it.kt_end) continue;
         item = i;
@@ -297,7 +321,7 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
         if (kt + 1 < it.kt_end)
           ++kt;
         else if constexpr (STREAM)
-          live = enter(item + (int)gridDim.x);  // no further item: the cursor stays where it is
+          live = enter(next_item(item));  // no further item: the cursor stays where it is
         else
           live = false;
       }
@@ -316,7 +340,7 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
     // elements before it is parked in LDS
     AVec ra0[ALOADS], ra1[ALOADS];
     T rb0[BLOADS], rb1[BLOADS];
-    live = enter((int)blockIdx.x);
+    live = enter(item_first);
     if (live) {
       fetch(ra0, rb0);
       stash(ra0, rb0, 0);
@@ -345,7 +369,7 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
   int pi = 0;
   int buf = 0;
   T *__restrict__ dst = static_cast<T *>(p.dst);
-  locate((int)blockIdx.x, pi, it);  // the grid never has more blocks than items
+  if (item_first < item_end) locate(item_first, pi, it);  // (with even shares a block may have nothing to do)
   __syncthreads();
   // AHEAD: operands of one K step (k4: which four rows of the K tile in `buf`), see `step` below
   constexpr bool AHEAD = sizeof(T) == 4 && BM == 64 && BN == 256 && NPH == 1 && !FOLD;
@@ -358,8 +382,8 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
     }
   };
   read_step(0, cur_a, cur_b);
-  for (int item = (int)blockIdx.x; item < p.items; item += (int)gridDim.x) {
-    if (item != (int)blockIdx.x) locate(item, pi, it);
+  for (int item = item_first; item < item_end; item = next_item(item)) {
+    if (item != item_first) locate(item, pi, it);
     const Phase &ph = it.ph;
     const int pos0 = it.pos0, m0 = it.m0;
     const int j12 = ph.J[1] * ph.J[2];
@@ -389,7 +413,7 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
     auto fused_ok = [&](int f, int j0, int j1, int j2) -> bool {
       return (j0 < p.pJ[f][0]) & (j1 < p.pJ[f][1]) & (j2 < p.pJ[f][2]);
     };
-    T *slot = static_cast<T *>(p.partial) + ((long long)(it.tile - p.full_tiles) * p.tail_split + it.piece) * (NPH * BM * BN);
+    T *slot = static_cast<T *>(p.partial) + (long long)it.slot * (NPH * BM * BN);
 
     if constexpr (sizeof(T) == 8) {
       // The wave tile is cut into 8-row and 8-column groups; group pairs are interleaved
@@ -567,14 +591,35 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
             if (m < p.M) store_vec<T, 2>(out + (long long)m * p.dst_mstride, two);
           }
         } else {
-#pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            if (first + h >= ph.npos) continue;
-            T *out = dst_of(first + h);
+          // positions adjacent in dst but not 16-byte aligned: the pair as one vector of element
+          // alignment when both lie in one sample
+          bool together = false;
+          if (p.run_store && first + 2 <= ph.npos) {
+            const unsigned nn = ph.by_jvol.div((unsigned)first);
+            together = (unsigned)first - nn * (unsigned)jvol + 2u <= (unsigned)jvol;
+          }
+          if (together) {
+            typedef T OutPair __attribute__((ext_vector_type(2), aligned(sizeof(T))));
+            T *out = dst_of(first);
 #pragma unroll
             for (int i = 0; i < GM; ++i) {
               const int m = m0 + drow + (i / 2) * 16 + i % 2;
-              if (m < p.M) out[(long long)m * p.dst_mstride] = acc[0][i][2 * g + h];
+              if (m < p.M) {
+                OutPair v;
+                v[0] = acc[0][i][2 * g], v[1] = acc[0][i][2 * g + 1];
+                *reinterpret_cast<OutPair *>(out + (long long)m * p.dst_mstride) = v;
+              }
+            }
+          } else {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              if (first + h >= ph.npos) continue;
+              T *out = dst_of(first + h);
+#pragma unroll
+              for (int i = 0; i < GM; ++i) {
+                const int m = m0 + drow + (i / 2) * 16 + i % 2;
+                if (m < p.M) out[(long long)m * p.dst_mstride] = acc[0][i][2 * g + h];
+              }
             }
           }
         }
@@ -678,53 +723,80 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
       }
       const int first = pos0 + wn0 + l16 * TN;
       if constexpr (NPH > 1) {
-        if (p.vec_store && ph.J[2] % TN == 0) {
-          // the lane's TN coarse positions exist and lie in one row of the coarse grid
-          if (first < ph.npos) {
+        // Phases f and f + 1 alternate along the last axis of dst (coarse position j2 of phase f is
+        // element 2 * j2 of the row, of phase f + 1 element 2 * j2 + 1), so what a lane holds for
+        // PER coarse positions of one row are 2 * PER adjacent elements.  Rows of dst need not
+        // start on 16-byte boundaries (an exact window grid under stride 2 has an odd extent):
+        // the stores only assume the alignment of an element.  The phase with the odd elements is
+        // one position shorter when the extent is odd: the pair that reaches beyond a row's end is
+        // stored element by element.
+        constexpr int PER = TN < 2 ? TN : 2;  // coarse positions per (up to) 16-byte store
+        typedef T OutVec __attribute__((ext_vector_type(2 * PER), aligned(sizeof(T))));
+        if (ph.J[2] % PER == 0) {
+          // the PER coarse positions of a store lie in one row of the coarse grid
+#pragma unroll
+          for (int h = 0; h < TN / PER; ++h) {
+            if (first + h * PER >= ph.npos) continue;
             int n, j0, j1, j2;
-            split_pos(first, n, j0, j1, j2);
-            // phases f and f+1 alternate along the last axis: 2*TN adjacent elements of dst
+            split_pos(first + h * PER, n, j0, j1, j2);
 #pragma unroll
             for (int f = 0; f < NPH; f += 2) {
-              if (!fused_ok(f, j0, j1, j2)) continue;
+              if (!((j0 < p.pJ[f][0]) & (j1 < p.pJ[f][1]))) continue;
               T *out = fused_dst(f, n, j0, j1, j2);
+              const bool whole = (j2 + PER <= p.pJ[f][2]) & (j2 + PER <= p.pJ[f + 1][2]);
 #pragma unroll
               for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                   const int m = m0 + wm0 + Mma<T>::row_of(lane, q) * TM + i;
-                  if (m < p.M) {
-                    constexpr int PER = TN < 2 ? TN : 2;  // coarse positions per 16-byte store
+                  if (m >= p.M) continue;
+                  T *row = out + (long long)m * p.dst_mstride;
+                  if (whole) {
+                    OutVec v;
 #pragma unroll
-                    for (int h = 0; h < TN / PER; ++h) {
-                      T v[2 * PER];
+                    for (int t = 0; t < PER; ++t) {
+                      v[2 * t] = acc[f][i][h * PER + t][q];
+                      v[2 * t + 1] = acc[f + 1][i][h * PER + t][q];
+                    }
+                    *reinterpret_cast<OutVec *>(row) = v;
+                  } else {
 #pragma unroll
-                      for (int t = 0; t < PER; ++t) {
-                        v[2 * t] = acc[f][i][h * PER + t][q];
-                        v[2 * t + 1] = acc[f + 1][i][h * PER + t][q];
-                      }
-                      store_vec<T, 2 * PER>(out + (long long)m * p.dst_mstride + 2 * h * PER, v);
+                    for (int t = 0; t < PER; ++t) {
+                      if (j2 + t < p.pJ[f][2]) row[2 * t] = acc[f][i][h * PER + t][q];
+                      if (j2 + t < p.pJ[f + 1][2]) row[2 * t + 1] = acc[f + 1][i][h * PER + t][q];
                     }
                   }
                 }
             }
           }
         } else {
+          // an odd number of coarse positions per row: one position, two adjacent elements, at a time
+          typedef T Pair __attribute__((ext_vector_type(2), aligned(sizeof(T))));
 #pragma unroll
           for (int j = 0; j < TN; ++j) {
             if (first + j >= ph.npos) continue;
             int n, j0, j1, j2;
             split_pos(first + j, n, j0, j1, j2);
 #pragma unroll
-            for (int f = 0; f < NPH; ++f) {
-              if (!fused_ok(f, j0, j1, j2)) continue;
+            for (int f = 0; f < NPH; f += 2) {
+              if (!((j0 < p.pJ[f][0]) & (j1 < p.pJ[f][1]))) continue;
               T *out = fused_dst(f, n, j0, j1, j2);
+              const bool even = j2 < p.pJ[f][2], odd = j2 < p.pJ[f + 1][2];
 #pragma unroll
               for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                   const int m = m0 + wm0 + Mma<T>::row_of(lane, q) * TM + i;
-                  if (m < p.M) out[(long long)m * p.dst_mstride] = acc[f][i][j][q];
+                  if (m >= p.M) continue;
+                  T *row = out + (long long)m * p.dst_mstride;
+                  if (even & odd) {
+                    Pair v;
+                    v[0] = acc[f][i][j][q], v[1] = acc[f + 1][i][j][q];
+                    *reinterpret_cast<Pair *>(row) = v;
+                  } else {
+                    if (even) row[0] = acc[f][i][j][q];
+                    if (odd) row[1] = acc[f + 1][i][j][q];
+                  }
                 }
             }
           }
@@ -783,17 +855,41 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
             }
         }
       } else {
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          if (first + j >= ph.npos) continue;
-          T *out = dst_of(first + j);
+        // a sample's positions are adjacent in dst but no whole 16-byte pieces (49, 729, ... of them):
+        // the lanes whose TN positions lie in one sample still store them as one vector
+        bool together = false;
+        if (p.run_store && TN > 1 && first + TN <= ph.npos) {
+          const unsigned nn = ph.by_jvol.div((unsigned)first);
+          together = (unsigned)first - nn * (unsigned)jvol + (unsigned)TN <= (unsigned)jvol;
+        }
+        if (together) {
+          typedef T OutVec __attribute__((ext_vector_type(TN), aligned(sizeof(T))));
+          T *out = dst_of(first);
 #pragma unroll
           for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               const int m = m0 + wm0 + Mma<T>::row_of(lane, q) * TM + i;
-              if (m < p.M) out[(long long)m * p.dst_mstride] = acc[0][i][j][q];
+              if (m < p.M) {
+                OutVec v;
+#pragma unroll
+                for (int j = 0; j < TN; ++j) v[j] = acc[0][i][j][q];
+                *reinterpret_cast<OutVec *>(out + (long long)m * p.dst_mstride) = v;
+              }
             }
+        } else {
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            if (first + j >= ph.npos) continue;
+            T *out = dst_of(first + j);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                const int m = m0 + wm0 + Mma<T>::row_of(lane, q) * TM + i;
+                if (m < p.M) out[(long long)m * p.dst_mstride] = acc[0][i][j][q];
+              }
+          }
         }
       }
     }
@@ -807,7 +903,12 @@ template <typename T, int BM, int BN, int NPH = 1>
 __global__ void __launch_bounds__(256) tail_fixup_kernel(const GemmParams p) {
   const int e = blockIdx.x * 256 + threadIdx.x;  // element of the [BM][BN] tile
   if (e >= BM * BN) return;
-  const int tile = p.full_tiles + blockIdx.y;
+  // the tile, where its slices' partial sums start and how many there are
+  int tile = p.full_tiles + blockIdx.y, first_slot = (int)blockIdx.y * p.tail_split, slots = p.tail_split;
+  if (p.share_fix != nullptr) {
+    const ShareFix fx = p.share_fix[blockIdx.y];
+    tile = fx.tile, first_slot = fx.first_slot, slots = fx.slots;
+  }
   const int pblk = tile / p.m_tiles;
   int pi = 0;
   while (pi + 1 < p.nphases && pblk >= p.phases[pi + 1].blk_begin) ++pi;
@@ -824,12 +925,12 @@ __global__ void __launch_bounds__(256) tail_fixup_kernel(const GemmParams p) {
   const int j1 = (int)ph.by_j2.div(r);
   const int j2 = (int)r - j1 * ph.J[2];
   const long long slice = (long long)NPH * BM * BN;  // elements of one K slice of a tile: one [BM][BN] per phase
-  const T *slot = static_cast<const T *>(p.partial) + (long long)blockIdx.y * p.tail_split * slice + e;
+  const T *slot = static_cast<const T *>(p.partial) + (long long)first_slot * slice + e;
 #pragma unroll
   for (int f = 0; f < NPH; ++f) {
     const int o0 = NPH == 1 ? ph.o0[0] : p.po0[f][0], o1 = NPH == 1 ? ph.o0[1] : p.po0[f][1], o2 = NPH == 1 ? ph.o0[2] : p.po0[f][2];
     if (NPH > 1 && !((j0 < p.pJ[f][0]) & (j1 < p.pJ[f][1]) & (j2 < p.pJ[f][2]))) continue;
-    const T sum = sum_in_order(slot + (long long)f * (BM * BN), slice, p.tail_split);
+    const T sum = sum_in_order(slot + (long long)f * (BM * BN), slice, slots);
     T *out = static_cast<T *>(p.dst) + (long long)n * p.dst_nstride + (long long)(o0 + j0 * p.oj[0]) * p.os[0] +
              (long long)(o1 + j1 * p.oj[1]) * p.os[1] + (long long)(o2 + j2 * p.oj[2]) * p.os[2];
     out[(long long)m * p.dst_mstride] = sum;

@@ -68,6 +68,13 @@ template <int NPH, int RG>
 __global__ void __launch_bounds__(256) thin_gemm_kernel(ThinParams p) {
   constexpr int NACC = NPH * RG;   // accumulators: (stride phase, group of four rows)
   constexpr int EPV = 16 / NACC;   // entries per register of packed filters
+  // feed() writes the MFMA as the instruction itself from 8 accumulators on, where the compiler
+  // inserts no wait states: the code relies on an accumulator being written again only NACC
+  // MFMAs after its last write (feed_all runs through all NACC for every entry) and on the two
+  // s_nop 7 before the epilogue.  Fewer than 8 accumulators go through the builtin, which the
+  // compiler schedules itself; any other count must revisit both.
+  static_assert(NACC == 1 || NACC == 2 || NACC == 4 || NACC == 8 || NACC == 16, "accumulator counts the hazard analysis covers");
+  static_assert(NACC * EPV == 16, "a register of packed filters feeds sixteen MFMAs");
   const int lane = threadIdx.x & 63;
   const int pos = blockIdx.x * 256 + threadIdx.x;
   const bool active = pos < p.npos;
@@ -97,7 +104,7 @@ __global__ void __launch_bounds__(256) thin_gemm_kernel(ThinParams p) {
   // gathered elements, 16 MFMAs.  The steps of all chunks form one pipeline: two sets of
   // registers take turns, the loads of one step are in flight while the other feeds the MFMAs,
   // also across the change from one chunk to the next (where the entries' offsets are renewed).
-  const unsigned a_lane = (unsigned)lane * 4u;
+  unsigned a_lane = (unsigned)lane * 4u;  // past the last step: kOutside (the range check is on the per-lane offset)
   unsigned at[EPV];
   // The rows of the table come through the scalar data path; with few entries per chunk the
   // chunks change often, and the rows of the next chunk are asked for a chunk ahead so that
@@ -134,7 +141,8 @@ __global__ void __launch_bounds__(256) thin_gemm_kernel(ThinParams p) {
     __builtin_amdgcn_sched_barrier(0);  // all of a step's loads are issued before the MFMAs that follow in the source
   };
   // moves on to the next step; past the last one every load lies outside its buffer and reads as
-  // zero (the packed filters end there, the entries' offsets are set outside)
+  // zero: the per-lane offsets of the filters and of the entries are set outside (the hardware
+  // checks the per-lane offset against the buffer's size, not the scalar one added to it)
   auto advance = [&]() {
     a_uni += 256u;
     s_uni += p.group_bytes;
@@ -152,7 +160,9 @@ __global__ void __launch_bounds__(256) thin_gemm_kernel(ThinParams p) {
       } else {
 #pragma unroll
         for (int i = 0; i < EPV; ++i) at[i] = kOutside;
-        a_uni = kOutside;
+        a_lane = kOutside;
+        a_uni = 0u;
+        s_uni = 0u;
       }
     }
   };
@@ -241,8 +251,10 @@ int launch_thin_pack(const float *w, float *packed, const int *arow, int chunks,
   return err == hipSuccess ? MG_OK : hip_fail(err, "thin_pack_kernel", __FILE__, __LINE__);
 }
 
-// (stride phases, row groups) the kernel is built for: their product is at most 16
-#define MG_THIN_SHAPES(X) X(1, 1) X(1, 2) X(1, 4) X(1, 8) X(1, 16) X(2, 1) X(2, 2) X(2, 4) X(2, 8) X(4, 1) X(4, 2) X(4, 4)
+// (stride phases, row groups) the kernel is built for: their product is at most 16.  The callers
+// use stride phases for the data gradient of up to four channels (one row group) and row groups
+// for the forward pass (one phase); each pair listed here has an exact-integer test.
+#define MG_THIN_SHAPES(X) X(1, 1) X(1, 2) X(1, 4) X(1, 8) X(1, 16) X(2, 1) X(4, 1)
 
 bool thin_gemm_has(int nph, int rg) {
 #define MG_THIN_HAS(NPH, RG) \

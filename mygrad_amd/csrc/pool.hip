@@ -11,6 +11,7 @@
 #include <cstdlib>
 
 #include <algorithm>
+#include <optional>
 
 namespace mg {
 
@@ -55,7 +56,7 @@ __global__ void __launch_bounds__(256) maxpool_fwd_kernel(PoolParams p, const T 
           }
         }
       }
-    out[idx] = best;
+    if (out) out[idx] = best;  // null: only the argmax offsets are wanted
     if constexpr (MARK) mark[idx] = (unsigned char)code;
   }
 }
@@ -662,15 +663,16 @@ __global__ void __launch_bounds__(256) maxpool_from_mark_kernel(PoolMarkParams p
   }
 }
 
-// Forward pass for windows over the last two axes whose extent and step are known at compile time
-// (P0 = S0 = 1; P1 x P2 placed every S1, S2), straight from global memory.  Lane l of a wavefront
-// takes the l-th 16-byte piece of a window row's P1 rows of x -- consecutive lanes, consecutive
-// pieces: every load of the wavefront is one contiguous run -- and reduces the VEC / S2 windows
-// that start inside its piece.  The P2 - S2 columns those reach beyond the piece come from the
-// next lane by a cross-lane move, not from memory; the last lane of a wavefront only supplies them
-// (the next wavefront starts on its piece again).  A window that would need columns of the next
-// row does not exist.  Every element of x crosses HBM once (rows shared by two window rows come
-// the second time out of L1 / L2); nothing is staged.
+// Forward pass for windows whose extent and step are known at compile time (P0 x P1 x P2 placed
+// every S0, S1, S2; P0 = S0 = 1 for windows over the last two axes), straight from global memory.
+// Lane l of a wavefront takes the l-th 16-byte piece of a window row's P1 rows of x -- consecutive
+// lanes, consecutive pieces: every load of the wavefront is one contiguous run -- in each of the
+// window's P0 planes, one after the other, and reduces the VEC / S2 windows that start inside its
+// piece.  The P2 - S2 columns those reach beyond the piece come from the next lane by a
+// cross-lane move, not from memory; the last lane of a wavefront only supplies them (the next
+// wavefront starts on its piece again).  A window that would need columns of the next row does
+// not exist.  Rows and planes that two windows share are loaded by both (the second time out of
+// L1 / L2: the items that share them run next to each other); nothing is staged.
 // Pieces are counted in columns, not in addresses: a row need not start on a 16-byte boundary
 // (the loads only assume the alignment of an element), and a row that is no whole number of
 // pieces ends in a short one of `tail` columns.  The lane of a short piece loads the last VEC
@@ -680,13 +682,13 @@ __global__ void __launch_bounds__(256) maxpool_from_mark_kernel(PoolMarkParams p
 // Needs VEC % S2 == 0, P2 - S2 <= VEC and X2 >= VEC.
 #define POOL_ROWS_PER_THREAD 3
 struct PoolRowsParams {
-  int X1, X2, G1, G2;
+  int X0, X1, X2, G0, G1, G2;
   int pieces;        // 16-byte pieces per row of x, the short one included
   int tail;          // columns of the short piece (X2 % VEC); 0: none
-  int groups;        // groups of POOL_ROWS_PER_THREAD window rows per plane
-  long long planes;  // lead * X0
+  int groups;        // groups of POOL_ROWS_PER_THREAD window rows per window plane
+  long long planes;  // lead * G0: window planes
   long long items;   // planes * groups * pieces: one per (group of window rows, piece)
-  FastDivP by_pieces, by_groups;
+  FastDivP by_pieces, by_groups, by_g0;
 };
 
 template <typename T>
@@ -694,7 +696,7 @@ __device__ __forceinline__ T from_next_lane(T value) {
   return __shfl_down(value, 1, 64);
 }
 
-template <typename T, int P1, int P2, int S1, int S2, bool MARK, bool STORE_OUT = true>
+template <typename T, int P0, int P1, int P2, int S0, int S1, int S2, bool MARK, bool STORE_OUT = true>
 __global__ void __launch_bounds__(256) maxpool_rows_fwd_kernel(PoolRowsParams p, const T *__restrict__ x, T *__restrict__ out,
                                                               unsigned char *__restrict__ mark) {
   constexpr int VEC = 16 / sizeof(T);
@@ -709,150 +711,222 @@ __global__ void __launch_bounds__(256) maxpool_rows_fwd_kernel(PoolRowsParams p,
   const long long item = wave * 63 + lane;  // wavefronts overlap by one lane
   const unsigned u = (unsigned)(item < p.items ? item : p.items - 1);  // clamped: every lane loads, some do not store
   const unsigned q = p.by_pieces.div(u), piece = u - q * (unsigned)p.pieces;
-  const unsigned plane = p.by_groups.div(q);
+  const unsigned plane = p.by_groups.div(q);  // window plane: (leading index, g0)
   const int g1_first = (int)(q - plane * (unsigned)p.groups) * RW;
+  const unsigned lead = p.by_g0.div(plane);
+  const long long xplane = (long long)lead * p.X0 + (long long)(plane - lead * (unsigned)p.G0) * S0;  // the first plane of x under the window plane
   const bool short_piece = p.tail != 0 && (int)piece == p.pieces - 1;
-  const T *rows = x + (long long)plane * p.X1 * p.X2 + (short_piece ? p.X2 - VEC : (int)piece * VEC);
+  const T *rows = x + xplane * p.X1 * p.X2 + (short_piece ? p.X2 - VEC : (int)piece * VEC);
   const int row_first = g1_first * S1;
-  T v[NR][VEC + HALO];
+  const bool idle = lane == 63 || item >= p.items;  // supplies its neighbour's columns only
+
+  T best[RW][WO];
+  int code[RW][WO];
 #pragma unroll
-  for (int r = 0; r < NR; ++r) {
-    // rows beyond the last one belong to window rows that do not exist: read the last row instead
-    const Vec mine = *reinterpret_cast<const Vec *>(rows + (long long)min(row_first + r, p.X1 - 1) * p.X2);
+  for (int a0 = 0; a0 < P0; ++a0) {
+    T v[NR][VEC + HALO];
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) v[r][i] = mine[i];
-  }
-  if (p.tail != 0) {
-    // a short piece's own columns are the last `tail` of what it loaded
+    for (int r = 0; r < NR; ++r) {
+      // rows beyond the last one belong to window rows that do not exist: read the last row instead
+      const Vec mine = *reinterpret_cast<const Vec *>(rows + ((long long)a0 * p.X1 + min(row_first + r, p.X1 - 1)) * p.X2);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) v[r][i] = mine[i];
+    }
+    if (p.tail != 0) {
+      // a short piece's own columns are the last `tail` of what it loaded
+#pragma unroll
+      for (int r = 0; r < NR; ++r)
+#pragma unroll
+        for (int i = 0; i < VEC - 1; ++i) {
+          T moved = v[r][i];
+#pragma unroll
+          for (int k = i + 1; k < VEC; ++k)
+            if (p.tail == k) moved = v[r][i + VEC - k];
+          v[r][i] = short_piece ? moved : v[r][i];
+        }
+    }
 #pragma unroll
     for (int r = 0; r < NR; ++r)
 #pragma unroll
-      for (int i = 0; i < VEC - 1; ++i) {
-        T moved = v[r][i];
+      for (int i = 0; i < HALO; ++i) v[r][VEC + i] = from_next_lane(v[r][i]);
 #pragma unroll
-        for (int k = i + 1; k < VEC; ++k)
-          if (p.tail == k) moved = v[r][i + VEC - k];
-        v[r][i] = short_piece ? moved : v[r][i];
+    for (int w = 0; w < RW; ++w)
+#pragma unroll
+      for (int t = 0; t < WO; ++t) {
+        if (a0 == 0) {
+          best[w][t] = v[w * S1][t * S2];
+          code[w][t] = 0;
+        }
+#pragma unroll
+        for (int a1 = 0; a1 < P1; ++a1)
+#pragma unroll
+          for (int a2 = 0; a2 < P2; ++a2) {
+            const T c = v[w * S1 + a1][t * S2 + a2];
+            if (takes_over(c, best[w][t])) {
+              best[w][t] = c;
+              code[w][t] = (a0 * P1 + a1) * P2 + a2;
+            }
+          }
       }
   }
-#pragma unroll
-  for (int r = 0; r < NR; ++r)
-#pragma unroll
-    for (int i = 0; i < HALO; ++i) v[r][VEC + i] = from_next_lane(v[r][i]);
-  if (lane == 63 || item >= p.items) return;
+  if (idle) return;
 #pragma unroll
   for (int w = 0; w < RW; ++w) {
     const int g1 = g1_first + w;
     if (g1 >= p.G1) break;
     const long long w0 = ((long long)plane * p.G1 + g1) * p.G2 + (long long)piece * WO;
+    // the piece's windows are neighbours in out and in the record: one store each when all exist
+    if (WO > 1 && (int)piece * WO + WO <= p.G2) {
+      if constexpr (STORE_OUT) {
+        typedef T OVec __attribute__((ext_vector_type(WO), aligned(sizeof(T))));
+        OVec o;
 #pragma unroll
-    for (int t = 0; t < WO; ++t) {
-      T best = v[w * S1][t * S2];
-      int code = 0;
-#pragma unroll
-      for (int a1 = 0; a1 < P1; ++a1)
-#pragma unroll
-        for (int a2 = 0; a2 < P2; ++a2) {
-          const T c = v[w * S1 + a1][t * S2 + a2];
-          if (takes_over(c, best)) {
-            best = c;
-            code = a1 * P2 + a2;
-          }
-        }
-      if ((int)piece * WO + t < p.G2) {
-        if constexpr (STORE_OUT) out[w0 + t] = best;
-        if constexpr (MARK) mark[w0 + t] = (unsigned char)code;
+        for (int t = 0; t < WO; ++t) o[t] = best[w][t];
+        *reinterpret_cast<OVec *>(out + w0) = o;
       }
+      if constexpr (MARK) {
+        typedef unsigned char CVec __attribute__((ext_vector_type(WO), aligned(1)));
+        CVec c;
+#pragma unroll
+        for (int t = 0; t < WO; ++t) c[t] = (unsigned char)code[w][t];
+        *reinterpret_cast<CVec *>(mark + w0) = c;
+      }
+    } else {
+#pragma unroll
+      for (int t = 0; t < WO; ++t)
+        if ((int)piece * WO + t < p.G2) {
+          if constexpr (STORE_OUT) out[w0 + t] = best[w][t];
+          if constexpr (MARK) mark[w0 + t] = (unsigned char)code[w][t];
+        }
     }
   }
 }
 
-// The same gather for windows over the last two axes whose extent and step are known at compile
-// time (P0 = S0 = 1; P1 x P2 placed every S1, S2).  A thread owns a 16-byte piece of S1
-// consecutive rows of dx: the rows k*S1 .. k*S1 + S1 - 1 are covered by the same ceil(P1/S1)
-// window rows, and the piece's columns by the same ceil(P2/S2) - 1 + VD/S2 windows along the row,
-// whichever thread -- so their recorded offsets and gradients are loaded up front (clamped, never
-// predicated), and every element adds, in ascending window order, the gradient of the windows
-// whose recorded offset names it and +0.0 for the others: no loop bounds to compute, no
-// divisions by runtime values, no LDS.  Needs VD % S2 == 0 (a piece starts on a window boundary).
+// The same gather for windows whose extent and step are known at compile time (P0 x P1 x P2
+// placed every S0, S1, S2; P0 = S0 = 1 for windows over the last two axes).  A thread owns a
+// 16-byte piece of S1 consecutive rows in S0 consecutive planes of dx: the rows k1*S1 ..
+// k1*S1 + S1 - 1 are covered by the same ceil(P1/S1) window rows (the planes by the same
+// ceil(P0/S0) window planes), and the piece's columns by the same ceil(P2/S2) - 1 + VD/S2 windows
+// along the row, whichever thread -- so their recorded offsets and gradients are loaded up front
+// (clamped, never predicated), and every element adds, in ascending window order, the gradient
+// of the windows whose recorded offset names it and +0.0 for the others: no loop bounds to
+// compute, no divisions by runtime values, no LDS.  Needs VD % S2 == 0 (a piece starts on a
+// window boundary) and at least pool_gather_run() windows per row.
 // Pieces are counted in columns: rows of dx need not start on 16-byte boundaries (the stores only
 // assume the alignment of an element), and the short piece at the end of a row that is no whole
 // number of pieces is stored element by element.
 struct PoolGatherParams {
-  int X1, X2, G1, G2;
+  int X0, X1, X2, G0, G1, G2;
   int pieces;        // 16-byte pieces per row of dx, the short one included
   int tail;          // columns of the short piece (X2 % VD); 0: none
   int groups;        // groups of S1 rows per plane: ceil(X1 / S1)
-  long long planes;  // lead * X0
-  FastDivP by_pieces, by_groups;
+  int groups0;       // groups of S0 planes per leading index: ceil(X0 / S0)
+  long long planes;  // lead * groups0
+  FastDivP by_pieces, by_groups, by_groups0;
 };
 
-template <typename T, typename TD, int P1, int P2, int S1, int S2>
+template <typename T, typename TD, int P0, int P1, int P2, int S0, int S1, int S2>
 __global__ void __launch_bounds__(256) maxpool_mark_gather_kernel(PoolGatherParams p, const unsigned char *__restrict__ mark,
                                                                  const T *__restrict__ grad, TD *__restrict__ dx) {
   constexpr int VD = 16 / sizeof(TD);
-  constexpr int C1 = (P1 + S1 - 1) / S1, C2 = (P2 + S2 - 1) / S2;
+  constexpr int C0 = (P0 + S0 - 1) / S0, C1 = (P1 + S1 - 1) / S1, C2 = (P2 + S2 - 1) / S2;
   constexpr int NW2 = (VD - 1) / S2 + C2;  // windows along the row that can reach the piece
-  static_assert(VD % S2 == 0, "a piece starts on a window boundary");
+  constexpr int LW = NW2 <= 2 ? 2 : NW2 <= 4 ? 4 : 8;  // windows loaded per window row
+  static_assert(VD % S2 == 0 && NW2 <= 8, "a piece starts on a window boundary");
   typedef TD DVec __attribute__((ext_vector_type(VD), aligned(sizeof(TD))));
   const long long item = (long long)blockIdx.x * 256 + threadIdx.x;
   if (item >= p.planes * p.groups * p.pieces) return;
   const unsigned u = (unsigned)item;
   const unsigned q = p.by_pieces.div(u), piece = u - q * (unsigned)p.pieces;
-  const unsigned plane = p.by_groups.div(q);
-  const int k = (int)(q - plane * (unsigned)p.groups);
+  const unsigned plane = p.by_groups.div(q);  // (leading index, group of S0 planes)
+  const int k1 = (int)(q - plane * (unsigned)p.groups);
+  const unsigned lead = p.by_groups0.div(plane);
+  const int k0 = (int)(plane - lead * (unsigned)p.groups0);
   const int i2 = (int)piece * VD;
   const int live = (p.tail != 0 && (int)piece == p.pieces - 1) ? p.tail : VD;  // columns of this piece
-  const unsigned char *m = mark + (long long)plane * (p.G1 * p.G2);
-  const T *g = grad + (long long)plane * (p.G1 * p.G2);
-  const int g1_first = k - (C1 - 1), g2_first = i2 / S2 - (C2 - 1);
+  const long long gvol = (long long)p.G0 * p.G1 * p.G2;
+  const unsigned char *m = mark + (long long)lead * gvol;
+  const T *g = grad + (long long)lead * gvol;
+  const int g0_first = k0 - (C0 - 1), g1_first = k1 - (C1 - 1), g2_first = i2 / S2 - (C2 - 1);
 
-  int code[C1][NW2];
-  double term[C1][NW2];
+  // The NW2 windows of a window row are neighbours in the record and in grad: LW of them (a power
+  // of two that holds NW2) come as one load each, from the run [b, b + LW) that starts at the first
+  // window wanted where that lies inside the row and at the nearest run inside it otherwise; the
+  // window wanted at place e is then the loaded one at place e + shift.
+  int code[C0][C1][NW2];
+  double term[C0][C1][NW2];
+  typedef unsigned char CVec __attribute__((ext_vector_type(LW), aligned(1)));
+  typedef T GVec __attribute__((ext_vector_type(LW), aligned(sizeof(T))));
+  const int b = min(max(g2_first, 0), p.G2 - LW);
+  const int shift = g2_first - b;
 #pragma unroll
-  for (int d = 0; d < C1; ++d) {
-    const int g1 = g1_first + d;
-    const bool ok1 = (g1 >= 0) & (g1 < p.G1);
-    const int r = min(max(g1, 0), p.G1 - 1) * p.G2;
+  for (int d0 = 0; d0 < C0; ++d0) {
+    const int g0 = g0_first + d0;
+    const bool ok0 = (g0 >= 0) & (g0 < p.G0);
+    const int r0 = min(max(g0, 0), p.G0 - 1) * p.G1;
 #pragma unroll
-    for (int e = 0; e < NW2; ++e) {
-      const int g2 = g2_first + e;
-      const bool ok = ok1 & (g2 >= 0) & (g2 < p.G2);
-      const int at = r + min(max(g2, 0), p.G2 - 1);
-      const int c = (int)m[at];
-      const double t = (double)g[at];
-      code[d][e] = ok ? c : -1;  // a window that does not exist names no element
-      term[d][e] = t;
+    for (int d = 0; d < C1; ++d) {
+      const int g1 = g1_first + d;
+      const bool ok1 = ok0 & (g1 >= 0) & (g1 < p.G1);
+      const int r = (r0 + min(max(g1, 0), p.G1 - 1)) * p.G2 + b;
+      const CVec lc = *reinterpret_cast<const CVec *>(m + r);
+      const GVec lg = *reinterpret_cast<const GVec *>(g + r);
+#pragma unroll
+      for (int e = 0; e < NW2; ++e) {
+        const int g2 = g2_first + e;
+        const bool ok = ok1 & (g2 >= 0) & (g2 < p.G2);
+        int c = -1;
+        T t = T(0);
+#pragma unroll
+        for (int k = 0; k < LW; ++k) {
+          const bool here = e + shift == k;
+          c = here ? (int)lc[k] : c;
+          t = here ? lg[k] : t;
+        }
+        code[d0][d][e] = ok ? c : -1;  // a window that does not exist names no element
+        term[d0][d][e] = (double)t;
+      }
     }
   }
-  TD *to = dx + ((long long)plane * p.X1 + (long long)k * S1) * p.X2 + i2;
+  TD *to = dx + (((long long)lead * p.X0 + (long long)k0 * S0) * p.X1 + (long long)k1 * S1) * p.X2 + i2;
 #pragma unroll
-  for (int rr = 0; rr < S1; ++rr) {
-    if (k * S1 + rr >= p.X1) break;
-    DVec out;
+  for (int pp = 0; pp < S0; ++pp) {
+    if (k0 * S0 + pp >= p.X0) break;
 #pragma unroll
-    for (int v = 0; v < VD; ++v) {
-      double acc = 0.0;
+    for (int rr = 0; rr < S1; ++rr) {
+      if (k1 * S1 + rr >= p.X1) break;
+      DVec out;
 #pragma unroll
-      for (int d = 0; d < C1; ++d) {
-        const int a1 = rr + (C1 - 1 - d) * S1;  // the row's offset inside window row d: known at compile time
-        if (a1 >= P1) continue;                 // that window row does not reach this row
+      for (int v = 0; v < VD; ++v) {
+        double acc = 0.0;
 #pragma unroll
-        for (int e = 0; e < C2; ++e) {
-          const int w = v / S2 + e;                     // which of the loaded windows
-          const int a2 = (v % S2) + (C2 - 1 - e) * S2;   // the element's offset inside it
-          if (a2 >= P2) continue;
-          acc += code[d][w] == a1 * P2 + a2 ? term[d][w] : 0.0;  // + (+0.0) leaves a sum that started at +0.0 as it is
+        for (int d0 = 0; d0 < C0; ++d0) {
+          const int a0 = pp + (C0 - 1 - d0) * S0;  // the plane's offset inside window plane d0: known at compile time
+          if (a0 >= P0) continue;
+#pragma unroll
+          for (int d = 0; d < C1; ++d) {
+            const int a1 = rr + (C1 - 1 - d) * S1;  // the row's offset inside window row d
+            if (a1 >= P1) continue;                 // that window row does not reach this row
+#pragma unroll
+            for (int e = 0; e < C2; ++e) {
+              const int w = v / S2 + e;                     // which of the loaded windows
+              const int a2 = (v % S2) + (C2 - 1 - e) * S2;   // the element's offset inside it
+              if (a2 >= P2) continue;
+              // + (+0.0) leaves a sum that started at +0.0 as it is
+              acc += code[d0][d][w] == (a0 * P1 + a1) * P2 + a2 ? term[d0][d][w] : 0.0;
+            }
+          }
         }
+        out[v] = (TD)acc;
       }
-      out[v] = (TD)acc;
-    }
-    if (live == VD) {
-      *reinterpret_cast<DVec *>(to + (long long)rr * p.X2) = out;
-    } else {
+      TD *row = to + ((long long)pp * p.X1 + rr) * p.X2;
+      if (live == VD) {
+        *reinterpret_cast<DVec *>(row) = out;
+      } else {
 #pragma unroll
-      for (int v = 0; v < VD - 1; ++v)
-        if (v < live) to[(long long)rr * p.X2 + v] = out[v];
+        for (int v = 0; v < VD - 1; ++v)
+          if (v < live) row[v] = out[v];
+      }
     }
   }
 }
@@ -1113,11 +1187,23 @@ static int exact_signature(const PoolParams &p, size_t elem, const void *a, cons
   return sig;
 }
 
-// ---- the kernels for 2-D windows known at compile time: when they apply, and their launches
-static int window_signature4(const PoolParams &p) { return ((p.P[1] * 10 + p.P[2]) * 10 + p.S[1]) * 10 + p.S[2]; }
+// ---- the kernels for windows known at compile time: when they apply, and their launches
+// P0 P1 P2 S0 S1 S2 as one number; the instances: 3x3 every other position, 3x3 and 2x2 at every
+// position (windows over the last two axes), 3x3x3 every other position.
+static int window_signature6(const PoolParams &p) {
+  int sig = 0;
+  for (int k = 0; k < 3; ++k) sig = sig * 10 + (p.P[k] < 10 ? p.P[k] : 0);
+  for (int k = 0; k < 3; ++k) sig = sig * 10 + (p.S[k] < 10 ? p.S[k] : 0);
+  return sig;
+}
+#define MG_POOL_WINDOW_INSTANCES(X) X(1, 3, 3, 1, 2, 2) X(1, 3, 3, 1, 1, 1) X(1, 2, 2, 1, 1, 1) X(3, 3, 3, 2, 2, 2)
 static bool has_rows_instance(const PoolParams &p) {
-  const int sig4 = window_signature4(p);
-  return p.P[0] == 1 && p.S[0] == 1 && (sig4 == 3322 || sig4 == 3311 || sig4 == 2211);
+  const int sig6 = window_signature6(p);
+#define MG_POOL_HAS(A, B, C, D, E, F) \
+  if (sig6 == ((((A * 10 + B) * 10 + C) * 10 + D) * 10 + E) * 10 + F) return true;
+  MG_POOL_WINDOW_INSTANCES(MG_POOL_HAS)
+#undef MG_POOL_HAS
+  return false;
 }
 
 static bool rows_forward_applies(const PoolParams &p, bool f32, const void *x) {
@@ -1126,7 +1212,7 @@ static bool rows_forward_applies(const PoolParams &p, bool f32, const void *x) {
     return !(flag && flag[0] == '0');
   }();
   const int vec = f32 ? 4 : 2;
-  const long long items = p.lead * p.X[0] * ceil_div(p.G[1], POOL_ROWS_PER_THREAD) * ceil_div(p.X[2], vec);
+  const long long items = p.lead * p.G[0] * ceil_div(p.G[1], POOL_ROWS_PER_THREAD) * ceil_div(p.X[2], vec);
   return on && has_rows_instance(p) && p.X[2] >= vec && vec % p.S[2] == 0 &&
          reinterpret_cast<uintptr_t>(x) % (f32 ? 4 : 8) == 0 && items < (1ll << 31);
 }
@@ -1134,25 +1220,32 @@ static bool rows_forward_applies(const PoolParams &p, bool f32, const void *x) {
 // out may be null (with mark set): only the argmax offsets are wanted
 static int launch_rows_forward(const PoolParams &p, bool f32, const void *x, void *out, unsigned char *mark, hipStream_t s) {
   const int vec = f32 ? 4 : 2;
-  const int sig4 = window_signature4(p);
+  const int sig6 = window_signature6(p);
   PoolRowsParams q{};
-  q.X1 = p.X[1], q.X2 = p.X[2], q.G1 = p.G[1], q.G2 = p.G[2];
+  q.X0 = p.X[0], q.X1 = p.X[1], q.X2 = p.X[2], q.G0 = p.G[0], q.G1 = p.G[1], q.G2 = p.G[2];
   q.pieces = (int)ceil_div(p.X[2], vec);
   q.tail = p.X[2] % vec;
   q.groups = (int)ceil_div(p.G[1], POOL_ROWS_PER_THREAD);
-  q.planes = p.lead * p.X[0];
+  q.planes = p.lead * p.G[0];
   q.items = q.planes * q.groups * q.pieces;
   q.by_pieces = make_fastdiv_p((unsigned)q.pieces);
   q.by_groups = make_fastdiv_p((unsigned)q.groups);
+  q.by_g0 = make_fastdiv_p((unsigned)p.G[0]);
   // a wavefront covers 63 items (its last lane only supplies its neighbour), a block 4 wavefronts
   const dim3 grid((unsigned)ceil_div(ceil_div(q.items, 63), 4)), block(256);
-#define MG_POOL_ROWS_SIG(T, A, B, C, D, MK, OUT) \
-  hipLaunchKernelGGL((maxpool_rows_fwd_kernel<T, A, B, C, D, MK, OUT>), grid, block, 0, s, q, (const T *)x, (T *)out, mark)
-#define MG_POOL_ROWS_MK(T, MK, OUT)                                  \
-  do {                                                               \
-    if (sig4 == 3322) MG_POOL_ROWS_SIG(T, 3, 3, 2, 2, MK, OUT);      \
-    else if (sig4 == 3311) MG_POOL_ROWS_SIG(T, 3, 3, 1, 1, MK, OUT); \
-    else MG_POOL_ROWS_SIG(T, 2, 2, 1, 1, MK, OUT);                   \
+  bool launched = false;
+#define MG_POOL_ROWS_SIG(T, MK, OUT, A, B, C, D, E, F)                                                              \
+  if (!launched && sig6 == ((((A * 10 + B) * 10 + C) * 10 + D) * 10 + E) * 10 + F) {                                \
+    hipLaunchKernelGGL((maxpool_rows_fwd_kernel<T, A, B, C, D, E, F, MK, OUT>), grid, block, 0, s, q, (const T *)x, \
+                       (T *)out, mark);                                                                             \
+    launched = true;                                                                                                \
+  }
+#define MG_POOL_ROWS_MK(T, MK, OUT)                                                             \
+  do {                                                                                          \
+    MG_POOL_ROWS_SIG(T, MK, OUT, 1, 3, 3, 1, 2, 2)                                              \
+    MG_POOL_ROWS_SIG(T, MK, OUT, 1, 3, 3, 1, 1, 1)                                              \
+    MG_POOL_ROWS_SIG(T, MK, OUT, 1, 2, 2, 1, 1, 1)                                              \
+    MG_POOL_ROWS_SIG(T, MK, OUT, 3, 3, 3, 2, 2, 2)                                              \
   } while (0)
 #define MG_POOL_ROWS(T)                                 \
   do {                                                  \
@@ -1164,8 +1257,15 @@ static int launch_rows_forward(const PoolParams &p, bool f32, const void *x, voi
 #undef MG_POOL_ROWS
 #undef MG_POOL_ROWS_MK
 #undef MG_POOL_ROWS_SIG
+  if (!launched) return fail(MG_ERR_UNSUPPORTED, "no compile-time instance for pooling window signature %d", sig6);
   MG_HIP(hipGetLastError());
   return MG_OK;
+}
+
+// Windows the gather kernel loads per window row (its LW): needs that many in a row.
+static int pool_gather_run(const PoolParams &p, int vd) {
+  const int nw2 = (vd - 1) / p.S[2] + (p.P[2] + p.S[2] - 1) / p.S[2];
+  return nw2 <= 2 ? 2 : nw2 <= 4 ? 4 : 8;
 }
 
 static bool mark_gather_applies(const PoolParams &p, bool f32, bool wide, const void *dx) {
@@ -1174,31 +1274,39 @@ static bool mark_gather_applies(const PoolParams &p, bool f32, bool wide, const 
     return !(flag && flag[0] == '0');
   }();
   const int vd = (f32 && !wide) ? 4 : 2;
-  const long long items = p.lead * p.X[0] * ceil_div(p.X[1], p.S[1]) * ceil_div(p.X[2], vd);
+  const long long items = p.lead * ceil_div(p.X[0], p.S[0]) * ceil_div(p.X[1], p.S[1]) * ceil_div(p.X[2], vd);
   return on && has_rows_instance(p) && vd % p.S[2] == 0 && reinterpret_cast<uintptr_t>(dx) % (16 / vd) == 0 &&
-         items < (1ll << 31) && (long long)p.G[1] * p.G[2] < (1ll << 30);
+         p.G[2] >= pool_gather_run(p, vd) && items < (1ll << 31) && p.gvol < (1ll << 30);
 }
 
 static int launch_mark_gather(const PoolParams &p, bool f32, bool wide, const unsigned char *mark, const void *grad, void *dx,
                               hipStream_t s) {
   const int vd = (f32 && !wide) ? 4 : 2;
-  const int sig4 = window_signature4(p);
+  const int sig6 = window_signature6(p);
   PoolGatherParams q{};
-  q.X1 = p.X[1], q.X2 = p.X[2], q.G1 = p.G[1], q.G2 = p.G[2];
+  q.X0 = p.X[0], q.X1 = p.X[1], q.X2 = p.X[2], q.G0 = p.G[0], q.G1 = p.G[1], q.G2 = p.G[2];
   q.pieces = (int)ceil_div(p.X[2], vd);
   q.tail = p.X[2] % vd;
   q.groups = (int)ceil_div(p.X[1], p.S[1]);
-  q.planes = p.lead * p.X[0];
+  q.groups0 = (int)ceil_div(p.X[0], p.S[0]);
+  q.planes = p.lead * q.groups0;
   q.by_pieces = make_fastdiv_p((unsigned)q.pieces);
   q.by_groups = make_fastdiv_p((unsigned)q.groups);
+  q.by_groups0 = make_fastdiv_p((unsigned)q.groups0);
   const dim3 grid((unsigned)ceil_div(q.planes * q.groups * q.pieces, 256)), block(256);
-#define MG_POOL_GATHER_SIG(T, TD, A, B, C, D) \
-  hipLaunchKernelGGL((maxpool_mark_gather_kernel<T, TD, A, B, C, D>), grid, block, 0, s, q, mark, (const T *)grad, (TD *)dx)
-#define MG_POOL_GATHER(T, TD)                                     \
-  do {                                                            \
-    if (sig4 == 3322) MG_POOL_GATHER_SIG(T, TD, 3, 3, 2, 2);      \
-    else if (sig4 == 3311) MG_POOL_GATHER_SIG(T, TD, 3, 3, 1, 1); \
-    else MG_POOL_GATHER_SIG(T, TD, 2, 2, 1, 1);                   \
+  bool launched = false;
+#define MG_POOL_GATHER_SIG(T, TD, A, B, C, D, E, F)                                                                  \
+  if (!launched && sig6 == ((((A * 10 + B) * 10 + C) * 10 + D) * 10 + E) * 10 + F) {                                 \
+    hipLaunchKernelGGL((maxpool_mark_gather_kernel<T, TD, A, B, C, D, E, F>), grid, block, 0, s, q, mark,            \
+                       (const T *)grad, (TD *)dx);                                                                   \
+    launched = true;                                                                                                 \
+  }
+#define MG_POOL_GATHER(T, TD)                               \
+  do {                                                      \
+    MG_POOL_GATHER_SIG(T, TD, 1, 3, 3, 1, 2, 2)             \
+    MG_POOL_GATHER_SIG(T, TD, 1, 3, 3, 1, 1, 1)             \
+    MG_POOL_GATHER_SIG(T, TD, 1, 2, 2, 1, 1, 1)             \
+    MG_POOL_GATHER_SIG(T, TD, 3, 3, 3, 2, 2, 2)             \
   } while (0)
   if (!f32)
     MG_POOL_GATHER(double, double);
@@ -1208,6 +1316,7 @@ static int launch_mark_gather(const PoolParams &p, bool f32, bool wide, const un
     MG_POOL_GATHER(float, float);
 #undef MG_POOL_GATHER
 #undef MG_POOL_GATHER_SIG
+  if (!launched) return fail(MG_ERR_UNSUPPORTED, "no compile-time instance for pooling window signature %d", sig6);
   MG_HIP(hipGetLastError());
   return MG_OK;
 }
@@ -1310,7 +1419,8 @@ static int maxpool_fwd_impl(const mg_pool_desc *desc, const void *x, void *out, 
 }
 
 // Backward pass from recorded argmax offsets.
-static int maxpool_bwd_from_mark(const mg_pool_desc *desc, const unsigned char *mark, const void *grad, void *dx) {
+static int maxpool_bwd_from_mark(const mg_pool_desc *desc, const unsigned char *mark, const void *grad, void *dx,
+                                 bool own_timing = true) {
   PoolParams p;
   if (int rc = check_pool_desc(desc, &p)) return rc;
   if (!mark || !grad || !dx) return fail(MG_ERR_BAD_ARG, "null tensor pointer in the max-pool backward pass");
@@ -1318,7 +1428,8 @@ static int maxpool_bwd_from_mark(const mg_pool_desc *desc, const unsigned char *
     return fail(MG_ERR_UNSUPPORTED, "a window of %lld elements does not fit the one-byte argmax record (at most 256)",
                 (long long)p.P[0] * p.P[1] * p.P[2]);
   hipStream_t s = runtime().stream;
-  ScopedTiming timed(TAG_POOL_BWD);
+  std::optional<ScopedTiming> timed;
+  if (own_timing) timed.emplace(TAG_POOL_BWD);  // else: a part of the caller's pass
   const bool f32 = desc->dtype == MG_F32, wide = desc->dx_dtype == MG_F64;
   PoolExactParams ep;
   // the exact-tiling test looks at the alignment of x; grad stands in for it here
@@ -1572,6 +1683,25 @@ int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, vo
 #undef MG_POOL_BWD_SIG
     MG_HIP(hipGetLastError());
     return MG_OK;
+  }
+  if ((long long)p.P[0] * p.P[1] * p.P[2] <= 256) {
+    // No room in LDS for a band of this shape: one pass that records every window's argmax in the
+    // library workspace (a thread per window), then the routing from those bytes (a thread per 16
+    // bytes of dx walks the few windows that cover it).  The kernel below, a thread per element
+    // that scans every covering window itself, reads x prod(P) / prod(S) times over.
+    void *marks = nullptr;
+    if (int rc = workspace((size_t)(p.lead * p.gvol), &marks)) return rc;
+    const unsigned mgrid = grid_for(p.lead * p.gvol);
+    if (desc->dtype == MG_F32)
+      hipLaunchKernelGGL((maxpool_fwd_kernel<float, true>), dim3(mgrid), dim3(256), 0, s, p, (const float *)x, (float *)nullptr,
+                         (unsigned char *)marks);
+    else
+      hipLaunchKernelGGL((maxpool_fwd_kernel<double, true>), dim3(mgrid), dim3(256), 0, s, p, (const double *)x, (double *)nullptr,
+                         (unsigned char *)marks);
+    MG_HIP(hipGetLastError());
+    const int rc = maxpool_bwd_from_mark(desc, (const unsigned char *)marks, grad, dx, false);
+    note_plan("pool bwd: argmax pass (thread per window) + routing from the record, no staging");
+    return rc;
   }
   note_plan("pool bwd: thread per element, no staging");
   const unsigned grid = grid_for(p.lead * p.xvol);

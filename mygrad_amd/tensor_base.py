@@ -268,6 +268,10 @@ class Tensor:
             # remembers who holds it, and locks the array on their behalf when it is read
             for t in (*tensor_vars, out):
                 if t.on_device:
+                    # a device tensor that is never read on the host (a weight in a training loop)
+                    # would collect one dead reference per operation: drop them as the list grows
+                    if len(t._guards) >= 32:
+                        t._guards = [ref for ref in t._guards if ref() is not None]
                     t._guards.append(ref_f)
             finalize(f, _graph.release, guarded)
         _device.drop_pending()
@@ -304,7 +308,7 @@ class Tensor:
                         f"`grad` must be broadcast-compatible with `tensor.shape={self.shape}`\n"
                         f"Got `grad.shape={seed.shape}`"
                     )
-        elif self._creator is not None and self.on_device and self.size:
+        elif self._creator is not None and self.on_device and self.size and self.dtype in (np.float16, np.float32, np.float64):
             seed = _device.full(self.shape, self.dtype, 1.0)
         else:
             seed = np.ones(self.shape, dtype=self.dtype)

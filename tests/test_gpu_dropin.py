@@ -619,6 +619,55 @@ def test_max_pool_of_float16_is_exact():
     assert np.array_equal(x.grad.view(np.uint16), want.view(np.uint16))
 
 
+def test_float16_results_seed_backward_without_being_read():
+    """backward() with no argument on a float16 result that is still on the device: the all-ones
+    seed (tensor_base.py:1330-1334) is made on the device too, and the gradients are those of a
+    seed of ones handed in from the host."""
+    rng = np.random.default_rng(80)
+    x16 = rng.standard_normal((2, 6, 9, 9)).astype(np.float16)
+    w16 = (rng.standard_normal((4, 6, 3, 3)) / 7).astype(np.float16)
+    for make in (lambda x, w: conv_nd(x, w, stride=2), lambda x, w: max_pool(conv_nd(x, w, stride=1), (3, 3), 2)):
+        x, w = mg.Tensor(x16), mg.Tensor(w16)
+        out = make(x, w)
+        assert out.on_device and out.dtype == np.float16
+        out.backward()
+        x2, w2 = mg.Tensor(x16), mg.Tensor(w16)
+        out2 = make(x2, w2)
+        out2.backward(np.ones(out2.shape, dtype=np.float16))
+        assert x.grad.dtype == np.float16 and w.grad.dtype == np.float16
+        assert np.array_equal(x.grad.view(np.uint16), x2.grad.view(np.uint16))
+        assert np.array_equal(w.grad.view(np.uint16), w2.grad.view(np.uint16))
+
+
+def test_integer_result_on_the_device_meets_a_float_operand():
+    """repeat() of an integer tensor leaves an integer array on the device; multiplying it by a
+    float tensor converts it through the host, as NumPy would promote it."""
+    a = np.arange(12, dtype=np.int64).reshape(3, 4)
+    b = np.linspace(-1.0, 1.0, 24).reshape(3, 8)
+    for dtype in (np.float64, np.float32):
+        r = mg.repeat(mg.Tensor(a), 2, axis=1)
+        assert r.dtype == np.int64
+        f = mg.Tensor(b.astype(dtype))
+        prod = r * f
+        want = np.repeat(a, 2, axis=1) * b.astype(dtype)
+        assert prod.dtype == want.dtype
+        assert np.array_equal(prod.data, want)
+        prod.backward()
+        assert np.array_equal(f.grad, np.repeat(a, 2, axis=1).astype(dtype))
+
+
+def test_weight_that_stays_on_the_device_keeps_no_dead_references():
+    """A device tensor that is never read on the host (a weight in a training loop) remembers the
+    operations that hold it read-only; the list must not grow with the number of steps."""
+    rng = np.random.default_rng(81)
+    w = mg.device_tensor(rng.standard_normal((8, 4, 3, 3)))
+    x = mg.device_tensor(rng.standard_normal((2, 4, 8, 8)), constant=True)
+    for _ in range(300):
+        conv_nd(x, w, stride=1).backward()
+    assert len(w._guards) <= 64 and len(x._guards) <= 64
+    assert w.grad.shape == w.shape
+
+
 def test_complex_operands_under_no_autodiff_carry_a_complex_step():
     """The reference's tests differentiate conv_nd numerically with a complex step through the
     operation itself (tests/nnet/layers/test_conv.py:291-300, tests/utils/numerical_gradient.py):

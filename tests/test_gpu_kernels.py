@@ -124,6 +124,12 @@ def test_pool_ties_and_overlap_bit_exact(pools, m, lead, dtype):
     ((3,), (7, 9), (2, 2), (1, 1)),
     ((2,), (5, 6), (3, 3), (1, 1)),       # a short piece of two float32 columns
     ((2,), (3, 3), (3, 3), (2, 2)),       # a float32 row shorter than one piece
+    # 3 x 3 x 3 windows at every other position: the same kernels with a pooled leading axis
+    ((2, 2), (7, 9, 13), (3, 3, 3), (2, 2, 2)),
+    ((3,), (5, 7, 8), (3, 3, 3), (2, 2, 2)),     # flooring placement along the last axis
+    ((2,), (8, 10, 12), (3, 3, 3), (2, 2, 2)),   # the last plane, row and column are never covered
+    ((1,), (9, 65, 65), (3, 3, 3), (2, 2, 2)),   # planes too large for a band in LDS
+    ((2,), (3, 5, 9), (3, 3, 3), (2, 2, 2)),     # a single window plane
 ])
 def test_pool_backward_gather_for_windows_known_at_compile_time(pools, dtype, lead, X, pool, stride):
     """2-D windows of 3x3 / stride 2, 3x3 / stride 1 and 2x2 / stride 1 over rows of whole 16-byte
@@ -181,7 +187,8 @@ def test_pool_windows_that_tile_the_input_exactly(pools, dtype, lead, X, pool):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
-@pytest.mark.parametrize("X,pool,stride", [((7, 9001), (3, 3), (2, 2)), ((2, 5, 7000), (2, 3, 2), (1, 2, 3))])
+@pytest.mark.parametrize("X,pool,stride", [((7, 9001), (3, 3), (2, 2)), ((2, 5, 7000), (2, 3, 2), (1, 2, 3)),
+                                           ((7, 70, 70), (2, 3, 3), (1, 2, 2)), ((5, 9000), (4, 2), (1, 1))])
 def test_pool_rows_too_long_for_the_staged_kernels(pools, dtype, X, pool, stride):
     """One row of windows with its halo exceeds the LDS budget: the kernels that work
     element by element from global memory take over."""
@@ -397,6 +404,13 @@ FUSED_PHASE_CASES = [
     ((2, 24, 9, 16, 20), (32, 24, 3, 3, 3), (1, 2, 2), (1, 1, 1), (1, 1, 1)),
     ((40, 128, 28, 28), (256, 128, 3, 3), (2, 2), (1, 1), (1, 1)),
     ((2, 8, 12, 10), (16, 8, 3, 3), (2, 2), (0, 0), (1, 1)),
+    # exact window grids under stride 2 (odd extents): rows of dx start on no 16-byte boundary; an even
+    # and an odd number of coarse positions per row (pairs of positions / single positions per store)
+    ((3, 64, 13, 13), (32, 64, 3, 3), (2, 2), (1, 1), (1, 1)),
+    ((2, 32, 55, 55), (64, 32, 3, 3), (2, 2), (1, 1), (1, 1)),
+    ((2, 128, 9, 27), (16, 128, 3, 3), (1, 2), (1, 1), (1, 1)),
+    ((2, 16, 5, 7, 11), (32, 16, 3, 3, 3), (1, 2, 2), (1, 1, 1), (1, 1, 1)),
+    ((2, 64, 15, 15), (32, 64, 1, 1), (2, 2), (0, 0), (1, 1)),
 ]
 
 
@@ -416,6 +430,35 @@ def test_conv_dgrad_with_fused_stride_phases(abi, case, plan_mode):
     ones_g = np.ones_like(g)
     assert np.array_equal(abi.conv_dgrad(ones_g, x_shape, ones_w, s, p, d),
                           direct.conv_backward_x(ones_g, x_shape, ones_w, s, p, d).astype(np.float32))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("x_shape,w_shape,s,p,d", [
+    ((5, 64, 7, 7), (64, 64, 3, 3), (1, 1), (1, 1), (1, 1)),       # 49 positions per sample
+    ((3, 64, 27, 27), (128, 64, 3, 3), (1, 1), (1, 1), (1, 1)),    # 729
+    ((2, 48, 5, 9, 3), (64, 48, 3, 3, 1), (1, 1, 1), (1, 1, 0), (1, 1, 1)),
+    ((7, 128, 13), (64, 128, 5), (1,), (2,), (1,)),
+    ((4, 64, 30, 31), (64, 64, 3, 3), (2, 2), (1, 1), (1, 1)),     # forward only: a 15 x 15 grid
+])
+def test_conv_samples_that_are_no_whole_16_byte_pieces(abi, dtype, x_shape, w_shape, s, p, d, monkeypatch):
+    """An odd number of positions per sample: a lane's positions are adjacent in the result but
+    not 16-byte aligned, and the last lane of a sample holds positions of two samples."""
+    monkeypatch.setenv("MYGRAD_HIP_TINY", "0")
+    rng = np.random.default_rng(1450 + x_shape[-1])
+    tol = TOL[np.dtype(dtype)]
+    x = rng.standard_normal(x_shape).astype(dtype)
+    w = (rng.standard_normal(w_shape) / np.sqrt(np.prod(w_shape[1:]))).astype(dtype)
+    want = direct.conv_forward(x, w, s, p, d)
+    g = rng.standard_normal(want.shape).astype(dtype)
+    assert rel_err(abi.conv_fwd(x, w, s, p, d), want) <= tol
+    assert rel_err(abi.conv_dgrad(g, x_shape, w, s, p, d), direct.conv_backward_x(g, x_shape, w, s, p, d)) <= tol
+    assert rel_err(abi.conv_wgrad(g, x, w_shape, s, p, d), direct.conv_backward_w(g, x, w_shape, s, p, d)) <= tol
+    # exact with ones: an element stored to the wrong place changes a count
+    ones_x, ones_w = np.ones(x_shape, dtype), np.ones(w_shape, dtype)
+    assert np.array_equal(abi.conv_fwd(ones_x, ones_w, s, p, d), direct.conv_forward(ones_x, ones_w, s, p, d).astype(dtype))
+    ones_g = np.ones_like(g)
+    assert np.array_equal(abi.conv_dgrad(ones_g, x_shape, ones_w, s, p, d),
+                          direct.conv_backward_x(ones_g, x_shape, ones_w, s, p, d).astype(dtype))
 
 
 # Few channels (filters, in the forward pass), a 3-tap "same" last axis whose rows are a power of
@@ -584,6 +627,10 @@ THIN_FILTER_CASES = [
     # a first layer with more than 64 filters: passes of 64 rows over the same positions
     ((128, 3, 64, 64), (96, 3, 4, 4), (2, 2), (1, 1), (1, 1)),      # a pass of 64 and one of 32
     ((64, 1, 64, 64), (130, 1, 3, 3), (1, 1), (1, 1), (1, 1)),      # three passes, two rows in the last
+    # a first layer of 8, 16 and 32 filters: two, four and eight groups of four rows
+    ((64, 3, 64, 64), (8, 3, 3, 3), (1, 1), (1, 1), (1, 1)),
+    ((32, 3, 96, 96), (16, 3, 5, 5), (2, 2), (2, 2), (1, 1)),
+    ((64, 2, 64, 64), (32, 2, 3, 3), (1, 1), (1, 1), (1, 1)),
 ]
 
 
