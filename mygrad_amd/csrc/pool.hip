@@ -696,6 +696,16 @@ __device__ __forceinline__ T from_next_lane(T value) {
   return __shfl_down(value, 1, 64);
 }
 
+// Blocks are handed to the 8 XCDs round-robin, and each XCD has its own L2.  Neighbouring work
+// items share rows and planes of x (windows overlap) and entries of the record, so the blocks
+// b, b + 8, ... of one XCD take consecutive runs of items: block b is the (b / 8)-th block of XCD
+// b % 8 and takes the (b / 8)-th run of that XCD's eighth of the work.
+__device__ __forceinline__ unsigned xcd_run(unsigned block, unsigned blocks) {
+  const unsigned xcd = block % 8u, nth = block / 8u;
+  const unsigned per = blocks / 8u, extra = blocks % 8u;
+  return xcd * per + min(xcd, extra) + nth;
+}
+
 template <typename T, int P0, int P1, int P2, int S0, int S1, int S2, bool MARK, bool STORE_OUT = true>
 __global__ void __launch_bounds__(256) maxpool_rows_fwd_kernel(PoolRowsParams p, const T *__restrict__ x, T *__restrict__ out,
                                                               unsigned char *__restrict__ mark) {
@@ -707,7 +717,7 @@ __global__ void __launch_bounds__(256) maxpool_rows_fwd_kernel(PoolRowsParams p,
   static_assert(VEC % S2 == 0 && HALO >= 0 && HALO <= VEC, "piece / window geometry");
   typedef T Vec __attribute__((ext_vector_type(VEC), aligned(sizeof(T))));
   const int lane = threadIdx.x & 63;
-  const long long wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const long long wave = (long long)xcd_run(blockIdx.x, gridDim.x) * 4 + (threadIdx.x >> 6);
   const long long item = wave * 63 + lane;  // wavefronts overlap by one lane
   const unsigned u = (unsigned)(item < p.items ? item : p.items - 1);  // clamped: every lane loads, some do not store
   const unsigned q = p.by_pieces.div(u), piece = u - q * (unsigned)p.pieces;
@@ -834,7 +844,7 @@ __global__ void __launch_bounds__(256) maxpool_mark_gather_kernel(PoolGatherPara
   constexpr int LW = NW2 <= 2 ? 2 : NW2 <= 4 ? 4 : 8;  // windows loaded per window row
   static_assert(VD % S2 == 0 && NW2 <= 8, "a piece starts on a window boundary");
   typedef TD DVec __attribute__((ext_vector_type(VD), aligned(sizeof(TD))));
-  const long long item = (long long)blockIdx.x * 256 + threadIdx.x;
+  const long long item = (long long)xcd_run(blockIdx.x, gridDim.x) * 256 + threadIdx.x;
   if (item >= p.planes * p.groups * p.pieces) return;
   const unsigned u = (unsigned)item;
   const unsigned q = p.by_pieces.div(u), piece = u - q * (unsigned)p.pieces;
