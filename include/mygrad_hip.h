@@ -197,6 +197,17 @@ int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, vo
 int mg_maxpool_fwd_argmax(const mg_pool_desc *desc, const void *x, void *out, void *argmax);
 int mg_maxpool_bwd_argmax(const mg_pool_desc *desc, const void *argmax, const void *grad, void *dx);
 
+/* Backward pass of a pooling over four or five axes that ran as two mg_maxpool_fwd_argmax calls:
+ * `inner` over the last three axes (its leading index runs over the un-pooled axes and the leading
+ * pooled ones), then `outer` over the leading pooled axes of its result (nd = 2 or 3, the last axis
+ * being the inner stage's merged grid with a window of one element placed at every position).
+ * grad:(outer lead, outer grid) is routed to dx:(inner lead, inner X...) through both records, every
+ * element adding its windows in the row-major order of the whole windows: what np.add.at does for
+ * a pooling over all the axes at once, MaxPoolND.backward_var, src/mygrad/nnet/layers/pooling.py:136-148,
+ * bit for bit (routing the two stages one after the other adds the same terms in another order). */
+int mg_maxpool_bwd_argmax_staged(const mg_pool_desc *inner, const mg_pool_desc *outer, const void *inner_argmax,
+                                 const void *outer_argmax, const void *grad, void *dx);
+
 /* ---- element-wise and whole-array kernels either side of conv / pool ----
  * dtype: 0 float32, 1 float64; n elements, C-contiguous, same shape; device pointers,
  * 16-byte aligned (what mg_malloc returns). */

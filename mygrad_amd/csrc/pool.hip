@@ -980,6 +980,74 @@ __global__ void __launch_bounds__(256) maxpool_exact_from_mark_kernel(PoolExactP
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// Pooling over four or five axes runs as two stages: the last three axes first (`inner`: every
+// leading position pooled on its own), then the leading pooled axes over the merged grid of the
+// first stage (`outer`: windows of one element along that merged axis).  Both stages record where
+// each of their windows found its maximum, and together the two records name the element of x a
+// whole window routes its gradient to: the first stage's byte inside the leading position that
+// the second stage's byte picks.  A thread owns one element of dx and walks the whole windows
+// that cover it in ascending row-major order -- windows along the leading axes outermost, as
+// np.add.at visits them (pooling.py:147-148) -- adding grad where both records name the
+// element: one sequential sum from +0.0, carried in double, the reference's order bit for bit.
+// (Routing stage by stage adds a leading position's windows first and the positions afterwards:
+// the same terms, another association.)
+// ------------------------------------------------------------------------------------------
+struct PoolStagedParams {
+  int X[3], P[3], S[3], G[3];      // inner stage: the last three pooled axes
+  int OX[2], OP[2], OS[2], OG[2];  // outer stage: the leading pooled axes (extent 1 where there is none)
+  int xvol, gvol;                  // elements of x / windows per leading position of the inner stage
+  long long total;                 // elements of dx
+  FastDivP by_xvol, by_x12, by_x2, by_ox1, by_ox01, by_s[3], by_os[2];
+};
+
+template <typename T, typename TD>
+__global__ void __launch_bounds__(256) maxpool_staged_gather_kernel(PoolStagedParams p, const unsigned char *__restrict__ inner_mark,
+                                                                   const unsigned char *__restrict__ outer_mark,
+                                                                   const T *__restrict__ grad, TD *__restrict__ dx) {
+  for (long long idx = (long long)blockIdx.x * 256 + threadIdx.x; idx < p.total; idx += (long long)gridDim.x * 256) {
+    // element -> (leading index, q0, q1 | i0, i1, i2); leading positions fit 32 bits (checked by the host)
+    const unsigned pos = (unsigned)(idx / p.xvol);  // (leading index, q0, q1)
+    unsigned r = (unsigned)(idx - (long long)pos * p.xvol);
+    const int i0 = (int)p.by_x12.div(r);
+    r -= (unsigned)i0 * (unsigned)(p.X[1] * p.X[2]);
+    const int i1 = (int)p.by_x2.div(r);
+    const int i2 = (int)r - i1 * p.X[2];
+    const unsigned lead = p.by_ox01.div(pos);
+    const unsigned q01 = pos - lead * (unsigned)(p.OX[0] * p.OX[1]);
+    const int q0 = (int)p.by_ox1.div(q01), q1 = (int)q01 - q0 * p.OX[1];
+    const int i[3] = {i0, i1, i2}, q[2] = {q0, q1};
+    int lo[3], hi[3], olo[2], ohi[2];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+      lo[k] = i[k] >= p.P[k] ? (int)p.by_s[k].div((unsigned)(i[k] - p.P[k] + p.S[k])) : 0;
+      hi[k] = min(p.G[k] - 1, (int)p.by_s[k].div((unsigned)i[k]));
+    }
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      olo[k] = q[k] >= p.OP[k] ? (int)p.by_os[k].div((unsigned)(q[k] - p.OP[k] + p.OS[k])) : 0;
+      ohi[k] = min(p.OG[k] - 1, (int)p.by_os[k].div((unsigned)q[k]));
+    }
+    const unsigned char *m1 = inner_mark + (long long)pos * p.gvol;
+    double acc = 0.0;
+    for (int h0 = olo[0]; h0 <= ohi[0]; ++h0)
+      for (int h1 = olo[1]; h1 <= ohi[1]; ++h1) {
+        const int mine_outer = (q0 - h0 * p.OS[0]) * p.OP[1] + (q1 - h1 * p.OS[1]);
+        const long long orow = (((long long)lead * p.OG[0] + h0) * p.OG[1] + h1) * p.gvol;
+        for (int g0 = lo[0]; g0 <= hi[0]; ++g0)
+          for (int g1 = lo[1]; g1 <= hi[1]; ++g1) {
+            const int row = (g0 * p.G[1] + g1) * p.G[2];
+            const int mine01 = ((i0 - g0 * p.S[0]) * p.P[1] + (i1 - g1 * p.S[1])) * p.P[2];
+            for (int g2 = lo[2]; g2 <= hi[2]; ++g2) {
+              const bool here = (int)m1[row + g2] == mine01 + (i2 - g2 * p.S[2]) && (int)outer_mark[orow + row + g2] == mine_outer;
+              if (here) acc += (double)grad[orow + row + g2];
+            }
+          }
+      }
+    dx[idx] = (TD)acc;
+  }
+}
+
 static int check_pool_desc(const mg_pool_desc *d, PoolParams *p) {
   if (!d) return fail(MG_ERR_BAD_ARG, "pool descriptor is null");
   if (d->dtype != MG_F32 && d->dtype != MG_F64)
@@ -1593,6 +1661,57 @@ int mg_maxpool_bwd_argmax(const mg_pool_desc *desc, const void *argmax, const vo
   std::lock_guard<std::recursive_mutex> guard(api_mutex());
   MG_REQUIRE_INIT();
   return maxpool_bwd_from_mark(desc, static_cast<const unsigned char *>(argmax), grad, dx);
+}
+
+int mg_maxpool_bwd_argmax_staged(const mg_pool_desc *inner, const mg_pool_desc *outer, const void *inner_argmax,
+                                 const void *outer_argmax, const void *grad, void *dx) {
+  std::lock_guard<std::recursive_mutex> guard(api_mutex());
+  MG_REQUIRE_INIT();
+  PoolParams pi, po;
+  if (int rc = check_pool_desc(inner, &pi)) return rc;
+  if (int rc = check_pool_desc(outer, &po)) return rc;
+  if (!inner_argmax || !outer_argmax || !grad || !dx) return fail(MG_ERR_BAD_ARG, "null pointer in mg_maxpool_bwd_argmax_staged");
+  if (inner->dtype != outer->dtype || inner->dx_dtype != outer->dx_dtype)
+    return fail(MG_ERR_BAD_ARG, "the two stages disagree on the types");
+  // the outer stage pools the leading axes over the inner stage's windows: its last axis is their
+  // merged grid with a window of one element, and its positions are the inner stage's leading indices
+  if (po.X[2] != pi.gvol || po.P[2] != 1 || po.S[2] != 1 || po.G[2] != pi.gvol || po.lead * po.X[0] * po.X[1] != pi.lead)
+    return fail(MG_ERR_BAD_ARG, "the outer stage (lead %lld, extents %d x %d x %d) does not pool the inner stage's %lld positions of %lld windows",
+                po.lead, po.X[0], po.X[1], po.X[2], pi.lead, pi.gvol);
+  if ((long long)pi.P[0] * pi.P[1] * pi.P[2] > 256 || (long long)po.P[0] * po.P[1] > 256)
+    return fail(MG_ERR_UNSUPPORTED, "a window of more than 256 elements does not fit the one-byte argmax record");
+  if (pi.lead >= (1ll << 31) || po.lead * po.G[0] * po.G[1] * pi.gvol >= (1ll << 40))
+    return fail(MG_ERR_UNSUPPORTED, "too many leading positions for the staged gather");
+  PoolStagedParams q{};
+  for (int k = 0; k < 3; ++k) {
+    q.X[k] = pi.X[k], q.P[k] = pi.P[k], q.S[k] = pi.S[k], q.G[k] = pi.G[k];
+    q.by_s[k] = make_fastdiv_p((unsigned)pi.S[k]);
+  }
+  for (int k = 0; k < 2; ++k) {
+    q.OX[k] = po.X[k], q.OP[k] = po.P[k], q.OS[k] = po.S[k], q.OG[k] = po.G[k];
+    q.by_os[k] = make_fastdiv_p((unsigned)po.S[k]);
+  }
+  q.xvol = (int)pi.xvol;
+  q.gvol = (int)pi.gvol;
+  q.total = pi.lead * pi.xvol;
+  q.by_xvol = make_fastdiv_p((unsigned)pi.xvol);
+  q.by_x12 = make_fastdiv_p((unsigned)(pi.X[1] * pi.X[2]));
+  q.by_x2 = make_fastdiv_p((unsigned)pi.X[2]);
+  q.by_ox1 = make_fastdiv_p((unsigned)po.X[1]);
+  q.by_ox01 = make_fastdiv_p((unsigned)(po.X[0] * po.X[1]));
+  hipStream_t s = runtime().stream;
+  ScopedTiming timed(TAG_POOL_BWD);
+  note_plan("pool bwd from two stages' argmax: thread per element of dx, whole windows in row-major order");
+  const unsigned grid = grid_for(q.total);
+  const unsigned char *m1 = static_cast<const unsigned char *>(inner_argmax), *m2 = static_cast<const unsigned char *>(outer_argmax);
+  if (inner->dtype == MG_F64)
+    hipLaunchKernelGGL((maxpool_staged_gather_kernel<double, double>), dim3(grid), dim3(256), 0, s, q, m1, m2, (const double *)grad, (double *)dx);
+  else if (inner->dx_dtype == MG_F64)
+    hipLaunchKernelGGL((maxpool_staged_gather_kernel<float, double>), dim3(grid), dim3(256), 0, s, q, m1, m2, (const float *)grad, (double *)dx);
+  else
+    hipLaunchKernelGGL((maxpool_staged_gather_kernel<float, float>), dim3(grid), dim3(256), 0, s, q, m1, m2, (const float *)grad, (float *)dx);
+  MG_HIP(hipGetLastError());
+  return MG_OK;
 }
 
 int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, void *dx) {

@@ -503,6 +503,49 @@ def test_pooling_over_more_axes_than_the_kernels_take(case, dtype):
     assert _graph.held_count() == 0
 
 
+@pytest.mark.parametrize("dtype", [np.float64, np.float32])
+@pytest.mark.parametrize("x_shape,pool,stride", [
+    ((2, 7, 6, 7, 8), (3, 2, 3, 2), (1, 2, 2, 3)),          # four pooled axes, windows that overlap along three of them
+    ((3, 5, 6, 5, 7, 9), (2, 3, 2, 3, 3), (1, 1, 1, 2, 2)),  # five
+    ((6, 5, 5, 5), (3, 3, 3, 3), (1, 1, 1, 1)),              # every element under up to 81 windows, no leading axes
+])
+def test_pooling_over_four_and_five_axes_adds_in_the_reference_order(x_shape, pool, stride, dtype):
+    """Real-valued gradients of very different magnitudes: the sum an element receives depends on
+    the order of its terms, and must be np.add.at's (pooling.py:147-148) bit for bit -- also for a
+    float32 x, whose sums the reference carries in float64 and rounds once."""
+    rng = np.random.default_rng(4100 + len(pool))
+    xv = rng.integers(0, 3, x_shape).astype(dtype)  # ties: an element is the argmax of many windows
+    out_shape = ora.pool_forward(xv, pool, stride).shape
+    g = (rng.standard_normal(out_shape) * 10.0 ** rng.integers(-6, 6, out_shape)).astype(dtype)
+    g[rng.random(out_shape) < 0.1] = -0.0
+    x = mg.Tensor(xv)
+    max_pool(x, pool, stride).backward(g)
+    want = ora.pool_backward(xv, g, pool, stride)  # float64
+    kind = np.uint64 if dtype == np.float64 else np.uint32
+    assert np.array_equal(x.grad.view(kind), want.astype(dtype).view(kind))
+    # the float64 route (a gradient that is added to one the tensor already holds): x feeds two
+    # poolings whose outputs are multiplied, so each sends g * (the other's output) back
+    x2 = mg.Tensor(xv)
+    a, b = max_pool(x2, pool, stride), max_pool(x2, pool, stride)
+    mg.sum(a * b * mg.Tensor(g, constant=True)).backward()
+    sent = (g * ora.pool_forward(xv, pool, stride)).astype(dtype)  # one rounding, like the device's multiply
+    each = ora.pool_backward(xv, sent, pool, stride)  # float64
+    assert np.array_equal(x2.grad.view(kind), (each.astype(dtype).astype(np.float64) + each).astype(dtype).view(kind))
+    assert _graph.held_count() == 0
+
+
+def test_window_with_zeros_of_both_signs_keeps_the_first_ones_sign():
+    """np.max over a window that holds +0.0 and -0.0 returns either, depending on the order and the
+    vector width (implementation-defined); here the first of the equal maxima wins, as np.argmax
+    picks it, and the gradient goes to that element."""
+    for first, second in ((0.0, -0.0), (-0.0, 0.0)):
+        x = mg.Tensor(np.array([[first, second, -1.0, second]]))
+        out = max_pool(x, (4,), 4)
+        assert np.signbit(out.data[0, 0]) == np.signbit(first)
+        out.backward(np.array([[5.0]]))
+        assert np.array_equal(x.grad, [[5.0, 0.0, 0.0, 0.0]])
+
+
 def test_pooling_over_four_axes_with_a_leading_window_of_one():
     rng = np.random.default_rng(32)
     xv = rng.integers(0, 4, (2, 3, 5, 6, 8)).astype(np.float64)
