@@ -64,6 +64,11 @@ WORKLOADS = {
                  stride=(2, 2), padding=(3, 3), dilation=(1, 1), constant_input=True),
     "stem-dx": dict(kind="conv", dtype="f32", seed=1017, x=(128, 3, 224, 224), w=(64, 3, 7, 7), wscale=(2 / 147) ** 0.5,
                     stride=(2, 2), padding=(3, 3), dilation=(1, 1)),
+    # the same stem in double precision, the reference's default dtype (half the batch: the same bytes)
+    "stem64": dict(kind="conv", dtype="f64", seed=1017, x=(64, 3, 224, 224), w=(64, 3, 7, 7), wscale=(2 / 147) ** 0.5,
+                   stride=(2, 2), padding=(3, 3), dilation=(1, 1), constant_input=True),
+    "stem64-dx": dict(kind="conv", dtype="f64", seed=1017, x=(64, 3, 224, 224), w=(64, 3, 7, 7), wscale=(2 / 147) ** 0.5,
+                      stride=(2, 2), padding=(3, 3), dilation=(1, 1)),
     "pool2": dict(kind="pool", dtype="f64", seed=1002, x=(64, 64, 56, 56), pool=(3, 3), stride=(2, 2)),
     "pool5": dict(kind="pool", dtype="f32", seed=1006, x=(8, 32, 32, 64, 64), pool=(2, 2, 2), stride=(2, 2, 2)),
     # the same two with each window's argmax recomputed from x in the backward pass (the stateless

@@ -107,6 +107,25 @@ __global__ void __launch_bounds__(256) pack_transpose_kernel(const T *__restrict
   }
 }
 
+// Stride phases as rows (see GemmParams::phase_count): Ap[(e * F + f)][c * phases + phase] = w[f][c][tap of offset e in
+// that phase], zero where the phase has no tap at that offset; taps[e * phases + phase] names the tap (-1: none).
+template <typename T>
+__global__ void __launch_bounds__(256) pack_phase_rows_kernel(const T *__restrict__ w, T *__restrict__ ap, const int *__restrict__ taps,
+                                                              int entries, int phases, int F, int C, int wvol, int ld) {
+  const long long total = (long long)entries * F * ld;
+  for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long long)gridDim.x * blockDim.x) {
+    const int m = (int)(idx % ld);
+    const long long row = idx / ld;
+    const int f = (int)(row % F), e = (int)(row / F);
+    T v = T(0);
+    if (m < phases * C) {
+      const int tap = taps[e * phases + m % phases];
+      if (tap >= 0) v = w[((long long)f * C + m / phases) * wvol + tap];
+    }
+    ap[idx] = v;
+  }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256) pack_filters_kernel(const T *__restrict__ w, T *__restrict__ ap, int F, int C,
                                                            int wvol, int mode, int ld) {
@@ -591,6 +610,8 @@ struct Plan {
   bool table_rows = false;          // tap-major kernel whose K tiles are rows of the gather table (channel count no multiple of the K tile)
   int table_count = 0;              // data gradient on table rows: rows of the (padded) table = rows of the packed filters
   int fold_row = 0;                 // data gradient with the last axis' three taps folded into the rows: length of a row of positions
+  int phase_rows = 0;               // data gradient with the stride phases as rows of the GEMM (GemmParams::phase_count): the channel count
+  int phase_count = 0;              // ... and the number of phases; table_count is then the number of distinct gathered offsets
   bool deep_k = false;              // table-driven, a few microseconds of work: 16 x 64 tiles with a K tile four times as deep
   // fused stride phases of the data gradient (see GemmParams::nph)
   int nph = 1;
@@ -1520,6 +1541,73 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
     return upload_plan(pl, t);
   }
 
+  // ---- a few channels under a stride, not taken by the kernel above (double precision, or too few
+  // positions for it): the stride phases become rows of the GEMM.  With three channels a 16-row tile
+  // has three live rows per phase; with the rows (phase, channel) over the coarse grid ceil(X / stride)
+  // it has phases x channels of them, and every gathered element of grad serves all phases of its
+  // coarse position (a zero in the packed filters where a phase has no tap for it).
+  static const bool phase_rows_on = [] {
+    const char *flag = getenv("MYGRAD_HIP_PHASE_ROWS");
+    return !(flag && flag[0] == '0');
+  }();
+  if (phase_rows_on && pl.tap_major && !pl.table_rows && nphase >= 2 && nphase <= 4 && (long long)found.size() == nphase &&
+      nphase * g.C <= 16 && g.C <= 8 && 2.0 * g.N * g.F * g.gvol * g.C * g.wvol >= 2e8) {
+    std::stable_sort(found.begin(), found.end(), [](const PhaseTaps &a, const PhaseTaps &b) {
+      if (a.ph.o0[0] != b.ph.o0[0]) return a.ph.o0[0] < b.ph.o0[0];
+      if (a.ph.o0[1] != b.ph.o0[1]) return a.ph.o0[1] < b.ph.o0[1];
+      return a.ph.o0[2] < b.ph.o0[2];
+    });
+    std::map<std::array<int, 3>, std::array<int, 4>> seen;  // gathered offset -> the tap it meets in each phase (-1: none)
+    for (int f = 0; f < (int)nphase; ++f) {
+      const PhaseTaps &pt = found[f];
+      for (int k = 0; k < 3; ++k) {
+        pl.po0[f][k] = pt.ph.o0[k];
+        pl.pJ[f][k] = pt.ph.J[k];
+      }
+      for (size_t a = 0; a < pt.taps[0].size(); ++a)
+        for (size_t b = 0; b < pt.taps[1].size(); ++b)
+          for (size_t c = 0; c < pt.taps[2].size(); ++c) {
+            const std::array<int, 3> d{pt.offs[0][a], pt.offs[1][b], pt.offs[2][c]};
+            auto it = seen.find(d);
+            if (it == seen.end()) it = seen.emplace(d, std::array<int, 4>{-1, -1, -1, -1}).first;
+            it->second[f] = (pt.taps[0][a] * g.W[1] + pt.taps[1][b]) * g.W[2] + pt.taps[2][c];
+          }
+    }
+    std::vector<std::array<int, 3>> offsets;
+    for (const auto &kv : seen) {
+      offsets.push_back(kv.first);
+      for (int f = 0; f < (int)nphase; ++f) t.arow.push_back(kv.second[f]);
+    }
+    const int entries = (int)offsets.size();
+    for (int f0 = 0; f0 < g.F; f0 += bk)  // filter block outermost: its offsets share a neighbourhood of grad
+      for (int e = 0; e < entries; ++e) {
+        KTile kt{};
+        kt.d0 = offsets[e][0], kt.d1 = offsets[e][1], kt.d2 = offsets[e][2];
+        kt.a_row0 = e * g.F + f0;
+        kt.coff = (int)(f0 * g.gvol) + kt.d0 * gs[0] + kt.d1 * gs[1] + kt.d2 * gs[2];
+        t.ktiles.push_back(kt);
+      }
+    Phase coarse{};
+    for (int k = 0; k < 3; ++k) coarse.J[k] = (g.X[k] + g.S[k] - 1) / g.S[k];
+    coarse.k_begin = 0;
+    coarse.k_count = (int)t.ktiles.size();
+    coarse.blk_begin = 0;
+    coarse.npos = (int)((long long)g.N * coarse.J[0] * coarse.J[1] * coarse.J[2]);
+    set_divisors(coarse);
+    const TileChoice tc = choose_tile((int)nphase * g.C, {(long long)coarse.npos}, coarse.k_count, true, g.dtype == MG_F64 ? 8 : 4, 1, bk);
+    if (tc.bm != 0 && coarse.k_count > 0) {
+      pl.bm = tc.bm, pl.bn = tc.bn, pl.m_tiles = tc.m_tiles, pl.full_tiles = tc.full_tiles, pl.tail_split = tc.tail_split, pl.blocks_per_cu = tc.blocks_per_cu;
+      pl.phase_rows = g.C;
+      pl.phase_count = (int)nphase;
+      pl.table_count = entries;
+      t.phases.push_back(coarse);
+      pl.pos_blocks = (int)ceil_div(coarse.npos, pl.bn);
+      return upload_plan(pl, t);
+    }
+    t.arow.clear();
+    t.ktiles.clear();
+  }
+
   // ---- stride 2 along the last axis: the phases' elements alternate in dx, and phases that
   // write them at different times make every line of dx cross HBM several times, partly
   // filled.  With 2 or 4 phases in all, every tile computes all of them for its patch of the
@@ -1878,7 +1966,7 @@ int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
              "%s: %s%s%s tile %dx%dx%d, %d phase(s) (%d fused per tile), %d position blocks x %d row tiles, %d whole tiles + %s, "
              "%d block(s) per unit, K splits %d",
              op == OP_FWD ? "fwd" : op == OP_DGRAD ? "dgrad" : "wgrad",
-             pl.thin ? "one position per lane" : pl.tap_major ? "tap-major" : "table-driven", pl.table_rows ? ", table rows" : "",
+             pl.thin ? "one position per lane" : pl.tap_major ? "tap-major" : "table-driven", pl.table_rows ? ", table rows" : pl.phase_rows ? ", stride phases as rows" : "",
              pl.fold_row ? ", folded taps" : "", pl.bm, pl.bn, pl.bk, pl.nphases, pl.nph, pl.pos_blocks, pl.m_tiles, pl.full_tiles, tail,
              pl.blocks_per_cu, pl.splits);
     // MYGRAD_HIP_TRACE=1 reports, once per new descriptor, what was planned
@@ -1946,6 +2034,13 @@ int run_gemm(GemmParams &gp, const Plan &pl, int tag, hipStream_t s) {
                  reinterpret_cast<uintptr_t>(gp.dst) % 16 == 0;
   gp.run_store = pl.single_dense_phase && !gp.vec_store;
   gp.nph = pl.nph;
+  gp.phase_count = pl.phase_rows ? pl.phase_count : 0;
+  // (the phases are sorted by their offsets, the last axis innermost: with a stride of two there, phases 2q and
+  // 2q + 1 differ by one element along it)
+  gp.phase_pairs = pl.phase_rows && gp.oj[2] == 2 && gp.os[2] == 1;
+  if (pl.phase_rows)
+    for (int f = 0; f < 4; ++f)
+      for (int k = 0; k < 3; ++k) gp.po0[f][k] = pl.po0[f][k], gp.pJ[f][k] = pl.pJ[f][k];
   if (pl.nph > 1) {
     for (int f = 0; f < 4; ++f) {
       gp.kcut[f] = pl.kcut[f];
@@ -2225,6 +2320,16 @@ int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
                          static_cast<T *>(packed), pl.arow, pl.table_count, (int)g.C, (int)g.wvol, ld);
       MG_HIP(hipGetLastError());
     }
+  } else if (pl.phase_rows) {
+    const int ld = packed_ld(pl.phase_count * g.C, true);
+    const size_t packed_bytes = ((size_t)pl.table_count * g.F * ld * sizeof(T) + 255) & ~size_t(255);
+    if (int rc = workspace(packed_bytes + tail_bytes(pl, sizeof(T)), &packed)) return rc;
+    partial = static_cast<char *>(packed) + packed_bytes;
+    ScopedTiming timed(TAG_PACK_FILTERS);
+    const unsigned blocks = (unsigned)std::min<long long>(ceil_div((long long)pl.table_count * g.F * ld, 256), 4096);
+    hipLaunchKernelGGL(pack_phase_rows_kernel<T>, dim3(blocks), dim3(256), 0, runtime().stream, static_cast<const T *>(w),
+                       static_cast<T *>(packed), pl.arow, pl.table_count, pl.phase_count, (int)g.F, (int)g.C, (int)g.wvol, ld);
+    MG_HIP(hipGetLastError());
   } else if (int rc = pack_filters<T>(g, w, pl.fold_row ? 4 : 3, &packed, tail_bytes(pl, sizeof(T)), &partial)) {
     return rc;
   }
@@ -2234,7 +2339,7 @@ int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   gp.a_mstride = (int)g.wvol;
   gp.src = grad;
   gp.dst = dx;
-  gp.M = g.C;
+  gp.M = pl.phase_rows ? pl.phase_count * g.C : g.C;
   const int qs[3] = {g.G[1] * g.G[2], g.G[2], 1};
   const int os[3] = {g.X[1] * g.X[2], g.X[2], 1};
   for (int k = 0; k < 3; ++k) {
@@ -2251,6 +2356,10 @@ int conv_dgrad_impl(const Geometry &g, const Plan &pl, const void *grad, const v
   gp.a_ld = pl.fold_row ? folded_ld<T>(g.C) : packed_ld(g.C, pl.tap_major);
   gp.a_bytes = pl.table_rows ? (unsigned)((size_t)pl.table_count * gp.a_ld * sizeof(T))
                              : (unsigned)((size_t)g.F * (pl.fold_row ? g.wvol / 3 : g.wvol) * gp.a_ld * sizeof(T));
+  if (pl.phase_rows) {
+    gp.a_ld = packed_ld(pl.phase_count * g.C, true);
+    gp.a_bytes = (unsigned)((size_t)pl.table_count * g.F * gp.a_ld * sizeof(T));
+  }
   gp.src_bytes = pl.tap_major ? (unsigned)((size_t)g.N * g.F * g.gvol * sizeof(T)) : 0;
   return run_gemm<T>(gp, pl, TAG_CONV_DGRAD, runtime().stream);
 }

@@ -142,6 +142,15 @@ struct GemmParams {
   // position's own place along that axis; the epilogue adds the three rows of an m, each shifted
   // by its tap's offset along the last axis (+1, 0, -1 positions), into the one row of dst.
   int fold_row;         // 0: not folded; else the length of a row of positions (a power of two, 4 .. 64)
+  // Stride phases as rows (data gradient of a few channels under a stride): the positions are the
+  // coarse grid J[k] = ceil(X[k] / stride[k]) and row m of the GEMM is stride phase m % phase_count
+  // of channel m / phase_count, so that every gathered element of grad serves all phases of its
+  // coarse position (the packed filters hold a zero where a phase has no tap for it) and the
+  // rows of an MFMA tile are channels x phases instead of channels alone.  po0 / pJ above say
+  // where a phase's elements lie in dst and which exist; phases 2q and 2q + 1 are rows next to
+  // each other and, with a stride of two along the last axis, elements next to each other.
+  int phase_count;      // 0: off; else the number of stride phases (2 or 4)
+  int phase_pairs;      // phases 2q, 2q + 1 are neighbours along the last axis of dst
 };
 
 // Gather-GEMM with one position per lane, for few rows (the data gradient of a layer with a

@@ -590,6 +590,33 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
             const T two[2] = {acc[0][i][2 * g], acc[0][i][2 * g + 1]};
             if (m < p.M) store_vec<T, 2>(out + (long long)m * p.dst_mstride, two);
           }
+        } else if (p.phase_count != 0) {
+          // rows are (channel, stride phase): each goes to its phase's element of the coarse position.
+          // The lane's rows 2r, 2r + 1 are phases 2q, 2q + 1 of one channel: neighbours along the
+          // last axis when that is where the stride is, stored together.
+          typedef T OutPair __attribute__((ext_vector_type(2), aligned(sizeof(T))));
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            if (first + h >= ph.npos) continue;
+            int n, j0, j1, j2;
+            split_pos(first + h, n, j0, j1, j2);
+#pragma unroll
+            for (int i = 0; i < GM; i += 2) {
+              const int m = m0 + drow + (i / 2) * 16;  // even: phase f even
+              if (m >= p.M) continue;
+              const int c = m / p.phase_count, f = m - c * p.phase_count;
+              const bool even = fused_ok(f, j0, j1, j2), odd = fused_ok(f + 1, j0, j1, j2);
+              T *out = fused_dst(f, n, j0, j1, j2) + (long long)c * p.dst_mstride;
+              if (p.phase_pairs && even && odd) {
+                OutPair v;
+                v[0] = acc[0][i][2 * g + h], v[1] = acc[0][i + 1][2 * g + h];
+                *reinterpret_cast<OutPair *>(out) = v;
+              } else {
+                if (even) out[0] = acc[0][i][2 * g + h];
+                if (odd) fused_dst(f + 1, n, j0, j1, j2)[(long long)c * p.dst_mstride] = acc[0][i + 1][2 * g + h];
+              }
+            }
+          }
         } else {
           // positions adjacent in dst but not 16-byte aligned: the pair as one vector of element
           // alignment when both lie in one sample
@@ -854,6 +881,23 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
               }
             }
         }
+      } else if (p.phase_count != 0) {
+        // rows are (channel, stride phase): each goes to its phase's element of the coarse position
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          if (first + j >= ph.npos) continue;
+          int n, j0, j1, j2;
+          split_pos(first + j, n, j0, j1, j2);
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const int m = m0 + wm0 + Mma<T>::row_of(lane, q) * TM + i;
+              if (m >= p.M) continue;
+              const int c = m / p.phase_count, f = m - c * p.phase_count;
+              if (fused_ok(f, j0, j1, j2)) fused_dst(f, n, j0, j1, j2)[(long long)c * p.dst_mstride] = acc[0][i][j][q];
+            }
+        }
       } else {
         // a sample's positions are adjacent in dst but no whole 16-byte pieces (49, 729, ... of them):
         // the lanes whose TN positions lie in one sample still store them as one vector
@@ -926,6 +970,16 @@ __global__ void __launch_bounds__(256) tail_fixup_kernel(const GemmParams p) {
   const int j2 = (int)r - j1 * ph.J[2];
   const long long slice = (long long)NPH * BM * BN;  // elements of one K slice of a tile: one [BM][BN] per phase
   const T *slot = static_cast<const T *>(p.partial) + (long long)first_slot * slice + e;
+  if (NPH == 1 && p.phase_count != 0) {
+    // row m is stride phase m % phase_count of channel m / phase_count
+    const int c = m / p.phase_count, f = m - c * p.phase_count;
+    if (!((j0 < p.pJ[f][0]) & (j1 < p.pJ[f][1]) & (j2 < p.pJ[f][2]))) return;
+    const T sum = sum_in_order(slot, slice, slots);
+    T *out = static_cast<T *>(p.dst) + (long long)n * p.dst_nstride + (long long)(p.po0[f][0] + j0 * p.oj[0]) * p.os[0] +
+             (long long)(p.po0[f][1] + j1 * p.oj[1]) * p.os[1] + (long long)(p.po0[f][2] + j2 * p.oj[2]) * p.os[2];
+    out[(long long)c * p.dst_mstride] = sum;
+    return;
+  }
 #pragma unroll
   for (int f = 0; f < NPH; ++f) {
     const int o0 = NPH == 1 ? ph.o0[0] : p.po0[f][0], o1 = NPH == 1 ? ph.o0[1] : p.po0[f][1], o2 = NPH == 1 ? ph.o0[2] : p.po0[f][2];
