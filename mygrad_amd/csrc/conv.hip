@@ -1161,6 +1161,13 @@ void set_fold_tile(const Geometry &g, Plan &pl, int rows, int bk) {
 // block runs through, each a round trip to memory, not by the matrix pipes.
 // MYGRAD_HIP_TINY=0 plans such a problem like a large one (read whenever a plan is built, and
 // part of the plan's key: the parity tests run their small cases both ways).
+// MYGRAD_HIP_PHASE_ROWS=0 plans the data gradient of a few channels under a stride phase by phase
+// (read whenever a plan is built, and part of the plan's key: the parity tests run both ways).
+bool phase_rows_enabled() {
+  const char *flag = getenv("MYGRAD_HIP_PHASE_ROWS");
+  return !(flag && flag[0] == '0');
+}
+
 bool tiny_plans_enabled() {
   const char *flag = getenv("MYGRAD_HIP_TINY");
   return !(flag && flag[0] == '0');
@@ -1546,10 +1553,7 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
   // has three live rows per phase; with the rows (phase, channel) over the coarse grid ceil(X / stride)
   // it has phases x channels of them, and every gathered element of grad serves all phases of its
   // coarse position (a zero in the packed filters where a phase has no tap for it).
-  static const bool phase_rows_on = [] {
-    const char *flag = getenv("MYGRAD_HIP_PHASE_ROWS");
-    return !(flag && flag[0] == '0');
-  }();
+  const bool phase_rows_on = phase_rows_enabled();
   if (phase_rows_on && pl.tap_major && !pl.table_rows && nphase >= 2 && nphase <= 4 && (long long)found.size() == nphase &&
       nphase * g.C <= 16 && g.C <= 8 && 2.0 * g.N * g.F * g.gvol * g.C * g.wvol >= 2e8) {
     std::stable_sort(found.begin(), found.end(), [](const PhaseTaps &a, const PhaseTaps &b) {
@@ -1947,6 +1951,7 @@ int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
   key.push_back((char)op);
   key.push_back(tiny_plans_enabled() ? 't' : 'T');
   key.push_back(thin_on() ? 'n' : 'N');
+  key.push_back(phase_rows_enabled() ? 'p' : 'P');
   auto it = plans().find(key);
   if (it == plans().end()) {
     if (plans().size() >= 256) {

@@ -614,6 +614,38 @@ def test_data_gradient_with_up_to_four_channels(abi, dtype, case):
         assert rel_err(other, direct.conv_backward_x(g, x_shape, w, s, p, d)) <= tol
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("x_shape,w_shape,s,p,d", [
+    ((8, 3, 101, 100), (64, 3, 7, 7), (2, 2), (3, 3), (1, 1)),     # too few positions for the kernel above in float32
+    ((6, 4, 75, 81), (32, 4, 5, 5), (2, 2), (2, 2), (1, 1)),       # sixteen rows: four channels x four phases, odd extents
+    ((4, 8, 90, 64), (48, 8, 3, 4), (2, 1), (1, 2), (1, 1)),       # two phases along the first axis only: no paired stores
+    ((3, 2, 30, 41, 44), (16, 2, 3, 3, 3), (1, 2, 2), (1, 1, 1), (1, 1, 1)),
+    ((16, 5, 4000), (32, 5, 9), (2,), (4,), (2,)),                 # dilation 2 under stride 2: one phase has no tap at all
+])
+def test_data_gradient_with_the_stride_phases_as_rows(abi, dtype, x_shape, w_shape, s, p, d):
+    """A few channels under a stride where the one-position-per-lane kernel does not apply (double
+    precision, or too few positions): the rows of the GEMM are (channel, stride phase) over the
+    coarse grid.  MYGRAD_HIP_PHASE_ROWS=0 plans the same problem phase by phase: same bar."""
+    rng = np.random.default_rng(2500 + x_shape[-1])
+    tol = TOL[np.dtype(dtype)]
+    w = (rng.standard_normal(w_shape) / np.sqrt(np.prod(w_shape[1:]))).astype(dtype)
+    grid = direct.conv_forward(np.zeros(x_shape, dtype=dtype), w, s, p, d).shape
+    g = rng.standard_normal(grid).astype(dtype)
+    want = direct.conv_backward_x(g, x_shape, w, s, p, d)
+    got = abi.conv_dgrad(g, x_shape, w, s, p, d)
+    assert rel_err(got, want) <= tol
+    assert np.array_equal(got, abi.conv_dgrad(g, x_shape, w, s, p, d))
+    gi = rng.integers(-2, 3, grid).astype(dtype)
+    wi = (np.arange(np.prod(w_shape)).reshape(w_shape) % 11 - 5).astype(dtype)
+    assert np.array_equal(abi.conv_dgrad(gi, x_shape, wi, s, p, d), direct.conv_backward_x(gi, x_shape, wi, s, p, d).astype(dtype))
+    os.environ["MYGRAD_HIP_PHASE_ROWS"] = "0"
+    try:
+        other = abi.conv_dgrad(g, x_shape, w, s, p, d)
+    finally:
+        del os.environ["MYGRAD_HIP_PHASE_ROWS"]
+    assert rel_err(other, want) <= tol
+
+
 # Up to four filters in single precision (a layer that ends in one map or in the three colours
 # of an image), or a first layer (channels that fill no K tile): the forward pass on the same
 # kernel, one output position per lane.
