@@ -219,6 +219,12 @@ struct WgradParams {
   int x_cstride;
   unsigned grad_bytes, x_bytes;  // sizes of grad and x (each below 2 GiB)
   int col_tiles, row_tiles;  // tiles of the output matrix along columns / filters
+  // One row of four 32-bit words per position (n, g), or null: the byte offset into x of the
+  // position's window origin (without the padding shift, which the column groups' offsets carry),
+  // the taps whose element exists there as a bit mask (64 taps at most, row-major), and what the
+  // position's sample adds to the byte offset of grad[0][f][position]: n * (F - 1) * gvol elements.
+  const void *pos_tab;
+  int wvol;  // taps of the window
 };
 
 }  // namespace mg

@@ -1089,10 +1089,66 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
   constexpr int NB = MYGROUPS * CLOADS;
   AReg ra0[ALOADS], ra1[ALOADS];
   T rb0[NB], rb1[NB];
+  // Position table (WgradParams::pos_tab): what a position contributes to the addresses and which
+  // taps it has, so that a K tile costs a table row instead of three divisions, the products with
+  // the strides and a bounds test per axis.  A row is asked for one round of its register set
+  // ahead and rides along in pe0 / pe1 (and, for the grad tile's own positions, pa0 / pa1).
+  const bool tabled = !TABLE && p.pos_tab != nullptr;
+  typedef unsigned u4 __attribute__((ext_vector_type(4)));
+  const __amdgpu_buffer_rsrc_t pos_buf = buffer_of<T>(p.pos_tab, tabled ? (unsigned)p.kpos * 16u : 0u);
+  unsigned tap_bit[MYGROUPS], col_bytes[MYGROUPS];
+  bool tap_high[MYGROUPS];
+  if constexpr (!TABLE) {
+#pragma unroll
+    for (int i = 0; i < MYGROUPS; ++i) {
+      const int tap = (n0 / 16 + gsel + i * GSPLIT) % p.wvol;
+      tap_bit[i] = grp[i][4] != 0 ? 1u << (tap & 31) : 0u;
+      tap_high[i] = tap >= 32;
+      col_bytes[i] = (unsigned)((grp[i][0] + csel * p.x_cstride) * (int)sizeof(T));
+    }
+  }
+  u4 pe0 = {0, 0, 0, 0}, pe1 = {0, 0, 0, 0};
+  unsigned pa0 = 0, pa1 = 0;
   const unsigned a_step = (unsigned)((WIDE ? APASS : ROWS) * p.gvol) * (unsigned)sizeof(T);
   const int apiece = tid % APIECES, arow = tid / APIECES;  // WIDE: this thread's piece of the grad tile
   const unsigned b_step = (unsigned)(CSPLIT * p.x_cstride) * (unsigned)sizeof(T);
 
+  // the table rows of K tile kt for this thread: of its own position, and (WIDE) of its grad piece
+  auto ask = [&](u4 &pe, unsigned &pa, int kt) {
+    const int ipos = kbeg + kt * BK + kcol;
+    pe = __builtin_amdgcn_raw_buffer_load_b128(pos_buf, (ipos < kend ? ipos : kbeg) * 16, 0, 0);
+    if constexpr (WIDE) {
+      const int apos = kbeg + kt * BK + apiece * VEC;
+      pa = __builtin_amdgcn_raw_buffer_load_b32(pos_buf, (apos < kend ? apos : kbeg) * 16 + 12, 0, 0);
+    }
+  };
+  auto fetch_tabled = [&](AReg(&ra)[ALOADS], T(&rb)[NB], u4 &pe, unsigned &pa, int kt, int kt_next) {
+    // the rows of the set's next tile first: whoever waits for them leaves this tile's loads in flight
+    u4 pe_next;
+    unsigned pa_next;
+    ask(pe_next, pa_next, kt_next);
+    const int ipos = kbeg + kt * BK + kcol;
+    const bool pos_ok = ipos < kend;
+    if constexpr (WIDE) {
+      const int apos = kbeg + kt * BK + apiece * VEC;
+      const unsigned g_at = apos < kend ? (unsigned)(apos + (m0 + arow) * p.gvol) * (unsigned)sizeof(T) + pa : kOutside;
+#pragma unroll
+      for (int r = 0; r < ALOADS; ++r) ra[r] = buffer_load16<T>(grad_buf, g_at, (unsigned)r * a_step);
+    } else {
+      const unsigned g_at = pos_ok ? (unsigned)(ipos + (m0 + row0) * p.gvol) * (unsigned)sizeof(T) + pe[3] : kOutside;
+#pragma unroll
+      for (int r = 0; r < ALOADS; ++r) ra[r] = buffer_load<T>(grad_buf, g_at, (unsigned)r * a_step);
+    }
+#pragma unroll
+    for (int j = 0; j < MYGROUPS; ++j) {
+      const unsigned word = tap_high[j] ? pe[2] : pe[1];
+      const bool ok = pos_ok & ((word & tap_bit[j]) != 0u);
+      const unsigned at = ok ? pe[0] + col_bytes[j] : kOutside;
+#pragma unroll
+      for (int r = 0; r < CLOADS; ++r) rb[j * CLOADS + r] = buffer_load<T>(x_buf, at, (unsigned)r * b_step);
+    }
+    pe = pe_next, pa = pa_next;
+  };
   auto fetch = [&](AReg(&ra)[ALOADS], T(&rb)[NB], int kt) {
     if constexpr (WIDE) {
       const int apos = kbeg + kt * BK + apiece * VEC;  // the piece lies inside one sample and inside the split or not at all
@@ -1162,6 +1218,30 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
     // tile i travels in register set i % 2 and lands in LDS buffer i % 2; the loads
     // of every path are the same (see tap_gemm_kernel), tiles past the end are clamped
     const int last = ktiles - 1;
+    if (tabled) {
+      // the same schedule with the table rows one round ahead: set 0 takes tiles 0, 2, 4, ...,
+      // set 1 tiles 1, 3, 5, ... (each clamped to the last)
+      if (ktiles > 0) {
+        ask(pe0, pa0, 0);
+        ask(pe1, pa1, min(1, last));
+        fetch_tabled(ra0, rb0, pe0, pa0, 0, min(2, last));
+        stash(ra0, rb0, 0);
+        fetch_tabled(ra1, rb1, pe1, pa1, min(1, last), min(3, last));
+        fetch_tabled(ra0, rb0, pe0, pa0, min(2, last), min(4, last));
+      }
+      __syncthreads();
+      int kt = 0;
+      for (; kt + 1 < ktiles; kt += 2) {
+        stash(ra1, rb1, 1);
+        fetch_tabled(ra1, rb1, pe1, pa1, min(kt + 3, last), min(kt + 5, last));
+        __syncthreads();
+        stash(ra0, rb0, 0);
+        fetch_tabled(ra0, rb0, pe0, pa0, min(kt + 4, last), min(kt + 6, last));
+        __syncthreads();
+      }
+      if (kt < ktiles) __syncthreads();
+      return;
+    }
     if (ktiles > 0) {
       fetch(ra0, rb0, 0);
       stash(ra0, rb0, 0);

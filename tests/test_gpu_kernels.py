@@ -646,6 +646,41 @@ def test_data_gradient_with_the_stride_phases_as_rows(abi, dtype, x_shape, w_sha
     assert rel_err(other, want) <= tol
 
 
+# The filter gradient's K index is the position: the single-precision tap-major kernel reads, per
+# position, a row of a table (window origin in x, which taps exist, what the sample adds to the
+# offset into grad) instead of dividing the position into coordinates for every K tile.
+POS_TABLE_CASES = [
+    ((6, 16, 23, 23), (32, 16, 3, 3), (1, 1), (1, 1), (1, 1)),         # rows of grad that are no whole 16-byte pieces
+    ((4, 32, 20, 24), (16, 32, 3, 3), (2, 2), (1, 1), (1, 1)),         # stride: taps missing on one side only
+    ((3, 16, 31, 36), (64, 16, 7, 7), (2, 1), (3, 3), (1, 1)),         # 49 taps: both words of the tap mask
+    ((2, 16, 9, 20, 20), (32, 16, 3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),  # 27 taps, padding on three axes
+    ((5, 48, 40, 40), (128, 48, 5, 5), (1, 1), (4, 4), (2, 2)),        # dilation; wide tiles, several column groups per thread
+    ((2, 16, 12, 12), (16, 16, 3, 3), (1, 1), (2, 2), (1, 1)),         # padding wider than a tap step; one short K tile per split
+]
+
+
+@pytest.mark.parametrize("x_shape,w_shape,s,p,d", POS_TABLE_CASES)
+def test_filter_gradient_with_and_without_the_position_table(abi, monkeypatch, x_shape, w_shape, s, p, d):
+    monkeypatch.setenv("MYGRAD_HIP_TINY", "0")  # small shapes: planned like large ones, or they take the table-driven kernel
+    rng = np.random.default_rng(2600 + x_shape[-1])
+    x = rng.standard_normal(x_shape).astype(np.float32)
+    grid = direct.conv_forward(x, np.zeros(w_shape, dtype=np.float32), s, p, d).shape
+    g = rng.standard_normal(grid).astype(np.float32)
+    want = direct.conv_backward_w(g, x, w_shape, s, p, d)
+    got = abi.conv_wgrad(g, x, w_shape, s, p, d)
+    from mygrad_amd import _hip
+
+    assert "tap-major" in _hip.last_plan()
+    assert rel_err(got, want) <= TOL[np.dtype(np.float32)]
+    # small integers: every sum is exact, so the result is the definition's bit for bit
+    xi = rng.integers(-3, 4, x_shape).astype(np.float32)
+    gi = rng.integers(-2, 3, grid).astype(np.float32)
+    assert np.array_equal(abi.conv_wgrad(gi, xi, w_shape, s, p, d), direct.conv_backward_w(gi, xi, w_shape, s, p, d).astype(np.float32))
+    # the same kernel on its own position arithmetic adds the same terms in the same order
+    monkeypatch.setenv("MYGRAD_HIP_POS_TABLE", "0")
+    assert np.array_equal(bits(got), bits(abi.conv_wgrad(g, x, w_shape, s, p, d)))
+
+
 # Up to four filters in single precision (a layer that ends in one map or in the three colours
 # of an image), or a first layer (channels that fill no K tile): the forward pass on the same
 # kernel, one output position per lane.
