@@ -1819,9 +1819,10 @@ int wgrad_blocks_per_cu(int bm, int bn, bool tap_major) {
 }
 
 // The position table of the tap-major filter-gradient kernel: row idx describes position
-// (n, g0, g1, g2) = idx in row-major order (see WgradParams::pos_tab).  `groups` starts with the
-// groups of the first channel block, one per tap, whose coordinate offsets are the taps'.
-__global__ void __launch_bounds__(256) wgrad_pos_table_kernel(unsigned *__restrict__ tab, const WGroup *__restrict__ groups, int wvol, int kpos,
+// (n, g0, g1, g2) = idx in row-major order (see WgradParams::pos_tab).  The coordinate offsets
+// (d0, d1, d2) of tap t lie at taps[t * tap_ints ...]: in the column groups of the first channel
+// block, one per tap, or in the first channel's rows of the gather table.
+__global__ void __launch_bounds__(256) wgrad_pos_table_kernel(unsigned *__restrict__ tab, const int *__restrict__ taps, int tap_ints, int wvol, int kpos,
                                                               int gvol, int g12, int g2n, int sj0, int sj1, int sj2, int qs0, int qs1, int qs2,
                                                               int q0, int q1, int q2, long long x_nstride, long long grad_extra,
                                                               int elem) {
@@ -1836,8 +1837,8 @@ __global__ void __launch_bounds__(256) wgrad_pos_table_kernel(unsigned *__restri
   const int qb0 = g0 * sj0, qb1 = g1 * sj1, qb2 = g2 * sj2;
   unsigned lo = 0, hi = 0;
   for (int t = 0; t < wvol; ++t) {
-    const WGroup e = groups[t];
-    const bool ok = ((unsigned)(qb0 + e.d0) < (unsigned)q0) & ((unsigned)(qb1 + e.d1) < (unsigned)q1) & ((unsigned)(qb2 + e.d2) < (unsigned)q2);
+    const int *d = taps + (long long)t * tap_ints;
+    const bool ok = ((unsigned)(qb0 + d[0]) < (unsigned)q0) & ((unsigned)(qb1 + d[1]) < (unsigned)q1) & ((unsigned)(qb2 + d[2]) < (unsigned)q2);
     if (ok) (t < 32 ? lo : hi) |= 1u << (t & 31);
   }
   uint4 row;
@@ -1850,7 +1851,8 @@ __global__ void __launch_bounds__(256) wgrad_pos_table_kernel(unsigned *__restri
 
 // MYGRAD_HIP_POS_TABLE=0 keeps the filter-gradient kernel on its in-kernel position arithmetic.
 // Single precision only: measured with the table, config 5 271 -> 263 us, config 3b 129.5 -> 123.6 us,
-// a 4096^3 product's da 1015 -> 973 us, config 3a unchanged; double precision (config 4) 1 % slower.
+// a 4096^3 product's da 1015 -> 973 us, config 3a unchanged, a 7x7 stride-2 first layer on table rows
+// 372 -> 344 us; double precision 1 % (config 4) to 7 % (the same first layer) slower.
 inline bool pos_table_enabled() {
   const char *flag = getenv("MYGRAD_HIP_POS_TABLE");
   return !(flag && flag[0] == '0');
@@ -1858,10 +1860,13 @@ inline bool pos_table_enabled() {
 
 int build_pos_table(const Geometry &g, Plan &pl) {
   const long long kpos = (long long)g.N * g.gvol;
-  if (!pl.tap_major || pl.table_rows || g.dtype != MG_F32 || g.wvol > 64 || kpos * 16 > (32ll << 20) || !pos_table_enabled()) return MG_OK;
+  if (!pl.tap_major || g.dtype != MG_F32 || g.wvol > 64 || kpos * 16 > (32ll << 20) || !pos_table_enabled()) return MG_OK;
   MG_HIP(hipMalloc(&pl.pos_tab, (size_t)kpos * 16));
+  // both kinds of row start with an element offset, followed by the three coordinate offsets
+  const int *taps = pl.table_rows ? reinterpret_cast<const int *>(pl.tab) + 1 : reinterpret_cast<const int *>(pl.groups) + 1;
+  const int tap_ints = (int)((pl.table_rows ? sizeof(TabEntry) : sizeof(WGroup)) / sizeof(int));
   hipLaunchKernelGGL(wgrad_pos_table_kernel, dim3((unsigned)ceil_div(kpos, 256)), dim3(256), 0, runtime().stream,
-                     static_cast<unsigned *>(pl.pos_tab), pl.groups, (int)g.wvol, (int)kpos, (int)g.gvol, g.G[1] * g.G[2], g.G[2], g.S[0], g.S[1],
+                     static_cast<unsigned *>(pl.pos_tab), taps, tap_ints, (int)g.wvol, (int)kpos, (int)g.gvol, g.G[1] * g.G[2], g.G[2], g.S[0], g.S[1],
                      g.S[2], g.X[1] * g.X[2], g.X[2], 1, g.X[0], g.X[1], g.X[2], (long long)g.C * g.xvol, (long long)(g.F - 1) * g.gvol,
                      g.dtype == MG_F64 ? 8 : 4);
   MG_HIP(hipGetLastError());
@@ -2427,10 +2432,17 @@ void launch_table_wgrad(WgradParams &wp, hipStream_t s) {
   wp.col_tiles = (int)ceil_div(wp.CT, BN);
   wp.row_tiles = (int)ceil_div(wp.F, BM);
   const long long blocks = (long long)wp.splits * wp.col_tiles * wp.row_tiles;
-  if (wp.gvol % (int)(16 / sizeof(T)) == 0)
+  const bool wide = wp.gvol % (int)(16 / sizeof(T)) == 0;
+  if (wp.pos_tab != nullptr) {
+    if (wide)
+      hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN, true, true, true>), dim3((unsigned)blocks), dim3(512), 0, s, wp);
+    else
+      hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN, false, true, true>), dim3((unsigned)blocks), dim3(512), 0, s, wp);
+  } else if (wide) {
     hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN, true, true>), dim3((unsigned)blocks), dim3(512), 0, s, wp);
-  else
+  } else {
     hipLaunchKernelGGL((tap_wgrad_kernel<T, BM, BN, BK, WM, WN, false, true>), dim3((unsigned)blocks), dim3(512), 0, s, wp);
+  }
 }
 
 template <typename T, int BM, int BN, int BK, int WM, int WN>

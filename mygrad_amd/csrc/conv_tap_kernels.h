@@ -1001,8 +1001,12 @@ __global__ void __launch_bounds__(256) tail_fixup_kernel(const GemmParams p) {
 // in dw's own order, padded to whole tiles with rows that lie outside every input), not groups
 // of 16 channels under one tap -- for channel counts that fill no group.  Every column then
 // costs the gathering waves its own bounds test.
-template <typename T, int BM, int BN, int BK, int WM, int WN, bool WIDE, bool TABLE = false>
+// POS (TABLE only): the columns' bounds tests come from the position table (WgradParams::pos_tab,
+// which must be there) instead of the gather table's coordinate offsets; the other kernels take
+// the position table whenever the plan has one.
+template <typename T, int BM, int BN, int BK, int WM, int WN, bool WIDE, bool TABLE = false, bool POS = false>
 __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
+  static_assert(TABLE || !POS, "POS selects between the two forms of the TABLE kernel");
   static_assert((BM / WM) * (BN / WN) == 4, "four wavefronts per block");
   static_assert(256 % BK == 0 && BK % 16 == 0 && BN % 16 == 0, "K tile");
   constexpr int TM = WM / 16, TN = WN / 16;
@@ -1077,23 +1081,34 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
     for (int i = 0; i < MYGROUPS; ++i) grp[i] = gtab[gsel + i * GSPLIT];
   }
   // TABLE: this thread's columns (gsel + j*GSPLIT)*16 + csel + r*CSPLIT of the tile, one table row each
-  int4v ent[TABLE ? MYGROUPS * CLOADS : 1];
+  constexpr int NB = MYGROUPS * CLOADS;
+  int4v ent[TABLE && !POS ? NB : 1];
+  // POS: a column is its element offset into x and its tap (a column past the last one: an offset
+  // outside x)
+  unsigned col_off[TABLE && POS ? NB : 1], col_tap[TABLE && POS ? NB : 1];
   if constexpr (TABLE) {
     const int4v MG_CONSTANT *rows = (const int4v MG_CONSTANT *)(p.tab) + n0;
 #pragma unroll
     for (int j = 0; j < MYGROUPS; ++j)
 #pragma unroll
-      for (int r = 0; r < CLOADS; ++r) ent[j * CLOADS + r] = rows[(gsel + j * GSPLIT) * 16 + csel + r * CSPLIT];
+      for (int r = 0; r < CLOADS; ++r) {
+        const int col = (gsel + j * GSPLIT) * 16 + csel + r * CSPLIT;
+        if constexpr (POS) {
+          col_off[j * CLOADS + r] = n0 + col < p.CT ? (unsigned)(rows[col][0] * (int)sizeof(T)) : kOutside;
+          col_tap[j * CLOADS + r] = (unsigned)((n0 + col) % p.wvol);
+        } else {
+          ent[j * CLOADS + r] = rows[col];
+        }
+      }
   }
 
-  constexpr int NB = MYGROUPS * CLOADS;
   AReg ra0[ALOADS], ra1[ALOADS];
   T rb0[NB], rb1[NB];
   // Position table (WgradParams::pos_tab): what a position contributes to the addresses and which
   // taps it has, so that a K tile costs a table row instead of three divisions, the products with
   // the strides and a bounds test per axis.  A row is asked for one round of its register set
   // ahead and rides along in pe0 / pe1 (and, for the grad tile's own positions, pa0 / pa1).
-  const bool tabled = !TABLE && p.pos_tab != nullptr;
+  const bool tabled = TABLE ? POS : p.pos_tab != nullptr;
   typedef unsigned u4 __attribute__((ext_vector_type(4)));
   const __amdgpu_buffer_rsrc_t pos_buf = buffer_of<T>(p.pos_tab, tabled ? (unsigned)p.kpos * 16u : 0u);
   unsigned tap_bit[MYGROUPS], col_bytes[MYGROUPS];
@@ -1139,13 +1154,22 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
 #pragma unroll
       for (int r = 0; r < ALOADS; ++r) ra[r] = buffer_load<T>(grad_buf, g_at, (unsigned)r * a_step);
     }
+    if constexpr (TABLE && POS) {
+      const unsigned long long taps = ((unsigned long long)pe[2] << 32) | pe[1];
 #pragma unroll
-    for (int j = 0; j < MYGROUPS; ++j) {
-      const unsigned word = tap_high[j] ? pe[2] : pe[1];
-      const bool ok = pos_ok & ((word & tap_bit[j]) != 0u);
-      const unsigned at = ok ? pe[0] + col_bytes[j] : kOutside;
+      for (int i = 0; i < NB; ++i) {
+        const bool ok = pos_ok & (((taps >> col_tap[i]) & 1ull) != 0ull);
+        rb[i] = buffer_load<T>(x_buf, ok ? pe[0] + col_off[i] : kOutside, 0u);
+      }
+    } else if constexpr (!TABLE) {
 #pragma unroll
-      for (int r = 0; r < CLOADS; ++r) rb[j * CLOADS + r] = buffer_load<T>(x_buf, at, (unsigned)r * b_step);
+      for (int j = 0; j < MYGROUPS; ++j) {
+        const unsigned word = tap_high[j] ? pe[2] : pe[1];
+        const bool ok = pos_ok & ((word & tap_bit[j]) != 0u);
+        const unsigned at = ok ? pe[0] + col_bytes[j] : kOutside;
+#pragma unroll
+        for (int r = 0; r < CLOADS; ++r) rb[j * CLOADS + r] = buffer_load<T>(x_buf, at, (unsigned)r * b_step);
+      }
     }
     pe = pe_next, pa = pa_next;
   };
@@ -1179,7 +1203,7 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
     }
     const unsigned x_at = (unsigned)((long long)n * p.x_nstride + (qb0 * p.qs[0] + qb1 * p.qs[1] + qb2 * p.qs[2]) +
                                      (TABLE ? 0ll : (long long)csel * p.x_cstride)) * (unsigned)sizeof(T);
-    if constexpr (TABLE) {
+    if constexpr (TABLE && !POS) {
 #pragma unroll
       for (int i = 0; i < NB; ++i) {
         const int4v e = ent[i];  // off, d0, d1, d2
@@ -1187,7 +1211,7 @@ __global__ void __launch_bounds__(512) tap_wgrad_kernel(const WgradParams p) {
                         ((unsigned)(qb2 + e[3]) < (unsigned)p.Q[2]);
         rb[i] = buffer_load<T>(x_buf, ok ? x_at + (unsigned)(e[0] * (int)sizeof(T)) : kOutside, 0u);
       }
-    } else {
+    } else if constexpr (!TABLE) {
 #pragma unroll
       for (int j = 0; j < MYGROUPS; ++j) {
         const int8v e = grp[j];  // coff, d0, d1, d2, valid

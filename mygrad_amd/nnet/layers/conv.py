@@ -33,6 +33,11 @@ def _kernel_dtype(*arrays):
     dtype = np.dtype(np.result_type(*(a.dtype for a in arrays)))
     if dtype == np.float16:
         return np.dtype(np.float32), dtype
+    if dtype.kind in "iu":
+        # Integer operands (constants: the reference multiplies them with np.tensordot in integer
+        # arithmetic, conv.py:96-99).  float64 holds every integer below 2**53, so while no sum of
+        # products can reach that, the float64 kernels give the integer result exactly.
+        return np.dtype(np.float64), dtype
     if dtype not in (np.float32, np.float64):
         raise TypeError(
             f"conv_nd runs on the GPU in float32 or float64 (float16 operands are widened to float32); "
@@ -103,6 +108,14 @@ class ConvND(Operation):
         if np.iscomplexobj(xd) or np.iscomplexobj(wd):
             return self._complex_forward(xd, wd)
         dtype, result_dtype = _kernel_dtype(xd, wd)
+        if result_dtype.kind in "iu" and xd.size and wd.size:
+            xd, wd = np.asarray(xd), np.asarray(wd)
+            largest = [max(abs(int(a.max())), abs(int(a.min()))) for a in (xd, wd)]
+            if largest[0] * largest[1] * int(np.prod(wd.shape[1:])) >= 2**53:
+                raise TypeError(
+                    f"conv_nd of integer operands runs in float64 on the GPU, which is exact while no sum can reach 2**53; "
+                    f"values up to {largest[0]} and {largest[1]} over {int(np.prod(wd.shape[1:]))} terms may (there is no CPU fallback)"
+                )
         grid = tuple(int(g) for g in out_shape)
         out_full = (xd.shape[0], wd.shape[0], *grid)
         self._dtype = dtype

@@ -139,6 +139,15 @@ class MaxPoolND(Operation):
         while m - skip > 1 and pool[skip] == 1 and stride[skip] == 1:
             skip += 1
         self._skip = skip
+        result_dtype = xd.dtype
+        if xd.dtype.kind in "iu":
+            # Integers (constants: no gradient is ever asked for) are pooled as float64, which holds
+            # every integer below 2**53; a maximum is one of the inputs, so the way back is exact.
+            xd = np.asarray(xd)
+            if xd.size and max(abs(int(xd.max())), abs(int(xd.min()))) >= 2**53:
+                raise TypeError("max_pool of integers runs in float64 on the GPU, which holds integers below 2**53 only "
+                                "(there is no CPU fallback)")
+            xd = xd.astype(np.float64)
         if xd.dtype not in (np.float32, np.float64, np.float16):
             raise TypeError(
                 f"max_pool runs on the GPU in float32 or float64 (float16 values are widened to float32), got {xd.dtype} "
@@ -146,7 +155,6 @@ class MaxPoolND(Operation):
             )
         # float16 is a storage type here: the values are widened to float32 (exactly), the kernels
         # pick the same maxima, and the result is narrowed again (exactly: it consists of inputs)
-        result_dtype = xd.dtype
         if xd.dtype == np.float16:
             xd = xd.astype(np.float32)  # on the device for a value that lives there, else on the host
         grid = tuple(int(g) for g in out_shape)

@@ -242,6 +242,24 @@ def test_operand_variety():
     assert _graph.held_count() == 0
 
 
+def test_integer_operands_give_the_integer_result():
+    """All-integer operands are constants; the reference multiplies them in integer arithmetic
+    (np.tensordot, conv.py:96-99) and takes maxima of integers (pooling.py:93).  Here they run in
+    float64, exactly, and come back in NumPy's result type."""
+    rng = np.random.default_rng(14)
+    xi = rng.integers(-1000, 1000, (3, 4, 11, 12))
+    wi = rng.integers(-50, 50, (5, 4, 3, 2)).astype(np.int32)
+    out = conv_nd(xi, wi, stride=(2, 1), padding=(1, 0), dilation=(1, 2))
+    want = ora.conv_forward(xi, wi, stride=(2, 1), padding=(1, 0), dilation=(1, 2))
+    assert out.dtype == want.dtype == np.int64 and out.constant and np.array_equal(out.data, want)
+    pooled = max_pool(mg.Tensor(xi.astype(np.int16)), (3, 2), (2, 2))
+    assert pooled.dtype == np.int16 and np.array_equal(pooled.data, ora.pool_forward(xi.astype(np.int16), (3, 2), (2, 2)))
+    big = np.array([[2**53 - 1, -(2**53) + 1, 0, 5]])
+    assert np.array_equal(max_pool(big, (2,), 2).data, [[2**53 - 1, 5]])
+    del out, pooled  # the results hold their operands read-only for as long as they live
+    assert _graph.held_count() == 0
+
+
 def test_tensor_feeding_two_pools_accumulates_like_the_reference():
     # second contribution is added to an existing float32 gradient: the reference adds
     # the unrounded float64 dx (pooling.py:147, operation_base.py:227-228)

@@ -656,6 +656,10 @@ POS_TABLE_CASES = [
     ((2, 16, 9, 20, 20), (32, 16, 3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),  # 27 taps, padding on three axes
     ((5, 48, 40, 40), (128, 48, 5, 5), (1, 1), (4, 4), (2, 2)),        # dilation; wide tiles, several column groups per thread
     ((2, 16, 12, 12), (16, 16, 3, 3), (1, 1), (2, 2), (1, 1)),         # padding wider than a tap step; one short K tile per split
+    # channels that fill no group of 16 columns: one table row per column, its tap looked up in the position's mask
+    ((8, 3, 45, 45), (64, 3, 7, 7), (2, 2), (3, 3), (1, 1)),           # 147 columns in two tiles of 80
+    ((6, 5, 22, 26), (24, 5, 3, 3), (1, 1), (1, 1), (1, 1)),           # a short last row tile; rows of grad that are no whole pieces
+    ((4, 20, 15, 15), (10, 20, 5, 5), (1, 1), (0, 0), (1, 1)),         # no padding: every tap exists everywhere
 ]
 
 

@@ -149,7 +149,12 @@ def test_unsupported_inputs_are_rejected_not_computed_on_the_cpu():
     with pytest.raises(TypeError):
         conv_nd(np.zeros((1, 1, 4), np.complex64), np.zeros((1, 1, 2), np.complex64), stride=1)
     with pytest.raises(TypeError):
-        max_pool(np.zeros((1, 4), np.int64), (2,), 2)
+        max_pool(np.zeros((1, 4), bool), (2,), 2)
+    # integers run as float64, which is exact below 2**53 only
+    with pytest.raises(TypeError):
+        max_pool(np.full((1, 4), 2**60), (2,), 2)
+    with pytest.raises(TypeError):
+        conv_nd(np.full((1, 1, 4), 2**30), np.full((1, 1, 2), 2**30), stride=1)
     with pytest.raises(NotImplementedError):
         max_pool(np.zeros((4, 4)), (), ())  # nothing to pool over
 
