@@ -1861,7 +1861,12 @@ inline bool pos_table_enabled() {
 int build_pos_table(const Geometry &g, Plan &pl) {
   const long long kpos = (long long)g.N * g.gvol;
   if (!pl.tap_major || g.dtype != MG_F32 || g.wvol > 64 || kpos * 16 > (32ll << 20) || !pos_table_enabled()) return MG_OK;
-  MG_HIP(hipMalloc(&pl.pos_tab, (size_t)kpos * 16));
+  if (hipMalloc(&pl.pos_tab, (size_t)kpos * 16) != hipSuccess) {
+    // no room for the table: the kernels do the arithmetic themselves
+    (void)hipGetLastError();
+    pl.pos_tab = nullptr;
+    return MG_OK;
+  }
   // both kinds of row start with an element offset, followed by the three coordinate offsets
   const int *taps = pl.table_rows ? reinterpret_cast<const int *>(pl.tab) + 1 : reinterpret_cast<const int *>(pl.groups) + 1;
   const int tap_ints = (int)((pl.table_rows ? sizeof(TabEntry) : sizeof(WGroup)) / sizeof(int));
