@@ -809,7 +809,9 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
     return !(flag && flag[0] == '0');
   }();
   bool forced_fits = false;
-  for (int ci = 0; ci < ncfgs; ++ci) forced_fits |= cfgs[ci].bm == forced.bm && cfgs[ci].bn == forced.bn && (!cfgs[ci].tap_only || tap_major);
+  for (int ci = 0; ci < ncfgs; ++ci)
+    forced_fits |= cfgs[ci].bm == forced.bm && cfgs[ci].bn == forced.bn && (!cfgs[ci].tap_only || tap_major) &&
+                   !(tap_major && elem == 8 && cfgs[ci].bn * cfgs[ci].bm >= 128 * 128);  // (no such double-precision tile)
   const int bm = forced_fits ? forced.bm : nph == 4 ? std::min(pick_bm(M), 64) : pick_bm(M);
   const int cus = runtime().props.multiProcessorCount;
   TileChoice best{};
