@@ -794,11 +794,12 @@ TileChoice choose_tile(int M, const std::vector<long long> &phase_npos, int min_
   static const Cfg fused4[] = {{64, 64, 1.10, true}, {32, 128, 1.10, true}, {16, 256, 1.00, true}};
   const Cfg *cfgs = nph == 4 ? fused4 : nph == 2 ? fused2 : plain;
   const int ncfgs = nph == 4 ? 3 : nph == 2 ? 4 : 7;
-  // MYGRAD_HIP_TILE="rows,positions[,blocks per unit]" (diagnostics; read once): only that tile shape
+  // MYGRAD_HIP_TILE="rows,positions[,blocks per unit]" (diagnostics and the tests of every tile shape;
+  // read whenever a plan is built, and part of the plan's key): only that tile shape, where it exists
   struct Forced {
     int bm = 0, bn = 0, r = 0;
   };
-  static const Forced forced = [] {
+  const Forced forced = [] {
     Forced f;
     if (const char *v = getenv("MYGRAD_HIP_TILE")) sscanf(v, "%d,%d,%d", &f.bm, &f.bn, &f.r);
     return f;
@@ -2017,6 +2018,7 @@ int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
   key.push_back(thin_on() ? 'n' : 'N');
   key.push_back(phase_rows_enabled() ? 'p' : 'P');
   key.push_back(pos_table_enabled() ? 'q' : 'Q');
+  if (const char *tile = getenv("MYGRAD_HIP_TILE")) key.append(tile);
   auto it = plans().find(key);
   if (it == plans().end()) {
     if (plans().size() >= 256) {

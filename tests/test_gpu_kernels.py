@@ -646,6 +646,48 @@ def test_data_gradient_with_the_stride_phases_as_rows(abi, dtype, x_shape, w_sha
     assert rel_err(other, want) <= tol
 
 
+# Every tile shape of the forward / data-gradient kernels, forced in turn (the planner would take
+# one or two of them for any given problem): rows x positions, and for the data gradient under a
+# stride the shapes of its fused stride phases.
+ALL_TILES = ["128,128", "128,64", "64,256", "64,128", "32,256", "32,128", "16,256", "64,64"]
+TILE_PROBLEMS = [
+    # (x, w, stride, padding, dilation): odd extents, so that row ends and sample ends fall inside tiles
+    ((3, 32, 29, 27), (160, 32, 3, 3), (1, 1), (1, 1), (1, 1)),       # 160 rows: one and a quarter tiles of 128
+    ((2, 48, 31, 33), (48, 48, 3, 3), (2, 2), (1, 1), (1, 1)),        # stride 2 both ways: four fused phases
+    ((2, 32, 20, 45), (64, 32, 3, 5), (1, 2), (1, 2), (1, 1)),        # stride 2 along the last axis only: two fused phases
+    ((2, 16, 9, 17, 19), (32, 16, 3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1)),  # three axes; folded taps where the tile allows
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("tile", ALL_TILES)
+@pytest.mark.parametrize("problem", range(len(TILE_PROBLEMS)))
+def test_every_tile_shape_of_the_gather_gemm(abi, monkeypatch, problem, tile, dtype):
+    from mygrad_amd import _hip
+
+    monkeypatch.setenv("MYGRAD_HIP_TINY", "0")
+    monkeypatch.setenv("MYGRAD_HIP_TILE", tile)
+    x_shape, w_shape, s, p, d = TILE_PROBLEMS[problem]
+    rng = np.random.default_rng(2700 + problem)
+    tol = TOL[np.dtype(dtype)]
+    x = rng.standard_normal(x_shape).astype(dtype)
+    w = (rng.standard_normal(w_shape) / np.sqrt(np.prod(w_shape[1:]))).astype(dtype)
+    want = direct.conv_forward(x, w, s, p, d)
+    got = abi.conv_fwd(x, w, s, p, d)
+    print("forward:", _hip.last_plan(), flush=True)
+    assert rel_err(got, want) <= tol
+    g = rng.standard_normal(want.shape).astype(dtype)
+    dx = abi.conv_dgrad(g, x_shape, w, s, p, d)
+    print("data gradient:", _hip.last_plan(), flush=True)
+    assert rel_err(dx, direct.conv_backward_x(g, x_shape, w, s, p, d)) <= tol
+    # small integers: every sum is exact whatever the tile and however its K tiles are shared out
+    xi = rng.integers(-3, 4, x_shape).astype(dtype)
+    wi = rng.integers(-2, 3, w_shape).astype(dtype)
+    gi = rng.integers(-2, 3, want.shape).astype(dtype)
+    assert np.array_equal(abi.conv_fwd(xi, wi, s, p, d), direct.conv_forward(xi, wi, s, p, d).astype(dtype))
+    assert np.array_equal(abi.conv_dgrad(gi, x_shape, wi, s, p, d), direct.conv_backward_x(gi, x_shape, wi, s, p, d).astype(dtype))
+
+
 # The filter gradient's K index is the position: the single-precision tap-major kernel reads, per
 # position, a row of a table (window origin in x, which taps exist, what the sample adds to the
 # offset into grad) instead of dividing the position into coordinates for every K tile.
