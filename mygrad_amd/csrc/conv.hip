@@ -1925,8 +1925,16 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
                         {32, 128, f64 ? 16 : 32},  {32, 64, f64 ? 32 : 64},   {16, 64, f64 ? 32 : 64}};
   long long best_splits = 1;
   pl.bm = 0;
+  // MYGRAD_HIP_WGRAD_TILE="rows,columns" (diagnostics and the tests of every tile shape; part of the
+  // plan's key): that candidate or, where it does not apply, the usual choice
+  int forced_bm = 0, forced_bn = 0;
+  if (const char *v = getenv("MYGRAD_HIP_WGRAD_TILE")) sscanf(v, "%d,%d", &forced_bm, &forced_bn);
+  bool forced = false;
+  for (const Cand &c : cands)
+    forced |= c.bm == forced_bm && c.bn == forced_bn && g.F % c.bm == 0 && !(f64 && c.bn == 192) && !(c.bm == 32 && c.bn == 128 && !f64);
   if (g.C % 16 == 0 && fits_buffer_loads(g)) {
     for (const Cand &c : cands) {
+      if (forced && (c.bm != forced_bm || c.bn != forced_bn)) continue;
       if (g.F % c.bm != 0) continue;
       if (f64 && c.bn == 192) continue;  // its accumulators leave room for one block per compute unit only
       // 32x64 double-precision tiles are bound by LDS reads (the 4x4x4 MFMA takes an operand
@@ -1935,7 +1943,7 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
       if (c.bm == 32 && c.bn == 128 && !f64) continue;
       const long long col_tiles = ceil_div(ct, c.bn), row_tiles = g.F / c.bm;
       const long long splits = splits_for(c.bm, c.bn, c.bk, true);
-      if (c.bn > 64) {
+      if (c.bn > 64 && !forced) {
         const int per_cu = f64 ? wgrad_blocks_per_cu<double>(c.bm, c.bn, true) : wgrad_blocks_per_cu<float>(c.bm, c.bn, true);
         const double waste = (double)(col_tiles * c.bn - ct) / (double)ct;
         const double filled = (double)(col_tiles * row_tiles * splits) / ((double)per_cu * cus);
@@ -2019,6 +2027,7 @@ int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
   key.push_back(phase_rows_enabled() ? 'p' : 'P');
   key.push_back(pos_table_enabled() ? 'q' : 'Q');
   if (const char *tile = getenv("MYGRAD_HIP_TILE")) key.append(tile);
+  if (const char *tile = getenv("MYGRAD_HIP_WGRAD_TILE")) key.append("w").append(tile);
   auto it = plans().find(key);
   if (it == plans().end()) {
     if (plans().size() >= 256) {

@@ -688,6 +688,32 @@ def test_every_tile_shape_of_the_gather_gemm(abi, monkeypatch, problem, tile, dt
     assert np.array_equal(abi.conv_dgrad(gi, x_shape, wi, s, p, d), direct.conv_backward_x(gi, x_shape, wi, s, p, d).astype(dtype))
 
 
+WGRAD_TILES = ["128,128", "64,192", "64,128", "64,64", "32,128", "32,64", "16,64"]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("tile", WGRAD_TILES)
+@pytest.mark.parametrize("x_shape,w_shape,s,p,d", [
+    ((3, 32, 29, 27), (128, 32, 3, 3), (1, 1), (1, 1), (1, 1)),   # 288 columns: tiles of 192 and 128 overhang
+    ((2, 48, 31, 33), (64, 48, 3, 3), (2, 2), (1, 1), (1, 1)),    # rows of grad that are no whole 16-byte pieces
+])
+def test_every_tile_shape_of_the_filter_gradient(abi, monkeypatch, x_shape, w_shape, s, p, d, tile, dtype):
+    from mygrad_amd import _hip
+
+    monkeypatch.setenv("MYGRAD_HIP_TINY", "0")
+    monkeypatch.setenv("MYGRAD_HIP_WGRAD_TILE", tile)
+    rng = np.random.default_rng(2800 + x_shape[-1])
+    x = rng.standard_normal(x_shape).astype(dtype)
+    grid = direct.conv_forward(x, np.zeros(w_shape, dtype=dtype), s, p, d).shape
+    g = rng.standard_normal(grid).astype(dtype)
+    got = abi.conv_wgrad(g, x, w_shape, s, p, d)
+    print("filter gradient:", _hip.last_plan(), flush=True)
+    assert rel_err(got, direct.conv_backward_w(g, x, w_shape, s, p, d)) <= TOL[np.dtype(dtype)]
+    xi = rng.integers(-3, 4, x_shape).astype(dtype)
+    gi = rng.integers(-2, 3, grid).astype(dtype)
+    assert np.array_equal(abi.conv_wgrad(gi, xi, w_shape, s, p, d), direct.conv_backward_w(gi, xi, w_shape, s, p, d).astype(dtype))
+
+
 # The filter gradient's K index is the position: the single-precision tap-major kernel reads, per
 # position, a row of a table (window origin in x, which taps exist, what the sample adds to the
 # offset into grad) instead of dividing the position into coordinates for every K tile.
