@@ -684,12 +684,17 @@ def run_sweep(names, steps=20, prewarm=0.25):
             # operands in the 256 MB last-level cache when they fit there, a pair that alternates
             # (x, out, grad and dx together) mostly does not.
             reps = max(steps, 50)
-            _hip.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(reps):
-                step()
-            _hip.synchronize()
-            pair_ms = (time.perf_counter() - t0) / reps * 1e3
+            while True:
+                _hip.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(reps):
+                    step()
+                _hip.synchronize()
+                elapsed = time.perf_counter() - t0
+                if elapsed >= 0.03 or reps >= 4000:
+                    break
+                reps *= 4
+            pair_ms = elapsed / reps * 1e3
             work = sum(work_of.values())
             rows.append({"shape": name, "dtype": wl["dtype"], "kind": "pool-pair", "pass": "pair", "plan": "", "launches": 0.0,
                          "host_us": pair_ms * 1e3, "kernel_us": None, "work": work, "unit": step.unit,

@@ -1625,8 +1625,19 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
     const char *flag = getenv("MYGRAD_HIP_FUSE");
     return !(flag && flag[0] == '0');
   }();
+  // Four phases of short rows are left apart: what the fusion buys is whole lines of dx, and a row of
+  // 13 elements is no whole line either way, while the fused tiles (64 x 64, four sets of
+  // accumulators) are the slower ones.  Measured on twelve 3x3 stride-2 layers, fused against
+  // apart: rows of 55 elements 0.67, of 27 elements 0.74 - 1.02 (0.83 on configuration 3b), of 13
+  // elements 1.00 - 1.16, of 7 elements 1.19.
+  // (MYGRAD_HIP_FUSE_MIN_ROW sets the shortest row that is still fused; read whenever a plan is
+  // built and part of the plan's key, for the tests of the fused kernels on small problems)
+  const int fuse_min_row = [] {
+    const char *v = getenv("MYGRAD_HIP_FUSE_MIN_ROW");
+    return v ? atoi(v) : 20;
+  }();
   const bool fused = fuse_on && pl.tap_major && !pl.table_rows && g.dtype == MG_F32 && g.S[2] == 2 && g.S[0] <= 2 && g.S[1] <= 2 &&
-                     (nphase == 2 || nphase == 4) && (long long)found.size() == nphase;
+                     (nphase == 2 || nphase == 4) && (long long)found.size() == nphase && (nphase == 2 || g.X[2] >= fuse_min_row);
   if (fused) {
     std::stable_sort(found.begin(), found.end(), [](const PhaseTaps &a, const PhaseTaps &b) {
       if (a.ph.o0[0] != b.ph.o0[0]) return a.ph.o0[0] < b.ph.o0[0];
@@ -2030,6 +2041,7 @@ int get_plan(ConvOp op, const mg_conv_desc *d, const Geometry &g, Plan **out) {
   key.push_back(pos_table_enabled() ? 'q' : 'Q');
   if (const char *tile = getenv("MYGRAD_HIP_TILE")) key.append(tile);
   if (const char *tile = getenv("MYGRAD_HIP_WGRAD_TILE")) key.append("w").append(tile);
+  if (const char *row = getenv("MYGRAD_HIP_FUSE_MIN_ROW")) key.append("r").append(row);
   auto it = plans().find(key);
   if (it == plans().end()) {
     if (plans().size() >= 256) {

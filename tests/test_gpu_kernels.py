@@ -414,8 +414,12 @@ FUSED_PHASE_CASES = [
 ]
 
 
+@pytest.mark.parametrize("rows", ["short rows fused too", "short rows phase by phase"])
 @pytest.mark.parametrize("case", range(len(FUSED_PHASE_CASES)))
-def test_conv_dgrad_with_fused_stride_phases(abi, case, plan_mode):
+def test_conv_dgrad_with_fused_stride_phases(abi, case, plan_mode, rows, monkeypatch):
+    # four phases of rows shorter than 20 elements are planned phase by phase unless told otherwise
+    if rows == "short rows fused too":
+        monkeypatch.setenv("MYGRAD_HIP_FUSE_MIN_ROW", "0")
     x_shape, w_shape, s, p, d = FUSED_PHASE_CASES[case]
     rng = np.random.default_rng(900 + case)
     w = (rng.standard_normal(w_shape) / np.sqrt(np.prod(w_shape[1:]))).astype(np.float32)
@@ -667,6 +671,7 @@ def test_every_tile_shape_of_the_gather_gemm(abi, monkeypatch, problem, tile, dt
 
     monkeypatch.setenv("MYGRAD_HIP_TINY", "0")
     monkeypatch.setenv("MYGRAD_HIP_TILE", tile)
+    monkeypatch.setenv("MYGRAD_HIP_FUSE_MIN_ROW", "0")
     x_shape, w_shape, s, p, d = TILE_PROBLEMS[problem]
     rng = np.random.default_rng(2700 + problem)
     tol = TOL[np.dtype(dtype)]
