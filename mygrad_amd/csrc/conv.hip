@@ -2091,8 +2091,15 @@ void launch_gemm(GemmParams &gp, const Plan &pl, hipStream_t s) {
       return;
     }
     gp.items = (int)(pl.full_tiles + tail_tiles * pl.tail_split);
-    hipLaunchKernelGGL((tap_gemm_kernel<T, BM, BN, BK, WM, WN, NPH, FOLD, ROWS>), dim3((unsigned)std::min<long long>(gp.items, slots)),
-                       dim3(512), 0, s, gp);
+    const long long grid = std::min<long long>(gp.items, slots);
+    // MYGRAD_HIP_XCD_CHUNK=0: every block starts on the tile of its own number
+    static const bool chunks_on = [] {
+      const char *flag = getenv("MYGRAD_HIP_XCD_CHUNK");
+      return !(flag && flag[0] == '0');
+    }();
+    const int c = pl.m_tiles;
+    gp.xcd_chunk = chunks_on && tap_gemm_streams(BM, (int)sizeof(T)) && grid == slots && (c == 2 || c == 4 || c == 8) && grid % (8 * c) == 0 ? c : 1;
+    hipLaunchKernelGGL((tap_gemm_kernel<T, BM, BN, BK, WM, WN, NPH, FOLD, ROWS>), dim3((unsigned)grid), dim3(512), 0, s, gp);
     if (tail_tiles > 0)
       hipLaunchKernelGGL((tail_fixup_kernel<T, BM, BN, NPH>), dim3((unsigned)ceil_div(BM * BN, 256), (unsigned)tail_tiles),
                          dim3(256), 0, s, gp);

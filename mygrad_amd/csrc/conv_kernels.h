@@ -149,6 +149,12 @@ struct GemmParams {
   // rows of an MFMA tile are channels x phases instead of channels alone.  po0 / pJ above say
   // where a phase's elements lie in dst and which exist; phases 2q and 2q + 1 are rows next to
   // each other and, with a stride of two along the last axis, elements next to each other.
+  // Row tiles of one position block on one XCD (persistent blocks without even shares): blocks are
+  // handed to the 8 XCDs round-robin, each with its own L2, and the m_tiles row tiles of a position
+  // block gather the same elements.  With xcd_chunk = c > 1 the j-th block of an XCD starts on tile
+  // ((j / c) * 8 + xcd) * c + j % c instead of on its own number: c consecutive tiles meet in one L2
+  // (c divides 32, so that the two blocks of a compute unit still take tiles 256 apart).
+  int xcd_chunk;
   int phase_count;      // 0: off; else the number of stride phases (2 or 4)
   int phase_pairs;      // phases 2q, 2q + 1 are neighbours along the last axis of dst
 };

@@ -202,7 +202,11 @@ __global__ void __launch_bounds__(512) tap_gemm_kernel(const GemmParams p) {
   const int share_begin = shares ? ((const int MG_CONSTANT *)p.share_first)[uniform((int)blockIdx.x)] : 0;
   const int share_end = shares ? ((const int MG_CONSTANT *)p.share_first)[uniform((int)blockIdx.x) + 1] : 0;
   const int item_end = shares ? p.full_tiles + share_end : p.items;
-  const int item_first = (!shares || (int)blockIdx.x < p.full_tiles) ? (int)blockIdx.x : p.full_tiles + share_begin;
+  // the block's place in the order of the tiles (see GemmParams::xcd_chunk)
+  const int chunk = p.xcd_chunk;
+  const int place = chunk > 1 ? (((int)blockIdx.x >> 3) / chunk * 8 + ((int)blockIdx.x & 7)) * chunk + ((int)blockIdx.x >> 3) % chunk
+                              : (int)blockIdx.x;
+  const int item_first = (!shares || place < p.full_tiles) ? place : p.full_tiles + share_begin;
   auto next_item = [&](int item) -> int {
     if (!shares) return item + (int)gridDim.x;
     if (item >= p.full_tiles) return item + 1;
