@@ -1805,8 +1805,6 @@ int build_dgrad_plan(const Geometry &g, Plan &pl) {
 // wave tile.  The table-driven kernel has the 64-column shapes only.
 #define MG_WGRAD_SHAPES(T, X)                                                          \
   X(T, 128, 128, (sizeof(T) == 8 ? 16 : 32), 64, 64)                                   \
-  X(T, 64, 192, (sizeof(T) == 8 ? 16 : 32), 32, 96)                                    \
-  X(T, 64, 128, (sizeof(T) == 8 ? 16 : 32), 32, 64)                                    \
   X(T, 64, 64, (sizeof(T) == 8 ? 32 : 64), 32, 32)                                     \
   X(T, 32, 128, (sizeof(T) == 8 ? 16 : 32), 32, 32)                                    \
   X(T, 32, 64, (sizeof(T) == 8 ? 32 : 64), 32, 16)                                     \
@@ -1929,15 +1927,16 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
   };
   // Tap-major candidates in the order of preference: the first shape wins that divides F, wastes
   // little on padding the columns to whole tiles and still fills most block slots of the device
-  // with tiles x K splits.  128 x 128 re-reads grad and x least.  With 64 filters the square tile
-  // with the K tile 64 deep (half the barriers, one column group per gathering thread) comes
-  // before the wider ones: forced in turn on four layers with 64 filters it was 3 - 13 % faster than
-  // 64 x 192 and 64 x 128 (3x3 at 56x56: 240 / 250 / 294 us; 5x5 dilated: 173 / 192 / 197 us).
+  // with tiles x K splits.  128 x 128 re-reads grad and x least.  With 64 filters the tile is square
+  // with the K tile 64 deep (half the barriers, one column group per gathering thread): tiles of
+  // 64 x 192 and 64 x 128 with K tiles of 32, forced in turn on four layers with 64 filters, were
+  // 3 - 13 % slower (3x3 at 56x56: 240 / 250 / 294 us; 5x5 dilated: 173 / 192 / 197 us) and are
+  // no longer built.
   struct Cand {
     int bm, bn, bk;
   };
-  const Cand cands[] = {{128, 128, f64 ? 16 : 32}, {64, 64, f64 ? 32 : 64}, {64, 192, f64 ? 16 : 32}, {64, 128, f64 ? 16 : 32},
-                        {32, 128, f64 ? 16 : 32},  {32, 64, f64 ? 32 : 64},   {16, 64, f64 ? 32 : 64}};
+  const Cand cands[] = {{128, 128, f64 ? 16 : 32}, {64, 64, f64 ? 32 : 64}, {32, 128, f64 ? 16 : 32},
+                        {32, 64, f64 ? 32 : 64},   {16, 64, f64 ? 32 : 64}};
   long long best_splits = 1;
   pl.bm = 0;
   // MYGRAD_HIP_WGRAD_TILE="rows,columns" (diagnostics and the tests of every tile shape; part of the
@@ -1946,12 +1945,11 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
   if (const char *v = getenv("MYGRAD_HIP_WGRAD_TILE")) sscanf(v, "%d,%d", &forced_bm, &forced_bn);
   bool forced = false;
   for (const Cand &c : cands)
-    forced |= c.bm == forced_bm && c.bn == forced_bn && g.F % c.bm == 0 && !(f64 && c.bn == 192) && !(c.bm == 32 && c.bn == 128 && !f64);
+    forced |= c.bm == forced_bm && c.bn == forced_bn && g.F % c.bm == 0 && !(c.bm == 32 && c.bn == 128 && !f64);
   if (g.C % 16 == 0 && fits_buffer_loads(g)) {
     for (const Cand &c : cands) {
       if (forced && (c.bm != forced_bm || c.bn != forced_bn)) continue;
       if (g.F % c.bm != 0) continue;
-      if (f64 && c.bn == 192) continue;  // its accumulators leave room for one block per compute unit only
       // 32x64 double-precision tiles are bound by LDS reads (the 4x4x4 MFMA takes an operand
       // per 512 flops); the wider tile halves them per flop and is worth more padding.
       // In single precision 32x128 measured slower than 32x64.
@@ -1962,7 +1960,7 @@ int build_wgrad_plan(const Geometry &g, Plan &pl) {
         const int per_cu = f64 ? wgrad_blocks_per_cu<double>(c.bm, c.bn, true) : wgrad_blocks_per_cu<float>(c.bm, c.bn, true);
         const double waste = (double)(col_tiles * c.bn - ct) / (double)ct;
         const double filled = (double)(col_tiles * row_tiles * splits) / ((double)per_cu * cus);
-        if (waste > (c.bm == 32 ? 0.15 : c.bm == 128 ? 0.12 : 0.06) || filled < 0.75) continue;
+        if (waste > (c.bm == 32 ? 0.15 : 0.12) || filled < 0.75) continue;
       }
       best_splits = splits;
       pl.bm = c.bm, pl.bn = c.bn, pl.bk = c.bk;
