@@ -2092,8 +2092,8 @@ void launch_gemm(GemmParams &gp, const Plan &pl, hipStream_t s) {
     }
     gp.items = (int)(pl.full_tiles + tail_tiles * pl.tail_split);
     const long long grid = std::min<long long>(gp.items, slots);
-    // MYGRAD_HIP_XCD_CHUNK=0: every block starts on the tile of its own number
-    static const bool chunks_on = [] {
+    // MYGRAD_HIP_XCD_CHUNK=0 (read at every launch): every block starts on the tile of its own number
+    const bool chunks_on = [] {
       const char *flag = getenv("MYGRAD_HIP_XCD_CHUNK");
       return !(flag && flag[0] == '0');
     }();

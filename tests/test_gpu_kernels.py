@@ -693,6 +693,27 @@ def test_every_tile_shape_of_the_gather_gemm(abi, monkeypatch, problem, tile, dt
     assert np.array_equal(abi.conv_dgrad(gi, x_shape, wi, s, p, d), direct.conv_backward_x(gi, x_shape, wi, s, p, d).astype(dtype))
 
 
+@pytest.mark.parametrize("x_shape,w_shape,row_tiles", [
+    ((16, 32, 32, 32), (512, 32, 3, 3), 4),
+    ((8, 16, 32, 32), (1024, 16, 3, 3), 8),
+])
+def test_row_tiles_of_a_position_block_on_one_xcd(abi, monkeypatch, x_shape, w_shape, row_tiles):
+    """As many tiles as the device has block slots, 4 or 8 row tiles per position block: the blocks
+    start on the tiles in chunks per XCD (every tile must still be computed exactly once), and with
+    MYGRAD_HIP_XCD_CHUNK=0 on the tile of their own number; same results bit for bit."""
+    from mygrad_amd import _hip
+
+    monkeypatch.setenv("MYGRAD_HIP_TILE", "128,128,2")
+    rng = np.random.default_rng(2900 + row_tiles)
+    x = rng.standard_normal(x_shape).astype(np.float32)
+    w = (rng.standard_normal(w_shape) / np.sqrt(np.prod(w_shape[1:]))).astype(np.float32)
+    got = abi.conv_fwd(x, w, 1, 1, 1)
+    assert f"x {row_tiles} row tiles" in _hip.last_plan() and "tile 128x128" in _hip.last_plan()
+    assert rel_err(got, direct.conv_forward(x, w, (1, 1), (1, 1), (1, 1))) <= 2e-4
+    monkeypatch.setenv("MYGRAD_HIP_XCD_CHUNK", "0")  # read at every launch
+    assert np.array_equal(bits(got), bits(abi.conv_fwd(x, w, 1, 1, 1)))
+
+
 WGRAD_TILES = ["128,128", "64,64", "32,128", "32,64", "16,64"]
 
 
