@@ -208,6 +208,13 @@ int mg_maxpool_bwd_argmax(const mg_pool_desc *desc, const void *argmax, const vo
 int mg_maxpool_bwd_argmax_staged(const mg_pool_desc *inner, const mg_pool_desc *outer, const void *inner_argmax,
                                  const void *outer_argmax, const void *grad, void *dx);
 
+/* The same for six or seven pooled axes, which run as three mg_maxpool_fwd_argmax calls: `third` pools the
+ * two foremost axes over the merged grid of the first two stages, as `outer` does over the first
+ * stage's.  grad:(third lead, third grid); same order of additions (pooling.py:136-148). */
+int mg_maxpool_bwd_argmax_staged3(const mg_pool_desc *inner, const mg_pool_desc *outer, const mg_pool_desc *third,
+                                  const void *inner_argmax, const void *outer_argmax, const void *third_argmax, const void *grad,
+                                  void *dx);
+
 /* ---- element-wise and whole-array kernels either side of conv / pool ----
  * dtype: 0 float32, 1 float64; n elements, C-contiguous, same shape; device pointers,
  * 16-byte aligned (what mg_malloc returns). */

@@ -146,6 +146,7 @@ _SIGNATURES = {
     "mg_maxpool_fwd_argmax": [ctypes.POINTER(PoolDesc), _vp, _vp, _vp],
     "mg_maxpool_bwd_argmax": [ctypes.POINTER(PoolDesc), _vp, _vp, _vp],
     "mg_maxpool_bwd_argmax_staged": [ctypes.POINTER(PoolDesc), ctypes.POINTER(PoolDesc), _vp, _vp, _vp, _vp],
+    "mg_maxpool_bwd_argmax_staged3": [ctypes.POINTER(PoolDesc), ctypes.POINTER(PoolDesc), ctypes.POINTER(PoolDesc), _vp, _vp, _vp, _vp, _vp],
     "mg_multiply": [ctypes.c_int, ctypes.c_int64, _vp, _vp, _vp],
     "mg_multiply_broadcast": [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_int64),
                               ctypes.POINTER(ctypes.c_int64), _vp, _vp, _vp],

@@ -995,15 +995,20 @@ __global__ void __launch_bounds__(256) maxpool_exact_from_mark_kernel(PoolExactP
 // ------------------------------------------------------------------------------------------
 struct PoolStagedParams {
   int X[3], P[3], S[3], G[3];      // inner stage: the last three pooled axes
-  int OX[2], OP[2], OS[2], OG[2];  // outer stage: the leading pooled axes (extent 1 where there is none)
+  int OX[2], OP[2], OS[2], OG[2];  // second stage: the two pooled axes in front of them (extent 1 where there is none)
+  int RX[2], RP[2], RS[2], RG[2];  // third stage: the two in front of those (all ones without a third stage)
   int xvol, gvol;                  // elements of x / windows per leading position of the inner stage
   long long total;                 // elements of dx
-  FastDivP by_xvol, by_x12, by_x2, by_ox1, by_ox01, by_s[3], by_os[2];
+  FastDivP by_xvol, by_x12, by_x2, by_ox1, by_ox01, by_rx1, by_rx01, by_s[3], by_os[2], by_rs[2];
 };
 
+// With six or seven pooled axes there is a third stage over the merged grid of the first two
+// (`third_mark`, else null): three records name the element, and its windows along the two
+// foremost axes are the outermost loops.
 template <typename T, typename TD>
 __global__ void __launch_bounds__(256) maxpool_staged_gather_kernel(PoolStagedParams p, const unsigned char *__restrict__ inner_mark,
                                                                    const unsigned char *__restrict__ outer_mark,
+                                                                   const unsigned char *__restrict__ third_mark,
                                                                    const T *__restrict__ grad, TD *__restrict__ dx) {
   for (long long idx = (long long)blockIdx.x * 256 + threadIdx.x; idx < p.total; idx += (long long)gridDim.x * 256) {
     // element -> (leading index, q0, q1 | i0, i1, i2); leading positions fit 32 bits (checked by the host)
@@ -1013,11 +1018,14 @@ __global__ void __launch_bounds__(256) maxpool_staged_gather_kernel(PoolStagedPa
     r -= (unsigned)i0 * (unsigned)(p.X[1] * p.X[2]);
     const int i1 = (int)p.by_x2.div(r);
     const int i2 = (int)r - i1 * p.X[2];
-    const unsigned lead = p.by_ox01.div(pos);
+    const unsigned lead = p.by_ox01.div(pos);  // (leading index, r0, r1): the second stage's leading position
     const unsigned q01 = pos - lead * (unsigned)(p.OX[0] * p.OX[1]);
     const int q0 = (int)p.by_ox1.div(q01), q1 = (int)q01 - q0 * p.OX[1];
-    const int i[3] = {i0, i1, i2}, q[2] = {q0, q1};
-    int lo[3], hi[3], olo[2], ohi[2];
+    const unsigned lead3 = p.by_rx01.div(lead);  // the third stage's leading position
+    const unsigned r01 = lead - lead3 * (unsigned)(p.RX[0] * p.RX[1]);
+    const int r0 = (int)p.by_rx1.div(r01), r1 = (int)r01 - r0 * p.RX[1];
+    const int i[3] = {i0, i1, i2}, q[2] = {q0, q1}, rr[2] = {r0, r1};
+    int lo[3], hi[3], olo[2], ohi[2], rlo[2], rhi[2];
 #pragma unroll
     for (int k = 0; k < 3; ++k) {
       lo[k] = i[k] >= p.P[k] ? (int)p.by_s[k].div((unsigned)(i[k] - p.P[k] + p.S[k])) : 0;
@@ -1028,20 +1036,33 @@ __global__ void __launch_bounds__(256) maxpool_staged_gather_kernel(PoolStagedPa
       olo[k] = q[k] >= p.OP[k] ? (int)p.by_os[k].div((unsigned)(q[k] - p.OP[k] + p.OS[k])) : 0;
       ohi[k] = min(p.OG[k] - 1, (int)p.by_os[k].div((unsigned)q[k]));
     }
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      rlo[k] = rr[k] >= p.RP[k] ? (int)p.by_rs[k].div((unsigned)(rr[k] - p.RP[k] + p.RS[k])) : 0;
+      rhi[k] = min(p.RG[k] - 1, (int)p.by_rs[k].div((unsigned)rr[k]));
+    }
     const unsigned char *m1 = inner_mark + (long long)pos * p.gvol;
+    const long long ovol = (long long)p.OG[0] * p.OG[1] * p.gvol;  // windows of the first two stages per leading position of the third
     double acc = 0.0;
-    for (int h0 = olo[0]; h0 <= ohi[0]; ++h0)
-      for (int h1 = olo[1]; h1 <= ohi[1]; ++h1) {
-        const int mine_outer = (q0 - h0 * p.OS[0]) * p.OP[1] + (q1 - h1 * p.OS[1]);
-        const long long orow = (((long long)lead * p.OG[0] + h0) * p.OG[1] + h1) * p.gvol;
-        for (int g0 = lo[0]; g0 <= hi[0]; ++g0)
-          for (int g1 = lo[1]; g1 <= hi[1]; ++g1) {
-            const int row = (g0 * p.G[1] + g1) * p.G[2];
-            const int mine01 = ((i0 - g0 * p.S[0]) * p.P[1] + (i1 - g1 * p.S[1])) * p.P[2];
-            for (int g2 = lo[2]; g2 <= hi[2]; ++g2) {
-              const bool here = (int)m1[row + g2] == mine01 + (i2 - g2 * p.S[2]) && (int)outer_mark[orow + row + g2] == mine_outer;
-              if (here) acc += (double)grad[orow + row + g2];
-            }
+    for (int k0 = rlo[0]; k0 <= rhi[0]; ++k0)
+      for (int k1 = rlo[1]; k1 <= rhi[1]; ++k1) {
+        const int mine_third = (r0 - k0 * p.RS[0]) * p.RP[1] + (r1 - k1 * p.RS[1]);
+        const long long trow = (((long long)lead3 * p.RG[0] + k0) * p.RG[1] + k1) * ovol;  // into the third record and grad
+        for (int h0 = olo[0]; h0 <= ohi[0]; ++h0)
+          for (int h1 = olo[1]; h1 <= ohi[1]; ++h1) {
+            const int mine_outer = (q0 - h0 * p.OS[0]) * p.OP[1] + (q1 - h1 * p.OS[1]);
+            const long long orow = (((long long)lead * p.OG[0] + h0) * p.OG[1] + h1) * p.gvol;  // into the second record
+            const long long grow = trow + ((long long)h0 * p.OG[1] + h1) * p.gvol;            // (= orow without a third stage)
+            for (int g0 = lo[0]; g0 <= hi[0]; ++g0)
+              for (int g1 = lo[1]; g1 <= hi[1]; ++g1) {
+                const int row = (g0 * p.G[1] + g1) * p.G[2];
+                const int mine01 = ((i0 - g0 * p.S[0]) * p.P[1] + (i1 - g1 * p.S[1])) * p.P[2];
+                for (int g2 = lo[2]; g2 <= hi[2]; ++g2) {
+                  const bool here = (int)m1[row + g2] == mine01 + (i2 - g2 * p.S[2]) && (int)outer_mark[orow + row + g2] == mine_outer &&
+                                    (third_mark == nullptr || (int)third_mark[grow + row + g2] == mine_third);
+                  if (here) acc += (double)grad[grow + row + g2];
+                }
+              }
           }
       }
     dx[idx] = (TD)acc;
@@ -1663,16 +1684,19 @@ int mg_maxpool_bwd_argmax(const mg_pool_desc *desc, const void *argmax, const vo
   return maxpool_bwd_from_mark(desc, static_cast<const unsigned char *>(argmax), grad, dx);
 }
 
-int mg_maxpool_bwd_argmax_staged(const mg_pool_desc *inner, const mg_pool_desc *outer, const void *inner_argmax,
-                                 const void *outer_argmax, const void *grad, void *dx) {
+static int staged_gather(const mg_pool_desc *inner, const mg_pool_desc *outer, const mg_pool_desc *third, const void *inner_argmax,
+                         const void *outer_argmax, const void *third_argmax, const void *grad, void *dx) {
   std::lock_guard<std::recursive_mutex> guard(api_mutex());
   MG_REQUIRE_INIT();
-  PoolParams pi, po;
+  PoolParams pi, po, pt;
   if (int rc = check_pool_desc(inner, &pi)) return rc;
   if (int rc = check_pool_desc(outer, &po)) return rc;
-  if (!inner_argmax || !outer_argmax || !grad || !dx) return fail(MG_ERR_BAD_ARG, "null pointer in mg_maxpool_bwd_argmax_staged");
-  if (inner->dtype != outer->dtype || inner->dx_dtype != outer->dx_dtype)
-    return fail(MG_ERR_BAD_ARG, "the two stages disagree on the types");
+  if (third)
+    if (int rc = check_pool_desc(third, &pt)) return rc;
+  if (!inner_argmax || !outer_argmax || (third && !third_argmax) || !grad || !dx)
+    return fail(MG_ERR_BAD_ARG, "null pointer in mg_maxpool_bwd_argmax_staged");
+  if (inner->dtype != outer->dtype || inner->dx_dtype != outer->dx_dtype || (third && (third->dtype != inner->dtype || third->dx_dtype != inner->dx_dtype)))
+    return fail(MG_ERR_BAD_ARG, "the stages disagree on the types");
   // the outer stage pools the leading axes over the inner stage's windows: its last axis is their
   // merged grid with a window of one element, and its positions are the inner stage's leading indices
   if (po.X[2] != pi.gvol || po.P[2] != 1 || po.S[2] != 1 || po.G[2] != pi.gvol || po.lead * po.X[0] * po.X[1] != pi.lead)
@@ -1682,7 +1706,19 @@ int mg_maxpool_bwd_argmax_staged(const mg_pool_desc *inner, const mg_pool_desc *
     return fail(MG_ERR_UNSUPPORTED, "a window of more than 256 elements does not fit the one-byte argmax record");
   if (pi.lead >= (1ll << 31) || po.lead * po.G[0] * po.G[1] * pi.gvol >= (1ll << 40))
     return fail(MG_ERR_UNSUPPORTED, "too many leading positions for the staged gather");
+  // a third stage pools two more axes over the merged grid of the first two, in the same way
+  if (third && (pt.X[2] != po.gvol || pt.P[2] != 1 || pt.S[2] != 1 || pt.G[2] != po.gvol || pt.lead * pt.X[0] * pt.X[1] != po.lead))
+    return fail(MG_ERR_BAD_ARG, "the third stage (lead %lld, extents %d x %d x %d) does not pool the second stage's %lld positions of %lld windows",
+                pt.lead, pt.X[0], pt.X[1], pt.X[2], po.lead, po.gvol);
+  if (third && (long long)pt.P[0] * pt.P[1] > 256)
+    return fail(MG_ERR_UNSUPPORTED, "a window of more than 256 elements does not fit the one-byte argmax record");
   PoolStagedParams q{};
+  for (int k = 0; k < 2; ++k) {
+    q.RX[k] = third ? pt.X[k] : 1, q.RP[k] = third ? pt.P[k] : 1, q.RS[k] = third ? pt.S[k] : 1, q.RG[k] = third ? pt.G[k] : 1;
+    q.by_rs[k] = make_fastdiv_p((unsigned)q.RS[k]);
+  }
+  q.by_rx1 = make_fastdiv_p((unsigned)q.RX[1]);
+  q.by_rx01 = make_fastdiv_p((unsigned)(q.RX[0] * q.RX[1]));
   for (int k = 0; k < 3; ++k) {
     q.X[k] = pi.X[k], q.P[k] = pi.P[k], q.S[k] = pi.S[k], q.G[k] = pi.G[k];
     q.by_s[k] = make_fastdiv_p((unsigned)pi.S[k]);
@@ -1701,17 +1737,31 @@ int mg_maxpool_bwd_argmax_staged(const mg_pool_desc *inner, const mg_pool_desc *
   q.by_ox01 = make_fastdiv_p((unsigned)(po.X[0] * po.X[1]));
   hipStream_t s = runtime().stream;
   ScopedTiming timed(TAG_POOL_BWD);
-  note_plan("pool bwd from two stages' argmax: thread per element of dx, whole windows in row-major order");
+  note_plan(third ? "pool bwd from three stages' argmax: thread per element of dx, whole windows in row-major order"
+                  : "pool bwd from two stages' argmax: thread per element of dx, whole windows in row-major order");
   const unsigned grid = grid_for(q.total);
-  const unsigned char *m1 = static_cast<const unsigned char *>(inner_argmax), *m2 = static_cast<const unsigned char *>(outer_argmax);
+  const unsigned char *m1 = static_cast<const unsigned char *>(inner_argmax), *m2 = static_cast<const unsigned char *>(outer_argmax),
+                      *m3 = static_cast<const unsigned char *>(third_argmax);
   if (inner->dtype == MG_F64)
-    hipLaunchKernelGGL((maxpool_staged_gather_kernel<double, double>), dim3(grid), dim3(256), 0, s, q, m1, m2, (const double *)grad, (double *)dx);
+    hipLaunchKernelGGL((maxpool_staged_gather_kernel<double, double>), dim3(grid), dim3(256), 0, s, q, m1, m2, m3, (const double *)grad, (double *)dx);
   else if (inner->dx_dtype == MG_F64)
-    hipLaunchKernelGGL((maxpool_staged_gather_kernel<float, double>), dim3(grid), dim3(256), 0, s, q, m1, m2, (const float *)grad, (double *)dx);
+    hipLaunchKernelGGL((maxpool_staged_gather_kernel<float, double>), dim3(grid), dim3(256), 0, s, q, m1, m2, m3, (const float *)grad, (double *)dx);
   else
-    hipLaunchKernelGGL((maxpool_staged_gather_kernel<float, float>), dim3(grid), dim3(256), 0, s, q, m1, m2, (const float *)grad, (float *)dx);
+    hipLaunchKernelGGL((maxpool_staged_gather_kernel<float, float>), dim3(grid), dim3(256), 0, s, q, m1, m2, m3, (const float *)grad, (float *)dx);
   MG_HIP(hipGetLastError());
   return MG_OK;
+}
+
+int mg_maxpool_bwd_argmax_staged(const mg_pool_desc *inner, const mg_pool_desc *outer, const void *inner_argmax,
+                                 const void *outer_argmax, const void *grad, void *dx) {
+  return staged_gather(inner, outer, nullptr, inner_argmax, outer_argmax, nullptr, grad, dx);
+}
+
+int mg_maxpool_bwd_argmax_staged3(const mg_pool_desc *inner, const mg_pool_desc *outer, const mg_pool_desc *third,
+                                  const void *inner_argmax, const void *outer_argmax, const void *third_argmax, const void *grad,
+                                  void *dx) {
+  if (!third) return fail(MG_ERR_BAD_ARG, "null descriptor of the third stage");
+  return staged_gather(inner, outer, third, inner_argmax, outer_argmax, third_argmax, grad, dx);
 }
 
 int mg_maxpool_bwd(const mg_pool_desc *desc, const void *x, const void *grad, void *dx) {

@@ -84,9 +84,9 @@ class MaxPoolND(Operation):
     first leading position that holds the maximum, then the first place inside it).  So the
     last three axes are pooled with all others counted as leading axes, the three resulting
     grid axes are merged into one with a window of one element, and the rest is pooled again.
-    With two stages (four or five pooled axes) the gradient is routed through both records at
-    once, every element adding its windows in the reference's order (bit-exact); with more, it
-    takes the stages in reverse, in float64 between them as the reference accumulates it
+    With two or three stages (four to seven pooled axes) the gradient is routed through all
+    records at once, every element adding its windows in the reference's order (bit-exact); with
+    more, it takes the stages in reverse, in float64 between them as the reference accumulates it
     (pooling.py:147): the same terms in another order.
     """
 
@@ -216,15 +216,17 @@ class MaxPoolND(Operation):
             fresh = True
         gb = _device.to_device(grad, x.dtype)
         g_dtype = x.dtype
-        if len(stages) == 2 and fresh and all(stage.argmax is not None for stage in stages):
-            # Four or five pooled axes: both stages' records together name the element a whole window
+        if len(stages) in (2, 3) and fresh and all(stage.argmax is not None for stage in stages):
+            # Four to seven pooled axes: the stages' records together name the element a whole window
             # routes to, and one gather adds every element's windows in the row-major order of the
             # whole windows -- np.add.at's order (pooling.py:147-148), bit for bit.  (Stage by stage,
             # as below, the same terms are added in another order.)
-            inner, outer = stages
+            inner = stages[0]
             db = _device.DeviceBuffer(inner.count * dx_dtype.itemsize)
-            _hip.check(_hip.lib().mg_maxpool_bwd_argmax_staged(inner.desc(x.dtype, dx_dtype), outer.desc(x.dtype, dx_dtype),
-                                                               inner.argmax.ptr, outer.argmax.ptr, gb.ptr, db.ptr))
+            descs = [stage.desc(x.dtype, dx_dtype) for stage in stages]
+            records = [stage.argmax.ptr for stage in stages]
+            entry = _hip.lib().mg_maxpool_bwd_argmax_staged if len(stages) == 2 else _hip.lib().mg_maxpool_bwd_argmax_staged3
+            _hip.check(entry(*descs, *records, gb.ptr, db.ptr))
             out = _device.download(db, x.shape, dx_dtype)
             _device.attach_transient(out, db)
             return out

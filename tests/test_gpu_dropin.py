@@ -526,11 +526,15 @@ def test_pooling_over_more_axes_than_the_kernels_take(case, dtype):
     ((2, 7, 6, 7, 8), (3, 2, 3, 2), (1, 2, 2, 3)),          # four pooled axes, windows that overlap along three of them
     ((3, 5, 6, 5, 7, 9), (2, 3, 2, 3, 3), (1, 1, 1, 2, 2)),  # five
     ((6, 5, 5, 5), (3, 3, 3, 3), (1, 1, 1, 1)),              # every element under up to 81 windows, no leading axes
+    # six and seven pooled axes: three stages, three records
+    ((2, 4, 5, 4, 5, 6, 5), (2, 3, 2, 3, 2, 3), (1, 1, 2, 1, 2, 1)),
+    ((3, 4, 3, 4, 3, 5, 4), (2, 2, 2, 2, 2, 3, 2), (1, 1, 1, 2, 1, 1, 2)),
 ])
 def test_pooling_over_four_and_five_axes_adds_in_the_reference_order(x_shape, pool, stride, dtype):
     """Real-valued gradients of very different magnitudes: the sum an element receives depends on
     the order of its terms, and must be np.add.at's (pooling.py:147-148) bit for bit -- also for a
-    float32 x, whose sums the reference carries in float64 and rounds once."""
+    float32 x, whose sums the reference carries in float64 and rounds once.  (Four to seven pooled
+    axes: two or three stages of the kernels' three axes.)"""
     rng = np.random.default_rng(4100 + len(pool))
     xv = rng.integers(0, 3, x_shape).astype(dtype)  # ties: an element is the argmax of many windows
     out_shape = ora.pool_forward(xv, pool, stride).shape
@@ -538,6 +542,9 @@ def test_pooling_over_four_and_five_axes_adds_in_the_reference_order(x_shape, po
     g[rng.random(out_shape) < 0.1] = -0.0
     x = mg.Tensor(xv)
     max_pool(x, pool, stride).backward(g)
+    from mygrad_amd import _hip
+
+    assert ("three" if len(pool) > 5 else "two") + " stages' argmax" in _hip.last_plan()
     want = ora.pool_backward(xv, g, pool, stride)  # float64
     kind = np.uint64 if dtype == np.float64 else np.uint32
     assert np.array_equal(x.grad.view(kind), want.astype(dtype).view(kind))
