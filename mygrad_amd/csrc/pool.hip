@@ -832,8 +832,21 @@ struct PoolGatherParams {
   int groups;        // groups of S1 rows per plane: ceil(X1 / S1)
   int groups0;       // groups of S0 planes per leading index: ceil(X0 / S0)
   long long planes;  // lead * groups0
+  int leads;         // leading positions: each has G0 * G1 * G2 windows
   FastDivP by_pieces, by_groups, by_groups0;
 };
+
+// acc += term on the lanes where code == wanted; the others keep acc (adding +0.0 to a sum that
+// started at +0.0 would leave it as it is, too).  The comparison narrows the execution mask for the
+// one addition, which takes half the vector instructions of two selects and an addition; the mask
+// is put back before the statement ends.
+__device__ __forceinline__ void add_where_equal(double &acc, double term, int code, int wanted) {
+  unsigned long long all;
+  asm("s_mov_b64 %1, exec\n\tv_cmpx_eq_u32_e32 vcc, %4, %3\n\tv_add_f64 %0, %0, %2\n\ts_mov_b64 exec, %1"
+      : "+v"(acc), "=&s"(all)
+      : "v"(term), "v"(code), "s"(wanted)
+      : "vcc");
+}
 
 template <typename T, typename TD, int P0, int P1, int P2, int S0, int S1, int S2>
 __global__ void __launch_bounds__(256) maxpool_mark_gather_kernel(PoolGatherParams p, const unsigned char *__restrict__ mark,
@@ -844,101 +857,150 @@ __global__ void __launch_bounds__(256) maxpool_mark_gather_kernel(PoolGatherPara
   constexpr int LW = NW2 <= 2 ? 2 : NW2 <= 4 ? 4 : 8;  // windows loaded per window row
   static_assert(VD % S2 == 0 && NW2 <= 8, "a piece starts on a window boundary");
   typedef TD DVec __attribute__((ext_vector_type(VD), aligned(sizeof(TD))));
-  const long long item = (long long)xcd_run(blockIdx.x, gridDim.x) * 256 + threadIdx.x;
-  if (item >= p.planes * p.groups * p.pieces) return;
-  const unsigned u = (unsigned)item;
-  const unsigned q = p.by_pieces.div(u), piece = u - q * (unsigned)p.pieces;
-  const unsigned plane = p.by_groups.div(q);  // (leading index, group of S0 planes)
-  const int k1 = (int)(q - plane * (unsigned)p.groups);
-  const unsigned lead = p.by_groups0.div(plane);
-  const int k0 = (int)(plane - lead * (unsigned)p.groups0);
-  const int i2 = (int)piece * VD;
-  const int live = (p.tail != 0 && (int)piece == p.pieces - 1) ? p.tail : VD;  // columns of this piece
-  const long long gvol = (long long)p.G0 * p.G1 * p.G2;
-  const unsigned char *m = mark + (long long)lead * gvol;
-  const T *g = grad + (long long)lead * gvol;
-  const int g0_first = k0 - (C0 - 1), g1_first = k1 - (C1 - 1), g2_first = i2 / S2 - (C2 - 1);
-
-  // The NW2 windows of a window row are neighbours in the record and in grad: LW of them (a power
-  // of two that holds NW2) come as one load each, from the run [b, b + LW) that starts at the first
-  // window wanted where that lies inside the row and at the nearest run inside it otherwise; the
-  // window wanted at place e is then the loaded one at place e + shift.
-  int code[C0][C1][NW2];
-  double term[C0][C1][NW2];
   typedef unsigned char CVec __attribute__((ext_vector_type(LW), aligned(1)));
   typedef T GVec __attribute__((ext_vector_type(LW), aligned(sizeof(T))));
-  const int b = min(max(g2_first, 0), p.G2 - LW);
-  const int shift = g2_first - b;
+  struct Where {  // an item: the piece `piece` of the rows k1 * S1 ... in the planes k0 * S0 ... of leading position `lead`
+    unsigned lead;
+    int k0, k1, piece;
+  };
+  struct Asked {  // the windows that can reach it, as loaded
+    CVec lc[C0][C1];
+    GVec lg[C0][C1];
+  };
+  const long long total = p.planes * p.groups * p.pieces;
+  const int gvol = p.G0 * p.G1 * p.G2;
+  const auto where_of = [&](long long item) {
+    const unsigned u = (unsigned)item;
+    const unsigned q = p.by_pieces.div(u);
+    const unsigned plane = p.by_groups.div(q);  // (leading index, group of S0 planes)
+    Where w;
+    w.piece = (int)(u - q * (unsigned)p.pieces);
+    w.k1 = (int)(q - plane * (unsigned)p.groups);
+    w.lead = p.by_groups0.div(plane);
+    w.k0 = (int)(plane - w.lead * (unsigned)p.groups0);
+    return w;
+  };
+  // The NW2 windows of a window row are neighbours in the record and in grad: LW of them (a power
+  // of two that holds NW2) come as one load each, starting at the first window wanted.  That one
+  // may lie before the row and the last ones beyond it: what is loaded there belongs to
+  // neighbouring rows and is masked (such windows do not exist), and only at the two ends of the
+  // whole record does the run have to move inside -- by `shift`, and the window wanted at place e
+  // is then the loaded one at place e + shift.  Returns where the run starts in the leading
+  // position's part of the record.
+  const auto run_start = [&](const Where &w, int d0, int d, int &shift, bool &exists) {
+    const int g0 = w.k0 - (C0 - 1) + d0, g1 = w.k1 - (C1 - 1) + d, g2_first = w.piece * VD / S2 - (C2 - 1);
+    exists = (g0 >= 0) & (g0 < p.G0) & (g1 >= 0) & (g1 < p.G1);
+    const int wanted = (min(max(g0, 0), p.G0 - 1) * p.G1 + min(max(g1, 0), p.G1 - 1)) * p.G2 + g2_first;
+    const int lowest = w.lead == 0 ? 0 : -LW, highest = (int)w.lead == p.leads - 1 ? gvol - LW : gvol;
+    const int r = min(max(wanted, lowest), highest);
+    shift = wanted - r;
+    return r;
+  };
+  const auto ask = [&](const Where &w, Asked &a) {
+    const unsigned char *m = mark + (long long)w.lead * gvol;
+    const T *g = grad + (long long)w.lead * gvol;
 #pragma unroll
-  for (int d0 = 0; d0 < C0; ++d0) {
-    const int g0 = g0_first + d0;
-    const bool ok0 = (g0 >= 0) & (g0 < p.G0);
-    const int r0 = min(max(g0, 0), p.G0 - 1) * p.G1;
+    for (int d0 = 0; d0 < C0; ++d0)
 #pragma unroll
-    for (int d = 0; d < C1; ++d) {
-      const int g1 = g1_first + d;
-      const bool ok1 = ok0 & (g1 >= 0) & (g1 < p.G1);
-      const int r = (r0 + min(max(g1, 0), p.G1 - 1)) * p.G2 + b;
-      const CVec lc = *reinterpret_cast<const CVec *>(m + r);
-      const GVec lg = *reinterpret_cast<const GVec *>(g + r);
-#pragma unroll
-      for (int e = 0; e < NW2; ++e) {
-        const int g2 = g2_first + e;
-        const bool ok = ok1 & (g2 >= 0) & (g2 < p.G2);
-        int c = -1;
-        T t = T(0);
-#pragma unroll
-        for (int k = 0; k < LW; ++k) {
-          const bool here = e + shift == k;
-          c = here ? (int)lc[k] : c;
-          t = here ? lg[k] : t;
-        }
-        code[d0][d][e] = ok ? c : -1;  // a window that does not exist names no element
-        term[d0][d][e] = (double)t;
+      for (int d = 0; d < C1; ++d) {
+        int shift;
+        bool exists;
+        const int r = run_start(w, d0, d, shift, exists);
+        a.lc[d0][d] = *reinterpret_cast<const CVec *>(m + r);
+        a.lg[d0][d] = *reinterpret_cast<const GVec *>(g + r);
       }
+  };
+  const auto finish = [&](const Where &w, const Asked &a) {
+    const int i2 = w.piece * VD, g2_first = i2 / S2 - (C2 - 1);
+    const int live = (p.tail != 0 && w.piece == p.pieces - 1) ? p.tail : VD;  // columns of this piece
+    int code[C0][C1][NW2];
+    double term[C0][C1][NW2];
+    int shift[C0][C1];
+    bool exists[C0][C1];
+    int moved = 0;
+#pragma unroll
+    for (int d0 = 0; d0 < C0; ++d0)
+#pragma unroll
+      for (int d = 0; d < C1; ++d) {
+        run_start(w, d0, d, shift[d0][d], exists[d0][d]);
+        moved |= shift[d0][d];
+#pragma unroll
+        for (int e = 0; e < NW2; ++e) {
+          const int g2 = g2_first + e;
+          const bool ok = exists[d0][d] & (g2 >= 0) & (g2 < p.G2);
+          code[d0][d][e] = ok ? (int)a.lc[d0][d][e] : -1;  // a window that does not exist names no element
+          term[d0][d][e] = (double)a.lg[d0][d][e];
+        }
+      }
+    if (moved != 0) {  // some of the first and the last threads of the grid only
+#pragma unroll
+      for (int d0 = 0; d0 < C0; ++d0)
+#pragma unroll
+        for (int d = 0; d < C1; ++d)
+#pragma unroll
+          for (int e = 0; e < NW2; ++e) {
+            const int g2 = g2_first + e;
+            const bool ok = exists[d0][d] & (g2 >= 0) & (g2 < p.G2);
+            int c = -1;
+            T t = T(0);
+#pragma unroll
+            for (int k = 0; k < LW; ++k) {
+              const bool here = e + shift[d0][d] == k;
+              c = here ? (int)a.lc[d0][d][k] : c;
+              t = here ? a.lg[d0][d][k] : t;
+            }
+            code[d0][d][e] = ok ? c : -1;
+            term[d0][d][e] = (double)t;
+          }
     }
-  }
-  TD *to = dx + (((long long)lead * p.X0 + (long long)k0 * S0) * p.X1 + (long long)k1 * S1) * p.X2 + i2;
+    TD *to = dx + (((long long)w.lead * p.X0 + (long long)w.k0 * S0) * p.X1 + (long long)w.k1 * S1) * p.X2 + i2;
 #pragma unroll
-  for (int pp = 0; pp < S0; ++pp) {
-    if (k0 * S0 + pp >= p.X0) break;
+    for (int pp = 0; pp < S0; ++pp) {
+      if (w.k0 * S0 + pp >= p.X0) break;
 #pragma unroll
-    for (int rr = 0; rr < S1; ++rr) {
-      if (k1 * S1 + rr >= p.X1) break;
-      DVec out;
+      for (int rr = 0; rr < S1; ++rr) {
+        if (w.k1 * S1 + rr >= p.X1) break;
+        DVec out;
 #pragma unroll
-      for (int v = 0; v < VD; ++v) {
-        double acc = 0.0;
+        for (int v = 0; v < VD; ++v) {
+          double acc = 0.0;
 #pragma unroll
-        for (int d0 = 0; d0 < C0; ++d0) {
-          const int a0 = pp + (C0 - 1 - d0) * S0;  // the plane's offset inside window plane d0: known at compile time
-          if (a0 >= P0) continue;
+          for (int d0 = 0; d0 < C0; ++d0) {
+            const int a0 = pp + (C0 - 1 - d0) * S0;  // the plane's offset inside window plane d0: known at compile time
+            if (a0 >= P0) continue;
 #pragma unroll
-          for (int d = 0; d < C1; ++d) {
-            const int a1 = rr + (C1 - 1 - d) * S1;  // the row's offset inside window row d
-            if (a1 >= P1) continue;                 // that window row does not reach this row
+            for (int d = 0; d < C1; ++d) {
+              const int a1 = rr + (C1 - 1 - d) * S1;  // the row's offset inside window row d
+              if (a1 >= P1) continue;                 // that window row does not reach this row
 #pragma unroll
-            for (int e = 0; e < C2; ++e) {
-              const int w = v / S2 + e;                     // which of the loaded windows
-              const int a2 = (v % S2) + (C2 - 1 - e) * S2;   // the element's offset inside it
-              if (a2 >= P2) continue;
-              // + (+0.0) leaves a sum that started at +0.0 as it is
-              acc += code[d0][d][w] == (a0 * P1 + a1) * P2 + a2 ? term[d0][d][w] : 0.0;
+              for (int e = 0; e < C2; ++e) {
+                const int wd = v / S2 + e;                    // which of the loaded windows
+                const int a2 = (v % S2) + (C2 - 1 - e) * S2;  // the element's offset inside it
+                if (a2 >= P2) continue;
+                add_where_equal(acc, term[d0][d][wd], code[d0][d][wd], (a0 * P1 + a1) * P2 + a2);
+              }
             }
           }
+          out[v] = (TD)acc;
         }
-        out[v] = (TD)acc;
-      }
-      TD *row = to + ((long long)pp * p.X1 + rr) * p.X2;
-      if (live == VD) {
-        *reinterpret_cast<DVec *>(row) = out;
-      } else {
+        TD *row = to + ((long long)pp * p.X1 + rr) * p.X2;
+        if (live == VD) {
+          *reinterpret_cast<DVec *>(row) = out;
+        } else {
 #pragma unroll
-        for (int v = 0; v < VD - 1; ++v)
-          if (v < live) row[v] = out[v];
+          for (int v = 0; v < VD - 1; ++v)
+            if (v < live) row[v] = out[v];
+        }
       }
     }
-  }
+  };
+
+  const long long item = (long long)xcd_run(blockIdx.x, gridDim.x) * 256 + threadIdx.x;
+  if (item >= total) return;
+  const Where w = where_of(item);
+  Asked a;
+  ask(w, a);
+  finish(w, a);
 }
 
 // The same for windows that tile the input exactly: an element belongs to one window, so a
@@ -1389,6 +1451,7 @@ static int launch_mark_gather(const PoolParams &p, bool f32, bool wide, const un
   q.groups = (int)ceil_div(p.X[1], p.S[1]);
   q.groups0 = (int)ceil_div(p.X[0], p.S[0]);
   q.planes = p.lead * q.groups0;
+  q.leads = (int)p.lead;
   q.by_pieces = make_fastdiv_p((unsigned)q.pieces);
   q.by_groups = make_fastdiv_p((unsigned)q.groups);
   q.by_groups0 = make_fastdiv_p((unsigned)q.groups0);
