@@ -1172,6 +1172,33 @@ def run_copy_calibration(mib=1024, reps=20):
             "value": 2 * n * 1e-9 / (avg * 1e-3), "unit": "GB/s", "launches": len(ms)}
 
 
+def run_mix_calibration(mib=268, reps=10):
+    """One stream over a buffer larger than the last-level cache, stored or loaded 16 bytes
+    per lane, with the opposite stream at a fraction of its volume: what the memory system
+    sustains per mix of loads and stores -- the practical ceiling of the bandwidth-bound
+    kernels, whose passes are such mixes (a pooling gradient stores 7 bytes per byte it loads,
+    a 1x1 convolution to four times the channels 4 per byte)."""
+    from mygrad_amd import _device, _hip
+
+    n = mib << 20
+    big, small, other = _device.DeviceBuffer(n), _device.DeviceBuffer(n), _device.DeviceBuffer(n)
+    lib = _hip.lib()
+    for buf in (big, small, other):
+        _hip.check(lib.mg_memset_zero(buf.ptr, n))
+    rows = []
+    for store_big in (1, 0):
+        for share in (0, 64, 8, 4, 2, 1):
+            ms = []
+            for _ in range(reps):
+                _hip.probe_stream(other.ptr, small.ptr, n, 0, 0)  # reading a third buffer pushes the operands out of the caches
+                ms.append(_hip.probe_stream(big.ptr, small.ptr, n, share, store_big))
+            avg = float(np.mean(ms[2:]))
+            second = n // share if share else 0
+            rows.append({"stored_bytes": n if store_big else second, "loaded_bytes": second if store_big else n,
+                         "avg_kernel_us": avg * 1e3, "GB/s": (n + second) * 1e-9 / (avg * 1e-3)})
+    return {"metric": "one launch of a load stream and a store stream, 16 bytes per lane", "unit": "GB/s", "mixes": rows}
+
+
 def run_mfma_probe():
     """What the matrix cores sustain per MFMA shape with operands in registers and no
     memory traffic, next to the published peaks: the ceiling of the convolution
@@ -1207,6 +1234,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a 1 GiB device copy (the reference point for HBM traffic counters)")
     ap.add_argument("--copy-mib", type=int, default=1024, help="size of the --calibrate-copy buffer in MiB (read + written)")
+    ap.add_argument("--calibrate-mix", action="store_true",
+                    help="time a store (or load) stream with the opposite stream at 0, 1/64 ... 1/1 of its volume and exit")
+    ap.add_argument("--mix-mib", type=int, default=268, help="size of the larger stream of --calibrate-mix in MiB")
     ap.add_argument("--sweep", action="store_true",
                     help="run only the sweep over reference-valid shapes around the benchmark's, pass by pass: a text "
                          "table on stdout (what profiles/sweep_hotpath.txt holds), the rows as one JSON line on stderr")
@@ -1221,6 +1251,9 @@ def main():
 
     if args.calibrate_copy:
         print(json.dumps(run_copy_calibration(args.copy_mib)))
+        return
+    if args.calibrate_mix:
+        print(json.dumps(run_mix_calibration(args.mix_mib)))
         return
     if args.probe_mfma:
         print(json.dumps(run_mfma_probe()))

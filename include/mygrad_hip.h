@@ -153,6 +153,15 @@ int mg_timing_pause(int paused);
  * besides the published peak (bench.py --probe-mfma). */
 int mg_probe_mfma(int kind, int waves_per_simd, double *tflops);
 
+/* Device diagnostic, no counterpart in the reference: one launch that stores (store_big
+ * != 0) or loads (store_big == 0) every 16-byte piece of `big` (big_bytes, a multiple of
+ * 16) while the opposite stream runs over `small` at 1 / share of that volume -- piece i of
+ * big goes with piece i / share of small, which therefore needs ceil(big_bytes / share)
+ * bytes (16 with share 0: no second stream).  *ms receives the launch's duration by HIP
+ * events.  It measures what the memory system sustains for a given mix of loads and
+ * stores, the ceiling of the bandwidth-bound kernels (bench.py --calibrate-mix). */
+int mg_probe_stream(void *big_dev, void *small_dev, size_t big_bytes, int share, int store_big, float *ms);
+
 /* ---- convolution ---- */
 
 /* out[n,f,g] = sum_{c,t} w[f,c,t] * x[n,c,g*stride+t*dil-pad] (zero outside x).

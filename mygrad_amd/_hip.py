@@ -134,6 +134,8 @@ _SIGNATURES = {
     "mg_timing_read": [ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_float), ctypes.c_int,
                        ctypes.POINTER(ctypes.c_int)],
     "mg_probe_mfma": [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double)],
+    "mg_probe_stream": [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int,
+                        ctypes.POINTER(ctypes.c_float)],
     "mg_event_create": [ctypes.POINTER(_vp)],
     "mg_event_record": [_vp],
     "mg_event_elapsed_ms": [_vp, _vp, ctypes.POINTER(ctypes.c_float)],
@@ -317,6 +319,14 @@ def probe_mfma(kind, waves_per_simd=2):
     """TFLOP/s the matrix cores sustain on one MFMA shape with nothing else in the way."""
     out = ctypes.c_double()
     check(lib().mg_probe_mfma(MFMA_KINDS[kind], int(waves_per_simd), ctypes.byref(out)))
+    return out.value
+
+
+def probe_stream(big_ptr, small_ptr, big_bytes, share, store_big):
+    """Milliseconds of one launch that stores (or loads) `big_bytes` while the opposite
+    stream moves 1 / share of that volume (share 0: no second stream)."""
+    out = ctypes.c_float()
+    check(lib().mg_probe_stream(big_ptr, small_ptr, int(big_bytes), int(share), int(bool(store_big)), ctypes.byref(out)))
     return out.value
 
 

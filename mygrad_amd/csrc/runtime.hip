@@ -175,6 +175,25 @@ using namespace mg;
 
 // ---- matrix-core rate probe ---------------------------------------------------------
 namespace {
+// Streams for the memory probe: every 16-byte piece of `big` is stored (or loaded); piece i
+// goes with piece i / share of `small`, so the second stream is 1 / share of the first.
+__global__ void __launch_bounds__(256) stream_store_kernel(float4 *big, const float4 *small, long long pieces, int share) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= pieces) return;
+  float4 v = make_float4(1.f, 2.f, 3.f, 4.f);
+  if (share > 0) v = small[i / share];
+  v.x += 1.f;
+  big[i] = v;
+}
+
+__global__ void __launch_bounds__(256) stream_load_kernel(const float4 *big, float4 *small, long long pieces, int share) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= pieces) return;
+  const float4 v = big[i];
+  // without a second stream the value still has to arrive: the store below never happens for finite data
+  if (share > 0 ? i % share == 0 : (v.x != v.x && v.y == 123.25f)) small[share > 0 ? i / share : 0] = v;
+}
+
 typedef float probe_f32x4 __attribute__((ext_vector_type(4)));
 typedef double probe_f64x4 __attribute__((ext_vector_type(4)));
 
@@ -552,6 +571,39 @@ int mg_timing_read(int32_t *tags, float *ms, int capacity, int *count) {
     MG_HIP(hipEventElapsedTime(&ms[i], g_timing.events[g_timing.records[i].start], g_timing.events[g_timing.records[i].stop]));
   }
   timing_reset();
+  return MG_OK;
+}
+
+int mg_probe_stream(void *big_dev, void *small_dev, size_t big_bytes, int share, int store_big, float *ms) {
+  MG_LOCK();
+  MG_REQUIRE_INIT();
+  if (!big_dev || !small_dev || !ms) return fail(MG_ERR_BAD_ARG, "null argument in mg_probe_stream");
+  if (big_bytes < 16 || big_bytes % 16 != 0) return fail(MG_ERR_BAD_ARG, "mg_probe_stream: %zu bytes (a multiple of 16 wanted)", big_bytes);
+  if (share < 0) return fail(MG_ERR_BAD_ARG, "mg_probe_stream: share %d (0: no second stream)", share);
+  if ((reinterpret_cast<uintptr_t>(big_dev) | reinterpret_cast<uintptr_t>(small_dev)) & 15u)
+    return fail(MG_ERR_BAD_ARG, "mg_probe_stream needs 16-byte aligned buffers");
+  const long long pieces = (long long)(big_bytes / 16);
+  const long long blocks = (pieces + 255) / 256;
+  if (blocks > 0x7fffffffll) return fail(MG_ERR_UNSUPPORTED, "mg_probe_stream: %zu bytes are more than one launch covers", big_bytes);
+  hipStream_t s = runtime().stream;
+  struct EventPair {  // destroyed on every way out
+    hipEvent_t t0 = nullptr, t1 = nullptr;
+    ~EventPair() {
+      if (t0) (void)hipEventDestroy(t0);
+      if (t1) (void)hipEventDestroy(t1);
+    }
+  } ev;
+  MG_HIP(hipEventCreate(&ev.t0));
+  MG_HIP(hipEventCreate(&ev.t1));
+  MG_HIP(hipEventRecord(ev.t0, s));
+  if (store_big)
+    hipLaunchKernelGGL(stream_store_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (float4 *)big_dev, (const float4 *)small_dev, pieces, share);
+  else
+    hipLaunchKernelGGL(stream_load_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (const float4 *)big_dev, (float4 *)small_dev, pieces, share);
+  MG_HIP(hipEventRecord(ev.t1, s));
+  MG_HIP(hipEventSynchronize(ev.t1));
+  MG_HIP(hipEventElapsedTime(ms, ev.t0, ev.t1));
+  MG_HIP(hipGetLastError());
   return MG_OK;
 }
 

@@ -1145,6 +1145,41 @@ def test_mfma_probe_reports_plausible_rates():
         _hip.probe_mfma("f32_16x16x4", 9)
 
 
+@pytest.mark.gpu
+def test_stream_probe_moves_what_it_says():
+    """The memory diagnostic stores every 16-byte piece of the large buffer from piece
+    i / share of the small one (first value plus one), or loads the large buffer and stores
+    every share-th piece to the small one; sizes and alignment are checked."""
+    from mygrad_amd import _device, _hip
+
+    pieces = 1000
+    small_host = np.arange(4 * pieces, dtype=np.float32).reshape(pieces, 4)
+    big, small = _device.DeviceBuffer(16 * pieces), _device.DeviceBuffer(16 * pieces)
+    small.upload(small_host)
+    got = np.empty((pieces, 4), dtype=np.float32)
+    for share in (1, 2, 8):
+        assert _hip.probe_stream(big.ptr, small.ptr, 16 * pieces, share, True) > 0.0
+        big.download_into(got)
+        want = small_host[np.arange(pieces) // share].copy()
+        want[:, 0] += 1.0
+        assert np.array_equal(got, want)
+    _hip.probe_stream(big.ptr, small.ptr, 16 * pieces, 0, True)
+    big.download_into(got)
+    assert np.array_equal(got, np.tile(np.array([2.0, 2.0, 3.0, 4.0], dtype=np.float32), (pieces, 1)))
+    big.upload(small_host)
+    _hip.check(_hip.lib().mg_memset_zero(small.ptr, 16 * pieces))
+    _hip.probe_stream(big.ptr, small.ptr, 16 * pieces, 4, False)
+    small.download_into(got)
+    assert np.array_equal(got[: pieces // 4], small_host[::4]) and not got[pieces // 4:].any()
+    _hip.probe_stream(big.ptr, small.ptr, 16 * pieces, 0, False)  # loads only
+    small.download_into(got)
+    assert np.array_equal(got[: pieces // 4], small_host[::4])
+    with pytest.raises(_hip.HipError):
+        _hip.probe_stream(big.ptr, small.ptr, 24, 1, True)
+    with pytest.raises(_hip.HipError):
+        _hip.probe_stream(big.ptr + 4, small.ptr, 16, 1, True)
+
+
 def test_per_launch_timing_records_chains_and_pauses():
     """``mg_timing_enable`` / ``mg_timing_read`` give one (kernel, milliseconds) record per timed
     launch, in order; ``mg_timing_pause`` suspends the recording without dropping what was
