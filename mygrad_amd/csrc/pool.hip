@@ -818,10 +818,11 @@ __global__ void __launch_bounds__(256) maxpool_rows_fwd_kernel(PoolRowsParams p,
 // k1*S1 + S1 - 1 are covered by the same ceil(P1/S1) window rows (the planes by the same
 // ceil(P0/S0) window planes), and the piece's columns by the same ceil(P2/S2) - 1 + VD/S2 windows
 // along the row, whichever thread -- so their recorded offsets and gradients are loaded up front
-// (clamped, never predicated), and every element adds, in ascending window order, the gradient
-// of the windows whose recorded offset names it and +0.0 for the others: no loop bounds to
-// compute, no divisions by runtime values, no LDS.  Needs VD % S2 == 0 (a piece starts on a
-// window boundary) and at least pool_gather_run() windows per row.
+// (never predicated: a window that does not exist is loaded from a neighbour's place and
+// masked), and every element adds, in ascending window order, the gradient of the windows whose
+// recorded offset names it: no loop bounds to compute, no divisions by runtime values, no LDS.
+// Needs VD % S2 == 0 (a piece starts on a window boundary) and at least pool_gather_run() windows
+// per row.
 // Pieces are counted in columns: rows of dx need not start on 16-byte boundaries (the stores only
 // assume the alignment of an element), and the short piece at the end of a row that is no whole
 // number of pieces is stored element by element.
