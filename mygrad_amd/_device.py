@@ -28,6 +28,8 @@ says.
 import ctypes
 import weakref
 
+from math import prod
+
 import numpy as np
 
 from . import _hip
@@ -189,7 +191,7 @@ class DeviceArray:
 
     @property
     def size(self):
-        return int(np.prod(self.shape, dtype=np.int64))
+        return prod(self.shape)  # the shape is a tuple of Python ints
 
     @property
     def itemsize(self):

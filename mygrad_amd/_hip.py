@@ -388,6 +388,26 @@ def pool_desc(dtype, lead, pooled_shape, pool, stride, grid, dx_dtype=None):
     )
 
 
+_shared_descs = {}
+
+
+def shared_desc(build, *args, **kwargs):
+    """``build(*args, **kwargs)`` (one of the descriptor builders above and below), built once per
+    distinct set of arguments and handed out again: for the operations, which describe the same
+    layer at every step and never write to a descriptor.  Arguments that do not hash (lists,
+    arrays) get a descriptor of their own."""
+    try:
+        key = (build, args, tuple(kwargs.items()))
+        desc = _shared_descs.get(key)
+    except TypeError:
+        return build(*args, **kwargs)
+    if desc is None:
+        if len(_shared_descs) >= 4096:
+            _shared_descs.clear()
+        desc = _shared_descs[key] = build(*args, **kwargs)
+    return desc
+
+
 def bn_desc(shape, dtype, has_gamma, has_beta, eps):
     """Descriptor of a batch normalisation of an array of `shape` = (N, C, ...)."""
     spatial = 1

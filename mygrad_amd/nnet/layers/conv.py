@@ -16,6 +16,10 @@ from .utils import check_window_args
 __all__ = ["conv_nd", "ConvND"]
 
 
+_PLAIN = (int, tuple)  # settings that hash: the usual way to pass stride, padding and dilation
+_CHECKED = {}          # (x.shape, w.shape, stride, padding, dilation) -> what ConvND.__call__ derives from them
+
+
 def _per_axis(value, m, lowest):
     """int-or-sequence -> length-m int array, with the reference's assertion
     (conv.py:35-61): right length, every entry an integer >= ``lowest``."""
@@ -81,29 +85,47 @@ class ConvND(Operation):
         assert wd.shape[1] == xd.shape[1], "The channel-depth of the batch and filters must agree"
 
         m = wd.ndim - 2
-        x_shape = np.array(xd.shape[2:])
-        w_shape = np.array(wd.shape[2:])
-        dilation = _per_axis(dilation, m, 1)
-        padding = _per_axis(padding, m, 0)
-        stride = _per_axis(stride, m, 1)
+        # A layer is called with the same shapes and settings at every step: what the checks below
+        # made of them the first time (they passed) is kept and handed out again.
+        key = None
+        if type(stride) in _PLAIN and type(padding) in _PLAIN and type(dilation) in _PLAIN:
+            key = (tuple(xd.shape), tuple(wd.shape), stride, padding, dilation)
+        try:
+            checked = _CHECKED.get(key) if key is not None else None
+        except TypeError:  # a tuple of something that does not hash
+            key = checked = None
+        if checked is None:
+            x_shape = np.array(xd.shape[2:])
+            w_shape = np.array(wd.shape[2:])
+            dilation = _per_axis(dilation, m, 1)
+            padding = _per_axis(padding, m, 0)
+            stride = _per_axis(stride, m, 1)
 
-        out_shape = (x_shape + 2 * padding - ((w_shape - 1) * dilation + 1)) / stride + 1
-        if not all(i.is_integer() and i > 0 for i in out_shape):
-            raise ValueError(
-                "Stride and kernel dimensions are incompatible: \n"
-                f"Input dimensions: {tuple(x_shape)}\n"
-                f"Stride dimensions: {tuple(stride)}\n"
-                f"Kernel dimensions: {tuple(w_shape)}\n"
-                f"Padding dimensions: {tuple(padding)}\n"
-                f"Dilation dimensions: {tuple(dilation)}\n"
-            )
+            out_shape = (x_shape + 2 * padding - ((w_shape - 1) * dilation + 1)) / stride + 1
+            if not all(i.is_integer() and i > 0 for i in out_shape):
+                raise ValueError(
+                    "Stride and kernel dimensions are incompatible: \n"
+                    f"Input dimensions: {tuple(x_shape)}\n"
+                    f"Stride dimensions: {tuple(stride)}\n"
+                    f"Kernel dimensions: {tuple(w_shape)}\n"
+                    f"Padding dimensions: {tuple(padding)}\n"
+                    f"Dilation dimensions: {tuple(dilation)}\n"
+                )
+
+            # the window helper's own checks, applied to the padded extent (the
+            # reference windows the padded array: conv.py:81-88)
+            padded = tuple(xd.shape[:2]) + tuple(int(n + 2 * p) for n, p in zip(x_shape, padding))
+            check_window_args(padded, tuple(int(i) for i in w_shape), tuple(int(s) for s in stride),
+                              tuple(int(d) for d in dilation))
+            for arr in (padding, stride, dilation):
+                arr.flags.writeable = False  # shared between the operations that hit this entry
+            checked = (padding, stride, dilation, tuple(int(g) for g in out_shape))
+            if key is not None:
+                if len(_CHECKED) >= 1024:
+                    _CHECKED.clear()
+                _CHECKED[key] = checked
+        padding, stride, dilation, out_shape = checked
         self.padding, self.stride, self.dilation = padding, stride, dilation
-
-        # the window helper's own checks, applied to the padded extent (the
-        # reference windows the padded array: conv.py:81-88)
-        padded = tuple(xd.shape[:2]) + tuple(int(n + 2 * p) for n, p in zip(x_shape, padding))
-        check_window_args(padded, tuple(int(i) for i in w_shape), tuple(int(s) for s in stride),
-                          tuple(int(d) for d in dilation))
 
         if np.iscomplexobj(xd) or np.iscomplexobj(wd):
             return self._complex_forward(xd, wd)
@@ -134,7 +156,8 @@ class ConvND(Operation):
             self._desc = "folded"
             ob = _highrank.conv_forward(xb, wb, dtype, tuple(xd.shape), tuple(wd.shape), grid, stride, padding, dilation)
         else:
-            self._desc = _hip.conv_desc(dtype, xd.shape, wd.shape, grid, stride, padding, dilation)
+            self._desc = _hip.shared_desc(_hip.conv_desc, dtype, tuple(xd.shape), tuple(wd.shape), grid, tuple(stride), tuple(padding),
+                                          tuple(dilation))
             ob = _device.DeviceBuffer(int(np.prod(out_full)) * dtype.itemsize)
             _hip.check(_hip.lib().mg_conv_fwd(self._desc, xb.ptr, wb.ptr, ob.ptr))
         out, ob = _narrowed(ob, out_full, dtype, result_dtype)

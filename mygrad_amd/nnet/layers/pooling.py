@@ -3,6 +3,7 @@ signature, argument checks and errors (``mygrad/nnet/layers/pooling.py``),
 whose forward pass and gradient routing run as bandwidth-bound kernels in
 ``libmygrad_hip.so``."""
 
+from math import prod
 from numbers import Integral
 
 import numpy as np
@@ -25,17 +26,18 @@ class _Stage:
         self.pool = tuple(int(n) for n in pool)
         self.stride = tuple(int(n) for n in stride)
         self.grid = tuple((n - w) // s + 1 for n, w, s in zip(self.shape, self.pool, self.stride))
-        self.windows = self.lead * int(np.prod(self.grid, dtype=np.int64))
-        self.count = self.lead * int(np.prod(self.shape, dtype=np.int64))
+        self.windows = self.lead * prod(self.grid)
+        self.count = self.lead * prod(self.shape)
+        self.keeps_argmax = prod(self.pool) <= 256  # what one byte per window can tell apart
         self.argmax = None
         self.source = None  # the device buffer read by the forward pass (stages after the first)
 
     def desc(self, dtype, dx_dtype=None):
-        return _hip.pool_desc(dtype, self.lead, self.shape, self.pool, self.stride, self.grid, dx_dtype=dx_dtype)
+        return _hip.shared_desc(_hip.pool_desc, dtype, self.lead, self.shape, self.pool, self.stride, self.grid, dx_dtype=dx_dtype)
 
     def forward(self, dtype, xb):
         ob = _device.DeviceBuffer(self.windows * dtype.itemsize)
-        if int(np.prod(self.pool)) <= 256:
+        if self.keeps_argmax:
             # Each window's argmax (pooling.py:109-111) is found here, while x is being read
             # anyway, and kept on the device as one byte per window: the backward pass then
             # needs grad and these bytes only.
@@ -64,9 +66,9 @@ def plan_stages(lead, pooled, pool, stride, most=_hip.MG_MAX_ND):
     stages = []
     shape, window, step = [int(n) for n in pooled], [int(n) for n in pool], [int(n) for n in stride]
     while len(shape) > most:
-        stage = _Stage(int(lead) * int(np.prod(shape[:-most], dtype=np.int64)), shape[-most:], window[-most:], step[-most:])
+        stage = _Stage(int(lead) * prod(shape[:-most]), shape[-most:], window[-most:], step[-most:])
         stages.append(stage)
-        shape = shape[:-most] + [int(np.prod(stage.grid, dtype=np.int64))]
+        shape = shape[:-most] + [prod(stage.grid)]
         window, step = window[:-most] + [1], step[:-most] + [1]
     stages.append(_Stage(lead, shape, window, step))
     return stages
@@ -159,12 +161,12 @@ class MaxPoolND(Operation):
             xd = xd.astype(np.float32)  # on the device for a value that lives there, else on the host
         grid = tuple(int(g) for g in out_shape)
         self._grid = grid
-        self._lead = int(np.prod(lead_shape, dtype=np.int64))
+        self._lead = prod(int(n) for n in lead_shape)
         out_full = (*lead_shape, *grid)
         if self._lead == 0:
             return np.empty(out_full, dtype=result_dtype)
 
-        self._lead *= int(np.prod(pooled[:skip], dtype=np.int64))
+        self._lead *= prod(int(n) for n in pooled[:skip])
         stages = plan_stages(self._lead, pooled[skip:], pool[skip:], stride[skip:])
         self._stages = stages
 
