@@ -55,6 +55,14 @@ __all__ = [
 stats = {"h2d_bytes": 0, "d2h_bytes": 0, "mirror_hits": 0, "uploads": 0}
 
 
+def _count(shape):
+    """Elements of an array of ``shape`` (a sequence of extents, or one extent)."""
+    try:
+        return prod(int(n) for n in shape)
+    except TypeError:
+        return int(shape)
+
+
 def _free_device(ptr):
     try:
         _hip.load_library().mg_free(ptr)
@@ -72,14 +80,14 @@ def _free_pinned(ptr):
 class DeviceBuffer:
     """Owns one device allocation; freed when the last reference goes away."""
 
-    __slots__ = ("ptr", "nbytes", "_finalizer", "__weakref__")
+    __slots__ = ("ptr", "nbytes", "_owned", "__weakref__")
 
     def __init__(self, nbytes):
+        self._owned = None
         handle = ctypes.c_void_p()
         _hip.check(_hip.lib().mg_malloc(ctypes.byref(handle), int(nbytes)))
-        self.ptr = handle.value
+        self.ptr = self._owned = handle.value
         self.nbytes = int(nbytes)
-        self._finalizer = weakref.finalize(self, _free_device, self.ptr)
 
     def upload(self, arr):
         arr = np.ascontiguousarray(arr)
@@ -93,7 +101,12 @@ class DeviceBuffer:
         stats["d2h_bytes"] += arr.nbytes
 
     def free(self):
-        self._finalizer()
+        """Gives the block back (once; ``ptr`` keeps its value for whoever still compares it)."""
+        owned, self._owned = self._owned, None
+        if owned is not None:
+            _free_device(owned)
+
+    __del__ = free
 
 
 class _PinnedBlock:
@@ -114,7 +127,7 @@ def pinned_empty(shape, dtype):
     buffer); the pinned block is released when the last view dies.
     """
     dtype = np.dtype(dtype)
-    count = int(np.prod(shape, dtype=np.int64))
+    count = _count(shape)
     nbytes = max(count * dtype.itemsize, 1)
     block = _PinnedBlock(nbytes)
     raw = (ctypes.c_char * nbytes).from_address(block.ptr)
@@ -283,7 +296,7 @@ def full(shape, dtype, value):
     dtype = np.dtype(dtype)
     if dtype == np.float16:
         return full(shape, np.float32, value).astype(np.float16)
-    count = int(np.prod(shape, dtype=np.int64))
+    count = _count(shape)
     buf = DeviceBuffer(max(count * dtype.itemsize, 16))
     _hip.check(_hip.lib().mg_fill_value(_hip.dtype_code(dtype), count, float(value), buf.ptr))
     return DeviceArray(buf, shape, dtype)

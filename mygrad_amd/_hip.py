@@ -235,6 +235,8 @@ def check(status):
 def lib():
     """The loaded library with the device initialised; raises HipUnavailable otherwise."""
     global _ready
+    if _ready:
+        return _lib
     handle = load_library()
     if not _ready:
         device = int(os.environ.get("MYGRAD_HIP_DEVICE", "0"))
