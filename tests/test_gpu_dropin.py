@@ -242,6 +242,40 @@ def test_operand_variety():
     assert _graph.held_count() == 0
 
 
+def test_a_layer_called_again_reuses_its_checks_but_not_for_other_settings():
+    """ConvND keeps what its argument checks derived for a (shapes, settings) pair and the shared
+    descriptor of the layer: a second call gives the same result, other settings on the same shapes
+    get their own entry, and settings that the checks reject are rejected every time."""
+    rng = np.random.default_rng(77)
+    x, w = rng.standard_normal((2, 3, 9, 9)), rng.standard_normal((4, 3, 3, 3))
+    first = conv_nd(x, w, stride=1, padding=1, constant=True).data
+    again = conv_nd(x, w, stride=1, padding=1, constant=True).data
+    assert np.array_equal(first, again)
+    assert rel_err(first, direct.conv_forward(x, w, (1, 1), (1, 1), (1, 1))) < TOL[np.dtype(np.float64)]
+    for conf in (dict(stride=2, padding=0), dict(stride=(1, 1), padding=(0, 1)), dict(stride=1, padding=1, dilation=2),
+                 dict(stride=[1, 1], padding=np.array([1, 1]))):
+        stride, padding, dilation = (np.broadcast_to(np.asarray(conf.get(k, d)), (2,)) for k, d in
+                                     (("stride", 1), ("padding", 0), ("dilation", 1)))
+        if any((n + 2 * p - ((t - 1) * d + 1)) % s for n, t, s, p, d in zip((9, 9), (3, 3), stride, padding, dilation)):
+            with pytest.raises(ValueError):
+                conv_nd(x, w, **conf)
+            continue
+        for _ in range(2):
+            got = conv_nd(x, w, constant=True, **conf).data
+            want = direct.conv_forward(x, w, tuple(int(v) for v in stride), tuple(int(v) for v in padding),
+                                       tuple(int(v) for v in dilation))
+            assert got.shape == want.shape and rel_err(got, want) < TOL[np.dtype(np.float64)]
+    for _ in range(2):  # rejected before and after good calls with the same shapes
+        with pytest.raises(AssertionError):
+            conv_nd(x, w, stride=0, padding=1)
+        with pytest.raises(AssertionError):
+            conv_nd(x, w, stride=1, padding=(1, 1, 1))
+        with pytest.raises(ValueError):
+            conv_nd(x, w, stride=3, padding=1)
+    out = conv_nd(mg.Tensor(x), mg.Tensor(w), stride=1, padding=1)
+    assert not out.creator.stride.flags.writeable  # the arrays are shared between the operations of a layer
+
+
 def test_integer_operands_give_the_integer_result():
     """All-integer operands are constants; the reference multiplies them in integer arithmetic
     (np.tensordot, conv.py:96-99) and takes maxima of integers (pooling.py:93).  Here they run in

@@ -666,3 +666,24 @@ def test_pooling_stages_cover_any_number_of_axes():
         assert stages[-1].windows == lead * int(np.prod(grid))
         # window volumes multiply up to the whole window
         assert int(np.prod([np.prod(st.pool) for st in stages])) == int(np.prod(pool))
+
+
+def test_shared_descriptors_are_built_once_per_distinct_layer():
+    """``_hip.shared_desc`` hands the same descriptor object to every call with the same
+    arguments (the operations describe the same layer at every step), builds a fresh one for
+    arguments that do not hash, and never confuses two builders or two sets of settings."""
+    f32, f64 = np.dtype(np.float32), np.dtype(np.float64)
+    a = _hip.shared_desc(_hip.pool_desc, f32, 6, (8, 8), (2, 2), (2, 2), (4, 4), dx_dtype=None)
+    b = _hip.shared_desc(_hip.pool_desc, f32, 6, (8, 8), (2, 2), (2, 2), (4, 4), dx_dtype=None)
+    assert a is b
+    wide = _hip.shared_desc(_hip.pool_desc, f32, 6, (8, 8), (2, 2), (2, 2), (4, 4), dx_dtype=f64)
+    assert wide is not a and wide.dx_dtype == _hip.MG_F64 and a.dx_dtype == _hip.MG_F32
+    other = _hip.shared_desc(_hip.pool_desc, f32, 7, (8, 8), (2, 2), (2, 2), (4, 4), dx_dtype=None)
+    assert other is not a and other.lead == 7 and a.lead == 6
+    listed = _hip.shared_desc(_hip.pool_desc, f32, 6, [8, 8], [2, 2], [2, 2], [4, 4])
+    assert listed is not a and list(listed.X) == list(a.X) and list(listed.G) == list(a.G)
+    c = _hip.shared_desc(_hip.conv_desc, f64, (2, 3, 8, 8), (4, 3, 3, 3), (8, 8), (1, 1), (1, 1), (1, 1))
+    assert c is _hip.shared_desc(_hip.conv_desc, f64, (2, 3, 8, 8), (4, 3, 3, 3), (8, 8), (1, 1), (1, 1), (1, 1))
+    assert (c.N, c.C, c.F, list(c.pad)) == (2, 3, 4, [0, 1, 1])
+    fresh = _hip.conv_desc(f64, (2, 3, 8, 8), (4, 3, 3, 3), (8, 8), (1, 1), (1, 1), (1, 1))
+    assert fresh is not c  # the builders themselves always build
